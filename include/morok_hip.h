@@ -1,0 +1,207 @@
+/*
+ * morok_hip.h - C ABI of libmorok_hip.so, the MI355X (gfx950) device backend for morok.
+ *
+ * The library sits behind morok's device boundary
+ *     Device { Renderer, Compiler, RuntimeFactory -> Program, Allocator }
+ * (device/src/device.rs) and exports one C entry point per trait method a Rust shim
+ * would bind.  Each declaration cites the reference interface it stands for; paths are
+ * relative to the morok workspace root.
+ *
+ * Conventions
+ *   - every function returning int returns 0 on success, otherwise one of MRK_ERR_*;
+ *     the message is available from mrk_hip_last_error() (thread-local, valid until the
+ *     next failing call on the same thread).  No call panics or aborts across the ABI.
+ *   - all device work of one device id is queued on a single in-order HIP stream
+ *     (the execution loop of runtime/src/execution_plan.rs:168-181 relies on in-order
+ *     execution and never synchronises between kernels); copyout synchronises.
+ *   - launch dimensions: global_size = grid extent in workgroups, local_size = workgroup
+ *     extent in work-items (the gidx/lidx extents of schedule/src/gpudims.rs:153-156).
+ *   - all entry points are thread-safe (Renderer/Compiler are Send + Sync in the
+ *     reference, device.rs:142,186; kernels are shared across threads by the kernel cache,
+ *     runtime/src/kernel_cache.rs:46-50).
+ */
+#ifndef MOROK_HIP_H
+#define MOROK_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- status codes: variants of device/src/error.rs:5-51 ---- */
+#define MRK_OK 0
+#define MRK_ERR_SIZE_MISMATCH 1      /* Error::SizeMismatch */
+#define MRK_ERR_COPY_FAILED 2        /* Error::CopyFailed */
+#define MRK_ERR_INVALID_DEVICE 3     /* Error::InvalidDevice */
+#define MRK_ERR_NOT_ALLOCATED 4      /* Error::NotAllocated */
+#define MRK_ERR_NOT_CPU_ACCESSIBLE 5 /* Error::NotCpuAccessible */
+#define MRK_ERR_INVALID_VIEW 6       /* Error::InvalidView */
+#define MRK_ERR_RUNTIME 7            /* Error::Runtime */
+#define MRK_ERR_HIP 8                /* backend variant, cf. Error::CudaError (error.rs:47-50) */
+#define MRK_ERR_RENDER 9             /* RenderKernel context, tensor/src/realize.rs:42-46 */
+#define MRK_ERR_COMPILE 10           /* CompileKernel context */
+#define MRK_ERR_INVALID_ARGUMENT 11
+#define MRK_ERR_TIMEOUT 12           /* TimelineSignal::wait timeout, device/src/sync.rs:118-168 */
+#define MRK_ERR_UNSUPPORTED_DEVICE 13 /* runtime/src/device_registry.rs:114-120 */
+
+const char* mrk_hip_last_error(void);
+
+/* ---- opaque handles ---- */
+typedef struct mrk_buffer mrk_buffer;               /* device::Buffer        (device/src/buffer.rs:97-110) */
+typedef struct mrk_program_spec mrk_program_spec;   /* device::ProgramSpec   (device/src/device.rs:327-367) */
+typedef struct mrk_compiled_spec mrk_compiled_spec; /* device::CompiledSpec  (device/src/device.rs:72-100) */
+typedef struct mrk_program mrk_program;             /* Box<dyn Program>      (device/src/device.rs:34-60) */
+typedef struct mrk_event mrk_event;                 /* hipEvent pair member for timing */
+
+/* =====================================================================================
+ * Device registry and factory
+ * ===================================================================================== */
+
+/* DeviceSpecExt::parse (device/src/registry.rs:26-81) with the HIP arm: accepts
+ * "HIP", "HIP:n", "AMD[:n]", "GPU[:n]" (case-insensitive); anything else -> INVALID_DEVICE. */
+int mrk_hip_device_parse(const char* spec, int* device_id);
+/* Number of visible HIP devices. */
+int mrk_hip_device_count(int* count);
+/* DEVICE_FACTORIES.device(spec, registry) (runtime/src/device_registry.rs:99-127): creates
+ * (once) the device bundle - allocator, renderer, compiler, runtime factory - for the id.
+ * Registered under the base type string "HIP" (register_factory, device_registry.rs:81-83). */
+int mrk_hip_device_create(int device_id);
+/* Looks a factory up by base type string; unknown types -> UNSUPPORTED_DEVICE
+ * (device_registry.rs:114-120). */
+int mrk_hip_device_create_by_type(const char* device_type, int device_id);
+/* Allocator::name (device/src/allocator.rs:186) / Device::base_device_key (device.rs:310-312). */
+const char* mrk_hip_name(void);
+/* The device's HIP stream (hipStream_t) for interop with caller-side HIP code. */
+int mrk_hip_device_stream(int device_id, void** stream);
+
+/* =====================================================================================
+ * Allocator (device/src/allocator.rs:180-190) behind the LRU cache (allocator.rs:330-442)
+ * ===================================================================================== */
+
+/* Allocator::alloc(size, &BufferOptions{zero_init, cpu_accessible}).
+ * cpu_accessible = 0 -> hipMalloc; 1 -> hipMallocManaged (as CudaUnified, allocator.rs:278-286). */
+int mrk_hip_alloc(int device_id, size_t size, int zero_init, int cpu_accessible, void** out);
+/* Allocator::free: parks the allocation in the LRU cache (<= 32 per (size, cpu_accessible)). */
+int mrk_hip_free(int device_id, void* ptr, size_t size, int cpu_accessible);
+/* Allocator::synchronize (allocator.rs:183-185). */
+int mrk_hip_sync(int device_id);
+/* LruAllocator::cache_count / total_cached (allocator.rs:350-363) and cache clear. */
+int mrk_hip_lru_cache_count(int device_id, size_t size, int cpu_accessible, size_t* count);
+int mrk_hip_lru_total_cached(int device_id, size_t* count);
+int mrk_hip_lru_clear(int device_id);
+/* Raw copies for callers that hold device pointers from mrk_hip_alloc
+ * (device/src/buffer.rs:351-366,390-407,444-532).  copyout waits for all queued work first. */
+int mrk_hip_copyin(int device_id, void* dst, size_t dst_offset, const void* src_host, size_t size);
+int mrk_hip_copyout(int device_id, void* dst_host, const void* src, size_t src_offset, size_t size);
+int mrk_hip_copy_dd(int device_id, void* dst, size_t dst_offset, const void* src, size_t src_offset, size_t size);
+
+/* =====================================================================================
+ * Buffer (device/src/buffer.rs)
+ * ===================================================================================== */
+
+/* Buffer::new (buffer.rs:112-121): lazy, nothing is allocated until first use. */
+int mrk_hip_buffer_new(int device_id, size_t size, int zero_init, int cpu_accessible, mrk_buffer** out);
+/* Buffer::ensure_allocated / is_allocated (buffer.rs:153-160). */
+int mrk_hip_buffer_ensure_allocated(mrk_buffer* b);
+int mrk_hip_buffer_is_allocated(const mrk_buffer* b);
+/* Buffer::view (buffer.rs:136-150): shares the allocation and the id; INVALID_VIEW when
+ * offset + size exceeds the buffer. */
+int mrk_hip_buffer_view(const mrk_buffer* b, size_t offset, size_t size, mrk_buffer** out);
+/* Buffer::copyin / copyout / copy_from (buffer.rs:332-368,371-408,411-534): SIZE_MISMATCH
+ * unless the byte counts match exactly. */
+int mrk_hip_buffer_copyin(mrk_buffer* b, const void* src, size_t size);
+int mrk_hip_buffer_copyout(const mrk_buffer* b, void* dst, size_t size);
+int mrk_hip_buffer_copy_from(mrk_buffer* dst, const mrk_buffer* src);
+/* Buffer::as_raw_ptr (buffer.rs:554-574): device address + view offset; NOT_ALLOCATED before
+ * allocation (the reference panics). */
+int mrk_hip_buffer_raw_ptr(const mrk_buffer* b, void** out);
+/* Buffer::id / size (buffer.rs:327-329). */
+uint64_t mrk_hip_buffer_id(const mrk_buffer* b);
+size_t mrk_hip_buffer_size(const mrk_buffer* b);
+/* Buffer::synchronize (buffer.rs:537-539). */
+int mrk_hip_buffer_synchronize(const mrk_buffer* b);
+/* Drop: the allocation returns to the allocator when the last view is released
+ * (buffer.rs:86-93). */
+void mrk_hip_buffer_release(mrk_buffer* b);
+
+/* =====================================================================================
+ * Compiler (device/src/device.rs:142-177) and ProgramSpec / CompiledSpec accessors
+ * ===================================================================================== */
+
+/* Builds a ProgramSpec from already-rendered HIP-C source (what Renderer::render returns).
+ * var_is_i64[i] != 0 -> scalar argument i is `long long`, else `int`.  global/local may be
+ * NULL when the launch sizes are supplied at execute time. */
+int mrk_hip_program_spec_from_source(const char* name, const char* src, size_t buf_count, const char* const* var_names,
+                                     const uint8_t* var_is_i64, size_t nvars, const size_t global_size[3],
+                                     const size_t local_size[3], mrk_program_spec** out);
+const char* mrk_hip_program_spec_name(const mrk_program_spec* s);
+const char* mrk_hip_program_spec_src(const mrk_program_spec* s);
+size_t mrk_hip_program_spec_buf_count(const mrk_program_spec* s);
+size_t mrk_hip_program_spec_var_count(const mrk_program_spec* s);
+const char* mrk_hip_program_spec_var_name(const mrk_program_spec* s, size_t i);
+/* Returns 1 and fills the arrays if the spec carries launch sizes, else 0. */
+int mrk_hip_program_spec_sizes(const mrk_program_spec* s, size_t global_size[3], size_t local_size[3]);
+/* globals / outs / ins PARAM slot lists (device.rs:353-363): which = 0,1,2. */
+size_t mrk_hip_program_spec_slots(const mrk_program_spec* s, int which, size_t* out, size_t cap);
+void mrk_hip_program_spec_release(mrk_program_spec* s);
+
+/* Compiler::compile (device.rs:170): HIP-C -> gfx950 code object, in process.  AOT
+ * convention (device.rs:118-120,153-169): bytes populated, src absent. */
+int mrk_hip_compile(const mrk_program_spec* spec, mrk_compiled_spec** out);
+/* Compiler::cache_key (device.rs:176): "hip-gfx950". */
+const char* mrk_hip_cache_key(void);
+const char* mrk_hip_compiled_spec_name(const mrk_compiled_spec* c);
+size_t mrk_hip_compiled_spec_bytes(const mrk_compiled_spec* c, const uint8_t** bytes);
+int mrk_hip_compiled_spec_has_src(const mrk_compiled_spec* c);
+void mrk_hip_compiled_spec_release(mrk_compiled_spec* c);
+
+/* =====================================================================================
+ * RuntimeFactory and Program (device/src/device.rs:34-60,234)
+ * ===================================================================================== */
+
+/* RuntimeFactory(&CompiledSpec) -> Box<dyn Program>: hipModuleLoadData +
+ * hipModuleGetFunction(spec.name). */
+int mrk_hip_program_create(int device_id, const mrk_compiled_spec* spec, mrk_program** out);
+/* Program::execute(buffers, vals, global_size, local_size) (device.rs:50-56):
+ * hipModuleLaunchKernel with the buffer pointers first, then vals in var_names order
+ * (same positional order as runtime/src/dispatch.rs:67-69).  global/local may be NULL to
+ * use the sizes recorded in the spec.  Asynchronous: returns once the launch is queued. */
+int mrk_hip_program_execute(mrk_program* p, void* const* buffers, size_t nbufs, const int64_t* vals, size_t nvals,
+                            const size_t global_size[3], const size_t local_size[3]);
+/* Program::name (device.rs:59). */
+const char* mrk_hip_program_name(const mrk_program* p);
+void mrk_hip_program_destroy(mrk_program* p);
+
+/* Hand-written gfx950 kernels exposed as Programs, so that an ExecutionPlan can hold them
+ * next to generated kernels.  `kind` and the meaning of `params`:
+ *   "softmax_f32"     params = {rows, cols}                         buffers = {y, x}
+ * Buffer order follows the reference's PARAM numbering: outputs first. */
+int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_program** out);
+
+/* =====================================================================================
+ * Hand-written kernels, direct entry points (device pointers, queued on the device stream)
+ * ===================================================================================== */
+
+/* Fused row softmax over the last axis, f32 [rows, cols] row-major: the lazy graph of
+ * Tensor::softmax (tensor/src/activation.rs:90-101) in one kernel instead of the
+ * reference's three (tensor/src/test/unit/fusion.rs:83-88). */
+int mrk_hip_softmax_f32(int device_id, const void* x, void* y, int64_t rows, int64_t cols);
+/* Same with an explicit implementation variant (0 default, 1 one-wave-per-row); tuning only. */
+int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t rows, int64_t cols, int variant);
+
+/* =====================================================================================
+ * Events (hipEvent timing; stands where benchmark_kernel / execute_profiled use Instant,
+ * runtime/src/benchmark.rs:64-91, runtime/src/execution_plan.rs:200-221)
+ * ===================================================================================== */
+int mrk_hip_event_create(int device_id, mrk_event** out);
+int mrk_hip_event_record(mrk_event* e);
+int mrk_hip_event_synchronize(mrk_event* e);
+int mrk_hip_event_elapsed_ms(mrk_event* start, mrk_event* stop, float* ms);
+void mrk_hip_event_destroy(mrk_event* e);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MOROK_HIP_H */

@@ -1,0 +1,10 @@
+"""morok_amd: MI355X (gfx950) device backend for morok behind its Device boundary.
+
+Importing the package loads morok_amd/libmorok_hip.so; nothing here computes on the CPU.
+"""
+from ._ffi import MorokHipError, lib, declared_symbols  # noqa: F401
+from .device import (  # noqa: F401
+    Buffer, CompiledSpec, Device, Event, Program, ProgramSpec, cache_key, compile_spec, device_count, parse_device,
+    time_launches,
+)
+from . import ops  # noqa: F401

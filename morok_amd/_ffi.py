@@ -1,0 +1,120 @@
+"""ctypes binding of libmorok_hip.so (the C ABI declared in include/morok_hip.h).
+
+The library is loaded from the package directory; there is no fallback of any kind: if
+the shared object is missing, importing this module raises.
+"""
+import ctypes as C
+import os
+import re
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmorok_hip.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "morok_hip.h")
+
+
+class MorokHipError(RuntimeError):
+    """An entry point returned a non-zero status; `code` is one of the MRK_ERR_* values."""
+
+    def __init__(self, code, message):
+        super().__init__(f"[{code}] {message}")
+        self.code = code
+        self.message = message
+
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+        "or `make -C morok_amd/csrc` (there is no CPU fallback)"
+    )
+
+lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+
+c_size_p = C.POINTER(C.c_size_t)
+c_void_pp = C.POINTER(C.c_void_p)
+c_i64_p = C.POINTER(C.c_int64)
+
+_SIGS = {
+    "mrk_hip_last_error": (C.c_char_p, []),
+    "mrk_hip_device_parse": (C.c_int, [C.c_char_p, C.POINTER(C.c_int)]),
+    "mrk_hip_device_count": (C.c_int, [C.POINTER(C.c_int)]),
+    "mrk_hip_device_create": (C.c_int, [C.c_int]),
+    "mrk_hip_device_create_by_type": (C.c_int, [C.c_char_p, C.c_int]),
+    "mrk_hip_name": (C.c_char_p, []),
+    "mrk_hip_device_stream": (C.c_int, [C.c_int, c_void_pp]),
+    "mrk_hip_alloc": (C.c_int, [C.c_int, C.c_size_t, C.c_int, C.c_int, c_void_pp]),
+    "mrk_hip_free": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_int]),
+    "mrk_hip_sync": (C.c_int, [C.c_int]),
+    "mrk_hip_lru_cache_count": (C.c_int, [C.c_int, C.c_size_t, C.c_int, c_size_p]),
+    "mrk_hip_lru_total_cached": (C.c_int, [C.c_int, c_size_p]),
+    "mrk_hip_lru_clear": (C.c_int, [C.c_int]),
+    "mrk_hip_copyin": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t]),
+    "mrk_hip_copyout": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t]),
+    "mrk_hip_copy_dd": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_void_p, C.c_size_t, C.c_size_t]),
+    "mrk_hip_buffer_new": (C.c_int, [C.c_int, C.c_size_t, C.c_int, C.c_int, c_void_pp]),
+    "mrk_hip_buffer_ensure_allocated": (C.c_int, [C.c_void_p]),
+    "mrk_hip_buffer_is_allocated": (C.c_int, [C.c_void_p]),
+    "mrk_hip_buffer_view": (C.c_int, [C.c_void_p, C.c_size_t, C.c_size_t, c_void_pp]),
+    "mrk_hip_buffer_copyin": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "mrk_hip_buffer_copyout": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "mrk_hip_buffer_copy_from": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "mrk_hip_buffer_raw_ptr": (C.c_int, [C.c_void_p, c_void_pp]),
+    "mrk_hip_buffer_id": (C.c_uint64, [C.c_void_p]),
+    "mrk_hip_buffer_size": (C.c_size_t, [C.c_void_p]),
+    "mrk_hip_buffer_synchronize": (C.c_int, [C.c_void_p]),
+    "mrk_hip_buffer_release": (None, [C.c_void_p]),
+    "mrk_hip_program_spec_from_source": (
+        C.c_int,
+        [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_char_p), C.POINTER(C.c_uint8), C.c_size_t, c_size_p,
+         c_size_p, c_void_pp],
+    ),
+    "mrk_hip_program_spec_name": (C.c_char_p, [C.c_void_p]),
+    "mrk_hip_program_spec_src": (C.c_char_p, [C.c_void_p]),
+    "mrk_hip_program_spec_buf_count": (C.c_size_t, [C.c_void_p]),
+    "mrk_hip_program_spec_var_count": (C.c_size_t, [C.c_void_p]),
+    "mrk_hip_program_spec_var_name": (C.c_char_p, [C.c_void_p, C.c_size_t]),
+    "mrk_hip_program_spec_sizes": (C.c_int, [C.c_void_p, c_size_p, c_size_p]),
+    "mrk_hip_program_spec_slots": (C.c_size_t, [C.c_void_p, C.c_int, c_size_p, C.c_size_t]),
+    "mrk_hip_program_spec_release": (None, [C.c_void_p]),
+    "mrk_hip_compile": (C.c_int, [C.c_void_p, c_void_pp]),
+    "mrk_hip_cache_key": (C.c_char_p, []),
+    "mrk_hip_compiled_spec_name": (C.c_char_p, [C.c_void_p]),
+    "mrk_hip_compiled_spec_bytes": (C.c_size_t, [C.c_void_p, C.POINTER(C.POINTER(C.c_uint8))]),
+    "mrk_hip_compiled_spec_has_src": (C.c_int, [C.c_void_p]),
+    "mrk_hip_compiled_spec_release": (None, [C.c_void_p]),
+    "mrk_hip_program_create": (C.c_int, [C.c_int, C.c_void_p, c_void_pp]),
+    "mrk_hip_program_execute": (C.c_int, [C.c_void_p, c_void_pp, C.c_size_t, c_i64_p, C.c_size_t, c_size_p, c_size_p]),
+    "mrk_hip_program_name": (C.c_char_p, [C.c_void_p]),
+    "mrk_hip_program_destroy": (None, [C.c_void_p]),
+    "mrk_hip_program_builtin": (C.c_int, [C.c_int, C.c_char_p, c_i64_p, C.c_size_t, c_void_pp]),
+    "mrk_hip_softmax_f32": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
+    "mrk_hip_softmax_f32_variant": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int]),
+    "mrk_hip_event_create": (C.c_int, [C.c_int, c_void_pp]),
+    "mrk_hip_event_record": (C.c_int, [C.c_void_p]),
+    "mrk_hip_event_synchronize": (C.c_int, [C.c_void_p]),
+    "mrk_hip_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
+    "mrk_hip_event_destroy": (None, [C.c_void_p]),
+}
+
+
+def declared_symbols(header_path=HEADER_PATH):
+    """Names of every function declared in the public header."""
+    text = open(header_path).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mrk_\w+)\s*\(", text)))
+
+
+def _bind():
+    for name, (res, args) in _SIGS.items():
+        fn = getattr(lib, name)  # AttributeError if the library does not export it
+        fn.restype = res
+        fn.argtypes = args
+
+
+_bind()
+
+
+def check(rc):
+    """Raises MorokHipError for a non-zero status."""
+    if rc != 0:
+        raise MorokHipError(rc, lib.mrk_hip_last_error().decode("utf-8", "replace"))
+    return rc

@@ -1,0 +1,72 @@
+// Hand-written gfx950 kernels wrapped as Programs so that execution plans can hold them
+// beside generated kernels (device/src/device.rs:34-60).  Buffer order follows the
+// reference's PARAM numbering: outputs first, then inputs.
+#include <cstring>
+
+#include "builtin.h"
+#include "error.h"
+#include "kernels/kernels.h"
+
+namespace mrk {
+
+namespace {
+
+class BuiltinProgram final : public Program {
+  public:
+    using Fn = std::function<int(ffi::Stream, void* const*, const std::vector<int64_t>&)>;
+    BuiltinProgram(int device_id, ffi::Stream stream, std::string name, size_t nbufs, std::vector<int64_t> params, Fn fn)
+        : device_id_(device_id),
+          stream_(stream),
+          name_(std::move(name)),
+          nbufs_(nbufs),
+          params_(std::move(params)),
+          fn_(std::move(fn)) {}
+    int execute(void* const* buffers, size_t nbufs, const int64_t*, size_t nvals, const size_t*,
+                const size_t*) override {
+        if (nbufs != nbufs_)
+            return failf(kInvalidArgument, "kernel '%s' expects %zu buffers, got %zu", name_.c_str(), nbufs_, nbufs);
+        if (nvals != 0)
+            return failf(kInvalidArgument, "kernel '%s' takes no variable values, got %zu", name_.c_str(), nvals);
+        for (size_t i = 0; i < nbufs; i++)
+            if (!buffers[i]) return failf(kInvalidArgument, "kernel '%s': buffer %zu is null", name_.c_str(), i);
+        MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
+        int rc = fn_(stream_, buffers, params_);
+        if (rc != 0) return fail_hip(rc, name_.c_str());
+        return kOk;
+    }
+    const char* name() const override { return name_.c_str(); }
+
+  private:
+    int device_id_;
+    ffi::Stream stream_;
+    std::string name_;
+    size_t nbufs_;
+    std::vector<int64_t> params_;
+    Fn fn_;
+};
+
+}  // namespace
+
+int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, const int64_t* params, size_t nparams,
+                           std::unique_ptr<Program>* out) {
+    std::vector<int64_t> p(params, params + nparams);
+    std::string k(kind ? kind : "");
+    auto need = [&](size_t n) -> int {
+        if (nparams != n)
+            return failf(kInvalidArgument, "builtin '%s' takes %zu parameters, got %zu", k.c_str(), n, nparams);
+        return kOk;
+    };
+    if (k == "softmax_f32") {
+        MRK_TRY(need(2));
+        if (p[0] < 0 || p[1] < 0) return fail(kInvalidArgument, "softmax_f32: negative shape");
+        std::string name = "softmax_f32_" + std::to_string(p[0]) + "_" + std::to_string(p[1]);
+        out->reset(new BuiltinProgram(device_id, stream, name, 2, p,
+                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_softmax_f32(s, b[1], b[0], q[0], q[1], 0);
+                                      }));
+        return kOk;
+    }
+    return fail(kInvalidArgument, "unknown builtin kernel kind: " + k);
+}
+
+}  // namespace mrk

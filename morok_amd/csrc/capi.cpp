@@ -1,0 +1,382 @@
+// extern "C" surface of libmorok_hip.so (declared in include/morok_hip.h).
+#include <cstring>
+
+#include "../../include/morok_hip.h"
+#include "buffer.h"
+#include "builtin.h"
+#include "device.h"
+#include "error.h"
+#include "kernels/kernels.h"
+
+using namespace mrk;
+
+struct mrk_buffer {
+    std::unique_ptr<Buffer> b;
+};
+struct mrk_program_spec {
+    ProgramSpec s;
+};
+struct mrk_compiled_spec {
+    CompiledSpec c;
+};
+struct mrk_program {
+    std::unique_ptr<Program> p;
+};
+struct mrk_event {
+    int device_id;
+    ffi::Event e;
+    ffi::Stream stream;
+};
+
+namespace {
+
+int get_device(int device_id, std::shared_ptr<Device>* out) {
+    return DeviceFactoryRegistry::global().device("HIP", device_id, out);
+}
+int get_lru(int device_id, LruAllocator** out) {
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    *out = static_cast<LruAllocator*>(d->allocator.get());
+    return kOk;
+}
+#define MRK_NONNULL(p)                                                                     \
+    do {                                                                                   \
+        if (!(p)) return fail(kInvalidArgument, "null argument: " #p);                     \
+    } while (0)
+
+}  // namespace
+
+extern "C" {
+
+const char* mrk_hip_last_error(void) { return last_error(); }
+
+int mrk_hip_device_parse(const char* spec, int* device_id) {
+    MRK_NONNULL(device_id);
+    return parse_device_spec(spec, device_id);
+}
+int mrk_hip_device_count(int* count) {
+    MRK_NONNULL(count);
+    MRK_HIP(ffi::device_count(count), "hipGetDeviceCount");
+    return kOk;
+}
+int mrk_hip_device_create(int device_id) {
+    std::shared_ptr<Device> d;
+    return get_device(device_id, &d);
+}
+int mrk_hip_device_create_by_type(const char* device_type, int device_id) {
+    MRK_NONNULL(device_type);
+    std::shared_ptr<Device> d;
+    return DeviceFactoryRegistry::global().device(device_type, device_id, &d);
+}
+const char* mrk_hip_name(void) { return Device::base_device_key(); }
+int mrk_hip_device_stream(int device_id, void** stream) {
+    MRK_NONNULL(stream);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    *stream = d->allocator->stream();
+    return kOk;
+}
+
+int mrk_hip_alloc(int device_id, size_t size, int zero_init, int cpu_accessible, void** out) {
+    MRK_NONNULL(out);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    BufferOptions o;
+    o.zero_init = zero_init != 0;
+    o.cpu_accessible = cpu_accessible != 0;
+    RawBuffer rb;
+    MRK_TRY(d->allocator->alloc(size, o, &rb));
+    *out = rb.ptr;
+    return kOk;
+}
+int mrk_hip_free(int device_id, void* ptr, size_t size, int cpu_accessible) {
+    if (!ptr) return kOk;
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    BufferOptions o;
+    o.cpu_accessible = cpu_accessible != 0;
+    RawBuffer rb;
+    rb.ptr = ptr;
+    rb.size = size;
+    rb.cpu_accessible = o.cpu_accessible;
+    d->allocator->free(rb, o);
+    return kOk;
+}
+int mrk_hip_sync(int device_id) {
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    return d->allocator->synchronize();
+}
+int mrk_hip_lru_cache_count(int device_id, size_t size, int cpu_accessible, size_t* count) {
+    MRK_NONNULL(count);
+    LruAllocator* lru;
+    MRK_TRY(get_lru(device_id, &lru));
+    *count = lru->cache_count(size, cpu_accessible != 0);
+    return kOk;
+}
+int mrk_hip_lru_total_cached(int device_id, size_t* count) {
+    MRK_NONNULL(count);
+    LruAllocator* lru;
+    MRK_TRY(get_lru(device_id, &lru));
+    *count = lru->total_cached();
+    return kOk;
+}
+int mrk_hip_lru_clear(int device_id) {
+    LruAllocator* lru;
+    MRK_TRY(get_lru(device_id, &lru));
+    lru->clear();
+    return kOk;
+}
+int mrk_hip_copyin(int device_id, void* dst, size_t dst_offset, const void* src_host, size_t size) {
+    if (size == 0) return kOk;
+    MRK_NONNULL(dst);
+    MRK_NONNULL(src_host);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(ffi::memcpy_htod_async(static_cast<char*>(dst) + dst_offset, src_host, size, d->allocator->stream()),
+            "hipMemcpyAsync(HtoD)");
+    MRK_HIP(ffi::stream_synchronize(d->allocator->stream()), "hipStreamSynchronize");
+    return kOk;
+}
+int mrk_hip_copyout(int device_id, void* dst_host, const void* src, size_t src_offset, size_t size) {
+    if (size == 0) return kOk;
+    MRK_NONNULL(dst_host);
+    MRK_NONNULL(src);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(ffi::memcpy_dtoh_async(dst_host, static_cast<const char*>(src) + src_offset, size, d->allocator->stream()),
+            "hipMemcpyAsync(DtoH)");
+    MRK_HIP(ffi::stream_synchronize(d->allocator->stream()), "hipStreamSynchronize");
+    return kOk;
+}
+int mrk_hip_copy_dd(int device_id, void* dst, size_t dst_offset, const void* src, size_t src_offset, size_t size) {
+    if (size == 0) return kOk;
+    MRK_NONNULL(dst);
+    MRK_NONNULL(src);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(ffi::memcpy_dtod_async(static_cast<char*>(dst) + dst_offset, static_cast<const char*>(src) + src_offset,
+                                   size, d->allocator->stream()),
+            "hipMemcpyAsync(DtoD)");
+    return kOk;
+}
+
+int mrk_hip_buffer_new(int device_id, size_t size, int zero_init, int cpu_accessible, mrk_buffer** out) {
+    MRK_NONNULL(out);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    BufferOptions o;
+    o.zero_init = zero_init != 0;
+    o.cpu_accessible = cpu_accessible != 0;
+    auto* h = new mrk_buffer();
+    h->b.reset(new Buffer(d->allocator, size, o));
+    *out = h;
+    return kOk;
+}
+int mrk_hip_buffer_ensure_allocated(mrk_buffer* b) {
+    MRK_NONNULL(b);
+    return b->b->ensure_allocated();
+}
+int mrk_hip_buffer_is_allocated(const mrk_buffer* b) { return b && b->b->is_allocated() ? 1 : 0; }
+int mrk_hip_buffer_view(const mrk_buffer* b, size_t offset, size_t size, mrk_buffer** out) {
+    MRK_NONNULL(b);
+    MRK_NONNULL(out);
+    std::unique_ptr<Buffer> v;
+    MRK_TRY(b->b->view(offset, size, &v));
+    auto* h = new mrk_buffer();
+    h->b = std::move(v);
+    *out = h;
+    return kOk;
+}
+int mrk_hip_buffer_copyin(mrk_buffer* b, const void* src, size_t size) {
+    MRK_NONNULL(b);
+    if (size) MRK_NONNULL(src);
+    return b->b->copyin(src, size);
+}
+int mrk_hip_buffer_copyout(const mrk_buffer* b, void* dst, size_t size) {
+    MRK_NONNULL(b);
+    if (size) MRK_NONNULL(dst);
+    return b->b->copyout(dst, size);
+}
+int mrk_hip_buffer_copy_from(mrk_buffer* dst, const mrk_buffer* src) {
+    MRK_NONNULL(dst);
+    MRK_NONNULL(src);
+    return dst->b->copy_from(*src->b);
+}
+int mrk_hip_buffer_raw_ptr(const mrk_buffer* b, void** out) {
+    MRK_NONNULL(b);
+    MRK_NONNULL(out);
+    return b->b->as_raw_ptr(out);
+}
+uint64_t mrk_hip_buffer_id(const mrk_buffer* b) { return b ? b->b->id() : 0; }
+size_t mrk_hip_buffer_size(const mrk_buffer* b) { return b ? b->b->size() : 0; }
+int mrk_hip_buffer_synchronize(const mrk_buffer* b) {
+    MRK_NONNULL(b);
+    return b->b->synchronize();
+}
+void mrk_hip_buffer_release(mrk_buffer* b) { delete b; }
+
+int mrk_hip_program_spec_from_source(const char* name, const char* src, size_t buf_count, const char* const* var_names,
+                                     const uint8_t* var_is_i64, size_t nvars, const size_t global_size[3],
+                                     const size_t local_size[3], mrk_program_spec** out) {
+    MRK_NONNULL(name);
+    MRK_NONNULL(src);
+    MRK_NONNULL(out);
+    auto* h = new mrk_program_spec();
+    h->s.name = name;
+    h->s.src = src;
+    h->s.buf_count = buf_count;
+    for (size_t i = 0; i < nvars; i++) {
+        h->s.var_names.push_back(var_names[i]);
+        h->s.var_is_i64.push_back(var_is_i64 ? var_is_i64[i] : 0);
+        h->s.vars.push_back(Variable{var_names[i], 0, 0});
+    }
+    if (global_size && local_size) {
+        h->s.has_sizes = true;
+        for (int i = 0; i < 3; i++) {
+            h->s.global_size[i] = global_size[i];
+            h->s.local_size[i] = local_size[i];
+        }
+    }
+    for (size_t i = 0; i < buf_count; i++) h->s.globals.push_back(i);
+    *out = h;
+    return kOk;
+}
+const char* mrk_hip_program_spec_name(const mrk_program_spec* s) { return s ? s->s.name.c_str() : ""; }
+const char* mrk_hip_program_spec_src(const mrk_program_spec* s) { return s ? s->s.src.c_str() : ""; }
+size_t mrk_hip_program_spec_buf_count(const mrk_program_spec* s) { return s ? s->s.buf_count : 0; }
+size_t mrk_hip_program_spec_var_count(const mrk_program_spec* s) { return s ? s->s.var_names.size() : 0; }
+const char* mrk_hip_program_spec_var_name(const mrk_program_spec* s, size_t i) {
+    return (s && i < s->s.var_names.size()) ? s->s.var_names[i].c_str() : "";
+}
+int mrk_hip_program_spec_sizes(const mrk_program_spec* s, size_t global_size[3], size_t local_size[3]) {
+    if (!s || !s->s.has_sizes) return 0;
+    for (int i = 0; i < 3; i++) {
+        if (global_size) global_size[i] = s->s.global_size[i];
+        if (local_size) local_size[i] = s->s.local_size[i];
+    }
+    return 1;
+}
+size_t mrk_hip_program_spec_slots(const mrk_program_spec* s, int which, size_t* out, size_t cap) {
+    if (!s) return 0;
+    const std::vector<size_t>& v = which == 0 ? s->s.globals : which == 1 ? s->s.outs : s->s.ins;
+    for (size_t i = 0; i < v.size() && i < cap; i++) out[i] = v[i];
+    return v.size();
+}
+void mrk_hip_program_spec_release(mrk_program_spec* s) { delete s; }
+
+int mrk_hip_compile(const mrk_program_spec* spec, mrk_compiled_spec** out) {
+    MRK_NONNULL(spec);
+    MRK_NONNULL(out);
+    auto compiler = make_hiprtc_compiler();
+    auto* h = new mrk_compiled_spec();
+    int rc = compiler->compile(spec->s, &h->c);
+    if (rc != kOk) {
+        delete h;
+        return rc;
+    }
+    *out = h;
+    return kOk;
+}
+const char* mrk_hip_cache_key(void) {
+    static std::shared_ptr<Compiler> c = make_hiprtc_compiler();
+    return c->cache_key();
+}
+const char* mrk_hip_compiled_spec_name(const mrk_compiled_spec* c) { return c ? c->c.name.c_str() : ""; }
+size_t mrk_hip_compiled_spec_bytes(const mrk_compiled_spec* c, const uint8_t** bytes) {
+    if (!c) return 0;
+    if (bytes) *bytes = c->c.bytes.data();
+    return c->c.bytes.size();
+}
+int mrk_hip_compiled_spec_has_src(const mrk_compiled_spec* c) { return c && c->c.has_src ? 1 : 0; }
+void mrk_hip_compiled_spec_release(mrk_compiled_spec* c) { delete c; }
+
+int mrk_hip_program_create(int device_id, const mrk_compiled_spec* spec, mrk_program** out) {
+    MRK_NONNULL(spec);
+    MRK_NONNULL(out);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    std::unique_ptr<Program> p;
+    MRK_TRY(d->runtime(spec->c, &p));
+    auto* h = new mrk_program();
+    h->p = std::move(p);
+    *out = h;
+    return kOk;
+}
+int mrk_hip_program_execute(mrk_program* p, void* const* buffers, size_t nbufs, const int64_t* vals, size_t nvals,
+                            const size_t global_size[3], const size_t local_size[3]) {
+    MRK_NONNULL(p);
+    if (nbufs) MRK_NONNULL(buffers);
+    if (nvals) MRK_NONNULL(vals);
+    return p->p->execute(buffers, nbufs, vals, nvals, global_size, local_size);
+}
+const char* mrk_hip_program_name(const mrk_program* p) { return p ? p->p->name() : ""; }
+void mrk_hip_program_destroy(mrk_program* p) { delete p; }
+
+int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_program** out) {
+    MRK_NONNULL(kind);
+    MRK_NONNULL(out);
+    if (nparams) MRK_NONNULL(params);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    std::unique_ptr<Program> p;
+    MRK_TRY(create_builtin_program(device_id, d->allocator->stream(), kind, params, nparams, &p));
+    auto* h = new mrk_program();
+    h->p = std::move(p);
+    *out = h;
+    return kOk;
+}
+
+int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t rows, int64_t cols, int variant) {
+    if (rows < 0 || cols < 0) return fail(kInvalidArgument, "softmax_f32: negative shape");
+    if (rows == 0 || cols == 0) return kOk;
+    MRK_NONNULL(x);
+    MRK_NONNULL(y);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_softmax_f32(d->allocator->stream(), x, y, rows, cols, variant), "softmax_f32 launch");
+    return kOk;
+}
+int mrk_hip_softmax_f32(int device_id, const void* x, void* y, int64_t rows, int64_t cols) {
+    return mrk_hip_softmax_f32_variant(device_id, x, y, rows, cols, 0);
+}
+
+int mrk_hip_event_create(int device_id, mrk_event** out) {
+    MRK_NONNULL(out);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    ffi::Event e = nullptr;
+    MRK_HIP(ffi::event_create(&e), "hipEventCreate");
+    *out = new mrk_event{device_id, e, d->allocator->stream()};
+    return kOk;
+}
+int mrk_hip_event_record(mrk_event* e) {
+    MRK_NONNULL(e);
+    MRK_HIP(ffi::set_device(e->device_id), "hipSetDevice");
+    MRK_HIP(ffi::event_record(e->e, e->stream), "hipEventRecord");
+    return kOk;
+}
+int mrk_hip_event_synchronize(mrk_event* e) {
+    MRK_NONNULL(e);
+    MRK_HIP(ffi::event_synchronize(e->e), "hipEventSynchronize");
+    return kOk;
+}
+int mrk_hip_event_elapsed_ms(mrk_event* start, mrk_event* stop, float* ms) {
+    MRK_NONNULL(start);
+    MRK_NONNULL(stop);
+    MRK_NONNULL(ms);
+    MRK_HIP(ffi::event_elapsed_ms(ms, start->e, stop->e), "hipEventElapsedTime");
+    return kOk;
+}
+void mrk_hip_event_destroy(mrk_event* e) {
+    if (!e) return;
+    ffi::event_destroy(e->e);
+    delete e;
+}
+
+}  // extern "C"

@@ -1,0 +1,34 @@
+#include "error.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "hip_ffi.h"
+
+namespace mrk {
+
+static thread_local std::string g_last_error;
+
+int fail(Status code, const std::string& msg) {
+    g_last_error = msg;
+    return static_cast<int>(code);
+}
+
+int failf(Status code, const char* fmt, ...) {
+    char buf[2048];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return static_cast<int>(code);
+}
+
+int fail_hip(int hip_code, const char* what) {
+    return failf(kHipError, "HIP error: %s failed: %s (%d)", what, ffi::error_name(hip_code), hip_code);
+}
+
+const char* last_error() { return g_last_error.c_str(); }
+void clear_error() { g_last_error.clear(); }
+
+}  // namespace mrk
