@@ -192,6 +192,16 @@ int mrk_hip_softmax_f32(int device_id, const void* x, void* y, int64_t rows, int
 int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t rows, int64_t cols, int variant);
 
 /* =====================================================================================
+ * Synthetic inputs for benchmarks (no counterpart in the reference, whose tensor API has no
+ * RNG, tensor/src/nn/mod.rs:304): counter-based SplitMix64 values written on the device.
+ * dtype 0 = f32, 1 = bf16; mode 0 = uniform [a, b), mode 1 = normal(0, sigma = a).
+ * ===================================================================================== */
+int mrk_hip_fill(int device_id, void* out, size_t n, int dtype, int mode, uint64_t seed, uint64_t tensor_id, float a,
+                 float b);
+/* int32 values uniform over [0, high). */
+int mrk_hip_fill_randint(int device_id, void* out, size_t n, uint64_t seed, uint64_t tensor_id, int high);
+
+/* =====================================================================================
  * Events (hipEvent timing; stands where benchmark_kernel / execute_profiled use Instant,
  * runtime/src/benchmark.rs:64-91, runtime/src/execution_plan.rs:200-221)
  * ===================================================================================== */

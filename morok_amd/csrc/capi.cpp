@@ -345,6 +345,28 @@ int mrk_hip_softmax_f32(int device_id, const void* x, void* y, int64_t rows, int
     return mrk_hip_softmax_f32_variant(device_id, x, y, rows, cols, 0);
 }
 
+int mrk_hip_fill(int device_id, void* out, size_t n, int dtype, int mode, uint64_t seed, uint64_t tensor_id, float a,
+                 float b) {
+    if (n == 0) return kOk;
+    MRK_NONNULL(out);
+    if (dtype < 0 || dtype > 1 || mode < 0 || mode > 1) return fail(kInvalidArgument, "fill: bad dtype or mode");
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_fill(d->allocator->stream(), out, n, dtype, mode, seed, tensor_id, a, b), "fill launch");
+    return kOk;
+}
+int mrk_hip_fill_randint(int device_id, void* out, size_t n, uint64_t seed, uint64_t tensor_id, int high) {
+    if (n == 0) return kOk;
+    MRK_NONNULL(out);
+    if (high <= 0) return fail(kInvalidArgument, "fill_randint: high must be positive");
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_fill_randint(d->allocator->stream(), out, n, seed, tensor_id, high), "fill_randint launch");
+    return kOk;
+}
+
 int mrk_hip_event_create(int device_id, mrk_event** out) {
     MRK_NONNULL(out);
     std::shared_ptr<Device> d;

@@ -25,6 +25,9 @@ int failf(Status code, const char* fmt, ...) {
 }
 
 int fail_hip(int hip_code, const char* what) {
+    // The runtime keeps the last error per thread; drop it so that a later, unrelated
+    // hipGetLastError() check does not report this failure again.
+    ffi::clear_last_error();
     return failf(kHipError, "HIP error: %s failed: %s (%d)", what, ffi::error_name(hip_code), hip_code);
 }
 

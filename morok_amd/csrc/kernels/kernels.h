@@ -9,4 +9,11 @@ namespace mrk {
 // y = softmax(x, axis=-1), x and y f32 [rows, cols] row-major.  variant 0 = default.
 int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long cols, int variant);
 
+
+// Synthetic benchmark inputs. dtype 0 = f32, 1 = bf16; mode 0 = uniform [a, b), 1 = normal(0, a).
+int launch_fill(void* stream, void* out, size_t n, int dtype, int mode, unsigned long long seed,
+                unsigned long long tensor_id, float a, float b);
+int launch_fill_randint(void* stream, void* out, size_t n, unsigned long long seed, unsigned long long tensor_id,
+                        int high);
+
 }  // namespace mrk

@@ -122,6 +122,7 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
     if (rows <= 0 || cols <= 0) return 0;
     if (rows > 0x7fffffffL) return -1;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    (void)hipGetLastError();  // launch status below must be this launch's own
     const float* xi = static_cast<const float*>(x);
     float* yo = static_cast<float*>(y);
     const bool aligned = (cols % 4 == 0) && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) % 16 == 0);

@@ -12,3 +12,16 @@ def _p(b):
 def softmax_f32(x, y, rows, cols, device_id=0, variant=0):
     """Fused row softmax (Tensor::softmax, tensor/src/activation.rs:90-101), last axis."""
     check(lib.mrk_hip_softmax_f32_variant(device_id, _p(x), _p(y), rows, cols, variant))
+
+
+def fill_normal(buf, n, sigma=1.0, seed=0, tensor_id=0, bf16=False, device_id=0):
+    """Device-side synthetic normal(0, sigma) values (benchmark inputs)."""
+    check(lib.mrk_hip_fill(device_id, _p(buf), n, int(bf16), 1, seed, tensor_id, sigma, 0.0))
+
+
+def fill_uniform(buf, n, lo=-1.0, hi=1.0, seed=0, tensor_id=0, bf16=False, device_id=0):
+    check(lib.mrk_hip_fill(device_id, _p(buf), n, int(bf16), 0, seed, tensor_id, lo, hi))
+
+
+def fill_randint(buf, n, high, seed=0, tensor_id=0, device_id=0):
+    check(lib.mrk_hip_fill_randint(device_id, _p(buf), n, seed, tensor_id, high))
