@@ -177,6 +177,7 @@ void mrk_hip_program_destroy(mrk_program* p);
 /* Hand-written gfx950 kernels exposed as Programs, so that an ExecutionPlan can hold them
  * next to generated kernels.  `kind` and the meaning of `params`:
  *   "softmax_f32"     params = {rows, cols}                         buffers = {y, x}
+ *   "gemm_bf16"       params = {M, N, K}                            buffers = {c, a, b}
  * Buffer order follows the reference's PARAM numbering: outputs first. */
 int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_program** out);
 
@@ -190,6 +191,16 @@ int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* para
 int mrk_hip_softmax_f32(int device_id, const void* x, void* y, int64_t rows, int64_t cols);
 /* Same with an explicit implementation variant (0 default, 1 one-wave-per-row); tuning only. */
 int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t rows, int64_t cols, int variant);
+
+/* C[M,N] = A[M,K] @ B[K,N], row-major bf16, f32 accumulation on MFMA, bf16 result: the
+ * lazy graph of Tensor::matmul on bf16 operands (tensor/src/matmul.rs:82-110; accumulator
+ * promotion tensor/src/reduce.rs:101-117) as the tensor-core rewrite leaves it
+ * (schedule/src/optimizer/tc.rs:36-94).  Any shape; shapes with M,N % 256 == 0 and
+ * K % 64 == 0 take the LDS-tiled kernel. */
+int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k);
+/* Same with an explicit kernel variant (0 choose by shape, 2 any-shape kernel); tuning/tests. */
+int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
+                               int variant);
 
 /* =====================================================================================
  * Synthetic inputs for benchmarks (no counterpart in the reference, whose tensor API has no

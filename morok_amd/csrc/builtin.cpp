@@ -66,6 +66,16 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
+    if (k == "gemm_bf16") {
+        MRK_TRY(need(3));
+        if (p[0] < 0 || p[1] < 0 || p[2] < 0) return fail(kInvalidArgument, "gemm_bf16: negative shape");
+        std::string name = "gemm_bf16_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+        out->reset(new BuiltinProgram(device_id, stream, name, 3, p,
+                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16(s, b[1], b[2], b[0], q[0], q[1], q[2], 0);
+                                      }));
+        return kOk;
+    }
     return fail(kInvalidArgument, "unknown builtin kernel kind: " + k);
 }
 

@@ -345,6 +345,25 @@ int mrk_hip_softmax_f32(int device_id, const void* x, void* y, int64_t rows, int
     return mrk_hip_softmax_f32_variant(device_id, x, y, rows, cols, 0);
 }
 
+int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
+                               int variant) {
+    if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16: negative shape");
+    if (m == 0 || n == 0) return kOk;
+    MRK_NONNULL(c);
+    if (k > 0) {
+        MRK_NONNULL(a);
+        MRK_NONNULL(b);
+    }
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_gemm_bf16(d->allocator->stream(), a, b, c, m, n, k, variant), "gemm_bf16 launch");
+    return kOk;
+}
+int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k) {
+    return mrk_hip_gemm_bf16_variant(device_id, a, b, c, m, n, k, 0);
+}
+
 int mrk_hip_fill(int device_id, void* out, size_t n, int dtype, int mode, uint64_t seed, uint64_t tensor_id, float a,
                  float b) {
     if (n == 0) return kOk;

@@ -10,6 +10,10 @@ namespace mrk {
 int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long cols, int variant);
 
 
+// C[M,N] = A[M,K] * B[K,N]; bf16 row-major operands, f32 accumulate, bf16 result.
+// variant 0 = choose by shape, 2 = force the any-shape kernel.
+int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant);
+
 // Synthetic benchmark inputs. dtype 0 = f32, 1 = bf16; mode 0 = uniform [a, b), 1 = normal(0, a).
 int launch_fill(void* stream, void* out, size_t n, int dtype, int mode, unsigned long long seed,
                 unsigned long long tensor_id, float a, float b);

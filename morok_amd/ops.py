@@ -14,6 +14,12 @@ def softmax_f32(x, y, rows, cols, device_id=0, variant=0):
     check(lib.mrk_hip_softmax_f32_variant(device_id, _p(x), _p(y), rows, cols, variant))
 
 
+def gemm_bf16(a, b, c, m, n, k, device_id=0, variant=0):
+    """c[m,n] = a[m,k] @ b[k,n], bf16 row-major, f32 accumulate (Tensor::matmul on bf16,
+    tensor/src/matmul.rs:82-110)."""
+    check(lib.mrk_hip_gemm_bf16_variant(device_id, _p(a), _p(b), _p(c), m, n, k, variant))
+
+
 def fill_normal(buf, n, sigma=1.0, seed=0, tensor_id=0, bf16=False, device_id=0):
     """Device-side synthetic normal(0, sigma) values (benchmark inputs)."""
     check(lib.mrk_hip_fill(device_id, _p(buf), n, int(bf16), 1, seed, tensor_id, sigma, 0.0))

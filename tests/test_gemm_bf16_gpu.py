@@ -1,0 +1,93 @@
+"""Parity of the MFMA bf16 GEMM with the CPU oracle (exact products, f32 accumulate, one
+rounding to bf16) on identical seeded inputs.  Tolerance from the north star: <= 2e-2 max
+relative error, measured as max|gpu - ref| / max|ref|; a tighter elementwise bound
+(2 bf16 ulps of the result plus summation-order noise) is asserted as well."""
+import numpy as np
+import pytest
+
+import morok_amd
+from morok_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _gemm(dev, a, b, variant=0, via_program=False):
+    M, K = a.shape
+    N = b.shape[1]
+    ba = morok_amd.Buffer.from_numpy(a, dev.device_id)
+    bb = morok_amd.Buffer.from_numpy(b, dev.device_id)
+    bc = dev.buffer(max(M * N * 2, 1))
+    if via_program:
+        morok_amd.Program.builtin("gemm_bf16", [M, N, K], dev.device_id).execute([bc, ba, bb])
+    else:
+        ops.gemm_bf16(ba, bb, bc, M, N, K, dev.device_id, variant)
+    return bc.copyout(np.uint16, nbytes=M * N * 2).reshape(M, N)
+
+
+def _check(c, ref, K):
+    cf, rf = synth.from_bf16(c), synth.from_bf16(ref)
+    assert np.all(np.isfinite(cf))
+    scale = np.abs(rf).max()
+    assert np.abs(cf - rf).max() <= 2e-2 * scale
+    # f32 accumulation order differs between MFMA and the sequential oracle: error of the
+    # f32 sum ~ K * 2^-24 * sqrt(K), then one bf16 rounding each (they may round apart by 1 ulp)
+    assert np.all(np.abs(cf - rf) <= np.abs(rf) * 2**-7 + 1e-5 * np.sqrt(K) * max(scale / np.sqrt(K), 1.0))
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 64), (256, 512, 128), (512, 256, 1024), (768, 1024, 192)])
+def test_gemm_tiled_kernel_parity(dev, oracle, shape):
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 3, 0)
+    b = synth.normal_bf16((K, N), 3, 1)
+    _check(_gemm(dev, a, b), oracle.gemm_bf16(a, b), K)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (32, 32, 16), (33, 65, 17), (100, 200, 300), (5, 7, 1000),
+                                   (255, 257, 63), (64, 64, 0)])
+def test_gemm_generic_kernel_parity(dev, oracle, shape):
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 3, 2)
+    b = synth.normal_bf16((K, N), 3, 3)
+    _check(_gemm(dev, a, b), oracle.gemm_bf16(a, b), max(K, 1))
+
+
+def test_gemm_both_kernels_agree_and_program_path(dev, oracle):
+    a = synth.normal_bf16((256, 128), 3, 4)
+    b = synth.normal_bf16((128, 256), 3, 5)
+    ref = oracle.gemm_bf16(a, b)
+    _check(_gemm(dev, a, b, variant=2), ref, 128)
+    _check(_gemm(dev, a, b, via_program=True), ref, 128)
+
+
+def test_gemm_special_cases_exact(dev):
+    # identity / permutation / ones: exact in bf16, so bit-for-bit
+    n = 256
+    a = synth.normal_bf16((n, n), 3, 6)
+    eye = synth.to_bf16(np.eye(n, dtype=np.float32))
+    assert np.array_equal(_gemm(dev, a, eye), a)
+    assert np.array_equal(_gemm(dev, eye, a), a)
+    perm = synth.to_bf16(np.eye(n, dtype=np.float32)[:, ::-1].copy())
+    assert np.array_equal(_gemm(dev, a, perm), a[:, ::-1])
+    ones = synth.to_bf16(np.ones((n, 512), np.float32))
+    c = synth.from_bf16(_gemm(dev, ones, synth.to_bf16(np.ones((512, n), np.float32))))
+    assert np.all(c == 512)
+    # asymmetric operands catch a transposed A or B
+    a2 = synth.to_bf16(np.arange(256 * 64, dtype=np.float32).reshape(256, 64) % 7 - 3)
+    b2 = synth.to_bf16(np.arange(64 * 256, dtype=np.float32).reshape(64, 256) % 5 - 2)
+    ref = synth.from_bf16(a2).astype(np.float64) @ synth.from_bf16(b2).astype(np.float64)
+    assert np.array_equal(synth.from_bf16(_gemm(dev, a2, b2)), synth.from_bf16(synth.to_bf16(ref.astype(np.float32))))
+
+
+def test_gemm_full_size_config_slice_and_linearity(dev, oracle):
+    # configs[2] shape 4096^3: rows of the full product against the oracle, plus linearity
+    M = N = K = 4096
+    a = synth.normal_bf16((M, K), 3, 0)
+    b = synth.normal_bf16((K, N), 3, 1)
+    c = _gemm(dev, a, b)
+    rows = np.array([0, 1, 255, 256, 1000, 2047, 2048, 4095])
+    ref = oracle.gemm_bf16(np.ascontiguousarray(a[rows]), b)
+    _check(c[rows], ref, K)
+    # size-independent property: (2A) B == 2 (A B) exactly (scaling by 2 is exact in bf16 and f32)
+    a2 = synth.to_bf16(synth.from_bf16(a) * 2)
+    c2 = _gemm(dev, a2, b)
+    assert np.array_equal(synth.from_bf16(c2), synth.from_bf16(c) * 2)
