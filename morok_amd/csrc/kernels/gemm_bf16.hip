@@ -20,6 +20,8 @@
 // writes and 16-byte coalesced global stores.
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "kernels.h"
 
 namespace mrk::dev {
@@ -117,46 +119,109 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
     // lane-constant parts of the fragment addresses
-    const int a_row_l = wm * 128 + (lane & 31);  // + i*32
-    const int a_kch_l = lane >> 5;               // + ks*2
-    const int b_krow_l = 8 * (lane >> 5) + ((lane & 15) >> 2);                    // + ks*16 + 4*r
-    const int b_ncol_l = wn * 128 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);      // + j*32
+    const int a_base_l = (wm * 128 + (lane & 31)) * 128;                                  // + i*4096
+    const int b_base_l = (8 * (lane >> 5) + ((lane & 15) >> 2)) * kBPitch +
+                         (wn * 128 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;        // + ks*16*pitch + j*64
+    int a_xo[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) a_xo[ks] = ((ks * 2 + (lane >> 5)) ^ (lane & 7)) << 4;
 
+    bf16x8 fa[2][4], fb[2][4];
+    auto load_frags = [&](int buf, int ks, int slot) {
+        const char* sA = sA0 + buf * kAStage + a_base_l + a_xo[ks];
+        const char* sB = sB0 + buf * kBStage + b_base_l + ks * 16 * kBPitch;
+#pragma unroll
+        for (int i = 0; i < 4; i++) fa[slot][i] = *LDS_PTR(bf16x8, sA + i * 4096);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + j * 64));
+            bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + j * 64 + 4 * kBPitch));
+            fb[slot][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+    };
+    auto mma = [&](int slot) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
+    };
+    // LDS writes of this wave are complete and every wave has arrived: the only
+    // synchronisation the K loop needs (global loads stay in flight across it).
+    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    // Software pipeline.  While tile kt is consumed from LDS stage `cur`, tile kt+1 sits
+    // in registers (loaded one iteration earlier) and is written to the other stage
+    // during k-step 0; tile kt+2 is requested from global memory during k-step 1.
+    // Fragments are double-buffered in registers: the LDS reads for k-step ks+1 are
+    // issued among the MFMAs of k-step ks.  The sched_group_barrier sequences spell out
+    // that interleaving (one memory instruction between consecutive MFMAs) so that LDS
+    // and global traffic proceed while the matrix pipe is busy.
     const int KT = K / kBK;
     gload(0);
     swrite(0);
-    __syncthreads();
-    int cur = 0;
-    for (int kt = 0; kt < KT; kt++) {
-        if (kt + 1 < KT) gload(kt + 1);
-        const char* sA = sA0 + cur * kAStage;
-        const char* sB = sB0 + cur * kBStage;
+    gload(KT > 1 ? 1 : 0);
+    lds_barrier();
+    load_frags(0, 0, 0);
+
+    // No branches inside an iteration, so that every k-step stays one basic block the
+    // scheduler can interleave: near the end of K the prefetches simply re-request the
+    // last tile (a cache hit) and fill an LDS stage nobody reads.
+    auto iteration = [&](auto cur_c, int kt) {
+        constexpr int cur = decltype(cur_c)::value;
+        // k-step 0: MFMAs on slot 0 | LDS reads of k-step 1 | LDS writes of tile kt+1
+        swrite(cur ^ 1);
+        load_frags(cur, 1, 1);
+        mma(0);
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            bf16x8 af[4], bfr[4];
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int row = a_row_l + i * 32;
-                const int kch = ks * 2 + a_kch_l;
-                af[i] = *LDS_PTR(bf16x8, sA + row * 128 + ((kch ^ (row & 7)) << 4));
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int off = (ks * 16 + b_krow_l) * kBPitch + (b_ncol_l + j * 32) * 2;
-                bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off));
-                bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off + 4 * kBPitch));
-                bfr[j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+        for (int n = 0; n < 16; n++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // DS write
         }
-        if (kt + 1 < KT) swrite(cur ^ 1);
-        __syncthreads();
-        cur ^= 1;
+        __builtin_amdgcn_sched_barrier(0);
+        // k-step 1: MFMAs on slot 1 | LDS reads of k-step 2 | global loads of tile kt+2
+        gload(kt + 2 < KT ? kt + 2 : KT - 1);
+        load_frags(cur, 2, 0);
+        mma(1);
+#pragma unroll
+        for (int n = 0; n < 16; n++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);  // VALU (address)
+            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM read
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // k-step 2: MFMAs on slot 0 | LDS reads of k-step 3
+        load_frags(cur, 3, 1);
+        mma(0);
+#pragma unroll
+        for (int n = 0; n < 16; n++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // every wave has finished reading stage `cur` and writing the other stage
+        lds_barrier();
+        // k-step 3: MFMAs on slot 1 | LDS reads of k-step 0 of the next tile
+        load_frags(cur ^ 1, 0, 0);
+        mma(1);
+#pragma unroll
+        for (int n = 0; n < 16; n++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using I0 = std::integral_constant<int, 0>;
+    using I1 = std::integral_constant<int, 1>;
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+        iteration(I0{}, kt);
+        iteration(I1{}, kt + 1);
     }
+    if (kt < KT) iteration(I0{}, kt);
+    lds_barrier();
 
     // Epilogue.  With swapped operands lane l of tile (i, j) holds, in registers 4g..4g+3,
     // C[m = i*32 + l%32][n = j*32 + 8g + 4*(l/32) + 0..3].
