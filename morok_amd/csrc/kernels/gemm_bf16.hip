@@ -11,15 +11,19 @@
 // byte.
 //
 // Main kernel: 256x256 output tile per workgroup of 4 waves (2x2), each wave 128x128 =
-// 4x4 MFMA tiles (256 accumulator registers), K step 64.  Global -> registers -> LDS
-// with two LDS stages, one barrier per K step.  A is kept in LDS row-major with an XOR
-// swizzle of its 16-byte chunks, B row-major (n contiguous) with a 32-byte row skew and
-// read through the transposing LDS load, which hands each lane the 4 consecutive-k
-// values of its column.  The MFMA is issued with swapped operands (D' = B^T A^T) so each
+// 4x4 MFMA tiles (256 accumulator registers), K step 64.  Tiles travel global -> LDS
+// directly (global_load_lds, 16 B per lane, no register staging) into two LDS stages,
+// one barrier per K step; the copy of tile kt+2 is issued among the MFMAs of the last
+// k-step of tile kt, a full tile of work ahead of its first use.  A is kept in LDS
+// row-major with an XOR swizzle of its 16-byte chunks, B row-major (n contiguous) with
+// an XOR swizzle of its 32-byte granules and read through the transposing LDS load,
+// which hands each lane the 4 consecutive-k values of its column.  Fragments are
+// double-buffered in registers so LDS reads of k-step ks+1 run under the MFMAs of ks.  The MFMA is issued with swapped operands (D' = B^T A^T) so each
 // lane ends up with 4 consecutive n of one row, which makes the epilogue 8-byte LDS
 // writes and 16-byte coalesced global stores.
 #include <hip/hip_runtime.h>
 
+#include <cstdint>
 #include <type_traits>
 
 #include "kernels.h"
@@ -37,11 +41,10 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kBM = 256, kBN = 256, kBK = 64;
 constexpr int kAStage = kBM * kBK * 2;         // 32768 B, row pitch 128 B, chunk-swizzled
-constexpr int kBPitch = kBN * 2 + 32;          // 544 B: rows skewed by 32 B across banks
-constexpr int kBStage = kBK * kBPitch;         // 34816 B
+constexpr int kBStageSw = kBK * kBN * 2;       // 32768 B, row pitch 512 B, granule-swizzled
 constexpr int kCPitch = 128 * 2 + 16;          // epilogue staging pitch per wave
 constexpr int kCWave = 128 * kCPitch;          // 34816 B
-constexpr int kSmemMain = 2 * kAStage + 2 * kBStage;  // 135168
+constexpr int kSmemMain = 2 * kAStage + 2 * kBStageSw;  // 131072
 constexpr int kSmemEpi = 4 * kCWave;                  // 139264
 constexpr int kSmem = kSmemEpi > kSmemMain ? kSmemEpi : kSmemMain;
 
@@ -67,47 +70,53 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                          __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
                                                          int tiles_n) {
-    __shared__ __attribute__((aligned(16))) char smem[kSmem];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    // two stages; A stage: 256 rows x 128 B, 16 B chunks XOR-swizzled by (row & 7);
+    // B stage: 64 k-rows x 512 B, 32 B granules XOR-swizzled by (k & 3).
+    __shared__ __attribute__((aligned(1024))) char smem[kSmem];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
     const size_t m0 = (size_t)tile_m * kBM, n0 = (size_t)tile_n * kBN;
-    const __bf16* Ag = A + m0 * K;
-    const __bf16* Bg = B + n0;
     char* sA0 = smem;
     char* sB0 = smem + 2 * kAStage;
 
-    u32x4 ra[8], rb[8];
-    // per-thread chunk coordinates (fixed over the K loop)
-    // A: 2048 chunks of 16 B per stage, chunk c = i*256 + tid -> row c>>3, k-chunk c&7
-    // B: 2048 chunks, c -> k row c>>5, n-chunk c&31
-    auto gload = [&](int kt) {
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int c = i * 256 + tid;
-            ra[i] = *reinterpret_cast<const u32x4*>(Ag + (size_t)(c >> 3) * K + (size_t)kt * kBK + (c & 7) * 8);
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int c = i * 256 + tid;
-            rb[i] = *reinterpret_cast<const u32x4*>(Bg + ((size_t)kt * kBK + (c >> 5)) * N + (c & 31) * 8);
+    // ---- direct global -> LDS copies: each wave moves 8 KB of A and 8 KB of B per tile,
+    // one instruction = 64 lanes x 16 B = 1 KB of contiguous LDS.
+    // A chunk q (1 KB = 8 rows): lane -> row q*8 + lane/8, LDS chunk lane%8 holds logical
+    // chunk (lane%8) ^ (row & 7).
+    const unsigned a_voff = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (lane >> 3)) << 3)) * 2);
+    // B chunk q (1 KB = 2 k-rows): lane -> k-row q*2 + lane/32, LDS 16 B chunk lane%32 ->
+    // granule (lane%32)/2 ^ (krow & 3).
+    const int b_h = lane & 1, b_g = (lane & 31) >> 1, b_r = lane >> 5;
+    const unsigned b_voff0 = (unsigned)(((size_t)(wave * 16 + b_r) * N + ((((b_g ^ (0 + b_r)) << 1) | b_h) << 3)) * 2);
+    const unsigned b_voff1 = (unsigned)(((size_t)(wave * 16 + b_r) * N + ((((b_g ^ (2 + b_r)) << 1) | b_h) << 3)) * 2);
+    const char* a_tile = reinterpret_cast<const char*>(A + m0 * K);
+    const char* b_tile = reinterpret_cast<const char*>(B + n0);
+    const unsigned lds_a = (unsigned)(uintptr_t)LDS_PTR(char, sA0) + wave * 8192;
+    const unsigned lds_b = (unsigned)(uintptr_t)LDS_PTR(char, sB0) + wave * 8192;
+    // One direct copy: 64 lanes x 16 B land at LDS [m0, m0 + 1 KB); the compiler is not told
+    // about it (it would otherwise wait for the copy before every later LDS read), so the
+    // waits are explicit: tile_barrier() drains vmcnt before the tile is consumed.
+    auto dma = [&](unsigned lds_addr, unsigned voff, const char* sbase) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(sbase)
+                     : "m0");
+    };
+    // n = 0..7: A chunks, n = 8..15: B chunks of tile kt into `stage`
+    auto dma_one = [&](int n, int kt, int stage) {
+        if (n < 8) {
+            dma(lds_a + stage * kAStage + n * 1024, a_voff, a_tile + ((size_t)kt * kBK + (size_t)n * 8 * K) * 2);
+        } else {
+            const int q = n - 8;
+            dma(lds_b + stage * kBStageSw + q * 1024, (q & 1) ? b_voff1 : b_voff0,
+                b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
         }
     };
-    auto swrite = [&](int buf) {
-        char* sA = sA0 + buf * kAStage;
-        char* sB = sB0 + buf * kBStage;
+    auto dma_tile = [&](int kt, int stage) {
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int c = i * 256 + tid;
-            const int row = c >> 3, kc = c & 7;
-            *LDS_PTR(u32x4, sA + row * 128 + ((kc ^ (row & 7)) << 4)) = ra[i];
-        }
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const int c = i * 256 + tid;
-            *LDS_PTR(u32x4, sB + (c >> 5) * kBPitch + ((c & 31) << 4)) = rb[i];
-        }
+        for (int n = 0; n < 16; n++) dma_one(n, kt, stage);
     };
 
     f32x16 acc[4][4];
@@ -119,23 +128,27 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
     // lane-constant parts of the fragment addresses
-    const int a_base_l = (wm * 128 + (lane & 31)) * 128;                                  // + i*4096
-    const int b_base_l = (8 * (lane >> 5) + ((lane & 15) >> 2)) * kBPitch +
-                         (wn * 128 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;        // + ks*16*pitch + j*64
+    const int a_base_l = (wm * 128 + (lane & 31)) * 128;  // + i*4096
     int a_xo[4];
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) a_xo[ks] = ((ks * 2 + (lane >> 5)) ^ (lane & 7)) << 4;
+    const int b_rr = (lane & 15) >> 2;
+    const int b_g0 = wn * 8 + ((lane >> 4) & 1);
+    const int b_row_l = (8 * (lane >> 5) + b_rr) * 512 + 8 * (lane & 3);  // + ks*16*512 + r*4*512
+    const int b_p0 = b_row_l + ((b_g0 ^ b_rr) << 5);                      // j = 0 (+128: j = 2)
+    const int b_p1 = b_row_l + (((b_g0 ^ b_rr) ^ 2) << 5);                // j = 1 (+128: j = 3)
 
     bf16x8 fa[2][4], fb[2][4];
     auto load_frags = [&](int buf, int ks, int slot) {
         const char* sA = sA0 + buf * kAStage + a_base_l + a_xo[ks];
-        const char* sB = sB0 + buf * kBStage + b_base_l + ks * 16 * kBPitch;
+        const char* sB = sB0 + buf * kBStageSw + ks * 16 * 512;
 #pragma unroll
         for (int i = 0; i < 4; i++) fa[slot][i] = *LDS_PTR(bf16x8, sA + i * 4096);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + j * 64));
-            bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + j * 64 + 4 * kBPitch));
+            const int off = ((j & 1) ? b_p1 : b_p0) + (j >> 1) * 128;
+            bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off));
+            bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off + 4 * 512));
             fb[slot][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
     };
@@ -146,53 +159,33 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
             for (int j = 0; j < 4; j++)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
     };
-    // LDS writes of this wave are complete and every wave has arrived: the only
-    // synchronisation the K loop needs (global loads stay in flight across it).
-    auto lds_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    // this wave's LDS reads and its direct-to-LDS copies are complete, then all waves meet
+    auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-    // Software pipeline.  While tile kt is consumed from LDS stage `cur`, tile kt+1 sits
-    // in registers (loaded one iteration earlier) and is written to the other stage
-    // during k-step 0; tile kt+2 is requested from global memory during k-step 1.
-    // Fragments are double-buffered in registers: the LDS reads for k-step ks+1 are
-    // issued among the MFMAs of k-step ks.  The sched_group_barrier sequences spell out
-    // that interleaving (one memory instruction between consecutive MFMAs) so that LDS
-    // and global traffic proceed while the matrix pipe is busy.
     const int KT = K / kBK;
-    gload(0);
-    swrite(0);
-    gload(KT > 1 ? 1 : 0);
-    lds_barrier();
+    dma_tile(0, 0);
+    dma_tile(KT > 1 ? 1 : 0, 1);
+    tile_barrier();
     load_frags(0, 0, 0);
 
-    // No branches inside an iteration, so that every k-step stays one basic block the
-    // scheduler can interleave: near the end of K the prefetches simply re-request the
-    // last tile (a cache hit) and fill an LDS stage nobody reads.
     auto iteration = [&](auto cur_c, int kt) {
         constexpr int cur = decltype(cur_c)::value;
-        // k-step 0: MFMAs on slot 0 | LDS reads of k-step 1 | LDS writes of tile kt+1
-        swrite(cur ^ 1);
         load_frags(cur, 1, 1);
         mma(0);
 #pragma unroll
         for (int n = 0; n < 16; n++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
-            __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);  // DS write
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // k-step 1: MFMAs on slot 1 | LDS reads of k-step 2 | global loads of tile kt+2
-        gload(kt + 2 < KT ? kt + 2 : KT - 1);
         load_frags(cur, 2, 0);
         mma(1);
 #pragma unroll
         for (int n = 0; n < 16; n++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);  // VALU (address)
-            __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // VMEM read
         }
         __builtin_amdgcn_sched_barrier(0);
-        // k-step 2: MFMAs on slot 0 | LDS reads of k-step 3
         load_frags(cur, 3, 1);
         mma(0);
 #pragma unroll
@@ -201,15 +194,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
             if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // every wave has finished reading stage `cur` and writing the other stage
-        lds_barrier();
-        // k-step 3: MFMAs on slot 1 | LDS reads of k-step 0 of the next tile
-        load_frags(cur ^ 1, 0, 0);
-        mma(1);
+        // tile kt+1 has landed in the other stage; nobody reads stage `cur` any more
+        tile_barrier();
+        {
+            const int ktn = kt + 2 < KT ? kt + 2 : KT - 1;
+            const char* sAn = sA0 + (cur ^ 1) * kAStage + a_base_l + a_xo[0];
+            const char* sBn = sB0 + (cur ^ 1) * kBStageSw;
+            bf16x4 lo[4], hi[4];
 #pragma unroll
-        for (int n = 0; n < 16; n++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            for (int n = 0; n < 16; n++) {
+                acc[n >> 2][n & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][n & 3], fa[1][n >> 2], acc[n >> 2][n & 3], 0, 0, 0);
+                if (n < 4) fa[0][n] = *LDS_PTR(bf16x8, sAn + n * 4096);
+                else if (n < 12) {
+                    const int j = (n - 4) >> 1;
+                    const int off = ((j & 1) ? b_p1 : b_p0) + (j >> 1) * 128;
+                    if ((n & 1) == 0) lo[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off));
+                    else hi[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off + 4 * 512));
+                }
+                dma_one(n, ktn, cur);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) fb[0][j] = __builtin_shufflevector(lo[j], hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
         }
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -221,7 +227,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
         iteration(I1{}, kt + 1);
     }
     if (kt < KT) iteration(I0{}, kt);
-    lds_barrier();
+    tile_barrier();
 
     // Epilogue.  With swapped operands lane l of tile (i, j) holds, in registers 4g..4g+3,
     // C[m = i*32 + l%32][n = j*32 + 8g + 4*(l/32) + 0..3].
@@ -310,3 +316,4 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
 }
 
 }  // namespace mrk
+
