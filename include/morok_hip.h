@@ -178,6 +178,7 @@ void mrk_hip_program_destroy(mrk_program* p);
  * next to generated kernels.  `kind` and the meaning of `params`:
  *   "softmax_f32"     params = {rows, cols}                         buffers = {y, x}
  *   "gemm_bf16"       params = {M, N, K}                            buffers = {c, a, b}
+ *   "flash_fwd_bf16"  params = {B*H, Sq, Sk, D, causal, f32 bits of scale}   buffers = {o, q, k, v}
  * Buffer order follows the reference's PARAM numbering: outputs first. */
 int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_program** out);
 
@@ -201,6 +202,15 @@ int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int6
 /* Same with an explicit kernel variant (0 choose by shape, 2 any-shape kernel); tuning/tests. */
 int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
                                int variant);
+
+/* Scaled dot-product attention forward in one kernel (online softmax, f32 scores and
+ * statistics, P rounded to bf16 before the second product, bf16 output):
+ * Tensor::scaled_dot_product_attention (tensor/src/transformer.rs:78-137) with is_causal as
+ * given and no attn_mask / softcap.  q [B,H,Sq,D], k and v [B,H,Sk,D], o [B,H,Sq,D], row-major
+ * bf16, D = 128, scale > 0 (the reference default is 1/sqrt(D), transformer.rs:90-91).
+ * Causal rule of the reference: key j is visible to query i iff j <= i (transformer.rs:103-109). */
+int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
+                                int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal);
 
 /* =====================================================================================
  * Synthetic inputs for benchmarks (no counterpart in the reference, whose tensor API has no

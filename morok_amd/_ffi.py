@@ -91,6 +91,8 @@ _SIGS = {
     "mrk_hip_gemm_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64]),
     "mrk_hip_gemm_bf16_variant": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
                                             C.c_int64, C.c_int]),
+    "mrk_hip_flash_attn_fwd_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                              C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_int]),
     "mrk_hip_fill": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_float,
                                C.c_float]),
     "mrk_hip_fill_randint": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_uint64, C.c_uint64, C.c_int]),

@@ -76,6 +76,21 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
+    if (k == "flash_fwd_bf16") {
+        MRK_TRY(need(6));
+        if (p[0] < 0 || p[1] < 0 || p[2] <= 0 || p[3] != 128)
+            return fail(kInvalidArgument, "flash_fwd_bf16: bad shape (params BH, Sq, Sk, D=128, causal, scale bits)");
+        std::string name = "flash_fwd_bf16_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+        out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
+                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          uint32_t bits = static_cast<uint32_t>(q[5]);
+                                          float scale;
+                                          std::memcpy(&scale, &bits, 4);
+                                          return launch_flash_fwd_bf16(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3],
+                                                                       scale, q[4] != 0);
+                                      }));
+        return kOk;
+    }
     return fail(kInvalidArgument, "unknown builtin kernel kind: " + k);
 }
 

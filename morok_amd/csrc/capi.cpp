@@ -364,6 +364,25 @@ int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int6
     return mrk_hip_gemm_bf16_variant(device_id, a, b, c, m, n, k, 0);
 }
 
+int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
+                                int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal) {
+    if (batch < 0 || heads < 0 || sq < 0 || sk < 0) return fail(kInvalidArgument, "flash_attn_fwd: negative shape");
+    if (batch == 0 || heads == 0 || sq == 0) return kOk;
+    if (d != 128) return failf(kInvalidArgument, "flash_attn_fwd: head_dim %lld is not supported (128 only)", (long long)d);
+    if (sk == 0) return fail(kInvalidArgument, "flash_attn_fwd: empty key sequence (softmax over no keys is undefined)");
+    if (!(scale > 0.0f)) return fail(kInvalidArgument, "flash_attn_fwd: scale must be positive");
+    MRK_NONNULL(q);
+    MRK_NONNULL(k);
+    MRK_NONNULL(v);
+    MRK_NONNULL(o);
+    std::shared_ptr<Device> dv;
+    MRK_TRY(get_device(device_id, &dv));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_flash_fwd_bf16(dv->allocator->stream(), q, k, v, o, batch * heads, sq, sk, d, scale, causal ? 1 : 0),
+            "flash_attn_fwd launch");
+    return kOk;
+}
+
 int mrk_hip_fill(int device_id, void* out, size_t n, int dtype, int mode, uint64_t seed, uint64_t tensor_id, float a,
                  float b) {
     if (n == 0) return kOk;

@@ -1,0 +1,258 @@
+// Flash-attention forward for gfx950: O = softmax(Q K^T * scale [+ causal mask]) V in one
+// kernel with an online softmax, bf16 operands, f32 scores / statistics / accumulators.
+//
+// Replaces the composed graph of Tensor::scaled_dot_product_attention
+// (tensor/src/transformer.rs:78-137: matmul, scale, tril -> where(-inf), softmax, matmul),
+// which the reference schedules as >= 6 kernels that materialise the [B,H,Sq,Sk] score
+// tensor (tensor/src/test/unit/fusion.rs:90-104).  Causal rule as in the reference:
+// key j is visible to query i iff j <= i (tril(0) over [Sq, Sk], transformer.rs:103-109).
+//
+// Layout: Q [BH, Sq, D], K [BH, Sk, D], V [BH, Sk, D], O [BH, Sq, D], row-major, D = 128.
+//
+// Work split: one workgroup = 128 queries of one (batch, head); 4 waves x 32 queries.
+// K and V tiles of 64 keys travel global -> LDS directly (global_load_lds), two stages.
+// Everything is computed transposed so that softmax statistics stay inside a lane:
+//   S^T[key][q] = K_tile Q^T        MFMA 32x32x16, A = K rows from LDS, B = Q^T in registers
+//   lane l owns query q = l % 32 and 16 of every 32 keys; the other 16 sit in lane l ^ 32
+//   O^T[d][q]  += V^T P^T           A = V^T through the transposing LDS load, B = P^T taken
+//                                   straight from the S^T accumulator registers
+// The k index of the second product is whatever order the accumulator registers hold the
+// keys in; the V^T fragment is fetched in that same order, so no register shuffle is needed.
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "kernels.h"
+
+namespace mrk::dev {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+#define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+constexpr int kD = 128;        // head dim
+constexpr int kQT = 128;       // queries per workgroup
+constexpr int kKT = 64;        // keys per tile
+constexpr int kRow = kD * 2;   // 256 B per K/V row
+constexpr int kTile = kKT * kRow;  // 16 KB
+
+__global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
+                                                         const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
+                                                         int Sq, int Sk, float scale_log2e, int causal, int q_tiles) {
+    // K stage s at s*32 KB, V stage s at s*32 KB + 16 KB
+    __shared__ __attribute__((aligned(1024))) char smem[4 * kTile];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // Heavy (late) query tiles first; workgroups of one head stay on one XCD (ids mod 8).
+    int bh, qt;
+    {
+        const int bid = blockIdx.x;
+        if ((BH & 7) == 0) {
+            const int per = BH >> 3;
+            const int idx = bid >> 3;
+            bh = (bid & 7) + 8 * (idx % per);
+            qt = q_tiles - 1 - idx / per;
+        } else {
+            bh = bid % BH;
+            qt = q_tiles - 1 - bid / BH;
+        }
+    }
+    const int q0 = qt * kQT;
+    const int qw0 = q0 + wave * 32;  // first query of this wave
+    const int lq = lane & 31, lg = lane >> 5;
+    const __bf16* Qh = Q + (size_t)bh * Sq * kD;
+    const char* Kh = reinterpret_cast<const char*>(K + (size_t)bh * Sk * kD);
+    const char* Vh = reinterpret_cast<const char*>(V + (size_t)bh * Sk * kD);
+    __bf16* Oh = O + (size_t)bh * Sq * kD;
+
+    // number of key tiles this workgroup visits
+    int kend = Sk;
+    if (causal && q0 + kQT < kend) kend = q0 + kQT;
+    const int ntiles = (kend + kKT - 1) / kKT;
+
+    // ---- direct global -> LDS tile copies.  One instruction = 1 KB = 4 rows of 256 B.
+    // wave w copies rows 16w .. 16w+15 of both tiles (4 instructions each).
+    const unsigned lds_base = (unsigned)(uintptr_t)LDS_PTR(char, smem);
+    const int c16 = lane & 15, r4 = lane >> 4;
+    auto dma = [&](unsigned lds_addr, unsigned voff, const char* sbase) {
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(lds_addr), "v"(voff), "s"(sbase)
+                     : "m0");
+    };
+    auto dma_tile = [&](int j, int stage) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int row = wave * 16 + c * 4 + r4;  // row inside the tile
+            int key = j * kKT + row;
+            key = key < Sk ? key : Sk - 1;  // ragged tail: re-read the last row, masked later
+            // K: 16 B chunk c16 of the LDS row holds logical chunk c16 ^ (row & 7)
+            const unsigned kvoff = (unsigned)key * kRow + ((c16 ^ (row & 7)) << 4);
+            // V: 32 B granule (c16 >> 1) holds logical granule (c16 >> 1) ^ (row & 3)
+            const unsigned vvoff = (unsigned)key * kRow + (((((c16 >> 1) ^ (row & 3)) << 1) | (c16 & 1)) << 4);
+            const unsigned dst = lds_base + stage * 2 * kTile + (wave * 16 + c * 4) * kRow;
+            dma(dst, kvoff, Kh);
+            dma(dst + kTile, vvoff, Vh);
+        }
+    };
+    auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    // ---- Q^T fragments: lane holds q = qw0 + l%32, d = 16*ds + 8*(l/32) .. +8
+    bf16x8 qf[8];
+    {
+        int qrow = qw0 + lq;
+        qrow = qrow < Sq ? qrow : Sq - 1;
+        const __bf16* qp = Qh + (size_t)qrow * kD + 8 * lg;
+#pragma unroll
+        for (int ds = 0; ds < 8; ds++) qf[ds] = *reinterpret_cast<const bf16x8*>(qp + 16 * ds);
+    }
+
+    f32x16 o[4];
+#pragma unroll
+    for (int db = 0; db < 4; db++)
+#pragma unroll
+        for (int e = 0; e < 16; e++) o[db][e] = 0.0f;
+    float m_run = -INFINITY;  // running max of raw scores (before scale)
+    float l_run = 0.0f;       // this lane's partial row sum
+
+    // lane-constant LDS offsets
+    // K fragment (A operand): row = kb*32 + l%32, logical chunk 2*ds + l/32
+    const int k_row_off = lq * kRow;
+    const int k_sw = lq & 7;
+    // V^T fragment via transposing read: 16-lane block b = l/16 covers d half (b & 1) and
+    // key group g = b >> 1; inside the block lane j' = l%16 points at key row j'/4,
+    // 8-byte unit j'%4 of the 32-byte granule.
+    const int v_rr = (lane & 15) >> 2;
+    const int v_row_off = (4 * lg + v_rr) * kRow + 8 * (lane & 3);
+    const int v_half = (lane >> 4) & 1;
+
+    dma_tile(0, 0);
+    for (int j = 0; j < ntiles; j++) {
+        const int stage = j & 1;
+        tile_barrier();  // tile j landed; every wave is done with tile j-1
+        if (j + 1 < ntiles) dma_tile(j + 1, stage ^ 1);
+        const int key0 = j * kKT;
+        // this wave's queries see nothing of the tile: keys all beyond its last query
+        if (causal && key0 > qw0 + 31) continue;
+        const char* sK = smem + stage * 2 * kTile;
+        const char* sV = sK + kTile;
+
+        // ---- S^T = K Q^T
+        f32x16 st[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) st[kb][e] = 0.0f;
+#pragma unroll
+        for (int ds = 0; ds < 8; ds++) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                const int off = kb * 32 * kRow + k_row_off + (((2 * ds + lg) ^ k_sw) << 4);
+                bf16x8 kf = *LDS_PTR(bf16x8, sK + off);
+                st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ds], st[kb], 0, 0, 0);
+            }
+        }
+        // ---- mask: register e of block kb is key key0 + kb*32 + 8*(e/4) + 4*(l/32) + e%4
+        const bool need_mask = (causal && key0 + kKT - 1 > qw0) || (key0 + kKT > Sk);
+        if (need_mask) {
+            const int qidx = qw0 + lq;
+            const int lim = causal ? (qidx < Sk - 1 ? qidx : Sk - 1) : Sk - 1;  // last visible key
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int e = 0; e < 16; e++) {
+                    const int key = key0 + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3);
+                    if (key > lim) st[kb][e] = -INFINITY;
+                }
+        }
+        // ---- online softmax, all in the lane that owns the query
+        float mx = st[0][0];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) mx = fmaxf(mx, st[kb][e]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        // m_new is finite from the first tile on: key 0 is visible to every query
+        const float mb = m_new * scale_log2e;
+        const float alpha = __builtin_amdgcn_exp2f(m_run * scale_log2e - mb);
+        m_run = m_new;
+        float psum = 0.0f;
+        bf16x8 pb[2][2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                f32x8 p;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kb][8 * t + e], scale_log2e, -mb));
+                    psum += p[e];
+                }
+                pb[kb][t] = __builtin_convertvector(p, bf16x8);
+            }
+        }
+        l_run = l_run * alpha + psum;
+#pragma unroll
+        for (int db = 0; db < 4; db++) o[db] *= alpha;
+
+        // ---- O^T += V^T P^T.  MFMA (kb, t) contracts over the 16 keys held in registers
+        // 8t .. 8t+7 of block kb: keys kb*32 + 16t + {0, 8} + 4*(l/32) + 0..3.
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+#pragma unroll
+                for (int db = 0; db < 4; db++) {
+                    const int off = (kb * 32 + 16 * t) * kRow + v_row_off + (((db * 2 + v_half) ^ v_rr) << 5);
+                    bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sV + off));
+                    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sV + off + 8 * kRow));
+                    bf16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[kb][t], o[db], 0, 0, 0);
+                }
+            }
+        }
+    }
+
+    // ---- normalise and store: lane holds O[q = qw0 + l%32][d = db*32 + 8*(e/4) + 4*(l/32) + e%4]
+    const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const float inv = 1.0f / l_tot;
+    const int qrow = qw0 + lq;
+    if (qrow < Sq) {
+        __bf16* op = Oh + (size_t)qrow * kD + 4 * lg;
+#pragma unroll
+        for (int db = 0; db < 4; db++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                f32x4 v = {o[db][4 * g] * inv, o[db][4 * g + 1] * inv, o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv};
+                *reinterpret_cast<bf16x4*>(op + db * 32 + 8 * g) = __builtin_convertvector(v, bf16x4);
+            }
+    }
+}
+
+}  // namespace mrk::dev
+
+namespace mrk {
+
+int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
+                          long D, float scale, int causal) {
+    using namespace mrk::dev;
+    if (BH <= 0 || Sq <= 0) return 0;
+    if (D != kD || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
+    if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
+    const long q_tiles = (Sq + kQT - 1) / kQT;
+    const long blocks = BH * q_tiles;
+    if (blocks > 0x7fffffffL) return (int)hipErrorInvalidValue;
+    (void)hipGetLastError();
+    const float scale_log2e = scale * 1.4426950408889634f;
+    flash_fwd_d128<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
+        static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mrk

@@ -14,6 +14,11 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 // variant 0 = choose by shape, 2 = force the any-shape kernel.
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant);
 
+// O = softmax(Q K^T * scale [causal]) V; Q [BH,Sq,D], K/V [BH,Sk,D], O [BH,Sq,D] bf16, D = 128,
+// scale > 0.  Causal: key j visible to query i iff j <= i.
+int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
+                          long D, float scale, int causal);
+
 // Synthetic benchmark inputs. dtype 0 = f32, 1 = bf16; mode 0 = uniform [a, b), 1 = normal(0, a).
 int launch_fill(void* stream, void* out, size_t n, int dtype, int mode, unsigned long long seed,
                 unsigned long long tensor_id, float a, float b);

@@ -20,6 +20,12 @@ def gemm_bf16(a, b, c, m, n, k, device_id=0, variant=0):
     check(lib.mrk_hip_gemm_bf16_variant(device_id, _p(a), _p(b), _p(c), m, n, k, variant))
 
 
+def flash_attn_fwd_bf16(q, k, v, o, batch, heads, sq, sk, d, scale, causal=True, device_id=0):
+    """Fused SDPA forward (Tensor::scaled_dot_product_attention, tensor/src/transformer.rs:78-137)."""
+    check(lib.mrk_hip_flash_attn_fwd_bf16(device_id, _p(q), _p(k), _p(v), _p(o), batch, heads, sq, sk, d, scale,
+                                          int(causal)))
+
+
 def fill_normal(buf, n, sigma=1.0, seed=0, tensor_id=0, bf16=False, device_id=0):
     """Device-side synthetic normal(0, sigma) values (benchmark inputs)."""
     check(lib.mrk_hip_fill(device_id, _p(buf), n, int(bf16), 1, seed, tensor_id, sigma, 0.0))
