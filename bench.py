@@ -76,7 +76,98 @@ def bench_softmax(m, dev, steps, warmup, cpu):
     return rec
 
 
-WORKLOADS = {"softmax": bench_softmax}
+def bench_gemm(m, dev, steps, warmup, cpu):
+    """configs[2]: bf16 GEMM M=N=K=4096, inputs normal(0,1) rounded to bf16, f32 accumulate, bf16 out."""
+    from morok_amd import ops, synth
+
+    M = N = K = 4096
+    ba = dev.buffer(M * K * 2).ensure_allocated()
+    bb = dev.buffer(K * N * 2).ensure_allocated()
+    bc = dev.buffer(M * N * 2).ensure_allocated()
+    ops.fill_normal(ba, M * K, seed=3, tensor_id=0, bf16=True)
+    ops.fill_normal(bb, K * N, seed=3, tensor_id=1, bf16=True)
+    ms = m.time_launches(lambda: ops.gemm_bf16(ba, bb, bc, M, N, K), steps, warmup)
+    flops = 2.0 * M * N * K
+    tf = flops / (ms * 1e-3) / 1e12
+    rec = {
+        "metric": "bf16 GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "bf16",
+        "config": {"workload": "bf16 GEMM M=N=K=4096, normal(0,1) inputs, f32 accumulate, bf16 out (configs[2])"},
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None, "kernel": "gemm_bf16_tile256",
+                     "algorithmic_flops_per_launch": flops},
+    }
+    if cpu:
+        from tests.oracle_lib import Oracle
+
+        orc = Oracle()
+        sm = 512  # 512 of the 4096 output rows: ~17 GFLOP of CPU work per run
+        a = synth.normal_bf16((sm, K), 3, 0)
+        b = synth.normal_bf16((K, N), 3, 1)
+        t = orc.thread_count(sm * N * K, sm)
+        sec = _cpu_time(lambda: orc.gemm_bf16(a, b, threads=t))
+        rec["cpu_baseline"] = {"value": 2.0 * sm * N * K / sec / 1e12, "unit": "TFLOP/s", "cores": t, "kind": "port",
+                               "sample": f"{sm} of 4096 output rows (K=N=4096), f32-accumulate bf16 matmul kernel, "
+                                         f"{t} threads, min of 3 after 1 warm-up"}
+    return rec
+
+
+def bench_flash(m, dev, steps, warmup, cpu):
+    """configs[3]: causal flash-attention forward, bf16 Q/K/V [8, 32, 4096, 128], scale 1/sqrt(128)."""
+    from morok_amd import ops, synth
+
+    B, H, S, D = 8, 32, 4096, 128
+    n = B * H * S * D
+    bq, bk, bv, bo = (dev.buffer(n * 2).ensure_allocated() for _ in range(4))
+    for i, b in enumerate((bq, bk, bv)):
+        ops.fill_normal(b, n, seed=4, tensor_id=i, bf16=True)
+    scale = 1.0 / np.sqrt(D)
+    steps = max(1, min(steps, 20))
+    ms = m.time_launches(lambda: ops.flash_attn_fwd_bf16(bq, bk, bv, bo, B, H, S, S, D, scale, True), steps,
+                         min(warmup, 3))
+    flops = 0.5 * 4.0 * B * H * S * S * D  # causal convention: half of the dense 4*B*H*S^2*D
+    tf = flops / (ms * 1e-3) / 1e12
+    rec = {
+        "metric": "flash-attn fwd TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "bf16",
+        "steps": steps,
+        "config": {"workload": "causal flash-attention fwd, bf16 [8,32,4096,128], scale 1/sqrt(128) (configs[3])"},
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None, "kernel": "flash_fwd_d128",
+                     "algorithmic_flops_per_launch": flops},
+    }
+    if cpu:
+        from tests.oracle_lib import Oracle
+
+        orc = Oracle()
+        q = synth.normal_bf16((S, D), 4, 0)
+        k = synth.normal_bf16((S, D), 4, 1)
+        v = synth.normal_bf16((S, D), 4, 2)
+        t = orc.max_threads
+        sec = _cpu_time(lambda: orc.sdpa_bf16_rows(q, k, v, scale, causal=True, threads=t))
+        rec["cpu_baseline"] = {"value": 0.5 * 4.0 * S * S * D / sec / 1e12, "unit": "TFLOP/s", "cores": t,
+                               "kind": "port",
+                               "sample": f"one (batch, head) slice of 256 at S=4096, D=128, causal, rows split over {t} "
+                                         "threads, min of 3 after 1 warm-up; per-unit rate, the full job is 256 such slices"}
+    return rec
+
+
+def bench_copy(m, dev, steps, warmup, cpu):
+    """Calibration only: 256 MiB streaming copy kernel (known traffic 2 x 256 MiB per launch)."""
+    from morok_amd import ops
+
+    nbytes = 256 << 20
+    bx = dev.buffer(nbytes).ensure_allocated()
+    by = dev.buffer(nbytes).ensure_allocated()
+    ops.fill_normal(bx, nbytes // 4, seed=9)
+    ms = m.time_launches(lambda: ops.copy_kernel(bx, by, nbytes), steps, warmup)
+    gbs = 2 * nbytes / (ms * 1e-3) / 1e9
+    return {"metric": "copy GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "u8",
+            "config": {"workload": "calibration: 256 MiB streaming copy kernel"},
+            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "copy_kernel",
+                         "algorithmic_bytes_per_launch": 2 * nbytes}}
+
+
+WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "copy": bench_copy}
 PRIMARY_ORDER = ["gemm", "flash", "softmax"]
 
 

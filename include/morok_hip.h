@@ -219,6 +219,9 @@ int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, con
  * ===================================================================================== */
 int mrk_hip_fill(int device_id, void* out, size_t n, int dtype, int mode, uint64_t seed, uint64_t tensor_id, float a,
                  float b);
+/* Streaming copy kernel over `bytes` (multiple of 16): the kernel of known traffic that
+ * FETCH_SIZE / WRITE_SIZE counter readings are scaled against (no reference counterpart). */
+int mrk_hip_copy_kernel(int device_id, const void* src, void* dst, size_t bytes);
 /* int32 values uniform over [0, high). */
 int mrk_hip_fill_randint(int device_id, void* out, size_t n, uint64_t seed, uint64_t tensor_id, int high);
 

@@ -405,6 +405,18 @@ int mrk_hip_fill_randint(int device_id, void* out, size_t n, uint64_t seed, uint
     return kOk;
 }
 
+int mrk_hip_copy_kernel(int device_id, const void* src, void* dst, size_t bytes) {
+    if (bytes == 0) return kOk;
+    MRK_NONNULL(src);
+    MRK_NONNULL(dst);
+    if (bytes % 16 != 0) return fail(kInvalidArgument, "copy_kernel: size must be a multiple of 16 bytes");
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_copy(d->allocator->stream(), src, dst, bytes), "copy_kernel launch");
+    return kOk;
+}
+
 int mrk_hip_event_create(int device_id, mrk_event** out) {
     MRK_NONNULL(out);
     std::shared_ptr<Device> d;

@@ -47,18 +47,20 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
     // K stage s at s*32 KB, V stage s at s*32 KB + 16 KB
     __shared__ __attribute__((aligned(1024))) char smem[4 * kTile];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Heavy (late) query tiles first; workgroups of one head stay on one XCD (ids mod 8).
+    // Workgroup ids congruent mod 8 run on the same XCD and share its L2.  Each XCD walks
+    // its own heads one after another, all query tiles of a head back to back (heaviest,
+    // i.e. latest, first), so the tiles of a head run concurrently and stream the head's
+    // K and V through that L2 once instead of re-reading them from HBM per query tile.
     int bh, qt;
     {
         const int bid = blockIdx.x;
         if ((BH & 7) == 0) {
-            const int per = BH >> 3;
             const int idx = bid >> 3;
-            bh = (bid & 7) + 8 * (idx % per);
-            qt = q_tiles - 1 - idx / per;
+            bh = (bid & 7) + 8 * (idx / q_tiles);
+            qt = q_tiles - 1 - idx % q_tiles;
         } else {
-            bh = bid % BH;
-            qt = q_tiles - 1 - bid / BH;
+            bh = bid / q_tiles;
+            qt = q_tiles - 1 - bid % q_tiles;
         }
     }
     const int q0 = qt * kQT;
@@ -90,8 +92,10 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
             const int row = wave * 16 + c * 4 + r4;  // row inside the tile
             int key = j * kKT + row;
             key = key < Sk ? key : Sk - 1;  // ragged tail: re-read the last row, masked later
-            // K: 16 B chunk c16 of the LDS row holds logical chunk c16 ^ (row & 7)
-            const unsigned kvoff = (unsigned)key * kRow + ((c16 ^ (row & 7)) << 4);
+            // K: 16 B chunk c16 of the LDS row holds logical chunk c16 ^ (row & 15): the LDS
+            // serves 16 lanes x 16 B per cycle over 64 banks, so 16 consecutive rows must
+            // land in 16 different chunk slots
+            const unsigned kvoff = (unsigned)key * kRow + ((c16 ^ (row & 15)) << 4);
             // V: 32 B granule (c16 >> 1) holds logical granule (c16 >> 1) ^ (row & 3)
             const unsigned vvoff = (unsigned)key * kRow + (((((c16 >> 1) ^ (row & 3)) << 1) | (c16 & 1)) << 4);
             const unsigned dst = lds_base + stage * 2 * kTile + (wave * 16 + c * 4) * kRow;
@@ -118,11 +122,12 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
         for (int e = 0; e < 16; e++) o[db][e] = 0.0f;
     float m_run = -INFINITY;  // running max of raw scores (before scale)
     float l_run = 0.0f;       // this lane's partial row sum
+    const float lazy_thresh = 8.0f / scale_log2e;  // kLazy = 8: probabilities stay below 256
 
     // lane-constant LDS offsets
     // K fragment (A operand): row = kb*32 + l%32, logical chunk 2*ds + l/32
     const int k_row_off = lq * kRow;
-    const int k_sw = lq & 7;
+    const int k_sw = lq & 15;
     // V^T fragment via transposing read: 16-lane block b = l/16 covers d half (b & 1) and
     // key group g = b >> 1; inside the block lane j' = l%16 points at key row j'/4,
     // 8-byte unit j'%4 of the 32-byte granule.
@@ -141,19 +146,28 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
         const char* sK = smem + stage * 2 * kTile;
         const char* sV = sK + kTile;
 
-        // ---- S^T = K Q^T
+        // ---- S^T = K Q^T (K fragments fetched one d-step ahead of the MFMAs that use them)
         f32x16 st[2];
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int e = 0; e < 16; e++) st[kb][e] = 0.0f;
+        {
+            bf16x8 kf[2][2];
 #pragma unroll
-        for (int ds = 0; ds < 8; ds++) {
+            for (int kb = 0; kb < 2; kb++)
+                kf[0][kb] = *LDS_PTR(bf16x8, sK + kb * 32 * kRow + k_row_off + (((0 + lg) ^ k_sw) << 4));
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
-                const int off = kb * 32 * kRow + k_row_off + (((2 * ds + lg) ^ k_sw) << 4);
-                bf16x8 kf = *LDS_PTR(bf16x8, sK + off);
-                st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ds], st[kb], 0, 0, 0);
+            for (int ds = 0; ds < 8; ds++) {
+                if (ds + 1 < 8) {
+#pragma unroll
+                    for (int kb = 0; kb < 2; kb++)
+                        kf[(ds + 1) & 1][kb] =
+                            *LDS_PTR(bf16x8, sK + kb * 32 * kRow + k_row_off + (((2 * (ds + 1) + lg) ^ k_sw) << 4));
+                }
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+                    st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds & 1][kb], qf[ds], st[kb], 0, 0, 0);
             }
         }
         // ---- mask: register e of block kb is key key0 + kb*32 + 8*(e/4) + 4*(l/32) + e%4
@@ -176,11 +190,21 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
 #pragma unroll
             for (int e = 0; e < 16; e++) mx = fmaxf(mx, st[kb][e]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        // m_new is finite from the first tile on: key 0 is visible to every query
-        const float mb = m_new * scale_log2e;
-        const float alpha = __builtin_amdgcn_exp2f(m_run * scale_log2e - mb);
-        m_run = m_new;
+        // Lazy rescaling: the exponentials are taken relative to m_run, which is only moved
+        // (and the accumulators rescaled) when some row's maximum has grown by more than
+        // kLazy / scale_log2e, i.e. when a probability could exceed 2^kLazy.  Rounding P to
+        // bf16 is relative and the row sum is f32, so the result does not depend on which
+        // reference the exponentials use.  The first tile always takes the branch
+        // (m_run = -inf); key 0 is visible to every query, so m_run is finite from then on.
+        if (__builtin_amdgcn_ballot_w64(mx > m_run + lazy_thresh) != 0) {
+            const float m_new = fmaxf(m_run, mx);
+            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int db = 0; db < 4; db++) o[db] *= alpha;
+        }
+        const float mb = m_run * scale_log2e;
         float psum = 0.0f;
         bf16x8 pb[2][2];
 #pragma unroll
@@ -196,24 +220,25 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
                 pb[kb][t] = __builtin_convertvector(p, bf16x8);
             }
         }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int db = 0; db < 4; db++) o[db] *= alpha;
+        l_run += psum;
 
         // ---- O^T += V^T P^T.  MFMA (kb, t) contracts over the 16 keys held in registers
         // 8t .. 8t+7 of block kb: keys kb*32 + 16t + {0, 8} + 4*(l/32) + 0..3.
+        {
+            auto vfrag = [&](int n) {  // n = (kb*2 + t)*4 + db
+                const int kbt = n >> 2, db = n & 3;
+                const int off = (kbt * 16) * kRow + v_row_off + (((db * 2 + v_half) ^ v_rr) << 5);
+                bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sV + off));
+                bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sV + off + 8 * kRow));
+                return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            };
+            bf16x8 vf[3];
+            vf[0] = vfrag(0);
+            vf[1] = vfrag(1);
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-            for (int t = 0; t < 2; t++) {
-#pragma unroll
-                for (int db = 0; db < 4; db++) {
-                    const int off = (kb * 32 + 16 * t) * kRow + v_row_off + (((db * 2 + v_half) ^ v_rr) << 5);
-                    bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sV + off));
-                    bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sV + off + 8 * kRow));
-                    bf16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                    o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pb[kb][t], o[db], 0, 0, 0);
-                }
+            for (int n = 0; n < 16; n++) {
+                if (n + 2 < 16) vf[(n + 2) % 3] = vfrag(n + 2);
+                o[n & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[n % 3], pb[n >> 3][(n >> 2) & 1], o[n & 3], 0, 0, 0);
             }
         }
     }

@@ -70,7 +70,7 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                          __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
                                                          int tiles_n) {
-    // two stages; A stage: 256 rows x 128 B, 16 B chunks XOR-swizzled by (row & 7);
+    // two stages; A stage: 256 rows x 128 B, 16 B chunks XOR-swizzled by ((row >> 1) & 7);
     // B stage: 64 k-rows x 512 B, 32 B granules XOR-swizzled by (k & 3).
     __shared__ __attribute__((aligned(1024))) char smem[kSmem];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -84,8 +84,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     // ---- direct global -> LDS copies: each wave moves 8 KB of A and 8 KB of B per tile,
     // one instruction = 64 lanes x 16 B = 1 KB of contiguous LDS.
     // A chunk q (1 KB = 8 rows): lane -> row q*8 + lane/8, LDS chunk lane%8 holds logical
-    // chunk (lane%8) ^ (row & 7).
-    const unsigned a_voff = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (lane >> 3)) << 3)) * 2);
+    // chunk (lane%8) ^ ((row >> 1) & 7).  The LDS serves 16 lanes x 16 B per cycle over 64
+    // banks; with 128 B rows this swizzle puts 16 consecutive rows of one logical chunk
+    // into 16 different 16 B slots.
+    // (two variants: (row >> 1) & 7 depends on the parity of q)
+    const unsigned a_voff0 = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (lane >> 4)) << 3)) * 2);
+    const unsigned a_voff1 = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (4 + (lane >> 4))) << 3)) * 2);
     // B chunk q (1 KB = 2 k-rows): lane -> k-row q*2 + lane/32, LDS 16 B chunk lane%32 ->
     // granule (lane%32)/2 ^ (krow & 3).
     const int b_h = lane & 1, b_g = (lane & 31) >> 1, b_r = lane >> 5;
@@ -107,7 +111,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     // n = 0..7: A chunks, n = 8..15: B chunks of tile kt into `stage`
     auto dma_one = [&](int n, int kt, int stage) {
         if (n < 8) {
-            dma(lds_a + stage * kAStage + n * 1024, a_voff, a_tile + ((size_t)kt * kBK + (size_t)n * 8 * K) * 2);
+            dma(lds_a + stage * kAStage + n * 1024, (n & 1) ? a_voff1 : a_voff0, a_tile + ((size_t)kt * kBK + (size_t)n * 8 * K) * 2);
         } else {
             const int q = n - 8;
             dma(lds_b + stage * kBStageSw + q * 1024, (q & 1) ? b_voff1 : b_voff0,
@@ -131,7 +135,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     const int a_base_l = (wm * 128 + (lane & 31)) * 128;  // + i*4096
     int a_xo[4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) a_xo[ks] = ((ks * 2 + (lane >> 5)) ^ (lane & 7)) << 4;
+    for (int ks = 0; ks < 4; ks++) a_xo[ks] = ((ks * 2 + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4;
     const int b_rr = (lane & 15) >> 2;
     const int b_g0 = wn * 8 + ((lane >> 4) & 1);
     const int b_row_l = (8 * (lane >> 5) + b_rr) * 512 + 8 * (lane & 3);  // + ks*16*512 + r*4*512

@@ -25,4 +25,7 @@ int launch_fill(void* stream, void* out, size_t n, int dtype, int mode, unsigned
 int launch_fill_randint(void* stream, void* out, size_t n, unsigned long long seed, unsigned long long tensor_id,
                         int high);
 
+// Streaming device-to-device copy kernel (bytes % 16 == 0): traffic-counter calibration.
+int launch_copy(void* stream, const void* in, void* out, size_t bytes);
+
 }  // namespace mrk

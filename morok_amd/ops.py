@@ -37,3 +37,8 @@ def fill_uniform(buf, n, lo=-1.0, hi=1.0, seed=0, tensor_id=0, bf16=False, devic
 
 def fill_randint(buf, n, high, seed=0, tensor_id=0, device_id=0):
     check(lib.mrk_hip_fill_randint(device_id, _p(buf), n, seed, tensor_id, high))
+
+
+def copy_kernel(src, dst, nbytes, device_id=0):
+    """Streaming copy kernel of known traffic (counter calibration)."""
+    check(lib.mrk_hip_copy_kernel(device_id, _p(src), _p(dst), nbytes))
