@@ -113,6 +113,11 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
         const __bf16* qp = Qh + (size_t)qrow * kD + 8 * lg;
 #pragma unroll
         for (int ds = 0; ds < 8; ds++) qf[ds] = *reinterpret_cast<const bf16x8*>(qp + 16 * ds);
+        // Make the compiler wait for these loads here, before the loop: inside the loop the
+        // only outstanding vector-memory operations must be the direct-to-LDS copies it does
+        // not know about, which are drained explicitly in tile_barrier().
+#pragma unroll
+        for (int ds = 0; ds < 8; ds++) asm volatile("" : "+v"(qf[ds]));
     }
 
     f32x16 o[4];
@@ -141,8 +146,8 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
         tile_barrier();  // tile j landed; every wave is done with tile j-1
         if (j + 1 < ntiles) dma_tile(j + 1, stage ^ 1);
         const int key0 = j * kKT;
-        // this wave's queries see nothing of the tile: keys all beyond its last query
-        if (causal && key0 > qw0 + 31) continue;
+        // (a wave whose queries all precede the tile still runs it fully masked: P = 0 adds
+        // nothing, and a branch-free body keeps the accumulators in place)
         const char* sK = smem + stage * 2 * kTile;
         const char* sV = sK + kTile;
 
