@@ -130,6 +130,17 @@ void mrk_hip_buffer_release(mrk_buffer* b);
  * Compiler (device/src/device.rs:142-177) and ProgramSpec / CompiledSpec accessors
  * ===================================================================================== */
 
+/* Renderer::render(&Arc<UOp>, Option<&str>) -> ProgramSpec (device/src/device.rs:186-222;
+ * reference implementation CRenderer::render, codegen/src/c/mod.rs:47-270).  `kernel` is the
+ * serialized linearized stream - the Vec<Arc<UOp>> after linearize_with_cfg +
+ * line_rewrite_cleanups (schedule/src/linearize/mod.rs:172-177,308-310) - in the wire format
+ * documented in morok_amd/csrc/uop.h; `name` may be NULL (falls back to "kernel",
+ * device.rs:192-193).  Emits HIP-C for gfx950: SPECIAL -> blockIdx/threadIdx with the launch
+ * dims taken from the extents, DEFINE_LOCAL -> __shared__, BARRIER -> __syncthreads(),
+ * WMMA -> MFMA builtin.  Works without a GPU.  Renderer::decompositor is None for this
+ * backend (all transcendental ops map to device math functions, cf. c/mod.rs:276-280). */
+int mrk_hip_render(int device_id, const uint8_t* kernel, size_t len, const char* name, mrk_program_spec** out);
+
 /* Builds a ProgramSpec from already-rendered HIP-C source (what Renderer::render returns).
  * var_is_i64[i] != 0 -> scalar argument i is `long long`, else `int`.  global/local may be
  * NULL when the launch sizes are supplied at execute time. */

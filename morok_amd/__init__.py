@@ -8,3 +8,4 @@ from .device import (  # noqa: F401
     time_launches,
 )
 from . import ops  # noqa: F401
+from . import uop  # noqa: F401

@@ -62,6 +62,7 @@ _SIGS = {
     "mrk_hip_buffer_size": (C.c_size_t, [C.c_void_p]),
     "mrk_hip_buffer_synchronize": (C.c_int, [C.c_void_p]),
     "mrk_hip_buffer_release": (None, [C.c_void_p]),
+    "mrk_hip_render": (C.c_int, [C.c_int, C.c_char_p, C.c_size_t, C.c_char_p, c_void_pp]),
     "mrk_hip_program_spec_from_source": (
         C.c_int,
         [C.c_char_p, C.c_char_p, C.c_size_t, C.POINTER(C.c_char_p), C.POINTER(C.c_uint8), C.c_size_t, c_size_p,

@@ -7,6 +7,7 @@
 #include "device.h"
 #include "error.h"
 #include "kernels/kernels.h"
+#include "uop.h"
 
 using namespace mrk;
 
@@ -218,6 +219,23 @@ int mrk_hip_buffer_synchronize(const mrk_buffer* b) {
     return b->b->synchronize();
 }
 void mrk_hip_buffer_release(mrk_buffer* b) { delete b; }
+
+int mrk_hip_render(int device_id, const uint8_t* kernel, size_t len, const char* name, mrk_program_spec** out) {
+    MRK_NONNULL(kernel);
+    MRK_NONNULL(out);
+    LinearKernel k;
+    MRK_TRY(parse_linear_kernel(kernel, len, &k));
+    // The renderer needs no device: rendering works on a host without a GPU.
+    auto renderer = make_hip_renderer(device_id);
+    auto* h = new mrk_program_spec();
+    int rc = renderer->render(k, name, &h->s);
+    if (rc != kOk) {
+        delete h;
+        return rc;
+    }
+    *out = h;
+    return kOk;
+}
 
 int mrk_hip_program_spec_from_source(const char* name, const char* src, size_t buf_count, const char* const* var_names,
                                      const uint8_t* var_is_i64, size_t nvars, const size_t global_size[3],

@@ -43,33 +43,40 @@ constexpr int kTile = kKT * kRow;  // 16 KB
 
 __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
                                                          const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
-                                                         int Sq, int Sk, float scale_log2e, int causal, int q_tiles) {
+                                                         int Sq, int Sk, float scale_log2e, int causal, int q_tiles, int units) {
     // K stage s at s*32 KB, V stage s at s*32 KB + 16 KB
     __shared__ __attribute__((aligned(1024))) char smem[4 * kTile];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // Workgroup ids congruent mod 8 run on the same XCD and share its L2.  Each XCD walks
-    // its own heads one after another, all query tiles of a head back to back (heaviest,
-    // i.e. latest, first), so the tiles of a head run concurrently and stream the head's
-    // K and V through that L2 once instead of re-reading them from HBM per query tile.
-    int bh, qt;
+    // its own heads one after another, all work units of a head back to back, so the units
+    // of a head run concurrently and stream the head's K and V through that L2 once
+    // instead of re-reading them from HBM per query tile.
+    // A work unit is one query tile, or under the causal mask a pair (latest remaining
+    // tile, earliest remaining tile): tile t costs about t+1 key steps, so every pair
+    // costs the same and the workgroups of a launch finish together.
+    int bh, unit;
     {
         const int bid = blockIdx.x;
         if ((BH & 7) == 0) {
             const int idx = bid >> 3;
-            bh = (bid & 7) + 8 * (idx / q_tiles);
-            qt = q_tiles - 1 - idx % q_tiles;
+            bh = (bid & 7) + 8 * (idx / units);
+            unit = idx % units;
         } else {
-            bh = bid / q_tiles;
-            qt = q_tiles - 1 - bid % q_tiles;
+            bh = bid / units;
+            unit = bid % units;
         }
     }
-    const int q0 = qt * kQT;
-    const int qw0 = q0 + wave * 32;  // first query of this wave
     const int lq = lane & 31, lg = lane >> 5;
     const __bf16* Qh = Q + (size_t)bh * Sq * kD;
     const char* Kh = reinterpret_cast<const char*>(K + (size_t)bh * Sk * kD);
     const char* Vh = reinterpret_cast<const char*>(V + (size_t)bh * Sk * kD);
     __bf16* Oh = O + (size_t)bh * Sq * kD;
+    const int first_qt = causal ? q_tiles - 1 - unit : unit;
+    const int npass = (causal && unit != first_qt) ? 2 : 1;
+    for (int pass = 0; pass < npass; pass++) {
+    const int qt = pass == 0 ? first_qt : unit;
+    const int q0 = qt * kQT;
+    const int qw0 = q0 + wave * 32;  // first query of this wave
 
     // number of key tiles this workgroup visits
     int kend = Sk;
@@ -140,6 +147,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
     const int v_row_off = (4 * lg + v_rr) * kRow + 8 * (lane & 3);
     const int v_half = (lane >> 4) & 1;
 
+    if (pass) tile_barrier();  // every wave is done reading the previous pass's last tile
     dma_tile(0, 0);
     for (int j = 0; j < ntiles; j++) {
         const int stage = j & 1;
@@ -262,6 +270,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
                 *reinterpret_cast<bf16x4*>(op + db * 32 + 8 * g) = __builtin_convertvector(v, bf16x4);
             }
     }
+    }  // pass
 }
 
 }  // namespace mrk::dev
@@ -275,13 +284,14 @@ int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void
     if (D != kD || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
     if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
     const long q_tiles = (Sq + kQT - 1) / kQT;
-    const long blocks = BH * q_tiles;
+    const long units = causal ? (q_tiles + 1) / 2 : q_tiles;
+    const long blocks = BH * units;
     if (blocks > 0x7fffffffL) return (int)hipErrorInvalidValue;
     (void)hipGetLastError();
     const float scale_log2e = scale * 1.4426950408889634f;
     flash_fwd_d128<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
-        static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles);
+        static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles, (int)units);
     return (int)hipGetLastError();
 }
 

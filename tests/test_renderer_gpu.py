@@ -1,0 +1,199 @@
+"""Generated kernels on the GPU: render -> compile -> RuntimeFactory -> Program::execute, the
+three boundary hooks of tensor/src/realize.rs:1056-1059, compared with the CPU oracle on the
+same seeded inputs.  Tolerances from the north star: bit-exact for integer/index ops,
+<= 1e-5 relative for f32 elementwise, <= 1e-4 relative for f32 reductions, <= 2e-2 for bf16
+GEMM with fp32 accumulate."""
+import numpy as np
+import pytest
+
+import morok_amd
+from morok_amd import synth, uop as U
+from tests import kernels_lib as KL
+
+pytestmark = pytest.mark.gpu
+
+UNARY_IDS = {"neg": 0, "abs": 1, "sqrt": 2, "rsqrt": 3, "reciprocal": 4, "exp": 5, "exp2": 6, "log": 7, "log2": 8,
+             "sin": 9, "cos": 10, "tan": 11, "floor": 12, "ceil": 13, "trunc": 14, "round": 15, "erf": 16, "sign": 17,
+             "square": 18}
+BINARY_F_IDS = {"add": 0, "sub": 1, "mul": 2, "fdiv": 3, "mod": 4, "max": 5, "pow": 6}
+BINARY_I_IDS = {"add": 0, "sub": 1, "mul": 2, "idiv": 3, "mod": 4, "max": 5, "and": 7, "or": 8, "xor": 9, "shl": 10,
+                "shr": 11}
+
+
+def run(dev, kernel, name, out_shape, out_dtype, inputs, vals=()):
+    spec = U.render(kernel, name, dev.device_id)
+    prog = morok_amd.Program.create(morok_amd.compile_spec(spec), dev.device_id)
+    out = dev.buffer(int(np.prod(out_shape)) * np.dtype(out_dtype).itemsize)
+    bufs = [out] + [morok_amd.Buffer.from_numpy(a, dev.device_id) for a in inputs]
+    prog.execute(bufs, vals)  # launch sizes recorded by the renderer
+    return out.copyout(out_dtype, out_shape)
+
+
+def rel_err(y, ref):
+    return np.abs(y - ref) / np.maximum(np.abs(ref), 1e-30)
+
+
+@pytest.mark.parametrize("op", sorted(UNARY_IDS))
+def test_unary_f32_parity(dev, oracle, op):
+    n = 5000  # not a multiple of the block: exercises the gated tail
+    if op in ("sqrt", "rsqrt", "log", "log2"):
+        x = synth.uniform((n,), 21, 0, 0.01, 50.0)
+    elif op == "reciprocal":
+        x = synth.uniform((n,), 21, 0, 0.5, 50.0) * np.where(synth.uniform((n,), 21, 9) > 0, 1, -1).astype(np.float32)
+    elif op in ("exp", "exp2"):
+        x = synth.uniform((n,), 21, 0, -20.0, 20.0)
+    elif op == "tan":
+        x = synth.uniform((n,), 21, 0, -1.4, 1.4)
+    else:
+        x = synth.uniform((n,), 21, 0, -30.0, 30.0)
+    y = run(dev, KL.elementwise_unary(op, n), "u_" + op, (n,), np.float32, [x])
+    ref = oracle.map_unary_f32(UNARY_IDS[op], x)
+    if op in ("neg", "abs", "floor", "ceil", "trunc", "round", "sign", "square", "sqrt"):
+        assert np.array_equal(y, ref)  # exactly rounded or exact operations
+    elif op in ("sin", "cos"):
+        assert np.abs(y - ref).max() <= 1e-5  # absolute near the zeros of the function
+    else:
+        assert rel_err(y, ref).max() <= 1e-5, rel_err(y, ref).max()
+
+
+@pytest.mark.parametrize("op", sorted(BINARY_F_IDS))
+def test_binary_f32_parity(dev, oracle, op):
+    n = 4099
+    a = synth.uniform((n,), 22, 0, -8.0, 8.0)
+    b = synth.uniform((n,), 22, 1, 0.25, 4.0)
+    if op == "pow":
+        a = np.abs(a) + np.float32(0.1)
+    y = run(dev, KL.elementwise_binary(op, n), "b_" + op, (n,), np.float32, [a, b])
+    ref = oracle.map_binary_f32(BINARY_F_IDS[op], a, b)
+    if op in ("add", "sub", "mul", "fdiv", "max", "mod"):
+        assert np.array_equal(y, ref)  # IEEE-exact operations
+    else:
+        assert rel_err(y, ref).max() <= 1e-5
+
+
+@pytest.mark.parametrize("op", sorted(BINARY_I_IDS))
+def test_binary_i32_bit_exact(dev, oracle, op):
+    n = 3001
+    a = synth.randint((n,), 23, 0, high=200001) - 100000
+    b = synth.randint((n,), 23, 1, high=2001) - 1000
+    if op in ("idiv", "mod"):
+        b = np.where(b == 0, 7, b).astype(np.int32)  # C truncating semantics for negatives (ir/src/types.rs:625-646)
+    if op in ("shl", "shr"):
+        b = (np.abs(b) % 12).astype(np.int32)
+    if op == "mul":
+        a = (a % 20000).astype(np.int32)
+    y = run(dev, KL.elementwise_binary(op, n, U.i32, out_dt=U.i32), "bi_" + op, (n,), np.int32, [a, b])
+    assert np.array_equal(y, oracle.map_binary_i32(BINARY_I_IDS[op], a, b))
+
+
+def test_comparison_to_float_cast(dev):
+    n = 1000
+    a = synth.uniform((n,), 24, 0)
+    b = synth.uniform((n,), 24, 1)
+    y = run(dev, KL.elementwise_binary("lt", n, U.f32, out_dt=U.f32), "cmp", (n,), np.float32, [a, b])
+    assert np.array_equal(y, (a < b).astype(np.float32))
+
+
+@pytest.mark.parametrize("form", [True, False])
+@pytest.mark.parametrize("op", ["max", "add"])
+def test_row_reduce_parity(dev, form, op):
+    rows, cols = 150, 777
+    x = synth.normal((rows, cols), 25, 0, sigma=2.0)
+    y = run(dev, KL.row_reduce(op, rows, cols, form), "rr", (rows,), np.float32, [x])
+    if op == "max":
+        assert np.array_equal(y, x.max(-1))
+    else:
+        # same left-to-right f32 accumulation as the CPU kernel
+        ref = np.zeros(rows, np.float32)
+        for c in range(cols):
+            ref += x[:, c]
+        assert rel_err(y, ref).max() <= 1e-4
+        assert np.array_equal(y, ref)
+
+
+def test_three_kernel_softmax_matches_oracle_and_fused(dev, oracle):
+    rows, cols = 96, 1000
+    x = synth.normal((rows, cols), 2, 0, sigma=2.0)
+    k1, k2, k3 = KL.softmax_kernels(rows, cols)
+    m = run(dev, k1, "r_max", (rows,), np.float32, [x])
+    s = run(dev, k2, "r_expsum", (rows,), np.float32, [x, m])
+    y = run(dev, k3, "E_div", (rows, cols), np.float32, [x, m, s])
+    ref = oracle.softmax_f32(x)
+    assert np.array_equal(m, x.max(-1))
+    big = ref > 1e-30
+    assert rel_err(y, ref)[big].max() <= 1e-5
+
+
+@pytest.mark.parametrize("size,tol", [(128, 0.5), (256, 1.0), (512, 2.0), (1024, 3.0)])
+def test_matmul_f32_reference_generators(dev, oracle, size, tol):
+    # the reference's validated square cases incl. configs[0]'s 1024 x 1024 shape
+    # (tensor/src/test/unit/matmul.rs:24-41,669-677)
+    x = np.arange(size * size)
+    a = ((x % 31).astype(np.float32) * np.float32(0.05) - np.float32(0.8)).reshape(size, size)
+    b = ((x % 37).astype(np.float32) * np.float32(0.04) - np.float32(0.7)).reshape(size, size)
+    c = run(dev, KL.matmul_f32_upcast4x4(size, size, size), "r_mm", (size, size), np.float32, [a, b])
+    ref = oracle.matmul_f32(a, b)
+    assert np.abs(c - a.astype(np.float64) @ b.astype(np.float64)).max() < tol  # the reference's own bound
+    assert np.array_equal(c, ref)  # same sequential fmaf chain per element as the CPU kernel
+
+
+def test_matmul_f32_config0_uniform_inputs(dev, oracle):
+    # configs[0]: A[1024x1024] @ B[1024x1024], entries uniform(-1, 1) from seed 1
+    a = synth.uniform((1024, 1024), 1, 0)
+    b = synth.uniform((1024, 1024), 1, 1)
+    c = run(dev, KL.matmul_f32_upcast4x4(1024, 1024, 1024), "r_mm", (1024, 1024), np.float32, [a, b])
+    ref = oracle.matmul_f32(a, b)
+    assert (np.abs(c - ref) / np.maximum(np.abs(ref), 1e-3)).max() <= 1e-4
+    assert np.array_equal(c, ref)
+
+
+@pytest.mark.parametrize("shape", [(16, 16, 32), (64, 48, 128), (128, 128, 256)])
+def test_wmma_gemm_bf16_parity(dev, oracle, shape):
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 3, 0)
+    b = synth.normal_bf16((K, N), 3, 1)
+    c = run(dev, KL.wmma_gemm_bf16(M, N, K), "r_wmma", (M, N), np.uint16, [a, b])
+    cf, rf = synth.from_bf16(c), synth.from_bf16(oracle.gemm_bf16(a, b))
+    assert np.abs(cf - rf).max() <= 2e-2 * np.abs(rf).max()
+    assert np.all(np.abs(cf - rf) <= np.abs(rf) * 2**-7 + 1e-3)
+    # one-hot operands pin the lane <-> element mapping of the tensor-core operands exactly
+    a1 = np.zeros((M, K), np.float32)
+    a1[np.arange(M), (np.arange(M) * 5) % K] = 1
+    c1 = run(dev, KL.wmma_gemm_bf16(M, N, K), "r_wmma", (M, N), np.uint16, [synth.to_bf16(a1), b])
+    assert np.array_equal(c1, b[(np.arange(M) * 5) % K])
+
+
+def test_wave_reduce_row_sum(dev):
+    rows, cols = 40, 512
+    x = synth.normal((rows, cols), 26, 0)
+    y = run(dev, KL.wave_row_sum(rows, cols), "r_wave", (rows,), np.float32, [x])
+    ref = x.astype(np.float64).sum(-1)
+    assert np.abs(y - ref).max() <= 1e-4 * np.abs(x).sum(-1).max()
+    ones = np.ones((rows, cols), np.float32)
+    assert np.all(run(dev, KL.wave_row_sum(rows, cols), "r_wave", (rows,), np.float32, [ones]) == cols)
+
+
+def test_local_memory_transpose(dev):
+    n = 16
+    x = synth.normal((n, n), 27, 0)
+    y = run(dev, KL.local_memory_transpose(n), "t", (n, n), np.float32, [x])
+    assert np.array_equal(y, x.T)
+
+
+def test_variables_positional_vals(dev):
+    k = U.Kernel()
+    out = k.param(0, U.f32, 1024)
+    n = k.define_var("n", U.i32, 1, 1024)
+    off = k.define_var("off", U.i64, 0, 1 << 40)
+    l = k.special("lidx0", 256)
+    g = k.special("gidx0", 4)
+    idx = k.add(k.mul(g, k.const(256)), l)
+    k.if_(k.binary("lt", idx, n))
+    k.store(k.index(out, idx), k.cast(k.binary("sub", k.add(k.cast(idx, U.i64), off), k.const(1 << 33, U.i64)), U.f32))
+    k.endif()
+    spec = U.render(k, "v", dev.device_id)
+    prog = morok_amd.Program.create(morok_amd.compile_spec(spec), dev.device_id)
+    out_b = dev.buffer(4096, zero_init=True)
+    prog.execute([out_b], [700, (1 << 33) + 5])  # a value that needs all 64 bits
+    y = out_b.copyout(np.float32)
+    assert np.array_equal(y[:700], np.arange(700, dtype=np.float32) + 5) and not y[700:].any()
