@@ -53,6 +53,9 @@ typedef struct mrk_buffer mrk_buffer;               /* device::Buffer        (de
 typedef struct mrk_program_spec mrk_program_spec;   /* device::ProgramSpec   (device/src/device.rs:327-367) */
 typedef struct mrk_compiled_spec mrk_compiled_spec; /* device::CompiledSpec  (device/src/device.rs:72-100) */
 typedef struct mrk_program mrk_program;             /* Box<dyn Program>      (device/src/device.rs:34-60) */
+typedef struct mrk_kernel mrk_kernel;               /* Arc<CachedKernel>     (runtime/src/kernel_cache.rs:27-44) */
+typedef struct mrk_plan mrk_plan;                   /* ExecutionPlan         (runtime/src/execution_plan.rs:84-106) */
+typedef struct mrk_signal mrk_signal;               /* TimelineSignal        (device/src/sync.rs:44-71) */
 typedef struct mrk_event mrk_event;                 /* hipEvent pair member for timing */
 
 /* =====================================================================================
@@ -192,6 +195,66 @@ void mrk_hip_program_destroy(mrk_program* p);
  *   "flash_fwd_bf16"  params = {B*H, Sq, Sk, D, causal, f32 bits of scale}   buffers = {o, q, k, v}
  * Buffer order follows the reference's PARAM numbering: outputs first. */
 int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_program** out);
+
+/* =====================================================================================
+ * Kernel cache (runtime/src/kernel_cache.rs) and execution plan (runtime/src/execution_plan.rs)
+ * ===================================================================================== */
+
+/* get_or_compile_kernel(ast_id, device, || render; compile; runtime) (kernel_cache.rs:87-118;
+ * call site tensor/src/realize.rs:1052-1070): the kernel is looked up by the content hash of
+ * the linearized stream, the device string and the compiler's cache_key; on a miss it goes
+ * through the three boundary hooks.  *was_cached (may be NULL) tells which happened. */
+int mrk_hip_kernel_get_or_compile(int device_id, const uint8_t* kernel, size_t len, const char* name, mrk_kernel** out,
+                                  int* was_cached);
+/* Same cache for a hand-written kernel (kinds and params as for mrk_hip_program_builtin). */
+int mrk_hip_kernel_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_kernel** out);
+/* CachedKernel fields (kernel_cache.rs:27-44). */
+const char* mrk_hip_kernel_entry_point(const mrk_kernel* k);
+const char* mrk_hip_kernel_code(const mrk_kernel* k);
+size_t mrk_hip_kernel_var_count(const mrk_kernel* k);
+const char* mrk_hip_kernel_var_name(const mrk_kernel* k, size_t i);
+/* 1 if both handles share one cached kernel (Arc pointer identity). */
+int mrk_hip_kernel_same(const mrk_kernel* a, const mrk_kernel* b);
+void mrk_hip_kernel_release(mrk_kernel* k);
+size_t mrk_hip_kernel_cache_size(void);
+/* clear_all (kernel_cache.rs:124-130). */
+void mrk_hip_kernel_cache_clear(void);
+
+/* ExecutionPlanBuilder (execution_plan.rs:330-411): buffers are owned by the plan; kernels
+ * refer to them by index in the order the kernel expects (outputs first). */
+int mrk_hip_plan_create(int device_id, mrk_plan** out);
+int mrk_hip_plan_add_buffer(mrk_plan* plan, const mrk_buffer* b, size_t* index);
+int mrk_hip_plan_add_kernel(mrk_plan* plan, const mrk_kernel* k, const size_t* buffer_indices, size_t nbufs,
+                            const int64_t* vals, size_t nvals);
+/* ensure_allocated on every buffer and precompute the raw pointers (execution_plan.rs:391-397). */
+int mrk_hip_plan_build(mrk_plan* plan);
+/* ExecutionPlan::execute (execution_plan.rs:168-181): launches every kernel in order on the
+ * device stream; no synchronisation between kernels. */
+int mrk_hip_plan_execute(mrk_plan* plan);
+/* ExecutionPlan::execute_profiled (execution_plan.rs:200-221): per-kernel elapsed time in ms,
+ * measured with HIP events (the reference uses Instant around blocking CPU calls). */
+int mrk_hip_plan_execute_profiled(mrk_plan* plan, double* elapsed_ms, size_t cap, size_t* count);
+/* ExecutionPlan::execute_with_vars (execution_plan.rs:239-250): rebind variables by name. */
+int mrk_hip_plan_execute_with_vars(mrk_plan* plan, const char* const* names, const int64_t* vals, size_t n);
+size_t mrk_hip_plan_kernel_count(const mrk_plan* plan);
+const char* mrk_hip_plan_kernel_name(const mrk_plan* plan, size_t i);
+void mrk_hip_plan_release(mrk_plan* plan);
+
+/* benchmark_kernel (runtime/src/benchmark.rs:64-91; protocol 23-27: warm-up runs, timed runs,
+ * minimum), timed with HIP events so that asynchronous launches are measured correctly - the
+ * hook beam search needs (tensor/src/realize.rs:1190-1242). */
+int mrk_hip_benchmark_kernel(int device_id, mrk_program* p, void* const* buffers, size_t nbufs, const int64_t* vals,
+                             size_t nvals, const size_t global_size[3], const size_t local_size[3], int warmup, int runs,
+                             double* min_ms, double* mean_ms);
+
+/* TimelineSignal::{set, value, wait(value, timeout_ms)} (device/src/sync.rs:44-71), modelled on
+ * CudaTimelineSignal (sync.rs:192-310): one event per recorded value, the last 16 kept.
+ * wait returns MRK_ERR_TIMEOUT when the value is not reached in time (sync.rs:118-168). */
+int mrk_hip_signal_create(int device_id, mrk_signal** out);
+int mrk_hip_signal_set(mrk_signal* s, uint64_t value);
+uint64_t mrk_hip_signal_value(mrk_signal* s);
+int mrk_hip_signal_wait(mrk_signal* s, uint64_t value, uint64_t timeout_ms);
+void mrk_hip_signal_destroy(mrk_signal* s);
 
 /* =====================================================================================
  * Hand-written kernels, direct entry points (device pointers, queued on the device stream)

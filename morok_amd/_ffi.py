@@ -87,6 +87,34 @@ _SIGS = {
     "mrk_hip_program_name": (C.c_char_p, [C.c_void_p]),
     "mrk_hip_program_destroy": (None, [C.c_void_p]),
     "mrk_hip_program_builtin": (C.c_int, [C.c_int, C.c_char_p, c_i64_p, C.c_size_t, c_void_pp]),
+    "mrk_hip_kernel_get_or_compile": (C.c_int, [C.c_int, C.c_char_p, C.c_size_t, C.c_char_p, c_void_pp,
+                                                C.POINTER(C.c_int)]),
+    "mrk_hip_kernel_builtin": (C.c_int, [C.c_int, C.c_char_p, c_i64_p, C.c_size_t, c_void_pp]),
+    "mrk_hip_kernel_entry_point": (C.c_char_p, [C.c_void_p]),
+    "mrk_hip_kernel_code": (C.c_char_p, [C.c_void_p]),
+    "mrk_hip_kernel_var_count": (C.c_size_t, [C.c_void_p]),
+    "mrk_hip_kernel_var_name": (C.c_char_p, [C.c_void_p, C.c_size_t]),
+    "mrk_hip_kernel_same": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "mrk_hip_kernel_release": (None, [C.c_void_p]),
+    "mrk_hip_kernel_cache_size": (C.c_size_t, []),
+    "mrk_hip_kernel_cache_clear": (None, []),
+    "mrk_hip_plan_create": (C.c_int, [C.c_int, c_void_pp]),
+    "mrk_hip_plan_add_buffer": (C.c_int, [C.c_void_p, C.c_void_p, c_size_p]),
+    "mrk_hip_plan_add_kernel": (C.c_int, [C.c_void_p, C.c_void_p, c_size_p, C.c_size_t, c_i64_p, C.c_size_t]),
+    "mrk_hip_plan_build": (C.c_int, [C.c_void_p]),
+    "mrk_hip_plan_execute": (C.c_int, [C.c_void_p]),
+    "mrk_hip_plan_execute_profiled": (C.c_int, [C.c_void_p, C.POINTER(C.c_double), C.c_size_t, c_size_p]),
+    "mrk_hip_plan_execute_with_vars": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), c_i64_p, C.c_size_t]),
+    "mrk_hip_plan_kernel_count": (C.c_size_t, [C.c_void_p]),
+    "mrk_hip_plan_kernel_name": (C.c_char_p, [C.c_void_p, C.c_size_t]),
+    "mrk_hip_plan_release": (None, [C.c_void_p]),
+    "mrk_hip_benchmark_kernel": (C.c_int, [C.c_int, C.c_void_p, c_void_pp, C.c_size_t, c_i64_p, C.c_size_t, c_size_p,
+                                           c_size_p, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "mrk_hip_signal_create": (C.c_int, [C.c_int, c_void_pp]),
+    "mrk_hip_signal_set": (C.c_int, [C.c_void_p, C.c_uint64]),
+    "mrk_hip_signal_value": (C.c_uint64, [C.c_void_p]),
+    "mrk_hip_signal_wait": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64]),
+    "mrk_hip_signal_destroy": (None, [C.c_void_p]),
     "mrk_hip_softmax_f32": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
     "mrk_hip_softmax_f32_variant": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int]),
     "mrk_hip_gemm_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64]),

@@ -7,6 +7,7 @@
 #include "device.h"
 #include "error.h"
 #include "kernels/kernels.h"
+#include "runtime.h"
 #include "uop.h"
 
 using namespace mrk;
@@ -22,6 +23,15 @@ struct mrk_compiled_spec {
 };
 struct mrk_program {
     std::unique_ptr<Program> p;
+};
+struct mrk_kernel {
+    std::shared_ptr<CachedKernel> k;
+};
+struct mrk_plan {
+    std::unique_ptr<ExecutionPlan> p;
+};
+struct mrk_signal {
+    std::unique_ptr<TimelineSignal> s;
 };
 struct mrk_event {
     int device_id;
@@ -347,6 +357,145 @@ int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* para
     *out = h;
     return kOk;
 }
+
+int mrk_hip_kernel_get_or_compile(int device_id, const uint8_t* kernel, size_t len, const char* name, mrk_kernel** out,
+                                  int* was_cached) {
+    MRK_NONNULL(kernel);
+    MRK_NONNULL(out);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    LinearKernel k;
+    MRK_TRY(parse_linear_kernel(kernel, len, &k));
+    std::shared_ptr<CachedKernel> ck;
+    bool cached = false;
+    MRK_TRY(get_or_compile_linear_kernel(*d, k, name, &ck, &cached));
+    if (was_cached) *was_cached = cached ? 1 : 0;
+    *out = new mrk_kernel{ck};
+    return kOk;
+}
+int mrk_hip_kernel_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_kernel** out) {
+    MRK_NONNULL(kind);
+    MRK_NONNULL(out);
+    if (nparams) MRK_NONNULL(params);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    std::string key = std::string("builtin:") + kind;
+    for (size_t i = 0; i < nparams; i++) key += ":" + std::to_string(params[i]);
+    const std::string device = std::string("HIP:") + std::to_string(device_id);
+    std::shared_ptr<CachedKernel> ck;
+    MRK_TRY(KernelCache::global().get_or_compile(
+        fnv1a64(reinterpret_cast<const uint8_t*>(key.data()), key.size()), device,
+        [&](std::shared_ptr<CachedKernel>* fresh) -> int {
+            std::unique_ptr<Program> p;
+            MRK_TRY(create_builtin_program(device_id, d->allocator->stream(), kind, params, nparams, &p));
+            auto k = std::make_shared<CachedKernel>();
+            k->entry_point = p->name();
+            k->program = std::move(p);
+            k->device = device;
+            *fresh = std::move(k);
+            return kOk;
+        },
+        &ck));
+    *out = new mrk_kernel{ck};
+    return kOk;
+}
+const char* mrk_hip_kernel_entry_point(const mrk_kernel* k) { return k ? k->k->entry_point.c_str() : ""; }
+const char* mrk_hip_kernel_code(const mrk_kernel* k) { return k ? k->k->code.c_str() : ""; }
+size_t mrk_hip_kernel_var_count(const mrk_kernel* k) { return k ? k->k->var_names.size() : 0; }
+const char* mrk_hip_kernel_var_name(const mrk_kernel* k, size_t i) {
+    return (k && i < k->k->var_names.size()) ? k->k->var_names[i].c_str() : "";
+}
+int mrk_hip_kernel_same(const mrk_kernel* a, const mrk_kernel* b) { return a && b && a->k.get() == b->k.get(); }
+void mrk_hip_kernel_release(mrk_kernel* k) { delete k; }
+size_t mrk_hip_kernel_cache_size(void) { return KernelCache::global().size(); }
+void mrk_hip_kernel_cache_clear(void) { KernelCache::global().clear_all(); }
+
+int mrk_hip_plan_create(int device_id, mrk_plan** out) {
+    MRK_NONNULL(out);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    auto* h = new mrk_plan();
+    h->p.reset(new ExecutionPlan(device_id));
+    *out = h;
+    return kOk;
+}
+int mrk_hip_plan_add_buffer(mrk_plan* plan, const mrk_buffer* b, size_t* index) {
+    MRK_NONNULL(plan);
+    MRK_NONNULL(b);
+    MRK_NONNULL(index);
+    *index = plan->p->add_buffer(std::make_shared<Buffer>(*b->b));
+    return kOk;
+}
+int mrk_hip_plan_add_kernel(mrk_plan* plan, const mrk_kernel* k, const size_t* buffer_indices, size_t nbufs,
+                            const int64_t* vals, size_t nvals) {
+    MRK_NONNULL(plan);
+    MRK_NONNULL(k);
+    if (nbufs) MRK_NONNULL(buffer_indices);
+    if (nvals) MRK_NONNULL(vals);
+    return plan->p->add_kernel(k->k, std::vector<size_t>(buffer_indices, buffer_indices + nbufs),
+                               std::vector<int64_t>(vals, vals + nvals));
+}
+int mrk_hip_plan_build(mrk_plan* plan) {
+    MRK_NONNULL(plan);
+    return plan->p->build();
+}
+int mrk_hip_plan_execute(mrk_plan* plan) {
+    MRK_NONNULL(plan);
+    return plan->p->execute();
+}
+int mrk_hip_plan_execute_profiled(mrk_plan* plan, double* elapsed_ms, size_t cap, size_t* count) {
+    MRK_NONNULL(plan);
+    std::vector<KernelProfile> prof;
+    MRK_TRY(plan->p->execute_profiled(&prof));
+    if (count) *count = prof.size();
+    for (size_t i = 0; i < prof.size() && i < cap && elapsed_ms; i++) elapsed_ms[i] = prof[i].elapsed_ms;
+    return kOk;
+}
+int mrk_hip_plan_execute_with_vars(mrk_plan* plan, const char* const* names, const int64_t* vals, size_t n) {
+    MRK_NONNULL(plan);
+    std::vector<std::pair<std::string, int64_t>> kv;
+    for (size_t i = 0; i < n; i++) kv.emplace_back(names[i], vals[i]);
+    return plan->p->execute_with_vars(kv);
+}
+size_t mrk_hip_plan_kernel_count(const mrk_plan* plan) { return plan ? plan->p->kernel_count() : 0; }
+const char* mrk_hip_plan_kernel_name(const mrk_plan* plan, size_t i) {
+    return (plan && i < plan->p->kernel_count()) ? plan->p->kernel(i).kernel->entry_point.c_str() : "";
+}
+void mrk_hip_plan_release(mrk_plan* plan) { delete plan; }
+
+int mrk_hip_benchmark_kernel(int device_id, mrk_program* p, void* const* buffers, size_t nbufs, const int64_t* vals,
+                             size_t nvals, const size_t global_size[3], const size_t local_size[3], int warmup, int runs,
+                             double* min_ms, double* mean_ms) {
+    MRK_NONNULL(p);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    BenchmarkResult r;
+    MRK_TRY(benchmark_kernel(device_id, d->allocator->stream(), p->p.get(), buffers, nbufs, vals, nvals, global_size,
+                             local_size, warmup, runs, &r));
+    if (min_ms) *min_ms = r.min_ms;
+    if (mean_ms) *mean_ms = r.mean_ms;
+    return kOk;
+}
+
+int mrk_hip_signal_create(int device_id, mrk_signal** out) {
+    MRK_NONNULL(out);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    auto* h = new mrk_signal();
+    h->s.reset(new TimelineSignal(device_id, d->allocator->stream()));
+    *out = h;
+    return kOk;
+}
+int mrk_hip_signal_set(mrk_signal* s, uint64_t value) {
+    MRK_NONNULL(s);
+    return s->s->set(value);
+}
+uint64_t mrk_hip_signal_value(mrk_signal* s) { return s ? s->s->value() : 0; }
+int mrk_hip_signal_wait(mrk_signal* s, uint64_t value, uint64_t timeout_ms) {
+    MRK_NONNULL(s);
+    return s->s->wait(value, timeout_ms);
+}
+void mrk_hip_signal_destroy(mrk_signal* s) { delete s; }
 
 int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t rows, int64_t cols, int variant) {
     if (rows < 0 || cols < 0) return fail(kInvalidArgument, "softmax_f32: negative shape");

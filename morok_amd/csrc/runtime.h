@@ -1,0 +1,132 @@
+// Kernel cache and execution plan: the counterparts of runtime/src/kernel_cache.rs:27-158
+// and runtime/src/execution_plan.rs:50-250,391-411.
+#pragma once
+#include <array>
+#include <chrono>
+#include <functional>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "buffer.h"
+#include "device.h"
+
+namespace mrk {
+
+// runtime/src/kernel_cache.rs:27-44
+struct CachedKernel {
+    std::unique_ptr<Program> program;
+    std::string device;  // "HIP:0"
+    std::string code;    // rendered source (empty for hand-written kernels)
+    std::string entry_point;
+    std::vector<std::string> var_names;
+    bool has_sizes = false;
+    std::array<size_t, 3> global_size{1, 1, 1};
+    std::array<size_t, 3> local_size{1, 1, 1};
+};
+
+// Global dedup cache keyed by (AST content hash, device string)
+// (kernel_cache.rs:52-56,87-118).  Two threads racing on one key may both compile; the
+// first insert wins and both receive the winner.
+class KernelCache {
+  public:
+    static KernelCache& global();
+    using CompileFn = std::function<int(std::shared_ptr<CachedKernel>*)>;
+    int get_or_compile(uint64_t ast_hash, const std::string& device, const CompileFn& compile_fn,
+                       std::shared_ptr<CachedKernel>* out, bool* was_cached = nullptr);
+    size_t size();
+    void clear_all();  // kernel_cache.rs:124-130
+
+  private:
+    std::mutex mu_;
+    std::unordered_map<std::string, std::shared_ptr<CachedKernel>> map_;
+};
+
+// Render -> compile -> load through the three hooks of a Device, memoised in the cache:
+// what prepare_execution_plan does per kernel (tensor/src/realize.rs:1052-1070).
+int get_or_compile_linear_kernel(const Device& dev, const LinearKernel& k, const char* name,
+                                 std::shared_ptr<CachedKernel>* out, bool* was_cached = nullptr);
+
+// execution_plan.rs:50-82
+struct PreparedKernel {
+    uint64_t id = 0;
+    std::shared_ptr<CachedKernel> kernel;
+    std::vector<size_t> buffer_indices;
+    std::vector<int64_t> vals;
+    std::vector<void*> buffer_ptrs;  // precomputed with Buffer::as_raw_ptr (execution_plan.rs:391-397)
+    std::vector<uint64_t> buffer_ids;
+};
+
+// runtime/src/profiler.rs:30-39; elapsed is measured with HIP events on the device stream
+// (the reference uses Instant around a blocking CPU call).
+struct KernelProfile {
+    std::string entry_point;
+    size_t num_buffers = 0;
+    double elapsed_ms = 0.0;
+};
+
+class ExecutionPlan {
+  public:
+    explicit ExecutionPlan(int device_id) : device_id_(device_id) {}
+    // Builder (execution_plan.rs:330-411): the plan owns clones of all buffers, which keeps
+    // the precomputed pointers valid.
+    size_t add_buffer(std::shared_ptr<Buffer> b);
+    int add_kernel(std::shared_ptr<CachedKernel> kernel, const std::vector<size_t>& buffer_indices,
+                   const std::vector<int64_t>& vals);
+    void set_outputs(const std::vector<size_t>& idx) { outputs_ = idx; }
+    int build();  // ensure_allocated on every buffer, compute raw pointers
+
+    // execution_plan.rs:168-181: tight loop, no allocation, no per-launch sync.
+    int execute();
+    // execution_plan.rs:200-221
+    int execute_profiled(std::vector<KernelProfile>* out);
+    // execution_plan.rs:239-250: rebinding by name, kernels are not recompiled.
+    int execute_with_vars(const std::vector<std::pair<std::string, int64_t>>& var_vals);
+
+    size_t kernel_count() const { return kernels_.size(); }
+    const PreparedKernel& kernel(size_t i) const { return kernels_[i]; }
+    size_t buffer_count() const { return buffers_.size(); }
+    std::shared_ptr<Buffer> buffer(size_t i) const { return buffers_[i]; }
+    const std::vector<size_t>& outputs() const { return outputs_; }
+    int device_id() const { return device_id_; }
+
+  private:
+    int device_id_;
+    bool built_ = false;
+    std::vector<PreparedKernel> kernels_;
+    std::vector<std::shared_ptr<Buffer>> buffers_;
+    std::vector<size_t> outputs_;
+};
+
+// runtime/src/benchmark.rs:23-27,64-91: warm-up runs, timed runs, minimum; timed with HIP
+// events instead of a wall clock so that the asynchronous launch is measured correctly.
+struct BenchmarkResult {
+    double min_ms = 0, mean_ms = 0, max_ms = 0;
+    int runs = 0;
+};
+int benchmark_kernel(int device_id, ffi::Stream stream, Program* program, void* const* buffers, size_t nbufs,
+                     const int64_t* vals, size_t nvals, const size_t* global, const size_t* local, int warmup,
+                     int runs, BenchmarkResult* out);
+
+// device/src/sync.rs:44-71,192-310: monotonically increasing timeline value backed by one
+// HIP event per recorded value (the last 16 are kept).
+class TimelineSignal {
+  public:
+    TimelineSignal(int device_id, ffi::Stream stream) : device_id_(device_id), stream_(stream) {}
+    ~TimelineSignal();
+    uint64_t value();                       // highest value whose event has completed
+    int set(uint64_t value);                // record an event for `value` on the stream
+    int wait(uint64_t value, uint64_t timeout_ms);  // kTimeout if not reached in time
+    bool is_reached(uint64_t value) { return this->value() >= value; }
+
+  private:
+    int device_id_;
+    ffi::Stream stream_;
+    std::mutex mu_;
+    uint64_t completed_ = 0;
+    std::vector<std::pair<uint64_t, ffi::Event>> pending_;
+};
+
+}  // namespace mrk

@@ -357,3 +357,157 @@ def time_launches(fn, iters, warmup=3, device_id=0):
     e1.record()
     e1.synchronize()
     return e0.elapsed_ms(e1) / iters
+
+
+class Kernel:
+    """Arc<CachedKernel> (runtime/src/kernel_cache.rs:27-44), obtained through the global
+    kernel cache."""
+
+    def __init__(self, handle, was_cached=False):
+        self._h = handle
+        self.was_cached = was_cached
+
+    @classmethod
+    def get_or_compile(cls, kernel, name=None, device_id=0):
+        """get_or_compile_kernel (kernel_cache.rs:87-118) over render -> compile -> runtime."""
+        data = kernel.serialize() if hasattr(kernel, "serialize") else bytes(kernel)
+        h = C.c_void_p()
+        cached = C.c_int(0)
+        check(lib.mrk_hip_kernel_get_or_compile(device_id, data, len(data), name.encode() if name else None,
+                                                C.byref(h), C.byref(cached)))
+        return cls(h, bool(cached.value))
+
+    @classmethod
+    def builtin(cls, kind, params, device_id=0):
+        arr = (C.c_int64 * max(len(params), 1))(*[int(p) for p in params])
+        h = C.c_void_p()
+        check(lib.mrk_hip_kernel_builtin(device_id, kind.encode(), arr, len(params), C.byref(h)))
+        return cls(h)
+
+    @property
+    def entry_point(self):
+        return lib.mrk_hip_kernel_entry_point(self._h).decode()
+
+    @property
+    def code(self):
+        return lib.mrk_hip_kernel_code(self._h).decode()
+
+    @property
+    def var_names(self):
+        return [lib.mrk_hip_kernel_var_name(self._h, i).decode() for i in range(lib.mrk_hip_kernel_var_count(self._h))]
+
+    def same_as(self, other):
+        return bool(lib.mrk_hip_kernel_same(self._h, other._h))
+
+    def __del__(self):
+        try:
+            if self._h:
+                lib.mrk_hip_kernel_release(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+def kernel_cache_size():
+    return lib.mrk_hip_kernel_cache_size()
+
+
+def kernel_cache_clear():
+    lib.mrk_hip_kernel_cache_clear()
+
+
+class ExecutionPlan:
+    """ExecutionPlan + builder (runtime/src/execution_plan.rs:84-250,330-411)."""
+
+    def __init__(self, device_id=0):
+        h = C.c_void_p()
+        check(lib.mrk_hip_plan_create(device_id, C.byref(h)))
+        self._h = h
+        self._buffers = []
+
+    def add_buffer(self, buf):
+        idx = C.c_size_t()
+        check(lib.mrk_hip_plan_add_buffer(self._h, buf._h, C.byref(idx)))
+        self._buffers.append(buf)
+        return idx.value
+
+    def add_kernel(self, kernel, buffer_indices, vals=()):
+        bi = (C.c_size_t * max(len(buffer_indices), 1))(*buffer_indices)
+        va = (C.c_int64 * max(len(vals), 1))(*[int(v) for v in vals])
+        check(lib.mrk_hip_plan_add_kernel(self._h, kernel._h, bi, len(buffer_indices), va, len(vals)))
+
+    def build(self):
+        check(lib.mrk_hip_plan_build(self._h))
+        return self
+
+    def execute(self):
+        check(lib.mrk_hip_plan_execute(self._h))
+
+    def execute_profiled(self):
+        n = lib.mrk_hip_plan_kernel_count(self._h)
+        ms = (C.c_double * max(n, 1))()
+        cnt = C.c_size_t()
+        check(lib.mrk_hip_plan_execute_profiled(self._h, ms, n, C.byref(cnt)))
+        return [(self.kernel_name(i), ms[i]) for i in range(cnt.value)]
+
+    def execute_with_vars(self, var_vals):
+        names = (C.c_char_p * max(len(var_vals), 1))(*[k.encode() for k in var_vals])
+        vals = (C.c_int64 * max(len(var_vals), 1))(*[int(v) for v in var_vals.values()])
+        check(lib.mrk_hip_plan_execute_with_vars(self._h, names, vals, len(var_vals)))
+
+    @property
+    def kernel_count(self):
+        return lib.mrk_hip_plan_kernel_count(self._h)
+
+    def kernel_name(self, i):
+        return lib.mrk_hip_plan_kernel_name(self._h, i).decode()
+
+    def __del__(self):
+        try:
+            if self._h:
+                lib.mrk_hip_plan_release(self._h)
+                self._h = None
+        except Exception:
+            pass
+
+
+def benchmark_kernel(program, buffers, vals=(), global_size=None, local_size=None, warmup=1, runs=3, device_id=0):
+    """benchmark_kernel (runtime/src/benchmark.rs:64-91): (min_ms, mean_ms) with the reference's
+    default protocol of 1 warm-up and 3 timed runs."""
+    ptrs = [b.ptr if isinstance(b, Buffer) else int(b) for b in buffers]
+    parr = (C.c_void_p * max(len(ptrs), 1))(*ptrs)
+    varr = (C.c_int64 * max(len(vals), 1))(*[int(v) for v in vals])
+    mn, mean = C.c_double(), C.c_double()
+    check(lib.mrk_hip_benchmark_kernel(device_id, program._h, parr, len(ptrs), varr, len(vals), _size3(global_size),
+                                       _size3(local_size), warmup, runs, C.byref(mn), C.byref(mean)))
+    return mn.value, mean.value
+
+
+class TimelineSignal:
+    """TimelineSignal over HIP events (device/src/sync.rs:44-71,192-310)."""
+
+    def __init__(self, device_id=0):
+        h = C.c_void_p()
+        check(lib.mrk_hip_signal_create(device_id, C.byref(h)))
+        self._h = h
+
+    def set(self, value):
+        check(lib.mrk_hip_signal_set(self._h, value))
+
+    @property
+    def value(self):
+        return lib.mrk_hip_signal_value(self._h)
+
+    def wait(self, value, timeout_ms):
+        check(lib.mrk_hip_signal_wait(self._h, value, timeout_ms))
+
+    def is_reached(self, value):
+        return self.value >= value
+
+    def __del__(self):
+        try:
+            if self._h:
+                lib.mrk_hip_signal_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass

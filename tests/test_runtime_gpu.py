@@ -1,0 +1,132 @@
+"""Kernel cache, execution plan, benchmark hook and timeline signal on the GPU
+(runtime/src/kernel_cache.rs, runtime/src/execution_plan.rs, runtime/src/benchmark.rs,
+device/src/sync.rs)."""
+import time
+
+import numpy as np
+import pytest
+
+import morok_amd
+from morok_amd import MorokHipError, ops, synth
+from tests import kernels_lib as KL
+
+pytestmark = pytest.mark.gpu
+
+
+def test_kernel_cache_dedup(dev):
+    morok_amd.kernel_cache_clear()
+    k = KL.elementwise_unary("exp", 4096)
+    a = morok_amd.Kernel.get_or_compile(k, "E_exp", dev.device_id)
+    assert not a.was_cached and morok_amd.kernel_cache_size() == 1
+    b = morok_amd.Kernel.get_or_compile(KL.elementwise_unary("exp", 4096), "E_exp", dev.device_id)
+    assert b.was_cached and a.same_as(b) and morok_amd.kernel_cache_size() == 1
+    c = morok_amd.Kernel.get_or_compile(KL.elementwise_unary("exp", 8192), "E_exp", dev.device_id)
+    assert not c.was_cached and not c.same_as(a) and morok_amd.kernel_cache_size() == 2
+    assert a.entry_point == "E_exp" and "expf(" in a.code
+    f1 = morok_amd.Kernel.builtin("softmax_f32", [8, 256], dev.device_id)
+    f2 = morok_amd.Kernel.builtin("softmax_f32", [8, 256], dev.device_id)
+    assert f1.same_as(f2)
+    morok_amd.kernel_cache_clear()
+    assert morok_amd.kernel_cache_size() == 0
+
+
+def test_plan_three_kernel_softmax_vs_fused(dev, oracle):
+    rows, cols = 64, 512
+    x = synth.normal((rows, cols), 2, 0, sigma=2.0)
+    k1, k2, k3 = (morok_amd.Kernel.get_or_compile(k, n, dev.device_id)
+                  for k, n in zip(KL.softmax_kernels(rows, cols), ("r_max", "r_expsum", "E_div")))
+    plan = morok_amd.ExecutionPlan(dev.device_id)
+    bx = plan.add_buffer(morok_amd.Buffer.from_numpy(x, dev.device_id))
+    y_buf, m_buf, s_buf = dev.buffer(x.nbytes), dev.buffer(rows * 4), dev.buffer(rows * 4)
+    assert not m_buf.is_allocated()  # intermediates are allocated by build()
+    by, bm, bs = plan.add_buffer(y_buf), plan.add_buffer(m_buf), plan.add_buffer(s_buf)
+    plan.add_kernel(k1, [bm, bx])
+    plan.add_kernel(k2, [bs, bx, bm])
+    plan.add_kernel(k3, [by, bx, bm, bs])
+    plan.build()
+    assert m_buf.is_allocated() and plan.kernel_count == 3
+    plan.execute()
+    y3 = y_buf.copyout(np.float32, (rows, cols))
+    ref = oracle.softmax_f32(x)
+    assert (np.abs(y3 - ref) / np.maximum(ref, 1e-30))[ref > 1e-30].max() <= 1e-5
+
+    fused = morok_amd.ExecutionPlan(dev.device_id)
+    fx = fused.add_buffer(morok_amd.Buffer.from_numpy(x, dev.device_id))
+    yf = dev.buffer(x.nbytes)
+    fy = fused.add_buffer(yf)
+    fused.add_kernel(morok_amd.Kernel.builtin("softmax_f32", [rows, cols], dev.device_id), [fy, fx])
+    fused.build().execute()
+    y1 = yf.copyout(np.float32, (rows, cols))
+    assert (np.abs(y1 - ref) / np.maximum(ref, 1e-30))[ref > 1e-30].max() <= 1e-5
+
+    prof = plan.execute_profiled()
+    assert [p[0] for p in prof] == ["r_max", "r_expsum", "E_div"]
+    assert all(p[1] > 0 for p in prof)
+    # re-execution is idempotent
+    plan.execute()
+    assert np.array_equal(y_buf.copyout(np.float32, (rows, cols)), y3)
+
+
+def test_plan_errors(dev):
+    k = morok_amd.Kernel.get_or_compile(KL.elementwise_unary("neg", 256), "E_neg", dev.device_id)
+    plan = morok_amd.ExecutionPlan(dev.device_id)
+    b = plan.add_buffer(dev.buffer(1024))
+    with pytest.raises(MorokHipError):
+        plan.add_kernel(k, [b, 7])  # buffer index out of range
+    with pytest.raises(MorokHipError):
+        plan.add_kernel(k, [b, b], vals=[1])  # kernel takes no variables
+    plan.add_kernel(k, [b])  # wrong buffer count surfaces at execute
+    with pytest.raises(MorokHipError) as e:
+        plan.execute()
+    assert "Kernel 0 failed" in e.value.message
+
+
+def test_execute_with_vars_rebinds_by_name(dev):
+    from morok_amd import uop as U
+
+    k = U.Kernel()
+    out = k.param(0, U.f32, 1024)
+    n = k.define_var("n", U.i32, 0, 1024)
+    l = k.special("lidx0", 256)
+    g = k.special("gidx0", 4)
+    idx = k.add(k.mul(g, k.const(256)), l)
+    k.if_(k.binary("lt", idx, n))
+    k.store(k.index(out, idx), k.const(1.0, U.f32))
+    k.endif()
+    kern = morok_amd.Kernel.get_or_compile(k, "fill_n", dev.device_id)
+    assert kern.var_names == ["n"]
+    plan = morok_amd.ExecutionPlan(dev.device_id)
+    ob = dev.buffer(4096, zero_init=True)
+    plan.add_kernel(kern, [plan.add_buffer(ob)], vals=[10])
+    plan.build().execute()
+    assert ob.copyout(np.float32).sum() == 10
+    plan.execute_with_vars({"n": 600, "unrelated": 3})
+    assert ob.copyout(np.float32).sum() == 600
+
+
+def test_benchmark_kernel_protocol(dev):
+    rows = cols = 2048
+    bx = dev.buffer(rows * cols * 4).ensure_allocated()
+    by = dev.buffer(rows * cols * 4).ensure_allocated()
+    ops.fill_normal(bx, rows * cols, seed=5)
+    prog = morok_amd.Program.builtin("softmax_f32", [rows, cols], dev.device_id)
+    mn, mean = morok_amd.benchmark_kernel(prog, [by, bx], warmup=1, runs=3, device_id=dev.device_id)
+    assert 0 < mn <= mean < 50
+    with pytest.raises(MorokHipError):
+        morok_amd.benchmark_kernel(prog, [by, bx], runs=0, device_id=dev.device_id)
+
+
+def test_timeline_signal(dev):
+    s = morok_amd.TimelineSignal(dev.device_id)
+    assert s.value == 0
+    t0 = time.time()
+    with pytest.raises(MorokHipError) as e:
+        s.wait(1, 20)  # nothing recorded: times out (device/src/sync.rs:363-369)
+    assert e.value.code == 12 and "timed out" in e.value.message and time.time() - t0 < 2
+    bx = dev.buffer(1 << 24).ensure_allocated()
+    by = dev.buffer(1 << 24).ensure_allocated()
+    for v in range(1, 25):  # more than the 16 kept events
+        ops.copy_kernel(bx, by, 1 << 24, dev.device_id)
+        s.set(v)
+    s.wait(24, 5000)
+    assert s.value == 24 and s.is_reached(10) and not s.is_reached(25)
