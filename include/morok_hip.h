@@ -257,6 +257,46 @@ int mrk_hip_signal_wait(mrk_signal* s, uint64_t value, uint64_t timeout_ms);
 void mrk_hip_signal_destroy(mrk_signal* s);
 
 /* =====================================================================================
+ * Scheduling helpers for the gfx950 target (what morok's `schedule` crate supplies per backend)
+ * ===================================================================================== */
+
+/* Renderer::amd_cdna4() capability descriptor (schedule/src/optimizer/renderer.rs:290-303) as
+ * "key=value;..." text: device, has_local, has_shared, has_threads, shared_max, global_max,
+ * local_max, upcast_max, tensor_cores (WMMA names in table order). */
+const char* mrk_hip_sched_caps(void);
+/* select_tensor_core (schedule/src/optimizer/tc.rs:126-168) over cdna4_tensor_cores()
+ * (renderer.rs:724-733): scalar dtype tags as in morok_amd/csrc/uop.h; -1 if none matches. */
+int mrk_hip_sched_tc_select(int in0_scalar, int in1_scalar, int acc_scalar);
+/* TensorCore fields (renderer.rs:358-417): dims (N, M, K), threads, elements per lane (A, B, C). */
+int mrk_hip_sched_tc_info(int tc_index, int dims[3], int* threads, int elements_per_thread[3]);
+/* Which matrix element a lane's operand element is, derived from the table's opts and
+ * swizzle (tc.rs:175-215): operand 0 = A -> (m, k), 1 = B -> (n, k), 2 = C -> (m, n). */
+int mrk_hip_sched_tc_operand_element(int tc_index, int operand, int lane, int elem, int* mn, int* k);
+/* gpudims helpers (schedule/src/gpudims.rs:387-463,529-584). group_dims / get_contraction return 1
+ * on success and 0 when no grouping / contraction exists. */
+size_t mrk_hip_sched_find_smallest_divisor(size_t n);
+int mrk_hip_sched_group_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, size_t* out, size_t cap,
+                             size_t* nout);
+int mrk_hip_sched_split_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, size_t* out, size_t cap,
+                             size_t* nout);
+int mrk_hip_sched_limit_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, size_t* out, size_t cap,
+                             size_t* nout);
+int mrk_hip_sched_get_contraction(const size_t* original, size_t n, const size_t* limited, size_t nl, size_t* group_of_dim);
+/* get_grouped_dims (gpudims.rs:331-382): launch extents for `dims` under `max_sizes` (NULL = no
+ * limit; reverse != 0 for global indices) and, when raw/index_per_dim are given, the index of
+ * every original dimension for one tuple of hardware indices. */
+int mrk_hip_sched_grouped_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, int reverse,
+                               size_t* launch, size_t cap, size_t* nlaunch, const size_t* raw, size_t* index_per_dim);
+/* Linearized kernels for the matmul shapes on the hot path, serialized in the wire format
+ * (free with mrk_hip_sched_free): the f32 matmul kernel (LOCAL 16x16, UPCAST 4x4) and the
+ * tensor-core matmul that tc::apply produces (tc.rs:358-674) with post-TC upcasts
+ * (schedule/src/optimizer/heuristics.rs:787-821). */
+int mrk_hip_sched_build_matmul_f32(int64_t m, int64_t n, int64_t k, uint8_t** kernel, size_t* len);
+int mrk_hip_sched_build_wmma_matmul(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, uint8_t** kernel,
+                                    size_t* len);
+void mrk_hip_sched_free(void* p);
+
+/* =====================================================================================
  * Hand-written kernels, direct entry points (device pointers, queued on the device stream)
  * ===================================================================================== */
 

@@ -10,3 +10,4 @@ from .device import (  # noqa: F401
 )
 from . import ops  # noqa: F401
 from . import uop  # noqa: F401
+from . import sched  # noqa: F401

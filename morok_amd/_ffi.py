@@ -115,6 +115,23 @@ _SIGS = {
     "mrk_hip_signal_value": (C.c_uint64, [C.c_void_p]),
     "mrk_hip_signal_wait": (C.c_int, [C.c_void_p, C.c_uint64, C.c_uint64]),
     "mrk_hip_signal_destroy": (None, [C.c_void_p]),
+    "mrk_hip_sched_caps": (C.c_char_p, []),
+    "mrk_hip_sched_tc_select": (C.c_int, [C.c_int, C.c_int, C.c_int]),
+    "mrk_hip_sched_tc_info": (C.c_int, [C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "mrk_hip_sched_tc_operand_element": (C.c_int, [C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_int),
+                                                   C.POINTER(C.c_int)]),
+    "mrk_hip_sched_find_smallest_divisor": (C.c_size_t, [C.c_size_t]),
+    "mrk_hip_sched_group_dims": (C.c_int, [c_size_p, C.c_size_t, c_size_p, C.c_size_t, c_size_p, C.c_size_t, c_size_p]),
+    "mrk_hip_sched_split_dims": (C.c_int, [c_size_p, C.c_size_t, c_size_p, C.c_size_t, c_size_p, C.c_size_t, c_size_p]),
+    "mrk_hip_sched_limit_dims": (C.c_int, [c_size_p, C.c_size_t, c_size_p, C.c_size_t, c_size_p, C.c_size_t, c_size_p]),
+    "mrk_hip_sched_get_contraction": (C.c_int, [c_size_p, C.c_size_t, c_size_p, C.c_size_t, c_size_p]),
+    "mrk_hip_sched_grouped_dims": (C.c_int, [c_size_p, C.c_size_t, c_size_p, C.c_size_t, C.c_int, c_size_p, C.c_size_t,
+                                             c_size_p, c_size_p, c_size_p]),
+    "mrk_hip_sched_build_matmul_f32": (C.c_int, [C.c_int64, C.c_int64, C.c_int64, C.POINTER(C.POINTER(C.c_uint8)),
+                                                 c_size_p]),
+    "mrk_hip_sched_build_wmma_matmul": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int,
+                                                  C.POINTER(C.POINTER(C.c_uint8)), c_size_p]),
+    "mrk_hip_sched_free": (None, [C.c_void_p]),
     "mrk_hip_softmax_f32": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
     "mrk_hip_softmax_f32_variant": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int]),
     "mrk_hip_gemm_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64]),

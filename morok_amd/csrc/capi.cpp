@@ -1,4 +1,5 @@
 // extern "C" surface of libmorok_hip.so (declared in include/morok_hip.h).
+#include <cstdlib>
 #include <cstring>
 
 #include "../../include/morok_hip.h"
@@ -8,6 +9,7 @@
 #include "error.h"
 #include "kernels/kernels.h"
 #include "runtime.h"
+#include "schedule.h"
 #include "uop.h"
 
 using namespace mrk;
@@ -496,6 +498,122 @@ int mrk_hip_signal_wait(mrk_signal* s, uint64_t value, uint64_t timeout_ms) {
     return s->s->wait(value, timeout_ms);
 }
 void mrk_hip_signal_destroy(mrk_signal* s) { delete s; }
+
+// ---- scheduling helpers
+size_t mrk_hip_sched_find_smallest_divisor(size_t n) { return find_smallest_divisor(n); }
+static int put_dims(const std::vector<size_t>& v, size_t* out, size_t cap, size_t* n) {
+    if (n) *n = v.size();
+    for (size_t i = 0; i < v.size() && i < cap && out; i++) out[i] = v[i];
+    return kOk;
+}
+int mrk_hip_sched_group_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, size_t* out, size_t cap,
+                             size_t* nout) {
+    std::vector<size_t> r;
+    if (!group_dims(std::vector<size_t>(dims, dims + n), std::vector<size_t>(max_sizes, max_sizes + nmax), &r)) return 0;
+    put_dims(r, out, cap, nout);
+    return 1;
+}
+int mrk_hip_sched_split_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, size_t* out, size_t cap,
+                             size_t* nout) {
+    return put_dims(split_dims(std::vector<size_t>(dims, dims + n), std::vector<size_t>(max_sizes, max_sizes + nmax)), out,
+                    cap, nout);
+}
+int mrk_hip_sched_limit_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, size_t* out, size_t cap,
+                             size_t* nout) {
+    return put_dims(limit_dims(std::vector<size_t>(dims, dims + n), std::vector<size_t>(max_sizes, max_sizes + nmax)), out,
+                    cap, nout);
+}
+int mrk_hip_sched_get_contraction(const size_t* original, size_t n, const size_t* limited, size_t nl, size_t* group_of_dim) {
+    std::vector<std::vector<size_t>> c;
+    if (!get_contraction(std::vector<size_t>(original, original + n), std::vector<size_t>(limited, limited + nl), &c)) return 0;
+    for (size_t g = 0; g < c.size(); g++)
+        for (size_t d : c[g])
+            if (group_of_dim) group_of_dim[d] = g;
+    return 1;
+}
+int mrk_hip_sched_grouped_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, int reverse,
+                               size_t* launch, size_t cap, size_t* nlaunch, const size_t* raw, size_t* index_per_dim) {
+    std::vector<size_t> mx(max_sizes, max_sizes + nmax);
+    GroupedDims g = get_grouped_dims(std::vector<size_t>(dims, dims + n), max_sizes ? &mx : nullptr, reverse != 0);
+    put_dims(g.launch, launch, cap, nlaunch);
+    if (raw && index_per_dim) {
+        std::vector<size_t> r(raw, raw + g.launch.size());
+        for (size_t i = 0; i < r.size(); i++)
+            if (r[i] >= g.launch[i]) return fail(kInvalidArgument, "grouped_dims: raw index out of range");
+        std::vector<size_t> m = g.map(r);
+        for (size_t i = 0; i < m.size(); i++) index_per_dim[i] = m[i];
+    }
+    return kOk;
+}
+const char* mrk_hip_sched_caps(void) {
+    static std::string desc = [] {
+        RendererCaps c = amd_cdna4_caps();
+        std::string s = "device=" + c.device + ";has_local=" + std::to_string(c.has_local) +
+                        ";has_shared=" + std::to_string(c.has_shared) + ";has_threads=" + std::to_string(c.has_threads) +
+                        ";shared_max=" + std::to_string(c.shared_max) + ";global_max=";
+        for (size_t i = 0; i < c.global_max.size(); i++) s += (i ? "," : "") + std::to_string(c.global_max[i]);
+        s += ";local_max=" + std::to_string(c.local_max) + ";upcast_max=" + std::to_string(c.upcast_max) + ";tensor_cores=";
+        for (size_t i = 0; i < c.tensor_cores.size(); i++) s += (i ? "," : "") + wmma_name(c.tensor_cores[i]);
+        return s;
+    }();
+    return desc.c_str();
+}
+int mrk_hip_sched_tc_select(int in0_scalar, int in1_scalar, int acc_scalar) {
+    return select_tensor_core(cdna4_tensor_cores(), static_cast<Scalar>(in0_scalar), static_cast<Scalar>(in1_scalar),
+                              static_cast<Scalar>(acc_scalar));
+}
+int mrk_hip_sched_tc_info(int tc_index, int dims[3], int* threads, int elements_per_thread[3]) {
+    auto tcs = cdna4_tensor_cores();
+    if (tc_index < 0 || tc_index >= (int)tcs.size()) return fail(kInvalidArgument, "tc index out of range");
+    for (int i = 0; i < 3; i++) {
+        if (dims) dims[i] = tcs[tc_index].dims[i];
+        if (elements_per_thread) elements_per_thread[i] = tcs[tc_index].elements_per_thread[i];
+    }
+    if (threads) *threads = tcs[tc_index].threads;
+    return kOk;
+}
+int mrk_hip_sched_tc_operand_element(int tc_index, int operand, int lane, int elem, int* mn, int* k) {
+    auto tcs = cdna4_tensor_cores();
+    if (tc_index < 0 || tc_index >= (int)tcs.size() || operand < 0 || operand > 2)
+        return fail(kInvalidArgument, "tc index or operand out of range");
+    if (operand == 2) tc_acc_element(tcs[tc_index], lane, elem, mn, k);
+    else tc_operand_element(tcs[tc_index], operand, lane, elem, mn, k);
+    return kOk;
+}
+static int export_kernel(const LinearKernel& k, KernelBuilder* /*unused*/, const std::vector<uint8_t>& bytes, uint8_t** out,
+                         size_t* len) {
+    (void)k;
+    uint8_t* p = static_cast<uint8_t*>(std::malloc(bytes.size() ? bytes.size() : 1));
+    if (!p) return fail(kRuntime, "out of host memory");
+    std::memcpy(p, bytes.data(), bytes.size());
+    *out = p;
+    *len = bytes.size();
+    return kOk;
+}
+static std::vector<uint8_t> reserialize(const LinearKernel& k) {
+    KernelBuilder b;
+    for (const UOp& u : k.nodes) b.add(u.op, u.dtype, u.src, u.arg_i, u.arg_f, u.sub, u.str, u.extra);
+    return b.serialize();
+}
+int mrk_hip_sched_build_matmul_f32(int64_t m, int64_t n, int64_t k, uint8_t** kernel, size_t* len) {
+    MRK_NONNULL(kernel);
+    MRK_NONNULL(len);
+    if (m <= 0 || n <= 0 || k < 0 || m % 64 || n % 64)
+        return fail(kInvalidArgument, "matmul_f32 kernel: M and N must be positive multiples of 64");
+    LinearKernel lk = build_matmul_f32_kernel(m, n, k);
+    return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
+}
+int mrk_hip_sched_build_wmma_matmul(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, uint8_t** kernel,
+                                    size_t* len) {
+    MRK_NONNULL(kernel);
+    MRK_NONNULL(len);
+    auto tcs = cdna4_tensor_cores();
+    if (tc_index < 0 || tc_index >= (int)tcs.size()) return fail(kInvalidArgument, "tc index out of range");
+    LinearKernel lk;
+    MRK_TRY(build_wmma_matmul_kernel(tcs[tc_index], m, n, k, static_cast<Scalar>(out_scalar), &lk));
+    return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
+}
+void mrk_hip_sched_free(void* p) { std::free(p); }
 
 int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t rows, int64_t cols, int variant) {
     if (rows < 0 || cols < 0) return fail(kInvalidArgument, "softmax_f32: negative shape");

@@ -361,6 +361,7 @@ bool wmma_wrapper(const std::string& name, std::string* def) {
         {"WMMA_16_16_32_bfloat_float", "__builtin_amdgcn_mfma_f32_16x16x32_bf16", "__bf16", 8},
         {"WMMA_16_16_32_half_float", "__builtin_amdgcn_mfma_f32_16x16x32_f16", "_Float16", 8},
         {"WMMA_16_16_16_half_float", "__builtin_amdgcn_mfma_f32_16x16x16f16", "_Float16", 4},
+        {"WMMA_16_16_16_bfloat_float", "__builtin_amdgcn_mfma_f32_16x16x16bf16_1k", "__bf16", 4},
     };
     for (const Entry& e : table) {
         if (name == e.name) {

@@ -1,0 +1,542 @@
+#include "schedule.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "error.h"
+
+namespace mrk {
+
+// ============================================================================ tensor cores
+namespace {
+
+std::vector<TcOpt> opts_from(const char* s) {  // "l0 l0 l0 l0 u1 u1 l1 l1"
+    std::vector<TcOpt> v;
+    for (const char* p = s; *p; p++)
+        if (*p == 'l' || *p == 'u') v.push_back(TcOpt{*p, p[1] - '0'});
+    return v;
+}
+std::vector<SwizzleAxis> sw(std::initializer_list<const char*> items) {
+    std::vector<SwizzleAxis> v;
+    for (const char* it : items) v.push_back(SwizzleAxis{it[0], it[1] - '0'});
+    return v;
+}
+
+// renderer.rs:538-547
+TensorCore cdna_161616(Scalar in, Scalar out) {
+    TensorCore t;
+    t.dims = {16, 16, 16};
+    t.threads = 64;
+    t.elements_per_thread = {4, 4, 4};
+    t.dtype_in = in;
+    t.dtype_out = out;
+    t.opts = opts_from("l0 l0 l0 l0 u1 u1 l1 l1");
+    t.swizzle[0] = {sw({"u0", "u1", "l4", "l5", "r2", "r3"}), sw({"r0", "r1"}), sw({"l0", "l1", "l2", "l3"})};
+    t.swizzle[1] = {sw({"l0", "l1", "l2", "l3", "r2", "r3"}), sw({"r0", "r1"}), sw({"l4", "l5", "u0", "u1"})};
+    return t;
+}
+// renderer.rs:549-558
+TensorCore cdna_161632(Scalar in, Scalar out) {
+    TensorCore t;
+    t.dims = {16, 16, 32};
+    t.threads = 64;
+    t.elements_per_thread = {8, 8, 4};
+    t.dtype_in = in;
+    t.dtype_out = out;
+    t.opts = opts_from("l0 l0 l0 l0 u1 u1 l1 l1");
+    t.swizzle[0] = {sw({"u0", "u1", "l4", "l5", "r3", "r4"}), sw({"r0", "r1"}), sw({"l0", "l1", "l2", "l3", "r2"})};
+    t.swizzle[1] = {sw({"l0", "l1", "l2", "l3", "r3", "r4"}), sw({"r0", "r1"}), sw({"l4", "l5", "u0", "u1", "r2"})};
+    return t;
+}
+
+const char* tc_dtype_name(Scalar s) {  // tc.rs:677-688
+    switch (s) {
+        case Scalar::Float16: return "half";
+        case Scalar::BFloat16: return "bfloat";
+        case Scalar::Float32: return "float";
+        case Scalar::Float64: return "double";
+        default: return "unknown";
+    }
+}
+
+int ilog2(int v) {
+    int r = 0;
+    while ((1 << (r + 1)) <= v) r++;
+    return r;
+}
+
+// logical axis of every l_i / u_i produced by the opts: (axis 0 = N, 1 = M; bit within axis).
+// Each opt splits its axis by 2 and the new range becomes the low part, so successive
+// splits of one axis take bits 0, 1, 2, ...
+struct Logical {
+    int axis;  // 0 N, 1 M, 2 K
+    int bit;
+};
+void logical_axes(const TensorCore& tc, std::vector<Logical>* locals, std::vector<Logical>* upcasts) {
+    int next_bit[2] = {0, 0};
+    for (const TcOpt& o : tc.opts) {
+        Logical l{o.axis, next_bit[o.axis]++};
+        (o.kind == 'l' ? locals : upcasts)->push_back(l);
+    }
+}
+Logical resolve(const SwizzleAxis& a, const std::vector<Logical>& locals, const std::vector<Logical>& upcasts) {
+    if (a.kind == 'l') return locals[a.idx];
+    if (a.kind == 'u') return upcasts[a.idx];
+    return Logical{2, a.idx};
+}
+
+}  // namespace
+
+std::vector<TensorCore> cdna4_tensor_cores() {
+    return {
+        cdna_161632(Scalar::Float16, Scalar::Float32),
+        cdna_161632(Scalar::BFloat16, Scalar::Float32),
+        cdna_161616(Scalar::Float16, Scalar::Float32),
+        cdna_161616(Scalar::BFloat16, Scalar::Float32),
+    };
+}
+
+RendererCaps amd_cdna4_caps() {
+    RendererCaps c;
+    c.device = "AMD_CDNA4";
+    c.has_local = true;
+    c.has_shared = true;
+    c.has_threads = false;
+    c.shared_max = 163840;
+    c.global_max = {2147483647, 65535, 65535};
+    c.local_max = 1024;
+    c.upcast_max = 8;
+    c.tensor_cores = cdna4_tensor_cores();
+    return c;
+}
+
+int select_tensor_core(const std::vector<TensorCore>& tcs, Scalar in0, Scalar in1, Scalar acc) {
+    for (size_t i = 0; i < tcs.size(); i++)
+        if (tcs[i].dtype_in == in0 && tcs[i].dtype_in == in1 && tcs[i].dtype_out == acc) return static_cast<int>(i);
+    return -1;
+}
+
+std::string wmma_name(const TensorCore& tc) {
+    return "WMMA_" + std::to_string(tc.dims[0]) + "_" + std::to_string(tc.dims[1]) + "_" + std::to_string(tc.dims[2]) +
+           "_" + tc_dtype_name(tc.dtype_in) + "_" + tc_dtype_name(tc.dtype_out);
+}
+
+void tc_operand_element(const TensorCore& tc, int operand, int lane, int elem, int* mn, int* k) {
+    std::vector<Logical> locals, upcasts;
+    logical_axes(tc, &locals, &upcasts);
+    const auto& s = tc.swizzle[operand];
+    const int relevant = operand == 0 ? 1 : 0;  // A depends on M, B on N
+    int out_mn = 0, out_k = 0;
+    auto apply = [&](const Logical& l) {
+        if (l.axis == 2) out_k |= 1 << l.bit;
+        else if (l.axis == relevant) out_mn |= 1 << l.bit;
+    };
+    // lane bit p <- logical axis at local position p of the operand's view
+    for (size_t p = 0; p < s[0].size(); p++)
+        if (lane & (1 << p)) apply(resolve(s[0][p], locals, upcasts));
+    // element bits: the upcast positions, then the reduce positions, skipping axes the operand
+    // does not depend on (those are broadcast in its view)
+    int ebit = 0;
+    for (int part = 1; part <= 2; part++)
+        for (const SwizzleAxis& a : s[part]) {
+            Logical l = resolve(a, locals, upcasts);
+            if (l.axis != 2 && l.axis != relevant) continue;
+            if (elem & (1 << ebit)) apply(l);
+            ebit++;
+        }
+    *mn = out_mn;
+    *k = out_k;
+}
+
+void tc_acc_element(const TensorCore& tc, int lane, int elem, int* m, int* n) {
+    std::vector<Logical> locals, upcasts;
+    logical_axes(tc, &locals, &upcasts);
+    int om = 0, on = 0;
+    for (size_t p = 0; p < locals.size(); p++)
+        if (lane & (1 << p)) (locals[p].axis == 0 ? on : om) |= 1 << locals[p].bit;
+    for (size_t p = 0; p < upcasts.size(); p++)
+        if (elem & (1 << p)) (upcasts[p].axis == 0 ? on : om) |= 1 << upcasts[p].bit;
+    *m = om;
+    *n = on;
+}
+
+// ============================================================================ gpudims
+size_t find_smallest_divisor(size_t n) {
+    if (n <= 1) return 1;
+    size_t lim = static_cast<size_t>(std::ceil(std::sqrt(static_cast<double>(n))));
+    for (size_t d = 2; d <= lim; d++)
+        if (n % d == 0) return d;
+    return 1;  // prime (the reference reports primes, 2 and 3 included via the sqrt bound, as "no divisor")
+}
+
+bool group_dims(const std::vector<size_t>& dims, const std::vector<size_t>& max_sizes, std::vector<size_t>* out) {
+    std::vector<size_t> r = dims;
+    auto fits = [&]() {
+        if (r.size() > max_sizes.size()) return false;
+        for (size_t i = 0; i < r.size(); i++)
+            if (r[i] > max_sizes[i]) return false;
+        return true;
+    };
+    while (!fits()) {
+        bool grouped = false;
+        size_t lim = std::min(max_sizes.size(), r.size() ? r.size() - 1 : 0);
+        for (size_t i = 0; i < lim; i++) {
+            if (i + 1 >= r.size()) break;
+            unsigned __int128 prod = static_cast<unsigned __int128>(r[i]) * r[i + 1];
+            if (prod <= max_sizes[i]) {
+                r[i] = static_cast<size_t>(prod);
+                r.erase(r.begin() + static_cast<long>(i) + 1);
+                grouped = true;
+                break;
+            }
+        }
+        if (!grouped) return false;
+    }
+    *out = r;
+    return true;
+}
+
+std::vector<size_t> split_dims(const std::vector<size_t>& dims, const std::vector<size_t>& max_sizes) {
+    std::vector<size_t> r = dims;
+    while (r.size() < 3) r.push_back(1);
+    for (size_t i = 0; i < r.size(); i++) {
+        size_t mx = i < max_sizes.size() ? max_sizes[i] : static_cast<size_t>(-1);
+        while (r[i] > mx) {
+            size_t d = find_smallest_divisor(r[i]);
+            if (d == 1) break;
+            size_t next = (i + 1) % r.size();
+            r[i] /= d;
+            r[next] *= d;
+        }
+    }
+    while (r.size() > 1 && r.back() == 1) r.pop_back();
+    return r;
+}
+
+std::vector<size_t> limit_dims(const std::vector<size_t>& dims, const std::vector<size_t>& max_sizes) {
+    std::vector<size_t> g;
+    if (group_dims(dims, max_sizes, &g)) return g;
+    return split_dims(dims, max_sizes);
+}
+
+bool get_contraction(const std::vector<size_t>& original, const std::vector<size_t>& limited,
+                     std::vector<std::vector<size_t>>* out) {
+    out->clear();
+    if (original.empty() && limited.empty()) return true;
+    if (limited.empty()) return false;
+    std::vector<size_t> acc_old, acc_new;
+    size_t a = 1;
+    for (size_t x : original) acc_old.push_back(a *= x);
+    a = 1;
+    for (size_t x : limited) acc_new.push_back(a *= x);
+    std::vector<size_t> split;
+    for (size_t acc : acc_new) {
+        if (acc == 1) {
+            split.push_back(0);
+            continue;
+        }
+        auto it = std::find(acc_old.begin(), acc_old.end(), acc);
+        if (it == acc_old.end()) return false;
+        split.push_back(static_cast<size_t>(it - acc_old.begin()) + 1);
+    }
+    size_t prev = 0;
+    for (size_t i = 0; i < split.size(); i++) {
+        std::vector<size_t> g;
+        size_t hi = (i + 1 == split.size()) ? original.size() : split[i];
+        for (size_t j = prev; j < hi; j++) g.push_back(j);
+        out->push_back(g);
+        if (i + 1 != split.size()) prev = split[i];
+    }
+    return true;
+}
+
+GroupedDims get_grouped_dims(const std::vector<size_t>& dims, const std::vector<size_t>* max_sizes, bool reverse) {
+    GroupedDims g;
+    g.original = dims;
+    g.reverse = reverse;
+    std::vector<size_t> d = dims;
+    if (reverse) std::reverse(d.begin(), d.end());
+    g.launch = max_sizes ? limit_dims(d, *max_sizes) : d;
+    return g;
+}
+
+std::vector<size_t> GroupedDims::map(const std::vector<size_t>& raw) const {
+    std::vector<size_t> d = original;
+    if (reverse) std::reverse(d.begin(), d.end());
+    std::vector<size_t> res;
+    if (launch == d) {
+        res = raw;
+    } else {
+        std::vector<std::vector<size_t>> contraction;
+        if (launch.size() < d.size() && get_contraction(d, launch, &contraction)) {
+            // grouped: peel the original dims off each fused index, fastest-varying first
+            res.assign(d.size(), 0);
+            for (size_t gi = 0; gi < contraction.size(); gi++) {
+                size_t cur = raw[gi];
+                const auto& grp = contraction[gi];
+                for (size_t j = 0; j + 1 < grp.size(); j++) {
+                    res[grp[j]] = cur % d[grp[j]];
+                    cur /= d[grp[j]];
+                }
+                if (!grp.empty()) res[grp.back()] = cur;
+            }
+        } else {
+            // split or reshaped: flatten the raw indices row-major, unflatten over the original dims
+            size_t flat = 0;
+            for (size_t i = 0; i < launch.size(); i++) flat = flat * launch[i] + raw[i];
+            res.assign(d.size(), 0);
+            for (size_t i = d.size(); i-- > 0;) {
+                res[i] = flat % d[i];
+                flat /= d[i];
+            }
+        }
+    }
+    if (reverse) std::reverse(res.begin(), res.end());
+    return res;
+}
+
+// ============================================================================ kernel builder
+uint32_t KernelBuilder::add(Op op, DType dt, std::vector<uint32_t> src, int64_t arg_i, double arg_f, uint16_t sub,
+                            std::string str, std::vector<int64_t> extra) {
+    UOp u;
+    u.id = static_cast<uint32_t>(k_.nodes.size()) + 1;
+    u.op = op;
+    u.dtype = dt;
+    u.src = std::move(src);
+    u.arg_i = arg_i;
+    u.arg_f = arg_f;
+    u.sub = sub;
+    u.str = std::move(str);
+    u.extra = std::move(extra);
+    k_.nodes.push_back(std::move(u));
+    return k_.nodes.back().id;
+}
+
+uint32_t KernelBuilder::binary(BinaryOp op, uint32_t a, uint32_t b) {
+    DType d = dtype(a);
+    switch (op) {
+        case BinaryOp::Lt:
+        case BinaryOp::Le:
+        case BinaryOp::Gt:
+        case BinaryOp::Ge:
+        case BinaryOp::Eq:
+        case BinaryOp::Ne: d = scalar(Scalar::Bool, d.vcount); break;
+        default: break;
+    }
+    return add(Op::Binary, d, {a, b}, 0, 0, static_cast<uint16_t>(op));
+}
+
+uint32_t KernelBuilder::iadd(uint32_t a, uint32_t b) {
+    const UOp& na = node(a);
+    const UOp& nb = node(b);
+    if (na.op == Op::Const && na.arg_i == 0) return b;
+    if (nb.op == Op::Const && nb.arg_i == 0) return a;
+    if (na.op == Op::Const && nb.op == Op::Const) return ci(na.arg_i + nb.arg_i, na.dtype.scalar);
+    return binary(BinaryOp::Add, a, b);
+}
+uint32_t KernelBuilder::imul(uint32_t a, int64_t c) {
+    const UOp& na = node(a);
+    if (c == 1) return a;
+    if (na.op == Op::Const) return ci(na.arg_i * c, na.dtype.scalar);
+    if (c == 0) return ci(0, na.dtype.scalar);
+    return binary(BinaryOp::Mul, a, ci(c, na.dtype.scalar));
+}
+uint32_t KernelBuilder::idiv(uint32_t a, int64_t c) {
+    const UOp& na = node(a);
+    if (c == 1) return a;
+    if (na.op == Op::Const) return ci(na.arg_i / c, na.dtype.scalar);
+    return binary(BinaryOp::Idiv, a, ci(c, na.dtype.scalar));
+}
+uint32_t KernelBuilder::imod(uint32_t a, int64_t c) {
+    const UOp& na = node(a);
+    if (c == 1) return ci(0, na.dtype.scalar);
+    if (na.op == Op::Const) return ci(na.arg_i % c, na.dtype.scalar);
+    return binary(BinaryOp::Mod, a, ci(c, na.dtype.scalar));
+}
+
+std::vector<uint8_t> KernelBuilder::serialize() const {
+    std::vector<uint8_t> out;
+    auto put = [&](const void* p, size_t n) {
+        const uint8_t* b = static_cast<const uint8_t*>(p);
+        out.insert(out.end(), b, b + n);
+    };
+    auto u32 = [&](uint32_t v) { put(&v, 4); };
+    auto u16 = [&](uint16_t v) { put(&v, 2); };
+    auto u8 = [&](uint8_t v) { put(&v, 1); };
+    auto i64 = [&](int64_t v) { put(&v, 8); };
+    u32(0x4C4B524Du);
+    u32(1);
+    u32(static_cast<uint32_t>(k_.nodes.size()));
+    for (const UOp& u : k_.nodes) {
+        u32(u.id);
+        u16(static_cast<uint16_t>(u.op));
+        u8(static_cast<uint8_t>(u.dtype.scalar));
+        u8(static_cast<uint8_t>((u.dtype.is_ptr ? 1 : 0) | (static_cast<int>(u.dtype.space) << 1)));
+        u16(u.dtype.vcount);
+        i64(u.dtype.ptr_size);
+        u16(static_cast<uint16_t>(u.src.size()));
+        for (uint32_t s : u.src) u32(s);
+        i64(u.arg_i);
+        put(&u.arg_f, 8);
+        u16(u.sub);
+        u16(static_cast<uint16_t>(u.str.size()));
+        put(u.str.data(), u.str.size());
+        u16(static_cast<uint16_t>(u.extra.size()));
+        for (int64_t e : u.extra) i64(e);
+    }
+    return out;
+}
+
+LinearKernel KernelBuilder::finish() {
+    std::vector<uint8_t> bytes = serialize();
+    k_.content_hash = fnv1a64(bytes.data(), bytes.size());
+    return k_;
+}
+
+// ============================================================================ matmul kernels
+LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K) {
+    KernelBuilder b;
+    const Scalar f = Scalar::Float32;
+    uint32_t c = b.param(0, f, M * N), a = b.param(1, f, M * K), bm = b.param(2, f, K * N);
+    uint32_t gx = b.special("gidx0", N / 64), gy = b.special("gidx1", M / 64);
+    uint32_t lx = b.special("lidx0", 16), ly = b.special("lidx1", 16);
+    uint32_t col0 = b.iadd(b.imul(gx, 64), b.imul(lx, 4));
+    uint32_t row0 = b.iadd(b.imul(gy, 64), b.imul(ly, 4));
+    uint32_t acc = b.define_reg(0, f, 16);
+    uint32_t zero = b.cf(0.0);
+    for (int i = 0; i < 16; i++) b.store(b.index(acc, b.ci(i)), zero);
+    uint32_t r = b.range(K, 0, AxisType::Reduce);
+    uint32_t bvec = b.load(b.index(bm, b.iadd(b.imul(r, N), col0)), 4);
+    for (int i = 0; i < 4; i++) {
+        uint32_t arow = b.iadd(row0, b.ci(i));
+        uint32_t av = b.load(b.index(a, b.iadd(b.imul(arow, K), r)));
+        for (int j = 0; j < 4; j++) {
+            uint32_t slot = b.index(acc, b.ci(i * 4 + j));
+            b.store(slot, b.mulacc(av, b.gep(bvec, j), b.load(slot)));
+        }
+    }
+    b.end({r});
+    for (int i = 0; i < 4; i++) {
+        uint32_t arow = b.iadd(row0, b.ci(i));
+        std::vector<uint32_t> vals;
+        for (int j = 0; j < 4; j++) vals.push_back(b.load(b.index(acc, b.ci(i * 4 + j))));
+        b.store(b.index(c, b.iadd(b.imul(arow, N), col0)), b.vectorize(vals));
+    }
+    return b.finish();
+}
+
+int build_wmma_matmul_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, LinearKernel* k) {
+    const int tn = tc.dims[0], tm = tc.dims[1], tk = tc.dims[2];
+    if (M % tm || N % tn || K % tk)
+        return failf(kInvalidArgument, "tensor-core matmul: shape %lldx%lldx%lld is not a multiple of the %dx%dx%d tile (PADTO is not applied here)",
+                     (long long)M, (long long)N, (long long)K, tm, tn, tk);
+    if (tc.threads != 64) return fail(kInvalidArgument, "tensor-core matmul: only 64-lane tensor cores are lowered");
+    // post-TC upcasts (heuristics.rs:787-821): first of [5,4,3,2] that divides the tile count
+    auto pick = [](int64_t tiles) {
+        for (int u : {5, 4, 3, 2})
+            if (tiles % u == 0) return u;
+        return 1;
+    };
+    const int um = pick(M / tm), un = pick(N / tn);
+    const int ea = tc.elements_per_thread[0], eb = tc.elements_per_thread[1], ec = tc.elements_per_thread[2];
+    KernelBuilder b;
+    uint32_t c = b.param(0, out, M * N), a = b.param(1, tc.dtype_in, M * K), bm = b.param(2, tc.dtype_in, K * N);
+    uint32_t gx = b.special("gidx0", N / (tn * un)), gy = b.special("gidx1", M / (tm * um));
+    uint32_t lane = b.special("lidx0", 64);  // the WARP range of tc.threads lanes (tc.rs:452-456)
+    // per-lane operand coordinates from the swizzle tables, as bit gathers of the lane id.
+    // coordinates of element 0; further elements differ only in k (checked below).
+    auto lane_expr = [&](int operand, bool want_k) -> uint32_t {
+        // value(lane) = sum over lane bits p of bit(lane, p) * contribution(p)
+        uint32_t acc_id = b.ci(0);
+        for (int p = 0; p < 6; p++) {
+            int mn, kk, mn0, kk0;
+            tc_operand_element(tc, operand, 1 << p, 0, &mn, &kk);
+            tc_operand_element(tc, operand, 0, 0, &mn0, &kk0);
+            int contrib = want_k ? kk - kk0 : mn - mn0;
+            if (!contrib) continue;
+            uint32_t bit = b.binary(BinaryOp::And, b.binary(BinaryOp::Shr, lane, b.ci(p)), b.ci(1));
+            acc_id = b.iadd(acc_id, b.imul(bit, contrib));
+        }
+        return acc_id;
+    };
+    // element e of a lane must advance k by a lane-independent amount and leave m/n alone
+    std::vector<int> a_dk(ea), b_dk(eb);
+    for (int operand = 0; operand < 2; operand++)
+        for (int e = 0; e < (operand ? eb : ea); e++) {
+            int mn, kk, mn0, kk0;
+            tc_operand_element(tc, operand, 37, e, &mn, &kk);
+            tc_operand_element(tc, operand, 37, 0, &mn0, &kk0);
+            if (mn != mn0) return fail(kInvalidArgument, "tensor-core matmul: operand elements span rows/columns");
+            (operand ? b_dk : a_dk)[e] = kk - kk0;
+        }
+    bool a_contig = true;
+    for (int e = 0; e < ea; e++) a_contig = a_contig && a_dk[e] == e;
+    uint32_t a_m = lane_expr(0, false), a_k = lane_expr(0, true);
+    uint32_t b_n = lane_expr(1, false), b_k = lane_expr(1, true);
+    // accumulator coordinates
+    uint32_t c_m = b.ci(0), c_n = b.ci(0);
+    for (int p = 0; p < 6; p++) {
+        int m, n;
+        tc_acc_element(tc, 1 << p, 0, &m, &n);
+        uint32_t bit = b.binary(BinaryOp::And, b.binary(BinaryOp::Shr, lane, b.ci(p)), b.ci(1));
+        if (m) c_m = b.iadd(c_m, b.imul(bit, m));
+        if (n) c_n = b.iadd(c_n, b.imul(bit, n));
+    }
+    uint32_t acc = b.define_reg(0, tc.dtype_out, um * un, ec);
+    {
+        std::vector<uint32_t> z(ec, b.cf(0.0, tc.dtype_out));
+        uint32_t zv = b.vectorize(z);
+        for (int i = 0; i < um * un; i++) b.store(b.index(acc, b.ci(i)), zv);
+    }
+    const std::string name = wmma_name(tc);
+    uint32_t r = b.range(K / tk, 0, AxisType::Reduce);
+    uint32_t kbase = b.imul(r, tk);
+    std::vector<uint32_t> afrag(um), bfrag(un);
+    for (int i = 0; i < um; i++) {
+        uint32_t row = b.iadd(b.iadd(b.imul(gy, tm * um), b.ci(i * tm)), a_m);
+        uint32_t base = b.iadd(b.imul(row, K), b.iadd(kbase, a_k));
+        if (a_contig) {
+            afrag[i] = b.load(b.index(a, base), ea);
+        } else {
+            std::vector<uint32_t> el;
+            for (int e = 0; e < ea; e++) el.push_back(b.load(b.index(a, b.iadd(base, b.ci(a_dk[e])))));
+            afrag[i] = b.vectorize(el);
+        }
+    }
+    for (int j = 0; j < un; j++) {
+        uint32_t col = b.iadd(b.iadd(b.imul(gx, tn * un), b.ci(j * tn)), b_n);
+        std::vector<uint32_t> el;
+        for (int e = 0; e < eb; e++) {
+            uint32_t krow = b.iadd(b.iadd(kbase, b_k), b.ci(b_dk[e]));
+            el.push_back(b.load(b.index(bm, b.iadd(b.imul(krow, N), col))));
+        }
+        bfrag[j] = b.vectorize(el);
+    }
+    for (int i = 0; i < um; i++)
+        for (int j = 0; j < un; j++) {
+            uint32_t slot = b.index(acc, b.ci(i * un + j));
+            DType cd = KernelBuilder::scalar(tc.dtype_out, ec);
+            uint32_t w = b.add(Op::Wmma, cd, {afrag[i], bfrag[j], b.load(slot)}, 0, 0, 0, name);
+            b.store(slot, w);
+        }
+    b.end({r});
+    for (int i = 0; i < um; i++)
+        for (int j = 0; j < un; j++) {
+            uint32_t res = b.load(b.index(acc, b.ci(i * un + j)));
+            for (int e = 0; e < ec; e++) {
+                int m, n, m0, n0;
+                tc_acc_element(tc, 0, e, &m, &n);
+                tc_acc_element(tc, 0, 0, &m0, &n0);
+                uint32_t row = b.iadd(b.iadd(b.imul(gy, tm * um), b.ci(i * tm + (m - m0))), c_m);
+                uint32_t col = b.iadd(b.iadd(b.imul(gx, tn * un), b.ci(j * tn + (n - n0))), c_n);
+                uint32_t v = b.gep(res, e);
+                if (out != tc.dtype_out) v = b.cast(v, out);
+                b.store(b.index(c, b.iadd(b.imul(row, N), col)), v);
+            }
+        }
+    *k = b.finish();
+    return kOk;
+}
+
+}  // namespace mrk

@@ -1,0 +1,99 @@
+"""Bindings of the scheduling helpers (capabilities, tensor cores, GPU dims, matmul kernels)."""
+import ctypes as C
+
+from ._ffi import check, lib
+from . import uop as U
+
+
+def caps():
+    """Renderer::amd_cdna4() (schedule/src/optimizer/renderer.rs:290-303) as a dict."""
+    out = {}
+    for item in lib.mrk_hip_sched_caps().decode().split(";"):
+        k, v = item.split("=", 1)
+        out[k] = v
+    out["global_max"] = [int(x) for x in out["global_max"].split(",")]
+    out["tensor_cores"] = out["tensor_cores"].split(",")
+    for k in ("has_local", "has_shared", "has_threads", "shared_max", "local_max", "upcast_max"):
+        out[k] = int(out[k])
+    return out
+
+
+def tc_select(in0, in1, acc):
+    return lib.mrk_hip_sched_tc_select(in0, in1, acc)
+
+
+def tc_info(i):
+    dims, ept, thr = (C.c_int * 3)(), (C.c_int * 3)(), C.c_int()
+    check(lib.mrk_hip_sched_tc_info(i, dims, C.byref(thr), ept))
+    return list(dims), thr.value, list(ept)
+
+
+def tc_element(i, operand, lane, elem):
+    a, b = C.c_int(), C.c_int()
+    check(lib.mrk_hip_sched_tc_operand_element(i, operand, lane, elem, C.byref(a), C.byref(b)))
+    return a.value, b.value
+
+
+def _arr(v):
+    return (C.c_size_t * max(len(v), 1))(*v)
+
+
+def _dims_call(fn, dims, max_sizes):
+    out = (C.c_size_t * 16)()
+    n = C.c_size_t()
+    rc = fn(_arr(dims), len(dims), _arr(max_sizes), len(max_sizes), out, 16, C.byref(n))
+    return rc, list(out[: n.value])
+
+
+def find_smallest_divisor(n):
+    return lib.mrk_hip_sched_find_smallest_divisor(n)
+
+
+def group_dims(dims, max_sizes):
+    rc, out = _dims_call(lib.mrk_hip_sched_group_dims, dims, max_sizes)
+    return out if rc == 1 else None
+
+
+def split_dims(dims, max_sizes):
+    return _dims_call(lib.mrk_hip_sched_split_dims, dims, max_sizes)[1]
+
+
+def limit_dims(dims, max_sizes):
+    return _dims_call(lib.mrk_hip_sched_limit_dims, dims, max_sizes)[1]
+
+
+def get_contraction(original, limited):
+    g = (C.c_size_t * max(len(original), 1))()
+    if not lib.mrk_hip_sched_get_contraction(_arr(original), len(original), _arr(limited), len(limited), g):
+        return None
+    groups = [[] for _ in limited]
+    for d in range(len(original)):
+        groups[g[d]].append(d)
+    return groups
+
+
+def grouped_dims(dims, max_sizes, reverse, raw=None):
+    launch = (C.c_size_t * 16)()
+    n = C.c_size_t()
+    idx = (C.c_size_t * max(len(dims), 1))()
+    check(lib.mrk_hip_sched_grouped_dims(_arr(dims), len(dims), _arr(max_sizes) if max_sizes else None,
+                                         len(max_sizes) if max_sizes else 0, int(reverse), launch, 16, C.byref(n),
+                                         _arr(raw) if raw is not None else None, idx if raw is not None else None))
+    return list(launch[: n.value]), (list(idx[: len(dims)]) if raw is not None else None)
+
+
+def _take(fn, *args):
+    p = C.POINTER(C.c_uint8)()
+    n = C.c_size_t()
+    check(fn(*args, C.byref(p), C.byref(n)))
+    data = C.string_at(p, n.value)
+    lib.mrk_hip_sched_free(p)
+    return data
+
+
+def build_matmul_f32(m, n, k):
+    return _take(lib.mrk_hip_sched_build_matmul_f32, m, n, k)
+
+
+def build_wmma_matmul(tc_index, m, n, k, out_scalar=U.BF16):
+    return _take(lib.mrk_hip_sched_build_wmma_matmul, tc_index, m, n, k, out_scalar)

@@ -197,3 +197,37 @@ def test_variables_positional_vals(dev):
     prog.execute([out_b], [700, (1 << 33) + 5])  # a value that needs all 64 bits
     y = out_b.copyout(np.float32)
     assert np.array_equal(y[:700], np.arange(700, dtype=np.float32) + 5) and not y[700:].any()
+
+
+@pytest.mark.parametrize("tc,shape,out", [(1, (64, 160, 128), U.BF16), (1, (16, 16, 32), U.BF16), (3, (48, 32, 64), U.BF16),
+                                          (1, (80, 48, 96), U.F32)])
+def test_tc_apply_matmul_from_tables(dev, oracle, tc, shape, out):
+    """The tensor-core matmul built from the CDNA tables (opts + swizzle) on the GPU."""
+    from morok_amd import sched
+
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 3, 10)
+    b = synth.normal_bf16((K, N), 3, 11)
+    kern = sched.build_wmma_matmul(tc, M, N, K, out)
+    np_out = np.uint16 if out == U.BF16 else np.float32
+    c = run(dev, kern, "r_tc", (M, N), np_out, [a, b])
+    ref = synth.from_bf16(a).astype(np.float64) @ synth.from_bf16(b).astype(np.float64)
+    cf = synth.from_bf16(c) if out == U.BF16 else c
+    assert np.abs(cf - ref).max() <= 2e-2 * np.abs(ref).max()
+    if out == U.F32:
+        assert np.abs(cf - ref).max() <= 1e-4 * np.abs(ref).max()
+    # one-hot rows pin the operand gather exactly
+    a1 = np.zeros((M, K), np.float32)
+    a1[np.arange(M), (np.arange(M) * 7) % K] = 1
+    c1 = run(dev, kern, "r_tc", (M, N), np_out, [synth.to_bf16(a1), b])
+    want = b[(np.arange(M) * 7) % K]
+    assert np.array_equal(c1, want if out == U.BF16 else synth.from_bf16(want))
+
+
+def test_scheduled_matmul_f32_kernel(dev, oracle):
+    from morok_amd import sched
+
+    a = synth.uniform((128, 96), 1, 5)
+    b = synth.uniform((96, 192), 1, 6)
+    c = run(dev, sched.build_matmul_f32(128, 192, 96), "r_mm", (128, 192), np.float32, [a, b])
+    assert np.array_equal(c, oracle.matmul_f32(a, b))

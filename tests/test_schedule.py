@@ -1,0 +1,139 @@
+"""Scheduling helpers without a GPU: capability descriptor, tensor-core tables and the operand
+layouts derived from them, GPU dimension limiting.  The gpudims cases restate the reference's
+own unit tests (schedule/src/gpudims.rs:644-739); the layout checks pin the CDNA swizzle
+tables (untested upstream) to the MFMA register layout measured on the hardware."""
+import itertools
+import random
+
+import pytest
+
+import morok_amd
+from morok_amd import MorokHipError, sched, uop as U
+
+
+def test_caps_match_reference_descriptor():
+    c = sched.caps()  # schedule/src/optimizer/renderer.rs:290-303
+    assert c["device"] == "AMD_CDNA4" and c["has_local"] == 1 and c["has_shared"] == 1 and c["has_threads"] == 0
+    assert c["global_max"] == [2147483647, 65535, 65535] and c["local_max"] == 1024 and c["upcast_max"] == 8
+    assert c["shared_max"] == 163840  # gfx950 LDS per workgroup (the reference lists 65536)
+    assert c["tensor_cores"][:2] == ["WMMA_16_16_32_half_float", "WMMA_16_16_32_bfloat_float"]
+    assert "WMMA_16_16_16_bfloat_float" in c["tensor_cores"]
+
+
+def test_tensor_core_selection():
+    # tc.rs:126-168: first entry whose input and accumulator dtypes match
+    assert sched.tc_select(U.BF16, U.BF16, U.F32) == 1
+    assert sched.tc_select(U.F16, U.F16, U.F32) == 0
+    assert sched.tc_select(U.F32, U.F32, U.F32) == -1
+    assert sched.tc_select(U.BF16, U.BF16, U.BF16) == -1
+    assert sched.tc_select(U.BF16, U.F16, U.F32) == -1
+    dims, threads, ept = sched.tc_info(1)
+    assert dims == [16, 16, 32] and threads == 64 and ept == [8, 8, 4]  # renderer.rs:549-558
+    dims, threads, ept = sched.tc_info(3)
+    assert dims == [16, 16, 16] and ept == [4, 4, 4]
+    with pytest.raises(MorokHipError):
+        sched.tc_info(9)
+
+
+@pytest.mark.parametrize("tc", [0, 1, 2, 3])
+def test_swizzle_tables_equal_mfma_register_layout(tc):
+    """Layout of v_mfma_f32_16x16x{16,32}: lane l holds row/column l % 16 and the contiguous k
+    group l // 16 of A/B; accumulator element i of lane l is C[4 * (l // 16) + i][l % 16].
+    (The same formulas drive the one-hot MFMA test on the GPU.)"""
+    (_, _, K), _, (ea, eb, ec) = sched.tc_info(tc)
+    per = K // 4
+    assert ea == per and eb == per
+    seen_a, seen_b, seen_c = set(), set(), set()
+    for lane in range(64):
+        for e in range(per):
+            assert sched.tc_element(tc, 0, lane, e) == (lane % 16, per * (lane // 16) + e)
+            assert sched.tc_element(tc, 1, lane, e) == (lane % 16, per * (lane // 16) + e)
+            seen_a.add(sched.tc_element(tc, 0, lane, e))
+            seen_b.add(sched.tc_element(tc, 1, lane, e))
+        for e in range(ec):
+            assert sched.tc_element(tc, 2, lane, e) == (4 * (lane // 16) + e, lane % 16)
+            seen_c.add(sched.tc_element(tc, 2, lane, e))
+    assert len(seen_a) == 16 * K and len(seen_b) == 16 * K and len(seen_c) == 256  # every element exactly once
+
+
+# ---- the reference's gpudims unit tests
+def test_group_dims_cases():
+    assert sched.group_dims([4, 4], [16, 16, 16]) == [4, 4]
+    g = sched.group_dims([4, 4, 4, 4], [256, 256, 256])
+    assert g is not None and len(g) <= 3 and g == [16, 4, 4]
+    assert sched.group_dims([8, 8, 8], [256, 256, 256]) == [8, 8, 8]
+    assert sched.group_dims([1000], [10]) is None
+
+
+def test_split_dims_and_smallest_divisor():
+    assert all(d <= 64 for d in sched.split_dims([100], [64, 64, 64]))
+    assert sched.split_dims([100], [64, 64, 64]) == [50, 2]
+    assert [sched.find_smallest_divisor(n) for n in (1, 2, 3, 4, 9, 100)] == [1, 2, 1, 2, 3, 2]
+
+
+def test_get_contraction_cases():
+    assert sched.get_contraction([2, 5, 2], [10, 2]) == [[0, 1], [2]]
+    assert sched.get_contraction([4, 4, 4], [4, 4, 4]) == [[0], [1], [2]]
+    assert sched.get_contraction([2, 3, 4], [24]) == [[0, 1, 2]]
+    assert sched.get_contraction([2, 3, 4], [5, 4]) is None
+    assert sched.get_contraction([2, 4, 3], [8, 3]) == [[0, 1], [2]]
+
+
+def test_limit_dims_under_cdna4_limits():
+    gmax = sched.caps()["global_max"]
+    assert sched.limit_dims([8192, 8192], gmax) == [8192, 8192]
+    assert sched.limit_dims([70000, 70000, 3, 5], gmax)[0] <= gmax[0]
+    out = sched.limit_dims([4, 100000, 100000], gmax)  # y would exceed 65535: must be regrouped or split
+    assert all(o <= m for o, m in zip(out, gmax)) and len(out) <= 3
+    prod = 1
+    for o in out:
+        prod *= o
+    assert prod == 4 * 100000 * 100000
+
+
+def test_grouped_dims_index_mapping_is_a_bijection():
+    """Integer/index work is bit-exact: every tuple of hardware indices maps to a distinct,
+    in-range tuple of original indices, and all of them are covered."""
+    rng = random.Random(7)
+    cases = [([2, 5, 2], [16, 2]), ([6, 4], [8, 8, 8]), ([3, 3, 3, 3], [32, 32, 32]), ([100], [64, 64, 64]),
+             ([7, 9], [63, 63]), ([12], [4, 4, 4])]
+    for _ in range(20):
+        n = rng.randint(1, 4)
+        cases.append(([rng.choice([1, 2, 3, 4, 5, 6, 8]) for _ in range(n)], [rng.choice([8, 16, 64])] * 3))
+    for dims, mx in cases:
+        for reverse in (False, True):
+            launch, _ = sched.grouped_dims(dims, mx, reverse)
+            total = 1
+            for d in dims:
+                total *= d
+            lt = 1
+            for l in launch:
+                lt *= l
+            assert lt == total, (dims, mx, launch)
+            seen = set()
+            for raw in itertools.product(*[range(l) for l in launch]):
+                _, idx = sched.grouped_dims(dims, mx, reverse, list(raw))
+                assert all(0 <= i < d for i, d in zip(idx, dims)), (dims, launch, raw, idx)
+                seen.add(tuple(idx))
+            assert len(seen) == total, (dims, mx, reverse, launch)
+    # global indices are assigned in reverse: the last (fastest) dimension gets gidx0
+    launch, idx = sched.grouped_dims([3, 5], None, True, [4, 2])
+    assert launch == [5, 3] and idx == [2, 4]
+    launch, idx = sched.grouped_dims([3, 5], None, False, [2, 4])
+    assert launch == [3, 5] and idx == [2, 4]
+
+
+def test_matmul_kernels_render_and_compile():
+    spec = U.render(sched.build_matmul_f32(128, 192, 64), "r_mm")
+    assert spec.global_size == [3, 2, 1] and spec.local_size == [16, 16, 1] and "fmaf(" in spec.src
+    morok_amd.compile_spec(spec)
+    spec = U.render(sched.build_wmma_matmul(1, 64, 160, 128), "r_tc")
+    # post-TC upcasts (heuristics.rs:787-821): M has 4 tiles -> upcast 4, N has 10 -> upcast 5
+    assert spec.global_size == [2, 1, 1] and spec.local_size == [64, 1, 1]
+    assert spec.src.count("__WMMA_16_16_32_bfloat_float(") == 20 + 1
+    morok_amd.compile_spec(spec)
+    with pytest.raises(MorokHipError) as e:
+        sched.build_wmma_matmul(1, 60, 64, 64)
+    assert "not a multiple" in e.value.message
+    morok_amd.compile_spec(U.render(sched.build_wmma_matmul(0, 32, 32, 64, U.F16), "r_tc16"))
+    morok_amd.compile_spec(U.render(sched.build_wmma_matmul(2, 32, 32, 64, U.F32), "r_tc16k16"))
