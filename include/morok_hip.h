@@ -349,6 +349,75 @@ int mrk_hip_event_synchronize(mrk_event* e);
 int mrk_hip_event_elapsed_ms(mrk_event* start, mrk_event* stop, float* ms);
 void mrk_hip_event_destroy(mrk_event* e);
 
+/* =====================================================================================
+ * Lazy tensors: the caller side of the boundary.  Ops build a graph; realize splits it into
+ * kernels (a reduce is a kernel boundary, movement ops become index arithmetic), obtains each
+ * through the kernel cache and runs them as one execution plan
+ * (tensor/src/realize.rs:83-127,299-357,937-1117).  With fusion on (the default) the composed
+ * graphs of softmax / matmul / scaled_dot_product_attention run as the hand-written kernels
+ * when dtype and layout qualify; with fusion off every op runs through generated kernels.
+ * dtype and op tags are those of the linearized-kernel wire format (morok_amd/csrc/uop.h).
+ * Every constructor returns a new handle the caller releases; handles are immutable.
+ * ===================================================================================== */
+typedef struct mrk_tensor mrk_tensor;
+/* Tensor::from_raw_bytes / from_slice (tensor/src/data.rs:23-96): data is copied to the device
+ * at creation; nbytes must equal numel * sizeof(dtype) (MRK_ERR_SIZE_MISMATCH otherwise). */
+int mrk_hip_tensor_from_bytes(int device_id, const void* data, size_t nbytes, const int64_t* shape, size_t ndim,
+                              int dtype, mrk_tensor** out);
+/* Wraps an existing device buffer (shared, not copied). */
+int mrk_hip_tensor_from_buffer(const mrk_buffer* b, const int64_t* shape, size_t ndim, int dtype, mrk_tensor** out);
+int mrk_hip_tensor_const(int device_id, double value, int dtype, mrk_tensor** out);          /* lib.rs:432 */
+int mrk_hip_tensor_full(int device_id, const int64_t* shape, size_t ndim, double value, int dtype,
+                        mrk_tensor** out);                                                    /* lib.rs:251 */
+void mrk_hip_tensor_release(mrk_tensor* t);
+size_t mrk_hip_tensor_ndim(const mrk_tensor* t);
+int mrk_hip_tensor_shape(const mrk_tensor* t, int64_t* shape_out, size_t capacity);
+int mrk_hip_tensor_dtype(const mrk_tensor* t);
+/* movement */
+int mrk_hip_tensor_reshape(const mrk_tensor* t, const int64_t* shape, size_t ndim, mrk_tensor** out);
+int mrk_hip_tensor_permute(const mrk_tensor* t, const int64_t* perm, size_t ndim, mrk_tensor** out);
+int mrk_hip_tensor_transpose(const mrk_tensor* t, int64_t a, int64_t b, mrk_tensor** out);
+int mrk_hip_tensor_expand(const mrk_tensor* t, const int64_t* shape, size_t ndim, mrk_tensor** out);
+int mrk_hip_tensor_shrink(const mrk_tensor* t, const int64_t* begin, const int64_t* end, size_t ndim,
+                          mrk_tensor** out);
+int mrk_hip_tensor_contiguous(const mrk_tensor* t, mrk_tensor** out);                         /* lib.rs:548 */
+int mrk_hip_tensor_cat(const mrk_tensor* const* parts, size_t nparts, int64_t axis, mrk_tensor** out);
+/* elementwise, with broadcasting and dtype promotion (dtype/src/cast.rs:88) */
+int mrk_hip_tensor_cast(const mrk_tensor* t, int dtype, mrk_tensor** out);                    /* lib.rs:495 */
+int mrk_hip_tensor_unary(const mrk_tensor* t, int unary_op, mrk_tensor** out);
+int mrk_hip_tensor_binary(const mrk_tensor* a, int binary_op, const mrk_tensor* b, mrk_tensor** out);
+/* cond ? a : b */
+int mrk_hip_tensor_where(const mrk_tensor* cond, const mrk_tensor* a, const mrk_tensor* b, mrk_tensor** out);
+int mrk_hip_tensor_sigmoid(const mrk_tensor* t, mrk_tensor** out);                            /* activation.rs:42-52 */
+int mrk_hip_tensor_silu(const mrk_tensor* t, mrk_tensor** out);                               /* activation.rs:309-318 */
+/* reductions (reduce.rs:620-692); promote != 0 accumulates half types in f32 and small ints
+ * in 32 bits (reduce.rs:101-117) */
+int mrk_hip_tensor_reduce(const mrk_tensor* t, int reduce_op, const int64_t* axes, size_t naxes, int keepdim,
+                          int promote, mrk_tensor** out);
+int mrk_hip_tensor_mean(const mrk_tensor* t, const int64_t* axes, size_t naxes, int keepdim, mrk_tensor** out);
+/* composite ops of the hot path */
+int mrk_hip_tensor_matmul(const mrk_tensor* a, const mrk_tensor* b, mrk_tensor** out);        /* matmul.rs:82-110 */
+int mrk_hip_tensor_softmax(const mrk_tensor* t, int64_t axis, mrk_tensor** out);              /* activation.rs:90-101 */
+int mrk_hip_tensor_rms_norm(const mrk_tensor* t, int64_t axis, double eps, mrk_tensor** out); /* nn/norm.rs:92-111 */
+int mrk_hip_tensor_embedding(const mrk_tensor* weight, const mrk_tensor* indices, mrk_tensor** out); /* transformer.rs:12-25 */
+int mrk_hip_tensor_rotary(const mrk_tensor* x, const mrk_tensor* cos, const mrk_tensor* sin, int interleaved,
+                          mrk_tensor** out);                                                  /* transformer.rs:32-69 */
+/* scale <= 0 selects 1/sqrt(head_dim) (transformer.rs:90-91) */
+int mrk_hip_tensor_sdpa(const mrk_tensor* q, const mrk_tensor* k, const mrk_tensor* v, double scale, int is_causal,
+                        mrk_tensor** out);                                                    /* transformer.rs:78-137 */
+/* realization (realize.rs:83-127) and extraction (data.rs:211-236) */
+int mrk_hip_tensor_realize(const mrk_tensor* t);
+int mrk_hip_tensor_to_bytes(const mrk_tensor* t, void* dst, size_t nbytes);
+/* Device buffer of a realized tensor (new handle sharing the allocation). */
+int mrk_hip_tensor_buffer(const mrk_tensor* t, mrk_buffer** out);
+/* Per-thread: hand-written fused kernels on/off; what the last realize on this thread ran
+ * (Tensor::kernels(), tensor/src/lib.rs:213). */
+void mrk_hip_tensor_set_fusion(int enabled);
+size_t mrk_hip_tensor_last_kernel_count(void);
+const char* mrk_hip_tensor_last_kernel_name(size_t i);
+size_t mrk_hip_tensor_last_cached_count(void);
+double mrk_hip_tensor_last_elapsed_ms(void);
+
 #ifdef __cplusplus
 }
 #endif

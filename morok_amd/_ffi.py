@@ -148,6 +148,44 @@ _SIGS = {
     "mrk_hip_event_synchronize": (C.c_int, [C.c_void_p]),
     "mrk_hip_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "mrk_hip_event_destroy": (None, [C.c_void_p]),
+    # lazy tensors
+    "mrk_hip_tensor_from_bytes": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_from_buffer": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_const": (C.c_int, [C.c_int, C.c_double, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_full": (C.c_int, [C.c_int, c_i64_p, C.c_size_t, C.c_double, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_release": (None, [C.c_void_p]),
+    "mrk_hip_tensor_ndim": (C.c_size_t, [C.c_void_p]),
+    "mrk_hip_tensor_shape": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t]),
+    "mrk_hip_tensor_dtype": (C.c_int, [C.c_void_p]),
+    "mrk_hip_tensor_reshape": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t, c_void_pp]),
+    "mrk_hip_tensor_permute": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t, c_void_pp]),
+    "mrk_hip_tensor_transpose": (C.c_int, [C.c_void_p, C.c_int64, C.c_int64, c_void_pp]),
+    "mrk_hip_tensor_expand": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t, c_void_pp]),
+    "mrk_hip_tensor_shrink": (C.c_int, [C.c_void_p, c_i64_p, c_i64_p, C.c_size_t, c_void_pp]),
+    "mrk_hip_tensor_contiguous": (C.c_int, [C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_cat": (C.c_int, [c_void_pp, C.c_size_t, C.c_int64, c_void_pp]),
+    "mrk_hip_tensor_cast": (C.c_int, [C.c_void_p, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_unary": (C.c_int, [C.c_void_p, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_binary": (C.c_int, [C.c_void_p, C.c_int, C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_where": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_sigmoid": (C.c_int, [C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_silu": (C.c_int, [C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_reduce": (C.c_int, [C.c_void_p, C.c_int, c_i64_p, C.c_size_t, C.c_int, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_mean": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_matmul": (C.c_int, [C.c_void_p, C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_softmax": (C.c_int, [C.c_void_p, C.c_int64, c_void_pp]),
+    "mrk_hip_tensor_rms_norm": (C.c_int, [C.c_void_p, C.c_int64, C.c_double, c_void_pp]),
+    "mrk_hip_tensor_embedding": (C.c_int, [C.c_void_p, C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_rotary": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_sdpa": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_double, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_realize": (C.c_int, [C.c_void_p]),
+    "mrk_hip_tensor_to_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
+    "mrk_hip_tensor_buffer": (C.c_int, [C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_set_fusion": (None, [C.c_int]),
+    "mrk_hip_tensor_last_kernel_count": (C.c_size_t, []),
+    "mrk_hip_tensor_last_kernel_name": (C.c_char_p, [C.c_size_t]),
+    "mrk_hip_tensor_last_cached_count": (C.c_size_t, []),
+    "mrk_hip_tensor_last_elapsed_ms": (C.c_double, []),
 }
 
 

@@ -10,6 +10,7 @@
 #include "kernels/kernels.h"
 #include "runtime.h"
 #include "schedule.h"
+#include "tensor.h"
 #include "uop.h"
 
 using namespace mrk;
@@ -34,6 +35,9 @@ struct mrk_plan {
 };
 struct mrk_signal {
     std::unique_ptr<TimelineSignal> s;
+};
+struct mrk_tensor {
+    Tensor t;
 };
 struct mrk_event {
     int device_id;
@@ -735,5 +739,195 @@ void mrk_hip_event_destroy(mrk_event* e) {
     ffi::event_destroy(e->e);
     delete e;
 }
+
+// ---- lazy tensors
+namespace {
+int wrap_tensor(Tensor t, mrk_tensor** out) {
+    if (!t.valid()) return last_status() != kOk ? last_status() : fail(kInvalidArgument, "invalid tensor operand");
+    *out = new mrk_tensor{std::move(t)};
+    return kOk;
+}
+std::vector<int64_t> vec64(const int64_t* p, size_t n) { return p ? std::vector<int64_t>(p, p + n) : std::vector<int64_t>(); }
+bool scalar_ok(int dtype) { return dtype >= 0 && dtype <= static_cast<int>(Scalar::Float64); }
+}  // namespace
+#define MRK_DTYPE(d)                                                             \
+    do {                                                                         \
+        if (!scalar_ok(d)) return fail(kInvalidArgument, "unknown dtype tag");   \
+    } while (0)
+
+int mrk_hip_tensor_from_bytes(int device_id, const void* data, size_t nbytes, const int64_t* shape, size_t ndim,
+                              int dtype, mrk_tensor** out) {
+    MRK_NONNULL(out);
+    MRK_DTYPE(dtype);
+    if (nbytes) MRK_NONNULL(data);
+    clear_error();
+    return wrap_tensor(Tensor::from_raw_bytes(device_id, data, nbytes, vec64(shape, ndim), static_cast<Scalar>(dtype)), out);
+}
+int mrk_hip_tensor_from_buffer(const mrk_buffer* b, const int64_t* shape, size_t ndim, int dtype, mrk_tensor** out) {
+    MRK_NONNULL(b);
+    MRK_NONNULL(out);
+    MRK_DTYPE(dtype);
+    clear_error();
+    return wrap_tensor(Tensor::from_buffer(std::make_shared<Buffer>(*b->b), vec64(shape, ndim), static_cast<Scalar>(dtype)), out);
+}
+int mrk_hip_tensor_const(int device_id, double value, int dtype, mrk_tensor** out) {
+    MRK_NONNULL(out);
+    MRK_DTYPE(dtype);
+    clear_error();
+    return wrap_tensor(Tensor::const_(value, static_cast<Scalar>(dtype), device_id), out);
+}
+int mrk_hip_tensor_full(int device_id, const int64_t* shape, size_t ndim, double value, int dtype, mrk_tensor** out) {
+    MRK_NONNULL(out);
+    MRK_DTYPE(dtype);
+    clear_error();
+    return wrap_tensor(Tensor::full(vec64(shape, ndim), value, static_cast<Scalar>(dtype), device_id), out);
+}
+void mrk_hip_tensor_release(mrk_tensor* t) { delete t; }
+size_t mrk_hip_tensor_ndim(const mrk_tensor* t) { return t ? static_cast<size_t>(t->t.ndim()) : 0; }
+int mrk_hip_tensor_shape(const mrk_tensor* t, int64_t* shape_out, size_t capacity) {
+    MRK_NONNULL(t);
+    if (capacity < t->t.shape().size()) return fail(kInvalidArgument, "shape buffer too small");
+    for (size_t i = 0; i < t->t.shape().size(); i++) shape_out[i] = t->t.shape()[i];
+    return kOk;
+}
+int mrk_hip_tensor_dtype(const mrk_tensor* t) { return t ? static_cast<int>(t->t.dtype()) : -1; }
+
+#define MRK_T1(t)       \
+    MRK_NONNULL(t);     \
+    MRK_NONNULL(out);   \
+    clear_error()
+
+int mrk_hip_tensor_reshape(const mrk_tensor* t, const int64_t* shape, size_t ndim, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.try_reshape(vec64(shape, ndim)), out);
+}
+int mrk_hip_tensor_permute(const mrk_tensor* t, const int64_t* perm, size_t ndim, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.try_permute(vec64(perm, ndim)), out);
+}
+int mrk_hip_tensor_transpose(const mrk_tensor* t, int64_t a, int64_t b, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.try_transpose(a, b), out);
+}
+int mrk_hip_tensor_expand(const mrk_tensor* t, const int64_t* shape, size_t ndim, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.try_expand(vec64(shape, ndim)), out);
+}
+int mrk_hip_tensor_shrink(const mrk_tensor* t, const int64_t* begin, const int64_t* end, size_t ndim, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.try_shrink(vec64(begin, ndim), vec64(end, ndim)), out);
+}
+int mrk_hip_tensor_contiguous(const mrk_tensor* t, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.contiguous(), out);
+}
+int mrk_hip_tensor_cat(const mrk_tensor* const* parts, size_t nparts, int64_t axis, mrk_tensor** out) {
+    MRK_NONNULL(parts);
+    MRK_NONNULL(out);
+    clear_error();
+    std::vector<Tensor> ts;
+    for (size_t i = 0; i < nparts; i++) {
+        MRK_NONNULL(parts[i]);
+        ts.push_back(parts[i]->t);
+    }
+    return wrap_tensor(Tensor::cat(ts, axis), out);
+}
+int mrk_hip_tensor_cast(const mrk_tensor* t, int dtype, mrk_tensor** out) {
+    MRK_T1(t);
+    MRK_DTYPE(dtype);
+    return wrap_tensor(t->t.cast(static_cast<Scalar>(dtype)), out);
+}
+int mrk_hip_tensor_unary(const mrk_tensor* t, int unary_op, mrk_tensor** out) {
+    MRK_T1(t);
+    if (unary_op < 0 || unary_op > static_cast<int>(UnaryOp::Not)) return fail(kInvalidArgument, "unknown unary op tag");
+    return wrap_tensor(t->t.unary(static_cast<UnaryOp>(unary_op)), out);
+}
+int mrk_hip_tensor_binary(const mrk_tensor* a, int binary_op, const mrk_tensor* b, mrk_tensor** out) {
+    MRK_T1(a);
+    MRK_NONNULL(b);
+    if (binary_op < 0 || binary_op > static_cast<int>(BinaryOp::Ne)) return fail(kInvalidArgument, "unknown binary op tag");
+    return wrap_tensor(a->t.binary(static_cast<BinaryOp>(binary_op), b->t), out);
+}
+int mrk_hip_tensor_where(const mrk_tensor* cond, const mrk_tensor* a, const mrk_tensor* b, mrk_tensor** out) {
+    MRK_T1(cond);
+    MRK_NONNULL(a);
+    MRK_NONNULL(b);
+    return wrap_tensor(a->t.where_(cond->t, b->t), out);
+}
+int mrk_hip_tensor_sigmoid(const mrk_tensor* t, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.sigmoid(), out);
+}
+int mrk_hip_tensor_silu(const mrk_tensor* t, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.silu(), out);
+}
+int mrk_hip_tensor_reduce(const mrk_tensor* t, int reduce_op, const int64_t* axes, size_t naxes, int keepdim, int promote,
+                          mrk_tensor** out) {
+    MRK_T1(t);
+    if (reduce_op < 0 || reduce_op > static_cast<int>(ReduceOp::Min)) return fail(kInvalidArgument, "unknown reduce op tag");
+    return wrap_tensor(t->t.reduce(static_cast<ReduceOp>(reduce_op), vec64(axes, naxes), keepdim != 0, promote != 0), out);
+}
+int mrk_hip_tensor_mean(const mrk_tensor* t, const int64_t* axes, size_t naxes, int keepdim, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.mean(vec64(axes, naxes), keepdim != 0), out);
+}
+int mrk_hip_tensor_matmul(const mrk_tensor* a, const mrk_tensor* b, mrk_tensor** out) {
+    MRK_T1(a);
+    MRK_NONNULL(b);
+    return wrap_tensor(a->t.matmul(b->t), out);
+}
+int mrk_hip_tensor_softmax(const mrk_tensor* t, int64_t axis, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.softmax(axis), out);
+}
+int mrk_hip_tensor_rms_norm(const mrk_tensor* t, int64_t axis, double eps, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.rms_norm(axis, eps), out);
+}
+int mrk_hip_tensor_embedding(const mrk_tensor* weight, const mrk_tensor* indices, mrk_tensor** out) {
+    MRK_T1(weight);
+    MRK_NONNULL(indices);
+    return wrap_tensor(weight->t.embedding(indices->t), out);
+}
+int mrk_hip_tensor_rotary(const mrk_tensor* x, const mrk_tensor* cos, const mrk_tensor* sin, int interleaved,
+                          mrk_tensor** out) {
+    MRK_T1(x);
+    MRK_NONNULL(cos);
+    MRK_NONNULL(sin);
+    return wrap_tensor(x->t.apply_rotary_emb(cos->t, sin->t, interleaved != 0), out);
+}
+int mrk_hip_tensor_sdpa(const mrk_tensor* q, const mrk_tensor* k, const mrk_tensor* v, double scale, int is_causal,
+                        mrk_tensor** out) {
+    MRK_T1(q);
+    MRK_NONNULL(k);
+    MRK_NONNULL(v);
+    return wrap_tensor(q->t.scaled_dot_product_attention(k->t, v->t, scale, is_causal != 0), out);
+}
+int mrk_hip_tensor_realize(const mrk_tensor* t) {
+    MRK_NONNULL(t);
+    return t->t.realize();
+}
+int mrk_hip_tensor_to_bytes(const mrk_tensor* t, void* dst, size_t nbytes) {
+    MRK_NONNULL(t);
+    if (nbytes) MRK_NONNULL(dst);
+    return t->t.to_bytes(dst, nbytes);
+}
+int mrk_hip_tensor_buffer(const mrk_tensor* t, mrk_buffer** out) {
+    MRK_NONNULL(t);
+    MRK_NONNULL(out);
+    auto b = t->t.buffer();
+    if (!b) return fail(kInvalidArgument, "tensor is not realized");
+    *out = new mrk_buffer{std::unique_ptr<Buffer>(new Buffer(*b))};
+    return kOk;
+}
+void mrk_hip_tensor_set_fusion(int enabled) { set_fusion_enabled(enabled != 0); }
+size_t mrk_hip_tensor_last_kernel_count(void) { return last_realize_stats().kernel_names.size(); }
+const char* mrk_hip_tensor_last_kernel_name(size_t i) {
+    const auto& n = last_realize_stats().kernel_names;
+    return i < n.size() ? n[i].c_str() : nullptr;
+}
+size_t mrk_hip_tensor_last_cached_count(void) { return last_realize_stats().cached_kernels; }
+double mrk_hip_tensor_last_elapsed_ms(void) { return last_realize_stats().elapsed_ms; }
 
 }  // extern "C"

@@ -8,9 +8,11 @@
 namespace mrk {
 
 static thread_local std::string g_last_error;
+static thread_local int g_last_status = 0;
 
 int fail(Status code, const std::string& msg) {
     g_last_error = msg;
+    g_last_status = static_cast<int>(code);
     return static_cast<int>(code);
 }
 
@@ -21,6 +23,7 @@ int failf(Status code, const char* fmt, ...) {
     vsnprintf(buf, sizeof(buf), fmt, ap);
     va_end(ap);
     g_last_error = buf;
+    g_last_status = static_cast<int>(code);
     return static_cast<int>(code);
 }
 
@@ -32,6 +35,10 @@ int fail_hip(int hip_code, const char* what) {
 }
 
 const char* last_error() { return g_last_error.c_str(); }
-void clear_error() { g_last_error.clear(); }
+int last_status() { return g_last_status; }
+void clear_error() {
+    g_last_error.clear();
+    g_last_status = 0;
+}
 
 }  // namespace mrk

@@ -33,6 +33,8 @@ int failf(Status code, const char* fmt, ...) __attribute__((format(printf, 2, 3)
 // Maps a hipError_t-like integer from the FFI layer to kHipError with the error's name.
 int fail_hip(int hip_code, const char* what);
 const char* last_error();
+// Status of the most recent fail*() on this thread since clear_error() (0 if none).
+int last_status();
 void clear_error();
 
 }  // namespace mrk

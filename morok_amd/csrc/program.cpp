@@ -104,7 +104,9 @@ int create_module_program(int device_id, ffi::Stream stream, const CompiledSpec&
     int rc = ffi::module_get_function(&f, m, spec.name.c_str());
     if (rc != 0) {
         ffi::module_unload(m);
-        return fail_hip(rc, "hipModuleGetFunction");
+        ffi::clear_last_error();
+        return failf(kHipError, "HIP error: hipModuleGetFunction failed for entry point '%s': %s (%d)", spec.name.c_str(),
+                     ffi::error_name(rc), rc);
     }
     out->reset(new ModuleProgram(device_id, stream, m, f, spec));
     return kOk;

@@ -1,0 +1,985 @@
+#include "tensor.h"
+
+#include <algorithm>
+#include <chrono>
+#include <cmath>
+#include <cstring>
+#include <map>
+#include <set>
+#include <unordered_map>
+
+#include "builtin.h"
+#include "device.h"
+#include "error.h"
+#include "runtime.h"
+#include "schedule.h"
+
+namespace mrk {
+
+// ============================================================================ small helpers
+size_t scalar_size(Scalar s) {
+    switch (s) {
+        case Scalar::Bool:
+        case Scalar::Int8:
+        case Scalar::UInt8: return 1;
+        case Scalar::Int16:
+        case Scalar::UInt16:
+        case Scalar::Float16:
+        case Scalar::BFloat16: return 2;
+        case Scalar::Int32:
+        case Scalar::UInt32:
+        case Scalar::Float32: return 4;
+        case Scalar::Void: return 0;
+        default: return 8;
+    }
+}
+
+static bool is_float(Scalar s) {
+    return s == Scalar::Float16 || s == Scalar::BFloat16 || s == Scalar::Float32 || s == Scalar::Float64;
+}
+static bool is_half(Scalar s) { return s == Scalar::Float16 || s == Scalar::BFloat16; }
+
+// dtype/src/cast.rs:88: the smallest type both promote to (restricted to the types used here)
+Scalar least_upper_dtype(Scalar a, Scalar b) {
+    if (a == b) return a;
+    auto frank = [](Scalar s) {
+        switch (s) {
+            case Scalar::Float16:
+            case Scalar::BFloat16: return 1;
+            case Scalar::Float32: return 2;
+            case Scalar::Float64: return 3;
+            default: return 0;
+        }
+    };
+    if (is_float(a) && is_float(b)) {
+        if (frank(a) == 1 && frank(b) == 1) return Scalar::Float32;  // half with bfloat16
+        return frank(a) > frank(b) ? a : b;
+    }
+    if (is_float(a)) return a;
+    if (is_float(b)) return b;
+    auto irank = [](Scalar s) {
+        switch (s) {
+            case Scalar::Bool: return 0;
+            case Scalar::Int8:
+            case Scalar::UInt8: return 1;
+            case Scalar::Int16:
+            case Scalar::UInt16: return 2;
+            case Scalar::Int32:
+            case Scalar::UInt32: return 3;
+            default: return 4;
+        }
+    };
+    return irank(a) >= irank(b) ? a : b;
+}
+
+static thread_local bool g_fusion = true;
+static thread_local RealizeStats g_stats;
+void set_fusion_enabled(bool on) { g_fusion = on; }
+bool fusion_enabled() { return g_fusion; }
+const RealizeStats& last_realize_stats() { return g_stats; }
+
+static Tensor bad(Status code, const std::string& msg) {
+    fail(code, msg);
+    return Tensor();
+}
+static std::string shape_str(const std::vector<int64_t>& s) {
+    std::string r = "[";
+    for (size_t i = 0; i < s.size(); i++) r += (i ? ", " : "") + std::to_string(s[i]);
+    return r + "]";
+}
+static TensorRef mk(TKind kind, Scalar dt, std::vector<int64_t> shape, std::vector<TensorRef> src, int dev) {
+    auto n = std::make_shared<TensorNode>();
+    n->kind = kind;
+    n->dtype = dt;
+    n->shape = std::move(shape);
+    n->src = std::move(src);
+    n->device_id = dev;
+    return n;
+}
+static bool norm_axis(int64_t* a, int64_t nd) {
+    if (*a < 0) *a += nd;
+    return *a >= 0 && *a < nd;
+}
+
+// ============================================================================ graph building
+Tensor Tensor::from_raw_bytes(int device_id, const void* data, size_t nbytes, const std::vector<int64_t>& shape,
+                              Scalar dtype) {
+    int64_t numel = 1;
+    for (int64_t d : shape) {
+        if (d < 0) return bad(kInvalidArgument, "from_raw_bytes: negative dimension");
+        numel *= d;
+    }
+    const size_t expected = static_cast<size_t>(numel) * scalar_size(dtype);
+    if (nbytes != expected)  // data.rs:81-96
+        return bad(kSizeMismatch, "from_raw_bytes: data length " + std::to_string(nbytes) + " != expected " +
+                                      std::to_string(expected) + " (" + std::to_string(numel) + " elements * " +
+                                      std::to_string(scalar_size(dtype)) + " bytes)");
+    std::shared_ptr<Device> dev;
+    if (DeviceFactoryRegistry::global().device("HIP", device_id, &dev) != kOk) return Tensor();
+    BufferOptions opt;
+    auto buf = std::make_shared<Buffer>(dev->allocator, expected, opt);
+    if (buf->copyin(data, expected) != kOk) return Tensor();  // data.rs:66-67: copied at creation
+    return from_buffer(buf, shape, dtype);
+}
+
+Tensor Tensor::from_buffer(std::shared_ptr<Buffer> buf, const std::vector<int64_t>& shape, Scalar dtype) {
+    int64_t numel = 1;
+    for (int64_t d : shape) numel *= d;
+    if (static_cast<size_t>(numel) * scalar_size(dtype) != buf->size())
+        return bad(kSizeMismatch, "from_buffer: buffer size does not match shape " + shape_str(shape));
+    auto n = mk(TKind::Buffer, dtype, shape, {}, buf->device_id());
+    n->buffer = std::move(buf);
+    return Tensor(n);
+}
+
+Tensor Tensor::const_(double value, Scalar dtype, int device_id) {
+    auto n = mk(TKind::Const, dtype, {}, {}, device_id);
+    n->cval = value;
+    return Tensor(n);
+}
+
+Tensor Tensor::full(const std::vector<int64_t>& shape, double value, Scalar dtype, int device_id) {
+    std::vector<int64_t> ones(shape.size(), 1);
+    return const_(value, dtype, device_id).try_reshape(ones).try_expand(shape);
+}
+
+Tensor Tensor::try_reshape(const std::vector<int64_t>& shape_in) const {
+    if (!n_) return Tensor();
+    std::vector<int64_t> shape = shape_in;
+    int64_t known = 1, infer = -1;
+    for (size_t i = 0; i < shape.size(); i++) {
+        if (shape[i] == -1) {
+            if (infer >= 0) return bad(kInvalidArgument, "reshape: more than one -1");
+            infer = static_cast<int64_t>(i);
+        } else if (shape[i] < 0) {
+            return bad(kInvalidArgument, "reshape: negative dimension");
+        } else {
+            known *= shape[i];
+        }
+    }
+    const int64_t numel = n_->numel();
+    if (infer >= 0) {
+        if (known == 0 || numel % known) return bad(kInvalidArgument, "reshape: cannot infer dimension");
+        shape[infer] = numel / known;
+        known *= shape[infer];
+    }
+    if (known != numel)
+        return bad(kInvalidArgument, "reshape: " + shape_str(n_->shape) + " -> " + shape_str(shape) + " changes the element count");
+    if (shape == n_->shape) return *this;
+    return Tensor(mk(TKind::Reshape, n_->dtype, shape, {n_}, n_->device_id));
+}
+
+Tensor Tensor::try_permute(const std::vector<int64_t>& perm_in) const {
+    if (!n_) return Tensor();
+    const int64_t nd = ndim();
+    std::vector<int64_t> perm = perm_in, shape(perm.size());
+    if (static_cast<int64_t>(perm.size()) != nd) return bad(kInvalidArgument, "permute: wrong number of axes");
+    std::vector<bool> seen(nd, false);
+    for (int64_t i = 0; i < nd; i++) {
+        if (!norm_axis(&perm[i], nd) || seen[perm[i]]) return bad(kInvalidArgument, "permute: invalid permutation");
+        seen[perm[i]] = true;
+        shape[i] = n_->shape[perm[i]];
+    }
+    auto n = mk(TKind::Permute, n_->dtype, shape, {n_}, n_->device_id);
+    n->arg = perm;
+    return Tensor(n);
+}
+
+Tensor Tensor::try_transpose(int64_t a, int64_t b) const {
+    if (!n_) return Tensor();
+    const int64_t nd = ndim();
+    if (!norm_axis(&a, nd) || !norm_axis(&b, nd)) return bad(kInvalidArgument, "transpose: axis out of range");
+    std::vector<int64_t> perm(nd);
+    for (int64_t i = 0; i < nd; i++) perm[i] = i;
+    std::swap(perm[a], perm[b]);
+    return try_permute(perm);
+}
+
+Tensor Tensor::try_expand(const std::vector<int64_t>& shape_in) const {
+    if (!n_) return Tensor();
+    if (shape_in.size() != n_->shape.size()) return bad(kInvalidArgument, "expand: rank mismatch");
+    std::vector<int64_t> shape = shape_in;
+    for (size_t i = 0; i < shape.size(); i++) {
+        if (shape[i] == -1) shape[i] = n_->shape[i];
+        if (shape[i] != n_->shape[i] && n_->shape[i] != 1)
+            return bad(kInvalidArgument, "expand: " + shape_str(n_->shape) + " cannot broadcast to " + shape_str(shape));
+    }
+    if (shape == n_->shape) return *this;
+    return Tensor(mk(TKind::Expand, n_->dtype, shape, {n_}, n_->device_id));
+}
+
+Tensor Tensor::try_shrink(const std::vector<int64_t>& begin, const std::vector<int64_t>& end) const {
+    if (!n_) return Tensor();
+    if (begin.size() != n_->shape.size() || end.size() != begin.size()) return bad(kInvalidArgument, "shrink: rank mismatch");
+    std::vector<int64_t> shape(begin.size());
+    for (size_t i = 0; i < begin.size(); i++) {
+        if (begin[i] < 0 || end[i] > n_->shape[i] || begin[i] > end[i]) return bad(kInvalidArgument, "shrink: range out of bounds");
+        shape[i] = end[i] - begin[i];
+    }
+    auto n = mk(TKind::Shrink, n_->dtype, shape, {n_}, n_->device_id);
+    n->arg = begin;
+    return Tensor(n);
+}
+
+Tensor Tensor::try_unsqueeze(int64_t axis) const {
+    if (!n_) return Tensor();
+    int64_t nd = ndim() + 1;
+    if (!norm_axis(&axis, nd)) return bad(kInvalidArgument, "unsqueeze: axis out of range");
+    std::vector<int64_t> shape = n_->shape;
+    shape.insert(shape.begin() + axis, 1);
+    return try_reshape(shape);
+}
+
+Tensor Tensor::try_squeeze(int64_t axis) const {
+    if (!n_) return Tensor();
+    if (!norm_axis(&axis, ndim()) || n_->shape[axis] != 1) return bad(kInvalidArgument, "squeeze: axis is not of size 1");
+    std::vector<int64_t> shape = n_->shape;
+    shape.erase(shape.begin() + axis);
+    return try_reshape(shape);
+}
+
+Tensor Tensor::contiguous() const {
+    if (!n_) return Tensor();
+    if (n_->kind == TKind::Buffer || n_->kind == TKind::Contiguous) return *this;
+    return Tensor(mk(TKind::Contiguous, n_->dtype, n_->shape, {n_}, n_->device_id));
+}
+
+Tensor Tensor::cat(const std::vector<Tensor>& parts, int64_t axis) {
+    if (parts.empty()) return bad(kInvalidArgument, "cat: no tensors");
+    for (const Tensor& p : parts)
+        if (!p.valid()) return Tensor();
+    const int64_t nd = parts[0].ndim();
+    if (!norm_axis(&axis, nd)) return bad(kInvalidArgument, "cat: axis out of range");
+    std::vector<int64_t> shape = parts[0].shape();
+    std::vector<TensorRef> src;
+    int64_t total = 0;
+    for (const Tensor& p : parts) {
+        if (p.ndim() != nd || p.dtype() != parts[0].dtype()) return bad(kInvalidArgument, "cat: rank or dtype mismatch");
+        for (int64_t i = 0; i < nd; i++)
+            if (i != axis && p.shape()[i] != shape[i]) return bad(kInvalidArgument, "cat: shape mismatch");
+        total += p.shape()[axis];
+        src.push_back(p.node());
+    }
+    shape[axis] = total;
+    auto n = mk(TKind::Cat, parts[0].dtype(), shape, src, parts[0].node()->device_id);
+    n->arg = {axis};
+    return Tensor(n);
+}
+
+Tensor Tensor::cast(Scalar dtype) const {
+    if (!n_) return Tensor();
+    if (dtype == n_->dtype) return *this;
+    return Tensor(mk(TKind::Cast, dtype, n_->shape, {n_}, n_->device_id));
+}
+
+Tensor Tensor::unary(UnaryOp op) const {
+    if (!n_) return Tensor();
+    auto n = mk(TKind::Unary, n_->dtype, n_->shape, {n_}, n_->device_id);
+    n->sub = static_cast<uint16_t>(op);
+    return Tensor(n);
+}
+
+// numpy-style broadcast of `t` to `shape` (explicit reshape + expand nodes, as the reference's
+// binary ops insert them)
+static Tensor broadcast_to(const Tensor& t, const std::vector<int64_t>& shape) {
+    std::vector<int64_t> padded(shape.size() - t.shape().size(), 1);
+    padded.insert(padded.end(), t.shape().begin(), t.shape().end());
+    return t.try_reshape(padded).try_expand(shape);
+}
+static bool broadcast_shape(const std::vector<int64_t>& a, const std::vector<int64_t>& b, std::vector<int64_t>* out) {
+    size_t n = std::max(a.size(), b.size());
+    out->assign(n, 1);
+    for (size_t i = 0; i < n; i++) {
+        int64_t da = i < n - a.size() ? 1 : a[i - (n - a.size())];
+        int64_t db = i < n - b.size() ? 1 : b[i - (n - b.size())];
+        if (da != db && da != 1 && db != 1) return false;
+        (*out)[i] = da == 1 ? db : da;
+    }
+    return true;
+}
+
+Tensor Tensor::binary(BinaryOp op, const Tensor& other) const {
+    if (!n_ || !other.n_) return Tensor();
+    std::vector<int64_t> shape;
+    if (!broadcast_shape(n_->shape, other.n_->shape, &shape))
+        return bad(kInvalidArgument, "binary op: shapes " + shape_str(n_->shape) + " and " + shape_str(other.n_->shape) + " do not broadcast");
+    Scalar dt = least_upper_dtype(n_->dtype, other.n_->dtype);
+    Tensor a = broadcast_to(cast(dt), shape), b = broadcast_to(other.cast(dt), shape);
+    if (!a.valid() || !b.valid()) return Tensor();
+    Scalar out = dt;
+    switch (op) {
+        case BinaryOp::Lt:
+        case BinaryOp::Le:
+        case BinaryOp::Gt:
+        case BinaryOp::Ge:
+        case BinaryOp::Eq:
+        case BinaryOp::Ne: out = Scalar::Bool; break;
+        default: break;
+    }
+    auto n = mk(TKind::Binary, out, shape, {a.n_, b.n_}, n_->device_id);
+    n->sub = static_cast<uint16_t>(op);
+    return Tensor(n);
+}
+
+Tensor Tensor::where_(const Tensor& cond, const Tensor& other) const {
+    if (!n_ || !cond.n_ || !other.n_) return Tensor();
+    std::vector<int64_t> s1, shape;
+    if (!broadcast_shape(n_->shape, other.n_->shape, &s1) || !broadcast_shape(s1, cond.n_->shape, &shape))
+        return bad(kInvalidArgument, "where: shapes do not broadcast");
+    Scalar dt = least_upper_dtype(n_->dtype, other.n_->dtype);
+    Tensor c = broadcast_to(cond.cast(Scalar::Bool), shape), t = broadcast_to(cast(dt), shape),
+           f = broadcast_to(other.cast(dt), shape);
+    if (!c.valid() || !t.valid() || !f.valid()) return Tensor();
+    return Tensor(mk(TKind::Where, dt, shape, {c.n_, t.n_, f.n_}, n_->device_id));
+}
+
+Tensor Tensor::sigmoid() const {
+    // sigmoid(x) = 1 / (1 + exp2(x * (-1/ln 2)))  (activation.rs:42-52)
+    if (!n_) return Tensor();
+    Tensor scaled = try_mul(const_(-1.0 / 0.6931471805599453, n_->dtype, n_->device_id));
+    Tensor e = scaled.try_exp2();
+    return const_(1.0, n_->dtype, n_->device_id).try_add(e).unary(UnaryOp::Reciprocal);
+}
+Tensor Tensor::swish() const { return try_mul(sigmoid()); }
+
+Tensor Tensor::reduce(ReduceOp op, std::vector<int64_t> axes, bool keepdim, bool promote) const {
+    if (!n_) return Tensor();
+    const int64_t nd = ndim();
+    std::set<int64_t> ax;
+    for (int64_t a : axes) {
+        if (!norm_axis(&a, nd)) return bad(kInvalidArgument, "reduce: axis out of range");
+        ax.insert(a);
+    }
+    // accumulation dtype (reduce.rs:101-117)
+    Scalar acc = n_->dtype;
+    if (promote) {
+        switch (n_->dtype) {
+            case Scalar::Bool:
+            case Scalar::Int8:
+            case Scalar::Int16: acc = Scalar::Int32; break;
+            case Scalar::UInt8:
+            case Scalar::UInt16: acc = Scalar::UInt32; break;
+            case Scalar::Float16:
+            case Scalar::BFloat16: acc = Scalar::Float32; break;
+            default: break;
+        }
+    }
+    Tensor work = cast(acc);
+    std::vector<int64_t> kshape = n_->shape, oshape;
+    for (int64_t i = 0; i < nd; i++) {
+        if (ax.count(i)) kshape[i] = 1;
+        else oshape.push_back(n_->shape[i]);
+    }
+    auto r = mk(TKind::Reduce, acc, kshape, {work.n_}, n_->device_id);
+    r->sub = static_cast<uint16_t>(op);
+    r->arg.assign(ax.begin(), ax.end());
+    Tensor res(r);
+    if (!keepdim) res = res.try_reshape(oshape);
+    // cast back after a promoted sum of a half type (reduce.rs:665-691)
+    if (promote && is_half(n_->dtype)) res = res.cast(n_->dtype);
+    return res;
+}
+
+Tensor Tensor::mean(std::vector<int64_t> axes, bool keepdim) const {
+    if (!n_) return Tensor();
+    int64_t count = 1;
+    for (int64_t a : axes) {
+        if (!norm_axis(&a, ndim())) return bad(kInvalidArgument, "mean: axis out of range");
+        count *= n_->shape[a];
+    }
+    Tensor s = reduce(ReduceOp::Add, axes, keepdim, true);
+    if (!s.valid()) return s;
+    // x / c is rewritten to x * (1/c) before rendering (schedule/src/optimizer/mod.rs:414-434)
+    return s.try_mul(const_(1.0 / static_cast<double>(count), s.dtype(), n_->device_id));
+}
+
+Tensor Tensor::matmul(const Tensor& other) const {
+    if (!n_ || !other.n_) return Tensor();
+    const int64_t dx = ndim(), dw = other.ndim();
+    if (dx == 0 || dw == 0) return bad(kInvalidArgument, "matmul: 0-d operand");
+    const int64_t k = n_->shape[dx - 1];
+    const int64_t axis_w = dw >= 2 ? dw - 2 : 0;
+    if (other.n_->shape[axis_w] != k)
+        return bad(kInvalidArgument, "matmul: shapes " + shape_str(n_->shape) + " and " + shape_str(other.n_->shape) + " do not contract");
+    if (dx < 2 || dw < 2) return bad(kInvalidArgument, "matmul: vector operands are not supported by this backend");
+    // x[..., M, K] -> [..., M, 1, K];  w[..., K, N] -> [..., 1, N, K];  product.sum(-1)  (matmul.rs:96-109)
+    std::vector<int64_t> xs = n_->shape;
+    xs.insert(xs.end() - 1, 1);
+    Tensor wt = other.try_transpose(-1, -2);
+    std::vector<int64_t> ws = wt.shape();
+    ws.insert(ws.end() - 2, 1);
+    Tensor prod = try_reshape(xs).try_mul(wt.try_reshape(ws));
+    Tensor res = prod.reduce(ReduceOp::Add, {-1}, false, true);
+    if (!res.valid()) return res;
+    res.node()->hint = HintKind::Matmul;
+    res.node()->hint_inputs = {n_, other.n_};
+    return res;
+}
+
+Tensor Tensor::softmax(int64_t axis) const {
+    if (!n_) return Tensor();
+    if (!norm_axis(&axis, ndim())) return bad(kInvalidArgument, "softmax: axis out of range");
+    Tensor m = reduce(ReduceOp::Max, {axis}, true, false);
+    Tensor e = try_sub(m).try_exp();
+    Tensor s = e.reduce(ReduceOp::Add, {axis}, true, false);  // sum_with: no promotion (reduce.rs:197-205)
+    Tensor res = e.try_div(s);
+    if (!res.valid()) return res;
+    res.node()->hint = HintKind::Softmax;
+    res.node()->hint_inputs = {n_};
+    res.node()->arg = {axis};
+    return res;
+}
+
+Tensor Tensor::rms_norm(int64_t axis, double eps) const {
+    if (!n_) return Tensor();
+    if (!norm_axis(&axis, ndim())) return bad(kInvalidArgument, "rms_norm: axis out of range");
+    std::vector<int64_t> axes;
+    for (int64_t a = axis; a < ndim(); a++) axes.push_back(a);
+    Tensor x32 = cast(Scalar::Float32);
+    Tensor norm = x32.square().mean(axes, true).try_add(const_(eps, Scalar::Float32, n_->device_id)).try_rsqrt();
+    return try_mul(norm);  // bf16 * f32 promotes to f32 (dtype/src/cast.rs:88)
+}
+
+Tensor Tensor::embedding(const Tensor& indices) const {
+    if (!n_ || !indices.n_) return Tensor();
+    if (ndim() != 2) return bad(kInvalidArgument, "embedding: weight must be [vocab, dim]");
+    std::vector<int64_t> shape = indices.shape();
+    shape.push_back(n_->shape[1]);
+    Tensor idx = indices.cast(Scalar::Int32);
+    return Tensor(mk(TKind::Gather, n_->dtype, shape, {n_, idx.n_}, n_->device_id));
+}
+
+Tensor Tensor::apply_rotary_emb(const Tensor& cos, const Tensor& sin, bool interleaved) const {
+    if (!n_ || !cos.valid() || !sin.valid()) return Tensor();
+    const int64_t nd = ndim();
+    if (nd == 0) return bad(kInvalidArgument, "apply_rotary_emb requires non-scalar input");
+    const int64_t last = n_->shape[nd - 1], half = last / 2;
+    if (last % 2) return bad(kInvalidArgument, "apply_rotary_emb: last dim must be even");
+    Tensor x1, x2;
+    std::vector<int64_t> b0(nd, 0), e0 = n_->shape;
+    if (interleaved) {
+        std::vector<int64_t> rs(n_->shape.begin(), n_->shape.end() - 1);
+        rs.push_back(half);
+        rs.push_back(2);
+        Tensor r = try_reshape(rs);
+        std::vector<int64_t> b(nd + 1, 0), e = rs;
+        e[nd] = 1;
+        x1 = r.try_shrink(b, e).try_squeeze(-1);
+        b[nd] = 1;
+        e[nd] = 2;
+        x2 = r.try_shrink(b, e).try_squeeze(-1);
+    } else {
+        std::vector<int64_t> e = e0, b = b0;
+        e[nd - 1] = half;
+        x1 = try_shrink(b, e);
+        b[nd - 1] = half;
+        e[nd - 1] = last;
+        x2 = try_shrink(b, e);
+    }
+    Tensor real = x1.try_mul(cos).try_sub(x2.try_mul(sin));
+    Tensor imag = x1.try_mul(sin).try_add(x2.try_mul(cos));
+    if (!real.valid() || !imag.valid()) return Tensor();
+    if (interleaved) {
+        Tensor st = cat({real.try_unsqueeze(-1), imag.try_unsqueeze(-1)}, -1);
+        std::vector<int64_t> fs = real.shape();
+        fs.back() = last;
+        return st.try_reshape(fs);
+    }
+    return cat({real, imag}, -1);
+}
+
+Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& value, double scale, bool is_causal) const {
+    if (!n_ || !key.valid() || !value.valid()) return Tensor();
+    const int64_t nd = ndim();
+    if (nd < 2 || key.ndim() != nd || value.ndim() != nd) return bad(kInvalidArgument, "sdpa: rank mismatch");
+    const int64_t head_dim = n_->shape[nd - 1];
+    const double scale_val = scale > 0.0 ? scale : 1.0 / std::sqrt(static_cast<double>(head_dim));  // transformer.rs:90-91
+    const Scalar sdt = n_->dtype;
+    Tensor scores = matmul(key.try_transpose(-1, -2));
+    scores = scores.try_mul(const_(scale_val, sdt, n_->device_id));
+    if (is_causal) {
+        const int64_t ql = n_->shape[nd - 2], kl = key.shape()[nd - 2];
+        // tril(0) over a [Sq, Sk] mask of ones: key j visible iff j <= i (transformer.rs:103-109)
+        auto iota = [&](int64_t axis) {
+            auto n = mk(TKind::Iota, Scalar::Int32, {ql, kl}, {}, n_->device_id);
+            n->arg = {axis};
+            return Tensor(n);
+        };
+        Tensor mask = iota(1).binary(BinaryOp::Le, iota(0));
+        scores = scores.where_(mask, const_(-INFINITY, sdt, n_->device_id));
+    }
+    Tensor out = scores.softmax(-1).matmul(value);
+    if (!out.valid()) return out;
+    out.node()->hint = HintKind::Sdpa;
+    out.node()->hint_inputs = {n_, key.node(), value.node()};
+    out.node()->hint_scale = scale_val;
+    out.node()->hint_causal = is_causal;
+    return out;
+}
+
+// ============================================================================ scheduling
+namespace {
+
+// One kernel under construction: the builder plus the device buffers it reads (slot 1..),
+// discovered while the expression is emitted.
+struct KernelGen {
+    KernelBuilder b;
+    Scalar idx_t = Scalar::Int32;
+    std::vector<std::shared_ptr<Buffer>> inputs;
+    std::vector<uint32_t> input_params;
+    std::vector<Scalar> input_dtypes;
+    std::map<std::pair<const TensorNode*, std::vector<uint32_t>>, uint32_t> memo;
+
+    uint32_t ci(int64_t v) { return b.ci(v, idx_t); }
+    uint32_t buffer_param(const std::shared_ptr<Buffer>& buf, Scalar dt, int64_t numel) {
+        for (size_t i = 0; i < inputs.size(); i++)
+            if (inputs[i].get() == buf.get() && input_dtypes[i] == dt) return input_params[i];
+        inputs.push_back(buf);
+        input_dtypes.push_back(dt);
+        input_params.push_back(b.param(static_cast<int>(inputs.size()), dt, numel));
+        return input_params.back();
+    }
+};
+
+// half types are evaluated in f32
+Scalar compute_dtype(Scalar s) { return is_half(s) ? Scalar::Float32 : s; }
+
+uint32_t flatten(KernelGen& g, const std::vector<uint32_t>& coords, const std::vector<int64_t>& shape) {
+    uint32_t flat = g.ci(0);
+    int64_t stride = 1;
+    for (size_t i = shape.size(); i-- > 0;) {
+        if (shape[i] != 1) flat = g.b.iadd(flat, g.b.imul(coords[i], stride));
+        stride *= shape[i];
+    }
+    return flat;
+}
+std::vector<uint32_t> unflatten(KernelGen& g, uint32_t flat, const std::vector<int64_t>& shape) {
+    std::vector<uint32_t> coords(shape.size());
+    int64_t inner = 1;
+    for (size_t i = shape.size(); i-- > 0;) {
+        if (shape[i] == 1) {
+            coords[i] = g.ci(0);
+        } else {
+            uint32_t q = g.b.idiv(flat, inner);
+            // the outermost non-unit dimension needs no modulo
+            bool outermost = true;
+            for (size_t j = 0; j < i; j++) outermost = outermost && shape[j] == 1;
+            coords[i] = outermost ? q : g.b.imod(q, shape[i]);
+        }
+        inner *= shape[i];
+    }
+    return coords;
+}
+
+uint32_t emit(KernelGen& g, const TensorNode* n, const std::vector<uint32_t>& coords);
+
+uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const std::vector<uint32_t>& coords) {
+    KernelBuilder& b = g.b;
+    const Scalar ct = compute_dtype(n->dtype);
+    if (n->buffer) {  // materialised tensor: a load from its row-major buffer
+        uint32_t p = g.buffer_param(n->buffer, n->dtype, n->numel());
+        uint32_t v = b.load(b.index(p, flatten(g, coords, n->shape)));
+        return ct != n->dtype ? b.cast(v, ct) : v;
+    }
+    switch (n->kind) {
+        case TKind::Const:
+            return is_float(ct) ? b.cf(n->cval, ct) : b.ci(static_cast<int64_t>(n->cval), ct);
+        case TKind::Unary: {
+            uint32_t x = emit(g, n->src[0].get(), coords);
+            return b.unary(static_cast<UnaryOp>(n->sub), x);
+        }
+        case TKind::Binary: {
+            uint32_t x = emit(g, n->src[0].get(), coords), y = emit(g, n->src[1].get(), coords);
+            return b.binary(static_cast<BinaryOp>(n->sub), x, y);
+        }
+        case TKind::Where: {
+            uint32_t c = emit(g, n->src[0].get(), coords), t = emit(g, n->src[1].get(), coords),
+                     f = emit(g, n->src[2].get(), coords);
+            return b.where(c, t, f);
+        }
+        case TKind::Cast: {
+            uint32_t x = emit(g, n->src[0].get(), coords);
+            const Scalar from = compute_dtype(n->src[0]->dtype);
+            if (is_half(n->dtype)) {  // an explicit cast to a half type rounds here
+                uint32_t r = b.dtype(x).scalar == n->dtype ? x : b.cast(x, n->dtype);
+                return b.cast(r, Scalar::Float32);
+            }
+            return from == ct ? x : b.cast(x, ct);
+        }
+        case TKind::Contiguous: return emit(g, n->src[0].get(), coords);
+        case TKind::Reshape: {
+            const TensorNode* s = n->src[0].get();
+            // same sequence of non-unit dims: coordinates carry over
+            std::vector<size_t> a, c;
+            for (size_t i = 0; i < n->shape.size(); i++)
+                if (n->shape[i] != 1) a.push_back(i);
+            for (size_t i = 0; i < s->shape.size(); i++)
+                if (s->shape[i] != 1) c.push_back(i);
+            bool same = a.size() == c.size();
+            for (size_t i = 0; same && i < a.size(); i++) same = n->shape[a[i]] == s->shape[c[i]];
+            std::vector<uint32_t> sc(s->shape.size());
+            if (same) {
+                for (size_t i = 0; i < sc.size(); i++) sc[i] = g.ci(0);
+                for (size_t i = 0; i < a.size(); i++) sc[c[i]] = coords[a[i]];
+            } else {
+                sc = unflatten(g, flatten(g, coords, n->shape), s->shape);
+            }
+            return emit(g, s, sc);
+        }
+        case TKind::Permute: {
+            std::vector<uint32_t> sc(coords.size());
+            for (size_t i = 0; i < coords.size(); i++) sc[n->arg[i]] = coords[i];
+            return emit(g, n->src[0].get(), sc);
+        }
+        case TKind::Expand: {
+            const TensorNode* s = n->src[0].get();
+            std::vector<uint32_t> sc = coords;
+            for (size_t i = 0; i < sc.size(); i++)
+                if (s->shape[i] == 1 && n->shape[i] != 1) sc[i] = g.ci(0);
+            return emit(g, s, sc);
+        }
+        case TKind::Shrink: {
+            std::vector<uint32_t> sc = coords;
+            for (size_t i = 0; i < sc.size(); i++)
+                if (n->arg[i]) sc[i] = b.iadd(coords[i], g.ci(n->arg[i]));
+            return emit(g, n->src[0].get(), sc);
+        }
+        case TKind::Iota: {
+            uint32_t c = coords[n->arg[0]];
+            return b.dtype(c).scalar == ct ? c : b.cast(c, ct);
+        }
+        case TKind::Cat: {
+            const size_t axis = static_cast<size_t>(n->arg[0]);
+            // every part is evaluated at a clamped coordinate; the right one is selected
+            int64_t off = 0;
+            std::vector<uint32_t> vals;
+            std::vector<int64_t> ends;
+            for (const TensorRef& p : n->src) {
+                const int64_t len = p->shape[axis];
+                std::vector<uint32_t> sc = coords;
+                uint32_t rel = b.iadd(coords[axis], g.ci(-off));
+                uint32_t lo = b.where(b.binary(BinaryOp::Lt, rel, g.ci(0)), g.ci(0), rel);
+                sc[axis] = b.where(b.binary(BinaryOp::Gt, lo, g.ci(len - 1)), g.ci(len - 1), lo);
+                vals.push_back(emit(g, p.get(), sc));
+                off += len;
+                ends.push_back(off);
+            }
+            uint32_t res = vals.back();
+            for (size_t i = vals.size() - 1; i-- > 0;)
+                res = b.where(b.binary(BinaryOp::Lt, coords[axis], g.ci(ends[i])), vals[i], res);
+            return res;
+        }
+        case TKind::Gather: {
+            const TensorNode* w = n->src[0].get();
+            std::vector<uint32_t> ic(coords.begin(), coords.end() - 1);
+            uint32_t row = emit(g, n->src[1].get(), ic);
+            if (b.dtype(row).scalar != g.idx_t) row = b.cast(row, g.idx_t);
+            return emit(g, w, {row, coords.back()});
+        }
+        case TKind::Reduce:
+        case TKind::Buffer: break;  // always materialised before being read
+    }
+    return 0;
+}
+
+uint32_t emit(KernelGen& g, const TensorNode* n, const std::vector<uint32_t>& coords) {
+    auto key = std::make_pair(n, coords);
+    auto it = g.memo.find(key);
+    if (it != g.memo.end()) return it->second;
+    uint32_t v = emit_uncached(g, n, coords);
+    g.memo[key] = v;
+    return v;
+}
+
+struct Scheduler {
+    std::shared_ptr<Device> dev;
+    std::unique_ptr<ExecutionPlan> plan;
+    RealizeStats stats;
+
+    int add_kernel(const std::shared_ptr<CachedKernel>& k, const std::vector<std::shared_ptr<Buffer>>& bufs, bool cached) {
+        std::vector<size_t> idx;
+        for (auto& bptr : bufs) idx.push_back(plan->add_buffer(bptr));
+        MRK_TRY(plan->add_kernel(k, idx, {}));
+        stats.kernel_names.push_back(k->entry_point);
+        if (cached) stats.cached_kernels++;
+        return kOk;
+    }
+    std::shared_ptr<Buffer> new_buffer(const TensorNode* n) {
+        BufferOptions o;
+        size_t bytes = static_cast<size_t>(n->numel()) * scalar_size(n->dtype);
+        return std::make_shared<Buffer>(dev->allocator, bytes ? bytes : 1, o);
+    }
+    int builtin(const char* kind, const std::vector<int64_t>& params, const std::vector<std::shared_ptr<Buffer>>& bufs) {
+        std::string key = std::string("builtin:") + kind;
+        for (int64_t p : params) key += ":" + std::to_string(p);
+        const std::string device = "HIP:" + std::to_string(dev->device_id);
+        std::shared_ptr<CachedKernel> ck;
+        bool cached = false;
+        MRK_TRY(KernelCache::global().get_or_compile(
+            fnv1a64(reinterpret_cast<const uint8_t*>(key.data()), key.size()), device,
+            [&](std::shared_ptr<CachedKernel>* fresh) -> int {
+                std::unique_ptr<Program> p;
+                MRK_TRY(create_builtin_program(dev->device_id, dev->allocator->stream(), kind, params.data(), params.size(), &p));
+                auto k = std::make_shared<CachedKernel>();
+                k->entry_point = p->name();
+                k->program = std::move(p);
+                k->device = device;
+                *fresh = std::move(k);
+                return kOk;
+            },
+            &ck, &cached));
+        return add_kernel(ck, bufs, cached);
+    }
+
+    // nodes that must exist in memory before the kernel rooted at `root` can read them
+    void boundaries(const TensorNode* n, const TensorNode* root, std::set<const TensorNode*>& seen,
+                    std::vector<TensorNode*>& out, int64_t* max_numel) {
+        if (!seen.insert(n).second) return;
+        *max_numel = std::max(*max_numel, n->numel());
+        if (n->buffer) return;
+        if (n != root && (n->kind == TKind::Reduce || n->kind == TKind::Contiguous || fusable(n))) {
+            out.push_back(const_cast<TensorNode*>(n));
+            return;
+        }
+        for (const TensorRef& s : n->src) boundaries(s.get(), root, seen, out, max_numel);
+    }
+
+    static bool all_dims_one_except_last2(const TensorNode* n) { return n->shape.size() == 2; }
+    bool fusable(const TensorNode* n) const {
+        if (!g_fusion || n->hint == HintKind::None) return false;
+        switch (n->hint) {
+            case HintKind::Softmax:
+                return n->dtype == Scalar::Float32 && !n->shape.empty() &&
+                       n->arg[0] == static_cast<int64_t>(n->shape.size()) - 1 && n->numel() > 0;
+            case HintKind::Matmul: {
+                const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
+                if (a->shape.size() != 2 || w->shape.size() != 2 || a->dtype != w->dtype) return false;
+                if (a->dtype == Scalar::BFloat16) return n->dtype == Scalar::BFloat16 && n->numel() > 0;
+                if (a->dtype == Scalar::Float32)
+                    return a->shape[0] % 64 == 0 && w->shape[1] % 64 == 0 && a->shape[0] > 0 && w->shape[1] > 0;
+                return false;
+            }
+            case HintKind::Sdpa: {
+                const TensorNode* q = n->hint_inputs[0].get();
+                const TensorNode* k = n->hint_inputs[1].get();
+                const TensorNode* v = n->hint_inputs[2].get();
+                return q->dtype == Scalar::BFloat16 && k->dtype == q->dtype && v->dtype == q->dtype &&
+                       q->shape.size() == 4 && q->shape[3] == 128 && v->shape[3] == 128 && k->shape[2] > 0 &&
+                       k->shape[0] == q->shape[0] && k->shape[1] == q->shape[1] && q->numel() > 0;
+            }
+            default: return false;
+        }
+    }
+
+    int materialize(TensorNode* n) {
+        if (n->buffer) return kOk;
+        if (n->numel() > 0 && fusable(n)) return materialize_fused(n);
+        // a reshape of materialised data is the same bytes
+        if (n->kind == TKind::Reshape) {
+            TensorNode* s = n->src[0].get();
+            if (s->buffer || s->kind == TKind::Reduce || s->kind == TKind::Contiguous || fusable(s)) {
+                MRK_TRY(materialize(s));
+                n->buffer = s->buffer;
+                return kOk;
+            }
+        }
+        if (n->numel() == 0) {
+            n->buffer = new_buffer(n);
+            return kOk;
+        }
+        std::set<const TensorNode*> seen;
+        std::vector<TensorNode*> deps;
+        int64_t max_numel = 0;
+        boundaries(n, n, seen, deps, &max_numel);
+        for (TensorNode* d : deps) MRK_TRY(materialize(d));
+        return n->kind == TKind::Reduce ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
+    }
+
+    int materialize_fused(TensorNode* n) {
+        for (const TensorRef& in : n->hint_inputs) MRK_TRY(materialize(in.get()));
+        auto out = new_buffer(n);
+        int rc = kOk;
+        if (n->hint == HintKind::Softmax) {
+            const int64_t cols = n->shape.back(), rows = n->numel() / cols;
+            rc = builtin("softmax_f32", {rows, cols}, {out, n->hint_inputs[0]->buffer});
+        } else if (n->hint == HintKind::Matmul) {
+            const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
+            const int64_t M = a->shape[0], K = a->shape[1], N = w->shape[1];
+            if (a->dtype == Scalar::BFloat16) {
+                rc = builtin("gemm_bf16", {M, N, K}, {out, a->buffer, w->buffer});
+            } else {
+                LinearKernel k = build_matmul_f32_kernel(M, N, K);
+                std::shared_ptr<CachedKernel> ck;
+                bool cached = false;
+                const std::string name = "r_" + std::to_string(M) + "_" + std::to_string(N) + "_" + std::to_string(K);
+                MRK_TRY(get_or_compile_linear_kernel(*dev, k, name.c_str(), &ck, &cached));
+                rc = add_kernel(ck, {out, a->buffer, w->buffer}, cached);
+            }
+        } else if (n->hint == HintKind::Sdpa) {
+            const TensorNode* q = n->hint_inputs[0].get();
+            const TensorNode* k = n->hint_inputs[1].get();
+            float scale = static_cast<float>(n->hint_scale);
+            uint32_t bits;
+            std::memcpy(&bits, &scale, 4);
+            rc = builtin("flash_fwd_bf16",
+                         {q->shape[0] * q->shape[1], q->shape[2], k->shape[2], q->shape[3], n->hint_causal ? 1 : 0,
+                          static_cast<int64_t>(bits)},
+                         {out, q->buffer, k->buffer, n->hint_inputs[2]->buffer});
+        }
+        MRK_TRY(rc);
+        n->buffer = out;
+        return kOk;
+    }
+
+    int finish_kernel(KernelGen& g, TensorNode* n, const std::shared_ptr<Buffer>& out, const std::string& name) {
+        LinearKernel k = g.b.finish();
+        std::shared_ptr<CachedKernel> ck;
+        bool cached = false;
+        MRK_TRY(get_or_compile_linear_kernel(*dev, k, name.c_str(), &ck, &cached));
+        std::vector<std::shared_ptr<Buffer>> bufs{out};
+        bufs.insert(bufs.end(), g.inputs.begin(), g.inputs.end());
+        MRK_TRY(add_kernel(ck, bufs, cached));
+        n->buffer = out;
+        return kOk;
+    }
+
+    int gen_elementwise(TensorNode* n, int64_t max_numel) {
+        const int64_t N = n->numel();
+        KernelGen g;
+        g.idx_t = max_numel >= (1LL << 31) ? Scalar::Int64 : Scalar::Int32;
+        KernelBuilder& b = g.b;
+        auto out = new_buffer(n);
+        uint32_t po = b.param(0, n->dtype, N);
+        const int64_t block = 256, grid = (N + block - 1) / block;
+        if (grid > 2147483647LL) return fail(kInvalidArgument, "realize: tensor too large for one launch");
+        uint32_t gx = b.special("gidx0", grid), lx = b.special("lidx0", block);
+        if (g.idx_t != Scalar::Int32) {
+            gx = b.cast(gx, g.idx_t);
+            lx = b.cast(lx, g.idx_t);
+        }
+        uint32_t i = b.iadd(b.imul(gx, block), lx);
+        b.if_(b.binary(BinaryOp::Lt, i, g.ci(N)));
+        std::vector<uint32_t> coords = unflatten(g, i, n->shape);
+        uint32_t v = n->kind == TKind::Contiguous ? emit(g, n->src[0].get(), coords) : emit_uncached(g, n, coords);
+        if (b.dtype(v).scalar != n->dtype) v = b.cast(v, n->dtype);
+        b.store(b.index(po, i), v);
+        b.endif();
+        return finish_kernel(g, n, out, "E_" + std::to_string(N));
+    }
+
+    int gen_reduce(TensorNode* n, int64_t max_numel) {
+        const TensorNode* s = n->src[0].get();
+        const ReduceOp op = static_cast<ReduceOp>(n->sub);
+        const int64_t Nout = n->numel();
+        std::vector<int64_t> rdims;
+        int64_t R = 1;
+        for (int64_t a : n->arg) {
+            rdims.push_back(s->shape[a]);
+            R *= s->shape[a];
+        }
+        KernelGen g;
+        g.idx_t = max_numel >= (1LL << 31) ? Scalar::Int64 : Scalar::Int32;
+        KernelBuilder& b = g.b;
+        auto out = new_buffer(n);
+        uint32_t po = b.param(0, n->dtype, Nout);
+        const Scalar ct = compute_dtype(n->dtype);
+        const bool wave = R >= 128 && ct == Scalar::Float32 && (op == ReduceOp::Add || op == ReduceOp::Max);
+        auto identity = [&]() -> uint32_t {
+            if (is_float(ct)) return b.cf(op == ReduceOp::Add ? 0.0 : op == ReduceOp::Mul ? 1.0 : op == ReduceOp::Max ? -INFINITY : INFINITY, ct);
+            return b.ci(op == ReduceOp::Mul ? 1 : 0, ct);
+        };
+        if (!wave) {
+            // one work-item per output element, the reduced axes as nested sequential loops
+            const int64_t block = 64, grid = (Nout + block - 1) / block;
+            uint32_t gx = b.special("gidx0", grid), lx = b.special("lidx0", block);
+            if (g.idx_t != Scalar::Int32) {
+                gx = b.cast(gx, g.idx_t);
+                lx = b.cast(lx, g.idx_t);
+            }
+            uint32_t o = b.iadd(b.imul(gx, block), lx);
+            uint32_t gate = b.binary(BinaryOp::Lt, o, g.ci(Nout));
+            uint32_t oc = b.where(gate, o, g.ci(Nout - 1));  // clamp: masked lanes recompute the last element
+            std::vector<uint32_t> coords = unflatten(g, oc, n->shape);
+            std::vector<uint32_t> ranges;
+            for (size_t r = 0; r < n->arg.size(); r++) {
+                uint32_t rg = b.add(Op::Range, KernelBuilder::scalar(g.idx_t), {g.ci(rdims[r])}, static_cast<int64_t>(r), 0,
+                                    static_cast<uint16_t>(AxisType::Reduce));
+                ranges.push_back(rg);
+                coords[n->arg[r]] = rg;
+            }
+            uint32_t v = emit(g, s, coords);
+            uint32_t red = b.reduce(op, v, ranges);
+            std::vector<uint32_t> rev(ranges.rbegin(), ranges.rend());
+            b.end(rev);
+            b.if_(gate);
+            uint32_t res = red;
+            if (b.dtype(res).scalar != n->dtype) res = b.cast(res, n->dtype);
+            b.store(b.index(po, o), res);
+            b.endif();
+            return finish_kernel(g, n, out, "r_" + std::to_string(Nout) + "_" + std::to_string(R));
+        }
+        // one wavefront per output element: lanes stride the flattened reduce space, partial
+        // results are combined with the wave64 cross-lane reduction (the GROUP_REDUCE idea of
+        // schedule/src/optimizer/heuristics.rs:370-392 without the LDS round trip)
+        const int64_t per_block = 4, grid = (Nout + per_block - 1) / per_block;
+        if (grid > 2147483647LL) return fail(kInvalidArgument, "realize: reduction too large for one launch");
+        uint32_t gx = b.special("gidx0", grid), lane = b.special("lidx0", 64), ly = b.special("lidx1", per_block);
+        if (g.idx_t != Scalar::Int32) {
+            gx = b.cast(gx, g.idx_t);
+            lane = b.cast(lane, g.idx_t);
+            ly = b.cast(ly, g.idx_t);
+        }
+        uint32_t o = b.iadd(b.imul(gx, per_block), ly);
+        uint32_t ogate = b.binary(BinaryOp::Lt, o, g.ci(Nout));
+        uint32_t oc = b.where(ogate, o, g.ci(Nout - 1));
+        std::vector<uint32_t> coords = unflatten(g, oc, n->shape);
+        const int64_t steps = (R + 63) / 64;
+        uint32_t rg = b.add(Op::Range, KernelBuilder::scalar(g.idx_t), {g.ci(steps)}, 0, 0, static_cast<uint16_t>(AxisType::Reduce));
+        uint32_t f = b.iadd(b.imul(rg, 64), lane);
+        uint32_t fgate = b.binary(BinaryOp::Lt, f, g.ci(R));
+        uint32_t fc = (R % 64 == 0) ? f : b.where(fgate, f, g.ci(R - 1));
+        std::vector<uint32_t> rc = unflatten(g, fc, rdims);
+        for (size_t r = 0; r < n->arg.size(); r++) coords[n->arg[r]] = rc[r];
+        uint32_t v = emit(g, s, coords);
+        if (R % 64 != 0) v = b.where(fgate, v, identity());
+        uint32_t red = b.reduce(op, v, {rg});
+        b.end({rg});
+        uint32_t total = b.wave_reduce(op, red);
+        uint32_t first = b.binary(BinaryOp::Eq, lane, g.ci(0));
+        b.if_(b.binary(BinaryOp::And, first, ogate));
+        uint32_t res = total;
+        if (b.dtype(res).scalar != n->dtype) res = b.cast(res, n->dtype);
+        b.store(b.index(po, o), res);
+        b.endif();
+        return finish_kernel(g, n, out, "r_" + std::to_string(Nout) + "_g" + std::to_string(R));
+    }
+};
+
+}  // namespace
+
+int Tensor::realize() const {
+    if (!n_) return fail(kInvalidArgument, "realize: invalid tensor");
+    g_stats = RealizeStats();
+    if (n_->buffer) return kOk;
+    auto t0 = std::chrono::steady_clock::now();
+    Scheduler s;
+    MRK_TRY(DeviceFactoryRegistry::global().device("HIP", n_->device_id, &s.dev));
+    s.plan.reset(new ExecutionPlan(n_->device_id));
+    MRK_TRY(s.materialize(n_.get()));
+    MRK_TRY(s.plan->build());
+    MRK_TRY(s.plan->execute());
+    s.stats.elapsed_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    g_stats = s.stats;
+    return kOk;
+}
+
+int Tensor::to_bytes(void* dst, size_t nbytes) const {
+    if (!n_) return fail(kInvalidArgument, "to_vec: invalid tensor");
+    if (!n_->buffer) MRK_TRY(realize());
+    const size_t expect = static_cast<size_t>(n_->numel()) * scalar_size(n_->dtype);
+    if (nbytes != expect) return failf(kSizeMismatch, "size mismatch: expected %zu, got %zu", expect, nbytes);
+    if (expect == 0) return kOk;
+    return n_->buffer->copyout(dst, nbytes);
+}
+
+}  // namespace mrk

@@ -1,0 +1,308 @@
+"""Lazy tensor API on the GPU: the reference's own tensor tests restated through the C ABI
+(tensor/src/test/unit/matmul.rs, transformer.rs, fusion.rs, book_examples.rs), every result
+also checked against the CPU oracle.  Both lowering modes are covered: generated kernels only
+(fusion off) and the hand-written kernels (fusion on)."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+GOLD = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_known_answers.json")))
+
+
+@pytest.fixture()
+def T(dev):
+    from morok_amd import tensor
+
+    yield tensor
+    tensor.set_fusion(True)
+
+
+@pytest.fixture(params=[False, True], ids=["generated", "fused"])
+def fusion(request, T):
+    T.set_fusion(request.param)
+    return request.param
+
+
+def f32(a):
+    return np.asarray(a, dtype=np.float32)
+
+
+# ---------------------------------------------------------------- creation / extraction
+def test_roundtrip_and_size_check(T):
+    from morok_amd import MorokHipError, uop
+
+    x = np.arange(24, dtype=np.float32).reshape(2, 3, 4)
+    t = T.Tensor.from_numpy(x)
+    assert t.shape == (2, 3, 4) and t.dtype == uop.F32
+    np.testing.assert_array_equal(t.to_numpy(), x)
+    with pytest.raises(MorokHipError) as e:  # data.rs:81-96
+        T.Tensor.from_bytes(b"\0" * 10, (3,), uop.F32)
+    assert "data length 10 != expected 12" in str(e.value)
+    assert e.value.code == 1
+
+
+def test_movement_ops_are_index_arithmetic(T):
+    x = np.arange(2 * 3 * 4, dtype=np.float32).reshape(2, 3, 4)
+    t = T.Tensor.from_numpy(x)
+    y = t.try_permute([2, 0, 1]).try_reshape([4, 6]).try_shrink([(1, 3), (2, 5)]).try_add(1.0)
+    np.testing.assert_array_equal(y.to_numpy(), x.transpose(2, 0, 1).reshape(4, 6)[1:3, 2:5] + 1)
+    assert len(y.kernels()) == 1  # one elementwise kernel, no copies for the views
+    e = T.Tensor.from_numpy(f32([[1], [2]])).try_expand([2, 3]).try_mul(T.Tensor.from_numpy(f32([10, 20, 30])))
+    np.testing.assert_array_equal(e.to_numpy(), f32([[10, 20, 30], [20, 40, 60]]))
+    c = T.Tensor.cat([t, t.try_mul(2.0)], 1)
+    np.testing.assert_array_equal(c.to_numpy(), np.concatenate([x, 2 * x], 1))
+
+
+def test_elementwise_int_and_promotion(T):
+    from morok_amd import uop
+
+    a = T.Tensor.from_numpy(np.arange(-5, 5, dtype=np.int32))
+    b = T.Tensor.from_numpy(np.full(10, 3, dtype=np.int32))
+    np.testing.assert_array_equal(a.binary("mul", b).binary("add", b).to_numpy(), np.arange(-5, 5) * 3 + 3)
+    m = a.binary("lt", 0)
+    assert m.dtype == uop.BOOL
+    np.testing.assert_array_equal(m.to_numpy(), np.arange(-5, 5) < 0)
+    f = a.try_add(T.Tensor.from_numpy(np.full(10, 0.5, dtype=np.float32)))
+    assert f.dtype == uop.F32
+    np.testing.assert_array_equal(f.to_numpy(), np.arange(-5, 5) + np.float32(0.5))
+    i64 = T.Tensor.from_numpy(np.array([2**40, -7], dtype=np.int64)).binary("add", T.Tensor.from_numpy(np.array([1, 1], dtype=np.int64)))
+    np.testing.assert_array_equal(i64.to_numpy(), np.array([2**40 + 1, -6], dtype=np.int64))
+
+
+# ---------------------------------------------------------------- matmul (matmul.rs)
+def test_matmul_known_answers(T, fusion):
+    for key in ("matmul_2x2", "matmul_3x3"):
+        g = GOLD[key]
+        c = T.Tensor.from_numpy(f32(g["a"])).matmul(T.Tensor.from_numpy(f32(g["b"])))
+        np.testing.assert_allclose(c.to_numpy(), f32(g["expected"]), atol=g["tol"])
+
+
+@pytest.mark.parametrize("n,tol", [(128, 0.5), (256, 1.0), (500, 1.5)])
+def test_matmul_square_closed_form(T, fusion, oracle, n, tol):
+    x = np.arange(n * n, dtype=np.int64)
+    a = ((x % 31) * 0.05 - 0.8).astype(np.float32).reshape(n, n)
+    b = ((x % 37) * 0.04 - 0.7).astype(np.float32).reshape(n, n)
+    c = T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b))
+    got = c.to_numpy()
+    assert len(c.kernels()) == 1  # fusion.rs:28-33
+    ref = oracle.matmul_f32(a, b)
+    assert np.abs(got - ref).max() < tol  # the reference's own tolerance (matmul.rs:669-677)
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-4 * np.abs(ref).max())
+
+
+def test_matmul_nonsquare_and_batched(T, fusion, oracle):
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal((64, 512), dtype=np.float32)
+    b = rng.standard_normal((512, 64), dtype=np.float32)
+    got = T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b)).to_numpy()
+    np.testing.assert_allclose(got, oracle.matmul_f32(a, b), rtol=1e-4, atol=1e-3)
+    ab = rng.standard_normal((3, 5, 7), dtype=np.float32)
+    bb = rng.standard_normal((3, 7, 4), dtype=np.float32)
+    got = T.Tensor.from_numpy(ab).matmul(T.Tensor.from_numpy(bb)).to_numpy()
+    np.testing.assert_allclose(got, np.stack([oracle.matmul_f32(ab[i], bb[i]) for i in range(3)]), rtol=1e-4, atol=1e-5)
+
+
+def test_matmul_shape_error(T):
+    from morok_amd import MorokHipError
+
+    with pytest.raises(MorokHipError):
+        T.Tensor.from_numpy(np.zeros((2, 3), np.float32)).matmul(T.Tensor.from_numpy(np.zeros((4, 2), np.float32)))
+
+
+def test_matmul_bf16(T, fusion, oracle):
+    from morok_amd import synth, uop
+
+    rng = np.random.default_rng(7)
+    M, N, K = (256, 256, 128) if fusion else (48, 40, 64)
+    a = synth.to_bf16(rng.standard_normal((M, K), dtype=np.float32))
+    b = synth.to_bf16(rng.standard_normal((K, N), dtype=np.float32))
+    c = T.Tensor.from_numpy(a, uop.BF16).matmul(T.Tensor.from_numpy(b, uop.BF16))
+    assert c.dtype == uop.BF16
+    got = synth.from_bf16(c.to_numpy())
+    ref = synth.from_bf16(oracle.gemm_bf16(a, b))
+    assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
+    if fusion:
+        assert c.kernels() == ["gemm_bf16_tile256"] or c.kernels()[0].startswith("gemm_bf16")
+
+
+# ---------------------------------------------------------------- softmax
+@pytest.mark.parametrize("shape", [(4, 8), (3, 1000), (2, 5, 257)])
+def test_softmax(T, fusion, oracle, shape):
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal(shape) * 3).astype(np.float32)
+    s = T.Tensor.from_numpy(x).softmax(-1)
+    got = s.to_numpy()
+    assert len(s.kernels()) == (1 if fusion else 3)  # fusion.rs:83-88: max, sum, divide
+    ref = oracle.softmax_f32(x.reshape(-1, shape[-1])).reshape(shape)
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-7)
+    np.testing.assert_allclose(got.sum(-1), 1.0, atol=GOLD["softmax_invariants"]["row_sum_tol"])
+    assert (got > 0).all() and (got <= 1).all()
+
+
+def test_softmax_inner_axis(T, oracle):
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((6, 33, 5)).astype(np.float32)
+    got = T.Tensor.from_numpy(x).softmax(1).to_numpy()
+    ref = oracle.softmax_f32(np.ascontiguousarray(x.transpose(0, 2, 1)).reshape(-1, 33)).reshape(6, 5, 33).transpose(0, 2, 1)
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-7)
+
+
+# ---------------------------------------------------------------- reductions
+def test_reductions(T):
+    rng = np.random.default_rng(13)
+    x = rng.standard_normal((7, 300, 9)).astype(np.float32)
+    t = T.Tensor.from_numpy(x)
+    np.testing.assert_allclose(t.sum(1).to_numpy(), x.astype(np.float64).sum(1), rtol=1e-4, atol=1e-4)
+    np.testing.assert_array_equal(t.max(1).to_numpy(), x.max(1))
+    np.testing.assert_allclose(t.sum([0, 2]).to_numpy(), x.astype(np.float64).sum((0, 2)), rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(t.mean([2], keepdim=True).to_numpy(), x.mean(2, keepdims=True), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(t.sum([0, 1, 2]).to_numpy(), x.astype(np.float64).sum(), rtol=1e-4, atol=1e-3)
+    i = np.arange(1000, dtype=np.int32).reshape(10, 100)
+    np.testing.assert_array_equal(T.Tensor.from_numpy(i).sum(1).to_numpy(), i.sum(1))
+    np.testing.assert_array_equal(T.Tensor.from_numpy(i).max(0).to_numpy(), i.max(0))
+
+
+def test_sum_of_bf16_accumulates_in_f32(T):
+    from morok_amd import synth, uop
+
+    x = synth.to_bf16(np.full((4, 4096), 1.0 / 256, dtype=np.float32))
+    s = T.Tensor.from_numpy(x, uop.BF16).sum(1)
+    assert s.dtype == uop.BF16  # cast back after the promoted accumulation (reduce.rs:665-691)
+    np.testing.assert_array_equal(synth.from_bf16(s.to_numpy()), np.full(4, 16.0, np.float32))
+
+
+# ---------------------------------------------------------------- transformer.rs
+def test_rms_norm(T):
+    g = GOLD["rms_norm_basic"]
+    x = f32(g["x"])
+    got = T.Tensor.from_numpy(x).rms_norm(-1, g["eps"]).to_numpy()
+    np.testing.assert_allclose(got, x / np.sqrt(7.5 + 1e-5), atol=g["tol"])
+    g = GOLD["rms_norm_axis"]
+    x = f32(g["x"])
+    got = T.Tensor.from_numpy(x).rms_norm(-1, g["eps"]).to_numpy()
+    np.testing.assert_allclose(got, x / np.sqrt(f32(g["row_mean_sq"])[:, None] + g["eps"]), atol=g["tol"])
+
+
+def test_rms_norm_vs_oracle(T, oracle):
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((33, 4096)).astype(np.float32)
+    got = T.Tensor.from_numpy(x).rms_norm(-1, 1e-6).to_numpy()
+    np.testing.assert_allclose(got, oracle.rms_norm_f32(x, 1e-6), rtol=1e-5, atol=1e-6)
+
+
+def test_embedding(T):
+    g = GOLD["embedding_basic"]
+    w = T.Tensor.from_numpy(np.arange(12, dtype=np.float32).reshape(3, 4))
+    got = w.embedding(T.Tensor.from_numpy(np.array(g["indices"], dtype=np.int32))).to_numpy()
+    np.testing.assert_array_equal(got, f32(g["expected"]))
+    g = GOLD["embedding_2d"]
+    got = T.Tensor.from_numpy(f32(g["weight"])).embedding(T.Tensor.from_numpy(np.array(g["indices"], dtype=np.int32))).to_numpy()
+    np.testing.assert_array_equal(got, f32(g["expected"]))
+
+
+@pytest.mark.parametrize("key", ["rope_split", "rope_interleaved", "rope_rotation"])
+def test_rope_known_answers(T, key):
+    g = GOLD[key]
+    x = T.Tensor.from_numpy(f32(g["x"]).reshape(1, 1, 1, 4))
+    cos = T.Tensor.from_numpy(f32(g["cos"]).reshape(1, 1, 1, 2))
+    sin = T.Tensor.from_numpy(f32(g["sin"]).reshape(1, 1, 1, 2))
+    got = x.apply_rotary_emb(cos, sin, g["interleaved"]).to_numpy().reshape(-1)
+    np.testing.assert_allclose(got, f32(g["expected"]), atol=g["tol"])
+
+
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_rope_vs_oracle(T, oracle, interleaved):
+    rng = np.random.default_rng(19)
+    B, H, S, D = 2, 3, 17, 64
+    x = rng.standard_normal((B, H, S, D)).astype(np.float32)
+    ang = rng.uniform(0, 6.28, (S, D // 2)).astype(np.float32)
+    cos, sin = np.cos(ang), np.sin(ang)
+    got = T.Tensor.from_numpy(x).apply_rotary_emb(T.Tensor.from_numpy(cos.reshape(1, 1, S, D // 2)),
+                                                  T.Tensor.from_numpy(sin.reshape(1, 1, S, D // 2)), interleaved).to_numpy()
+    ref = oracle.rope_f32(x, cos, sin, interleaved)
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
+
+
+def test_sdpa_causal_row0(T, fusion):
+    g = GOLD["sdpa_causal_row0"]
+    q = T.Tensor.from_numpy(f32(g["q"]).reshape(1, 1, 3, 2))
+    v = T.Tensor.from_numpy(f32(g["v"]).reshape(1, 1, 3, 2))
+    out = q.scaled_dot_product_attention(q, v, is_causal=True).to_numpy()
+    assert out.shape == (1, 1, 3, 2)
+    np.testing.assert_allclose(out[0, 0, 0], f32(g["expected_row0"]), atol=g["tol"])
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_sdpa_f32_vs_oracle(T, fusion, oracle, causal):
+    rng = np.random.default_rng(23)
+    B, H, S, D = 2, 2, 40, 16
+    q, k, v = (rng.standard_normal((B, H, S, D)).astype(np.float32) for _ in range(3))
+    out = T.Tensor.from_numpy(q).scaled_dot_product_attention(T.Tensor.from_numpy(k), T.Tensor.from_numpy(v),
+                                                              is_causal=causal).to_numpy()
+    ref = oracle.sdpa_f32(q, k, v, 1 / np.sqrt(D), causal)
+    np.testing.assert_allclose(out, ref, rtol=1e-4, atol=1e-5)
+
+
+def test_sdpa_bf16_uses_flash(T, oracle):
+    from morok_amd import synth, uop
+
+    rng = np.random.default_rng(29)
+    B, H, S, D = 1, 2, 256, 128
+    q, k, v = (synth.to_bf16(rng.standard_normal((B, H, S, D)).astype(np.float32)) for _ in range(3))
+    t = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(T.Tensor.from_numpy(k, uop.BF16),
+                                                                      T.Tensor.from_numpy(v, uop.BF16), is_causal=True)
+    got = synth.from_bf16(t.to_numpy())
+    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("flash_fwd")
+    ref = synth.from_bf16(oracle.sdpa_bf16(q, k, v, 1 / np.sqrt(D), True))
+    assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
+
+
+def test_silu_and_sigmoid(T, oracle):
+    rng = np.random.default_rng(31)
+    x = (rng.standard_normal(5000) * 4).astype(np.float32)
+    got = T.Tensor.from_numpy(x).silu().to_numpy()
+    np.testing.assert_allclose(got, oracle.silu_f32(x), rtol=1e-5, atol=1e-6)
+    s = T.Tensor.from_numpy(x).sigmoid().to_numpy()
+    np.testing.assert_allclose(s, 1 / (1 + np.exp(-x.astype(np.float64))), rtol=1e-5, atol=1e-7)
+
+
+# ---------------------------------------------------------------- realize / caching
+def test_realize_reuses_cached_kernels(T):
+    from morok_amd import tensor
+
+    x = np.arange(1000, dtype=np.float32)
+    a = T.Tensor.from_numpy(x).try_mul(3.0).try_add(1.0)
+    a.realize()
+    first = tensor.last_cached_count()
+    b = T.Tensor.from_numpy(x + 1).try_mul(3.0).try_add(1.0)
+    b.realize()
+    assert tensor.last_cached_count() == 1 and first in (0, 1)  # same AST -> same kernel (kernel_cache.rs:87-118)
+    np.testing.assert_array_equal(b.to_numpy(), (x + 1) * 3 + 1)
+    # realizing again is a no-op; a consumer of a realized tensor reads its buffer
+    b.realize()
+    assert tensor.last_kernels() == []
+    c = b.try_sub(1.0)
+    np.testing.assert_array_equal(c.to_numpy(), (x + 1) * 3)
+    assert len(c.kernels()) == 1
+
+
+def test_contiguous_is_a_kernel_boundary(T):
+    x = np.arange(12, dtype=np.float32).reshape(3, 4)
+    t = T.Tensor.from_numpy(x).try_transpose(0, 1).contiguous()
+    y = t.try_add(1.0)
+    np.testing.assert_array_equal(y.to_numpy(), x.T + 1)
+    assert len(y.kernels()) == 2
+
+
+def test_large_elementwise_bandwidth_shape(T):
+    # 64 Mi elements: exercises the 2^31 byte range with int32 element indices
+    n = 1 << 26
+    from morok_amd import uop
+
+    t = T.Tensor.full([n], 1.5, uop.F32).try_mul(T.Tensor.full([n], 2.0, uop.F32)).contiguous()
+    s = t.sum(0)
+    assert float(s.to_numpy()) == 3.0 * n
