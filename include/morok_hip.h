@@ -407,6 +407,10 @@ int mrk_hip_tensor_sdpa(const mrk_tensor* q, const mrk_tensor* k, const mrk_tens
                         mrk_tensor** out);                                                    /* transformer.rs:78-137 */
 /* realization (realize.rs:83-127) and extraction (data.rs:211-236) */
 int mrk_hip_tensor_realize(const mrk_tensor* t);
+/* Tensor::prepare (realize.rs:299-357): schedule + compile into an execution plan without
+ * running it; the plan may be executed repeatedly (mrk_hip_plan_execute*), the tensor holds
+ * valid data once it has run.  Release with mrk_hip_plan_release. */
+int mrk_hip_tensor_prepare(const mrk_tensor* t, mrk_plan** out);
 int mrk_hip_tensor_to_bytes(const mrk_tensor* t, void* dst, size_t nbytes);
 /* Device buffer of a realized tensor (new handle sharing the allocation). */
 int mrk_hip_tensor_buffer(const mrk_tensor* t, mrk_buffer** out);
@@ -415,6 +419,9 @@ int mrk_hip_tensor_buffer(const mrk_tensor* t, mrk_buffer** out);
 void mrk_hip_tensor_set_fusion(int enabled);
 size_t mrk_hip_tensor_last_kernel_count(void);
 const char* mrk_hip_tensor_last_kernel_name(size_t i);
+/* Rendered HIP C of that kernel; "" for a hand-written kernel (CachedKernel::code,
+ * runtime/src/kernel_cache.rs:27-44). */
+const char* mrk_hip_tensor_last_kernel_source(size_t i);
 size_t mrk_hip_tensor_last_cached_count(void);
 double mrk_hip_tensor_last_elapsed_ms(void);
 

@@ -179,11 +179,13 @@ _SIGS = {
     "mrk_hip_tensor_rotary": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, c_void_pp]),
     "mrk_hip_tensor_sdpa": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_double, C.c_int, c_void_pp]),
     "mrk_hip_tensor_realize": (C.c_int, [C.c_void_p]),
+    "mrk_hip_tensor_prepare": (C.c_int, [C.c_void_p, c_void_pp]),
     "mrk_hip_tensor_to_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "mrk_hip_tensor_buffer": (C.c_int, [C.c_void_p, c_void_pp]),
     "mrk_hip_tensor_set_fusion": (None, [C.c_int]),
     "mrk_hip_tensor_last_kernel_count": (C.c_size_t, []),
     "mrk_hip_tensor_last_kernel_name": (C.c_char_p, [C.c_size_t]),
+    "mrk_hip_tensor_last_kernel_source": (C.c_char_p, [C.c_size_t]),
     "mrk_hip_tensor_last_cached_count": (C.c_size_t, []),
     "mrk_hip_tensor_last_elapsed_ms": (C.c_double, []),
 }

@@ -908,6 +908,14 @@ int mrk_hip_tensor_realize(const mrk_tensor* t) {
     MRK_NONNULL(t);
     return t->t.realize();
 }
+int mrk_hip_tensor_prepare(const mrk_tensor* t, mrk_plan** out) {
+    MRK_NONNULL(t);
+    MRK_NONNULL(out);
+    std::unique_ptr<ExecutionPlan> p;
+    MRK_TRY(t->t.prepare(&p));
+    *out = new mrk_plan{std::move(p)};
+    return kOk;
+}
 int mrk_hip_tensor_to_bytes(const mrk_tensor* t, void* dst, size_t nbytes) {
     MRK_NONNULL(t);
     if (nbytes) MRK_NONNULL(dst);
@@ -925,6 +933,10 @@ void mrk_hip_tensor_set_fusion(int enabled) { set_fusion_enabled(enabled != 0); 
 size_t mrk_hip_tensor_last_kernel_count(void) { return last_realize_stats().kernel_names.size(); }
 const char* mrk_hip_tensor_last_kernel_name(size_t i) {
     const auto& n = last_realize_stats().kernel_names;
+    return i < n.size() ? n[i].c_str() : nullptr;
+}
+const char* mrk_hip_tensor_last_kernel_source(size_t i) {
+    const auto& n = last_realize_stats().kernel_sources;
     return i < n.size() ? n[i].c_str() : nullptr;
 }
 size_t mrk_hip_tensor_last_cached_count(void) { return last_realize_stats().cached_kernels; }

@@ -60,12 +60,6 @@ const char* tc_dtype_name(Scalar s) {  // tc.rs:677-688
     }
 }
 
-int ilog2(int v) {
-    int r = 0;
-    while ((1 << (r + 1)) <= v) r++;
-    return r;
-}
-
 // logical axis of every l_i / u_i produced by the opts: (axis 0 = N, 1 = M; bit within axis).
 // Each opt splits its axis by 2 and the new range becomes the low part, so successive
 // splits of one axis take bits 0, 1, 2, ...
@@ -299,6 +293,48 @@ std::vector<size_t> GroupedDims::map(const std::vector<size_t>& raw) const {
 // ============================================================================ kernel builder
 uint32_t KernelBuilder::add(Op op, DType dt, std::vector<uint32_t> src, int64_t arg_i, double arg_f, uint16_t sub,
                             std::string str, std::vector<int64_t> extra) {
+    // Common-subexpression elimination for side-effect-free value nodes: an identical node
+    // that is still in scope is returned instead of a new one.
+    std::string key;
+    bool pure = false;
+    if (cse_) {
+        switch (op) {
+            case Op::Const:
+            case Op::Binary:
+            case Op::Unary:
+            case Op::Where:
+            case Op::Cast:
+            case Op::BitCast:
+            case Op::Gep:
+            case Op::Index:
+            case Op::Vectorize: pure = true; break;
+            default: break;
+        }
+    }
+    if (pure) {
+        auto put = [&](const void* p, size_t n) { key.append(static_cast<const char*>(p), n); };
+        uint16_t head[6] = {static_cast<uint16_t>(op), static_cast<uint16_t>(dt.scalar), dt.vcount,
+                            static_cast<uint16_t>(dt.is_ptr), static_cast<uint16_t>(dt.space), sub};
+        put(head, sizeof head);
+        put(&dt.ptr_size, sizeof dt.ptr_size);
+        put(&arg_i, sizeof arg_i);
+        put(&arg_f, sizeof arg_f);
+        for (uint32_t v : src) put(&v, sizeof v);
+        key.push_back('|');
+        for (int64_t v : extra) put(&v, sizeof v);
+        key.push_back('|');
+        key += str;
+        auto it = cse_map_.find(key);
+        if (it != cse_map_.end()) return it->second;
+    }
+    // scopes: values defined inside a loop or a conditional are not visible after it closes
+    if (cse_ && (op == Op::End || op == Op::EndIf)) {
+        size_t closes = op == Op::End ? std::max<size_t>(src.size(), 1) : 1;
+        for (size_t i = 0; i < closes && !cse_scopes_.empty(); i++) {
+            for (const std::string& k : cse_scopes_.back()) cse_map_.erase(k);
+            cse_scopes_.pop_back();
+        }
+    }
     UOp u;
     u.id = static_cast<uint32_t>(k_.nodes.size()) + 1;
     u.op = op;
@@ -310,7 +346,13 @@ uint32_t KernelBuilder::add(Op op, DType dt, std::vector<uint32_t> src, int64_t 
     u.str = std::move(str);
     u.extra = std::move(extra);
     k_.nodes.push_back(std::move(u));
-    return k_.nodes.back().id;
+    const uint32_t id = k_.nodes.back().id;
+    if (pure) {
+        cse_map_.emplace(key, id);
+        if (!cse_scopes_.empty()) cse_scopes_.back().push_back(std::move(key));
+    }
+    if (cse_ && (op == Op::Range || op == Op::If)) cse_scopes_.emplace_back();
+    return id;
 }
 
 uint32_t KernelBuilder::binary(BinaryOp op, uint32_t a, uint32_t b) {

@@ -7,6 +7,7 @@
 #pragma once
 #include <array>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "uop.h"
@@ -156,8 +157,14 @@ class KernelBuilder {
     LinearKernel finish();
     std::vector<uint8_t> serialize() const;
 
+    // Turns on common-subexpression elimination of pure value nodes (scope-aware).
+    void enable_cse() { cse_ = true; }
+
   private:
     LinearKernel k_;
+    bool cse_ = false;
+    std::unordered_map<std::string, uint32_t> cse_map_;
+    std::vector<std::vector<std::string>> cse_scopes_;
 };
 
 // Linearized kernels for the matmul shapes on the hot path.

@@ -6,6 +6,7 @@
 #include <cstring>
 #include <map>
 #include <set>
+#include <tuple>
 #include <unordered_map>
 
 #include "builtin.h"
@@ -520,17 +521,35 @@ Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& val
 // ============================================================================ scheduling
 namespace {
 
+// A coordinate while an expression is emitted: value = node + off.  `off` is a compile-time
+// constant, which lets the V elements one work-item produces (UPCAST of the innermost axis,
+// schedule/src/optimizer/heuristics.rs:37-82) share all index arithmetic and lets a load of
+// V consecutive elements become one vector load.  `aligned`: node is a multiple of the
+// upcast width and off lies in [0, width).
+struct Cx {
+    uint32_t node = 0;
+    int64_t off = 0;
+    bool aligned = false;
+    bool operator<(const Cx& o) const { return std::tie(node, off, aligned) < std::tie(o.node, o.off, o.aligned); }
+};
+using Coords = std::vector<Cx>;
+
 // One kernel under construction: the builder plus the device buffers it reads (slot 1..),
 // discovered while the expression is emitted.
 struct KernelGen {
+    KernelGen() { b.enable_cse(); }
     KernelBuilder b;
     Scalar idx_t = Scalar::Int32;
+    int64_t width = 1;  // upcast width of the innermost output axis
     std::vector<std::shared_ptr<Buffer>> inputs;
     std::vector<uint32_t> input_params;
     std::vector<Scalar> input_dtypes;
-    std::map<std::pair<const TensorNode*, std::vector<uint32_t>>, uint32_t> memo;
+    std::map<std::pair<const TensorNode*, Coords>, uint32_t> memo;
+    std::map<std::tuple<uint32_t, uint32_t, int64_t>, uint32_t> vec_loads;  // (param, base index, group) -> vector value
 
     uint32_t ci(int64_t v) { return b.ci(v, idx_t); }
+    uint32_t value(const Cx& c) { return c.off ? b.iadd(c.node, ci(c.off)) : c.node; }
+    Cx zero() { return Cx{ci(0), 0, true}; }
     uint32_t buffer_param(const std::shared_ptr<Buffer>& buf, Scalar dt, int64_t numel) {
         for (size_t i = 0; i < inputs.size(); i++)
             if (inputs[i].get() == buf.get() && input_dtypes[i] == dt) return input_params[i];
@@ -544,7 +563,7 @@ struct KernelGen {
 // half types are evaluated in f32
 Scalar compute_dtype(Scalar s) { return is_half(s) ? Scalar::Float32 : s; }
 
-uint32_t flatten(KernelGen& g, const std::vector<uint32_t>& coords, const std::vector<int64_t>& shape) {
+uint32_t flatten_nodes(KernelGen& g, const std::vector<uint32_t>& coords, const std::vector<int64_t>& shape) {
     uint32_t flat = g.ci(0);
     int64_t stride = 1;
     for (size_t i = shape.size(); i-- > 0;) {
@@ -571,14 +590,53 @@ std::vector<uint32_t> unflatten(KernelGen& g, uint32_t flat, const std::vector<i
     return coords;
 }
 
-uint32_t emit(KernelGen& g, const TensorNode* n, const std::vector<uint32_t>& coords);
+// Row-major flat index of `coords` in `shape` as (node, constant offset); *vec_ok tells whether
+// the node part is a multiple of the upcast width with the offset inside one group, i.e. the
+// elements off = 0..width-1 are consecutive in memory.
+Cx flatten(KernelGen& g, const Coords& coords, const std::vector<int64_t>& shape) {
+    std::vector<uint32_t> nodes(coords.size());
+    int64_t off = 0, stride = 1;
+    bool vec_ok = g.width > 1 && !shape.empty() && shape.back() % g.width == 0 && coords.back().aligned;
+    for (size_t i = shape.size(); i-- > 0;) {
+        nodes[i] = coords[i].node;
+        if (shape[i] != 1) off += coords[i].off * stride;
+        if (i + 1 != shape.size() && coords[i].off != 0 && shape[i] != 1) vec_ok = false;
+        stride *= shape[i];
+    }
+    if (!vec_ok && g.width > 1 && shape.empty()) vec_ok = false;
+    return Cx{flatten_nodes(g, nodes, shape), off, vec_ok && off >= 0 && off < g.width};
+}
 
-uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const std::vector<uint32_t>& coords) {
+uint32_t emit(KernelGen& g, const TensorNode* n, const Coords& coords);
+
+uint32_t emit_load(KernelGen& g, const TensorNode* n, const Coords& coords) {
+    KernelBuilder& b = g.b;
+    uint32_t p = g.buffer_param(n->buffer, n->dtype, n->numel());
+    Cx flat = flatten(g, coords, n->shape);
+    const int64_t per_load = std::min<int64_t>(g.width, 16 / static_cast<int64_t>(scalar_size(n->dtype)));
+    if (flat.aligned && per_load > 1 && n->dtype != Scalar::Bool) {
+        // one vector load per group of `per_load` consecutive elements, shared by the group
+        const int64_t group = flat.off / per_load;
+        auto key = std::make_tuple(p, flat.node, group);
+        auto it = g.vec_loads.find(key);
+        uint32_t vec;
+        if (it != g.vec_loads.end()) {
+            vec = it->second;
+        } else {
+            uint32_t at = group ? b.iadd(flat.node, g.ci(group * per_load)) : flat.node;
+            vec = b.load(b.index(p, at), static_cast<int>(per_load));
+            g.vec_loads[key] = vec;
+        }
+        return b.gep(vec, static_cast<int>(flat.off % per_load));
+    }
+    return b.load(b.index(p, g.value(flat)));
+}
+
+uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) {
     KernelBuilder& b = g.b;
     const Scalar ct = compute_dtype(n->dtype);
     if (n->buffer) {  // materialised tensor: a load from its row-major buffer
-        uint32_t p = g.buffer_param(n->buffer, n->dtype, n->numel());
-        uint32_t v = b.load(b.index(p, flatten(g, coords, n->shape)));
+        uint32_t v = emit_load(g, n, coords);
         return ct != n->dtype ? b.cast(v, ct) : v;
     }
     switch (n->kind) {
@@ -617,64 +675,81 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const std::vector<uint
                 if (s->shape[i] != 1) c.push_back(i);
             bool same = a.size() == c.size();
             for (size_t i = 0; same && i < a.size(); i++) same = n->shape[a[i]] == s->shape[c[i]];
-            std::vector<uint32_t> sc(s->shape.size());
+            Coords sc(s->shape.size());
             if (same) {
-                for (size_t i = 0; i < sc.size(); i++) sc[i] = g.ci(0);
+                for (size_t i = 0; i < sc.size(); i++) sc[i] = g.zero();
                 for (size_t i = 0; i < a.size(); i++) sc[c[i]] = coords[a[i]];
             } else {
-                sc = unflatten(g, flatten(g, coords, n->shape), s->shape);
+                Cx flat = flatten(g, coords, n->shape);
+                if (flat.aligned && !s->shape.empty() && s->shape.back() % g.width == 0) {
+                    // the whole group stays inside the innermost source dimension
+                    std::vector<uint32_t> u = unflatten(g, flat.node, s->shape);
+                    for (size_t i = 0; i < sc.size(); i++) sc[i] = Cx{u[i], 0, false};
+                    sc.back() = Cx{u.back(), flat.off, true};
+                } else {
+                    std::vector<uint32_t> u = unflatten(g, g.value(flat), s->shape);
+                    for (size_t i = 0; i < sc.size(); i++) sc[i] = Cx{u[i], 0, false};
+                }
             }
             return emit(g, s, sc);
         }
         case TKind::Permute: {
-            std::vector<uint32_t> sc(coords.size());
+            Coords sc(coords.size());
             for (size_t i = 0; i < coords.size(); i++) sc[n->arg[i]] = coords[i];
             return emit(g, n->src[0].get(), sc);
         }
         case TKind::Expand: {
             const TensorNode* s = n->src[0].get();
-            std::vector<uint32_t> sc = coords;
+            Coords sc = coords;
             for (size_t i = 0; i < sc.size(); i++)
-                if (s->shape[i] == 1 && n->shape[i] != 1) sc[i] = g.ci(0);
+                if (s->shape[i] == 1 && n->shape[i] != 1) sc[i] = g.zero();
             return emit(g, s, sc);
         }
         case TKind::Shrink: {
-            std::vector<uint32_t> sc = coords;
-            for (size_t i = 0; i < sc.size(); i++)
-                if (n->arg[i]) sc[i] = b.iadd(coords[i], g.ci(n->arg[i]));
+            Coords sc = coords;
+            for (size_t i = 0; i < sc.size(); i++) {
+                if (!n->arg[i]) continue;
+                if (sc[i].aligned && n->arg[i] % g.width == 0) sc[i].node = b.iadd(sc[i].node, g.ci(n->arg[i]));
+                else sc[i].off += n->arg[i], sc[i].aligned = false;
+            }
             return emit(g, n->src[0].get(), sc);
         }
         case TKind::Iota: {
-            uint32_t c = coords[n->arg[0]];
+            uint32_t c = g.value(coords[n->arg[0]]);
             return b.dtype(c).scalar == ct ? c : b.cast(c, ct);
         }
         case TKind::Cat: {
             const size_t axis = static_cast<size_t>(n->arg[0]);
             // every part is evaluated at a clamped coordinate; the right one is selected
-            int64_t off = 0;
+            bool groups = coords[axis].aligned;  // a whole upcast group falls into one part
+            for (const TensorRef& p : n->src) groups = groups && p->shape[axis] % g.width == 0;
+            const uint32_t pos = groups ? coords[axis].node : g.value(coords[axis]);
+            const int64_t span = groups ? g.width : 1;
+            int64_t start = 0;
             std::vector<uint32_t> vals;
             std::vector<int64_t> ends;
             for (const TensorRef& p : n->src) {
                 const int64_t len = p->shape[axis];
-                std::vector<uint32_t> sc = coords;
-                uint32_t rel = b.iadd(coords[axis], g.ci(-off));
+                Coords sc = coords;
+                uint32_t rel = b.iadd(pos, g.ci(-start));
                 uint32_t lo = b.where(b.binary(BinaryOp::Lt, rel, g.ci(0)), g.ci(0), rel);
-                sc[axis] = b.where(b.binary(BinaryOp::Gt, lo, g.ci(len - 1)), g.ci(len - 1), lo);
+                uint32_t cl = b.where(b.binary(BinaryOp::Gt, lo, g.ci(len - span)), g.ci(len - span), lo);
+                sc[axis] = groups ? Cx{cl, coords[axis].off, true} : Cx{cl, 0, false};
                 vals.push_back(emit(g, p.get(), sc));
-                off += len;
-                ends.push_back(off);
+                start += len;
+                ends.push_back(start);
             }
             uint32_t res = vals.back();
             for (size_t i = vals.size() - 1; i-- > 0;)
-                res = b.where(b.binary(BinaryOp::Lt, coords[axis], g.ci(ends[i])), vals[i], res);
+                res = b.where(b.binary(BinaryOp::Lt, pos, g.ci(ends[i])), vals[i], res);
             return res;
         }
         case TKind::Gather: {
             const TensorNode* w = n->src[0].get();
-            std::vector<uint32_t> ic(coords.begin(), coords.end() - 1);
+            Coords ic(coords.begin(), coords.end() - 1);
             uint32_t row = emit(g, n->src[1].get(), ic);
             if (b.dtype(row).scalar != g.idx_t) row = b.cast(row, g.idx_t);
-            return emit(g, w, {row, coords.back()});
+            return emit(g, w, {Cx{row, 0, false}, coords.back()});
         }
         case TKind::Reduce:
         case TKind::Buffer: break;  // always materialised before being read
@@ -682,13 +757,19 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const std::vector<uint
     return 0;
 }
 
-uint32_t emit(KernelGen& g, const TensorNode* n, const std::vector<uint32_t>& coords) {
+uint32_t emit(KernelGen& g, const TensorNode* n, const Coords& coords) {
     auto key = std::make_pair(n, coords);
     auto it = g.memo.find(key);
     if (it != g.memo.end()) return it->second;
     uint32_t v = emit_uncached(g, n, coords);
     g.memo[key] = v;
     return v;
+}
+
+Coords plain(const std::vector<uint32_t>& nodes) {
+    Coords c(nodes.size());
+    for (size_t i = 0; i < nodes.size(); i++) c[i] = Cx{nodes[i], 0, false};
+    return c;
 }
 
 struct Scheduler {
@@ -701,6 +782,7 @@ struct Scheduler {
         for (auto& bptr : bufs) idx.push_back(plan->add_buffer(bptr));
         MRK_TRY(plan->add_kernel(k, idx, {}));
         stats.kernel_names.push_back(k->entry_point);
+        stats.kernel_sources.push_back(k->code);
         if (cached) stats.cached_kernels++;
         return kOk;
     }
@@ -850,21 +932,40 @@ struct Scheduler {
         KernelBuilder& b = g.b;
         auto out = new_buffer(n);
         uint32_t po = b.param(0, n->dtype, N);
-        const int64_t block = 256, grid = (N + block - 1) / block;
+        // UPCAST of the innermost axis: one work-item produces `width` consecutive outputs
+        // (16 bytes of them) when the axis divides evenly
+        int64_t width = 1;
+        if (!n->shape.empty() && n->dtype != Scalar::Bool)
+            for (int64_t w = 16 / static_cast<int64_t>(scalar_size(n->dtype)); w > 1; w /= 2)
+                if (n->shape.back() % w == 0) {
+                    width = w;
+                    break;
+                }
+        g.width = width;
+        const int64_t items = N / width, block = 256, grid = (items + block - 1) / block;
         if (grid > 2147483647LL) return fail(kInvalidArgument, "realize: tensor too large for one launch");
         uint32_t gx = b.special("gidx0", grid), lx = b.special("lidx0", block);
         if (g.idx_t != Scalar::Int32) {
             gx = b.cast(gx, g.idx_t);
             lx = b.cast(lx, g.idx_t);
         }
-        uint32_t i = b.iadd(b.imul(gx, block), lx);
-        b.if_(b.binary(BinaryOp::Lt, i, g.ci(N)));
-        std::vector<uint32_t> coords = unflatten(g, i, n->shape);
-        uint32_t v = n->kind == TKind::Contiguous ? emit(g, n->src[0].get(), coords) : emit_uncached(g, n, coords);
-        if (b.dtype(v).scalar != n->dtype) v = b.cast(v, n->dtype);
-        b.store(b.index(po, i), v);
+        uint32_t item = b.iadd(b.imul(gx, block), lx);
+        b.if_(b.binary(BinaryOp::Lt, item, g.ci(items)));
+        uint32_t base = b.imul(item, width);
+        Coords coords = plain(unflatten(g, base, n->shape));
+        if (width > 1) coords.back().aligned = true;
+        std::vector<uint32_t> vals;
+        for (int64_t e = 0; e < width; e++) {
+            Coords ce = coords;
+            if (!ce.empty()) ce.back().off = e;
+            uint32_t v = n->kind == TKind::Contiguous ? emit(g, n->src[0].get(), ce) : emit_uncached(g, n, ce);
+            if (b.dtype(v).scalar != n->dtype) v = b.cast(v, n->dtype);
+            vals.push_back(v);
+        }
+        if (width > 1) b.store(b.index(po, base), b.vectorize(vals));
+        else b.store(b.index(po, base), vals[0]);
         b.endif();
-        return finish_kernel(g, n, out, "E_" + std::to_string(N));
+        return finish_kernel(g, n, out, "E_" + std::to_string(N) + (width > 1 ? "_" + std::to_string(width) : ""));
     }
 
     int gen_reduce(TensorNode* n, int64_t max_numel) {
@@ -899,13 +1000,13 @@ struct Scheduler {
             uint32_t o = b.iadd(b.imul(gx, block), lx);
             uint32_t gate = b.binary(BinaryOp::Lt, o, g.ci(Nout));
             uint32_t oc = b.where(gate, o, g.ci(Nout - 1));  // clamp: masked lanes recompute the last element
-            std::vector<uint32_t> coords = unflatten(g, oc, n->shape);
+            Coords coords = plain(unflatten(g, oc, n->shape));
             std::vector<uint32_t> ranges;
             for (size_t r = 0; r < n->arg.size(); r++) {
                 uint32_t rg = b.add(Op::Range, KernelBuilder::scalar(g.idx_t), {g.ci(rdims[r])}, static_cast<int64_t>(r), 0,
                                     static_cast<uint16_t>(AxisType::Reduce));
                 ranges.push_back(rg);
-                coords[n->arg[r]] = rg;
+                coords[n->arg[r]] = Cx{rg, 0, false};
             }
             uint32_t v = emit(g, s, coords);
             uint32_t red = b.reduce(op, v, ranges);
@@ -932,14 +1033,14 @@ struct Scheduler {
         uint32_t o = b.iadd(b.imul(gx, per_block), ly);
         uint32_t ogate = b.binary(BinaryOp::Lt, o, g.ci(Nout));
         uint32_t oc = b.where(ogate, o, g.ci(Nout - 1));
-        std::vector<uint32_t> coords = unflatten(g, oc, n->shape);
+        Coords coords = plain(unflatten(g, oc, n->shape));
         const int64_t steps = (R + 63) / 64;
         uint32_t rg = b.add(Op::Range, KernelBuilder::scalar(g.idx_t), {g.ci(steps)}, 0, 0, static_cast<uint16_t>(AxisType::Reduce));
         uint32_t f = b.iadd(b.imul(rg, 64), lane);
         uint32_t fgate = b.binary(BinaryOp::Lt, f, g.ci(R));
         uint32_t fc = (R % 64 == 0) ? f : b.where(fgate, f, g.ci(R - 1));
         std::vector<uint32_t> rc = unflatten(g, fc, rdims);
-        for (size_t r = 0; r < n->arg.size(); r++) coords[n->arg[r]] = rc[r];
+        for (size_t r = 0; r < n->arg.size(); r++) coords[n->arg[r]] = Cx{rc[r], 0, false};
         uint32_t v = emit(g, s, coords);
         if (R % 64 != 0) v = b.where(fgate, v, identity());
         uint32_t red = b.reduce(op, v, {rg});
@@ -957,19 +1058,33 @@ struct Scheduler {
 
 }  // namespace
 
-int Tensor::realize() const {
-    if (!n_) return fail(kInvalidArgument, "realize: invalid tensor");
+int Tensor::prepare(std::unique_ptr<ExecutionPlan>* out) const {
+    if (!n_) return fail(kInvalidArgument, "prepare: invalid tensor");
     g_stats = RealizeStats();
-    if (n_->buffer) return kOk;
     auto t0 = std::chrono::steady_clock::now();
     Scheduler s;
     MRK_TRY(DeviceFactoryRegistry::global().device("HIP", n_->device_id, &s.dev));
     s.plan.reset(new ExecutionPlan(n_->device_id));
-    MRK_TRY(s.materialize(n_.get()));
+    if (!n_->buffer) MRK_TRY(s.materialize(n_.get()));
+    s.plan->set_outputs({s.plan->add_buffer(n_->buffer)});
     MRK_TRY(s.plan->build());
-    MRK_TRY(s.plan->execute());
     s.stats.elapsed_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     g_stats = s.stats;
+    *out = std::move(s.plan);
+    return kOk;
+}
+
+int Tensor::realize() const {
+    if (!n_) return fail(kInvalidArgument, "realize: invalid tensor");
+    if (n_->buffer) {
+        g_stats = RealizeStats();
+        return kOk;
+    }
+    auto t0 = std::chrono::steady_clock::now();
+    std::unique_ptr<ExecutionPlan> plan;
+    MRK_TRY(prepare(&plan));
+    MRK_TRY(plan->execute());
+    g_stats.elapsed_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     return kOk;
 }
 

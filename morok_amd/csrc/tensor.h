@@ -65,6 +65,7 @@ struct TensorNode {
 // What the last realize() on this thread did (Tensor::kernels(), tensor/src/lib.rs:213).
 struct RealizeStats {
     std::vector<std::string> kernel_names;
+    std::vector<std::string> kernel_sources;  // rendered HIP C; empty for hand-written kernels
     size_t cached_kernels = 0;
     double elapsed_ms = 0.0;
 };
@@ -131,6 +132,10 @@ class Tensor {
 
     // ---- realization (realize.rs:83-127) and extraction (data.rs:211-236)
     int realize() const;
+    // Schedules and compiles without executing (Tensor::prepare, realize.rs:299-357): the
+    // returned plan can be executed any number of times; the tensor's buffer holds valid data
+    // once the plan has run.
+    int prepare(std::unique_ptr<class ExecutionPlan>* out) const;
     int to_bytes(void* dst, size_t nbytes) const;  // realize if needed, then copy out
     std::shared_ptr<Buffer> buffer() const { return n_ ? n_->buffer : nullptr; }
 

@@ -1,0 +1,72 @@
+"""A pre-norm decoder transformer block composed from the lazy tensor API (llama layout:
+RMSNorm -> QKV -> RoPE -> causal attention -> O-proj + residual -> RMSNorm -> SwiGLU MLP +
+residual).  morok has no decoder-block function of its own; this is the caller-side
+composition of its ops (tensor/src/transformer.rs:12-137, tensor/src/nn/norm.rs:92-111,
+tensor/src/activation.rs:309-318, tensor/src/matmul.rs:82-110) in bfloat16, with the casts
+back to bfloat16 that rms_norm's f32 promotion requires placed at each stage output.
+"""
+import numpy as np
+
+from . import synth, uop
+from .tensor import Tensor
+
+WEIGHT_NAMES = ("emb", "w_an", "Wq", "Wk", "Wv", "Wo", "w_fn", "W1", "W3", "W2")
+
+
+def rope_tables(seq, dim, theta=10000.0):
+    """cos/sin [seq, dim/2] in f32: angle(p, i) = p * theta^(-2i/dim)."""
+    inv = (theta ** (-np.arange(0, dim, 2, dtype=np.float64) / dim))
+    ang = np.arange(seq, dtype=np.float64)[:, None] * inv[None, :]
+    return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+
+def synthetic_weights(hidden, ffn, vocab, seed=0):
+    """Random-init bf16 weights (uint16 bit patterns), scaled so that activations stay O(1)."""
+    shapes = {"emb": (vocab, hidden), "w_an": (hidden,), "Wq": (hidden, hidden), "Wk": (hidden, hidden),
+              "Wv": (hidden, hidden), "Wo": (hidden, hidden), "w_fn": (hidden,), "W1": (hidden, ffn),
+              "W3": (hidden, ffn), "W2": (ffn, hidden)}
+    w = {}
+    for tid, name in enumerate(WEIGHT_NAMES):
+        shp = shapes[name]
+        if len(shp) == 1:
+            vals = 1.0 + synth.normal(shp, seed, 100 + tid, sigma=0.1)
+        else:
+            vals = synth.normal(shp, seed, 100 + tid, sigma=1.0 if name == "emb" else 1.0 / np.sqrt(shp[0]))
+        w[name] = synth.to_bf16(vals)
+    return w
+
+
+class DecoderBlock:
+    """Holds the device-resident weights and builds the lazy graph of one forward pass."""
+
+    def __init__(self, weights, batch, seq, hidden, heads, ffn, eps=1e-6, theta=10000.0, device_id=0):
+        assert hidden % heads == 0
+        self.batch, self.seq, self.hidden, self.heads, self.ffn, self.eps = batch, seq, hidden, heads, ffn, eps
+        self.dim = hidden // heads
+        self.w = {k: Tensor.from_numpy(np.ascontiguousarray(weights[k]), uop.BF16, device_id) for k in WEIGHT_NAMES}
+        cos, sin = rope_tables(seq, self.dim, theta)
+        self.cos_host, self.sin_host = cos, sin
+        self.cos = Tensor.from_numpy(cos.reshape(1, 1, seq, self.dim // 2), device_id=device_id)
+        self.sin = Tensor.from_numpy(sin.reshape(1, 1, seq, self.dim // 2), device_id=device_id)
+
+    def _heads(self, x):
+        """[T, hidden] token-major -> [B, H, S, D] head-major (a view: no copy by itself)."""
+        return x.try_reshape([self.batch, self.seq, self.heads, self.dim]).try_permute([0, 2, 1, 3])
+
+    def _norm(self, x, weight):
+        return x.rms_norm(-1, self.eps).try_mul(weight).cast(uop.BF16)
+
+    def forward(self, tokens):
+        """tokens: int32 Tensor [batch*seq].  Returns the lazy bf16 [batch*seq, hidden] output."""
+        w, T = self.w, self.batch * self.seq
+        h = w["emb"].embedding(tokens).contiguous()
+        xn = self._norm(h, w["w_an"])
+        q = self._heads(xn.matmul(w["Wq"])).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
+        k = self._heads(xn.matmul(w["Wk"])).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
+        v = self._heads(xn.matmul(w["Wv"]))
+        a = q.scaled_dot_product_attention(k, v, is_causal=True)
+        a = a.try_permute([0, 2, 1, 3]).try_reshape([T, self.hidden])
+        h2 = h.try_add(a.matmul(w["Wo"])).contiguous()
+        xn2 = self._norm(h2, w["w_fn"])
+        g = xn2.matmul(w["W1"]).silu().try_mul(xn2.matmul(w["W3"]))
+        return h2.try_add(g.matmul(w["W2"]))

@@ -419,10 +419,13 @@ def kernel_cache_clear():
 class ExecutionPlan:
     """ExecutionPlan + builder (runtime/src/execution_plan.rs:84-250,330-411)."""
 
-    def __init__(self, device_id=0):
-        h = C.c_void_p()
-        check(lib.mrk_hip_plan_create(device_id, C.byref(h)))
-        self._h = h
+    def __init__(self, device_id=0, _handle=None):
+        if _handle is not None:
+            self._h = _handle
+        else:
+            h = C.c_void_p()
+            check(lib.mrk_hip_plan_create(device_id, C.byref(h)))
+            self._h = h
         self._buffers = []
 
     def add_buffer(self, buf):

@@ -11,7 +11,7 @@ import numpy as np
 
 from . import uop
 from ._ffi import c_i64_p, check, lib
-from .device import Buffer
+from .device import Buffer, ExecutionPlan
 
 _NP_OF = {uop.F32: np.float32, uop.F64: np.float64, uop.F16: np.float16, uop.BF16: np.uint16, uop.I32: np.int32,
           uop.I64: np.int64, uop.U32: np.uint32, uop.U8: np.uint8, uop.I8: np.int8, uop.BOOL: np.bool_,
@@ -35,6 +35,11 @@ def set_fusion(enabled):
 def last_kernels():
     """Entry-point names of the kernels the last realize on this thread launched."""
     return [lib.mrk_hip_tensor_last_kernel_name(i).decode() for i in range(lib.mrk_hip_tensor_last_kernel_count())]
+
+
+def last_kernel_sources():
+    """Rendered HIP C per kernel of the last realize ("" for hand-written kernels)."""
+    return [lib.mrk_hip_tensor_last_kernel_source(i).decode() for i in range(lib.mrk_hip_tensor_last_kernel_count())]
 
 
 def last_cached_count():
@@ -248,6 +253,12 @@ class Tensor:
     def realize(self):
         check(lib.mrk_hip_tensor_realize(self._h))
         return self
+
+    def prepare(self):
+        """Tensor::prepare: schedule + compile into an ExecutionPlan without running it."""
+        h = C.c_void_p()
+        check(lib.mrk_hip_tensor_prepare(self._h, C.byref(h)))
+        return ExecutionPlan(_handle=h)
 
     def kernels(self):
         """Names of the kernels the last realize launched (tensor/src/lib.rs:213)."""

@@ -1,0 +1,74 @@
+"""Decoder transformer block composed from the lazy tensor API, against the CPU oracle's
+stage-by-stage restatement (bf16 storage, f32 math, one rounding per stage output)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def run_block(cfg, tokens, weights):
+    from morok_amd import decoder, tensor, uop
+
+    blk = decoder.DecoderBlock(weights, cfg["batch"], cfg["seq"], cfg["hidden"], cfg["heads"], cfg["ffn"], cfg["eps"])
+    out = blk.forward(tensor.Tensor.from_numpy(tokens.astype(np.int32)))
+    out.realize()
+    return blk, out, out.kernels()
+
+
+def rel_err(got_bits, ref_bits):
+    from morok_amd import synth
+
+    got, ref = synth.from_bf16(got_bits), synth.from_bf16(ref_bits)
+    return float(np.abs(got - ref).max() / np.abs(ref).max())
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(batch=2, seq=128, hidden=256, heads=2, ffn=512, vocab=1000, eps=1e-6),
+    dict(batch=1, seq=192, hidden=512, heads=4, ffn=1280, vocab=777, eps=1e-6),
+    dict(batch=1, seq=256, hidden=4096, heads=32, ffn=11008, vocab=32000, eps=1e-6),
+], ids=["h256", "h512", "h4096_seq256"])
+def test_decoder_block_vs_oracle(dev, oracle, cfg):
+    from morok_amd import decoder, synth
+
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], cfg["vocab"], seed=3)
+    T = cfg["batch"] * cfg["seq"]
+    tok = synth.randint((T,), 3, 1, cfg["vocab"])
+    blk, out, kernels = run_block(cfg, tok, w)
+    got = out.to_numpy()
+    ref = oracle.decoder_block_bf16(tok, w, blk.cos_host, blk.sin_host, cfg["batch"], cfg["seq"], cfg["hidden"],
+                                    cfg["heads"], cfg["ffn"], cfg["eps"])
+    assert got.shape == ref.shape == (T, cfg["hidden"])
+    assert rel_err(got, ref) <= 2e-2   # bf16 GEMM/attention tolerance
+    # the seven matmuls and the attention run as the hand-written kernels
+    assert sum(k.startswith("gemm_bf16") for k in kernels) == 7
+    assert sum(k.startswith("flash_fwd") for k in kernels) == 1
+
+
+def test_decoder_block_full_size_properties(dev):
+    """hidden 4096, 32 heads, SwiGLU 11008, batch 4 x seq 2048: too large for the CPU oracle in
+    a test, so checked through properties that hold at any size: determinism, independence of
+    batch entries, and causality (outputs before position p ignore tokens from p on)."""
+    from morok_amd import decoder, synth
+
+    cfg = dict(batch=4, seq=2048, hidden=4096, heads=32, ffn=11008, vocab=32000, eps=1e-6)
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], cfg["vocab"], seed=5)
+    T = cfg["batch"] * cfg["seq"]
+    tok = synth.randint((T,), 5, 1, cfg["vocab"])
+    _, out, kernels = run_block(cfg, tok, w)
+    a = out.to_numpy()
+    assert np.isfinite(synth.from_bf16(a)).all()
+    _, out2, _ = run_block(cfg, tok, w)
+    assert np.array_equal(a, out2.to_numpy())                       # deterministic
+    p = 1500
+    tok2 = tok.copy().reshape(cfg["batch"], cfg["seq"])
+    tok2[1, p:] = (tok2[1, p:] + 17) % cfg["vocab"]                 # change the tail of sequence 1
+    _, out3, _ = run_block(cfg, tok2.reshape(-1), w)
+    b = out3.to_numpy().reshape(cfg["batch"], cfg["seq"], -1)
+    a4 = a.reshape(cfg["batch"], cfg["seq"], -1)
+    assert np.array_equal(a4[0], b[0]) and np.array_equal(a4[2:], b[2:])   # other sequences untouched
+    assert np.array_equal(a4[1, :p], b[1, :p])                              # causal prefix untouched
+    assert not np.array_equal(a4[1, p:], b[1, p:])
+    # one sequence alone gives the same rows as inside the batch
+    cfg1 = dict(cfg, batch=1)
+    _, out4, _ = run_block(cfg1, tok[: cfg["seq"]], w)
+    assert np.array_equal(out4.to_numpy(), a4[0])

@@ -261,8 +261,10 @@ def test_tensor_kernel_cache_and_realize_idempotent(T, shim):
 
 def test_tensor_launch_dims(T, shim):
     T.set_fusion(False)
-    zeros(T, (1000,)).try_add(1.0).realize()
+    zeros(T, (1001,)).try_add(1.0).realize()
     assert hostshim_lib.last_dims(shim) == ((4, 1, 1), (256, 1, 1))
+    zeros(T, (8, 1000)).try_add(1.0).realize()      # innermost axis % 4 == 0: four outputs per work-item
+    assert hostshim_lib.last_dims(shim) == ((8, 1, 1), (256, 1, 1))
     zeros(T, (10, 4096)).sum(1).realize()           # one wavefront per output, four per workgroup
     assert hostshim_lib.last_dims(shim) == ((3, 1, 1), (64, 4, 1))
     zeros(T, (100, 16)).sum(1).realize()            # short rows: one work-item per output
@@ -276,3 +278,21 @@ def test_tensor_int64_indexing_for_huge_views(T, shim):
     t.realize()
     k = morok_amd.Kernel.get_or_compile  # noqa: F841  (the kernel compiled: the source is valid)
     assert len(t.kernels()) == 1
+
+
+def test_decoder_block_lowering(T, shim):
+    """The decoder block graph lowers to 7 GEMMs + 1 flash attention + the generated
+    elementwise / reduce kernels; weights and tokens never reach a real device here."""
+    from morok_amd import decoder, synth
+
+    cfg = dict(batch=2, seq=64, hidden=256, heads=2, ffn=512)
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], 100, seed=1)
+    blk = decoder.DecoderBlock(w, cfg["batch"], cfg["seq"], cfg["hidden"], cfg["heads"], cfg["ffn"])
+    n0 = shim.mrk_shim_launches()
+    out = blk.forward(T.Tensor.from_numpy(synth.randint((128,), 1, 1, 100))).realize()
+    names = out.kernels()
+    assert out.shape == (128, 256) and out.dtype == uop.BF16
+    assert sum(k.startswith("gemm_bf16") for k in names) == 7
+    assert sum(k.startswith("flash_fwd") for k in names) == 1
+    assert shim.mrk_shim_launches() - n0 == len(names)
+    print(names)
