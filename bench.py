@@ -29,6 +29,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
+# HBM bytes per launch of each dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
+# of this file (one counter per run), each scaled by what the same counter reads for the 256 MiB
+# copy kernel (FETCH_SIZE x2.000, WRITE_SIZE x0.999 on gfx950); summaries under profiles/.
+MIB = 1 << 20
+MEASURED_TRAFFIC = {"softmax": (256.1 + 255.7) * MIB, "gemm": (192.2 + 32.0) * MIB, "flash": (1029.1 + 255.7) * MIB}
 METRIC = "bf16 GEMM TFLOP/s & flash-attn fwd TFLOP/s (% of peak); softmax HBM GB/s"
 
 
@@ -58,20 +63,21 @@ def bench_softmax(m, dev, steps, warmup, cpu):
         "metric": "softmax HBM GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "f32",
         "config": {"workload": "row softmax f32 [8192x8192], normal(0,2), one fused kernel (configs[1])"},
         "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "softmax_rows_in_regs<256,8,1>",
+                     "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC["softmax"],
+                     "kernel": "softmax_rows_in_regs<256,8,1>",
                      "algorithmic_bytes_per_launch": algo_bytes},
     }
     if cpu:
         from tests.oracle_lib import Oracle
 
         orc = Oracle()
-        srows = 2048  # a quarter of the rows: ~1 s of CPU work per run
+        srows = 8192  # the whole matrix; 4 passes of it (1 warm-up + 3 timed)
         x = synth.normal((srows, cols), 2, 0, sigma=2.0)
         t = orc.thread_count(srows * cols, srows)
         sec = _cpu_time(lambda: orc.softmax_f32(x, threads=t))
         # the oracle runs the reference's 3-kernel schedule; its algorithmic bytes are the same 2*n*4
         rec["cpu_baseline"] = {"value": 2 * srows * cols * 4 / sec / 1e9, "unit": "GB/s", "cores": t, "kind": "port",
-                               "sample": f"{srows} of 8192 rows x 8192 cols, 3-kernel Clang-backend schedule, "
+                               "sample": f"all {srows} rows x 8192 cols, 3-kernel Clang-backend schedule, "
                                          f"{t} threads, min of 3 after 1 warm-up"}
     return rec
 
@@ -93,20 +99,20 @@ def bench_gemm(m, dev, steps, warmup, cpu):
         "metric": "bf16 GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "bf16",
         "config": {"workload": "bf16 GEMM M=N=K=4096, normal(0,1) inputs, f32 accumulate, bf16 out (configs[2])"},
         "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None, "kernel": "gemm_bf16_tile256",
+                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC["gemm"], "kernel": "gemm_bf16_tile256",
                      "algorithmic_flops_per_launch": flops},
     }
     if cpu:
         from tests.oracle_lib import Oracle
 
         orc = Oracle()
-        sm = 512  # 512 of the 4096 output rows: ~17 GFLOP of CPU work per run
+        sm = 4096  # the whole 4096^3 product: 137 GFLOP per run, 4 runs
         a = synth.normal_bf16((sm, K), 3, 0)
         b = synth.normal_bf16((K, N), 3, 1)
         t = orc.thread_count(sm * N * K, sm)
         sec = _cpu_time(lambda: orc.gemm_bf16(a, b, threads=t))
         rec["cpu_baseline"] = {"value": 2.0 * sm * N * K / sec / 1e12, "unit": "TFLOP/s", "cores": t, "kind": "port",
-                               "sample": f"{sm} of 4096 output rows (K=N=4096), f32-accumulate bf16 matmul kernel, "
+                               "sample": f"all {sm} output rows (K=N=4096), f32-accumulate bf16 matmul kernel, "
                                          f"{t} threads, min of 3 after 1 warm-up"}
     return rec
 
@@ -131,22 +137,67 @@ def bench_flash(m, dev, steps, warmup, cpu):
         "steps": steps,
         "config": {"workload": "causal flash-attention fwd, bf16 [8,32,4096,128], scale 1/sqrt(128) (configs[3])"},
         "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None, "kernel": "flash_fwd_d128",
+                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC["flash"], "kernel": "flash_fwd_d128",
                      "algorithmic_flops_per_launch": flops},
     }
     if cpu:
         from tests.oracle_lib import Oracle
 
         orc = Oracle()
-        q = synth.normal_bf16((S, D), 4, 0)
-        k = synth.normal_bf16((S, D), 4, 1)
-        v = synth.normal_bf16((S, D), 4, 2)
+        sl = 16  # 16 of the 256 (batch, head) slices at full sequence length
+        q = synth.normal_bf16((1, sl, S, D), 4, 0)
+        k = synth.normal_bf16((1, sl, S, D), 4, 1)
+        v = synth.normal_bf16((1, sl, S, D), 4, 2)
         t = orc.max_threads
-        sec = _cpu_time(lambda: orc.sdpa_bf16_rows(q, k, v, scale, causal=True, threads=t))
-        rec["cpu_baseline"] = {"value": 0.5 * 4.0 * S * S * D / sec / 1e12, "unit": "TFLOP/s", "cores": t,
+        sec = _cpu_time(lambda: orc.sdpa_bf16(q, k, v, scale, causal=True, threads=t))
+        rec["cpu_baseline"] = {"value": 0.5 * 4.0 * sl * S * S * D / sec / 1e12, "unit": "TFLOP/s", "cores": t,
                                "kind": "port",
-                               "sample": f"one (batch, head) slice of 256 at S=4096, D=128, causal, rows split over {t} "
-                                         "threads, min of 3 after 1 warm-up; per-unit rate, the full job is 256 such slices"}
+                               "sample": f"{sl} of the 256 (batch, head) slices at S=4096, D=128, causal, one slice per "
+                                         f"thread over {t} threads, min of 3 after 1 warm-up"}
+    return rec
+
+
+def bench_decoder(m, dev, steps, warmup, cpu):
+    """configs[4]: decoder transformer block from the tensor API, bf16, hidden 4096, 32 heads x 128,
+    SwiGLU 11008, RMSNorm eps 1e-6, RoPE theta 1e4, batch 4 x seq 2048 prefill, vocab 32000."""
+    from morok_amd import decoder, synth, tensor
+
+    B, S, hidden, heads, ffn, vocab = 4, 2048, 4096, 32, 11008, 32000
+    T = B * S
+    w = decoder.synthetic_weights(hidden, ffn, vocab, seed=5)
+    blk = decoder.DecoderBlock(w, B, S, hidden, heads, ffn, eps=1e-6, theta=10000.0)
+    tok = tensor.Tensor.from_numpy(synth.randint((T,), 5, 1, vocab))
+    plan = blk.forward(tok).prepare()      # schedule + compile once (Tensor::prepare), then execute per step
+    steps = max(1, min(steps, 20))
+    ms = m.time_launches(plan.execute, steps, min(warmup, 3))
+    prof = plan.execute_profiled()
+    gemm_ms = sum(t for n, t in prof if n.startswith("gemm_bf16"))
+    flash_ms = sum(t for n, t in prof if n.startswith("flash_fwd"))
+    flops = 2.0 * T * hidden * (4 * hidden + 3 * ffn) + 0.5 * 4.0 * B * heads * S * S * (hidden // heads)
+    tf = flops / (ms * 1e-3) / 1e12
+    rec = {
+        "metric": "decoder block TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "bf16",
+        "steps": steps, "tokens_per_s": T / (ms * 1e-3),
+        "config": {"workload": "decoder block via tensor API: hidden 4096, 32x128 heads, SwiGLU 11008, batch 4 x seq 2048 "
+                               "prefill (configs[4])"},
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None, "kernel": "gemm_bf16_tile256 (7 of the 20 kernels)",
+                     "algorithmic_flops_per_launch": flops},
+        "kernels": len(prof), "gemm_ms": gemm_ms, "flash_ms": flash_ms, "other_ms": sum(t for _, t in prof) - gemm_ms - flash_ms,
+    }
+    if cpu:
+        from tests.oracle_lib import Oracle
+
+        orc = Oracle()
+        sb, ss = 1, 512  # one sequence of 512 tokens through the full-width block
+        stok = synth.randint((sb * ss,), 5, 1, vocab)
+        cos, sin = decoder.rope_tables(ss, hidden // heads)
+        t = orc.max_threads
+        sec = _cpu_time(lambda: orc.decoder_block_bf16(stok, w, cos, sin, sb, ss, hidden, heads, ffn, 1e-6, threads=t))
+        sflops = 2.0 * sb * ss * hidden * (4 * hidden + 3 * ffn) + 0.5 * 4.0 * sb * heads * ss * ss * (hidden // heads)
+        rec["cpu_baseline"] = {"value": sflops / sec / 1e12, "unit": "TFLOP/s", "cores": t, "kind": "port",
+                               "sample": f"batch {sb} x seq {ss} through the full-width block (same weights), {t} threads, "
+                                         "min of 3 after 1 warm-up"}
     return rec
 
 
@@ -167,8 +218,9 @@ def bench_copy(m, dev, steps, warmup, cpu):
                          "algorithmic_bytes_per_launch": 2 * nbytes}}
 
 
-WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "copy": bench_copy}
-PRIMARY_ORDER = ["gemm", "flash", "softmax"]
+WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "decoder": bench_decoder,
+             "copy": bench_copy}
+PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder"]
 
 
 def main():
