@@ -21,6 +21,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <type_traits>
 
 #include "kernels.h"
 
@@ -41,10 +42,18 @@ constexpr int kKT = 64;        // keys per tile
 constexpr int kRow = kD * 2;   // 256 B per K/V row
 constexpr int kTile = kKT * kRow;  // 16 KB
 
+// max(x of lane l, x of lane l ^ 32): the swap exchanges the upper 32 lanes of its first
+// register with the lower 32 lanes of its second, which leaves one register holding the
+// lower half twice and the other the upper half twice.
+__device__ __forceinline__ float max_with_other_half(float x) {
+    float a = x, b = x;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+
 __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
                                                          const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
                                                          int Sq, int Sk, float scale_log2e, int causal, int q_tiles, int units) {
-    // K stage s at s*32 KB, V stage s at s*32 KB + 16 KB
     __shared__ __attribute__((aligned(1024))) char smem[4 * kTile];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // Workgroup ids congruent mod 8 run on the same XCD and share its L2.  Each XCD walks
@@ -93,21 +102,29 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
                      : "s"(lds_addr), "v"(voff), "s"(sbase)
                      : "m0");
     };
-    auto dma_tile = [&](int j, int stage) {
+    // LDS map: K stage s at s*16 KB, V stage s at 32 KB + s*16 KB
+    auto dma_k = [&](int j, int stage) {
 #pragma unroll
         for (int c = 0; c < 4; c++) {
             const int row = wave * 16 + c * 4 + r4;  // row inside the tile
             int key = j * kKT + row;
             key = key < Sk ? key : Sk - 1;  // ragged tail: re-read the last row, masked later
-            // K: 16 B chunk c16 of the LDS row holds logical chunk c16 ^ (row & 15): the LDS
+            // 16 B chunk c16 of the LDS row holds logical chunk c16 ^ (row & 15): the LDS
             // serves 16 lanes x 16 B per cycle over 64 banks, so 16 consecutive rows must
             // land in 16 different chunk slots
             const unsigned kvoff = (unsigned)key * kRow + ((c16 ^ (row & 15)) << 4);
-            // V: 32 B granule (c16 >> 1) holds logical granule (c16 >> 1) ^ (row & 3)
+            dma(lds_base + stage * kTile + (wave * 16 + c * 4) * kRow, kvoff, Kh);
+        }
+    };
+    auto dma_v = [&](int j, int stage) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const int row = wave * 16 + c * 4 + r4;
+            int key = j * kKT + row;
+            key = key < Sk ? key : Sk - 1;
+            // 32 B granule (c16 >> 1) holds logical granule (c16 >> 1) ^ (row & 3)
             const unsigned vvoff = (unsigned)key * kRow + (((((c16 >> 1) ^ (row & 3)) << 1) | (c16 & 1)) << 4);
-            const unsigned dst = lds_base + stage * 2 * kTile + (wave * 16 + c * 4) * kRow;
-            dma(dst, kvoff, Kh);
-            dma(dst + kTile, vvoff, Vh);
+            dma(lds_base + 2 * kTile + stage * kTile + (wave * 16 + c * 4) * kRow, vvoff, Vh);
         }
     };
     auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
@@ -147,47 +164,40 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
     const int v_row_off = (4 * lg + v_rr) * kRow + 8 * (lane & 3);
     const int v_half = (lane >> 4) & 1;
 
-    if (pass) tile_barrier();  // every wave is done reading the previous pass's last tile
-    dma_tile(0, 0);
-    for (int j = 0; j < ntiles; j++) {
-        const int stage = j & 1;
-        tile_barrier();  // tile j landed; every wave is done with tile j-1
-        if (j + 1 < ntiles) dma_tile(j + 1, stage ^ 1);
-        const int key0 = j * kKT;
-        // (a wave whose queries all precede the tile still runs it fully masked: P = 0 adds
-        // nothing, and a branch-free body keeps the accumulators in place)
-        const char* sK = smem + stage * 2 * kTile;
-        const char* sV = sK + kTile;
+    // first tile that needs masking for this wave: the causal diagonal (a tile is clear of
+    // it iff its last key <= the wave's first query) or the ragged tail of the keys
+    int first_masked = (Sk % kKT) ? Sk / kKT : ntiles;
+    if (causal && qw0 / kKT < first_masked) first_masked = qw0 / kKT;
+    const int qidx = qw0 + lq;
+    const int lim = causal ? (qidx < Sk - 1 ? qidx : Sk - 1) : Sk - 1;  // last visible key
 
-        // ---- S^T = K Q^T (K fragments fetched one d-step ahead of the MFMAs that use them)
-        f32x16 st[2];
+    // S^T = K Q^T for one tile (K fragments fetched one d-step ahead of their MFMAs),
+    // then the mask and the row maximum.  Register e of block kb is key
+    // key0 + kb*32 + 8*(e/4) + 4*(l/32) + e%4.
+    auto qk_tile = [&](const char* sK, f32x16 (&st)[2]) {
 #pragma unroll
         for (int kb = 0; kb < 2; kb++)
 #pragma unroll
             for (int e = 0; e < 16; e++) st[kb][e] = 0.0f;
-        {
-            bf16x8 kf[2][2];
+        bf16x8 kf[2][2];
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-                kf[0][kb] = *LDS_PTR(bf16x8, sK + kb * 32 * kRow + k_row_off + (((0 + lg) ^ k_sw) << 4));
+        for (int kb = 0; kb < 2; kb++)
+            kf[0][kb] = *LDS_PTR(bf16x8, sK + kb * 32 * kRow + k_row_off + (((0 + lg) ^ k_sw) << 4));
 #pragma unroll
-            for (int ds = 0; ds < 8; ds++) {
-                if (ds + 1 < 8) {
-#pragma unroll
-                    for (int kb = 0; kb < 2; kb++)
-                        kf[(ds + 1) & 1][kb] =
-                            *LDS_PTR(bf16x8, sK + kb * 32 * kRow + k_row_off + (((2 * (ds + 1) + lg) ^ k_sw) << 4));
-                }
+        for (int ds = 0; ds < 8; ds++) {
+            if (ds + 1 < 8) {
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++)
-                    st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds & 1][kb], qf[ds], st[kb], 0, 0, 0);
+                    kf[(ds + 1) & 1][kb] =
+                        *LDS_PTR(bf16x8, sK + kb * 32 * kRow + k_row_off + (((2 * (ds + 1) + lg) ^ k_sw) << 4));
             }
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+                st[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds & 1][kb], qf[ds], st[kb], 0, 0, 0);
         }
-        // ---- mask: register e of block kb is key key0 + kb*32 + 8*(e/4) + 4*(l/32) + e%4
-        const bool need_mask = (causal && key0 + kKT - 1 > qw0) || (key0 + kKT > Sk);
-        if (need_mask) {
-            const int qidx = qw0 + lq;
-            const int lim = causal ? (qidx < Sk - 1 ? qidx : Sk - 1) : Sk - 1;  // last visible key
+    };
+    auto mask_and_max = [&](f32x16 (&st)[2], int key0, bool mask) -> float {
+        if (mask) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
@@ -196,47 +206,90 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
                     if (key > lim) st[kb][e] = -INFINITY;
                 }
         }
-        // ---- online softmax, all in the lane that owns the query
-        float mx = st[0][0];
+        float mx0 = st[0][0], mx1 = st[1][0];
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-            for (int e = 0; e < 16; e++) mx = fmaxf(mx, st[kb][e]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        // Lazy rescaling: the exponentials are taken relative to m_run, which is only moved
-        // (and the accumulators rescaled) when some row's maximum has grown by more than
-        // kLazy / scale_log2e, i.e. when a probability could exceed 2^kLazy.  Rounding P to
-        // bf16 is relative and the row sum is f32, so the result does not depend on which
-        // reference the exponentials use.  The first tile always takes the branch
-        // (m_run = -inf); key 0 is visible to every query, so m_run is finite from then on.
-        if (__builtin_amdgcn_ballot_w64(mx > m_run + lazy_thresh) != 0) {
-            const float m_new = fmaxf(m_run, mx);
+        for (int e = 1; e < 16; e++) {
+            mx0 = fmaxf(mx0, st[0][e]);
+            mx1 = fmaxf(mx1, st[1][e]);
+        }
+        const float mx = fmaxf(mx0, mx1);
+        // the other 16 keys of every 32 sit in lane l ^ 32
+        return max_with_other_half(mx);
+    };
+
+    // One loop iteration, software-pipelined inside the wave: while the matrix pipe runs
+    // S(j+1) = K(j+1) Q^T the vector ALUs turn S(j) into P(j); while it runs
+    // O += V(j)^T P(j)^T they find the row maximum of S(j+1).  The iteration starts with the
+    // (rare) rescale decided by that maximum, so the pipelined part is one basic block.
+    // Lazy rescaling: exponentials are taken relative to m_run, which only moves (and the
+    // accumulators are rescaled) when some row's maximum has grown by more than
+    // kLazy / scale_log2e, i.e. when a probability could exceed 2^kLazy.  Rounding P to bf16
+    // is relative and the row sum is f32, so the result does not depend on the reference
+    // point.  The first tile always rescales (m_run = -inf); key 0 is visible to every
+    // query, so m_run is finite from then on.
+    auto body = [&](int j, f32x16 (&cur)[2], float mx_cur, f32x16 (&nxt)[2], float& mx_nxt, auto mask_next) {
+        if (__builtin_amdgcn_ballot_w64(mx_cur > m_run + lazy_thresh) != 0) {
+            const float m_new = fmaxf(m_run, mx_cur);
             const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
             m_run = m_new;
             l_run *= alpha;
 #pragma unroll
             for (int db = 0; db < 4; db++) o[db] *= alpha;
         }
+        // K(j+1) and V(j) have landed; every wave is done with K(j) and V(j-1)
+        tile_barrier();
+        if (j + 2 < ntiles) dma_k(j + 2, j & 1);
+        if (j + 1 < ntiles) dma_v(j + 1, (j + 1) & 1);
+        const char* sKn = smem + ((j + 1) & 1) * kTile;
+        const char* sV = smem + 2 * kTile + (j & 1) * kTile;
         const float mb = m_run * scale_log2e;
-        float psum = 0.0f;
+
+        // ---- phase A: S(j+1) = K(j+1) Q^T on the matrix pipe, P(j) = exp2(S(j)*c - m*c) on
+        // the vector ALUs: each of the 16 MFMAs is followed by the exponentials of two score
+        // registers (the last iteration computes a tile nobody uses).  The fences keep the
+        // compiler from regrouping the two instruction streams.
+        float psum0 = 0.0f, psum1 = 0.0f;
         bf16x8 pb[2][2];
+        {
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
-                f32x8 p;
+                for (int e = 0; e < 16; e++) nxt[kb][e] = 0.0f;
+            bf16x8 kf[2][2];
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(st[kb][8 * t + e], scale_log2e, -mb));
-                    psum += p[e];
+            for (int kb = 0; kb < 2; kb++)
+                kf[0][kb] = *LDS_PTR(bf16x8, sKn + kb * 32 * kRow + k_row_off + (((0 + lg) ^ k_sw) << 4));
+            f32x8 p;
+#pragma unroll
+            for (int ds = 0; ds < 8; ds++) {
+                if (ds + 1 < 8) {
+#pragma unroll
+                    for (int kb = 0; kb < 2; kb++)
+                        kf[(ds + 1) & 1][kb] =
+                            *LDS_PTR(bf16x8, sKn + kb * 32 * kRow + k_row_off + (((2 * (ds + 1) + lg) ^ k_sw) << 4));
                 }
-                pb[kb][t] = __builtin_convertvector(p, bf16x8);
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+                    nxt[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds & 1][kb], qf[ds], nxt[kb], 0, 0, 0);
+                    const int idx = ds * 2 + kb;           // 0..15: score registers 2*idx, 2*idx+1
+                    const int pk = idx >> 3, pe = (idx & 7) * 2;  // block, register inside the block
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe], scale_log2e, -mb));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe + 1], scale_log2e, -mb));
+                    psum0 += p0;
+                    psum1 += p1;
+                    p[pe & 7] = p0;
+                    p[(pe & 7) + 1] = p1;
+                    if ((idx & 3) == 3) pb[pk][(idx >> 2) & 1] = __builtin_convertvector(p, bf16x8);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
         }
-        l_run += psum;
+        l_run += psum0 + psum1;
 
-        // ---- O^T += V^T P^T.  MFMA (kb, t) contracts over the 16 keys held in registers
-        // 8t .. 8t+7 of block kb: keys kb*32 + 16t + {0, 8} + 4*(l/32) + 0..3.
+        // ---- phase B: O^T += V(j)^T P(j)^T on the matrix pipe, mask and row maximum of
+        // S(j+1) on the vector ALUs.  MFMA (kb, t) contracts over the 16 keys held in
+        // registers 8t .. 8t+7 of block kb: keys kb*32 + 16t + {0, 8} + 4*(l/32) + 0..3.
+        float mx0 = -INFINITY, mx1 = -INFINITY;
         {
             auto vfrag = [&](int n) {  // n = (kb*2 + t)*4 + db
                 const int kbt = n >> 2, db = n & 3;
@@ -248,14 +301,67 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
             bf16x8 vf[3];
             vf[0] = vfrag(0);
             vf[1] = vfrag(1);
+            const int key0n = (j + 1) * kKT;
 #pragma unroll
             for (int n = 0; n < 16; n++) {
                 if (n + 2 < 16) vf[(n + 2) % 3] = vfrag(n + 2);
                 o[n & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[n % 3], pb[n >> 3][(n >> 2) & 1], o[n & 3], 0, 0, 0);
+                if (n >= 8) {  // the score MFMAs have drained by now: 4 registers per slot
+                    const int kb = (n - 8) >> 2, e0 = ((n - 8) & 3) * 4;
+#pragma unroll
+                    for (int e = e0; e < e0 + 4; e++) {
+                        if (decltype(mask_next)::value) {
+                            const int key = key0n + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3);
+                            if (key > lim) nxt[kb][e] = -INFINITY;
+                        }
+                        if (e & 1) mx1 = fmaxf(mx1, nxt[kb][e]);
+                        else mx0 = fmaxf(mx0, nxt[kb][e]);
+                    }
+                    // pins the partial maxima to this slot (pure operations are otherwise
+                    // free to sink below the last MFMA)
+                    asm volatile("" : "+v"(mx0), "+v"(mx1));
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
+        {
+            const float mx = fmaxf(mx0, mx1);
+            // the other 16 keys of every 32 sit in lane l ^ 32
+            mx_nxt = max_with_other_half(mx);
+        }
+    };
+
+    if (pass) tile_barrier();  // every wave is done reading the previous pass's tiles
+    dma_k(0, 0);
+    dma_v(0, 0);
+    if (ntiles > 1) dma_k(1, 1);
+    tile_barrier();
+    f32x16 sa[2], sb[2];
+    float mxa, mxb = 0.0f;
+    qk_tile(smem, sa);
+    mxa = mask_and_max(sa, 0, first_masked <= 0);
+    {
+        int j = 0;
+        const int jm = first_masked - 1 < ntiles ? first_masked - 1 : ntiles;  // iterations whose next tile is unmasked
+        for (; j + 1 < jm; j += 2) {
+            body(j, sa, mxa, sb, mxb, std::false_type{});
+            body(j + 1, sb, mxb, sa, mxa, std::false_type{});
+        }
+        if (j < jm) {
+            body(j, sa, mxa, sb, mxb, std::false_type{});
+            sa[0] = sb[0];
+            sa[1] = sb[1];
+            mxa = mxb;
+            j++;
+        }
+        for (; j + 1 < ntiles; j += 2) {
+            body(j, sa, mxa, sb, mxb, std::true_type{});
+            body(j + 1, sb, mxb, sa, mxa, std::true_type{});
+        }
+        if (j < ntiles) body(j, sa, mxa, sb, mxb, std::true_type{});
     }
 
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     // ---- normalise and store: lane holds O[q = qw0 + l%32][d = db*32 + 8*(e/4) + 4*(l/32) + e%4]
     const float l_tot = l_run + __shfl_xor(l_run, 32);
     const float inv = 1.0f / l_tot;
