@@ -37,6 +37,24 @@ MEASURED_TRAFFIC = {"softmax": (256.1 + 255.7) * MIB, "gemm": (192.2 + 32.0) * M
 METRIC = "bf16 GEMM TFLOP/s & flash-attn fwd TFLOP/s (% of peak); softmax HBM GB/s"
 
 
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _launch_stats(m, fn, steps, warmup):
+    """Average over exactly `steps` launches (one event pair around all of them), then a second
+    pass with one event pair per launch for the median and the minimum."""
+    ms = m.time_launches(fn, steps, warmup)
+    med, mn = m.time_each_launch(fn, max(steps, 20), 0)
+    return ms, {"median_ms": med, "min_ms": mn}
+
+
 def _cpu_time(fn):
     fn()  # warm-up
     best = float("inf")
@@ -56,7 +74,7 @@ def bench_softmax(m, dev, steps, warmup, cpu):
     bx = dev.buffer(n * 4).ensure_allocated()
     by = dev.buffer(n * 4).ensure_allocated()
     ops.fill_normal(bx, n, sigma=2.0, seed=2, tensor_id=0)
-    ms = m.time_launches(lambda: ops.softmax_f32(bx, by, rows, cols), steps, warmup)
+    ms, stats = _launch_stats(m, lambda: ops.softmax_f32(bx, by, rows, cols), steps, warmup)
     algo_bytes = 2 * n * 4  # one read + one write of the matrix
     gbs = algo_bytes / (ms * 1e-3) / 1e9
     rec = {
@@ -67,6 +85,7 @@ def bench_softmax(m, dev, steps, warmup, cpu):
                      "kernel": "softmax_rows_in_regs<256,8,1>",
                      "algorithmic_bytes_per_launch": algo_bytes},
     }
+    rec.update(stats)
     if cpu:
         from tests.oracle_lib import Oracle
 
@@ -92,7 +111,7 @@ def bench_gemm(m, dev, steps, warmup, cpu):
     bc = dev.buffer(M * N * 2).ensure_allocated()
     ops.fill_normal(ba, M * K, seed=3, tensor_id=0, bf16=True)
     ops.fill_normal(bb, K * N, seed=3, tensor_id=1, bf16=True)
-    ms = m.time_launches(lambda: ops.gemm_bf16(ba, bb, bc, M, N, K), steps, warmup)
+    ms, stats = _launch_stats(m, lambda: ops.gemm_bf16(ba, bb, bc, M, N, K), steps, warmup)
     flops = 2.0 * M * N * K
     tf = flops / (ms * 1e-3) / 1e12
     rec = {
@@ -102,6 +121,7 @@ def bench_gemm(m, dev, steps, warmup, cpu):
                      "frac": tf / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC["gemm"], "kernel": "gemm_bf16_tile256",
                      "algorithmic_flops_per_launch": flops},
     }
+    rec.update(stats)
     if cpu:
         from tests.oracle_lib import Oracle
 
@@ -128,8 +148,8 @@ def bench_flash(m, dev, steps, warmup, cpu):
         ops.fill_normal(b, n, seed=4, tensor_id=i, bf16=True)
     scale = 1.0 / np.sqrt(D)
     steps = max(1, min(steps, 20))
-    ms = m.time_launches(lambda: ops.flash_attn_fwd_bf16(bq, bk, bv, bo, B, H, S, S, D, scale, True), steps,
-                         min(warmup, 3))
+    ms, stats = _launch_stats(m, lambda: ops.flash_attn_fwd_bf16(bq, bk, bv, bo, B, H, S, S, D, scale, True), steps,
+                              min(warmup, 3))
     flops = 0.5 * 4.0 * B * H * S * S * D  # causal convention: half of the dense 4*B*H*S^2*D
     tf = flops / (ms * 1e-3) / 1e12
     rec = {
@@ -140,6 +160,7 @@ def bench_flash(m, dev, steps, warmup, cpu):
                      "frac": tf / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC["flash"], "kernel": "flash_fwd_d128",
                      "algorithmic_flops_per_launch": flops},
     }
+    rec.update(stats)
     if cpu:
         from tests.oracle_lib import Oracle
 
@@ -169,7 +190,7 @@ def bench_decoder(m, dev, steps, warmup, cpu):
     tok = tensor.Tensor.from_numpy(synth.randint((T,), 5, 1, vocab))
     plan = blk.forward(tok).prepare()      # schedule + compile once (Tensor::prepare), then execute per step
     steps = max(1, min(steps, 20))
-    ms = m.time_launches(plan.execute, steps, min(warmup, 3))
+    ms, stats = _launch_stats(m, plan.execute, steps, min(warmup, 3))
     prof = plan.execute_profiled()
     gemm_ms = sum(t for n, t in prof if n.startswith("gemm_bf16"))
     flash_ms = sum(t for n, t in prof if n.startswith("flash_fwd"))
@@ -185,6 +206,7 @@ def bench_decoder(m, dev, steps, warmup, cpu):
                      "algorithmic_flops_per_launch": flops},
         "kernels": len(prof), "gemm_ms": gemm_ms, "flash_ms": flash_ms, "other_ms": sum(t for _, t in prof) - gemm_ms - flash_ms,
     }
+    rec.update(stats)
     if cpu:
         from tests.oracle_lib import Oracle
 
@@ -201,6 +223,41 @@ def bench_decoder(m, dev, steps, warmup, cpu):
     return rec
 
 
+def bench_matmul_f32(m, dev, steps, warmup, cpu):
+    """configs[0]: f32 matmul through Tensor::matmul, A[1024x1024] @ B[1024x1024], uniform(-1,1), seed 1
+    (plumbing + correctness: lazy graph -> schedule -> render -> hiprtc -> launch)."""
+    from morok_amd import synth, tensor
+
+    n = 1024
+    a = synth.uniform((n, n), 1, 0)
+    b = synth.uniform((n, n), 1, 1)
+    ta, tb = tensor.Tensor.from_numpy(a), tensor.Tensor.from_numpy(b)
+    c = ta.matmul(tb)
+    plan = c.prepare()
+    ms, stats = _launch_stats(m, plan.execute, steps, warmup)
+    flops = 2.0 * n ** 3
+    tf = flops / (ms * 1e-3) / 1e12
+    rec = {
+        "metric": "f32 matmul TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "f32",
+        "config": {"workload": "f32 matmul 1024^3 via the lazy tensor API, generated kernel (configs[0])"},
+        "roofline": {"bound": "mfma", "achieved": tf, "peak": 157.3, "unit": "TFLOP/s", "frac": tf / 157.3,
+                     "traffic": None, "kernel": plan.kernel_name(0), "algorithmic_flops_per_launch": flops},
+    }
+    rec.update(stats)
+    if cpu:
+        from tests.oracle_lib import Oracle
+
+        orc = Oracle()
+        t = orc.thread_count(n * n * n, n)
+        sec = _cpu_time(lambda: orc.matmul_f32(a, b, threads=t))
+        got = c.to_numpy()
+        ref = orc.matmul_f32(a, b, threads=t)
+        rec["max_rel_err_vs_cpu"] = float(np.abs(got - ref).max() / np.abs(ref).max())
+        rec["cpu_baseline"] = {"value": flops / sec / 1e12, "unit": "TFLOP/s", "cores": t, "kind": "port",
+                               "sample": f"the whole 1024^3 product, {t} threads, min of 3 after 1 warm-up"}
+    return rec
+
+
 def bench_copy(m, dev, steps, warmup, cpu):
     """Calibration only: 256 MiB streaming copy kernel (known traffic 2 x 256 MiB per launch)."""
     from morok_amd import ops
@@ -209,9 +266,9 @@ def bench_copy(m, dev, steps, warmup, cpu):
     bx = dev.buffer(nbytes).ensure_allocated()
     by = dev.buffer(nbytes).ensure_allocated()
     ops.fill_normal(bx, nbytes // 4, seed=9)
-    ms = m.time_launches(lambda: ops.copy_kernel(bx, by, nbytes), steps, warmup)
+    ms, stats = _launch_stats(m, lambda: ops.copy_kernel(bx, by, nbytes), steps, warmup)
     gbs = 2 * nbytes / (ms * 1e-3) / 1e9
-    return {"metric": "copy GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "u8",
+    return {"metric": "copy GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "u8", **stats,
             "config": {"workload": "calibration: 256 MiB streaming copy kernel"},
             "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": gbs / HBM_PEAK_GBS, "traffic": None, "kernel": "copy_kernel",
@@ -219,8 +276,8 @@ def bench_copy(m, dev, steps, warmup, cpu):
 
 
 WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "decoder": bench_decoder,
-             "copy": bench_copy}
-PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder"]
+             "matmul_f32": bench_matmul_f32, "copy": bench_copy}
+PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32"]
 
 
 def main():
@@ -253,6 +310,14 @@ def main():
         "dtype": primary["dtype"], "data": "synthetic", "config": primary["config"],
         "roofline": primary["roofline"],
     }
+    cpu_model = _cpu_model()
+    for r in recs:
+        if "cpu_baseline" in r:
+            r["cpu_baseline"]["cpu_model"] = cpu_model
+            r["cpu_baseline"]["host_cores"] = os.cpu_count()
+    for k in ("median_ms", "min_ms"):
+        if k in primary:
+            line[k] = primary[k]
     if "cpu_baseline" in primary:
         line["cpu_baseline"] = primary["cpu_baseline"]
     if len(recs) > 1:

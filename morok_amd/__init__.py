@@ -6,7 +6,7 @@ from ._ffi import MorokHipError, lib, declared_symbols  # noqa: F401
 from .device import (  # noqa: F401
     Buffer, CompiledSpec, Device, Event, ExecutionPlan, Kernel, Program, ProgramSpec, TimelineSignal,
     benchmark_kernel, cache_key, compile_spec, device_count, kernel_cache_clear, kernel_cache_size, parse_device,
-    time_launches,
+    time_each_launch, time_launches,
 )
 from . import ops  # noqa: F401
 from . import uop  # noqa: F401

@@ -359,6 +359,20 @@ def time_launches(fn, iters, warmup=3, device_id=0):
     return e0.elapsed_ms(e1) / iters
 
 
+def time_each_launch(fn, iters, warmup=3, device_id=0):
+    """Per-launch milliseconds (one event pair per call): returns (median, minimum)."""
+    for _ in range(warmup):
+        fn()
+    events = [Event(device_id) for _ in range(iters + 1)]
+    events[0].record()
+    for i in range(iters):
+        fn()
+        events[i + 1].record()
+    events[-1].synchronize()
+    ms = sorted(events[i].elapsed_ms(events[i + 1]) for i in range(iters))
+    return ms[len(ms) // 2], ms[0]
+
+
 class Kernel:
     """Arc<CachedKernel> (runtime/src/kernel_cache.rs:27-44), obtained through the global
     kernel cache."""
