@@ -33,7 +33,7 @@ BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
 # of this file (one counter per run), each scaled by what the same counter reads for the 256 MiB
 # copy kernel (FETCH_SIZE x2.000, WRITE_SIZE x0.999 on gfx950); summaries under profiles/.
 MIB = 1 << 20
-MEASURED_TRAFFIC = {"softmax": (256.1 + 255.7) * MIB, "gemm": (192.2 + 32.0) * MIB, "flash": (1029.1 + 255.7) * MIB}
+MEASURED_TRAFFIC = {"softmax": (256.1 + 255.7) * MIB, "gemm": (192.2 + 32.0) * MIB, "flash": (1024.8 + 255.9) * MIB}
 METRIC = "bf16 GEMM TFLOP/s & flash-attn fwd TFLOP/s (% of peak); softmax HBM GB/s"
 
 
