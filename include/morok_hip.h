@@ -295,6 +295,33 @@ int mrk_hip_sched_build_matmul_f32(int64_t m, int64_t n, int64_t k, uint8_t** ke
 int mrk_hip_sched_build_wmma_matmul(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, uint8_t** kernel,
                                     size_t* len);
 void mrk_hip_sched_free(void* p);
+/* The f32 matmul kernel with the optimisation choices explicit: opts = {LOCAL x, LOCAL y,
+ * UPCAST of N (vector width 1/2/4), UPCAST of M (rows per work-item 1..8), UNROLL of K}.
+ * INVALID_ARGUMENT when the choices do not divide the shape (the action space of
+ * schedule/src/optimizer/beam.rs:36-120 restricted to this kernel). */
+int mrk_hip_sched_build_matmul_f32_opts(int64_t m, int64_t n, int64_t k, const int opts[5], uint8_t** kernel, size_t* len);
+
+/* =====================================================================================
+ * Beam-search support (tensor/src/realize.rs:1190-1242, schedule/src/optimizer/beam.rs)
+ * ===================================================================================== */
+/* compile_and_time: render + compile + load (not timed), then warm-up and `runs` timed
+ * launches with HIP events on the device stream; *min_ms is the minimum
+ * (runtime/src/benchmark.rs:23-27,64-91).  Candidates are timed one at a time however many
+ * threads call this.  A candidate that does not render / compile / launch returns a status,
+ * it never aborts the process. */
+int mrk_hip_compile_and_time(int device_id, const void* kernel, size_t len, const char* name, mrk_buffer* const* buffers,
+                             size_t nbufs, const int64_t* vals, size_t nvals, int warmup, int runs, double* min_ms);
+/* On-disk result cache keyed (ast_hash, beam_width, device string) (beam.rs:390-440; sled in the
+ * reference, one file per key here, under $MOROK_CACHE_DIR | $XDG_CACHE_HOME/morok |
+ * $HOME/.cache/morok, in beam_cache_hip/).  get: *len = 0 on a miss (and always when
+ * IGNORE_BEAM_CACHE is set); INVALID_ARGUMENT if the value exceeds capacity. */
+int mrk_hip_beam_cache_get(uint64_t ast_hash, int width, const char* device, void* value, size_t capacity, size_t* len);
+int mrk_hip_beam_cache_put(uint64_t ast_hash, int width, const char* device, const void* value, size_t len);
+/* Beam search of width `width` over LOCAL / UPCAST / UNROLL for the f32 matmul of this shape;
+ * result in opts (same layout as above), its time in *best_ms, *from_cache = 1 when the disk
+ * cache answered, *timed = number of candidates compiled and timed. */
+int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t k, int width, int opts[5],
+                                   double* best_ms, int* from_cache, int* timed);
 
 /* =====================================================================================
  * Hand-written kernels, direct entry points (device pointers, queued on the device stream)

@@ -148,6 +148,11 @@ _SIGS = {
     "mrk_hip_event_synchronize": (C.c_int, [C.c_void_p]),
     "mrk_hip_event_elapsed_ms": (C.c_int, [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]),
     "mrk_hip_event_destroy": (None, [C.c_void_p]),
+    "mrk_hip_sched_build_matmul_f32_opts": (C.c_int, [C.c_int64, C.c_int64, C.c_int64, C.POINTER(C.c_int), C.POINTER(C.POINTER(C.c_uint8)), c_size_p]),
+    "mrk_hip_compile_and_time": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_char_p, c_void_pp, C.c_size_t, c_i64_p, C.c_size_t, C.c_int, C.c_int, C.POINTER(C.c_double)]),
+    "mrk_hip_beam_cache_get": (C.c_int, [C.c_uint64, C.c_int, C.c_char_p, C.c_void_p, C.c_size_t, c_size_p]),
+    "mrk_hip_beam_cache_put": (C.c_int, [C.c_uint64, C.c_int, C.c_char_p, C.c_void_p, C.c_size_t]),
+    "mrk_hip_beam_search_matmul_f32": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_double), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     # lazy tensors
     "mrk_hip_tensor_from_bytes": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),
     "mrk_hip_tensor_from_buffer": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),

@@ -618,6 +618,76 @@ int mrk_hip_sched_build_wmma_matmul(int tc_index, int64_t m, int64_t n, int64_t 
     return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
 }
 void mrk_hip_sched_free(void* p) { std::free(p); }
+int mrk_hip_sched_build_matmul_f32_opts(int64_t m, int64_t n, int64_t k, const int opts[5], uint8_t** kernel, size_t* len) {
+    MRK_NONNULL(opts);
+    MRK_NONNULL(kernel);
+    MRK_NONNULL(len);
+    MatmulF32Opts o{opts[0], opts[1], opts[2], opts[3], opts[4]};
+    if (!matmul_f32_opts_valid(o, m, n, k))
+        return fail(kInvalidArgument, "matmul f32: LOCAL/UPCAST/UNROLL choices do not fit the shape");
+    LinearKernel lk = build_matmul_f32_kernel(m, n, k, o);
+    return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
+}
+
+int mrk_hip_compile_and_time(int device_id, const void* kernel, size_t len, const char* name, mrk_buffer* const* buffers,
+                             size_t nbufs, const int64_t* vals, size_t nvals, int warmup, int runs, double* min_ms) {
+    MRK_NONNULL(kernel);
+    MRK_NONNULL(min_ms);
+    if (nbufs) MRK_NONNULL(buffers);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    LinearKernel k;
+    MRK_TRY(parse_linear_kernel(static_cast<const uint8_t*>(kernel), len, &k));
+    std::vector<void*> ptrs(nbufs);
+    for (size_t i = 0; i < nbufs; i++) {
+        MRK_NONNULL(buffers[i]);
+        MRK_TRY(buffers[i]->b->ensure_allocated());
+        MRK_TRY(buffers[i]->b->as_raw_ptr(&ptrs[i]));
+    }
+    BenchmarkResult r;
+    MRK_TRY(compile_and_time(*d, k, name, ptrs.data(), nbufs, vals, nvals, warmup, runs, &r));
+    *min_ms = r.min_ms;
+    return kOk;
+}
+int mrk_hip_beam_cache_get(uint64_t ast_hash, int width, const char* device, void* value, size_t capacity, size_t* len) {
+    MRK_NONNULL(device);
+    MRK_NONNULL(len);
+    std::vector<uint8_t> v;
+    *len = 0;
+    if (!BeamCache::get(ast_hash, width, device, &v)) return kOk;
+    if (v.size() > capacity) return fail(kInvalidArgument, "beam cache: value larger than the buffer");
+    if (!v.empty()) {
+        MRK_NONNULL(value);
+        std::memcpy(value, v.data(), v.size());
+    }
+    *len = v.size();
+    return kOk;
+}
+int mrk_hip_beam_cache_put(uint64_t ast_hash, int width, const char* device, const void* value, size_t len) {
+    MRK_NONNULL(device);
+    if (len) MRK_NONNULL(value);
+    return BeamCache::put(ast_hash, width, device, value, len);
+}
+int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t k, int width, int opts[5],
+                                   double* best_ms, int* from_cache, int* timed) {
+    MRK_NONNULL(opts);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    MatmulF32Opts o;
+    bool cached = false;
+    int n_timed = 0;
+    double ms = 0;
+    MRK_TRY(beam_search_matmul_f32(*d, m, n, k, width, &o, &ms, &cached, &n_timed));
+    opts[0] = o.local_x;
+    opts[1] = o.local_y;
+    opts[2] = o.up_n;
+    opts[3] = o.up_m;
+    opts[4] = o.unroll_k;
+    if (best_ms) *best_ms = ms;
+    if (from_cache) *from_cache = cached ? 1 : 0;
+    if (timed) *timed = n_timed;
+    return kOk;
+}
 
 int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t rows, int64_t cols, int variant) {
     if (rows < 0 || cols < 0) return fail(kInvalidArgument, "softmax_f32: negative shape");

@@ -1,8 +1,16 @@
 #include "runtime.h"
 
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <algorithm>
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <thread>
+
+#include "schedule.h"
 
 #include "error.h"
 #include "uop.h"
@@ -214,6 +222,192 @@ int benchmark_kernel(int device_id, ffi::Stream stream, Program* program, void* 
     out->max_ms = mx;
     out->mean_ms = sum / runs;
     out->runs = runs;
+    return kOk;
+}
+
+int compile_and_time(const Device& dev, const LinearKernel& k, const char* name, void* const* buffers, size_t nbufs,
+                     const int64_t* vals, size_t nvals, int warmup, int runs, BenchmarkResult* out) {
+    ProgramSpec spec;
+    MRK_TRY(dev.renderer->render(k, name, &spec));
+    if (spec.buf_count != nbufs)
+        return failf(kInvalidArgument, "compile_and_time: kernel takes %zu buffers, got %zu", spec.buf_count, nbufs);
+    CompiledSpec compiled;
+    MRK_TRY(dev.compiler->compile(spec, &compiled));
+    std::unique_ptr<Program> program;
+    MRK_TRY(dev.runtime(compiled, &program));
+    static std::mutex timing_lock;
+    std::lock_guard<std::mutex> lock(timing_lock);
+    return benchmark_kernel(dev.device_id, dev.allocator->stream(), program.get(), buffers, nbufs, vals, nvals,
+                            spec.has_sizes ? spec.global_size.data() : nullptr,
+                            spec.has_sizes ? spec.local_size.data() : nullptr, warmup, runs, out);
+}
+
+std::string BeamCache::directory() {
+    std::string base;
+    if (const char* d = std::getenv("MOROK_CACHE_DIR")) base = d;
+    else if (const char* x = std::getenv("XDG_CACHE_HOME")) base = std::string(x) + "/morok";
+    else if (const char* h = std::getenv("HOME")) base = std::string(h) + "/.cache/morok";
+    else base = "/tmp/morok";
+    return base + "/beam_cache_hip";
+}
+
+static std::string beam_key_path(uint64_t ast_hash, int width, const std::string& device) {
+    std::string id = std::to_string(ast_hash) + ":" + std::to_string(width) + ":" + device;
+    char name[40];
+    std::snprintf(name, sizeof name, "%016llx", static_cast<unsigned long long>(
+                      fnv1a64(reinterpret_cast<const uint8_t*>(id.data()), id.size())));
+    return BeamCache::directory() + "/" + name;
+}
+
+bool BeamCache::get(uint64_t ast_hash, int width, const std::string& device, std::vector<uint8_t>* value) {
+    if (const char* ig = std::getenv("IGNORE_BEAM_CACHE"))
+        if (ig[0] && ig[0] != '0') return false;
+    std::FILE* f = std::fopen(beam_key_path(ast_hash, width, device).c_str(), "rb");
+    if (!f) return false;
+    // record: the full key (collision check), then the value
+    uint64_t h = 0;
+    int32_t w = 0;
+    uint32_t dlen = 0, vlen = 0;
+    bool ok = std::fread(&h, 8, 1, f) == 1 && std::fread(&w, 4, 1, f) == 1 && std::fread(&dlen, 4, 1, f) == 1 && dlen < 256;
+    std::string dev(dlen, '\0');
+    ok = ok && (dlen == 0 || std::fread(&dev[0], 1, dlen, f) == dlen) && std::fread(&vlen, 4, 1, f) == 1 && vlen < (1u << 20);
+    if (ok) {
+        value->resize(vlen);
+        ok = (vlen == 0 || std::fread(value->data(), 1, vlen, f) == vlen) && h == ast_hash && w == width && dev == device;
+    }
+    std::fclose(f);
+    return ok;
+}
+
+int BeamCache::put(uint64_t ast_hash, int width, const std::string& device, const void* value, size_t len) {
+    const std::string dir = directory();
+    // mkdir -p
+    for (size_t i = 1; i <= dir.size(); i++)
+        if (i == dir.size() || dir[i] == '/') ::mkdir(dir.substr(0, i).c_str(), 0755);
+    const std::string path = beam_key_path(ast_hash, width, device);
+    const std::string tmp = path + ".tmp." + std::to_string(static_cast<long long>(::getpid()));
+    std::FILE* f = std::fopen(tmp.c_str(), "wb");
+    if (!f) return failf(kRuntime, "runtime error: cannot write beam cache entry %s", tmp.c_str());
+    const int32_t w = width;
+    const uint32_t dlen = static_cast<uint32_t>(device.size()), vlen = static_cast<uint32_t>(len);
+    bool ok = std::fwrite(&ast_hash, 8, 1, f) == 1 && std::fwrite(&w, 4, 1, f) == 1 && std::fwrite(&dlen, 4, 1, f) == 1 &&
+              (dlen == 0 || std::fwrite(device.data(), 1, dlen, f) == dlen) && std::fwrite(&vlen, 4, 1, f) == 1 &&
+              (vlen == 0 || std::fwrite(value, 1, vlen, f) == vlen);
+    ok = std::fclose(f) == 0 && ok;
+    if (!ok || std::rename(tmp.c_str(), path.c_str()) != 0) {  // rename: readers never see a partial entry
+        std::remove(tmp.c_str());
+        return failf(kRuntime, "runtime error: cannot write beam cache entry %s", path.c_str());
+    }
+    return kOk;
+}
+
+int beam_search_matmul_f32(const Device& dev, int64_t M, int64_t N, int64_t K, int width, MatmulF32Opts* best,
+                           double* best_ms, bool* from_cache, int* candidates_timed) {
+    if (width < 1) return fail(kInvalidArgument, "beam search: width must be >= 1");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(kInvalidArgument, "beam search: empty matmul");
+    const std::string device = "HIP:" + std::to_string(dev.device_id);
+    const std::string id = "matmul_f32:" + std::to_string(M) + "x" + std::to_string(N) + "x" + std::to_string(K);
+    const uint64_t ast_hash = fnv1a64(reinterpret_cast<const uint8_t*>(id.data()), id.size());
+    if (from_cache) *from_cache = false;
+    if (candidates_timed) *candidates_timed = 0;
+    std::vector<uint8_t> cached;
+    struct Record {
+        int32_t opts[5];
+        double ms;
+    };
+    if (BeamCache::get(ast_hash, width, device, &cached) && cached.size() == sizeof(Record)) {
+        Record r;
+        std::memcpy(&r, cached.data(), sizeof r);
+        MatmulF32Opts o{r.opts[0], r.opts[1], r.opts[2], r.opts[3], r.opts[4]};
+        if (matmul_f32_opts_valid(o, M, N, K)) {
+            *best = o;
+            if (best_ms) *best_ms = r.ms;
+            if (from_cache) *from_cache = true;
+            return kOk;
+        }
+    }
+    // scratch operands (contents are irrelevant for timing; zero-filled to keep the FPU quiet)
+    BufferOptions bo;
+    bo.zero_init = true;
+    Buffer a(dev.allocator, static_cast<size_t>(M * K) * 4, bo), b(dev.allocator, static_cast<size_t>(K * N) * 4, bo),
+        c(dev.allocator, static_cast<size_t>(M * N) * 4, bo);
+    MRK_TRY(a.ensure_allocated());
+    MRK_TRY(b.ensure_allocated());
+    MRK_TRY(c.ensure_allocated());
+    void* ptrs[3];
+    MRK_TRY(c.as_raw_ptr(&ptrs[0]));
+    MRK_TRY(a.as_raw_ptr(&ptrs[1]));
+    MRK_TRY(b.as_raw_ptr(&ptrs[2]));
+
+    using Cand = std::pair<double, MatmulF32Opts>;
+    auto time_one = [&](const MatmulF32Opts& o, double* ms) -> bool {
+        if (!matmul_f32_opts_valid(o, M, N, K)) return false;
+        BenchmarkResult r;
+        LinearKernel k = build_matmul_f32_kernel(M, N, K, o);
+        // warm-up 1, 3 runs, minimum: runtime/src/benchmark.rs:23-27
+        if (compile_and_time(dev, k, "beam_candidate", ptrs, 3, nullptr, 0, 1, 3, &r) != kOk) return false;  // a failing candidate is skipped
+        if (candidates_timed) (*candidates_timed)++;
+        *ms = r.min_ms;
+        return true;
+    };
+    auto keep_best = [&](std::vector<Cand>& v) {
+        std::sort(v.begin(), v.end(), [](const Cand& x, const Cand& y) { return x.first < y.first; });
+        if (static_cast<int>(v.size()) > width) v.resize(width);
+    };
+    // stage 1: LOCAL
+    std::vector<Cand> beam;
+    static const int locals[][2] = {{16, 16}, {32, 8}, {8, 32}, {64, 4}, {16, 8}, {32, 4}, {8, 8}, {64, 1}, {32, 2}};
+    for (auto& l : locals) {
+        MatmulF32Opts o;
+        o.local_x = l[0];
+        o.local_y = l[1];
+        double ms;
+        if (time_one(o, &ms)) beam.emplace_back(ms, o);
+    }
+    if (beam.empty()) {  // shapes the default tiling does not divide: scalar columns, one row
+        static const int small[][2] = {{16, 16}, {32, 8}, {8, 8}, {16, 4}, {4, 4}, {2, 2}, {1, 1}};
+        for (auto& l : small) {
+            MatmulF32Opts o{l[0], l[1], 1, 1, 1};
+            double ms;
+            if (time_one(o, &ms)) beam.emplace_back(ms, o);
+        }
+    }
+    if (beam.empty()) return fail(kInvalidArgument, "beam search: no valid candidate for this shape");
+    keep_best(beam);
+    // stage 2: UPCAST
+    {
+        std::vector<Cand> next = beam;
+        for (const Cand& cnd : beam)
+            for (int un : {4, 2, 1})
+                for (int um : {8, 4, 2, 1}) {
+                    MatmulF32Opts o = cnd.second;
+                    if (o.up_n == un && o.up_m == um) continue;
+                    o.up_n = un;
+                    o.up_m = um;
+                    double ms;
+                    if (time_one(o, &ms)) next.emplace_back(ms, o);
+                }
+        beam = next;
+        keep_best(beam);
+    }
+    // stage 3: UNROLL
+    {
+        std::vector<Cand> next = beam;
+        for (const Cand& cnd : beam)
+            for (int u : {2, 4, 8}) {
+                MatmulF32Opts o = cnd.second;
+                o.unroll_k = u;
+                double ms;
+                if (time_one(o, &ms)) next.emplace_back(ms, o);
+            }
+        beam = next;
+        keep_best(beam);
+    }
+    *best = beam[0].second;
+    if (best_ms) *best_ms = beam[0].first;
+    Record r{{best->local_x, best->local_y, best->up_n, best->up_m, best->unroll_k}, beam[0].first};
+    (void)BeamCache::put(ast_hash, width, device, &r, sizeof r);  // a read-only cache directory is not an error
+    clear_error();
     return kOk;
 }
 

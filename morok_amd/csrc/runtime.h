@@ -110,6 +110,33 @@ int benchmark_kernel(int device_id, ffi::Stream stream, Program* program, void* 
                      const int64_t* vals, size_t nvals, const size_t* global, const size_t* local, int warmup,
                      int runs, BenchmarkResult* out);
 
+// Beam-search timing hook (tensor/src/realize.rs:1190-1242): render and compile `k` (not timed),
+// load it, then time only the execution with HIP events.  Candidates are timed one at a time
+// (a process-wide lock): concurrent timing on one GPU would measure the contention, not the
+// kernel.  A candidate that fails to render, compile or launch yields a status, never an
+// abort (the reference wraps this in catch_unwind).
+int compile_and_time(const Device& dev, const LinearKernel& k, const char* name, void* const* buffers, size_t nbufs,
+                     const int64_t* vals, size_t nvals, int warmup, int runs, BenchmarkResult* out);
+
+// On-disk cache of search results keyed (ast_hash, beam_width, device), the role sled plays in
+// schedule/src/optimizer/beam.rs:390-440: one small file per key under
+// $MOROK_CACHE_DIR, else $XDG_CACHE_HOME/morok, else $HOME/.cache/morok, in beam_cache_hip/.
+// IGNORE_BEAM_CACHE=1 turns lookups off (beam.rs:16-19).
+class BeamCache {
+  public:
+    static std::string directory();
+    static bool get(uint64_t ast_hash, int width, const std::string& device, std::vector<uint8_t>* value);
+    static int put(uint64_t ast_hash, int width, const std::string& device, const void* value, size_t len);
+};
+
+// Beam search over the f32 matmul action space (beam.rs:1-20): stage by stage (LOCAL, UPCAST,
+// UNROLL) every valid action is applied to the `width` best candidates so far, each result is
+// compiled and timed, and the `width` fastest survive.  Scratch operands are allocated on the
+// device for the timing runs.  *from_cache tells whether the answer came from the disk cache.
+struct MatmulF32Opts;
+int beam_search_matmul_f32(const Device& dev, int64_t M, int64_t N, int64_t K, int width, MatmulF32Opts* best,
+                           double* best_ms, bool* from_cache, int* candidates_timed);
+
 // device/src/sync.rs:44-71,192-310: monotonically increasing timeline value backed by one
 // HIP event per recorded value (the last 16 are kept).
 class TimelineSignal {

@@ -437,36 +437,52 @@ LinearKernel KernelBuilder::finish() {
 }
 
 // ============================================================================ matmul kernels
-LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K) {
+bool matmul_f32_opts_valid(const MatmulF32Opts& o, int64_t M, int64_t N, int64_t K) {
+    if (o.local_x < 1 || o.local_y < 1 || o.local_x * o.local_y > 1024) return false;
+    if (o.up_n != 1 && o.up_n != 2 && o.up_n != 4) return false;
+    if (o.up_m < 1 || o.up_m > 8 || o.unroll_k < 1 || o.unroll_k > 8) return false;
+    if (o.up_m * o.up_n > 32) return false;  // accumulator registers per work-item
+    return M % (static_cast<int64_t>(o.local_y) * o.up_m) == 0 && N % (static_cast<int64_t>(o.local_x) * o.up_n) == 0 &&
+           K % o.unroll_k == 0 && M > 0 && N > 0 && K > 0;
+}
+
+LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K, const MatmulF32Opts& o) {
     KernelBuilder b;
     const Scalar f = Scalar::Float32;
+    const int un = o.up_n, um = o.up_m;
+    const int64_t tile_n = static_cast<int64_t>(o.local_x) * un, tile_m = static_cast<int64_t>(o.local_y) * um;
     uint32_t c = b.param(0, f, M * N), a = b.param(1, f, M * K), bm = b.param(2, f, K * N);
-    uint32_t gx = b.special("gidx0", N / 64), gy = b.special("gidx1", M / 64);
-    uint32_t lx = b.special("lidx0", 16), ly = b.special("lidx1", 16);
-    uint32_t col0 = b.iadd(b.imul(gx, 64), b.imul(lx, 4));
-    uint32_t row0 = b.iadd(b.imul(gy, 64), b.imul(ly, 4));
-    uint32_t acc = b.define_reg(0, f, 16);
+    uint32_t gx = b.special("gidx0", N / tile_n), gy = b.special("gidx1", M / tile_m);
+    uint32_t lx = b.special("lidx0", o.local_x), ly = b.special("lidx1", o.local_y);
+    uint32_t col0 = b.iadd(b.imul(gx, tile_n), b.imul(lx, un));
+    uint32_t row0 = b.iadd(b.imul(gy, tile_m), b.imul(ly, um));
+    uint32_t acc = b.define_reg(0, f, um * un);
     uint32_t zero = b.cf(0.0);
-    for (int i = 0; i < 16; i++) b.store(b.index(acc, b.ci(i)), zero);
-    uint32_t r = b.range(K, 0, AxisType::Reduce);
-    uint32_t bvec = b.load(b.index(bm, b.iadd(b.imul(r, N), col0)), 4);
-    for (int i = 0; i < 4; i++) {
-        uint32_t arow = b.iadd(row0, b.ci(i));
-        uint32_t av = b.load(b.index(a, b.iadd(b.imul(arow, K), r)));
-        for (int j = 0; j < 4; j++) {
-            uint32_t slot = b.index(acc, b.ci(i * 4 + j));
-            b.store(slot, b.mulacc(av, b.gep(bvec, j), b.load(slot)));
+    for (int i = 0; i < um * un; i++) b.store(b.index(acc, b.ci(i)), zero);
+    uint32_t r = b.range(K / o.unroll_k, 0, AxisType::Reduce);
+    for (int u = 0; u < o.unroll_k; u++) {
+        uint32_t kk = b.iadd(b.imul(r, o.unroll_k), b.ci(u));
+        uint32_t bvec = b.load(b.index(bm, b.iadd(b.imul(kk, N), col0)), un);
+        for (int i = 0; i < um; i++) {
+            uint32_t arow = b.iadd(row0, b.ci(i));
+            uint32_t av = b.load(b.index(a, b.iadd(b.imul(arow, K), kk)));
+            for (int j = 0; j < un; j++) {
+                uint32_t slot = b.index(acc, b.ci(i * un + j));
+                b.store(slot, b.mulacc(av, un > 1 ? b.gep(bvec, j) : bvec, b.load(slot)));
+            }
         }
     }
     b.end({r});
-    for (int i = 0; i < 4; i++) {
+    for (int i = 0; i < um; i++) {
         uint32_t arow = b.iadd(row0, b.ci(i));
         std::vector<uint32_t> vals;
-        for (int j = 0; j < 4; j++) vals.push_back(b.load(b.index(acc, b.ci(i * 4 + j))));
-        b.store(b.index(c, b.iadd(b.imul(arow, N), col0)), b.vectorize(vals));
+        for (int j = 0; j < un; j++) vals.push_back(b.load(b.index(acc, b.ci(i * un + j))));
+        b.store(b.index(c, b.iadd(b.imul(arow, N), col0)), un > 1 ? b.vectorize(vals) : vals[0]);
     }
     return b.finish();
 }
+
+LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K) { return build_matmul_f32_kernel(M, N, K, MatmulF32Opts()); }
 
 int build_wmma_matmul_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, LinearKernel* k) {
     const int tn = tc.dims[0], tm = tc.dims[1], tk = tc.dims[2];

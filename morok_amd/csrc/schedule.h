@@ -173,6 +173,16 @@ class KernelBuilder {
 // schedule/src/optimizer/heuristics.rs:37-82 aim for: upcast 4, local <= 128..256).
 // Requires M % 64 == 0 and N % 64 == 0.
 LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K);
+// The same kernel shape with the optimisation choices left open: the action space a beam
+// search explores (LOCAL extents, UPCAST of N as a vector and of M as rows per work-item,
+// UNROLL of the reduce axis; schedule/src/optimizer/beam.rs:36-120).
+struct MatmulF32Opts {
+    int local_x = 16, local_y = 16;  // LOCAL
+    int up_n = 4, up_m = 4;          // UPCAST
+    int unroll_k = 1;                // UNROLL
+};
+bool matmul_f32_opts_valid(const MatmulF32Opts& o, int64_t M, int64_t N, int64_t K);
+LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K, const MatmulF32Opts& o);
 // Tensor-core matmul (tc.rs:358-674 applied to C[M,N] = A[M,K] B[K,N]): one wave per
 // um x un grid of 16x16 output tiles, operands gathered per lane as the tensor core's
 // swizzle prescribes, WMMA per K step, accumulate in dtype_out, result cast to `out`.

@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <set>
@@ -890,7 +891,13 @@ struct Scheduler {
             if (a->dtype == Scalar::BFloat16) {
                 rc = builtin("gemm_bf16", {M, N, K}, {out, a->buffer, w->buffer});
             } else {
-                LinearKernel k = build_matmul_f32_kernel(M, N, K);
+                // MOROK_BEAM=<width> selects the LOCAL/UPCAST/UNROLL choices by timed search
+                // (cached on disk) instead of the fixed heuristic (tensor/src/realize.rs:1160-1250)
+                MatmulF32Opts opts;
+                int beam = 0;
+                if (const char* e = std::getenv("MOROK_BEAM")) beam = std::atoi(e);
+                if (beam > 0) MRK_TRY(beam_search_matmul_f32(*dev, M, N, K, beam, &opts, nullptr, nullptr, nullptr));
+                LinearKernel k = build_matmul_f32_kernel(M, N, K, opts);
                 std::shared_ptr<CachedKernel> ck;
                 bool cached = false;
                 const std::string name = "r_" + std::to_string(M) + "_" + std::to_string(N) + "_" + std::to_string(K);

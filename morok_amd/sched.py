@@ -97,3 +97,40 @@ def build_matmul_f32(m, n, k):
 
 def build_wmma_matmul(tc_index, m, n, k, out_scalar=U.BF16):
     return _take(lib.mrk_hip_sched_build_wmma_matmul, tc_index, m, n, k, out_scalar)
+
+
+def build_matmul_f32_opts(m, n, k, opts):
+    """f32 matmul kernel with explicit (LOCAL x, LOCAL y, UPCAST n, UPCAST m, UNROLL k)."""
+    arr = (C.c_int * 5)(*opts)
+    return _take(lib.mrk_hip_sched_build_matmul_f32_opts, m, n, k, arr)
+
+
+def compile_and_time(kernel_bytes, buffers, vals=(), name=None, warmup=1, runs=3, device_id=0):
+    """Beam-search timing hook: compile (not timed), then the minimum of `runs` event-timed
+    launches in milliseconds (tensor/src/realize.rs:1190-1242)."""
+    ms = C.c_double()
+    bufs = (C.c_void_p * max(len(buffers), 1))(*[b._h for b in buffers])
+    va = (C.c_int64 * max(len(vals), 1))(*[int(v) for v in vals])
+    check(lib.mrk_hip_compile_and_time(device_id, kernel_bytes, len(kernel_bytes), name.encode() if name else None,
+                                       bufs, len(buffers), va, len(vals), warmup, runs, C.byref(ms)))
+    return ms.value
+
+
+def beam_cache_get(ast_hash, width, device):
+    buf = C.create_string_buffer(4096)
+    n = C.c_size_t()
+    check(lib.mrk_hip_beam_cache_get(ast_hash, width, device.encode(), buf, 4096, C.byref(n)))
+    return buf.raw[: n.value] if n.value else None
+
+
+def beam_cache_put(ast_hash, width, device, value):
+    check(lib.mrk_hip_beam_cache_put(ast_hash, width, device.encode(), value, len(value)))
+
+
+def beam_search_matmul_f32(m, n, k, width=2, device_id=0):
+    """Returns (opts, best_ms, from_cache, candidates_timed)."""
+    opts = (C.c_int * 5)()
+    ms = C.c_double()
+    cached, timed = C.c_int(), C.c_int()
+    check(lib.mrk_hip_beam_search_matmul_f32(device_id, m, n, k, width, opts, C.byref(ms), C.byref(cached), C.byref(timed)))
+    return list(opts), ms.value, bool(cached.value), timed.value

@@ -296,3 +296,58 @@ def test_decoder_block_lowering(T, shim):
     assert sum(k.startswith("flash_fwd") for k in names) == 1
     assert shim.mrk_shim_launches() - n0 == len(names)
     print(names)
+
+
+# ------------------------------------------------------------------ beam-search support
+def test_beam_cache_roundtrip_and_ignore(shim, tmp_path, monkeypatch):
+    from morok_amd import sched
+
+    monkeypatch.setenv("MOROK_CACHE_DIR", str(tmp_path))
+    monkeypatch.delenv("IGNORE_BEAM_CACHE", raising=False)
+    assert sched.beam_cache_get(1234, 4, "HIP:0") is None
+    sched.beam_cache_put(1234, 4, "HIP:0", b"\x01\x02\x03")
+    assert sched.beam_cache_get(1234, 4, "HIP:0") == b"\x01\x02\x03"
+    # the key covers the AST hash, the beam width and the device (beam.rs:401-409)
+    assert sched.beam_cache_get(1234, 8, "HIP:0") is None
+    assert sched.beam_cache_get(1234, 4, "HIP:1") is None
+    assert sched.beam_cache_get(1235, 4, "HIP:0") is None
+    sched.beam_cache_put(1234, 4, "HIP:0", b"new")          # overwrite
+    assert sched.beam_cache_get(1234, 4, "HIP:0") == b"new"
+    assert (tmp_path / "beam_cache_hip").is_dir()
+    monkeypatch.setenv("IGNORE_BEAM_CACHE", "1")             # beam.rs:16-19
+    assert sched.beam_cache_get(1234, 4, "HIP:0") is None
+
+
+def test_compile_and_time_and_failing_candidates(dev, shim):
+    from morok_amd import sched
+
+    bufs = [dev.buffer(64 * 64 * 4) for _ in range(3)]
+    k = sched.build_matmul_f32_opts(64, 64, 64, [16, 16, 4, 4, 2])
+    n = shim.mrk_shim_launches()
+    ms = sched.compile_and_time(k, bufs, warmup=1, runs=3)
+    assert ms >= 0.0 and shim.mrk_shim_launches() == n + 4           # 1 warm-up + 3 timed launches
+    assert hostshim_lib.last_dims(shim) == ((1, 1, 1), (16, 16, 1))
+    with pytest.raises(MorokHipError):                                # wrong buffer count: a status, not a crash
+        sched.compile_and_time(k, bufs[:2])
+    with pytest.raises(MorokHipError) as e:                           # choices that do not divide the shape
+        sched.build_matmul_f32_opts(64, 64, 64, [16, 16, 4, 8, 1])
+    assert e.value.code == 11
+    with pytest.raises(MorokHipError):
+        sched.compile_and_time(b"not a kernel", bufs)
+
+
+def test_beam_search_uses_and_fills_the_disk_cache(dev, shim, tmp_path, monkeypatch):
+    from morok_amd import sched
+
+    monkeypatch.setenv("MOROK_CACHE_DIR", str(tmp_path))
+    monkeypatch.delenv("IGNORE_BEAM_CACHE", raising=False)
+    opts, ms, cached, timed = sched.beam_search_matmul_f32(128, 128, 64, width=2)
+    assert not cached and timed > 10 and len(opts) == 5
+    assert 128 % (opts[0] * opts[2]) == 0 and 128 % (opts[1] * opts[3]) == 0 and 64 % opts[4] == 0
+    opts2, _, cached2, timed2 = sched.beam_search_matmul_f32(128, 128, 64, width=2)
+    assert cached2 and timed2 == 0 and opts2 == opts
+    _, _, cached3, _ = sched.beam_search_matmul_f32(128, 128, 64, width=3)    # other width, other key
+    assert not cached3
+    # odd shapes fall back to scalar columns / single rows instead of failing
+    opts4, _, _, _ = sched.beam_search_matmul_f32(6, 10, 7, width=1)
+    assert 10 % (opts4[0] * opts4[2]) == 0 and 6 % (opts4[1] * opts4[3]) == 0

@@ -130,3 +130,42 @@ def test_timeline_signal(dev):
         s.set(v)
     s.wait(24, 5000)
     assert s.value == 24 and s.is_reached(10) and not s.is_reached(25)
+
+
+def test_beam_search_matmul_f32(dev, oracle, tmp_path, monkeypatch):
+    """Beam search over LOCAL / UPCAST / UNROLL with event-timed candidates: the winner is a
+    valid kernel, computes the right product, is at least as fast as the fixed heuristic, and
+    the second search is answered by the disk cache."""
+    import morok_amd
+    from morok_amd import sched, synth
+
+    monkeypatch.setenv("MOROK_CACHE_DIR", str(tmp_path))
+    monkeypatch.delenv("IGNORE_BEAM_CACHE", raising=False)
+    n = 512
+    opts, best_ms, cached, timed = sched.beam_search_matmul_f32(n, n, n, width=2)
+    assert not cached and timed >= 9 and best_ms > 0
+    a = synth.uniform((n, n), 1, 0)
+    b = synth.uniform((n, n), 1, 1)
+    ba, bb, bc = morok_amd.Buffer.from_numpy(a), morok_amd.Buffer.from_numpy(b), dev.buffer(n * n * 4)
+    k = morok_amd.Kernel.get_or_compile(sched.build_matmul_f32_opts(n, n, n, opts), "beam_winner")
+    plan = morok_amd.ExecutionPlan()
+    plan.add_kernel(k, [plan.add_buffer(bc), plan.add_buffer(ba), plan.add_buffer(bb)])
+    plan.build().execute()
+    got = bc.copyout(np.float32, (n, n))
+    ref = oracle.matmul_f32(a, b)
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-4 * np.abs(ref).max())
+    base_ms = sched.compile_and_time(sched.build_matmul_f32(n, n, n), [bc, ba, bb], warmup=1, runs=5)
+    assert best_ms <= base_ms * 1.15
+    opts2, _, cached2, timed2 = sched.beam_search_matmul_f32(n, n, n, width=2)
+    assert cached2 and timed2 == 0 and opts2 == opts
+
+
+def test_tensor_matmul_with_beam(dev, oracle, tmp_path, monkeypatch):
+    from morok_amd import synth, tensor
+
+    monkeypatch.setenv("MOROK_CACHE_DIR", str(tmp_path))
+    monkeypatch.setenv("MOROK_BEAM", "1")
+    a = synth.uniform((256, 192), 7, 0)
+    b = synth.uniform((192, 128), 7, 1)
+    got = tensor.Tensor.from_numpy(a).matmul(tensor.Tensor.from_numpy(b)).to_numpy()
+    np.testing.assert_allclose(got, oracle.matmul_f32(a, b), rtol=1e-4, atol=1e-4)
