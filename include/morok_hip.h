@@ -257,6 +257,33 @@ int mrk_hip_signal_wait(mrk_signal* s, uint64_t value, uint64_t timeout_ms);
 void mrk_hip_signal_destroy(mrk_signal* s);
 
 /* =====================================================================================
+ * Hardware queues (device/src/queue.rs:76-161) over HIP streams of default priority.
+ * Commands are batched and reach the queue's stream on submit; ordering between queues is
+ * expressed with timeline signals, which become hipStreamWaitEvent dependencies on the GPU
+ * (QueueFactory::create_compute_queue / create_copy_queue / create_signal, queue.rs:136-161).
+ * ===================================================================================== */
+typedef struct mrk_queue mrk_queue;
+int mrk_hip_queue_create(int device_id, int copy_queue, mrk_queue** out);
+/* HardwareQueue::wait / signal (queue.rs:93-105). */
+int mrk_hip_queue_wait(mrk_queue* q, mrk_signal* s, uint64_t value);
+int mrk_hip_queue_signal(mrk_queue* q, mrk_signal* s, uint64_t value);
+/* HardwareQueue::exec (queue.rs:107-121): global/local may be null (sizes recorded at compile
+ * time are used, ExecParams default). */
+int mrk_hip_queue_exec(mrk_queue* q, const mrk_kernel* k, mrk_buffer* const* buffers, size_t nbufs, const int64_t* vals,
+                       size_t nvals, const size_t* global, const size_t* local);
+/* HardwareQueue::copy (queue.rs:123-128): device-to-device, SIZE_MISMATCH at submit unless
+ * the sizes are equal. */
+int mrk_hip_queue_copy(mrk_queue* q, mrk_buffer* dst, const mrk_buffer* src);
+/* HardwareQueue::memory_barrier (queue.rs:130-134): a HIP stream executes in order; records nothing. */
+int mrk_hip_queue_memory_barrier(mrk_queue* q);
+/* HardwareQueue::submit (queue.rs:136-141): hands the batch to the stream without waiting for it.
+ * A wait on a value that no queue has signalled yet is retried for wait_timeout_ms, then TIMEOUT. */
+int mrk_hip_queue_submit(mrk_queue* q, uint64_t wait_timeout_ms);
+int mrk_hip_queue_synchronize(mrk_queue* q);
+size_t mrk_hip_queue_pending(const mrk_queue* q);
+void mrk_hip_queue_destroy(mrk_queue* q);
+
+/* =====================================================================================
  * Scheduling helpers for the gfx950 target (what morok's `schedule` crate supplies per backend)
  * ===================================================================================== */
 

@@ -153,6 +153,16 @@ _SIGS = {
     "mrk_hip_beam_cache_get": (C.c_int, [C.c_uint64, C.c_int, C.c_char_p, C.c_void_p, C.c_size_t, c_size_p]),
     "mrk_hip_beam_cache_put": (C.c_int, [C.c_uint64, C.c_int, C.c_char_p, C.c_void_p, C.c_size_t]),
     "mrk_hip_beam_search_matmul_f32": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_double), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "mrk_hip_queue_create": (C.c_int, [C.c_int, C.c_int, c_void_pp]),
+    "mrk_hip_queue_wait": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64]),
+    "mrk_hip_queue_signal": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64]),
+    "mrk_hip_queue_exec": (C.c_int, [C.c_void_p, C.c_void_p, c_void_pp, C.c_size_t, c_i64_p, C.c_size_t, c_size_p, c_size_p]),
+    "mrk_hip_queue_copy": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p]),
+    "mrk_hip_queue_memory_barrier": (C.c_int, [C.c_void_p]),
+    "mrk_hip_queue_submit": (C.c_int, [C.c_void_p, C.c_uint64]),
+    "mrk_hip_queue_synchronize": (C.c_int, [C.c_void_p]),
+    "mrk_hip_queue_pending": (C.c_size_t, [C.c_void_p]),
+    "mrk_hip_queue_destroy": (None, [C.c_void_p]),
     # lazy tensors
     "mrk_hip_tensor_from_bytes": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),
     "mrk_hip_tensor_from_buffer": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),

@@ -21,8 +21,12 @@ class BuiltinProgram final : public Program {
           nbufs_(nbufs),
           params_(std::move(params)),
           fn_(std::move(fn)) {}
-    int execute(void* const* buffers, size_t nbufs, const int64_t*, size_t nvals, const size_t*,
-                const size_t*) override {
+    int execute(void* const* buffers, size_t nbufs, const int64_t* vals, size_t nvals, const size_t* global,
+                const size_t* local) override {
+        return execute_on(stream_, buffers, nbufs, vals, nvals, global, local);
+    }
+    int execute_on(ffi::Stream stream, void* const* buffers, size_t nbufs, const int64_t*, size_t nvals, const size_t*,
+                   const size_t*) override {
         if (nbufs != nbufs_)
             return failf(kInvalidArgument, "kernel '%s' expects %zu buffers, got %zu", name_.c_str(), nbufs_, nbufs);
         if (nvals != 0)
@@ -30,7 +34,7 @@ class BuiltinProgram final : public Program {
         for (size_t i = 0; i < nbufs; i++)
             if (!buffers[i]) return failf(kInvalidArgument, "kernel '%s': buffer %zu is null", name_.c_str(), i);
         MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
-        int rc = fn_(stream_, buffers, params_);
+        int rc = fn_(stream, buffers, params_);
         if (rc != 0) return fail_hip(rc, name_.c_str());
         return kOk;
     }

@@ -8,6 +8,7 @@
 #include "device.h"
 #include "error.h"
 #include "kernels/kernels.h"
+#include "queue.h"
 #include "runtime.h"
 #include "schedule.h"
 #include "tensor.h"
@@ -34,7 +35,10 @@ struct mrk_plan {
     std::unique_ptr<ExecutionPlan> p;
 };
 struct mrk_signal {
-    std::unique_ptr<TimelineSignal> s;
+    std::shared_ptr<TimelineSignal> s;
+};
+struct mrk_queue {
+    std::unique_ptr<HardwareQueue> q;
 };
 struct mrk_tensor {
     Tensor t;
@@ -502,6 +506,65 @@ int mrk_hip_signal_wait(mrk_signal* s, uint64_t value, uint64_t timeout_ms) {
     return s->s->wait(value, timeout_ms);
 }
 void mrk_hip_signal_destroy(mrk_signal* s) { delete s; }
+
+// ---- hardware queues
+int mrk_hip_queue_create(int device_id, int copy_queue, mrk_queue** out) {
+    MRK_NONNULL(out);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    std::unique_ptr<HardwareQueue> q(new HardwareQueue(device_id, copy_queue != 0));
+    MRK_TRY(q->init());
+    *out = new mrk_queue{std::move(q)};
+    return kOk;
+}
+int mrk_hip_queue_wait(mrk_queue* q, mrk_signal* s, uint64_t value) {
+    MRK_NONNULL(q);
+    MRK_NONNULL(s);
+    q->q->wait(s->s, value);
+    return kOk;
+}
+int mrk_hip_queue_signal(mrk_queue* q, mrk_signal* s, uint64_t value) {
+    MRK_NONNULL(q);
+    MRK_NONNULL(s);
+    q->q->signal(s->s, value);
+    return kOk;
+}
+int mrk_hip_queue_exec(mrk_queue* q, const mrk_kernel* k, mrk_buffer* const* buffers, size_t nbufs, const int64_t* vals,
+                       size_t nvals, const size_t* global, const size_t* local) {
+    MRK_NONNULL(q);
+    MRK_NONNULL(k);
+    if (nbufs) MRK_NONNULL(buffers);
+    if (nvals) MRK_NONNULL(vals);
+    std::vector<std::shared_ptr<Buffer>> bufs;
+    for (size_t i = 0; i < nbufs; i++) {
+        MRK_NONNULL(buffers[i]);
+        bufs.push_back(std::make_shared<Buffer>(*buffers[i]->b));
+    }
+    q->q->exec(k->k, std::move(bufs), std::vector<int64_t>(vals, vals + nvals), global, local);
+    return kOk;
+}
+int mrk_hip_queue_copy(mrk_queue* q, mrk_buffer* dst, const mrk_buffer* src) {
+    MRK_NONNULL(q);
+    MRK_NONNULL(dst);
+    MRK_NONNULL(src);
+    q->q->copy(std::make_shared<Buffer>(*dst->b), std::make_shared<Buffer>(*src->b));
+    return kOk;
+}
+int mrk_hip_queue_memory_barrier(mrk_queue* q) {
+    MRK_NONNULL(q);
+    q->q->memory_barrier();
+    return kOk;
+}
+int mrk_hip_queue_submit(mrk_queue* q, uint64_t wait_timeout_ms) {
+    MRK_NONNULL(q);
+    return q->q->submit(wait_timeout_ms);
+}
+int mrk_hip_queue_synchronize(mrk_queue* q) {
+    MRK_NONNULL(q);
+    return q->q->synchronize();
+}
+size_t mrk_hip_queue_pending(const mrk_queue* q) { return q ? q->q->pending_commands() : 0; }
+void mrk_hip_queue_destroy(mrk_queue* q) { delete q; }
 
 // ---- scheduling helpers
 size_t mrk_hip_sched_find_smallest_divisor(size_t n) { return find_smallest_divisor(n); }

@@ -67,6 +67,9 @@ class Program {
     // then the sizes recorded at compile time are used.
     virtual int execute(void* const* buffers, size_t nbufs, const int64_t* vals, size_t nvals, const size_t* global,
                         const size_t* local) = 0;
+    // The same launch on another stream of the same device (hardware queues own their streams).
+    virtual int execute_on(ffi::Stream stream, void* const* buffers, size_t nbufs, const int64_t* vals, size_t nvals,
+                           const size_t* global, const size_t* local) = 0;
     virtual const char* name() const = 0;
 };
 

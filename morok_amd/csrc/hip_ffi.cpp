@@ -36,6 +36,9 @@ int stream_create(Stream* out) {
 }
 int stream_destroy(Stream s) { return hipStreamDestroy(static_cast<hipStream_t>(s)); }
 int stream_synchronize(Stream s) { return hipStreamSynchronize(static_cast<hipStream_t>(s)); }
+int stream_wait_event(Stream s, Event e) {
+    return hipStreamWaitEvent(static_cast<hipStream_t>(s), static_cast<hipEvent_t>(e), 0);
+}
 int device_synchronize() { return hipDeviceSynchronize(); }
 
 int event_create(Event* out) {

@@ -38,6 +38,8 @@ int stream_create(Stream* out);
 int stream_destroy(Stream s);
 int stream_synchronize(Stream s);
 int device_synchronize();
+// Makes all work queued on `s` after this call wait for `e` (hipStreamWaitEvent).
+int stream_wait_event(Stream s, Event e);
 
 int event_create(Event* out);
 int event_destroy(Event e);

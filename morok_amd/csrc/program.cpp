@@ -35,6 +35,10 @@ class ModuleProgram final : public Program {
 
     int execute(void* const* buffers, size_t nbufs, const int64_t* vals, size_t nvals, const size_t* global,
                 const size_t* local) override {
+        return execute_on(stream_, buffers, nbufs, vals, nvals, global, local);
+    }
+    int execute_on(ffi::Stream stream, void* const* buffers, size_t nbufs, const int64_t* vals, size_t nvals,
+                   const size_t* global, const size_t* local) override {
         if (nbufs != buf_count_)
             return failf(kInvalidArgument, "kernel '%s' expects %zu buffers, got %zu", name_.c_str(), buf_count_, nbufs);
         if (nvals != nvars_)
@@ -74,7 +78,7 @@ class ModuleProgram final : public Program {
             }
         }
         MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
-        MRK_HIP(ffi::module_launch(function_, grid, block, 0, stream_, params.data()), "hipModuleLaunchKernel");
+        MRK_HIP(ffi::module_launch(function_, grid, block, 0, stream, params.data()), "hipModuleLaunchKernel");
         return kOk;
     }
     const char* name() const override { return name_.c_str(); }

@@ -1,0 +1,123 @@
+#include "queue.h"
+
+#include <chrono>
+#include <thread>
+
+#include "error.h"
+
+namespace mrk {
+
+HardwareQueue::HardwareQueue(int device_id, bool copy_queue) : device_id_(device_id), copy_queue_(copy_queue) {}
+
+HardwareQueue::~HardwareQueue() {
+    if (stream_) {
+        ffi::set_device(device_id_);
+        ffi::stream_synchronize(stream_);
+        ffi::stream_destroy(stream_);
+    }
+}
+
+int HardwareQueue::init() {
+    MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
+    MRK_HIP(ffi::stream_create(&stream_), "hipStreamCreate");
+    return kOk;
+}
+
+void HardwareQueue::wait(std::shared_ptr<TimelineSignal> signal, uint64_t value) {
+    Command c;
+    c.kind = Kind::Wait;
+    c.signal = std::move(signal);
+    c.value = value;
+    cmds_.push_back(std::move(c));
+}
+
+void HardwareQueue::signal(std::shared_ptr<TimelineSignal> signal, uint64_t value) {
+    Command c;
+    c.kind = Kind::Signal;
+    c.signal = std::move(signal);
+    c.value = value;
+    cmds_.push_back(std::move(c));
+}
+
+void HardwareQueue::exec(std::shared_ptr<CachedKernel> kernel, std::vector<std::shared_ptr<Buffer>> buffers,
+                         std::vector<int64_t> vals, const size_t* global, const size_t* local) {
+    Command c;
+    c.kind = Kind::Exec;
+    c.kernel = std::move(kernel);
+    c.buffers = std::move(buffers);
+    c.vals = std::move(vals);
+    if (global && local) {
+        c.has_sizes = true;
+        for (int i = 0; i < 3; i++) {
+            c.global[i] = global[i];
+            c.local[i] = local[i];
+        }
+    }
+    cmds_.push_back(std::move(c));
+}
+
+void HardwareQueue::copy(std::shared_ptr<Buffer> dst, std::shared_ptr<Buffer> src) {
+    Command c;
+    c.kind = Kind::Copy;
+    c.buffers = {std::move(dst), std::move(src)};
+    cmds_.push_back(std::move(c));
+}
+
+int HardwareQueue::submit(uint64_t wait_timeout_ms) {
+    if (!stream_) return fail(kRuntime, "runtime error: queue used before init()");
+    MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
+    // the batch leaves the queue whatever happens: a failed submit is not replayed
+    std::vector<Command> batch;
+    batch.swap(cmds_);
+    for (Command& c : batch) {
+        switch (c.kind) {
+            case Kind::Wait: {
+                const auto deadline = std::chrono::steady_clock::now() + std::chrono::milliseconds(wait_timeout_ms);
+                for (;;) {
+                    bool pending = false;
+                    MRK_TRY(c.signal->stream_wait(c.value, stream_, &pending));
+                    if (!pending) break;
+                    if (std::chrono::steady_clock::now() >= deadline)
+                        return failf(kTimeout, "runtime error: queue wait on value %llu that nobody signalled within %llu ms",
+                                     (unsigned long long)c.value, (unsigned long long)wait_timeout_ms);
+                    std::this_thread::sleep_for(std::chrono::microseconds(50));
+                }
+                break;
+            }
+            case Kind::Signal: MRK_TRY(c.signal->set_on(c.value, stream_)); break;
+            case Kind::Exec: {
+                std::vector<void*> ptrs(c.buffers.size());
+                for (size_t i = 0; i < c.buffers.size(); i++) {
+                    MRK_TRY(c.buffers[i]->ensure_allocated());
+                    MRK_TRY(c.buffers[i]->as_raw_ptr(&ptrs[i]));
+                }
+                const size_t* g = c.has_sizes ? c.global : (c.kernel->has_sizes ? c.kernel->global_size.data() : nullptr);
+                const size_t* l = c.has_sizes ? c.local : (c.kernel->has_sizes ? c.kernel->local_size.data() : nullptr);
+                MRK_TRY(c.kernel->program->execute_on(stream_, ptrs.data(), ptrs.size(), c.vals.data(), c.vals.size(), g, l));
+                break;
+            }
+            case Kind::Copy: {
+                Buffer& dst = *c.buffers[0];
+                const Buffer& src = *c.buffers[1];
+                if (dst.size() != src.size())
+                    return failf(kSizeMismatch, "size mismatch: expected %zu, got %zu", dst.size(), src.size());
+                MRK_TRY(dst.ensure_allocated());
+                void *d = nullptr, *s = nullptr;
+                MRK_TRY(dst.as_raw_ptr(&d));
+                MRK_TRY(src.as_raw_ptr(&s));
+                MRK_HIP(ffi::memcpy_dtod_async(d, s, dst.size(), stream_), "hipMemcpyAsync");
+                break;
+            }
+        }
+    }
+    return kOk;
+}
+
+int HardwareQueue::synchronize() {
+    if (!stream_) return kOk;
+    MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
+    MRK_HIP(ffi::stream_synchronize(stream_), "hipStreamSynchronize");
+    return kOk;
+}
+
+}  // namespace mrk

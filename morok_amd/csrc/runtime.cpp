@@ -417,7 +417,9 @@ TimelineSignal::~TimelineSignal() {
 
 uint64_t TimelineSignal::value() {
     std::lock_guard<std::mutex> lock(mu_);
-    // events complete in stream order: retire from the front
+    // values are recorded in increasing order; with one stream the events also complete in
+    // that order, with several queues a later value may finish first, and reaching it means
+    // the timeline has passed the earlier ones only once they have finished too
     while (!pending_.empty() && ffi::event_query(pending_.front().second) == 0) {
         completed_ = pending_.front().first > completed_ ? pending_.front().first : completed_;
         ffi::event_destroy(pending_.front().second);
@@ -426,11 +428,27 @@ uint64_t TimelineSignal::value() {
     return completed_;
 }
 
-int TimelineSignal::set(uint64_t value) {
+int TimelineSignal::set(uint64_t value) { return set_on(value, stream_); }
+
+int TimelineSignal::stream_wait(uint64_t target, ffi::Stream stream, bool* pending) {
+    *pending = false;
+    if (value() >= target) return kOk;  // also retires finished events
+    std::lock_guard<std::mutex> lock(mu_);
+    for (auto& p : pending_)
+        if (p.first >= target) {
+            MRK_HIP(ffi::stream_wait_event(stream, p.second), "hipStreamWaitEvent");
+            return kOk;
+        }
+    if (completed_ >= target) return kOk;
+    *pending = true;
+    return kOk;
+}
+
+int TimelineSignal::set_on(uint64_t value, ffi::Stream stream) {
     MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
     ffi::Event e = nullptr;
     MRK_HIP(ffi::event_create(&e), "hipEventCreate");
-    int rc = ffi::event_record(e, stream_);
+    int rc = ffi::event_record(e, stream);
     if (rc != 0) {
         ffi::event_destroy(e);
         return fail_hip(rc, "hipEventRecord");

@@ -145,6 +145,11 @@ class TimelineSignal {
     ~TimelineSignal();
     uint64_t value();                       // highest value whose event has completed
     int set(uint64_t value);                // record an event for `value` on the stream
+    int set_on(uint64_t value, ffi::Stream stream);  // the same on another stream (hardware queues)
+    // Makes later work on `stream` wait on the GPU until the signal reaches `value`.  *pending
+    // = true when no event for such a value has been recorded yet (the producer has not
+    // submitted): the caller decides whether to retry.
+    int stream_wait(uint64_t value, ffi::Stream stream, bool* pending);
     int wait(uint64_t value, uint64_t timeout_ms);  // kTimeout if not reached in time
     bool is_reached(uint64_t value) { return this->value() >= value; }
 

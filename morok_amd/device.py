@@ -528,3 +528,60 @@ class TimelineSignal:
                 self._h = None
         except Exception:
             pass
+
+
+class HardwareQueue:
+    """HardwareQueue (device/src/queue.rs:76-141): batches commands for its own HIP stream;
+    submit() hands them over without waiting.  Every method returns self for chaining."""
+
+    def __init__(self, device_id=0, copy_queue=False):
+        h = C.c_void_p()
+        check(lib.mrk_hip_queue_create(device_id, int(copy_queue), C.byref(h)))
+        self._h = h
+        self._keep = []
+
+    def wait(self, signal, value):
+        check(lib.mrk_hip_queue_wait(self._h, signal._h, value))
+        return self
+
+    def signal(self, signal, value):
+        check(lib.mrk_hip_queue_signal(self._h, signal._h, value))
+        return self
+
+    def exec(self, kernel, buffers, vals=(), global_size=None, local_size=None):
+        bufs = (C.c_void_p * max(len(buffers), 1))(*[b._h for b in buffers])
+        va = (C.c_int64 * max(len(vals), 1))(*[int(v) for v in vals])
+        g = _size3(global_size) if global_size is not None else None
+        l = _size3(local_size) if local_size is not None else None
+        check(lib.mrk_hip_queue_exec(self._h, kernel._h, bufs, len(buffers), va, len(vals), g, l))
+        self._keep.append((kernel, list(buffers)))
+        return self
+
+    def copy(self, dst, src):
+        check(lib.mrk_hip_queue_copy(self._h, dst._h, src._h))
+        return self
+
+    def memory_barrier(self):
+        check(lib.mrk_hip_queue_memory_barrier(self._h))
+        return self
+
+    def submit(self, wait_timeout_ms=10000):
+        check(lib.mrk_hip_queue_submit(self._h, wait_timeout_ms))
+        return self
+
+    def synchronize(self):
+        check(lib.mrk_hip_queue_synchronize(self._h))
+        self._keep.clear()
+        return self
+
+    @property
+    def pending(self):
+        return lib.mrk_hip_queue_pending(self._h)
+
+    def __del__(self):
+        try:
+            if self._h:
+                lib.mrk_hip_queue_destroy(self._h)
+                self._h = None
+        except Exception:
+            pass

@@ -351,3 +351,28 @@ def test_beam_search_uses_and_fills_the_disk_cache(dev, shim, tmp_path, monkeypa
     # odd shapes fall back to scalar columns / single rows instead of failing
     opts4, _, _, _ = sched.beam_search_matmul_f32(6, 10, 7, width=1)
     assert 10 % (opts4[0] * opts4[2]) == 0 and 6 % (opts4[1] * opts4[3]) == 0
+
+
+# ------------------------------------------------------------------ hardware queues
+def test_queue_batches_until_submit_and_reports_errors(dev, shim):
+    k = morok_amd.Kernel.get_or_compile(__import__("morok_amd").sched.build_matmul_f32_opts(64, 64, 64, [16, 16, 4, 4, 1]), "qk")
+    a, b, c = (dev.buffer(64 * 64 * 4) for _ in range(3))
+    sig = morok_amd.TimelineSignal()
+    q = morok_amd.HardwareQueue()
+    n = shim.mrk_shim_launches()
+    q.exec(k, [c, a, b]).signal(sig, 1).memory_barrier()
+    assert q.pending == 2 and shim.mrk_shim_launches() == n        # nothing reaches the device before submit
+    q.submit().synchronize()
+    assert q.pending == 0 and shim.mrk_shim_launches() == n + 1 and sig.value == 1
+    # a copy between buffers of different sizes is refused at submit (buffer.rs:411-534)
+    q.copy(dev.buffer(16), dev.buffer(32))
+    with pytest.raises(MorokHipError) as e:
+        q.submit()
+    assert e.value.code == 1 and q.pending == 0
+    # waiting on a value nobody signals times out instead of hanging
+    q2 = morok_amd.HardwareQueue(copy_queue=True)
+    q2.wait(sig, 5)
+    with pytest.raises(MorokHipError) as e:
+        q2.submit(wait_timeout_ms=20)
+    assert e.value.code == 12
+    q2.wait(sig, 1).copy(a, b).submit(wait_timeout_ms=20)          # already reached: no wait

@@ -169,3 +169,44 @@ def test_tensor_matmul_with_beam(dev, oracle, tmp_path, monkeypatch):
     b = synth.uniform((192, 128), 7, 1)
     got = tensor.Tensor.from_numpy(a).matmul(tensor.Tensor.from_numpy(b)).to_numpy()
     np.testing.assert_allclose(got, oracle.matmul_f32(a, b), rtol=1e-4, atol=1e-4)
+
+
+def test_copy_and_compute_queues_with_signals(dev):
+    """A copy queue feeds a compute queue chunk by chunk; timeline signals order producer and
+    consumer on the GPU (hipStreamWaitEvent), the host never waits between chunks.  Each chunk
+    is staged through the same two buffers, so a missing dependency would corrupt the result."""
+    import morok_amd
+    from morok_amd import uop as U
+
+    n, chunks = 1 << 20, 8
+    k = U.Kernel()
+    out = k.param(0, U.f32, n)
+    inp = k.param(1, U.f32, n)
+    gx, lx = k.special("gidx0", n // 256), k.special("lidx0", 256)
+    i = k.add(k.mul(gx, k.const(256)), lx)
+    k.store(k.index(out, i), k.add(k.mul(k.load(k.index(inp, i)), k.const(2.0, U.f32)), k.const(1.0, U.f32)))
+    kern = morok_amd.Kernel.get_or_compile(k, "scale_add")
+    src = [morok_amd.Buffer.from_numpy(np.full(n, float(c), np.float32)) for c in range(chunks)]
+    dst = [dev.buffer(n * 4).ensure_allocated() for _ in range(chunks)]
+    stage = [dev.buffer(n * 4).ensure_allocated() for _ in range(2)]
+    dev.synchronize()
+    copied, consumed = morok_amd.TimelineSignal(), morok_amd.TimelineSignal()
+    qc, qx = morok_amd.HardwareQueue(copy_queue=True), morok_amd.HardwareQueue()
+    for c in range(chunks):
+        if c >= 2:
+            qc.wait(consumed, c - 1)          # stage[c % 2] was read by chunk c-2, i.e. consumed value c-1
+        qc.copy(stage[c % 2], src[c]).signal(copied, c + 1)
+        qx.wait(copied, c + 1).exec(kern, [dst[c], stage[c % 2]]).signal(consumed, c + 1)
+    # submit the consumer first: its waits refer to values the producer has not recorded yet
+    import threading
+
+    t = threading.Thread(target=lambda: qx.submit(wait_timeout_ms=20000))
+    t.start()
+    qc.submit(wait_timeout_ms=20000)
+    t.join()
+    qx.synchronize()
+    qc.synchronize()
+    consumed.wait(chunks, 5000)
+    for c in range(chunks):
+        got = dst[c].copyout(np.float32, (n,))
+        assert np.all(got == 2.0 * c + 1.0), c
