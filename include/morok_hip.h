@@ -478,6 +478,11 @@ const char* mrk_hip_tensor_last_kernel_name(size_t i);
 const char* mrk_hip_tensor_last_kernel_source(size_t i);
 size_t mrk_hip_tensor_last_cached_count(void);
 double mrk_hip_tensor_last_elapsed_ms(void);
+/* Memory planner result of the last realize / prepare on this thread: intermediates that were
+ * given an already used block, and the bytes that saved (tensor/src/memory_planner.rs:84-96).
+ * Intermediates share blocks by liveness; MOROK_NO_MEMORY_PLANNER=1 turns that off. */
+size_t mrk_hip_tensor_last_buffers_reused(void);
+size_t mrk_hip_tensor_last_memory_saved(void);
 
 #ifdef __cplusplus
 }

@@ -203,6 +203,8 @@ _SIGS = {
     "mrk_hip_tensor_last_kernel_source": (C.c_char_p, [C.c_size_t]),
     "mrk_hip_tensor_last_cached_count": (C.c_size_t, []),
     "mrk_hip_tensor_last_elapsed_ms": (C.c_double, []),
+    "mrk_hip_tensor_last_buffers_reused": (C.c_size_t, []),
+    "mrk_hip_tensor_last_memory_saved": (C.c_size_t, []),
 }
 
 

@@ -52,6 +52,9 @@ class Buffer {
     // buffer.rs:554-574: pointer handed to kernels; for this backend the device VA + offset.
     int as_raw_ptr(void** out) const;
     int synchronize() const { return data_->allocator()->synchronize(); }
+    // true when this handle covers its whole base allocation (not a sub-range view)
+    bool is_whole() const { return offset_ == 0 && size_ == data_->total_size(); }
+    const BufferOptions& options() const { return data_->options(); }
 
   private:
     Buffer(std::shared_ptr<BufferData> data, size_t offset, size_t size)

@@ -1074,5 +1074,7 @@ const char* mrk_hip_tensor_last_kernel_source(size_t i) {
 }
 size_t mrk_hip_tensor_last_cached_count(void) { return last_realize_stats().cached_kernels; }
 double mrk_hip_tensor_last_elapsed_ms(void) { return last_realize_stats().elapsed_ms; }
+size_t mrk_hip_tensor_last_buffers_reused(void) { return last_realize_stats().buffers_reused; }
+size_t mrk_hip_tensor_last_memory_saved(void) { return last_realize_stats().memory_saved; }
 
 }  // extern "C"

@@ -111,7 +111,57 @@ int ExecutionPlan::add_kernel(std::shared_ptr<CachedKernel> kernel, const std::v
     return kOk;
 }
 
+int ExecutionPlan::plan_memory() {
+    memory_planned_ = true;
+    const size_t n = buffers_.size();
+    constexpr size_t kBlock = 0x1000;  // memory_planner.rs:23
+    std::vector<long> first(n, -1), last(n, -1);
+    for (size_t t = 0; t < kernels_.size(); t++)
+        for (size_t i : kernels_[t].buffer_indices) {
+            if (first[i] < 0) first[i] = static_cast<long>(t);
+            last[i] = static_cast<long>(t);
+        }
+    std::vector<bool> candidate(n, false);
+    for (size_t i = 0; i < n; i++) {
+        const Buffer& b = *buffers_[i];
+        bool is_output = std::find(outputs_.begin(), outputs_.end(), i) != outputs_.end();
+        // inputs (already allocated), outputs (must persist) and views are left alone
+        candidate[i] = first[i] >= 0 && !b.is_allocated() && !is_output && b.is_whole() && !b.options().cpu_accessible;
+    }
+    std::shared_ptr<Allocator> alloc;
+    MRK_TRY(AllocatorRegistry::global().get(device_id_, &alloc));
+    std::unordered_map<size_t, std::vector<std::shared_ptr<Buffer>>> pool;  // rounded size -> free blocks
+    std::vector<std::shared_ptr<Buffer>> block_of(n);
+    for (size_t t = 0; t < kernels_.size(); t++) {
+        // frees before allocations at the same step (memory_planner.rs:8)
+        for (size_t i = 0; i < n; i++)
+            if (candidate[i] && last[i] == static_cast<long>(t) - 1 && block_of[i]) pool[block_of[i]->size()].push_back(block_of[i]);
+        for (size_t i = 0; i < n; i++) {
+            if (!candidate[i] || first[i] != static_cast<long>(t)) continue;
+            const size_t want = buffers_[i]->size();
+            const size_t rounded = (want + kBlock - 1) / kBlock * kBlock;
+            auto& free_list = pool[rounded];
+            mem_stats_.planned++;
+            if (!free_list.empty()) {
+                block_of[i] = free_list.back();
+                free_list.pop_back();
+                mem_stats_.buffers_reused++;
+                mem_stats_.memory_saved += rounded;
+            } else {
+                BufferOptions o;
+                block_of[i] = std::make_shared<Buffer>(alloc, rounded, o);
+                mem_stats_.memory_planned += rounded;
+            }
+            std::unique_ptr<Buffer> v;
+            MRK_TRY(block_of[i]->view(0, want, &v));
+            buffers_[i] = std::shared_ptr<Buffer>(std::move(v));
+        }
+    }
+    return kOk;
+}
+
 int ExecutionPlan::build() {
+    if (plan_memory_ && !memory_planned_ && !outputs_.empty()) MRK_TRY(plan_memory());
     for (auto& b : buffers_) MRK_TRY(b->ensure_allocated());  // tensor/src/realize.rs:974-981
     for (auto& pk : kernels_) {
         pk.buffer_ptrs.clear();

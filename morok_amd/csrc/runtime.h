@@ -67,6 +67,14 @@ struct KernelProfile {
     double elapsed_ms = 0.0;
 };
 
+// tensor/src/memory_planner.rs:84-96
+struct MemoryPlanStats {
+    size_t planned = 0;         // intermediates that took part
+    size_t buffers_reused = 0;  // of those, how many were given an already used block
+    size_t memory_saved = 0;    // bytes not allocated thanks to reuse
+    size_t memory_planned = 0;  // bytes the planned intermediates occupy after reuse
+};
+
 class ExecutionPlan {
   public:
     explicit ExecutionPlan(int device_id) : device_id_(device_id) {}
@@ -76,6 +84,13 @@ class ExecutionPlan {
     int add_kernel(std::shared_ptr<CachedKernel> kernel, const std::vector<size_t>& buffer_indices,
                    const std::vector<int64_t>& vals);
     void set_outputs(const std::vector<size_t>& idx) { outputs_ = idx; }
+    // Liveness-based reuse of intermediate buffers (tensor/src/memory_planner.rs:1-45): at
+    // build(), every buffer that is not yet allocated, not an output and not a view is given
+    // a block from a pool keyed by its size rounded up to 4 KiB; a block returns to the pool
+    // after the last kernel that touches its buffer.  Kernels run in order on one stream,
+    // so a block may be rewritten as soon as the kernel after its last reader is queued.
+    void enable_memory_planner() { plan_memory_ = true; }
+    const MemoryPlanStats& memory_plan() const { return mem_stats_; }
     int build();  // ensure_allocated on every buffer, compute raw pointers
 
     // execution_plan.rs:168-181: tight loop, no allocation, no per-launch sync.
@@ -93,8 +108,11 @@ class ExecutionPlan {
     int device_id() const { return device_id_; }
 
   private:
+    int plan_memory();
     int device_id_;
     bool built_ = false;
+    bool plan_memory_ = false, memory_planned_ = false;
+    MemoryPlanStats mem_stats_;
     std::vector<PreparedKernel> kernels_;
     std::vector<std::shared_ptr<Buffer>> buffers_;
     std::vector<size_t> outputs_;

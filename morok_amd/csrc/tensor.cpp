@@ -777,6 +777,7 @@ struct Scheduler {
     std::shared_ptr<Device> dev;
     std::unique_ptr<ExecutionPlan> plan;
     RealizeStats stats;
+    std::vector<TensorNode*> produced;  // nodes this realization gave a buffer
 
     int add_kernel(const std::shared_ptr<CachedKernel>& k, const std::vector<std::shared_ptr<Buffer>>& bufs, bool cached) {
         std::vector<size_t> idx;
@@ -863,11 +864,13 @@ struct Scheduler {
             if (s->buffer || s->kind == TKind::Reduce || s->kind == TKind::Contiguous || fusable(s)) {
                 MRK_TRY(materialize(s));
                 n->buffer = s->buffer;
+                produced.push_back(n);
                 return kOk;
             }
         }
         if (n->numel() == 0) {
             n->buffer = new_buffer(n);
+            produced.push_back(n);
             return kOk;
         }
         std::set<const TensorNode*> seen;
@@ -917,6 +920,7 @@ struct Scheduler {
         }
         MRK_TRY(rc);
         n->buffer = out;
+        produced.push_back(n);
         return kOk;
     }
 
@@ -929,6 +933,7 @@ struct Scheduler {
         bufs.insert(bufs.end(), g.inputs.begin(), g.inputs.end());
         MRK_TRY(add_kernel(ck, bufs, cached));
         n->buffer = out;
+        produced.push_back(n);
         return kOk;
     }
 
@@ -1074,7 +1079,19 @@ int Tensor::prepare(std::unique_ptr<ExecutionPlan>* out) const {
     s.plan.reset(new ExecutionPlan(n_->device_id));
     if (!n_->buffer) MRK_TRY(s.materialize(n_.get()));
     s.plan->set_outputs({s.plan->add_buffer(n_->buffer)});
-    MRK_TRY(s.plan->build());
+    // Intermediates share blocks by liveness (tensor/src/memory_planner.rs); their contents do
+    // not outlive the plan's execution, so their nodes go back to being lazy: only the root
+    // keeps its buffer.  MOROK_NO_MEMORY_PLANNER=1 keeps every intermediate resident.
+    const char* no_planner = std::getenv("MOROK_NO_MEMORY_PLANNER");
+    const bool planner = !(no_planner && no_planner[0] && no_planner[0] != '0');
+    if (planner) s.plan->enable_memory_planner();
+    int rc = s.plan->build();
+    if (planner || rc != kOk)
+        for (TensorNode* t : s.produced)
+            if (t != n_.get()) t->buffer = nullptr;
+    MRK_TRY(rc);
+    s.stats.buffers_reused = s.plan->memory_plan().buffers_reused;
+    s.stats.memory_saved = s.plan->memory_plan().memory_saved;
     s.stats.elapsed_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     g_stats = s.stats;
     *out = std::move(s.plan);

@@ -67,6 +67,8 @@ struct RealizeStats {
     std::vector<std::string> kernel_names;
     std::vector<std::string> kernel_sources;  // rendered HIP C; empty for hand-written kernels
     size_t cached_kernels = 0;
+    size_t buffers_reused = 0;  // memory planner (tensor/src/memory_planner.rs:84-96)
+    size_t memory_saved = 0;
     double elapsed_ms = 0.0;
 };
 

@@ -46,6 +46,11 @@ def last_cached_count():
     return lib.mrk_hip_tensor_last_cached_count()
 
 
+def last_memory_plan():
+    """(buffers reused, bytes saved) by the memory planner in the last realize / prepare."""
+    return lib.mrk_hip_tensor_last_buffers_reused(), lib.mrk_hip_tensor_last_memory_saved()
+
+
 def last_elapsed_ms():
     return lib.mrk_hip_tensor_last_elapsed_ms()
 

@@ -376,3 +376,41 @@ def test_queue_batches_until_submit_and_reports_errors(dev, shim):
         q2.submit(wait_timeout_ms=20)
     assert e.value.code == 12
     q2.wait(sig, 1).copy(a, b).submit(wait_timeout_ms=20)          # already reached: no wait
+
+
+def test_memory_planner_reuses_intermediates(T, shim, monkeypatch):
+    """tensor/src/memory_planner.rs: intermediates with disjoint lifetimes share blocks; outputs
+    and inputs never do."""
+    from morok_amd import decoder, synth, tensor
+
+    cfg = dict(batch=2, seq=64, hidden=256, heads=2, ffn=512)
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], 100, seed=1)
+    blk = decoder.DecoderBlock(w, cfg["batch"], cfg["seq"], cfg["hidden"], cfg["heads"], cfg["ffn"])
+    tok = T.Tensor.from_numpy(synth.randint((128,), 1, 1, 100))
+    dev = morok_amd.Device("HIP")
+    dev.lru_clear()
+    base = shim.mrk_shim_bytes_in_use()
+    out = blk.forward(tok).realize()
+    reused, saved = tensor.last_memory_plan()
+    planned_bytes = shim.mrk_shim_bytes_in_use() - base
+    assert reused >= 8 and saved >= 8 * 128 * 256 * 2
+    del out
+    dev.lru_clear()
+    monkeypatch.setenv("MOROK_NO_MEMORY_PLANNER", "1")
+    base = shim.mrk_shim_bytes_in_use()
+    out2 = blk.forward(tok).realize()
+    assert tensor.last_memory_plan() == (0, 0)
+    unplanned_bytes = shim.mrk_shim_bytes_in_use() - base
+    assert planned_bytes < unplanned_bytes and unplanned_bytes - planned_bytes >= saved // 2
+    del out2
+
+
+def test_planned_intermediates_become_lazy_again(T, shim):
+    x = zeros(T, (64, 64))
+    mid = x.try_add(1.0).contiguous()              # an intermediate of the first realization
+    a = mid.try_mul(2.0).sum(1).realize()
+    assert len(a.kernels()) == 2
+    b = mid.try_mul(3.0).realize()                 # mid's block may have been reused: it is recomputed
+    assert len(b.kernels()) == 2
+    c = a.try_add(1.0).realize()                   # a was an output: it is read, not recomputed
+    assert len(c.kernels()) == 1
