@@ -82,15 +82,22 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
     __bf16* Oh = O + (size_t)bh * Sq * kD;
     const int first_qt = causal ? q_tiles - 1 - unit : unit;
     const int npass = (causal && unit != first_qt) ? 2 : 1;
+    // key tiles a query tile visits
+    auto tiles_of = [&](int qt) {
+        int kend = Sk;
+        if (causal && qt * kQT + kQT < kend) kend = qt * kQT + kQT;
+        return (kend + kKT - 1) / kKT;
+    };
+    // The key tiles of the (up to) two passes form one sequence g = 0 .. ntot-1; the copies run
+    // two (K) and one (V) tiles ahead along that sequence, across the pass boundary, and tile
+    // g lives in LDS stage g & 1.
+    const int n0 = tiles_of(first_qt), n1 = npass > 1 ? tiles_of(unit) : 0, ntot = n0 + n1;
     for (int pass = 0; pass < npass; pass++) {
     const int qt = pass == 0 ? first_qt : unit;
     const int q0 = qt * kQT;
     const int qw0 = q0 + wave * 32;  // first query of this wave
-
-    // number of key tiles this workgroup visits
-    int kend = Sk;
-    if (causal && q0 + kQT < kend) kend = q0 + kQT;
-    const int ntiles = (kend + kKT - 1) / kKT;
+    const int ntiles = pass == 0 ? n0 : n1;
+    const int base = pass == 0 ? 0 : n0;  // sequence index of this pass's tile 0
 
     // ---- direct global -> LDS tile copies.  One instruction = 1 KB = 4 rows of 256 B.
     // wave w copies rows 16w .. 16w+15 of both tiles (4 instructions each).
@@ -128,6 +135,19 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
         }
     };
     auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    auto seq_k = [&](int g) {
+        if (g < ntot) dma_k(g < n0 ? g : g - n0, g & 1);
+    };
+    auto seq_v = [&](int g) {
+        if (g < ntot) dma_v(g < n0 ? g : g - n0, g & 1);
+    };
+    // the first pass starts its copies before anything else; a second pass finds its first
+    // tiles already copied (or on their way) by the first
+    if (pass == 0) {
+        seq_k(0);
+        seq_v(0);
+        seq_k(1);
+    }
 
     // ---- Q^T fragments: lane holds q = qw0 + l%32, d = 16*ds + 8*(l/32) .. +8
     bf16x8 qf[8];
@@ -238,10 +258,11 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
         }
         // K(j+1) and V(j) have landed; every wave is done with K(j) and V(j-1)
         tile_barrier();
-        if (j + 2 < ntiles) dma_k(j + 2, j & 1);
-        if (j + 1 < ntiles) dma_v(j + 1, (j + 1) & 1);
-        const char* sKn = smem + ((j + 1) & 1) * kTile;
-        const char* sV = smem + 2 * kTile + (j & 1) * kTile;
+        const int g = base + j;
+        seq_k(g + 2);
+        seq_v(g + 1);
+        const char* sKn = smem + ((g + 1) & 1) * kTile;
+        const char* sV = smem + 2 * kTile + (g & 1) * kTile;
         const float mb = m_run * scale_log2e;
 
         // ---- phase A: S(j+1) = K(j+1) Q^T on the matrix pipe, P(j) = exp2(S(j)*c - m*c) on
@@ -331,18 +352,18 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
         }
     };
 
-    if (pass) tile_barrier();  // every wave is done reading the previous pass's tiles
-    dma_k(0, 0);
-    dma_v(0, 0);
-    if (ntiles > 1) dma_k(1, 1);
-    tile_barrier();
+    if (pass == 0) tile_barrier();
     f32x16 sa[2], sb[2];
     float mxa, mxb = 0.0f;
-    qk_tile(smem, sa);
+    qk_tile(smem + (base & 1) * kTile, sa);
     mxa = mask_and_max(sa, 0, first_masked <= 0);
     {
         int j = 0;
-        const int jm = first_masked - 1 < ntiles ? first_masked - 1 : ntiles;  // iterations whose next tile is unmasked
+        // under the causal mask the tiles past the wave's own diagonal are invisible to it: it
+        // only keeps the barrier rhythm and copies its share of them for the other waves
+        int nmine = ntiles;
+        if (causal && (qw0 + 31) / kKT + 1 < nmine) nmine = (qw0 + 31) / kKT + 1;
+        const int jm = first_masked - 1 < nmine ? first_masked - 1 : nmine;  // iterations whose next tile is unmasked
         for (; j + 1 < jm; j += 2) {
             body(j, sa, mxa, sb, mxb, std::false_type{});
             body(j + 1, sb, mxb, sa, mxa, std::false_type{});
@@ -354,11 +375,19 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
             mxa = mxb;
             j++;
         }
-        for (; j + 1 < ntiles; j += 2) {
+        for (; j + 1 < nmine; j += 2) {
             body(j, sa, mxa, sb, mxb, std::true_type{});
             body(j + 1, sb, mxb, sa, mxa, std::true_type{});
         }
-        if (j < ntiles) body(j, sa, mxa, sb, mxb, std::true_type{});
+        if (j < nmine) {
+            body(j, sa, mxa, sb, mxb, std::true_type{});
+            j++;
+        }
+        for (; j < ntiles; j++) {
+            tile_barrier();
+            seq_k(base + j + 2);
+            seq_v(base + j + 1);
+        }
     }
 
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");

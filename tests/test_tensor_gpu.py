@@ -306,3 +306,26 @@ def test_large_elementwise_bandwidth_shape(T):
     t = T.Tensor.full([n], 1.5, uop.F32).try_mul(T.Tensor.full([n], 2.0, uop.F32)).contiguous()
     s = t.sum(0)
     assert float(s.to_numpy()) == 3.0 * n
+
+
+# ---------------------------------------------------------------- realize_binary.rs
+_NP_BIN = {"add": np.add, "sub": np.subtract, "mul": np.multiply, "fdiv": np.divide}
+
+
+@pytest.mark.parametrize("case", GOLD["realize_binary"]["cases"], ids=lambda c: c["name"])
+def test_realize_binary_cases(T, case):
+    a, b = f32(case["a"]), f32(case["b"])
+    got = T.Tensor.from_numpy(a).binary(case["op"], T.Tensor.from_numpy(b)).to_numpy()
+    want = f32(case["expected"]) if "expected" in case else _NP_BIN[case["op"]](a, b)
+    np.testing.assert_allclose(got, want, atol=case["tol"], rtol=0)
+
+
+@pytest.mark.parametrize("case", GOLD["realize_binary"]["chained"], ids=lambda c: c["name"])
+def test_realize_chained_expressions(T, case):
+    t = {k: T.Tensor.from_numpy(f32(case[k])) for k in "abcde" if k in case}
+    expr = {"add_mul": lambda: (t["a"] + t["b"]) * t["c"], "mul_add": lambda: t["a"] * t["b"] + t["c"],
+            "sub_div": lambda: (t["a"] - t["b"]) / t["c"],
+            "complex": lambda: ((t["a"] + t["b"]) * t["c"] - t["d"]).try_div(t["e"])}[case["name"]]()
+    got = expr.to_numpy()
+    assert len(expr.kernels()) == 1          # one fused elementwise kernel
+    np.testing.assert_allclose(got, f32(case["expected"]), atol=case["tol"], rtol=0)
