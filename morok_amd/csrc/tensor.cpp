@@ -120,7 +120,7 @@ Tensor Tensor::from_raw_bytes(int device_id, const void* data, size_t nbytes, co
     if (DeviceFactoryRegistry::global().device("HIP", device_id, &dev) != kOk) return Tensor();
     BufferOptions opt;
     auto buf = std::make_shared<Buffer>(dev->allocator, expected, opt);
-    if (buf->copyin(data, expected) != kOk) return Tensor();  // data.rs:66-67: copied at creation
+    if (expected && buf->copyin(data, expected) != kOk) return Tensor();  // data.rs:66-67: copied at creation
     return from_buffer(buf, shape, dtype);
 }
 
@@ -724,6 +724,7 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) 
             // every part is evaluated at a clamped coordinate; the right one is selected
             bool groups = coords[axis].aligned;  // a whole upcast group falls into one part
             for (const TensorRef& p : n->src) groups = groups && p->shape[axis] % g.width == 0;
+            if (n->numel() == 0) return is_float(ct) ? b.cf(0.0, ct) : b.ci(0, ct);
             const uint32_t pos = groups ? coords[axis].node : g.value(coords[axis]);
             const int64_t span = groups ? g.width : 1;
             int64_t start = 0;
@@ -731,6 +732,7 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) 
             std::vector<int64_t> ends;
             for (const TensorRef& p : n->src) {
                 const int64_t len = p->shape[axis];
+                if (len == 0) continue;  // an empty part contributes no element (and has no valid coordinate)
                 Coords sc = coords;
                 uint32_t rel = b.iadd(pos, g.ci(-start));
                 uint32_t lo = b.where(b.binary(BinaryOp::Lt, rel, g.ci(0)), g.ci(0), rel);
@@ -750,7 +752,15 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) 
             Coords ic(coords.begin(), coords.end() - 1);
             uint32_t row = emit(g, n->src[1].get(), ic);
             if (b.dtype(row).scalar != g.idx_t) row = b.cast(row, g.idx_t);
-            return emit(g, w, {Cx{row, 0, false}, coords.back()});
+            // An index outside [0, rows) selects nothing: the reference gathers through a
+            // comparison against arange(rows) (tensor/src/transformer.rs:12-25), which yields
+            // zeros there.  The row is clamped for the load and the value masked afterwards.
+            const int64_t rows = w->shape[0];
+            uint32_t below = b.binary(BinaryOp::Lt, row, g.ci(0)), above = b.binary(BinaryOp::Gt, row, g.ci(rows - 1));
+            uint32_t clamped = b.where(below, g.ci(0), b.where(above, g.ci(rows - 1), row));
+            uint32_t v = emit(g, w, {Cx{clamped, 0, false}, coords.back()});
+            uint32_t zero = is_float(ct) ? b.cf(0.0, ct) : b.ci(0, ct);
+            return b.where(b.binary(BinaryOp::Or, below, above), zero, v);
         }
         case TKind::Reduce:
         case TKind::Buffer: break;  // always materialised before being read

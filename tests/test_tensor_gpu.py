@@ -329,3 +329,21 @@ def test_realize_chained_expressions(T, case):
     got = expr.to_numpy()
     assert len(expr.kernels()) == 1          # one fused elementwise kernel
     np.testing.assert_allclose(got, f32(case["expected"]), atol=case["tol"], rtol=0)
+
+
+def test_embedding_out_of_range_index_reads_zero(T):
+    """An index outside the vocabulary selects nothing (the reference gathers by comparing
+    against arange(vocab)); on the GPU it must in particular not read out of bounds."""
+    w = np.arange(12, dtype=np.float32).reshape(3, 4) + 1
+    idx = np.array([2, -1, 0, 3, 7_000_000], dtype=np.int32)
+    got = T.Tensor.from_numpy(w).embedding(T.Tensor.from_numpy(idx)).to_numpy()
+    want = np.stack([w[2], np.zeros(4), w[0], np.zeros(4), np.zeros(4)]).astype(np.float32)
+    np.testing.assert_array_equal(got, want)
+
+
+def test_empty_tensors_and_empty_cat_parts(T):
+    e = T.Tensor.from_numpy(np.zeros((0, 4), np.float32))
+    assert e.try_add(1.0).to_numpy().shape == (0, 4)
+    x = np.arange(8, dtype=np.float32).reshape(2, 4)
+    c = T.Tensor.cat([T.Tensor.from_numpy(x), e, T.Tensor.from_numpy(x + 10)], 0)
+    np.testing.assert_array_equal(c.to_numpy(), np.concatenate([x, x + 10], 0))
