@@ -9,36 +9,58 @@ def _p(b):
     return C.c_void_p(b.ptr if isinstance(b, Buffer) else int(b))
 
 
+def _need(b, nbytes, what):
+    """Host-side shape check before a hand-written kernel is launched: a Buffer that is too
+    small for the stated shape is refused here instead of faulting on the GPU.  Raw device
+    addresses carry no size and are taken on trust."""
+    if isinstance(b, Buffer) and b.size < nbytes:
+        raise ValueError(f"{what}: buffer of {b.size} bytes is smaller than the {nbytes} bytes the shape needs")
+
+
 def softmax_f32(x, y, rows, cols, device_id=0, variant=0):
     """Fused row softmax (Tensor::softmax, tensor/src/activation.rs:90-101), last axis."""
+    for b, w in ((x, "softmax input"), (y, "softmax output")):
+        _need(b, rows * cols * 4, w)
     check(lib.mrk_hip_softmax_f32_variant(device_id, _p(x), _p(y), rows, cols, variant))
 
 
 def gemm_bf16(a, b, c, m, n, k, device_id=0, variant=0):
     """c[m,n] = a[m,k] @ b[k,n], bf16 row-major, f32 accumulate (Tensor::matmul on bf16,
     tensor/src/matmul.rs:82-110)."""
+    _need(a, m * k * 2, "gemm A")
+    _need(b, k * n * 2, "gemm B")
+    _need(c, m * n * 2, "gemm C")
     check(lib.mrk_hip_gemm_bf16_variant(device_id, _p(a), _p(b), _p(c), m, n, k, variant))
 
 
 def flash_attn_fwd_bf16(q, k, v, o, batch, heads, sq, sk, d, scale, causal=True, device_id=0):
     """Fused SDPA forward (Tensor::scaled_dot_product_attention, tensor/src/transformer.rs:78-137)."""
+    _need(q, batch * heads * sq * d * 2, "attention Q")
+    _need(o, batch * heads * sq * d * 2, "attention O")
+    _need(k, batch * heads * sk * d * 2, "attention K")
+    _need(v, batch * heads * sk * d * 2, "attention V")
     check(lib.mrk_hip_flash_attn_fwd_bf16(device_id, _p(q), _p(k), _p(v), _p(o), batch, heads, sq, sk, d, scale,
                                           int(causal)))
 
 
 def fill_normal(buf, n, sigma=1.0, seed=0, tensor_id=0, bf16=False, device_id=0):
     """Device-side synthetic normal(0, sigma) values (benchmark inputs)."""
+    _need(buf, n * (2 if bf16 else 4), "fill")
     check(lib.mrk_hip_fill(device_id, _p(buf), n, int(bf16), 1, seed, tensor_id, sigma, 0.0))
 
 
 def fill_uniform(buf, n, lo=-1.0, hi=1.0, seed=0, tensor_id=0, bf16=False, device_id=0):
+    _need(buf, n * (2 if bf16 else 4), "fill")
     check(lib.mrk_hip_fill(device_id, _p(buf), n, int(bf16), 0, seed, tensor_id, lo, hi))
 
 
 def fill_randint(buf, n, high, seed=0, tensor_id=0, device_id=0):
+    _need(buf, n * 4, "fill_randint")
     check(lib.mrk_hip_fill_randint(device_id, _p(buf), n, seed, tensor_id, high))
 
 
 def copy_kernel(src, dst, nbytes, device_id=0):
     """Streaming copy kernel of known traffic (counter calibration)."""
+    _need(src, nbytes, "copy source")
+    _need(dst, nbytes, "copy destination")
     check(lib.mrk_hip_copy_kernel(device_id, _p(src), _p(dst), nbytes))

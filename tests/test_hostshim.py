@@ -414,3 +414,21 @@ def test_planned_intermediates_become_lazy_again(T, shim):
     assert len(b.kernels()) == 2
     c = a.try_add(1.0).realize()                   # a was an output: it is read, not recomputed
     assert len(c.kernels()) == 1
+
+
+def test_ops_refuse_undersized_buffers(dev, shim):
+    from morok_amd import ops
+
+    small, big = dev.buffer(1024), dev.buffer(64 * 64 * 4)
+    n = shim.mrk_shim_launches()
+    with pytest.raises(ValueError):
+        ops.softmax_f32(small, big, 64, 64)
+    with pytest.raises(ValueError):
+        ops.gemm_bf16(big, big, small, 64, 64, 64)
+    with pytest.raises(ValueError):
+        ops.flash_attn_fwd_bf16(big, big, small, big, 1, 1, 64, 64, 128, 0.1)
+    with pytest.raises(ValueError):
+        ops.fill_normal(small, 1 << 20)
+    assert shim.mrk_shim_launches() == n             # nothing was launched
+    ops.softmax_f32(big, big, 64, 64)
+    assert shim.mrk_shim_last_kernel() == b"softmax_f32"
