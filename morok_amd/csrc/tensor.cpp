@@ -129,6 +129,8 @@ Tensor Tensor::from_buffer(std::shared_ptr<Buffer> buf, const std::vector<int64_
     for (int64_t d : shape) numel *= d;
     if (static_cast<size_t>(numel) * scalar_size(dtype) != buf->size())
         return bad(kSizeMismatch, "from_buffer: buffer size does not match shape " + shape_str(shape));
+    // kernels read and write 16 bytes per access: a view has to start on such a boundary
+    if (buf->offset() % 16 != 0) return bad(kInvalidArgument, "from_buffer: a buffer view must start at a multiple of 16 bytes");
     auto n = mk(TKind::Buffer, dtype, shape, {}, buf->device_id());
     n->buffer = std::move(buf);
     return Tensor(n);
@@ -838,7 +840,6 @@ struct Scheduler {
         for (const TensorRef& s : n->src) boundaries(s.get(), root, seen, out, max_numel);
     }
 
-    static bool all_dims_one_except_last2(const TensorNode* n) { return n->shape.size() == 2; }
     bool fusable(const TensorNode* n) const {
         if (!g_fusion || n->hint == HintKind::None) return false;
         switch (n->hint) {

@@ -432,3 +432,15 @@ def test_ops_refuse_undersized_buffers(dev, shim):
     assert shim.mrk_shim_launches() == n             # nothing was launched
     ops.softmax_f32(big, big, 64, 64)
     assert shim.mrk_shim_last_kernel() == b"softmax_f32"
+
+
+def test_tensor_from_buffer_view_alignment(T, dev):
+    b = dev.buffer(1024).ensure_allocated()
+    t = T.Tensor.from_buffer(b.view(64, 256), (64,), uop.F32)
+    assert t.shape == (64,)
+    with pytest.raises(MorokHipError) as e:
+        T.Tensor.from_buffer(b.view(4, 256), (64,), uop.F32)
+    assert e.value.code == 11
+    with pytest.raises(MorokHipError) as e:
+        T.Tensor.from_buffer(b, (100,), uop.F32)
+    assert e.value.code == 1
