@@ -935,14 +935,17 @@ struct Scheduler {
         return kOk;
     }
 
-    int finish_kernel(KernelGen& g, TensorNode* n, const std::shared_ptr<Buffer>& out, const std::string& name) {
+    int queue_kernel(KernelGen& g, const std::shared_ptr<Buffer>& out, const std::string& name) {
         LinearKernel k = g.b.finish();
         std::shared_ptr<CachedKernel> ck;
         bool cached = false;
         MRK_TRY(get_or_compile_linear_kernel(*dev, k, name.c_str(), &ck, &cached));
         std::vector<std::shared_ptr<Buffer>> bufs{out};
         bufs.insert(bufs.end(), g.inputs.begin(), g.inputs.end());
-        MRK_TRY(add_kernel(ck, bufs, cached));
+        return add_kernel(ck, bufs, cached);
+    }
+    int finish_kernel(KernelGen& g, TensorNode* n, const std::shared_ptr<Buffer>& out, const std::string& name) {
+        MRK_TRY(queue_kernel(g, out, name));
         n->buffer = out;
         produced.push_back(n);
         return kOk;
@@ -1005,9 +1008,27 @@ struct Scheduler {
         g.idx_t = max_numel >= (1LL << 31) ? Scalar::Int64 : Scalar::Int32;
         KernelBuilder& b = g.b;
         auto out = new_buffer(n);
-        uint32_t po = b.param(0, n->dtype, Nout);
         const Scalar ct = compute_dtype(n->dtype);
         const bool wave = R >= 128 && ct == Scalar::Float32 && (op == ReduceOp::Add || op == ReduceOp::Max);
+        // Two-stage reduction (split_reduceop, schedule/src/rangeify/kernel.rs:44-61): when one
+        // output folds at least 32768 inputs, the reduce range is cut into P segments (8 <= P <=
+        // 256, partial buffer of at most 2^22 elements) reduced by P times as many waves, and
+        // a second small kernel folds the P partials.
+        int64_t P = 1;
+        if (wave && R >= 32768) {
+            for (int64_t d = 256; d >= 8; d /= 2)
+                if (R / d >= 1024 && Nout * d <= (1LL << 22)) {
+                    P = d;
+                    break;
+                }
+        }
+        const int64_t chunk = (R + P - 1) / P;
+        std::shared_ptr<Buffer> partial;
+        if (P > 1) {
+            BufferOptions bo;
+            partial = std::make_shared<Buffer>(dev->allocator, static_cast<size_t>(Nout * P) * 4, bo);
+        }
+        uint32_t po = P > 1 ? b.param(0, Scalar::Float32, Nout * P) : b.param(0, n->dtype, Nout);
         auto identity = [&]() -> uint32_t {
             if (is_float(ct)) return b.cf(op == ReduceOp::Add ? 0.0 : op == ReduceOp::Mul ? 1.0 : op == ReduceOp::Max ? -INFINITY : INFINITY, ct);
             return b.ci(op == ReduceOp::Mul ? 1 : 0, ct);
@@ -1045,7 +1066,8 @@ struct Scheduler {
         // one wavefront per output element: lanes stride the flattened reduce space, partial
         // results are combined with the wave64 cross-lane reduction (the GROUP_REDUCE idea of
         // schedule/src/optimizer/heuristics.rs:370-392 without the LDS round trip)
-        const int64_t per_block = 4, grid = (Nout + per_block - 1) / per_block;
+        const int64_t W = Nout * P;  // wave-sized outputs of this kernel
+        const int64_t per_block = 4, grid = (W + per_block - 1) / per_block;
         if (grid > 2147483647LL) return fail(kInvalidArgument, "realize: reduction too large for one launch");
         uint32_t gx = b.special("gidx0", grid), lane = b.special("lidx0", 64), ly = b.special("lidx1", per_block);
         if (g.idx_t != Scalar::Int32) {
@@ -1053,29 +1075,53 @@ struct Scheduler {
             lane = b.cast(lane, g.idx_t);
             ly = b.cast(ly, g.idx_t);
         }
-        uint32_t o = b.iadd(b.imul(gx, per_block), ly);
-        uint32_t ogate = b.binary(BinaryOp::Lt, o, g.ci(Nout));
-        uint32_t oc = b.where(ogate, o, g.ci(Nout - 1));
+        uint32_t w = b.iadd(b.imul(gx, per_block), ly);
+        uint32_t wgate = b.binary(BinaryOp::Lt, w, g.ci(W));
+        uint32_t wc = b.where(wgate, w, g.ci(W - 1));
+        uint32_t oc = P > 1 ? b.idiv(wc, P) : wc;
+        uint32_t seg0 = P > 1 ? b.imul(b.imod(wc, P), chunk) : g.ci(0);  // first reduce index of the segment
         Coords coords = plain(unflatten(g, oc, n->shape));
-        const int64_t steps = (R + 63) / 64;
+        const int64_t steps = (chunk + 63) / 64;
         uint32_t rg = b.add(Op::Range, KernelBuilder::scalar(g.idx_t), {g.ci(steps)}, 0, 0, static_cast<uint16_t>(AxisType::Reduce));
-        uint32_t f = b.iadd(b.imul(rg, 64), lane);
-        uint32_t fgate = b.binary(BinaryOp::Lt, f, g.ci(R));
-        uint32_t fc = (R % 64 == 0) ? f : b.where(fgate, f, g.ci(R - 1));
+        uint32_t in_seg = b.iadd(b.imul(rg, 64), lane);
+        uint32_t f = b.iadd(seg0, in_seg);
+        const bool exact = chunk % 64 == 0 && chunk * P == R;
+        uint32_t fgate = b.binary(BinaryOp::And, b.binary(BinaryOp::Lt, in_seg, g.ci(chunk)), b.binary(BinaryOp::Lt, f, g.ci(R)));
+        uint32_t fc = exact ? f : b.where(fgate, f, g.ci(R - 1));
         std::vector<uint32_t> rc = unflatten(g, fc, rdims);
         for (size_t r = 0; r < n->arg.size(); r++) coords[n->arg[r]] = Cx{rc[r], 0, false};
         uint32_t v = emit(g, s, coords);
-        if (R % 64 != 0) v = b.where(fgate, v, identity());
+        if (!exact) v = b.where(fgate, v, identity());
         uint32_t red = b.reduce(op, v, {rg});
         b.end({rg});
         uint32_t total = b.wave_reduce(op, red);
         uint32_t first = b.binary(BinaryOp::Eq, lane, g.ci(0));
-        b.if_(b.binary(BinaryOp::And, first, ogate));
+        b.if_(b.binary(BinaryOp::And, first, wgate));
         uint32_t res = total;
-        if (b.dtype(res).scalar != n->dtype) res = b.cast(res, n->dtype);
-        b.store(b.index(po, o), res);
+        if (P == 1 && b.dtype(res).scalar != n->dtype) res = b.cast(res, n->dtype);
+        b.store(b.index(po, w), res);
         b.endif();
-        return finish_kernel(g, n, out, "r_" + std::to_string(Nout) + "_g" + std::to_string(R));
+        if (P == 1) return finish_kernel(g, n, out, "r_" + std::to_string(Nout) + "_g" + std::to_string(R));
+        MRK_TRY(queue_kernel(g, partial, "r_" + std::to_string(Nout) + "x" + std::to_string(P) + "_g" + std::to_string(chunk)));
+        // second stage: one work-item per output folds its P partials
+        KernelGen g2;
+        KernelBuilder& b2 = g2.b;
+        uint32_t po2 = b2.param(0, n->dtype, Nout);
+        uint32_t pin = g2.buffer_param(partial, Scalar::Float32, Nout * P);
+        const int64_t block2 = 64, grid2 = (Nout + block2 - 1) / block2;
+        uint32_t o2 = b2.iadd(b2.imul(b2.special("gidx0", grid2), block2), b2.special("lidx0", block2));
+        uint32_t gate2 = b2.binary(BinaryOp::Lt, o2, b2.ci(Nout));
+        uint32_t oc2 = b2.where(gate2, o2, b2.ci(Nout - 1));
+        uint32_t r2 = b2.range(P, 0, AxisType::Reduce);
+        uint32_t pv = b2.load(b2.index(pin, b2.iadd(b2.imul(oc2, P), r2)));
+        uint32_t red2 = b2.reduce(op, pv, {r2});
+        b2.end({r2});
+        b2.if_(gate2);
+        uint32_t res2 = red2;
+        if (b2.dtype(res2).scalar != n->dtype) res2 = b2.cast(res2, n->dtype);
+        b2.store(b2.index(po2, o2), res2);
+        b2.endif();
+        return finish_kernel(g2, n, out, "r_" + std::to_string(Nout) + "_" + std::to_string(P));
     }
 };
 

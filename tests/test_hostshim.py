@@ -444,3 +444,14 @@ def test_tensor_from_buffer_view_alignment(T, dev):
     with pytest.raises(MorokHipError) as e:
         T.Tensor.from_buffer(b, (100,), uop.F32)
     assert e.value.code == 1
+
+
+def test_large_reductions_are_split_in_two_stages(T, shim):
+    """split_reduceop (schedule/src/rangeify/kernel.rs:44-61): >= 32768 inputs per output."""
+    T.set_fusion(False)
+    t = zeros(T, (1 << 20,)).sum(0).realize()
+    assert len(t.kernels()) == 2 and t.kernels()[0].startswith("r_1x256_g")
+    t = zeros(T, (4, 70000)).max(1).realize()
+    assert len(t.kernels()) == 2
+    t = zeros(T, (64, 4096)).sum(1).realize()        # below the threshold: one kernel
+    assert len(t.kernels()) == 1

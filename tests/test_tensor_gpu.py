@@ -347,3 +347,22 @@ def test_empty_tensors_and_empty_cat_parts(T):
     x = np.arange(8, dtype=np.float32).reshape(2, 4)
     c = T.Tensor.cat([T.Tensor.from_numpy(x), e, T.Tensor.from_numpy(x + 10)], 0)
     np.testing.assert_array_equal(c.to_numpy(), np.concatenate([x, x + 10], 0))
+
+
+def test_split_reduction_values(T):
+    """Two-stage reductions (>= 32768 inputs per output), ragged segment ends included."""
+    rng = np.random.default_rng(41)
+    x = rng.standard_normal((3, 100003)).astype(np.float32)
+    t = T.Tensor.from_numpy(x)
+    s = t.sum(1)
+    np.testing.assert_allclose(s.to_numpy(), x.astype(np.float64).sum(1), rtol=1e-4, atol=1e-2)
+    assert len(s.kernels()) == 2
+    np.testing.assert_array_equal(t.max(1).to_numpy(), x.max(1))
+    y = rng.standard_normal((1 << 21,)).astype(np.float32)
+    ty = T.Tensor.from_numpy(y)
+    np.testing.assert_allclose(ty.sum(0).to_numpy(), y.astype(np.float64).sum(), rtol=1e-4, atol=1e-2)
+    z = rng.standard_normal((2, 200, 300)).astype(np.float32)   # several reduced axes, strided
+    np.testing.assert_allclose(T.Tensor.from_numpy(z).sum([1, 2]).to_numpy(), z.astype(np.float64).sum((1, 2)), rtol=1e-4,
+                               atol=1e-2)
+    np.testing.assert_allclose(T.Tensor.from_numpy(z).try_permute([1, 0, 2]).sum([0, 2]).to_numpy(),
+                               z.astype(np.float64).sum((1, 2)), rtol=1e-4, atol=1e-2)
