@@ -276,8 +276,8 @@ def test_tensor_int64_indexing_for_huge_views(T, shim):
     T.set_fusion(False)
     t = T.Tensor.full([1 << 16, 1 << 16], 1.0, uop.F32).sum(1)
     t.realize()
-    k = morok_amd.Kernel.get_or_compile  # noqa: F841  (the kernel compiled: the source is valid)
-    assert len(t.kernels()) == 1
+    # 65536 inputs per output: two-stage reduction; both generated sources compiled
+    assert len(t.kernels()) == 2
 
 
 def test_decoder_block_lowering(T, shim):
