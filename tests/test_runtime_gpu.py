@@ -210,3 +210,33 @@ def test_copy_and_compute_queues_with_signals(dev):
     for c in range(chunks):
         got = dst[c].copyout(np.float32, (n,))
         assert np.all(got == 2.0 * c + 1.0), c
+
+
+def test_concurrent_realize_from_threads(dev, oracle):
+    """Entry points are thread-safe (Renderer / Compiler are Send + Sync upstream, kernels are
+    shared through the cache): several host threads build, schedule and run graphs at once."""
+    import threading
+
+    from morok_amd import synth, tensor
+
+    errors, results = [], {}
+
+    def work(i):
+        try:
+            a = synth.uniform((128, 96), 50 + i, 0)
+            b = synth.uniform((96, 64), 50 + i, 1)
+            for _ in range(5):
+                t = tensor.Tensor.from_numpy(a).matmul(tensor.Tensor.from_numpy(b)).try_add(float(i)).softmax(-1)
+                results[i] = (t.to_numpy(), a, b)
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(6)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for i, (got, a, b) in results.items():
+        ref = oracle.softmax_f32(oracle.matmul_f32(a, b) + np.float32(i))
+        np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-6)
