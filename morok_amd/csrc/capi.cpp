@@ -263,6 +263,8 @@ int mrk_hip_program_spec_from_source(const char* name, const char* src, size_t b
     MRK_NONNULL(name);
     MRK_NONNULL(src);
     MRK_NONNULL(out);
+    if (nvars) MRK_NONNULL(var_names);
+    for (size_t i = 0; i < nvars; i++) MRK_NONNULL(var_names[i]);
     auto* h = new mrk_program_spec();
     h->s.name = name;
     h->s.src = src;
@@ -463,8 +465,15 @@ int mrk_hip_plan_execute_profiled(mrk_plan* plan, double* elapsed_ms, size_t cap
 }
 int mrk_hip_plan_execute_with_vars(mrk_plan* plan, const char* const* names, const int64_t* vals, size_t n) {
     MRK_NONNULL(plan);
+    if (n) {
+        MRK_NONNULL(names);
+        MRK_NONNULL(vals);
+    }
     std::vector<std::pair<std::string, int64_t>> kv;
-    for (size_t i = 0; i < n; i++) kv.emplace_back(names[i], vals[i]);
+    for (size_t i = 0; i < n; i++) {
+        MRK_NONNULL(names[i]);
+        kv.emplace_back(names[i], vals[i]);
+    }
     return plan->p->execute_with_vars(kv);
 }
 size_t mrk_hip_plan_kernel_count(const mrk_plan* plan) { return plan ? plan->p->kernel_count() : 0; }

@@ -303,7 +303,10 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     hipStream_t s = static_cast<hipStream_t>(stream);
     (void)hipGetLastError();
     const bool aligned = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) % 16) == 0;
-    if (variant != 2 && aligned && K > 0 && M % kBM == 0 && N % kBN == 0 && K % kBK == 0) {
+    // the tiled kernel addresses a tile's rows with 32-bit byte offsets from the tile origin:
+    // 255 rows of A (K elements each) and 49 rows of B (N elements each) must stay below 4 GiB
+    const bool offsets_fit = K <= (1L << 23) && N <= (1L << 25);
+    if (variant != 2 && aligned && offsets_fit && K > 0 && M % kBM == 0 && N % kBN == 0 && K % kBK == 0) {
         const int tm = (int)(M / kBM), tn = (int)(N / kBN);
         gemm_bf16_tile256<<<tm * tn, 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
                                                   static_cast<__bf16*>(C), (int)M, (int)N, (int)K, tm, tn);
