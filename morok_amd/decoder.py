@@ -39,11 +39,20 @@ def synthetic_weights(hidden, ffn, vocab, seed=0):
 class DecoderBlock:
     """Holds the device-resident weights and builds the lazy graph of one forward pass."""
 
-    def __init__(self, weights, batch, seq, hidden, heads, ffn, eps=1e-6, theta=10000.0, device_id=0):
+    def __init__(self, weights, batch, seq, hidden, heads, ffn, eps=1e-6, theta=10000.0, device_id=0,
+                 fuse_projections=True):
+        """fuse_projections: store Wq|Wk|Wv and W1|W3 side by side and run each group as one
+        product (same dot products, so the same bits): one launch instead of three / two, and the
+        gate+up product at hidden 4096 / ffn 11008 fills whole rounds of output tiles over the
+        compute units where two separate products each leave the last round two thirds empty."""
         assert hidden % heads == 0
         self.batch, self.seq, self.hidden, self.heads, self.ffn, self.eps = batch, seq, hidden, heads, ffn, eps
         self.dim = hidden // heads
         self.w = {k: Tensor.from_numpy(np.ascontiguousarray(weights[k]), uop.BF16, device_id) for k in WEIGHT_NAMES}
+        self.fused = bool(fuse_projections)
+        if self.fused:
+            self.w["Wqkv"] = Tensor.cat([self.w["Wq"], self.w["Wk"], self.w["Wv"]], 1).realize()
+            self.w["W13"] = Tensor.cat([self.w["W1"], self.w["W3"]], 1).realize()
         cos, sin = rope_tables(seq, self.dim, theta)
         self.cos_host, self.sin_host = cos, sin
         self.cos = Tensor.from_numpy(cos.reshape(1, 1, seq, self.dim // 2), device_id=device_id)
@@ -61,12 +70,21 @@ class DecoderBlock:
         w, T = self.w, self.batch * self.seq
         h = w["emb"].embedding(tokens).contiguous()
         xn = self._norm(h, w["w_an"])
-        q = self._heads(xn.matmul(w["Wq"])).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
-        k = self._heads(xn.matmul(w["Wk"])).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
-        v = self._heads(xn.matmul(w["Wv"]))
+        if self.fused:
+            qkv = xn.matmul(w["Wqkv"])
+            xq, xk, xv = (qkv.try_shrink([(0, T), (i * self.hidden, (i + 1) * self.hidden)]) for i in range(3))
+        else:
+            xq, xk, xv = xn.matmul(w["Wq"]), xn.matmul(w["Wk"]), xn.matmul(w["Wv"])
+        q = self._heads(xq).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
+        k = self._heads(xk).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
+        v = self._heads(xv)
         a = q.scaled_dot_product_attention(k, v, is_causal=True)
         a = a.try_permute([0, 2, 1, 3]).try_reshape([T, self.hidden])
         h2 = h.try_add(a.matmul(w["Wo"])).contiguous()
         xn2 = self._norm(h2, w["w_fn"])
-        g = xn2.matmul(w["W1"]).silu().try_mul(xn2.matmul(w["W3"]))
+        if self.fused:
+            gu = xn2.matmul(w["W13"])
+            g = gu.try_shrink([(0, T), (0, self.ffn)]).silu().try_mul(gu.try_shrink([(0, T), (self.ffn, 2 * self.ffn)]))
+        else:
+            g = xn2.matmul(w["W1"]).silu().try_mul(xn2.matmul(w["W3"]))
         return h2.try_add(g.matmul(w["W2"]))

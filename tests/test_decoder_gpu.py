@@ -6,10 +6,11 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-def run_block(cfg, tokens, weights):
+def run_block(cfg, tokens, weights, fused=True):
     from morok_amd import decoder, tensor, uop
 
-    blk = decoder.DecoderBlock(weights, cfg["batch"], cfg["seq"], cfg["hidden"], cfg["heads"], cfg["ffn"], cfg["eps"])
+    blk = decoder.DecoderBlock(weights, cfg["batch"], cfg["seq"], cfg["hidden"], cfg["heads"], cfg["ffn"], cfg["eps"],
+                               fuse_projections=fused)
     out = blk.forward(tensor.Tensor.from_numpy(tokens.astype(np.int32)))
     out.realize()
     return blk, out, out.kernels()
@@ -39,9 +40,14 @@ def test_decoder_block_vs_oracle(dev, oracle, cfg):
                                     cfg["heads"], cfg["ffn"], cfg["eps"])
     assert got.shape == ref.shape == (T, cfg["hidden"])
     assert rel_err(got, ref) <= 2e-2   # bf16 GEMM/attention tolerance
-    # the seven matmuls and the attention run as the hand-written kernels
-    assert sum(k.startswith("gemm_bf16") for k in kernels) == 7
+    # the matmuls (Wq|Wk|Wv and W1|W3 each as one product) and the attention run as the
+    # hand-written kernels
+    assert sum(k.startswith("gemm_bf16") for k in kernels) == 4
     assert sum(k.startswith("flash_fwd") for k in kernels) == 1
+    # seven separate products give the same bits: every output element is the same dot product
+    _, out7, kernels7 = run_block(cfg, tok, w, fused=False)
+    assert sum(k.startswith("gemm_bf16") for k in kernels7) == 7
+    assert np.array_equal(out7.to_numpy(), got)
 
 
 def test_decoder_block_full_size_properties(dev):
