@@ -12,15 +12,22 @@
 //
 // Main kernel: 256x256 output tile per workgroup of 4 waves (2x2), each wave 128x128 =
 // 4x4 MFMA tiles (256 accumulator registers), K step 64.  Tiles travel global -> LDS
-// directly (global_load_lds, 16 B per lane, no register staging) into two LDS stages,
-// one barrier per K step; the copy of tile kt+2 is issued among the MFMAs of the last
-// k-step of tile kt, a full tile of work ahead of its first use.  A is kept in LDS
+// directly (global_load_lds, 16 B per lane, no register staging).  A is kept in LDS
 // row-major with an XOR swizzle of its 16-byte chunks, B row-major (n contiguous) with
 // an XOR swizzle of its 32-byte granules and read through the transposing LDS load,
-// which hands each lane the 4 consecutive-k values of its column.  Fragments are
-// double-buffered in registers so LDS reads of k-step ks+1 run under the MFMAs of ks.  The MFMA is issued with swapped operands (D' = B^T A^T) so each
-// lane ends up with 4 consecutive n of one row, which makes the epilogue 8-byte LDS
-// writes and 16-byte coalesced global stores.
+// which hands each lane the 4 consecutive-k values of its column.  The MFMA is issued with
+// swapped operands (D' = B^T A^T) so each lane ends up with 4 consecutive n of one row,
+// which makes the epilogue 8-byte LDS writes and 16-byte coalesced global stores.
+//
+// Pipeline.  The vector-memory path takes a 1 KB copy every ~16 cycles, so the 64 copies a
+// workgroup issues per K step need about half of the step's MFMA time; issued in one burst
+// they stall the waves' instruction streams behind them.  They are therefore spread evenly,
+// four per 16-MFMA phase and wave: the LDS holds two A stages and three B stages (160 KB, all
+// of it), the copies of B tile kt+2 go out during the first two phases of tile kt into the
+// stage tile kt-1 left, the one barrier of the step sits in the middle of it, and the copies
+// of A tile kt+2 follow in the last two phases into the stage tile kt has just left.  For the
+// barrier to sit there every fragment of tile kt must have been read by then: fragments are
+// read two phases ahead of their MFMAs into four register slots (one per 16-deep k-step).
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
@@ -44,7 +51,7 @@ constexpr int kAStage = kBM * kBK * 2;         // 32768 B, row pitch 128 B, chun
 constexpr int kBStageSw = kBK * kBN * 2;       // 32768 B, row pitch 512 B, granule-swizzled
 constexpr int kCPitch = 128 * 2 + 16;          // epilogue staging pitch per wave
 constexpr int kCWave = 128 * kCPitch;          // 34816 B
-constexpr int kSmemMain = 2 * kAStage + 2 * kBStageSw;  // 131072
+constexpr int kSmemMain = 2 * kAStage + 3 * kBStageSw;  // 163840 = all 160 KB of the LDS
 constexpr int kSmemEpi = 4 * kCWave;                  // 139264
 constexpr int kSmem = kSmemEpi > kSmemMain ? kSmemEpi : kSmemMain;
 
@@ -70,7 +77,7 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
 __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                          __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
                                                          int tiles_n) {
-    // two stages; A stage: 256 rows x 128 B, 16 B chunks XOR-swizzled by ((row >> 1) & 7);
+    // A stage: 256 rows x 128 B, 16 B chunks XOR-swizzled by ((row >> 1) & 7);
     // B stage: 64 k-rows x 512 B, 32 B granules XOR-swizzled by (k & 3).
     __shared__ __attribute__((aligned(1024))) char smem[kSmem];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -78,20 +85,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
     const size_t m0 = (size_t)tile_m * kBM, n0 = (size_t)tile_n * kBN;
-    char* sA0 = smem;
-    char* sB0 = smem + 2 * kAStage;
+    char* sA0 = smem;                // two A stages
+    char* sB0 = smem + 2 * kAStage;  // three B stages
 
     // ---- direct global -> LDS copies: each wave moves 8 KB of A and 8 KB of B per tile,
     // one instruction = 64 lanes x 16 B = 1 KB of contiguous LDS.
     // A chunk q (1 KB = 8 rows): lane -> row q*8 + lane/8, LDS chunk lane%8 holds logical
     // chunk (lane%8) ^ ((row >> 1) & 7).  The LDS serves 16 lanes x 16 B per cycle over 64
     // banks; with 128 B rows this swizzle puts 16 consecutive rows of one logical chunk
-    // into 16 different 16 B slots.
-    // (two variants: (row >> 1) & 7 depends on the parity of q)
-    const unsigned a_voff0 = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (lane >> 4)) << 3)) * 2);
-    const unsigned a_voff1 = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (4 + (lane >> 4))) << 3)) * 2);
+    // into 16 different 16 B slots.  ((row >> 1) & 7 depends on the parity of q: two variants.)
     // B chunk q (1 KB = 2 k-rows): lane -> k-row q*2 + lane/32, LDS 16 B chunk lane%32 ->
     // granule (lane%32)/2 ^ (krow & 3).
+    const unsigned a_voff0 = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (lane >> 4)) << 3)) * 2);
+    const unsigned a_voff1 = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (4 + (lane >> 4))) << 3)) * 2);
     const int b_h = lane & 1, b_g = (lane & 31) >> 1, b_r = lane >> 5;
     const unsigned b_voff0 = (unsigned)(((size_t)(wave * 16 + b_r) * N + ((((b_g ^ (0 + b_r)) << 1) | b_h) << 3)) * 2);
     const unsigned b_voff1 = (unsigned)(((size_t)(wave * 16 + b_r) * N + ((((b_g ^ (2 + b_r)) << 1) | b_h) << 3)) * 2);
@@ -101,26 +107,18 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     const unsigned lds_b = (unsigned)(uintptr_t)LDS_PTR(char, sB0) + wave * 8192;
     // One direct copy: 64 lanes x 16 B land at LDS [m0, m0 + 1 KB); the compiler is not told
     // about it (it would otherwise wait for the copy before every later LDS read), so the
-    // waits are explicit: tile_barrier() drains vmcnt before the tile is consumed.
+    // waits are explicit in the barriers below.
     auto dma = [&](unsigned lds_addr, unsigned voff, const char* sbase) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :
                      : "s"(lds_addr), "v"(voff), "s"(sbase)
                      : "m0");
     };
-    // n = 0..7: A chunks, n = 8..15: B chunks of tile kt into `stage`
-    auto dma_one = [&](int n, int kt, int stage) {
-        if (n < 8) {
-            dma(lds_a + stage * kAStage + n * 1024, (n & 1) ? a_voff1 : a_voff0, a_tile + ((size_t)kt * kBK + (size_t)n * 8 * K) * 2);
-        } else {
-            const int q = n - 8;
-            dma(lds_b + stage * kBStageSw + q * 1024, (q & 1) ? b_voff1 : b_voff0,
-                b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
-        }
+    auto dma_a = [&](int q, int kt, int stage) {
+        dma(lds_a + stage * kAStage + q * 1024, (q & 1) ? a_voff1 : a_voff0, a_tile + ((size_t)kt * kBK + (size_t)q * 8 * K) * 2);
     };
-    auto dma_tile = [&](int kt, int stage) {
-#pragma unroll
-        for (int n = 0; n < 16; n++) dma_one(n, kt, stage);
+    auto dma_b = [&](int q, int kt, int stage) {
+        dma(lds_b + stage * kBStageSw + q * 1024, (q & 1) ? b_voff1 : b_voff0, b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
     };
 
     f32x16 acc[4][4];
@@ -142,96 +140,98 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     const int b_p0 = b_row_l + ((b_g0 ^ b_rr) << 5);                      // j = 0 (+128: j = 2)
     const int b_p1 = b_row_l + (((b_g0 ^ b_rr) ^ 2) << 5);                // j = 1 (+128: j = 3)
 
-    bf16x8 fa[2][4], fb[2][4];
-    auto load_frags = [&](int buf, int ks, int slot) {
-        const char* sA = sA0 + buf * kAStage + a_base_l + a_xo[ks];
-        const char* sB = sB0 + buf * kBStageSw + ks * 16 * 512;
+    bf16x8 fa[4][4], fb[4][4];  // fragment slot = k-step
+    // all but this wave's newest 8 copies (the B chunks issued since the last barrier) have
+    // landed, its LDS reads are complete; then all waves meet
+    auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    auto full_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+
+    const int KT = K / kBK;
 #pragma unroll
-        for (int i = 0; i < 4; i++) fa[slot][i] = *LDS_PTR(bf16x8, sA + i * 4096);
+    for (int q = 0; q < 8; q++) dma_a(q, 0, 0);
+#pragma unroll
+    for (int q = 0; q < 8; q++) dma_b(q, 0, 0);
+#pragma unroll
+    for (int q = 0; q < 8; q++) dma_a(q, KT > 1 ? 1 : 0, 1);
+#pragma unroll
+    for (int q = 0; q < 8; q++) dma_b(q, KT > 1 ? 1 : 0, 1);
+    full_barrier();
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) {
+        const char* sA = sA0 + a_base_l + a_xo[ks];
+        const char* sB = sB0 + ks * 16 * 512;
+#pragma unroll
+        for (int i = 0; i < 4; i++) fa[ks][i] = *LDS_PTR(bf16x8, sA + i * 4096);
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const int off = ((j & 1) ? b_p1 : b_p0) + (j >> 1) * 128;
             bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off));
             bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off + 4 * 512));
-            fb[slot][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            fb[ks][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         }
-    };
-    auto mma = [&](int slot) {
-#pragma unroll
-        for (int i = 0; i < 4; i++)
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][j], fa[slot][i], acc[i][j], 0, 0, 0);
-    };
-    // this wave's LDS reads and its direct-to-LDS copies are complete, then all waves meet
-    auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-
-    const int KT = K / kBK;
-    dma_tile(0, 0);
-    dma_tile(KT > 1 ? 1 : 0, 1);
-    tile_barrier();
-    load_frags(0, 0, 0);
-
-    auto iteration = [&](auto cur_c, int kt) {
-        constexpr int cur = decltype(cur_c)::value;
-        load_frags(cur, 1, 1);
-        mma(0);
-#pragma unroll
-        for (int n = 0; n < 16; n++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        load_frags(cur, 2, 0);
-        mma(1);
-#pragma unroll
-        for (int n = 0; n < 16; n++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        load_frags(cur, 3, 1);
-        mma(0);
-#pragma unroll
-        for (int n = 0; n < 16; n++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            if (n < 12) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // tile kt+1 has landed in the other stage; nobody reads stage `cur` any more
-        tile_barrier();
-        {
-            const int ktn = kt + 2 < KT ? kt + 2 : KT - 1;
-            const char* sAn = sA0 + (cur ^ 1) * kAStage + a_base_l + a_xo[0];
-            const char* sBn = sB0 + (cur ^ 1) * kBStageSw;
-            bf16x4 lo[4], hi[4];
-#pragma unroll
-            for (int n = 0; n < 16; n++) {
-                acc[n >> 2][n & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[1][n & 3], fa[1][n >> 2], acc[n >> 2][n & 3], 0, 0, 0);
-                if (n < 4) fa[0][n] = *LDS_PTR(bf16x8, sAn + n * 4096);
-                else if (n < 12) {
-                    const int j = (n - 4) >> 1;
-                    const int off = ((j & 1) ? b_p1 : b_p0) + (j >> 1) * 128;
-                    if ((n & 1) == 0) lo[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off));
-                    else hi[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off + 4 * 512));
-                }
-                dma_one(n, ktn, cur);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-#pragma unroll
-            for (int j = 0; j < 4; j++) fb[0][j] = __builtin_shufflevector(lo[j], hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-    };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    int kt = 0;
-    for (; kt + 1 < KT; kt += 2) {
-        iteration(I0{}, kt);
-        iteration(I1{}, kt + 1);
     }
-    if (kt < KT) iteration(I0{}, kt);
-    tile_barrier();
+
+    // One phase = the 16 MFMAs of k-step p of the current tile (fragment slot p) with the other
+    // pipes' work slotted between them: the 12 LDS reads of the fragments needed two phases
+    // later (slot p ^ 2, from sAn / sBn) and four chunk copies of tile kt2: phases 0-1 its B
+    // chunks into B stage st2, phases 2-3 (after the barrier) its A chunks into A stage `cur`.
+    auto phase = [&](auto p_c, auto cur_c, int kt2, int st2, const char* sAn, const char* sBn) {
+        constexpr int p = decltype(p_c)::value, cur = decltype(cur_c)::value;
+        constexpr int slot = p, nslot = p ^ 2;
+        bf16x4 lo[4], hi[4];
+#pragma unroll
+        for (int n = 0; n < 16; n++) {
+            acc[n >> 2][n & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][n & 3], fa[slot][n >> 2], acc[n >> 2][n & 3], 0, 0, 0);
+            if (n < 4) fa[nslot][n] = *LDS_PTR(bf16x8, sAn + n * 4096);
+            else if (n < 12) {
+                const int j = (n - 4) >> 1;
+                const int off = ((j & 1) ? b_p1 : b_p0) + (j >> 1) * 128;
+                if ((n & 1) == 0) lo[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off));
+                else hi[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off + 4 * 512));
+            }
+            if ((n & 3) == 1) {
+                const int q = (p & 1) * 4 + (n >> 2);
+                if (p < 2) dma_b(q, kt2, st2);
+                else dma_a(q, kt2, cur);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) fb[nslot][j] = __builtin_shufflevector(lo[j], hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using C0 = std::integral_constant<int, 0>;
+    using C1 = std::integral_constant<int, 1>;
+    using C2 = std::integral_constant<int, 2>;
+    using C3 = std::integral_constant<int, 3>;
+    // tile kt: A in stage cur = kt & 1, B in stage st = kt % 3 (next tile's B in stn, the one after goes to st2)
+    auto iteration = [&](auto cur_c, int kt, int st, int stn, int st2) {
+        constexpr int cur = decltype(cur_c)::value;
+        using C = std::integral_constant<int, cur>;
+        const int kt2 = kt + 2 < KT ? kt + 2 : KT - 1;
+        const char* sAc = sA0 + cur * kAStage + a_base_l;
+        const char* sBc = sB0 + st * kBStageSw;
+        const char* sAx = sA0 + (cur ^ 1) * kAStage + a_base_l;
+        const char* sBx = sB0 + stn * kBStageSw;
+        phase(C0{}, C{}, kt2, st2, sAc + a_xo[2], sBc + 2 * 16 * 512);
+        phase(C1{}, C{}, kt2, st2, sAc + a_xo[3], sBc + 3 * 16 * 512);
+        // tile kt+1 has landed; nobody reads A stage cur any more
+        tile_barrier();
+        phase(C2{}, C{}, kt2, st2, sAx + a_xo[0], sBx);
+        phase(C3{}, C{}, kt2, st2, sAx + a_xo[1], sBx + 1 * 16 * 512);
+    };
+    {
+        int kt = 0, st = 0;
+        auto nx = [](int s) { return s == 2 ? 0 : s + 1; };
+        for (; kt + 1 < KT; kt += 2) {
+            iteration(C0{}, kt, st, nx(st), nx(nx(st)));
+            st = nx(st);
+            iteration(C1{}, kt + 1, st, nx(st), nx(nx(st)));
+            st = nx(st);
+        }
+        if (kt < KT) iteration(C0{}, kt, st, nx(st), nx(nx(st)));
+    }
+    full_barrier();
 
     // Epilogue.  With swapped operands lane l of tile (i, j) holds, in registers 4g..4g+3,
     // C[m = i*32 + l%32][n = j*32 + 8g + 4*(l/32) + 0..3].
