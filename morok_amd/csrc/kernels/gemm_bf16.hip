@@ -155,7 +155,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     for (int q = 0; q < 8; q++) dma_a(q, KT > 1 ? 1 : 0, 1);
 #pragma unroll
     for (int q = 0; q < 8; q++) dma_b(q, KT > 1 ? 1 : 0, 1);
-    full_barrier();
+    // tile 0 has landed (the 16 copies of tile 1 may still be in flight; the first
+    // tile_barrier() covers them)
+    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
         const char* sA = sA0 + a_base_l + a_xo[ks];
