@@ -547,8 +547,12 @@ struct KernelGen {
     std::vector<std::shared_ptr<Buffer>> inputs;
     std::vector<uint32_t> input_params;
     std::vector<Scalar> input_dtypes;
-    std::map<std::pair<const TensorNode*, Coords>, uint32_t> memo;
-    std::map<std::tuple<uint32_t, uint32_t, int64_t>, uint32_t> vec_loads;  // (param, base index, group) -> vector value
+    // Condition under which the value being emitted is used at all (-1: always): the parts of
+    // a cat are selected by position, so the loads of a part are predicated on the position
+    // falling into it and the lanes of the other parts issue no memory request.
+    int64_t gate = -1;
+    std::map<std::tuple<const TensorNode*, Coords, int64_t>, uint32_t> memo;  // (node, coordinates, gate) -> value
+    std::map<std::tuple<uint32_t, uint32_t, int64_t, int64_t>, uint32_t> vec_loads;  // (param, base index, group, gate) -> vector value
 
     uint32_t ci(int64_t v) { return b.ci(v, idx_t); }
     uint32_t value(const Cx& c) { return c.off ? b.iadd(c.node, ci(c.off)) : c.node; }
@@ -620,18 +624,20 @@ uint32_t emit_load(KernelGen& g, const TensorNode* n, const Coords& coords) {
     if (flat.aligned && per_load > 1 && n->dtype != Scalar::Bool) {
         // one vector load per group of `per_load` consecutive elements, shared by the group
         const int64_t group = flat.off / per_load;
-        auto key = std::make_tuple(p, flat.node, group);
+        auto key = std::make_tuple(p, flat.node, group, g.gate);
         auto it = g.vec_loads.find(key);
         uint32_t vec;
         if (it != g.vec_loads.end()) {
             vec = it->second;
         } else {
             uint32_t at = group ? b.iadd(flat.node, g.ci(group * per_load)) : flat.node;
-            vec = b.load(b.index(p, at), static_cast<int>(per_load));
+            uint32_t ix = g.gate >= 0 ? b.index_gated(p, at, static_cast<uint32_t>(g.gate)) : b.index(p, at);
+            vec = b.load(ix, static_cast<int>(per_load));
             g.vec_loads[key] = vec;
         }
         return b.gep(vec, static_cast<int>(flat.off % per_load));
     }
+    if (g.gate >= 0) return b.load(b.index_gated(p, g.value(flat), static_cast<uint32_t>(g.gate)));
     return b.load(b.index(p, g.value(flat)));
 }
 
@@ -740,7 +746,14 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) 
                 uint32_t lo = b.where(b.binary(BinaryOp::Lt, rel, g.ci(0)), g.ci(0), rel);
                 uint32_t cl = b.where(b.binary(BinaryOp::Gt, lo, g.ci(len - span)), g.ci(len - span), lo);
                 sc[axis] = groups ? Cx{cl, coords[axis].off, true} : Cx{cl, 0, false};
+                // this part is live where start <= pos < start + len (and the enclosing gate holds)
+                const int64_t outer = g.gate;
+                uint32_t live = b.binary(BinaryOp::And, b.binary(BinaryOp::Ge, pos, g.ci(start)),
+                                         b.binary(BinaryOp::Lt, pos, g.ci(start + len)));
+                if (outer >= 0) live = b.binary(BinaryOp::And, static_cast<uint32_t>(outer), live);
+                g.gate = live;
                 vals.push_back(emit(g, p.get(), sc));
+                g.gate = outer;
                 start += len;
                 ends.push_back(start);
             }
@@ -771,7 +784,7 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) 
 }
 
 uint32_t emit(KernelGen& g, const TensorNode* n, const Coords& coords) {
-    auto key = std::make_pair(n, coords);
+    auto key = std::make_tuple(n, coords, g.gate);
     auto it = g.memo.find(key);
     if (it != g.memo.end()) return it->second;
     uint32_t v = emit_uncached(g, n, coords);
