@@ -25,13 +25,19 @@ def _run(dev, x, variant=0, via_program=False):
     return by.copyout(np.float32, (rows, cols))
 
 
-def _check(y, ref):
+def _check(y, ref, rtol=RTOL):
     assert np.all(np.isfinite(y))
     rel = np.abs(y - ref) / np.maximum(ref, np.float32(1e-30))
     # entries that underflow towards denormals carry no relative precision; bound them absolutely
     big = ref > 1e-30
-    assert rel[big].max() <= RTOL, rel[big].max()
-    assert np.abs(y - ref).max() <= RTOL * ref.max()
+    assert rel[big].max() <= rtol, rel[big].max()
+    assert np.abs(y - ref).max() <= rtol * ref.max()
+
+
+def _softmax_f64(x):
+    x = x.astype(np.float64)
+    e = np.exp(x - x.max(-1, keepdims=True))
+    return e / e.sum(-1, keepdims=True)
 
 
 @pytest.mark.parametrize("shape", [(1, 4), (3, 8), (64, 256), (33, 1000), (17, 1024), (8, 2048), (5, 4100),
@@ -40,6 +46,34 @@ def _check(y, ref):
 def test_softmax_parity_shapes(dev, oracle, shape, variant):
     x = synth.normal(shape, 2, 0, sigma=2.0)
     _check(_run(dev, x, variant), oracle.softmax_f32(x))
+
+
+@pytest.mark.parametrize("shape", [(64, 8191), (16, 12288), (8, 16384), (6, 32000), (5, 50257), (4, 65536),
+                                   (3, 65537), (3, 131072), (2, 100003), (7, 8193)])
+def test_softmax_long_and_unaligned_rows(dev, oracle, shape):
+    """Rows beyond 8192 columns stay in registers up to 65536 (512 / 1024 work-items per row),
+    longer ones take the two-sweep kernel; odd column counts give every row its own alignment."""
+    x = synth.normal(shape, 2, 1, sigma=2.0)
+    y = _run(dev, x)
+    # The oracle adds a row's exponentials one after another in f32 like the CPU backend it
+    # restates; over 10^5 terms that sum is itself 2.5e-5 off the exact one, so against the
+    # oracle these rows are held to the 1e-4 of f32 reductions and to 1e-5 against float64.
+    _check(y, oracle.softmax_f32(x), rtol=1e-4)
+    _check(y, _softmax_f64(x), rtol=1e-5)
+
+
+def test_softmax_rows_misaligned_differently_in_x_and_y(dev, oracle):
+    """Views whose bases are not 16-byte aligned alike fall back to element-wise access."""
+    rows, cols = 5, 70001
+    x = synth.normal((rows, cols), 2, 2, sigma=2.0)
+    bx = dev.buffer(x.nbytes + 64)
+    by = dev.buffer(x.nbytes + 64)
+    vx, vy = bx.view(4, x.nbytes), by.view(8, x.nbytes)
+    vx.copyin(x)
+    ops.softmax_f32(vx.ptr, vy.ptr, rows, cols, dev.device_id)
+    y = vy.copyout(np.float32, (rows, cols))
+    _check(y, oracle.softmax_f32(x), rtol=1e-4)
+    _check(y, _softmax_f64(x), rtol=1e-5)
 
 
 def test_softmax_config_slice_of_full_shape(dev, oracle):
