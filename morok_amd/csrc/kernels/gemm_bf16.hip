@@ -96,11 +96,26 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     // into 16 different 16 B slots.  ((row >> 1) & 7 depends on the parity of q: two variants.)
     // B chunk q (1 KB = 2 k-rows): lane -> k-row q*2 + lane/32, LDS 16 B chunk lane%32 ->
     // granule (lane%32)/2 ^ (krow & 3).
-    const unsigned a_voff0 = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (lane >> 4)) << 3)) * 2);
-    const unsigned a_voff1 = (unsigned)(((size_t)(wave * 64 + (lane >> 3)) * K + (((lane & 7) ^ (4 + (lane >> 4))) << 3)) * 2);
+    // Ragged edges: a tile may reach past row M or column N.  Source rows / column chunks
+    // beyond the edge are redirected to the last valid one (the duplicates only feed outputs
+    // the epilogue does not store), which costs nothing per K step: the redirected offsets do
+    // not depend on it.  N % 8 == 0 keeps the redirected chunk 16-byte aligned.
+    unsigned a_voff[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) {
+        size_t row = m0 + wave * 64 + q * 8 + (lane >> 3);
+        row = row < (size_t)M ? row : (size_t)M - 1;
+        const int chunk = (lane & 7) ^ ((q & 1) * 4 + (lane >> 4));
+        a_voff[q] = (unsigned)(((row - m0) * K + (chunk << 3)) * 2);
+    }
     const int b_h = lane & 1, b_g = (lane & 31) >> 1, b_r = lane >> 5;
-    const unsigned b_voff0 = (unsigned)(((size_t)(wave * 16 + b_r) * N + ((((b_g ^ (0 + b_r)) << 1) | b_h) << 3)) * 2);
-    const unsigned b_voff1 = (unsigned)(((size_t)(wave * 16 + b_r) * N + ((((b_g ^ (2 + b_r)) << 1) | b_h) << 3)) * 2);
+    unsigned b_voff[2];
+#pragma unroll
+    for (int par = 0; par < 2; par++) {
+        size_t col = n0 + ((((b_g ^ (par * 2 + b_r)) << 1) | b_h) << 3);
+        col = col + 8 <= (size_t)N ? col : (size_t)N - 8;
+        b_voff[par] = (unsigned)(((size_t)(wave * 16 + b_r) * N + (col - n0)) * 2);
+    }
     const char* a_tile = reinterpret_cast<const char*>(A + m0 * K);
     const char* b_tile = reinterpret_cast<const char*>(B + n0);
     const unsigned lds_a = (unsigned)(uintptr_t)LDS_PTR(char, sA0) + wave * 8192;
@@ -115,10 +130,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
                      : "m0");
     };
     auto dma_a = [&](int q, int kt, int stage) {
-        dma(lds_a + stage * kAStage + q * 1024, (q & 1) ? a_voff1 : a_voff0, a_tile + ((size_t)kt * kBK + (size_t)q * 8 * K) * 2);
+        dma(lds_a + stage * kAStage + q * 1024, a_voff[q], a_tile + (size_t)kt * kBK * 2);
     };
     auto dma_b = [&](int q, int kt, int stage) {
-        dma(lds_b + stage * kBStageSw + q * 1024, (q & 1) ? b_voff1 : b_voff0, b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
+        dma(lds_b + stage * kBStageSw + q * 1024, b_voff[q & 1], b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
     };
 
     f32x16 acc[4][4];
@@ -251,13 +266,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
                 *LDS_PTR(bf16x4, sC + ml * kCPitch + nl * 2) = h;
             }
     __syncthreads();
-    __bf16* Cg = C + (m0 + wm * 128) * N + n0 + wn * 128;
+    const size_t row0 = m0 + wm * 128, col0 = n0 + wn * 128;
+    __bf16* Cg = C + row0 * N + col0;
 #pragma unroll 4
     for (int it = 0; it < 32; it++) {
         const int r = it * 4 + (lane >> 4);
         const int ch = lane & 15;
         u32x4 v = *LDS_PTR(u32x4, sC + r * kCPitch + ch * 16);
-        *reinterpret_cast<u32x4*>(Cg + (size_t)r * N + ch * 8) = v;
+        if (row0 + r < (size_t)M && col0 + ch * 8 + 8 <= (size_t)N) *reinterpret_cast<u32x4*>(Cg + (size_t)r * N + ch * 8) = v;
     }
 }
 
@@ -308,8 +324,10 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     // the tiled kernel addresses a tile's rows with 32-bit byte offsets from the tile origin:
     // 255 rows of A (K elements each) and 49 rows of B (N elements each) must stay below 4 GiB
     const bool offsets_fit = K <= (1L << 23) && N <= (1L << 25);
-    if (variant != 2 && aligned && offsets_fit && K > 0 && M % kBM == 0 && N % kBN == 0 && K % kBK == 0) {
-        const int tm = (int)(M / kBM), tn = (int)(N / kBN);
+    // any M; N in whole 16-byte chunks; K in whole 64-deep steps (a partial step would need zero
+    // fill, which a direct-to-LDS copy cannot do)
+    if (variant != 2 && aligned && offsets_fit && K > 0 && N % 8 == 0 && K % kBK == 0) {
+        const int tm = (int)((M + kBM - 1) / kBM), tn = (int)((N + kBN - 1) / kBN);
         gemm_bf16_tile256<<<tm * tn, 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
                                                   static_cast<__bf16*>(C), (int)M, (int)N, (int)K, tm, tn);
     } else {
