@@ -191,7 +191,8 @@ void mrk_hip_program_destroy(mrk_program* p);
 /* Hand-written gfx950 kernels exposed as Programs, so that an ExecutionPlan can hold them
  * next to generated kernels.  `kind` and the meaning of `params`:
  *   "softmax_f32"     params = {rows, cols}                         buffers = {y, x}
- *   "gemm_bf16"       params = {M, N, K}                            buffers = {c, a, b}
+ *   "gemm_bf16"       params = {M, N, K} or {M, N, K, batch}        buffers = {c, a, b}
+ *                     (batch: that many products over matrices stored back to back)
  *   "flash_fwd_bf16"  params = {B*H, Sq, Sk, D, causal, f32 bits of scale}   buffers = {o, q, k, v}
  * Buffer order follows the reference's PARAM numbering: outputs first. */
 int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_program** out);

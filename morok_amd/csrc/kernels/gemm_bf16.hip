@@ -82,6 +82,10 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     __shared__ __attribute__((aligned(1024))) char smem[kSmem];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave >> 1, wn = wave & 1;
+    // blockIdx.y: which of the back-to-back stored products
+    A += (size_t)blockIdx.y * M * K;
+    B += (size_t)blockIdx.y * K * N;
+    C += (size_t)blockIdx.y * M * N;
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
     const size_t m0 = (size_t)tile_m * kBM, n0 = (size_t)tile_n * kBN;
@@ -286,6 +290,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic(const __bf16* __restric
     const int lane = threadIdx.x & 63;
     const long tile = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (tile >= total_tiles) return;
+    A += (size_t)blockIdx.y * M * K;
+    B += (size_t)blockIdx.y * K * N;
+    C += (size_t)blockIdx.y * M * N;
     const long m0 = (tile / tiles_n) * 32, n0 = (tile % tiles_n) * 32;
     const long m = m0 + (lane & 31), n = n0 + (lane & 31);
     const int kg = 8 * (lane >> 5);
@@ -314,9 +321,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic(const __bf16* __restric
 
 namespace mrk {
 
-int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant) {
+int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
+                     long batch) {
     using namespace mrk::dev;
-    if (M <= 0 || N <= 0) return 0;
+    if (M <= 0 || N <= 0 || batch <= 0) return 0;
+    if (batch > 65535) return (int)hipErrorInvalidValue;  // grid y extent
     if (M > 0x7fffffffL || N > 0x7fffffffL || K > 0x7fffffffL || K < 0) return (int)hipErrorInvalidValue;
     hipStream_t s = static_cast<hipStream_t>(stream);
     (void)hipGetLastError();
@@ -328,14 +337,14 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     // fill, which a direct-to-LDS copy cannot do)
     if (variant != 2 && aligned && offsets_fit && K > 0 && N % 8 == 0 && K % kBK == 0) {
         const int tm = (int)((M + kBM - 1) / kBM), tn = (int)((N + kBN - 1) / kBN);
-        gemm_bf16_tile256<<<tm * tn, 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
+        gemm_bf16_tile256<<<dim3((unsigned)(tm * tn), (unsigned)batch), 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
                                                   static_cast<__bf16*>(C), (int)M, (int)N, (int)K, tm, tn);
     } else {
         const long tm = (M + 31) / 32, tn = (N + 31) / 32;
         const long total = tm * tn;
         const long blocks = (total + 3) / 4;
         if (blocks > 0x7fffffffL) return (int)hipErrorInvalidValue;
-        gemm_bf16_generic<<<(unsigned)blocks, 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
+        gemm_bf16_generic<<<dim3((unsigned)blocks, (unsigned)batch), 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
                                                            static_cast<__bf16*>(C), (int)M, (int)N, (int)K, (int)tn,
                                                            total);
     }

@@ -11,8 +11,11 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 
 
 // C[M,N] = A[M,K] * B[K,N]; bf16 row-major operands, f32 accumulate, bf16 result.
-// variant 0 = choose by shape, 2 = force the any-shape kernel.
-int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant);
+// variant 0 = choose by shape, 2 = force the any-shape kernel.  batch > 1: that many
+// independent products over matrices stored back to back (A [batch,M,K], B [batch,K,N],
+// C [batch,M,N]), one launch.
+int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
+                     long batch = 1);
 
 // O = softmax(Q K^T * scale [causal]) V; Q [BH,Sq,D], K/V [BH,Sk,D], O [BH,Sq,D] bf16, D = 128,
 // scale > 0.  Causal: key j visible to query i iff j <= i.

@@ -861,8 +861,21 @@ struct Scheduler {
                        n->arg[0] == static_cast<int64_t>(n->shape.size()) - 1 && n->numel() > 0;
             case HintKind::Matmul: {
                 const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
-                if (a->shape.size() != 2 || w->shape.size() != 2 || a->dtype != w->dtype) return false;
-                if (a->dtype == Scalar::BFloat16) return n->dtype == Scalar::BFloat16 && n->numel() > 0;
+                if (a->dtype != w->dtype) return false;
+                if (a->dtype == Scalar::BFloat16) {
+                    // [..., M, K] x [K, N] is one product over the flattened leading axes;
+                    // equal leading axes on both sides are that many products in one launch
+                    if (n->dtype != Scalar::BFloat16 || n->numel() == 0 || a->shape.size() < 2) return false;
+                    if (w->shape.size() == 2) return true;
+                    if (w->shape.size() != a->shape.size()) return false;
+                    int64_t batch = 1;
+                    for (size_t i = 0; i + 2 < a->shape.size(); i++) {
+                        if (a->shape[i] != w->shape[i]) return false;
+                        batch *= a->shape[i];
+                    }
+                    return batch <= 65535;
+                }
+                if (a->shape.size() != 2 || w->shape.size() != 2) return false;
                 if (a->dtype == Scalar::Float32)
                     return a->shape[0] % 64 == 0 && w->shape[1] % 64 == 0 && a->shape[0] > 0 && w->shape[1] > 0;
                 return false;
@@ -914,9 +927,12 @@ struct Scheduler {
             rc = builtin("softmax_f32", {rows, cols}, {out, n->hint_inputs[0]->buffer});
         } else if (n->hint == HintKind::Matmul) {
             const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
-            const int64_t M = a->shape[0], K = a->shape[1], N = w->shape[1];
+            const int64_t K = a->shape.back(), N = w->shape.back();
+            int64_t M = a->shape[a->shape.size() - 2], batch = 1;
+            for (size_t i = 0; i + 2 < a->shape.size(); i++) (w->shape.size() == 2 ? M : batch) *= a->shape[i];
             if (a->dtype == Scalar::BFloat16) {
-                rc = builtin("gemm_bf16", {M, N, K}, {out, a->buffer, w->buffer});
+                rc = batch == 1 ? builtin("gemm_bf16", {M, N, K}, {out, a->buffer, w->buffer})
+                                : builtin("gemm_bf16", {M, N, K, batch}, {out, a->buffer, w->buffer});
             } else {
                 // MOROK_BEAM=<width> selects the LOCAL/UPCAST/UNROLL choices by timed search
                 // (cached on disk) instead of the fixed heuristic (tensor/src/realize.rs:1160-1250)

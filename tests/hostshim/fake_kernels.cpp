@@ -9,7 +9,7 @@ int launch_softmax_f32(void*, const void*, void*, long, long, int) {
     mrk_shim_note_launch("softmax_f32");
     return 0;
 }
-int launch_gemm_bf16(void*, const void*, const void*, void*, long, long, long, int) {
+int launch_gemm_bf16(void*, const void*, const void*, void*, long, long, long, int, long) {
     mrk_shim_note_launch("gemm_bf16");
     return 0;
 }

@@ -129,6 +129,32 @@ def test_matmul_bf16(T, fusion, oracle):
         assert c.kernels() == ["gemm_bf16_tile256"] or c.kernels()[0].startswith("gemm_bf16")
 
 
+@pytest.mark.parametrize("ashape,wshape", [((3, 100, 64), (64, 40)), ((2, 3, 128, 64), (2, 3, 64, 72)),
+                                           ((5, 37, 128), (5, 128, 8)), ((2, 2, 50, 192), (192, 264))])
+def test_matmul_bf16_leading_axes(T, fusion, oracle, ashape, wshape):
+    """[..., M, K] x [K, N] (one product over the flattened leading axes) and [..., M, K] x
+    [..., K, N] with equal leading axes (that many products, one launch of the hand-written
+    kernel); generated and hand-written paths against the per-matrix oracle."""
+    from morok_amd import synth, uop
+
+    rng = np.random.default_rng(9)
+    a = synth.to_bf16(rng.standard_normal(ashape, dtype=np.float32))
+    w = synth.to_bf16(rng.standard_normal(wshape, dtype=np.float32))
+    c = T.Tensor.from_numpy(a, uop.BF16).matmul(T.Tensor.from_numpy(w, uop.BF16))
+    got = synth.from_bf16(c.to_numpy())
+    M, K, N = ashape[-2], ashape[-1], wshape[-1]
+    a2 = a.reshape(-1, M, K)
+    w2 = w.reshape(-1, K, N) if len(wshape) > 2 else np.broadcast_to(w, (a2.shape[0], K, N))
+    ref = np.stack([synth.from_bf16(oracle.gemm_bf16(np.ascontiguousarray(a2[i]), np.ascontiguousarray(w2[i])))
+                    for i in range(a2.shape[0])]).reshape(got.shape)
+    assert got.shape == tuple(ashape[:-1]) + (N,)
+    assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
+    if fusion:
+        names = c.kernels()
+        assert len(names) == 1 and names[0].startswith("gemm_bf16")
+        assert names[0].endswith("_x%d" % a2.shape[0]) == (len(wshape) > 2)
+
+
 # ---------------------------------------------------------------- softmax
 @pytest.mark.parametrize("shape", [(4, 8), (3, 1000), (2, 5, 257)])
 def test_softmax(T, fusion, oracle, shape):
