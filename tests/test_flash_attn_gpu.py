@@ -78,6 +78,29 @@ def test_flash_special_cases(dev):
     assert np.array_equal(o, want)
 
 
+@pytest.mark.parametrize("trend", ["rising", "falling", "spiky"])
+@pytest.mark.parametrize("causal", [True, False])
+def test_flash_score_ranges(dev, oracle, trend, causal):
+    """Scores far outside the comfortable range: maxima that keep growing along the keys force
+    a rescale of the accumulators at every tile, falling ones none after the first, isolated
+    spikes of +-200 exercise the reference-point logic in both directions."""
+    B, H, S = 1, 2, 512
+    q, k, v = _inputs(B, H, S, S, seed=21)
+    qf, kf = synth.from_bf16(q).copy(), synth.from_bf16(k).copy()
+    qf[..., 0] = 1.0
+    j = np.arange(S, dtype=np.float32)
+    if trend == "rising":
+        kf[..., 0] = 0.4 * j              # +25.6 per 64-key tile
+    elif trend == "falling":
+        kf[..., 0] = -0.4 * j
+    else:
+        kf[..., 0] = 0.0
+        kf[:, :, 70::97, 0] = 200.0
+        kf[:, :, 33::131, 0] = -200.0
+    q2, k2 = synth.to_bf16(qf), synth.to_bf16(kf)
+    _check(_attn(dev, q2, k2, v, 1.0, causal), oracle.sdpa_bf16(q2, k2, v, 1.0, causal=causal))
+
+
 def test_flash_program_path_and_errors(dev, oracle):
     q, k, v = _inputs(1, 2, 192, 192, seed=24)
     _check(_attn(dev, q, k, v, SCALE, True, via_program=True), oracle.sdpa_bf16(q, k, v, SCALE, causal=True))
