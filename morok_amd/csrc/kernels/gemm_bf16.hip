@@ -74,9 +74,16 @@ __device__ __forceinline__ void tile_of_block(int bid, int tiles_m, int tiles_n,
     *tn = in / gm;
 }
 
-__global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
-                                                         __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
-                                                         int tiles_n) {
+// Sixteen zero bytes in device memory: where the copies of a partial last K step point the
+// lanes whose k lies beyond K.
+__device__ __attribute__((aligned(16))) const unsigned g_zero16[4] = {0u, 0u, 0u, 0u};
+
+// kRaggedK: K is not a multiple of 64 (but of 8).  The copies of the last, partial K step use
+// per-lane 64-bit addresses so that chunks beyond K can be redirected to g_zero16: zero
+// operands on both sides contribute nothing.  Every other step is copied as in the full case.
+template <bool kRaggedK>
+__device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                  __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n) {
     // A stage: 256 rows x 128 B, 16 B chunks XOR-swizzled by ((row >> 1) & 7);
     // B stage: 64 k-rows x 512 B, 32 B granules XOR-swizzled by (k & 3).
     __shared__ __attribute__((aligned(1024))) char smem[kSmem];
@@ -133,10 +140,27 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
                      : "s"(lds_addr), "v"(voff), "s"(sbase)
                      : "m0");
     };
+    auto dma_from = [&](unsigned lds_addr, const char* addr) {  // per-lane 64-bit source address
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(addr) : "m0");
+    };
+    const int KT = (K + kBK - 1) / kBK;
+    const int k_last = K - (KT - 1) * kBK;  // depth of the last K step: 64, or 8..56 when ragged
+    const char* zero16 = reinterpret_cast<const char*>(g_zero16);
     auto dma_a = [&](int q, int kt, int stage) {
-        dma(lds_a + stage * kAStage + q * 1024, a_voff[q], a_tile + (size_t)kt * kBK * 2);
+        if (kRaggedK && kt == KT - 1) {
+            const int chunk = (lane & 7) ^ ((q & 1) * 4 + (lane >> 4));  // logical 8-deep k chunk of this lane
+            dma_from(lds_a + stage * kAStage + q * 1024,
+                     chunk * 8 < k_last ? a_tile + (size_t)kt * kBK * 2 + a_voff[q] : zero16);
+        } else {
+            dma(lds_a + stage * kAStage + q * 1024, a_voff[q], a_tile + (size_t)kt * kBK * 2);
+        }
     };
     auto dma_b = [&](int q, int kt, int stage) {
+        if (kRaggedK && kt == KT - 1) {
+            dma_from(lds_b + stage * kBStageSw + q * 1024,
+                     wave * 16 + q * 2 + b_r < k_last ? b_tile + ((size_t)kt * kBK + q * 2) * N * 2 + b_voff[q & 1] : zero16);
+            return;
+        }
         dma(lds_b + stage * kBStageSw + q * 1024, b_voff[q & 1], b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
     };
 
@@ -165,7 +189,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
     auto full_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-    const int KT = K / kBK;
 #pragma unroll
     for (int q = 0; q < 8; q++) dma_a(q, 0, 0);
 #pragma unroll
@@ -281,6 +304,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     }
 }
 
+__global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                         __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
+                                                         int tiles_n) {
+    gemm_tile256_body<false>(A, B, C, M, N, K, tiles_m, tiles_n);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile256_ragged_k(const __bf16* __restrict__ A,
+                                                                  const __bf16* __restrict__ B, __bf16* __restrict__ C,
+                                                                  int M, int N, int K, int tiles_m, int tiles_n) {
+    gemm_tile256_body<true>(A, B, C, M, N, K, tiles_m, tiles_n);
+}
+
 // Any shape: one wave per 32x32 output tile, operands fetched straight from global memory
 // with bounds checks (zero fill), no LDS.  Correct for every M, N, K; used when the shape
 // does not fit the tiled kernel.
@@ -333,12 +367,16 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     // the tiled kernel addresses a tile's rows with 32-bit byte offsets from the tile origin:
     // 255 rows of A (K elements each) and 49 rows of B (N elements each) must stay below 4 GiB
     const bool offsets_fit = K <= (1L << 23) && N <= (1L << 25);
-    // any M; N in whole 16-byte chunks; K in whole 64-deep steps (a partial step would need zero
-    // fill, which a direct-to-LDS copy cannot do)
-    if (variant != 2 && aligned && offsets_fit && K > 0 && N % 8 == 0 && K % kBK == 0) {
+    // any M; N and K in whole 16-byte chunks
+    if (variant != 2 && aligned && offsets_fit && K > 0 && N % 8 == 0 && K % 8 == 0) {
         const int tm = (int)((M + kBM - 1) / kBM), tn = (int)((N + kBN - 1) / kBN);
-        gemm_bf16_tile256<<<dim3((unsigned)(tm * tn), (unsigned)batch), 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
+        const dim3 grid((unsigned)(tm * tn), (unsigned)batch);
+        if (K % kBK == 0)
+            gemm_bf16_tile256<<<grid, 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
                                                   static_cast<__bf16*>(C), (int)M, (int)N, (int)K, tm, tn);
+        else
+            gemm_bf16_tile256_ragged_k<<<grid, 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
+                                                           static_cast<__bf16*>(C), (int)M, (int)N, (int)K, tm, tn);
     } else {
         const long tm = (M + 31) / 32, tn = (N + 31) / 32;
         const long total = tm * tn;

@@ -59,6 +59,38 @@ def test_gemm_tiled_kernel_ragged_edges(dev, oracle, shape):
     assert np.array_equal(got, _gemm(dev, a, b, variant=2))
 
 
+# K in whole 16-byte chunks but not in whole 64-deep steps: the last step's out-of-range chunks
+# are copied from a block of zeros
+@pytest.mark.parametrize("shape", [(256, 256, 8), (256, 256, 72), (100, 264, 200), (512, 512, 1000), (300, 40, 136),
+                                   (256, 256, 56), (64, 128, 120)])
+def test_gemm_tiled_kernel_ragged_k(dev, oracle, shape):
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 3, 8)
+    b = synth.normal_bf16((K, N), 3, 9)
+    got = _gemm(dev, a, b)
+    _check(got, oracle.gemm_bf16(a, b), K)
+    assert np.array_equal(got, _gemm(dev, a, b, variant=2))
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 72), (256, 256, 64), (300, 264, 128), (100, 8, 200), (255, 1000, 8)])
+def test_gemm_does_not_read_past_the_operands(dev, oracle, shape):
+    """Edge tiles and the partial last K step must not read beyond A and B: NaNs placed right
+    behind them in the same allocations do not reach the result (a stray operand would, even
+    against a zero: NaN * 0 = NaN)."""
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 3, 10)
+    b = synth.normal_bf16((K, N), 3, 11)
+    nan = np.full(8192, 0x7FC0, np.uint16)
+    ba = morok_amd.Buffer.from_numpy(np.concatenate([a.reshape(-1), nan]), dev.device_id)
+    bb = morok_amd.Buffer.from_numpy(np.concatenate([b.reshape(-1), nan]), dev.device_id)
+    bc = dev.buffer(M * N * 2 + 4096)
+    bc.copyin(np.full(M * N + 2048, 0x7FC0, np.uint16))
+    ops.gemm_bf16(ba, bb, bc, M, N, K, dev.device_id)
+    out = bc.copyout(np.uint16)
+    _check(out[: M * N].reshape(M, N), oracle.gemm_bf16(a, b), K)
+    assert np.all(out[M * N:] == 0x7FC0)   # and nothing is written behind C
+
+
 @pytest.mark.parametrize("shape", [(1, 1, 1), (32, 32, 16), (33, 65, 17), (100, 200, 300), (5, 7, 1000),
                                    (255, 257, 63), (64, 64, 0)])
 def test_gemm_generic_kernel_parity(dev, oracle, shape):
