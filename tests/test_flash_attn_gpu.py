@@ -101,6 +101,22 @@ def test_flash_score_ranges(dev, oracle, trend, causal):
     _check(_attn(dev, q2, k2, v, 1.0, causal), oracle.sdpa_bf16(q2, k2, v, 1.0, causal=causal))
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 100, 100), (1, 1, 129, 257), (2, 1, 64, 33), (1, 1, 1, 1)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_flash_does_not_touch_neighbours(dev, oracle, shape, causal):
+    """Ragged last tiles: NaNs right behind Q, K and V in their allocations do not reach O, and
+    nothing is written behind O."""
+    B, H, Sq, Sk = shape
+    q, k, v = _inputs(B, H, Sq, Sk, seed=23)
+    nan = np.full(4096, 0x7FC0, np.uint16)
+    bq, bk, bv = (morok_amd.Buffer.from_numpy(np.concatenate([t.reshape(-1), nan]), dev.device_id) for t in (q, k, v))
+    bo = morok_amd.Buffer.from_numpy(np.full(q.size + 4096, 0x7FC0, np.uint16), dev.device_id)
+    ops.flash_attn_fwd_bf16(bq, bk, bv, bo, B, H, Sq, Sk, D, SCALE, causal, dev.device_id)
+    out = bo.copyout(np.uint16)
+    _check(out[: q.size].reshape(q.shape), oracle.sdpa_bf16(q, k, v, SCALE, causal=causal))
+    assert np.all(out[q.size:] == 0x7FC0)
+
+
 def test_flash_program_path_and_errors(dev, oracle):
     q, k, v = _inputs(1, 2, 192, 192, seed=24)
     _check(_attn(dev, q, k, v, SCALE, True, via_program=True), oracle.sdpa_bf16(q, k, v, SCALE, causal=True))

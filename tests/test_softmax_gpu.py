@@ -76,6 +76,20 @@ def test_softmax_rows_misaligned_differently_in_x_and_y(dev, oracle):
     _check(y, _softmax_f64(x), rtol=1e-5)
 
 
+@pytest.mark.parametrize("shape", [(3, 8191), (5, 1001), (2, 70001), (4, 4096), (7, 33)])
+def test_softmax_does_not_touch_neighbours(dev, oracle, shape):
+    """NaNs right behind x in its allocation do not reach y, and nothing is written behind y."""
+    rows, cols = shape
+    x = synth.normal(shape, 2, 3, sigma=2.0)
+    pad = np.full(1024, np.nan, np.float32)
+    bx = morok_amd.Buffer.from_numpy(np.concatenate([x.reshape(-1), pad]), dev.device_id)
+    by = morok_amd.Buffer.from_numpy(np.full(rows * cols + 1024, np.nan, np.float32), dev.device_id)
+    ops.softmax_f32(bx, by, rows, cols, dev.device_id)
+    out = by.copyout(np.float32)
+    _check(out[: rows * cols].reshape(shape), oracle.softmax_f32(x), rtol=1e-4)
+    assert np.all(np.isnan(out[rows * cols:]))
+
+
 def test_softmax_config_slice_of_full_shape(dev, oracle):
     # rows of the benchmark shape [8192 x 8192], N(0, 2): a slice the oracle finishes quickly
     x = synth.normal((256, 8192), 2, 0, sigma=2.0)
