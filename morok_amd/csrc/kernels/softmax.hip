@@ -195,7 +195,7 @@ namespace mrk {
 int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long cols, int variant) {
     using namespace mrk::dev;
     if (rows <= 0 || cols <= 0) return 0;
-    if (rows > 0x7fffffffL) return -1;
+    if (rows > 0x7fffffffL || cols > 0x7fffffffL) return (int)hipErrorInvalidValue;  // grid extent, 32-bit row split
     hipStream_t s = static_cast<hipStream_t>(stream);
     (void)hipGetLastError();  // launch status below must be this launch's own
     const float* xi = static_cast<const float*>(x);
