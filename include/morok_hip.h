@@ -232,6 +232,12 @@ int mrk_hip_plan_build(mrk_plan* plan);
 /* ExecutionPlan::execute (execution_plan.rs:168-181): launches every kernel in order on the
  * device stream; no synchronisation between kernels. */
 int mrk_hip_plan_execute(mrk_plan* plan);
+/* The launches of mrk_hip_plan_execute replayed as one HIP graph: the first call records them
+ * on the device's stream and instantiates the graph, later calls are one hipGraphLaunch.  No
+ * counterpart in the reference (its CPU kernels are plain function calls); for plans of many
+ * short kernels, where per-launch submission cost dominates.  The plan must be rebuilt-free:
+ * mrk_hip_plan_execute_with_vars or adding kernels drops the recorded graph. */
+int mrk_hip_plan_execute_graph(mrk_plan* plan);
 /* ExecutionPlan::execute_profiled (execution_plan.rs:200-221): per-kernel elapsed time in ms,
  * measured with HIP events (the reference uses Instant around blocking CPU calls). */
 int mrk_hip_plan_execute_profiled(mrk_plan* plan, double* elapsed_ms, size_t cap, size_t* count);

@@ -103,6 +103,7 @@ _SIGS = {
     "mrk_hip_plan_add_kernel": (C.c_int, [C.c_void_p, C.c_void_p, c_size_p, C.c_size_t, c_i64_p, C.c_size_t]),
     "mrk_hip_plan_build": (C.c_int, [C.c_void_p]),
     "mrk_hip_plan_execute": (C.c_int, [C.c_void_p]),
+    "mrk_hip_plan_execute_graph": (C.c_int, [C.c_void_p]),
     "mrk_hip_plan_execute_profiled": (C.c_int, [C.c_void_p, C.POINTER(C.c_double), C.c_size_t, c_size_p]),
     "mrk_hip_plan_execute_with_vars": (C.c_int, [C.c_void_p, C.POINTER(C.c_char_p), c_i64_p, C.c_size_t]),
     "mrk_hip_plan_kernel_count": (C.c_size_t, [C.c_void_p]),

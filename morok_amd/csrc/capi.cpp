@@ -455,6 +455,10 @@ int mrk_hip_plan_execute(mrk_plan* plan) {
     MRK_NONNULL(plan);
     return plan->p->execute();
 }
+int mrk_hip_plan_execute_graph(mrk_plan* plan) {
+    MRK_NONNULL(plan);
+    return plan->p->execute_graph();
+}
 int mrk_hip_plan_execute_profiled(mrk_plan* plan, double* elapsed_ms, size_t cap, size_t* count) {
     MRK_NONNULL(plan);
     std::vector<KernelProfile> prof;

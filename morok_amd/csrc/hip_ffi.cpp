@@ -74,6 +74,27 @@ int module_launch(Function f, const unsigned grid[3], const unsigned block[3], u
                                  block[2], shared_bytes, static_cast<hipStream_t>(s), kernel_params, nullptr);
 }
 
+int stream_begin_capture(Stream s) {
+    return static_cast<int>(hipStreamBeginCapture(static_cast<hipStream_t>(s), hipStreamCaptureModeThreadLocal));
+}
+int stream_end_capture(Stream s, Graph* out) {
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(static_cast<hipStream_t>(s), &g);
+    *out = g;
+    return static_cast<int>(e);
+}
+int graph_instantiate(GraphExec* out, Graph g) {
+    hipGraphExec_t x = nullptr;
+    hipError_t e = hipGraphInstantiate(&x, static_cast<hipGraph_t>(g), nullptr, nullptr, 0);
+    *out = x;
+    return static_cast<int>(e);
+}
+int graph_launch(GraphExec e, Stream s) {
+    return static_cast<int>(hipGraphLaunch(static_cast<hipGraphExec_t>(e), static_cast<hipStream_t>(s)));
+}
+int graph_exec_destroy(GraphExec e) { return static_cast<int>(hipGraphExecDestroy(static_cast<hipGraphExec_t>(e))); }
+int graph_destroy(Graph g) { return static_cast<int>(hipGraphDestroy(static_cast<hipGraph_t>(g))); }
+
 const char* error_name(int code) { return hipGetErrorName(static_cast<hipError_t>(code)); }
 void clear_last_error() { (void)hipGetLastError(); }
 

@@ -20,6 +20,8 @@ using Stream = void*;
 using Event = void*;
 using Module = void*;
 using Function = void*;
+using Graph = void*;
+using GraphExec = void*;
 
 int device_count(int* out);
 int set_device(int device_id);
@@ -55,6 +57,15 @@ int module_get_function(Function* out, Module m, const char* name);
 // kernel_params: array of pointers to each argument (hipModuleLaunchKernel convention).
 int module_launch(Function f, const unsigned grid[3], const unsigned block[3], unsigned shared_bytes, Stream s,
                   void** kernel_params);
+
+// Stream capture into a graph (thread-local capture mode: other threads' calls are unaffected)
+// and replay.  Only kernel launches are ever recorded by this library.
+int stream_begin_capture(Stream s);
+int stream_end_capture(Stream s, Graph* out);
+int graph_instantiate(GraphExec* out, Graph g);
+int graph_launch(GraphExec e, Stream s);
+int graph_exec_destroy(GraphExec e);
+int graph_destroy(Graph g);
 
 const char* error_name(int code);
 // Clears the sticky per-thread error state of the runtime after a failed call.

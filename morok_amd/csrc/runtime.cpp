@@ -108,6 +108,7 @@ int ExecutionPlan::add_kernel(std::shared_ptr<CachedKernel> kernel, const std::v
     pk.vals = vals;
     kernels_.push_back(std::move(pk));
     built_ = false;
+    drop_graph();
     return kOk;
 }
 
@@ -177,8 +178,7 @@ int ExecutionPlan::build() {
     return kOk;
 }
 
-int ExecutionPlan::execute() {
-    if (!built_) MRK_TRY(build());
+int ExecutionPlan::launch_all() {
     for (auto& pk : kernels_) {
         const CachedKernel& ck = *pk.kernel;
         int rc = ck.program->execute(pk.buffer_ptrs.data(), pk.buffer_ptrs.size(), pk.vals.data(), pk.vals.size(),
@@ -189,6 +189,49 @@ int ExecutionPlan::execute() {
             return failf(static_cast<Status>(rc), "Kernel %llu failed: %s", (unsigned long long)pk.id, inner.c_str());
         }
     }
+    return kOk;
+}
+
+int ExecutionPlan::execute() {
+    if (!built_) MRK_TRY(build());
+    return launch_all();
+}
+
+ExecutionPlan::~ExecutionPlan() { drop_graph(); }
+
+void ExecutionPlan::drop_graph() {
+    if (graph_exec_) {
+        (void)ffi::set_device(device_id_);
+        (void)ffi::graph_exec_destroy(graph_exec_);
+        graph_exec_ = nullptr;
+    }
+}
+
+int ExecutionPlan::execute_graph() {
+    if (!built_) MRK_TRY(build());
+    if (kernels_.empty()) return kOk;
+    std::shared_ptr<Allocator> alloc;
+    MRK_TRY(AllocatorRegistry::global().get(device_id_, &alloc));
+    ffi::Stream stream = alloc->stream();
+    MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
+    if (!graph_exec_) {
+        MRK_HIP(ffi::stream_begin_capture(stream), "hipStreamBeginCapture");
+        int rc = launch_all();
+        const std::string launch_error = rc != kOk ? last_error() : std::string();
+        ffi::Graph g = nullptr;
+        int ec = ffi::stream_end_capture(stream, &g);  // always: leaves the stream usable again
+        if (rc != kOk) {
+            if (g) (void)ffi::graph_destroy(g);
+            ffi::clear_last_error();
+            return fail(static_cast<Status>(rc), launch_error);
+        }
+        MRK_HIP(ec, "hipStreamEndCapture");
+        ec = ffi::graph_instantiate(&graph_exec_, g);
+        (void)ffi::graph_destroy(g);
+        if (ec != 0) graph_exec_ = nullptr;
+        MRK_HIP(ec, "hipGraphInstantiate");
+    }
+    MRK_HIP(ffi::graph_launch(graph_exec_, stream), "hipGraphLaunch");
     return kOk;
 }
 
@@ -236,6 +279,7 @@ int ExecutionPlan::execute_with_vars(const std::vector<std::pair<std::string, in
             for (const auto& kv : var_vals)
                 if (kv.first == names[i]) pk.vals[i] = kv.second;
     }
+    drop_graph();  // a recorded graph holds the old values
     return execute();
 }
 

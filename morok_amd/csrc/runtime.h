@@ -78,6 +78,9 @@ struct MemoryPlanStats {
 class ExecutionPlan {
   public:
     explicit ExecutionPlan(int device_id) : device_id_(device_id) {}
+    ~ExecutionPlan();
+    ExecutionPlan(const ExecutionPlan&) = delete;
+    ExecutionPlan& operator=(const ExecutionPlan&) = delete;
     // Builder (execution_plan.rs:330-411): the plan owns clones of all buffers, which keeps
     // the precomputed pointers valid.
     size_t add_buffer(std::shared_ptr<Buffer> b);
@@ -95,6 +98,13 @@ class ExecutionPlan {
 
     // execution_plan.rs:168-181: tight loop, no allocation, no per-launch sync.
     int execute();
+    // The same launches replayed as one HIP graph: the first call records execute() on the
+    // device's stream (kernel launches only) and instantiates the graph, later calls are a
+    // single hipGraphLaunch.  For launch-bound plans (many short kernels); no counterpart in
+    // the reference, whose CPU kernels are plain function calls.  Rebinding variables or
+    // adding kernels drops the recorded graph.
+    int execute_graph();
+    bool has_graph() const { return graph_exec_ != nullptr; }
     // execution_plan.rs:200-221
     int execute_profiled(std::vector<KernelProfile>* out);
     // execution_plan.rs:239-250: rebinding by name, kernels are not recompiled.
@@ -109,6 +119,9 @@ class ExecutionPlan {
 
   private:
     int plan_memory();
+    int launch_all();
+    void drop_graph();
+    ffi::GraphExec graph_exec_ = nullptr;
     int device_id_;
     bool built_ = false;
     bool plan_memory_ = false, memory_planned_ = false;

@@ -460,6 +460,10 @@ class ExecutionPlan:
     def execute(self):
         check(lib.mrk_hip_plan_execute(self._h))
 
+    def execute_graph(self):
+        """The same launches replayed as one HIP graph (recorded on the first call)."""
+        check(lib.mrk_hip_plan_execute_graph(self._h))
+
     def execute_profiled(self):
         n = lib.mrk_hip_plan_kernel_count(self._h)
         ms = (C.c_double * max(n, 1))()

@@ -31,6 +31,17 @@ struct FakeEvent {
     bool recorded = false;
 };
 constexpr int kOutOfMemory = 2, kInvalidValue = 1, kNotFound = 500, kInvalidDevice = 101, kInvalidImage = 200;
+// stream capture: launches made while capturing are recorded, not run; a graph launch runs them
+struct FakeGraph {
+    size_t launches = 0;
+};
+bool g_capturing = false;
+size_t g_captured = 0, g_graph_launches = 0, g_graphs_alive = 0;
+// one launch seen by the stand-in: counted as run, or as recorded while a capture is open (g_mu held)
+void count_launch() {
+    if (g_capturing) g_captured++;
+    else g_launches++;
+}
 }  // namespace
 
 extern "C" {
@@ -38,8 +49,11 @@ void mrk_shim_reset() {
     std::lock_guard<std::mutex> l(g_mu);
     g_limit = ~size_t(0);
     g_alloc_calls = g_free_calls = g_launches = g_syncs = 0;
+    g_graph_launches = 0;
     g_last_kernel.clear();
 }
+size_t mrk_shim_graph_launches() { return g_graph_launches; }
+size_t mrk_shim_graphs_alive() { return g_graphs_alive; }
 void mrk_shim_set_memory_limit(size_t bytes) { g_limit = bytes; }
 void mrk_shim_set_device_count(int n) { g_devices = n; }
 size_t mrk_shim_bytes_in_use() { return g_in_use; }
@@ -55,7 +69,7 @@ void mrk_shim_last_dims(unsigned* grid, unsigned* block) {
 // called by the recording launchers of fake_kernels.cpp
 void mrk_shim_note_launch(const char* name) {
     std::lock_guard<std::mutex> l(g_mu);
-    g_launches++;
+    count_launch();
     g_last_kernel = name;
 }
 }
@@ -191,7 +205,45 @@ int module_launch(Function f, const unsigned grid[3], const unsigned block[3], u
     std::memcpy(g_last_grid, grid, sizeof g_last_grid);
     std::memcpy(g_last_block, block, sizeof g_last_block);
     g_last_kernel = static_cast<FakeFunction*>(f)->name;
-    g_launches++;
+    count_launch();
+    return 0;
+}
+
+int stream_begin_capture(Stream) {
+    std::lock_guard<std::mutex> l(g_mu);
+    if (g_capturing) return kInvalidValue;
+    g_capturing = true;
+    g_captured = 0;
+    return 0;
+}
+int stream_end_capture(Stream, Graph* out) {
+    std::lock_guard<std::mutex> l(g_mu);
+    *out = nullptr;
+    if (!g_capturing) return kInvalidValue;
+    g_capturing = false;
+    *out = new FakeGraph{g_captured};
+    return 0;
+}
+int graph_instantiate(GraphExec* out, Graph g) {
+    std::lock_guard<std::mutex> l(g_mu);
+    *out = new FakeGraph{static_cast<FakeGraph*>(g)->launches};
+    g_graphs_alive++;
+    return 0;
+}
+int graph_launch(GraphExec e, Stream) {
+    std::lock_guard<std::mutex> l(g_mu);
+    g_launches += static_cast<FakeGraph*>(e)->launches;
+    g_graph_launches++;
+    return 0;
+}
+int graph_exec_destroy(GraphExec e) {
+    std::lock_guard<std::mutex> l(g_mu);
+    delete static_cast<FakeGraph*>(e);
+    g_graphs_alive--;
+    return 0;
+}
+int graph_destroy(Graph g) {
+    delete static_cast<FakeGraph*>(g);
     return 0;
 }
 

@@ -31,6 +31,8 @@ def load():
         ("mrk_shim_alloc_calls", C.c_size_t, []),
         ("mrk_shim_free_calls", C.c_size_t, []),
         ("mrk_shim_launches", C.c_size_t, []),
+        ("mrk_shim_graph_launches", C.c_size_t, []),
+        ("mrk_shim_graphs_alive", C.c_size_t, []),
         ("mrk_shim_syncs", C.c_size_t, []),
         ("mrk_shim_last_kernel", C.c_char_p, []),
         ("mrk_shim_last_dims", None, [C.POINTER(C.c_uint * 3), C.POINTER(C.c_uint * 3)]),

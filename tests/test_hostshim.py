@@ -301,6 +301,35 @@ def test_decoder_block_lowering(T, shim, fused, gemms):
     print(names)
 
 
+def test_plan_graph_replay_records_once(T, shim):
+    """execute_graph records the plan's launches once (nothing runs while recording), replays
+    them with one graph launch per call, and drops the recording when variables are rebound or
+    the plan goes away."""
+    x = T.Tensor.from_numpy(np.arange(64, dtype=np.float32).reshape(8, 8))
+    y = x.try_add(x).sum([1]).try_exp()      # a reduce and an elementwise kernel
+    plan = y.prepare()
+    n = plan.kernel_count
+    assert n >= 2
+    base = shim.mrk_shim_launches()
+    plan.execute()
+    assert shim.mrk_shim_launches() - base == n
+    plan.execute_graph()                      # records n launches, then one graph launch runs them
+    assert shim.mrk_shim_launches() - base == 2 * n and shim.mrk_shim_graph_launches() == 1
+    assert shim.mrk_shim_graphs_alive() == 1
+    plan.execute_graph()
+    plan.execute_graph()
+    assert shim.mrk_shim_launches() - base == 4 * n and shim.mrk_shim_graph_launches() == 3
+    plan.execute_with_vars({})                # rebinding drops the recording
+    assert shim.mrk_shim_graphs_alive() == 0
+    plan.execute_graph()
+    assert shim.mrk_shim_graphs_alive() == 1
+    del plan
+    import gc
+
+    gc.collect()
+    assert shim.mrk_shim_graphs_alive() == 0
+
+
 # ------------------------------------------------------------------ beam-search support
 def test_beam_cache_roundtrip_and_ignore(shim, tmp_path, monkeypatch):
     from morok_amd import sched

@@ -240,3 +240,49 @@ def test_concurrent_realize_from_threads(dev, oracle):
     for i, (got, a, b) in results.items():
         ref = oracle.softmax_f32(oracle.matmul_f32(a, b) + np.float32(i))
         np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-6)
+
+
+def test_plan_graph_replay_matches_eager(dev, oracle):
+    """ExecutionPlan::execute_graph: the recorded graph (kernel launches only: generated
+    kernels, GEMMs, flash attention) is replayed several times with the program's own eager work
+    and synchronisations in between, on fresh inputs each time; every replay must give exactly
+    what the eager launches give."""
+    from morok_amd import decoder, tensor
+
+    cfg = dict(batch=2, seq=128, hidden=256, heads=2, ffn=512, vocab=1000)
+    T = cfg["batch"] * cfg["seq"]
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], cfg["vocab"], seed=3)
+    blk = decoder.DecoderBlock(w, cfg["batch"], cfg["seq"], cfg["hidden"], cfg["heads"], cfg["ffn"])
+    tok_host = synth.randint((T,), 3, 1, cfg["vocab"]).astype(np.int32)
+    tok = tensor.Tensor.from_numpy(tok_host)
+    out = blk.forward(tok)
+    plan = out.prepare()
+    tok_buf = tok.buffer()
+
+    def result():
+        dev.synchronize()
+        return out.buffer().copyout(np.uint16, (T, cfg["hidden"])).copy()
+
+    plan.execute()
+    eager = result()
+    ref = oracle.decoder_block_bf16(tok_host, w, blk.cos_host, blk.sin_host, cfg["batch"], cfg["seq"], cfg["hidden"],
+                                    cfg["heads"], cfg["ffn"], 1e-6)
+    err = np.abs(synth.from_bf16(eager) - synth.from_bf16(ref)).max() / np.abs(synth.from_bf16(ref)).max()
+    assert err <= 2e-2
+    for i in range(4):
+        # new tokens, eager result first, then the graph on the same inputs
+        toks = synth.randint((T,), 30 + i, 1, cfg["vocab"]).astype(np.int32)
+        tok_buf.copyin(toks)
+        plan.execute()
+        want = result()
+        out.buffer().copyin(np.zeros(T * cfg["hidden"], np.uint16))   # the replay must rewrite it
+        plan.execute_graph()
+        got = result()
+        assert np.array_equal(got, want), i
+        # unrelated eager work between the replays
+        x = synth.normal((64, 512), 5, i, sigma=1.0)
+        bx = morok_amd.Buffer.from_numpy(x, dev.device_id)
+        by = dev.buffer(x.nbytes)
+        ops.softmax_f32(bx, by, 64, 512, dev.device_id)
+        dev.synchronize()
+    assert not np.array_equal(want, eager)    # the inputs did change between rounds
