@@ -178,12 +178,15 @@ int ExecutionPlan::build() {
     return kOk;
 }
 
-int ExecutionPlan::launch_all() {
+int ExecutionPlan::launch_all(ffi::Stream on) {
     for (auto& pk : kernels_) {
         const CachedKernel& ck = *pk.kernel;
-        int rc = ck.program->execute(pk.buffer_ptrs.data(), pk.buffer_ptrs.size(), pk.vals.data(), pk.vals.size(),
-                                     ck.has_sizes ? ck.global_size.data() : nullptr,
-                                     ck.has_sizes ? ck.local_size.data() : nullptr);
+        const size_t* g = ck.has_sizes ? ck.global_size.data() : nullptr;
+        const size_t* l = ck.has_sizes ? ck.local_size.data() : nullptr;
+        int rc = on ? ck.program->execute_on(on, pk.buffer_ptrs.data(), pk.buffer_ptrs.size(), pk.vals.data(),
+                                             pk.vals.size(), g, l)
+                    : ck.program->execute(pk.buffer_ptrs.data(), pk.buffer_ptrs.size(), pk.vals.data(), pk.vals.size(),
+                                          g, l);
         if (rc != kOk) {
             std::string inner = last_error();
             return failf(static_cast<Status>(rc), "Kernel %llu failed: %s", (unsigned long long)pk.id, inner.c_str());
@@ -194,7 +197,7 @@ int ExecutionPlan::launch_all() {
 
 int ExecutionPlan::execute() {
     if (!built_) MRK_TRY(build());
-    return launch_all();
+    return launch_all(nullptr);
 }
 
 ExecutionPlan::~ExecutionPlan() { drop_graph(); }
@@ -215,11 +218,20 @@ int ExecutionPlan::execute_graph() {
     ffi::Stream stream = alloc->stream();
     MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
     if (!graph_exec_) {
-        MRK_HIP(ffi::stream_begin_capture(stream), "hipStreamBeginCapture");
-        int rc = launch_all();
+        // Recorded on a stream of its own: the device's stream is shared by every thread, and a
+        // launch another thread queues there while a capture is open would end up in the graph.
+        ffi::Stream cap = nullptr;
+        MRK_HIP(ffi::stream_create(&cap), "hipStreamCreate");
+        int ec = ffi::stream_begin_capture(cap);
+        if (ec != 0) {
+            (void)ffi::stream_destroy(cap);
+            MRK_HIP(ec, "hipStreamBeginCapture");
+        }
+        int rc = launch_all(cap);
         const std::string launch_error = rc != kOk ? last_error() : std::string();
         ffi::Graph g = nullptr;
-        int ec = ffi::stream_end_capture(stream, &g);  // always: leaves the stream usable again
+        ec = ffi::stream_end_capture(cap, &g);  // always: a capture must be closed
+        (void)ffi::stream_destroy(cap);
         if (rc != kOk) {
             if (g) (void)ffi::graph_destroy(g);
             ffi::clear_last_error();

@@ -119,7 +119,7 @@ class ExecutionPlan {
 
   private:
     int plan_memory();
-    int launch_all();
+    int launch_all(ffi::Stream on);  // nullptr: every program's own stream
     void drop_graph();
     ffi::GraphExec graph_exec_ = nullptr;
     int device_id_;

@@ -6,6 +6,7 @@
 #include <chrono>
 #include <cstdlib>
 #include <cstring>
+#include <map>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -35,11 +36,12 @@ constexpr int kOutOfMemory = 2, kInvalidValue = 1, kNotFound = 500, kInvalidDevi
 struct FakeGraph {
     size_t launches = 0;
 };
-bool g_capturing = false;
-size_t g_captured = 0, g_graph_launches = 0, g_graphs_alive = 0;
-// one launch seen by the stand-in: counted as run, or as recorded while a capture is open (g_mu held)
-void count_launch() {
-    if (g_capturing) g_captured++;
+std::map<void*, size_t> g_capturing;  // stream -> launches recorded so far
+size_t g_graph_launches = 0, g_graphs_alive = 0;
+// one launch seen by the stand-in: counted as run, or as recorded while its stream is capturing (g_mu held)
+void count_launch(void* stream) {
+    auto it = g_capturing.find(stream);
+    if (it != g_capturing.end()) it->second++;
     else g_launches++;
 }
 }  // namespace
@@ -67,9 +69,9 @@ void mrk_shim_last_dims(unsigned* grid, unsigned* block) {
     std::memcpy(block, g_last_block, sizeof g_last_block);
 }
 // called by the recording launchers of fake_kernels.cpp
-void mrk_shim_note_launch(const char* name) {
+void mrk_shim_note_launch(void* stream, const char* name) {
     std::lock_guard<std::mutex> l(g_mu);
-    count_launch();
+    count_launch(stream);
     g_last_kernel = name;
 }
 }
@@ -139,12 +141,12 @@ int stream_destroy(Stream s) {
     return 0;
 }
 int stream_synchronize(Stream) {
-    g_syncs++;
+    { std::lock_guard<std::mutex> l(g_mu); g_syncs++; }
     return 0;
 }
 int stream_wait_event(Stream, Event) { return 0; }
 int device_synchronize() {
-    g_syncs++;
+    { std::lock_guard<std::mutex> l(g_mu); g_syncs++; }
     return 0;
 }
 
@@ -197,7 +199,7 @@ int module_get_function(Function* out, Module m, const char* name) {
     *out = new FakeFunction{name};  // lives as long as the process (tests only)
     return 0;
 }
-int module_launch(Function f, const unsigned grid[3], const unsigned block[3], unsigned, Stream, void**) {
+int module_launch(Function f, const unsigned grid[3], const unsigned block[3], unsigned, Stream stream, void**) {
     for (int i = 0; i < 3; i++)
         if (grid[i] == 0 || block[i] == 0) return kInvalidValue;
     if (size_t(block[0]) * block[1] * block[2] > 1024) return kInvalidValue;
@@ -205,23 +207,23 @@ int module_launch(Function f, const unsigned grid[3], const unsigned block[3], u
     std::memcpy(g_last_grid, grid, sizeof g_last_grid);
     std::memcpy(g_last_block, block, sizeof g_last_block);
     g_last_kernel = static_cast<FakeFunction*>(f)->name;
-    count_launch();
+    count_launch(stream);
     return 0;
 }
 
-int stream_begin_capture(Stream) {
+int stream_begin_capture(Stream s) {
     std::lock_guard<std::mutex> l(g_mu);
-    if (g_capturing) return kInvalidValue;
-    g_capturing = true;
-    g_captured = 0;
+    if (g_capturing.count(s)) return kInvalidValue;
+    g_capturing[s] = 0;
     return 0;
 }
-int stream_end_capture(Stream, Graph* out) {
+int stream_end_capture(Stream s, Graph* out) {
     std::lock_guard<std::mutex> l(g_mu);
     *out = nullptr;
-    if (!g_capturing) return kInvalidValue;
-    g_capturing = false;
-    *out = new FakeGraph{g_captured};
+    auto it = g_capturing.find(s);
+    if (it == g_capturing.end()) return kInvalidValue;
+    *out = new FakeGraph{it->second};
+    g_capturing.erase(it);
     return 0;
 }
 int graph_instantiate(GraphExec* out, Graph g) {

@@ -2,31 +2,31 @@
 // (morok_amd/csrc/kernels/kernels.h).  TEST INFRASTRUCTURE ONLY: they compute nothing.
 #include "kernels/kernels.h"
 
-extern "C" void mrk_shim_note_launch(const char* name);
+extern "C" void mrk_shim_note_launch(void* stream, const char* name);
 
 namespace mrk {
-int launch_softmax_f32(void*, const void*, void*, long, long, int) {
-    mrk_shim_note_launch("softmax_f32");
+int launch_softmax_f32(void* stream, const void*, void*, long, long, int) {
+    mrk_shim_note_launch(stream, "softmax_f32");
     return 0;
 }
-int launch_gemm_bf16(void*, const void*, const void*, void*, long, long, long, int, long) {
-    mrk_shim_note_launch("gemm_bf16");
+int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, long, int, long) {
+    mrk_shim_note_launch(stream, "gemm_bf16");
     return 0;
 }
-int launch_flash_fwd_bf16(void*, const void*, const void*, const void*, void*, long, long, long, long, float, int) {
-    mrk_shim_note_launch("flash_fwd_bf16");
+int launch_flash_fwd_bf16(void* stream, const void*, const void*, const void*, void*, long, long, long, long, float, int) {
+    mrk_shim_note_launch(stream, "flash_fwd_bf16");
     return 0;
 }
-int launch_fill(void*, void*, size_t, int, int, unsigned long long, unsigned long long, float, float) {
-    mrk_shim_note_launch("fill");
+int launch_fill(void* stream, void*, size_t, int, int, unsigned long long, unsigned long long, float, float) {
+    mrk_shim_note_launch(stream, "fill");
     return 0;
 }
-int launch_fill_randint(void*, void*, size_t, unsigned long long, unsigned long long, int) {
-    mrk_shim_note_launch("fill_randint");
+int launch_fill_randint(void* stream, void*, size_t, unsigned long long, unsigned long long, int) {
+    mrk_shim_note_launch(stream, "fill_randint");
     return 0;
 }
-int launch_copy(void*, const void*, void*, size_t) {
-    mrk_shim_note_launch("copy");
+int launch_copy(void* stream, const void*, void*, size_t) {
+    mrk_shim_note_launch(stream, "copy");
     return 0;
 }
 }  // namespace mrk
