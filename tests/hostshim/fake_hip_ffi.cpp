@@ -7,6 +7,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <unordered_map>
@@ -196,7 +197,10 @@ int module_get_function(Function* out, Module m, const char* name) {
     std::string needle(name);
     needle.push_back('\0');  // the symbol name as it sits in the string table
     if (mod->image.find(needle) == std::string::npos) return kNotFound;
-    *out = new FakeFunction{name};  // lives as long as the process (tests only)
+    static std::vector<std::unique_ptr<FakeFunction>> functions;  // owned here, freed at process exit
+    std::lock_guard<std::mutex> l(g_mu);
+    functions.emplace_back(new FakeFunction{name});
+    *out = functions.back().get();
     return 0;
 }
 int module_launch(Function f, const unsigned grid[3], const unsigned block[3], unsigned, Stream stream, void**) {
