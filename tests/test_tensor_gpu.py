@@ -392,3 +392,52 @@ def test_split_reduction_values(T):
                                atol=1e-2)
     np.testing.assert_allclose(T.Tensor.from_numpy(z).try_permute([1, 0, 2]).sum([0, 2]).to_numpy(),
                                z.astype(np.float64).sum((1, 2)), rtol=1e-4, atol=1e-2)
+
+
+# ---------------------------------------------------------------- generated kernels stay inside their inputs
+def _guarded(dev, arr):
+    """A tensor over a view that has NaNs right in front of and right behind its data in the
+    same allocation."""
+    import morok_amd
+
+    from morok_amd import uop
+
+    pad = 4096
+    raw = np.full(pad * 2 + arr.nbytes, 0xFF, np.uint8)      # 0xFFFFFFFF = NaN in f32, -1 in int32
+    raw[pad:pad + arr.nbytes] = np.frombuffer(np.ascontiguousarray(arr).tobytes(), np.uint8)
+    base = morok_amd.Buffer.from_numpy(raw, dev.device_id)
+    dt = {np.dtype(np.float32): uop.F32, np.dtype(np.int32): uop.I32}[arr.dtype]
+    return base, base.view(pad, arr.nbytes), dt
+
+
+def test_generated_kernels_do_not_read_past_their_inputs(T, dev):
+    """Movement ops become index arithmetic inside the consuming kernel; edges of shrink, cat,
+    gather (clamped rows, masked out-of-range indices), reductions and odd widths must not pull
+    in what lies next to the data (NaNs here, which would poison sums and selections)."""
+    rng = np.random.default_rng(31)
+    x = rng.standard_normal((37, 53)).astype(np.float32)
+    keep, view, dt = _guarded(dev, x)
+    t = T.Tensor.from_buffer(view, x.shape, dt)
+    # reduce over both axes, odd extents
+    np.testing.assert_allclose(t.sum([1]).to_numpy(), x.sum(1), rtol=1e-5, atol=1e-5)
+    np.testing.assert_allclose(t.sum([0]).to_numpy(), x.sum(0), rtol=1e-5, atol=1e-5)
+    # shrink to the last rows / columns, transpose, cat of the two edges
+    a = t.try_shrink([(30, 37), (40, 53)])
+    b = t.try_shrink([(0, 7), (0, 13)])
+    got = T.Tensor.cat([a, b], 1).try_transpose(0, 1).contiguous().to_numpy()
+    np.testing.assert_array_equal(got, np.concatenate([x[30:37, 40:53], x[0:7, 0:13]], 1).T)
+    # wide rows (vector loads) with a tail
+    y = rng.standard_normal((9, 1027)).astype(np.float32)
+    keep2, view2, _ = _guarded(dev, y)
+    ty = T.Tensor.from_buffer(view2, y.shape, dt)
+    np.testing.assert_allclose(ty.try_mul(ty).sum([1]).to_numpy(), (y * y).sum(1), rtol=1e-5)
+    np.testing.assert_allclose(ty.softmax(-1).to_numpy(), np.exp(y - y.max(1, keepdims=True)) /
+                               np.exp(y - y.max(1, keepdims=True)).sum(1, keepdims=True), rtol=1e-5, atol=1e-9)
+    # gather: first row, last row and out-of-range indices (which select nothing)
+    w = rng.standard_normal((11, 24)).astype(np.float32)
+    keep3, view3, _ = _guarded(dev, w)
+    tw = T.Tensor.from_buffer(view3, w.shape, dt)
+    idx = np.array([0, 10, 11, -1, 5, 1000], np.int32)
+    want = np.where(((idx >= 0) & (idx < 11))[:, None], w[np.clip(idx, 0, 10)], 0.0)
+    np.testing.assert_array_equal(tw.embedding(T.Tensor.from_numpy(idx)).to_numpy(), want)
+    del keep, keep2, keep3
