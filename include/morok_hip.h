@@ -374,7 +374,8 @@ int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t r
  * (schedule/src/optimizer/tc.rs:36-94).  Any shape; shapes with M,N % 256 == 0 and
  * K % 64 == 0 take the LDS-tiled kernel. */
 int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k);
-/* Same with an explicit kernel variant (0 choose by shape, 2 any-shape kernel); tuning/tests. */
+/* Same with an explicit kernel variant (0 choose by shape, 2 any-shape kernel, 3 / 4 tiled kernel
+ * with the 256-row / 128-row tile); tuning/tests. */
 int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
                                int variant);
 

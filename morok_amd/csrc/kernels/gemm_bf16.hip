@@ -47,13 +47,9 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
 constexpr int kBM = 256, kBN = 256, kBK = 64;
-constexpr int kAStage = kBM * kBK * 2;         // 32768 B, row pitch 128 B, chunk-swizzled
-constexpr int kBStageSw = kBK * kBN * 2;       // 32768 B, row pitch 512 B, granule-swizzled
-constexpr int kCPitch = 128 * 2 + 16;          // epilogue staging pitch per wave
-constexpr int kCWave = 128 * kCPitch;          // 34816 B
-constexpr int kSmemMain = 2 * kAStage + 3 * kBStageSw;  // 163840 = all 160 KB of the LDS
-constexpr int kSmemEpi = 4 * kCWave;                  // 139264
-constexpr int kSmem = kSmemEpi > kSmemMain ? kSmemEpi : kSmemMain;
+constexpr int kBStageSw = kBK * kBN * 2;       // 32768 B per B stage, row pitch 512 B, granule-swizzled
+// (an A stage is rows x 128 B, chunk-swizzled: 32768 B for the 256-row tile, which with two A
+// and three B stages fills all 160 KB of the LDS)
 
 // Maps the linear workgroup id to an output tile so that the workgroups that land on one
 // XCD (ids congruent mod 8 share an L2) cover a compact block of tiles: first regroup
@@ -81,25 +77,38 @@ __device__ __attribute__((aligned(16))) const unsigned g_zero16[4] = {0u, 0u, 0u
 // kRaggedK: K is not a multiple of 64 (but of 8).  The copies of the last, partial K step use
 // per-lane 64-bit addresses so that chunks beyond K can be redirected to g_zero16: zero
 // operands on both sides contribute nothing.  Every other step is copied as in the full case.
-template <bool kRaggedK>
-__device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
-                                                  __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n) {
-    // A stage: 256 rows x 128 B, 16 B chunks XOR-swizzled by ((row >> 1) & 7);
+//
+// kJ: 32-column MFMA tiles per wave.  kJ = 4: 256x256 workgroup tile, waves 2x2, each 128x128.
+// kJ = 2: 128x256 workgroup tile, waves 1x4, each 128x64 (half the accumulators, an A stage of
+// half the size, the same B stages and pipeline) for shapes whose 256x256 tiles would leave
+// most compute units without work.
+template <bool kRaggedK, int kJ>
+__device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                               __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n) {
+    constexpr int kTM = kJ == 4 ? 256 : 128;      // rows of the workgroup tile
+    constexpr int kAq = kTM / 32;                 // 1 KB A chunks (8 rows) each wave copies per K step
+    constexpr int kAStageT = kTM * kBK * 2;       // bytes of an A stage
+    constexpr int kCPitchT = kJ * 64 + 16;        // epilogue staging pitch per wave
+    constexpr int kCWaveT = 128 * kCPitchT;
+    constexpr int kSmemMainT = 2 * kAStageT + 3 * kBStageSw;
+    constexpr int kSmemT = 4 * kCWaveT > kSmemMainT ? 4 * kCWaveT : kSmemMainT;
+    constexpr int kSlots = 4 * kJ;                // MFMAs per phase
+    // A stage: kTM rows x 128 B, 16 B chunks XOR-swizzled by ((row >> 1) & 7);
     // B stage: 64 k-rows x 512 B, 32 B granules XOR-swizzled by (k & 3).
-    __shared__ __attribute__((aligned(1024))) char smem[kSmem];
+    __shared__ __attribute__((aligned(1024))) char smem[kSmemT];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = kJ == 4 ? wave >> 1 : 0, wn = kJ == 4 ? (wave & 1) : wave;
     // blockIdx.y: which of the back-to-back stored products
     A += (size_t)blockIdx.y * M * K;
     B += (size_t)blockIdx.y * K * N;
     C += (size_t)blockIdx.y * M * N;
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
-    const size_t m0 = (size_t)tile_m * kBM, n0 = (size_t)tile_n * kBN;
-    char* sA0 = smem;                // two A stages
-    char* sB0 = smem + 2 * kAStage;  // three B stages
+    const size_t m0 = (size_t)tile_m * kTM, n0 = (size_t)tile_n * kBN;
+    char* sA0 = smem;                 // two A stages
+    char* sB0 = smem + 2 * kAStageT;  // three B stages
 
-    // ---- direct global -> LDS copies: each wave moves 8 KB of A and 8 KB of B per tile,
+    // ---- direct global -> LDS copies: each wave moves kAq KB of A and 8 KB of B per tile,
     // one instruction = 64 lanes x 16 B = 1 KB of contiguous LDS.
     // A chunk q (1 KB = 8 rows): lane -> row q*8 + lane/8, LDS chunk lane%8 holds logical
     // chunk (lane%8) ^ ((row >> 1) & 7).  The LDS serves 16 lanes x 16 B per cycle over 64
@@ -111,10 +120,10 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
     // beyond the edge are redirected to the last valid one (the duplicates only feed outputs
     // the epilogue does not store), which costs nothing per K step: the redirected offsets do
     // not depend on it.  N % 8 == 0 keeps the redirected chunk 16-byte aligned.
-    unsigned a_voff[8];
+    unsigned a_voff[kAq];
 #pragma unroll
-    for (int q = 0; q < 8; q++) {
-        size_t row = m0 + wave * 64 + q * 8 + (lane >> 3);
+    for (int q = 0; q < kAq; q++) {
+        size_t row = m0 + wave * (kAq * 8) + q * 8 + (lane >> 3);
         row = row < (size_t)M ? row : (size_t)M - 1;
         const int chunk = (lane & 7) ^ ((q & 1) * 4 + (lane >> 4));
         a_voff[q] = (unsigned)(((row - m0) * K + (chunk << 3)) * 2);
@@ -129,7 +138,7 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
     }
     const char* a_tile = reinterpret_cast<const char*>(A + m0 * K);
     const char* b_tile = reinterpret_cast<const char*>(B + n0);
-    const unsigned lds_a = (unsigned)(uintptr_t)LDS_PTR(char, sA0) + wave * 8192;
+    const unsigned lds_a = (unsigned)(uintptr_t)LDS_PTR(char, sA0) + wave * (kAq * 1024);
     const unsigned lds_b = (unsigned)(uintptr_t)LDS_PTR(char, sB0) + wave * 8192;
     // One direct copy: 64 lanes x 16 B land at LDS [m0, m0 + 1 KB); the compiler is not told
     // about it (it would otherwise wait for the copy before every later LDS read), so the
@@ -149,10 +158,10 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
     auto dma_a = [&](int q, int kt, int stage) {
         if (kRaggedK && kt == KT - 1) {
             const int chunk = (lane & 7) ^ ((q & 1) * 4 + (lane >> 4));  // logical 8-deep k chunk of this lane
-            dma_from(lds_a + stage * kAStage + q * 1024,
+            dma_from(lds_a + stage * kAStageT + q * 1024,
                      chunk * 8 < k_last ? a_tile + (size_t)kt * kBK * 2 + a_voff[q] : zero16);
         } else {
-            dma(lds_a + stage * kAStage + q * 1024, a_voff[q], a_tile + (size_t)kt * kBK * 2);
+            dma(lds_a + stage * kAStageT + q * 1024, a_voff[q], a_tile + (size_t)kt * kBK * 2);
         }
     };
     auto dma_b = [&](int q, int kt, int stage) {
@@ -164,11 +173,11 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
         dma(lds_b + stage * kBStageSw + q * 1024, b_voff[q & 1], b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
     };
 
-    f32x16 acc[4][4];
+    f32x16 acc[4][kJ];
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < kJ; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
 
@@ -178,28 +187,29 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
 #pragma unroll
     for (int ks = 0; ks < 4; ks++) a_xo[ks] = ((ks * 2 + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4;
     const int b_rr = (lane & 15) >> 2;
-    const int b_g0 = wn * 8 + ((lane >> 4) & 1);
+    const int b_g0 = wn * (2 * kJ) + ((lane >> 4) & 1);  // first 16-column granule of this wave
     const int b_row_l = (8 * (lane >> 5) + b_rr) * 512 + 8 * (lane & 3);  // + ks*16*512 + r*4*512
     const int b_p0 = b_row_l + ((b_g0 ^ b_rr) << 5);                      // j = 0 (+128: j = 2)
     const int b_p1 = b_row_l + (((b_g0 ^ b_rr) ^ 2) << 5);                // j = 1 (+128: j = 3)
 
-    bf16x8 fa[4][4], fb[4][4];  // fragment slot = k-step
+    bf16x8 fa[4][4], fb[4][kJ];  // fragment slot = k-step
     // all but this wave's newest 8 copies (the B chunks issued since the last barrier) have
     // landed, its LDS reads are complete; then all waves meet
     auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
     auto full_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
 #pragma unroll
-    for (int q = 0; q < 8; q++) dma_a(q, 0, 0);
+    for (int q = 0; q < kAq; q++) dma_a(q, 0, 0);
 #pragma unroll
     for (int q = 0; q < 8; q++) dma_b(q, 0, 0);
 #pragma unroll
-    for (int q = 0; q < 8; q++) dma_a(q, KT > 1 ? 1 : 0, 1);
+    for (int q = 0; q < kAq; q++) dma_a(q, KT > 1 ? 1 : 0, 1);
 #pragma unroll
     for (int q = 0; q < 8; q++) dma_b(q, KT > 1 ? 1 : 0, 1);
-    // tile 0 has landed (the 16 copies of tile 1 may still be in flight; the first
+    // tile 0 has landed (the kAq + 8 copies of tile 1 may still be in flight; the first
     // tile_barrier() covers them)
-    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (kAq == 8) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
     for (int ks = 0; ks < 2; ks++) {
         const char* sA = sA0 + a_base_l + a_xo[ks];
@@ -207,7 +217,7 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
 #pragma unroll
         for (int i = 0; i < 4; i++) fa[ks][i] = *LDS_PTR(bf16x8, sA + i * 4096);
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < kJ; j++) {
             const int off = ((j & 1) ? b_p1 : b_p0) + (j >> 1) * 128;
             bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off));
             bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off + 4 * 512));
@@ -215,33 +225,36 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
         }
     }
 
-    // One phase = the 16 MFMAs of k-step p of the current tile (fragment slot p) with the other
-    // pipes' work slotted between them: the 12 LDS reads of the fragments needed two phases
-    // later (slot p ^ 2, from sAn / sBn) and four chunk copies of tile kt2: phases 0-1 its B
-    // chunks into B stage st2, phases 2-3 (after the barrier) its A chunks into A stage `cur`.
+    // One phase = the 4 * kJ MFMAs of k-step p of the current tile (fragment slot p) with the
+    // other pipes' work slotted between them: the 4 + 2 * kJ LDS reads of the fragments needed two
+    // phases later (slot p ^ 2, from sAn / sBn) and chunk copies of tile kt2: phases 0-1 four of
+    // its B chunks each into B stage st2, phases 2-3 (after the barrier) kAq / 2 of its A chunks
+    // each into A stage `cur`.
     auto phase = [&](auto p_c, auto cur_c, int kt2, int st2, const char* sAn, const char* sBn) {
         constexpr int p = decltype(p_c)::value, cur = decltype(cur_c)::value;
         constexpr int slot = p, nslot = p ^ 2;
-        bf16x4 lo[4], hi[4];
+        bf16x4 lo[kJ], hi[kJ];
+        constexpr int kBEvery = kSlots / 4, kAEvery = kSlots / (kAq / 2);  // slots between two copies
 #pragma unroll
-        for (int n = 0; n < 16; n++) {
-            acc[n >> 2][n & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][n & 3], fa[slot][n >> 2], acc[n >> 2][n & 3], 0, 0, 0);
+        for (int n = 0; n < kSlots; n++) {
+            const int mi = n / kJ, mj = n % kJ;
+            acc[mi][mj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][mj], fa[slot][mi], acc[mi][mj], 0, 0, 0);
             if (n < 4) fa[nslot][n] = *LDS_PTR(bf16x8, sAn + n * 4096);
-            else if (n < 12) {
+            else if (n < 4 + 2 * kJ) {
                 const int j = (n - 4) >> 1;
                 const int off = ((j & 1) ? b_p1 : b_p0) + (j >> 1) * 128;
                 if ((n & 1) == 0) lo[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off));
                 else hi[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off + 4 * 512));
             }
-            if ((n & 3) == 1) {
-                const int q = (p & 1) * 4 + (n >> 2);
-                if (p < 2) dma_b(q, kt2, st2);
-                else dma_a(q, kt2, cur);
+            if (p < 2) {
+                if (n % kBEvery == 1 % kBEvery) dma_b((p & 1) * 4 + n / kBEvery, kt2, st2);
+            } else {
+                if (n % kAEvery == 1) dma_a((p & 1) * (kAq / 2) + n / kAEvery, kt2, cur);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
-        for (int j = 0; j < 4; j++) fb[nslot][j] = __builtin_shufflevector(lo[j], hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
+        for (int j = 0; j < kJ; j++) fb[nslot][j] = __builtin_shufflevector(lo[j], hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
         __builtin_amdgcn_sched_barrier(0);
     };
     using C0 = std::integral_constant<int, 0>;
@@ -253,9 +266,9 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
         constexpr int cur = decltype(cur_c)::value;
         using C = std::integral_constant<int, cur>;
         const int kt2 = kt + 2 < KT ? kt + 2 : KT - 1;
-        const char* sAc = sA0 + cur * kAStage + a_base_l;
+        const char* sAc = sA0 + cur * kAStageT + a_base_l;
         const char* sBc = sB0 + st * kBStageSw;
-        const char* sAx = sA0 + (cur ^ 1) * kAStage + a_base_l;
+        const char* sAx = sA0 + (cur ^ 1) * kAStageT + a_base_l;
         const char* sBx = sB0 + stn * kBStageSw;
         phase(C0{}, C{}, kt2, st2, sAc + a_xo[2], sBc + 2 * 16 * 512);
         phase(C1{}, C{}, kt2, st2, sAc + a_xo[3], sBc + 3 * 16 * 512);
@@ -279,27 +292,29 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
 
     // Epilogue.  With swapped operands lane l of tile (i, j) holds, in registers 4g..4g+3,
     // C[m = i*32 + l%32][n = j*32 + 8g + 4*(l/32) + 0..3].
-    char* sC = smem + wave * kCWave;
+    char* sC = smem + wave * kCWaveT;
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++)
+        for (int j = 0; j < kJ; j++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
                 bf16x4 h = __builtin_convertvector(v, bf16x4);
                 const int ml = i * 32 + (lane & 31);
                 const int nl = j * 32 + 8 * g + 4 * (lane >> 5);
-                *LDS_PTR(bf16x4, sC + ml * kCPitch + nl * 2) = h;
+                *LDS_PTR(bf16x4, sC + ml * kCPitchT + nl * 2) = h;
             }
     __syncthreads();
-    const size_t row0 = m0 + wm * 128, col0 = n0 + wn * 128;
+    const size_t row0 = m0 + wm * 128, col0 = n0 + wn * (kJ * 32);
     __bf16* Cg = C + row0 * N + col0;
+    constexpr int kChunks = kJ * 4;          // 16-byte chunks per row of the wave's tile
+    constexpr int kRowsPerIt = 64 / kChunks;  // rows one store instruction covers
 #pragma unroll 4
-    for (int it = 0; it < 32; it++) {
-        const int r = it * 4 + (lane >> 4);
-        const int ch = lane & 15;
-        u32x4 v = *LDS_PTR(u32x4, sC + r * kCPitch + ch * 16);
+    for (int it = 0; it < 128 / kRowsPerIt; it++) {
+        const int r = it * kRowsPerIt + lane / kChunks;
+        const int ch = lane % kChunks;
+        u32x4 v = *LDS_PTR(u32x4, sC + r * kCPitchT + ch * 16);
         if (row0 + r < (size_t)M && col0 + ch * 8 + 8 <= (size_t)N) *reinterpret_cast<u32x4*>(Cg + (size_t)r * N + ch * 8) = v;
     }
 }
@@ -307,12 +322,22 @@ __device__ __forceinline__ void gemm_tile256_body(const __bf16* __restrict__ A, 
 __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                          __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
                                                          int tiles_n) {
-    gemm_tile256_body<false>(A, B, C, M, N, K, tiles_m, tiles_n);
+    gemm_tile_body<false, 4>(A, B, C, M, N, K, tiles_m, tiles_n);
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_ragged_k(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ B, __bf16* __restrict__ C,
                                                                   int M, int N, int K, int tiles_m, int tiles_n) {
-    gemm_tile256_body<true>(A, B, C, M, N, K, tiles_m, tiles_n);
+    gemm_tile_body<true, 4>(A, B, C, M, N, K, tiles_m, tiles_n);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile128(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                         __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
+                                                         int tiles_n) {
+    gemm_tile_body<false, 2>(A, B, C, M, N, K, tiles_m, tiles_n);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile128_ragged_k(const __bf16* __restrict__ A,
+                                                                  const __bf16* __restrict__ B, __bf16* __restrict__ C,
+                                                                  int M, int N, int K, int tiles_m, int tiles_n) {
+    gemm_tile_body<true, 2>(A, B, C, M, N, K, tiles_m, tiles_n);
 }
 
 // Any shape: one wave per 32x32 output tile, operands fetched straight from global memory
@@ -369,14 +394,22 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     const bool offsets_fit = K <= (1L << 23) && N <= (1L << 25);
     // any M; N and K in whole 16-byte chunks
     if (variant != 2 && aligned && offsets_fit && K > 0 && N % 8 == 0 && K % 8 == 0) {
-        const int tm = (int)((M + kBM - 1) / kBM), tn = (int)((N + kBN - 1) / kBN);
+        const long tn = (N + kBN - 1) / kBN;
+        const long tm128 = (M + 127) / 128;
+        // variant 0: the 128-row tile when all its workgroups are resident at once (at most one per
+        // compute unit): twice the workgroups of the 256-row tile for the same work.  3 / 4 force one.
+        const bool small = variant == 4 || (variant != 3 && tm128 * tn * batch <= 256);
+        const long tm = small ? tm128 : (M + kBM - 1) / kBM;
+        if (tm * tn > 0x7fffffffL) return (int)hipErrorInvalidValue;
         const dim3 grid((unsigned)(tm * tn), (unsigned)batch);
-        if (K % kBK == 0)
-            gemm_bf16_tile256<<<grid, 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
-                                                  static_cast<__bf16*>(C), (int)M, (int)N, (int)K, tm, tn);
-        else
-            gemm_bf16_tile256_ragged_k<<<grid, 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
-                                                           static_cast<__bf16*>(C), (int)M, (int)N, (int)K, tm, tn);
+        const __bf16* a = static_cast<const __bf16*>(A);
+        const __bf16* b = static_cast<const __bf16*>(B);
+        __bf16* c = static_cast<__bf16*>(C);
+        const bool ragged_k = K % kBK != 0;
+        if (small && !ragged_k) gemm_bf16_tile128<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+        else if (small) gemm_bf16_tile128_ragged_k<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+        else if (!ragged_k) gemm_bf16_tile256<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+        else gemm_bf16_tile256_ragged_k<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
     } else {
         const long tm = (M + 31) / 32, tn = (N + 31) / 32;
         const long total = tm * tn;

@@ -11,7 +11,8 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 
 
 // C[M,N] = A[M,K] * B[K,N]; bf16 row-major operands, f32 accumulate, bf16 result.
-// variant 0 = choose by shape, 2 = force the any-shape kernel.  batch > 1: that many
+// variant 0 = choose by shape, 2 = force the any-shape kernel, 3 / 4 = force the 256-row /
+// 128-row tile of the tiled kernel (where the shape allows the tiled kernel at all).  batch > 1: that many
 // independent products over matrices stored back to back (A [batch,M,K], B [batch,K,N],
 // C [batch,M,N]), one launch.
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,

@@ -72,8 +72,9 @@ def test_gemm_tiled_kernel_ragged_k(dev, oracle, shape):
     assert np.array_equal(got, _gemm(dev, a, b, variant=2))
 
 
+@pytest.mark.parametrize("variant", [3, 4])
 @pytest.mark.parametrize("shape", [(256, 256, 72), (256, 256, 64), (300, 264, 128), (100, 8, 200), (255, 1000, 8)])
-def test_gemm_does_not_read_past_the_operands(dev, oracle, shape):
+def test_gemm_does_not_read_past_the_operands(dev, oracle, shape, variant):
     """Edge tiles and the partial last K step must not read beyond A and B: NaNs placed right
     behind them in the same allocations do not reach the result (a stray operand would, even
     against a zero: NaN * 0 = NaN)."""
@@ -85,10 +86,25 @@ def test_gemm_does_not_read_past_the_operands(dev, oracle, shape):
     bb = morok_amd.Buffer.from_numpy(np.concatenate([b.reshape(-1), nan]), dev.device_id)
     bc = dev.buffer(M * N * 2 + 4096)
     bc.copyin(np.full(M * N + 2048, 0x7FC0, np.uint16))
-    ops.gemm_bf16(ba, bb, bc, M, N, K, dev.device_id)
+    ops.gemm_bf16(ba, bb, bc, M, N, K, dev.device_id, variant)
     out = bc.copyout(np.uint16)
     _check(out[: M * N].reshape(M, N), oracle.gemm_bf16(a, b), K)
     assert np.all(out[M * N:] == 0x7FC0)   # and nothing is written behind C
+
+
+# The 128-row tile (chosen by itself when the shape has few tiles) and the 256-row tile are the
+# same pipeline: forced either way they agree bit for bit with each other and with the oracle
+# within tolerance, on full, ragged-M/N and ragged-K shapes and on a batch.
+@pytest.mark.parametrize("shape", [(128, 256, 64), (512, 512, 256), (1000, 776, 320), (100, 264, 200), (384, 1024, 1000),
+                                   (129, 8, 72), (2048, 512, 128)])
+def test_gemm_both_tile_sizes_agree(dev, oracle, shape):
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 3, 12)
+    b = synth.normal_bf16((K, N), 3, 13)
+    big, small = _gemm(dev, a, b, variant=3), _gemm(dev, a, b, variant=4)
+    _check(small, oracle.gemm_bf16(a, b), K)
+    assert np.array_equal(big, small)
+    assert np.array_equal(_gemm(dev, a, b), small)
 
 
 @pytest.mark.parametrize("shape", [(1, 1, 1), (32, 32, 16), (33, 65, 17), (100, 200, 300), (5, 7, 1000),
