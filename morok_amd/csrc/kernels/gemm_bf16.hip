@@ -28,6 +28,12 @@
 // of A tile kt+2 follow in the last two phases into the stage tile kt has just left.  For the
 // barrier to sit there every fragment of tile kt must have been read by then: fragments are
 // read two phases ahead of their MFMAs into four register slots (one per 16-deep k-step).
+//
+// Shapes.  M is arbitrary, N and K multiples of 8: edge tiles redirect out-of-range rows and
+// column chunks to the last valid one and mask their stores; a partial last K step is copied
+// from zeros beyond K.  A second instance of the same body with a 128x256 workgroup tile serves
+// shapes that would otherwise leave most compute units idle; a leading batch dimension runs as
+// grid.y.  Everything else takes the any-shape kernel at the end of this file.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
