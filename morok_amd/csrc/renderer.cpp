@@ -852,7 +852,15 @@ class HipRenderer final : public Renderer {
                     return kOk;
                 }
                 std::string e = "(" + c_value_type(u.dtype) + "){";
-                for (size_t i = 0; i < u.src.size(); i++) e += (i ? ", " : "") + S(i);
+                // Arithmetic on 8- and 16-bit integers is carried out in int (the usual
+                // promotions); a braced initialiser refuses the narrowing back, an explicit
+                // cast of each element states it.
+                const Scalar sc = u.dtype.scalar;
+                const bool narrow = sc == Scalar::Int8 || sc == Scalar::UInt8 || sc == Scalar::Int16 || sc == Scalar::UInt16;
+                DType elem = u.dtype;
+                elem.vcount = 1;
+                for (size_t i = 0; i < u.src.size(); i++)
+                    e += (i ? ", " : "") + (narrow ? "((" + c_value_type(elem) + ")" + S(i) + ")" : S(i));
                 ctx.emit(u, e + "}", "vec");
                 return kOk;
             }

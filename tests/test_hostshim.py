@@ -271,6 +271,17 @@ def test_tensor_launch_dims(T, shim):
     assert hostshim_lib.last_dims(shim) == ((2, 1, 1), (64, 1, 1))
 
 
+@pytest.mark.parametrize("tag,npdt", [("U8", np.uint8), ("I8", np.int8), ("I16", np.int16), ("U16", np.uint16)])
+def test_narrow_integer_kernels_compile(T, shim, tag, npdt):
+    """Vectorised kernels on 8- and 16-bit integers: the promoted-to-int arithmetic must be cast
+    back inside vector literals for the source to compile."""
+    dt = getattr(uop, tag)
+    x = T.Tensor.from_numpy(np.zeros((4, 64), npdt), dt)
+    y = x.try_add(T.Tensor.const(3, dt)).try_mul(x)
+    y.realize()
+    assert len(y.kernels()) == 1 and y.dtype == dt
+
+
 def test_tensor_int64_indexing_for_huge_views(T, shim):
     """A broadcast view with more than 2^31 elements feeding a reduce must index in 64 bits."""
     T.set_fusion(False)

@@ -441,3 +441,43 @@ def test_generated_kernels_do_not_read_past_their_inputs(T, dev):
     want = np.where(((idx >= 0) & (idx < 11))[:, None], w[np.clip(idx, 0, 10)], 0.0)
     np.testing.assert_array_equal(tw.embedding(T.Tensor.from_numpy(idx)).to_numpy(), want)
     del keep, keep2, keep3
+
+
+@pytest.mark.parametrize("npdt,tag", [(np.uint8, "U8"), (np.int8, "I8"), (np.int16, "I16"), (np.uint16, "U16")])
+def test_narrow_integer_arithmetic_wraps(T, npdt, tag):
+    """8- and 16-bit integer elementwise kernels (vectorised 16 / 8 wide): results wrap modulo
+    2^bits like the reference's C backend, bit-exact against numpy."""
+    from morok_amd import uop
+
+    dt = getattr(uop, tag)
+    rng = np.random.default_rng(41)
+    info = np.iinfo(npdt)
+    a = rng.integers(info.min, info.max, size=(33, 64), endpoint=True).astype(npdt)
+    b = rng.integers(info.min, info.max, size=(33, 64), endpoint=True).astype(npdt)
+    ta, tb = T.Tensor.from_numpy(a, dt), T.Tensor.from_numpy(b, dt)
+    with np.errstate(over="ignore"):
+        np.testing.assert_array_equal(ta.try_add(tb).to_numpy(), (a + b).astype(npdt))
+        np.testing.assert_array_equal(ta.try_mul(tb).try_sub(ta).to_numpy(), (a * b - a).astype(npdt))
+    np.testing.assert_array_equal(ta.maximum(tb).to_numpy(), np.maximum(a, b))
+
+
+def test_more_than_2_pow_31_elements(T, dev):
+    """Index arithmetic switches to 64 bits when a kernel's iteration space or one of its
+    inputs has 2^31 elements or more: a broadcast view of 2^32 elements reduced by rows, and a
+    real 2^31 + 64 byte tensor through an elementwise kernel (first, last and middle checked)."""
+    from morok_amd import uop
+
+    T.set_fusion(False)
+    s = T.Tensor.full([1 << 16, 1 << 16], 0.5, uop.F32).sum([1])
+    got = s.to_numpy()
+    assert got.shape == (1 << 16,) and np.all(got == 32768.0)
+
+    n = (1 << 31) + 64
+    x = np.empty(n, np.uint8)
+    x[:] = np.arange(n, dtype=np.uint64).astype(np.uint8)       # value = index mod 256
+    t = T.Tensor.from_numpy(x, uop.U8)
+    y = t.try_add(T.Tensor.const(3, uop.U8)).to_numpy()
+    assert y.shape == (n,)
+    for lo in (0, (1 << 31) - 128, n - 256, 1_234_567_890):
+        np.testing.assert_array_equal(y[lo:lo + 128], ((np.arange(lo, lo + 128) + 3) % 256).astype(np.uint8))
+    T.set_fusion(True)
