@@ -481,3 +481,60 @@ def test_more_than_2_pow_31_elements(T, dev):
     for lo in (0, (1 << 31) - 128, n - 256, 1_234_567_890):
         np.testing.assert_array_equal(y[lo:lo + 128], ((np.arange(lo, lo + 128) + 3) % 256).astype(np.uint8))
     T.set_fusion(True)
+
+
+_NP = {"BOOL": np.bool_, "I8": np.int8, "U8": np.uint8, "I16": np.int16, "U16": np.uint16, "I32": np.int32,
+       "U32": np.uint32, "I64": np.int64, "U64": np.uint64, "F16": np.float16, "F32": np.float32, "F64": np.float64}
+
+
+def _values(name, shape, rng):
+    """In-range test values for a dtype (small magnitudes so every cast below is defined)."""
+    if name == "BOOL":
+        return rng.integers(0, 2, size=shape).astype(np.bool_)
+    if name.startswith("U"):
+        return rng.integers(0, 100, size=shape).astype(_NP[name])
+    if name.startswith("I"):
+        return rng.integers(-100, 100, size=shape).astype(_NP[name])
+    return (rng.integers(-400, 400, size=shape) / 4.0).astype(_NP[name])   # quarter steps: exact in f16
+
+
+@pytest.mark.parametrize("src", list(_NP))
+def test_cast_matrix(T, src):
+    """Every dtype to every other through a generated kernel, against numpy's C-style
+    conversions (float -> integer truncates toward zero, anything -> bool is != 0, a negative
+    integer -> unsigned wraps); values are chosen in range of every target."""
+    from morok_amd import uop
+
+    rng = np.random.default_rng(51)
+    x = _values(src, (5, 48), rng)
+    t = T.Tensor.from_numpy(x, getattr(uop, src))
+    for dst, npdst in _NP.items():
+        xs, ts = x, t
+        if src[0] == "F" and dst[0] == "U":
+            # a negative floating value has no defined conversion to an unsigned type in C
+            xs = np.abs(x)
+            ts = T.Tensor.from_numpy(xs, getattr(uop, src))
+        got = ts.cast(getattr(uop, dst)).to_numpy()
+        if dst == "BOOL":
+            want = xs != 0
+        elif dst[0] == "U" and src[0] == "I":
+            want = xs.astype(np.int64).astype(npdst)     # negative -> unsigned wraps modulo 2^bits
+        else:
+            want = xs.astype(npdst)
+        np.testing.assert_array_equal(got, want, err_msg=f"{src} -> {dst}")
+
+
+@pytest.mark.parametrize("name", ["I8", "U8", "I16", "U16", "I32", "U32", "I64", "U64", "F16", "F64"])
+def test_reductions_and_comparisons_across_dtypes(T, name):
+    from morok_amd import uop
+
+    rng = np.random.default_rng(52)
+    a, b = _values(name, (7, 300), rng), _values(name, (7, 300), rng)
+    ta, tb = T.Tensor.from_numpy(a, getattr(uop, name)), T.Tensor.from_numpy(b, getattr(uop, name))
+    np.testing.assert_array_equal(ta.max([1]).to_numpy(), a.max(1))
+    np.testing.assert_array_equal(ta.where(ta.binary("lt", tb), tb).to_numpy(), np.where(a < b, a, b))
+    s = ta.sum([1]).to_numpy()
+    if name[0] in "IU":
+        assert np.array_equal(s.astype(np.int64), a.astype(np.int64).sum(1))   # sums promote, no wrap at these sizes
+    else:
+        np.testing.assert_allclose(s.astype(np.float64), a.astype(np.float64).sum(1), rtol=2e-3 if name == "F16" else 1e-12)
