@@ -538,3 +538,63 @@ def test_reductions_and_comparisons_across_dtypes(T, name):
         assert np.array_equal(s.astype(np.int64), a.astype(np.int64).sum(1))   # sums promote, no wrap at these sizes
     else:
         np.testing.assert_allclose(s.astype(np.float64), a.astype(np.float64).sum(1), rtol=2e-3 if name == "F16" else 1e-12)
+
+
+def _random_graph(T, rng, x_np, x_t):
+    """A random chain of movement and elementwise ops applied to (numpy array, tensor) alike."""
+    a, t = x_np, x_t
+    for _ in range(int(rng.integers(2, 6))):
+        kind = rng.choice(["permute", "reshape", "shrink", "expand", "cat", "add", "mul", "flipcat", "contig"])
+        if kind == "permute" and a.ndim >= 2:
+            perm = list(rng.permutation(a.ndim))
+            a, t = np.transpose(a, perm), t.try_permute([int(p) for p in perm])
+        elif kind == "reshape":
+            n = a.size
+            divs = [d for d in (1, 2, 3, 4, 6, 8, 12, 16, 24) if n % d == 0]
+            d0 = int(rng.choice(divs))
+            rest = n // d0
+            divs2 = [d for d in (1, 2, 3, 4, 8) if rest % d == 0]
+            d1 = int(rng.choice(divs2))
+            shape = [d0, d1, rest // d1]
+            a, t = np.ascontiguousarray(a).reshape(shape), t.try_reshape(shape)
+        elif kind == "shrink" and a.size > 1:
+            rngs = []
+            for s in a.shape:
+                lo = int(rng.integers(0, max(1, s // 2)))
+                hi = int(rng.integers(lo + 1, s + 1))
+                rngs.append((lo, hi))
+            a, t = a[tuple(slice(lo, hi) for lo, hi in rngs)], t.try_shrink(rngs)
+        elif kind == "expand" and a.size <= 4096:
+            a, t = np.broadcast_to(a[None], (3,) + a.shape), t.try_reshape([1] + list(a.shape)).try_expand([3] + list(a.shape))
+        elif kind == "cat" and a.size <= 8192:
+            ax = int(rng.integers(0, a.ndim))
+            a, t = np.concatenate([a, a * 2], ax), T.Tensor.cat([t, t.try_add(t)], ax)
+        elif kind == "flipcat" and a.ndim >= 1 and a.shape[-1] >= 2:
+            h = a.shape[-1] // 2
+            lo = [(0, s) for s in a.shape[:-1]]
+            a2 = np.concatenate([a[..., h:], a[..., :h]], -1)
+            t = T.Tensor.cat([t.try_shrink(lo + [(h, a.shape[-1])]), t.try_shrink(lo + [(0, h)])], a.ndim - 1)
+            a = a2
+        elif kind == "add":
+            a, t = a + 1.5, t.try_add(T.Tensor.const(1.5))
+        elif kind == "mul":
+            a, t = a * a, t.try_mul(t)
+        elif kind == "contig":
+            a, t = np.ascontiguousarray(a), t.contiguous()
+    return a, t
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_movement_chains(T, seed):
+    """Random chains of reshape / permute / shrink / expand / cat with arithmetic in between,
+    realised as generated kernels (vector loads where the layout allows, scalar otherwise),
+    against numpy on the same chain; then reduced over a random axis."""
+    rng = np.random.default_rng(1000 + seed)
+    shape = [int(rng.choice([1, 2, 3, 4, 5, 7, 8, 16, 24])) for _ in range(int(rng.integers(1, 5)))]
+    x = rng.integers(-8, 8, size=shape).astype(np.float32)        # small integers: every result is exact
+    a, t = _random_graph(T, rng, x, T.Tensor.from_numpy(x))
+    assert t.shape == a.shape
+    np.testing.assert_array_equal(t.to_numpy(), a)
+    if a.ndim:
+        ax = int(rng.integers(0, a.ndim))
+        np.testing.assert_array_equal(t.sum([ax]).to_numpy(), a.sum(ax))
