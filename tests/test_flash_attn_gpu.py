@@ -155,3 +155,14 @@ def test_flash_full_size_properties(dev, oracle):
     for b, h in ((0, 0), (7, 31)):
         ref = oracle.sdpa_bf16(q[b:b + 1, h:h + 1], k[b:b + 1, h:h + 1], v[b:b + 1, h:h + 1], SCALE, causal=True)
         _check(o[b:b + 1, h:h + 1], ref)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_flash_random_shapes(dev, oracle, seed):
+    rng = np.random.default_rng(3000 + seed)
+    B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
+    Sq, Sk = int(rng.integers(1, 520)), int(rng.integers(1, 520))
+    causal = bool(seed & 1)
+    scale = float(rng.choice([SCALE, 0.05, 0.2]))
+    q, k, v = _inputs(B, H, Sq, Sk, seed=40 + seed)
+    _check(_attn(dev, q, k, v, scale, causal), oracle.sdpa_bf16(q, k, v, scale, causal=causal))

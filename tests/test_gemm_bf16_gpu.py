@@ -156,3 +156,21 @@ def test_gemm_full_size_config_slice_and_linearity(dev, oracle):
     a2 = synth.to_bf16(synth.from_bf16(a) * 2)
     c2 = _gemm(dev, a2, b)
     assert np.array_equal(synth.from_bf16(c2), synth.from_bf16(c) * 2)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_gemm_random_shapes(dev, oracle, seed):
+    """Random M, N, K (any, including ones that fall back to the any-shape kernel) and a random
+    forced variant: all paths agree with the oracle, and the tiled ones with each other."""
+    rng = np.random.default_rng(2000 + seed)
+    M = int(rng.integers(1, 700))
+    N = int(rng.integers(1, 90)) * (8 if seed % 3 else 1)
+    K = int(rng.integers(1, 60)) * (8 if seed % 4 else 1)
+    a = synth.normal_bf16((M, K), 3, 100 + seed)
+    b = synth.normal_bf16((K, N), 3, 200 + seed)
+    ref = oracle.gemm_bf16(a, b)
+    outs = [_gemm(dev, a, b, variant=v) for v in (0, 2, 3, 4)]
+    for o in outs:
+        _check(o, ref, K)
+    for o in outs[1:]:
+        assert np.array_equal(o, outs[0])

@@ -121,3 +121,14 @@ def test_softmax_edge_values(dev):
 def test_softmax_empty(dev):
     ops.softmax_f32(0, 0, 0, 128, dev.device_id)
     ops.softmax_f32(0, 0, 16, 0, dev.device_id)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_softmax_random_shapes(dev, oracle, seed):
+    rng = np.random.default_rng(4000 + seed)
+    rows = int(rng.integers(1, 70))
+    cols = int(rng.choice([rng.integers(1, 300), rng.integers(300, 9000), rng.integers(9000, 80000)]))
+    x = synth.normal((rows, cols), 2, 50 + seed, sigma=float(rng.choice([0.5, 2.0, 8.0])))
+    y = _run(dev, x, variant=int(seed & 1))
+    _check(y, oracle.softmax_f32(x), rtol=1e-4)
+    _check(y, _softmax_f64(x), rtol=1e-5)
