@@ -193,6 +193,8 @@ void mrk_hip_program_destroy(mrk_program* p);
  *   "softmax_f32"     params = {rows, cols}                         buffers = {y, x}
  *   "gemm_bf16"       params = {M, N, K} or {M, N, K, batch}        buffers = {c, a, b}
  *                     (batch: that many products over matrices stored back to back)
+ *                     params = {M, N, K, batch, workspace bytes}    buffers = {c, a, b, workspace}
+ *                     (split-K for shapes with few output tiles; size from mrk_hip_gemm_bf16_workspace_bytes)
  *   "flash_fwd_bf16"  params = {B*H, Sq, Sk, D, causal, f32 bits of scale}   buffers = {o, q, k, v}
  * Buffer order follows the reference's PARAM numbering: outputs first. */
 int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_program** out);
@@ -374,6 +376,11 @@ int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t r
  * (schedule/src/optimizer/tc.rs:36-94).  Any shape; shapes with M,N % 256 == 0 and
  * K % 64 == 0 take the LDS-tiled kernel. */
 int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k);
+/* Bytes of f32 scratch with which the product of this shape is spread over the chip along K
+ * (few output tiles, long K: a handful of rows against a weight matrix); 0 when the shape has
+ * enough tiles by itself.  mrk_hip_gemm_bf16 takes that scratch from the device allocator by
+ * itself; a "gemm_bf16" builtin Program takes it as its fourth buffer. */
+size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t batch);
 /* Same with an explicit kernel variant (0 choose by shape, 2 any-shape kernel, 3 / 4 tiled kernel
  * with the 256-row / 128-row tile); tuning/tests. */
 int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,

@@ -792,8 +792,20 @@ int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void*
     std::shared_ptr<Device> d;
     MRK_TRY(get_device(device_id, &d));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_gemm_bf16(d->allocator->stream(), a, b, c, m, n, k, variant), "gemm_bf16 launch");
+    // Few output tiles against a long K: scratch for split-K partials comes from the device's
+    // allocator (kept in its LRU cache between calls) and goes back right after the launch; the
+    // next user of the block queues behind this product on the same in-order stream.
+    const size_t ws = variant == 0 ? gemm_bf16_workspace_bytes(m, n, k, 1) : 0;
+    RawBuffer scratch;
+    BufferOptions so;
+    if (ws) MRK_TRY(d->allocator->alloc(ws, so, &scratch));
+    int rc = launch_gemm_bf16(d->allocator->stream(), a, b, c, m, n, k, variant, 1, ws ? scratch.ptr : nullptr, ws);
+    if (ws) d->allocator->free(scratch, so);
+    MRK_HIP(rc, "gemm_bf16 launch");
     return kOk;
+}
+size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t batch) {
+    return gemm_bf16_workspace_bytes(m, n, k, batch);
 }
 int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k) {
     return mrk_hip_gemm_bf16_variant(device_id, a, b, c, m, n, k, 0);

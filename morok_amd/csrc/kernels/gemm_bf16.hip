@@ -88,9 +88,15 @@ __device__ __attribute__((aligned(16))) const unsigned g_zero16[4] = {0u, 0u, 0u
 // kJ = 2: 128x256 workgroup tile, waves 1x4, each 128x64 (half the accumulators, an A stage of
 // half the size, the same B stages and pipeline) for shapes whose 256x256 tiles would leave
 // most compute units without work.
-template <bool kRaggedK, int kJ>
+//
+// kSplitK: blockIdx.z selects a range of `kt_per_split` K steps; the workgroup writes its f32
+// partial tile to W[z][batch][M][N] instead of C and gemm_splitk_reduce adds the partials up in
+// a fixed order.  For shapes with so few tiles that the K loop itself has to be spread over
+// the chip (a handful of rows against a large weight matrix).
+template <bool kRaggedK, int kJ, bool kSplitK = false>
 __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
-                                               __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n) {
+                                               __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+                                               float* __restrict__ W = nullptr, int kt_per_split = 0) {
     constexpr int kTM = kJ == 4 ? 256 : 128;      // rows of the workgroup tile
     constexpr int kAq = kTM / 32;                 // 1 KB A chunks (8 rows) each wave copies per K step
     constexpr int kAStageT = kTM * kBK * 2;       // bytes of an A stage
@@ -107,7 +113,7 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     // blockIdx.y: which of the back-to-back stored products
     A += (size_t)blockIdx.y * M * K;
     B += (size_t)blockIdx.y * K * N;
-    C += (size_t)blockIdx.y * M * N;
+    if (!kSplitK) C += (size_t)blockIdx.y * M * N;
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
     const size_t m0 = (size_t)tile_m * kTM, n0 = (size_t)tile_n * kBN;
@@ -142,8 +148,12 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         col = col + 8 <= (size_t)N ? col : (size_t)N - 8;
         b_voff[par] = (unsigned)(((size_t)(wave * 16 + b_r) * N + (col - n0)) * 2);
     }
-    const char* a_tile = reinterpret_cast<const char*>(A + m0 * K);
-    const char* b_tile = reinterpret_cast<const char*>(B + n0);
+    const int KT_all = (K + kBK - 1) / kBK;
+    const int kt0 = kSplitK ? (int)blockIdx.z * kt_per_split : 0;  // first K step of this workgroup
+    const int KT = kSplitK ? (KT_all - kt0 < kt_per_split ? KT_all - kt0 : kt_per_split) : KT_all;
+    const bool has_last = kt0 + KT == KT_all;  // the (possibly partial) last K step is in this range
+    const char* a_tile = reinterpret_cast<const char*>(A + m0 * K) + (size_t)kt0 * kBK * 2;
+    const char* b_tile = reinterpret_cast<const char*>(B + n0) + (size_t)kt0 * kBK * N * 2;
     const unsigned lds_a = (unsigned)(uintptr_t)LDS_PTR(char, sA0) + wave * (kAq * 1024);
     const unsigned lds_b = (unsigned)(uintptr_t)LDS_PTR(char, sB0) + wave * 8192;
     // One direct copy: 64 lanes x 16 B land at LDS [m0, m0 + 1 KB); the compiler is not told
@@ -158,11 +168,10 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     auto dma_from = [&](unsigned lds_addr, const char* addr) {  // per-lane 64-bit source address
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_addr), "v"(addr) : "m0");
     };
-    const int KT = (K + kBK - 1) / kBK;
-    const int k_last = K - (KT - 1) * kBK;  // depth of the last K step: 64, or 8..56 when ragged
+    const int k_last = K - (KT_all - 1) * kBK;  // depth of the last K step: 64, or 8..56 when ragged
     const char* zero16 = reinterpret_cast<const char*>(g_zero16);
     auto dma_a = [&](int q, int kt, int stage) {
-        if (kRaggedK && kt == KT - 1) {
+        if (kRaggedK && has_last && kt == KT - 1) {
             const int chunk = (lane & 7) ^ ((q & 1) * 4 + (lane >> 4));  // logical 8-deep k chunk of this lane
             dma_from(lds_a + stage * kAStageT + q * 1024,
                      chunk * 8 < k_last ? a_tile + (size_t)kt * kBK * 2 + a_voff[q] : zero16);
@@ -171,7 +180,7 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         }
     };
     auto dma_b = [&](int q, int kt, int stage) {
-        if (kRaggedK && kt == KT - 1) {
+        if (kRaggedK && has_last && kt == KT - 1) {
             dma_from(lds_b + stage * kBStageSw + q * 1024,
                      wave * 16 + q * 2 + b_r < k_last ? b_tile + ((size_t)kt * kBK + q * 2) * N * 2 + b_voff[q & 1] : zero16);
             return;
@@ -298,6 +307,22 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
 
     // Epilogue.  With swapped operands lane l of tile (i, j) holds, in registers 4g..4g+3,
     // C[m = i*32 + l%32][n = j*32 + 8g + 4*(l/32) + 0..3].
+    if (kSplitK) {
+        // f32 partials straight from the registers: 16 bytes per lane, rows and columns masked
+        const size_t row0 = m0 + wm * 128, col0 = n0 + wn * (kJ * 32);
+        float* Wt = W + ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * (size_t)M * N;
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < kJ; j++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const size_t row = row0 + i * 32 + (lane & 31), col = col0 + j * 32 + 8 * g + 4 * (lane >> 5);
+                    f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+                    if (row < (size_t)M && col + 4 <= (size_t)N) *reinterpret_cast<f32x4*>(Wt + row * N + col) = v;
+                }
+        return;
+    }
     char* sC = smem + wave * kCWaveT;
 #pragma unroll
     for (int i = 0; i < 4; i++)
@@ -345,6 +370,33 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile128_ragged_k(const __bf16* 
                                                                   int M, int N, int K, int tiles_m, int tiles_n) {
     gemm_tile_body<true, 2>(A, B, C, M, N, K, tiles_m, tiles_n);
 }
+__global__ __launch_bounds__(256) void gemm_bf16_tile128_splitk(const __bf16* __restrict__ A,
+                                                                const __bf16* __restrict__ B, float* __restrict__ W,
+                                                                int M, int N, int K, int tiles_m, int tiles_n,
+                                                                int kt_per_split) {
+    gemm_tile_body<false, 2, true>(A, B, nullptr, M, N, K, tiles_m, tiles_n, W, kt_per_split);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile128_splitk_ragged_k(const __bf16* __restrict__ A,
+                                                                         const __bf16* __restrict__ B,
+                                                                         float* __restrict__ W, int M, int N, int K,
+                                                                         int tiles_m, int tiles_n, int kt_per_split) {
+    gemm_tile_body<true, 2, true>(A, B, nullptr, M, N, K, tiles_m, tiles_n, W, kt_per_split);
+}
+// C[i] = bf16(W[0][i] + W[1][i] + ... + W[splits-1][i]), 8 elements per work-item, partials added
+// in the order of their K ranges so the result does not depend on timing.
+__global__ __launch_bounds__(256) void gemm_splitk_reduce(const float* __restrict__ W, __bf16* __restrict__ C, long total,
+                                                          int splits) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i >= total) return;
+    f32x4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = lo;
+    for (int s = 0; s < splits; s++) {
+        const f32x4* p = reinterpret_cast<const f32x4*>(W + (size_t)s * total + i);
+        lo += p[0];
+        hi += p[1];
+    }
+    bf16x4 l = __builtin_convertvector(lo, bf16x4), h = __builtin_convertvector(hi, bf16x4);
+    *reinterpret_cast<bf16x8*>(C + i) = __builtin_shufflevector(l, h, 0, 1, 2, 3, 4, 5, 6, 7);
+}
 
 // Any shape: one wave per 32x32 output tile, operands fetched straight from global memory
 // with bounds checks (zero fill), no LDS.  Correct for every M, N, K; used when the shape
@@ -386,8 +438,39 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic(const __bf16* __restric
 
 namespace mrk {
 
+namespace {
+// Split-K plan for a shape: how many K ranges and how many 64-deep steps each, or splits = 1
+// when the plain tiled kernel already has enough workgroups (or the K loop is too short).
+struct SplitPlan {
+    long splits = 1, kt_per_split = 0;
+};
+SplitPlan plan_split_k(long M, long N, long K, long batch) {
+    SplitPlan p;
+    const long tiles = ((M + 127) / 128) * ((N + 255) / 256) * batch;
+    const long kt_all = (K + 63) / 64;
+    if (K % 8 != 0 || N % 8 != 0 || tiles > 64 || kt_all < 8) return p;  // at most a quarter of the CUs busy
+    long want = 256 / tiles;                 // ranges that would put one workgroup on every CU
+    if (want > kt_all / 2) want = kt_all / 2;  // at least two K steps per range
+    // the partial results are written and read back once per range: worth it only while that
+    // traffic stays below what the operands themselves move
+    const double operand_bytes = 2.0 * batch * ((double)M * K + (double)K * N);
+    while (want >= 4 && 2.0 * want * batch * M * N * 4.0 > operand_bytes) want--;
+    if (want < 4) return p;
+    p.kt_per_split = (kt_all + want - 1) / want;
+    p.splits = (kt_all + p.kt_per_split - 1) / p.kt_per_split;
+    if (p.splits < 2) p.splits = 1;
+    return p;
+}
+}  // namespace
+
+size_t gemm_bf16_workspace_bytes(long M, long N, long K, long batch) {
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
+    const SplitPlan p = plan_split_k(M, N, K, batch);
+    return p.splits > 1 ? (size_t)p.splits * batch * M * N * sizeof(float) : 0;
+}
+
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
-                     long batch) {
+                     long batch, void* workspace, size_t workspace_bytes) {
     using namespace mrk::dev;
     if (M <= 0 || N <= 0 || batch <= 0) return 0;
     if (batch > 65535) return (int)hipErrorInvalidValue;  // grid y extent
@@ -402,6 +485,23 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     if (variant != 2 && aligned && offsets_fit && K > 0 && N % 8 == 0 && K % 8 == 0) {
         const long tn = (N + kBN - 1) / kBN;
         const long tm128 = (M + 127) / 128;
+        // a handful of rows against a large weight matrix: spread the K loop over the chip when
+        // the caller brought the workspace for the partial results
+        const SplitPlan sp = variant == 0 || variant == 5 ? plan_split_k(M, N, K, batch) : SplitPlan();
+        if (sp.splits > 1 && workspace && workspace_bytes >= (size_t)sp.splits * batch * M * N * sizeof(float) &&
+            reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && batch * sp.splits <= 65535) {
+            const dim3 grid((unsigned)(tm128 * tn), (unsigned)batch, (unsigned)sp.splits);
+            float* w = static_cast<float*>(workspace);
+            const __bf16* a = static_cast<const __bf16*>(A);
+            const __bf16* b = static_cast<const __bf16*>(B);
+            if (K % kBK == 0)
+                gemm_bf16_tile128_splitk<<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)tm128, (int)tn, (int)sp.kt_per_split);
+            else
+                gemm_bf16_tile128_splitk_ragged_k<<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)tm128, (int)tn, (int)sp.kt_per_split);
+            const long total = batch * M * N;
+            gemm_splitk_reduce<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>(w, static_cast<__bf16*>(C), total, (int)sp.splits);
+            return (int)hipGetLastError();
+        }
         // variant 0: the 128-row tile when all its workgroups are resident at once (at most one per
         // compute unit): twice the workgroups of the 256-row tile for the same work.  3 / 4 force one.
         const bool small = variant == 4 || (variant != 3 && tm128 * tn * batch <= 256);

@@ -12,11 +12,16 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 
 // C[M,N] = A[M,K] * B[K,N]; bf16 row-major operands, f32 accumulate, bf16 result.
 // variant 0 = choose by shape, 2 = force the any-shape kernel, 3 / 4 = force the 256-row /
-// 128-row tile of the tiled kernel (where the shape allows the tiled kernel at all).  batch > 1: that many
+// 128-row tile of the tiled kernel (where the shape allows the tiled kernel at all), 5 = as 0.  batch > 1: that many
 // independent products over matrices stored back to back (A [batch,M,K], B [batch,K,N],
 // C [batch,M,N]), one launch.
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
-                     long batch = 1);
+                     long batch = 1, void* workspace = nullptr, size_t workspace_bytes = 0);
+// Bytes of f32 scratch with which launch_gemm_bf16 spreads the K loop of this shape over the
+// chip (split-K: partial products per K range, added up in a fixed order by a second kernel);
+// 0 when the shape has enough output tiles by itself.  Without the workspace the same shape
+// runs unsplit.
+size_t gemm_bf16_workspace_bytes(long M, long N, long K, long batch);
 
 // O = softmax(Q K^T * scale [causal]) V; Q [BH,Sq,D], K/V [BH,Sk,D], O [BH,Sq,D] bf16, D = 128,
 // scale > 0.  Causal: key j visible to query i iff j <= i.

@@ -1,4 +1,5 @@
 #include "tensor.h"
+#include "kernels/kernels.h"
 
 #include <algorithm>
 #include <chrono>
@@ -931,8 +932,16 @@ struct Scheduler {
             int64_t M = a->shape[a->shape.size() - 2], batch = 1;
             for (size_t i = 0; i + 2 < a->shape.size(); i++) (w->shape.size() == 2 ? M : batch) *= a->shape[i];
             if (a->dtype == Scalar::BFloat16) {
-                rc = batch == 1 ? builtin("gemm_bf16", {M, N, K}, {out, a->buffer, w->buffer})
-                                : builtin("gemm_bf16", {M, N, K, batch}, {out, a->buffer, w->buffer});
+                // few output tiles against a long K: scratch for split-K partials, an intermediate
+                // of the plan like any other (lazily allocated, placed by the memory planner)
+                const size_t ws = gemm_bf16_workspace_bytes(M, N, K, batch);
+                if (ws) {
+                    auto scratch = std::make_shared<Buffer>(dev->allocator, ws, BufferOptions());
+                    rc = builtin("gemm_bf16", {M, N, K, batch, static_cast<int64_t>(ws)}, {out, a->buffer, w->buffer, scratch});
+                } else {
+                    rc = batch == 1 ? builtin("gemm_bf16", {M, N, K}, {out, a->buffer, w->buffer})
+                                    : builtin("gemm_bf16", {M, N, K, batch}, {out, a->buffer, w->buffer});
+                }
             } else {
                 // MOROK_BEAM=<width> selects the LOCAL/UPCAST/UNROLL choices by timed search
                 // (cached on disk) instead of the fixed heuristic (tensor/src/realize.rs:1160-1250)

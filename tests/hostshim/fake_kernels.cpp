@@ -9,7 +9,8 @@ int launch_softmax_f32(void* stream, const void*, void*, long, long, int) {
     mrk_shim_note_launch(stream, "softmax_f32");
     return 0;
 }
-int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, long, int, long) {
+size_t gemm_bf16_workspace_bytes(long, long, long, long) { return 0; }
+int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, long, int, long, void*, size_t) {
     mrk_shim_note_launch(stream, "gemm_bf16");
     return 0;
 }

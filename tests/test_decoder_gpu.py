@@ -47,7 +47,12 @@ def test_decoder_block_vs_oracle(dev, oracle, cfg):
     # seven separate products give the same bits: every output element is the same dot product
     _, out7, kernels7 = run_block(cfg, tok, w, fused=False)
     assert sum(k.startswith("gemm_bf16") for k in kernels7) == 7
-    assert np.array_equal(out7.to_numpy(), got)
+    if any(k.endswith("_splitk") for k in kernels + kernels7):
+        # a product with few rows may be spread over the chip along K in one layout and not in
+        # the other: the same dot products, added up in a different order
+        assert rel_err(out7.to_numpy(), got) <= 1e-2   # single bf16 roundings falling the other way
+    else:
+        assert np.array_equal(out7.to_numpy(), got)
 
 
 def test_decoder_block_full_size_properties(dev):

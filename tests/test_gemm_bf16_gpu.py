@@ -174,3 +174,39 @@ def test_gemm_random_shapes(dev, oracle, seed):
         _check(o, ref, K)
     for o in outs[1:]:
         assert np.array_equal(o, outs[0])
+
+
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (16, 1024, 2048), (100, 264, 4000), (16, 512, 2056), (37, 2048, 4096)])
+def test_gemm_split_k(dev, oracle, shape):
+    """Few output tiles against a long K: the K loop is spread over the chip, f32 partials go to
+    scratch from the device allocator and are added in a fixed order.  Against the oracle, the
+    unsplit kernel (which it may differ from by the rounding of one more f32 addition chain)
+    and itself (the same bits on every run)."""
+    from morok_amd._ffi import lib
+
+    M, N, K = shape
+    assert lib.mrk_hip_gemm_bf16_workspace_bytes(M, N, K, 1) > 0
+    a = synth.normal_bf16((M, K), 3, 14)
+    b = synth.normal_bf16((K, N), 3, 15)
+    got = _gemm(dev, a, b)                    # variant 0: split-K with allocator scratch
+    ref = oracle.gemm_bf16(a, b)
+    _check(got, ref, K)
+    unsplit = _gemm(dev, a, b, variant=4)
+    gf, uf = synth.from_bf16(got), synth.from_bf16(unsplit)
+    assert np.abs(gf - uf).max() <= 2 ** -7 * np.abs(uf).max()
+    assert np.array_equal(got, _gemm(dev, a, b))
+    # the same through a builtin Program with an explicit workspace buffer
+    ws = lib.mrk_hip_gemm_bf16_workspace_bytes(M, N, K, 1)
+    ba, bb = morok_amd.Buffer.from_numpy(a, dev.device_id), morok_amd.Buffer.from_numpy(b, dev.device_id)
+    bc, bw = dev.buffer(M * N * 2), dev.buffer(ws)
+    prog = morok_amd.Program.builtin("gemm_bf16", [M, N, K, 1, ws], dev.device_id)
+    assert prog.name.endswith("_splitk")
+    prog.execute([bc, ba, bb, bw])
+    assert np.array_equal(bc.copyout(np.uint16, nbytes=M * N * 2).reshape(M, N), got)
+
+
+def test_gemm_split_k_not_used_for_large_shapes():
+    from morok_amd._ffi import lib
+
+    for shape in [(4096, 4096, 4096), (512, 4096, 4096), (1024, 1024, 1024), (128, 256, 256), (8, 64, 128), (1024, 8192, 64)]:
+        assert lib.mrk_hip_gemm_bf16_workspace_bytes(*shape, 1) == 0, shape

@@ -598,3 +598,19 @@ def test_random_movement_chains(T, seed):
     if a.ndim:
         ax = int(rng.integers(0, a.ndim))
         np.testing.assert_array_equal(t.sum([ax]).to_numpy(), a.sum(ax))
+
+
+def test_matmul_bf16_few_rows_uses_split_k(T, oracle):
+    """A handful of rows against a large weight matrix through the tensor API: the scheduler
+    adds the split-K scratch to the plan as an intermediate buffer."""
+    from morok_amd import synth, uop
+
+    T.set_fusion(True)
+    rng = np.random.default_rng(61)
+    a = synth.to_bf16(rng.standard_normal((4, 2048), dtype=np.float32))
+    w = synth.to_bf16(rng.standard_normal((2048, 1024), dtype=np.float32))
+    c = T.Tensor.from_numpy(a, uop.BF16).matmul(T.Tensor.from_numpy(w, uop.BF16))
+    got = synth.from_bf16(c.to_numpy())
+    ref = synth.from_bf16(oracle.gemm_bf16(a, w))
+    assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
+    assert c.kernels() == ["gemm_bf16_4_1024_2048_splitk"]
