@@ -330,6 +330,11 @@ int mrk_hip_sched_grouped_dims(const size_t* dims, size_t n, const size_t* max_s
 int mrk_hip_sched_build_matmul_f32(int64_t m, int64_t n, int64_t k, uint8_t** kernel, size_t* len);
 int mrk_hip_sched_build_wmma_matmul(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, uint8_t** kernel,
                                     size_t* len);
+/* The same product with both operands staged through local memory by a workgroup of 2 x 2 waves
+ * (128 x 128 output tile; M, N multiples of 128): the GROUP / LOCAL step of the optimizer
+ * (schedule/src/optimizer/heuristics.rs:37-82) applied after the tensor-core rewrite. */
+int mrk_hip_sched_build_wmma_matmul_lds(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, uint8_t** kernel,
+                                        size_t* len);
 void mrk_hip_sched_free(void* p);
 /* The f32 matmul kernel with the optimisation choices explicit: opts = {LOCAL x, LOCAL y,
  * UPCAST of N (vector width 1/2/4), UPCAST of M (rows per work-item 1..8), UNROLL of K}.

@@ -132,6 +132,8 @@ _SIGS = {
                                                  c_size_p]),
     "mrk_hip_sched_build_wmma_matmul": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int,
                                                   C.POINTER(C.POINTER(C.c_uint8)), c_size_p]),
+    "mrk_hip_sched_build_wmma_matmul_lds": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int,
+                                                      C.POINTER(C.POINTER(C.c_uint8)), c_size_p]),
     "mrk_hip_sched_free": (None, [C.c_void_p]),
     "mrk_hip_softmax_f32": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
     "mrk_hip_softmax_f32_variant": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int]),

@@ -693,6 +693,16 @@ int mrk_hip_sched_build_wmma_matmul(int tc_index, int64_t m, int64_t n, int64_t 
     MRK_TRY(build_wmma_matmul_kernel(tcs[tc_index], m, n, k, static_cast<Scalar>(out_scalar), &lk));
     return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
 }
+int mrk_hip_sched_build_wmma_matmul_lds(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, uint8_t** kernel,
+                                        size_t* len) {
+    MRK_NONNULL(kernel);
+    MRK_NONNULL(len);
+    auto tcs = cdna4_tensor_cores();
+    if (tc_index < 0 || tc_index >= (int)tcs.size()) return fail(kInvalidArgument, "tc index out of range");
+    LinearKernel lk;
+    MRK_TRY(build_wmma_matmul_lds_kernel(tcs[tc_index], m, n, k, static_cast<Scalar>(out_scalar), &lk));
+    return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
+}
 void mrk_hip_sched_free(void* p) { std::free(p); }
 int mrk_hip_sched_build_matmul_f32_opts(int64_t m, int64_t n, int64_t k, const int opts[5], uint8_t** kernel, size_t* len) {
     MRK_NONNULL(opts);

@@ -597,4 +597,155 @@ int build_wmma_matmul_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t
     return kOk;
 }
 
+int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, LinearKernel* k) {
+    const int tn = tc.dims[0], tm = tc.dims[1], tk = tc.dims[2];
+    constexpr int um = 4, un = 4, kWavesM = 2, kWavesN = 2;
+    // K steps of the tensor core per barrier pair (UNROLL of the reduce axis): as many as
+    // divide K, up to 64 elements
+    int ku = 1;
+    while (ku * 2 * tk <= 64 && K % (ku * 2 * tk) == 0) ku *= 2;
+    const int BM = kWavesM * um * tm, BN = kWavesN * un * tn, BK = tk * ku;
+    if (tc.threads != 64 || tm != 16 || tn != 16) return fail(kInvalidArgument, "tensor-core matmul (LDS): only 64-lane 16x16 tensor cores are lowered");
+    if (M % BM || N % BN || K % BK)
+        return failf(kInvalidArgument, "tensor-core matmul (LDS): shape %lldx%lldx%lld is not a multiple of the %dx%dx%d workgroup tile",
+                     (long long)M, (long long)N, (long long)K, BM, BN, BK);
+    const int ea = tc.elements_per_thread[0], eb = tc.elements_per_thread[1], ec = tc.elements_per_thread[2];
+    if (BK % 8 || ea != eb) return fail(kInvalidArgument, "tensor-core matmul (LDS): unsupported operand shape");
+    // both operands: element e of a lane is k + e (consecutive k), same row / column
+    for (int operand = 0; operand < 2; operand++)
+        for (int e = 0; e < ea; e++) {
+            int mn, kk, mn0, kk0;
+            tc_operand_element(tc, operand, 37, e, &mn, &kk);
+            tc_operand_element(tc, operand, 37, 0, &mn0, &kk0);
+            if (mn != mn0 || kk - kk0 != e) return fail(kInvalidArgument, "tensor-core matmul (LDS): lanes must hold consecutive k");
+        }
+    KernelBuilder b;
+    b.enable_cse();
+    uint32_t c = b.param(0, out, M * N), a = b.param(1, tc.dtype_in, M * K), bm = b.param(2, tc.dtype_in, K * N);
+    uint32_t gx = b.special("gidx0", N / BN), gy = b.special("gidx1", M / BM);
+    uint32_t lane = b.special("lidx0", 64), wave = b.special("lidx1", kWavesM * kWavesN);
+    uint32_t tid = b.iadd(b.imul(wave, 64), lane);
+    uint32_t wy = b.idiv(wave, kWavesN), wx = b.imod(wave, kWavesN);
+    auto lane_expr = [&](int operand, bool want_k) -> uint32_t {
+        uint32_t v = b.ci(0);
+        for (int p = 0; p < 6; p++) {
+            int mn, kk, mn0, kk0;
+            tc_operand_element(tc, operand, 1 << p, 0, &mn, &kk);
+            tc_operand_element(tc, operand, 0, 0, &mn0, &kk0);
+            int contrib = want_k ? kk - kk0 : mn - mn0;
+            if (!contrib) continue;
+            uint32_t bit = b.binary(BinaryOp::And, b.binary(BinaryOp::Shr, lane, b.ci(p)), b.ci(1));
+            v = b.iadd(v, b.imul(bit, contrib));
+        }
+        return v;
+    };
+    uint32_t a_m = lane_expr(0, false), a_k = lane_expr(0, true);
+    uint32_t b_n = lane_expr(1, false), b_k = lane_expr(1, true);
+    uint32_t c_m = b.ci(0), c_n = b.ci(0);
+    for (int p = 0; p < 6; p++) {
+        int m, n;
+        tc_acc_element(tc, 1 << p, 0, &m, &n);
+        uint32_t bit = b.binary(BinaryOp::And, b.binary(BinaryOp::Shr, lane, b.ci(p)), b.ci(1));
+        if (m) c_m = b.iadd(c_m, b.imul(bit, m));
+        if (n) c_n = b.iadd(c_n, b.imul(bit, n));
+    }
+    // local memory: A tile [BM][P] and B tile [BK][PB], both as they lie in global memory; the
+    // pitches (+ 8 elements) keep 16-byte alignment for the vector copies and move consecutive
+    // rows to different banks.  A fragments are read back as one vector per lane; a B fragment
+    // is k-strided in this layout and is gathered element by element (writing B transposed
+    // instead would put the 16 lanes of a copy on two banks)
+    const int P = BK + 8, PB = BN + 4;  // B rows 8 apart (the four k groups of a fragment) land 16 banks apart
+    uint32_t sA = b.define_local(0, tc.dtype_in, (int64_t)BM * P), sB = b.define_local(1, tc.dtype_in, (int64_t)BK * PB);
+    // cooperative copies: vectors of 8 elements, 256 work-items
+    const int a_vecs_per_row = BK / 8, VA = BM * a_vecs_per_row / 256;   // per work-item
+    const int b_vecs_per_row = BN / 8, VB = BK * b_vecs_per_row / 256;
+    if (VA < 1 || VB < 1) return fail(kInvalidArgument, "tensor-core matmul (LDS): K tile too shallow for 256 work-items");
+    uint32_t ra = b.define_reg(1, tc.dtype_in, VA, 8), rb = b.define_reg(2, tc.dtype_in, VB, 8);
+    std::vector<uint32_t> a_row(VA), a_kc(VA), b_krow(VB), b_nc(VB);
+    for (int i = 0; i < VA; i++) {
+        uint32_t v = b.iadd(tid, b.ci(256 * i));
+        a_row[i] = b.idiv(v, a_vecs_per_row);
+        a_kc[i] = b.imul(b.imod(v, a_vecs_per_row), 8);
+    }
+    for (int i = 0; i < VB; i++) {
+        uint32_t v = b.iadd(tid, b.ci(256 * i));
+        b_krow[i] = b.idiv(v, b_vecs_per_row);
+        b_nc[i] = b.imul(b.imod(v, b_vecs_per_row), 8);
+    }
+    auto global_to_regs = [&](uint32_t kbase) {
+        for (int i = 0; i < VA; i++) {
+            uint32_t row = b.iadd(b.imul(gy, BM), a_row[i]);
+            b.store(b.index(ra, b.ci(i)), b.load(b.index(a, b.iadd(b.imul(row, K), b.iadd(kbase, a_kc[i]))), 8));
+        }
+        for (int i = 0; i < VB; i++) {
+            uint32_t col = b.iadd(b.imul(gx, BN), b_nc[i]);
+            b.store(b.index(rb, b.ci(i)), b.load(b.index(bm, b.iadd(b.imul(b.iadd(kbase, b_krow[i]), N), col)), 8));
+        }
+    };
+    uint32_t acc = b.define_reg(0, tc.dtype_out, um * un, ec);
+    {
+        std::vector<uint32_t> z(ec, b.cf(0.0, tc.dtype_out));
+        uint32_t zv = b.vectorize(z);
+        for (int i = 0; i < um * un; i++) b.store(b.index(acc, b.ci(i)), zv);
+    }
+    const std::string name = wmma_name(tc);
+    const int64_t KT = K / BK;
+    global_to_regs(b.ci(0));
+    uint32_t r = b.range(KT, 0, AxisType::Reduce);
+    // registers -> local memory
+    for (int i = 0; i < VA; i++) b.store(b.index(sA, b.iadd(b.imul(a_row[i], P), a_kc[i])), b.load(b.index(ra, b.ci(i))));
+    for (int i = 0; i < VB; i++) {  // rows of PB elements are 8-byte aligned: two stores of four
+        uint32_t vb = b.load(b.index(rb, b.ci(i)));
+        for (int h = 0; h < 2; h++) {
+            std::vector<uint32_t> half;
+            for (int e = 0; e < 4; e++) half.push_back(b.gep(vb, 4 * h + e));
+            b.store(b.index(sB, b.iadd(b.imul(b_krow[i], PB), b.iadd(b_nc[i], b.ci(4 * h)))), b.vectorize(half));
+        }
+    }
+    b.barrier();
+    // the next step's tiles travel while this step computes (the last step reloads its own)
+    uint32_t rn = b.iadd(r, b.ci(1));
+    uint32_t knext = b.imul(b.where(b.binary(BinaryOp::Lt, rn, b.ci(KT)), rn, b.ci(KT - 1)), BK);
+    global_to_regs(knext);
+    for (int kk = 0; kk < ku; kk++) {
+        std::vector<uint32_t> afrag(um), bfrag(un);
+        for (int i = 0; i < um; i++) {
+            uint32_t row = b.iadd(b.iadd(b.imul(wy, um * tm), b.ci(i * tm)), a_m);
+            afrag[i] = b.load(b.index(sA, b.iadd(b.imul(row, P), b.iadd(a_k, b.ci(kk * tk)))), ea);
+        }
+        for (int j = 0; j < un; j++) {
+            uint32_t col = b.iadd(b.iadd(b.imul(wx, un * tn), b.ci(j * tn)), b_n);
+            std::vector<uint32_t> el;
+            for (int e = 0; e < eb; e++)
+                el.push_back(b.load(b.index(sB, b.iadd(b.imul(b.iadd(b_k, b.ci(kk * tk + e)), PB), col))));
+            bfrag[j] = b.vectorize(el);
+        }
+        for (int i = 0; i < um; i++)
+            for (int j = 0; j < un; j++) {
+                uint32_t slot = b.index(acc, b.ci(i * un + j));
+                DType cd = KernelBuilder::scalar(tc.dtype_out, ec);
+                uint32_t w = b.add(Op::Wmma, cd, {afrag[i], bfrag[j], b.load(slot)}, 0, 0, 0, name);
+                b.store(slot, w);
+            }
+    }
+    b.barrier();  // every wave is done with the tiles before the next step overwrites them
+    b.end({r});
+    for (int i = 0; i < um; i++)
+        for (int j = 0; j < un; j++) {
+            uint32_t res = b.load(b.index(acc, b.ci(i * un + j)));
+            for (int e = 0; e < ec; e++) {
+                int m, n, m0, n0;
+                tc_acc_element(tc, 0, e, &m, &n);
+                tc_acc_element(tc, 0, 0, &m0, &n0);
+                uint32_t row = b.iadd(b.iadd(b.iadd(b.imul(gy, BM), b.imul(wy, um * tm)), b.ci(i * tm + (m - m0))), c_m);
+                uint32_t col = b.iadd(b.iadd(b.iadd(b.imul(gx, BN), b.imul(wx, un * tn)), b.ci(j * tn + (n - n0))), c_n);
+                uint32_t v = b.gep(res, e);
+                if (out != tc.dtype_out) v = b.cast(v, out);
+                b.store(b.index(c, b.iadd(b.imul(row, N), col)), v);
+            }
+        }
+    *k = b.finish();
+    return kOk;
+}
+
 }  // namespace mrk

@@ -140,6 +140,8 @@ class KernelBuilder {
         return add(Op::Reduce, dtype(v), std::move(s), 0, 0, static_cast<uint16_t>(op));
     }
     uint32_t wave_reduce(ReduceOp op, uint32_t v) { return add(Op::WaveReduce, dtype(v), {v}, 0, 0, static_cast<uint16_t>(op)); }
+    uint32_t define_local(int id, Scalar s, int64_t size) { return add(Op::DefineLocal, pointer(s, size, AddrSpace::Local), {}, id); }
+    uint32_t barrier() { return add(Op::Barrier, scalar(Scalar::Void)); }
     uint32_t define_reg(int id, Scalar s, int64_t size, int vcount = 1) {
         return add(Op::DefineReg, pointer(s, size, AddrSpace::Reg, vcount), {}, id);
     }
@@ -188,5 +190,15 @@ LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K, const Matm
 // swizzle prescribes, WMMA per K step, accumulate in dtype_out, result cast to `out`.
 // Post-TC upcasts of M and N by the first of [5,4,3,2] that divides (heuristics.rs:787-821).
 int build_wmma_matmul_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, LinearKernel* k);
+// The same product with the operands staged through local memory (GROUP / LOCAL of the
+// optimizer, schedule/src/optimizer/heuristics.rs:37-82, transforms.rs:1085-1089): a workgroup
+// of 2 x 2 waves owns a 128 x 128 output tile (4 x 4 tensor-core tiles per wave); per K step
+// the 256 work-items copy the A and B tiles global -> registers -> LDS with 16-byte loads (the
+// next step's loads are issued before this step's WMMAs); A fragments are read back as one
+// vector per lane, B fragments (k-strided in a row-major tile) element by element; two barriers
+// per step.
+// Requires M % 128 == 0, N % 128 == 0, K % tile_k == 0 and a tensor core whose lanes hold
+// consecutive k.
+int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, LinearKernel* k);
 
 }  // namespace mrk

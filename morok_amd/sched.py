@@ -99,6 +99,12 @@ def build_wmma_matmul(tc_index, m, n, k, out_scalar=U.BF16):
     return _take(lib.mrk_hip_sched_build_wmma_matmul, tc_index, m, n, k, out_scalar)
 
 
+def build_wmma_matmul_lds(tc_index, m, n, k, out_scalar):
+    """The tensor-core matmul with both operands staged through local memory by a workgroup of
+    2 x 2 waves (128 x 128 output tile); serialized linear kernel."""
+    return _take(lib.mrk_hip_sched_build_wmma_matmul_lds, tc_index, m, n, k, out_scalar)
+
+
 def build_matmul_f32_opts(m, n, k, opts):
     """f32 matmul kernel with explicit (LOCAL x, LOCAL y, UPCAST n, UPCAST m, UNROLL k)."""
     arr = (C.c_int * 5)(*opts)

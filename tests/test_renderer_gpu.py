@@ -224,6 +224,33 @@ def test_tc_apply_matmul_from_tables(dev, oracle, tc, shape, out):
     assert np.array_equal(c1, want if out == U.BF16 else synth.from_bf16(want))
 
 
+@pytest.mark.parametrize("tc,shape,out", [(1, (128, 128, 32), U.BF16), (1, (256, 384, 160), U.BF16), (1, (128, 256, 1024), U.F32),
+                                          (3, (128, 128, 48), U.BF16)])
+def test_tc_matmul_staged_through_local_memory(dev, oracle, tc, shape, out):
+    """The generated tensor-core matmul with a 2 x 2-wave workgroup, both operands copied
+    through LDS (B transposed on the way) and two barriers per K step: against float64, the
+    register-only generated kernel (same products, same K order: the same bits) and one-hot
+    operands that pin the copy and fragment indexing exactly."""
+    from morok_amd import sched
+
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 3, 12)
+    b = synth.normal_bf16((K, N), 3, 13)
+    kern = sched.build_wmma_matmul_lds(tc, M, N, K, out)
+    np_out = np.uint16 if out == U.BF16 else np.float32
+    c = run(dev, kern, "r_tc_lds", (M, N), np_out, [a, b])
+    ref = synth.from_bf16(a).astype(np.float64) @ synth.from_bf16(b).astype(np.float64)
+    cf = synth.from_bf16(c) if out == U.BF16 else c
+    assert np.abs(cf - ref).max() <= 2e-2 * np.abs(ref).max()
+    plain = run(dev, sched.build_wmma_matmul(tc, M, N, K, out), "r_tc", (M, N), np_out, [a, b])
+    assert np.array_equal(c, plain)
+    a1 = np.zeros((M, K), np.float32)
+    a1[np.arange(M), (np.arange(M) * 7) % K] = 1
+    c1 = run(dev, kern, "r_tc_lds", (M, N), np_out, [synth.to_bf16(a1), b])
+    want = b[(np.arange(M) * 7) % K]
+    assert np.array_equal(c1, want if out == U.BF16 else synth.from_bf16(want))
+
+
 def test_scheduled_matmul_f32_kernel(dev, oracle):
     from morok_amd import sched
 

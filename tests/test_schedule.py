@@ -137,3 +137,22 @@ def test_matmul_kernels_render_and_compile():
     assert "not a multiple" in e.value.message
     morok_amd.compile_spec(U.render(sched.build_wmma_matmul(0, 32, 32, 64, U.F16), "r_tc16"))
     morok_amd.compile_spec(U.render(sched.build_wmma_matmul(2, 32, 32, 64, U.F32), "r_tc16k16"))
+
+
+def test_wmma_matmul_lds_kernel_builds_and_compiles():
+    """The LDS-staged tensor-core matmul renders to two __shared__ tiles, two barriers per K
+    step and 16 MFMA builtins per wave and K step, and compiles for gfx950; shapes off the
+    128 x 128 workgroup tile are refused."""
+    import morok_amd
+    from morok_amd import sched, uop as U
+
+    kern = sched.build_wmma_matmul_lds(1, 256, 128, 64, U.BF16)
+    spec = U.render(kern, "r_tc_lds")
+    src = spec.src
+    assert src.count("__shared__") == 2 and src.count("__syncthreads();") == 2
+    assert "__builtin_amdgcn_mfma_f32_16x16x32_bf16" in src
+    assert src.count("__WMMA_16_16_32_bfloat_float(") == 2 * 16 + 1   # two K steps x 4 x 4 tiles per wave + the definition
+    assert spec.sizes() == ([1, 2, 1], [64, 4, 1])
+    morok_amd.compile_spec(spec)
+    with pytest.raises(morok_amd.MorokHipError):
+        sched.build_wmma_matmul_lds(1, 64, 128, 64, U.BF16)
