@@ -893,9 +893,40 @@ struct Scheduler {
         }
     }
 
+    // With the hand-written kernels switched off, a bf16 matmul whose shape fits still takes the
+    // tensor-core route of the optimizer (schedule/src/optimizer/tc.rs:36-94): the generated
+    // WMMA kernel staged through local memory instead of the generic reduce kernel.
+    bool generated_tc(const TensorNode* n) const {
+        if (g_fusion || n->hint != HintKind::Matmul || n->numel() == 0) return false;
+        const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
+        if (a->dtype != Scalar::BFloat16 || w->dtype != Scalar::BFloat16 || n->dtype != Scalar::BFloat16) return false;
+        if (a->shape.size() != 2 || w->shape.size() != 2) return false;
+        return a->shape[0] % 128 == 0 && w->shape[1] % 128 == 0 && a->shape[1] % 32 == 0 && a->shape[1] > 0;
+    }
+    int materialize_generated_tc(TensorNode* n) {
+        for (const TensorRef& in : n->hint_inputs) MRK_TRY(materialize(in.get()));
+        const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
+        const int64_t M = a->shape[0], K = a->shape[1], N = w->shape[1];
+        const auto tcs = cdna4_tensor_cores();
+        const int tc = select_tensor_core(tcs, Scalar::BFloat16, Scalar::BFloat16, Scalar::Float32);
+        if (tc < 0) return fail(kRuntime, "no bf16 tensor core in the CDNA table");
+        LinearKernel k;
+        MRK_TRY(build_wmma_matmul_lds_kernel(tcs[tc], M, N, K, Scalar::BFloat16, &k));
+        std::shared_ptr<CachedKernel> ck;
+        bool cached = false;
+        const std::string name = "r_tc_" + std::to_string(M) + "_" + std::to_string(N) + "_" + std::to_string(K);
+        MRK_TRY(get_or_compile_linear_kernel(*dev, k, name.c_str(), &ck, &cached));
+        auto out = new_buffer(n);
+        MRK_TRY(add_kernel(ck, {out, a->buffer, w->buffer}, cached));
+        n->buffer = out;
+        produced.push_back(n);
+        return kOk;
+    }
+
     int materialize(TensorNode* n) {
         if (n->buffer) return kOk;
         if (n->numel() > 0 && fusable(n)) return materialize_fused(n);
+        if (generated_tc(n)) return materialize_generated_tc(n);
         // a reshape of materialised data is the same bytes
         if (n->kind == TKind::Reshape) {
             TensorNode* s = n->src[0].get();

@@ -614,3 +614,25 @@ def test_matmul_bf16_few_rows_uses_split_k(T, oracle):
     ref = synth.from_bf16(oracle.gemm_bf16(a, w))
     assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
     assert c.kernels() == ["gemm_bf16_4_1024_2048_splitk"]
+
+
+def test_matmul_bf16_generated_tensor_core(T, oracle):
+    """With the hand-written kernels off, a bf16 matmul whose shape fits the 128 x 128 workgroup
+    tile takes the generated tensor-core kernel (WMMA staged through local memory); other shapes
+    keep the generic reduce kernel.  Same numerics policy as the hand-written GEMM: exact
+    products, f32 accumulation, one rounding."""
+    from morok_amd import synth, uop
+
+    T.set_fusion(False)
+    rng = np.random.default_rng(71)
+    for (M, N, K), tc in (((256, 128, 96), True), ((128, 256, 1024), True), ((96, 128, 64), False)):
+        a = synth.to_bf16(rng.standard_normal((M, K), dtype=np.float32))
+        w = synth.to_bf16(rng.standard_normal((K, N), dtype=np.float32))
+        c = T.Tensor.from_numpy(a, uop.BF16).matmul(T.Tensor.from_numpy(w, uop.BF16))
+        got = synth.from_bf16(c.to_numpy())
+        ref = synth.from_bf16(oracle.gemm_bf16(a, w))
+        assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
+        assert (c.kernels() == [f"r_tc_{M}_{N}_{K}"]) == tc, c.kernels()
+        if tc:
+            assert "__builtin_amdgcn_mfma" in T.last_kernel_sources()[0] and "__shared__" in T.last_kernel_sources()[0]
+    T.set_fusion(True)
