@@ -538,10 +538,19 @@ class HipRenderer final : public Renderer {
         }
         std::set<std::string> wmma_names;
         bool uses_wave_reduce = false;
+        int64_t reg_bytes = 0;  // per work-item, in declared register objects
         for (const UOp& u : nodes) {
             if (u.op == Op::Wmma) wmma_names.insert(u.str);
             if (u.op == Op::WaveReduce) uses_wave_reduce = true;
+            if (u.op == Op::DefineReg)
+                reg_bytes += (u.dtype.ptr_size > 0 ? u.dtype.ptr_size : 1) * static_cast<int64_t>(scalar_bytes(u.dtype.scalar)) * u.dtype.vcount;
         }
+        // A tensor-core kernel with workgroups of four waves or more whose declared registers
+        // leave room asks for two waves per SIMD (256 registers each).  Left at one, the device
+        // compiler spreads the accumulators over both halves of the 512-entry file and copies
+        // them between the halves on every trip of the K loop.  (One-wave workgroups measured
+        // slower with the hint, so they go without.)
+        const bool two_waves = !wmma_names.empty() && reg_bytes <= 128 * 4 && local[0] * local[1] * local[2] >= 256;
         for (const std::string& w : wmma_names) {
             std::string def;
             if (!wmma_wrapper(w, &def)) return fail(kRenderError, "render: no gfx950 MFMA lowering for " + w);
@@ -608,8 +617,8 @@ class HipRenderer final : public Renderer {
         std::ostringstream src;
         for (const std::string& l : pre) src << l << "\n";
         if (!pre.empty()) src << "\n";
-        src << "extern \"C\" __global__ void __launch_bounds__(" << local[0] * local[1] * local[2] << ") " << kernel_name
-            << "(";
+        src << "extern \"C\" __global__ void __launch_bounds__(" << local[0] * local[1] * local[2] << ") "
+            << (two_waves ? "__attribute__((amdgpu_waves_per_eu(2))) " : "") << kernel_name << "(";
         for (size_t i = 0; i < params.size(); i++) src << (i ? ", " : "") << params[i];
         src << ") {\n";
         for (const std::string& l : decls) src << l << "\n";

@@ -649,12 +649,24 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
         if (m) c_m = b.iadd(c_m, b.imul(bit, m));
         if (n) c_n = b.iadd(c_n, b.imul(bit, n));
     }
-    // local memory: A tile [BM][P] and B tile [BK][PB], both as they lie in global memory; the
-    // pitches (+ 8 elements) keep 16-byte alignment for the vector copies and move consecutive
-    // rows to different banks.  A fragments are read back as one vector per lane; a B fragment
-    // is k-strided in this layout and is gathered element by element (writing B transposed
-    // instead would put the 16 lanes of a copy on two banks)
-    const int P = BK + 8, PB = BN + 4;  // B rows 8 apart (the four k groups of a fragment) land 16 banks apart
+    // local memory.  A tile [BM][P] as it lies in global memory (the pitch of BK + 8 keeps the
+    // vector copies 16-byte aligned and moves consecutive rows to different banks); a lane's A
+    // fragment is one vector read.  A B fragment is k-strided in global memory, so B is kept
+    // with rows k and k+1 interleaved, [BK/2][PB][2]: a work-item copies the same 8 columns
+    // of both rows, zips them in registers and writes two 16-byte vectors, and a lane reads
+    // its fragment as element pairs, ready for the tensor core without repacking.  (Writing B
+    // transposed instead would put the 16 lanes of a copy on two banks.)  PB = BN + 4 puts
+    // the four k groups of a fragment, 4 pair-rows apart, 16 banks apart.  A K tile of fewer
+    // than 32 rows has too few pairs for 256 work-items and keeps plain rows, gathered
+    // element by element.
+    bool pairs = BK % 32 == 0 && eb % 2 == 0;
+    for (int p = 0; p < 6 && pairs; p++) {
+        int mn, kk, mn0, kk0;
+        tc_operand_element(tc, 1, 1 << p, 0, &mn, &kk);
+        tc_operand_element(tc, 1, 0, 0, &mn0, &kk0);
+        if ((kk - kk0) % 2) pairs = false;
+    }
+    const int P = BK + 8, PB = BN + 4;
     uint32_t sA = b.define_local(0, tc.dtype_in, (int64_t)BM * P), sB = b.define_local(1, tc.dtype_in, (int64_t)BK * PB);
     // cooperative copies: vectors of 8 elements, 256 work-items
     const int a_vecs_per_row = BK / 8, VA = BM * a_vecs_per_row / 256;   // per work-item
@@ -668,9 +680,15 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
         a_kc[i] = b.imul(b.imod(v, a_vecs_per_row), 8);
     }
     for (int i = 0; i < VB; i++) {
-        uint32_t v = b.iadd(tid, b.ci(256 * i));
-        b_krow[i] = b.idiv(v, b_vecs_per_row);
-        b_nc[i] = b.imul(b.imod(v, b_vecs_per_row), 8);
+        if (pairs) {  // vectors 2i and 2i+1 of a work-item: rows 2p and 2p+1, same columns
+            uint32_t v = b.iadd(tid, b.ci(256 * (i / 2)));
+            b_krow[i] = b.iadd(b.imul(b.idiv(v, b_vecs_per_row), 2), b.ci(i % 2));
+            b_nc[i] = b.imul(b.imod(v, b_vecs_per_row), 8);
+        } else {
+            uint32_t v = b.iadd(tid, b.ci(256 * i));
+            b_krow[i] = b.idiv(v, b_vecs_per_row);
+            b_nc[i] = b.imul(b.imod(v, b_vecs_per_row), 8);
+        }
     }
     auto global_to_regs = [&](uint32_t kbase) {
         for (int i = 0; i < VA; i++) {
@@ -682,11 +700,16 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
             b.store(b.index(rb, b.ci(i)), b.load(b.index(bm, b.iadd(b.imul(b.iadd(kbase, b_krow[i]), N), col)), 8));
         }
     };
-    uint32_t acc = b.define_reg(0, tc.dtype_out, um * un, ec);
+    // one register object per accumulator tile: as slots of one array the 64 floats become a
+    // single register tuple, which the device compiler shuffles around on every K step
+    std::vector<uint32_t> acc(um * un);
     {
         std::vector<uint32_t> z(ec, b.cf(0.0, tc.dtype_out));
         uint32_t zv = b.vectorize(z);
-        for (int i = 0; i < um * un; i++) b.store(b.index(acc, b.ci(i)), zv);
+        for (int i = 0; i < um * un; i++) {
+            acc[i] = b.index(b.define_reg(3 + i, tc.dtype_out, 1, ec), b.ci(0));
+            b.store(acc[i], zv);
+        }
     }
     const std::string name = wmma_name(tc);
     const int64_t KT = K / BK;
@@ -694,35 +717,63 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
     uint32_t r = b.range(KT, 0, AxisType::Reduce);
     // registers -> local memory
     for (int i = 0; i < VA; i++) b.store(b.index(sA, b.iadd(b.imul(a_row[i], P), a_kc[i])), b.load(b.index(ra, b.ci(i))));
-    for (int i = 0; i < VB; i++) {  // rows of PB elements are 8-byte aligned: two stores of four
-        uint32_t vb = b.load(b.index(rb, b.ci(i)));
-        for (int h = 0; h < 2; h++) {
-            std::vector<uint32_t> half;
-            for (int e = 0; e < 4; e++) half.push_back(b.gep(vb, 4 * h + e));
-            b.store(b.index(sB, b.iadd(b.imul(b_krow[i], PB), b.iadd(b_nc[i], b.ci(4 * h)))), b.vectorize(half));
+    if (pairs) {
+        for (int i = 0; i < VB; i += 2) {
+            uint32_t v0 = b.load(b.index(rb, b.ci(i))), v1 = b.load(b.index(rb, b.ci(i + 1)));
+            uint32_t prow = b.idiv(b_krow[i], 2);
+            for (int h = 0; h < 2; h++) {
+                std::vector<uint32_t> zip;
+                for (int e = 0; e < 4; e++) {
+                    zip.push_back(b.gep(v0, 4 * h + e));
+                    zip.push_back(b.gep(v1, 4 * h + e));
+                }
+                b.store(b.index(sB, b.imul(b.iadd(b.imul(prow, PB), b.iadd(b_nc[i], b.ci(4 * h))), 2)), b.vectorize(zip));
+            }
+        }
+    } else {
+        for (int i = 0; i < VB; i++) {  // rows of PB elements are 8-byte aligned: two stores of four
+            uint32_t vb = b.load(b.index(rb, b.ci(i)));
+            for (int h = 0; h < 2; h++) {
+                std::vector<uint32_t> half;
+                for (int e = 0; e < 4; e++) half.push_back(b.gep(vb, 4 * h + e));
+                b.store(b.index(sB, b.iadd(b.imul(b_krow[i], PB), b.iadd(b_nc[i], b.ci(4 * h)))), b.vectorize(half));
+            }
         }
     }
-    b.barrier();
-    // the next step's tiles travel while this step computes (the last step reloads its own)
+    // the next step's tiles travel while this step computes (the last step reloads its own).
+    // The loads are issued ahead of the barrier: the device compiler moves no memory operation
+    // across one, and left after it they sink below the tensor-core work, to the end of the
+    // step, where the next step waits for them at once
     uint32_t rn = b.iadd(r, b.ci(1));
     uint32_t knext = b.imul(b.where(b.binary(BinaryOp::Lt, rn, b.ci(KT)), rn, b.ci(KT - 1)), BK);
     global_to_regs(knext);
+    b.barrier();
+    // fragment addresses as one lane-dependent base plus a constant per fragment, so that the
+    // constants fold into the instructions' offset fields instead of taking a register each
+    uint32_t a_base = b.iadd(b.imul(b.iadd(b.imul(wy, um * tm), a_m), P), a_k);
+    uint32_t b_col = b.iadd(b.imul(wx, un * tn), b_n);
+    uint32_t b_base = pairs ? b.imul(b.iadd(b.imul(b.idiv(b_k, 2), PB), b_col), 2) : b.iadd(b.imul(b_k, PB), b_col);
     for (int kk = 0; kk < ku; kk++) {
         std::vector<uint32_t> afrag(um), bfrag(un);
-        for (int i = 0; i < um; i++) {
-            uint32_t row = b.iadd(b.iadd(b.imul(wy, um * tm), b.ci(i * tm)), a_m);
-            afrag[i] = b.load(b.index(sA, b.iadd(b.imul(row, P), b.iadd(a_k, b.ci(kk * tk)))), ea);
-        }
+        for (int i = 0; i < um; i++)
+            afrag[i] = b.load(b.index(sA, b.iadd(a_base, b.ci(i * tm * P + kk * tk))), ea);
         for (int j = 0; j < un; j++) {
-            uint32_t col = b.iadd(b.iadd(b.imul(wx, un * tn), b.ci(j * tn)), b_n);
             std::vector<uint32_t> el;
-            for (int e = 0; e < eb; e++)
-                el.push_back(b.load(b.index(sB, b.iadd(b.imul(b.iadd(b_k, b.ci(kk * tk + e)), PB), col))));
+            if (pairs) {
+                for (int q = 0; q < eb / 2; q++) {
+                    uint32_t two = b.load(b.index(sB, b.iadd(b_base, b.ci(((kk * tk / 2 + q) * PB + j * tn) * 2))), 2);
+                    el.push_back(b.gep(two, 0));
+                    el.push_back(b.gep(two, 1));
+                }
+            } else {
+                for (int e = 0; e < eb; e++)
+                    el.push_back(b.load(b.index(sB, b.iadd(b_base, b.ci((kk * tk + e) * PB + j * tn)))));
+            }
             bfrag[j] = b.vectorize(el);
         }
         for (int i = 0; i < um; i++)
             for (int j = 0; j < un; j++) {
-                uint32_t slot = b.index(acc, b.ci(i * un + j));
+                uint32_t slot = acc[i * un + j];
                 DType cd = KernelBuilder::scalar(tc.dtype_out, ec);
                 uint32_t w = b.add(Op::Wmma, cd, {afrag[i], bfrag[j], b.load(slot)}, 0, 0, 0, name);
                 b.store(slot, w);
@@ -732,7 +783,7 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
     b.end({r});
     for (int i = 0; i < um; i++)
         for (int j = 0; j < un; j++) {
-            uint32_t res = b.load(b.index(acc, b.ci(i * un + j)));
+            uint32_t res = b.load(acc[i * un + j]);
             for (int e = 0; e < ec; e++) {
                 int m, n, m0, n0;
                 tc_acc_element(tc, 0, e, &m, &n);

@@ -225,10 +225,11 @@ def test_tc_apply_matmul_from_tables(dev, oracle, tc, shape, out):
 
 
 @pytest.mark.parametrize("tc,shape,out", [(1, (128, 128, 32), U.BF16), (1, (256, 384, 160), U.BF16), (1, (128, 256, 1024), U.F32),
-                                          (3, (128, 128, 48), U.BF16)])
+                                          (3, (128, 128, 48), U.BF16), (3, (256, 128, 96), U.BF16)])
 def test_tc_matmul_staged_through_local_memory(dev, oracle, tc, shape, out):
     """The generated tensor-core matmul with a 2 x 2-wave workgroup, both operands copied
-    through LDS (B transposed on the way) and two barriers per K step: against float64, the
+    through LDS (B with pairs of K rows interleaved, or as plain rows when the K tile is 16
+    deep) and two barriers per K step: against float64, the
     register-only generated kernel (same products, same K order: the same bits) and one-hot
     operands that pin the copy and fragment indexing exactly."""
     from morok_amd import sched
