@@ -196,6 +196,9 @@ void mrk_hip_program_destroy(mrk_program* p);
  *                     params = {M, N, K, batch, workspace bytes}    buffers = {c, a, b, workspace}
  *                     (split-K for shapes with few output tiles; size from mrk_hip_gemm_bf16_workspace_bytes)
  *   "flash_fwd_bf16"  params = {B*H, Sq, Sk, D, causal, f32 bits of scale}   buffers = {o, q, k, v}
+ *   "flash_fwd_bf16_strided"  params = {B, H, Sq, Sk, D, causal, f32 bits of scale, element offsets
+ *                     of q k v o into their buffers (4), (batch, head, row) element strides of
+ *                     q k v o (12)}                                  buffers = {o, q, k, v}
  * Buffer order follows the reference's PARAM numbering: outputs first. */
 int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_program** out);
 
@@ -399,6 +402,16 @@ int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void*
  * Causal rule of the reference: key j is visible to query i iff j <= i (transformer.rs:103-109). */
 int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
                                 int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal);
+/* The same over operands given as views of larger buffers, the way the reference's movement
+ * ops hand them over without a copy (tensor/src/transformer.rs:78-137 takes any view; permute /
+ * shrink / expand never move data there): strides = (batch, head, row) element strides of q, k,
+ * v and o, 12 values; the D elements of a row are contiguous.  All strides are non-negative
+ * multiples of 8 elements and the pointers 16-byte aligned; a zero batch or head stride of k / v
+ * shares one set of keys between batches or heads; output rows, heads and batches must not
+ * overlap.  (rows - 1) * row stride * 2 bytes must stay below 4 GiB per operand. */
+int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
+                                        int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal,
+                                        const int64_t* strides);
 
 /* =====================================================================================
  * Synthetic inputs for benchmarks (no counterpart in the reference, whose tensor API has no

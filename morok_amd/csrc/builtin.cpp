@@ -108,6 +108,30 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
+    if (k == "flash_fwd_bf16_strided") {
+        // params: B, H, Sq, Sk, D, causal, scale bits, element offsets of q k v o into their
+        // buffers (4), then (batch, head, row) element strides of q k v o (12)
+        MRK_TRY(need(23));
+        if (p[0] < 0 || p[1] < 0 || p[2] < 0 || p[3] <= 0 || p[4] != 128)
+            return fail(kInvalidArgument, "flash_fwd_bf16_strided: bad shape (params B, H, Sq, Sk, D=128, causal, scale bits, 4 offsets, 12 strides)");
+        for (int i = 7; i < 23; i++)
+            if (p[i] < 0 || p[i] % 8) return fail(kInvalidArgument, "flash_fwd_bf16_strided: offsets and strides must be non-negative multiples of 8 elements");
+        std::string name = "flash_fwd_bf16_strided_" + std::to_string(p[0] * p[1]) + "_" + std::to_string(p[2]) + "_" + std::to_string(p[3]);
+        out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
+                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          uint32_t bits = static_cast<uint32_t>(q[6]);
+                                          float scale;
+                                          std::memcpy(&scale, &bits, 4);
+                                          long strides[12];
+                                          for (int i = 0; i < 12; i++) strides[i] = static_cast<long>(q[11 + i]);
+                                          auto at = [&](int buf, int which) {
+                                              return static_cast<char*>(b[buf]) + q[7 + which] * 2;
+                                          };
+                                          return launch_flash_fwd_bf16_strided(s, at(1, 0), at(2, 1), at(3, 2), at(0, 3), q[0], q[1],
+                                                                               q[2], q[3], q[4], scale, q[5] != 0, strides);
+                                      }));
+        return kOk;
+    }
     return fail(kInvalidArgument, "unknown builtin kernel kind: " + k);
 }
 

@@ -840,6 +840,36 @@ int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, con
     return kOk;
 }
 
+int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
+                                        int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal,
+                                        const int64_t* strides) {
+    if (batch < 0 || heads < 0 || sq < 0 || sk < 0) return fail(kInvalidArgument, "flash_attn_fwd_strided: negative shape");
+    if (batch == 0 || heads == 0 || sq == 0) return kOk;
+    if (d != 128) return failf(kInvalidArgument, "flash_attn_fwd_strided: head_dim %lld is not supported (128 only)", (long long)d);
+    if (sk == 0) return fail(kInvalidArgument, "flash_attn_fwd_strided: empty key sequence (softmax over no keys is undefined)");
+    if (!(scale > 0.0f)) return fail(kInvalidArgument, "flash_attn_fwd_strided: scale must be positive");
+    MRK_NONNULL(q);
+    MRK_NONNULL(k);
+    MRK_NONNULL(v);
+    MRK_NONNULL(o);
+    MRK_NONNULL(strides);
+    long st[12];
+    for (int i = 0; i < 12; i++) {
+        if (strides[i] < 0 || strides[i] % 8)
+            return failf(kInvalidArgument, "flash_attn_fwd_strided: stride %d (%lld) must be a non-negative multiple of 8 elements", i,
+                         (long long)strides[i]);
+        st[i] = static_cast<long>(strides[i]);
+    }
+    if (st[11] < 128 || (heads > 1 && st[10] == 0) || (batch > 1 && st[9] == 0))
+        return fail(kInvalidArgument, "flash_attn_fwd_strided: output rows, heads and batches must not overlap");
+    std::shared_ptr<Device> dv;
+    MRK_TRY(get_device(device_id, &dv));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_flash_fwd_bf16_strided(dv->allocator->stream(), q, k, v, o, batch, heads, sq, sk, d, scale, causal ? 1 : 0, st),
+            "flash_attn_fwd_strided launch");
+    return kOk;
+}
+
 int mrk_hip_fill(int device_id, void* out, size_t n, int dtype, int mode, uint64_t seed, uint64_t tensor_id, float a,
                  float b) {
     if (n == 0) return kOk;

@@ -51,9 +51,23 @@ __device__ __forceinline__ float max_with_other_half(float x) {
     return fmaxf(a, b);
 }
 
-__global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
-                                                         const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
-                                                         int Sq, int Sk, float scale_log2e, int causal, int q_tiles, int units) {
+// Where the rows of one (batch, head) lie, in elements: the first row of head h of batch b is
+// at b * batch + h * head, consecutive rows are `row` apart, the 128 elements of a row are
+// contiguous.  With these a caller hands over views (a slice of a fused QKV product, a
+// [batch, seq, heads, dim] activation) without copying them into [batch, heads, seq, dim].
+struct RowLayout {
+    long long batch, head;
+    unsigned row_bytes;
+};
+struct FlashLayout {
+    RowLayout q, k, v, o;
+    int heads;
+};
+
+template <bool kStrided>
+__device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
+                                               const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH, int Sq, int Sk,
+                                               float scale_log2e, int causal, int q_tiles, int units, const FlashLayout& lay) {
     __shared__ __attribute__((aligned(1024))) char smem[4 * kTile];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // Workgroup ids congruent mod 8 run on the same XCD and share its L2.  Each XCD walks
@@ -76,10 +90,25 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
         }
     }
     const int lq = lane & 31, lg = lane >> 5;
-    const __bf16* Qh = Q + (size_t)bh * Sq * kD;
-    const char* Kh = reinterpret_cast<const char*>(K + (size_t)bh * Sk * kD);
-    const char* Vh = reinterpret_cast<const char*>(V + (size_t)bh * Sk * kD);
-    __bf16* Oh = O + (size_t)bh * Sq * kD;
+    const __bf16 *Qh, *Kh_, *Vh_;
+    __bf16* Oh;
+    unsigned q_row, k_row, v_row, o_row;  // bytes between consecutive rows
+    if constexpr (kStrided) {
+        const int bb = bh / lay.heads, hh = bh - bb * lay.heads;
+        Qh = Q + bb * lay.q.batch + hh * lay.q.head;
+        Kh_ = K + bb * lay.k.batch + hh * lay.k.head;
+        Vh_ = V + bb * lay.v.batch + hh * lay.v.head;
+        Oh = O + bb * lay.o.batch + hh * lay.o.head;
+        q_row = lay.q.row_bytes, k_row = lay.k.row_bytes, v_row = lay.v.row_bytes, o_row = lay.o.row_bytes;
+    } else {
+        Qh = Q + (size_t)bh * Sq * kD;
+        Kh_ = K + (size_t)bh * Sk * kD;
+        Vh_ = V + (size_t)bh * Sk * kD;
+        Oh = O + (size_t)bh * Sq * kD;
+        q_row = k_row = v_row = o_row = kRow;
+    }
+    const char* Kh = reinterpret_cast<const char*>(Kh_);
+    const char* Vh = reinterpret_cast<const char*>(Vh_);
     const int first_qt = causal ? q_tiles - 1 - unit : unit;
     const int npass = (causal && unit != first_qt) ? 2 : 1;
     // key tiles a query tile visits
@@ -119,7 +148,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
             // 16 B chunk c16 of the LDS row holds logical chunk c16 ^ (row & 15): the LDS
             // serves 16 lanes x 16 B per cycle over 64 banks, so 16 consecutive rows must
             // land in 16 different chunk slots
-            const unsigned kvoff = (unsigned)key * kRow + ((c16 ^ (row & 15)) << 4);
+            const unsigned kvoff = (unsigned)key * k_row + ((c16 ^ (row & 15)) << 4);
             dma(lds_base + stage * kTile + (wave * 16 + c * 4) * kRow, kvoff, Kh);
         }
     };
@@ -130,7 +159,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
             int key = j * kKT + row;
             key = key < Sk ? key : Sk - 1;
             // 32 B granule (c16 >> 1) holds logical granule (c16 >> 1) ^ (row & 3)
-            const unsigned vvoff = (unsigned)key * kRow + (((((c16 >> 1) ^ (row & 3)) << 1) | (c16 & 1)) << 4);
+            const unsigned vvoff = (unsigned)key * v_row + (((((c16 >> 1) ^ (row & 3)) << 1) | (c16 & 1)) << 4);
             dma(lds_base + 2 * kTile + stage * kTile + (wave * 16 + c * 4) * kRow, vvoff, Vh);
         }
     };
@@ -154,7 +183,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
     {
         int qrow = qw0 + lq;
         qrow = qrow < Sq ? qrow : Sq - 1;
-        const __bf16* qp = Qh + (size_t)qrow * kD + 8 * lg;
+        const __bf16* qp = Qh + (size_t)qrow * (q_row / 2) + 8 * lg;
 #pragma unroll
         for (int ds = 0; ds < 8; ds++) qf[ds] = *reinterpret_cast<const bf16x8*>(qp + 16 * ds);
         // Make the compiler wait for these loads here, before the loop: inside the loop the
@@ -396,7 +425,7 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
     const float inv = 1.0f / l_tot;
     const int qrow = qw0 + lq;
     if (qrow < Sq) {
-        __bf16* op = Oh + (size_t)qrow * kD + 4 * lg;
+        __bf16* op = Oh + (size_t)qrow * (o_row / 2) + 4 * lg;
 #pragma unroll
         for (int db = 0; db < 4; db++)
 #pragma unroll
@@ -406,6 +435,19 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restric
             }
     }
     }  // pass
+}
+
+__global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
+                                                         const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
+                                                         int Sq, int Sk, float scale_log2e, int causal, int q_tiles, int units) {
+    flash_fwd_body<false>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, FlashLayout{});
+}
+
+__global__ __launch_bounds__(256, 2) void flash_fwd_d128_strided(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
+                                                                 const __bf16* __restrict__ V, __bf16* __restrict__ O,
+                                                                 int BH, int Sq, int Sk, float scale_log2e, int causal,
+                                                                 int q_tiles, int units, FlashLayout lay) {
+    flash_fwd_body<true>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, lay);
 }
 
 }  // namespace mrk::dev
@@ -427,6 +469,49 @@ int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void
     flash_fwd_d128<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
         static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles, (int)units);
+    return (int)hipGetLastError();
+}
+
+int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq,
+                                  long Sk, long D, float scale, int causal, const long* strides) {
+    using namespace mrk::dev;
+    if (B < 0 || H < 0 || !strides) return (int)hipErrorInvalidValue;
+    const long BH = B * H;
+    if (BH == 0 || Sq <= 0) return 0;
+    if (D != kD || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
+    if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
+    // strides: (batch, head, row) of q, k, v, o in elements.  Rows are read and written in
+    // 16-byte pieces from 16-byte aligned addresses; row offsets inside a head are 32-bit
+    const void* ptrs[4] = {q, k, v, o};
+    const long rows[4] = {Sq, Sk, Sk, Sq};
+    bool dense = true;
+    for (int t = 0; t < 4; t++) {
+        const long sb = strides[3 * t], sh = strides[3 * t + 1], sr = strides[3 * t + 2];
+        if (sb < 0 || sh < 0 || sr < 0 || sb % 8 || sh % 8 || sr % 8) return (int)hipErrorInvalidValue;
+        if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16) return (int)hipErrorInvalidValue;
+        if (sr > (1L << 30) || (rows[t] - 1) * sr * 2 + kRow > 0xffffffffL) return (int)hipErrorInvalidValue;
+        // the output must not alias itself: distinct rows, heads and batches at distinct places
+        if (t == 3 && (sr < kD || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
+        dense = dense && sr == kD && sh == rows[t] * kD && sb == H * rows[t] * kD;
+    }
+    if (dense) return launch_flash_fwd_bf16(stream, q, k, v, o, BH, Sq, Sk, D, scale, causal);
+    const long q_tiles = (Sq + kQT - 1) / kQT;
+    const long units = causal ? (q_tiles + 1) / 2 : q_tiles;
+    const long blocks = BH * units;
+    if (blocks > 0x7fffffffL) return (int)hipErrorInvalidValue;
+    FlashLayout lay;
+    RowLayout* rl[4] = {&lay.q, &lay.k, &lay.v, &lay.o};
+    for (int t = 0; t < 4; t++) {
+        rl[t]->batch = strides[3 * t];
+        rl[t]->head = strides[3 * t + 1];
+        rl[t]->row_bytes = (unsigned)(strides[3 * t + 2] * 2);
+    }
+    lay.heads = (int)H;
+    (void)hipGetLastError();
+    const float scale_log2e = scale * 1.4426950408889634f;
+    flash_fwd_d128_strided<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
+        static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles, (int)units, lay);
     return (int)hipGetLastError();
 }
 

@@ -27,6 +27,12 @@ size_t gemm_bf16_workspace_bytes(long M, long N, long K, long batch);
 // scale > 0.  Causal: key j visible to query i iff j <= i.
 int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
                           long D, float scale, int causal);
+// The same kernel over operands given as views: strides holds (batch, head, row) element
+// strides of q, k, v and o, in that order (12 values); the 128 elements of a row are
+// contiguous.  Strides must be multiples of 8 elements and the pointers 16-byte aligned;
+// zero batch / head strides broadcast an input.  Dense strides take the kernel above.
+int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq,
+                                  long Sk, long D, float scale, int causal, const long* strides);
 
 // Synthetic benchmark inputs. dtype 0 = f32, 1 = bf16; mode 0 = uniform [a, b), 1 = normal(0, a).
 int launch_fill(void* stream, void* out, size_t n, int dtype, int mode, unsigned long long seed,

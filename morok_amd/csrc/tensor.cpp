@@ -799,11 +799,111 @@ Coords plain(const std::vector<uint32_t>& nodes) {
     return c;
 }
 
+// ---- strided views.  A chain of movement ops over data in memory is an offset plus one
+// stride per axis whenever no reshape in it splits or merges axes that are not contiguous
+// with each other; the hand-written attention kernel reads and writes such views in place.
+static std::vector<int64_t> dense_strides(const std::vector<int64_t>& shape) {
+    std::vector<int64_t> st(shape.size(), 1);
+    for (size_t i = shape.size(); i-- > 1;) st[i - 1] = st[i] * shape[i];
+    return st;
+}
+
+// Strides of the same memory seen through `to` instead of `from` (equal element counts, no
+// zero extents); false when the reshape would need a copy.
+static bool reshape_strides(const std::vector<int64_t>& from, const std::vector<int64_t>& from_st, const std::vector<int64_t>& to,
+                            std::vector<int64_t>* to_st) {
+    std::vector<int64_t> od, os;  // extents of 1 carry no stride
+    for (size_t i = 0; i < from.size(); i++)
+        if (from[i] != 1) od.push_back(from[i]), os.push_back(from_st[i]);
+    to_st->assign(to.size(), 0);
+    size_t oi = 0, ni = 0;
+    while (ni < to.size()) {
+        if (to[ni] == 1) {
+            ni++;
+            continue;
+        }
+        if (oi >= od.size()) return false;
+        // smallest groups of axes on both sides with equal products
+        size_t oj = oi + 1, nj = ni + 1;
+        int64_t op = od[oi], np = to[ni];
+        while (op != np) {
+            if (np < op) {
+                if (nj >= to.size()) return false;
+                np *= to[nj++];
+            } else {
+                if (oj >= od.size()) return false;
+                op *= od[oj++];
+            }
+        }
+        for (size_t k = oi; k + 1 < oj; k++)
+            if (os[k] != od[k + 1] * os[k + 1]) return false;  // the old group is not one run of memory
+        int64_t st = os[oj - 1];
+        for (size_t k = nj; k-- > ni;) {
+            (*to_st)[k] = to[k] == 1 ? 0 : st;
+            st *= to[k];
+        }
+        oi = oj;
+        ni = nj;
+    }
+    return oi == od.size();
+}
+
+struct StridedView {
+    TensorNode* base = nullptr;  // in memory, or to be materialised
+    int64_t offset = 0;          // elements
+    std::vector<int64_t> strides;
+};
+
+static bool strided_view(TensorNode* n, StridedView* v) {
+    const bool movement = n->kind == TKind::Reshape || n->kind == TKind::Permute || n->kind == TKind::Expand || n->kind == TKind::Shrink;
+    if (n->buffer || !movement) {
+        v->base = n;
+        v->offset = 0;
+        v->strides = dense_strides(n->shape);
+        return true;
+    }
+    StridedView c;
+    TensorNode* s = n->src[0].get();
+    if (n->numel() == 0 || !strided_view(s, &c)) return false;
+    v->base = c.base;
+    v->offset = c.offset;
+    v->strides.assign(n->shape.size(), 0);
+    switch (n->kind) {
+        case TKind::Permute:
+            for (size_t i = 0; i < n->shape.size(); i++) v->strides[i] = c.strides[n->arg[i]];
+            return true;
+        case TKind::Expand:
+            for (size_t i = 0; i < n->shape.size(); i++) v->strides[i] = s->shape[i] == n->shape[i] ? c.strides[i] : 0;
+            return true;
+        case TKind::Shrink:
+            for (size_t i = 0; i < n->shape.size(); i++) {
+                v->offset += n->arg[i] * c.strides[i];
+                v->strides[i] = c.strides[i];
+            }
+            return true;
+        default: return reshape_strides(s->shape, c.strides, n->shape, &v->strides);
+    }
+}
+
 struct Scheduler {
     std::shared_ptr<Device> dev;
     std::unique_ptr<ExecutionPlan> plan;
     RealizeStats stats;
     std::vector<TensorNode*> produced;  // nodes this realization gave a buffer
+    std::unordered_map<const TensorNode*, int> uses;  // consumers of a node within the realised graph
+
+    void count_uses(const TensorNode* root) {
+        std::vector<const TensorNode*> stack{root};
+        std::set<const TensorNode*> seen{root};
+        while (!stack.empty()) {
+            const TensorNode* n = stack.back();
+            stack.pop_back();
+            for (const TensorRef& c : n->src) {
+                uses[c.get()]++;
+                if (seen.insert(c.get()).second) stack.push_back(c.get());
+            }
+        }
+    }
 
     int add_kernel(const std::shared_ptr<CachedKernel>& k, const std::vector<std::shared_ptr<Buffer>>& bufs, bool cached) {
         std::vector<size_t> idx;
@@ -926,6 +1026,10 @@ struct Scheduler {
     int materialize(TensorNode* n) {
         if (n->buffer) return kOk;
         if (n->numel() > 0 && fusable(n)) return materialize_fused(n);
+        {
+            std::vector<int64_t> out_strides;
+            if (TensorNode* att = attention_under(n, &out_strides)) return materialize_attention(att, n, out_strides);
+        }
         if (generated_tc(n)) return materialize_generated_tc(n);
         // a reshape of materialised data is the same bytes
         if (n->kind == TKind::Reshape) {
@@ -950,7 +1054,96 @@ struct Scheduler {
         return n->kind == TKind::Reduce ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
     }
 
+    // A reshape / permute chain whose only source is a fusable attention node nobody else
+    // reads: the kernel can write that layout itself.  Returns the attention node and the
+    // strides of its [B, H, Sq, D] output inside the chain end's dense buffer.
+    TensorNode* attention_under(TensorNode* n, std::vector<int64_t>* out_strides) const {
+        if (!g_fusion || n->numel() == 0 || (n->kind != TKind::Reshape && n->kind != TKind::Permute)) return nullptr;
+        std::vector<int64_t> st = dense_strides(n->shape);
+        TensorNode* m = n;
+        while (m->kind == TKind::Reshape || m->kind == TKind::Permute) {
+            TensorNode* c = m->src[0].get();
+            if (c->buffer) return nullptr;
+            auto u = uses.find(c);
+            if (u == uses.end() || u->second != 1) return nullptr;
+            std::vector<int64_t> cst(c->shape.size(), 0);
+            if (m->kind == TKind::Permute) {
+                for (size_t i = 0; i < m->shape.size(); i++) cst[m->arg[i]] = st[i];
+            } else if (!reshape_strides(m->shape, st, c->shape, &cst)) {
+                return nullptr;
+            }
+            st = cst;
+            m = c;
+        }
+        if (m->hint != HintKind::Sdpa || !fusable(m)) return nullptr;
+        if (st.size() != 4 || st[3] != 1 || st[0] % 8 || st[1] % 8 || st[2] % 8) return nullptr;
+        if (st[2] > (1LL << 30) || (m->shape[2] - 1) * st[2] * 2 + m->shape[3] * 2 > 0xffffffffLL) return nullptr;
+        *out_strides = st;
+        return m;
+    }
+
+    // The attention kernel over whatever views its operands are: an operand that is a strided
+    // view of data in memory (rows of 128 contiguous elements, 16-byte aligned) is read in
+    // place, anything else is materialised first.  `dst` is the node that receives the buffer,
+    // `out_strides` the layout of the [B, H, Sq, D] result inside it.
+    int materialize_attention(TensorNode* att, TensorNode* dst, const std::vector<int64_t>& out_strides) {
+        const TensorNode* q = att->hint_inputs[0].get();
+        const TensorNode* k = att->hint_inputs[1].get();
+        const int64_t B = q->shape[0], H = q->shape[1], Sq = q->shape[2], Sk = k->shape[2], D = q->shape[3];
+        std::vector<int64_t> params;
+        std::vector<std::shared_ptr<Buffer>> bufs(4);
+        int64_t offsets[4] = {0, 0, 0, 0};
+        std::vector<int64_t> strides;
+        bool dense = true;
+        for (int i = 0; i < 3; i++) {
+            TensorNode* in = att->hint_inputs[i].get();
+            StridedView v;
+            bool ok = !in->buffer && strided_view(in, &v) && v.base != in && v.strides.size() == 4 && v.offset % 8 == 0;
+            // only data that is (or will be) in memory anyway: a view of an unrealised
+            // elementwise expression is cheaper computed over the view alone
+            ok = ok && (v.base->buffer || v.base->kind == TKind::Reduce || v.base->kind == TKind::Contiguous || fusable(v.base));
+            if (ok) {
+                for (int a = 0; a < 4; a++)
+                    if (in->shape[a] == 1) v.strides[a] = 0;
+                const int64_t rows = in->shape[2];
+                ok = (D == 1 || v.strides[3] == 1) && v.strides[0] >= 0 && v.strides[1] >= 0 && v.strides[2] >= 0 &&
+                     v.strides[0] % 8 == 0 && v.strides[1] % 8 == 0 && v.strides[2] % 8 == 0 && v.strides[2] <= (1LL << 30) &&
+                     (rows - 1) * v.strides[2] * 2 + D * 2 <= 0xffffffffLL;
+            }
+            if (ok) {
+                MRK_TRY(materialize(v.base));
+                bufs[i + 1] = v.base->buffer;
+                offsets[i] = v.offset;
+                strides.insert(strides.end(), v.strides.begin(), v.strides.begin() + 3);
+                dense = false;
+            } else {
+                MRK_TRY(materialize(in));
+                bufs[i + 1] = in->buffer;
+                const std::vector<int64_t> ds = dense_strides(in->shape);
+                strides.insert(strides.end(), ds.begin(), ds.begin() + 3);
+            }
+        }
+        strides.insert(strides.end(), out_strides.begin(), out_strides.begin() + 3);
+        dense = dense && out_strides == dense_strides(att->shape);
+        auto out = new_buffer(dst);
+        bufs[0] = out;
+        float scale = static_cast<float>(att->hint_scale);
+        uint32_t bits;
+        std::memcpy(&bits, &scale, 4);
+        if (dense) {
+            MRK_TRY(builtin("flash_fwd_bf16", {B * H, Sq, Sk, D, att->hint_causal ? 1 : 0, static_cast<int64_t>(bits)}, bufs));
+        } else {
+            params = {B, H, Sq, Sk, D, att->hint_causal ? 1 : 0, static_cast<int64_t>(bits), offsets[0], offsets[1], offsets[2], 0};
+            params.insert(params.end(), strides.begin(), strides.end());
+            MRK_TRY(builtin("flash_fwd_bf16_strided", params, bufs));
+        }
+        dst->buffer = out;
+        produced.push_back(dst);
+        return kOk;
+    }
+
     int materialize_fused(TensorNode* n) {
+        if (n->hint == HintKind::Sdpa) return materialize_attention(n, n, dense_strides(n->shape));
         for (const TensorRef& in : n->hint_inputs) MRK_TRY(materialize(in.get()));
         auto out = new_buffer(n);
         int rc = kOk;
@@ -987,16 +1180,6 @@ struct Scheduler {
                 MRK_TRY(get_or_compile_linear_kernel(*dev, k, name.c_str(), &ck, &cached));
                 rc = add_kernel(ck, {out, a->buffer, w->buffer}, cached);
             }
-        } else if (n->hint == HintKind::Sdpa) {
-            const TensorNode* q = n->hint_inputs[0].get();
-            const TensorNode* k = n->hint_inputs[1].get();
-            float scale = static_cast<float>(n->hint_scale);
-            uint32_t bits;
-            std::memcpy(&bits, &scale, 4);
-            rc = builtin("flash_fwd_bf16",
-                         {q->shape[0] * q->shape[1], q->shape[2], k->shape[2], q->shape[3], n->hint_causal ? 1 : 0,
-                          static_cast<int64_t>(bits)},
-                         {out, q->buffer, k->buffer, n->hint_inputs[2]->buffer});
         }
         MRK_TRY(rc);
         n->buffer = out;
@@ -1203,6 +1386,7 @@ int Tensor::prepare(std::unique_ptr<ExecutionPlan>* out) const {
     Scheduler s;
     MRK_TRY(DeviceFactoryRegistry::global().device("HIP", n_->device_id, &s.dev));
     s.plan.reset(new ExecutionPlan(n_->device_id));
+    s.count_uses(n_.get());
     if (!n_->buffer) MRK_TRY(s.materialize(n_.get()));
     s.plan->set_outputs({s.plan->add_buffer(n_->buffer)});
     // Intermediates share blocks by liveness (tensor/src/memory_planner.rs); their contents do

@@ -43,6 +43,29 @@ def flash_attn_fwd_bf16(q, k, v, o, batch, heads, sq, sk, d, scale, causal=True,
                                           int(causal)))
 
 
+def flash_attn_fwd_bf16_strided(q, k, v, o, batch, heads, sq, sk, d, scale, strides, offsets=(0, 0, 0, 0), causal=True,
+                                device_id=0):
+    """The fused SDPA forward over views: `strides` = (batch, head, row) element strides of q, k,
+    v, o (12 values), `offsets` = element offset of each operand's first element inside its
+    buffer.  Each Buffer must hold the last element its view reaches."""
+    strides = [int(x) for x in strides]
+    if len(strides) != 12 or len(offsets) != 4:
+        raise ValueError("flash_attn_fwd_bf16_strided takes 12 strides and 4 offsets")
+    ptrs = []
+    for i, (b, rows, what) in enumerate(((q, sq, "attention Q"), (k, sk, "attention K"), (v, sk, "attention V"),
+                                         (o, sq, "attention O"))):
+        sb, sh, sr = strides[3 * i:3 * i + 3]
+        off = int(offsets[i])
+        if off < 0 or off % 8:
+            raise ValueError(f"{what}: offset {off} must be a non-negative multiple of 8 elements")
+        if batch and heads and rows:
+            _need(b, (off + (batch - 1) * sb + (heads - 1) * sh + (rows - 1) * sr + d) * 2, what)
+        ptrs.append(C.c_void_p((b.ptr if isinstance(b, Buffer) else int(b)) + off * 2))
+    arr = (C.c_int64 * 12)(*strides)
+    check(lib.mrk_hip_flash_attn_fwd_bf16_strided(device_id, ptrs[0], ptrs[1], ptrs[2], ptrs[3], batch, heads, sq, sk, d,
+                                                  scale, int(causal), arr))
+
+
 def fill_normal(buf, n, sigma=1.0, seed=0, tensor_id=0, bf16=False, device_id=0):
     """Device-side synthetic normal(0, sigma) values (benchmark inputs)."""
     _need(buf, n * (2 if bf16 else 4), "fill")

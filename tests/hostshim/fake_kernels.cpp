@@ -18,6 +18,11 @@ int launch_flash_fwd_bf16(void* stream, const void*, const void*, const void*, v
     mrk_shim_note_launch(stream, "flash_fwd_bf16");
     return 0;
 }
+int launch_flash_fwd_bf16_strided(void* stream, const void*, const void*, const void*, void*, long, long, long, long, long, float,
+                                  int, const long*) {
+    mrk_shim_note_launch(stream, "flash_fwd_bf16_strided");
+    return 0;
+}
 int launch_fill(void* stream, void*, size_t, int, int, unsigned long long, unsigned long long, float, float) {
     mrk_shim_note_launch(stream, "fill");
     return 0;

@@ -166,3 +166,93 @@ def test_flash_random_shapes(dev, oracle, seed):
     scale = float(rng.choice([SCALE, 0.05, 0.2]))
     q, k, v = _inputs(B, H, Sq, Sk, seed=40 + seed)
     _check(_attn(dev, q, k, v, scale, causal), oracle.sdpa_bf16(q, k, v, scale, causal=causal))
+
+
+# ---------------------------------------------------------------- operands given as views
+def _strided(dev, bufs, offsets, strides, B, H, Sq, Sk, causal, o_init=None, via_program=False):
+    """Runs the strided entry point on host arrays `bufs` = (q, k, v, o-shaped uint16 arrays of
+    whatever layout) and returns the output buffer's contents in its own layout."""
+    bq, bk, bv = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in bufs[:3])
+    o_host = bufs[3] if o_init is None else o_init
+    bo = morok_amd.Buffer.from_numpy(o_host, dev.device_id)
+    if via_program:
+        bits = int(np.float32(SCALE).view(np.uint32))
+        prog = morok_amd.Program.builtin("flash_fwd_bf16_strided",
+                                         [B, H, Sq, Sk, D, int(causal), bits, *offsets, *strides], dev.device_id)
+        prog.execute([bo, bq, bk, bv])
+    else:
+        ops.flash_attn_fwd_bf16_strided(bq, bk, bv, bo, B, H, Sq, Sk, D, SCALE, strides, offsets, causal, dev.device_id)
+    return bo.copyout(np.uint16, o_host.shape)
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 200, 200), (1, 4, 129, 257), (2, 2, 384, 384)])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("via_program", [False, True])
+def test_flash_over_seq_major_views(dev, oracle, shape, causal, via_program):
+    """All four operands as [B, S, H, D] activations (what a projection writes), the kernel
+    told so through strides: the same bits as the kernel over [B, H, S, D] copies, and the
+    oracle's values."""
+    B, H, Sq, Sk = shape
+    q, k, v = _inputs(B, H, Sq, Sk, seed=31)
+    qs, ks, vs = (np.ascontiguousarray(t.transpose(0, 2, 1, 3)) for t in (q, k, v))
+    strides = [Sq * H * D, D, H * D, Sk * H * D, D, H * D, Sk * H * D, D, H * D, Sq * H * D, D, H * D]
+    o = _strided(dev, (qs, ks, vs, np.zeros_like(qs)), [0, 0, 0, 0], strides, B, H, Sq, Sk, causal, via_program=via_program)
+    o = o.transpose(0, 2, 1, 3)
+    assert np.array_equal(o, _attn(dev, q, k, v, SCALE, causal))
+    _check(o, oracle.sdpa_bf16(q, k, v, SCALE, causal=causal))
+
+
+def test_flash_over_a_packed_qkv_product(dev):
+    """q, k and v as column slices of one [B*S, 3*H*D] matrix (a fused QKV projection), the
+    output as a column slice of a wider matrix whose other columns must stay as they were."""
+    B, H, S = 2, 4, 320
+    q, k, v = _inputs(B, H, S, S, seed=32)
+    hid = H * D
+    packed = np.zeros((B, S, 3 * hid), np.uint16)
+    for i, t in enumerate((q, k, v)):
+        packed[:, :, i * hid:(i + 1) * hid] = t.transpose(0, 2, 1, 3).reshape(B, S, hid)
+    wide = np.full((B, S, hid + 64), 0x7FC0, np.uint16)  # bf16 NaN pattern: writes outside the view would show
+    st_in = [S * 3 * hid, D, 3 * hid]
+    strides = st_in * 3 + [S * (hid + 64), D, hid + 64]
+    o = _strided(dev, (packed, packed, packed, None), [0, hid, 2 * hid, 32], strides, B, H, S, S, True, o_init=wide)
+    assert np.all(o[:, :, :32] == 0x7FC0) and np.all(o[:, :, 32 + hid:] == 0x7FC0)
+    got = o[:, :, 32:32 + hid].reshape(B, S, H, D).transpose(0, 2, 1, 3)
+    assert np.array_equal(got, _attn(dev, q, k, v, SCALE, True))
+
+
+def test_flash_shared_keys_through_zero_strides(dev, oracle):
+    """One set of keys and values for every head (head stride 0) and for every batch (batch
+    stride 0): the same as the kernel over broadcast copies."""
+    B, H, Sq, Sk = 2, 3, 150, 260
+    q, _, _ = _inputs(B, H, Sq, Sk, seed=33)
+    k1 = synth.normal_bf16((1, 1, Sk, D), 33, 1)
+    v1 = synth.normal_bf16((1, 1, Sk, D), 33, 2)
+    strides = [H * Sq * D, Sq * D, D, 0, 0, D, 0, 0, D, H * Sq * D, Sq * D, D]
+    o = _strided(dev, (q, k1, v1, np.zeros_like(q)), [0, 0, 0, 0], strides, B, H, Sq, Sk, False)
+    kb, vb = (np.ascontiguousarray(np.broadcast_to(t, (B, H, Sk, D))) for t in (k1, v1))
+    assert np.array_equal(o, _attn(dev, q, kb, vb, SCALE, False))
+    _check(o, oracle.sdpa_bf16(q, kb, vb, SCALE, causal=False))
+
+
+def test_flash_dense_strides_take_the_plain_kernel(dev):
+    B, H, S = 1, 2, 256
+    q, k, v = _inputs(B, H, S, S, seed=34)
+    strides = [H * S * D, S * D, D] * 4
+    o = _strided(dev, (q, k, v, np.zeros_like(q)), [0, 0, 0, 0], strides, B, H, S, S, True)
+    assert np.array_equal(o, _attn(dev, q, k, v, SCALE, True))
+
+
+def test_flash_strided_refuses_what_it_cannot_address(dev):
+    B, H, S = 1, 2, 64
+    q, k, v = _inputs(B, H, S, S, seed=35)
+    good = [H * S * D, S * D, D] * 4
+    bufs = (q, k, v, np.zeros_like(q))
+    for i, bad in ((2, D + 4), (1, S * D + 1), (11, 64), (10, 0)):  # unaligned row / head stride, overlapping output rows / heads
+        st = list(good)
+        st[i] = bad
+        with pytest.raises((MorokHipError, ValueError)):
+            _strided(dev, bufs, [0, 0, 0, 0], st, B, H, S, S, True)
+    with pytest.raises((MorokHipError, ValueError)):  # unaligned offset
+        _strided(dev, bufs, [4, 0, 0, 0], good, B, H, S, S, True)
+    with pytest.raises(ValueError):  # the view reaches past the buffer
+        _strided(dev, bufs, [0, 0, 0, 0], [H * S * D, S * D, 2 * D] + good[3:], B, H, S, S, True)

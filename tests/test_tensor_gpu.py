@@ -287,6 +287,93 @@ def test_sdpa_bf16_uses_flash(T, oracle):
     assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
 
 
+def test_sdpa_bf16_reads_and_writes_views_in_place(T, oracle):
+    """q / k / v as column slices of one packed [B*S, 3*H*D] buffer seen as [B, H, S, D], the
+    result permuted back to [B*S, H*D]: one attention kernel and no copy kernels, and the bits
+    of the attention over dense copies of the same operands."""
+    from morok_amd import synth, uop
+
+    B, H, S, D = 2, 3, 192, 128
+    hid = H * D
+    packed = synth.normal_bf16((B * S, 3 * hid), 41, 0)
+    pt = T.Tensor.from_numpy(packed, uop.BF16)
+
+    def head_view(t, i):
+        return (t.try_shrink([(0, B * S), (i * hid, (i + 1) * hid)]).try_reshape([B, S, H, D]).try_permute([0, 2, 1, 3]))
+
+    q, k, v = (head_view(pt, i) for i in range(3))
+    out = q.scaled_dot_product_attention(k, v, is_causal=True).try_permute([0, 2, 1, 3]).try_reshape([B * S, hid])
+    got = out.to_numpy()
+    assert out.kernels() == [f"flash_fwd_bf16_strided_{B * H}_{S}_{S}"]
+    qn, kn, vn = (np.ascontiguousarray(packed[:, i * hid:(i + 1) * hid].reshape(B, S, H, D).transpose(0, 2, 1, 3))
+                  for i in range(3))
+    dense = T.Tensor.from_numpy(qn, uop.BF16).scaled_dot_product_attention(
+        T.Tensor.from_numpy(kn, uop.BF16), T.Tensor.from_numpy(vn, uop.BF16), is_causal=True)
+    want = dense.to_numpy()
+    assert dense.kernels()[0].startswith("flash_fwd_bf16_") and "strided" not in dense.kernels()[0]
+    assert np.array_equal(got.reshape(B, S, H, D).transpose(0, 2, 1, 3), want)
+    ref = synth.from_bf16(oracle.sdpa_bf16(qn, kn, vn, 1 / np.sqrt(D), True))
+    assert np.abs(synth.from_bf16(want) - ref).max() <= 2e-2 * np.abs(ref).max()
+
+
+def test_sdpa_bf16_shared_keys_by_expand(T):
+    """Keys and values of one head expanded over all heads: read through zero strides."""
+    from morok_amd import synth, uop
+
+    B, H, S, D = 1, 4, 160, 128
+    q = synth.normal_bf16((B, H, S, D), 42, 0)
+    k1, v1 = synth.normal_bf16((B, 1, S, D), 42, 1), synth.normal_bf16((B, 1, S, D), 42, 2)
+    kt = T.Tensor.from_numpy(k1, uop.BF16).try_expand([B, H, S, D])
+    vt = T.Tensor.from_numpy(v1, uop.BF16).try_expand([B, H, S, D])
+    t = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(kt, vt, is_causal=False)
+    got = t.to_numpy()
+    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("flash_fwd_bf16_strided")
+    kb, vb = (np.ascontiguousarray(np.broadcast_to(x, (B, H, S, D))) for x in (k1, v1))
+    want = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(
+        T.Tensor.from_numpy(kb, uop.BF16), T.Tensor.from_numpy(vb, uop.BF16), is_causal=False).to_numpy()
+    assert np.array_equal(got, want)
+
+
+def test_sdpa_bf16_views_the_kernel_cannot_take_are_copied(T):
+    """A view with an unaligned offset, a transposed head dimension, an attention result with
+    two readers, and a view of an unrealised elementwise expression: each falls back to dense
+    copies (or the dense layout) and gives the same values."""
+    from morok_amd import synth, uop
+
+    B, H, S, D = 1, 2, 128, 128
+    big = synth.normal_bf16((B, H, S + 1, D + 4), 43, 0)
+    bt = T.Tensor.from_numpy(big, uop.BF16)
+    q = synth.normal_bf16((B, H, S, D), 43, 1)
+    qt = T.Tensor.from_numpy(q, uop.BF16)
+    kv = bt.try_shrink([(0, B), (0, H), (1, S + 1), (4, D + 4)])                 # offset 4 mod 8, row stride 132
+    t = qt.scaled_dot_product_attention(kv, kv, is_causal=True)
+    got = t.to_numpy()
+    assert sum(k.startswith("flash_fwd_bf16_") for k in t.kernels()) == 1 and not any("strided" in k for k in t.kernels())
+    kn = np.ascontiguousarray(big[:, :, 1:, 4:])
+    want = qt.scaled_dot_product_attention(T.Tensor.from_numpy(kn, uop.BF16), T.Tensor.from_numpy(kn, uop.BF16),
+                                           is_causal=True).to_numpy()
+    assert np.array_equal(got, want)
+    # head dimension not innermost
+    kT = T.Tensor.from_numpy(np.ascontiguousarray(kn.transpose(0, 1, 3, 2)), uop.BF16).try_permute([0, 1, 3, 2])
+    t2 = qt.scaled_dot_product_attention(kT, kT, is_causal=True)
+    assert np.array_equal(t2.to_numpy(), want) and not any("strided" in k for k in t2.kernels())
+    # two readers of the attention result: it is kept in its own layout
+    a = qt.scaled_dot_product_attention(T.Tensor.from_numpy(kn, uop.BF16), T.Tensor.from_numpy(kn, uop.BF16), is_causal=True)
+    both = a.try_permute([0, 2, 1, 3]).try_reshape([B * S, H * D]).try_add(a.try_reshape([B * S, H * D]))
+    gb = synth.from_bf16(both.to_numpy())
+    assert not any("strided" in k for k in both.kernels())
+    wf = synth.from_bf16(want)
+    exp = wf.transpose(0, 2, 1, 3).reshape(B * S, H * D) + wf.reshape(B * S, H * D)
+    assert np.abs(gb - exp).max() <= 1e-2 * np.abs(exp).max()
+    # a slice of an elementwise expression is computed over the slice, not over its base
+    e = bt.try_mul(1.0).try_shrink([(0, B), (0, H), (0, S), (0, D)])
+    t3 = qt.scaled_dot_product_attention(e, e, is_causal=True)
+    kn3 = np.ascontiguousarray(big[:, :, :S, :D])
+    want3 = qt.scaled_dot_product_attention(T.Tensor.from_numpy(kn3, uop.BF16), T.Tensor.from_numpy(kn3, uop.BF16),
+                                            is_causal=True).to_numpy()
+    assert np.array_equal(t3.to_numpy(), want3) and not any("strided" in k for k in t3.kernels())
+
+
 def test_silu_and_sigmoid(T, oracle):
     rng = np.random.default_rng(31)
     x = (rng.standard_normal(5000) * 4).astype(np.float32)
