@@ -338,6 +338,12 @@ int mrk_hip_sched_build_wmma_matmul(int tc_index, int64_t m, int64_t n, int64_t 
  * (schedule/src/optimizer/heuristics.rs:37-82) applied after the tensor-core rewrite. */
 int mrk_hip_sched_build_wmma_matmul_lds(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, uint8_t** kernel,
                                         size_t* len);
+/* The same with the choices explicit: opts = {waves_m, waves_n (LOCAL: the grid of waves in a
+ * workgroup), tiles_m, tiles_n (UPCAST: 16x16 tensor-core tiles per wave), K steps per barrier
+ * pair (UNROLL; 0 = as many as divide K, up to 64 elements)}.  All powers of two; M, N, K must be
+ * multiples of the resulting workgroup tile; INVALID_ARGUMENT otherwise. */
+int mrk_hip_sched_build_wmma_matmul_lds_opts(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, const int opts[5],
+                                             uint8_t** kernel, size_t* len);
 void mrk_hip_sched_free(void* p);
 /* The f32 matmul kernel with the optimisation choices explicit: opts = {LOCAL x, LOCAL y,
  * UPCAST of N (vector width 1/2/4), UPCAST of M (rows per work-item 1..8), UNROLL of K}.
@@ -366,6 +372,12 @@ int mrk_hip_beam_cache_put(uint64_t ast_hash, int width, const char* device, con
  * cache answered, *timed = number of candidates compiled and timed. */
 int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t k, int width, int opts[5],
                                    double* best_ms, int* from_cache, int* timed);
+/* The same search over the LDS-staged tensor-core matmul of mrk_hip_sched_build_wmma_matmul_lds_opts
+ * (bf16 / f16 in and out, tensor core `tc_index` of mrk_hip_sched_tensor_cores): the TC action
+ * of tc.rs:358-674 first, then LOCAL / UPCAST / UNROLL as above.  opts = {waves_m, waves_n,
+ * tiles_m per wave, tiles_n per wave, K steps per barrier pair}. */
+int mrk_hip_beam_search_wmma_matmul(int device_id, int tc_index, int64_t m, int64_t n, int64_t k, int width, int opts[5],
+                                    double* best_ms, int* from_cache, int* timed);
 
 /* =====================================================================================
  * Hand-written kernels, direct entry points (device pointers, queued on the device stream)

@@ -134,6 +134,8 @@ _SIGS = {
                                                   C.POINTER(C.POINTER(C.c_uint8)), c_size_p]),
     "mrk_hip_sched_build_wmma_matmul_lds": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int,
                                                       C.POINTER(C.POINTER(C.c_uint8)), c_size_p]),
+    "mrk_hip_sched_build_wmma_matmul_lds_opts": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int,
+                                                           C.POINTER(C.c_int), C.POINTER(C.POINTER(C.c_uint8)), c_size_p]),
     "mrk_hip_sched_free": (None, [C.c_void_p]),
     "mrk_hip_softmax_f32": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]),
     "mrk_hip_softmax_f32_variant": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int]),
@@ -160,6 +162,8 @@ _SIGS = {
     "mrk_hip_beam_cache_get": (C.c_int, [C.c_uint64, C.c_int, C.c_char_p, C.c_void_p, C.c_size_t, c_size_p]),
     "mrk_hip_beam_cache_put": (C.c_int, [C.c_uint64, C.c_int, C.c_char_p, C.c_void_p, C.c_size_t]),
     "mrk_hip_beam_search_matmul_f32": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_double), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
+    "mrk_hip_beam_search_wmma_matmul": (C.c_int, [C.c_int, C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int, C.POINTER(C.c_int),
+                                                  C.POINTER(C.c_double), C.POINTER(C.c_int), C.POINTER(C.c_int)]),
     "mrk_hip_queue_create": (C.c_int, [C.c_int, C.c_int, c_void_pp]),
     "mrk_hip_queue_wait": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64]),
     "mrk_hip_queue_signal": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint64]),

@@ -11,6 +11,7 @@
 #include <thread>
 
 #include "schedule.h"
+#include "tensor.h"
 
 #include "error.h"
 #include "uop.h"
@@ -513,6 +514,117 @@ int beam_search_matmul_f32(const Device& dev, int64_t M, int64_t N, int64_t K, i
     if (best_ms) *best_ms = beam[0].first;
     Record r{{best->local_x, best->local_y, best->up_n, best->up_m, best->unroll_k}, beam[0].first};
     (void)BeamCache::put(ast_hash, width, device, &r, sizeof r);  // a read-only cache directory is not an error
+    clear_error();
+    return kOk;
+}
+
+int beam_search_wmma_matmul(const Device& dev, const TensorCore& tc, int tc_index, int64_t M, int64_t N, int64_t K, int width,
+                            WmmaLdsOpts* best, double* best_ms, bool* from_cache, int* candidates_timed) {
+    if (width < 1) return fail(kInvalidArgument, "beam search: width must be >= 1");
+    if (M <= 0 || N <= 0 || K <= 0) return fail(kInvalidArgument, "beam search: empty matmul");
+    const std::string device = "HIP:" + std::to_string(dev.device_id);
+    const std::string id = "wmma_matmul_lds:" + std::to_string(tc_index) + ":" + std::to_string(M) + "x" + std::to_string(N) + "x" +
+                           std::to_string(K);
+    const uint64_t ast_hash = fnv1a64(reinterpret_cast<const uint8_t*>(id.data()), id.size());
+    if (from_cache) *from_cache = false;
+    if (candidates_timed) *candidates_timed = 0;
+    struct Record {
+        int32_t opts[5];
+        double ms;
+    };
+    std::vector<uint8_t> cached;
+    if (BeamCache::get(ast_hash, width, device, &cached) && cached.size() == sizeof(Record)) {
+        Record r;
+        std::memcpy(&r, cached.data(), sizeof r);
+        WmmaLdsOpts o{r.opts[0], r.opts[1], r.opts[2], r.opts[3], r.opts[4]};
+        if (wmma_lds_opts_valid(tc, o, M, N, K)) {
+            *best = o;
+            if (best_ms) *best_ms = r.ms;
+            if (from_cache) *from_cache = true;
+            return kOk;
+        }
+    }
+    const size_t esz = scalar_size(tc.dtype_in);
+    BufferOptions bo;
+    bo.zero_init = true;
+    Buffer a(dev.allocator, static_cast<size_t>(M * K) * esz, bo), b(dev.allocator, static_cast<size_t>(K * N) * esz, bo),
+        c(dev.allocator, static_cast<size_t>(M * N) * esz, bo);
+    MRK_TRY(a.ensure_allocated());
+    MRK_TRY(b.ensure_allocated());
+    MRK_TRY(c.ensure_allocated());
+    void* ptrs[3];
+    MRK_TRY(c.as_raw_ptr(&ptrs[0]));
+    MRK_TRY(a.as_raw_ptr(&ptrs[1]));
+    MRK_TRY(b.as_raw_ptr(&ptrs[2]));
+
+    using Cand = std::pair<double, WmmaLdsOpts>;
+    auto same = [](const WmmaLdsOpts& x, const WmmaLdsOpts& y) {
+        return x.waves_m == y.waves_m && x.waves_n == y.waves_n && x.up_m == y.up_m && x.up_n == y.up_n && x.unroll_k == y.unroll_k;
+    };
+    std::vector<WmmaLdsOpts> tried;
+    auto time_one = [&](const WmmaLdsOpts& o, double* ms) -> bool {
+        if (!wmma_lds_opts_valid(tc, o, M, N, K)) return false;
+        for (const WmmaLdsOpts& t : tried)
+            if (same(t, o)) return false;
+        tried.push_back(o);
+        LinearKernel k;
+        if (build_wmma_matmul_lds_kernel(tc, M, N, K, tc.dtype_in, o, &k) != kOk) return false;
+        BenchmarkResult r;
+        if (compile_and_time(dev, k, "beam_candidate", ptrs, 3, nullptr, 0, 1, 3, &r) != kOk) return false;
+        if (candidates_timed) (*candidates_timed)++;
+        *ms = r.min_ms;
+        return true;
+    };
+    auto keep_best = [&](std::vector<Cand>& v) {
+        std::sort(v.begin(), v.end(), [](const Cand& x, const Cand& y) { return x.first < y.first; });
+        if (static_cast<int>(v.size()) > width) v.resize(width);
+    };
+    // stage 1: LOCAL (the grid of waves), with the largest per-wave tile that still divides
+    std::vector<Cand> beam;
+    static const int grids[][2] = {{2, 2}, {1, 4}, {4, 1}, {2, 4}, {4, 2}, {1, 2}, {2, 1}, {1, 1}, {4, 4}};
+    for (auto& g : grids)
+        for (int up : {4, 2, 1}) {
+            WmmaLdsOpts o;
+            o.waves_m = g[0], o.waves_n = g[1], o.up_m = up, o.up_n = up;
+            double ms;
+            if (time_one(o, &ms)) {
+                beam.emplace_back(ms, o);
+                break;
+            }
+        }
+    if (beam.empty()) return fail(kInvalidArgument, "beam search: no valid tensor-core candidate for this shape");
+    keep_best(beam);
+    // stage 2: UPCAST (tensor-core tiles per wave)
+    {
+        std::vector<Cand> next = beam;
+        for (const Cand& cnd : beam)
+            for (int um : {8, 4, 2, 1})
+                for (int un : {8, 4, 2, 1}) {
+                    WmmaLdsOpts o = cnd.second;
+                    o.up_m = um, o.up_n = un;
+                    double ms;
+                    if (time_one(o, &ms)) next.emplace_back(ms, o);
+                }
+        beam = next;
+        keep_best(beam);
+    }
+    // stage 3: UNROLL (tensor-core K steps per barrier pair)
+    {
+        std::vector<Cand> next = beam;
+        for (const Cand& cnd : beam)
+            for (int u : {1, 2, 4, 8}) {
+                WmmaLdsOpts o = cnd.second;
+                o.unroll_k = u;
+                double ms;
+                if (time_one(o, &ms)) next.emplace_back(ms, o);
+            }
+        beam = next;
+        keep_best(beam);
+    }
+    *best = beam[0].second;
+    if (best_ms) *best_ms = beam[0].first;
+    Record r{{best->waves_m, best->waves_n, best->up_m, best->up_n, best->unroll_k}, beam[0].first};
+    (void)BeamCache::put(ast_hash, width, device, &r, sizeof r);
     clear_error();
     return kOk;
 }

@@ -167,6 +167,14 @@ class BeamCache {
 struct MatmulF32Opts;
 int beam_search_matmul_f32(const Device& dev, int64_t M, int64_t N, int64_t K, int width, MatmulF32Opts* best,
                            double* best_ms, bool* from_cache, int* candidates_timed);
+// The same search over the LDS-staged tensor-core matmul (bf16 in and out): LOCAL = the grid of
+// waves in a workgroup, UPCAST = tensor-core tiles per wave, UNROLL = tensor-core K steps per
+// barrier pair (schedule/src/optimizer/beam.rs:36-120 with the TC action applied first,
+// tc.rs:358-674).
+struct WmmaLdsOpts;
+struct TensorCore;
+int beam_search_wmma_matmul(const Device& dev, const TensorCore& tc, int tc_index, int64_t M, int64_t N, int64_t K, int width,
+                            WmmaLdsOpts* best, double* best_ms, bool* from_cache, int* candidates_timed);
 
 // device/src/sync.rs:44-71,192-310: monotonically increasing timeline value backed by one
 // HIP event per recorded value (the last 16 are kept).

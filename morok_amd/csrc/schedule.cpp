@@ -597,18 +597,49 @@ int build_wmma_matmul_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t
     return kOk;
 }
 
-int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, LinearKernel* k) {
+bool wmma_lds_tile(const TensorCore& tc, const WmmaLdsOpts& o, int64_t K, int* bm, int* bn, int* bk) {
     const int tn = tc.dims[0], tm = tc.dims[1], tk = tc.dims[2];
-    constexpr int um = 4, un = 4, kWavesM = 2, kWavesN = 2;
-    // K steps of the tensor core per barrier pair (UNROLL of the reduce axis): as many as
-    // divide K, up to 64 elements
-    int ku = 1;
-    while (ku * 2 * tk <= 64 && K % (ku * 2 * tk) == 0) ku *= 2;
-    const int BM = kWavesM * um * tm, BN = kWavesN * un * tn, BK = tk * ku;
+    auto pow2_upto = [](int v, int hi) { return v >= 1 && v <= hi && (v & (v - 1)) == 0; };
+    if (!pow2_upto(o.waves_m, 8) || !pow2_upto(o.waves_n, 8) || o.waves_m * o.waves_n > 16) return false;
+    if (!pow2_upto(o.up_m, 8) || !pow2_upto(o.up_n, 8) || o.up_m * o.up_n > 32) return false;
+    int ku = o.unroll_k;
+    if (ku == 0) {
+        ku = 1;
+        while (ku * 2 * tk <= 64 && K % (ku * 2 * tk) == 0) ku *= 2;
+    }
+    if (!pow2_upto(ku, 8) || ku * tk > 128) return false;
+    *bm = o.waves_m * o.up_m * tm;
+    *bn = o.waves_n * o.up_n * tn;
+    *bk = ku * tk;
+    return true;
+}
+
+bool wmma_lds_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, int64_t N, int64_t K) {
+    int BM, BN, BK;
+    if (tc.threads != 64 || tc.dims[0] != 16 || tc.dims[1] != 16 || !wmma_lds_tile(tc, o, K, &BM, &BN, &BK)) return false;
+    if (M <= 0 || N <= 0 || K <= 0 || M % BM || N % BN || K % BK || BK % 8) return false;
+    const int threads = 64 * o.waves_m * o.waves_n;
+    // every work-item copies the same whole number of 8-element vectors of each tile
+    if ((BM * BK / 8) % threads || (BK * BN / 8) % threads) return false;
+    // both tiles (with their padding) in the 160 KB of local memory, two workgroups per CU
+    const size_t lds = (static_cast<size_t>(BM) * (BK + 8) + static_cast<size_t>(BK) * (BN + 4)) * 2;
+    return lds <= 80 * 1024;
+}
+
+int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, const WmmaLdsOpts& opts,
+                                 LinearKernel* k) {
+    const int tn = tc.dims[0], tm = tc.dims[1], tk = tc.dims[2];
     if (tc.threads != 64 || tm != 16 || tn != 16) return fail(kInvalidArgument, "tensor-core matmul (LDS): only 64-lane 16x16 tensor cores are lowered");
+    int BM, BN, BK;
+    if (!wmma_lds_tile(tc, opts, K, &BM, &BN, &BK))
+        return fail(kInvalidArgument, "tensor-core matmul (LDS): waves, tiles per wave and K steps must be powers of two within 16 waves, 32 tiles per wave and a 128-deep K tile");
+    const int um = opts.up_m, un = opts.up_n, kWavesM = opts.waves_m, kWavesN = opts.waves_n;
+    const int ku = BK / tk, threads = 64 * kWavesM * kWavesN;
     if (M % BM || N % BN || K % BK)
         return failf(kInvalidArgument, "tensor-core matmul (LDS): shape %lldx%lldx%lld is not a multiple of the %dx%dx%d workgroup tile",
                      (long long)M, (long long)N, (long long)K, BM, BN, BK);
+    if (!wmma_lds_opts_valid(tc, opts, M, N, K))
+        return fail(kInvalidArgument, "tensor-core matmul (LDS): the tiles do not divide into whole vectors per work-item or do not fit local memory");
     const int ea = tc.elements_per_thread[0], eb = tc.elements_per_thread[1], ec = tc.elements_per_thread[2];
     if (BK % 8 || ea != eb) return fail(kInvalidArgument, "tensor-core matmul (LDS): unsupported operand shape");
     // both operands: element e of a lane is k + e (consecutive k), same row / column
@@ -656,10 +687,12 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
     // of both rows, zips them in registers and writes two 16-byte vectors, and a lane reads
     // its fragment as element pairs, ready for the tensor core without repacking.  (Writing B
     // transposed instead would put the 16 lanes of a copy on two banks.)  PB = BN + 4 puts
-    // the four k groups of a fragment, 4 pair-rows apart, 16 banks apart.  A K tile of fewer
-    // than 32 rows has too few pairs for 256 work-items and keeps plain rows, gathered
-    // element by element.
-    bool pairs = BK % 32 == 0 && eb % 2 == 0;
+    // the four k groups of a fragment, 4 pair-rows apart, 16 banks apart.  A K tile with an
+    // odd number of row vectors per work-item has no whole pairs and keeps plain rows,
+    // gathered element by element.
+    const int a_vecs_per_row = BK / 8, VA = BM * a_vecs_per_row / threads;   // per work-item
+    const int b_vecs_per_row = BN / 8, VB = BK * b_vecs_per_row / threads;
+    bool pairs = eb % 2 == 0 && VB % 2 == 0;
     for (int p = 0; p < 6 && pairs; p++) {
         int mn, kk, mn0, kk0;
         tc_operand_element(tc, 1, 1 << p, 0, &mn, &kk);
@@ -668,24 +701,22 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
     }
     const int P = BK + 8, PB = BN + 4;
     uint32_t sA = b.define_local(0, tc.dtype_in, (int64_t)BM * P), sB = b.define_local(1, tc.dtype_in, (int64_t)BK * PB);
-    // cooperative copies: vectors of 8 elements, 256 work-items
-    const int a_vecs_per_row = BK / 8, VA = BM * a_vecs_per_row / 256;   // per work-item
-    const int b_vecs_per_row = BN / 8, VB = BK * b_vecs_per_row / 256;
-    if (VA < 1 || VB < 1) return fail(kInvalidArgument, "tensor-core matmul (LDS): K tile too shallow for 256 work-items");
+    // cooperative copies: vectors of 8 elements, every work-item the same number
+    if (VA < 1 || VB < 1) return fail(kInvalidArgument, "tensor-core matmul (LDS): K tile too shallow for the workgroup");
     uint32_t ra = b.define_reg(1, tc.dtype_in, VA, 8), rb = b.define_reg(2, tc.dtype_in, VB, 8);
     std::vector<uint32_t> a_row(VA), a_kc(VA), b_krow(VB), b_nc(VB);
     for (int i = 0; i < VA; i++) {
-        uint32_t v = b.iadd(tid, b.ci(256 * i));
+        uint32_t v = b.iadd(tid, b.ci(threads * i));
         a_row[i] = b.idiv(v, a_vecs_per_row);
         a_kc[i] = b.imul(b.imod(v, a_vecs_per_row), 8);
     }
     for (int i = 0; i < VB; i++) {
         if (pairs) {  // vectors 2i and 2i+1 of a work-item: rows 2p and 2p+1, same columns
-            uint32_t v = b.iadd(tid, b.ci(256 * (i / 2)));
+            uint32_t v = b.iadd(tid, b.ci(threads * (i / 2)));
             b_krow[i] = b.iadd(b.imul(b.idiv(v, b_vecs_per_row), 2), b.ci(i % 2));
             b_nc[i] = b.imul(b.imod(v, b_vecs_per_row), 8);
         } else {
-            uint32_t v = b.iadd(tid, b.ci(256 * i));
+            uint32_t v = b.iadd(tid, b.ci(threads * i));
             b_krow[i] = b.idiv(v, b_vecs_per_row);
             b_nc[i] = b.imul(b.imod(v, b_vecs_per_row), 8);
         }

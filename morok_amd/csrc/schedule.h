@@ -192,13 +192,24 @@ LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K, const Matm
 int build_wmma_matmul_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, LinearKernel* k);
 // The same product with the operands staged through local memory (GROUP / LOCAL of the
 // optimizer, schedule/src/optimizer/heuristics.rs:37-82, transforms.rs:1085-1089): a workgroup
-// of 2 x 2 waves owns a 128 x 128 output tile (4 x 4 tensor-core tiles per wave); per K step
-// the 256 work-items copy the A and B tiles global -> registers -> LDS with 16-byte loads (the
-// next step's loads are issued before this step's WMMAs); A fragments are read back as one
-// vector per lane, B fragments (k-strided in a row-major tile) element by element; two barriers
-// per step.
-// Requires M % 128 == 0, N % 128 == 0, K % tile_k == 0 and a tensor core whose lanes hold
-// consecutive k.
+// of waves_m x waves_n waves owns a (waves_m * up_m * 16) x (waves_n * up_n * 16) output tile;
+// per K step the work-items copy the A and B tiles global -> registers -> LDS with 16-byte
+// loads (the next step's loads are issued before this step's WMMAs); A fragments are read back
+// as one vector per lane, B fragments as pairs of consecutive k (rows k and k+1 are kept
+// interleaved in LDS); two barriers per step.  The defaults are 2 x 2 waves of 4 x 4 tiles
+// (128 x 128) and as many tensor-core K steps per barrier pair as divide K, up to 64 elements.
+// Requires M and N to be multiples of the workgroup tile, K of the K tile, and a tensor core
+// whose lanes hold consecutive k.
+struct WmmaLdsOpts {
+    int waves_m = 2, waves_n = 2;  // LOCAL
+    int up_m = 4, up_n = 4;        // UPCAST: tensor-core tiles per wave
+    int unroll_k = 0;              // UNROLL: tensor-core K steps per barrier pair; 0 = choose by K
+};
+// Extents of the workgroup tile these choices give (false if the choices are not buildable at all)
+bool wmma_lds_tile(const TensorCore& tc, const WmmaLdsOpts& o, int64_t K, int* bm, int* bn, int* bk);
+bool wmma_lds_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, int64_t N, int64_t K);
+int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, const WmmaLdsOpts& o,
+                                 LinearKernel* k);
 int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, LinearKernel* k);
 
 }  // namespace mrk

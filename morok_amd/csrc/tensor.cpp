@@ -996,12 +996,33 @@ struct Scheduler {
     // With the hand-written kernels switched off, a bf16 matmul whose shape fits still takes the
     // tensor-core route of the optimizer (schedule/src/optimizer/tc.rs:36-94): the generated
     // WMMA kernel staged through local memory instead of the generic reduce kernel.
+    // The fixed heuristic: the largest of a few workgroup tiles that divides the shape and still
+    // gives every CU a workgroup (16 waves on 256 x 256 measured 1.05 PF at 4096^3 against 0.74
+    // for 4 waves on 128 x 128); a shape too small for that takes the valid tile with the most
+    // workgroups.  MOROK_BEAM searches the whole space instead.
+    static bool default_tc_opts(const TensorCore& tc, int64_t M, int64_t N, int64_t K, WmmaLdsOpts* o) {
+        static const int choices[][4] = {{4, 4, 4, 4}, {2, 2, 4, 4}, {2, 2, 2, 2}, {2, 2, 1, 1}, {1, 1, 1, 1}};
+        bool found = false;
+        for (auto& c : choices) {
+            WmmaLdsOpts t{c[0], c[1], c[2], c[3], 0};
+            if (!wmma_lds_opts_valid(tc, t, M, N, K)) continue;
+            *o = t;  // later (smaller) valid tiles overwrite: more workgroups
+            found = true;
+            int bm, bn, bk;
+            wmma_lds_tile(tc, t, K, &bm, &bn, &bk);
+            if ((M / bm) * (N / bn) >= 256) return true;
+        }
+        return found;
+    }
     bool generated_tc(const TensorNode* n) const {
         if (g_fusion || n->hint != HintKind::Matmul || n->numel() == 0) return false;
         const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
         if (a->dtype != Scalar::BFloat16 || w->dtype != Scalar::BFloat16 || n->dtype != Scalar::BFloat16) return false;
         if (a->shape.size() != 2 || w->shape.size() != 2) return false;
-        return a->shape[0] % 128 == 0 && w->shape[1] % 128 == 0 && a->shape[1] % 32 == 0 && a->shape[1] > 0;
+        const auto tcs = cdna4_tensor_cores();
+        const int tc = select_tensor_core(tcs, Scalar::BFloat16, Scalar::BFloat16, Scalar::Float32);
+        WmmaLdsOpts o;
+        return tc >= 0 && default_tc_opts(tcs[tc], a->shape[0], w->shape[1], a->shape[1], &o);
     }
     int materialize_generated_tc(TensorNode* n) {
         for (const TensorRef& in : n->hint_inputs) MRK_TRY(materialize(in.get()));
@@ -1010,8 +1031,13 @@ struct Scheduler {
         const auto tcs = cdna4_tensor_cores();
         const int tc = select_tensor_core(tcs, Scalar::BFloat16, Scalar::BFloat16, Scalar::Float32);
         if (tc < 0) return fail(kRuntime, "no bf16 tensor core in the CDNA table");
+        WmmaLdsOpts opts;
+        if (!default_tc_opts(tcs[tc], M, N, K, &opts)) return fail(kRuntime, "tensor-core matmul: no workgroup tile divides the shape");
+        int beam = 0;
+        if (const char* e = std::getenv("MOROK_BEAM")) beam = std::atoi(e);
+        if (beam > 0) MRK_TRY(beam_search_wmma_matmul(*dev, tcs[tc], tc, M, N, K, beam, &opts, nullptr, nullptr, nullptr));
         LinearKernel k;
-        MRK_TRY(build_wmma_matmul_lds_kernel(tcs[tc], M, N, K, Scalar::BFloat16, &k));
+        MRK_TRY(build_wmma_matmul_lds_kernel(tcs[tc], M, N, K, Scalar::BFloat16, opts, &k));
         std::shared_ptr<CachedKernel> ck;
         bool cached = false;
         const std::string name = "r_tc_" + std::to_string(M) + "_" + std::to_string(N) + "_" + std::to_string(K);

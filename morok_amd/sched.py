@@ -105,6 +105,13 @@ def build_wmma_matmul_lds(tc_index, m, n, k, out_scalar):
     return _take(lib.mrk_hip_sched_build_wmma_matmul_lds, tc_index, m, n, k, out_scalar)
 
 
+def build_wmma_matmul_lds_opts(tc_index, m, n, k, out_scalar, opts):
+    """The same with explicit (waves_m, waves_n, tiles_m per wave, tiles_n per wave, K steps per
+    barrier pair; 0 = by K)."""
+    arr = (C.c_int * 5)(*opts)
+    return _take(lib.mrk_hip_sched_build_wmma_matmul_lds_opts, tc_index, m, n, k, out_scalar, arr)
+
+
 def build_matmul_f32_opts(m, n, k, opts):
     """f32 matmul kernel with explicit (LOCAL x, LOCAL y, UPCAST n, UPCAST m, UNROLL k)."""
     arr = (C.c_int * 5)(*opts)
@@ -139,4 +146,15 @@ def beam_search_matmul_f32(m, n, k, width=2, device_id=0):
     ms = C.c_double()
     cached, timed = C.c_int(), C.c_int()
     check(lib.mrk_hip_beam_search_matmul_f32(device_id, m, n, k, width, opts, C.byref(ms), C.byref(cached), C.byref(timed)))
+    return list(opts), ms.value, bool(cached.value), timed.value
+
+
+def beam_search_wmma_matmul(tc_index, m, n, k, width=2, device_id=0):
+    """Beam search over the LDS-staged tensor-core matmul; returns (opts, best_ms, from_cache,
+    candidates_timed) with opts as build_wmma_matmul_lds_opts takes them."""
+    opts = (C.c_int * 5)()
+    ms = C.c_double()
+    cached, timed = C.c_int(), C.c_int()
+    check(lib.mrk_hip_beam_search_wmma_matmul(device_id, tc_index, m, n, k, width, opts, C.byref(ms), C.byref(cached),
+                                              C.byref(timed)))
     return list(opts), ms.value, bool(cached.value), timed.value

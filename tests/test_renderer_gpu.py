@@ -252,6 +252,27 @@ def test_tc_matmul_staged_through_local_memory(dev, oracle, tc, shape, out):
     assert np.array_equal(c1, want if out == U.BF16 else synth.from_bf16(want))
 
 
+@pytest.mark.parametrize("opts", [(1, 1, 1, 1, 0), (1, 1, 2, 4, 1), (1, 4, 4, 1, 2), (4, 1, 1, 4, 0), (2, 4, 2, 2, 2),
+                                  (4, 2, 2, 4, 2), (2, 2, 8, 4, 0), (2, 1, 2, 8, 2), (4, 4, 2, 2, 0), (1, 2, 4, 2, 1), (2, 2, 2, 2, 4)])
+def test_tc_matmul_lds_choices_agree(dev, opts):
+    """Every LOCAL / UPCAST / UNROLL choice of the LDS-staged tensor-core kernel computes the same
+    products in the same K order: the bits of the register-only generated kernel, and one-hot
+    operands come back exactly (copy and fragment indexing of each variant)."""
+    from morok_amd import sched
+
+    M, N, K = 512, 256, 256
+    a = synth.normal_bf16((M, K), 5, 21)
+    b = synth.normal_bf16((K, N), 5, 22)
+    kern = sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts)
+    c = run(dev, kern, "r_tc_lds", (M, N), np.uint16, [a, b])
+    plain = run(dev, sched.build_wmma_matmul(1, M, N, K, U.BF16), "r_tc", (M, N), np.uint16, [a, b])
+    assert np.array_equal(c, plain)
+    a1 = np.zeros((M, K), np.float32)
+    a1[np.arange(M), (np.arange(M) * 7) % K] = 1
+    c1 = run(dev, kern, "r_tc_lds", (M, N), np.uint16, [synth.to_bf16(a1), b])
+    assert np.array_equal(c1, b[(np.arange(M) * 7) % K])
+
+
 def test_scheduled_matmul_f32_kernel(dev, oracle):
     from morok_amd import sched
 

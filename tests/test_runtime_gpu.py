@@ -171,6 +171,42 @@ def test_tensor_matmul_with_beam(dev, oracle, tmp_path, monkeypatch):
     np.testing.assert_allclose(got, oracle.matmul_f32(a, b), rtol=1e-4, atol=1e-4)
 
 
+def test_beam_search_wmma_matmul(dev, tmp_path, monkeypatch):
+    """The same search over the LDS-staged tensor-core kernel (waves per workgroup, tiles per
+    wave, K steps per barrier pair): the winner computes the bits of the default choice (same
+    products, same K order), is no slower than it, and the second search comes from the disk
+    cache."""
+    import morok_amd
+    from morok_amd import sched, synth, uop as U
+
+    monkeypatch.setenv("MOROK_CACHE_DIR", str(tmp_path))
+    monkeypatch.delenv("IGNORE_BEAM_CACHE", raising=False)
+    M, N, K = 1024, 512, 512
+    opts, best_ms, cached, timed = sched.beam_search_wmma_matmul(1, M, N, K, width=2)
+    assert not cached and timed >= 12 and best_ms > 0
+    a = synth.normal_bf16((M, K), 8, 0)
+    b = synth.normal_bf16((K, N), 8, 1)
+    ba, bb = morok_amd.Buffer.from_numpy(a), morok_amd.Buffer.from_numpy(b)
+
+    def run(kern, name):
+        bc = dev.buffer(M * N * 2)
+        k = morok_amd.Kernel.get_or_compile(kern, name)
+        plan = morok_amd.ExecutionPlan()
+        plan.add_kernel(k, [plan.add_buffer(bc), plan.add_buffer(ba), plan.add_buffer(bb)])
+        plan.build().execute()
+        return bc, bc.copyout(np.uint16, (M, N))
+
+    bc, got = run(sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts), "beam_tc_winner")
+    _, want = run(sched.build_wmma_matmul_lds(1, M, N, K, U.BF16), "beam_tc_default")
+    assert np.array_equal(got, want)
+    ref = synth.from_bf16(a).astype(np.float64) @ synth.from_bf16(b).astype(np.float64)
+    assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
+    base_ms = sched.compile_and_time(sched.build_wmma_matmul_lds(1, M, N, K, U.BF16), [bc, ba, bb], warmup=1, runs=5)
+    assert best_ms <= base_ms * 1.15
+    opts2, _, cached2, timed2 = sched.beam_search_wmma_matmul(1, M, N, K, width=2)
+    assert cached2 and timed2 == 0 and opts2 == opts
+
+
 def test_copy_and_compute_queues_with_signals(dev):
     """A copy queue feeds a compute queue chunk by chunk; timeline signals order producer and
     consumer on the GPU (hipStreamWaitEvent), the host never waits between chunks.  Each chunk

@@ -154,5 +154,37 @@ def test_wmma_matmul_lds_kernel_builds_and_compiles():
     assert src.count("__WMMA_16_16_32_bfloat_float(") == 2 * 16 + 1   # two K steps x 4 x 4 tiles per wave + the definition
     assert spec.sizes() == ([1, 2, 1], [64, 4, 1])
     morok_amd.compile_spec(spec)
+    assert "amdgpu_waves_per_eu(2)" in src                               # four waves, accumulators within half the file
     with pytest.raises(morok_amd.MorokHipError):
         sched.build_wmma_matmul_lds(1, 64, 128, 64, U.BF16)
+
+
+@pytest.mark.parametrize("opts,grid,block,mfma,hint", [((1, 1, 1, 1, 0), [8, 16, 1], [64, 1, 1], 2, False),
+                                                       ((1, 4, 4, 1, 2), [2, 4, 1], [64, 4, 1], 8, True),
+                                                       ((4, 2, 2, 4, 2), [1, 2, 1], [64, 8, 1], 16, True),
+                                                       ((2, 2, 8, 4, 0), [1, 1, 1], [64, 4, 1], 64, False)])
+def test_wmma_matmul_lds_kernel_choices(opts, grid, block, mfma, hint):
+    """LOCAL (grid of waves), UPCAST (tiles per wave) and UNROLL (K steps per barrier pair) of
+    the LDS-staged tensor-core kernel: launch dimensions and MFMA count follow the choices and
+    every variant compiles; choices that do not divide the shape or the copies are refused."""
+    import morok_amd
+    from morok_amd import sched, uop as U
+
+    M, N, K = 256, 128, 64
+    spec = U.render(sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts), "r_tc_lds")
+    assert spec.sizes() == (grid, block)
+    assert spec.src.count("__WMMA_16_16_32_bfloat_float(") == mfma + 1
+    # two waves per SIMD are asked for when four or more waves share a workgroup and the declared
+    # registers (accumulators + copy staging) stay within 128 per work-item
+    assert ("amdgpu_waves_per_eu(2)" in spec.src) == hint
+    morok_amd.compile_spec(spec)
+
+
+@pytest.mark.parametrize("opts", [(3, 2, 4, 4, 0), (2, 2, 4, 4, 3), (8, 8, 1, 1, 0), (2, 2, 8, 8, 0), (4, 4, 1, 1, 1),
+                                  (2, 2, 4, 4, 8), (1, 1, 8, 8, 0)])
+def test_wmma_matmul_lds_kernel_refuses_bad_choices(opts):
+    import morok_amd
+    from morok_amd import sched, uop as U
+
+    with pytest.raises(morok_amd.MorokHipError):
+        sched.build_wmma_matmul_lds_opts(1, 256, 128, 64, U.BF16, opts)

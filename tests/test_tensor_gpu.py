@@ -287,6 +287,25 @@ def test_sdpa_bf16_uses_flash(T, oracle):
     assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
 
 
+def test_matmul_bf16_generated_tensor_core_small_tiles(T, oracle):
+    """With the hand-written kernels off, bf16 products whose extents are multiples of 16 (not
+    of 128) still take the tensor-core route, on a smaller workgroup tile."""
+    from morok_amd import synth, uop
+
+    T.set_fusion(False)
+    try:
+        for (M, N, K) in ((64, 192, 96), (48, 16, 64), (96, 64, 32)):
+            a = synth.normal_bf16((M, K), 51, 0)
+            w = synth.normal_bf16((K, N), 51, 1)
+            t = T.Tensor.from_numpy(a, uop.BF16).matmul(T.Tensor.from_numpy(w, uop.BF16))
+            got = synth.from_bf16(t.to_numpy())
+            assert t.kernels() == [f"r_tc_{M}_{N}_{K}"]
+            ref = synth.from_bf16(a).astype(np.float64) @ synth.from_bf16(w).astype(np.float64)
+            assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
+    finally:
+        T.set_fusion(True)
+
+
 def test_sdpa_bf16_reads_and_writes_views_in_place(T, oracle):
     """q / k / v as column slices of one packed [B*S, 3*H*D] buffer seen as [B, H, S, D], the
     result permuted back to [B*S, H*D]: one attention kernel and no copy kernels, and the bits
@@ -704,15 +723,16 @@ def test_matmul_bf16_few_rows_uses_split_k(T, oracle):
 
 
 def test_matmul_bf16_generated_tensor_core(T, oracle):
-    """With the hand-written kernels off, a bf16 matmul whose shape fits the 128 x 128 workgroup
-    tile takes the generated tensor-core kernel (WMMA staged through local memory); other shapes
-    keep the generic reduce kernel.  Same numerics policy as the hand-written GEMM: exact
+    """With the hand-written kernels off, a bf16 matmul whose extents are multiples of the
+    tensor-core tile (16 x 16 x 32) takes the generated tensor-core kernel (WMMA staged through
+    local memory, the largest workgroup tile that divides); other shapes keep the generic
+    reduce kernel.  Same numerics policy as the hand-written GEMM: exact
     products, f32 accumulation, one rounding."""
     from morok_amd import synth, uop
 
     T.set_fusion(False)
     rng = np.random.default_rng(71)
-    for (M, N, K), tc in (((256, 128, 96), True), ((128, 256, 1024), True), ((96, 128, 64), False)):
+    for (M, N, K), tc in (((256, 128, 96), True), ((128, 256, 1024), True), ((96, 128, 64), True), ((100, 128, 64), False), ((96, 128, 40), False)):
         a = synth.to_bf16(rng.standard_normal((M, K), dtype=np.float32))
         w = synth.to_bf16(rng.standard_normal((K, N), dtype=np.float32))
         c = T.Tensor.from_numpy(a, uop.BF16).matmul(T.Tensor.from_numpy(w, uop.BF16))
