@@ -856,7 +856,8 @@ struct StridedView {
 
 static bool strided_view(TensorNode* n, StridedView* v) {
     const bool movement = n->kind == TKind::Reshape || n->kind == TKind::Permute || n->kind == TKind::Expand || n->kind == TKind::Shrink;
-    if (n->buffer || !movement) {
+    // a node carrying a fused-kernel hint is a unit: its inner graph is not looked into
+    if (n->buffer || !movement || n->hint != HintKind::None) {
         v->base = n;
         v->offset = 0;
         v->strides = dense_strides(n->shape);
@@ -1084,10 +1085,10 @@ struct Scheduler {
     // reads: the kernel can write that layout itself.  Returns the attention node and the
     // strides of its [B, H, Sq, D] output inside the chain end's dense buffer.
     TensorNode* attention_under(TensorNode* n, std::vector<int64_t>* out_strides) const {
-        if (!g_fusion || n->numel() == 0 || (n->kind != TKind::Reshape && n->kind != TKind::Permute)) return nullptr;
+        if (!g_fusion || n->numel() == 0 || n->hint != HintKind::None || (n->kind != TKind::Reshape && n->kind != TKind::Permute)) return nullptr;
         std::vector<int64_t> st = dense_strides(n->shape);
         TensorNode* m = n;
-        while (m->kind == TKind::Reshape || m->kind == TKind::Permute) {
+        while (m->hint == HintKind::None && (m->kind == TKind::Reshape || m->kind == TKind::Permute)) {
             TensorNode* c = m->src[0].get();
             if (c->buffer) return nullptr;
             auto u = uses.find(c);

@@ -309,7 +309,10 @@ def test_decoder_block_lowering(T, shim, fused, gemms):
     assert sum(k.startswith("gemm_bf16") for k in names) == gemms
     assert sum(k.startswith("flash_fwd") for k in names) == 1
     assert shim.mrk_shim_launches() - n0 == len(names)
-    print(names)
+    # the attention kernel writes [tokens, hidden] itself and reads V in place out of the
+    # projection's [tokens, ...] result: neither is copied into [batch, heads, seq, dim]
+    assert sum(k.startswith("flash_fwd_bf16_strided") for k in names) == 1
+    assert len(names) == (15 if fused else 18)
 
 
 def test_plan_graph_replay_records_once(T, shim):
