@@ -334,14 +334,17 @@ int mrk_hip_sched_build_matmul_f32(int64_t m, int64_t n, int64_t k, uint8_t** ke
 int mrk_hip_sched_build_wmma_matmul(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, uint8_t** kernel,
                                     size_t* len);
 /* The same product with both operands staged through local memory by a workgroup of 2 x 2 waves
- * (128 x 128 output tile; M, N multiples of 128): the GROUP / LOCAL step of the optimizer
- * (schedule/src/optimizer/heuristics.rs:37-82) applied after the tensor-core rewrite. */
+ * (128 x 128 output tile): the GROUP / LOCAL step of the optimizer
+ * (schedule/src/optimizer/heuristics.rs:37-82) applied after the tensor-core rewrite.  Extents
+ * the tile does not divide are padded (PADTO, tc.rs:400-432: gated loads, guarded stores); N and
+ * K must be multiples of 8 (16-byte copies). */
 int mrk_hip_sched_build_wmma_matmul_lds(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, uint8_t** kernel,
                                         size_t* len);
 /* The same with the choices explicit: opts = {waves_m, waves_n (LOCAL: the grid of waves in a
  * workgroup), tiles_m, tiles_n (UPCAST: 16x16 tensor-core tiles per wave), K steps per barrier
- * pair (UNROLL; 0 = as many as divide K, up to 64 elements)}.  All powers of two; M, N, K must be
- * multiples of the resulting workgroup tile; INVALID_ARGUMENT otherwise. */
+ * pair (UNROLL; 0 = as many as divide K, up to 64 elements)}.  All powers of two;
+ * INVALID_ARGUMENT for choices whose tiles do not split into whole 16-byte copies per work-item
+ * or exceed local memory. */
 int mrk_hip_sched_build_wmma_matmul_lds_opts(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, const int opts[5],
                                              uint8_t** kernel, size_t* len);
 void mrk_hip_sched_free(void* p);

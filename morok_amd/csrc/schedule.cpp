@@ -617,7 +617,9 @@ bool wmma_lds_tile(const TensorCore& tc, const WmmaLdsOpts& o, int64_t K, int* b
 bool wmma_lds_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, int64_t N, int64_t K) {
     int BM, BN, BK;
     if (tc.threads != 64 || tc.dims[0] != 16 || tc.dims[1] != 16 || !wmma_lds_tile(tc, o, K, &BM, &BN, &BK)) return false;
-    if (M <= 0 || N <= 0 || K <= 0 || M % BM || N % BN || K % BK || BK % 8) return false;
+    // extents that the tile does not divide are padded (PADTO); the 16-byte copies still need
+    // rows of whole 8-element vectors
+    if (M <= 0 || N <= 0 || K <= 0 || N % 8 || K % 8 || BK % 8) return false;
     const int threads = 64 * o.waves_m * o.waves_n;
     // every work-item copies the same whole number of 8-element vectors of each tile
     if ((BM * BK / 8) % threads || (BK * BN / 8) % threads) return false;
@@ -635,11 +637,15 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
         return fail(kInvalidArgument, "tensor-core matmul (LDS): waves, tiles per wave and K steps must be powers of two within 16 waves, 32 tiles per wave and a 128-deep K tile");
     const int um = opts.up_m, un = opts.up_n, kWavesM = opts.waves_m, kWavesN = opts.waves_n;
     const int ku = BK / tk, threads = 64 * kWavesM * kWavesN;
-    if (M % BM || N % BN || K % BK)
-        return failf(kInvalidArgument, "tensor-core matmul (LDS): shape %lldx%lldx%lld is not a multiple of the %dx%dx%d workgroup tile",
-                     (long long)M, (long long)N, (long long)K, BM, BN, BK);
+    if (M <= 0 || N <= 0 || K <= 0 || N % 8 || K % 8)
+        return failf(kInvalidArgument, "tensor-core matmul (LDS): shape %lldx%lldx%lld needs N and K to be multiples of 8 (16-byte copies)",
+                     (long long)M, (long long)N, (long long)K);
     if (!wmma_lds_opts_valid(tc, opts, M, N, K))
         return fail(kInvalidArgument, "tensor-core matmul (LDS): the tiles do not divide into whole vectors per work-item or do not fit local memory");
+    // PADTO (tc.rs:400-432): an extent the workgroup tile does not divide is rounded up; loads
+    // beyond the operands are gated to zero and stores beyond the result are skipped
+    const bool pad_m = M % BM != 0, pad_n = N % BN != 0, pad_k = K % BK != 0;
+    const int64_t Mp = (M + BM - 1) / BM * BM, Np = (N + BN - 1) / BN * BN;
     const int ea = tc.elements_per_thread[0], eb = tc.elements_per_thread[1], ec = tc.elements_per_thread[2];
     if (BK % 8 || ea != eb) return fail(kInvalidArgument, "tensor-core matmul (LDS): unsupported operand shape");
     // both operands: element e of a lane is k + e (consecutive k), same row / column
@@ -653,7 +659,7 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
     KernelBuilder b;
     b.enable_cse();
     uint32_t c = b.param(0, out, M * N), a = b.param(1, tc.dtype_in, M * K), bm = b.param(2, tc.dtype_in, K * N);
-    uint32_t gx = b.special("gidx0", N / BN), gy = b.special("gidx1", M / BM);
+    uint32_t gx = b.special("gidx0", Np / BN), gy = b.special("gidx1", Mp / BM);
     uint32_t lane = b.special("lidx0", 64), wave = b.special("lidx1", kWavesM * kWavesN);
     uint32_t tid = b.iadd(b.imul(wave, 64), lane);
     uint32_t wy = b.idiv(wave, kWavesN), wx = b.imod(wave, kWavesN);
@@ -721,14 +727,19 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
             b_nc[i] = b.imul(b.imod(v, b_vecs_per_row), 8);
         }
     }
+    auto both = [&](uint32_t x, uint32_t y) { return x == UINT32_MAX ? y : y == UINT32_MAX ? x : b.binary(BinaryOp::And, x, y); };
     auto global_to_regs = [&](uint32_t kbase) {
         for (int i = 0; i < VA; i++) {
-            uint32_t row = b.iadd(b.imul(gy, BM), a_row[i]);
-            b.store(b.index(ra, b.ci(i)), b.load(b.index(a, b.iadd(b.imul(row, K), b.iadd(kbase, a_kc[i]))), 8));
+            uint32_t row = b.iadd(b.imul(gy, BM), a_row[i]), kcol = b.iadd(kbase, a_kc[i]);
+            uint32_t gate = both(pad_m ? b.binary(BinaryOp::Lt, row, b.ci(M)) : UINT32_MAX, pad_k ? b.binary(BinaryOp::Lt, kcol, b.ci(K)) : UINT32_MAX);
+            uint32_t at = b.iadd(b.imul(row, K), kcol);
+            b.store(b.index(ra, b.ci(i)), b.load(gate == UINT32_MAX ? b.index(a, at) : b.index_gated(a, at, gate), 8));
         }
         for (int i = 0; i < VB; i++) {
-            uint32_t col = b.iadd(b.imul(gx, BN), b_nc[i]);
-            b.store(b.index(rb, b.ci(i)), b.load(b.index(bm, b.iadd(b.imul(b.iadd(kbase, b_krow[i]), N), col)), 8));
+            uint32_t col = b.iadd(b.imul(gx, BN), b_nc[i]), krow = b.iadd(kbase, b_krow[i]);
+            uint32_t gate = both(pad_n ? b.binary(BinaryOp::Lt, col, b.ci(N)) : UINT32_MAX, pad_k ? b.binary(BinaryOp::Lt, krow, b.ci(K)) : UINT32_MAX);
+            uint32_t at = b.iadd(b.imul(krow, N), col);
+            b.store(b.index(rb, b.ci(i)), b.load(gate == UINT32_MAX ? b.index(bm, at) : b.index_gated(bm, at, gate), 8));
         }
     };
     // one register object per accumulator tile: as slots of one array the 64 floats become a
@@ -743,7 +754,7 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
         }
     }
     const std::string name = wmma_name(tc);
-    const int64_t KT = K / BK;
+    const int64_t KT = (K + BK - 1) / BK;
     global_to_regs(b.ci(0));
     uint32_t r = b.range(KT, 0, AxisType::Reduce);
     // registers -> local memory
@@ -823,7 +834,10 @@ int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int
                 uint32_t col = b.iadd(b.iadd(b.iadd(b.imul(gx, BN), b.imul(wx, un * tn)), b.ci(j * tn + (n - n0))), c_n);
                 uint32_t v = b.gep(res, e);
                 if (out != tc.dtype_out) v = b.cast(v, out);
+                uint32_t inside = both(pad_m ? b.binary(BinaryOp::Lt, row, b.ci(M)) : UINT32_MAX, pad_n ? b.binary(BinaryOp::Lt, col, b.ci(N)) : UINT32_MAX);
+                if (inside != UINT32_MAX) b.if_(inside);
                 b.store(b.index(c, b.iadd(b.imul(row, N), col)), v);
+                if (inside != UINT32_MAX) b.endif();
             }
         }
     *k = b.finish();

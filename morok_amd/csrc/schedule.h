@@ -198,8 +198,10 @@ int build_wmma_matmul_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t
 // as one vector per lane, B fragments as pairs of consecutive k (rows k and k+1 are kept
 // interleaved in LDS); two barriers per step.  The defaults are 2 x 2 waves of 4 x 4 tiles
 // (128 x 128) and as many tensor-core K steps per barrier pair as divide K, up to 64 elements.
-// Requires M and N to be multiples of the workgroup tile, K of the K tile, and a tensor core
-// whose lanes hold consecutive k.
+// Extents the workgroup tile does not divide are padded (PADTO, tc.rs:400-432): the grid is
+// rounded up, loads past the operands are gated to zero, stores past the result are skipped.
+// Requires N and K to be multiples of 8 (16-byte copies) and a tensor core whose lanes hold
+// consecutive k.
 struct WmmaLdsOpts {
     int waves_m = 2, waves_n = 2;  // LOCAL
     int up_m = 4, up_n = 4;        // UPCAST: tensor-core tiles per wave

@@ -997,21 +997,29 @@ struct Scheduler {
     // With the hand-written kernels switched off, a bf16 matmul whose shape fits still takes the
     // tensor-core route of the optimizer (schedule/src/optimizer/tc.rs:36-94): the generated
     // WMMA kernel staged through local memory instead of the generic reduce kernel.
-    // The fixed heuristic: the largest of a few workgroup tiles that divides the shape and still
-    // gives every CU a workgroup (16 waves on 256 x 256 measured 1.05 PF at 4096^3 against 0.74
-    // for 4 waves on 128 x 128); a shape too small for that takes the valid tile with the most
-    // workgroups.  MOROK_BEAM searches the whole space instead.
+    // The fixed heuristic: the largest of a few workgroup tiles that gives every CU a workgroup
+    // (16 waves on 256 x 256 measured 1.05 PF at 4096^3 against 0.74 for 4 waves on 128 x 128)
+    // and pads the output by at most an eighth; a shape too small for that takes the tile with
+    // the least padding, the smaller one among equals.  MOROK_BEAM searches the whole space.
     static bool default_tc_opts(const TensorCore& tc, int64_t M, int64_t N, int64_t K, WmmaLdsOpts* o) {
         static const int choices[][4] = {{4, 4, 4, 4}, {2, 2, 4, 4}, {2, 2, 2, 2}, {2, 2, 1, 1}, {1, 1, 1, 1}};
         bool found = false;
+        int64_t least = 0;
         for (auto& c : choices) {
             WmmaLdsOpts t{c[0], c[1], c[2], c[3], 0};
             if (!wmma_lds_opts_valid(tc, t, M, N, K)) continue;
-            *o = t;  // later (smaller) valid tiles overwrite: more workgroups
-            found = true;
             int bm, bn, bk;
             wmma_lds_tile(tc, t, K, &bm, &bn, &bk);
-            if ((M / bm) * (N / bn) >= 256) return true;
+            const int64_t tm = (M + bm - 1) / bm, tn = (N + bn - 1) / bn, padded = tm * bm * tn * bn;
+            if (padded * 8 <= M * N * 9 && tm * tn >= 256) {
+                *o = t;
+                return true;
+            }
+            if (!found || padded <= least) {
+                *o = t;
+                least = padded;
+                found = true;
+            }
         }
         return found;
     }

@@ -273,6 +273,40 @@ def test_tc_matmul_lds_choices_agree(dev, opts):
     assert np.array_equal(c1, b[(np.arange(M) * 7) % K])
 
 
+@pytest.mark.parametrize("shape,opts", [((200, 136, 72), (2, 2, 4, 4, 0)), ((1, 8, 8), (1, 1, 1, 1, 0)), ((130, 264, 200), (2, 2, 2, 2, 2)),
+                                        ((257, 256, 64), (4, 4, 4, 4, 0)), ((128, 128, 40), (2, 2, 4, 4, 0)), ((100, 128, 64), (1, 4, 4, 1, 2))])
+def test_tc_matmul_lds_padded_shapes(dev, shape, opts):
+    """PADTO: extents the workgroup tile does not divide.  Loads past the operands are gated
+    to zero and stores past the result skipped: values against float64, one-hot rows exact,
+    and memory behind the result and the operands untouched / unread (NaN patterns placed
+    there would surface in the result)."""
+    from morok_amd import sched
+
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 6, 31)
+    b = synth.normal_bf16((K, N), 6, 32)
+    kern = sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts)
+    # operands and result each sit in the front of a larger NaN-filled buffer
+    nan = np.uint16(0x7FC0)
+    abig = np.full(M * K + 4096, nan, np.uint16); abig[:M * K] = a.ravel()
+    bbig = np.full(K * N + 4096, nan, np.uint16); bbig[:K * N] = b.ravel()
+    ba, bb = morok_amd.Buffer.from_numpy(abig), morok_amd.Buffer.from_numpy(bbig)
+    bc = morok_amd.Buffer.from_numpy(np.full(M * N + 4096, nan, np.uint16))
+    k = morok_amd.Kernel.get_or_compile(kern, "r_tc_pad")
+    plan = morok_amd.ExecutionPlan()
+    plan.add_kernel(k, [plan.add_buffer(bc), plan.add_buffer(ba), plan.add_buffer(bb)])
+    plan.build().execute()
+    got = bc.copyout(np.uint16, (M * N + 4096,))
+    assert np.all(got[M * N:] == nan)
+    c = synth.from_bf16(got[:M * N].reshape(M, N))
+    ref = synth.from_bf16(a).astype(np.float64) @ synth.from_bf16(b).astype(np.float64)
+    assert np.all(np.isfinite(c)) and np.abs(c - ref).max() <= 2e-2 * np.abs(ref).max()
+    a1 = np.zeros((M, K), np.float32)
+    a1[np.arange(M), (np.arange(M) * 7) % K] = 1
+    c1 = run(dev, kern, "r_tc_pad", (M, N), np.uint16, [synth.to_bf16(a1), b])
+    assert np.array_equal(c1, b[(np.arange(M) * 7) % K])
+
+
 def test_scheduled_matmul_f32_kernel(dev, oracle):
     from morok_amd import sched
 

@@ -155,8 +155,13 @@ def test_wmma_matmul_lds_kernel_builds_and_compiles():
     assert spec.sizes() == ([1, 2, 1], [64, 4, 1])
     morok_amd.compile_spec(spec)
     assert "amdgpu_waves_per_eu(2)" in src                               # four waves, accumulators within half the file
+    # extents the tile does not divide are padded: gated loads, guarded stores, a rounded-up grid
+    pad = U.render(sched.build_wmma_matmul_lds(1, 200, 136, 72, U.BF16), "r_tc_pad")
+    assert pad.sizes() == ([2, 2, 1], [64, 4, 1]) and " ? *((mrk_bhalf8*)" in pad.src and "if (" in pad.src
+    morok_amd.compile_spec(pad)
+    assert " ? *((mrk_bhalf8*)" not in src and "if (" not in src        # none of it when the tile divides
     with pytest.raises(morok_amd.MorokHipError):
-        sched.build_wmma_matmul_lds(1, 64, 128, 64, U.BF16)
+        sched.build_wmma_matmul_lds(1, 64, 130, 64, U.BF16)               # rows of B are not whole 16-byte vectors
 
 
 @pytest.mark.parametrize("opts,grid,block,mfma,hint", [((1, 1, 1, 1, 0), [8, 16, 1], [64, 1, 1], 2, False),

@@ -723,16 +723,16 @@ def test_matmul_bf16_few_rows_uses_split_k(T, oracle):
 
 
 def test_matmul_bf16_generated_tensor_core(T, oracle):
-    """With the hand-written kernels off, a bf16 matmul whose extents are multiples of the
-    tensor-core tile (16 x 16 x 32) takes the generated tensor-core kernel (WMMA staged through
-    local memory, the largest workgroup tile that divides); other shapes keep the generic
-    reduce kernel.  Same numerics policy as the hand-written GEMM: exact
+    """With the hand-written kernels off, a bf16 matmul whose N and K are multiples of 8 takes
+    the generated tensor-core kernel (WMMA staged through local memory; extents the workgroup
+    tile does not divide are padded); other shapes keep the generic reduce kernel.  Same numerics policy as the hand-written GEMM: exact
     products, f32 accumulation, one rounding."""
     from morok_amd import synth, uop
 
     T.set_fusion(False)
     rng = np.random.default_rng(71)
-    for (M, N, K), tc in (((256, 128, 96), True), ((128, 256, 1024), True), ((96, 128, 64), True), ((100, 128, 64), False), ((96, 128, 40), False)):
+    for (M, N, K), tc in (((256, 128, 96), True), ((128, 256, 1024), True), ((96, 128, 64), True), ((100, 128, 64), True), ((96, 128, 40), True),
+                           ((3, 8, 8), True), ((100, 132, 64), False), ((96, 128, 36), False)):
         a = synth.to_bf16(rng.standard_normal((M, K), dtype=np.float32))
         w = synth.to_bf16(rng.standard_normal((K, N), dtype=np.float32))
         c = T.Tensor.from_numpy(a, uop.BF16).matmul(T.Tensor.from_numpy(w, uop.BF16))
