@@ -252,10 +252,9 @@ int ExecutionPlan::execute_profiled(std::vector<KernelProfile>* out) {
     if (!built_) MRK_TRY(build());
     out->clear();
     if (kernels_.empty()) return kOk;
-    ffi::Stream stream = buffers_.empty() ? nullptr : nullptr;
     std::shared_ptr<Allocator> alloc;
     MRK_TRY(AllocatorRegistry::global().get(device_id_, &alloc));
-    stream = alloc->stream();
+    ffi::Stream stream = alloc->stream();
     MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
     std::vector<ffi::Event> ev(kernels_.size() + 1, nullptr);
     for (auto& e : ev) MRK_HIP(ffi::event_create(&e), "hipEventCreate");

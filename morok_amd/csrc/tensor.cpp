@@ -621,7 +621,7 @@ uint32_t emit_load(KernelGen& g, const TensorNode* n, const Coords& coords) {
     KernelBuilder& b = g.b;
     uint32_t p = g.buffer_param(n->buffer, n->dtype, n->numel());
     Cx flat = flatten(g, coords, n->shape);
-    const int64_t per_load = std::min<int64_t>(g.width, 16 / static_cast<int64_t>(scalar_size(n->dtype)));
+    const int64_t per_load = std::min<int64_t>(g.width, 16 / std::max<int64_t>(1, static_cast<int64_t>(scalar_size(n->dtype))));
     if (flat.aligned && per_load > 1 && n->dtype != Scalar::Bool) {
         // one vector load per group of `per_load` consecutive elements, shared by the group
         const int64_t group = flat.off / per_load;
