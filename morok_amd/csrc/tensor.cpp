@@ -554,6 +554,13 @@ struct KernelGen {
     int64_t gate = -1;
     std::map<std::tuple<const TensorNode*, Coords, int64_t>, uint32_t> memo;  // (node, coordinates, gate) -> value
     std::map<std::tuple<uint32_t, uint32_t, int64_t, int64_t>, uint32_t> vec_loads;  // (param, base index, group, gate) -> vector value
+    // A cat that the kernel splits at its root: instead of evaluating every part and selecting,
+    // the kernel runs one guarded region per part and this cat forwards to the part picked
+    // (pick_part >= 0), or only reports its coordinate along the cat axis (pick_part == -2).
+    const TensorNode* pick_cat = nullptr;
+    int pick_part = -1;
+    Cx probed_pos;
+    bool probed = false;
 
     uint32_t ci(int64_t v) { return b.ci(v, idx_t); }
     uint32_t value(const Cx& c) { return c.off ? b.iadd(c.node, ci(c.off)) : c.node; }
@@ -734,6 +741,18 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) 
             bool groups = coords[axis].aligned;  // a whole upcast group falls into one part
             for (const TensorRef& p : n->src) groups = groups && p->shape[axis] % g.width == 0;
             if (n->numel() == 0) return is_float(ct) ? b.cf(0.0, ct) : b.ci(0, ct);
+            if (n == g.pick_cat && g.pick_part == -2) {
+                g.probed_pos = coords[axis];
+                g.probed = true;
+                return is_float(ct) ? b.cf(0.0, ct) : b.ci(0, ct);
+            }
+            if (n == g.pick_cat && g.pick_part >= 0) {  // inside the guarded region of one part
+                int64_t start = 0;
+                for (int i = 0; i < g.pick_part; i++) start += n->src[i]->shape[axis];
+                Coords sc = coords;
+                sc[axis] = Cx{start ? b.iadd(coords[axis].node, g.ci(-start)) : coords[axis].node, coords[axis].off, coords[axis].aligned};
+                return emit(g, n->src[g.pick_part].get(), sc);
+            }
             const uint32_t pos = groups ? coords[axis].node : g.value(coords[axis]);
             const int64_t span = groups ? g.width : 1;
             int64_t start = 0;
@@ -1238,6 +1257,30 @@ struct Scheduler {
         return kOk;
     }
 
+    // The cat a kernel rooted at `n` may split on: reached from the root through single-source
+    // nodes that neither reduce nor reorder within the innermost axis in ways the caller cannot
+    // check (the caller verifies the coordinate correspondence by probing), with at least two
+    // parts of equal extent along the cat's last axis, each a whole number of upcast groups,
+    // and at least one part that is not already in memory (else selecting costs nothing).
+    static const TensorNode* root_cat(const TensorNode* n, int64_t width) {
+        if (width <= 1 || n->shape.empty()) return nullptr;
+        const TensorNode* m = n;
+        while (!m->buffer && m->hint == HintKind::None &&
+               (m->kind == TKind::Contiguous || m->kind == TKind::Cast || m->kind == TKind::Permute || m->kind == TKind::Reshape) && m != nullptr) {
+            if (m->src.empty()) return nullptr;
+            m = m->src[0].get();
+        }
+        if (m->buffer || m->kind != TKind::Cat || m->src.size() < 2 || m->src.size() > 4 || m->shape.empty()) return nullptr;
+        const size_t axis = static_cast<size_t>(m->arg[0]);
+        if (axis + 1 != m->shape.size() || m->shape[axis] != n->shape.back()) return nullptr;
+        bool computed = false;
+        for (const TensorRef& p : m->src) {
+            if (p->shape[axis] != m->src[0]->shape[axis] || p->shape[axis] % width) return nullptr;
+            computed = computed || !p->buffer;
+        }
+        return computed ? m : nullptr;
+    }
+
     int gen_elementwise(TensorNode* n, int64_t max_numel) {
         const int64_t N = n->numel();
         KernelGen g;
@@ -1264,19 +1307,71 @@ struct Scheduler {
         }
         uint32_t item = b.iadd(b.imul(gx, block), lx);
         b.if_(b.binary(BinaryOp::Lt, item, g.ci(items)));
-        uint32_t base = b.imul(item, width);
-        Coords coords = plain(unflatten(g, base, n->shape));
-        if (width > 1) coords.back().aligned = true;
-        std::vector<uint32_t> vals;
-        for (int64_t e = 0; e < width; e++) {
-            Coords ce = coords;
-            if (!ce.empty()) ce.back().off = e;
-            uint32_t v = n->kind == TKind::Contiguous ? emit(g, n->src[0].get(), ce) : emit_uncached(g, n, ce);
-            if (b.dtype(v).scalar != n->dtype) v = b.cast(v, n->dtype);
-            vals.push_back(v);
+        auto emit_group = [&](const Coords& coords, uint32_t base) {
+            std::vector<uint32_t> vals;
+            for (int64_t e = 0; e < width; e++) {
+                Coords ce = coords;
+                if (!ce.empty()) ce.back().off = e;
+                uint32_t v = n->kind == TKind::Contiguous ? emit(g, n->src[0].get(), ce) : emit_uncached(g, n, ce);
+                if (b.dtype(v).scalar != n->dtype) v = b.cast(v, n->dtype);
+                vals.push_back(v);
+            }
+            if (width > 1) b.store(b.index(po, base), b.vectorize(vals));
+            else b.store(b.index(po, base), vals[0]);
+        };
+        // A cat of computed parts along the innermost output axis (rotary embedding: cat(real,
+        // imag)).  Evaluating every part for every output and selecting costs the arithmetic of
+        // all parts; instead the work-items are renumbered so that the 64 of a wave produce
+        // outputs of one part only (R rows x the part's vectors), and each part gets its own
+        // guarded region, which a wave of the other part skips altogether.
+        const TensorNode* cat = root_cat(n, width);
+        bool split = false;
+        if (cat) {
+            const int64_t P = static_cast<int64_t>(cat->src.size()), V = n->shape.back() / width, Vp = V / P;
+            const size_t axis = static_cast<size_t>(cat->arg[0]);
+            if (Vp >= 1 && V % P == 0 && 64 % Vp == 0 && block % (64 * P) == 0 && items % (64 * P) == 0) {
+                const int64_t R = 64 / Vp;
+                uint32_t grp = b.idiv(item, 64 * P), part = b.imod(b.idiv(item, 64), P), k = b.imod(item, 64);
+                uint32_t row = b.iadd(b.imul(grp, R), b.idiv(k, Vp));
+                uint32_t vec = b.iadd(b.imul(part, Vp), b.imod(k, Vp));
+                uint32_t base = b.imul(b.iadd(b.imul(row, V), vec), width);
+                Coords coords = plain(unflatten(g, base, n->shape));
+                coords.back().aligned = true;
+                // where along the cat axis this group lies: it has to be the innermost output
+                // coordinate itself for the renumbering to make waves uniform
+                g.pick_cat = cat;
+                g.pick_part = -2;
+                g.probed = false;
+                (void)(n->kind == TKind::Contiguous ? emit(g, n->src[0].get(), coords) : emit_uncached(g, n, coords));
+                g.memo.clear();
+                g.vec_loads.clear();
+                if (g.probed && g.probed_pos.aligned && g.probed_pos.off == 0 && g.probed_pos.node == coords.back().node) {
+                    split = true;
+                    int64_t start = 0;
+                    for (int64_t pi = 0; pi < P; pi++) {
+                        const int64_t len = cat->src[pi]->shape[axis];
+                        uint32_t live = b.binary(BinaryOp::And, b.binary(BinaryOp::Ge, g.probed_pos.node, g.ci(start)),
+                                                 b.binary(BinaryOp::Lt, g.probed_pos.node, g.ci(start + len)));
+                        b.if_(live);
+                        g.pick_part = static_cast<int>(pi);
+                        emit_group(coords, base);
+                        b.endif();
+                        // values named inside a guarded region are not visible after it
+                        g.memo.clear();
+                        g.vec_loads.clear();
+                        start += len;
+                    }
+                }
+                g.pick_cat = nullptr;
+                g.pick_part = -1;
+            }
         }
-        if (width > 1) b.store(b.index(po, base), b.vectorize(vals));
-        else b.store(b.index(po, base), vals[0]);
+        if (!split) {
+            uint32_t base = b.imul(item, width);
+            Coords coords = plain(unflatten(g, base, n->shape));
+            if (width > 1) coords.back().aligned = true;
+            emit_group(coords, base);
+        }
         b.endif();
         return finish_kernel(g, n, out, "E_" + std::to_string(N) + (width > 1 ? "_" + std::to_string(width) : ""));
     }
