@@ -216,6 +216,15 @@ def test_tensor_kernel_counts_generated(T, shim):
     assert len(rope.kernels()) == 1
     rope_i = x.apply_rotary_emb(zeros(T, (1, 1, 6, 4)), zeros(T, (1, 1, 6, 4)), True).realize()
     assert len(rope_i.kernels()) == 1
+    # a cat of computed halves on the innermost axis becomes one guarded region per half, with
+    # the work-items renumbered so that a wave stays inside one half
+    xr = zeros(T, (2, 16, 4, 128))
+    big = xr.apply_rotary_emb(zeros(T, (1, 16, 1, 64)), zeros(T, (1, 16, 1, 64)), False).realize()
+    src = T.last_kernel_sources()[0]
+    assert len(big.kernels()) == 1 and src.count("if (") == 3 and " ? " not in src.split("if (", 2)[2]
+    small = x.apply_rotary_emb(zeros(T, (1, 1, 6, 4)), zeros(T, (1, 1, 6, 4)), False).realize()
+    assert T.last_kernel_sources()[0].count("if (") == 1          # too few outputs for whole waves: select as before
+    assert len(small.kernels()) == 1
     a = x.scaled_dot_product_attention(x, x, is_causal=True).realize()
     assert len(a.kernels()) == 4                     # QK^T, max, sum, PV (the divide fuses into PV)
     sw = zeros(T, (1000,)).silu().realize()

@@ -306,6 +306,41 @@ def test_matmul_bf16_generated_tensor_core_small_tiles(T, oracle):
         T.set_fusion(True)
 
 
+@pytest.mark.parametrize("rows,part,nparts,dtype", [(64, 64, 2, "f32"), (256, 32, 4, "f32"), (48, 8, 2, "f32"), (8, 256, 2, "f32"),
+                                                     (64, 64, 2, "bf16"), (30, 64, 2, "f32"), (64, 24, 2, "f32"), (64, 64, 3, "f32"),
+                                                     (64, 512, 2, "f32")])
+def test_cat_of_computed_parts(T, rows, part, nparts, dtype):
+    """cat of parts that are computed (not just loaded) along the innermost axis: the kernel is
+    split into one guarded region per part when the parts are equal, a whole number of upcast
+    groups and fit the wave renumbering, and falls back to evaluate-and-select otherwise (odd
+    row counts, three parts, parts wider than a wave); permuted in front of the store as well.
+    All against numpy on the same values."""
+    from morok_amd import synth, uop
+
+    rng = np.random.default_rng(rows * 1000 + part * 10 + nparts)
+    x = rng.standard_normal((4, rows, part)).astype(np.float32)
+    y = rng.standard_normal((4, rows, part)).astype(np.float32)
+    if dtype == "bf16":
+        xb, yb = synth.to_bf16(x), synth.to_bf16(y)
+        x, y = synth.from_bf16(xb), synth.from_bf16(yb)
+        tx, ty = T.Tensor.from_numpy(xb, uop.BF16), T.Tensor.from_numpy(yb, uop.BF16)
+    else:
+        tx, ty = T.Tensor.from_numpy(x), T.Tensor.from_numpy(y)
+    exprs = [lambda a, b: a * b - b, lambda a, b: a + b * 2.0, lambda a, b: a * a, lambda a, b: b - a]
+    tparts = [(tx.try_mul(ty).try_sub(ty)), (tx.try_add(ty.try_mul(2.0))), (tx.try_mul(tx)), (ty.try_sub(tx))][:nparts]
+    want = np.concatenate([f(x, y) for f in exprs[:nparts]], axis=-1)
+    t = T.Tensor.cat(tparts, -1)
+    got = t.to_numpy()
+    assert len(t.kernels()) == 1
+    gotf = synth.from_bf16(got) if dtype == "bf16" else got
+    tol = 1e-2 if dtype == "bf16" else 1e-6
+    np.testing.assert_allclose(gotf, want, rtol=tol, atol=tol)
+    tp = T.Tensor.cat(tparts, -1).try_permute([1, 0, 2]).contiguous()
+    gp = tp.to_numpy()
+    gpf = synth.from_bf16(gp) if dtype == "bf16" else gp
+    np.testing.assert_allclose(gpf, want.transpose(1, 0, 2), rtol=tol, atol=tol)
+
+
 def test_sdpa_bf16_reads_and_writes_views_in_place(T, oracle):
     """q / k / v as column slices of one packed [B*S, 3*H*D] buffer seen as [B, H, S, D], the
     result permuted back to [B*S, H*D]: one attention kernel and no copy kernels, and the bits
