@@ -529,12 +529,15 @@ namespace {
 // constant, which lets the V elements one work-item produces (UPCAST of the innermost axis,
 // schedule/src/optimizer/heuristics.rs:37-82) share all index arithmetic and lets a load of
 // V consecutive elements become one vector load.  `aligned`: node is a multiple of the
-// upcast width and off lies in [0, width).
+// upcast width and off lies in [0, width).  `mult`: a known divisor of node (0 = nothing known),
+// which survives a reshape that splits the upcast axis (node / 2 is still a multiple of
+// width / 2) and decides whether a narrower group of elements can still be one vector load.
 struct Cx {
     uint32_t node = 0;
     int64_t off = 0;
     bool aligned = false;
-    bool operator<(const Cx& o) const { return std::tie(node, off, aligned) < std::tie(o.node, o.off, o.aligned); }
+    int64_t mult = 0;
+    bool operator<(const Cx& o) const { return std::tie(node, off, aligned, mult) < std::tie(o.node, o.off, o.aligned, o.mult); }
 };
 using Coords = std::vector<Cx>;
 
@@ -605,21 +608,72 @@ std::vector<uint32_t> unflatten(KernelGen& g, uint32_t flat, const std::vector<i
     return coords;
 }
 
-// Row-major flat index of `coords` in `shape` as (node, constant offset); *vec_ok tells whether
-// the node part is a multiple of the upcast width with the offset inside one group, i.e. the
-// elements off = 0..width-1 are consecutive in memory.
+int64_t gcd64(int64_t a, int64_t b) {
+    while (b) {
+        int64_t t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
+}
+
+// Row-major flat index of `coords` in `shape` as (node, constant offset).  `aligned` in the
+// result: the node part is known to be a multiple of the upcast width and the offset lies
+// inside one group, i.e. the elements off = 0..width-1 are consecutive in memory.
 Cx flatten(KernelGen& g, const Coords& coords, const std::vector<int64_t>& shape) {
     std::vector<uint32_t> nodes(coords.size());
     int64_t off = 0, stride = 1;
-    bool vec_ok = g.width > 1 && !shape.empty() && shape.back() % g.width == 0 && coords.back().aligned;
+    // what the flat node is known to be a multiple of: per axis, what its node is a multiple
+    // of times the axis stride (a constant-zero node contributes nothing)
+    const uint32_t zero = g.ci(0);
+    int64_t mult = 0;
     for (size_t i = shape.size(); i-- > 0;) {
         nodes[i] = coords[i].node;
-        if (shape[i] != 1) off += coords[i].off * stride;
-        if (i + 1 != shape.size() && coords[i].off != 0 && shape[i] != 1) vec_ok = false;
+        if (shape[i] != 1) {
+            off += coords[i].off * stride;
+            if (coords[i].node != zero) {
+                const int64_t m = coords[i].aligned ? std::max<int64_t>(g.width, coords[i].mult) : std::max<int64_t>(1, coords[i].mult);
+                mult = gcd64(mult, m * stride);
+            }
+        }
         stride *= shape[i];
     }
-    if (!vec_ok && g.width > 1 && shape.empty()) vec_ok = false;
-    return Cx{flatten_nodes(g, nodes, shape), off, vec_ok && off >= 0 && off < g.width};
+    if (mult == 0) mult = int64_t{1} << 40;  // every node is the constant zero
+    // the group of `width` elements starts on a multiple of the width and this element lies in it
+    const bool aligned = g.width > 1 && !shape.empty() && mult % g.width == 0 && off >= 0 && off < g.width;
+    return Cx{flatten_nodes(g, nodes, shape), off, aligned, mult};
+}
+
+// Coordinates in `shape` of flat = node + off, where node is a multiple of the upcast width W
+// and 0 <= off < W, when the trailing dimensions split W evenly: dimensions whose extent
+// times everything inside them divides W see only the constant part of the index, the one
+// dimension that straddles W gets node-part + constant without carry (its extent must be a
+// multiple of what is left of W), everything further out sees only the node.  False when
+// the dimensions do not line up that way.
+bool split_group(KernelGen& g, const Cx& flat, const std::vector<int64_t>& shape, Coords* out) {
+    const int64_t W = g.width;
+    if (W <= 1 || shape.empty()) return false;
+    std::vector<uint32_t> u = unflatten(g, flat.node, shape);
+    out->assign(shape.size(), Cx{});
+    int64_t inner = 1;
+    bool done = false;  // past the straddling dimension
+    for (size_t i = shape.size(); i-- > 0;) {
+        const int64_t d = shape[i];
+        if (d == 1) {
+            (*out)[i] = g.zero();
+        } else if (done) {
+            (*out)[i] = Cx{u[i], 0, false, 0};
+        } else if (W % (inner * d) == 0) {
+            (*out)[i] = Cx{g.ci(0), (flat.off / inner) % d, false, 0};  // the node part is a multiple of inner * d
+            done = inner * d == W;
+        } else {
+            if (W % inner || d % (W / inner)) return false;
+            (*out)[i] = Cx{u[i], flat.off / inner, false, W / inner};
+            done = true;
+        }
+        inner *= d;
+    }
+    return true;
 }
 
 uint32_t emit(KernelGen& g, const TensorNode* n, const Coords& coords);
@@ -629,7 +683,10 @@ uint32_t emit_load(KernelGen& g, const TensorNode* n, const Coords& coords) {
     uint32_t p = g.buffer_param(n->buffer, n->dtype, n->numel());
     Cx flat = flatten(g, coords, n->shape);
     const int64_t per_load = std::min<int64_t>(g.width, 16 / std::max<int64_t>(1, static_cast<int64_t>(scalar_size(n->dtype))));
-    if (flat.aligned && per_load > 1 && n->dtype != Scalar::Bool) {
+    // a group of per_load consecutive elements that starts on a multiple of per_load (and so lies
+    // inside a buffer of a multiple of per_load elements) is one vector load
+    const bool narrow = per_load > 1 && flat.mult > 0 && flat.mult % per_load == 0 && flat.off >= 0;
+    if ((flat.aligned || narrow) && per_load > 1 && n->numel() % per_load == 0 && n->dtype != Scalar::Bool) {
         // one vector load per group of `per_load` consecutive elements, shared by the group
         const int64_t group = flat.off / per_load;
         auto key = std::make_tuple(p, flat.node, group, g.gate);
@@ -703,6 +760,8 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) 
                     std::vector<uint32_t> u = unflatten(g, flat.node, s->shape);
                     for (size_t i = 0; i < sc.size(); i++) sc[i] = Cx{u[i], 0, false};
                     sc.back() = Cx{u.back(), flat.off, true};
+                } else if (flat.aligned && split_group(g, flat, s->shape, &sc)) {
+                    // the group is spread over several trailing source dimensions
                 } else {
                     std::vector<uint32_t> u = unflatten(g, g.value(flat), s->shape);
                     for (size_t i = 0; i < sc.size(); i++) sc[i] = Cx{u[i], 0, false};
@@ -752,6 +811,19 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) 
                 Coords sc = coords;
                 sc[axis] = Cx{start ? b.iadd(coords[axis].node, g.ci(-start)) : coords[axis].node, coords[axis].off, coords[axis].aligned};
                 return emit(g, n->src[g.pick_part].get(), sc);
+            }
+            if (!groups && coords[axis].node == g.ci(0)) {
+                // the position along the cat axis is a compile-time constant: no selection at all
+                int64_t start = 0;
+                for (const TensorRef& p : n->src) {
+                    const int64_t len = p->shape[axis];
+                    if (coords[axis].off >= start && coords[axis].off < start + len) {
+                        Coords sc = coords;
+                        sc[axis] = Cx{g.ci(0), coords[axis].off - start, false, 0};
+                        return emit(g, p.get(), sc);
+                    }
+                    start += len;
+                }
             }
             const uint32_t pos = groups ? coords[axis].node : g.value(coords[axis]);
             const int64_t span = groups ? g.width : 1;
