@@ -222,6 +222,11 @@ def test_tensor_kernel_counts_generated(T, shim):
     big = xr.apply_rotary_emb(zeros(T, (1, 16, 1, 64)), zeros(T, (1, 16, 1, 64)), False).realize()
     src = T.last_kernel_sources()[0]
     assert len(big.kernels()) == 1 and src.count("if (") == 3 and " ? " not in src.split("if (", 2)[2]
+    # interleaved pairs: the reshape [.., 128] -> [.., 64, 2] splits the upcast group; positions along
+    # the trailing axis stay compile-time constants, so nothing is selected and x is one vector load
+    inter = xr.apply_rotary_emb(zeros(T, (1, 16, 1, 64)), zeros(T, (1, 16, 1, 64)), True).realize()
+    src = T.last_kernel_sources()[0]
+    assert len(inter.kernels()) == 1 and " ? " not in src and src.count("*((mrk_float4*)") == 2   # the load of x, the store
     small = x.apply_rotary_emb(zeros(T, (1, 1, 6, 4)), zeros(T, (1, 1, 6, 4)), False).realize()
     assert T.last_kernel_sources()[0].count("if (") == 1          # too few outputs for whole waves: select as before
     assert len(small.kernels()) == 1
