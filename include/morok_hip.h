@@ -507,6 +507,13 @@ int mrk_hip_tensor_rotary(const mrk_tensor* x, const mrk_tensor* cos, const mrk_
 /* scale <= 0 selects 1/sqrt(head_dim) (transformer.rs:90-91) */
 int mrk_hip_tensor_sdpa(const mrk_tensor* q, const mrk_tensor* k, const mrk_tensor* v, double scale, int is_causal,
                         mrk_tensor** out);                                                    /* transformer.rs:78-137 */
+/* The same with the remaining options of the reference's builder: attn_mask (NULL for none; Bool:
+ * true = attend, otherwise added to the scores; broadcastable to [.., Sq, Sk], transformer.rs:112-125)
+ * and softcap (<= 0 for none; cap * tanh(scores / cap), transformer.rs:128-132).  With either of them
+ * the composed graph runs; the fused attention kernel covers neither. */
+int mrk_hip_tensor_sdpa_ex(const mrk_tensor* q, const mrk_tensor* k, const mrk_tensor* v, const mrk_tensor* attn_mask,
+                           double scale, int is_causal, double softcap, mrk_tensor** out);
+int mrk_hip_tensor_tanh(const mrk_tensor* t, mrk_tensor** out);                               /* activation.rs:64-74 */
 /* realization (realize.rs:83-127) and extraction (data.rs:211-236) */
 int mrk_hip_tensor_realize(const mrk_tensor* t);
 /* Tensor::prepare (realize.rs:299-357): schedule + compile into an execution plan without

@@ -204,6 +204,9 @@ _SIGS = {
     "mrk_hip_tensor_embedding": (C.c_int, [C.c_void_p, C.c_void_p, c_void_pp]),
     "mrk_hip_tensor_rotary": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, c_void_pp]),
     "mrk_hip_tensor_sdpa": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_double, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_sdpa_ex": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_double, C.c_int, C.c_double,
+                                         c_void_pp]),
+    "mrk_hip_tensor_tanh": (C.c_int, [C.c_void_p, c_void_pp]),
     "mrk_hip_tensor_realize": (C.c_int, [C.c_void_p]),
     "mrk_hip_tensor_prepare": (C.c_int, [C.c_void_p, c_void_pp]),
     "mrk_hip_tensor_to_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),

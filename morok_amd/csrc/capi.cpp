@@ -1137,6 +1137,18 @@ int mrk_hip_tensor_sdpa(const mrk_tensor* q, const mrk_tensor* k, const mrk_tens
     MRK_NONNULL(v);
     return wrap_tensor(q->t.scaled_dot_product_attention(k->t, v->t, scale, is_causal != 0), out);
 }
+int mrk_hip_tensor_sdpa_ex(const mrk_tensor* q, const mrk_tensor* k, const mrk_tensor* v, const mrk_tensor* attn_mask,
+                           double scale, int is_causal, double softcap, mrk_tensor** out) {
+    MRK_T1(q);
+    MRK_NONNULL(k);
+    MRK_NONNULL(v);
+    return wrap_tensor(q->t.scaled_dot_product_attention(k->t, v->t, scale, is_causal != 0, attn_mask ? &attn_mask->t : nullptr, softcap),
+                       out);
+}
+int mrk_hip_tensor_tanh(const mrk_tensor* t, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.tanh(), out);
+}
 int mrk_hip_tensor_realize(const mrk_tensor* t) {
     MRK_NONNULL(t);
     return t->t.realize();

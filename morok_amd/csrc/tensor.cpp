@@ -346,6 +346,13 @@ Tensor Tensor::sigmoid() const {
     return const_(1.0, n_->dtype, n_->device_id).try_add(e).unary(UnaryOp::Reciprocal);
 }
 Tensor Tensor::swish() const { return try_mul(sigmoid()); }
+Tensor Tensor::tanh() const {
+    // tanh(x) = 2 * sigmoid(2x) - 1  (activation.rs:64-74)
+    if (!n_) return Tensor();
+    Tensor two = const_(2.0, n_->dtype, n_->device_id);
+    Tensor sig = try_mul(two).sigmoid();
+    return two.try_mul(sig).try_sub(const_(1.0, n_->dtype, n_->device_id));
+}
 
 Tensor Tensor::reduce(ReduceOp op, std::vector<int64_t> axes, bool keepdim, bool promote) const {
     if (!n_) return Tensor();
@@ -493,7 +500,8 @@ Tensor Tensor::apply_rotary_emb(const Tensor& cos, const Tensor& sin, bool inter
     return cat({real, imag}, -1);
 }
 
-Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& value, double scale, bool is_causal) const {
+Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& value, double scale, bool is_causal,
+                                            const Tensor* attn_mask, double softcap) const {
     if (!n_ || !key.valid() || !value.valid()) return Tensor();
     const int64_t nd = ndim();
     if (nd < 2 || key.ndim() != nd || value.ndim() != nd) return bad(kInvalidArgument, "sdpa: rank mismatch");
@@ -513,8 +521,23 @@ Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& val
         Tensor mask = iota(1).binary(BinaryOp::Le, iota(0));
         scores = scores.where_(mask, const_(-INFINITY, sdt, n_->device_id));
     }
+    if (attn_mask) {  // transformer.rs:112-125
+        if (!attn_mask->valid()) return Tensor();
+        if (attn_mask->dtype() == Scalar::Bool) {
+            // true = attend: 0 where the mask holds, -inf elsewhere, added to the scores
+            Tensor additive = const_(0.0, sdt, n_->device_id).where_(*attn_mask, const_(-INFINITY, sdt, n_->device_id));
+            scores = scores.try_add(additive);
+        } else {
+            scores = scores.try_add(*attn_mask);
+        }
+    }
+    if (softcap > 0.0) {  // transformer.rs:128-132
+        Tensor cap = const_(softcap, sdt, n_->device_id);
+        scores = scores.try_div(cap).tanh().try_mul(cap);
+    }
     Tensor out = scores.softmax(-1).matmul(value);
     if (!out.valid()) return out;
+    if (attn_mask || softcap > 0.0) return out;  // the fused kernel covers neither: composed graph
     out.node()->hint = HintKind::Sdpa;
     out.node()->hint_inputs = {n_, key.node(), value.node()};
     out.node()->hint_scale = scale_val;

@@ -116,6 +116,7 @@ class Tensor {
     Tensor square() const { return unary(UnaryOp::Square); }
     Tensor sigmoid() const;  // activation.rs:42-52
     Tensor swish() const;    // activation.rs:309-313
+    Tensor tanh() const;     // activation.rs:64-74
     Tensor silu() const { return swish(); }
 
     // ---- reductions (reduce.rs:620-692)
@@ -130,7 +131,10 @@ class Tensor {
     Tensor rms_norm(int64_t axis, double eps) const;                        // nn/norm.rs:92-111
     Tensor embedding(const Tensor& indices) const;                          // transformer.rs:12-25
     Tensor apply_rotary_emb(const Tensor& cos, const Tensor& sin, bool interleaved) const;  // transformer.rs:32-69
-    Tensor scaled_dot_product_attention(const Tensor& key, const Tensor& value, double scale, bool is_causal) const;  // transformer.rs:78-137
+    // transformer.rs:78-137.  scale <= 0: 1/sqrt(head_dim); attn_mask (optional): Bool (true =
+    // attend) or additive, broadcastable to [.., Sq, Sk]; softcap > 0: cap * tanh(scores / cap).
+    Tensor scaled_dot_product_attention(const Tensor& key, const Tensor& value, double scale, bool is_causal,
+                                        const Tensor* attn_mask = nullptr, double softcap = 0.0) const;
 
     // ---- realization (realize.rs:83-127) and extraction (data.rs:211-236)
     int realize() const;

@@ -213,6 +213,9 @@ class Tensor:
     def silu(self):
         return self._new(lib.mrk_hip_tensor_silu)
 
+    def tanh(self):
+        return self._new(lib.mrk_hip_tensor_tanh)
+
     swish = silu
 
     # ---- reductions
@@ -251,8 +254,13 @@ class Tensor:
     def apply_rotary_emb(self, cos, sin, interleaved=False):
         return self._new(lib.mrk_hip_tensor_rotary, cos._h, sin._h, int(interleaved))
 
-    def scaled_dot_product_attention(self, key, value, scale=None, is_causal=False):
-        return self._new(lib.mrk_hip_tensor_sdpa, key._h, value._h, float(scale) if scale else 0.0, int(is_causal))
+    def scaled_dot_product_attention(self, key, value, scale=None, is_causal=False, attn_mask=None, softcap=None):
+        """transformer.rs:78-137.  attn_mask: Bool (True = attend) or additive, broadcastable to
+        [.., Sq, Sk]; softcap: cap * tanh(scores / cap).  Either of them selects the composed graph."""
+        if attn_mask is None and not softcap:
+            return self._new(lib.mrk_hip_tensor_sdpa, key._h, value._h, float(scale) if scale else 0.0, int(is_causal))
+        return self._new(lib.mrk_hip_tensor_sdpa_ex, key._h, value._h, attn_mask._h if attn_mask is not None else None,
+                         float(scale) if scale else 0.0, int(is_causal), float(softcap) if softcap else 0.0)
 
     # ---- realization / extraction
     def realize(self):

@@ -273,6 +273,87 @@ def test_sdpa_f32_vs_oracle(T, fusion, oracle, causal):
     np.testing.assert_allclose(out, ref, rtol=1e-4, atol=1e-5)
 
 
+def _np_sdpa(q, k, v, scale, causal=False, mask=None, softcap=None):
+    s = np.einsum("bhqd,bhkd->bhqk", q.astype(np.float64), k.astype(np.float64)) * scale
+    if causal:
+        s = np.where(np.tril(np.ones(s.shape[-2:], bool)), s, -np.inf)
+    if mask is not None:
+        s = s + (np.where(mask, 0.0, -np.inf) if mask.dtype == np.bool_ else mask.astype(np.float64))
+    if softcap:
+        s = np.tanh(s / softcap) * softcap
+    s = s - s.max(-1, keepdims=True)
+    p = np.exp(s)
+    p /= p.sum(-1, keepdims=True)
+    return np.einsum("bhqk,bhkd->bhqd", p, v.astype(np.float64))
+
+
+def test_tanh(T, fusion):
+    """tanh = 2 * sigmoid(2x) - 1 (activation.rs:64-74); the reference's doc values."""
+    x = np.array([-2.0, -1.0, 0.0, 1.0, 2.0, 9.0, -30.0], np.float32)
+    got = T.Tensor.from_numpy(x).tanh().to_numpy()
+    np.testing.assert_allclose(got[:5], [-0.964, -0.762, 0.0, 0.762, 0.964], atol=1e-3)
+    np.testing.assert_allclose(got, np.tanh(x.astype(np.float64)), rtol=1e-5, atol=1e-6)
+
+
+def test_sdpa_softcap_reference_case(T, fusion):
+    """transformer.rs test_sdpa_softcap: scores of 10 * scale capped through tanh stay finite; values
+    against the closed form."""
+    q = np.array([[[[10.0, 0.0], [0.0, 10.0]]]], np.float32)
+    v = np.array([[[[1.0, 0.0], [0.0, 1.0]]]], np.float32)
+    t = T.Tensor.from_numpy(q).scaled_dot_product_attention(T.Tensor.from_numpy(q), T.Tensor.from_numpy(v), softcap=1.0)
+    got = t.to_numpy()
+    assert got.shape == (1, 1, 2, 2) and np.all(np.isfinite(got))
+    np.testing.assert_allclose(got, _np_sdpa(q, q, v, 1 / np.sqrt(2), softcap=1.0), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("kind", ["bool", "bool_broadcast", "additive", "additive_causal_softcap"])
+def test_sdpa_attn_mask(T, fusion, kind):
+    """Attention masks (transformer.rs:112-125): Bool (true = attend) and additive, full and
+    broadcast over batch and heads, alone and together with the causal mask and a softcap;
+    against the float64 closed form.  Every query keeps at least one visible key."""
+    rng = np.random.default_rng(61)
+    B, H, Sq, Sk, D = 2, 3, 20, 28, 16
+    q, k, v = (rng.standard_normal(sh).astype(np.float32) for sh in ((B, H, Sq, D), (B, H, Sk, D), (B, H, Sk, D)))
+    scale = 1 / np.sqrt(D)
+    causal, softcap = False, None
+    if kind == "bool":
+        mask = rng.random((B, H, Sq, Sk)) < 0.6
+        mask[..., 0] = True
+    elif kind == "bool_broadcast":
+        mask = rng.random((1, 1, Sq, Sk)) < 0.5
+        mask[..., 0] = True
+    elif kind == "additive":
+        mask = rng.standard_normal((B, 1, Sq, Sk)).astype(np.float32)
+    else:
+        mask = rng.standard_normal((Sq, Sk)).astype(np.float32)
+        causal, softcap = True, 5.0
+    t = T.Tensor.from_numpy(q).scaled_dot_product_attention(T.Tensor.from_numpy(k), T.Tensor.from_numpy(v), is_causal=causal,
+                                                            attn_mask=T.Tensor.from_numpy(mask), softcap=softcap)
+    got = t.to_numpy()
+    want = _np_sdpa(q, k, v, scale, causal=causal, mask=mask, softcap=softcap)
+    assert np.all(np.isfinite(got))
+    np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-5)
+    assert not any(n.startswith("flash_fwd") for n in t.kernels())
+
+
+def test_sdpa_bf16_with_mask_takes_the_composed_graph(T):
+    """bf16 operands with a mask: the fused kernel does not apply, the composed graph still
+    computes the masked attention (bf16 scores: loose tolerance)."""
+    from morok_amd import synth, uop
+
+    rng = np.random.default_rng(62)
+    B, H, S, D = 1, 2, 64, 128
+    q, k, v = (synth.to_bf16(rng.standard_normal((B, H, S, D)).astype(np.float32)) for _ in range(3))
+    mask = rng.random((S, S)) < 0.7
+    mask[:, 0] = True
+    t = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(T.Tensor.from_numpy(k, uop.BF16), T.Tensor.from_numpy(v, uop.BF16),
+                                                                      attn_mask=T.Tensor.from_numpy(mask))
+    got = synth.from_bf16(t.to_numpy())
+    assert not any(n.startswith("flash_fwd") for n in t.kernels())
+    want = _np_sdpa(synth.from_bf16(q), synth.from_bf16(k), synth.from_bf16(v), 1 / np.sqrt(D), mask=mask)
+    assert np.abs(got - want).max() <= 5e-2 * np.abs(want).max()
+
+
 def test_sdpa_bf16_uses_flash(T, oracle):
     from morok_amd import synth, uop
 
