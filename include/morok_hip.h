@@ -498,7 +498,15 @@ int mrk_hip_tensor_reduce(const mrk_tensor* t, int reduce_op, const int64_t* axe
                           int promote, mrk_tensor** out);
 int mrk_hip_tensor_mean(const mrk_tensor* t, const int64_t* axes, size_t naxes, int keepdim, mrk_tensor** out);
 /* composite ops of the hot path */
+/* 1-D x 1-D (scalar result), 1-D x 2-D, 2-D x 1-D, 2-D x 2-D, batched with broadcast batch axes */
 int mrk_hip_tensor_matmul(const mrk_tensor* a, const mrk_tensor* b, mrk_tensor** out);        /* matmul.rs:82-110 */
+/* matmul_with().dtype(): accumulate in and return `acc_dtype` (a dtype tag; -1 = the default rule) */
+int mrk_hip_tensor_matmul_with(const mrk_tensor* a, const mrk_tensor* b, int acc_dtype, mrk_tensor** out);
+/* alpha * op(A) @ op(B) + beta * C, c may be NULL (matmul.rs:112-135) */
+int mrk_hip_tensor_gemm(const mrk_tensor* a, const mrk_tensor* b, float alpha, float beta, int trans_a, int trans_b,
+                        const mrk_tensor* c, mrk_tensor** out);
+/* x @ weight^T + bias, weight [out, in] (1-D weight: elementwise product), bias may be NULL (matmul.rs:160-190) */
+int mrk_hip_tensor_linear(const mrk_tensor* x, const mrk_tensor* weight, const mrk_tensor* bias, int acc_dtype, mrk_tensor** out);
 int mrk_hip_tensor_softmax(const mrk_tensor* t, int64_t axis, mrk_tensor** out);              /* activation.rs:90-101 */
 int mrk_hip_tensor_rms_norm(const mrk_tensor* t, int64_t axis, double eps, mrk_tensor** out); /* nn/norm.rs:92-111 */
 int mrk_hip_tensor_embedding(const mrk_tensor* weight, const mrk_tensor* indices, mrk_tensor** out); /* transformer.rs:12-25 */

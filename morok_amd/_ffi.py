@@ -199,6 +199,9 @@ _SIGS = {
     "mrk_hip_tensor_reduce": (C.c_int, [C.c_void_p, C.c_int, c_i64_p, C.c_size_t, C.c_int, C.c_int, c_void_pp]),
     "mrk_hip_tensor_mean": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),
     "mrk_hip_tensor_matmul": (C.c_int, [C.c_void_p, C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_matmul_with": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_gemm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_int, C.c_void_p, c_void_pp]),
+    "mrk_hip_tensor_linear": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, c_void_pp]),
     "mrk_hip_tensor_softmax": (C.c_int, [C.c_void_p, C.c_int64, c_void_pp]),
     "mrk_hip_tensor_rms_norm": (C.c_int, [C.c_void_p, C.c_int64, C.c_double, c_void_pp]),
     "mrk_hip_tensor_embedding": (C.c_int, [C.c_void_p, C.c_void_p, c_void_pp]),

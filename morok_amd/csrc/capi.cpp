@@ -1110,6 +1110,24 @@ int mrk_hip_tensor_matmul(const mrk_tensor* a, const mrk_tensor* b, mrk_tensor**
     MRK_NONNULL(b);
     return wrap_tensor(a->t.matmul(b->t), out);
 }
+int mrk_hip_tensor_matmul_with(const mrk_tensor* a, const mrk_tensor* b, int acc_dtype, mrk_tensor** out) {
+    MRK_T1(a);
+    MRK_NONNULL(b);
+    if (acc_dtype < -1 || acc_dtype >= static_cast<int>(Scalar::Void)) return fail(kInvalidArgument, "matmul_with: unknown dtype tag");
+    return wrap_tensor(a->t.matmul(b->t, acc_dtype < 0 ? Scalar::Void : static_cast<Scalar>(acc_dtype)), out);
+}
+int mrk_hip_tensor_gemm(const mrk_tensor* a, const mrk_tensor* b, float alpha, float beta, int trans_a, int trans_b,
+                        const mrk_tensor* c, mrk_tensor** out) {
+    MRK_T1(a);
+    MRK_NONNULL(b);
+    return wrap_tensor(a->t.gemm(b->t, alpha, beta, trans_a != 0, trans_b != 0, c ? &c->t : nullptr), out);
+}
+int mrk_hip_tensor_linear(const mrk_tensor* x, const mrk_tensor* weight, const mrk_tensor* bias, int acc_dtype, mrk_tensor** out) {
+    MRK_T1(x);
+    MRK_NONNULL(weight);
+    if (acc_dtype < -1 || acc_dtype >= static_cast<int>(Scalar::Void)) return fail(kInvalidArgument, "linear: unknown dtype tag");
+    return wrap_tensor(x->t.linear(weight->t, bias ? &bias->t : nullptr, acc_dtype < 0 ? Scalar::Void : static_cast<Scalar>(acc_dtype)), out);
+}
 int mrk_hip_tensor_softmax(const mrk_tensor* t, int64_t axis, mrk_tensor** out) {
     MRK_T1(t);
     return wrap_tensor(t->t.softmax(axis), out);

@@ -405,7 +405,7 @@ Tensor Tensor::mean(std::vector<int64_t> axes, bool keepdim) const {
     return s.try_mul(const_(1.0 / static_cast<double>(count), s.dtype(), n_->device_id));
 }
 
-Tensor Tensor::matmul(const Tensor& other) const {
+Tensor Tensor::matmul(const Tensor& other, Scalar acc) const {
     if (!n_ || !other.n_) return Tensor();
     const int64_t dx = ndim(), dw = other.ndim();
     if (dx == 0 || dw == 0) return bad(kInvalidArgument, "matmul: 0-d operand");
@@ -413,19 +413,51 @@ Tensor Tensor::matmul(const Tensor& other) const {
     const int64_t axis_w = dw >= 2 ? dw - 2 : 0;
     if (other.n_->shape[axis_w] != k)
         return bad(kInvalidArgument, "matmul: shapes " + shape_str(n_->shape) + " and " + shape_str(other.n_->shape) + " do not contract");
-    if (dx < 2 || dw < 2) return bad(kInvalidArgument, "matmul: vector operands are not supported by this backend");
-    // x[..., M, K] -> [..., M, 1, K];  w[..., K, N] -> [..., 1, N, K];  product.sum(-1)  (matmul.rs:96-109)
+    // x[..., M, K] -> [..., M, 1, K];  w[..., K, N] -> [..., 1, N, K];  product.sum(-1)  (matmul.rs:96-109).
+    // The broadcast axis is only inserted when both sides have one to pair it with: a vector
+    // operand multiplies as it is ([K] * [N, K], [M, K] * [K], [K] * [K]).
+    const int64_t bd = std::min<int64_t>({dx - 1, dw - 1, 1});
     std::vector<int64_t> xs = n_->shape;
-    xs.insert(xs.end() - 1, 1);
-    Tensor wt = other.try_transpose(-1, -2);
+    if (bd) xs.insert(xs.end() - 1, 1);
+    Tensor wt = dw >= 2 ? other.try_transpose(-1, -2) : other;
     std::vector<int64_t> ws = wt.shape();
-    ws.insert(ws.end() - 2, 1);
+    if (bd) ws.insert(ws.end() - 2, 1);
     Tensor prod = try_reshape(xs).try_mul(wt.try_reshape(ws));
+    if (acc != Scalar::Void) return prod.cast(acc).reduce(ReduceOp::Add, {-1}, false, false);  // sum_with().dtype(): reduce.rs:636-673
     Tensor res = prod.reduce(ReduceOp::Add, {-1}, false, true);
-    if (!res.valid()) return res;
+    if (!res.valid() || dx < 2 || dw < 2) return res;
     res.node()->hint = HintKind::Matmul;
     res.node()->hint_inputs = {n_, other.n_};
     return res;
+}
+
+Tensor Tensor::gemm(const Tensor& b, float alpha, float beta, bool trans_a, bool trans_b, const Tensor* c) const {
+    if (!n_ || !b.valid()) return Tensor();
+    Tensor a = trans_a ? try_transpose(0, 1) : *this;
+    Tensor bb = trans_b ? b.try_transpose(0, 1) : b;
+    Tensor res = a.matmul(bb);
+    if (!res.valid()) return res;
+    // the reference multiplies by f32 one-element tensors (matmul.rs:125-131): f32 promotion rules apply
+    if (alpha != 1.0f) res = res.try_mul(full({1}, alpha, Scalar::Float32, n_->device_id));
+    if (c) {
+        if (!c->valid()) return Tensor();
+        Tensor cc = beta != 1.0f ? c->try_mul(full({1}, beta, Scalar::Float32, n_->device_id)) : *c;
+        res = res.try_add(cc);
+    }
+    return res;
+}
+
+Tensor Tensor::linear(const Tensor& weight, const Tensor* bias, Scalar acc) const {
+    if (!n_ || !weight.valid()) return Tensor();
+    Tensor res;
+    if (weight.ndim() == 1) {
+        res = acc != Scalar::Void ? cast(acc).try_mul(weight) : try_mul(weight);
+    } else {
+        res = matmul(weight.try_transpose(-1, -2), acc);
+    }
+    if (!res.valid() || !bias) return res;
+    if (!bias->valid()) return Tensor();
+    return res.try_add(*bias);  // broadcast to the result's shape
 }
 
 Tensor Tensor::softmax(int64_t axis) const {

@@ -126,7 +126,14 @@ class Tensor {
     Tensor mean(std::vector<int64_t> axes, bool keepdim) const;
 
     // ---- composite ops on the hot path
-    Tensor matmul(const Tensor& other) const;                               // matmul.rs:82-110
+    // matmul.rs:82-110: 1-D x 1-D (scalar), 1-D x 2-D, 2-D x 1-D, 2-D x 2-D, batched with broadcast
+    // batch axes.  `acc` other than Void: accumulate in and return that dtype (matmul_with().dtype()).
+    Tensor matmul(const Tensor& other, Scalar acc = Scalar::Void) const;
+    Tensor dot(const Tensor& other) const { return matmul(other); }              // matmul.rs:40-42
+    // alpha * op(A) @ op(B) + beta * C  (matmul.rs:112-135); c may be null
+    Tensor gemm(const Tensor& b, float alpha, float beta, bool trans_a, bool trans_b, const Tensor* c) const;
+    // self @ weight^T + bias, weight [out, in] (a 1-D weight multiplies elementwise); matmul.rs:160-190
+    Tensor linear(const Tensor& weight, const Tensor* bias, Scalar acc = Scalar::Void) const;
     Tensor softmax(int64_t axis) const;                                     // activation.rs:90-101
     Tensor rms_norm(int64_t axis, double eps) const;                        // nn/norm.rs:92-111
     Tensor embedding(const Tensor& indices) const;                          // transformer.rs:12-25

@@ -236,10 +236,23 @@ class Tensor:
         return self._new(lib.mrk_hip_tensor_mean, a, n, int(keepdim))
 
     # ---- composite ops
-    def matmul(self, other):
-        return self._new(lib.mrk_hip_tensor_matmul, other._h)
+    def matmul(self, other, dtype=None):
+        """matmul.rs:82-110 (vector operands included); dtype: accumulate in and return that dtype."""
+        if dtype is None:
+            return self._new(lib.mrk_hip_tensor_matmul, other._h)
+        return self._new(lib.mrk_hip_tensor_matmul_with, other._h, int(dtype))
 
     dot = matmul
+
+    def gemm(self, b, alpha=1.0, beta=1.0, trans_a=False, trans_b=False, c=None):
+        """alpha * op(A) @ op(B) + beta * C (matmul.rs:112-135)."""
+        return self._new(lib.mrk_hip_tensor_gemm, b._h, float(alpha), float(beta), int(trans_a), int(trans_b),
+                         c._h if c is not None else None)
+
+    def linear(self, weight, bias=None, dtype=None):
+        """self @ weight.T + bias, weight [out, in] (matmul.rs:160-190)."""
+        return self._new(lib.mrk_hip_tensor_linear, weight._h, bias._h if bias is not None else None,
+                         -1 if dtype is None else int(dtype))
 
     def softmax(self, axis=-1):
         return self._new(lib.mrk_hip_tensor_softmax, axis)

@@ -106,6 +106,77 @@ def test_matmul_nonsquare_and_batched(T, fusion, oracle):
     np.testing.assert_allclose(got, np.stack([oracle.matmul_f32(ab[i], bb[i]) for i in range(3)]), rtol=1e-4, atol=1e-5)
 
 
+def test_matmul_vector_operands(T, fusion):
+    """tensor/src/test/unit/matmul.rs:176-235: 1-D @ 1-D is a scalar (70 for the reference's
+    vectors), [4] @ [4, 3] -> [3], [3, 4] @ [4] -> [3]; larger random cases against numpy."""
+    a = np.array([1, 2, 3, 4, 5], np.float32)
+    b = np.array([2, 3, 4, 5, 6], np.float32)
+    d = T.Tensor.from_numpy(a).dot(T.Tensor.from_numpy(b))
+    assert d.shape == () and abs(float(d.to_numpy().reshape(-1)[0]) - 70.0) < 1e-5
+    v = np.array([1, 2, 3, 4], np.float32)
+    m = np.arange(1, 13, dtype=np.float32).reshape(4, 3)
+    vm = T.Tensor.from_numpy(v).dot(T.Tensor.from_numpy(m))
+    assert vm.shape == (3,)
+    np.testing.assert_allclose(vm.to_numpy(), v @ m, atol=1e-5)
+    m2 = np.arange(1, 13, dtype=np.float32).reshape(3, 4)
+    mv = T.Tensor.from_numpy(m2).dot(T.Tensor.from_numpy(v))
+    assert mv.shape == (3,)
+    np.testing.assert_allclose(mv.to_numpy(), m2 @ v, atol=1e-5)
+    rng = np.random.default_rng(81)
+    x, w, y = rng.standard_normal(300).astype(np.float32), rng.standard_normal((300, 70)).astype(np.float32), \
+        rng.standard_normal((5, 40, 300)).astype(np.float32)
+    for lhs, rhs in ((x, w), (w.T.copy(), x), (y, x), (x, x)):
+        got = T.Tensor.from_numpy(lhs).matmul(T.Tensor.from_numpy(rhs)).to_numpy()
+        want = lhs.astype(np.float64) @ rhs.astype(np.float64)
+        np.testing.assert_allclose(got.reshape(want.shape), want, rtol=1e-4, atol=1e-4)
+
+
+def test_matmul_dtype_options(T, fusion):
+    """matmul.rs tests 417-435: int32 @ float32 promotes to float32; matmul_with().dtype(f64)
+    accumulates the f32 products in float64 and returns float64."""
+    from morok_amd import uop
+
+    ai = np.array([[1, 2], [3, 4]], np.int32)
+    bf = np.array([[5.0, 6.0], [7.0, 8.0]], np.float32)
+    c = T.Tensor.from_numpy(ai).dot(T.Tensor.from_numpy(bf))
+    assert c.dtype == uop.F32
+    np.testing.assert_allclose(c.to_numpy(), ai @ bf)
+    rng = np.random.default_rng(82)
+    a = (rng.standard_normal((8, 4096)) * 1e3).astype(np.float32)
+    b = rng.standard_normal((4096, 8)).astype(np.float32)
+    c64 = T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b), dtype=uop.F64)
+    assert c64.dtype == uop.F64
+    got = c64.to_numpy()
+    # the reference casts the f32 products, not the operands (matmul.rs:107-109): each product is
+    # rounded to f32, the sum of 4096 of them is exact to f64 rounding
+    want = (a[:, :, None] * b[None, :, :]).astype(np.float64).sum(axis=1)
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-7)
+
+
+def test_linear_and_gemm(T, fusion):
+    """matmul.rs:513-566 (linear: bias, no bias, batched, 1-D weight) and gemm (alpha, beta,
+    transposes, C), values against numpy."""
+    x = np.array([[1.0, 2.0, 3.0]], np.float32)
+    w = np.array([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]], np.float32)
+    bias = np.array([0.1, 0.2], np.float32)
+    r = T.Tensor.from_numpy(x).linear(T.Tensor.from_numpy(w), T.Tensor.from_numpy(bias))
+    assert r.shape == (1, 2)
+    np.testing.assert_allclose(r.to_numpy(), x @ w.T + bias, rtol=1e-6)
+    r = T.Tensor.from_numpy(x).linear(T.Tensor.from_numpy(w))
+    assert r.shape == (1, 2)
+    np.testing.assert_allclose(r.to_numpy(), x @ w.T, rtol=1e-6)
+    r = T.Tensor.from_numpy(np.ones((4, 3), np.float32)).linear(T.Tensor.from_numpy(np.ones((2, 3), np.float32)))
+    assert r.shape == (4, 2) and np.all(r.to_numpy() == 3.0)
+    r = T.Tensor.from_numpy(np.array([1, 2, 3], np.float32)).linear(T.Tensor.from_numpy(np.array([2, 3, 4], np.float32)))
+    assert r.shape == (3,) and np.all(r.to_numpy() == [2, 6, 12])
+    rng = np.random.default_rng(83)
+    a, b, c = (rng.standard_normal(sh).astype(np.float32) for sh in ((64, 48), (32, 48), (64, 32)))
+    g = T.Tensor.from_numpy(a).gemm(T.Tensor.from_numpy(b), alpha=0.5, beta=2.0, trans_b=True, c=T.Tensor.from_numpy(c))
+    np.testing.assert_allclose(g.to_numpy(), 0.5 * (a @ b.T) + 2.0 * c, rtol=1e-4, atol=1e-4)
+    g = T.Tensor.from_numpy(a.T.copy()).gemm(T.Tensor.from_numpy(b.T.copy()), trans_a=True)
+    np.testing.assert_allclose(g.to_numpy(), a @ b.T, rtol=1e-4, atol=1e-4)
+
+
 def test_matmul_shape_error(T):
     from morok_amd import MorokHipError
 
