@@ -85,6 +85,75 @@ def test_zero_init_on_reuse(dev, shim):
     dev.free(r, 2000)
 
 
+def test_allocator_properties(dev, shim):
+    """device/src/test/proptests.rs restated with hypothesis over random sizes and flags:
+    a freed block is reused for any later request of the same (size, cpu_accessible) key and
+    of no other; a buffer and its views cache exactly one block when both are gone; a reused
+    block requested with zero_init comes back zeroed; the cache never holds more than 32
+    blocks per key whatever the order of allocations and frees."""
+    from hypothesis import given, settings, HealthCheck, strategies as st
+
+    sizes = st.integers(min_value=1, max_value=1 << 16)
+
+    @settings(max_examples=60, deadline=None, suppress_health_check=list(HealthCheck))
+    @given(size=sizes, other=sizes, cpu=st.booleans(), other_cpu=st.booleans())
+    def reuse_by_key(size, other, cpu, other_cpu):
+        dev.lru_clear()
+        p = dev.alloc(size, cpu_accessible=cpu)
+        dev.free(p, size, cpu_accessible=cpu)
+        assert dev.lru_cache_count(size, cpu) == 1
+        q = dev.alloc(other, cpu_accessible=other_cpu)
+        same_key = other == size and other_cpu == cpu
+        assert (q == p) == same_key
+        assert dev.lru_cache_count(size, cpu) == (0 if same_key else 1)
+        dev.free(q, other, cpu_accessible=other_cpu)
+
+    @settings(max_examples=40, deadline=None, suppress_health_check=list(HealthCheck))
+    @given(size=st.integers(min_value=20, max_value=1 << 16), zero=st.booleans())
+    def views_and_zero_init(size, zero):
+        dev.lru_clear()
+        b = morok_amd.Buffer(size)
+        b.ensure_allocated()
+        v = b.view(0, min(size, 10))
+        assert v.id == b.id
+        junk = np.full(size, 0x5A, np.uint8)
+        b.copyin(junk)
+        del v, b
+        assert dev.lru_cache_count(size) == 1           # one block for the buffer and its view together
+        b2 = morok_amd.Buffer(size, zero_init=zero)
+        b2.ensure_allocated()
+        assert dev.lru_cache_count(size) == 0           # reused
+        got = b2.copyout(np.uint8, (size,))
+        assert (not got.any()) if zero else np.all(got == 0x5A)
+        del b2
+
+    @settings(max_examples=15, deadline=None, suppress_health_check=list(HealthCheck))
+    @given(ops=st.lists(st.tuples(st.sampled_from([64, 4096, 65536]), st.booleans()), min_size=1, max_size=120))
+    def capacity(ops):
+        dev.lru_clear()
+        live = []
+        for size, do_free in ops:
+            if do_free and live:
+                p, sz = live.pop()
+                dev.free(p, sz)
+            else:
+                live.append((dev.alloc(size), size))
+            for sz in (64, 4096, 65536):
+                assert dev.lru_cache_count(sz) <= 32
+        many = [dev.alloc(64) for _ in range(50)]
+        for p in many:
+            dev.free(p, 64)
+        assert dev.lru_cache_count(64) == 32
+        for p, sz in live:
+            dev.free(p, sz)
+
+    reuse_by_key()
+    views_and_zero_init()
+    capacity()
+    dev.lru_clear()
+    assert shim.mrk_shim_bytes_in_use() == 0
+
+
 def test_out_of_memory_clears_cache_and_retries(dev, shim):
     """allocator.rs:173-190: on an allocation failure the LRU frees everything it holds and
     retries once; only a second failure is reported."""
