@@ -259,6 +259,13 @@ int mrk_hip_benchmark_kernel(int device_id, mrk_program* p, void* const* buffers
                              size_t nvals, const size_t global_size[3], const size_t local_size[3], int warmup, int runs,
                              double* min_ms, double* mean_ms);
 
+/* benchmark_kernel_with_cutoff (runtime/src/benchmark.rs:100-137): as above, but when the first timed
+ * run takes more than three times cutoff_ms the candidate is given up at once: *skipped = 1 and the
+ * times are those of that one run.  cutoff_ms <= 0 disables the check. */
+int mrk_hip_benchmark_kernel_with_cutoff(int device_id, mrk_program* p, void* const* buffers, size_t nbufs, const int64_t* vals,
+                                         size_t nvals, const size_t global_size[3], const size_t local_size[3], int warmup,
+                                         int runs, double cutoff_ms, double* min_ms, double* mean_ms, int* skipped);
+
 /* TimelineSignal::{set, value, wait(value, timeout_ms)} (device/src/sync.rs:44-71), modelled on
  * CudaTimelineSignal (sync.rs:192-310): one event per recorded value, the last 16 kept.
  * wait returns MRK_ERR_TIMEOUT when the value is not reached in time (sync.rs:118-168). */

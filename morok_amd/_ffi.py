@@ -111,6 +111,9 @@ _SIGS = {
     "mrk_hip_plan_release": (None, [C.c_void_p]),
     "mrk_hip_benchmark_kernel": (C.c_int, [C.c_int, C.c_void_p, c_void_pp, C.c_size_t, c_i64_p, C.c_size_t, c_size_p,
                                            c_size_p, C.c_int, C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]),
+    "mrk_hip_benchmark_kernel_with_cutoff": (C.c_int, [C.c_int, C.c_void_p, c_void_pp, C.c_size_t, c_i64_p, C.c_size_t,
+                                                       c_size_p, c_size_p, C.c_int, C.c_int, C.c_double,
+                                                       C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_int)]),
     "mrk_hip_signal_create": (C.c_int, [C.c_int, c_void_pp]),
     "mrk_hip_signal_set": (C.c_int, [C.c_void_p, C.c_uint64]),
     "mrk_hip_signal_value": (C.c_uint64, [C.c_void_p]),

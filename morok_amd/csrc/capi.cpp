@@ -500,6 +500,22 @@ int mrk_hip_benchmark_kernel(int device_id, mrk_program* p, void* const* buffers
     return kOk;
 }
 
+int mrk_hip_benchmark_kernel_with_cutoff(int device_id, mrk_program* p, void* const* buffers, size_t nbufs, const int64_t* vals,
+                                         size_t nvals, const size_t global_size[3], const size_t local_size[3], int warmup,
+                                         int runs, double cutoff_ms, double* min_ms, double* mean_ms, int* skipped) {
+    MRK_NONNULL(p);
+    std::shared_ptr<Device> d;
+    MRK_TRY(get_device(device_id, &d));
+    BenchmarkResult r;
+    bool sk = false;
+    MRK_TRY(benchmark_kernel_with_cutoff(device_id, d->allocator->stream(), p->p.get(), buffers, nbufs, vals, nvals, global_size,
+                                         local_size, warmup, runs, cutoff_ms, &r, &sk));
+    if (min_ms) *min_ms = r.min_ms;
+    if (mean_ms) *mean_ms = r.mean_ms;
+    if (skipped) *skipped = sk ? 1 : 0;
+    return kOk;
+}
+
 int mrk_hip_signal_create(int device_id, mrk_signal** out) {
     MRK_NONNULL(out);
     std::shared_ptr<Device> d;

@@ -295,17 +295,18 @@ int ExecutionPlan::execute_with_vars(const std::vector<std::pair<std::string, in
     return execute();
 }
 
-int benchmark_kernel(int device_id, ffi::Stream stream, Program* program, void* const* buffers, size_t nbufs,
-                     const int64_t* vals, size_t nvals, const size_t* global, const size_t* local, int warmup,
-                     int runs, BenchmarkResult* out) {
+int benchmark_kernel_with_cutoff(int device_id, ffi::Stream stream, Program* program, void* const* buffers, size_t nbufs,
+                                 const int64_t* vals, size_t nvals, const size_t* global, const size_t* local, int warmup,
+                                 int runs, double cutoff_ms, BenchmarkResult* out, bool* skipped) {
     if (runs <= 0) return fail(kInvalidArgument, "benchmark: runs must be positive");
+    if (skipped) *skipped = false;
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
     for (int i = 0; i < warmup; i++) MRK_TRY(program->execute(buffers, nbufs, vals, nvals, global, local));
     ffi::Event e0 = nullptr, e1 = nullptr;
     MRK_HIP(ffi::event_create(&e0), "hipEventCreate");
     MRK_HIP(ffi::event_create(&e1), "hipEventCreate");
     double mn = 1e300, mx = 0, sum = 0;
-    int rc = kOk;
+    int rc = kOk, done = 0;
     for (int i = 0; i < runs && rc == kOk; i++) {
         ffi::event_record(e0, stream);
         rc = program->execute(buffers, nbufs, vals, nvals, global, local);
@@ -320,19 +321,32 @@ int benchmark_kernel(int device_id, ffi::Stream stream, Program* program, void* 
         mn = ms < mn ? ms : mn;
         mx = ms > mx ? ms : mx;
         sum += ms;
+        done++;
+        if (i == 0 && cutoff_ms > 0.0 && ms > 3.0 * cutoff_ms) {  // clearly slower: benchmark.rs:119-122
+            if (skipped) *skipped = true;
+            break;
+        }
     }
     ffi::event_destroy(e0);
     ffi::event_destroy(e1);
     if (rc != kOk) return rc;
     out->min_ms = mn;
     out->max_ms = mx;
-    out->mean_ms = sum / runs;
-    out->runs = runs;
+    out->mean_ms = sum / (done ? done : 1);
+    out->runs = done;
     return kOk;
 }
 
+int benchmark_kernel(int device_id, ffi::Stream stream, Program* program, void* const* buffers, size_t nbufs,
+                     const int64_t* vals, size_t nvals, const size_t* global, const size_t* local, int warmup,
+                     int runs, BenchmarkResult* out) {
+    return benchmark_kernel_with_cutoff(device_id, stream, program, buffers, nbufs, vals, nvals, global, local, warmup, runs, 0.0, out,
+                                        nullptr);
+}
+
 int compile_and_time(const Device& dev, const LinearKernel& k, const char* name, void* const* buffers, size_t nbufs,
-                     const int64_t* vals, size_t nvals, int warmup, int runs, BenchmarkResult* out) {
+                     const int64_t* vals, size_t nvals, int warmup, int runs, BenchmarkResult* out, double cutoff_ms,
+                     bool* skipped) {
     ProgramSpec spec;
     MRK_TRY(dev.renderer->render(k, name, &spec));
     if (spec.buf_count != nbufs)
@@ -343,9 +357,9 @@ int compile_and_time(const Device& dev, const LinearKernel& k, const char* name,
     MRK_TRY(dev.runtime(compiled, &program));
     static std::mutex timing_lock;
     std::lock_guard<std::mutex> lock(timing_lock);
-    return benchmark_kernel(dev.device_id, dev.allocator->stream(), program.get(), buffers, nbufs, vals, nvals,
-                            spec.has_sizes ? spec.global_size.data() : nullptr,
-                            spec.has_sizes ? spec.local_size.data() : nullptr, warmup, runs, out);
+    return benchmark_kernel_with_cutoff(dev.device_id, dev.allocator->stream(), program.get(), buffers, nbufs, vals, nvals,
+                                        spec.has_sizes ? spec.global_size.data() : nullptr,
+                                        spec.has_sizes ? spec.local_size.data() : nullptr, warmup, runs, cutoff_ms, out, skipped);
 }
 
 std::string BeamCache::directory() {
@@ -446,14 +460,20 @@ int beam_search_matmul_f32(const Device& dev, int64_t M, int64_t N, int64_t K, i
     MRK_TRY(b.as_raw_ptr(&ptrs[2]));
 
     using Cand = std::pair<double, MatmulF32Opts>;
+    double best_so_far = 1e300;
     auto time_one = [&](const MatmulF32Opts& o, double* ms) -> bool {
         if (!matmul_f32_opts_valid(o, M, N, K)) return false;
         BenchmarkResult r;
         LinearKernel k = build_matmul_f32_kernel(M, N, K, o);
-        // warm-up 1, 3 runs, minimum: runtime/src/benchmark.rs:23-27
-        if (compile_and_time(dev, k, "beam_candidate", ptrs, 3, nullptr, 0, 1, 3, &r) != kOk) return false;  // a failing candidate is skipped
+        // warm-up 1, 3 runs, minimum: runtime/src/benchmark.rs:23-27; a candidate clearly slower
+        // than three times the best so far is dropped after its first run (beam.rs:309-355)
+        bool skipped = false;
+        if (compile_and_time(dev, k, "beam_candidate", ptrs, 3, nullptr, 0, 1, 3, &r, best_so_far < 1e300 ? 3.0 * best_so_far : 0.0, &skipped) != kOk)
+            return false;  // a failing candidate is skipped
         if (candidates_timed) (*candidates_timed)++;
+        if (skipped) return false;
         *ms = r.min_ms;
+        best_so_far = std::min(best_so_far, r.min_ms);
         return true;
     };
     auto keep_best = [&](std::vector<Cand>& v) {
@@ -561,6 +581,7 @@ int beam_search_wmma_matmul(const Device& dev, const TensorCore& tc, int tc_inde
         return x.waves_m == y.waves_m && x.waves_n == y.waves_n && x.up_m == y.up_m && x.up_n == y.up_n && x.unroll_k == y.unroll_k;
     };
     std::vector<WmmaLdsOpts> tried;
+    double best_so_far = 1e300;
     auto time_one = [&](const WmmaLdsOpts& o, double* ms) -> bool {
         if (!wmma_lds_opts_valid(tc, o, M, N, K)) return false;
         for (const WmmaLdsOpts& t : tried)
@@ -569,9 +590,13 @@ int beam_search_wmma_matmul(const Device& dev, const TensorCore& tc, int tc_inde
         LinearKernel k;
         if (build_wmma_matmul_lds_kernel(tc, M, N, K, tc.dtype_in, o, &k) != kOk) return false;
         BenchmarkResult r;
-        if (compile_and_time(dev, k, "beam_candidate", ptrs, 3, nullptr, 0, 1, 3, &r) != kOk) return false;
+        bool skipped = false;
+        if (compile_and_time(dev, k, "beam_candidate", ptrs, 3, nullptr, 0, 1, 3, &r, best_so_far < 1e300 ? 3.0 * best_so_far : 0.0, &skipped) != kOk)
+            return false;
         if (candidates_timed) (*candidates_timed)++;
+        if (skipped) return false;
         *ms = r.min_ms;
+        best_so_far = std::min(best_so_far, r.min_ms);
         return true;
     };
     auto keep_best = [&](std::vector<Cand>& v) {

@@ -140,6 +140,12 @@ struct BenchmarkResult {
 int benchmark_kernel(int device_id, ffi::Stream stream, Program* program, void* const* buffers, size_t nbufs,
                      const int64_t* vals, size_t nvals, const size_t* global, const size_t* local, int warmup,
                      int runs, BenchmarkResult* out);
+// runtime/src/benchmark.rs:100-137: the same, but a candidate whose first timed run takes more than
+// three times `cutoff_ms` is given up at once (*skipped = true, nothing else is filled in): a
+// beam search spends no further launches on it.  cutoff_ms <= 0 disables the check.
+int benchmark_kernel_with_cutoff(int device_id, ffi::Stream stream, Program* program, void* const* buffers, size_t nbufs,
+                                 const int64_t* vals, size_t nvals, const size_t* global, const size_t* local, int warmup,
+                                 int runs, double cutoff_ms, BenchmarkResult* out, bool* skipped);
 
 // Beam-search timing hook (tensor/src/realize.rs:1190-1242): render and compile `k` (not timed),
 // load it, then time only the execution with HIP events.  Candidates are timed one at a time
@@ -147,7 +153,8 @@ int benchmark_kernel(int device_id, ffi::Stream stream, Program* program, void* 
 // kernel.  A candidate that fails to render, compile or launch yields a status, never an
 // abort (the reference wraps this in catch_unwind).
 int compile_and_time(const Device& dev, const LinearKernel& k, const char* name, void* const* buffers, size_t nbufs,
-                     const int64_t* vals, size_t nvals, int warmup, int runs, BenchmarkResult* out);
+                     const int64_t* vals, size_t nvals, int warmup, int runs, BenchmarkResult* out, double cutoff_ms = 0.0,
+                     bool* skipped = nullptr);
 
 // On-disk cache of search results keyed (ast_hash, beam_width, device), the role sled plays in
 // schedule/src/optimizer/beam.rs:390-440: one small file per key under

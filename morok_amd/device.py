@@ -504,6 +504,20 @@ def benchmark_kernel(program, buffers, vals=(), global_size=None, local_size=Non
     return mn.value, mean.value
 
 
+def benchmark_kernel_with_cutoff(program, buffers, cutoff_ms, vals=(), global_size=None, local_size=None, warmup=1, runs=3,
+                                 device_id=0):
+    """benchmark_kernel_with_cutoff (runtime/src/benchmark.rs:100-137): None when the first timed
+    run took more than three times `cutoff_ms` (the candidate is given up), else (min_ms, mean_ms)."""
+    ptrs = [b.ptr if isinstance(b, Buffer) else int(b) for b in buffers]
+    parr = (C.c_void_p * max(len(ptrs), 1))(*ptrs)
+    varr = (C.c_int64 * max(len(vals), 1))(*[int(v) for v in vals])
+    mn, mean, skipped = C.c_double(), C.c_double(), C.c_int()
+    check(lib.mrk_hip_benchmark_kernel_with_cutoff(device_id, program._h, parr, len(ptrs), varr, len(vals), _size3(global_size),
+                                                   _size3(local_size), warmup, runs, float(cutoff_ms), C.byref(mn),
+                                                   C.byref(mean), C.byref(skipped)))
+    return None if skipped.value else (mn.value, mean.value)
+
+
 class TimelineSignal:
     """TimelineSignal over HIP events (device/src/sync.rs:44-71,192-310)."""
 

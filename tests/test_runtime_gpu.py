@@ -116,6 +116,20 @@ def test_benchmark_kernel_protocol(dev):
         morok_amd.benchmark_kernel(prog, [by, bx], runs=0, device_id=dev.device_id)
 
 
+def test_benchmark_kernel_with_cutoff(dev):
+    """runtime/src/benchmark.rs:178-197: a kernel within the cutoff is timed in full, one whose
+    first run exceeds three times the cutoff is given up."""
+    rows = cols = 4096
+    bx = dev.buffer(rows * cols * 4).ensure_allocated()
+    by = dev.buffer(rows * cols * 4).ensure_allocated()
+    ops.fill_normal(bx, rows * cols, seed=5)
+    prog = morok_amd.Program.builtin("softmax_f32", [rows, cols], dev.device_id)
+    res = morok_amd.benchmark_kernel_with_cutoff(prog, [by, bx], cutoff_ms=50.0, device_id=dev.device_id)
+    assert res is not None and 0 < res[0] <= res[1]
+    assert morok_amd.benchmark_kernel_with_cutoff(prog, [by, bx], cutoff_ms=res[0] / 100.0, device_id=dev.device_id) is None
+    assert morok_amd.benchmark_kernel_with_cutoff(prog, [by, bx], cutoff_ms=0.0, device_id=dev.device_id) is not None
+
+
 def test_timeline_signal(dev):
     s = morok_amd.TimelineSignal(dev.device_id)
     assert s.value == 0
