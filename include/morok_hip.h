@@ -515,6 +515,8 @@ int mrk_hip_tensor_gemm(const mrk_tensor* a, const mrk_tensor* b, float alpha, f
 /* x @ weight^T + bias, weight [out, in] (1-D weight: elementwise product), bias may be NULL (matmul.rs:160-190) */
 int mrk_hip_tensor_linear(const mrk_tensor* x, const mrk_tensor* weight, const mrk_tensor* bias, int acc_dtype, mrk_tensor** out);
 int mrk_hip_tensor_softmax(const mrk_tensor* t, int64_t axis, mrk_tensor** out);              /* activation.rs:90-101 */
+int mrk_hip_tensor_log_softmax(const mrk_tensor* t, int64_t axis, mrk_tensor** out);          /* activation.rs:117-128 */
+int mrk_hip_tensor_logsumexp(const mrk_tensor* t, int64_t axis, mrk_tensor** out);            /* activation.rs:143-157 */
 int mrk_hip_tensor_rms_norm(const mrk_tensor* t, int64_t axis, double eps, mrk_tensor** out); /* nn/norm.rs:92-111 */
 int mrk_hip_tensor_embedding(const mrk_tensor* weight, const mrk_tensor* indices, mrk_tensor** out); /* transformer.rs:12-25 */
 int mrk_hip_tensor_rotary(const mrk_tensor* x, const mrk_tensor* cos, const mrk_tensor* sin, int interleaved,

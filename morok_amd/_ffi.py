@@ -206,6 +206,8 @@ _SIGS = {
     "mrk_hip_tensor_gemm": (C.c_int, [C.c_void_p, C.c_void_p, C.c_float, C.c_float, C.c_int, C.c_int, C.c_void_p, c_void_pp]),
     "mrk_hip_tensor_linear": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, c_void_pp]),
     "mrk_hip_tensor_softmax": (C.c_int, [C.c_void_p, C.c_int64, c_void_pp]),
+    "mrk_hip_tensor_log_softmax": (C.c_int, [C.c_void_p, C.c_int64, c_void_pp]),
+    "mrk_hip_tensor_logsumexp": (C.c_int, [C.c_void_p, C.c_int64, c_void_pp]),
     "mrk_hip_tensor_rms_norm": (C.c_int, [C.c_void_p, C.c_int64, C.c_double, c_void_pp]),
     "mrk_hip_tensor_embedding": (C.c_int, [C.c_void_p, C.c_void_p, c_void_pp]),
     "mrk_hip_tensor_rotary": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, c_void_pp]),

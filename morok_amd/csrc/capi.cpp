@@ -1144,6 +1144,14 @@ int mrk_hip_tensor_linear(const mrk_tensor* x, const mrk_tensor* weight, const m
     if (acc_dtype < -1 || acc_dtype >= static_cast<int>(Scalar::Void)) return fail(kInvalidArgument, "linear: unknown dtype tag");
     return wrap_tensor(x->t.linear(weight->t, bias ? &bias->t : nullptr, acc_dtype < 0 ? Scalar::Void : static_cast<Scalar>(acc_dtype)), out);
 }
+int mrk_hip_tensor_log_softmax(const mrk_tensor* t, int64_t axis, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.log_softmax(axis), out);
+}
+int mrk_hip_tensor_logsumexp(const mrk_tensor* t, int64_t axis, mrk_tensor** out) {
+    MRK_T1(t);
+    return wrap_tensor(t->t.logsumexp(axis), out);
+}
 int mrk_hip_tensor_softmax(const mrk_tensor* t, int64_t axis, mrk_tensor** out) {
     MRK_T1(t);
     return wrap_tensor(t->t.softmax(axis), out);

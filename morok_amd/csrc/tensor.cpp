@@ -474,6 +474,24 @@ Tensor Tensor::softmax(int64_t axis) const {
     return res;
 }
 
+Tensor Tensor::log_softmax(int64_t axis) const {
+    // x - max(x) - log(sum(exp(x - max(x))))  (activation.rs:117-128)
+    if (!n_) return Tensor();
+    if (!norm_axis(&axis, ndim())) return bad(kInvalidArgument, "log_softmax: axis out of range");
+    Tensor shifted = try_sub(reduce(ReduceOp::Max, {axis}, true, false));
+    Tensor s = shifted.try_exp().reduce(ReduceOp::Add, {axis}, true, false);
+    return shifted.try_sub(s.unary(UnaryOp::Log));
+}
+
+Tensor Tensor::logsumexp(int64_t axis) const {
+    // max(x) + log(sum(exp(x - max(x)))), the kept axis dropped by a max over it  (activation.rs:143-157)
+    if (!n_) return Tensor();
+    if (!norm_axis(&axis, ndim())) return bad(kInvalidArgument, "logsumexp: axis out of range");
+    Tensor m = reduce(ReduceOp::Max, {axis}, true, false);
+    Tensor s = try_sub(m).try_exp().reduce(ReduceOp::Add, {axis}, true, false);
+    return m.try_add(s.unary(UnaryOp::Log)).reduce(ReduceOp::Max, {axis}, false, false);
+}
+
 Tensor Tensor::rms_norm(int64_t axis, double eps) const {
     if (!n_) return Tensor();
     if (!norm_axis(&axis, ndim())) return bad(kInvalidArgument, "rms_norm: axis out of range");

@@ -135,6 +135,8 @@ class Tensor {
     // self @ weight^T + bias, weight [out, in] (a 1-D weight multiplies elementwise); matmul.rs:160-190
     Tensor linear(const Tensor& weight, const Tensor* bias, Scalar acc = Scalar::Void) const;
     Tensor softmax(int64_t axis) const;                                     // activation.rs:90-101
+    Tensor log_softmax(int64_t axis) const;  // activation.rs:117-128
+    Tensor logsumexp(int64_t axis) const;    // activation.rs:143-157
     Tensor rms_norm(int64_t axis, double eps) const;                        // nn/norm.rs:92-111
     Tensor embedding(const Tensor& indices) const;                          // transformer.rs:12-25
     Tensor apply_rotary_emb(const Tensor& cos, const Tensor& sin, bool interleaved) const;  // transformer.rs:32-69

@@ -257,6 +257,12 @@ class Tensor:
     def softmax(self, axis=-1):
         return self._new(lib.mrk_hip_tensor_softmax, axis)
 
+    def log_softmax(self, axis=-1):
+        return self._new(lib.mrk_hip_tensor_log_softmax, axis)
+
+    def logsumexp(self, axis=-1):
+        return self._new(lib.mrk_hip_tensor_logsumexp, axis)
+
     def rms_norm(self, axis=-1, eps=1e-5):
         return self._new(lib.mrk_hip_tensor_rms_norm, axis, float(eps))
 

@@ -240,6 +240,24 @@ def test_softmax(T, fusion, oracle, shape):
     assert (got > 0).all() and (got <= 1).all()
 
 
+@pytest.mark.parametrize("axis", [-1, 0, 1])
+def test_log_softmax_and_logsumexp(T, fusion, axis):
+    """activation.rs:117-157 against float64 closed forms, including rows whose naive
+    exp would overflow."""
+    rng = np.random.default_rng(91)
+    x = (rng.standard_normal((6, 50, 33)) * 30).astype(np.float32)
+    x[0, 0] += 500.0
+    x64 = x.astype(np.float64)
+    m = x64.max(axis, keepdims=True)
+    lse = m + np.log(np.exp(x64 - m).sum(axis, keepdims=True))
+    got = T.Tensor.from_numpy(x).log_softmax(axis).to_numpy()
+    np.testing.assert_allclose(got, x64 - lse, rtol=1e-5, atol=1e-4)
+    got = T.Tensor.from_numpy(x).logsumexp(axis).to_numpy()
+    assert got.shape == np.squeeze(lse, axis).shape
+    np.testing.assert_allclose(got, np.squeeze(lse, axis), rtol=1e-5, atol=1e-4)
+    assert np.allclose(np.exp(T.Tensor.from_numpy(x).log_softmax(axis).to_numpy().astype(np.float64)).sum(axis), 1.0, atol=1e-4)
+
+
 def test_softmax_inner_axis(T, oracle):
     rng = np.random.default_rng(12)
     x = rng.standard_normal((6, 33, 5)).astype(np.float32)
