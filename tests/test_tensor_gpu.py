@@ -911,6 +911,23 @@ def test_random_movement_chains(T, seed):
         np.testing.assert_array_equal(t.sum([ax]).to_numpy(), a.sum(ax))
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_movement_chains_power_of_two_shapes(T, seed):
+    """The same with extents that are powers of two up to 128: whole upcast groups, whole waves,
+    the shapes on which the generator takes its vector-load, split-group and per-part paths."""
+    rng = np.random.default_rng(50000 + seed)
+    shape = [int(rng.choice([1, 2, 4, 8, 16, 32, 64, 128])) for _ in range(int(rng.integers(1, 5)))]
+    while np.prod(shape) > 1 << 20:
+        shape[int(rng.integers(0, len(shape)))] = 2
+    x = rng.integers(-8, 8, size=shape).astype(np.float32)
+    a, t = _random_graph(T, rng, x, T.Tensor.from_numpy(x))
+    assert t.shape == a.shape
+    np.testing.assert_array_equal(t.to_numpy(), a)
+    if a.ndim:
+        ax = int(rng.integers(0, a.ndim))
+        np.testing.assert_array_equal(t.sum([ax]).to_numpy(), a.sum(ax))
+
+
 def test_matmul_bf16_few_rows_uses_split_k(T, oracle):
     """A handful of rows against a large weight matrix through the tensor API: the scheduler
     adds the split-K scratch to the plan as an intermediate buffer."""
