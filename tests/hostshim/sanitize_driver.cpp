@@ -1,7 +1,9 @@
 // Native driver of the host runtime for sanitizer builds (AddressSanitizer + UBSan, or
-// ThreadSanitizer): four threads create buffers and tensors, realize and prepare graphs, replay
-// plans eagerly, profiled and as graphs, and use queues and signals, all through the C ABI and
-// against the host-memory stand-ins of this directory.  TEST INFRASTRUCTURE ONLY.
+// ThreadSanitizer): four threads create buffers and tensors, realize and prepare graphs (among
+// them attention over strided views, masked attention, rotary embeddings, vector products),
+// replay plans eagerly, profiled and as graphs, build tensor-core kernels over the whole tile
+// search space, and use queues and signals, all through the C ABI and against the host-memory
+// stand-ins of this directory.  TEST INFRASTRUCTURE ONLY.
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -51,6 +53,72 @@ static int work(int id) {
     std::vector<double> prof(16); size_t n = 0;
     CK(mrk_hip_plan_execute_profiled(plan, prof.data(), 16, &n));
     mrk_hip_plan_release(plan);
+    // the scheduler's view analysis and kernel splitting: attention over slices of a packed bf16
+    // product with the result permuted back (strided kernel), masked attention (composed graph),
+    // rotary embedding in both layouts (per-part regions, split upcast groups), vector matmul
+    {
+        const int64_t B = 1, S = 128, H = 2, D = 128, hid = H * D;
+        int64_t ps[2] = {B * S, 3 * hid};
+        std::vector<uint16_t> packed(static_cast<size_t>(ps[0] * ps[1]), 0x3f80);
+        mrk_tensor* pk = nullptr;
+        CK(mrk_hip_tensor_from_bytes(0, packed.data(), packed.size() * 2, ps, 2, 10 /*bf16*/, &pk));
+        mrk_tensor* qkv[3] = {nullptr, nullptr, nullptr};
+        std::vector<mrk_tensor*> tmp;
+        for (int i = 0; i < 3; i++) {
+            int64_t b0[2] = {0, i * hid}, e0[2] = {B * S, (i + 1) * hid}, r4[4] = {B, S, H, D}, perm[4] = {0, 2, 1, 3};
+            mrk_tensor *a = nullptr, *b4 = nullptr;
+            CK(mrk_hip_tensor_shrink(pk, b0, e0, 2, &a));
+            CK(mrk_hip_tensor_reshape(a, r4, 4, &b4));
+            CK(mrk_hip_tensor_permute(b4, perm, 4, &qkv[i]));
+            tmp.push_back(a);
+            tmp.push_back(b4);
+        }
+        mrk_tensor *att = nullptr, *back = nullptr, *flat = nullptr;
+        CK(mrk_hip_tensor_sdpa(qkv[0], qkv[1], qkv[2], 0.0, 1, &att));
+        int64_t perm[4] = {0, 2, 1, 3}, r2[2] = {B * S, hid};
+        CK(mrk_hip_tensor_permute(att, perm, 4, &back));
+        CK(mrk_hip_tensor_reshape(back, r2, 2, &flat));
+        CK(mrk_hip_tensor_realize(flat));
+        if (mrk_hip_tensor_last_kernel_count() != 1 || !strstr(mrk_hip_tensor_last_kernel_name(0), "strided")) {
+            printf("attention over views did not take the strided kernel\n");
+            return 1;
+        }
+        int64_t ms[2] = {S, S};
+        std::vector<float> maskv(static_cast<size_t>(S * S), 0.0f);
+        mrk_tensor *mask = nullptr, *att2 = nullptr;
+        CK(mrk_hip_tensor_from_bytes(0, maskv.data(), maskv.size() * 4, ms, 2, 11, &mask));
+        CK(mrk_hip_tensor_sdpa_ex(qkv[0], qkv[1], qkv[2], mask, 0.0, 0, 2.0, &att2));
+        CK(mrk_hip_tensor_realize(att2));
+        int64_t xs[4] = {2, 16, 4, 128}, cs[4] = {1, 16, 1, 64};
+        std::vector<float> xv(2 * 16 * 4 * 128, 0.5f), cv(16 * 64, 1.0f);
+        mrk_tensor *xr = nullptr, *c = nullptr, *r0 = nullptr, *r1 = nullptr;
+        CK(mrk_hip_tensor_from_bytes(0, xv.data(), xv.size() * 4, xs, 4, 11, &xr));
+        CK(mrk_hip_tensor_from_bytes(0, cv.data(), cv.size() * 4, cs, 4, 11, &c));
+        CK(mrk_hip_tensor_rotary(xr, c, c, 0, &r0));
+        CK(mrk_hip_tensor_rotary(xr, c, c, 1, &r1));
+        CK(mrk_hip_tensor_realize(r0));
+        CK(mrk_hip_tensor_realize(r1));
+        int64_t vs[1] = {64};
+        mrk_tensor *vec = nullptr, *dot = nullptr, *mv = nullptr, *lin = nullptr;
+        CK(mrk_hip_tensor_from_bytes(0, x.data(), 64 * 4, vs, 1, 11, &vec));
+        CK(mrk_hip_tensor_matmul(vec, vec, &dot));
+        CK(mrk_hip_tensor_matmul(t, vec, &mv));
+        CK(mrk_hip_tensor_linear(t, t, vec, -1, &lin));
+        CK(mrk_hip_tensor_realize(dot));
+        CK(mrk_hip_tensor_realize(mv));
+        CK(mrk_hip_tensor_realize(lin));
+        for (mrk_tensor* p : {pk, qkv[0], qkv[1], qkv[2], att, back, flat, mask, att2, xr, c, r0, r1, vec, dot, mv, lin}) mrk_hip_tensor_release(p);
+        for (mrk_tensor* p : tmp) mrk_hip_tensor_release(p);
+        // tensor-core kernel builders: every tile choice of the search space on a padded shape
+        for (int wm : {1, 2, 4})
+            for (int wn : {1, 2, 4})
+                for (int um : {1, 4, 8}) {
+                    int opts[5] = {wm, wn, um, 2, id % 3};
+                    uint8_t* kern = nullptr;
+                    size_t len = 0;
+                    if (mrk_hip_sched_build_wmma_matmul_lds_opts(1, 200 + id, 136, 72, 10, opts, &kern, &len) == 0) mrk_hip_sched_free(kern);
+                }
+    }
     for (mrk_tensor* p : {t, u, w, s, m}) mrk_hip_tensor_release(p);
     // queues and signals
     mrk_queue* q = nullptr; mrk_signal* sig = nullptr;
