@@ -223,7 +223,7 @@ def bench_decoder(m, dev, steps, warmup, cpu):
         "config": {"workload": "decoder block via tensor API: hidden 4096, 32x128 heads, SwiGLU 11008, batch 4 x seq 2048 "
                                "prefill (configs[4])"},
         "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None, "kernel": f"gemm_bf16_tile256 ({sum(n.startswith('gemm_bf16') for n, _ in prof)} of the {len(prof)} kernels)",
+                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None, "kernel": f"gemm_bf16_tile256[_residual] ({sum(n.startswith('gemm_bf16') for n, _ in prof)} of the {len(prof)} kernels)",
                      "algorithmic_flops_per_launch": flops},
         "kernels": len(prof), "gemm_ms": gemm_ms, "flash_ms": flash_ms, "other_ms": sum(t for _, t in prof) - gemm_ms - flash_ms,
     }

@@ -195,6 +195,7 @@ void mrk_hip_program_destroy(mrk_program* p);
  *                     (batch: that many products over matrices stored back to back)
  *                     params = {M, N, K, batch, workspace bytes}    buffers = {c, a, b, workspace}
  *                     (split-K for shapes with few output tiles; size from mrk_hip_gemm_bf16_workspace_bytes)
+ *   "gemm_bf16_residual"  params = {M, N, K} or {M, N, K, batch}  buffers = {c, a, b, r}   (c = a b + r)
  *   "flash_fwd_bf16"  params = {B*H, Sq, Sk, D, causal, f32 bits of scale}   buffers = {o, q, k, v}
  *   "flash_fwd_bf16_strided"  params = {B, H, Sq, Sk, D, causal, f32 bits of scale, element offsets
  *                     of q k v o into their buffers (4), (batch, head, row) element strides of
@@ -415,6 +416,14 @@ size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_
  * with the 256-row / 128-row tile); tuning/tests. */
 int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
                                int variant);
+
+/* c = bf16(float(bf16(a b)) + float(r)): the product above with a bf16 matrix r of c's shape added
+ * in the kernel's epilogue - the bits of mrk_hip_gemm_bf16 followed by an elementwise add
+ * (Tensor::matmul + try_add, tensor/src/matmul.rs:82-110), without the round trip of the product
+ * through memory.  INVALID_ARGUMENT for shapes the fused epilogue does not cover (N or K not a
+ * multiple of 8, K = 0, or so few output tiles that split-K is used). */
+int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, const void* r, void* c, int64_t m, int64_t n,
+                               int64_t k);
 
 /* Scaled dot-product attention forward in one kernel (online softmax, f32 scores and
  * statistics, P rounded to bf16 before the second product, bf16 output):

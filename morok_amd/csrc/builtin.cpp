@@ -93,6 +93,20 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
+    if (k == "gemm_bf16_residual") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, b, r}
+        if (nparams < 3 || nparams > 4)
+            return failf(kInvalidArgument, "builtin 'gemm_bf16_residual' takes 3 or 4 parameters, got %zu", nparams);
+        while (p.size() < 4) p.push_back(1);
+        if (!gemm_bf16_residual_supported(p[0], p[1], p[2], p[3]))
+            return fail(kInvalidArgument, "gemm_bf16_residual: shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel)");
+        std::string name = "gemm_bf16_residual_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+        if (p[3] > 1) name += "_x" + std::to_string(p[3]);
+        out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
+                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16_residual(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3]);
+                                      }));
+        return kOk;
+    }
     if (k == "flash_fwd_bf16") {
         MRK_TRY(need(6));
         if (p[0] < 0 || p[1] < 0 || p[2] <= 0 || p[3] != 128)

@@ -872,6 +872,23 @@ int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int6
     return mrk_hip_gemm_bf16_variant(device_id, a, b, c, m, n, k, 0);
 }
 
+int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, const void* r, void* c, int64_t m, int64_t n, int64_t k) {
+    if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_residual: negative shape");
+    if (m == 0 || n == 0) return kOk;
+    MRK_NONNULL(a);
+    MRK_NONNULL(b);
+    MRK_NONNULL(r);
+    MRK_NONNULL(c);
+    if (!gemm_bf16_residual_supported(m, n, k, 1))
+        return fail(kInvalidArgument, "gemm_bf16_residual: shape not covered by the fused epilogue (N and K multiples of 8, K > 0, "
+                                      "enough output tiles that split-K is not used); run mrk_hip_gemm_bf16 and add separately");
+    std::shared_ptr<Device> dv;
+    MRK_TRY(get_device(device_id, &dv));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_gemm_bf16_residual(dv->allocator->stream(), a, b, r, c, m, n, k, 1), "gemm_bf16_residual launch");
+    return kOk;
+}
+
 int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
                                 int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal) {
     if (batch < 0 || heads < 0 || sq < 0 || sk < 0) return fail(kInvalidArgument, "flash_attn_fwd: negative shape");

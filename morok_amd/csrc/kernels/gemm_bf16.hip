@@ -47,6 +47,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
@@ -93,10 +94,15 @@ __device__ __attribute__((aligned(16))) const unsigned g_zero16[4] = {0u, 0u, 0u
 // partial tile to W[z][batch][M][N] instead of C and gemm_splitk_reduce adds the partials up in
 // a fixed order.  For shapes with so few tiles that the K loop itself has to be spread over
 // the chip (a handful of rows against a large weight matrix).
-template <bool kRaggedK, int kJ, bool kSplitK = false>
+//
+// kResidual: the epilogue adds a bf16 matrix R of C's shape to the rounded product,
+// C = bf16(float(bf16(A B)) + float(R)): the bits of the product kernel followed by an
+// elementwise add, without writing and re-reading the product.
+template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false>
 __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
-                                               float* __restrict__ W = nullptr, int kt_per_split = 0) {
+                                               float* __restrict__ W = nullptr, int kt_per_split = 0,
+                                               const __bf16* __restrict__ R = nullptr) {
     constexpr int kTM = kJ == 4 ? 256 : 128;      // rows of the workgroup tile
     constexpr int kAq = kTM / 32;                 // 1 KB A chunks (8 rows) each wave copies per K step
     constexpr int kAStageT = kTM * kBK * 2;       // bytes of an A stage
@@ -114,6 +120,7 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     A += (size_t)blockIdx.y * M * K;
     B += (size_t)blockIdx.y * K * N;
     if (!kSplitK) C += (size_t)blockIdx.y * M * N;
+    if (kResidual) R += (size_t)blockIdx.y * M * N;
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
     const size_t m0 = (size_t)tile_m * kTM, n0 = (size_t)tile_n * kBN;
@@ -324,6 +331,26 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         return;
     }
     char* sC = smem + wave * kCWaveT;
+    const size_t row0 = m0 + wm * 128, col0 = n0 + wn * (kJ * 32);
+    constexpr int kChunks = kJ * 4;          // 16-byte chunks per row of the wave's tile
+    constexpr int kRowsPerIt = 64 / kChunks;  // rows one store instruction covers
+    constexpr int kIts = 128 / kRowsPerIt;
+    // the residual rows this lane will add are fetched ahead, in two batches, so that their latency
+    // overlaps the staging of the accumulators instead of sitting in front of every store
+    // (half of them while the accumulators are still live, the other half once they are staged:
+    // all of them at once would not fit the register file next to the accumulators)
+    u32x4 res[kResidual ? kIts : 1];
+    auto fetch_residual = [&](int first, int last) {
+#pragma unroll
+        for (int it = first; it < last; it++) {
+            const int r = it * kRowsPerIt + lane / kChunks;
+            const int ch = lane % kChunks;
+            res[it] = u32x4{0u, 0u, 0u, 0u};
+            if (row0 + r < (size_t)M && col0 + ch * 8 + 8 <= (size_t)N)
+                res[it] = *reinterpret_cast<const u32x4*>(R + (row0 + r) * N + col0 + ch * 8);
+        }
+    };
+    if constexpr (kResidual) fetch_residual(0, kIts / 2);
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -336,17 +363,28 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
                 const int nl = j * 32 + 8 * g + 4 * (lane >> 5);
                 *LDS_PTR(bf16x4, sC + ml * kCPitchT + nl * 2) = h;
             }
+    if constexpr (kResidual) fetch_residual(kIts / 2, kIts);
     __syncthreads();
-    const size_t row0 = m0 + wm * 128, col0 = n0 + wn * (kJ * 32);
     __bf16* Cg = C + row0 * N + col0;
-    constexpr int kChunks = kJ * 4;          // 16-byte chunks per row of the wave's tile
-    constexpr int kRowsPerIt = 64 / kChunks;  // rows one store instruction covers
+    if constexpr (kResidual) {
+#pragma unroll
+        for (int it = 0; it < kIts; it++) {
+            const int r = it * kRowsPerIt + lane / kChunks;
+            const int ch = lane % kChunks;
+            u32x4 v = *LDS_PTR(u32x4, sC + r * kCPitchT + ch * 16);
+            const f32x8 sum = __builtin_convertvector(__builtin_bit_cast(bf16x8, v), f32x8) +
+                              __builtin_convertvector(__builtin_bit_cast(bf16x8, res[it]), f32x8);
+            v = __builtin_bit_cast(u32x4, __builtin_convertvector(sum, bf16x8));
+            if (row0 + r < (size_t)M && col0 + ch * 8 + 8 <= (size_t)N) *reinterpret_cast<u32x4*>(Cg + (size_t)r * N + ch * 8) = v;
+        }
+    } else {
 #pragma unroll 4
-    for (int it = 0; it < 128 / kRowsPerIt; it++) {
-        const int r = it * kRowsPerIt + lane / kChunks;
-        const int ch = lane % kChunks;
-        u32x4 v = *LDS_PTR(u32x4, sC + r * kCPitchT + ch * 16);
-        if (row0 + r < (size_t)M && col0 + ch * 8 + 8 <= (size_t)N) *reinterpret_cast<u32x4*>(Cg + (size_t)r * N + ch * 8) = v;
+        for (int it = 0; it < kIts; it++) {
+            const int r = it * kRowsPerIt + lane / kChunks;
+            const int ch = lane % kChunks;
+            u32x4 v = *LDS_PTR(u32x4, sC + r * kCPitchT + ch * 16);
+            if (row0 + r < (size_t)M && col0 + ch * 8 + 8 <= (size_t)N) *reinterpret_cast<u32x4*>(Cg + (size_t)r * N + ch * 8) = v;
+        }
     }
 }
 
@@ -359,6 +397,28 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256_ragged_k(const __bf16* 
                                                                   const __bf16* __restrict__ B, __bf16* __restrict__ C,
                                                                   int M, int N, int K, int tiles_m, int tiles_n) {
     gemm_tile_body<true, 4>(A, B, C, M, N, K, tiles_m, tiles_n);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile256_residual(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                                  const __bf16* __restrict__ R, __bf16* __restrict__ C, int M,
+                                                                  int N, int K, int tiles_m, int tiles_n) {
+    gemm_tile_body<false, 4, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile256_residual_ragged_k(const __bf16* __restrict__ A,
+                                                                           const __bf16* __restrict__ B,
+                                                                           const __bf16* __restrict__ R, __bf16* __restrict__ C,
+                                                                           int M, int N, int K, int tiles_m, int tiles_n) {
+    gemm_tile_body<true, 4, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile128_residual(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                                  const __bf16* __restrict__ R, __bf16* __restrict__ C, int M,
+                                                                  int N, int K, int tiles_m, int tiles_n) {
+    gemm_tile_body<false, 2, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile128_residual_ragged_k(const __bf16* __restrict__ A,
+                                                                           const __bf16* __restrict__ B,
+                                                                           const __bf16* __restrict__ R, __bf16* __restrict__ C,
+                                                                           int M, int N, int K, int tiles_m, int tiles_n) {
+    gemm_tile_body<true, 2, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile128(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                          __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
@@ -467,6 +527,38 @@ size_t gemm_bf16_workspace_bytes(long M, long N, long K, long batch) {
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
     const SplitPlan p = plan_split_k(M, N, K, batch);
     return p.splits > 1 ? (size_t)p.splits * batch * M * N * sizeof(float) : 0;
+}
+
+bool gemm_bf16_residual_supported(long M, long N, long K, long batch) {
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || batch > 65535) return false;
+    if (M > 0x7fffffffL || N > 0x7fffffffL || N % 8 || K % 8 || K > (1L << 23) || N > (1L << 25)) return false;
+    if (plan_split_k(M, N, K, batch).splits > 1) return false;  // split-K sums partials in another kernel
+    const long tn = (N + mrk::dev::kBN - 1) / mrk::dev::kBN, tm128 = (M + 127) / 128;
+    return tm128 * tn <= 0x7fffffffL;
+}
+
+int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch) {
+    using namespace mrk::dev;
+    if (M <= 0 || N <= 0 || batch <= 0) return 0;
+    if (!gemm_bf16_residual_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(R)) % 16)
+        return (int)hipErrorInvalidValue;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    (void)hipGetLastError();
+    const long tn = (N + kBN - 1) / kBN, tm128 = (M + 127) / 128;
+    const bool small = tm128 * tn * batch <= 256;
+    const long tm = small ? tm128 : (M + kBM - 1) / kBM;
+    const dim3 grid((unsigned)(tm * tn), (unsigned)batch);
+    const __bf16* a = static_cast<const __bf16*>(A);
+    const __bf16* b = static_cast<const __bf16*>(B);
+    const __bf16* r = static_cast<const __bf16*>(R);
+    __bf16* c = static_cast<__bf16*>(C);
+    const bool ragged_k = K % kBK != 0;
+    if (small && !ragged_k) gemm_bf16_tile128_residual<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+    else if (small) gemm_bf16_tile128_residual_ragged_k<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+    else if (!ragged_k) gemm_bf16_tile256_residual<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+    else gemm_bf16_tile256_residual_ragged_k<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+    return (int)hipGetLastError();
 }
 
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,

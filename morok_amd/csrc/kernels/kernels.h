@@ -17,6 +17,11 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 // C [batch,M,N]), one launch.
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
                      long batch = 1, void* workspace = nullptr, size_t workspace_bytes = 0);
+// c = bf16(float(bf16(a b)) + float(r)) with r of c's shape, added in the product kernel's epilogue
+// (same bits as the product followed by an elementwise add).  Supported for the shapes the tiled
+// kernels take without split-K; gemm_bf16_residual_supported tells.
+bool gemm_bf16_residual_supported(long M, long N, long K, long batch);
+int launch_gemm_bf16_residual(void* stream, const void* a, const void* b, const void* r, void* c, long M, long N, long K, long batch);
 // Bytes of f32 scratch with which launch_gemm_bf16 spreads the K loop of this shape over the
 // chip (split-K: partial products per K range, added up in a fixed order by a second kernel);
 // 0 when the shape has enough output tiles by itself.  Without the workspace the same shape

@@ -1112,7 +1112,9 @@ struct Scheduler {
         if (!seen.insert(n).second) return;
         *max_numel = std::max(*max_numel, n->numel());
         if (n->buffer) return;
-        if (n != root && (n->kind == TKind::Reduce || n->kind == TKind::Contiguous || fusable(n))) {
+        TensorNode* other = nullptr;
+        if (n != root && (n->kind == TKind::Reduce || n->kind == TKind::Contiguous || fusable(n) ||
+                          residual_matmul(const_cast<TensorNode*>(n), &other))) {
             out.push_back(const_cast<TensorNode*>(n));
             return;
         }
@@ -1222,18 +1224,71 @@ struct Scheduler {
         return kOk;
     }
 
+    // x + (a @ w) in bf16 where nothing else reads the product: the product kernel adds x in its
+    // epilogue (same bits as the product followed by the add).  Returns the product node and the
+    // other operand.
+    TensorNode* residual_matmul(TensorNode* n, TensorNode** other) const {
+        if (!g_fusion || n->kind != TKind::Binary || static_cast<BinaryOp>(n->sub) != BinaryOp::Add || n->dtype != Scalar::BFloat16 ||
+            n->numel() == 0 || n->src.size() != 2)
+            return nullptr;
+        for (int side = 0; side < 2; side++) {
+            TensorNode* mm = n->src[side].get();
+            TensorNode* r = n->src[1 - side].get();
+            if (mm->buffer || mm->hint != HintKind::Matmul || !fusable(mm) || mm->dtype != Scalar::BFloat16) continue;
+            auto u = uses.find(mm);
+            if (u == uses.end() || u->second != 1) continue;
+            if (r->dtype != Scalar::BFloat16 || r->shape != n->shape || mm->shape != n->shape) continue;
+            // only an operand that is in memory anyway: a lazy expression (a broadcast bias, x * 2)
+            // is cheaper evaluated inside the add than written out first
+            const TensorNode* rb = r;
+            while (!rb->buffer && rb->kind == TKind::Reshape) rb = rb->src[0].get();
+            if (!(rb->buffer || rb->kind == TKind::Reduce || rb->kind == TKind::Contiguous || fusable(rb))) continue;
+            int64_t M, N, K, batch;
+            matmul_extents(mm, &M, &N, &K, &batch);
+            if (!gemm_bf16_residual_supported(M, N, K, batch) || gemm_bf16_workspace_bytes(M, N, K, batch)) continue;
+            *other = r;
+            return mm;
+        }
+        return nullptr;
+    }
+    static void matmul_extents(const TensorNode* mm, int64_t* M, int64_t* N, int64_t* K, int64_t* batch) {
+        const TensorNode *a = mm->hint_inputs[0].get(), *w = mm->hint_inputs[1].get();
+        *K = a->shape.back();
+        *N = w->shape.back();
+        *M = a->shape[a->shape.size() - 2];
+        *batch = 1;
+        for (size_t i = 0; i + 2 < a->shape.size(); i++) (w->shape.size() == 2 ? *M : *batch) *= a->shape[i];
+    }
+    int materialize_residual_matmul(TensorNode* n, TensorNode* mm, TensorNode* r) {
+        for (const TensorRef& in : mm->hint_inputs) MRK_TRY(materialize(in.get()));
+        MRK_TRY(materialize(r));
+        int64_t M, N, K, batch;
+        matmul_extents(mm, &M, &N, &K, &batch);
+        auto out = new_buffer(n);
+        const std::vector<int64_t> params = batch == 1 ? std::vector<int64_t>{M, N, K} : std::vector<int64_t>{M, N, K, batch};
+        MRK_TRY(builtin("gemm_bf16_residual", params, {out, mm->hint_inputs[0]->buffer, mm->hint_inputs[1]->buffer, r->buffer}));
+        n->buffer = out;
+        produced.push_back(n);
+        return kOk;
+    }
+
     int materialize(TensorNode* n) {
         if (n->buffer) return kOk;
         if (n->numel() > 0 && fusable(n)) return materialize_fused(n);
+        {
+            TensorNode* other = nullptr;
+            if (TensorNode* mm = residual_matmul(n, &other)) return materialize_residual_matmul(n, mm, other);
+        }
         {
             std::vector<int64_t> out_strides;
             if (TensorNode* att = attention_under(n, &out_strides)) return materialize_attention(att, n, out_strides);
         }
         if (generated_tc(n)) return materialize_generated_tc(n);
-        // a reshape of materialised data is the same bytes
-        if (n->kind == TKind::Reshape) {
+        // a reshape of materialised data is the same bytes, and so is making it contiguous
+        if (n->kind == TKind::Reshape || n->kind == TKind::Contiguous) {
             TensorNode* s = n->src[0].get();
-            if (s->buffer || s->kind == TKind::Reduce || s->kind == TKind::Contiguous || fusable(s)) {
+            TensorNode* other = nullptr;
+            if (s->buffer || s->kind == TKind::Reduce || s->kind == TKind::Contiguous || fusable(s) || residual_matmul(s, &other)) {
                 MRK_TRY(materialize(s));
                 n->buffer = s->buffer;
                 produced.push_back(n);

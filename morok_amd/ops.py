@@ -33,6 +33,16 @@ def gemm_bf16(a, b, c, m, n, k, device_id=0, variant=0):
     check(lib.mrk_hip_gemm_bf16_variant(device_id, _p(a), _p(b), _p(c), m, n, k, variant))
 
 
+def gemm_bf16_residual(a, b, r, c, m, n, k, device_id=0):
+    """c[m,n] = a[m,k] @ b[k,n] + r[m,n]: the residual added in the product kernel's epilogue,
+    same bits as gemm_bf16 followed by an elementwise add."""
+    _need(a, m * k * 2, "gemm A")
+    _need(b, k * n * 2, "gemm B")
+    _need(r, m * n * 2, "gemm R")
+    _need(c, m * n * 2, "gemm C")
+    check(lib.mrk_hip_gemm_bf16_residual(device_id, _p(a), _p(b), _p(r), _p(c), m, n, k))
+
+
 def flash_attn_fwd_bf16(q, k, v, o, batch, heads, sq, sk, d, scale, causal=True, device_id=0):
     """Fused SDPA forward (Tensor::scaled_dot_product_attention, tensor/src/transformer.rs:78-137)."""
     _need(q, batch * heads * sq * d * 2, "attention Q")

@@ -210,3 +210,41 @@ def test_gemm_split_k_not_used_for_large_shapes():
 
     for shape in [(4096, 4096, 4096), (512, 4096, 4096), (1024, 1024, 1024), (128, 256, 256), (8, 64, 128), (1024, 8192, 64)]:
         assert lib.mrk_hip_gemm_bf16_workspace_bytes(*shape, 1) == 0, shape
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 4096), (300, 264, 200), (128, 4096, 136), (1000, 520, 72), (257, 8, 8)])
+def test_gemm_residual_epilogue(dev, oracle, shape):
+    """c = a b + r with r added in the product kernel's epilogue: the bits of the plain
+    product followed by an f32 add and one more rounding (the oracle's product, then numpy),
+    for full, ragged and tiny tiles; memory behind c stays untouched and r is not read past
+    its end (NaN patterns there would surface)."""
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 7, 41)
+    b = synth.normal_bf16((K, N), 7, 42)
+    r = synth.normal_bf16((M, N), 7, 43)
+    nan = np.uint16(0x7FC0)
+    rbig = np.full(M * N + 2048, nan, np.uint16)
+    rbig[:M * N] = r.ravel()
+    ba, bb, br = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (a, b, rbig))
+    bc = morok_amd.Buffer.from_numpy(np.full(M * N + 2048, nan, np.uint16), dev.device_id)
+    ops.gemm_bf16_residual(ba, bb, br, bc, M, N, K, dev.device_id)
+    got = bc.copyout(np.uint16, (M * N + 2048,))
+    assert np.all(got[M * N:] == nan)
+    prod = oracle.gemm_bf16(a, b)
+    want = synth.to_bf16(synth.from_bf16(prod) + synth.from_bf16(r))
+    plain = dev.buffer(M * N * 2)
+    ops.gemm_bf16(ba, bb, plain, M, N, K, dev.device_id)
+    fused_from_plain = synth.to_bf16(synth.from_bf16(plain.copyout(np.uint16, (M, N))) + synth.from_bf16(r))
+    assert np.array_equal(got[:M * N].reshape(M, N), fused_from_plain)
+    gf, wf = synth.from_bf16(got[:M * N].reshape(M, N)), synth.from_bf16(want)
+    assert np.abs(gf - wf).max() <= 2e-2 * np.abs(wf).max()
+
+
+def test_gemm_residual_refuses_split_k_shapes(dev):
+    a = dev.buffer(4 * 4096 * 2)
+    b = dev.buffer(4096 * 1024 * 2)
+    c = dev.buffer(4 * 1024 * 2)
+    with pytest.raises(morok_amd.MorokHipError):
+        ops.gemm_bf16_residual(a, b, c, c, 4, 1024, 4096, dev.device_id)   # few tiles, long K: the split-K shape
+    with pytest.raises(morok_amd.MorokHipError):
+        ops.gemm_bf16_residual(a, b, c, c, 4, 1020, 64, dev.device_id)     # N not a multiple of 8

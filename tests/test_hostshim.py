@@ -395,7 +395,9 @@ def test_decoder_block_lowering(T, shim, fused, gemms):
     # the attention kernel writes [tokens, hidden] itself and reads V in place out of the
     # projection's [tokens, ...] result: neither is copied into [batch, heads, seq, dim]
     assert sum(k.startswith("flash_fwd_bf16_strided") for k in names) == 1
-    assert len(names) == (15 if fused else 18)
+    # both residual additions happen in the epilogue of the product in front of them
+    assert sum(k.startswith("gemm_bf16_residual") for k in names) == 2
+    assert len(names) == (13 if fused else 16)
 
 
 def test_plan_graph_replay_records_once(T, shim):
@@ -522,7 +524,7 @@ def test_memory_planner_reuses_intermediates(T, shim, monkeypatch):
     out = blk.forward(tok).realize()
     reused, saved = tensor.last_memory_plan()
     planned_bytes = shim.mrk_shim_bytes_in_use() - base
-    assert reused >= 6 and saved >= 5 * 128 * 256 * 2
+    assert reused >= 4 and saved >= 3 * 128 * 256 * 2
     del out
     dev.lru_clear()
     monkeypatch.setenv("MOROK_NO_MEMORY_PLANNER", "1")

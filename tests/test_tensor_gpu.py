@@ -928,6 +928,40 @@ def test_random_movement_chains_power_of_two_shapes(T, seed):
         np.testing.assert_array_equal(t.sum([ax]).to_numpy(), a.sum(ax))
 
 
+def test_matmul_bf16_residual_add_is_fused(T):
+    """x + a @ w in bf16 with no other reader of the product: one kernel (the product kernel
+    with the residual epilogue), on either side of the add and through contiguous(); the same
+    bits as with the hand-written kernels' fusion of the add left out; a product with two
+    readers is kept and added separately."""
+    from morok_amd import synth, uop
+
+    M, K, N = 256, 192, 384
+    a, w, x = synth.normal_bf16((M, K), 9, 1), synth.normal_bf16((K, N), 9, 2), synth.normal_bf16((M, N), 9, 3)
+    ta, tw, tx = (T.Tensor.from_numpy(t, uop.BF16) for t in (a, w, x))
+    T.set_fusion(True)
+    left = tx.try_add(ta.matmul(tw)).contiguous()
+    got_l = left.to_numpy()
+    assert left.kernels() == [f"gemm_bf16_residual_{M}_{N}_{K}"]
+    right = ta.matmul(tw).try_add(tx)
+    got_r = right.to_numpy()
+    assert right.kernels() == [f"gemm_bf16_residual_{M}_{N}_{K}"]
+    assert np.array_equal(got_l, got_r)
+    prod = ta.matmul(tw)
+    separate = synth.to_bf16(synth.from_bf16(prod.to_numpy()) + synth.from_bf16(x))
+    assert np.array_equal(got_l, separate)
+    mm = ta.matmul(tw)
+    both = tx.try_add(mm).try_mul(mm)                      # the product has two readers
+    gb = both.to_numpy()
+    assert not any(k.startswith("gemm_bf16_residual") for k in both.kernels())
+    pf = synth.from_bf16(prod.to_numpy())
+    want = synth.from_bf16(synth.to_bf16(pf + synth.from_bf16(x)))
+    assert np.abs(synth.from_bf16(gb) - want * pf).max() <= 2e-2 * np.abs(want * pf).max()
+    bx = T.Tensor.from_numpy(synth.normal_bf16((1, N), 9, 4), uop.BF16)
+    bc = ta.matmul(tw).try_add(bx)                          # a broadcast operand is not a residual
+    bc.realize()
+    assert not any(k.startswith("gemm_bf16_residual") for k in bc.kernels())
+
+
 def test_matmul_bf16_few_rows_uses_split_k(T, oracle):
     """A handful of rows against a large weight matrix through the tensor API: the scheduler
     adds the split-K scratch to the plan as an intermediate buffer."""
