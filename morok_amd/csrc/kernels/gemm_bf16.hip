@@ -335,10 +335,11 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     constexpr int kChunks = kJ * 4;          // 16-byte chunks per row of the wave's tile
     constexpr int kRowsPerIt = 64 / kChunks;  // rows one store instruction covers
     constexpr int kIts = 128 / kRowsPerIt;
+    constexpr int kFirstBatch = kIts / 4;  // as many as fit the register file next to the live accumulators
     // the residual rows this lane will add are fetched ahead, in two batches, so that their latency
     // overlaps the staging of the accumulators instead of sitting in front of every store
-    // (half of them while the accumulators are still live, the other half once they are staged:
-    // all of them at once would not fit the register file next to the accumulators)
+    // (a quarter of them while the accumulators are still live, the rest once they are staged:
+    // more at once would not fit the register file next to the accumulators)
     u32x4 res[kResidual ? kIts : 1];
     auto fetch_residual = [&](int first, int last) {
 #pragma unroll
@@ -350,7 +351,7 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
                 res[it] = *reinterpret_cast<const u32x4*>(R + (row0 + r) * N + col0 + ch * 8);
         }
     };
-    if constexpr (kResidual) fetch_residual(0, kIts / 2);
+    if constexpr (kResidual) fetch_residual(0, kFirstBatch);
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
@@ -363,7 +364,7 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
                 const int nl = j * 32 + 8 * g + 4 * (lane >> 5);
                 *LDS_PTR(bf16x4, sC + ml * kCPitchT + nl * 2) = h;
             }
-    if constexpr (kResidual) fetch_residual(kIts / 2, kIts);
+    if constexpr (kResidual) fetch_residual(kFirstBatch, kIts);
     __syncthreads();
     __bf16* Cg = C + row0 * N + col0;
     if constexpr (kResidual) {
