@@ -586,3 +586,36 @@ def test_large_reductions_are_split_in_two_stages(T, shim):
     assert len(t.kernels()) == 2
     t = zeros(T, (64, 4096)).sum(1).realize()        # below the threshold: one kernel
     assert len(t.kernels()) == 1
+
+
+def test_null_arguments_are_errors_not_crashes(T, dev, shim):
+    """Every entry point checks its pointers: a null handle or output slot yields
+    MRK_ERR_INVALID_ARGUMENT with a message, never a fault in the library."""
+    import ctypes as C
+
+    x = zeros(T, (4, 4))
+    out = C.c_void_p()
+    null = None
+    calls = [
+        lambda: shim.mrk_hip_tensor_sdpa_ex(null, x._h, x._h, null, 0.0, 0, 0.0, C.byref(out)),
+        lambda: shim.mrk_hip_tensor_sdpa_ex(x._h, null, x._h, null, 0.0, 0, 0.0, C.byref(out)),
+        lambda: shim.mrk_hip_tensor_sdpa_ex(x._h, x._h, x._h, null, 0.0, 0, 0.0, null),
+        lambda: shim.mrk_hip_tensor_tanh(null, C.byref(out)),
+        lambda: shim.mrk_hip_tensor_tanh(x._h, null),
+        lambda: shim.mrk_hip_tensor_matmul_with(x._h, null, -1, C.byref(out)),
+        lambda: shim.mrk_hip_tensor_matmul_with(x._h, x._h, 99, C.byref(out)),
+        lambda: shim.mrk_hip_tensor_gemm(x._h, null, 1.0, 1.0, 0, 0, null, C.byref(out)),
+        lambda: shim.mrk_hip_tensor_linear(x._h, null, null, -1, C.byref(out)),
+        lambda: shim.mrk_hip_tensor_linear(x._h, x._h, null, 99, C.byref(out)),
+        lambda: shim.mrk_hip_tensor_log_softmax(null, -1, C.byref(out)),
+        lambda: shim.mrk_hip_tensor_logsumexp(x._h, -1, null),
+        lambda: shim.mrk_hip_gemm_bf16_residual(0, null, 1, 1, 1, 8, 8, 8),
+        lambda: shim.mrk_hip_flash_attn_fwd_bf16_strided(0, 1, 1, 1, 1, 1, 1, 8, 8, 128, 1.0, 0, null),
+        lambda: shim.mrk_hip_sched_build_wmma_matmul_lds_opts(1, 128, 128, 64, 10, null, C.byref(C.POINTER(C.c_uint8)()), C.byref(C.c_size_t())),
+        lambda: shim.mrk_hip_beam_search_wmma_matmul(0, 1, 128, 128, 64, 1, null, null, null, null),
+        lambda: shim.mrk_hip_benchmark_kernel_with_cutoff(0, null, null, 0, null, 0, null, null, 1, 1, 0.0, null, null, null),
+    ]
+    for i, call in enumerate(calls):
+        rc = call()
+        assert rc == 11, (i, rc, shim.mrk_hip_last_error())       # MRK_ERR_INVALID_ARGUMENT
+        assert shim.mrk_hip_last_error()
