@@ -21,6 +21,20 @@ def test_matmul_reference_small_cases(oracle):
         assert np.abs(c - np.array(g["expected"], np.float32)).max() < g["tol"]
 
 
+def test_matmul_reference_vector_cases(oracle):
+    """Dot product, vector x matrix and matrix x vector of the reference's tests, through the
+    oracle's matmul with the vector as a one-row / one-column matrix."""
+    g = GOLD["matmul_dot_1d"]
+    c = oracle.matmul_f32(np.array([g["a"]], np.float32), np.array(g["b"], np.float32).reshape(-1, 1))
+    assert abs(float(c[0, 0]) - g["expected"]) < g["tol"]
+    g = GOLD["matmul_vector_matrix"]
+    c = oracle.matmul_f32(np.array([g["v"]], np.float32), np.array(g["m"], np.float32))
+    assert np.abs(c[0] - np.array(g["expected"], np.float32)).max() < g["tol"]
+    g = GOLD["matmul_matrix_vector"]
+    c = oracle.matmul_f32(np.array(g["m"], np.float32), np.array(g["v"], np.float32).reshape(-1, 1))
+    assert np.abs(c[:, 0] - np.array(g["expected"], np.float32)).max() < g["tol"]
+
+
 @pytest.mark.parametrize("size,tol", [tuple(x) for x in GOLD["matmul_square_closed_form"]["sizes_tol"]])
 def test_matmul_reference_square_generators(oracle, size, tol):
     x = np.arange(size * size)
