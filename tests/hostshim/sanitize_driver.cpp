@@ -83,6 +83,23 @@ static int work(int id) {
             printf("attention over views did not take the strided kernel\n");
             return 1;
         }
+        // x + a @ w in bf16: the product kernel with the residual epilogue, through contiguous()
+        {
+            int64_t as[2] = {B * S, hid}, wsh[2] = {hid, hid};
+            std::vector<uint16_t> av(static_cast<size_t>(as[0] * as[1]), 0x3f80), wv(static_cast<size_t>(hid * hid), 0x3c00);
+            mrk_tensor *ta = nullptr, *tw = nullptr, *mm = nullptr, *sum = nullptr, *cont = nullptr;
+            CK(mrk_hip_tensor_from_bytes(0, av.data(), av.size() * 2, as, 2, 10, &ta));
+            CK(mrk_hip_tensor_from_bytes(0, wv.data(), wv.size() * 2, wsh, 2, 10, &tw));
+            CK(mrk_hip_tensor_matmul(ta, tw, &mm));
+            CK(mrk_hip_tensor_binary(ta, 0 /*add*/, mm, &sum));
+            CK(mrk_hip_tensor_contiguous(sum, &cont));
+            CK(mrk_hip_tensor_realize(cont));
+            if (mrk_hip_tensor_last_kernel_count() != 1 || !strstr(mrk_hip_tensor_last_kernel_name(0), "residual")) {
+                printf("x + a @ w did not take the residual epilogue\n");
+                return 1;
+            }
+            for (mrk_tensor* p : {ta, tw, mm, sum, cont}) mrk_hip_tensor_release(p);
+        }
         int64_t ms[2] = {S, S};
         std::vector<float> maskv(static_cast<size_t>(S * S), 0.0f);
         mrk_tensor *mask = nullptr, *att2 = nullptr;
