@@ -16,7 +16,7 @@
  *   - thread fan-out: runtime/src/devices/cpu.rs:67-117 (one call per thread_id)
  *     with the thread count of schedule/src/optimizer/heuristics.rs:485-535.
  *
- * Pinning status (see tests/test_oracle_*.py):
+ * Pinning status (see tests/test_oracle.py):
  *   orc_matmul_f32        pinned: reference known answers (2x2, closed-form 1024^2
  *                         generators, ones) + float64 matmul
  *   orc_softmax_*         pinned: float64 softmax, shift invariance, row sums, tiny brute force
@@ -29,6 +29,21 @@
  *   orc_silu_mul_*, orc_decoder_block_bf16
  *                         parity unpinned by reference tests (the reference has no decoder-block
  *                         function); each stage is pinned separately against float64
+ *   orc_unary_f32, orc_map_unary_f32
+ *                         pinned: float64 evaluation within 0-2 ulp per op, values at which
+ *                         neighbouring ops differ (half-to-even rint, sign(0), exp vs exp2), and
+ *                         the reference's softplus / mish / softsign / sinh / cosh / tanh known
+ *                         answers through the reference's own compositions of these ops
+ *   orc_binary_f32, orc_map_binary_f32
+ *                         pinned: the reference's realize_binary cases, correctly rounded float64
+ *                         results for + - * /, exact fmod with the dividend's sign, pow within 2 ulp
+ *   orc_binary_i64, orc_map_binary_i32
+ *                         pinned: the reference's documented -9/5, 9/-5 quotients and remainders,
+ *                         brute force over operands of both signs against unbounded integers
+ *                         (truncating division, arithmetic shift, 32-bit wrap)
+ *   orc_add_bf16          pinned: float64 sum rounded once, ties-to-even cases
+ *   orc_heads_to_tokens_u16, orc_rope_heads_bf16
+ *                         pinned: index permutation on distinct values, rotation vs float64
  *
  * Exact summation order and bf16 rounding placement inside fused elementwise
  * chains of the real backend depend on optimizer choices that only running the

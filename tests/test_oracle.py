@@ -2,6 +2,7 @@
 against the known answers held by the reference's own tests (tests/golden/
 reference_known_answers.json) and against what the mathematics fixes (float64 closed forms,
 invariants, special cases).  Runs without a GPU."""
+import ctypes as C
 import json
 import os
 
@@ -318,3 +319,213 @@ def test_decoder_block_composition_vs_float64(oracle):
     g = r(g1 / (1 + np.exp(-g1)) * g3)
     ref = r(h2 + r(g @ f["W2"]))
     assert np.abs(out - ref).max() < 3e-2 * np.abs(ref).max()
+
+
+# ------------------------------------------------------------------ elementwise semantics tables
+# orc_unary_f32 / orc_binary_f32 / orc_binary_i64 and their orc_map_* loops are the truth the
+# renderer parity tests compare generated kernels with; they are pinned here against the known
+# answers the reference holds, against float64 evaluation of the same function and, for the
+# integer table, against brute force over small operands of both signs.
+_UN = {"neg": 0, "abs": 1, "sqrt": 2, "rsqrt": 3, "reciprocal": 4, "exp": 5, "exp2": 6, "log": 7, "log2": 8,
+       "sin": 9, "cos": 10, "tan": 11, "floor": 12, "ceil": 13, "trunc": 14, "round": 15, "erf": 16, "sign": 17,
+       "square": 18}
+_BF = {"add": 0, "sub": 1, "mul": 2, "fdiv": 3, "mod": 4, "max": 5, "pow": 6}
+_BI = {"add": 0, "sub": 1, "mul": 2, "idiv": 3, "mod": 4, "max": 5, "and": 7, "or": 8, "xor": 9, "shl": 10, "shr": 11}
+
+
+def _ulp_bound(ref64, ulps):
+    """|error| allowed for a float32 result whose exact value is ref64."""
+    return ulps * np.spacing(np.abs(ref64).astype(np.float32)).astype(np.float64)
+
+
+def test_unary_table_vs_float64(oracle):
+    import math
+
+    pos = np.concatenate([synth.uniform((4000,), 91, 0, 1e-3, 60.0), np.float32([1, 4, 9, 0.25, 2, 1e-3])])
+    sym = np.concatenate([synth.uniform((4000,), 91, 1, -30.0, 30.0), np.float32([0, -0.0, 1, -1, 2.5, -2.5, 0.5, -0.5, 1.5])])
+    f64 = {
+        "neg": (sym, lambda x: -x, 0), "abs": (sym, np.abs, 0), "sqrt": (pos, np.sqrt, 0.5),
+        "rsqrt": (pos, lambda x: 1 / np.sqrt(x), 1.5), "reciprocal": (sym[sym != 0], lambda x: 1 / x, 0.5),
+        "exp": (sym[np.abs(sym) < 20], np.exp, 2), "exp2": (sym[np.abs(sym) < 20], np.exp2, 2),
+        "log": (pos, np.log, 2), "log2": (pos, np.log2, 2), "floor": (sym, np.floor, 0), "ceil": (sym, np.ceil, 0),
+        "trunc": (sym, np.trunc, 0), "round": (sym, np.rint, 0), "sign": (sym, np.sign, 0),
+        "square": (sym, lambda x: x * x, 0.5),
+        "erf": (sym[np.abs(sym) < 4], np.vectorize(math.erf), 2), "tan": (sym[np.abs(sym) < 1.4], np.tan, 2),
+    }
+    for op, (x, fn, ulps) in f64.items():
+        y = oracle.map_unary_f32(_UN[op], x).astype(np.float64)
+        ref = fn(x.astype(np.float64))
+        assert np.all(np.abs(y - ref) <= _ulp_bound(ref, ulps)), op
+    # sin / cos: absolute bound near their zeros
+    for op, fn in (("sin", np.sin), ("cos", np.cos)):
+        y = oracle.map_unary_f32(_UN[op], sym).astype(np.float64)
+        assert np.abs(y - fn(sym.astype(np.float64))).max() <= 2e-7, op
+    # every op tag of the table is covered above
+    assert set(f64) | {"sin", "cos"} == set(_UN)
+
+
+def test_unary_table_distinguishing_values(oracle):
+    """Values at which neighbouring ops of the table differ, so a swapped case label fails."""
+    x = np.float32([-2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 3.7, -3.7])
+    want = {
+        "floor": [-3, -2, -1, 0, 1, 2, 3, -4], "ceil": [-2, -1, -0.0, 1, 2, 3, 4, -3],
+        "trunc": [-2, -1, -0.0, 0, 1, 2, 3, -3], "round": [-2, -2, -0.0, 0, 2, 2, 4, -4],  # half to even
+        "sign": [-1, -1, -1, 1, 1, 1, 1, -1], "neg": list(-x), "abs": list(np.abs(x)), "square": list(x * x),
+    }
+    for op, w in want.items():
+        assert np.array_equal(oracle.map_unary_f32(_UN[op], x), np.float32(w)), op
+    assert oracle.map_unary_f32(_UN["sign"], np.float32([0.0, -0.0])).tolist() == [0.0, 0.0]
+    # exp / exp2 / log / log2 at points where the bases tell them apart
+    assert abs(float(oracle.map_unary_f32(_UN["exp"], np.float32([1]))[0]) - np.e) < 3e-7
+    assert oracle.map_unary_f32(_UN["exp2"], np.float32([3, 10, -1])).tolist() == [8.0, 1024.0, 0.5]
+    assert oracle.map_unary_f32(_UN["log2"], np.float32([8, 0.25])).tolist() == [3.0, -2.0]
+    assert abs(float(oracle.map_unary_f32(_UN["log"], np.float32([np.e]))[0]) - 1.0) < 2e-7
+    assert oracle.map_unary_f32(_UN["sqrt"], np.float32([1, 4, 9])).tolist() == [1.0, 2.0, 3.0]
+    assert oracle.map_unary_f32(_UN["rsqrt"], np.float32([1, 4, 16])).tolist() == [1.0, 0.5, 0.25]
+    assert oracle.map_unary_f32(_UN["reciprocal"], np.float32([2, -4])).tolist() == [0.5, -0.25]
+    # scalar entry point and the mapped loop agree
+    assert oracle.lib.orc_unary_f32(_UN["square"], C.c_float(3.0)) == 9.0
+
+
+def test_binary_f32_table(oracle):
+    for c in GOLD["realize_binary"]["cases"]:  # tensor/src/test/unit/realize_binary.rs:16-270
+        a, b = np.float32(c["a"]), np.float32(c["b"])
+        y = oracle.map_binary_f32(_BF[c["op"]], a, b)
+        want = np.float32(c["expected"]) if "expected" in c else {
+            "add": np.add, "sub": np.subtract, "mul": np.multiply, "fdiv": np.divide}[c["op"]](a, b)
+        assert np.abs(y - want).max() <= c["tol"], c["name"]
+    a = synth.uniform((5000,), 92, 0, -8.0, 8.0)
+    b = synth.uniform((5000,), 92, 1, 0.25, 4.0) * np.where(synth.uniform((5000,), 92, 2) > 0, 1, -1).astype(np.float32)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    for op, fn in (("add", np.add), ("sub", np.subtract), ("mul", np.multiply), ("fdiv", np.divide)):
+        # IEEE: the float32 result is the correctly rounded exact result
+        assert np.array_equal(oracle.map_binary_f32(_BF[op], a, b), fn(a64, b64).astype(np.float32)), op
+    assert np.array_equal(oracle.map_binary_f32(_BF["max"], a, b), np.maximum(a, b))
+    # fmod: exact, sign of the dividend (C remainder, not Python's)
+    assert np.array_equal(oracle.map_binary_f32(_BF["mod"], a, b), np.fmod(a64, b64).astype(np.float32))
+    assert oracle.map_binary_f32(_BF["mod"], np.float32([-9, 9, 5.5]), np.float32([5, -5, 2])).tolist() == [-4.0, 4.0, 1.5]
+    ap = np.abs(a) + np.float32(0.1)
+    ref = np.power(ap.astype(np.float64), b64)
+    assert np.all(np.abs(oracle.map_binary_f32(_BF["pow"], ap, b) - ref) <= _ulp_bound(ref, 2))
+    # operand order: sub, fdiv, mod and pow are not commutative
+    assert oracle.lib.orc_binary_f32(_BF["sub"], C.c_float(5), C.c_float(3)) == 2.0
+    assert oracle.lib.orc_binary_f32(_BF["fdiv"], C.c_float(1), C.c_float(4)) == 0.25
+    assert oracle.lib.orc_binary_f32(_BF["pow"], C.c_float(2), C.c_float(5)) == 32.0
+
+
+def test_binary_integer_table_brute_force(oracle):
+    """Brute force over operands of both signs against Python's unbounded integers, with C
+    semantics written out: quotient truncated toward zero, remainder with the dividend's sign
+    (ir/src/types.rs:625-646), arithmetic right shift, two's-complement wrap to 32 bits."""
+    for c in GOLD["integer_div_mod_doc_examples"]["cases"]:
+        got = oracle.map_binary_i32(_BI[c["op"]], np.int32([c["a"]]), np.int32([c["b"]]))
+        assert int(got[0]) == c["expected"], c
+
+    def wrap(v):
+        return (v + 2**31) % 2**32 - 2**31
+
+    def trunc_div(a, b):
+        q = abs(a) // abs(b)
+        return q if (a < 0) == (b < 0) else -q
+
+    py = {"add": lambda a, b: a + b, "sub": lambda a, b: a - b, "mul": lambda a, b: a * b, "idiv": trunc_div,
+          "mod": lambda a, b: a - trunc_div(a, b) * b, "max": max, "and": lambda a, b: a & b,
+          "or": lambda a, b: a | b, "xor": lambda a, b: a ^ b}
+    vals = list(range(-20, 21)) + [2**31 - 1, -2**31 + 1, 123456789, -987654321, 65535, -65536]
+    aa, bb = np.meshgrid(np.int32(vals), np.int32(vals), indexing="ij")
+    aa, bb = aa.ravel(), bb.ravel()
+    for op, fn in py.items():
+        keep = bb != 0 if op in ("idiv", "mod") else np.ones(aa.shape, bool)
+        a, b = aa[keep], bb[keep]
+        got = oracle.map_binary_i32(_BI[op], a, b)
+        want = np.array([wrap(fn(int(x), int(y))) for x, y in zip(a, b)], np.int64).astype(np.int32)
+        assert np.array_equal(got, want), op
+    sh = np.int32(list(range(0, 31)))
+    for v in (1, 3, -1, -8, 1000, -123456, 2**30 + 5):
+        a = np.full(sh.shape, v, np.int32)
+        assert np.array_equal(oracle.map_binary_i32(_BI["shr"], a, sh), np.int32([v >> int(s) for s in sh])), v
+    # left shifts are compared where the result fits (no signed overflow, which C leaves undefined)
+    for v in (1, 3, 5, 1000):
+        s = np.int32([k for k in range(0, 31) if abs(v) << k < 2**31])
+        a = np.full(s.shape, v, np.int32)
+        assert np.array_equal(oracle.map_binary_i32(_BI["shl"], a, s), np.int32([v << int(k) for k in s])), v
+    assert set(py) | {"shl", "shr"} == set(_BI)
+    # 64-bit scalar entry point: products beyond 32 bits are kept
+    oracle.lib.orc_binary_i64.restype = C.c_longlong
+    oracle.lib.orc_binary_i64.argtypes = [C.c_int, C.c_longlong, C.c_longlong]
+    assert oracle.lib.orc_binary_i64(_BI["mul"], 3_000_000_000, 7) == 21_000_000_000
+    assert oracle.lib.orc_binary_i64(_BI["idiv"], -21_000_000_001, 7) == -3_000_000_000
+    assert oracle.lib.orc_binary_i64(_BI["mod"], -21_000_000_001, 7) == -1
+
+
+def test_composed_activation_known_answers(oracle):
+    """softplus / mish / softsign / sinh / cosh as the reference composes them from the table's
+    ops (tensor/src/activation.rs:320-358, tensor/src/math.rs:252-266), against the values its
+    own tests hold."""
+    U = lambda op, x: oracle.map_unary_f32(_UN[op], x)
+    B = lambda op, a, b: oracle.map_binary_f32(_BF[op], a, np.broadcast_to(np.float32(b), a.shape))
+
+    def softplus(x, beta):
+        s = B("mul", x, beta)
+        m = B("max", s, 0.0)
+        t = B("add", U("exp", B("sub", s, m)), U("exp", B("sub", np.zeros_like(x), m)))
+        return B("mul", B("add", U("log", t), m), np.float32(1.0 / beta))
+
+    def tanh(x):  # 2 * sigmoid(2x) - 1, sigmoid through exp2 (activation.rs:64-74)
+        t = B("mul", x, 2.0)
+        sig = U("reciprocal", B("add", U("exp2", B("mul", t, np.float32(-1.0 / np.log(2.0)))), 1.0))
+        return B("sub", B("mul", sig, 2.0), 1.0)
+
+    for c in GOLD["activation_values"]["cases"] + GOLD["math_values"]["cases"]:
+        x = np.float32(c["x"])
+        if c["name"] == "softplus":
+            y = softplus(x, c["beta"])
+        elif c["name"] == "mish":
+            y = B("mul", x, tanh(softplus(x, 1.0)))
+        elif c["name"] == "softsign":
+            y = B("fdiv", x, B("add", U("abs", x), 1.0))
+        else:
+            ep, en = U("exp", x), U("exp", U("neg", x))
+            y = B("fdiv", B("sub" if c["name"] == "sinh" else "add", ep, en), 2.0)
+        assert np.abs(y - np.float32(c["expected"])).max() <= c["tol"], c
+    g = GOLD["tanh_doc_values"]
+    assert np.abs(tanh(np.float32(g["x"])) - np.float32(g["expected"])).max() <= g["tol"]
+
+
+def test_add_bf16_definition(oracle):
+    """y = bf16(float(a) + float(b)), round to nearest even: the float32 sum of two bf16 values
+    is exact in float64, so rounding the float64 sum twice (to f32, then to bf16) is the
+    definition; cases with ties and opposite signs included."""
+    a = synth.normal_bf16((4096,), 93, 0)
+    b = synth.normal_bf16((4096,), 93, 1)
+    s32 = (synth.from_bf16(a).astype(np.float64) + synth.from_bf16(b).astype(np.float64)).astype(np.float32)
+    assert np.array_equal(oracle.add_bf16(a, b), synth.to_bf16(s32))
+    one, eps = synth.to_bf16(np.float32([1.0])), synth.to_bf16(np.float32([2.0 ** -8]))
+    # 1 + 2^-8 lies halfway between 1 and the next bf16 (1 + 2^-7): ties go to the even mantissa
+    assert synth.from_bf16(oracle.add_bf16(one, eps))[0] == 1.0
+    x = synth.to_bf16(np.float32([1.0 + 2.0 ** -7]))
+    assert synth.from_bf16(oracle.add_bf16(x, eps))[0] == np.float32(1.0 + 2.0 ** -6)
+    assert synth.from_bf16(oracle.add_bf16(x, synth.to_bf16(np.float32([-1.0]))))[0] == np.float32(2.0 ** -7)
+
+
+def test_heads_to_tokens_and_rope_heads_layout(oracle):
+    """Index checks with distinct values per position: [B,H,S,D] -> [B*S, H*D] and the
+    token-major -> head-major move of orc_rope_heads_bf16 (apply=0: a pure permutation;
+    apply=1: the split-half rotation of orc_rope_f32 on every head)."""
+    Bn, S, H, D = 2, 5, 3, 8
+    x = np.arange(Bn * H * S * D, dtype=np.uint16).reshape(Bn, H, S, D)
+    y = np.empty((Bn * S, H * D), np.uint16)
+    oracle.lib.orc_heads_to_tokens_u16(x.ctypes.data_as(C.c_void_p), y.ctypes.data_as(C.c_void_p), Bn, S, H, D)
+    assert np.array_equal(y, x.transpose(0, 2, 1, 3).reshape(Bn * S, H * D))
+    tok = synth.normal_bf16((Bn * S, H * D), 94, 0)
+    ang = synth.uniform((S, D // 2), 94, 1, -3.0, 3.0)
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    moved = oracle.rope_heads_bf16(tok, cos, sin, Bn, S, H, D, apply=False)
+    assert np.array_equal(moved, tok.reshape(Bn, S, H, D).transpose(0, 2, 1, 3))
+    rot = oracle.rope_heads_bf16(tok, cos, sin, Bn, S, H, D, apply=True)
+    xf = synth.from_bf16(moved).astype(np.float64)
+    c64, s64 = cos.astype(np.float64), sin.astype(np.float64)
+    lo, hi = xf[..., : D // 2], xf[..., D // 2:]
+    ref = np.concatenate([lo * c64 - hi * s64, lo * s64 + hi * c64], -1)
+    got = synth.from_bf16(rot).astype(np.float64)
+    assert np.abs(got - ref).max() <= 2.0 ** -8 * np.abs(ref).max() + 1e-6
