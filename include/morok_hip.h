@@ -95,7 +95,9 @@ int mrk_hip_lru_cache_count(int device_id, size_t size, int cpu_accessible, size
 int mrk_hip_lru_total_cached(int device_id, size_t* count);
 int mrk_hip_lru_clear(int device_id);
 /* Raw copies for callers that hold device pointers from mrk_hip_alloc
- * (device/src/buffer.rs:351-366,390-407,444-532).  copyout waits for all queued work first. */
+ * (device/src/buffer.rs:351-366,390-407,444-532).  copyout waits for everything queued on the
+ * device's own stream first; work submitted through an mrk_queue runs on that queue's stream
+ * and needs mrk_hip_queue_synchronize (or a signal wait) before its results are copied out. */
 int mrk_hip_copyin(int device_id, void* dst, size_t dst_offset, const void* src_host, size_t size);
 int mrk_hip_copyout(int device_id, void* dst_host, const void* src, size_t src_offset, size_t size);
 int mrk_hip_copy_dd(int device_id, void* dst, size_t dst_offset, const void* src, size_t src_offset, size_t size);

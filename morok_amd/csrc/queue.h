@@ -3,7 +3,19 @@
 // ordering between queues is expressed with timeline signals
 // (device/src/sync.rs:44-71), which become hipStreamWaitEvent dependencies on the GPU, so
 // a copy queue and a compute queue overlap exactly where no signal orders them.
+//
+// Ordering against the device's own stream (allocations, zero-fills, uploads, Tensor::realize):
+// a batch starts only after everything queued on the device stream at submit() time has
+// finished (one event per submit), so a zero_init fill or an upload lands before the batch's
+// kernels touch the buffer.  Lifetime: the buffers and kernels of a batch stay referenced by
+// the queue until the batch has completed on the GPU, so a caller may release them right after
+// submit(); when they are finally dropped the device stream is made to wait for that batch
+// first, so that a block going back to the allocator's cache is not handed to device-stream
+// work that would overtake the batch.  The reverse direction is the caller's: device-stream
+// work (copyout included) that must see a batch's results needs queue.synchronize() or a
+// signal wait first.
 #pragma once
+#include <deque>
 #include <memory>
 #include <vector>
 
@@ -38,6 +50,7 @@ class HardwareQueue {
     int submit(uint64_t wait_timeout_ms = 10000);
     int synchronize();
     size_t pending_commands() const { return cmds_.size(); }
+    size_t batches_in_flight() const { return in_flight_.size(); }
     bool is_copy_queue() const { return copy_queue_; }
     ffi::Stream stream() const { return stream_; }
 
@@ -53,10 +66,21 @@ class HardwareQueue {
         bool has_sizes = false;
         size_t global[3] = {1, 1, 1}, local[3] = {1, 1, 1};
     };
+    struct InFlight {
+        ffi::Event done = nullptr;   // recorded on the queue's stream behind the batch
+        ffi::Event ready = nullptr;  // recorded on the device stream in front of the batch
+        std::vector<Command> batch;
+    };
+    // drops the batches whose completion event has fired (all of them when `all`, after the
+    // caller has synchronized the stream)
+    void retire(bool all);
+    int issue(std::vector<Command>& batch, uint64_t wait_timeout_ms);
     int device_id_;
     bool copy_queue_;
     ffi::Stream stream_ = nullptr;
+    ffi::Stream device_stream_ = nullptr;  // the allocator's stream of this device
     std::vector<Command> cmds_;
+    std::deque<InFlight> in_flight_;
 };
 
 }  // namespace mrk

@@ -7,6 +7,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <mutex>
 #include <set>
 #include <tuple>
 #include <unordered_map>
@@ -1709,27 +1710,45 @@ struct Scheduler {
 
 }  // namespace
 
-int Tensor::prepare(std::unique_ptr<ExecutionPlan>* out) const {
-    if (!n_) return fail(kInvalidArgument, "prepare: invalid tensor");
+// Scheduling writes provisional buffers onto graph nodes, and graphs of different roots may
+// share nodes, so every path that reads or writes TensorNode::buffer runs under this lock:
+// concurrent realizations of tensors over a common lazy subgraph are serialised for the
+// (host-side) scheduling and for the enqueue of the plan, not for the GPU work itself.
+static std::recursive_mutex g_graph_mutex;
+
+namespace {
+// Schedules `root`.  On success `kept` lists the nodes (root included) that keep a buffer whose
+// contents exist only after the plan has run; on failure no node keeps one.
+int prepare_locked(const TensorRef& root, std::unique_ptr<ExecutionPlan>* out, std::vector<TensorNode*>* kept) {
     g_stats = RealizeStats();
     auto t0 = std::chrono::steady_clock::now();
     Scheduler s;
-    MRK_TRY(DeviceFactoryRegistry::global().device("HIP", n_->device_id, &s.dev));
-    s.plan.reset(new ExecutionPlan(n_->device_id));
-    s.count_uses(n_.get());
-    if (!n_->buffer) MRK_TRY(s.materialize(n_.get()));
-    s.plan->set_outputs({s.plan->add_buffer(n_->buffer)});
+    // every exit that is not the successful one returns the touched nodes to their lazy state
+    struct Rollback {
+        Scheduler& s;
+        bool armed = true;
+        ~Rollback() {
+            if (armed)
+                for (TensorNode* t : s.produced) t->buffer = nullptr;
+        }
+    } rollback{s};
+    MRK_TRY(DeviceFactoryRegistry::global().device("HIP", root->device_id, &s.dev));
+    s.plan.reset(new ExecutionPlan(root->device_id));
+    s.count_uses(root.get());
+    if (!root->buffer) MRK_TRY(s.materialize(root.get()));
+    s.plan->set_outputs({s.plan->add_buffer(root->buffer)});
     // Intermediates share blocks by liveness (tensor/src/memory_planner.rs); their contents do
     // not outlive the plan's execution, so their nodes go back to being lazy: only the root
     // keeps its buffer.  MOROK_NO_MEMORY_PLANNER=1 keeps every intermediate resident.
     const char* no_planner = std::getenv("MOROK_NO_MEMORY_PLANNER");
     const bool planner = !(no_planner && no_planner[0] && no_planner[0] != '0');
     if (planner) s.plan->enable_memory_planner();
-    int rc = s.plan->build();
-    if (planner || rc != kOk)
-        for (TensorNode* t : s.produced)
-            if (t != n_.get()) t->buffer = nullptr;
-    MRK_TRY(rc);
+    MRK_TRY(s.plan->build());
+    rollback.armed = false;
+    for (TensorNode* t : s.produced) {
+        if (planner && t != root.get()) t->buffer = nullptr;
+        else if (kept) kept->push_back(t);
+    }
     s.stats.buffers_reused = s.plan->memory_plan().buffers_reused;
     s.stats.memory_saved = s.plan->memory_plan().memory_saved;
     s.stats.elapsed_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
@@ -1737,28 +1756,54 @@ int Tensor::prepare(std::unique_ptr<ExecutionPlan>* out) const {
     *out = std::move(s.plan);
     return kOk;
 }
+}  // namespace
+
+int Tensor::prepare(std::unique_ptr<ExecutionPlan>* out) const {
+    if (!n_) return fail(kInvalidArgument, "prepare: invalid tensor");
+    std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
+    return prepare_locked(n_, out, nullptr);
+}
 
 int Tensor::realize() const {
     if (!n_) return fail(kInvalidArgument, "realize: invalid tensor");
+    std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
     if (n_->buffer) {
         g_stats = RealizeStats();
         return kOk;
     }
     auto t0 = std::chrono::steady_clock::now();
     std::unique_ptr<ExecutionPlan> plan;
-    MRK_TRY(prepare(&plan));
-    MRK_TRY(plan->execute());
+    std::vector<TensorNode*> kept;
+    MRK_TRY(prepare_locked(n_, &plan, &kept));
+    // The plan is enqueued before the lock is released: whoever sees the root's buffer next
+    // queues its reads behind these kernels on the device's in-order stream.
+    int rc = plan->execute();
+    if (rc != kOk) {
+        for (TensorNode* t : kept) t->buffer = nullptr;  // nothing was computed into them
+        return rc;
+    }
     g_stats.elapsed_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     return kOk;
 }
 
+std::shared_ptr<Buffer> Tensor::buffer() const {
+    if (!n_) return nullptr;
+    std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
+    return n_->buffer;
+}
+
 int Tensor::to_bytes(void* dst, size_t nbytes) const {
     if (!n_) return fail(kInvalidArgument, "to_vec: invalid tensor");
-    if (!n_->buffer) MRK_TRY(realize());
+    std::shared_ptr<Buffer> buf;
+    {
+        std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
+        if (!n_->buffer) MRK_TRY(realize());
+        buf = n_->buffer;
+    }
     const size_t expect = static_cast<size_t>(n_->numel()) * scalar_size(n_->dtype);
     if (nbytes != expect) return failf(kSizeMismatch, "size mismatch: expected %zu, got %zu", expect, nbytes);
     if (expect == 0) return kOk;
-    return n_->buffer->copyout(dst, nbytes);
+    return buf->copyout(dst, nbytes);
 }
 
 }  // namespace mrk

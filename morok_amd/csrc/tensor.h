@@ -152,7 +152,7 @@ class Tensor {
     // once the plan has run.
     int prepare(std::unique_ptr<class ExecutionPlan>* out) const;
     int to_bytes(void* dst, size_t nbytes) const;  // realize if needed, then copy out
-    std::shared_ptr<Buffer> buffer() const { return n_ ? n_->buffer : nullptr; }
+    std::shared_ptr<Buffer> buffer() const;
 
   private:
     TensorRef n_;

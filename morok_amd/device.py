@@ -550,13 +550,14 @@ class TimelineSignal:
 
 class HardwareQueue:
     """HardwareQueue (device/src/queue.rs:76-141): batches commands for its own HIP stream;
-    submit() hands them over without waiting.  Every method returns self for chaining."""
+    submit() hands them over without waiting.  The library keeps the buffers and kernels of a
+    submitted batch referenced until it has run, so callers may drop theirs after submit().
+    Every method returns self for chaining."""
 
     def __init__(self, device_id=0, copy_queue=False):
         h = C.c_void_p()
         check(lib.mrk_hip_queue_create(device_id, int(copy_queue), C.byref(h)))
         self._h = h
-        self._keep = []
 
     def wait(self, signal, value):
         check(lib.mrk_hip_queue_wait(self._h, signal._h, value))
@@ -572,7 +573,6 @@ class HardwareQueue:
         g = _size3(global_size) if global_size is not None else None
         l = _size3(local_size) if local_size is not None else None
         check(lib.mrk_hip_queue_exec(self._h, kernel._h, bufs, len(buffers), va, len(vals), g, l))
-        self._keep.append((kernel, list(buffers)))
         return self
 
     def copy(self, dst, src):
@@ -589,7 +589,6 @@ class HardwareQueue:
 
     def synchronize(self):
         check(lib.mrk_hip_queue_synchronize(self._h))
-        self._keep.clear()
         return self
 
     @property

@@ -29,6 +29,7 @@ struct FakeFunction {
     std::string name;
 };
 struct FakeEvent {
+    int no = 0;
     std::chrono::steady_clock::time_point t;
     bool recorded = false;
 };
@@ -39,6 +40,17 @@ struct FakeGraph {
 };
 std::map<void*, size_t> g_capturing;  // stream -> launches recorded so far
 size_t g_graph_launches = 0, g_graphs_alive = 0;
+bool g_events_pending = false;  // event_query answers "not ready" while set
+// trace of stream operations ("memset:S", "record:E:S", "wait:S:E", "launch:S", "dtod:S"; S = stream
+// number in creation order, E = event number), kept while enabled
+bool g_trace_on = false;
+std::string g_trace;
+int g_next_stream = 0, g_next_event = 0;
+int stream_no(void* s) { return s ? *static_cast<int*>(s) : -1; }
+void trace(const std::string& what) {
+    if (g_trace_on) g_trace += what + " ";
+}
+long g_fail_module_load_in = -1;  // >= 0: that many further module loads succeed, the next one fails once
 // one launch seen by the stand-in: counted as run, or as recorded while its stream is capturing (g_mu held)
 void count_launch(void* stream) {
     auto it = g_capturing.find(stream);
@@ -53,7 +65,29 @@ void mrk_shim_reset() {
     g_limit = ~size_t(0);
     g_alloc_calls = g_free_calls = g_launches = g_syncs = 0;
     g_graph_launches = 0;
+    g_fail_module_load_in = -1;
+    g_events_pending = false;
+    g_trace_on = false;
+    g_trace.clear();
     g_last_kernel.clear();
+}
+// failure injection: after `n` more successful module loads the next one reports an invalid image, once
+void mrk_shim_fail_module_load_after(long n) { g_fail_module_load_in = n; }
+void mrk_shim_set_events_pending(int on) { g_events_pending = on != 0; }
+void mrk_shim_trace(int on) {
+    std::lock_guard<std::mutex> l(g_mu);
+    g_trace_on = on != 0;
+    g_trace.clear();
+}
+// copies the trace (NUL-terminated, truncated to cap) and returns its full length
+size_t mrk_shim_trace_get(char* out, size_t cap) {
+    std::lock_guard<std::mutex> l(g_mu);
+    if (out && cap) {
+        size_t n = g_trace.size() < cap - 1 ? g_trace.size() : cap - 1;
+        std::memcpy(out, g_trace.data(), n);
+        out[n] = 0;
+    }
+    return g_trace.size();
 }
 size_t mrk_shim_graph_launches() { return g_graph_launches; }
 size_t mrk_shim_graphs_alive() { return g_graphs_alive; }
@@ -73,6 +107,7 @@ void mrk_shim_last_dims(unsigned* grid, unsigned* block) {
 void mrk_shim_note_launch(void* stream, const char* name) {
     std::lock_guard<std::mutex> l(g_mu);
     count_launch(stream);
+    trace("launch:" + std::to_string(stream_no(stream)));
     g_last_kernel = name;
 }
 }
@@ -116,7 +151,8 @@ int mem_info(size_t* free_bytes, size_t* total_bytes) {
     return 0;
 }
 
-int memset_async(void* dst, int value, size_t bytes, Stream) {
+int memset_async(void* dst, int value, size_t bytes, Stream s) {
+    { std::lock_guard<std::mutex> l(g_mu); trace("memset:" + std::to_string(stream_no(s))); }
     std::memset(dst, value, bytes);
     return 0;
 }
@@ -128,13 +164,15 @@ int memcpy_dtoh_async(void* dst, const void* src, size_t bytes, Stream) {
     std::memcpy(dst, src, bytes);
     return 0;
 }
-int memcpy_dtod_async(void* dst, const void* src, size_t bytes, Stream) {
+int memcpy_dtod_async(void* dst, const void* src, size_t bytes, Stream s) {
+    { std::lock_guard<std::mutex> l(g_mu); trace("dtod:" + std::to_string(stream_no(s))); }
     std::memmove(dst, src, bytes);
     return 0;
 }
 
 int stream_create(Stream* out) {
-    *out = new int(0);
+    std::lock_guard<std::mutex> l(g_mu);
+    *out = new int(g_next_stream++);
     return 0;
 }
 int stream_destroy(Stream s) {
@@ -145,27 +183,35 @@ int stream_synchronize(Stream) {
     { std::lock_guard<std::mutex> l(g_mu); g_syncs++; }
     return 0;
 }
-int stream_wait_event(Stream, Event) { return 0; }
+int stream_wait_event(Stream s, Event e) {
+    std::lock_guard<std::mutex> l(g_mu);
+    trace("wait:" + std::to_string(stream_no(s)) + ":" + std::to_string(static_cast<FakeEvent*>(e)->no));
+    return 0;
+}
 int device_synchronize() {
     { std::lock_guard<std::mutex> l(g_mu); g_syncs++; }
     return 0;
 }
 
 int event_create(Event* out) {
-    *out = new FakeEvent();
+    std::lock_guard<std::mutex> l(g_mu);
+    auto* ev = new FakeEvent();
+    ev->no = g_next_event++;
+    *out = ev;
     return 0;
 }
 int event_destroy(Event e) {
     delete static_cast<FakeEvent*>(e);
     return 0;
 }
-int event_record(Event e, Stream) {
+int event_record(Event e, Stream s) {
     auto* ev = static_cast<FakeEvent*>(e);
+    { std::lock_guard<std::mutex> l(g_mu); trace("record:" + std::to_string(ev->no) + ":" + std::to_string(stream_no(s))); }
     ev->t = std::chrono::steady_clock::now();
     ev->recorded = true;
     return 0;
 }
-int event_query(Event) { return 0; }
+int event_query(Event) { return g_events_pending ? kNotReady : 0; }
 int event_synchronize(Event) { return 0; }
 int event_elapsed_ms(float* ms, Event start, Event stop) {
     auto *a = static_cast<FakeEvent*>(start), *b = static_cast<FakeEvent*>(stop);
@@ -178,6 +224,14 @@ int module_load_data(Module* out, const void* image) {
     // a gfx950 code object is an ELF; its length is recovered from the section header table
     const unsigned char* p = static_cast<const unsigned char*>(image);
     if (!p || std::memcmp(p, "\x7f" "ELF", 4) != 0) return kInvalidImage;
+    {
+        std::lock_guard<std::mutex> l(g_mu);
+        if (g_fail_module_load_in == 0) {
+            g_fail_module_load_in = -1;
+            return kInvalidImage;
+        }
+        if (g_fail_module_load_in > 0) g_fail_module_load_in--;
+    }
     uint64_t shoff;
     uint16_t shentsize, shnum;
     std::memcpy(&shoff, p + 0x28, 8);
@@ -212,6 +266,7 @@ int module_launch(Function f, const unsigned grid[3], const unsigned block[3], u
     std::memcpy(g_last_block, block, sizeof g_last_block);
     g_last_kernel = static_cast<FakeFunction*>(f)->name;
     count_launch(stream);
+    trace("launch:" + std::to_string(stream_no(stream)));
     return 0;
 }
 

@@ -12,12 +12,57 @@
 #define CK(x) do { int rc_ = (x); if (rc_ != 0) { printf("FAIL line %d rc %d: %s\n", __LINE__, rc_, mrk_hip_last_error()); return 1; } } while (0)
 #include <thread>
 static int work(int id);
+// Four threads realize four different roots built over ONE shared lazy subgraph (a reduce over an
+// elementwise chain, so the shared nodes are kernel boundaries that receive provisional buffers
+// while a root is scheduled), several times over, and read the results back.
+static int shared_subgraph() {
+    int64_t shp[2] = {48, 80};
+    std::vector<float> x(48 * 80, 0.5f);
+    mrk_tensor *t = nullptr, *u = nullptr, *mid = nullptr;
+    CK(mrk_hip_tensor_from_bytes(0, x.data(), x.size() * 4, shp, 2, 11 /*f32*/, &t));
+    CK(mrk_hip_tensor_binary(t, 0 /*add*/, t, &u));
+    int64_t axes[1] = {1};
+    CK(mrk_hip_tensor_reduce(u, 0 /*add*/, axes, 1, 1, 1, &mid));  // shared, lazy
+    int rcs[4] = {0, 0, 0, 0};
+    std::vector<std::thread> th;
+    for (int i = 0; i < 4; i++)
+        th.emplace_back([i, u, mid, &rcs] {
+            rcs[i] = [&]() -> int {
+                for (int r = 0; r < 6; r++) {
+                    mrk_tensor *a = nullptr, *root = nullptr;
+                    CK(mrk_hip_tensor_binary(u, i % 2 ? 2 /*mul*/ : 1 /*sub*/, mid, &a));
+                    int64_t ax[1] = {0};
+                    CK(mrk_hip_tensor_reduce(a, i < 2 ? 0 : 2 /*add | max*/, ax, 1, 0, 1, &root));
+                    if (r % 2) {
+                        mrk_plan* plan = nullptr;
+                        CK(mrk_hip_tensor_prepare(root, &plan));
+                        CK(mrk_hip_plan_execute(plan));
+                        mrk_hip_plan_release(plan);
+                    } else {
+                        CK(mrk_hip_tensor_realize(root));
+                    }
+                    std::vector<float> out(80);
+                    CK(mrk_hip_tensor_to_bytes(root, out.data(), out.size() * 4));
+                    mrk_hip_tensor_release(a);
+                    mrk_hip_tensor_release(root);
+                }
+                return 0;
+            }();
+        });
+    for (auto& thr : th) thr.join();
+    for (int rc : rcs)
+        if (rc) return 1;
+    CK(mrk_hip_tensor_realize(mid));  // the shared node itself is still realizable afterwards
+    for (mrk_tensor* p : {t, u, mid}) mrk_hip_tensor_release(p);
+    return 0;
+}
 int main() {
     if (mrk_hip_device_create(0)) return 1;
     std::vector<std::thread> th; int rcs[4] = {0,0,0,0};
     for (int i = 0; i < 4; i++) th.emplace_back([i, &rcs] { for (int r = 0; r < 5; r++) rcs[i] |= work(i); });
     for (auto& t : th) t.join();
     for (int i = 0; i < 4; i++) if (rcs[i]) return 1;
+    if (shared_subgraph()) return 1;
     printf("threads ok\n");
     return 0;
 }

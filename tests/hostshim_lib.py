@@ -31,6 +31,10 @@ def load():
         ("mrk_shim_alloc_calls", C.c_size_t, []),
         ("mrk_shim_free_calls", C.c_size_t, []),
         ("mrk_shim_launches", C.c_size_t, []),
+        ("mrk_shim_fail_module_load_after", None, [C.c_long]),
+        ("mrk_shim_set_events_pending", None, [C.c_int]),
+        ("mrk_shim_trace", None, [C.c_int]),
+        ("mrk_shim_trace_get", C.c_size_t, [C.c_char_p, C.c_size_t]),
         ("mrk_shim_graph_launches", C.c_size_t, []),
         ("mrk_shim_graphs_alive", C.c_size_t, []),
         ("mrk_shim_syncs", C.c_size_t, []),
@@ -48,3 +52,11 @@ def last_dims(lib):
     g, b = (C.c_uint * 3)(), (C.c_uint * 3)()
     lib.mrk_shim_last_dims(C.byref(g), C.byref(b))
     return tuple(g), tuple(b)
+
+
+def trace(lib):
+    """The stream operations recorded since mrk_shim_trace(1), as a list of strings."""
+    n = lib.mrk_shim_trace_get(None, 0)
+    buf = C.create_string_buffer(n + 1)
+    lib.mrk_shim_trace_get(buf, n + 1)
+    return buf.value.decode().split()

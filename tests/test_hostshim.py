@@ -509,6 +509,43 @@ def test_queue_batches_until_submit_and_reports_errors(dev, shim):
     q2.wait(sig, 1).copy(a, b).submit(wait_timeout_ms=20)          # already reached: no wait
 
 
+def test_queue_orders_against_the_device_stream_and_keeps_buffers_alive(dev, shim):
+    """A zero_init buffer's fill is queued on the device stream when the buffer is first
+    allocated (here: inside submit); the queue's stream must wait for the device stream before the
+    kernel that writes the buffer.  The buffers of a batch stay referenced until the batch has
+    completed, and the device stream waits for the batch before their blocks can be reused."""
+    k = morok_amd.Kernel.get_or_compile(__import__("morok_amd").sched.build_matmul_f32_opts(64, 64, 64, [16, 16, 4, 4, 1]), "qk")
+    nbytes = 64 * 64 * 4 + 4096                     # a size nothing else in this test uses
+    a, b = dev.buffer(nbytes), dev.buffer(nbytes)
+    a.ensure_allocated(), b.ensure_allocated()
+    c = dev.buffer(nbytes, zero_init=True)          # lazy: allocated (and zero-filled) at submit
+    q = morok_amd.HardwareQueue()
+    shim.mrk_shim_set_events_pending(1)             # the GPU has not finished anything yet
+    shim.mrk_shim_trace(1)
+    q.exec(k, [c, a, b]).submit()
+    ops = hostshim_lib.trace(shim)
+    fill = next(i for i, o in enumerate(ops) if o.startswith("memset:"))
+    dev_stream = ops[fill].split(":")[1]
+    rec = next(i for i, o in enumerate(ops) if o.startswith("record:") and o.endswith(":" + dev_stream) and i > fill)
+    ev = ops[rec].split(":")[1]
+    launch = next(i for i, o in enumerate(ops) if o.startswith("launch:"))
+    q_stream = ops[launch].split(":")[1]
+    assert q_stream != dev_stream
+    assert fill < rec < ops.index(f"wait:{q_stream}:{ev}") < launch, ops
+    # the caller lets go of its buffer right after submit: the block is not recycled yet
+    before = dev.lru_cache_count(nbytes)
+    del c
+    assert dev.lru_cache_count(nbytes) == before
+    q.exec(k, [a, a, b]).submit()                   # a later submit does not retire an unfinished batch
+    assert dev.lru_cache_count(nbytes) == before
+    shim.mrk_shim_trace(1)
+    shim.mrk_shim_set_events_pending(0)
+    q.synchronize()                                 # now it has run: the block goes back to the cache,
+    assert dev.lru_cache_count(nbytes) == before + 1
+    ops = hostshim_lib.trace(shim)                  # and the device stream was told to wait for the batch
+    assert any(o.startswith(f"wait:{dev_stream}:") for o in ops), ops
+
+
 def test_memory_planner_reuses_intermediates(T, shim, monkeypatch):
     """tensor/src/memory_planner.rs: intermediates with disjoint lifetimes share blocks; outputs
     and inputs never do."""
@@ -545,6 +582,29 @@ def test_planned_intermediates_become_lazy_again(T, shim):
     assert len(b.kernels()) == 2
     c = a.try_add(1.0).realize()                   # a was an output: it is read, not recomputed
     assert len(c.kernels()) == 1
+
+
+def test_failed_schedule_leaves_the_graph_lazy(T, shim):
+    """A kernel that fails to load in the middle of a realization must not leave provisional
+    buffers on the nodes scheduled before it: the next realization of the same graph has to
+    schedule (and launch) every kernel again instead of reading never-computed memory."""
+    T.set_fusion(False)
+    morok_amd.kernel_cache_clear()
+    x = zeros(T, (37, 53))
+    mid = x.try_add(1.0).sum(1)                    # kernel 1 (reduce)
+    root = mid.try_mul(2.0).contiguous().sum(0)    # kernels 2 and 3
+    shim.mrk_shim_fail_module_load_after(1)        # the second kernel's code object is refused
+    n = shim.mrk_shim_launches()
+    with pytest.raises(MorokHipError):
+        root.realize()
+    assert shim.mrk_shim_launches() == n           # nothing ran
+    with pytest.raises(MorokHipError):             # extraction does not hand out an unrealised root either
+        shim.mrk_shim_fail_module_load_after(0)
+        root.to_numpy()
+    root.realize()                                 # now everything loads
+    assert len(root.kernels()) == 3 and shim.mrk_shim_launches() == n + 3
+    again = mid.try_mul(3.0).realize()             # the shared reduce is scheduled again, not read
+    assert len(again.kernels()) == 2
 
 
 def test_ops_refuse_undersized_buffers(dev, shim):
