@@ -419,6 +419,20 @@ size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_
 int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
                                int variant);
 
+/* mrk_hip_gemm_bf16 for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same kernels and the same bits as mrk_hip_gemm_bf16, but the split-K partials go
+ * to a fixed 32 MiB device array inside the library (resolved per device by
+ * mrk_hip_device_create) instead of a block from the allocator, and the call performs no
+ * allocation or free of any kind.  The device must have been created before
+ * (INVALID_ARGUMENT otherwise: creating it allocates).  A shape whose partials would exceed
+ * mrk_hip_gemm_bf16_noalloc_capacity() bytes is refused with INVALID_ARGUMENT and nothing is
+ * launched.  All calls on one device share the array: calls that may overlap on one device
+ * (different streams or threads without ordering between them) race; calls queued on the
+ * device's own in-order stream, as this entry point does, do not. */
+int mrk_hip_gemm_bf16_noalloc(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k);
+size_t mrk_hip_gemm_bf16_noalloc_capacity(void);
+
 /* c = bf16(float(bf16(a b)) + float(r)): the product above with a bf16 matrix r of c's shape added
  * in the kernel's epilogue - the bits of mrk_hip_gemm_bf16 followed by an elementwise add
  * (Tensor::matmul + try_add, tensor/src/matmul.rs:82-110), without the round trip of the product

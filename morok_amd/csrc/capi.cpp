@@ -872,6 +872,30 @@ int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int6
     return mrk_hip_gemm_bf16_variant(device_id, a, b, c, m, n, k, 0);
 }
 
+size_t mrk_hip_gemm_bf16_noalloc_capacity(void) { return gemm_bf16_static_workspace_capacity(); }
+int mrk_hip_gemm_bf16_noalloc(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k) {
+    if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_noalloc: negative shape");
+    if (m == 0 || n == 0) return kOk;
+    MRK_NONNULL(c);
+    if (k > 0) {
+        MRK_NONNULL(a);
+        MRK_NONNULL(b);
+    }
+    // lookup only: creating a device allocates (streams, the allocator), which this call must not
+    std::shared_ptr<Device> d = DeviceFactoryRegistry::global().find("HIP", device_id);
+    if (!d)
+        return failf(kInvalidArgument, "gemm_bf16_noalloc: device HIP:%d has not been created; call mrk_hip_device_create "
+                                       "during set-up (this entry point allocates nothing, device creation does)", device_id);
+    const size_t need = gemm_bf16_workspace_bytes(m, n, k, 1);
+    if (need > gemm_bf16_static_workspace_capacity())
+        return failf(kInvalidArgument, "gemm_bf16_noalloc: %lldx%lldx%lld needs %zu bytes of split-K scratch, the built-in "
+                                       "scratch holds %zu; use mrk_hip_gemm_bf16", (long long)m, (long long)n, (long long)k,
+                     need, gemm_bf16_static_workspace_capacity());
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_gemm_bf16_static_ws(d->allocator->stream(), device_id, a, b, c, m, n, k), "gemm_bf16_noalloc launch");
+    return kOk;
+}
+
 int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, const void* r, void* c, int64_t m, int64_t n, int64_t k) {
     if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_residual: negative shape");
     if (m == 0 || n == 0) return kOk;

@@ -1,4 +1,5 @@
 #include "device.h"
+#include "kernels/kernels.h"
 
 #include <algorithm>
 #include <cctype>
@@ -84,6 +85,13 @@ int DeviceFactoryRegistry::device(const std::string& device_type, int device_id,
     return kOk;
 }
 
+std::shared_ptr<Device> DeviceFactoryRegistry::find(const std::string& device_type, int device_id) {
+    std::string key = device_type + ":" + std::to_string(device_id);
+    std::lock_guard<std::mutex> lock(mu_);
+    auto it = devices_.find(key);
+    return it == devices_.end() ? nullptr : it->second;
+}
+
 void DeviceFactoryRegistry::reset() {
     std::lock_guard<std::mutex> lock(mu_);
     devices_.clear();
@@ -93,6 +101,10 @@ int create_hip_device(int device_id, AllocatorRegistry& registry, std::shared_pt
     auto dev = std::make_shared<Device>();
     dev->device_id = device_id;
     MRK_TRY(registry.get(device_id, &dev->allocator));
+    // set-up work that must not happen later, inside entry points that promise not to allocate:
+    // the per-device address of the split-K scratch array (this device is current here)
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(gemm_bf16_static_workspace_init(device_id), "hipGetSymbolAddress(split-K scratch)");
     dev->renderer = make_hip_renderer(device_id);
     dev->compiler = make_hiprtc_compiler();
     ffi::Stream stream = dev->allocator->stream();

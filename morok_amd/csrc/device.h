@@ -124,6 +124,8 @@ class DeviceFactoryRegistry {
     static DeviceFactoryRegistry& global();
     void register_factory(const std::string& device_type, DeviceFactory f);
     int device(const std::string& device_type, int device_id, std::shared_ptr<Device>* out);
+    // lookup only: null when the device has not been created yet (creates and allocates nothing)
+    std::shared_ptr<Device> find(const std::string& device_type, int device_id);
     void reset();
 
   private:

@@ -35,6 +35,7 @@
 // shapes that would otherwise leave most compute units idle; a leading batch dimension runs as
 // grid.y.  Everything else takes the any-shape kernel at the end of this file.
 #include <hip/hip_runtime.h>
+#include <atomic>
 
 #include <cstdint>
 #include <type_traits>
@@ -497,9 +498,19 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic(const __bf16* __restric
 
 }  // namespace mrk::dev
 
+// Split-K partials for callers that cannot allocate: 32 MiB per device, held until the process
+// ends.  That is the most plan_split_k ever asks for (at most 256 workgroups in flight, each
+// with one 128 x 256 f32 partial tile).  In host code the name is only a handle for
+// hipGetSymbolAddress; kernels receive the resolved per-device address as an argument.
+static constexpr size_t kStaticWsBytes = size_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticWsBytes];
+
 namespace mrk {
 
 namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_static_ws[kMaxDevices];  // resolved address of `scratch` on each device
+
 // Split-K plan for a shape: how many K ranges and how many 64-deep steps each, or splits = 1
 // when the plain tiled kernel already has enough workgroups (or the K loop is too short).
 struct SplitPlan {
@@ -528,6 +539,30 @@ size_t gemm_bf16_workspace_bytes(long M, long N, long K, long batch) {
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
     const SplitPlan p = plan_split_k(M, N, K, batch);
     return p.splits > 1 ? (size_t)p.splits * batch * M * N * sizeof(float) : 0;
+}
+
+int gemm_bf16_static_workspace_init(int device_id) {
+    if (device_id < 0 || device_id >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    if (g_static_ws[device_id].load(std::memory_order_acquire)) return 0;
+    void* p = nullptr;  // the array's address on the current device (every device has its own copy)
+    hipError_t rc = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (rc != hipSuccess) return (int)rc;
+    if (!p || reinterpret_cast<uintptr_t>(p) % 256) return (int)hipErrorInvalidSymbol;
+    g_static_ws[device_id].store(p, std::memory_order_release);
+    return 0;
+}
+
+size_t gemm_bf16_static_workspace_capacity() { return kStaticWsBytes; }
+
+int launch_gemm_bf16_static_ws(void* stream, int device_id, const void* A, const void* B, void* C, long M, long N, long K) {
+    if (device_id < 0 || device_id >= kMaxDevices) return (int)hipErrorInvalidDevice;
+    const size_t need = gemm_bf16_workspace_bytes(M, N, K, 1);
+    if (need > kStaticWsBytes) return (int)hipErrorInvalidValue;
+    void* ws = g_static_ws[device_id].load(std::memory_order_acquire);
+    if (!ws) return (int)hipErrorNotInitialized;
+    // every element of a partial tile that the reduce kernel reads is written by the split
+    // kernel of the same call, so nothing has to be cleared between calls
+    return launch_gemm_bf16(stream, A, B, C, M, N, K, 0, 1, need ? ws : nullptr, need);
 }
 
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch) {

@@ -27,6 +27,15 @@ int launch_gemm_bf16_residual(void* stream, const void* a, const void* b, const 
 // 0 when the shape has enough output tiles by itself.  Without the workspace the same shape
 // runs unsplit.
 size_t gemm_bf16_workspace_bytes(long M, long N, long K, long batch);
+// The same product with the split-K partials in a file-scope device array instead of a
+// caller's workspace, for callers that must not allocate.  gemm_bf16_static_workspace_init
+// resolves the array's address on one device (that device current; once per device, at
+// set-up); launch_gemm_bf16_static_ws launches nothing and returns hipErrorInvalidValue when
+// the shape's partials exceed gemm_bf16_static_workspace_capacity(), hipErrorNotInitialized
+// when the address has not been resolved for device_id.  Calls on one device share the array.
+int gemm_bf16_static_workspace_init(int device_id);
+size_t gemm_bf16_static_workspace_capacity();
+int launch_gemm_bf16_static_ws(void* stream, int device_id, const void* A, const void* B, void* C, long M, long N, long K);
 
 // O = softmax(Q K^T * scale [causal]) V; Q [BH,Sq,D], K/V [BH,Sk,D], O [BH,Sq,D] bf16, D = 128,
 // scale > 0.  Causal: key j visible to query i iff j <= i.

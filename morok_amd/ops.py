@@ -33,6 +33,15 @@ def gemm_bf16(a, b, c, m, n, k, device_id=0, variant=0):
     check(lib.mrk_hip_gemm_bf16_variant(device_id, _p(a), _p(b), _p(c), m, n, k, variant))
 
 
+def gemm_bf16_noalloc(a, b, c, m, n, k, device_id=0):
+    """gemm_bf16 without any device allocation: split-K partials go to the library's fixed
+    device scratch (for callers under graph capture or in loops that must not allocate)."""
+    _need(a, m * k * 2, "gemm A")
+    _need(b, k * n * 2, "gemm B")
+    _need(c, m * n * 2, "gemm C")
+    check(lib.mrk_hip_gemm_bf16_noalloc(device_id, _p(a), _p(b), _p(c), m, n, k))
+
+
 def gemm_bf16_residual(a, b, r, c, m, n, k, device_id=0):
     """c[m,n] = a[m,k] @ b[k,n] + r[m,n]: the residual added in the product kernel's epilogue,
     same bits as gemm_bf16 followed by an elementwise add."""

@@ -14,6 +14,12 @@ int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, 
     mrk_shim_note_launch(stream, "gemm_bf16");
     return 0;
 }
+int gemm_bf16_static_workspace_init(int) { return 0; }
+size_t gemm_bf16_static_workspace_capacity() { return size_t(32) << 20; }
+int launch_gemm_bf16_static_ws(void* stream, int, const void*, const void*, void*, long, long, long) {
+    mrk_shim_note_launch(stream, "gemm_bf16");
+    return 0;
+}
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch) {
     return M > 0 && N > 0 && K > 0 && batch > 0 && N % 8 == 0 && K % 8 == 0;
 }
