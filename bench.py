@@ -31,11 +31,39 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, published
 BF16_PEAK_TFLOPS = 2500.0    # MI355X dense bf16 MFMA, published
-# HBM bytes per launch of each dominant kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
-# of this file (one counter per run), each scaled by what the same counter reads for the 256 MiB
-# copy kernel (FETCH_SIZE x2.000, WRITE_SIZE x0.999 on gfx950); summaries under profiles/.
 MIB = 1 << 20
-MEASURED_TRAFFIC = {"softmax": (256.1 + 255.7) * MIB, "gemm": (192.2 + 32.0) * MIB, "flash": (1024.8 + 255.9) * MIB}
+# roofline.traffic is not measured by this run (counters need a profiler run of their own): it is
+# read from the committed rocprofv3 summary of the same workload, i.e. from the FETCH_SIZE and
+# WRITE_SIZE passes recorded there, each scaled by what the same counter read for the 256 MiB copy
+# kernel, and only when that summary names the kernel this run launched; otherwise null.
+PROFILE_OF = {"softmax": "softmax_rows_in_regs_8192x8192_f32.txt", "gemm": "gemm_bf16_tile256_4096cubed.txt",
+              "flash": "flash_fwd_d128_causal_8x32x4096x128.txt", "decoder": "decoder_block_4x2048_h4096.txt",
+              "generated_tc": "generated_tensor_core_gemm_4096cubed.txt"}
+
+
+def _profiled_traffic(workload, kernel):
+    """(bytes per launch, source) for `kernel` from profiles/<summary>, or (None, reason)."""
+    import re
+
+    path = os.path.join(ROOT, "profiles", PROFILE_OF.get(workload, ""))
+    if not os.path.isfile(path):
+        return None, "no committed profile summary at run time"
+    base = kernel.split("<")[0]
+    for line in open(path):
+        mt = re.match(r"\s*(\S.*?)\s+n=\s*\d+\s+FETCH.*->\s*([0-9.]+) MiB \| WRITE.*->\s*([0-9.]+) MiB", line)
+        if mt and mt.group(1).split("<")[0] == base:
+            return (float(mt.group(2)) + float(mt.group(3))) * MIB, "profiles/" + PROFILE_OF[workload]
+    return None, "profiles/%s does not list kernel %s" % (PROFILE_OF[workload], base)
+
+
+def _roofline(workload, bound, achieved, peak, unit, kernel, **extra):
+    traffic, source = _profiled_traffic(workload, kernel)
+    r = {"bound": bound, "achieved": achieved, "peak": peak, "unit": unit, "frac": achieved / peak, "traffic": traffic,
+         "traffic_source": source, "kernel": kernel}
+    r.update(extra)
+    return r
+
+
 METRIC = "bf16 GEMM TFLOP/s & flash-attn fwd TFLOP/s (% of peak); softmax HBM GB/s"
 
 
@@ -101,10 +129,8 @@ def bench_softmax(m, dev, steps, warmup, cpu):
     rec = {
         "metric": "softmax HBM GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "f32",
         "config": {"workload": "row softmax f32 [8192x8192], normal(0,2), one fused kernel (configs[1])"},
-        "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": gbs / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC["softmax"],
-                     "kernel": "softmax_rows_in_regs<256,8,1>",
-                     "algorithmic_bytes_per_launch": algo_bytes},
+        "roofline": _roofline("softmax", "hbm", gbs, HBM_PEAK_GBS, "GB/s", "softmax_rows_in_regs<256,8,1>",
+                              algorithmic_bytes_per_launch=algo_bytes),
     }
     rec.update(stats)
     if cpu:
@@ -122,39 +148,101 @@ def bench_softmax(m, dev, steps, warmup, cpu):
     return rec
 
 
+_CEILING = {}  # TFLOP/s of the MFMA-only calibration kernel, measured once per run
+
+
+def _mfma_ceiling_tflops(m, dev):
+    """Rate of the register-only MFMA kernel at the size of the 4096^3 product (256 workgroups x 64
+    K steps of a 256 x 256 tile), with the same settle / warm-up discipline as the workloads."""
+    from morok_amd import ops
+
+    if "tf" not in _CEILING:
+        scratch = dev.buffer(256).ensure_allocated()
+        ms, _ = _launch_stats(m, lambda: ops.mfma_ceiling(scratch, 256, 64), 50, 5)
+        _CEILING["tf"] = 2.0 * 4096 ** 3 / (ms * 1e-3) / 1e12
+    return _CEILING["tf"]
+
+
+def _gemm_cpu_baseline(M, N, K):
+    from morok_amd import synth
+    from tests.oracle_lib import Oracle
+
+    orc = Oracle()
+    a = synth.normal_bf16((M, K), 3, 0)
+    b = synth.normal_bf16((K, N), 3, 1)
+    t = orc.thread_count(M * N * K, M)
+    sec = _cpu_time(lambda: orc.gemm_bf16(a, b, threads=t))
+    return {"value": 2.0 * M * N * K / sec / 1e12, "unit": "TFLOP/s", "cores": t, "kind": "port",
+            "sample": f"all {M} output rows (K=N=4096), f32-accumulate bf16 matmul kernel, "
+                      f"{t} threads, min of 3 after 1 warm-up"}
+
+
+def _vendor_gemm_tflops(n, steps, warmup):
+    """torch.matmul (hipBLASLt) on the same shape and dtype, same settle discipline: a reference
+    point outside the product path, reported when torch imports on this box."""
+    try:
+        import torch
+    except Exception:
+        return None
+    if not torch.cuda.is_available():
+        return None
+    a = torch.randn(n, n, device="cuda", dtype=torch.bfloat16)
+    b = torch.randn(n, n, device="cuda", dtype=torch.bfloat16)
+    c = torch.empty(n, n, device="cuda", dtype=torch.bfloat16)
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < SETTLE_MS:
+        for _ in range(10):
+            torch.matmul(a, b, out=c)
+        torch.cuda.synchronize()
+    for _ in range(warmup):
+        torch.matmul(a, b, out=c)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        torch.matmul(a, b, out=c)
+    e1.record()
+    torch.cuda.synchronize()
+    return 2.0 * n ** 3 / (e0.elapsed_time(e1) / steps * 1e-3) / 1e12
+
+
 def bench_gemm(m, dev, steps, warmup, cpu):
-    """configs[2]: bf16 GEMM M=N=K=4096, inputs normal(0,1) rounded to bf16, f32 accumulate, bf16 out."""
-    from morok_amd import ops, synth
+    """configs[2]: bf16 GEMM M=N=K=4096, inputs normal(0,1) rounded to bf16, f32 accumulate, bf16 out,
+    through the caller path: Tensor::matmul -> prepare (schedule, kernel cache, plan) -> execute."""
+    from morok_amd import ops, tensor, uop
 
     M = N = K = 4096
     ba = dev.buffer(M * K * 2).ensure_allocated()
     bb = dev.buffer(K * N * 2).ensure_allocated()
-    bc = dev.buffer(M * N * 2).ensure_allocated()
     ops.fill_normal(ba, M * K, seed=3, tensor_id=0, bf16=True)
     ops.fill_normal(bb, K * N, seed=3, tensor_id=1, bf16=True)
-    ms, stats = _launch_stats(m, lambda: ops.gemm_bf16(ba, bb, bc, M, N, K), steps, warmup)
+    c = tensor.Tensor.from_buffer(ba, (M, K), uop.BF16).matmul(tensor.Tensor.from_buffer(bb, (K, N), uop.BF16))
+    plan = c.prepare()
+    program = plan.kernel_name(0)  # the plan's one item: the hand-written kernel behind the Program interface
+    if not program.startswith("gemm_bf16"):
+        raise RuntimeError("Tensor::matmul did not select the hand-written bf16 GEMM: " + program)
+    kernel = "gemm_bf16_tile256"     # the device function that Program launches for this shape
+    ms, stats = _launch_stats(m, plan.execute, steps, warmup)
     flops = 2.0 * M * N * K
     tf = flops / (ms * 1e-3) / 1e12
+    # the same kernel called straight through the C ABI (no plan): shows what the plan costs
+    bc = dev.buffer(M * N * 2).ensure_allocated()
+    direct_ms, _ = _launch_stats(m, lambda: ops.gemm_bf16(ba, bb, bc, M, N, K), steps, warmup)
+    ceiling = _mfma_ceiling_tflops(m, dev)
     rec = {
         "metric": "bf16 GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "bf16",
-        "config": {"workload": "bf16 GEMM M=N=K=4096, normal(0,1) inputs, f32 accumulate, bf16 out (configs[2])"},
-        "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC["gemm"], "kernel": "gemm_bf16_tile256",
-                     "algorithmic_flops_per_launch": flops},
+        "config": {"workload": "bf16 GEMM M=N=K=4096, normal(0,1) inputs, f32 accumulate, bf16 out, via "
+                               "Tensor::matmul -> prepare -> execute (configs[2])"},
+        "roofline": _roofline("gemm", "mfma", tf, BF16_PEAK_TFLOPS, "TFLOP/s", kernel, algorithmic_flops_per_launch=flops,
+                              mfma_only_ceiling=ceiling, frac_of_ceiling=tf / ceiling),
+        "plan_item": program, "direct_abi_ms_per_step": direct_ms,
     }
     rec.update(stats)
+    vendor = _vendor_gemm_tflops(M, steps, warmup)
+    if vendor is not None:
+        rec["vendor_reference"] = {"value": vendor, "unit": "TFLOP/s", "library": "torch.matmul (hipBLASLt), not on the "
+                                   "product path", "ratio": tf / vendor}
     if cpu:
-        from tests.oracle_lib import Oracle
-
-        orc = Oracle()
-        sm = 4096  # the whole 4096^3 product: 137 GFLOP per run, 4 runs
-        a = synth.normal_bf16((sm, K), 3, 0)
-        b = synth.normal_bf16((K, N), 3, 1)
-        t = orc.thread_count(sm * N * K, sm)
-        sec = _cpu_time(lambda: orc.gemm_bf16(a, b, threads=t))
-        rec["cpu_baseline"] = {"value": 2.0 * sm * N * K / sec / 1e12, "unit": "TFLOP/s", "cores": t, "kind": "port",
-                               "sample": f"all {sm} output rows (K=N=4096), f32-accumulate bf16 matmul kernel, "
-                                         f"{t} threads, min of 3 after 1 warm-up"}
+        rec["cpu_baseline"] = _gemm_cpu_baseline(M, N, K)
     return rec
 
 
@@ -177,9 +265,8 @@ def bench_flash(m, dev, steps, warmup, cpu):
         "metric": "flash-attn fwd TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "bf16",
         "steps": steps,
         "config": {"workload": "causal flash-attention fwd, bf16 [8,32,4096,128], scale 1/sqrt(128) (configs[3])"},
-        "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": MEASURED_TRAFFIC["flash"], "kernel": "flash_fwd_d128",
-                     "algorithmic_flops_per_launch": flops},
+        "roofline": _roofline("flash", "mfma", tf, BF16_PEAK_TFLOPS, "TFLOP/s", "flash_fwd_d128",
+                              algorithmic_flops_per_launch=flops),
     }
     rec.update(stats)
     if cpu:
@@ -223,7 +310,9 @@ def bench_decoder(m, dev, steps, warmup, cpu):
         "config": {"workload": "decoder block via tensor API: hidden 4096, 32x128 heads, SwiGLU 11008, batch 4 x seq 2048 "
                                "prefill (configs[4])"},
         "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None, "kernel": f"gemm_bf16_tile256[_residual] ({sum(n.startswith('gemm_bf16') for n, _ in prof)} of the {len(prof)} kernels)",
+                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None,
+                     "traffic_source": "per-kernel figures in profiles/" + PROFILE_OF["decoder"],
+                     "kernel": f"gemm_bf16_tile256[_residual] ({sum(n.startswith('gemm_bf16') for n, _ in prof)} of the {len(prof)} kernels)",
                      "algorithmic_flops_per_launch": flops},
         "kernels": len(prof), "gemm_ms": gemm_ms, "flash_ms": flash_ms, "other_ms": sum(t for _, t in prof) - gemm_ms - flash_ms,
     }
@@ -261,8 +350,11 @@ def bench_matmul_f32(m, dev, steps, warmup, cpu):
     rec = {
         "metric": "f32 matmul TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "f32",
         "config": {"workload": "f32 matmul 1024^3 via the lazy tensor API, generated kernel (configs[0])"},
-        "roofline": {"bound": "mfma", "achieved": tf, "peak": 157.3, "unit": "TFLOP/s", "frac": tf / 157.3,
-                     "traffic": None, "kernel": plan.kernel_name(0), "algorithmic_flops_per_launch": flops},
+        # a generated kernel of vector-ALU fused multiply-adds (no matrix instructions exist for
+        # f32 operands in the vocabulary): priced against the part's published vector fp32 rate
+        "roofline": {"bound": "valu_fp32", "achieved": tf, "peak": 157.3, "unit": "TFLOP/s", "frac": tf / 157.3,
+                     "traffic": None, "traffic_source": "not profiled (plumbing config)", "kernel": plan.kernel_name(0),
+                     "algorithmic_flops_per_launch": flops},
     }
     rec.update(stats)
     if cpu:
@@ -301,12 +393,24 @@ def bench_generated_tc(m, dev, steps, warmup, cpu):
         "metric": "generated tensor-core GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "bf16",
         "config": {"workload": "bf16 GEMM M=N=K=4096 via the lazy tensor API, generated tensor-core kernel "
                                "(hand-written kernels off)"},
-        "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": tf / BF16_PEAK_TFLOPS, "traffic": None, "kernel": plan.kernel_name(0),
-                     "algorithmic_flops_per_launch": flops},
+        "roofline": _roofline("generated_tc", "mfma", tf, BF16_PEAK_TFLOPS, "TFLOP/s", plan.kernel_name(0),
+                              algorithmic_flops_per_launch=flops),
     }
     rec.update(stats)
+    if cpu:
+        rec["cpu_baseline"] = _gemm_cpu_baseline(n, n, n)
     return rec
+
+
+def bench_mfma_ceiling(m, dev, steps, warmup, cpu):
+    """Calibration only: the MFMA-only kernel at the size of the 4096^3 product."""
+    tf = _mfma_ceiling_tflops(m, dev)
+    return {"metric": "MFMA-only ceiling TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": 2.0 * 4096 ** 3 / tf / 1e9,
+            "dtype": "bf16", "config": {"workload": "calibration: 256 workgroups x 64 K steps of register-only "
+                                                    "v_mfma_f32_32x32x16_bf16 (the MFMA stream of the 4096^3 GEMM)"},
+            "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": tf / BF16_PEAK_TFLOPS, "traffic": 0, "traffic_source": "no memory operands",
+                         "kernel": "mfma_ceiling_kernel", "algorithmic_flops_per_launch": 2.0 * 4096 ** 3}}
 
 
 def bench_copy(m, dev, steps, warmup, cpu):
@@ -327,7 +431,7 @@ def bench_copy(m, dev, steps, warmup, cpu):
 
 
 WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "decoder": bench_decoder,
-             "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy}
+             "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling}
 PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc"]
 
 
@@ -369,7 +473,7 @@ def main():
         if "cpu_baseline" in r:
             r["cpu_baseline"]["cpu_model"] = cpu_model
             r["cpu_baseline"]["host_cores"] = os.cpu_count()
-    for k in ("median_ms", "min_ms"):
+    for k in ("median_ms", "min_ms", "plan_item", "direct_abi_ms_per_step", "vendor_reference"):
         if k in primary:
             line[k] = primary[k]
     if "cpu_baseline" in primary:

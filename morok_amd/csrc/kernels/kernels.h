@@ -57,4 +57,11 @@ int launch_fill_randint(void* stream, void* out, size_t n, unsigned long long se
 // Streaming device-to-device copy kernel (bytes % 16 == 0): traffic-counter calibration.
 int launch_copy(void* stream, const void* in, void* out, size_t bytes);
 
+
+// MFMA-only calibration kernel: `workgroups` workgroups of four waves, each wave issuing
+// k_steps x 64 v_mfma_f32_32x32x16_bf16 from registers (the instruction stream of one
+// 256 x 256 x 64*k_steps GEMM tile without its memory traffic): 2 * 256 * 256 * 64 * k_steps
+// flops per workgroup.  `out` (>= 4 bytes) is never written in practice.
+int launch_mfma_ceiling(void* stream, void* out, long workgroups, long k_steps);
+
 }  // namespace mrk

@@ -1,0 +1,67 @@
+// Calibration kernel: what the matrix pipes of this part sustain when nothing else competes.
+// One workgroup of four waves per compute unit; every wave issues the MFMA stream of one
+// 256x256 GEMM tile (64 v_mfma_f32_32x32x16_bf16 per 64-deep K step, sixteen independent
+// accumulators) from registers only: no global loads, no LDS traffic, no barriers.  The rate
+// it reaches is the ceiling a bf16 GEMM kernel is measured against next to the published peak
+// (the part lowers its clock under matrix load, so that ceiling sits below the peak).
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace mrk::dev {
+
+typedef __bf16 cal_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float cal_f32x16 __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ out, int k_steps, float seed) {
+    const int lane = threadIdx.x & 63;
+    cal_f32x16 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+    cal_bf16x8 fa[4], fb[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            fa[i][e] = (__bf16)(seed * (float)(lane + e + i));
+            fb[i][e] = (__bf16)(seed * (float)(lane - e - i));
+        }
+    for (int kt = 0; kt < k_steps; kt++) {
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++)
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        // keeps the loop a loop: the operands change in a way the compiler cannot fold
+        asm volatile("" : "+v"(fa[0]), "+v"(fb[0]));
+    }
+    float s = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) s += acc[i][j][e];
+    if (s == 12345.678f) out[0] = s;  // never true for the operands above; keeps the work alive
+}
+
+}  // namespace mrk::dev
+
+namespace mrk {
+
+int launch_mfma_ceiling(void* stream, void* out, long workgroups, long k_steps) {
+    if (workgroups <= 0 || k_steps <= 0 || workgroups > 0x7fffffffL || k_steps > 0x7fffffffL || !out)
+        return (int)hipErrorInvalidValue;
+    (void)hipGetLastError();
+    dev::mfma_ceiling_kernel<<<(unsigned)workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<float*>(out),
+                                                                                               (int)k_steps, 0.001f);
+    return (int)hipGetLastError();
+}
+
+}  // namespace mrk

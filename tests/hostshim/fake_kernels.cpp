@@ -48,4 +48,8 @@ int launch_copy(void* stream, const void*, void*, size_t) {
     mrk_shim_note_launch(stream, "copy");
     return 0;
 }
+int launch_mfma_ceiling(void* stream, void*, long, long) {
+    mrk_shim_note_launch(stream, "mfma_ceiling");
+    return 0;
+}
 }  // namespace mrk

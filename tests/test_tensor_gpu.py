@@ -94,6 +94,26 @@ def test_matmul_square_closed_form(T, fusion, oracle, n, tol):
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-4 * np.abs(ref).max())
 
 
+def test_matmul_config1_1024_cubed(T, oracle):
+    """The first benchmark configuration itself: A[1024x1024] @ B[1024x1024], entries uniform(-1, 1)
+    from seed 1, through Tensor::matmul (one generated kernel) against the CPU oracle on the same
+    inputs; also the reference's closed-form generators at this size (matmul.rs:669-677)."""
+    from morok_amd import synth
+
+    n = 1024
+    a, b = synth.uniform((n, n), 1, 0), synth.uniform((n, n), 1, 1)
+    c = T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b))
+    got = c.to_numpy()
+    assert c.kernels() == ["r_1024_1024_1024"]
+    ref = oracle.matmul_f32(a, b)
+    assert np.abs(got - ref).max() <= 1e-4 * np.abs(ref).max()  # f32 reduction tolerance
+    x = np.arange(n * n, dtype=np.int64)
+    a2 = ((x % 31) * 0.05 - 0.8).astype(np.float32).reshape(n, n)
+    b2 = ((x % 37) * 0.04 - 0.7).astype(np.float32).reshape(n, n)
+    got2 = T.Tensor.from_numpy(a2).matmul(T.Tensor.from_numpy(b2)).to_numpy()
+    assert np.abs(got2 - oracle.matmul_f32(a2, b2)).max() < 3.0  # the reference's tolerance at 1024
+
+
 def test_matmul_nonsquare_and_batched(T, fusion, oracle):
     rng = np.random.default_rng(5)
     a = rng.standard_normal((64, 512), dtype=np.float32)
