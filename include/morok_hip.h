@@ -504,6 +504,21 @@ typedef struct mrk_tensor mrk_tensor;
  * at creation; nbytes must equal numel * sizeof(dtype) (MRK_ERR_SIZE_MISMATCH otherwise). */
 int mrk_hip_tensor_from_bytes(int device_id, const void* data, size_t nbytes, const int64_t* shape, size_t ndim,
                               int dtype, mrk_tensor** out);
+/* Tensor::from_slice / from_raw_bytes without a device (data.rs:27-36,81-96): the tensor lives on
+ * the CPU device, its bytes are copied into host memory owned by the tensor and no GPU is
+ * touched.  This backend does not compute on the CPU: such a tensor can be read back, reshaped,
+ * and moved with mrk_hip_tensor_to; realizing a computation over it is UNSUPPORTED_DEVICE. */
+int mrk_hip_tensor_from_host_bytes(const void* data, size_t nbytes, const int64_t* shape, size_t ndim, int dtype,
+                                   mrk_tensor** out);
+/* Tensor::to (tensor/src/lib.rs:479-486).  device: "CPU", "HIP", "HIP:0", "AMD:0", "GPU"...  Same
+ * device: a new handle to the same tensor.  Otherwise a lazy COPY: nothing moves until the result
+ * (or something computed from it) is realized; the execution plan then carries a copy item that
+ * runs in order with its kernels on every execute (tensor/src/realize.rs:1002-1011), so a prepared
+ * plan re-uploads the host data each time it runs.  A copy to "CPU" must be the last step of a
+ * realization.  Plans with copy items cannot be replayed through mrk_hip_plan_execute_graph. */
+int mrk_hip_tensor_to(const mrk_tensor* t, const char* device, mrk_tensor** out);
+/* Tensor::device (lib.rs:464-466): writes "CPU" or "HIP:<n>" (NUL-terminated) into out[cap]. */
+int mrk_hip_tensor_device(const mrk_tensor* t, char* out, size_t cap);
 /* Wraps an existing device buffer (shared, not copied). */
 int mrk_hip_tensor_from_buffer(const mrk_buffer* b, const int64_t* shape, size_t ndim, int dtype, mrk_tensor** out);
 int mrk_hip_tensor_const(int device_id, double value, int dtype, mrk_tensor** out);          /* lib.rs:432 */

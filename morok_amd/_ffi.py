@@ -184,6 +184,9 @@ _SIGS = {
     "mrk_hip_queue_destroy": (None, [C.c_void_p]),
     # lazy tensors
     "mrk_hip_tensor_from_bytes": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_from_host_bytes": (C.c_int, [C.c_void_p, C.c_size_t, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),
+    "mrk_hip_tensor_to": (C.c_int, [C.c_void_p, C.c_char_p, c_void_pp]),
+    "mrk_hip_tensor_device": (C.c_int, [C.c_void_p, C.c_char_p, C.c_size_t]),
     "mrk_hip_tensor_from_buffer": (C.c_int, [C.c_void_p, c_i64_p, C.c_size_t, C.c_int, c_void_pp]),
     "mrk_hip_tensor_const": (C.c_int, [C.c_int, C.c_double, C.c_int, c_void_pp]),
     "mrk_hip_tensor_full": (C.c_int, [C.c_int, c_i64_p, C.c_size_t, C.c_double, C.c_int, c_void_pp]),

@@ -49,7 +49,45 @@ class BuiltinProgram final : public Program {
     Fn fn_;
 };
 
+class CopyProgram final : public Program {
+  public:
+    CopyProgram(int device_id, ffi::Stream stream, bool to_device, std::shared_ptr<std::vector<uint8_t>> host)
+        : device_id_(device_id), stream_(stream), to_device_(to_device), host_(std::move(host)) {
+        name_ = std::string(to_device ? "copy_h2d_" : "copy_d2h_") + std::to_string(host_->size());
+    }
+    int execute(void* const* buffers, size_t nbufs, const int64_t* vals, size_t nvals, const size_t* global,
+                const size_t* local) override {
+        return execute_on(stream_, buffers, nbufs, vals, nvals, global, local);
+    }
+    int execute_on(ffi::Stream stream, void* const* buffers, size_t nbufs, const int64_t*, size_t nvals, const size_t*,
+                   const size_t*) override {
+        if (nbufs != 1 || nvals != 0 || !buffers[0])
+            return failf(kInvalidArgument, "copy item '%s' takes exactly one device buffer", name_.c_str());
+        if (host_->empty()) return kOk;
+        MRK_HIP(ffi::set_device(device_id_), "hipSetDevice");
+        if (to_device_) MRK_HIP(ffi::memcpy_htod_async(buffers[0], host_->data(), host_->size(), stream), "hipMemcpyAsync(HtoD)");
+        else MRK_HIP(ffi::memcpy_dtoh_async(host_->data(), buffers[0], host_->size(), stream), "hipMemcpyAsync(DtoH)");
+        return kOk;
+    }
+    const char* name() const override { return name_.c_str(); }
+    bool capturable() const override { return false; }
+
+  private:
+    int device_id_;
+    ffi::Stream stream_;
+    bool to_device_;
+    std::shared_ptr<std::vector<uint8_t>> host_;
+    std::string name_;
+};
+
 }  // namespace
+
+int create_copy_program(int device_id, ffi::Stream stream, bool to_device, std::shared_ptr<std::vector<uint8_t>> host,
+                        std::unique_ptr<Program>* out) {
+    if (!host) return fail(kInvalidArgument, "copy item: no host memory");
+    out->reset(new CopyProgram(device_id, stream, to_device, std::move(host)));
+    return kOk;
+}
 
 int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, const int64_t* params, size_t nparams,
                            std::unique_ptr<Program>* out) {

@@ -1,5 +1,6 @@
 // extern "C" surface of libmorok_hip.so (declared in include/morok_hip.h).
 #include <cstdlib>
+#include <cctype>
 #include <cstring>
 
 #include "../../include/morok_hip.h"
@@ -1062,6 +1063,41 @@ int mrk_hip_tensor_from_bytes(int device_id, const void* data, size_t nbytes, co
     if (nbytes) MRK_NONNULL(data);
     clear_error();
     return wrap_tensor(Tensor::from_raw_bytes(device_id, data, nbytes, vec64(shape, ndim), static_cast<Scalar>(dtype)), out);
+}
+int mrk_hip_tensor_from_host_bytes(const void* data, size_t nbytes, const int64_t* shape, size_t ndim, int dtype, mrk_tensor** out) {
+    MRK_NONNULL(out);
+    MRK_DTYPE(dtype);
+    if (nbytes) MRK_NONNULL(data);
+    clear_error();
+    return wrap_tensor(Tensor::from_host_bytes(data, nbytes, vec64(shape, ndim), static_cast<Scalar>(dtype)), out);
+}
+// "CPU" (any case) -> kCpuDevice, else the HIP spellings of parse_device_spec
+static int parse_tensor_device(const char* spec, int* device_id) {
+    std::string s(spec);
+    for (char& c : s) c = static_cast<char>(std::toupper(static_cast<unsigned char>(c)));
+    if (s == "CPU" || s == "CPU:0") {
+        *device_id = kCpuDevice;
+        return kOk;
+    }
+    return parse_device_spec(spec, device_id);
+}
+int mrk_hip_tensor_to(const mrk_tensor* t, const char* device, mrk_tensor** out) {
+    MRK_NONNULL(t);
+    MRK_NONNULL(device);
+    MRK_NONNULL(out);
+    clear_error();
+    int id = 0;
+    MRK_TRY(parse_tensor_device(device, &id));
+    return wrap_tensor(t->t.to(id), out);
+}
+int mrk_hip_tensor_device(const mrk_tensor* t, char* out, size_t cap) {
+    MRK_NONNULL(t);
+    MRK_NONNULL(out);
+    const int id = t->t.device();
+    const std::string name = id == kCpuDevice ? std::string("CPU") : "HIP:" + std::to_string(id);
+    if (cap < name.size() + 1) return fail(kInvalidArgument, "tensor_device: output too small");
+    std::memcpy(out, name.c_str(), name.size() + 1);
+    return kOk;
 }
 int mrk_hip_tensor_from_buffer(const mrk_buffer* b, const int64_t* shape, size_t ndim, int dtype, mrk_tensor** out) {
     MRK_NONNULL(b);

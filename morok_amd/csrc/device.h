@@ -71,6 +71,9 @@ class Program {
     virtual int execute_on(ffi::Stream stream, void* const* buffers, size_t nbufs, const int64_t* vals, size_t nvals,
                            const size_t* global, const size_t* local) = 0;
     virtual const char* name() const = 0;
+    // false for items that are not kernel launches (COPY items between host and device memory):
+    // they are not recorded into HIP graphs.
+    virtual bool capturable() const { return true; }
 };
 
 class Compiler {

@@ -214,6 +214,10 @@ void ExecutionPlan::drop_graph() {
 int ExecutionPlan::execute_graph() {
     if (!built_) MRK_TRY(build());
     if (kernels_.empty()) return kOk;
+    for (const auto& pk : kernels_)
+        if (!pk.kernel->program->capturable())
+            return failf(kInvalidArgument, "execution plan: item '%s' is a host/device copy and cannot be recorded into a "
+                                           "graph; use execute()", pk.kernel->entry_point.c_str());
     std::shared_ptr<Allocator> alloc;
     MRK_TRY(AllocatorRegistry::global().get(device_id_, &alloc));
     ffi::Stream stream = alloc->stream();

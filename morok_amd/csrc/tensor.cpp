@@ -100,6 +100,13 @@ static TensorRef mk(TKind kind, Scalar dt, std::vector<int64_t> shape, std::vect
     n->device_id = dev;
     return n;
 }
+// nodes whose value always exists in memory before a consumer kernel reads it
+static bool is_boundary_kind(const TensorNode* n) {
+    return n->kind == TKind::Reduce || n->kind == TKind::Contiguous || n->kind == TKind::Copy;
+}
+static std::string device_name(int device_id) {
+    return device_id == kCpuDevice ? std::string("CPU") : "HIP:" + std::to_string(device_id);
+}
 static bool norm_axis(int64_t* a, int64_t nd) {
     if (*a < 0) *a += nd;
     return *a >= 0 && *a < nd;
@@ -124,6 +131,35 @@ Tensor Tensor::from_raw_bytes(int device_id, const void* data, size_t nbytes, co
     auto buf = std::make_shared<Buffer>(dev->allocator, expected, opt);
     if (expected && buf->copyin(data, expected) != kOk) return Tensor();  // data.rs:66-67: copied at creation
     return from_buffer(buf, shape, dtype);
+}
+
+Tensor Tensor::from_host_bytes(const void* data, size_t nbytes, const std::vector<int64_t>& shape, Scalar dtype) {
+    int64_t numel = 1;
+    for (int64_t d : shape) {
+        if (d < 0) return bad(kInvalidArgument, "from_slice: negative dimension");
+        numel *= d;
+    }
+    const size_t expected = static_cast<size_t>(numel) * scalar_size(dtype);
+    if (nbytes != expected)  // data.rs:81-96
+        return bad(kSizeMismatch, "from_raw_bytes: data length " + std::to_string(nbytes) + " != expected " +
+                                      std::to_string(expected) + " (" + std::to_string(numel) + " elements * " +
+                                      std::to_string(scalar_size(dtype)) + " bytes)");
+    if (expected && !data) return bad(kInvalidArgument, "from_slice: null data");
+    auto n = mk(TKind::Buffer, dtype, shape, {}, kCpuDevice);
+    const uint8_t* p = static_cast<const uint8_t*>(data);
+    n->host = std::make_shared<std::vector<uint8_t>>(p, p + expected);  // data.rs:66-67: copied at creation
+    return Tensor(n);
+}
+
+Tensor Tensor::to(int device_id) const {
+    if (!n_) return bad(kInvalidArgument, "to: invalid tensor");
+    if (n_->device_id == device_id) return *this;  // lib.rs:480-482
+    if (device_id != kCpuDevice) {
+        int count = 0;
+        if (ffi::device_count(&count) != 0 || device_id < 0 || device_id >= count)
+            return bad(kInvalidDevice, "invalid device: HIP:" + std::to_string(device_id));
+    }
+    return Tensor(mk(TKind::Copy, n_->dtype, n_->shape, {n_}, device_id));
 }
 
 Tensor Tensor::from_buffer(std::shared_ptr<Buffer> buf, const std::vector<int64_t>& shape, Scalar dtype) {
@@ -1056,6 +1092,7 @@ struct Scheduler {
     std::unique_ptr<ExecutionPlan> plan;
     RealizeStats stats;
     std::vector<TensorNode*> produced;  // nodes this realization gave a buffer
+    std::vector<TensorNode*> produced_host;  // CPU nodes this realization gave host memory (device -> CPU copies)
     std::unordered_map<const TensorNode*, int> uses;  // consumers of a node within the realised graph
 
     void count_uses(const TensorNode* root) {
@@ -1114,7 +1151,7 @@ struct Scheduler {
         *max_numel = std::max(*max_numel, n->numel());
         if (n->buffer) return;
         TensorNode* other = nullptr;
-        if (n != root && (n->kind == TKind::Reduce || n->kind == TKind::Contiguous || fusable(n) ||
+        if (n != root && (is_boundary_kind(n) || fusable(n) ||
                           residual_matmul(const_cast<TensorNode*>(n), &other))) {
             out.push_back(const_cast<TensorNode*>(n));
             return;
@@ -1243,7 +1280,7 @@ struct Scheduler {
             // is cheaper evaluated inside the add than written out first
             const TensorNode* rb = r;
             while (!rb->buffer && rb->kind == TKind::Reshape) rb = rb->src[0].get();
-            if (!(rb->buffer || rb->kind == TKind::Reduce || rb->kind == TKind::Contiguous || fusable(rb))) continue;
+            if (!(rb->buffer || is_boundary_kind(rb) || fusable(rb))) continue;
             int64_t M, N, K, batch;
             matmul_extents(mm, &M, &N, &K, &batch);
             if (!gemm_bf16_residual_supported(M, N, K, batch) || gemm_bf16_workspace_bytes(M, N, K, batch)) continue;
@@ -1273,8 +1310,79 @@ struct Scheduler {
         return kOk;
     }
 
+    // Everything a realization computes runs on a HIP device.  Host-resident data may enter a
+    // graph only through a COPY node (Tensor::to), and a copy back to the CPU only as the root.
+    int check_placement(const TensorNode* root) {
+        if (root->device_id == kCpuDevice && root->kind != TKind::Copy)
+            return fail(kUnsupportedDevice, "this backend computes on HIP devices only: the tensor lives on the CPU device; "
+                                            "move its inputs with to(\"HIP:0\") first");
+        std::vector<const TensorNode*> stack{root};
+        std::set<const TensorNode*> seen{root};
+        while (!stack.empty()) {
+            const TensorNode* n = stack.back();
+            stack.pop_back();
+            if (n->buffer) continue;
+            if (n->kind == TKind::Copy && n->device_id != kCpuDevice) continue;  // checked when it is materialised
+            if (n->kind == TKind::Copy && n != root)
+                return fail(kUnsupportedDevice, "a copy to the CPU device can only be the last step of a realization");
+            if (n->kind == TKind::Buffer && n->host)
+                return fail(kUnsupportedDevice, "an operand lives on the CPU device: move it with to(\"HIP:0\") before computing "
+                                                "with it (this backend does not compute on the CPU)");
+            for (const TensorRef& c : n->src)
+                if (seen.insert(c.get()).second) stack.push_back(c.get());
+        }
+        return kOk;
+    }
+
+    int add_copy_item(bool to_device, std::shared_ptr<std::vector<uint8_t>> host, const std::shared_ptr<Buffer>& device_side) {
+        std::unique_ptr<Program> p;
+        MRK_TRY(create_copy_program(dev->device_id, dev->allocator->stream(), to_device, std::move(host), &p));
+        auto k = std::make_shared<CachedKernel>();
+        k->entry_point = p->name();
+        k->program = std::move(p);
+        k->device = "HIP:" + std::to_string(dev->device_id);
+        return add_kernel(k, {device_side}, false);
+    }
+
+    // COPY nodes become copy items of the plan, executed in order with its kernels
+    // (tensor/src/realize.rs:1002-1011): nothing is transferred while scheduling.
+    int materialize_copy(TensorNode* n) {
+        TensorNode* s = n->src[0].get();
+        const size_t bytes = static_cast<size_t>(n->numel()) * scalar_size(n->dtype);
+        if (n->device_id == kCpuDevice) {  // device -> CPU
+            if (s->device_id == kCpuDevice) return fail(kRuntime, "runtime error: copy between two CPU tensors");
+            MRK_TRY(materialize(s));
+            auto host = std::make_shared<std::vector<uint8_t>>(bytes);
+            if (bytes) MRK_TRY(add_copy_item(false, host, s->buffer));
+            n->host = host;
+            n->host_from = dev->device_id;
+            produced_host.push_back(n);
+            return kOk;
+        }
+        if (s->device_id != kCpuDevice)
+            return failf(kCopyFailed, "copy operation failed: cross-device copy %s -> %s is not supported", device_name(s->device_id).c_str(),
+                         device_name(n->device_id).c_str());
+        // CPU -> device: the source must be stored bytes (a reshape of stored bytes is the same bytes)
+        const TensorNode* h = s;
+        while (!h->host && h->kind == TKind::Reshape) h = h->src[0].get();
+        if (!h->host)
+            return fail(kUnsupportedDevice, "to(): the source is an unrealised expression on the CPU device; this backend does not "
+                                            "compute on the CPU - move the stored operands to the device first and compute there");
+        if (h->host_from != kCpuDevice) {  // bytes that a device is still writing (an earlier copy to the CPU)
+            std::shared_ptr<Allocator> a;
+            MRK_TRY(AllocatorRegistry::global().get(h->host_from, &a));
+            MRK_TRY(a->synchronize());
+        }
+        auto out = new_buffer(n);
+        if (bytes) MRK_TRY(add_copy_item(true, h->host, out));
+        n->buffer = out;
+        produced.push_back(n);
+        return kOk;
+    }
+
     int materialize(TensorNode* n) {
         if (n->buffer) return kOk;
+        if (n->kind == TKind::Copy) return materialize_copy(n);
         if (n->numel() > 0 && fusable(n)) return materialize_fused(n);
         {
             TensorNode* other = nullptr;
@@ -1289,7 +1397,7 @@ struct Scheduler {
         if (n->kind == TKind::Reshape || n->kind == TKind::Contiguous) {
             TensorNode* s = n->src[0].get();
             TensorNode* other = nullptr;
-            if (s->buffer || s->kind == TKind::Reduce || s->kind == TKind::Contiguous || fusable(s) || residual_matmul(s, &other)) {
+            if (s->buffer || is_boundary_kind(s) || fusable(s) || residual_matmul(s, &other)) {
                 MRK_TRY(materialize(s));
                 n->buffer = s->buffer;
                 produced.push_back(n);
@@ -1356,7 +1464,7 @@ struct Scheduler {
             bool ok = !in->buffer && strided_view(in, &v) && v.base != in && v.strides.size() == 4 && v.offset % 8 == 0;
             // only data that is (or will be) in memory anyway: a view of an unrealised
             // elementwise expression is cheaper computed over the view alone
-            ok = ok && (v.base->buffer || v.base->kind == TKind::Reduce || v.base->kind == TKind::Contiguous || fusable(v.base));
+            ok = ok && (v.base->buffer || is_boundary_kind(v.base) || fusable(v.base));
             if (ok) {
                 for (int a = 0; a < 4; a++)
                     if (in->shape[a] == 1) v.strides[a] = 0;
@@ -1728,15 +1836,25 @@ int prepare_locked(const TensorRef& root, std::unique_ptr<ExecutionPlan>* out, s
         Scheduler& s;
         bool armed = true;
         ~Rollback() {
-            if (armed)
-                for (TensorNode* t : s.produced) t->buffer = nullptr;
+            if (!armed) return;
+            for (TensorNode* t : s.produced) t->buffer = nullptr;
+            for (TensorNode* t : s.produced_host) t->host = nullptr;
         }
     } rollback{s};
-    MRK_TRY(DeviceFactoryRegistry::global().device("HIP", root->device_id, &s.dev));
-    s.plan.reset(new ExecutionPlan(root->device_id));
+    // a copy to the CPU is scheduled on the device its source lives on
+    const bool to_cpu = root->device_id == kCpuDevice && root->kind == TKind::Copy;
+    const int device_id = to_cpu ? root->src[0]->device_id : root->device_id;
+    MRK_TRY(s.check_placement(root.get()));
+    MRK_TRY(DeviceFactoryRegistry::global().device("HIP", device_id, &s.dev));
+    s.plan.reset(new ExecutionPlan(device_id));
     s.count_uses(root.get());
-    if (!root->buffer) MRK_TRY(s.materialize(root.get()));
-    s.plan->set_outputs({s.plan->add_buffer(root->buffer)});
+    if (to_cpu) {
+        if (!root->host) MRK_TRY(s.materialize(root.get()));
+        s.plan->set_outputs({s.plan->add_buffer(root->src[0]->buffer)});  // the device side of the copy stays whole
+    } else {
+        if (!root->buffer) MRK_TRY(s.materialize(root.get()));
+        s.plan->set_outputs({s.plan->add_buffer(root->buffer)});
+    }
     // Intermediates share blocks by liveness (tensor/src/memory_planner.rs); their contents do
     // not outlive the plan's execution, so their nodes go back to being lazy: only the root
     // keeps its buffer.  MOROK_NO_MEMORY_PLANNER=1 keeps every intermediate resident.
@@ -1749,6 +1867,7 @@ int prepare_locked(const TensorRef& root, std::unique_ptr<ExecutionPlan>* out, s
         if (planner && t != root.get()) t->buffer = nullptr;
         else if (kept) kept->push_back(t);
     }
+    if (kept) kept->insert(kept->end(), s.produced_host.begin(), s.produced_host.end());
     s.stats.buffers_reused = s.plan->memory_plan().buffers_reused;
     s.stats.memory_saved = s.plan->memory_plan().memory_saved;
     s.stats.elapsed_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
@@ -1767,7 +1886,7 @@ int Tensor::prepare(std::unique_ptr<ExecutionPlan>* out) const {
 int Tensor::realize() const {
     if (!n_) return fail(kInvalidArgument, "realize: invalid tensor");
     std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
-    if (n_->buffer) {
+    if (n_->buffer || (n_->device_id == kCpuDevice && n_->host)) {
         g_stats = RealizeStats();
         return kOk;
     }
@@ -1779,7 +1898,10 @@ int Tensor::realize() const {
     // queues its reads behind these kernels on the device's in-order stream.
     int rc = plan->execute();
     if (rc != kOk) {
-        for (TensorNode* t : kept) t->buffer = nullptr;  // nothing was computed into them
+        for (TensorNode* t : kept) {  // nothing was computed into them
+            t->buffer = nullptr;
+            if (t->kind == TKind::Copy && t->device_id == kCpuDevice) t->host = nullptr;
+        }
         return rc;
     }
     g_stats.elapsed_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
@@ -1795,14 +1917,31 @@ std::shared_ptr<Buffer> Tensor::buffer() const {
 int Tensor::to_bytes(void* dst, size_t nbytes) const {
     if (!n_) return fail(kInvalidArgument, "to_vec: invalid tensor");
     std::shared_ptr<Buffer> buf;
+    std::shared_ptr<std::vector<uint8_t>> host;
+    int host_from = kCpuDevice;
     {
         std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
-        if (!n_->buffer) MRK_TRY(realize());
-        buf = n_->buffer;
+        if (n_->device_id == kCpuDevice) {
+            if (!n_->host) MRK_TRY(realize());
+            host = n_->host;
+            host_from = n_->host_from;
+        } else {
+            if (!n_->buffer) MRK_TRY(realize());
+            buf = n_->buffer;
+        }
     }
     const size_t expect = static_cast<size_t>(n_->numel()) * scalar_size(n_->dtype);
     if (nbytes != expect) return failf(kSizeMismatch, "size mismatch: expected %zu, got %zu", expect, nbytes);
     if (expect == 0) return kOk;
+    if (host) {
+        if (host_from != kCpuDevice) {  // the copy that fills these bytes was queued on that device's stream
+            std::shared_ptr<Allocator> a;
+            MRK_TRY(AllocatorRegistry::global().get(host_from, &a));
+            MRK_TRY(a->synchronize());
+        }
+        std::memcpy(dst, host->data(), expect);
+        return kOk;
+    }
     return buf->copyout(dst, nbytes);
 }
 

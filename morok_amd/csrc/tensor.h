@@ -31,8 +31,11 @@
 namespace mrk {
 
 enum class TKind : uint8_t {
-    Buffer, Const, Unary, Binary, Where, Cast, Reduce, Reshape, Permute, Expand, Shrink, Iota, Cat, Gather, Contiguous,
+    Buffer, Const, Unary, Binary, Where, Cast, Reduce, Reshape, Permute, Expand, Shrink, Iota, Cat, Gather, Contiguous, Copy,
 };
+
+// Device id of data that lives in host memory (DeviceSpec::Cpu); HIP devices are 0, 1, ...
+constexpr int kCpuDevice = -1;
 
 enum class HintKind : uint8_t { None, Softmax, Matmul, Sdpa };
 
@@ -49,6 +52,11 @@ struct TensorNode {
     double cval = 0.0;          // constant value
     int device_id = 0;
     std::shared_ptr<Buffer> buffer;  // set once the node is materialised (row-major contiguous)
+    // Host-resident bytes of a CPU tensor (device_id == kCpuDevice): the data of a tensor created
+    // from a slice, or the destination of a device -> CPU copy.  host_from is the device whose
+    // stream must be synchronized before the bytes of such a copy are read (kCpuDevice: none).
+    std::shared_ptr<std::vector<uint8_t>> host;
+    int host_from = kCpuDevice;
     // fused-kernel hint: the node is the root of a composed graph a hand-written kernel covers
     HintKind hint = HintKind::None;
     std::vector<TensorRef> hint_inputs;
@@ -86,6 +94,13 @@ class Tensor {
     static Tensor from_raw_bytes(int device_id, const void* data, size_t nbytes, const std::vector<int64_t>& shape,
                                  Scalar dtype);
     static Tensor from_buffer(std::shared_ptr<Buffer> buf, const std::vector<int64_t>& shape, Scalar dtype);
+    // Tensor::from_slice / from_raw_bytes without a device (data.rs:27-36,81-96): the bytes stay in
+    // host memory; nothing touches a GPU until the tensor is moved with to() and realized.
+    static Tensor from_host_bytes(const void* data, size_t nbytes, const std::vector<int64_t>& shape, Scalar dtype);
+    // Tensor::to (lib.rs:479-486): same device -> the same tensor; otherwise a lazy COPY node, which
+    // realization turns into a copy item of the execution plan (realize.rs:1002-1011).
+    Tensor to(int device_id) const;
+    int device() const { return n_ ? n_->device_id : 0; }  // lib.rs:464-466; kCpuDevice for host data
     static Tensor const_(double value, Scalar dtype, int device_id = 0);                           // lib.rs:432
     static Tensor full(const std::vector<int64_t>& shape, double value, Scalar dtype, int device_id = 0);  // lib.rs:251
 

@@ -77,6 +77,35 @@ class Tensor:
         return cls(h)
 
     @classmethod
+    def from_slice(cls, data, dtype=None):
+        """Tensor::from_slice (tensor/src/data.rs:27-36): a tensor on the CPU device; its bytes stay
+        in host memory until it is moved with to() and the result is realized."""
+        arr = np.ascontiguousarray(data)
+        if arr.dtype == np.float64 and dtype is None:
+            arr = arr.astype(np.float32)  # Python floats stand for f32 literals
+        tag = dtype if dtype is not None else _TAG_OF[arr.dtype]
+        shape, nd = _i64(arr.shape)
+        h = C.c_void_p()
+        check(lib.mrk_hip_tensor_from_host_bytes(arr.ctypes.data_as(C.c_void_p), arr.nbytes, shape, nd, tag, C.byref(h)))
+        return cls(h)
+
+    @classmethod
+    def from_slice_with(cls, data, device="CPU", dtype=None):
+        """Tensor::from_slice_with(..).device(..) (data.rs:39-52): host data, then to(device)."""
+        return cls.from_slice(data, dtype).to(device)
+
+    def to(self, device):
+        """Tensor::to (tensor/src/lib.rs:479-486): a lazy COPY to "CPU" / "HIP:0"; the same tensor when
+        it already lives there."""
+        return self._new(lib.mrk_hip_tensor_to, str(device).encode())
+
+    @property
+    def device(self):
+        buf = C.create_string_buffer(32)
+        check(lib.mrk_hip_tensor_device(self._h, buf, 32))
+        return buf.value.decode()
+
+    @classmethod
     def from_bytes(cls, raw, shape, dtype, device_id=0):
         raw = bytes(raw)
         shp, nd = _i64(shape)
@@ -304,6 +333,10 @@ class Tensor:
 
     def to_vec(self):
         return self.to_numpy().reshape(-1)
+
+    def as_vec(self):
+        """Tensor::as_vec (tensor/src/data.rs:211-236): the flat contents (realizes if needed)."""
+        return self.to_vec()
 
     def buffer(self):
         h = C.c_void_p()

@@ -41,7 +41,7 @@ struct FakeGraph {
 std::map<void*, size_t> g_capturing;  // stream -> launches recorded so far
 size_t g_graph_launches = 0, g_graphs_alive = 0;
 bool g_events_pending = false;  // event_query answers "not ready" while set
-// trace of stream operations ("memset:S", "record:E:S", "wait:S:E", "launch:S", "dtod:S"; S = stream
+// trace of stream operations ("memset:S", "record:E:S", "wait:S:E", "launch:S", "dtod:S", "htod:S", "dtoh:S"; S = stream
 // number in creation order, E = event number), kept while enabled
 bool g_trace_on = false;
 std::string g_trace;
@@ -156,11 +156,13 @@ int memset_async(void* dst, int value, size_t bytes, Stream s) {
     std::memset(dst, value, bytes);
     return 0;
 }
-int memcpy_htod_async(void* dst, const void* src, size_t bytes, Stream) {
+int memcpy_htod_async(void* dst, const void* src, size_t bytes, Stream s) {
+    { std::lock_guard<std::mutex> l(g_mu); trace("htod:" + std::to_string(stream_no(s))); }
     std::memcpy(dst, src, bytes);
     return 0;
 }
-int memcpy_dtoh_async(void* dst, const void* src, size_t bytes, Stream) {
+int memcpy_dtoh_async(void* dst, const void* src, size_t bytes, Stream s) {
+    { std::lock_guard<std::mutex> l(g_mu); trace("dtoh:" + std::to_string(stream_no(s))); }
     std::memcpy(dst, src, bytes);
     return 0;
 }

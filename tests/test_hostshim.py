@@ -607,6 +607,84 @@ def test_failed_schedule_leaves_the_graph_lazy(T, shim):
     assert len(again.kernels()) == 2
 
 
+# ------------------------------------------------------------------ Tensor::to / COPY items
+def test_host_tensors_and_lazy_device_copies(T, shim):
+    """tensor/src/realize.rs:1322-1347 (device of from_slice, to() on the same / another device) and
+    realize.rs:1002-1011 (COPY as an item of the plan, executed in order with the kernels)."""
+    T.set_fusion(False)
+    x = np.arange(12, dtype=np.float32).reshape(3, 4)
+    allocs = shim.mrk_shim_alloc_calls()
+    shim.mrk_shim_trace(1)
+    a = T.Tensor.from_slice(x)
+    assert a.device == "CPU" and a.shape == (3, 4)          # from_slice defaults to the CPU device
+    assert a.to("CPU").device == "CPU" and a.to("cpu").to_numpy().tolist() == x.tolist()
+    b = a.to("HIP:0")
+    assert b.device == "HIP:0" and a.device == "CPU"        # the source stays where it was
+    assert T.Tensor.from_slice_with(x, device="HIP").device == "HIP:0"
+    # lazy: neither creation nor to() allocated device memory or moved a byte
+    assert shim.mrk_shim_alloc_calls() == allocs and hostshim_lib.trace(shim) == []
+    b.realize()
+    assert b.kernels() == ["copy_h2d_48"] and hostshim_lib.trace(shim).count("htod:0") == 1
+    assert b.to_numpy().tolist() == x.tolist()
+    # a computation over the copy: the copy item precedes the kernel in the same plan
+    shim.mrk_shim_trace(1)
+    c = T.Tensor.from_slice(x).to("HIP:0").try_mul(2.0)
+    plan = c.prepare()
+    assert [plan.kernel_name(i) for i in range(plan.kernel_count)] == ["copy_h2d_48", "E_12_4"]
+    assert "htod:0" not in hostshim_lib.trace(shim)          # deferred to execute time
+    plan.execute()
+    plan.execute()
+    ops = hostshim_lib.trace(shim)
+    assert ops.count("htod:0") == 2 and ops.index("htod:0") < ops.index("launch:0")
+    with pytest.raises(MorokHipError) as e:                   # copies are not graph nodes
+        plan.execute_graph()
+    assert "copy" in str(e.value)
+    # device -> CPU as the last step, and the whole round trip in one plan
+    back = T.Tensor.from_slice(x).to("HIP:0").to("CPU")
+    assert back.device == "CPU"
+    assert back.to_numpy().tolist() == x.tolist() and back.kernels() == ["copy_h2d_48", "copy_d2h_48"]
+    n = shim.mrk_shim_launches()
+    assert back.as_vec().tolist() == x.ravel().tolist() and shim.mrk_shim_launches() == n  # realized once
+    assert back.to("HIP:0").realize().kernels() == ["copy_h2d_48"]      # host bytes of a copy can go up again
+    # a reshape of stored host bytes is the same bytes
+    assert T.Tensor.from_slice(x).try_reshape([4, 3]).to("HIP:0").to_numpy().tolist() == x.reshape(4, 3).tolist()
+
+
+def test_host_tensor_errors(T, shim):
+    x = np.ones((4,), np.float32)
+    cpu = T.Tensor.from_slice(x)
+    for bad in (lambda: cpu.try_add(1.0).realize(),                       # no CPU compute in this backend
+                lambda: cpu.try_add(1.0).to("HIP:0").realize(),           # not stored bytes
+                lambda: cpu.try_add(T.Tensor.from_numpy(x)).realize(),    # operand left on the CPU
+                lambda: T.Tensor.from_numpy(x).to("CPU").to("HIP:0").try_add(cpu.to("HIP:0").to("CPU")).realize()):
+        with pytest.raises(MorokHipError) as e:
+            bad()
+        assert e.value.code == 13, str(e.value)                            # UnsupportedDevice
+    with pytest.raises(MorokHipError) as e:
+        cpu.to("HIP:5")
+    assert e.value.code == 3
+    with pytest.raises(MorokHipError):
+        cpu.to("TPU:0")
+    with pytest.raises(MorokHipError) as e:
+        T.Tensor.from_slice(np.zeros(3, np.float32)).to_numpy().shape and lib_check_size(T)
+    assert e.value.code == 1
+    # a failed realization leaves the graph lazy (no half-made host buffers)
+    t = T.Tensor.from_numpy(x).try_add(1.0).to("CPU")
+    shim.mrk_shim_fail_module_load_after(0)
+    morok_amd.kernel_cache_clear()
+    with pytest.raises(MorokHipError):
+        t.realize()
+    assert t.to_numpy().shape == (4,)
+
+
+def lib_check_size(T):
+    from morok_amd._ffi import check, lib
+
+    t = T.Tensor.from_slice(np.zeros(3, np.float32))
+    out = np.empty(2, np.float32)
+    check(lib.mrk_hip_tensor_to_bytes(t._h, out.ctypes.data_as(C.c_void_p), out.nbytes))
+
+
 def test_ops_refuse_undersized_buffers(dev, shim):
     from morok_amd import ops
 

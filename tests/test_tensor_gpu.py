@@ -1019,3 +1019,58 @@ def test_matmul_bf16_generated_tensor_core(T, oracle):
         if tc:
             assert "__builtin_amdgcn_mfma" in T.last_kernel_sources()[0] and "__shared__" in T.last_kernel_sources()[0]
     T.set_fusion(True)
+
+
+# ---------------------------------------------------------------- Tensor::to / COPY plan items
+def test_host_tensors_through_device_copies(T, oracle):
+    """Host-resident tensors (Tensor::from_slice), moved with to("HIP:0") as lazy COPY nodes that
+    the plan executes in order with its kernels (tensor/src/lib.rs:479-486,
+    tensor/src/realize.rs:1002-1011), on the reference's own matmul / softmax cases."""
+    for key in ("matmul_2x2", "matmul_3x3"):
+        g = GOLD[key]
+        a, b = T.Tensor.from_slice(f32(g["a"])), T.Tensor.from_slice(f32(g["b"]))
+        assert a.device == "CPU"
+        c = a.to("HIP:0").matmul(b.to("HIP:0"))
+        got = c.to_numpy()
+        assert [k.split("_")[0] for k in c.kernels()] == ["copy", "copy", "r"]
+        np.testing.assert_allclose(got, f32(g["expected"]), atol=g["tol"])
+    # closed-form generators at 256 (matmul.rs:669-677), result copied back to the CPU device
+    n = 256
+    x = np.arange(n * n, dtype=np.int64)
+    a = ((x % 31) * 0.05 - 0.8).astype(np.float32).reshape(n, n)
+    b = ((x % 37) * 0.04 - 0.7).astype(np.float32).reshape(n, n)
+    c = T.Tensor.from_slice(a).to("HIP:0").matmul(T.Tensor.from_slice(b).to("HIP:0")).to("CPU")
+    assert c.device == "CPU"
+    got = c.as_vec().reshape(n, n)
+    assert c.kernels()[-1].startswith("copy_d2h")
+    ref = oracle.matmul_f32(a, b)
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=1e-4 * np.abs(ref).max())
+    # softmax over host data: rows sum to one and match the oracle
+    from morok_amd import synth
+
+    s = synth.normal((64, 1000), 2, 0, sigma=2.0)
+    p = T.Tensor.from_slice(s).to("HIP:0").softmax(-1).to("CPU").to_numpy()
+    ref = oracle.softmax_f32(s)
+    np.testing.assert_allclose(p, ref, rtol=1e-5, atol=1e-9)
+    assert np.abs(p.sum(-1) - 1).max() < 1e-4
+
+
+def test_prepared_plan_reuploads_host_data_on_every_execute(T):
+    """The copy is an item of the plan, not a side effect of scheduling: executing a prepared plan
+    twice uploads twice, so each run starts from the host bytes even if the device copy of the
+    input was overwritten in between (here: by the memory planner handing its block on)."""
+    x = np.arange(4096, dtype=np.float32)
+    t = T.Tensor.from_slice(x).to("HIP:0").try_mul(3.0).try_add(1.0)
+    plan = t.prepare()
+    names = [plan.kernel_name(i) for i in range(plan.kernel_count)]
+    assert names[0] == "copy_h2d_16384" and len(names) == 2
+    for _ in range(2):
+        plan.execute()
+        np.testing.assert_array_equal(t.to_numpy(), x * 3 + 1)
+    # bf16 GEMM of host operands lands on the hand-written kernel after two copies
+    from morok_amd import synth, uop
+
+    a, b = synth.normal_bf16((256, 128), 7, 0), synth.normal_bf16((128, 256), 7, 1)
+    c = T.Tensor.from_slice(a, uop.BF16).to("HIP:0").matmul(T.Tensor.from_slice(b, uop.BF16).to("HIP:0"))
+    direct = T.Tensor.from_numpy(a, uop.BF16).matmul(T.Tensor.from_numpy(b, uop.BF16)).to_numpy()
+    assert np.array_equal(c.to_numpy(), direct) and c.kernels()[-1].startswith("gemm_bf16")
