@@ -332,8 +332,15 @@ int mrk_hip_sched_limit_dims(const size_t* dims, size_t n, const size_t* max_siz
                              size_t* nout);
 int mrk_hip_sched_get_contraction(const size_t* original, size_t n, const size_t* limited, size_t nl, size_t* group_of_dim);
 /* get_grouped_dims (gpudims.rs:331-382): launch extents for `dims` under `max_sizes` (NULL = no
- * limit; reverse != 0 for global indices) and, when raw/index_per_dim are given, the index of
- * every original dimension for one tuple of hardware indices. */
+ * limit) and, when raw/index_per_dim are given, the index of every original dimension for one
+ * tuple of hardware indices.  reverse: 0 = local indices (dims as given); 1 = global indices as
+ * this backend launches them: the dims are reversed before limiting and the indices after it, so
+ * the innermost axis is gidx0 whatever regrouping happened (tinygrad's order); 2 = the reference's
+ * literal code, which limits the dims as given and reverses only the index list.  Modes 1 and 2
+ * agree exactly when the dims read the same in both directions (one dim, [a, a], [a, b, a] ...);
+ * for every other dims list mode 2 gives dimension i an index that runs over the extent of
+ * dimension n-1-i (for [3, 5]: dimension 0 gets an index in [0, 5)), which is why generated
+ * kernels use mode 1.  A caller comparing with the reference's unit tests wants mode 2. */
 int mrk_hip_sched_grouped_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, int reverse,
                                size_t* launch, size_t cap, size_t* nlaunch, const size_t* raw, size_t* index_per_dim);
 /* Linearized kernels for the matmul shapes on the hot path, serialized in the wire format

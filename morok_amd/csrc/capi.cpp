@@ -631,7 +631,8 @@ int mrk_hip_sched_get_contraction(const size_t* original, size_t n, const size_t
 int mrk_hip_sched_grouped_dims(const size_t* dims, size_t n, const size_t* max_sizes, size_t nmax, int reverse,
                                size_t* launch, size_t cap, size_t* nlaunch, const size_t* raw, size_t* index_per_dim) {
     std::vector<size_t> mx(max_sizes, max_sizes + nmax);
-    GroupedDims g = get_grouped_dims(std::vector<size_t>(dims, dims + n), max_sizes ? &mx : nullptr, reverse != 0);
+    if (reverse < 0 || reverse > 2) return fail(kInvalidArgument, "grouped_dims: reverse must be 0, 1 or 2");
+    GroupedDims g = get_grouped_dims(std::vector<size_t>(dims, dims + n), max_sizes ? &mx : nullptr, static_cast<DimOrder>(reverse));
     put_dims(g.launch, launch, cap, nlaunch);
     if (raw && index_per_dim) {
         std::vector<size_t> r(raw, raw + g.launch.size());

@@ -245,25 +245,35 @@ bool get_contraction(const std::vector<size_t>& original, const std::vector<size
     return true;
 }
 
-GroupedDims get_grouped_dims(const std::vector<size_t>& dims, const std::vector<size_t>* max_sizes, bool reverse) {
+GroupedDims get_grouped_dims(const std::vector<size_t>& dims, const std::vector<size_t>* max_sizes, DimOrder order) {
     GroupedDims g;
     g.original = dims;
-    g.reverse = reverse;
+    g.order = order;
     std::vector<size_t> d = dims;
-    if (reverse) std::reverse(d.begin(), d.end());
+    if (order == DimOrder::kReverseDims) std::reverse(d.begin(), d.end());
     g.launch = max_sizes ? limit_dims(d, *max_sizes) : d;
     return g;
 }
 
+namespace {
+// How the launch extents relate to the dims they were made from: untouched, grouped (with the
+// contraction), or split / reshaped (flatten and unflatten).
+enum class DimRelation { kSame, kGrouped, kFlat };
+DimRelation relate(const std::vector<size_t>& d, const std::vector<size_t>& launch, std::vector<std::vector<size_t>>* contraction) {
+    if (launch == d) return DimRelation::kSame;
+    if (launch.size() < d.size() && get_contraction(d, launch, contraction)) return DimRelation::kGrouped;
+    return DimRelation::kFlat;
+}
+}  // namespace
+
 std::vector<size_t> GroupedDims::map(const std::vector<size_t>& raw) const {
     std::vector<size_t> d = original;
-    if (reverse) std::reverse(d.begin(), d.end());
+    if (order == DimOrder::kReverseDims) std::reverse(d.begin(), d.end());
     std::vector<size_t> res;
-    if (launch == d) {
-        res = raw;
-    } else {
-        std::vector<std::vector<size_t>> contraction;
-        if (launch.size() < d.size() && get_contraction(d, launch, &contraction)) {
+    std::vector<std::vector<size_t>> contraction;
+    switch (relate(d, launch, &contraction)) {
+        case DimRelation::kSame: res = raw; break;
+        case DimRelation::kGrouped:
             // grouped: peel the original dims off each fused index, fastest-varying first
             res.assign(d.size(), 0);
             for (size_t gi = 0; gi < contraction.size(); gi++) {
@@ -275,7 +285,8 @@ std::vector<size_t> GroupedDims::map(const std::vector<size_t>& raw) const {
                 }
                 if (!grp.empty()) res[grp.back()] = cur;
             }
-        } else {
+            break;
+        case DimRelation::kFlat: {
             // split or reshaped: flatten the raw indices row-major, unflatten over the original dims
             size_t flat = 0;
             for (size_t i = 0; i < launch.size(); i++) flat = flat * launch[i] + raw[i];
@@ -284,9 +295,45 @@ std::vector<size_t> GroupedDims::map(const std::vector<size_t>& raw) const {
                 res[i] = flat % d[i];
                 flat /= d[i];
             }
+            break;
         }
     }
-    if (reverse) std::reverse(res.begin(), res.end());
+    if (order != DimOrder::kForward) std::reverse(res.begin(), res.end());
+    return res;
+}
+
+std::vector<uint32_t> GroupedDims::map_nodes(KernelBuilder& b, const std::vector<uint32_t>& raw) const {
+    std::vector<size_t> d = original;
+    if (order == DimOrder::kReverseDims) std::reverse(d.begin(), d.end());
+    std::vector<uint32_t> res;
+    std::vector<std::vector<size_t>> contraction;
+    auto c = [](size_t v) { return static_cast<int64_t>(v); };
+    switch (relate(d, launch, &contraction)) {
+        case DimRelation::kSame: res = raw; break;
+        case DimRelation::kGrouped:
+            res.assign(d.size(), 0);
+            for (size_t gi = 0; gi < contraction.size(); gi++) {
+                uint32_t cur = raw[gi];
+                const auto& grp = contraction[gi];
+                for (size_t j = 0; j + 1 < grp.size(); j++) {
+                    res[grp[j]] = d[grp[j]] == 1 ? b.ci(0, b.dtype(cur).scalar) : b.imod(cur, c(d[grp[j]]));
+                    if (d[grp[j]] != 1) cur = b.idiv(cur, c(d[grp[j]]));
+                }
+                if (!grp.empty()) res[grp.back()] = cur;
+            }
+            break;
+        case DimRelation::kFlat: {
+            uint32_t flat = raw[0];
+            for (size_t i = 1; i < launch.size(); i++) flat = b.iadd(b.imul(flat, c(launch[i])), raw[i]);
+            res.assign(d.size(), 0);
+            for (size_t i = d.size(); i-- > 0;) {
+                res[i] = i == 0 ? flat : b.imod(flat, c(d[i]));
+                if (i) flat = b.idiv(flat, c(d[i]));
+            }
+            break;
+        }
+    }
+    if (order != DimOrder::kForward) std::reverse(res.begin(), res.end());
     return res;
 }
 

@@ -72,14 +72,32 @@ bool get_contraction(const std::vector<size_t>& original, const std::vector<size
                      std::vector<std::vector<size_t>>* out);
 // gpudims.rs:331-382,479-505,587-642: the launch extents for `dims` under `max_sizes` and,
 // for a given tuple of raw hardware indices, the index of every original dimension.
+class KernelBuilder;
+// How global dims are turned around (local dims never are):
+//   kReverseDims   - the dims are reversed before limiting and the indices after it, so the
+//                    innermost axis lands on gidx0 whatever regrouping happened.  This is what
+//                    this backend launches and what tinygrad's get_grouped_dims does.
+//   kReverseResult - the reference's literal code (schedule/src/gpudims.rs:331-382): dims are
+//                    limited as given and only the resulting index list is reversed.  Equal to
+//                    kReverseDims when the dims read the same in both directions; otherwise it
+//                    hands dimension i an index whose extent is that of dimension n-1-i.  Offered
+//                    for comparison with the reference, never launched.
+enum class DimOrder { kForward = 0, kReverseDims = 1, kReverseResult = 2 };
 struct GroupedDims {
     std::vector<size_t> original;  // in the caller's order
     std::vector<size_t> launch;    // extents of gidx0.. / lidx0..
-    bool reverse = false;
+    DimOrder order = DimOrder::kForward;
     // raw[i] in [0, launch[i])  ->  index per original dimension
     std::vector<size_t> map(const std::vector<size_t>& raw) const;
+    // The same mapping as nodes of a kernel under construction: raw[i] is the SPECIAL of launch
+    // extent i; the result holds one index node per original dimension (mod / idiv chains where
+    // dims were regrouped, the SPECIALs themselves where they were not).
+    std::vector<uint32_t> map_nodes(KernelBuilder& b, const std::vector<uint32_t>& raw) const;
 };
-GroupedDims get_grouped_dims(const std::vector<size_t>& dims, const std::vector<size_t>* max_sizes, bool reverse);
+GroupedDims get_grouped_dims(const std::vector<size_t>& dims, const std::vector<size_t>* max_sizes, DimOrder order);
+inline GroupedDims get_grouped_dims(const std::vector<size_t>& dims, const std::vector<size_t>* max_sizes, bool reverse) {
+    return get_grouped_dims(dims, max_sizes, reverse ? DimOrder::kReverseDims : DimOrder::kForward);
+}
 
 // ---- small builder for linearized kernels (C++ twin of morok_amd/uop.py)
 class KernelBuilder {

@@ -1590,6 +1590,40 @@ struct Scheduler {
         return computed ? m : nullptr;
     }
 
+    // Workgroup index of a generated kernel.  `gdims` are the kernel's global axes counted in
+    // workgroups, outermost first (the order of the GLOBAL ranges of the reference's kernels).
+    // Their launch extents (gidx0..2) and the index of every axis come from get_grouped_dims
+    // under this device's limits (schedule/src/gpudims.rs:60-196,331-382): the innermost axis
+    // lands on gidx0, axes beyond three or beyond 65535 in y / z are regrouped and recovered
+    // with mod / div.  Returns the row-major flat workgroup index (0 on failure, error set).
+    uint32_t workgroup_index(KernelBuilder& b, Scalar idx_t, const std::vector<int64_t>& gdims) {
+        static const RendererCaps caps = amd_cdna4_caps();
+        std::vector<size_t> d(gdims.begin(), gdims.end());
+        const GroupedDims gd = get_grouped_dims(d, &caps.global_max, DimOrder::kReverseDims);
+        for (size_t i = 0; i < gd.launch.size(); i++)
+            if (i >= caps.global_max.size() || gd.launch[i] > caps.global_max[i]) {
+                fail(kInvalidArgument, "realize: tensor too large for one launch");
+                return 0;
+            }
+        std::vector<uint32_t> raw;
+        for (size_t i = 0; i < gd.launch.size(); i++) {
+            uint32_t sp = b.special("gidx" + std::to_string(i), static_cast<int64_t>(gd.launch[i]));
+            raw.push_back(idx_t != Scalar::Int32 ? b.cast(sp, idx_t) : sp);
+        }
+        const std::vector<uint32_t> ax = gd.map_nodes(b, raw);
+        uint32_t flat = ax[0];
+        for (size_t i = 1; i < ax.size(); i++) flat = b.iadd(b.imul(flat, gdims[i]), ax[i]);
+        return flat;
+    }
+    // Global axes of a kernel over `rows` rows of `per_row` work-items each with `block` work-items
+    // per workgroup: [rows, workgroups per row] when workgroups tile a row exactly, else the flat
+    // workgroup count.
+    static std::vector<int64_t> workgroup_axes(int64_t items, int64_t per_row, int64_t block) {
+        if (per_row > 0 && per_row % block == 0 && items % per_row == 0 && items / per_row > 1)
+            return {items / per_row, per_row / block};
+        return {(items + block - 1) / block};
+    }
+
     int gen_elementwise(TensorNode* n, int64_t max_numel) {
         const int64_t N = n->numel();
         KernelGen g;
@@ -1607,13 +1641,11 @@ struct Scheduler {
                     break;
                 }
         g.width = width;
-        const int64_t items = N / width, block = 256, grid = (items + block - 1) / block;
-        if (grid > 2147483647LL) return fail(kInvalidArgument, "realize: tensor too large for one launch");
-        uint32_t gx = b.special("gidx0", grid), lx = b.special("lidx0", block);
-        if (g.idx_t != Scalar::Int32) {
-            gx = b.cast(gx, g.idx_t);
-            lx = b.cast(lx, g.idx_t);
-        }
+        const int64_t items = N / width, block = 256;
+        uint32_t gx = workgroup_index(b, g.idx_t, workgroup_axes(items, n->shape.empty() ? 0 : n->shape.back() / width, block));
+        if (!gx) return last_status();
+        uint32_t lx = b.special("lidx0", block);
+        if (g.idx_t != Scalar::Int32) lx = b.cast(lx, g.idx_t);
         uint32_t item = b.iadd(b.imul(gx, block), lx);
         b.if_(b.binary(BinaryOp::Lt, item, g.ci(items)));
         auto emit_group = [&](const Coords& coords, uint32_t base) {
@@ -1726,12 +1758,11 @@ struct Scheduler {
         };
         if (!wave) {
             // one work-item per output element, the reduced axes as nested sequential loops
-            const int64_t block = 64, grid = (Nout + block - 1) / block;
-            uint32_t gx = b.special("gidx0", grid), lx = b.special("lidx0", block);
-            if (g.idx_t != Scalar::Int32) {
-                gx = b.cast(gx, g.idx_t);
-                lx = b.cast(lx, g.idx_t);
-            }
+            const int64_t block = 64;
+            uint32_t gx = workgroup_index(b, g.idx_t, workgroup_axes(Nout, n->shape.empty() ? 0 : n->shape.back(), block));
+            if (!gx) return last_status();
+            uint32_t lx = b.special("lidx0", block);
+            if (g.idx_t != Scalar::Int32) lx = b.cast(lx, g.idx_t);
             uint32_t o = b.iadd(b.imul(gx, block), lx);
             uint32_t gate = b.binary(BinaryOp::Lt, o, g.ci(Nout));
             uint32_t oc = b.where(gate, o, g.ci(Nout - 1));  // clamp: masked lanes recompute the last element
@@ -1758,11 +1789,11 @@ struct Scheduler {
         // results are combined with the wave64 cross-lane reduction (the GROUP_REDUCE idea of
         // schedule/src/optimizer/heuristics.rs:370-392 without the LDS round trip)
         const int64_t W = Nout * P;  // wave-sized outputs of this kernel
-        const int64_t per_block = 4, grid = (W + per_block - 1) / per_block;
-        if (grid > 2147483647LL) return fail(kInvalidArgument, "realize: reduction too large for one launch");
-        uint32_t gx = b.special("gidx0", grid), lane = b.special("lidx0", 64), ly = b.special("lidx1", per_block);
+        const int64_t per_block = 4;
+        uint32_t gx = workgroup_index(b, g.idx_t, workgroup_axes(W, 0, per_block));
+        if (!gx) return last_status();
+        uint32_t lane = b.special("lidx0", 64), ly = b.special("lidx1", per_block);
         if (g.idx_t != Scalar::Int32) {
-            gx = b.cast(gx, g.idx_t);
             lane = b.cast(lane, g.idx_t);
             ly = b.cast(ly, g.idx_t);
         }
@@ -1799,8 +1830,10 @@ struct Scheduler {
         KernelBuilder& b2 = g2.b;
         uint32_t po2 = b2.param(0, n->dtype, Nout);
         uint32_t pin = g2.buffer_param(partial, Scalar::Float32, Nout * P);
-        const int64_t block2 = 64, grid2 = (Nout + block2 - 1) / block2;
-        uint32_t o2 = b2.iadd(b2.imul(b2.special("gidx0", grid2), block2), b2.special("lidx0", block2));
+        const int64_t block2 = 64;
+        uint32_t gx2 = workgroup_index(b2, Scalar::Int32, workgroup_axes(Nout, 0, block2));
+        if (!gx2) return last_status();
+        uint32_t o2 = b2.iadd(b2.imul(gx2, block2), b2.special("lidx0", block2));
         uint32_t gate2 = b2.binary(BinaryOp::Lt, o2, b2.ci(Nout));
         uint32_t oc2 = b2.where(gate2, o2, b2.ci(Nout - 1));
         uint32_t r2 = b2.range(P, 0, AxisType::Reduce);

@@ -342,6 +342,27 @@ def test_tensor_kernel_cache_and_realize_idempotent(T, shim):
     assert a.shape == (1000,) and c.shape == (1001,)
 
 
+def test_tensor_launch_dims_come_from_grouped_dims(T, shim):
+    """Generated kernels take their grid from get_grouped_dims under the device limits
+    (schedule/src/gpudims.rs:331-382, global_max [2147483647, 65535, 65535]): rows x workgroups-per-row
+    as (x = innermost, y = rows) while rows fit y, regrouped into x beyond that."""
+    T.set_fusion(False)
+    zeros(T, (300, 1024)).try_add(1.0).realize()          # 256 work-items tile a row of 1024 / 4 exactly
+    assert hostshim_lib.last_dims(shim) == ((1, 300, 1), (256, 1, 1))
+    zeros(T, (300, 4096)).try_add(1.0).realize()
+    assert hostshim_lib.last_dims(shim) == ((4, 300, 1), (256, 1, 1))
+    zeros(T, (70000, 1024)).try_add(1.0).realize()        # 70000 rows exceed 65535 in y: grouped into x
+    assert hostshim_lib.last_dims(shim) == ((70000, 1, 1), (256, 1, 1))
+    src = T.last_kernel_sources()[0]
+    assert "blockIdx.y" not in src
+    zeros(T, (70000, 2048)).try_add(1.0).realize()
+    assert hostshim_lib.last_dims(shim) == ((140000, 1, 1), (256, 1, 1))
+    zeros(T, (2, 3, 5, 1024)).try_add(1.0).realize()      # leading axes count as rows
+    assert hostshim_lib.last_dims(shim) == ((1, 30, 1), (256, 1, 1))
+    zeros(T, (300, 1000)).try_add(1.0).realize()          # rows the workgroups do not tile: flat
+    assert hostshim_lib.last_dims(shim) == ((293, 1, 1), (256, 1, 1))
+
+
 def test_tensor_launch_dims(T, shim):
     T.set_fusion(False)
     zeros(T, (1001,)).try_add(1.0).realize()

@@ -193,3 +193,47 @@ def test_wmma_matmul_lds_kernel_refuses_bad_choices(opts):
 
     with pytest.raises(morok_amd.MorokHipError):
         sched.build_wmma_matmul_lds_opts(1, 256, 128, 64, U.BF16, opts)
+
+
+def test_global_index_order_modes_and_where_they_differ():
+    """reverse=1 (dims reversed before limiting, indices after: what generated kernels launch) against
+    reverse=2 (the literal code of schedule/src/gpudims.rs:331-382: only the index list is reversed).
+    The two agree exactly on dims lists that read the same in both directions; on every other list
+    mode 2 hands dimension i an index running over the extent of dimension n-1-i, so it is not an
+    in-range bijection there."""
+    GLOBAL_MAX = [2147483647, 65535, 65535]
+    cases = [[7], [4, 4], [3, 5, 3], [3, 5], [2, 3, 4], [5, 1], [6, 6, 2], [2, 9, 9, 2], [2, 3, 3, 4], [70000, 4],
+             [4, 70000], [70000, 70000], [3, 70000, 3]]
+    for dims in cases:
+        l1, _ = sched.grouped_dims(dims, GLOBAL_MAX, 1)
+        l2, _ = sched.grouped_dims(dims, GLOBAL_MAX, 2)
+        symmetric = dims == dims[::-1]
+        total = 1
+        for d in dims:
+            total *= d
+        if total > 5000:  # compare on a sample of hardware index tuples
+            raws = [[min(r, l - 1) for l in l1] for r in (0, 1, 2, 69999)]
+        else:
+            raws = [list(r) for r in itertools.product(*[range(l) for l in l1])]
+        if symmetric:
+            assert l1 == l2, dims
+            for raw in raws:
+                assert sched.grouped_dims(dims, GLOBAL_MAX, 1, raw)[1] == sched.grouped_dims(dims, GLOBAL_MAX, 2, raw)[1]
+        else:
+            # mode 1 stays in range for every tuple; mode 2 leaves it for some tuple
+            out_of_range = False
+            for raw in itertools.product(*[range(min(l, 6)) for l in l2]):
+                _, idx = sched.grouped_dims(dims, GLOBAL_MAX, 2, list(raw))
+                out_of_range = out_of_range or any(i >= d for i, d in zip(idx, dims))
+            for raw in raws:
+                _, idx = sched.grouped_dims(dims, GLOBAL_MAX, 1, raw)
+                assert all(0 <= i < d for i, d in zip(idx, dims)), (dims, raw, idx)
+            assert out_of_range or l1 != l2, dims
+    # the innermost axis is gidx0 in mode 1 whatever regrouping happened
+    assert sched.grouped_dims([3, 5], GLOBAL_MAX, 1)[0] == [5, 3]
+    assert sched.grouped_dims([3, 5], GLOBAL_MAX, 2)[0] == [3, 5]
+    assert sched.grouped_dims([70000, 4], GLOBAL_MAX, 1)[0] == [280000]          # y would exceed 65535: grouped
+    assert sched.grouped_dims([70000, 4], GLOBAL_MAX, 1, [9])[1] == [2, 1]        # 9 = 2 * 4 + 1
+    assert sched.grouped_dims([2, 3, 70000, 8], GLOBAL_MAX, 1)[0] == [560000, 3, 2]
+    with pytest.raises(Exception):
+        sched.grouped_dims([3, 5], GLOBAL_MAX, 3)

@@ -1074,3 +1074,22 @@ def test_prepared_plan_reuploads_host_data_on_every_execute(T):
     c = T.Tensor.from_slice(a, uop.BF16).to("HIP:0").matmul(T.Tensor.from_slice(b, uop.BF16).to("HIP:0"))
     direct = T.Tensor.from_numpy(a, uop.BF16).matmul(T.Tensor.from_numpy(b, uop.BF16)).to_numpy()
     assert np.array_equal(c.to_numpy(), direct) and c.kernels()[-1].startswith("gemm_bf16")
+
+
+# ---------------------------------------------------------------- launch dims from get_grouped_dims
+@pytest.mark.parametrize("shape", [(300, 1024), (70000, 1024), (66000, 2, 512), (2, 3, 5, 1024), (70001, 256)])
+def test_regrouped_launch_dims_index_exactly(T, shape):
+    """Grids come from get_grouped_dims (gidx0 = innermost axis, rows on y until they exceed 65535,
+    then regrouped into x and recovered with mod / div): index work is bit-exact, so an integer
+    kernel whose value encodes its own position must match numpy for every element."""
+    n = int(np.prod(shape))
+    x = (np.arange(n, dtype=np.int64) * 2654435761 % 2147483647).astype(np.int32).reshape(shape)
+    t = T.Tensor.from_numpy(x)
+    got = t.binary("xor", T.Tensor.from_numpy(np.full(shape[-1], 0x5A5A5A5A, np.int32))).binary("add", t).to_numpy()
+    want = (x ^ np.int32(0x5A5A5A5A)) + x
+    assert np.array_equal(got, want)
+    # and through a transposed read (the index of every axis matters, not only the flat one)
+    if len(shape) == 2 and shape[0] >= 66000:
+        small = x[:, :8].copy()
+        tt = T.Tensor.from_numpy(np.ascontiguousarray(small.T)).try_transpose(0, 1).try_add(T.Tensor.from_numpy(small))
+        assert np.array_equal(tt.to_numpy(), small + small)
