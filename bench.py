@@ -413,6 +413,45 @@ def bench_mfma_ceiling(m, dev, steps, warmup, cpu):
                          "kernel": "mfma_ceiling_kernel", "algorithmic_flops_per_launch": 2.0 * 4096 ** 3}}
 
 
+def bench_group_reduce(m, dev, steps, warmup, cpu):
+    """Row sums of f32 [8, 2^24] through the lazy tensor API: few outputs, long rows, i.e. the GROUP
+    reduction (waves of a workgroup share an output through local memory) plus a small second
+    kernel that folds the per-workgroup partials.  HBM-bound: 512 MiB read per step."""
+    from morok_amd import ops, tensor, uop
+
+    rows, cols = 8, 1 << 24
+    n = rows * cols
+    bx = dev.buffer(n * 4).ensure_allocated()
+    ops.fill_normal(bx, n, seed=6, tensor_id=0)
+    tensor.set_fusion(False)
+    try:
+        t = tensor.Tensor.from_buffer(bx, (rows, cols), uop.F32).sum(1)
+        plan = t.prepare()
+    finally:
+        tensor.set_fusion(True)
+    names = [plan.kernel_name(i) for i in range(plan.kernel_count)]
+    ms, stats = _launch_stats(m, plan.execute, steps, warmup)
+    algo_bytes = n * 4 + rows * 4
+    gbs = algo_bytes / (ms * 1e-3) / 1e9
+    rec = {"metric": "grouped reduce HBM GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "f32", **stats,
+           "config": {"workload": "row sums of f32 [8 x 2^24] via the lazy tensor API (generated GROUP reduce + fold)"},
+           "kernels": names,
+           "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS,
+                        "traffic": None, "traffic_source": "profiles/group_reduce_sum_8x16777216_f32.txt", "kernel": names[0],
+                        "algorithmic_bytes_per_launch": algo_bytes}}
+    if cpu:
+        import numpy as np
+
+        x = bx.copyout(np.float32, (rows, cols))
+        sec = _cpu_time(lambda: x.sum(axis=1, dtype=np.float32))
+        ref = x.astype(np.float64).sum(1)
+        rec["max_rel_err_vs_float64"] = float(np.max(np.abs(t.to_numpy() - ref) / np.abs(x.astype(np.float64)).sum(1)))
+        rec["cpu_baseline"] = {"value": algo_bytes / sec / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+                               "sample": "the whole [8 x 2^24] matrix, sequential f32 row sums (numpy, one thread), min of 3 "
+                                         "after 1 warm-up"}
+    return rec
+
+
 def bench_copy(m, dev, steps, warmup, cpu):
     """Calibration only: 256 MiB streaming copy kernel (known traffic 2 x 256 MiB per launch)."""
     from morok_amd import ops
@@ -431,7 +470,8 @@ def bench_copy(m, dev, steps, warmup, cpu):
 
 
 WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "decoder": bench_decoder,
-             "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling}
+             "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling,
+             "group_reduce": bench_group_reduce}
 PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc"]
 
 

@@ -1745,6 +1745,31 @@ struct Scheduler {
                     break;
                 }
         }
+        // GROUP through local memory (GROUPTOP, schedule/src/optimizer/heuristics.rs:370-392: kernels
+        // with at most 2048 outputs let several work-items share an output).  Here the sharing unit
+        // is the wavefront: G waves of one workgroup fold interleaved 64-element blocks of the same
+        // output (or of the same segment of it), leave their partial in local memory and, behind a
+        // barrier, the first folds the G partials in order.  A split reduction keeps its number of
+        // waves and folds G times fewer partials in the second kernel; an unsplit one with few
+        // outputs gets up to 16 times the waves without a second launch.
+        int64_t G = 1;
+        const char* no_group = std::getenv("MOROK_NO_GROUP_REDUCE");  // measurement switch: every wave on its own
+        const bool grouping = wave && Nout <= 2048 && !(no_group && no_group[0] && no_group[0] != '0');
+        if (grouping && R >= 32768) {
+            // waves per output: each folds at least 4096 inputs, about 4096 waves over the whole chip;
+            // up to 16 of them form a workgroup, the rest are segments for the second kernel
+            int64_t wpo = 1;
+            while (wpo * 2 <= R / 4096 && wpo * 2 * Nout <= 4096) wpo *= 2;
+            G = wpo < 16 ? wpo : 16;
+            P = wpo / G;
+            if (P > 256) P = 256;
+        } else if (grouping) {  // more waves per output while each keeps at least 512 inputs
+            for (int64_t c = 16; c > 1; c /= 2)
+                if (R / c >= 512 && Nout * c <= 2048) {
+                    G = c;
+                    break;
+                }
+        }
         const int64_t chunk = (R + P - 1) / P;
         std::shared_ptr<Buffer> partial;
         if (P > 1) {
@@ -1788,26 +1813,29 @@ struct Scheduler {
         // one wavefront per output element: lanes stride the flattened reduce space, partial
         // results are combined with the wave64 cross-lane reduction (the GROUP_REDUCE idea of
         // schedule/src/optimizer/heuristics.rs:370-392 without the LDS round trip)
-        const int64_t W = Nout * P;  // wave-sized outputs of this kernel
-        const int64_t per_block = 4;
+        const int64_t W = Nout * P;  // wave-sized (G == 1) or workgroup-sized outputs of this kernel
+        const int64_t per_block = G > 1 ? 1 : 4;
         uint32_t gx = workgroup_index(b, g.idx_t, workgroup_axes(W, 0, per_block));
         if (!gx) return last_status();
-        uint32_t lane = b.special("lidx0", 64), ly = b.special("lidx1", per_block);
+        uint32_t lane = b.special("lidx0", 64), ly = b.special("lidx1", G > 1 ? G : per_block);
         if (g.idx_t != Scalar::Int32) {
             lane = b.cast(lane, g.idx_t);
             ly = b.cast(ly, g.idx_t);
         }
-        uint32_t w = b.iadd(b.imul(gx, per_block), ly);
+        // G == 1: wave ly of the workgroup owns output w; G > 1: the whole workgroup owns w = gx
+        uint32_t w = G > 1 ? gx : b.iadd(b.imul(gx, per_block), ly);
         uint32_t wgate = b.binary(BinaryOp::Lt, w, g.ci(W));
-        uint32_t wc = b.where(wgate, w, g.ci(W - 1));
+        uint32_t wc = G > 1 ? w : b.where(wgate, w, g.ci(W - 1));
         uint32_t oc = P > 1 ? b.idiv(wc, P) : wc;
         uint32_t seg0 = P > 1 ? b.imul(b.imod(wc, P), chunk) : g.ci(0);  // first reduce index of the segment
         Coords coords = plain(unflatten(g, oc, n->shape));
-        const int64_t steps = (chunk + 63) / 64;
+        const int64_t steps = (chunk + 64 * G - 1) / (64 * G);
         uint32_t rg = b.add(Op::Range, KernelBuilder::scalar(g.idx_t), {g.ci(steps)}, 0, 0, static_cast<uint16_t>(AxisType::Reduce));
-        uint32_t in_seg = b.iadd(b.imul(rg, 64), lane);
+        // block rg * G + ly of the segment: the G waves read neighbouring 256-byte blocks
+        uint32_t blk = G > 1 ? b.iadd(b.imul(rg, G), ly) : rg;
+        uint32_t in_seg = b.iadd(b.imul(blk, 64), lane);
         uint32_t f = b.iadd(seg0, in_seg);
-        const bool exact = chunk % 64 == 0 && chunk * P == R;
+        const bool exact = chunk % (64 * G) == 0 && chunk * P == R;
         uint32_t fgate = b.binary(BinaryOp::And, b.binary(BinaryOp::Lt, in_seg, g.ci(chunk)), b.binary(BinaryOp::Lt, f, g.ci(R)));
         uint32_t fc = exact ? f : b.where(fgate, f, g.ci(R - 1));
         std::vector<uint32_t> rc = unflatten(g, fc, rdims);
@@ -1818,13 +1846,30 @@ struct Scheduler {
         b.end({rg});
         uint32_t total = b.wave_reduce(op, red);
         uint32_t first = b.binary(BinaryOp::Eq, lane, g.ci(0));
-        b.if_(b.binary(BinaryOp::And, first, wgate));
-        uint32_t res = total;
-        if (P == 1 && b.dtype(res).scalar != n->dtype) res = b.cast(res, n->dtype);
-        b.store(b.index(po, w), res);
-        b.endif();
-        if (P == 1) return finish_kernel(g, n, out, "r_" + std::to_string(Nout) + "_g" + std::to_string(R));
-        MRK_TRY(queue_kernel(g, partial, "r_" + std::to_string(Nout) + "x" + std::to_string(P) + "_g" + std::to_string(chunk)));
+        if (G > 1) {
+            uint32_t lds = b.define_local(0, ct, G);
+            b.if_(first);
+            b.store(b.index(lds, ly), total);
+            b.endif();
+            b.barrier();
+            b.if_(b.binary(BinaryOp::And, first, b.binary(BinaryOp::Eq, ly, g.ci(0))));
+            uint32_t r2 = b.add(Op::Range, KernelBuilder::scalar(g.idx_t), {g.ci(G)}, 1, 0, static_cast<uint16_t>(AxisType::Reduce));
+            uint32_t folded = b.reduce(op, b.load(b.index(lds, r2)), {r2});
+            b.end({r2});
+            uint32_t res = folded;
+            if (P == 1 && b.dtype(res).scalar != n->dtype) res = b.cast(res, n->dtype);
+            b.store(b.index(po, w), res);
+            b.endif();
+        } else {
+            b.if_(b.binary(BinaryOp::And, first, wgate));
+            uint32_t res = total;
+            if (P == 1 && b.dtype(res).scalar != n->dtype) res = b.cast(res, n->dtype);
+            b.store(b.index(po, w), res);
+            b.endif();
+        }
+        const std::string grp = G > 1 ? "_l" + std::to_string(G) : "";  // waves sharing an output through local memory
+        if (P == 1) return finish_kernel(g, n, out, "r_" + std::to_string(Nout) + "_g" + std::to_string(R) + grp);
+        MRK_TRY(queue_kernel(g, partial, "r_" + std::to_string(Nout) + "x" + std::to_string(P) + "_g" + std::to_string(chunk) + grp));
         // second stage: one work-item per output folds its P partials
         KernelGen g2;
         KernelBuilder& b2 = g2.b;

@@ -369,8 +369,10 @@ def test_tensor_launch_dims(T, shim):
     assert hostshim_lib.last_dims(shim) == ((4, 1, 1), (256, 1, 1))
     zeros(T, (8, 1000)).try_add(1.0).realize()      # innermost axis % 4 == 0: four outputs per work-item
     assert hostshim_lib.last_dims(shim) == ((8, 1, 1), (256, 1, 1))
-    zeros(T, (10, 4096)).sum(1).realize()           # one wavefront per output, four per workgroup
-    assert hostshim_lib.last_dims(shim) == ((3, 1, 1), (64, 4, 1))
+    zeros(T, (10, 4096)).sum(1).realize()           # few outputs: eight wavefronts share each through local memory
+    assert hostshim_lib.last_dims(shim) == ((10, 1, 1), (64, 8, 1))
+    zeros(T, (5000, 4096)).sum(1).realize()         # many outputs: one wavefront per output, four per workgroup
+    assert hostshim_lib.last_dims(shim) == ((1250, 1, 1), (64, 4, 1))
     zeros(T, (100, 16)).sum(1).realize()            # short rows: one work-item per output
     assert hostshim_lib.last_dims(shim) == ((2, 1, 1), (64, 1, 1))
 
@@ -740,11 +742,42 @@ def test_large_reductions_are_split_in_two_stages(T, shim):
     """split_reduceop (schedule/src/rangeify/kernel.rs:44-61): >= 32768 inputs per output."""
     T.set_fusion(False)
     t = zeros(T, (1 << 20,)).sum(0).realize()
-    assert len(t.kernels()) == 2 and t.kernels()[0].startswith("r_1x256_g")
-    t = zeros(T, (4, 70000)).max(1).realize()
+    # 256 waves as 16 workgroups of 16: the waves of a workgroup meet in local memory, 16 partials are left
+    assert t.kernels() == ["r_1x16_g65536_l16", "r_1_16"]
+    assert hostshim_lib.last_dims(shim) == ((1, 1, 1), (64, 1, 1))
+    t = zeros(T, (4, 70000)).max(1).realize()        # few outputs: 16 waves share each, no second kernel
+    assert t.kernels() == ["r_4_g70000_l16"]
+    t = zeros(T, (4096, 70000)).max(1).realize()     # many outputs: split as before
     assert len(t.kernels()) == 2
     t = zeros(T, (64, 4096)).sum(1).realize()        # below the threshold: one kernel
     assert len(t.kernels()) == 1
+
+
+def test_grouped_reduce_through_local_memory(T, shim, monkeypatch):
+    """GROUP / GROUPTOP (schedule/src/optimizer/heuristics.rs:370-392): kernels with at most 2048
+    outputs let the waves of a workgroup share an output through local memory and a barrier."""
+    T.set_fusion(False)
+    t = zeros(T, (64, 8192)).sum(1).realize()
+    assert t.kernels() == ["r_64_g8192_l16"]         # 16 waves per output, one launch
+    assert hostshim_lib.last_dims(shim) == ((64, 1, 1), (64, 16, 1))
+    src = T.last_kernel_sources()[0]
+    assert "__shared__ float local0[16]" in src and "__syncthreads()" in src
+    t = zeros(T, (512, 2048)).max(1).realize()       # more outputs: fewer waves each
+    assert t.kernels() == ["r_512_g2048_l4"]
+    t = zeros(T, (2048, 1024)).max(1).realize()      # enough outputs to fill the chip by themselves
+    assert t.kernels() == ["r_2048_g1024"]
+    t = zeros(T, (4096, 4096)).sum(1).realize()      # many outputs: one wave per output as before
+    assert t.kernels() == ["r_4096_g4096"]
+    t = zeros(T, (8, 300)).sum(1).realize()          # short rows: nothing to share
+    assert t.kernels() == ["r_8_g300"]
+    t = zeros(T, (8, 1 << 20)).sum(1).realize()      # split: the first stage leaves 16 partials per output
+    assert t.kernels() == ["r_8x16_g65536_l16", "r_8_16"]
+    t = zeros(T, (256, 65536)).sum(1).realize()      # 16 waves per output already cover the chip: one launch
+    assert t.kernels() == ["r_256_g65536_l16"]
+    monkeypatch.setenv("MOROK_NO_GROUP_REDUCE", "1")
+    morok_amd.kernel_cache_clear()
+    t = zeros(T, (64, 8192)).sum(1).realize()
+    assert t.kernels() == ["r_64_g8192"]
 
 
 def test_null_arguments_are_errors_not_crashes(T, dev, shim):

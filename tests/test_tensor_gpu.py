@@ -1093,3 +1093,29 @@ def test_regrouped_launch_dims_index_exactly(T, shape):
         small = x[:, :8].copy()
         tt = T.Tensor.from_numpy(np.ascontiguousarray(small.T)).try_transpose(0, 1).try_add(T.Tensor.from_numpy(small))
         assert np.array_equal(tt.to_numpy(), small + small)
+
+
+# ---------------------------------------------------------------- GROUP reduce through local memory
+@pytest.mark.parametrize("shape,axis", [((64, 8192), 1), ((2048, 1024), 1), ((8, 1 << 20), 1), ((3, 5, 4100), 2),
+                                        ((1 << 21,), 0), ((17, 9000), 1), ((4, 70001), 1)])
+@pytest.mark.parametrize("op", ["sum", "max"])
+def test_grouped_reductions_match_float64(T, fusion, oracle, shape, axis, op):
+    """Reductions with few outputs share each output between the waves of a workgroup (local memory
+    + barrier), split or unsplit: <= 1e-4 relative against float64 for sums (north-star tolerance for
+    f32 reductions), exact for maxima; ragged extents exercise the masked tail blocks."""
+    from morok_amd import synth
+
+    x = synth.normal(shape, 31, len(shape), sigma=1.0) + np.float32(0.25)
+    t = T.Tensor.from_numpy(x)
+    got = (t.sum(axis) if op == "sum" else t.max(axis)).to_numpy()
+    if op == "sum":
+        ref = x.astype(np.float64).sum(axis)
+        scale = np.abs(x.astype(np.float64)).sum(axis)   # condition of the sum: |error| <= 1e-4 * sum |x|
+        assert np.all(np.abs(got - ref) <= 1e-4 * np.maximum(np.abs(ref), 1e-3 * scale))
+    else:
+        assert np.array_equal(got, x.max(axis))
+    if len(shape) == 2 and op == "sum" and shape[1] <= 8192:
+        # the oracle's softmax holds the same row sums: sum(exp(x - max)) is its normaliser
+        p = oracle.softmax_f32(x)
+        e = np.exp(x - x.max(1, keepdims=True))
+        np.testing.assert_allclose((T.Tensor.from_numpy(e).sum(1).to_numpy())[:, None] * p, e, rtol=2e-5, atol=1e-9)
