@@ -198,6 +198,7 @@ void mrk_hip_program_destroy(mrk_program* p);
  *                     params = {M, N, K, batch, workspace bytes}    buffers = {c, a, b, workspace}
  *                     (split-K for shapes with few output tiles; size from mrk_hip_gemm_bf16_workspace_bytes)
  *   "gemm_bf16_residual"  params = {M, N, K} or {M, N, K, batch}  buffers = {c, a, b, r}   (c = a b + r)
+ *   "gemm_bf16_swiglu"    params = {M, F, K}                      buffers = {c, a, w}      (w = gate | up, [K, 2F])
  *   "flash_fwd_bf16"  params = {B*H, Sq, Sk, D, causal, f32 bits of scale}   buffers = {o, q, k, v}
  *   "flash_fwd_bf16_strided"  params = {B, H, Sq, Sk, D, causal, f32 bits of scale, element offsets
  *                     of q k v o into their buffers (4), (batch, head, row) element strides of
@@ -447,6 +448,16 @@ size_t mrk_hip_gemm_bf16_noalloc_capacity(void);
  * multiple of 8, K = 0, or so few output tiles that split-K is used). */
 int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, const void* r, void* c, int64_t m, int64_t n,
                                int64_t k);
+
+/* Gated-MLP pair of products: c[M, F] = bf16(silu(float(bf16(a wg))) * float(bf16(a wu))) with
+ * w = [wg | wu] stored side by side as one row-major [K, 2F] matrix: what
+ * (x.matmul(w)[:, :F]).silu() * x.matmul(w)[:, F:] computes (Tensor::matmul, tensor/src/matmul.rs:82-110;
+ * Tensor::silu / swish, tensor/src/activation.rs:309-318; the products rounded to bf16 first, then
+ * x * sigmoid(x) * y in f32 and one rounding), with the gate applied in the product kernel's
+ * epilogue so that the [M, 2F] product is never written.  F and K multiples of 8, K > 0;
+ * INVALID_ARGUMENT otherwise.  Builtin Program kind "gemm_bf16_swiglu", params {M, F, K},
+ * buffers {c, a, w}. */
+int mrk_hip_gemm_bf16_swiglu(int device_id, const void* a, const void* w, void* c, int64_t m, int64_t f, int64_t k);
 
 /* Scaled dot-product attention forward in one kernel (online softmax, f32 scores and
  * statistics, P rounded to bf16 before the second product, bf16 output):

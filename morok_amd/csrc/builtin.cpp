@@ -145,6 +145,17 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
+    if (k == "gemm_bf16_swiglu") {  // {M, F, K}; buffers {c [M, F], a [M, K], w [K, 2F] = gate | up}
+        MRK_TRY(need(3));
+        if (!gemm_bf16_swiglu_supported(p[0], p[1], p[2]))
+            return fail(kInvalidArgument, "gemm_bf16_swiglu: shape not covered (M, F, K > 0; F and K multiples of 8)");
+        std::string name = "gemm_bf16_swiglu_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+        out->reset(new BuiltinProgram(device_id, stream, name, 3, p,
+                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16_swiglu(s, b[1], b[2], b[0], q[0], q[1], q[2]);
+                                      }));
+        return kOk;
+    }
     if (k == "flash_fwd_bf16") {
         MRK_TRY(need(6));
         if (p[0] < 0 || p[1] < 0 || p[2] <= 0 || p[3] != 128)

@@ -874,6 +874,21 @@ int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int6
     return mrk_hip_gemm_bf16_variant(device_id, a, b, c, m, n, k, 0);
 }
 
+int mrk_hip_gemm_bf16_swiglu(int device_id, const void* a, const void* w, void* c, int64_t m, int64_t f, int64_t k) {
+    if (m < 0 || f < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_swiglu: negative shape");
+    if (m == 0 || f == 0) return kOk;
+    MRK_NONNULL(a);
+    MRK_NONNULL(w);
+    MRK_NONNULL(c);
+    if (!gemm_bf16_swiglu_supported(m, f, k))
+        return fail(kInvalidArgument, "gemm_bf16_swiglu: shape not covered by the gated epilogue (F and K multiples of 8, K > 0); run "
+                                      "mrk_hip_gemm_bf16 on the [K, 2F] matrix and apply the gate separately");
+    std::shared_ptr<Device> dv;
+    MRK_TRY(get_device(device_id, &dv));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_gemm_bf16_swiglu(dv->allocator->stream(), a, w, c, m, f, k), "gemm_bf16_swiglu launch");
+    return kOk;
+}
 size_t mrk_hip_gemm_bf16_noalloc_capacity(void) { return gemm_bf16_static_workspace_capacity(); }
 int mrk_hip_gemm_bf16_noalloc(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k) {
     if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_noalloc: negative shape");

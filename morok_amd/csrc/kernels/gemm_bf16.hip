@@ -99,7 +99,14 @@ __device__ __attribute__((aligned(16))) const unsigned g_zero16[4] = {0u, 0u, 0u
 // kResidual: the epilogue adds a bf16 matrix R of C's shape to the rounded product,
 // C = bf16(float(bf16(A B)) + float(R)): the bits of the product kernel followed by an
 // elementwise add, without writing and re-reading the product.
-template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false>
+//
+// kSwiGLU (256-row tile only): B is [K, 2F] holding a gate matrix in its columns [0, F) and an up
+// matrix in [F, 2F) (N = 2F is B's row pitch); the workgroup's 256 tile columns are 128 gate
+// columns followed by the 128 up columns at the same offset, and the epilogue writes
+// C[M, F] = bf16(silu(float(bf16(A gate))) * float(bf16(A up))): the two products rounded to bf16
+// as separate kernels would leave them, then x * sigmoid(x) * y in f32 with one rounding, without
+// the 2F-wide product ever reaching memory.
+template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false, bool kSwiGLU = false>
 __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
                                                float* __restrict__ W = nullptr, int kt_per_split = 0,
@@ -124,7 +131,8 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     if (kResidual) R += (size_t)blockIdx.y * M * N;
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
-    const size_t m0 = (size_t)tile_m * kTM, n0 = (size_t)tile_n * kBN;
+    static_assert(!kSwiGLU || (kJ == 4 && !kSplitK && !kResidual), "the gated epilogue exists for the 256-row tile only");
+    const size_t m0 = (size_t)tile_m * kTM, n0 = (size_t)tile_n * (kSwiGLU ? kBN / 2 : kBN);
     char* sA0 = smem;                 // two A stages
     char* sB0 = smem + 2 * kAStageT;  // three B stages
 
@@ -153,7 +161,14 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
 #pragma unroll
     for (int par = 0; par < 2; par++) {
         size_t col = n0 + ((((b_g ^ (par * 2 + b_r)) << 1) | b_h) << 3);
-        col = col + 8 <= (size_t)N ? col : (size_t)N - 8;
+        if (kSwiGLU) {
+            // tile columns 0..127 come from the gate half of B, 128..255 from the up half
+            const size_t F = (size_t)N / 2, lc = col - n0, half = lc >> 7;
+            col = n0 + (lc & 127);
+            col = (col + 8 <= F ? col : F - 8) + half * F;
+        } else {
+            col = col + 8 <= (size_t)N ? col : (size_t)N - 8;
+        }
         b_voff[par] = (unsigned)(((size_t)(wave * 16 + b_r) * N + (col - n0)) * 2);
     }
     const int KT_all = (K + kBK - 1) / kBK;
@@ -367,6 +382,30 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
             }
     if constexpr (kResidual) fetch_residual(kFirstBatch, kIts);
     __syncthreads();
+    if constexpr (kSwiGLU) {
+        // waves (wm, 0) and (wm, 1) staged the gate and the up block of the same 128 rows x 128
+        // columns; each of the two now combines 64 of those rows: 16 chunks of 8 columns per row
+        const size_t F = (size_t)N / 2;
+        const char* sG = smem + (wm * 2 + 0) * kCWaveT;
+        const char* sU = smem + (wm * 2 + 1) * kCWaveT;
+#pragma unroll 4
+        for (int it = 0; it < 16; it++) {
+            const int r = wn * 64 + it * 4 + (lane >> 4);
+            const int ch = lane & 15;
+            const f32x8 gf = __builtin_convertvector(__builtin_bit_cast(bf16x8, *LDS_PTR(u32x4, sG + r * kCPitchT + ch * 16)), f32x8);
+            const f32x8 uf = __builtin_convertvector(__builtin_bit_cast(bf16x8, *LDS_PTR(u32x4, sU + r * kCPitchT + ch * 16)), f32x8);
+            f32x8 y;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                // x * sigmoid(x) * y with sigmoid(x) = 1 / (1 + exp2(x * (-1 / ln 2)))
+                const float sg = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(gf[e] * -1.4426950408889634f));
+                y[e] = gf[e] * sg * uf[e];
+            }
+            const u32x4 v = __builtin_bit_cast(u32x4, __builtin_convertvector(y, bf16x8));
+            if (row0 + r < (size_t)M && n0 + ch * 8 + 8 <= F) *reinterpret_cast<u32x4*>(C + (row0 + r) * F + n0 + ch * 8) = v;
+        }
+        return;
+    }
     __bf16* Cg = C + row0 * N + col0;
     if constexpr (kResidual) {
 #pragma unroll
@@ -410,6 +449,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256_residual_ragged_k(const
                                                                            const __bf16* __restrict__ R, __bf16* __restrict__ C,
                                                                            int M, int N, int K, int tiles_m, int tiles_n) {
     gemm_tile_body<true, 4, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile256_swiglu(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                                __bf16* __restrict__ C, int M, int N2, int K, int tiles_m,
+                                                                int tiles_n) {
+    gemm_tile_body<false, 4, false, false, true>(A, B, C, M, N2, K, tiles_m, tiles_n);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile256_swiglu_ragged_k(const __bf16* __restrict__ A,
+                                                                         const __bf16* __restrict__ B, __bf16* __restrict__ C,
+                                                                         int M, int N2, int K, int tiles_m, int tiles_n) {
+    gemm_tile_body<true, 4, false, false, true>(A, B, C, M, N2, K, tiles_m, tiles_n);
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile128_residual(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                                   const __bf16* __restrict__ R, __bf16* __restrict__ C, int M,
@@ -594,6 +643,30 @@ int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const 
     else if (small) gemm_bf16_tile128_residual_ragged_k<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
     else if (!ragged_k) gemm_bf16_tile256_residual<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
     else gemm_bf16_tile256_residual_ragged_k<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+    return (int)hipGetLastError();
+}
+
+bool gemm_bf16_swiglu_supported(long M, long F, long K) {
+    if (M <= 0 || F <= 0 || K <= 0) return false;
+    if (M > 0x7fffffffL || F % 8 || K % 8 || K > (1L << 23) || 2 * F > (1L << 25)) return false;
+    const long tn = (F + 127) / 128, tm = (M + mrk::dev::kBM - 1) / mrk::dev::kBM;
+    return tm * tn <= 0x7fffffffL;
+}
+
+int launch_gemm_bf16_swiglu(void* stream, const void* A, const void* B, void* C, long M, long F, long K) {
+    using namespace mrk::dev;
+    if (M <= 0 || F <= 0) return 0;
+    if (!gemm_bf16_swiglu_supported(M, F, K)) return (int)hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) % 16) return (int)hipErrorInvalidValue;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    (void)hipGetLastError();
+    const long tn = (F + 127) / 128, tm = (M + kBM - 1) / kBM;
+    const dim3 grid((unsigned)(tm * tn), 1);
+    const __bf16* a = static_cast<const __bf16*>(A);
+    const __bf16* b = static_cast<const __bf16*>(B);
+    __bf16* c = static_cast<__bf16*>(C);
+    if (K % kBK == 0) gemm_bf16_tile256_swiglu<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)(2 * F), (int)K, (int)tm, (int)tn);
+    else gemm_bf16_tile256_swiglu_ragged_k<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)(2 * F), (int)K, (int)tm, (int)tn);
     return (int)hipGetLastError();
 }
 

@@ -22,6 +22,11 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
 // kernels take without split-K; gemm_bf16_residual_supported tells.
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch);
 int launch_gemm_bf16_residual(void* stream, const void* a, const void* b, const void* r, void* c, long M, long N, long K, long batch);
+// C[M, F] = bf16(silu(float(bf16(A Wg))) * float(bf16(A Wu))) for W = [Wg | Wu] stored side by side as
+// one [K, 2F] matrix: the gated-MLP pair of products with the gate applied in the product kernel's
+// epilogue, so that the [M, 2F] product never reaches memory.  F and K multiples of 8.
+bool gemm_bf16_swiglu_supported(long M, long F, long K);
+int launch_gemm_bf16_swiglu(void* stream, const void* a, const void* w, void* c, long M, long F, long K);
 // Bytes of f32 scratch with which launch_gemm_bf16 spreads the K loop of this shape over the
 // chip (split-K: partial products per K range, added up in a fixed order by a second kernel);
 // 0 when the shape has enough output tiles by itself.  Without the workspace the same shape

@@ -382,7 +382,14 @@ Tensor Tensor::sigmoid() const {
     Tensor e = scaled.try_exp2();
     return const_(1.0, n_->dtype, n_->device_id).try_add(e).unary(UnaryOp::Reciprocal);
 }
-Tensor Tensor::swish() const { return try_mul(sigmoid()); }
+Tensor Tensor::swish() const {
+    Tensor res = try_mul(sigmoid());
+    if (res.valid()) {  // remembered so that silu(gate) * up over one packed product can run in that product's epilogue
+        res.node()->hint = HintKind::Swish;
+        res.node()->hint_inputs = {n_};
+    }
+    return res;
+}
 Tensor Tensor::tanh() const {
     // tanh(x) = 2 * sigmoid(2x) - 1  (activation.rs:64-74)
     if (!n_) return Tensor();
@@ -1152,7 +1159,7 @@ struct Scheduler {
         if (n->buffer) return;
         TensorNode* other = nullptr;
         if (n != root && (is_boundary_kind(n) || fusable(n) ||
-                          residual_matmul(const_cast<TensorNode*>(n), &other))) {
+                          residual_matmul(const_cast<TensorNode*>(n), &other) || swiglu_matmul(n))) {
             out.push_back(const_cast<TensorNode*>(n));
             return;
         }
@@ -1162,6 +1169,7 @@ struct Scheduler {
     bool fusable(const TensorNode* n) const {
         if (!g_fusion || n->hint == HintKind::None) return false;
         switch (n->hint) {
+            case HintKind::Swish: return false;  // no kernel of its own: only matched as part of swiglu_matmul
             case HintKind::Softmax:
                 return n->dtype == Scalar::Float32 && !n->shape.empty() &&
                        n->arg[0] == static_cast<int64_t>(n->shape.size()) - 1 && n->numel() > 0;
@@ -1289,6 +1297,48 @@ struct Scheduler {
         }
         return nullptr;
     }
+    // silu(p[:, :F]) * p[:, F:] in bf16 over one packed product p = a @ [Wg | Wu] that nothing else
+    // reads: the product kernel applies the gate in its epilogue and writes [M, F] directly.
+    // Returns the product node.
+    TensorNode* swiglu_matmul(const TensorNode* n) const {
+        if (!g_fusion || n->kind != TKind::Binary || static_cast<BinaryOp>(n->sub) != BinaryOp::Mul || n->dtype != Scalar::BFloat16 ||
+            n->numel() == 0 || n->src.size() != 2 || n->shape.size() != 2)
+            return nullptr;
+        for (int side = 0; side < 2; side++) {
+            const TensorNode* sw = n->src[side].get();
+            const TensorNode* up = n->src[1 - side].get();
+            if (sw->buffer || sw->hint != HintKind::Swish || sw->hint_inputs.size() != 1) continue;
+            const TensorNode* gate = sw->hint_inputs[0].get();
+            if (gate->buffer || up->buffer || gate->kind != TKind::Shrink || up->kind != TKind::Shrink) continue;
+            TensorNode* mm = gate->src[0].get();
+            if (up->src[0].get() != mm || mm->buffer || mm->hint != HintKind::Matmul || !fusable(mm) || mm->dtype != Scalar::BFloat16) continue;
+            if (mm->shape.size() != 2 || mm->hint_inputs[1]->shape.size() != 2) continue;
+            const int64_t M = mm->shape[0], F = n->shape[1];
+            if (mm->shape[1] != 2 * F || n->shape[0] != M || gate->shape != n->shape || up->shape != n->shape) continue;
+            if (gate->arg.size() != 2 || up->arg.size() != 2 || gate->arg[0] != 0 || gate->arg[1] != 0 || up->arg[0] != 0 || up->arg[1] != F) continue;
+            // nobody else may read the packed product, its halves or the gate's activation
+            auto used = [&](const TensorNode* t, int times) {
+                auto u = uses.find(t);
+                return u != uses.end() && u->second == times;
+            };
+            if (!used(mm, 2) || !used(gate, 2) || !used(up, 1) || !used(sw, 1)) continue;
+            int64_t Mx, N2, K, batch;
+            matmul_extents(mm, &Mx, &N2, &K, &batch);
+            if (batch != 1 || Mx != M || N2 != 2 * F || !gemm_bf16_swiglu_supported(M, F, K)) continue;
+            return mm;
+        }
+        return nullptr;
+    }
+    int materialize_swiglu_matmul(TensorNode* n, TensorNode* mm) {
+        for (const TensorRef& in : mm->hint_inputs) MRK_TRY(materialize(in.get()));
+        int64_t M, N2, K, batch;
+        matmul_extents(mm, &M, &N2, &K, &batch);
+        auto out = new_buffer(n);
+        MRK_TRY(builtin("gemm_bf16_swiglu", {M, N2 / 2, K}, {out, mm->hint_inputs[0]->buffer, mm->hint_inputs[1]->buffer}));
+        n->buffer = out;
+        produced.push_back(n);
+        return kOk;
+    }
     static void matmul_extents(const TensorNode* mm, int64_t* M, int64_t* N, int64_t* K, int64_t* batch) {
         const TensorNode *a = mm->hint_inputs[0].get(), *w = mm->hint_inputs[1].get();
         *K = a->shape.back();
@@ -1387,6 +1437,7 @@ struct Scheduler {
         {
             TensorNode* other = nullptr;
             if (TensorNode* mm = residual_matmul(n, &other)) return materialize_residual_matmul(n, mm, other);
+            if (TensorNode* mm = swiglu_matmul(n)) return materialize_swiglu_matmul(n, mm);
         }
         {
             std::vector<int64_t> out_strides;
@@ -1397,7 +1448,7 @@ struct Scheduler {
         if (n->kind == TKind::Reshape || n->kind == TKind::Contiguous) {
             TensorNode* s = n->src[0].get();
             TensorNode* other = nullptr;
-            if (s->buffer || is_boundary_kind(s) || fusable(s) || residual_matmul(s, &other)) {
+            if (s->buffer || is_boundary_kind(s) || fusable(s) || residual_matmul(s, &other) || swiglu_matmul(s)) {
                 MRK_TRY(materialize(s));
                 n->buffer = s->buffer;
                 produced.push_back(n);

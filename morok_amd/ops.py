@@ -42,6 +42,15 @@ def gemm_bf16_noalloc(a, b, c, m, n, k, device_id=0):
     check(lib.mrk_hip_gemm_bf16_noalloc(device_id, _p(a), _p(b), _p(c), m, n, k))
 
 
+def gemm_bf16_swiglu(a, w, c, m, f, k, device_id=0):
+    """c[m,f] = silu(a @ w[:, :f]) * (a @ w[:, f:]) for w [k, 2f] = gate | up, the gate applied in the
+    product kernel's epilogue."""
+    _need(a, m * k * 2, "gemm A")
+    _need(w, k * 2 * f * 2, "gemm W (gate | up)")
+    _need(c, m * f * 2, "gemm C")
+    check(lib.mrk_hip_gemm_bf16_swiglu(device_id, _p(a), _p(w), _p(c), m, f, k))
+
+
 def gemm_bf16_residual(a, b, r, c, m, n, k, device_id=0):
     """c[m,n] = a[m,k] @ b[k,n] + r[m,n]: the residual added in the product kernel's epilogue,
     same bits as gemm_bf16 followed by an elementwise add."""

@@ -27,6 +27,11 @@ int launch_gemm_bf16_residual(void* stream, const void*, const void*, const void
     mrk_shim_note_launch(stream, "gemm_bf16_residual");
     return 0;
 }
+bool gemm_bf16_swiglu_supported(long M, long F, long K) { return M > 0 && F > 0 && K > 0 && F % 8 == 0 && K % 8 == 0; }
+int launch_gemm_bf16_swiglu(void* stream, const void*, const void*, void*, long, long, long) {
+    mrk_shim_note_launch(stream, "gemm_bf16_swiglu");
+    return 0;
+}
 int launch_flash_fwd_bf16(void* stream, const void*, const void*, const void*, void*, long, long, long, long, float, int) {
     mrk_shim_note_launch(stream, "flash_fwd_bf16");
     return 0;

@@ -44,15 +44,16 @@ def test_decoder_block_vs_oracle(dev, oracle, cfg):
     # hand-written kernels
     assert sum(k.startswith("gemm_bf16") for k in kernels) == 4
     assert sum(k.startswith("flash_fwd") for k in kernels) == 1
-    # seven separate products give the same bits: every output element is the same dot product
+    assert sum(k.startswith("gemm_bf16_swiglu") for k in kernels) == 1   # silu(gate) * up in the W1|W3 epilogue
+    # Seven separate products compute the same dot products.  The gate differs in one place: the
+    # epilogue of the packed W1|W3 product takes its reciprocal with the hardware approximation
+    # (1 ulp) where the generated elementwise kernel divides exactly, so a small fraction of the
+    # gated activations round to the neighbouring bf16 value (and a product with few rows may be
+    # spread along K in one layout and not in the other): single roundings falling the other way.
     _, out7, kernels7 = run_block(cfg, tok, w, fused=False)
     assert sum(k.startswith("gemm_bf16") for k in kernels7) == 7
-    if any(k.endswith("_splitk") for k in kernels + kernels7):
-        # a product with few rows may be spread over the chip along K in one layout and not in
-        # the other: the same dot products, added up in a different order
-        assert rel_err(out7.to_numpy(), got) <= 1e-2   # single bf16 roundings falling the other way
-    else:
-        assert np.array_equal(out7.to_numpy(), got)
+    assert rel_err(out7.to_numpy(), got) <= 1e-2
+    assert rel_err(out7.to_numpy(), ref) <= 2e-2
 
 
 def test_decoder_block_full_size_properties(dev):

@@ -248,3 +248,43 @@ def test_gemm_residual_refuses_split_k_shapes(dev):
         ops.gemm_bf16_residual(a, b, c, c, 4, 1024, 4096, dev.device_id)   # few tiles, long K: the split-K shape
     with pytest.raises(morok_amd.MorokHipError):
         ops.gemm_bf16_residual(a, b, c, c, 4, 1020, 64, dev.device_id)     # N not a multiple of 8
+
+
+# ---------------------------------------------------------------- gated epilogue (SwiGLU)
+@pytest.mark.parametrize("shape", [(256, 128, 64), (512, 1024, 256), (300, 1000, 192), (37, 136, 72), (1024, 11008 // 8, 512)])
+def test_gemm_swiglu_epilogue_parity(dev, oracle, shape):
+    """c = silu(a @ Wg) * (a @ Wu) with [Wg | Wu] stored side by side, the gate applied in the product
+    kernel's epilogue: against the oracle's three stages (two bf16 products rounded to bf16, then
+    orc_silu_mul_bf16) at the bf16 GEMM tolerance, and against the unfused GPU sequence (two
+    products + the generated elementwise kernel), from which it may differ by the rounding of the
+    fast reciprocal only: one bf16 ulp on a small fraction of the elements."""
+    from morok_amd import tensor as T, uop
+
+    M, F, K = shape
+    a = synth.normal_bf16((M, K), 11, 0)
+    w = synth.to_bf16(synth.normal((K, 2 * F), 11, 1, sigma=1.0 / np.sqrt(K)))
+    ba, bw = morok_amd.Buffer.from_numpy(a, dev.device_id), morok_amd.Buffer.from_numpy(w, dev.device_id)
+    # NaNs right behind the result: the masked edge stores must not reach them
+    out = dev.buffer(M * F * 2 + 256)
+    out.copyin(np.full(M * F + 128, 0x7FC0, np.uint16))
+    ops.gemm_bf16_swiglu(ba, bw, out, M, F, K, dev.device_id)
+    raw = out.copyout(np.uint16, nbytes=M * F * 2 + 256)
+    got, guard = raw[: M * F].reshape(M, F), raw[M * F:]
+    assert np.all(guard == 0x7FC0)
+    gate, up = oracle.gemm_bf16(a, np.ascontiguousarray(w[:, :F])), oracle.gemm_bf16(a, np.ascontiguousarray(w[:, F:]))
+    ref = synth.from_bf16(oracle.silu_mul_bf16(gate, up))
+    gf = synth.from_bf16(got)
+    assert np.all(np.isfinite(gf))
+    assert np.abs(gf - ref).max() <= 2e-2 * np.abs(ref).max()
+    # the unfused path on the GPU
+    T.set_fusion(True)
+    ta, tw = T.Tensor.from_numpy(a, uop.BF16), T.Tensor.from_numpy(w, uop.BF16)
+    g, u = ta.matmul(tw.try_shrink([(0, K), (0, F)]).contiguous()), ta.matmul(tw.try_shrink([(0, K), (F, 2 * F)]).contiguous())
+    unfused = g.silu().try_mul(u).to_numpy()
+    diff = got.astype(np.int32) - unfused.astype(np.int32)
+    assert np.abs(diff).max() <= 1 and np.count_nonzero(diff) <= 0.02 * diff.size
+    # and through the lazy graph: the scheduler picks the fused kernel for the packed product
+    gu = ta.matmul(tw)
+    fused = gu.try_shrink([(0, M), (0, F)]).silu().try_mul(gu.try_shrink([(0, M), (F, 2 * F)]))
+    assert np.array_equal(fused.to_numpy(), got)
+    assert [k for k in fused.kernels() if k.startswith("gemm_bf16_swiglu")], fused.kernels()

@@ -420,7 +420,9 @@ def test_decoder_block_lowering(T, shim, fused, gemms):
     assert sum(k.startswith("flash_fwd_bf16_strided") for k in names) == 1
     # both residual additions happen in the epilogue of the product in front of them
     assert sum(k.startswith("gemm_bf16_residual") for k in names) == 2
-    assert len(names) == (13 if fused else 16)
+    # with gate and up stored side by side, silu(gate) * up happens in the epilogue of their product
+    assert sum(k.startswith("gemm_bf16_swiglu") for k in names) == (1 if fused else 0)
+    assert len(names) == (12 if fused else 16)
 
 
 def test_plan_graph_replay_records_once(T, shim):
