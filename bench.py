@@ -151,16 +151,20 @@ def bench_softmax(m, dev, steps, warmup, cpu):
 _CEILING = {}  # TFLOP/s of the MFMA-only calibration kernel, measured once per run
 
 
-def _mfma_ceiling_tflops(m, dev):
+def _mfma_ceiling_tflops(m, dev, random_operands=True):
     """Rate of the register-only MFMA kernel at the size of the 4096^3 product (256 workgroups x 64
-    K steps of a 256 x 256 tile), with the same settle / warm-up discipline as the workloads."""
+    K steps of a 256 x 256 tile), with the same settle / warm-up discipline as the workloads.
+    random_operands: operand registers hold hashed values in [-1.7, 1.7) (the default: what a
+    product of random matrices feeds the pipes) or small smooth values; the part is power-managed
+    and sustains a lower clock the more the operand bits toggle."""
     from morok_amd import ops
 
-    if "tf" not in _CEILING:
+    key = "random" if random_operands else "smooth"
+    if key not in _CEILING:
         scratch = dev.buffer(256).ensure_allocated()
-        ms, _ = _launch_stats(m, lambda: ops.mfma_ceiling(scratch, 256, 64), 50, 5)
-        _CEILING["tf"] = 2.0 * 4096 ** 3 / (ms * 1e-3) / 1e12
-    return _CEILING["tf"]
+        ms, _ = _launch_stats(m, lambda: ops.mfma_ceiling(scratch, 256, 64, random_operands=random_operands), 50, 5)
+        _CEILING[key] = 2.0 * 4096 ** 3 / (ms * 1e-3) / 1e12
+    return _CEILING[key]
 
 
 def _gemm_cpu_baseline(M, N, K):
@@ -233,7 +237,8 @@ def bench_gemm(m, dev, steps, warmup, cpu):
         "config": {"workload": "bf16 GEMM M=N=K=4096, normal(0,1) inputs, f32 accumulate, bf16 out, via "
                                "Tensor::matmul -> prepare -> execute (configs[2])"},
         "roofline": _roofline("gemm", "mfma", tf, BF16_PEAK_TFLOPS, "TFLOP/s", kernel, algorithmic_flops_per_launch=flops,
-                              mfma_only_ceiling=ceiling, frac_of_ceiling=tf / ceiling),
+                              mfma_only_ceiling=ceiling, frac_of_ceiling=tf / ceiling,
+                              mfma_only_ceiling_smooth_operands=_mfma_ceiling_tflops(m, dev, False)),
         "plan_item": program, "direct_abi_ms_per_step": direct_ms,
     }
     rec.update(stats)
@@ -405,9 +410,10 @@ def bench_generated_tc(m, dev, steps, warmup, cpu):
 def bench_mfma_ceiling(m, dev, steps, warmup, cpu):
     """Calibration only: the MFMA-only kernel at the size of the 4096^3 product."""
     tf = _mfma_ceiling_tflops(m, dev)
-    return {"metric": "MFMA-only ceiling TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": 2.0 * 4096 ** 3 / tf / 1e9,
+    smooth = _mfma_ceiling_tflops(m, dev, False)
+    return {"metric": "MFMA-only ceiling TFLOP/s", "smooth_operands_value": smooth, "value": tf, "unit": "TFLOP/s", "ms_per_step": 2.0 * 4096 ** 3 / tf / 1e9,
             "dtype": "bf16", "config": {"workload": "calibration: 256 workgroups x 64 K steps of register-only "
-                                                    "v_mfma_f32_32x32x16_bf16 (the MFMA stream of the 4096^3 GEMM)"},
+                                                    "v_mfma_f32_32x32x16_bf16 (the MFMA stream of the 4096^3 GEMM), hashed operand values"},
             "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": tf / BF16_PEAK_TFLOPS, "traffic": 0, "traffic_source": "no memory operands",
                          "kernel": "mfma_ceiling_kernel", "algorithmic_flops_per_launch": 2.0 * 4096 ** 3}}

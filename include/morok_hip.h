@@ -492,8 +492,10 @@ int mrk_hip_copy_kernel(int device_id, const void* src, void* dst, size_t bytes)
  * waves, each wave issuing the matrix-instruction stream of one 256 x 256 x (64 * k_steps) bf16
  * GEMM tile from registers, without memory traffic: 2 * 256 * 256 * 64 * k_steps flops per
  * workgroup.  The rate it sustains is the ceiling GEMM kernels are compared with next to the
- * published peak.  `scratch`: any device allocation of >= 4 bytes. */
-int mrk_hip_mfma_ceiling(int device_id, void* scratch, int64_t workgroups, int64_t k_steps);
+ * published peak.  random_operands: 0 = smooth small operand values, 1 = hashed values in
+ * [-1.7, 1.7) as in a product of random matrices (the pipes' power draw, and with it the sustained
+ * clock, depends on how much the operand bits toggle).  `scratch`: any device allocation of >= 4 bytes. */
+int mrk_hip_mfma_ceiling(int device_id, void* scratch, int64_t workgroups, int64_t k_steps, int random_operands);
 /* int32 values uniform over [0, high). */
 int mrk_hip_fill_randint(int device_id, void* out, size_t n, uint64_t seed, uint64_t tensor_id, int high);
 

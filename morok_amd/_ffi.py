@@ -158,7 +158,7 @@ _SIGS = {
                                                       C.POINTER(C.c_int64)]),
     "mrk_hip_fill": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_float,
                                C.c_float]),
-    "mrk_hip_mfma_ceiling": (C.c_int, [C.c_int, C.c_void_p, C.c_int64, C.c_int64]),
+    "mrk_hip_mfma_ceiling": (C.c_int, [C.c_int, C.c_void_p, C.c_int64, C.c_int64, C.c_int]),
     "mrk_hip_copy_kernel": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]),
     "mrk_hip_fill_randint": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_uint64, C.c_uint64, C.c_int]),
     "mrk_hip_event_create": (C.c_int, [C.c_int, c_void_pp]),

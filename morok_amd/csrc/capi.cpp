@@ -1013,13 +1013,13 @@ int mrk_hip_copy_kernel(int device_id, const void* src, void* dst, size_t bytes)
     return kOk;
 }
 
-int mrk_hip_mfma_ceiling(int device_id, void* scratch, int64_t workgroups, int64_t k_steps) {
+int mrk_hip_mfma_ceiling(int device_id, void* scratch, int64_t workgroups, int64_t k_steps, int random_operands) {
     MRK_NONNULL(scratch);
     if (workgroups <= 0 || k_steps <= 0) return fail(kInvalidArgument, "mfma_ceiling: workgroups and k_steps must be positive");
     std::shared_ptr<Device> d;
     MRK_TRY(get_device(device_id, &d));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_mfma_ceiling(d->allocator->stream(), scratch, workgroups, k_steps), "mfma_ceiling launch");
+    MRK_HIP(launch_mfma_ceiling(d->allocator->stream(), scratch, workgroups, k_steps, random_operands != 0), "mfma_ceiling launch");
     return kOk;
 }
 

@@ -13,7 +13,11 @@ namespace mrk::dev {
 typedef __bf16 cal_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float cal_f32x16 __attribute__((ext_vector_type(16)));
 
-__global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ out, int k_steps, float seed) {
+// operands: 0 = small smooth values (few bits toggle between consecutive instructions), 1 = values
+// spread over [-1.7, 1.7) by a hash of (lane, register, element), as the operands of a product of
+// random matrices are.  The matrix pipes' power draw, and with it the clock the part sustains,
+// depends on how much the operand bits toggle.
+__global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ out, int k_steps, float seed, int random_operands) {
     const int lane = threadIdx.x & 63;
     cal_f32x16 acc[4][4];
 #pragma unroll
@@ -27,8 +31,19 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ o
     for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            fa[i][e] = (__bf16)(seed * (float)(lane + e + i));
-            fb[i][e] = (__bf16)(seed * (float)(lane - e - i));
+            if (random_operands) {
+                unsigned x = (unsigned)((threadIdx.x * 4 + i) * 8 + e) * 2654435761u + blockIdx.x * 40503u + 12345u;
+                x ^= x >> 15;
+                x *= 2246822519u;
+                x ^= x >> 13;
+                unsigned y = x * 3266489917u;
+                y ^= y >> 16;
+                fa[i][e] = (__bf16)(((float)(x >> 8) / 8388608.0f - 1.0f) * 1.7f);
+                fb[i][e] = (__bf16)(((float)(y >> 8) / 8388608.0f - 1.0f) * 1.7f);
+            } else {
+                fa[i][e] = (__bf16)(seed * (float)(lane + e + i));
+                fb[i][e] = (__bf16)(seed * (float)(lane - e - i));
+            }
         }
     for (int kt = 0; kt < k_steps; kt++) {
 #pragma unroll
@@ -55,12 +70,12 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ o
 
 namespace mrk {
 
-int launch_mfma_ceiling(void* stream, void* out, long workgroups, long k_steps) {
+int launch_mfma_ceiling(void* stream, void* out, long workgroups, long k_steps, int random_operands) {
     if (workgroups <= 0 || k_steps <= 0 || workgroups > 0x7fffffffL || k_steps > 0x7fffffffL || !out)
         return (int)hipErrorInvalidValue;
     (void)hipGetLastError();
     dev::mfma_ceiling_kernel<<<(unsigned)workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<float*>(out),
-                                                                                               (int)k_steps, 0.001f);
+                                                                                               (int)k_steps, 0.001f, random_operands);
     return (int)hipGetLastError();
 }
 

@@ -72,11 +72,19 @@ class DecoderBlock:
         xn = self._norm(h, w["w_an"])
         if self.fused:
             qkv = xn.matmul(w["Wqkv"])
-            xq, xk, xv = (qkv.try_shrink([(0, T), (i * self.hidden, (i + 1) * self.hidden)]) for i in range(3))
+            xv = qkv.try_shrink([(0, T), (2 * self.hidden, 3 * self.hidden)])
+            # q and k lie side by side in the packed product: one rotary kernel over 2 * heads heads
+            # (the same per-head arithmetic), q and k are then the two halves of its result
+            xqk = qkv.try_shrink([(0, T), (0, 2 * self.hidden)])
+            qk = xqk.try_reshape([self.batch, self.seq, 2 * self.heads, self.dim]).try_permute([0, 2, 1, 3])
+            qk = qk.apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16).contiguous()
+            full = [(0, self.batch), None, (0, self.seq), (0, self.dim)]
+            q = qk.try_shrink([r if r else (0, self.heads) for r in full])
+            k = qk.try_shrink([r if r else (self.heads, 2 * self.heads) for r in full])
         else:
             xq, xk, xv = xn.matmul(w["Wq"]), xn.matmul(w["Wk"]), xn.matmul(w["Wv"])
-        q = self._heads(xq).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
-        k = self._heads(xk).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
+            q = self._heads(xq).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
+            k = self._heads(xk).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
         v = self._heads(xv)
         a = q.scaled_dot_product_attention(k, v, is_causal=True)
         a = a.try_permute([0, 2, 1, 3]).try_reshape([T, self.hidden])

@@ -117,8 +117,8 @@ def copy_kernel(src, dst, nbytes, device_id=0):
     check(lib.mrk_hip_copy_kernel(device_id, _p(src), _p(dst), nbytes))
 
 
-def mfma_ceiling(scratch, workgroups, k_steps, device_id=0):
+def mfma_ceiling(scratch, workgroups, k_steps, device_id=0, random_operands=True):
     """MFMA-only calibration kernel: the matrix-instruction stream of `workgroups` 256x256 GEMM
     tiles of depth 64 * k_steps, from registers (2 * 256 * 256 * 64 * k_steps flops each)."""
     _need(scratch, 4, "mfma_ceiling scratch")
-    check(lib.mrk_hip_mfma_ceiling(device_id, _p(scratch), workgroups, k_steps))
+    check(lib.mrk_hip_mfma_ceiling(device_id, _p(scratch), workgroups, k_steps, int(random_operands)))

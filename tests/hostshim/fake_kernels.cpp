@@ -53,7 +53,7 @@ int launch_copy(void* stream, const void*, void*, size_t) {
     mrk_shim_note_launch(stream, "copy");
     return 0;
 }
-int launch_mfma_ceiling(void* stream, void*, long, long) {
+int launch_mfma_ceiling(void* stream, void*, long, long, int) {
     mrk_shim_note_launch(stream, "mfma_ceiling");
     return 0;
 }
