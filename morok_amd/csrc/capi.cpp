@@ -934,7 +934,7 @@ int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, con
                                 int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal) {
     if (batch < 0 || heads < 0 || sq < 0 || sk < 0) return fail(kInvalidArgument, "flash_attn_fwd: negative shape");
     if (batch == 0 || heads == 0 || sq == 0) return kOk;
-    if (d != 128) return failf(kInvalidArgument, "flash_attn_fwd: head_dim %lld is not supported (128 only)", (long long)d);
+    if (d != 128 && d != 64) return failf(kInvalidArgument, "flash_attn_fwd: head_dim %lld is not supported (128 and 64 only)", (long long)d);
     if (sk == 0) return fail(kInvalidArgument, "flash_attn_fwd: empty key sequence (softmax over no keys is undefined)");
     if (!(scale > 0.0f)) return fail(kInvalidArgument, "flash_attn_fwd: scale must be positive");
     MRK_NONNULL(q);
@@ -954,7 +954,7 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
                                         const int64_t* strides) {
     if (batch < 0 || heads < 0 || sq < 0 || sk < 0) return fail(kInvalidArgument, "flash_attn_fwd_strided: negative shape");
     if (batch == 0 || heads == 0 || sq == 0) return kOk;
-    if (d != 128) return failf(kInvalidArgument, "flash_attn_fwd_strided: head_dim %lld is not supported (128 only)", (long long)d);
+    if (d != 128 && d != 64) return failf(kInvalidArgument, "flash_attn_fwd_strided: head_dim %lld is not supported (128 and 64 only)", (long long)d);
     if (sk == 0) return fail(kInvalidArgument, "flash_attn_fwd_strided: empty key sequence (softmax over no keys is undefined)");
     if (!(scale > 0.0f)) return fail(kInvalidArgument, "flash_attn_fwd_strided: scale must be positive");
     MRK_NONNULL(q);
@@ -969,7 +969,7 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
                          (long long)strides[i]);
         st[i] = static_cast<long>(strides[i]);
     }
-    if (st[11] < 128 || (heads > 1 && st[10] == 0) || (batch > 1 && st[9] == 0))
+    if (st[11] < d || (heads > 1 && st[10] == 0) || (batch > 1 && st[9] == 0))
         return fail(kInvalidArgument, "flash_attn_fwd_strided: output rows, heads and batches must not overlap");
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));

@@ -7,7 +7,8 @@
 // tensor (tensor/src/test/unit/fusion.rs:90-104).  Causal rule as in the reference:
 // key j is visible to query i iff j <= i (tril(0) over [Sq, Sk], transformer.rs:103-109).
 //
-// Layout: Q [BH, Sq, D], K [BH, Sk, D], V [BH, Sk, D], O [BH, Sq, D], row-major, D = 128.
+// Layout: Q [BH, Sq, D], K [BH, Sk, D], V [BH, Sk, D], O [BH, Sq, D], row-major, D = 128 or 64
+// (one instantiation of the same body per head dim; the comments below give the D = 128 numbers).
 //
 // Work split: one workgroup = 128 queries of one (batch, head); 4 waves x 32 queries.
 // K and V tiles of 64 keys travel global -> LDS directly (global_load_lds), two stages.
@@ -36,11 +37,8 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 #define LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
-constexpr int kD = 128;        // head dim
 constexpr int kQT = 128;       // queries per workgroup
 constexpr int kKT = 64;        // keys per tile
-constexpr int kRow = kD * 2;   // 256 B per K/V row
-constexpr int kTile = kKT * kRow;  // 16 KB
 
 // max(x of lane l, x of lane l ^ 32): the swap exchanges the upper 32 lanes of its first
 // register with the lower 32 lanes of its second, which leaves one register holding the
@@ -64,10 +62,23 @@ struct FlashLayout {
     int heads;
 };
 
-template <bool kStrided>
+// kD: head dim, 128 or 64.  Rows of K and V are kD * 2 bytes in LDS (256 or 128): with 256-byte
+// rows one row spans all 64 banks and the swizzles spread 16 consecutive rows over the 16-byte
+// chunks; with 128-byte rows two consecutive rows span the banks, so the K swizzle uses
+// (row >> 1) & 7 over the 8 chunks of a row and the V granule swizzle (row & 3 over 32-byte
+// granules) needs no change.
+template <int kD, bool kStrided>
 __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
                                                const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH, int Sq, int Sk,
                                                float scale_log2e, int causal, int q_tiles, int units, const FlashLayout& lay) {
+    static_assert(kD == 128 || kD == 64, "head dims with an instantiation: 128 and 64");
+    constexpr int kRow = kD * 2;          // bytes per K/V row in LDS: 256 (128)
+    constexpr int kTile = kKT * kRow;     // 16 KB (8 KB)
+    constexpr int kDS = kD / 16;          // 16-deep steps of the score product: 8 (4)
+    constexpr int kDB = kD / 32;          // 32-row blocks of O^T: 4 (2)
+    constexpr int kCh = kD / 8;           // 16-byte chunks per row: 16 (8)
+    constexpr int kRowsPerDma = 64 / kCh; // rows one 1 KB copy covers: 4 (8)
+    constexpr int kDmaPerWave = 16 / kRowsPerDma;  // copies per wave and tile: 4 (2)
     __shared__ __attribute__((aligned(1024))) char smem[4 * kTile];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // Workgroup ids congruent mod 8 run on the same XCD and share its L2.  Each XCD walks
@@ -131,7 +142,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     // ---- direct global -> LDS tile copies.  One instruction = 1 KB = 4 rows of 256 B.
     // wave w copies rows 16w .. 16w+15 of both tiles (4 instructions each).
     const unsigned lds_base = (unsigned)(uintptr_t)LDS_PTR(char, smem);
-    const int c16 = lane & 15, r4 = lane >> 4;
+    const int c16 = lane % kCh, r4 = lane / kCh;  // chunk inside the row, row inside the copy
     auto dma = [&](unsigned lds_addr, unsigned voff, const char* sbase) {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                      :
@@ -141,26 +152,28 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     // LDS map: K stage s at s*16 KB, V stage s at 32 KB + s*16 KB
     auto dma_k = [&](int j, int stage) {
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const int row = wave * 16 + c * 4 + r4;  // row inside the tile
+        for (int c = 0; c < kDmaPerWave; c++) {
+            const int row = wave * 16 + c * kRowsPerDma + r4;  // row inside the tile
             int key = j * kKT + row;
             key = key < Sk ? key : Sk - 1;  // ragged tail: re-read the last row, masked later
             // 16 B chunk c16 of the LDS row holds logical chunk c16 ^ (row & 15): the LDS
             // serves 16 lanes x 16 B per cycle over 64 banks, so 16 consecutive rows must
-            // land in 16 different chunk slots
-            const unsigned kvoff = (unsigned)key * k_row + ((c16 ^ (row & 15)) << 4);
-            dma(lds_base + stage * kTile + (wave * 16 + c * 4) * kRow, kvoff, Kh);
+            // land in 16 different chunk slots (128-byte rows: c16 ^ ((row >> 1) & 7), the
+            // parity of the row selects the half of the banks)
+            const int ksw = kD == 128 ? (row & 15) : ((row >> 1) & 7);
+            const unsigned kvoff = (unsigned)key * k_row + ((c16 ^ ksw) << 4);
+            dma(lds_base + stage * kTile + (wave * 16 + c * kRowsPerDma) * kRow, kvoff, Kh);
         }
     };
     auto dma_v = [&](int j, int stage) {
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const int row = wave * 16 + c * 4 + r4;
+        for (int c = 0; c < kDmaPerWave; c++) {
+            const int row = wave * 16 + c * kRowsPerDma + r4;
             int key = j * kKT + row;
             key = key < Sk ? key : Sk - 1;
             // 32 B granule (c16 >> 1) holds logical granule (c16 >> 1) ^ (row & 3)
             const unsigned vvoff = (unsigned)key * v_row + (((((c16 >> 1) ^ (row & 3)) << 1) | (c16 & 1)) << 4);
-            dma(lds_base + 2 * kTile + stage * kTile + (wave * 16 + c * 4) * kRow, vvoff, Vh);
+            dma(lds_base + 2 * kTile + stage * kTile + (wave * 16 + c * kRowsPerDma) * kRow, vvoff, Vh);
         }
     };
     auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
@@ -179,23 +192,23 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     }
 
     // ---- Q^T fragments: lane holds q = qw0 + l%32, d = 16*ds + 8*(l/32) .. +8
-    bf16x8 qf[8];
+    bf16x8 qf[kDS];
     {
         int qrow = qw0 + lq;
         qrow = qrow < Sq ? qrow : Sq - 1;
         const __bf16* qp = Qh + (size_t)qrow * (q_row / 2) + 8 * lg;
 #pragma unroll
-        for (int ds = 0; ds < 8; ds++) qf[ds] = *reinterpret_cast<const bf16x8*>(qp + 16 * ds);
+        for (int ds = 0; ds < kDS; ds++) qf[ds] = *reinterpret_cast<const bf16x8*>(qp + 16 * ds);
         // Make the compiler wait for these loads here, before the loop: inside the loop the
         // only outstanding vector-memory operations must be the direct-to-LDS copies it does
         // not know about, which are drained explicitly in tile_barrier().
 #pragma unroll
-        for (int ds = 0; ds < 8; ds++) asm volatile("" : "+v"(qf[ds]));
+        for (int ds = 0; ds < kDS; ds++) asm volatile("" : "+v"(qf[ds]));
     }
 
-    f32x16 o[4];
+    f32x16 o[kDB];
 #pragma unroll
-    for (int db = 0; db < 4; db++)
+    for (int db = 0; db < kDB; db++)
 #pragma unroll
         for (int e = 0; e < 16; e++) o[db][e] = 0.0f;
     float m_run = -INFINITY;  // running max of raw scores (before scale)
@@ -205,7 +218,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     // lane-constant LDS offsets
     // K fragment (A operand): row = kb*32 + l%32, logical chunk 2*ds + l/32
     const int k_row_off = lq * kRow;
-    const int k_sw = lq & 15;
+    const int k_sw = kD == 128 ? (lq & 15) : ((lq >> 1) & 7);
     // V^T fragment via transposing read: 16-lane block b = l/16 covers d half (b & 1) and
     // key group g = b >> 1; inside the block lane j' = l%16 points at key row j'/4,
     // 8-byte unit j'%4 of the 32-byte granule.
@@ -233,8 +246,8 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         for (int kb = 0; kb < 2; kb++)
             kf[0][kb] = *LDS_PTR(bf16x8, sK + kb * 32 * kRow + k_row_off + (((0 + lg) ^ k_sw) << 4));
 #pragma unroll
-        for (int ds = 0; ds < 8; ds++) {
-            if (ds + 1 < 8) {
+        for (int ds = 0; ds < kDS; ds++) {
+            if (ds + 1 < kDS) {
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++)
                     kf[(ds + 1) & 1][kb] =
@@ -283,7 +296,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
             m_run = m_new;
             l_run *= alpha;
 #pragma unroll
-            for (int db = 0; db < 4; db++) o[db] *= alpha;
+            for (int db = 0; db < kDB; db++) o[db] *= alpha;
         }
         // K(j+1) and V(j) have landed; every wave is done with K(j) and V(j-1)
         tile_barrier();
@@ -295,8 +308,8 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         const float mb = m_run * scale_log2e;
 
         // ---- phase A: S(j+1) = K(j+1) Q^T on the matrix pipe, P(j) = exp2(S(j)*c - m*c) on
-        // the vector ALUs: each of the 16 MFMAs is followed by the exponentials of two score
-        // registers (the last iteration computes a tile nobody uses).  The fences keep the
+        // the vector ALUs: each of the 16 (8) MFMAs is followed by the exponentials of two (four)
+        // score registers (the last iteration computes a tile nobody uses).  The fences keep the
         // compiler from regrouping the two instruction streams.
         float psum0 = 0.0f, psum1 = 0.0f;
         bf16x8 pb[2][2];
@@ -310,9 +323,10 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
             for (int kb = 0; kb < 2; kb++)
                 kf[0][kb] = *LDS_PTR(bf16x8, sKn + kb * 32 * kRow + k_row_off + (((0 + lg) ^ k_sw) << 4));
             f32x8 p;
+            constexpr int kPairs = 8 / kDS;  // pairs of score registers per MFMA: 1 (2)
 #pragma unroll
-            for (int ds = 0; ds < 8; ds++) {
-                if (ds + 1 < 8) {
+            for (int ds = 0; ds < kDS; ds++) {
+                if (ds + 1 < kDS) {
 #pragma unroll
                     for (int kb = 0; kb < 2; kb++)
                         kf[(ds + 1) & 1][kb] =
@@ -321,15 +335,18 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++) {
                     nxt[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds & 1][kb], qf[ds], nxt[kb], 0, 0, 0);
-                    const int idx = ds * 2 + kb;           // 0..15: score registers 2*idx, 2*idx+1
-                    const int pk = idx >> 3, pe = (idx & 7) * 2;  // block, register inside the block
-                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe], scale_log2e, -mb));
-                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe + 1], scale_log2e, -mb));
-                    psum0 += p0;
-                    psum1 += p1;
-                    p[pe & 7] = p0;
-                    p[(pe & 7) + 1] = p1;
-                    if ((idx & 3) == 3) pb[pk][(idx >> 2) & 1] = __builtin_convertvector(p, bf16x8);
+#pragma unroll
+                    for (int pr = 0; pr < kPairs; pr++) {
+                        const int idx = (ds * 2 + kb) * kPairs + pr;  // 0..15: score registers 2*idx, 2*idx+1
+                        const int pk = idx >> 3, pe = (idx & 7) * 2;  // block, register inside the block
+                        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe], scale_log2e, -mb));
+                        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe + 1], scale_log2e, -mb));
+                        psum0 += p0;
+                        psum1 += p1;
+                        p[pe & 7] = p0;
+                        p[(pe & 7) + 1] = p1;
+                        if ((idx & 3) == 3) pb[pk][(idx >> 2) & 1] = __builtin_convertvector(p, bf16x8);
+                    }
                     __builtin_amdgcn_sched_barrier(0);
                 }
             }
@@ -341,8 +358,9 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         // registers 8t .. 8t+7 of block kb: keys kb*32 + 16t + {0, 8} + 4*(l/32) + 0..3.
         float mx0 = -INFINITY, mx1 = -INFINITY;
         {
-            auto vfrag = [&](int n) {  // n = (kb*2 + t)*4 + db
-                const int kbt = n >> 2, db = n & 3;
+            constexpr int kNB = 4 * kDB;  // MFMAs of this phase: 16 (8)
+            auto vfrag = [&](int n) {  // n = (kb*2 + t)*kDB + db
+                const int kbt = n / kDB, db = n % kDB;
                 const int off = (kbt * 16) * kRow + v_row_off + (((db * 2 + v_half) ^ v_rr) << 5);
                 bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sV + off));
                 bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sV + off + 8 * kRow));
@@ -353,13 +371,15 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
             vf[1] = vfrag(1);
             const int key0n = (j + 1) * kKT;
 #pragma unroll
-            for (int n = 0; n < 16; n++) {
-                if (n + 2 < 16) vf[(n + 2) % 3] = vfrag(n + 2);
-                o[n & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[n % 3], pb[n >> 3][(n >> 2) & 1], o[n & 3], 0, 0, 0);
-                if (n >= 8) {  // the score MFMAs have drained by now: 4 registers per slot
-                    const int kb = (n - 8) >> 2, e0 = ((n - 8) & 3) * 4;
+            for (int n = 0; n < kNB; n++) {
+                if (n + 2 < kNB) vf[(n + 2) % 3] = vfrag(n + 2);
+                const int kbt = n / kDB, db = n % kDB;
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[n % 3], pb[kbt >> 1][kbt & 1], o[db], 0, 0, 0);
+                if (n >= kNB / 2) {  // the score MFMAs have drained by now: 4 (8) registers per slot
+                    constexpr int kSlotsPerKb = kNB / 4, kRegs = 16 / kSlotsPerKb;
+                    const int kb = (n - kNB / 2) / kSlotsPerKb, e0 = ((n - kNB / 2) % kSlotsPerKb) * kRegs;
 #pragma unroll
-                    for (int e = e0; e < e0 + 4; e++) {
+                    for (int e = e0; e < e0 + kRegs; e++) {
                         if (decltype(mask_next)::value) {
                             const int key = key0n + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3);
                             if (key > lim) nxt[kb][e] = -INFINITY;
@@ -427,7 +447,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     if (qrow < Sq) {
         __bf16* op = Oh + (size_t)qrow * (o_row / 2) + 4 * lg;
 #pragma unroll
-        for (int db = 0; db < 4; db++)
+        for (int db = 0; db < kDB; db++)
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 f32x4 v = {o[db][4 * g] * inv, o[db][4 * g + 1] * inv, o[db][4 * g + 2] * inv, o[db][4 * g + 3] * inv};
@@ -440,14 +460,25 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
 __global__ __launch_bounds__(256, 2) void flash_fwd_d128(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
                                                          const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
                                                          int Sq, int Sk, float scale_log2e, int causal, int q_tiles, int units) {
-    flash_fwd_body<false>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, FlashLayout{});
+    flash_fwd_body<128, false>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, FlashLayout{});
+}
+__global__ __launch_bounds__(256, 2) void flash_fwd_d64(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
+                                                        const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
+                                                        int Sq, int Sk, float scale_log2e, int causal, int q_tiles, int units) {
+    flash_fwd_body<64, false>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, FlashLayout{});
 }
 
 __global__ __launch_bounds__(256, 2) void flash_fwd_d128_strided(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
                                                                  const __bf16* __restrict__ V, __bf16* __restrict__ O,
                                                                  int BH, int Sq, int Sk, float scale_log2e, int causal,
                                                                  int q_tiles, int units, FlashLayout lay) {
-    flash_fwd_body<true>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, lay);
+    flash_fwd_body<128, true>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, lay);
+}
+__global__ __launch_bounds__(256, 2) void flash_fwd_d64_strided(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
+                                                                const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
+                                                                int Sq, int Sk, float scale_log2e, int causal, int q_tiles,
+                                                                int units, FlashLayout lay) {
+    flash_fwd_body<64, true>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, lay);
 }
 
 }  // namespace mrk::dev
@@ -458,7 +489,7 @@ int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void
                           long D, float scale, int causal) {
     using namespace mrk::dev;
     if (BH <= 0 || Sq <= 0) return 0;
-    if (D != kD || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
+    if ((D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
     if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
     const long q_tiles = (Sq + kQT - 1) / kQT;
     const long units = causal ? (q_tiles + 1) / 2 : q_tiles;
@@ -466,7 +497,8 @@ int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void
     if (blocks > 0x7fffffffL) return (int)hipErrorInvalidValue;
     (void)hipGetLastError();
     const float scale_log2e = scale * 1.4426950408889634f;
-    flash_fwd_d128<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
+    auto kernel = D == 128 ? flash_fwd_d128 : flash_fwd_d64;
+    kernel<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
         static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles, (int)units);
     return (int)hipGetLastError();
@@ -478,7 +510,7 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
     if (B < 0 || H < 0 || !strides) return (int)hipErrorInvalidValue;
     const long BH = B * H;
     if (BH == 0 || Sq <= 0) return 0;
-    if (D != kD || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
+    if ((D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
     if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
     // strides: (batch, head, row) of q, k, v, o in elements.  Rows are read and written in
     // 16-byte pieces from 16-byte aligned addresses; row offsets inside a head are 32-bit
@@ -489,10 +521,10 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
         const long sb = strides[3 * t], sh = strides[3 * t + 1], sr = strides[3 * t + 2];
         if (sb < 0 || sh < 0 || sr < 0 || sb % 8 || sh % 8 || sr % 8) return (int)hipErrorInvalidValue;
         if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16) return (int)hipErrorInvalidValue;
-        if (sr > (1L << 30) || (rows[t] - 1) * sr * 2 + kRow > 0xffffffffL) return (int)hipErrorInvalidValue;
+        if (sr > (1L << 30) || (rows[t] - 1) * sr * 2 + D * 2 > 0xffffffffL) return (int)hipErrorInvalidValue;
         // the output must not alias itself: distinct rows, heads and batches at distinct places
-        if (t == 3 && (sr < kD || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
-        dense = dense && sr == kD && sh == rows[t] * kD && sb == H * rows[t] * kD;
+        if (t == 3 && (sr < D || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
+        dense = dense && sr == D && sh == rows[t] * D && sb == H * rows[t] * D;
     }
     if (dense) return launch_flash_fwd_bf16(stream, q, k, v, o, BH, Sq, Sk, D, scale, causal);
     const long q_tiles = (Sq + kQT - 1) / kQT;
@@ -509,7 +541,8 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
     lay.heads = (int)H;
     (void)hipGetLastError();
     const float scale_log2e = scale * 1.4426950408889634f;
-    flash_fwd_d128_strided<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
+    auto kernel = D == 128 ? flash_fwd_d128_strided : flash_fwd_d64_strided;
+    kernel<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
         static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles, (int)units, lay);
     return (int)hipGetLastError();

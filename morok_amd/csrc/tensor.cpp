@@ -1199,7 +1199,7 @@ struct Scheduler {
                 const TensorNode* k = n->hint_inputs[1].get();
                 const TensorNode* v = n->hint_inputs[2].get();
                 return q->dtype == Scalar::BFloat16 && k->dtype == q->dtype && v->dtype == q->dtype &&
-                       q->shape.size() == 4 && q->shape[3] == 128 && v->shape[3] == 128 && k->shape[2] > 0 &&
+                       q->shape.size() == 4 && (q->shape[3] == 128 || q->shape[3] == 64) && v->shape[3] == q->shape[3] && k->shape[2] > 0 &&
                        k->shape[0] == q->shape[0] && k->shape[1] == q->shape[1] && q->numel() > 0;
             }
             default: return false;
@@ -1497,7 +1497,7 @@ struct Scheduler {
     }
 
     // The attention kernel over whatever views its operands are: an operand that is a strided
-    // view of data in memory (rows of 128 contiguous elements, 16-byte aligned) is read in
+    // view of data in memory (rows of head-dim contiguous elements, 16-byte aligned) is read in
     // place, anything else is materialised first.  `dst` is the node that receives the buffer,
     // `out_strides` the layout of the [B, H, Sq, D] result inside it.
     int materialize_attention(TensorNode* att, TensorNode* dst, const std::vector<int64_t>& out_strides) {
