@@ -367,10 +367,13 @@ int mrk_hip_sched_build_wmma_matmul_lds_opts(int tc_index, int64_t m, int64_t n,
                                              uint8_t** kernel, size_t* len);
 void mrk_hip_sched_free(void* p);
 /* The f32 matmul kernel with the optimisation choices explicit: opts = {LOCAL x, LOCAL y,
- * UPCAST of N (vector width 1/2/4), UPCAST of M (rows per work-item 1..8), UNROLL of K}.
- * INVALID_ARGUMENT when the choices do not divide the shape (the action space of
- * schedule/src/optimizer/beam.rs:36-120 restricted to this kernel). */
-int mrk_hip_sched_build_matmul_f32_opts(int64_t m, int64_t n, int64_t k, const int opts[5], uint8_t** kernel, size_t* len);
+ * UPCAST of N (vector width 1/2/4), UPCAST of M (rows per work-item 1..8), UNROLL of K,
+ * GROUP depth}.  GROUP depth 0: operands straight from global memory.  8 / 16 / 32: the
+ * workgroup stages A and B tiles of that K depth through local memory (UPCAST 4 or 8 each way,
+ * UNROLL ignored; schedule/src/optimizer/heuristics.rs:37-82).  INVALID_ARGUMENT when the choices
+ * do not divide the shape (the action space of schedule/src/optimizer/beam.rs:36-120 restricted
+ * to this kernel). */
+int mrk_hip_sched_build_matmul_f32_opts(int64_t m, int64_t n, int64_t k, const int opts[6], uint8_t** kernel, size_t* len);
 
 /* =====================================================================================
  * Beam-search support (tensor/src/realize.rs:1190-1242, schedule/src/optimizer/beam.rs)
@@ -388,10 +391,10 @@ int mrk_hip_compile_and_time(int device_id, const void* kernel, size_t len, cons
  * IGNORE_BEAM_CACHE is set); INVALID_ARGUMENT if the value exceeds capacity. */
 int mrk_hip_beam_cache_get(uint64_t ast_hash, int width, const char* device, void* value, size_t capacity, size_t* len);
 int mrk_hip_beam_cache_put(uint64_t ast_hash, int width, const char* device, const void* value, size_t len);
-/* Beam search of width `width` over LOCAL / UPCAST / UNROLL for the f32 matmul of this shape;
- * result in opts (same layout as above), its time in *best_ms, *from_cache = 1 when the disk
- * cache answered, *timed = number of candidates compiled and timed. */
-int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t k, int width, int opts[5],
+/* Beam search of width `width` over LOCAL / UPCAST / UNROLL / GROUP for the f32 matmul of this
+ * shape; result in opts (same six-entry layout as above), its time in *best_ms, *from_cache = 1
+ * when the disk cache answered, *timed = number of candidates compiled and timed. */
+int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t k, int width, int opts[6],
                                    double* best_ms, int* from_cache, int* timed);
 /* The same search over the LDS-staged tensor-core matmul of mrk_hip_sched_build_wmma_matmul_lds_opts
  * (bf16 / f16 in and out, tensor core `tc_index` of mrk_hip_sched_tensor_cores): the TC action

@@ -734,13 +734,13 @@ int mrk_hip_sched_build_wmma_matmul_lds_opts(int tc_index, int64_t m, int64_t n,
     return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
 }
 void mrk_hip_sched_free(void* p) { std::free(p); }
-int mrk_hip_sched_build_matmul_f32_opts(int64_t m, int64_t n, int64_t k, const int opts[5], uint8_t** kernel, size_t* len) {
+int mrk_hip_sched_build_matmul_f32_opts(int64_t m, int64_t n, int64_t k, const int opts[6], uint8_t** kernel, size_t* len) {
     MRK_NONNULL(opts);
     MRK_NONNULL(kernel);
     MRK_NONNULL(len);
-    MatmulF32Opts o{opts[0], opts[1], opts[2], opts[3], opts[4]};
+    MatmulF32Opts o{opts[0], opts[1], opts[2], opts[3], opts[4], opts[5]};
     if (!matmul_f32_opts_valid(o, m, n, k))
-        return fail(kInvalidArgument, "matmul f32: LOCAL/UPCAST/UNROLL choices do not fit the shape");
+        return fail(kInvalidArgument, "matmul f32: LOCAL/UPCAST/UNROLL/GROUP choices do not fit the shape");
     LinearKernel lk = build_matmul_f32_kernel(m, n, k, o);
     return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
 }
@@ -784,7 +784,7 @@ int mrk_hip_beam_cache_put(uint64_t ast_hash, int width, const char* device, con
     if (len) MRK_NONNULL(value);
     return BeamCache::put(ast_hash, width, device, value, len);
 }
-int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t k, int width, int opts[5],
+int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t k, int width, int opts[6],
                                    double* best_ms, int* from_cache, int* timed) {
     MRK_NONNULL(opts);
     std::shared_ptr<Device> d;
@@ -799,6 +799,7 @@ int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t 
     opts[2] = o.up_n;
     opts[3] = o.up_m;
     opts[4] = o.unroll_k;
+    opts[5] = o.lds_k;
     if (best_ms) *best_ms = ms;
     if (from_cache) *from_cache = cached ? 1 : 0;
     if (timed) *timed = n_timed;

@@ -436,13 +436,13 @@ int beam_search_matmul_f32(const Device& dev, int64_t M, int64_t N, int64_t K, i
     if (candidates_timed) *candidates_timed = 0;
     std::vector<uint8_t> cached;
     struct Record {
-        int32_t opts[5];
+        int32_t opts[6];
         double ms;
     };
     if (BeamCache::get(ast_hash, width, device, &cached) && cached.size() == sizeof(Record)) {
         Record r;
         std::memcpy(&r, cached.data(), sizeof r);
-        MatmulF32Opts o{r.opts[0], r.opts[1], r.opts[2], r.opts[3], r.opts[4]};
+        MatmulF32Opts o{r.opts[0], r.opts[1], r.opts[2], r.opts[3], r.opts[4], r.opts[5]};
         if (matmul_f32_opts_valid(o, M, N, K)) {
             *best = o;
             if (best_ms) *best_ms = r.ms;
@@ -533,9 +533,27 @@ int beam_search_matmul_f32(const Device& dev, int64_t M, int64_t N, int64_t K, i
         beam = next;
         keep_best(beam);
     }
+    // stage 4: GROUP - the operand tiles staged through local memory, with the register tiles it allows
+    {
+        std::vector<Cand> next = beam;
+        for (const Cand& cnd : beam)
+            for (int depth : {8, 16, 32})
+                for (int un : {4, 8})
+                    for (int um : {4, 8}) {
+                        MatmulF32Opts o = cnd.second;
+                        o.lds_k = depth;
+                        o.up_n = un;
+                        o.up_m = um;
+                        o.unroll_k = 1;
+                        double ms;
+                        if (time_one(o, &ms)) next.emplace_back(ms, o);
+                    }
+        beam = next;
+        keep_best(beam);
+    }
     *best = beam[0].second;
     if (best_ms) *best_ms = beam[0].first;
-    Record r{{best->local_x, best->local_y, best->up_n, best->up_m, best->unroll_k}, beam[0].first};
+    Record r{{best->local_x, best->local_y, best->up_n, best->up_m, best->unroll_k, best->lds_k}, beam[0].first};
     (void)BeamCache::put(ast_hash, width, device, &r, sizeof r);  // a read-only cache directory is not an error
     clear_error();
     return kOk;

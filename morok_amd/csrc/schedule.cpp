@@ -486,14 +486,115 @@ LinearKernel KernelBuilder::finish() {
 // ============================================================================ matmul kernels
 bool matmul_f32_opts_valid(const MatmulF32Opts& o, int64_t M, int64_t N, int64_t K) {
     if (o.local_x < 1 || o.local_y < 1 || o.local_x * o.local_y > 1024) return false;
-    if (o.up_n != 1 && o.up_n != 2 && o.up_n != 4) return false;
     if (o.up_m < 1 || o.up_m > 8 || o.unroll_k < 1 || o.unroll_k > 8) return false;
-    if (o.up_m * o.up_n > 32) return false;  // accumulator registers per work-item
+    if (o.up_m * o.up_n > (o.lds_k ? 64 : 32)) return false;  // accumulator registers per work-item
+    if (o.lds_k) {
+        const int64_t threads = static_cast<int64_t>(o.local_x) * o.local_y, tile_m = static_cast<int64_t>(o.local_y) * o.up_m,
+                      tile_n = static_cast<int64_t>(o.local_x) * o.up_n;
+        if (o.lds_k != 8 && o.lds_k != 16 && o.lds_k != 32) return false;
+        if (o.up_n != 4 && o.up_n != 8) return false;
+        if (o.up_m != 4 && o.up_m != 8) return false;
+        if (threads < 64 || threads % 64 || K % o.lds_k) return false;
+        // every work-item copies the same whole number of 4-float vectors of each tile
+        if ((tile_m * o.lds_k / 4) % threads || (tile_n * o.lds_k / 4) % threads) return false;
+        if ((tile_m + 4 + tile_n + 4) * o.lds_k * 4 > 65536) return false;
+        return M % tile_m == 0 && N % tile_n == 0 && M > 0 && N > 0 && K > 0;
+    }
+    if (o.up_n != 1 && o.up_n != 2 && o.up_n != 4) return false;
     return M % (static_cast<int64_t>(o.local_y) * o.up_m) == 0 && N % (static_cast<int64_t>(o.local_x) * o.up_n) == 0 &&
            K % o.unroll_k == 0 && M > 0 && N > 0 && K > 0;
 }
 
+// C = A B in f32 with the operand tiles staged through local memory.  Workgroup tile
+// (local_y * up_m) x (local_x * up_n), K depth lds_k per stage.  LDS holds A transposed
+// ([k][m], pitch tile_m + 4) and B as it lies ([k][n], pitch tile_n + 4): a work-item's up_m rows
+// and up_n columns are then whole 16-byte vectors, read once per k and reused up_n / up_m times;
+// the 16 lanes of a row of the workgroup read the same A vector (a broadcast) and 256 contiguous
+// bytes of B.  Copies: global -> registers (16-byte loads along k for A, along n for B) -> LDS;
+// the loads of the next stage are issued before this stage's barrier.
+static LinearKernel build_matmul_f32_lds_kernel(int64_t M, int64_t N, int64_t K, const MatmulF32Opts& o) {
+    KernelBuilder b;
+    b.enable_cse();
+    const Scalar f = Scalar::Float32;
+    const int un = o.up_n, um = o.up_m, BK = o.lds_k;
+    const int threads = o.local_x * o.local_y;
+    const int64_t BM = static_cast<int64_t>(o.local_y) * um, BN = static_cast<int64_t>(o.local_x) * un;
+    const int64_t PA = BM + 4, PB = BN + 4;
+    const int VA = static_cast<int>(BM * BK / 4 / threads), VB = static_cast<int>(BN * BK / 4 / threads);
+    uint32_t c = b.param(0, f, M * N), a = b.param(1, f, M * K), bm = b.param(2, f, K * N);
+    uint32_t gx = b.special("gidx0", N / BN), gy = b.special("gidx1", M / BM);
+    uint32_t lx = b.special("lidx0", o.local_x), ly = b.special("lidx1", o.local_y);
+    uint32_t tid = b.iadd(b.imul(ly, o.local_x), lx);
+    uint32_t sA = b.define_local(0, f, PA * BK), sB = b.define_local(1, f, PB * BK);
+    uint32_t ra = b.define_reg(1, f, VA, 4), rb = b.define_reg(2, f, VB, 4);
+    // vector v of a tile: A row v / (BK / 4), k offset 4 * (v % (BK / 4)); B k row v / (BN / 4), column 4 * (v % (BN / 4))
+    std::vector<uint32_t> a_row(VA), a_k(VA), b_k(VB), b_col(VB);
+    for (int i = 0; i < VA; i++) {
+        uint32_t v = b.iadd(tid, b.ci(threads * i));
+        a_row[i] = b.idiv(v, BK / 4);
+        a_k[i] = b.imul(b.imod(v, BK / 4), 4);
+    }
+    for (int i = 0; i < VB; i++) {
+        uint32_t v = b.iadd(tid, b.ci(threads * i));
+        b_k[i] = b.idiv(v, BN / 4);
+        b_col[i] = b.imul(b.imod(v, BN / 4), 4);
+    }
+    auto global_to_regs = [&](uint32_t kbase) {
+        for (int i = 0; i < VA; i++) {
+            uint32_t row = b.iadd(b.imul(gy, BM), a_row[i]);
+            b.store(b.index(ra, b.ci(i)), b.load(b.index(a, b.iadd(b.imul(row, K), b.iadd(kbase, a_k[i]))), 4));
+        }
+        for (int i = 0; i < VB; i++) {
+            uint32_t col = b.iadd(b.imul(gx, BN), b_col[i]);
+            b.store(b.index(rb, b.ci(i)), b.load(b.index(bm, b.iadd(b.imul(b.iadd(kbase, b_k[i]), N), col)), 4));
+        }
+    };
+    std::vector<uint32_t> acc(um * un);
+    uint32_t zero = b.cf(0.0);
+    for (int i = 0; i < um * un; i++) {
+        acc[i] = b.index(b.define_reg(3 + i, f, 1), b.ci(0));
+        b.store(acc[i], zero);
+    }
+    const int64_t KT = K / BK;
+    global_to_regs(b.ci(0));
+    uint32_t r = b.range(KT, 0, AxisType::Reduce);
+    for (int i = 0; i < VA; i++) {  // A transposed: element (row, k) to sA[k][row]
+        uint32_t v = b.load(b.index(ra, b.ci(i)));
+        for (int e = 0; e < 4; e++) b.store(b.index(sA, b.iadd(b.imul(b.iadd(a_k[i], b.ci(e)), PA), a_row[i])), b.gep(v, e));
+    }
+    for (int i = 0; i < VB; i++) b.store(b.index(sB, b.iadd(b.imul(b_k[i], PB), b_col[i])), b.load(b.index(rb, b.ci(i))));
+    uint32_t rn = b.iadd(r, b.ci(1));
+    uint32_t knext = b.imul(b.where(b.binary(BinaryOp::Lt, rn, b.ci(KT)), rn, b.ci(KT - 1)), BK);
+    global_to_regs(knext);
+    b.barrier();
+    uint32_t a_base = b.imul(ly, um), b_base = b.imul(lx, un);
+    for (int kk = 0; kk < BK; kk++) {
+        std::vector<uint32_t> av, bv;
+        for (int i = 0; i < um; i += 4) {
+            uint32_t v = b.load(b.index(sA, b.iadd(a_base, b.ci(kk * PA + i))), 4);
+            for (int e = 0; e < 4; e++) av.push_back(b.gep(v, e));
+        }
+        for (int j = 0; j < un; j += 4) {
+            uint32_t v = b.load(b.index(sB, b.iadd(b_base, b.ci(kk * PB + j))), 4);
+            for (int e = 0; e < 4; e++) bv.push_back(b.gep(v, e));
+        }
+        for (int i = 0; i < um; i++)
+            for (int j = 0; j < un; j++) b.store(acc[i * un + j], b.mulacc(av[i], bv[j], b.load(acc[i * un + j])));
+    }
+    b.barrier();
+    b.end({r});
+    uint32_t row0 = b.iadd(b.imul(gy, BM), b.imul(ly, um)), col0 = b.iadd(b.imul(gx, BN), b.imul(lx, un));
+    for (int i = 0; i < um; i++)
+        for (int j = 0; j < un; j += 4) {
+            std::vector<uint32_t> vals;
+            for (int e = 0; e < 4; e++) vals.push_back(b.load(acc[i * un + j + e]));
+            b.store(b.index(c, b.iadd(b.imul(b.iadd(row0, b.ci(i)), N), b.iadd(col0, b.ci(j)))), b.vectorize(vals));
+        }
+    return b.finish();
+}
+
 LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K, const MatmulF32Opts& o) {
+    if (o.lds_k) return build_matmul_f32_lds_kernel(M, N, K, o);
     KernelBuilder b;
     const Scalar f = Scalar::Float32;
     const int un = o.up_n, um = o.up_m;

@@ -200,6 +200,11 @@ struct MatmulF32Opts {
     int local_x = 16, local_y = 16;  // LOCAL
     int up_n = 4, up_m = 4;          // UPCAST
     int unroll_k = 1;                // UNROLL
+    // GROUP through local memory (schedule/src/optimizer/heuristics.rs:37-82, transforms.rs:1085-1089):
+    // 0 = operands straight from global memory; 8 / 16 / 32 = the workgroup stages A and B tiles
+    // of that depth in LDS (A transposed, so a work-item's rows are one vector), the next tiles'
+    // global loads issued before this tile's multiply-adds, two barriers per tile.
+    int lds_k = 0;
 };
 bool matmul_f32_opts_valid(const MatmulF32Opts& o, int64_t M, int64_t N, int64_t K);
 LinearKernel build_matmul_f32_kernel(int64_t M, int64_t N, int64_t K, const MatmulF32Opts& o);

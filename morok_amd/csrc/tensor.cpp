@@ -1583,7 +1583,17 @@ struct Scheduler {
             } else {
                 // MOROK_BEAM=<width> selects the LOCAL/UPCAST/UNROLL choices by timed search
                 // (cached on disk) instead of the fixed heuristic (tensor/src/realize.rs:1160-1250)
+                // fixed heuristic: the operand tiles go through local memory, with the largest of three
+                // workgroup tiles (128 x 128, 64 x 64, 64 rows x 32 columns) that still leaves at least
+                // 512 workgroups (two per compute unit), else the smallest that divides the shape;
+                // shapes none of them divides read their operands straight from global memory
                 MatmulF32Opts opts;
+                const MatmulF32Opts tiles[3] = {{32, 16, 4, 8, 1, 16}, {16, 16, 4, 4, 1, 16}, {8, 16, 4, 4, 1, 16}};
+                for (const MatmulF32Opts& c : tiles) {
+                    if (!matmul_f32_opts_valid(c, M, N, K)) continue;
+                    opts = c;
+                    if ((M / (c.local_y * c.up_m)) * (N / (c.local_x * c.up_n)) >= 512) break;
+                }
                 int beam = 0;
                 if (const char* e = std::getenv("MOROK_BEAM")) beam = std::atoi(e);
                 if (beam > 0) MRK_TRY(beam_search_matmul_f32(*dev, M, N, K, beam, &opts, nullptr, nullptr, nullptr));

@@ -113,8 +113,9 @@ def build_wmma_matmul_lds_opts(tc_index, m, n, k, out_scalar, opts):
 
 
 def build_matmul_f32_opts(m, n, k, opts):
-    """f32 matmul kernel with explicit (LOCAL x, LOCAL y, UPCAST n, UPCAST m, UNROLL k)."""
-    arr = (C.c_int * 5)(*opts)
+    """f32 matmul kernel with explicit (LOCAL x, LOCAL y, UPCAST n, UPCAST m, UNROLL k[, GROUP depth:
+    0 or the K depth of the tiles staged through local memory])."""
+    arr = (C.c_int * 6)(*(list(opts) + [0] * (6 - len(opts))))
     return _take(lib.mrk_hip_sched_build_matmul_f32_opts, m, n, k, arr)
 
 
@@ -142,7 +143,7 @@ def beam_cache_put(ast_hash, width, device, value):
 
 def beam_search_matmul_f32(m, n, k, width=2, device_id=0):
     """Returns (opts, best_ms, from_cache, candidates_timed)."""
-    opts = (C.c_int * 5)()
+    opts = (C.c_int * 6)()
     ms = C.c_double()
     cached, timed = C.c_int(), C.c_int()
     check(lib.mrk_hip_beam_search_matmul_f32(device_id, m, n, k, width, opts, C.byref(ms), C.byref(cached), C.byref(timed)))

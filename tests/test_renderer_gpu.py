@@ -314,3 +314,32 @@ def test_scheduled_matmul_f32_kernel(dev, oracle):
     b = synth.uniform((96, 192), 1, 6)
     c = run(dev, sched.build_matmul_f32(128, 192, 96), "r_mm", (128, 192), np.float32, [a, b])
     assert np.array_equal(c, oracle.matmul_f32(a, b))
+
+
+@pytest.mark.parametrize("opts", [[16, 16, 4, 4, 1, 16], [32, 16, 4, 8, 1, 16], [8, 16, 4, 4, 1, 16], [16, 16, 8, 8, 1, 8],
+                                  [16, 8, 4, 8, 1, 32]])
+def test_matmul_f32_staged_through_local_memory(dev, oracle, opts):
+    """GROUP: the workgroup stages A (transposed) and B tiles through local memory; every tile
+    choice computes the same sums in the same k order as the kernel that reads global memory
+    directly (bit-identical to it) and matches the CPU oracle within the f32 reduction tolerance."""
+    from morok_amd import sched
+
+    M, N, K = 256, 384, 160
+    a, b = synth.uniform((M, K), 55, 0), synth.uniform((K, N), 55, 1)
+    ba, bb = morok_amd.Buffer.from_numpy(a, dev.device_id), morok_amd.Buffer.from_numpy(b, dev.device_id)
+
+    def run_opts(o):
+        out = dev.buffer(M * N * 4 + 4096)
+        out.copyin(np.full(M * N + 1024, np.nan, np.float32))
+        k = morok_amd.Kernel.get_or_compile(sched.build_matmul_f32_opts(M, N, K, o), "mm_" + "_".join(map(str, o)))
+        plan = morok_amd.ExecutionPlan()
+        plan.add_kernel(k, [plan.add_buffer(out), plan.add_buffer(ba), plan.add_buffer(bb)])
+        plan.build().execute()
+        raw = out.copyout(np.float32)
+        assert np.all(np.isnan(raw[M * N:]))   # nothing written behind the result
+        return raw[: M * N].reshape(M, N)
+
+    got = run_opts(opts)
+    assert np.array_equal(got, run_opts([16, 16, 4, 4, 1, 0]))
+    ref = oracle.matmul_f32(a, b)
+    assert np.abs(got - ref).max() <= 1e-4 * np.abs(ref).max()
