@@ -677,6 +677,9 @@ struct KernelGen {
     // A cat that the kernel splits at its root: instead of evaluating every part and selecting,
     // the kernel runs one guarded region per part and this cat forwards to the part picked
     // (pick_part >= 0), or only reports its coordinate along the cat axis (pick_part == -2).
+    // Nodes whose value this kernel has computed itself and holds in a register, whatever the
+    // coordinates (a row's reduction inside the kernel that also consumes it).
+    std::map<const TensorNode*, uint32_t> fixed;
     const TensorNode* pick_cat = nullptr;
     int pick_part = -1;
     Cx probed_pos;
@@ -993,6 +996,8 @@ uint32_t emit_uncached(KernelGen& g, const TensorNode* n, const Coords& coords) 
 }
 
 uint32_t emit(KernelGen& g, const TensorNode* n, const Coords& coords) {
+    auto fx = g.fixed.find(n);
+    if (fx != g.fixed.end()) return fx->second;
     auto key = std::make_tuple(n, coords, g.gate);
     auto it = g.memo.find(key);
     if (it != g.memo.end()) return it->second;
@@ -1464,6 +1469,18 @@ struct Scheduler {
         std::vector<TensorNode*> deps;
         int64_t max_numel = 0;
         boundaries(n, n, seen, deps, &max_numel);
+        int64_t row_block = 0;
+        if (TensorNode* R = row_reduce_dep(n, deps, &row_block)) {
+            // everything either kernel half reads has to exist: the other inputs of the elementwise
+            // part and the inputs of the reduction's own expression
+            std::set<const TensorNode*> seen_r;
+            std::vector<TensorNode*> deps_r;
+            boundaries(R, R, seen_r, deps_r, &max_numel);
+            for (TensorNode* d : deps)
+                if (d != R) MRK_TRY(materialize(d));
+            for (TensorNode* d : deps_r) MRK_TRY(materialize(d));
+            return gen_row_fused(n, R, row_block, max_numel);
+        }
         for (TensorNode* d : deps) MRK_TRY(materialize(d));
         return n->kind == TKind::Reduce ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
     }
@@ -1683,6 +1700,118 @@ struct Scheduler {
         if (per_row > 0 && per_row % block == 0 && items % per_row == 0 && items / per_row > 1)
             return {items / per_row, per_row / block};
         return {(items + block - 1) / block};
+    }
+
+    // Row-resident fusion: an elementwise kernel whose one unrealised reduce input folds the last
+    // axis of a tensor of the output's own shape (keepdim), as rms_norm's x * rsqrt(mean(x^2) + eps)
+    // does.  One workgroup then owns a row: it folds the row (wave reduction + local memory),
+    // keeps the total in a register and produces the row's outputs from the values it already
+    // loaded, so the row is read once and the reduction needs no kernel and no buffer of its own.
+    // Returns the reduce node, or null when the shape does not fit (the two-kernel path remains).
+    TensorNode* row_reduce_dep(const TensorNode* n, const std::vector<TensorNode*>& deps, int64_t* block_out) const {
+        const char* off = std::getenv("MOROK_NO_ROW_FUSION");
+        if (off && off[0] && off[0] != '0') return nullptr;
+        if (n->kind == TKind::Reduce || n->shape.empty() || n->dtype == Scalar::Bool || n->numel() == 0) return nullptr;
+        TensorNode* R = nullptr;
+        for (TensorNode* d : deps) {
+            if (d->buffer || d->kind != TKind::Reduce) continue;
+            if (R) return nullptr;  // one reduction per kernel
+            R = d;
+        }
+        if (!R || R->src.size() != 1 || R->arg.size() != 1) return nullptr;
+        const TensorNode* src = R->src[0].get();
+        const int64_t last = static_cast<int64_t>(n->shape.size()) - 1;
+        if (src->shape != n->shape || R->arg[0] != last) return nullptr;
+        const ReduceOp op = static_cast<ReduceOp>(R->sub);
+        if (compute_dtype(R->dtype) != Scalar::Float32 || (op != ReduceOp::Add && op != ReduceOp::Max)) return nullptr;
+        auto u = uses.find(R);
+        if (u == uses.end() || u->second != 1) return nullptr;  // somebody else wants the reduction in memory
+        const int64_t C = n->shape.back(), rows = n->numel() / C;
+        int64_t width = 1;
+        for (int64_t w = 16 / static_cast<int64_t>(scalar_size(n->dtype)); w > 1; w /= 2)
+            if (C % w == 0) {
+                width = w;
+                break;
+            }
+        const int64_t V = C / width;
+        int64_t block = 0;
+        for (int64_t c : {256, 128, 64})
+            if (V % c == 0) {
+                block = c;
+                break;
+            }
+        // whole waves, at most 8 vectors per work-item (the row stays in registers), enough rows to fill the chip
+        if (!block || V / block > 8 || rows < 128) return nullptr;
+        *block_out = block;
+        return R;
+    }
+
+    int gen_row_fused(TensorNode* n, TensorNode* R, int64_t block, int64_t max_numel) {
+        const TensorNode* src = R->src[0].get();
+        const ReduceOp op = static_cast<ReduceOp>(R->sub);
+        const int64_t N = n->numel(), C = n->shape.back(), rows = N / C;
+        KernelGen g;
+        g.idx_t = max_numel >= (1LL << 31) ? Scalar::Int64 : Scalar::Int32;
+        KernelBuilder& b = g.b;
+        auto out = new_buffer(n);
+        uint32_t po = b.param(0, n->dtype, N);
+        int64_t width = 1;
+        for (int64_t w = 16 / static_cast<int64_t>(scalar_size(n->dtype)); w > 1; w /= 2)
+            if (C % w == 0) {
+                width = w;
+                break;
+            }
+        g.width = width;
+        const int64_t V = C / width, per_item = V / block, waves = block / 64;
+        uint32_t row = workgroup_index(b, g.idx_t, {rows});
+        if (!row) return last_status();
+        uint32_t lx = b.special("lidx0", block);
+        if (g.idx_t != Scalar::Int32) lx = b.cast(lx, g.idx_t);
+        // vector i of this work-item: lx + i * block, so that a wave reads consecutive 16-byte pieces
+        std::vector<uint32_t> base(per_item);
+        std::vector<Coords> coords(per_item);
+        for (int64_t i = 0; i < per_item; i++) {
+            base[i] = b.imul(b.iadd(b.iadd(b.imul(row, V), lx), g.ci(i * block)), width);
+            coords[i] = plain(unflatten(g, base[i], n->shape));
+            if (width > 1) coords[i].back().aligned = true;
+        }
+        // ---- the row's reduction: per work-item, per wave, then across the waves through local memory
+        uint32_t acc = 0;
+        for (int64_t i = 0; i < per_item; i++)
+            for (int64_t e = 0; e < width; e++) {
+                Coords ce = coords[i];
+                ce.back().off = e;
+                uint32_t v = emit(g, src, ce);
+                if (b.dtype(v).scalar != Scalar::Float32) v = b.cast(v, Scalar::Float32);
+                acc = acc ? b.binary(op == ReduceOp::Add ? BinaryOp::Add : BinaryOp::Max, acc, v) : v;
+            }
+        uint32_t total = b.wave_reduce(op, acc);
+        if (waves > 1) {
+            uint32_t lds = b.define_local(0, Scalar::Float32, waves);
+            uint32_t lane = b.imod(lx, 64), wave = b.idiv(lx, 64);
+            b.if_(b.binary(BinaryOp::Eq, lane, g.ci(0)));
+            b.store(b.index(lds, wave), total);
+            b.endif();
+            b.barrier();
+            total = b.load(b.index(lds, g.ci(0)));
+            for (int64_t w = 1; w < waves; w++)
+                total = b.binary(op == ReduceOp::Add ? BinaryOp::Add : BinaryOp::Max, total, b.load(b.index(lds, g.ci(w))));
+        }
+        g.fixed[R] = R->dtype != Scalar::Float32 ? b.cast(total, compute_dtype(R->dtype)) : total;
+        // ---- the row's outputs, from the loads the reduction already made
+        for (int64_t i = 0; i < per_item; i++) {
+            std::vector<uint32_t> vals;
+            for (int64_t e = 0; e < width; e++) {
+                Coords ce = coords[i];
+                ce.back().off = e;
+                uint32_t v = n->kind == TKind::Contiguous ? emit(g, n->src[0].get(), ce) : emit_uncached(g, n, ce);
+                if (b.dtype(v).scalar != n->dtype) v = b.cast(v, n->dtype);
+                vals.push_back(v);
+            }
+            if (width > 1) b.store(b.index(po, base[i]), b.vectorize(vals));
+            else b.store(b.index(po, base[i]), vals[0]);
+        }
+        return finish_kernel(g, n, out, "rE_" + std::to_string(rows) + "_g" + std::to_string(C) + (width > 1 ? "_" + std::to_string(width) : ""));
     }
 
     int gen_elementwise(TensorNode* n, int64_t max_numel) {

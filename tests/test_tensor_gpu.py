@@ -1122,3 +1122,38 @@ def test_grouped_reductions_match_float64(T, fusion, oracle, shape, axis, op):
         p = oracle.softmax_f32(x)
         e = np.exp(x - x.max(1, keepdims=True))
         np.testing.assert_allclose((T.Tensor.from_numpy(e).sum(1).to_numpy())[:, None] * p, e, rtol=2e-5, atol=1e-9)
+
+
+# ---------------------------------------------------------------- row-resident reduce + elementwise
+@pytest.mark.parametrize("rows,cols", [(256, 4096), (1000, 512), (128, 8192), (300, 1024), (130, 64 * 4)])
+def test_row_resident_norm_kernels(T, oracle, rows, cols, monkeypatch):
+    """rms_norm (and anything of its shape: an elementwise kernel fed by a keepdim reduction over the
+    last axis of its own input) runs as ONE kernel that folds a row and produces it from the same
+    loads.  Against the oracle's rms_norm, and against the two-kernel path, from which it differs only
+    in the order of the row sum."""
+    from morok_amd import synth, uop
+
+    x = synth.normal((rows, cols), 81, 0, sigma=1.5)
+    t = T.Tensor.from_numpy(x).rms_norm(-1, 1e-5)
+    got = t.to_numpy()
+    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("rE_"), t.kernels()
+    ref = oracle.rms_norm_f32(x, 1e-5)
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6)
+    monkeypatch.setenv("MOROK_NO_ROW_FUSION", "1")
+    t2 = T.Tensor.from_numpy(x).rms_norm(-1, 1e-5)
+    two = t2.to_numpy()
+    assert len(t2.kernels()) == 2
+    np.testing.assert_allclose(got, two, rtol=2e-6, atol=1e-7)
+    monkeypatch.delenv("MOROK_NO_ROW_FUSION")
+    # bf16 with a weight, as the decoder block uses it, against the oracle's bf16 stage
+    xb, wb = synth.normal_bf16((rows, cols), 82, 0), synth.to_bf16(1.0 + synth.normal((cols,), 82, 1, sigma=0.1))
+    tb = T.Tensor.from_numpy(xb, uop.BF16).rms_norm(-1, 1e-6).try_mul(T.Tensor.from_numpy(wb, uop.BF16)).cast(uop.BF16)
+    gb = tb.to_numpy()
+    assert len(tb.kernels()) == (1 if (cols // 8) % 64 == 0 else 2)   # whole waves of 16-byte vectors per row, or two kernels
+    rb = oracle.rms_norm_weight_bf16(xb, wb, 1e-6)
+    d = np.abs(gb.astype(np.int32) - rb.astype(np.int32))
+    assert d.max() <= 1 and np.count_nonzero(d) <= 0.01 * d.size      # a bf16 ulp where the f32 sums round apart
+    # a row maximum consumed by its own row: x - max(x)
+    m = T.Tensor.from_numpy(x)
+    sm = m.try_sub(m.max(1, keepdim=True))
+    assert np.array_equal(sm.to_numpy(), x - x.max(1, keepdims=True)) and len(sm.kernels()) == 1
