@@ -78,6 +78,7 @@ def _cpu_model():
 
 
 SETTLE_MS = 300.0  # untimed launches before the W warm-up steps, see _settle()
+REFERENCE_LEGS = True
 
 
 def _settle(m, fn):
@@ -228,24 +229,25 @@ def bench_gemm(m, dev, steps, warmup, cpu):
     ms, stats = _launch_stats(m, plan.execute, steps, warmup)
     flops = 2.0 * M * N * K
     tf = flops / (ms * 1e-3) / 1e12
-    # the same kernel called straight through the C ABI (no plan): shows what the plan costs
-    bc = dev.buffer(M * N * 2).ensure_allocated()
-    direct_ms, _ = _launch_stats(m, lambda: ops.gemm_bf16(ba, bb, bc, M, N, K), steps, warmup)
-    ceiling = _mfma_ceiling_tflops(m, dev)
     rec = {
         "metric": "bf16 GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "bf16",
         "config": {"workload": "bf16 GEMM M=N=K=4096, normal(0,1) inputs, f32 accumulate, bf16 out, via "
                                "Tensor::matmul -> prepare -> execute (configs[2])"},
-        "roofline": _roofline("gemm", "mfma", tf, BF16_PEAK_TFLOPS, "TFLOP/s", kernel, algorithmic_flops_per_launch=flops,
-                              mfma_only_ceiling=ceiling, frac_of_ceiling=tf / ceiling,
-                              mfma_only_ceiling_smooth_operands=_mfma_ceiling_tflops(m, dev, False)),
-        "plan_item": program, "direct_abi_ms_per_step": direct_ms,
+        "roofline": _roofline("gemm", "mfma", tf, BF16_PEAK_TFLOPS, "TFLOP/s", kernel, algorithmic_flops_per_launch=flops),
+        "plan_item": program,
     }
     rec.update(stats)
-    vendor = _vendor_gemm_tflops(M, steps, warmup)
-    if vendor is not None:
-        rec["vendor_reference"] = {"value": vendor, "unit": "TFLOP/s", "library": "torch.matmul (hipBLASLt), not on the "
-                                   "product path", "ratio": tf / vendor}
+    if REFERENCE_LEGS:
+        # the same kernel called straight through the C ABI (no plan): shows what the plan costs
+        bc = dev.buffer(M * N * 2).ensure_allocated()
+        rec["direct_abi_ms_per_step"], _ = _launch_stats(m, lambda: ops.gemm_bf16(ba, bb, bc, M, N, K), steps, warmup)
+        ceiling = _mfma_ceiling_tflops(m, dev)
+        rec["roofline"].update(mfma_only_ceiling=ceiling, frac_of_ceiling=tf / ceiling,
+                               mfma_only_ceiling_smooth_operands=_mfma_ceiling_tflops(m, dev, False))
+        vendor = _vendor_gemm_tflops(M, steps, warmup)
+        if vendor is not None:
+            rec["vendor_reference"] = {"value": vendor, "unit": "TFLOP/s", "library": "torch.matmul (hipBLASLt), not on the "
+                                       "product path", "ratio": tf / vendor}
     if cpu:
         rec["cpu_baseline"] = _gemm_cpu_baseline(M, N, K)
     return rec
@@ -488,10 +490,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="all", help="all | " + " | ".join(sorted(WORKLOADS)))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-reference-legs", action="store_true",
+                    help="skip the MFMA-only ceiling, the direct C-ABI leg and the vendor reference of the GEMM workload "
+                         "(profiler runs: only the measured kernel in the trace)")
     ap.add_argument("--settle-ms", type=float, default=SETTLE_MS,
                     help="untimed launches for this many ms before warm-up (0 for counter-collection runs)")
     args = ap.parse_args()
     globals()["SETTLE_MS"] = args.settle_ms
+    globals()["REFERENCE_LEGS"] = not args.no_reference_legs
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (every kernel shards into "
                  "independent units); run with --gpus 1")
