@@ -360,10 +360,13 @@ int mrk_hip_sched_build_wmma_matmul_lds(int tc_index, int64_t m, int64_t n, int6
                                         size_t* len);
 /* The same with the choices explicit: opts = {waves_m, waves_n (LOCAL: the grid of waves in a
  * workgroup), tiles_m, tiles_n (UPCAST: 16x16 tensor-core tiles per wave), K steps per barrier
- * pair (UNROLL; 0 = as many as divide K, up to 64 elements)}.  All powers of two;
- * INVALID_ARGUMENT for choices whose tiles do not split into whole 16-byte copies per work-item
- * or exceed local memory. */
-int mrk_hip_sched_build_wmma_matmul_lds_opts(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, const int opts[5],
+ * pair (UNROLL; 0 = as many as divide K, up to 64 elements), stages}.  stages = 0: tiles travel
+ * global -> registers -> local memory; stages = 2: two stages per tile filled by direct
+ * global -> local copies, B fragments through the transposing local load, one barrier per
+ * 64-deep K step, workgroups mapped to tiles per XCD (16x16x32 tensor cores; m, n, k must be
+ * multiples of the workgroup tile and of 64).  All powers of two; INVALID_ARGUMENT for choices
+ * whose tiles do not split into whole copies per work-item / wave or exceed local memory. */
+int mrk_hip_sched_build_wmma_matmul_lds_opts(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, const int opts[6],
                                              uint8_t** kernel, size_t* len);
 void mrk_hip_sched_free(void* p);
 /* The f32 matmul kernel with the optimisation choices explicit: opts = {LOCAL x, LOCAL y,
@@ -399,8 +402,8 @@ int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t 
 /* The same search over the LDS-staged tensor-core matmul of mrk_hip_sched_build_wmma_matmul_lds_opts
  * (bf16 / f16 in and out, tensor core `tc_index` of mrk_hip_sched_tensor_cores): the TC action
  * of tc.rs:358-674 first, then LOCAL / UPCAST / UNROLL as above.  opts = {waves_m, waves_n,
- * tiles_m per wave, tiles_n per wave, K steps per barrier pair}. */
-int mrk_hip_beam_search_wmma_matmul(int device_id, int tc_index, int64_t m, int64_t n, int64_t k, int width, int opts[5],
+ * tiles_m per wave, tiles_n per wave, K steps per barrier pair, stages}. */
+int mrk_hip_beam_search_wmma_matmul(int device_id, int tc_index, int64_t m, int64_t n, int64_t k, int width, int opts[6],
                                     double* best_ms, int* from_cache, int* timed);
 
 /* =====================================================================================

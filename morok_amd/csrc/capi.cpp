@@ -721,14 +721,14 @@ int mrk_hip_sched_build_wmma_matmul_lds(int tc_index, int64_t m, int64_t n, int6
     MRK_TRY(build_wmma_matmul_lds_kernel(tcs[tc_index], m, n, k, static_cast<Scalar>(out_scalar), WmmaLdsOpts(), &lk));
     return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
 }
-int mrk_hip_sched_build_wmma_matmul_lds_opts(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, const int opts[5],
+int mrk_hip_sched_build_wmma_matmul_lds_opts(int tc_index, int64_t m, int64_t n, int64_t k, int out_scalar, const int opts[6],
                                              uint8_t** kernel, size_t* len) {
     MRK_NONNULL(opts);
     MRK_NONNULL(kernel);
     MRK_NONNULL(len);
     auto tcs = cdna4_tensor_cores();
     if (tc_index < 0 || tc_index >= (int)tcs.size()) return fail(kInvalidArgument, "tc index out of range");
-    WmmaLdsOpts o{opts[0], opts[1], opts[2], opts[3], opts[4]};
+    WmmaLdsOpts o{opts[0], opts[1], opts[2], opts[3], opts[4], opts[5]};
     LinearKernel lk;
     MRK_TRY(build_wmma_matmul_lds_kernel(tcs[tc_index], m, n, k, static_cast<Scalar>(out_scalar), o, &lk));
     return export_kernel(lk, nullptr, reserialize(lk), kernel, len);
@@ -806,7 +806,7 @@ int mrk_hip_beam_search_matmul_f32(int device_id, int64_t m, int64_t n, int64_t 
     return kOk;
 }
 
-int mrk_hip_beam_search_wmma_matmul(int device_id, int tc_index, int64_t m, int64_t n, int64_t k, int width, int opts[5],
+int mrk_hip_beam_search_wmma_matmul(int device_id, int tc_index, int64_t m, int64_t n, int64_t k, int width, int opts[6],
                                     double* best_ms, int* from_cache, int* timed) {
     MRK_NONNULL(opts);
     std::shared_ptr<Device> d;
@@ -823,6 +823,7 @@ int mrk_hip_beam_search_wmma_matmul(int device_id, int tc_index, int64_t m, int6
     opts[2] = o.up_m;
     opts[3] = o.up_n;
     opts[4] = o.unroll_k;
+    opts[5] = o.stages;
     if (best_ms) *best_ms = ms;
     if (from_cache) *from_cache = cached ? 1 : 0;
     if (timed) *timed = n_timed;

@@ -86,7 +86,7 @@ int parse_linear_kernel(const uint8_t* data, size_t len, LinearKernel* out) {
         u.dtype.ptr_size = r.get<int64_t>();
         uint16_t nsrc = r.get<uint16_t>();
         if (!r.ok) break;
-        if (op > static_cast<uint16_t>(Op::WaveReduce))
+        if (op > static_cast<uint16_t>(Op::WaitAsync))
             return failf(kRenderError, "linearized kernel: unknown op tag %u at node %u", op, i);
         if (scalar > static_cast<uint8_t>(Scalar::Index))
             return failf(kRenderError, "linearized kernel: unknown scalar dtype %u at node %u", scalar, i);
@@ -557,6 +557,12 @@ class HipRenderer final : public Renderer {
             pre.push_back(def);
         }
         if (uses_wave_reduce) pre.push_back(kWaveReducePreamble);
+        for (const UOp& u : nodes)
+            if (u.op == Op::LoadTr) {
+                pre.push_back("typedef __bf16 mrk_tr_bf16x4 __attribute__((__vector_size__(4 * sizeof(__bf16))));\n"
+                              "typedef __fp16 mrk_tr_f16x4 __attribute__((__vector_size__(4 * sizeof(__fp16))));");
+                break;
+            }
 
         // ---- signature: buffers then variables (c/mod.rs:138-172)
         std::vector<std::string> params;
@@ -672,6 +678,27 @@ class HipRenderer final : public Renderer {
             if (it != min_use.end() && it->second < kv.second) out.insert(kv.first);
         }
         return out;
+    }
+
+    // the PARAM / DEFINE_LOCAL / DEFINE_REG a pointer expression is based on
+    template <class NodeFn>
+    static const UOp* base_buffer_of(uint32_t id, NodeFn& node) {
+        for (;;) {
+            const UOp& u = node(id);
+            switch (u.op) {
+                case Op::Param:
+                case Op::DefineLocal:
+                case Op::DefineReg: return &u;
+                case Op::Index:
+                case Op::Cast:
+                case Op::BitCast:
+                case Op::After:
+                    if (u.src.empty()) return nullptr;
+                    id = u.src[0];
+                    break;
+                default: return nullptr;
+            }
+        }
     }
 
     template <class NodeFn>
@@ -887,6 +914,36 @@ class HipRenderer final : public Renderer {
                 ctx.body.push_back(ctx.indent() + reduce_accumulate(static_cast<ReduceOp>(u.sub), acc, S(0), u.dtype));
                 return kOk;
             }
+            case Op::LoadTr: {
+                MRK_TRY(need(1));
+                const char* bi = u.dtype.scalar == Scalar::BFloat16 ? "__builtin_amdgcn_ds_read_tr16_b64_v4bf16"
+                                 : u.dtype.scalar == Scalar::Float16 ? "__builtin_amdgcn_ds_read_tr16_b64_v4f16"
+                                                                     : nullptr;
+                const UOp* base = base_buffer_of(u.src[0], node);
+                if (!bi || u.dtype.vcount != 4 || !base || base->op != Op::DefineLocal)
+                    return fail(kRenderError, "render: LOAD_TR reads 4 half / bfloat elements from local memory");
+                const char* vt = u.dtype.scalar == Scalar::BFloat16 ? "mrk_tr_bf16x4" : "mrk_tr_f16x4";
+                std::string call = fmt("%s((__attribute__((address_space(3))) %s*)(%s))", bi, vt, S(0).c_str());
+                ctx.emit(u, "__builtin_bit_cast(" + c_value_type(u.dtype) + ", " + call + ")", "tr", true);
+                return kOk;
+            }
+            case Op::AsyncCopy: {
+                MRK_TRY(need(2));
+                const UOp* g = base_buffer_of(u.src[0], node);
+                const UOp* l = base_buffer_of(u.src[1], node);
+                if (!g || g->op != Op::Param || !l || l->op != Op::DefineLocal)
+                    return fail(kRenderError, "render: ASYNC_COPY copies from a PARAM to a DEFINE_LOCAL");
+                // M0 holds the wave's local-memory destination; the copy itself is invisible to the
+                // compiler's wait-count bookkeeping, WAIT_ASYNC is its only ordering
+                ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, off\" : : \"s\"(" +
+                                   "__builtin_amdgcn_readfirstlane((unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + S(1) +
+                                   "))), \"v\"((const char*)(" + S(0) + ")) : \"m0\", \"memory\");");
+                return kOk;
+            }
+            case Op::WaitAsync:
+                if (u.arg_i < 0 || u.arg_i > 63) return fail(kRenderError, "render: WAIT_ASYNC takes a count of 0..63");
+                ctx.body.push_back(ctx.indent() + fmt("asm volatile(\"s_waitcnt vmcnt(%d)\" ::: \"memory\");", static_cast<int>(u.arg_i)));
+                return kOk;
             case Op::WaveReduce: {
                 MRK_TRY(need(1));
                 if (u.dtype.scalar != Scalar::Float32 || u.dtype.vcount != 1)

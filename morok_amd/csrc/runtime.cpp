@@ -570,14 +570,14 @@ int beam_search_wmma_matmul(const Device& dev, const TensorCore& tc, int tc_inde
     if (from_cache) *from_cache = false;
     if (candidates_timed) *candidates_timed = 0;
     struct Record {
-        int32_t opts[5];
+        int32_t opts[6];
         double ms;
     };
     std::vector<uint8_t> cached;
     if (BeamCache::get(ast_hash, width, device, &cached) && cached.size() == sizeof(Record)) {
         Record r;
         std::memcpy(&r, cached.data(), sizeof r);
-        WmmaLdsOpts o{r.opts[0], r.opts[1], r.opts[2], r.opts[3], r.opts[4]};
+        WmmaLdsOpts o{r.opts[0], r.opts[1], r.opts[2], r.opts[3], r.opts[4], r.opts[5]};
         if (wmma_lds_opts_valid(tc, o, M, N, K)) {
             *best = o;
             if (best_ms) *best_ms = r.ms;
@@ -600,7 +600,8 @@ int beam_search_wmma_matmul(const Device& dev, const TensorCore& tc, int tc_inde
 
     using Cand = std::pair<double, WmmaLdsOpts>;
     auto same = [](const WmmaLdsOpts& x, const WmmaLdsOpts& y) {
-        return x.waves_m == y.waves_m && x.waves_n == y.waves_n && x.up_m == y.up_m && x.up_n == y.up_n && x.unroll_k == y.unroll_k;
+        return x.waves_m == y.waves_m && x.waves_n == y.waves_n && x.up_m == y.up_m && x.up_n == y.up_n && x.unroll_k == y.unroll_k &&
+               x.stages == y.stages;
     };
     std::vector<WmmaLdsOpts> tried;
     double best_so_far = 1e300;
@@ -667,9 +668,32 @@ int beam_search_wmma_matmul(const Device& dev, const TensorCore& tc, int tc_inde
         beam = next;
         keep_best(beam);
     }
+    // stage 4: GROUP variant: the tiles filled by direct global -> local copies (two stages, one
+    // barrier per step, transposing B reads); its good shapes are few waves with large tiles,
+    // so they are tried outright beside the survivors' own shapes
+    {
+        std::vector<Cand> next = beam;
+        std::vector<WmmaLdsOpts> seeds;
+        for (const Cand& cnd : beam) seeds.push_back(cnd.second);
+        static const int shapes[][4] = {{2, 2, 8, 8}, {2, 2, 8, 4}, {2, 2, 4, 8}, {2, 4, 8, 4}, {4, 2, 4, 8}, {2, 2, 4, 4}, {2, 4, 4, 4},
+                                        {4, 4, 4, 4}, {1, 4, 8, 2}, {1, 4, 4, 2}, {2, 2, 2, 2}, {1, 4, 2, 1}};
+        for (auto& sh : shapes) {
+            WmmaLdsOpts o;
+            o.waves_m = sh[0], o.waves_n = sh[1], o.up_m = sh[2], o.up_n = sh[3];
+            seeds.push_back(o);
+        }
+        for (WmmaLdsOpts o : seeds) {
+            o.unroll_k = 0;
+            o.stages = 2;
+            double ms;
+            if (time_one(o, &ms)) next.emplace_back(ms, o);
+        }
+        beam = next;
+        keep_best(beam);
+    }
     *best = beam[0].second;
     if (best_ms) *best_ms = beam[0].first;
-    Record r{{best->waves_m, best->waves_n, best->up_m, best->up_n, best->unroll_k}, beam[0].first};
+    Record r{{best->waves_m, best->waves_n, best->up_m, best->up_n, best->unroll_k, best->stages}, beam[0].first};
     (void)BeamCache::put(ast_hash, width, device, &r, sizeof r);
     clear_error();
     return kOk;

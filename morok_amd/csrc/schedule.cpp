@@ -745,7 +745,13 @@ int build_wmma_matmul_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t
     return kOk;
 }
 
+static bool wmma_async_tile(const TensorCore& tc, const WmmaLdsOpts& o, int* bm, int* bn);
+
 bool wmma_lds_tile(const TensorCore& tc, const WmmaLdsOpts& o, int64_t K, int* bm, int* bn, int* bk) {
+    if (o.stages == 2) {
+        *bk = 64;
+        return wmma_async_tile(tc, o, bm, bn);
+    }
     const int tn = tc.dims[0], tm = tc.dims[1], tk = tc.dims[2];
     auto pow2_upto = [](int v, int hi) { return v >= 1 && v <= hi && (v & (v - 1)) == 0; };
     if (!pow2_upto(o.waves_m, 8) || !pow2_upto(o.waves_n, 8) || o.waves_m * o.waves_n > 16) return false;
@@ -762,7 +768,11 @@ bool wmma_lds_tile(const TensorCore& tc, const WmmaLdsOpts& o, int64_t K, int* b
     return true;
 }
 
+static bool wmma_async_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, int64_t N, int64_t K);
+
 bool wmma_lds_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, int64_t N, int64_t K) {
+    if (o.stages == 2) return wmma_async_opts_valid(tc, o, M, N, K);
+    if (o.stages != 0) return false;
     int BM, BN, BK;
     if (tc.threads != 64 || tc.dims[0] != 16 || tc.dims[1] != 16 || !wmma_lds_tile(tc, o, K, &BM, &BN, &BK)) return false;
     // extents that the tile does not divide are padded (PADTO); the 16-byte copies still need
@@ -776,8 +786,225 @@ bool wmma_lds_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, 
     return lds <= 80 * 1024;
 }
 
+// ---- stages = 2: direct global -> local copies, transposing B reads ------------------------
+// Layout of one stage.  A tile [BM][64]: rows of 128 bytes, the eight 16-byte pieces of row r
+// XOR-swizzled by (r >> 1) & 7, so the 16 rows a fragment read touches at one k lie in 16
+// different bank groups.  B tile [64][BN] as in global memory (n contiguous), its 32-byte
+// granules (16 columns) XOR-swizzled by k & 3, so the four k rows of a transposing read lie in
+// four different granules.  A copy instruction fills 1 KB of contiguous local memory from 64
+// per-lane sources; the swizzles are applied on the source side.
+static bool wmma_async_tile(const TensorCore& tc, const WmmaLdsOpts& o, int* bm, int* bn) {
+    auto pow2_upto = [](int v, int hi) { return v >= 1 && v <= hi && (v & (v - 1)) == 0; };
+    if (tc.threads != 64 || tc.dims[0] != 16 || tc.dims[1] != 16 || tc.dims[2] != 32) return false;
+    if (tc.dtype_in != Scalar::BFloat16 && tc.dtype_in != Scalar::Float16) return false;
+    if (!pow2_upto(o.waves_m, 8) || !pow2_upto(o.waves_n, 8) || o.waves_m * o.waves_n > 16) return false;
+    if (!pow2_upto(o.up_m, 8) || !pow2_upto(o.up_n, 8)) return false;
+    if (o.unroll_k != 0 && o.unroll_k != 2) return false;
+    *bm = o.waves_m * o.up_m * 16;
+    *bn = o.waves_n * o.up_n * 16;
+    return true;
+}
+
+static bool wmma_async_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, int64_t N, int64_t K) {
+    int BM, BN;
+    if (!wmma_async_tile(tc, o, &BM, &BN)) return false;
+    const int W = o.waves_m * o.waves_n;
+    if (M <= 0 || N <= 0 || K <= 0 || M % BM || N % BN || K % 64) return false;
+    if (M * K >= (1LL << 31) || K * N >= (1LL << 31) || M * N >= (1LL << 31)) return false;  // 32-bit element indices
+    if (BN < 64 || BN > 512) return false;              // whole granule groups per row, at most one row per copy
+    if ((BM / 8) % W || (BN / 8) % W) return false;     // every wave copies the same number of 1 KB chunks
+    if ((BM / 8 + BN / 8) / W > 32) return false;
+    if (2 * (BM + BN) * 64 * 2 > 160 * 1024) return false;  // two stages of both tiles in 160 KB
+    return true;
+}
+
+static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out,
+                                          const WmmaLdsOpts& opts, LinearKernel* k) {
+    int BM, BN;
+    if (!wmma_async_tile(tc, opts, &BM, &BN) || !wmma_async_opts_valid(tc, opts, M, N, K))
+        return failf(kInvalidArgument,
+                     "tensor-core matmul (direct copies): shape %lldx%lldx%lld does not divide into the workgroup tile with a K step of 64, "
+                     "or the tile does not fit two stages of local memory",
+                     (long long)M, (long long)N, (long long)K);
+    // the lane <-> element maps this builder writes out by hand; checked against the table
+    for (int l = 0; l < 64; l++)
+        for (int e = 0; e < 8; e++) {
+            int mn, kk;
+            for (int operand = 0; operand < 2; operand++) {
+                tc_operand_element(tc, operand, l, e, &mn, &kk);
+                if (mn != l % 16 || kk != 8 * (l / 16) + e) return fail(kInvalidArgument, "tensor-core matmul (direct copies): unexpected operand layout");
+            }
+            if (e < 4) {
+                int m, n;
+                tc_acc_element(tc, l, e, &m, &n);
+                if (m != 4 * (l / 16) + e || n != l % 16) return fail(kInvalidArgument, "tensor-core matmul (direct copies): unexpected accumulator layout");
+            }
+        }
+    const int um = opts.up_m, un = opts.up_n, WM = opts.waves_m, WN = opts.waves_n, W = WM * WN;
+    const int64_t KT = K / 64, tiles_m = M / BM, tiles_n = N / BN, T = tiles_m * tiles_n;
+    const int A_STAGE = BM * 64, B_STAGE = 64 * BN;  // elements
+    const int CA = BM / 8 / W, CB = BN / 8 / W, PRB = BN / 8;
+    KernelBuilder b;
+    b.enable_cse();
+    uint32_t c = b.param(0, out, M * N), a = b.param(1, tc.dtype_in, M * K), bmat = b.param(2, tc.dtype_in, K * N);
+    uint32_t bid = b.special("gidx0", T);
+    uint32_t lane = b.special("lidx0", 64), wave = b.special("lidx1", W);
+    auto bin = [&](BinaryOp op, uint32_t x, uint32_t y) { return b.binary(op, x, y); };
+    // workgroup -> tile: ids congruent mod 8 run on one XCD (one L2); give each XCD a contiguous
+    // range of tile ids, and walk tile ids in column groups of four tile rows
+    uint32_t id = bid;
+    if (T >= 8) {
+        const int64_t per = T / 8, rem = T % 8;
+        uint32_t xcd = b.imod(bid, 8), idx = b.idiv(bid, 8);
+        uint32_t extra = rem ? b.where(bin(BinaryOp::Lt, xcd, b.ci(rem)), xcd, b.ci(rem)) : b.ci(0);
+        id = b.iadd(b.iadd(b.imul(xcd, per), extra), idx);
+    }
+    uint32_t tm, tn;
+    {
+        const int64_t group = 4, group_sz = group * tiles_n;
+        uint32_t g = b.idiv(id, group_sz), first_m = b.imul(g, group), in = b.imod(id, group_sz);
+        if (tiles_m % group == 0) {
+            tm = b.iadd(first_m, b.imod(in, group));
+            tn = b.idiv(in, group);
+        } else {
+            uint32_t left = bin(BinaryOp::Sub, b.ci(tiles_m), first_m);
+            uint32_t gm = b.where(bin(BinaryOp::Lt, left, b.ci(group)), left, b.ci(group));
+            tm = b.iadd(first_m, bin(BinaryOp::Mod, in, gm));
+            tn = bin(BinaryOp::Idiv, in, gm);
+        }
+    }
+    uint32_t wy = b.idiv(wave, WN), wx = b.imod(wave, WN);
+    uint32_t l16 = b.imod(lane, 16), lg = b.idiv(lane, 16);
+    uint32_t sA = b.define_local(0, tc.dtype_in, 2LL * A_STAGE), sB = b.define_local(1, tc.dtype_in, 2LL * B_STAGE);
+
+    // copies: per wave CA chunks of A and CB chunks of B per tile
+    std::vector<uint32_t> a_src(CA), a_dst(CA), b_src(CB), b_dst(CB);
+    uint32_t a_tile0 = b.imul(tm, (int64_t)BM * K), b_tile0 = b.imul(tn, BN);
+    for (int q = 0; q < CA; q++) {
+        uint32_t chunk = b.iadd(b.imul(wave, CA), b.ci(q));
+        uint32_t row = b.iadd(b.imul(chunk, 8), b.idiv(lane, 8));
+        uint32_t sw = bin(BinaryOp::And, bin(BinaryOp::Shr, row, b.ci(1)), b.ci(7));
+        uint32_t piece = bin(BinaryOp::Xor, b.imod(lane, 8), sw);
+        a_src[q] = b.iadd(a_tile0, b.iadd(b.imul(row, K), b.imul(piece, 8)));
+        a_dst[q] = b.imul(chunk, 512);
+    }
+    for (int q = 0; q < CB; q++) {
+        uint32_t chunk = b.iadd(b.imul(wave, CB), b.ci(q));
+        uint32_t piece_id = b.iadd(b.imul(chunk, 64), lane);
+        uint32_t krow = b.idiv(piece_id, PRB), pp = b.imod(piece_id, PRB);
+        uint32_t gran = bin(BinaryOp::Xor, b.idiv(pp, 2), bin(BinaryOp::And, krow, b.ci(3)));
+        uint32_t col = b.imul(b.iadd(b.imul(gran, 2), b.imod(pp, 2)), 8);
+        b_src[q] = b.iadd(b_tile0, b.iadd(b.imul(krow, N), col));
+        b_dst[q] = b.imul(chunk, 512);
+    }
+    auto copy_tile = [&](uint32_t kt, uint32_t stage) {  // kt, stage: nodes (uniform)
+        uint32_t ka = b.imul(kt, 64), kb = b.imul(kt, 64 * N);
+        uint32_t oa = b.imul(stage, A_STAGE), ob = b.imul(stage, B_STAGE);
+        for (int q = 0; q < CA; q++) b.async_copy(b.index(a, b.iadd(a_src[q], ka)), b.index(sA, b.iadd(a_dst[q], oa)));
+        for (int q = 0; q < CB; q++) b.async_copy(b.index(bmat, b.iadd(b_src[q], kb)), b.index(sB, b.iadd(b_dst[q], ob)));
+    };
+    // fragment addresses: lane-dependent base per k step (A) / per column tile (B) + constants
+    uint32_t a_sw = b.idiv(l16, 2);
+    uint32_t a_row = b.iadd(b.imul(wy, um * 16), l16);
+    uint32_t a_base[2], b_base[8];
+    for (int kk = 0; kk < 2; kk++)
+        a_base[kk] = b.iadd(b.imul(a_row, 64), b.imul(bin(BinaryOp::Xor, b.iadd(lg, b.ci(kk * 4)), a_sw), 8));
+    uint32_t b_kq = b.idiv(l16, 4);
+    for (int j = 0; j < un; j++) {
+        uint32_t gran = bin(BinaryOp::Xor, b.iadd(b.imul(wx, un), b.ci(j)), b_kq);
+        b_base[j] = b.iadd(b.imul(b.iadd(b.imul(lg, 8), b_kq), BN), b.iadd(b.imul(gran, 16), b.imul(b.imod(l16, 4), 4)));
+    }
+    auto read_a = [&](int kk, int i, uint32_t oa) {
+        return b.load(b.index(sA, b.iadd(b.iadd(a_base[kk], oa), b.ci(i * 16 * 64))), 8);
+    };
+    auto read_b = [&](int kk, int j, uint32_t ob) {
+        uint32_t at = b.iadd(b_base[j], ob);
+        uint32_t lo = b.load_tr(b.index(sB, b.iadd(at, b.ci(kk * 32 * BN))));
+        uint32_t hi = b.load_tr(b.index(sB, b.iadd(at, b.ci((kk * 32 + 4) * BN))));
+        std::vector<uint32_t> el;
+        for (int e = 0; e < 4; e++) el.push_back(b.gep(lo, e));
+        for (int e = 0; e < 4; e++) el.push_back(b.gep(hi, e));
+        return b.vectorize(el);
+    };
+    // registers: accumulators (one object per tile) and the fragments of the first k step, which
+    // are read one half step ahead and so live across the loop edge
+    std::vector<uint32_t> acc(um * un), fa0(um), fb0(un);
+    int reg_id = 1;
+    {
+        std::vector<uint32_t> z(4, b.cf(0.0, tc.dtype_out));
+        uint32_t zv = b.vectorize(z);
+        for (int i = 0; i < um * un; i++) {
+            acc[i] = b.index(b.define_reg(reg_id++, tc.dtype_out, 1, 4), b.ci(0));
+            b.store(acc[i], zv);
+        }
+        for (int i = 0; i < um; i++) fa0[i] = b.index(b.define_reg(reg_id++, tc.dtype_in, 1, 8), b.ci(0));
+        for (int j = 0; j < un; j++) fb0[j] = b.index(b.define_reg(reg_id++, tc.dtype_in, 1, 8), b.ci(0));
+    }
+    const std::string name = wmma_name(tc);
+    const DType cd = KernelBuilder::scalar(tc.dtype_out, 4);
+    // the B fragment goes in as the first operand: the tensor core then leaves four consecutive
+    // columns of one row in a lane (result rows are written as vectors), same products, same order
+    auto mfmas = [&](const std::vector<uint32_t>& af, const std::vector<uint32_t>& bf) {
+        for (int i = 0; i < um; i++)
+            for (int j = 0; j < un; j++) {
+                uint32_t slot = acc[i * un + j];
+                b.store(slot, b.add(Op::Wmma, cd, {bf[j], af[i], b.load(slot)}, 0, 0, 0, name));
+            }
+    };
+    const int cpw = CA + CB;
+    copy_tile(b.ci(0), b.ci(0));
+    if (KT > 1) copy_tile(b.ci(1), b.ci(1));
+    b.wait_async(KT > 1 ? cpw : 0);
+    b.barrier();
+    for (int i = 0; i < um; i++) b.store(fa0[i], read_a(0, i, b.ci(0)));
+    for (int j = 0; j < un; j++) b.store(fb0[j], read_b(0, j, b.ci(0)));
+    uint32_t r = b.range(KT, 0, AxisType::Reduce);
+    {
+        uint32_t st = b.imod(r, 2), sn = bin(BinaryOp::Sub, b.ci(1), st);
+        uint32_t oa = b.imul(st, A_STAGE), ob = b.imul(st, B_STAGE), na = b.imul(sn, A_STAGE), nb = b.imul(sn, B_STAGE);
+        std::vector<uint32_t> f1a(um), f1b(un), f0a(um), f0b(un);
+        for (int i = 0; i < um; i++) f1a[i] = read_a(1, i, oa);
+        for (int j = 0; j < un; j++) f1b[j] = read_b(1, j, ob);
+        for (int i = 0; i < um; i++) f0a[i] = b.load(fa0[i]);
+        for (int j = 0; j < un; j++) f0b[j] = b.load(fb0[j]);
+        mfmas(f0a, f0b);
+        // tile r + 1 has landed in the other stage (issued half a step ago or earlier) and, behind
+        // the barrier, nobody reads this stage any more
+        b.wait_async(0);
+        b.barrier();
+        if (KT > 2) {
+            uint32_t r2 = b.iadd(r, b.ci(2));
+            b.if_(bin(BinaryOp::Lt, r2, b.ci(KT)));
+            copy_tile(r2, st);
+            b.endif();
+        }
+        // first half of tile r + 1 (after the last tile: a stale stage, read and never used)
+        for (int i = 0; i < um; i++) b.store(fa0[i], read_a(0, i, na));
+        for (int j = 0; j < un; j++) b.store(fb0[j], read_b(0, j, nb));
+        mfmas(f1a, f1b);
+    }
+    b.end({r});
+    uint32_t row0 = b.iadd(b.iadd(b.imul(tm, BM), b.imul(wy, um * 16)), l16);
+    uint32_t col0 = b.iadd(b.iadd(b.imul(tn, BN), b.imul(wx, un * 16)), b.imul(lg, 4));
+    for (int i = 0; i < um; i++)
+        for (int j = 0; j < un; j++) {
+            uint32_t res = b.load(acc[i * un + j]);
+            std::vector<uint32_t> el;
+            for (int e = 0; e < 4; e++) {
+                uint32_t v = b.gep(res, e);
+                el.push_back(out != tc.dtype_out ? b.cast(v, out) : v);
+            }
+            uint32_t at = b.iadd(b.imul(b.iadd(row0, b.ci(i * 16)), N), b.iadd(col0, b.ci(j * 16)));
+            b.store(b.index(c, at), b.vectorize(el));
+        }
+    *k = b.finish();
+    return kOk;
+}
+
 int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, const WmmaLdsOpts& opts,
                                  LinearKernel* k) {
+    if (opts.stages == 2) return build_wmma_matmul_async_kernel(tc, M, N, K, out, opts, k);
+    if (opts.stages != 0) return fail(kInvalidArgument, "tensor-core matmul (LDS): stages must be 0 (through registers) or 2 (direct copies)");
     const int tn = tc.dims[0], tm = tc.dims[1], tk = tc.dims[2];
     if (tc.threads != 64 || tm != 16 || tn != 16) return fail(kInvalidArgument, "tensor-core matmul (LDS): only 64-lane 16x16 tensor cores are lowered");
     int BM, BN, BK;

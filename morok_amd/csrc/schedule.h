@@ -160,6 +160,13 @@ class KernelBuilder {
     uint32_t wave_reduce(ReduceOp op, uint32_t v) { return add(Op::WaveReduce, dtype(v), {v}, 0, 0, static_cast<uint16_t>(op)); }
     uint32_t define_local(int id, Scalar s, int64_t size) { return add(Op::DefineLocal, pointer(s, size, AddrSpace::Local), {}, id); }
     uint32_t barrier() { return add(Op::Barrier, scalar(Scalar::Void)); }
+    // gfx950 local-memory extensions (uop.h): transposing 4-element load, direct global -> local
+    // copy of 16 bytes per lane, wait until at most n such copies of this wave are in flight
+    uint32_t load_tr(uint32_t local_index) { return add(Op::LoadTr, scalar(dtype(local_index).scalar, 4), {local_index}); }
+    uint32_t async_copy(uint32_t global_index, uint32_t local_index) {
+        return add(Op::AsyncCopy, scalar(Scalar::Void), {global_index, local_index});
+    }
+    uint32_t wait_async(int n) { return add(Op::WaitAsync, scalar(Scalar::Void), {}, n); }
     uint32_t define_reg(int id, Scalar s, int64_t size, int vcount = 1) {
         return add(Op::DefineReg, pointer(s, size, AddrSpace::Reg, vcount), {}, id);
     }
@@ -229,6 +236,12 @@ struct WmmaLdsOpts {
     int waves_m = 2, waves_n = 2;  // LOCAL
     int up_m = 4, up_n = 4;        // UPCAST: tensor-core tiles per wave
     int unroll_k = 0;              // UNROLL: tensor-core K steps per barrier pair; 0 = choose by K
+    // 0: tiles travel global -> registers -> local memory (above).  2: two stages of each tile in
+    // local memory filled by direct global -> local copies (ASYNC_COPY / WAIT_ASYNC), B fragments
+    // read with the transposing load (LOAD_TR), one barrier per 64-deep K step, workgroups
+    // mapped to tiles in compact blocks per XCD, result rows written as 8-byte vectors.  Needs a
+    // 16x16x32 tensor core, M, N, K divisible by the tile and a K step of 64.
+    int stages = 0;
 };
 // Extents of the workgroup tile these choices give (false if the choices are not buildable at all)
 bool wmma_lds_tile(const TensorCore& tc, const WmmaLdsOpts& o, int64_t K, int* bm, int* bn, int* bk);

@@ -1214,11 +1214,27 @@ struct Scheduler {
     // With the hand-written kernels switched off, a bf16 matmul whose shape fits still takes the
     // tensor-core route of the optimizer (schedule/src/optimizer/tc.rs:36-94): the generated
     // WMMA kernel staged through local memory instead of the generic reduce kernel.
-    // The fixed heuristic: the largest of a few workgroup tiles that gives every CU a workgroup
+    // The fixed heuristic for the register-staged variant (any shape whose N and K are multiples
+    // of 8): the largest of a few workgroup tiles that gives every CU a workgroup
     // (16 waves on 256 x 256 measured 1.05 PF at 4096^3 against 0.74 for 4 waves on 128 x 128)
     // and pads the output by at most an eighth; a shape too small for that takes the tile with
     // the least padding, the smaller one among equals.  MOROK_BEAM searches the whole space.
     static bool default_tc_opts(const TensorCore& tc, int64_t M, int64_t N, int64_t K, WmmaLdsOpts* o) {
+        // shapes that whole tiles and 64-deep K steps divide take the variant with direct
+        // global -> local copies (faster at every shape measured: 4096^3 1.26 against 1.08 PF,
+        // 2048^3 0.76 against 0.49, 1024^3 0.30 against 0.23): the largest tile that still fills
+        // the chip (one 256 x 256 workgroup or two smaller ones per CU), else the smallest
+        static const int direct[][5] = {{2, 4, 8, 4, 256}, {2, 2, 4, 4, 512}, {2, 2, 4, 2, 512}, {2, 2, 2, 2, 0}};
+        for (auto& c : direct) {
+            WmmaLdsOpts t{c[0], c[1], c[2], c[3], 0, 2};
+            if (!wmma_lds_opts_valid(tc, t, M, N, K)) continue;
+            int bm, bn, bk;
+            wmma_lds_tile(tc, t, K, &bm, &bn, &bk);
+            if ((M / bm) * (N / bn) >= c[4]) {
+                *o = t;
+                return true;
+            }
+        }
         static const int choices[][4] = {{4, 4, 4, 4}, {2, 2, 4, 4}, {2, 2, 2, 2}, {2, 2, 1, 1}, {1, 1, 1, 1}};
         bool found = false;
         int64_t least = 0;

@@ -50,6 +50,22 @@ enum class Op : uint16_t {
     // of src0 over the 64 lanes of a wavefront, sub = ReduceOp.  A host scheduler emits it
     // for a GROUP_REDUCE axis of extent 64 instead of the local-memory tree.
     WaveReduce = 27,
+    // Extensions for the gfx950 local-memory path of tensor-core kernels (not in the reference
+    // vocabulary; what the hand-written GEMM uses, made available to generated kernels).
+    // LoadTr: transposing load of 16-bit elements from local memory, src0 = Index into a
+    // DEFINE_LOCAL, dtype = vector of 4.  Within each group of 16 lanes, lane i addresses 4
+    // consecutive elements (row i / 4, columns 4 * (i % 4) .. + 3 of a 4 x 16 block); lane i
+    // receives column i of the block, rows 0..3.
+    LoadTr = 28,
+    // AsyncCopy: direct global -> local copy of 16 bytes per lane that bypasses registers,
+    // src0 = Index into a PARAM (per lane, 16-byte aligned), src1 = Index into a DEFINE_LOCAL
+    // that must be the same for all 64 lanes of a wavefront (its first lane is used): lane i's
+    // bytes land at that address + 16 * i.  Completion is not tracked by later loads: a WaitAsync
+    // followed by a Barrier makes the data visible to the workgroup.
+    AsyncCopy = 29,
+    // WaitAsync: blocks the wavefront until at most arg_i of its AsyncCopies are in flight
+    // (they complete in issue order).
+    WaitAsync = 30,
 };
 
 // dtype/src/lib.rs:129-154

@@ -107,8 +107,9 @@ def build_wmma_matmul_lds(tc_index, m, n, k, out_scalar):
 
 def build_wmma_matmul_lds_opts(tc_index, m, n, k, out_scalar, opts):
     """The same with explicit (waves_m, waves_n, tiles_m per wave, tiles_n per wave, K steps per
-    barrier pair; 0 = by K)."""
-    arr = (C.c_int * 5)(*opts)
+    barrier pair; 0 = by K[, stages: 0 = through registers, 2 = direct global -> local copies])."""
+    opts = list(opts) + [0] * (6 - len(opts))
+    arr = (C.c_int * 6)(*opts)
     return _take(lib.mrk_hip_sched_build_wmma_matmul_lds_opts, tc_index, m, n, k, out_scalar, arr)
 
 
@@ -153,7 +154,7 @@ def beam_search_matmul_f32(m, n, k, width=2, device_id=0):
 def beam_search_wmma_matmul(tc_index, m, n, k, width=2, device_id=0):
     """Beam search over the LDS-staged tensor-core matmul; returns (opts, best_ms, from_cache,
     candidates_timed) with opts as build_wmma_matmul_lds_opts takes them."""
-    opts = (C.c_int * 5)()
+    opts = (C.c_int * 6)()
     ms = C.c_double()
     cached, timed = C.c_int(), C.c_int()
     check(lib.mrk_hip_beam_search_wmma_matmul(device_id, tc_index, m, n, k, width, opts, C.byref(ms), C.byref(cached),

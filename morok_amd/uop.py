@@ -14,7 +14,8 @@ from .device import ProgramSpec
 
 # ---- enums (must match morok_amd/csrc/uop.h)
 (PARAM, DEFINE_VAR, DEFINE_LOCAL, DEFINE_REG, CONST, SPECIAL, RANGE, END, INDEX, LOAD, STORE, UNARY, BINARY, WHERE,
- MULACC, CAST, BITCAST, GEP, VECTORIZE, WMMA, IF, ENDIF, BARRIER, AFTER, NOOP, SINK, REDUCE, WAVE_REDUCE) = range(28)
+ MULACC, CAST, BITCAST, GEP, VECTORIZE, WMMA, IF, ENDIF, BARRIER, AFTER, NOOP, SINK, REDUCE, WAVE_REDUCE, LOAD_TR, ASYNC_COPY,
+ WAIT_ASYNC) = range(31)
 
 (BOOL, I8, U8, I16, U16, I32, U32, I64, U64, F16, BF16, F32, F64, VOID, INDEX_T) = range(15)
 GLOBAL, LOCAL, REG = 0, 1, 2
@@ -160,6 +161,19 @@ class Kernel:
 
     def wave_reduce(self, op, value):
         return self._add(WAVE_REDUCE, self.dtypes[value], src=(value,), sub=REDUCE_OPS[op])
+
+    def load_tr(self, local_index):
+        """Transposing load of four 16-bit elements from local memory (extension op LOAD_TR)."""
+        return self._add(LOAD_TR, DT(self.dtypes[local_index].scalar, 4), src=(local_index,))
+
+    def async_copy(self, global_index, local_index):
+        """Direct global -> local copy of 16 bytes per lane; the local index must be the same for the
+        64 lanes of a wave, lane i lands 16 * i bytes behind it (extension op ASYNC_COPY)."""
+        return self._add(ASYNC_COPY, DT(VOID), src=(global_index, local_index))
+
+    def wait_async(self, n):
+        """Waits until at most n of the wave's async copies are in flight (extension op WAIT_ASYNC)."""
+        return self._add(WAIT_ASYNC, DT(VOID), arg_i=n)
 
     def after(self, x, *deps):
         return self._add(AFTER, self.dtypes[x], src=(x,) + deps)

@@ -215,6 +215,28 @@ def wave_row_sum(rows, cols):
     return k
 
 
+def async_copy_transposing_load():
+    """One wave: a 1 KB ASYNC_COPY of a [16][32] matrix of 16-bit elements into local memory (lane i
+    fetches elements 8i .. 8i + 7, which land 16 i bytes into the tile: the identity layout), then
+    every group of 16 lanes takes a 4 x 16 block (rows 4g .. 4g + 3, columns 0 .. 15) through
+    LOAD_TR and writes its four elements to out[lane][0..3] (extension ops ASYNC_COPY, WAIT_ASYNC,
+    LOAD_TR)."""
+    k = U.Kernel()
+    out = k.param(0, U.bf16, 256)
+    inp = k.param(1, U.bf16, 512)
+    lane = k.special("lidx0", 64)
+    tile = k.define_local(0, U.bf16, 512)
+    k.async_copy(k.index(inp, k.mul(lane, k.const(8))), k.index(tile, k.const(0)))
+    k.wait_async(0)
+    k.barrier()
+    i16, g = k.binary("mod", lane, k.const(16)), k.binary("idiv", lane, k.const(16))
+    row = k.add(k.mul(g, k.const(4)), k.binary("idiv", i16, k.const(4)))
+    at = k.add(k.mul(row, k.const(32)), k.mul(k.binary("mod", i16, k.const(4)), k.const(4)))
+    v = k.load_tr(k.index(tile, at))
+    k.store(k.index(out, k.mul(lane, k.const(4))), v)
+    return k
+
+
 def local_memory_transpose(n):
     """n x n tile transposed through LDS with a barrier (DEFINE_LOCAL + BARRIER)."""
     k = U.Kernel()

@@ -101,6 +101,27 @@ def test_wmma_lowers_to_mfma():
     assert "no gfx950 MFMA lowering" in e.value.message
 
 
+def test_local_memory_extension_ops_render():
+    spec = U.render(KL.async_copy_transposing_load(), "tr")
+    assert "global_load_lds_dwordx4" in spec.src and "s_mov_b32 m0" in spec.src and "readfirstlane" in spec.src
+    assert 's_waitcnt vmcnt(0)' in spec.src
+    assert "__builtin_amdgcn_ds_read_tr16_b64_v4bf16(" in spec.src
+    morok_amd.compile_spec(spec)
+    # a transposing load reads local memory, a direct copy goes from a PARAM to local memory
+    k = U.Kernel()
+    out = k.param(0, U.bf16, 256)
+    inp = k.param(1, U.bf16, 512)
+    k.store(k.index(out, k.const(0)), k.load_tr(k.index(inp, k.const(0))))
+    with pytest.raises(morok_amd.MorokHipError):
+        U.render(k, "bad_tr")
+    k = U.Kernel()
+    out = k.param(0, U.bf16, 256)
+    inp = k.param(1, U.bf16, 512)
+    k.async_copy(k.index(inp, k.const(0)), k.index(out, k.const(0)))
+    with pytest.raises(morok_amd.MorokHipError):
+        U.render(k, "bad_copy")
+
+
 def test_wave_reduce_uses_dpp():
     spec = U.render(KL.wave_row_sum(8, 256), "wr")
     assert "__builtin_amdgcn_update_dpp" in spec.src and "__builtin_amdgcn_ds_swizzle" in spec.src

@@ -173,6 +173,18 @@ def test_wave_reduce_row_sum(dev):
     assert np.all(run(dev, KL.wave_row_sum(rows, cols), "r_wave", (rows,), np.float32, [ones]) == cols)
 
 
+def test_async_copy_and_transposing_load(dev):
+    """The documented lane maps of the local-memory extension ops: a direct copy lays lane i's 16
+    bytes 16 i bytes into the destination, and within a group of 16 lanes a transposing load hands
+    lane i column i of the 4 x 16 block whose row i / 4, columns 4 (i % 4) .. + 3 it addressed."""
+    x = (np.arange(512, dtype=np.uint16) * 7 + 3).astype(np.uint16)
+    y = run(dev, KL.async_copy_transposing_load(), "tr", (64, 4), np.uint16, [x])
+    m = x.reshape(16, 32)
+    lanes = np.arange(64)
+    want = np.stack([m[4 * (lanes // 16) + e, lanes % 16] for e in range(4)], axis=1)
+    assert np.array_equal(y, want)
+
+
 def test_local_memory_transpose(dev):
     n = 16
     x = synth.normal((n, n), 27, 0)
@@ -271,6 +283,48 @@ def test_tc_matmul_lds_choices_agree(dev, opts):
     a1[np.arange(M), (np.arange(M) * 7) % K] = 1
     c1 = run(dev, kern, "r_tc_lds", (M, N), np.uint16, [synth.to_bf16(a1), b])
     assert np.array_equal(c1, b[(np.arange(M) * 7) % K])
+
+
+@pytest.mark.parametrize("shape,opts", [((512, 512, 256), (2, 2, 2, 2, 0, 2)), ((256, 384, 64), (2, 2, 4, 4, 0, 2)),
+                                        ((128, 192, 128), (1, 4, 4, 1, 0, 2)), ((512, 512, 192), (4, 4, 4, 4, 0, 2)),
+                                        ((512, 256, 320), (2, 2, 8, 8, 0, 2)), ((256, 512, 256), (2, 4, 8, 4, 0, 2)),
+                                        ((192, 128, 448), (1, 1, 4, 4, 0, 2)), ((768, 256, 128), (2, 2, 8, 4, 2, 2)),
+                                        ((256, 1024, 128), (4, 2, 4, 8, 0, 2)), ((1536, 768, 64), (2, 2, 8, 8, 0, 2))])
+def test_tc_matmul_direct_copy_choices_agree(dev, shape, opts):
+    """The variant whose tiles arrive by direct global -> local copies (two stages, transposing B
+    reads, operands swapped at the tensor core, tiles assigned per XCD) computes the same products
+    in the same K order as the register-only generated kernel: same bits, one-hot operands come
+    back exactly, and nothing outside the operands is read or outside the result written (NaN
+    patterns behind each of them would surface).  K steps of 1, 2, 3 and more cover the prologue,
+    the last copy and the steady state; tile counts that 8 and 4 do not divide cover the mapping."""
+    from morok_amd import sched
+
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 9, 41)
+    b = synth.normal_bf16((K, N), 9, 42)
+    kern = sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts)
+    nan = np.uint16(0x7FC0)
+
+    def fenced(x):
+        big = np.full(x.size + 4096, nan, np.uint16)
+        big[:x.size] = x.ravel()
+        return morok_amd.Buffer.from_numpy(big)
+
+    def run_fenced(av):
+        bc = morok_amd.Buffer.from_numpy(np.full(M * N + 4096, nan, np.uint16))
+        k = morok_amd.Kernel.get_or_compile(kern, "r_tc_dma")
+        plan = morok_amd.ExecutionPlan()
+        plan.add_kernel(k, [plan.add_buffer(bc), plan.add_buffer(fenced(av)), plan.add_buffer(fenced(b))])
+        plan.build().execute()
+        got = bc.copyout(np.uint16, (M * N + 4096,))
+        assert np.all(got[M * N:] == nan)
+        return got[:M * N].reshape(M, N)
+
+    plain = run(dev, sched.build_wmma_matmul(1, M, N, K, U.BF16), "r_tc", (M, N), np.uint16, [a, b])
+    assert np.array_equal(run_fenced(a), plain)
+    a1 = np.zeros((M, K), np.float32)
+    a1[np.arange(M), (np.arange(M) * 7) % K] = 1
+    assert np.array_equal(run_fenced(synth.to_bf16(a1)), b[(np.arange(M) * 7) % K])
 
 
 @pytest.mark.parametrize("shape,opts", [((200, 136, 72), (2, 2, 4, 4, 0)), ((1, 8, 8), (1, 1, 1, 1, 0)), ((130, 264, 200), (2, 2, 2, 2, 2)),

@@ -195,6 +195,53 @@ def test_wmma_matmul_lds_kernel_refuses_bad_choices(opts):
         sched.build_wmma_matmul_lds_opts(1, 256, 128, 64, U.BF16, opts)
 
 
+def test_wmma_matmul_direct_copy_kernel_builds_and_compiles():
+    """stages = 2: both tiles in two stages of local memory filled by direct global -> local copies
+    (extension ops ASYNC_COPY / WAIT_ASYNC), B fragments through the transposing load (LOAD_TR),
+    one barrier per 64-deep K step plus the one that opens the loop, a flat grid whose workgroups
+    are mapped to tiles per XCD, and 8-byte vector stores of result rows."""
+    import morok_amd
+    from morok_amd import sched, uop as U
+
+    M, N, K = 1024, 512, 256
+    spec = U.render(sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, (2, 4, 8, 4, 0, 2)), "r_tc_dma")
+    src = spec.src
+    assert spec.sizes() == ([8, 1, 1], [64, 8, 1])                       # 4 x 2 tiles of 256 x 256, 8 waves
+    assert "__shared__ __bf16 local0[32768];" in src and "__shared__ __bf16 local1[32768];" in src   # 2 stages x 256 x 64 each
+    copies_per_wave = (256 // 8 + 256 // 8) // 8
+    assert src.count("global_load_lds_dwordx4") == 3 * copies_per_wave    # tiles 0 and 1 up front, tile r + 2 in the loop
+    assert src.count("__syncthreads();") == 2
+    assert 's_waitcnt vmcnt(%d)' % copies_per_wave in src and src.count("s_waitcnt vmcnt(0)") == 1
+    assert src.count("__builtin_amdgcn_ds_read_tr16_b64_v4bf16(") == 3 * 2 * 4   # 4 column tiles x (lo, hi) x (first half ahead, second, first)
+    assert src.count("__WMMA_16_16_32_bfloat_float(") == 2 * 32 + 1
+    assert "*((mrk_bhalf4*)((data0 +" in src                               # result rows as vectors of four
+    assert "gidx0 % 8" in src                                              # the XCD regrouping
+    morok_amd.compile_spec(spec)
+    # a single K step has no loop-carried copies; half precision takes the f16 transposing load
+    one = U.render(sched.build_wmma_matmul_lds_opts(1, 128, 128, 64, U.BF16, (2, 2, 4, 4, 0, 2)), "r_tc_dma1")
+    assert one.src.count("global_load_lds_dwordx4") == (128 // 8 + 128 // 8) // 4 and "s_waitcnt vmcnt(0)" in one.src
+    morok_amd.compile_spec(one)
+    half = U.render(sched.build_wmma_matmul_lds_opts(0, 128, 128, 128, U.F16, (2, 2, 4, 4, 0, 2)), "r_tc_dma_h")
+    assert "__builtin_amdgcn_ds_read_tr16_b64_v4f16(" in half.src
+    morok_amd.compile_spec(half)
+
+
+def test_tc_matmul_direct_copy_refuses_what_it_cannot_tile():
+    import morok_amd
+    from morok_amd import sched, uop as U
+
+    for shape, opts in (((500, 512, 256), (2, 2, 2, 2, 0, 2)),     # M is not a multiple of the tile
+                        ((512, 512, 200), (2, 2, 2, 2, 0, 2)),     # K is not a multiple of 64
+                        ((512, 512, 256), (2, 2, 2, 2, 1, 2)),     # the K step is 64 deep
+                        ((512, 512, 256), (1, 1, 2, 2, 0, 2)),     # 32 columns: no whole granule group
+                        ((1024, 1024, 256), (4, 4, 8, 8, 0, 2)),   # two stages of 512 x 512 exceed local memory
+                        ((512, 512, 256), (2, 2, 2, 2, 0, 3))):    # no such variant
+        with pytest.raises(morok_amd.MorokHipError):
+            sched.build_wmma_matmul_lds_opts(1, *shape, U.BF16, opts)
+    with pytest.raises(morok_amd.MorokHipError):
+        sched.build_wmma_matmul_lds_opts(3, 512, 512, 256, U.BF16, (2, 2, 2, 2, 0, 2))   # a 16x16x16 tensor core
+
+
 def test_global_index_order_modes_and_where_they_differ():
     """reverse=1 (dims reversed before limiting, indices after: what generated kernels launch) against
     reverse=2 (the literal code of schedule/src/gpudims.rs:331-382: only the index list is reversed).
