@@ -628,6 +628,14 @@ double mrk_hip_tensor_last_elapsed_ms(void);
  * Intermediates share blocks by liveness; MOROK_NO_MEMORY_PLANNER=1 turns that off. */
 size_t mrk_hip_tensor_last_buffers_reused(void);
 size_t mrk_hip_tensor_last_memory_saved(void);
+/* With MOROK_BEAM=<width> in the environment, realize / prepare searches the choices of every
+ * generated elementwise and reduce kernel of at least 65536 elements of work as well
+ * (tensor/src/realize.rs:1190-1242, schedule/src/optimizer/beam.rs:36-120): UPCAST then LOCAL for
+ * elementwise kernels, GROUP / split then LOCAL for wave reductions; winners are cached on disk
+ * (mrk_hip_beam_cache_*).  Candidates compiled and timed, and kernels answered by the cache,
+ * in the last realize / prepare on this thread. */
+size_t mrk_hip_tensor_last_beam_candidates(void);
+size_t mrk_hip_tensor_last_beam_cache_hits(void);
 
 #ifdef __cplusplus
 }

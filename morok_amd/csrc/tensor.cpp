@@ -1498,7 +1498,172 @@ struct Scheduler {
             return gen_row_fused(n, R, row_block, max_numel);
         }
         for (TensorNode* d : deps) MRK_TRY(materialize(d));
+        if (const char* e = std::getenv("MOROK_BEAM")) {
+            const int beam = std::atoi(e);
+            if (beam > 0 && !dry) return beam_generated(n, max_numel, beam);
+        }
         return n->kind == TKind::Reduce ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
+    }
+
+    // Beam search over the choices of one generated elementwise / reduce kernel
+    // (tensor/src/realize.rs:1190-1242, schedule/src/optimizer/beam.rs:36-120): every candidate is
+    // built as the real kernel would be, compiled and timed on buffers of the real sizes (inputs
+    // that already hold data are read in place, everything else is zero-filled scratch), staged
+    // like the matmul searches: UPCAST then LOCAL for an elementwise kernel, GROUP (waves per
+    // output and segments) then LOCAL (outputs per workgroup) for a wave reduction.  The winner
+    // is cached on disk under the hash of the kernel the fixed heuristics produce.
+    int beam_generated(TensorNode* n, int64_t max_numel, int width) {
+        const bool red = n->kind == TKind::Reduce;
+        auto build = [&](const GenOpts& o, std::vector<DryKernel>* out) -> int {
+            dry = true;
+            gen_opts = o;
+            dry_kernels.clear();
+            const int rc = red ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
+            dry = false;
+            gen_opts = GenOpts();
+            *out = std::move(dry_kernels);
+            dry_kernels.clear();
+            return rc;
+        };
+        auto for_real = [&](const GenOpts& o) -> int {
+            gen_opts = o;
+            const int rc = red ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
+            gen_opts = GenOpts();
+            return rc;
+        };
+        std::vector<DryKernel> base;
+        MRK_TRY(build(GenOpts(), &base));
+        int64_t work = n->numel();
+        if (red) for (int64_t a : n->arg) work *= n->src[0]->shape[a];
+        if (base.empty() || work < (1 << 16)) return for_real(GenOpts());  // too small to be worth a search
+        uint64_t h = 1469598103934665603ull;
+        for (const DryKernel& d : base) h = (h ^ d.k.content_hash) * 1099511628211ull;
+        const std::string device = "HIP:" + std::to_string(dev->device_id);
+        struct Record {
+            int32_t opts[5];
+            double ms;
+        };
+        auto to_opts = [](const Record& r) {
+            GenOpts o;
+            o.upcast_bytes = r.opts[0], o.local = r.opts[1], o.group = r.opts[2], o.split = r.opts[3], o.outs = r.opts[4];
+            return o;
+        };
+        std::vector<uint8_t> cached;
+        if (BeamCache::get(h, width, device, &cached) && cached.size() == sizeof(Record)) {
+            Record r;
+            std::memcpy(&r, cached.data(), sizeof r);
+            const GenOpts o = to_opts(r);
+            std::vector<DryKernel> probe;
+            if (build(o, &probe) == kOk && !probe.empty()) {
+                stats.beam_cache_hits++;
+                return for_real(o);
+            }
+            clear_error();
+        }
+        double best_so_far = 1e300;
+        std::set<std::string> tried;
+        auto time_one = [&](const GenOpts& o, double* ms) -> bool {
+            std::vector<DryKernel> ks;
+            if (build(o, &ks) != kOk || ks.empty()) {
+                clear_error();
+                return false;
+            }
+            std::string sig;
+            for (const DryKernel& d : ks) sig += std::to_string(d.k.content_hash) + ":";
+            if (!tried.insert(sig).second) return false;  // the choice changed nothing
+            double total = 0;
+            for (const DryKernel& d : ks) {
+                std::vector<std::unique_ptr<Buffer>> scratch;
+                std::vector<void*> ptrs;
+                for (const auto& bp : d.bufs) {
+                    const Buffer* use = bp.get();
+                    if (!bp->is_allocated() || bp.get() == d.bufs[0].get()) {
+                        BufferOptions bo;
+                        bo.zero_init = true;
+                        scratch.push_back(std::make_unique<Buffer>(dev->allocator, bp->size(), bo));
+                        if (scratch.back()->ensure_allocated() != kOk) return false;
+                        use = scratch.back().get();
+                    }
+                    void* ptr = nullptr;
+                    if (use->as_raw_ptr(&ptr) != kOk) return false;
+                    ptrs.push_back(ptr);
+                }
+                BenchmarkResult r;
+                bool skipped = false;
+                if (compile_and_time(*dev, d.k, "beam_candidate", ptrs.data(), ptrs.size(), nullptr, 0, 2, 5, &r,
+                                     best_so_far < 1e300 ? 3.0 * best_so_far : 0.0, &skipped) != kOk) {
+                    clear_error();
+                    return false;
+                }
+                if (skipped) return false;
+                total += r.min_ms;
+            }
+            stats.beam_candidates++;
+            *ms = total;
+            best_so_far = std::min(best_so_far, total);
+            return true;
+        };
+        using Cand = std::pair<double, GenOpts>;
+        auto keep_best = [&](std::vector<Cand>& v) {
+            std::sort(v.begin(), v.end(), [](const Cand& x, const Cand& y) { return x.first < y.first; });
+            if (static_cast<int>(v.size()) > width) v.resize(width);
+        };
+        std::vector<Cand> beam;
+        {
+            double ms;
+            if (!time_one(GenOpts(), &ms)) return for_real(GenOpts());
+            beam.emplace_back(ms, GenOpts());
+        }
+        if (!red) {
+            for (int up : {8, 4, 32}) {
+                GenOpts o;
+                o.upcast_bytes = up;
+                double ms;
+                if (time_one(o, &ms)) beam.emplace_back(ms, o);
+            }
+            keep_best(beam);
+            std::vector<Cand> next = beam;
+            for (const Cand& c : beam)
+                for (int local : {64, 128, 512, 1024}) {
+                    GenOpts o = c.second;
+                    o.local = local;
+                    double ms;
+                    if (time_one(o, &ms)) next.emplace_back(ms, o);
+                }
+            beam = next;
+            keep_best(beam);
+        } else {
+            int64_t R = 1;
+            for (int64_t a : n->arg) R *= n->src[0]->shape[a];
+            const int64_t Nout = n->numel();
+            for (int grp : {1, 2, 4, 8, 16})
+                for (int split : {1, 4, 16, 64, 256}) {
+                    if (R / split < 64LL * grp || Nout * split > (1LL << 22) || (split > 1 && R / split < 1024)) continue;
+                    GenOpts o;
+                    o.group = grp, o.split = split;
+                    double ms;
+                    if (time_one(o, &ms)) beam.emplace_back(ms, o);
+                }
+            keep_best(beam);
+            std::vector<Cand> next = beam;
+            for (const Cand& c : beam) {
+                if (c.second.group > 1) continue;  // a shared output owns its workgroup
+                for (int outs : {1, 2, 8, 16}) {
+                    GenOpts o = c.second;
+                    if (o.group == 0) o.group = 1, o.split = 0;
+                    o.outs = outs;
+                    double ms;
+                    if (time_one(o, &ms)) next.emplace_back(ms, o);
+                }
+            }
+            beam = next;
+            keep_best(beam);
+        }
+        const GenOpts& w = beam[0].second;
+        Record r{{w.upcast_bytes, w.local, w.group, w.split, w.outs}, beam[0].first};
+        (void)BeamCache::put(h, width, device, &r, sizeof r);  // a read-only cache directory is not an error
+        clear_error();
+        return for_real(w);
     }
 
     // A reshape / permute chain whose only source is a fusable attention node nobody else
@@ -1644,8 +1809,36 @@ struct Scheduler {
         return kOk;
     }
 
+    // Choices a search may make for a generated kernel in place of the fixed heuristics
+    // (the optimizer's actions on an elementwise / reduce kernel, schedule/src/optimizer/beam.rs:36-120);
+    // 0 leaves a choice to the heuristic.
+    struct GenOpts {
+        int upcast_bytes = 0;  // UPCAST: bytes of consecutive outputs per work-item (elementwise; heuristic 16)
+        int local = 0;         // LOCAL: work-items per workgroup (elementwise; heuristic 256)
+        int group = 0;         // GROUP: waves that share one output through local memory (wave reductions)
+        int split = 0;         // with group: segments per output folded by a second kernel (1 = none)
+        int outs = 0;          // LOCAL: outputs (one wave each) per workgroup when group == 1 (heuristic 4)
+    };
+    GenOpts gen_opts;
+    // dry run: kernels are built and collected here instead of being compiled and queued, and
+    // no node is marked as produced (a search builds every candidate this way)
+    struct DryKernel {
+        LinearKernel k;
+        std::vector<std::shared_ptr<Buffer>> bufs;
+    };
+    bool dry = false;
+    std::vector<DryKernel> dry_kernels;
+
     int queue_kernel(KernelGen& g, const std::shared_ptr<Buffer>& out, const std::string& name) {
         LinearKernel k = g.b.finish();
+        if (dry) {
+            DryKernel d;
+            d.k = std::move(k);
+            d.bufs.push_back(out);
+            d.bufs.insert(d.bufs.end(), g.inputs.begin(), g.inputs.end());
+            dry_kernels.push_back(std::move(d));
+            return kOk;
+        }
         std::shared_ptr<CachedKernel> ck;
         bool cached = false;
         MRK_TRY(get_or_compile_linear_kernel(*dev, k, name.c_str(), &ck, &cached));
@@ -1655,6 +1848,7 @@ struct Scheduler {
     }
     int finish_kernel(KernelGen& g, TensorNode* n, const std::shared_ptr<Buffer>& out, const std::string& name) {
         MRK_TRY(queue_kernel(g, out, name));
+        if (dry) return kOk;
         n->buffer = out;
         produced.push_back(n);
         return kOk;
@@ -1840,14 +2034,15 @@ struct Scheduler {
         // UPCAST of the innermost axis: one work-item produces `width` consecutive outputs
         // (16 bytes of them) when the axis divides evenly
         int64_t width = 1;
+        const int64_t up_bytes = gen_opts.upcast_bytes > 0 ? gen_opts.upcast_bytes : 16;
         if (!n->shape.empty() && n->dtype != Scalar::Bool)
-            for (int64_t w = 16 / static_cast<int64_t>(scalar_size(n->dtype)); w > 1; w /= 2)
+            for (int64_t w = up_bytes / static_cast<int64_t>(scalar_size(n->dtype)); w > 1; w /= 2)
                 if (n->shape.back() % w == 0) {
                     width = w;
                     break;
                 }
         g.width = width;
-        const int64_t items = N / width, block = 256;
+        const int64_t items = N / width, block = gen_opts.local > 0 ? gen_opts.local : 256;
         uint32_t gx = workgroup_index(b, g.idx_t, workgroup_axes(items, n->shape.empty() ? 0 : n->shape.back() / width, block));
         if (!gx) return last_status();
         uint32_t lx = b.special("lidx0", block);
@@ -1938,7 +2133,19 @@ struct Scheduler {
         KernelBuilder& b = g.b;
         auto out = new_buffer(n);
         const Scalar ct = compute_dtype(n->dtype);
-        const bool wave = R >= 128 && ct == Scalar::Float32 && (op == ReduceOp::Add || op == ReduceOp::Max);
+        // A reduction that keeps the innermost (contiguous) axis of its input - column sums, a fold
+        // over a middle axis - puts the lanes along that kept axis: a work-item per output walks
+        // the reduce range, so every load of a wave is one contiguous row piece.  (Lanes along the
+        // reduce range, as for row reductions, would stride the input by whole rows.)
+        const bool reduces_last = std::find(n->arg.begin(), n->arg.end(), static_cast<int64_t>(s->shape.size()) - 1) != n->arg.end();
+        const bool columns = !reduces_last && !s->shape.empty() && s->shape.back() >= 16;
+        const bool wave = R >= 128 && ct == Scalar::Float32 && (op == ReduceOp::Add || op == ReduceOp::Max) && !columns;
+        // ... and when that leaves too few work-items to fill the chip, the outermost reduce axis is
+        // cut into Pt segments (split_reduceop again): Pt times the work-items, partials laid out
+        // [segment][output] so both kernels stay coalesced
+        int64_t Pt = 1;
+        if (!wave && columns && R >= 128)
+            while (Pt * 2 * Nout <= (1 << 18) && rdims[0] % (Pt * 2) == 0 && R / (Pt * 2) >= 32) Pt *= 2;
         // Two-stage reduction (split_reduceop, schedule/src/rangeify/kernel.rs:44-61): when one
         // output folds at least 32768 inputs, the reduce range is cut into P segments (8 <= P <=
         // 256, partial buffer of at most 2^22 elements) reduced by P times as many waves, and
@@ -1976,34 +2183,39 @@ struct Scheduler {
                     break;
                 }
         }
+        if (wave && gen_opts.group > 0) {  // a search's explicit choice
+            G = gen_opts.group;
+            P = gen_opts.split > 0 ? gen_opts.split : 1;
+        }
         const int64_t chunk = (R + P - 1) / P;
         std::shared_ptr<Buffer> partial;
         if (P > 1) {
             BufferOptions bo;
             partial = std::make_shared<Buffer>(dev->allocator, static_cast<size_t>(Nout * P) * 4, bo);
         }
-        uint32_t po = P > 1 ? b.param(0, Scalar::Float32, Nout * P) : b.param(0, n->dtype, Nout);
+        uint32_t po = P > 1 ? b.param(0, Scalar::Float32, Nout * P) : Pt > 1 ? b.param(0, ct, Nout * Pt) : b.param(0, n->dtype, Nout);
         auto identity = [&]() -> uint32_t {
             if (is_float(ct)) return b.cf(op == ReduceOp::Add ? 0.0 : op == ReduceOp::Mul ? 1.0 : op == ReduceOp::Max ? -INFINITY : INFINITY, ct);
             return b.ci(op == ReduceOp::Mul ? 1 : 0, ct);
         };
         if (!wave) {
-            // one work-item per output element, the reduced axes as nested sequential loops
-            const int64_t block = 64;
-            uint32_t gx = workgroup_index(b, g.idx_t, workgroup_axes(Nout, n->shape.empty() ? 0 : n->shape.back(), block));
+            // one work-item per output element (per segment of one), the reduced axes as nested sequential loops
+            const int64_t block = 64, Wt = Nout * Pt, seg_len = rdims[0] / Pt;
+            uint32_t gx = workgroup_index(b, g.idx_t, workgroup_axes(Wt, Pt > 1 || n->shape.empty() ? 0 : n->shape.back(), block));
             if (!gx) return last_status();
             uint32_t lx = b.special("lidx0", block);
             if (g.idx_t != Scalar::Int32) lx = b.cast(lx, g.idx_t);
             uint32_t o = b.iadd(b.imul(gx, block), lx);
-            uint32_t gate = b.binary(BinaryOp::Lt, o, g.ci(Nout));
-            uint32_t oc = b.where(gate, o, g.ci(Nout - 1));  // clamp: masked lanes recompute the last element
-            Coords coords = plain(unflatten(g, oc, n->shape));
+            uint32_t gate = b.binary(BinaryOp::Lt, o, g.ci(Wt));
+            uint32_t oc = b.where(gate, o, g.ci(Wt - 1));  // clamp: masked lanes recompute the last element
+            uint32_t seg = Pt > 1 ? b.idiv(oc, Nout) : 0, oo = Pt > 1 ? b.imod(oc, Nout) : oc;
+            Coords coords = plain(unflatten(g, oo, n->shape));
             std::vector<uint32_t> ranges;
             for (size_t r = 0; r < n->arg.size(); r++) {
-                uint32_t rg = b.add(Op::Range, KernelBuilder::scalar(g.idx_t), {g.ci(rdims[r])}, static_cast<int64_t>(r), 0,
+                uint32_t rg = b.add(Op::Range, KernelBuilder::scalar(g.idx_t), {g.ci(r == 0 ? seg_len : rdims[r])}, static_cast<int64_t>(r), 0,
                                     static_cast<uint16_t>(AxisType::Reduce));
                 ranges.push_back(rg);
-                coords[n->arg[r]] = Cx{rg, 0, false};
+                coords[n->arg[r]] = Cx{r == 0 && Pt > 1 ? b.iadd(b.imul(seg, seg_len), rg) : rg, 0, false};
             }
             uint32_t v = emit(g, s, coords);
             uint32_t red = b.reduce(op, v, ranges);
@@ -2011,16 +2223,40 @@ struct Scheduler {
             b.end(rev);
             b.if_(gate);
             uint32_t res = red;
-            if (b.dtype(res).scalar != n->dtype) res = b.cast(res, n->dtype);
+            const Scalar store_t = Pt > 1 ? ct : n->dtype;
+            if (b.dtype(res).scalar != store_t) res = b.cast(res, store_t);
             b.store(b.index(po, o), res);
             b.endif();
-            return finish_kernel(g, n, out, "r_" + std::to_string(Nout) + "_" + std::to_string(R));
+            if (Pt == 1) return finish_kernel(g, n, out, "r_" + std::to_string(Nout) + "_" + std::to_string(R));
+            BufferOptions bo;
+            auto part = std::make_shared<Buffer>(dev->allocator, static_cast<size_t>(Wt) * scalar_size(ct), bo);
+            MRK_TRY(queue_kernel(g, part, "r_" + std::to_string(Nout) + "x" + std::to_string(Pt) + "_" + std::to_string(R / Pt)));
+            // second stage: a work-item per output folds its Pt partials, one coalesced row of them per step
+            KernelGen g2;
+            KernelBuilder& b2 = g2.b;
+            uint32_t po2 = b2.param(0, n->dtype, Nout);
+            uint32_t pin = g2.buffer_param(part, ct, Wt);
+            uint32_t gx2 = workgroup_index(b2, Scalar::Int32, workgroup_axes(Nout, 0, block));
+            if (!gx2) return last_status();
+            uint32_t o2 = b2.iadd(b2.imul(gx2, block), b2.special("lidx0", block));
+            uint32_t gate2 = b2.binary(BinaryOp::Lt, o2, b2.ci(Nout));
+            uint32_t oc2 = b2.where(gate2, o2, b2.ci(Nout - 1));
+            uint32_t r2 = b2.range(Pt, 0, AxisType::Reduce);
+            uint32_t pv = b2.load(b2.index(pin, b2.iadd(b2.imul(r2, Nout), oc2)));
+            uint32_t red2 = b2.reduce(op, pv, {r2});
+            b2.end({r2});
+            b2.if_(gate2);
+            uint32_t res2 = red2;
+            if (b2.dtype(res2).scalar != n->dtype) res2 = b2.cast(res2, n->dtype);
+            b2.store(b2.index(po2, o2), res2);
+            b2.endif();
+            return finish_kernel(g2, n, out, "r_" + std::to_string(Nout) + "_" + std::to_string(Pt));
         }
         // one wavefront per output element: lanes stride the flattened reduce space, partial
         // results are combined with the wave64 cross-lane reduction (the GROUP_REDUCE idea of
         // schedule/src/optimizer/heuristics.rs:370-392 without the LDS round trip)
         const int64_t W = Nout * P;  // wave-sized (G == 1) or workgroup-sized outputs of this kernel
-        const int64_t per_block = G > 1 ? 1 : 4;
+        const int64_t per_block = G > 1 ? 1 : gen_opts.outs > 0 ? gen_opts.outs : 4;
         uint32_t gx = workgroup_index(b, g.idx_t, workgroup_axes(W, 0, per_block));
         if (!gx) return last_status();
         uint32_t lane = b.special("lidx0", 64), ly = b.special("lidx1", G > 1 ? G : per_block);

@@ -51,6 +51,12 @@ def last_memory_plan():
     return lib.mrk_hip_tensor_last_buffers_reused(), lib.mrk_hip_tensor_last_memory_saved()
 
 
+def last_beam_search():
+    """(candidates compiled and timed, kernels answered by the disk cache) for the generated
+    elementwise / reduce kernels of the last realize / prepare under MOROK_BEAM."""
+    return lib.mrk_hip_tensor_last_beam_candidates(), lib.mrk_hip_tensor_last_beam_cache_hits()
+
+
 def last_elapsed_ms():
     return lib.mrk_hip_tensor_last_elapsed_ms()
 

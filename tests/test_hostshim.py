@@ -494,6 +494,41 @@ def test_compile_and_time_and_failing_candidates(dev, shim):
         sched.compile_and_time(b"not a kernel", bufs)
 
 
+def test_beam_search_over_generated_kernels(dev, shim, tmp_path, monkeypatch):
+    """MOROK_BEAM also searches the generated elementwise and reduce kernels: candidates are built
+    like the real kernel, compiled and timed; the winner is cached on disk under the hash of the
+    heuristic kernel, so a second realization of the same graph compiles and times nothing; small
+    kernels are left to the heuristics; the kernel list keeps its shape."""
+    from morok_amd import tensor as T
+
+    monkeypatch.setenv("MOROK_CACHE_DIR", str(tmp_path))
+    monkeypatch.delenv("IGNORE_BEAM_CACHE", raising=False)
+
+    def graph():
+        a = T.Tensor.from_numpy(np.ones((512, 1024), np.float32))
+        b = T.Tensor.from_numpy(np.ones((512, 1024), np.float32))
+        return a.try_add(b).try_exp().sum(-1)
+
+    graph().realize()
+    plain = T.last_kernels()
+    assert T.last_beam_search() == (0, 0)
+    monkeypatch.setenv("MOROK_BEAM", "2")
+    graph().realize()
+    timed, hits = T.last_beam_search()
+    assert timed >= 4 and hits == 0
+    assert len(T.last_kernels()) == len(plain)
+    graph().realize()
+    assert T.last_beam_search() == (0, 1)
+    # elementwise: UPCAST and LOCAL candidates; tiny kernels are not searched
+    big = T.Tensor.from_numpy(np.ones((256, 2048), np.float32))
+    big.try_mul(big).cast(uop.BF16).realize()
+    timed, hits = T.last_beam_search()
+    assert timed >= 6 and hits == 0 and T.last_kernels()[0].startswith("E_524288")
+    small = T.Tensor.from_numpy(np.ones((16, 16), np.float32))
+    small.try_mul(small).realize()
+    assert T.last_beam_search() == (0, 0)
+
+
 def test_beam_search_uses_and_fills_the_disk_cache(dev, shim, tmp_path, monkeypatch):
     from morok_amd import sched
 

@@ -1124,6 +1124,42 @@ def test_grouped_reductions_match_float64(T, fusion, oracle, shape, axis, op):
         np.testing.assert_allclose((T.Tensor.from_numpy(e).sum(1).to_numpy())[:, None] * p, e, rtol=2e-5, atol=1e-9)
 
 
+# ---------------------------------------------------------------- reductions that keep the contiguous axis
+@pytest.mark.parametrize("shape,axis,kernels", [((8192, 4096), 0, 2), ((4, 2048, 256), 1, 2), ((300, 1000), 0, 2), ((129, 64), 0, 1),
+                                                ((6, 500, 33, 16), 1, 2), ((2, 4096, 8, 64), (1, 2), 2), ((100, 4096), 0, 1)])
+@pytest.mark.parametrize("op", ["sum", "max"])
+def test_column_reductions(T, shape, axis, kernels, op):
+    """A fold that keeps the innermost axis (column sums, a fold over a middle axis) runs with the
+    lanes along the kept axis, and splits the outermost reduce axis over more work-items when the
+    outputs alone would not fill the chip (two kernels, partials as [segment][output])."""
+    from morok_amd import synth
+
+    x = synth.normal(shape, 33, len(shape)) + np.float32(0.25)
+    t = T.Tensor.from_numpy(x)
+    got = (t.sum(axis) if op == "sum" else t.max(axis)).to_numpy()
+    names = T.last_kernels()
+    assert len(names) == kernels                                     # an odd or short reduce axis is not split
+    assert not any("_g" in nm for nm in names)                       # no wave-per-output kernel
+    if op == "sum":
+        ref = x.astype(np.float64).sum(axis)
+        scale = np.abs(x.astype(np.float64)).sum(axis)
+        assert np.all(np.abs(got - ref) <= 1e-4 * np.maximum(np.abs(ref), 1e-3 * scale))
+    else:
+        assert np.array_equal(got, x.max(axis))
+
+
+def test_column_reduction_integers_and_bf16(T):
+    from morok_amd import synth, uop
+
+    xi = synth.randint((1024, 512), 34, 0, 1000).astype(np.int32) - 500
+    assert np.array_equal(T.Tensor.from_numpy(xi).sum(0).to_numpy(), xi.sum(0, dtype=np.int32))
+    assert len(T.last_kernels()) == 2
+    xb = synth.normal_bf16((512, 2048), 34, 1)
+    got = synth.from_bf16(T.Tensor.from_numpy(xb, uop.BF16).sum(0).to_numpy())
+    ref = synth.from_bf16(xb).astype(np.float64).sum(0)
+    assert np.all(np.abs(got - ref) <= 1e-2 * np.maximum(np.abs(ref), 1.0))   # one bf16 rounding of an f32 sum
+
+
 # ---------------------------------------------------------------- row-resident reduce + elementwise
 @pytest.mark.parametrize("rows,cols", [(256, 4096), (1000, 512), (128, 8192), (300, 1024), (130, 64 * 4)])
 def test_row_resident_norm_kernels(T, oracle, rows, cols, monkeypatch):
@@ -1157,3 +1193,46 @@ def test_row_resident_norm_kernels(T, oracle, rows, cols, monkeypatch):
     m = T.Tensor.from_numpy(x)
     sm = m.try_sub(m.max(1, keepdim=True))
     assert np.array_equal(sm.to_numpy(), x - x.max(1, keepdims=True)) and len(sm.kernels()) == 1
+
+
+def test_beam_search_over_generated_kernels_keeps_values(T, tmp_path, monkeypatch):
+    """Under MOROK_BEAM the choices of generated elementwise and reduce kernels are searched on the
+    device (candidates timed on scratch buffers of the real sizes); whatever wins, elementwise
+    results are the bits of the heuristic kernel and reductions stay within the reduction
+    tolerance of float64; the second realization takes its choices from the disk cache."""
+    from morok_amd import synth, uop
+
+    Tensor = T.Tensor
+    monkeypatch.setenv("MOROK_CACHE_DIR", str(tmp_path))
+    monkeypatch.delenv("IGNORE_BEAM_CACHE", raising=False)
+    x = synth.normal((768, 2048), 61, 0)
+    y = synth.normal((768, 2048), 61, 1)
+    idx = synth.randint((4096,), 61, 2, 768)
+
+    def graphs():
+        tx, ty = Tensor.from_numpy(x), Tensor.from_numpy(y)
+        e = tx.try_mul(ty).try_add(tx).cast(uop.BF16)                  # elementwise, bf16 out
+        r = tx.try_exp().sum(-1)                                        # 768 wave reductions
+        f = tx.try_reshape([3, 512 * 1024]).sum(-1)                     # few outputs, long folds
+        g = tx.embedding(Tensor.from_numpy(idx)).try_add(Tensor.from_numpy(y[:1]).try_expand([4096, 2048]))   # gather + broadcast
+        return e, r, f, g
+
+    monkeypatch.delenv("MOROK_BEAM", raising=False)
+    want = [t.to_numpy() for t in graphs()]
+    monkeypatch.setenv("MOROK_BEAM", "2")
+    timed_total = 0
+    got = []
+    for t in graphs():
+        got.append(t.to_numpy())
+        timed, hits = T.last_beam_search()
+        assert hits == 0
+        timed_total += timed
+    assert timed_total >= 20
+    assert np.array_equal(got[0], want[0]) and np.array_equal(got[3], want[3])
+    ref_r = np.exp(x.astype(np.float64)).sum(-1)
+    assert np.abs(got[1] - ref_r).max() <= 1e-4 * np.abs(ref_r).max()
+    ref_f = x.astype(np.float64).reshape(3, -1).sum(-1)
+    assert np.abs(got[2] - ref_f).max() <= 1e-4 * np.abs(x).astype(np.float64).reshape(3, -1).sum(-1).max()
+    for t, w in zip(graphs(), got):
+        assert np.array_equal(t.to_numpy(), w)                          # same choices, same bits
+        assert T.last_beam_search()[0] == 0 and T.last_beam_search()[1] >= 1
