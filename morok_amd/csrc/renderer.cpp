@@ -88,7 +88,7 @@ int parse_linear_kernel(const uint8_t* data, size_t len, LinearKernel* out) {
         if (!r.ok) break;
         if (op > static_cast<uint16_t>(Op::WaitAsync))
             return failf(kRenderError, "linearized kernel: unknown op tag %u at node %u", op, i);
-        if (scalar > static_cast<uint8_t>(Scalar::Index))
+        if (scalar > static_cast<uint8_t>(Scalar::Fp8E5M2))
             return failf(kRenderError, "linearized kernel: unknown scalar dtype %u at node %u", scalar, i);
         u.op = static_cast<Op>(op);
         u.dtype.scalar = static_cast<Scalar>(scalar);
@@ -131,6 +131,8 @@ const char* c_scalar(Scalar s) {  // codegen/src/c/types.rs:10-28
         case Scalar::UInt32: return "unsigned int";
         case Scalar::Int64:
         case Scalar::Index: return "long long";
+        case Scalar::Fp8E4M3:
+        case Scalar::Fp8E5M2: return "unsigned char";  // types.rs:26
         case Scalar::UInt64: return "unsigned long long";
         case Scalar::Float16: return "_Float16";
         case Scalar::BFloat16: return "__bf16";
@@ -151,6 +153,8 @@ const char* c_vector_base(Scalar s) {  // types.rs:31-49, prefixed to stay clear
         case Scalar::UInt32: return "mrk_uint";
         case Scalar::Int64:
         case Scalar::Index: return "mrk_llong";
+        case Scalar::Fp8E4M3: return "mrk_f8e4m3_";
+        case Scalar::Fp8E5M2: return "mrk_f8e5m2_";
         case Scalar::UInt64: return "mrk_ullong";
         case Scalar::Float16: return "mrk_half";
         case Scalar::BFloat16: return "mrk_bhalf";
@@ -164,6 +168,8 @@ size_t scalar_bytes(Scalar s) {
     switch (s) {
         case Scalar::Bool:
         case Scalar::Int8:
+        case Scalar::Fp8E4M3:
+        case Scalar::Fp8E5M2:
         case Scalar::UInt8: return 1;
         case Scalar::Int16:
         case Scalar::UInt16:
@@ -350,7 +356,27 @@ std::string reduce_accumulate(ReduceOp op, const std::string& acc, const std::st
 // names 677-688).  Operand sizes per lane follow the CDNA tables
 // (schedule/src/optimizer/renderer.rs:538-558): 16x16x32 -> A,B 8 elements, C 4;
 // 16x16x16 -> A,B 4 elements, C 4.
-bool wmma_wrapper(const std::string& name, std::string* def) {
+// The reference names both 8-bit float cores WMMA_16_16_32_unknown_float (its dtype-name table
+// has no entry for them); the operand dtype tells them apart: E4M3 -> ..._fp8_fp8, E5M2 ->
+// ..._bf8_bf8, eight bytes per lane handed over as one 64-bit integer.
+std::string wmma_callee(const std::string& name, Scalar operand) {
+    if (operand == Scalar::Fp8E4M3) return name + "_e4m3";
+    if (operand == Scalar::Fp8E5M2) return name + "_e5m2";
+    return name;
+}
+bool wmma_wrapper(const std::string& name, Scalar operand, std::string* def) {
+    if (operand == Scalar::Fp8E4M3 || operand == Scalar::Fp8E5M2) {
+        if (name != "WMMA_16_16_32_unknown_float") return false;
+        const std::string fn = wmma_callee(name, operand);
+        *def = fmt(
+            "typedef unsigned char __%s_in __attribute__((ext_vector_type(8)));\n"
+            "typedef float __%s_acc __attribute__((ext_vector_type(4)));\n"
+            "static __device__ __forceinline__ __%s_acc __%s(__%s_in a, __%s_in b, __%s_acc c) {\n"
+            "  return %s(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b), c, 0, 0, 0);\n}\n",
+            fn.c_str(), fn.c_str(), fn.c_str(), fn.c_str(), fn.c_str(), fn.c_str(), fn.c_str(),
+            operand == Scalar::Fp8E4M3 ? "__builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8" : "__builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8");
+        return true;
+    }
     struct Entry {
         const char* name;
         const char* builtin;
@@ -536,11 +562,11 @@ class HipRenderer final : public Renderer {
             pre.push_back(fmt("typedef %s %s%d __attribute__((aligned(%zu), ext_vector_type(%d)));", storage,
                               c_vector_base(s), vt.second, align, vt.second));
         }
-        std::set<std::string> wmma_names;
+        std::set<std::pair<std::string, Scalar>> wmma_names;
         bool uses_wave_reduce = false;
         int64_t reg_bytes = 0;  // per work-item, in declared register objects
         for (const UOp& u : nodes) {
-            if (u.op == Op::Wmma) wmma_names.insert(u.str);
+            if (u.op == Op::Wmma) wmma_names.insert({u.str, u.src.empty() ? Scalar::Void : by_id.at(u.src[0])->dtype.scalar});
             if (u.op == Op::WaveReduce) uses_wave_reduce = true;
             if (u.op == Op::DefineReg)
                 reg_bytes += (u.dtype.ptr_size > 0 ? u.dtype.ptr_size : 1) * static_cast<int64_t>(scalar_bytes(u.dtype.scalar)) * u.dtype.vcount;
@@ -551,9 +577,9 @@ class HipRenderer final : public Renderer {
         // them between the halves on every trip of the K loop.  (One-wave workgroups measured
         // slower with the hint, so they go without.)
         const bool two_waves = !wmma_names.empty() && reg_bytes <= 128 * 4 && local[0] * local[1] * local[2] >= 256;
-        for (const std::string& w : wmma_names) {
+        for (const auto& w : wmma_names) {
             std::string def;
-            if (!wmma_wrapper(w, &def)) return fail(kRenderError, "render: no gfx950 MFMA lowering for " + w);
+            if (!wmma_wrapper(w.first, w.second, &def)) return fail(kRenderError, "render: no gfx950 MFMA lowering for " + w.first);
             pre.push_back(def);
         }
         if (uses_wave_reduce) pre.push_back(kWaveReducePreamble);
@@ -710,6 +736,14 @@ class HipRenderer final : public Renderer {
                              static_cast<unsigned>(u.op), n, u.src.size());
             return kOk;
         };
+        // 8-bit floats are storage and tensor-core operands; C arithmetic on their `unsigned char`
+        // carrier would be integer arithmetic
+        if (u.op == Op::Unary || u.op == Op::Binary || u.op == Op::Where || u.op == Op::MulAcc || u.op == Op::Cast || u.op == Op::Reduce ||
+            u.op == Op::WaveReduce) {
+            bool fp8 = u.dtype.is_fp8();
+            for (uint32_t sid : u.src) fp8 = fp8 || node(sid).dtype.is_fp8();
+            if (fp8) return fail(kRenderError, "render: 8-bit float values can be loaded, stored and fed to a tensor core, nothing else");
+        }
         switch (u.op) {
             case Op::Param:
             case Op::DefineVar:
@@ -902,7 +936,7 @@ class HipRenderer final : public Renderer {
             }
             case Op::Wmma:  // ops.rs:404-411
                 MRK_TRY(need(3));
-                ctx.emit(u, "__" + u.str + "(" + S(0) + ", " + S(1) + ", " + S(2) + ")", "wmma", true);
+                ctx.emit(u, "__" + wmma_callee(u.str, node(u.src[0]).dtype.scalar) + "(" + S(0) + ", " + S(1) + ", " + S(2) + ")", "wmma", true);
                 return kOk;
             case Op::Reduce: {  // ops.rs:342-361
                 MRK_TRY(need(1));

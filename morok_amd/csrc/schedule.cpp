@@ -82,8 +82,10 @@ Logical resolve(const SwizzleAxis& a, const std::vector<Logical>& locals, const 
 
 }  // namespace
 
-std::vector<TensorCore> cdna4_tensor_cores() {
+std::vector<TensorCore> cdna4_tensor_cores() {  // renderer.rs:724-733, same order
     return {
+        cdna_161632(Scalar::Fp8E5M2, Scalar::Float32),
+        cdna_161632(Scalar::Fp8E4M3, Scalar::Float32),
         cdna_161632(Scalar::Float16, Scalar::Float32),
         cdna_161632(Scalar::BFloat16, Scalar::Float32),
         cdna_161616(Scalar::Float16, Scalar::Float32),
@@ -773,6 +775,7 @@ static bool wmma_async_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, in
 bool wmma_lds_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, int64_t N, int64_t K) {
     if (o.stages == 2) return wmma_async_opts_valid(tc, o, M, N, K);
     if (o.stages != 0) return false;
+    if (tc.dtype_in != Scalar::BFloat16 && tc.dtype_in != Scalar::Float16) return false;  // 8 elements per 16-byte copy
     int BM, BN, BK;
     if (tc.threads != 64 || tc.dims[0] != 16 || tc.dims[1] != 16 || !wmma_lds_tile(tc, o, K, &BM, &BN, &BK)) return false;
     // extents that the tile does not divide are padded (PADTO); the 16-byte copies still need

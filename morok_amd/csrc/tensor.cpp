@@ -25,6 +25,8 @@ size_t scalar_size(Scalar s) {
     switch (s) {
         case Scalar::Bool:
         case Scalar::Int8:
+        case Scalar::Fp8E4M3:
+        case Scalar::Fp8E5M2:
         case Scalar::UInt8: return 1;
         case Scalar::Int16:
         case Scalar::UInt16:

@@ -72,6 +72,11 @@ enum class Op : uint16_t {
 enum class Scalar : uint8_t {
     Bool = 0, Int8, UInt8, Int16, UInt16, Int32, UInt32, Int64, UInt64, Float16, BFloat16, Float32, Float64, Void,
     Index,
+    // dtype/src/lib.rs:142-143: OCP 8-bit floats (E4M3 has no infinity, maximum 448; E5M2 is the top
+    // byte of a half, maximum 57344).  One byte of storage, `unsigned char` in C
+    // (codegen/src/c/types.rs:26); they appear as tensor-core operands only.
+    Fp8E4M3,
+    Fp8E5M2,
 };
 
 enum class AddrSpace : uint8_t { Global = 0, Local = 1, Reg = 2 };  // dtype/src/lib.rs:103-110
@@ -100,6 +105,7 @@ struct DType {
         return scalar == Scalar::Float16 || scalar == Scalar::BFloat16 || scalar == Scalar::Float32 ||
                scalar == Scalar::Float64;
     }
+    bool is_fp8() const { return scalar == Scalar::Fp8E4M3 || scalar == Scalar::Fp8E5M2; }
     bool is_bool() const { return scalar == Scalar::Bool; }
     bool is_signed() const {
         return scalar == Scalar::Int8 || scalar == Scalar::Int16 || scalar == Scalar::Int32 ||

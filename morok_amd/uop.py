@@ -17,7 +17,7 @@ from .device import ProgramSpec
  MULACC, CAST, BITCAST, GEP, VECTORIZE, WMMA, IF, ENDIF, BARRIER, AFTER, NOOP, SINK, REDUCE, WAVE_REDUCE, LOAD_TR, ASYNC_COPY,
  WAIT_ASYNC) = range(31)
 
-(BOOL, I8, U8, I16, U16, I32, U32, I64, U64, F16, BF16, F32, F64, VOID, INDEX_T) = range(15)
+(BOOL, I8, U8, I16, U16, I32, U32, I64, U64, F16, BF16, F32, F64, VOID, INDEX_T, FP8E4M3, FP8E5M2) = range(17)
 GLOBAL, LOCAL, REG = 0, 1, 2
 (AX_GLOBAL, AX_WARP, AX_LOCAL, AX_LOOP, AX_GROUP_REDUCE, AX_REDUCE, AX_UPCAST, AX_UNROLL, AX_THREAD, AX_OUTER) = range(10)
 
@@ -58,6 +58,7 @@ class DT:
 
 
 f32, f16, bf16, f64 = DT(F32), DT(F16), DT(BF16), DT(F64)
+fp8e4m3, fp8e5m2 = DT(FP8E4M3), DT(FP8E5M2)   # one byte each; tensor-core operands only
 i32, i64, u32, u8, i8, boolean, index = DT(I32), DT(I64), DT(U32), DT(U8), DT(I8), DT(BOOL), DT(INDEX_T)
 
 

@@ -44,6 +44,13 @@
  *   orc_add_bf16          pinned: float64 sum rounded once, ties-to-even cases
  *   orc_heads_to_tokens_u16, orc_rope_heads_bf16
  *                         pinned: index permutation on distinct values, rotation vs float64
+ *   orc_fp8_to_f32, orc_matmul_fp8_f32
+ *                         pinned: the reference's range constants (448 / 57344, dtype/src/lib.rs:234-256)
+ *                         and (exponent, mantissa) widths (297-298); E5M2 against the top byte of
+ *                         an IEEE half for all 256 codes; E4M3 against the closed form of the OCP
+ *                         format for all 256 codes; the product against float64 on decoded values.
+ *                         The reference holds no 8-bit-float matmul test: parity unpinned by
+ *                         reference tests
  *
  * Exact summation order and bf16 rounding placement inside fused elementwise
  * chains of the real backend depend on optimizer choices that only running the
@@ -458,6 +465,34 @@ void orc_silu_mul_bf16(const bf16_t* g, const bf16_t* u, bf16_t* y, long n) {
 /* y = bf16(a + b) (residual) */
 void orc_add_bf16(const bf16_t* a, const bf16_t* b, bf16_t* y, long n) {
     for (long i = 0; i < n; i++) y[i] = f32_to_bf16(bf16_to_f32(a[i]) + bf16_to_f32(b[i]));
+}
+/* ===================== 8-bit floats (tensor-core operands) =====================
+ * dtype/src/lib.rs:142-143 (FP8E4M3, FP8E5M2), 234-256 (range -448..448 / -57344..57344),
+ * 297-298 ((exponent, mantissa) = (4, 3) / (5, 2)): the OCP formats.  E4M3 has bias 7, no
+ * infinity, and only S.1111.111 is NaN; E5M2 has bias 15 and IEEE-style infinities and NaNs.
+ * kind 0 = E4M3, 1 = E5M2. */
+static float fp8_decode(int kind, uint8_t v) {
+    const int mbits = kind == 0 ? 3 : 2, ebits = kind == 0 ? 4 : 5, bias = kind == 0 ? 7 : 15;
+    const int sign = v >> 7, e = (v >> mbits) & ((1 << ebits) - 1), m = v & ((1 << mbits) - 1);
+    float mag;
+    if (kind == 0 && e == 15 && m == 7) mag = NAN;
+    else if (kind == 1 && e == 31) mag = m ? NAN : INFINITY;
+    else if (e == 0) mag = ldexpf((float)m, 1 - bias - mbits);
+    else mag = ldexpf((float)((1 << mbits) + m), e - bias - mbits);
+    return sign ? -mag : mag;
+}
+void orc_fp8_to_f32(int kind, const uint8_t* x, long n, float* y) {
+    for (long i = 0; i < n; i++) y[i] = fp8_decode(kind, x[i]);
+}
+/* C[M,N] = A[M,K] B[K,N] on 8-bit-float operands: exact products, f32 accumulator in k order
+ * (the accumulate of tc.rs:358-674's WMMA with an f32 accumulator dtype). */
+void orc_matmul_fp8_f32(int kind, const uint8_t* a, const uint8_t* b, float* c, int M, int N, int K) {
+    for (int i = 0; i < M; i++)
+        for (int j = 0; j < N; j++) {
+            float acc = 0.0f;
+            for (int k = 0; k < K; k++) acc += fp8_decode(kind, a[(size_t)i * K + k]) * fp8_decode(kind, b[(size_t)k * N + j]);
+            c[(size_t)i * N + j] = acc;
+        }
 }
 /* head-major [B,H,S,D] -> token-major [B*S, H*D] */
 void orc_heads_to_tokens_u16(const uint16_t* x, uint16_t* y, int batch, int seq, int heads, int dim) {

@@ -178,14 +178,14 @@ static int work(int id) {
                     int opts[6] = {wm, wn, um, 2, id % 3, 0};
                     uint8_t* kern = nullptr;
                     size_t len = 0;
-                    if (mrk_hip_sched_build_wmma_matmul_lds_opts(1, 200 + id, 136, 72, 10, opts, &kern, &len) == 0) mrk_hip_sched_free(kern);
+                    if (mrk_hip_sched_build_wmma_matmul_lds_opts(3, 200 + id, 136, 72, 10, opts, &kern, &len) == 0) mrk_hip_sched_free(kern);
                 }
         // and the variant with direct global -> local copies on shapes its tiles divide
         for (int um : {2, 4, 8}) {
             int opts[6] = {2, 2 << (id % 2), um, 4, 0, 2};
             uint8_t* kern = nullptr;
             size_t len = 0;
-            if (mrk_hip_sched_build_wmma_matmul_lds_opts(1, 1024, 1024, 64 * (1 + id), 10, opts, &kern, &len) == 0) mrk_hip_sched_free(kern);
+            if (mrk_hip_sched_build_wmma_matmul_lds_opts(3, 1024, 1024, 64 * (1 + id), 10, opts, &kern, &len) == 0) mrk_hip_sched_free(kern);
         }
     }
     for (mrk_tensor* p : {t, u, w, s, m}) mrk_hip_tensor_release(p);

@@ -157,6 +157,20 @@ class Oracle:
         self.lib.orc_add_bf16(_ptr(a), _ptr(b), _ptr(y), C.c_long(a.size))
         return y
 
+    def fp8_to_f32(self, kind, x):
+        """kind 0 = E4M3, 1 = E5M2; x: uint8 codes."""
+        x = np.ascontiguousarray(x, np.uint8)
+        y = np.empty(x.shape, np.float32)
+        self.lib.orc_fp8_to_f32(C.c_int(kind), _ptr(x), C.c_long(x.size), _ptr(y))
+        return y
+
+    def matmul_fp8_f32(self, kind, a, b):
+        a = np.ascontiguousarray(a, np.uint8)
+        b = np.ascontiguousarray(b, np.uint8)
+        c = np.empty((a.shape[0], b.shape[1]), np.float32)
+        self.lib.orc_matmul_fp8_f32(C.c_int(kind), _ptr(a), _ptr(b), _ptr(c), a.shape[0], b.shape[1], a.shape[1])
+        return c
+
     def decoder_block_bf16(self, tok, w, cos, sin, batch, seq, hidden, heads, ffn, eps, threads=None):
         T = batch * seq
         n = self.lib.orc_decoder_block_scratch_elems(T, hidden, ffn)

@@ -79,7 +79,7 @@ def test_generated_tensor_core_random_choices(dev, seed):
         opts = (int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4, 8])), int(rng.choice([1, 2, 4, 8])),
                 int(rng.choice([0, 1, 2, 4])))
         try:
-            kern = sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts)
+            kern = sched.build_wmma_matmul_lds_opts(3, M, N, K, U.BF16, opts)
             break
         except morok_amd.MorokHipError:
             continue

@@ -842,8 +842,8 @@ def test_null_arguments_are_errors_not_crashes(T, dev, shim):
         lambda: shim.mrk_hip_tensor_logsumexp(x._h, -1, null),
         lambda: shim.mrk_hip_gemm_bf16_residual(0, null, 1, 1, 1, 8, 8, 8),
         lambda: shim.mrk_hip_flash_attn_fwd_bf16_strided(0, 1, 1, 1, 1, 1, 1, 8, 8, 128, 1.0, 0, null),
-        lambda: shim.mrk_hip_sched_build_wmma_matmul_lds_opts(1, 128, 128, 64, 10, null, C.byref(C.POINTER(C.c_uint8)()), C.byref(C.c_size_t())),
-        lambda: shim.mrk_hip_beam_search_wmma_matmul(0, 1, 128, 128, 64, 1, null, null, null, null),
+        lambda: shim.mrk_hip_sched_build_wmma_matmul_lds_opts(3, 128, 128, 64, 10, null, C.byref(C.POINTER(C.c_uint8)()), C.byref(C.c_size_t())),
+        lambda: shim.mrk_hip_beam_search_wmma_matmul(2, 1, 128, 128, 64, 1, null, null, null, null),
         lambda: shim.mrk_hip_benchmark_kernel_with_cutoff(0, null, null, 0, null, 0, null, null, 1, 1, 0.0, null, null, null),
     ]
     for i, call in enumerate(calls):

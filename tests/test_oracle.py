@@ -529,3 +529,56 @@ def test_heads_to_tokens_and_rope_heads_layout(oracle):
     ref = np.concatenate([lo * c64 - hi * s64, lo * s64 + hi * c64], -1)
     got = synth.from_bf16(rot).astype(np.float64)
     assert np.abs(got - ref).max() <= 2.0 ** -8 * np.abs(ref).max() + 1e-6
+
+
+def test_fp8_decode_all_codes(oracle):
+    """Every one of the 256 codes of both 8-bit floats.  E5M2 is the top byte of an IEEE half, so
+    numpy's float16 decodes it independently; E4M3 (OCP: bias 7, no infinity, S.1111.111 = NaN)
+    against its closed form written per field; both against the range and field widths the
+    reference records for them."""
+    codes = np.arange(256, dtype=np.uint8)
+    fmt = GOLD["fp8_formats"]
+    e5 = oracle.fp8_to_f32(1, codes)
+    half = (codes.astype(np.uint16) << 8).view(np.float16).astype(np.float32)
+    assert np.array_equal(np.isnan(e5), np.isnan(half)) and np.array_equal(e5[~np.isnan(e5)], half[~np.isnan(half)])
+    fin = e5[np.isfinite(e5)]
+    assert fin.max() == fmt["e5m2"]["max"] and fin.min() == fmt["e5m2"]["min"]
+    e4 = oracle.fp8_to_f32(0, codes)
+    eb, mb = fmt["e4m3"]["exponent_bits"], fmt["e4m3"]["mantissa_bits"]
+    assert (eb, mb) == (4, 3) and 1 + eb + mb == 8
+    want = []
+    for c in range(256):
+        s, e, m = c >> 7, (c >> mb) & (2 ** eb - 1), c & (2 ** mb - 1)
+        if e == 2 ** eb - 1 and m == 2 ** mb - 1:
+            v = float("nan")
+        elif e == 0:
+            v = m / 2 ** mb * 2.0 ** (1 - 7)
+        else:
+            v = (1 + m / 2 ** mb) * 2.0 ** (e - 7)
+        want.append(-v if s else v)
+    want = np.float32(want)
+    assert np.isnan(e4[0x7F]) and np.isnan(e4[0xFF]) and np.isnan(e4).sum() == 2 and not np.isinf(e4).any()
+    ok = ~np.isnan(want)
+    assert np.array_equal(e4[ok], want[ok])
+    assert np.nanmax(e4) == fmt["e4m3"]["max"] and np.nanmin(e4) == fmt["e4m3"]["min"]
+    # landmarks a shifted bias or a swapped field width would move
+    assert e4[0x38] == 1.0 and e4[0x40] == 2.0 and e4[0x30] == 0.5 and e4[0x01] == 2.0 ** -9 and e4[0x08] == 2.0 ** -6 and e4[0x7E] == 448.0
+    assert e5[0x3C] == 1.0 and e5[0x40] == 2.0 and e5[0x01] == 2.0 ** -16 and e5[0x7B] == 57344.0 and np.isinf(e5[0x7C])
+    # magnitudes grow with the code within a sign
+    assert np.all(np.diff(e4[:0x7F]) > 0) and np.all(np.diff(e5[:0x7D]) > 0)
+
+
+@pytest.mark.parametrize("kind", [0, 1])
+def test_fp8_matmul_vs_float64(oracle, kind):
+    rng = np.random.default_rng(95 + kind)
+    M, N, K = 33, 20, 96
+    # finite codes of moderate magnitude
+    a = rng.integers(0x10, 0x58, (M, K)).astype(np.uint8) | (rng.integers(0, 2, (M, K)).astype(np.uint8) << 7)
+    b = rng.integers(0x10, 0x58, (K, N)).astype(np.uint8) | (rng.integers(0, 2, (K, N)).astype(np.uint8) << 7)
+    c = oracle.matmul_fp8_f32(kind, a, b)
+    af, bf = oracle.fp8_to_f32(kind, a).astype(np.float64), oracle.fp8_to_f32(kind, b).astype(np.float64)
+    ref = af @ bf
+    assert np.abs(c - ref).max() <= 1e-5 * (np.abs(af) @ np.abs(bf)).max()
+    eye = np.zeros((K, K), np.uint8)
+    eye[np.arange(K), np.arange(K)] = 0x38 if kind == 0 else 0x3C        # 1.0
+    assert np.array_equal(oracle.matmul_fp8_f32(kind, a, eye), oracle.fp8_to_f32(kind, a))

@@ -211,8 +211,8 @@ def test_variables_positional_vals(dev):
     assert np.array_equal(y[:700], np.arange(700, dtype=np.float32) + 5) and not y[700:].any()
 
 
-@pytest.mark.parametrize("tc,shape,out", [(1, (64, 160, 128), U.BF16), (1, (16, 16, 32), U.BF16), (3, (48, 32, 64), U.BF16),
-                                          (1, (80, 48, 96), U.F32)])
+@pytest.mark.parametrize("tc,shape,out", [(3, (64, 160, 128), U.BF16), (3, (16, 16, 32), U.BF16), (5, (48, 32, 64), U.BF16),
+                                          (3, (80, 48, 96), U.F32)])
 def test_tc_apply_matmul_from_tables(dev, oracle, tc, shape, out):
     """The tensor-core matmul built from the CDNA tables (opts + swizzle) on the GPU."""
     from morok_amd import sched
@@ -236,8 +236,8 @@ def test_tc_apply_matmul_from_tables(dev, oracle, tc, shape, out):
     assert np.array_equal(c1, want if out == U.BF16 else synth.from_bf16(want))
 
 
-@pytest.mark.parametrize("tc,shape,out", [(1, (128, 128, 32), U.BF16), (1, (256, 384, 160), U.BF16), (1, (128, 256, 1024), U.F32),
-                                          (3, (128, 128, 48), U.BF16), (3, (256, 128, 96), U.BF16)])
+@pytest.mark.parametrize("tc,shape,out", [(3, (128, 128, 32), U.BF16), (3, (256, 384, 160), U.BF16), (3, (128, 256, 1024), U.F32),
+                                          (5, (128, 128, 48), U.BF16), (5, (256, 128, 96), U.BF16)])
 def test_tc_matmul_staged_through_local_memory(dev, oracle, tc, shape, out):
     """The generated tensor-core matmul with a 2 x 2-wave workgroup, both operands copied
     through LDS (B with pairs of K rows interleaved, or as plain rows when the K tile is 16
@@ -275,14 +275,54 @@ def test_tc_matmul_lds_choices_agree(dev, opts):
     M, N, K = 512, 256, 256
     a = synth.normal_bf16((M, K), 5, 21)
     b = synth.normal_bf16((K, N), 5, 22)
-    kern = sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts)
+    kern = sched.build_wmma_matmul_lds_opts(3, M, N, K, U.BF16, opts)
     c = run(dev, kern, "r_tc_lds", (M, N), np.uint16, [a, b])
-    plain = run(dev, sched.build_wmma_matmul(1, M, N, K, U.BF16), "r_tc", (M, N), np.uint16, [a, b])
+    plain = run(dev, sched.build_wmma_matmul(3, M, N, K, U.BF16), "r_tc", (M, N), np.uint16, [a, b])
     assert np.array_equal(c, plain)
     a1 = np.zeros((M, K), np.float32)
     a1[np.arange(M), (np.arange(M) * 7) % K] = 1
     c1 = run(dev, kern, "r_tc_lds", (M, N), np.uint16, [synth.to_bf16(a1), b])
     assert np.array_equal(c1, b[(np.arange(M) * 7) % K])
+
+
+@pytest.mark.parametrize("tc,kind,one", [(0, 1, 0x3C), (1, 0, 0x38)])
+@pytest.mark.parametrize("shape", [(16, 16, 32), (64, 80, 128), (48, 32, 256)])
+def test_tc_apply_matmul_fp8(dev, oracle, tc, kind, one, shape):
+    """The two 8-bit-float tensor cores of the CDNA4 table (E5M2 first, then E4M3): operands are
+    byte codes, eight per lane, the accumulator is f32.  Products of 8-bit floats are exact in f32
+    and the oracle adds them one by one.  The matrix core adds the 32 products of a K step as one
+    block, aligned to the block's largest product, and drops what lies more than about 11.6 bits
+    below it (measured: error <= 2^-11.6 of the largest product per block over the formats' whole
+    range, none at all when the operands span a few binades).  So: operands within [0.5, 2) give
+    the float64 result exactly; operands over the wide range stay within 2^-11 of the largest
+    product per block of 32, summed over the blocks; one-hot rows of 1.0 return the decoded rows
+    of B exactly."""
+    from morok_amd import sched
+
+    M, N, K = shape
+    rng = np.random.default_rng(97 + kind)
+    kern = sched.build_wmma_matmul(tc, M, N, K, U.F32)
+
+    def codes(lo, hi, shp):
+        return rng.integers(lo, hi, shp).astype(np.uint8) | (rng.integers(0, 2, shp).astype(np.uint8) << 7)
+
+    one_code, two_code = one, one + (8 if kind == 0 else 4)              # 1.0 and 2.0
+    a, b = codes(one_code - (two_code - one_code), two_code, (M, K)), codes(one_code - (two_code - one_code), two_code, (K, N))
+    c = run(dev, kern, "r_tc8", (M, N), np.float32, [a, b])
+    af, bf = oracle.fp8_to_f32(kind, a).astype(np.float64), oracle.fp8_to_f32(kind, b).astype(np.float64)
+    assert np.abs(af).min() >= 0.5 and np.abs(af).max() < 2.0
+    assert np.array_equal(c, (af @ bf).astype(np.float32)) and np.array_equal(c, oracle.matmul_fp8_f32(kind, a, b))
+    a, b = codes(0x08, 0x60, (M, K)), codes(0x08, 0x60, (K, N))
+    c = run(dev, kern, "r_tc8", (M, N), np.float32, [a, b])
+    ref = oracle.matmul_fp8_f32(kind, a, b)
+    af, bf = oracle.fp8_to_f32(kind, a).astype(np.float64), oracle.fp8_to_f32(kind, b).astype(np.float64)
+    terms = np.abs(af[:, :, None] * bf[None, :, :]).reshape(M, K // 32, 32, N)
+    bound = 2.0 ** -11 * terms.max(2).sum(1) + 1e-6 * np.abs(af) @ np.abs(bf)
+    assert np.all(np.abs(c - ref) <= bound)
+    a1 = np.zeros((M, K), np.uint8)
+    a1[np.arange(M), (np.arange(M) * 5) % K] = one
+    c1 = run(dev, kern, "r_tc8", (M, N), np.float32, [a1, b])
+    assert np.array_equal(c1, oracle.fp8_to_f32(kind, b)[(np.arange(M) * 5) % K])
 
 
 @pytest.mark.parametrize("shape,opts", [((512, 512, 256), (2, 2, 2, 2, 0, 2)), ((256, 384, 64), (2, 2, 4, 4, 0, 2)),
@@ -302,7 +342,7 @@ def test_tc_matmul_direct_copy_choices_agree(dev, shape, opts):
     M, N, K = shape
     a = synth.normal_bf16((M, K), 9, 41)
     b = synth.normal_bf16((K, N), 9, 42)
-    kern = sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts)
+    kern = sched.build_wmma_matmul_lds_opts(3, M, N, K, U.BF16, opts)
     nan = np.uint16(0x7FC0)
 
     def fenced(x):
@@ -320,7 +360,7 @@ def test_tc_matmul_direct_copy_choices_agree(dev, shape, opts):
         assert np.all(got[M * N:] == nan)
         return got[:M * N].reshape(M, N)
 
-    plain = run(dev, sched.build_wmma_matmul(1, M, N, K, U.BF16), "r_tc", (M, N), np.uint16, [a, b])
+    plain = run(dev, sched.build_wmma_matmul(3, M, N, K, U.BF16), "r_tc", (M, N), np.uint16, [a, b])
     assert np.array_equal(run_fenced(a), plain)
     a1 = np.zeros((M, K), np.float32)
     a1[np.arange(M), (np.arange(M) * 7) % K] = 1
@@ -339,7 +379,7 @@ def test_tc_matmul_lds_padded_shapes(dev, shape, opts):
     M, N, K = shape
     a = synth.normal_bf16((M, K), 6, 31)
     b = synth.normal_bf16((K, N), 6, 32)
-    kern = sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts)
+    kern = sched.build_wmma_matmul_lds_opts(3, M, N, K, U.BF16, opts)
     # operands and result each sit in the front of a larger NaN-filled buffer
     nan = np.uint16(0x7FC0)
     abig = np.full(M * K + 4096, nan, np.uint16); abig[:M * K] = a.ravel()

@@ -196,7 +196,7 @@ def test_beam_search_wmma_matmul(dev, tmp_path, monkeypatch):
     monkeypatch.setenv("MOROK_CACHE_DIR", str(tmp_path))
     monkeypatch.delenv("IGNORE_BEAM_CACHE", raising=False)
     M, N, K = 1024, 512, 512
-    opts, best_ms, cached, timed = sched.beam_search_wmma_matmul(1, M, N, K, width=2)
+    opts, best_ms, cached, timed = sched.beam_search_wmma_matmul(3, M, N, K, width=2)
     assert not cached and timed >= 12 and best_ms > 0
     a = synth.normal_bf16((M, K), 8, 0)
     b = synth.normal_bf16((K, N), 8, 1)
@@ -210,14 +210,14 @@ def test_beam_search_wmma_matmul(dev, tmp_path, monkeypatch):
         plan.build().execute()
         return bc, bc.copyout(np.uint16, (M, N))
 
-    bc, got = run(sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts), "beam_tc_winner")
-    _, want = run(sched.build_wmma_matmul_lds(1, M, N, K, U.BF16), "beam_tc_default")
+    bc, got = run(sched.build_wmma_matmul_lds_opts(3, M, N, K, U.BF16, opts), "beam_tc_winner")
+    _, want = run(sched.build_wmma_matmul_lds(3, M, N, K, U.BF16), "beam_tc_default")
     assert np.array_equal(got, want)
     ref = synth.from_bf16(a).astype(np.float64) @ synth.from_bf16(b).astype(np.float64)
     assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
-    base_ms = sched.compile_and_time(sched.build_wmma_matmul_lds(1, M, N, K, U.BF16), [bc, ba, bb], warmup=1, runs=5)
+    base_ms = sched.compile_and_time(sched.build_wmma_matmul_lds(3, M, N, K, U.BF16), [bc, ba, bb], warmup=1, runs=5)
     assert best_ms <= base_ms * 1.15
-    opts2, _, cached2, timed2 = sched.beam_search_wmma_matmul(1, M, N, K, width=2)
+    opts2, _, cached2, timed2 = sched.beam_search_wmma_matmul(3, M, N, K, width=2)
     assert cached2 and timed2 == 0 and opts2 == opts
 
 

@@ -16,26 +16,31 @@ def test_caps_match_reference_descriptor():
     assert c["device"] == "AMD_CDNA4" and c["has_local"] == 1 and c["has_shared"] == 1 and c["has_threads"] == 0
     assert c["global_max"] == [2147483647, 65535, 65535] and c["local_max"] == 1024 and c["upcast_max"] == 8
     assert c["shared_max"] == 163840  # gfx950 LDS per workgroup (the reference lists 65536)
-    assert c["tensor_cores"][:2] == ["WMMA_16_16_32_half_float", "WMMA_16_16_32_bfloat_float"]
-    assert "WMMA_16_16_16_bfloat_float" in c["tensor_cores"]
+    # cdna4_tensor_cores(), renderer.rs:724-733: fp8e5m2, fp8e4m3, f16, bf16 (16x16x32), f16, bf16 (16x16x16);
+    # the reference's WMMA name table has no entry for the 8-bit floats (tc.rs:677-688: "unknown")
+    assert c["tensor_cores"] == ["WMMA_16_16_32_unknown_float", "WMMA_16_16_32_unknown_float", "WMMA_16_16_32_half_float",
+                                 "WMMA_16_16_32_bfloat_float", "WMMA_16_16_16_half_float", "WMMA_16_16_16_bfloat_float"]
 
 
 def test_tensor_core_selection():
     # tc.rs:126-168: first entry whose input and accumulator dtypes match
-    assert sched.tc_select(U.BF16, U.BF16, U.F32) == 1
-    assert sched.tc_select(U.F16, U.F16, U.F32) == 0
+    assert sched.tc_select(U.BF16, U.BF16, U.F32) == 3
+    assert sched.tc_select(U.F16, U.F16, U.F32) == 2
+    assert sched.tc_select(U.FP8E5M2, U.FP8E5M2, U.F32) == 0
+    assert sched.tc_select(U.FP8E4M3, U.FP8E4M3, U.F32) == 1
+    assert sched.tc_select(U.FP8E4M3, U.FP8E5M2, U.F32) == -1
     assert sched.tc_select(U.F32, U.F32, U.F32) == -1
     assert sched.tc_select(U.BF16, U.BF16, U.BF16) == -1
     assert sched.tc_select(U.BF16, U.F16, U.F32) == -1
-    dims, threads, ept = sched.tc_info(1)
-    assert dims == [16, 16, 32] and threads == 64 and ept == [8, 8, 4]  # renderer.rs:549-558
     dims, threads, ept = sched.tc_info(3)
+    assert dims == [16, 16, 32] and threads == 64 and ept == [8, 8, 4]  # renderer.rs:549-558
+    dims, threads, ept = sched.tc_info(5)
     assert dims == [16, 16, 16] and ept == [4, 4, 4]
     with pytest.raises(MorokHipError):
-        sched.tc_info(9)
+        sched.tc_info(11)
 
 
-@pytest.mark.parametrize("tc", [0, 1, 2, 3])
+@pytest.mark.parametrize("tc", [0, 1, 2, 3, 4, 5])
 def test_swizzle_tables_equal_mfma_register_layout(tc):
     """Layout of v_mfma_f32_16x16x{16,32}: lane l holds row/column l % 16 and the contiguous k
     group l // 16 of A/B; accumulator element i of lane l is C[4 * (l // 16) + i][l % 16].
@@ -127,16 +132,25 @@ def test_matmul_kernels_render_and_compile():
     spec = U.render(sched.build_matmul_f32(128, 192, 64), "r_mm")
     assert spec.global_size == [3, 2, 1] and spec.local_size == [16, 16, 1] and "fmaf(" in spec.src
     morok_amd.compile_spec(spec)
-    spec = U.render(sched.build_wmma_matmul(1, 64, 160, 128), "r_tc")
+    spec = U.render(sched.build_wmma_matmul(3, 64, 160, 128), "r_tc")
     # post-TC upcasts (heuristics.rs:787-821): M has 4 tiles -> upcast 4, N has 10 -> upcast 5
     assert spec.global_size == [2, 1, 1] and spec.local_size == [64, 1, 1]
     assert spec.src.count("__WMMA_16_16_32_bfloat_float(") == 20 + 1
     morok_amd.compile_spec(spec)
     with pytest.raises(MorokHipError) as e:
-        sched.build_wmma_matmul(1, 60, 64, 64)
+        sched.build_wmma_matmul(3, 60, 64, 64)
     assert "not a multiple" in e.value.message
-    morok_amd.compile_spec(U.render(sched.build_wmma_matmul(0, 32, 32, 64, U.F16), "r_tc16"))
-    morok_amd.compile_spec(U.render(sched.build_wmma_matmul(2, 32, 32, 64, U.F32), "r_tc16k16"))
+    # the 8-bit-float cores: byte operands, eight per lane handed over as one 64-bit integer
+    for tc, builtin in ((0, "__builtin_amdgcn_mfma_f32_16x16x32_bf8_bf8"), (1, "__builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8")):
+        spec8 = U.render(sched.build_wmma_matmul(tc, 32, 32, 64, U.F32), "r_tc8")
+        assert builtin in spec8.src and "const unsigned char* __restrict__ data1" in spec8.src
+        morok_amd.compile_spec(spec8)
+        with pytest.raises(MorokHipError):
+            sched.build_wmma_matmul_lds(tc, 128, 128, 64, U.F32)          # the LDS layouts are for 16-bit elements
+    with pytest.raises(MorokHipError):                                    # an 8-bit-float result would need arithmetic on the carrier byte
+        U.render(sched.build_wmma_matmul(1, 32, 32, 64, U.FP8E4M3), "r_tc8_out")
+    morok_amd.compile_spec(U.render(sched.build_wmma_matmul(2, 32, 32, 64, U.F16), "r_tc16"))
+    morok_amd.compile_spec(U.render(sched.build_wmma_matmul(4, 32, 32, 64, U.F32), "r_tc16k16"))
 
 
 def test_wmma_matmul_lds_kernel_builds_and_compiles():
@@ -146,7 +160,7 @@ def test_wmma_matmul_lds_kernel_builds_and_compiles():
     import morok_amd
     from morok_amd import sched, uop as U
 
-    kern = sched.build_wmma_matmul_lds(1, 256, 128, 64, U.BF16)
+    kern = sched.build_wmma_matmul_lds(3, 256, 128, 64, U.BF16)
     spec = U.render(kern, "r_tc_lds")
     src = spec.src
     assert src.count("__shared__") == 2 and src.count("__syncthreads();") == 2
@@ -156,12 +170,12 @@ def test_wmma_matmul_lds_kernel_builds_and_compiles():
     morok_amd.compile_spec(spec)
     assert "amdgpu_waves_per_eu(2)" in src                               # four waves, accumulators within half the file
     # extents the tile does not divide are padded: gated loads, guarded stores, a rounded-up grid
-    pad = U.render(sched.build_wmma_matmul_lds(1, 200, 136, 72, U.BF16), "r_tc_pad")
+    pad = U.render(sched.build_wmma_matmul_lds(3, 200, 136, 72, U.BF16), "r_tc_pad")
     assert pad.sizes() == ([2, 2, 1], [64, 4, 1]) and " ? *((mrk_bhalf8*)" in pad.src and "if (" in pad.src
     morok_amd.compile_spec(pad)
     assert " ? *((mrk_bhalf8*)" not in src and "if (" not in src        # none of it when the tile divides
     with pytest.raises(morok_amd.MorokHipError):
-        sched.build_wmma_matmul_lds(1, 64, 130, 64, U.BF16)               # rows of B are not whole 16-byte vectors
+        sched.build_wmma_matmul_lds(3, 64, 130, 64, U.BF16)               # rows of B are not whole 16-byte vectors
 
 
 @pytest.mark.parametrize("opts,grid,block,mfma,hint", [((1, 1, 1, 1, 0), [8, 16, 1], [64, 1, 1], 2, False),
@@ -176,7 +190,7 @@ def test_wmma_matmul_lds_kernel_choices(opts, grid, block, mfma, hint):
     from morok_amd import sched, uop as U
 
     M, N, K = 256, 128, 64
-    spec = U.render(sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, opts), "r_tc_lds")
+    spec = U.render(sched.build_wmma_matmul_lds_opts(3, M, N, K, U.BF16, opts), "r_tc_lds")
     assert spec.sizes() == (grid, block)
     assert spec.src.count("__WMMA_16_16_32_bfloat_float(") == mfma + 1
     # two waves per SIMD are asked for when four or more waves share a workgroup and the declared
@@ -192,7 +206,7 @@ def test_wmma_matmul_lds_kernel_refuses_bad_choices(opts):
     from morok_amd import sched, uop as U
 
     with pytest.raises(morok_amd.MorokHipError):
-        sched.build_wmma_matmul_lds_opts(1, 256, 128, 64, U.BF16, opts)
+        sched.build_wmma_matmul_lds_opts(3, 256, 128, 64, U.BF16, opts)
 
 
 def test_wmma_matmul_direct_copy_kernel_builds_and_compiles():
@@ -204,7 +218,7 @@ def test_wmma_matmul_direct_copy_kernel_builds_and_compiles():
     from morok_amd import sched, uop as U
 
     M, N, K = 1024, 512, 256
-    spec = U.render(sched.build_wmma_matmul_lds_opts(1, M, N, K, U.BF16, (2, 4, 8, 4, 0, 2)), "r_tc_dma")
+    spec = U.render(sched.build_wmma_matmul_lds_opts(3, M, N, K, U.BF16, (2, 4, 8, 4, 0, 2)), "r_tc_dma")
     src = spec.src
     assert spec.sizes() == ([8, 1, 1], [64, 8, 1])                       # 4 x 2 tiles of 256 x 256, 8 waves
     assert "__shared__ __bf16 local0[32768];" in src and "__shared__ __bf16 local1[32768];" in src   # 2 stages x 256 x 64 each
@@ -218,10 +232,10 @@ def test_wmma_matmul_direct_copy_kernel_builds_and_compiles():
     assert "gidx0 % 8" in src                                              # the XCD regrouping
     morok_amd.compile_spec(spec)
     # a single K step has no loop-carried copies; half precision takes the f16 transposing load
-    one = U.render(sched.build_wmma_matmul_lds_opts(1, 128, 128, 64, U.BF16, (2, 2, 4, 4, 0, 2)), "r_tc_dma1")
+    one = U.render(sched.build_wmma_matmul_lds_opts(3, 128, 128, 64, U.BF16, (2, 2, 4, 4, 0, 2)), "r_tc_dma1")
     assert one.src.count("global_load_lds_dwordx4") == (128 // 8 + 128 // 8) // 4 and "s_waitcnt vmcnt(0)" in one.src
     morok_amd.compile_spec(one)
-    half = U.render(sched.build_wmma_matmul_lds_opts(0, 128, 128, 128, U.F16, (2, 2, 4, 4, 0, 2)), "r_tc_dma_h")
+    half = U.render(sched.build_wmma_matmul_lds_opts(2, 128, 128, 128, U.F16, (2, 2, 4, 4, 0, 2)), "r_tc_dma_h")
     assert "__builtin_amdgcn_ds_read_tr16_b64_v4f16(" in half.src
     morok_amd.compile_spec(half)
 
@@ -237,9 +251,9 @@ def test_tc_matmul_direct_copy_refuses_what_it_cannot_tile():
                         ((1024, 1024, 256), (4, 4, 8, 8, 0, 2)),   # two stages of 512 x 512 exceed local memory
                         ((512, 512, 256), (2, 2, 2, 2, 0, 3))):    # no such variant
         with pytest.raises(morok_amd.MorokHipError):
-            sched.build_wmma_matmul_lds_opts(1, *shape, U.BF16, opts)
+            sched.build_wmma_matmul_lds_opts(3, *shape, U.BF16, opts)
     with pytest.raises(morok_amd.MorokHipError):
-        sched.build_wmma_matmul_lds_opts(3, 512, 512, 256, U.BF16, (2, 2, 2, 2, 0, 2))   # a 16x16x16 tensor core
+        sched.build_wmma_matmul_lds_opts(5, 512, 512, 256, U.BF16, (2, 2, 2, 2, 0, 2))   # a 16x16x16 tensor core
 
 
 def test_global_index_order_modes_and_where_they_differ():
