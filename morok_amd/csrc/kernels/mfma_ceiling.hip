@@ -1,7 +1,9 @@
 // Calibration kernel: what the matrix pipes of this part sustain when nothing else competes.
 // One workgroup of four waves per compute unit; every wave issues the MFMA stream of one
 // 256x256 GEMM tile (64 v_mfma_f32_32x32x16_bf16 per 64-deep K step, sixteen independent
-// accumulators) from registers only: no global loads, no LDS traffic, no barriers.  The rate
+// accumulators, a different set of operand fragments for each of the four 16-deep sub-steps, the
+// 4 x 4 tiles walked back and forth as the GEMM kernel walks them) from registers only: no global
+// loads, no LDS traffic, no barriers.  The rate
 // it reaches is the ceiling a bf16 GEMM kernel is measured against next to the published peak
 // (the part lowers its clock under matrix load, so that ceiling sits below the peak).
 #include <hip/hip_runtime.h>
@@ -17,7 +19,9 @@ typedef float cal_f32x16 __attribute__((ext_vector_type(16)));
 // spread over [-1.7, 1.7) by a hash of (lane, register, element), as the operands of a product of
 // random matrices are.  The matrix pipes' power draw, and with it the clock the part sustains,
 // depends on how much the operand bits toggle.
-__global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ out, int k_steps, float seed, int random_operands) {
+// (a template parameter, so that the set-up in front of the loop is straight-line code)
+template <bool random_operands>
+__global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ out, int k_steps, float seed) {
     const int lane = threadIdx.x & 63;
     cal_f32x16 acc[4][4];
 #pragma unroll
@@ -26,23 +30,25 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ o
         for (int j = 0; j < 4; j++)
 #pragma unroll
             for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
-    cal_bf16x8 fa[4], fb[4];
+    cal_bf16x8 fa[4][4], fb[4][4];  // [sub-step][tile row / column]
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++)
 #pragma unroll
     for (int i = 0; i < 4; i++)
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             if (random_operands) {
-                unsigned x = (unsigned)((threadIdx.x * 4 + i) * 8 + e) * 2654435761u + blockIdx.x * 40503u + 12345u;
+                unsigned x = (unsigned)(((threadIdx.x * 4 + i) * 8 + e) * 4 + ks) * 2654435761u + blockIdx.x * 40503u + 12345u;
                 x ^= x >> 15;
                 x *= 2246822519u;
                 x ^= x >> 13;
                 unsigned y = x * 3266489917u;
                 y ^= y >> 16;
-                fa[i][e] = (__bf16)(((float)(x >> 8) / 8388608.0f - 1.0f) * 1.7f);
-                fb[i][e] = (__bf16)(((float)(y >> 8) / 8388608.0f - 1.0f) * 1.7f);
+                fa[ks][i][e] = (__bf16)(((float)(x >> 8) / 8388608.0f - 1.0f) * 1.7f);
+                fb[ks][i][e] = (__bf16)(((float)(y >> 8) / 8388608.0f - 1.0f) * 1.7f);
             } else {
-                fa[i][e] = (__bf16)(seed * (float)(lane + e + i));
-                fb[i][e] = (__bf16)(seed * (float)(lane - e - i));
+                fa[ks][i][e] = (__bf16)(seed * (float)(lane + e + i));
+                fb[ks][i][e] = (__bf16)(seed * (float)(lane - e - i));
             }
         }
     for (int kt = 0; kt < k_steps; kt++) {
@@ -51,10 +57,12 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ o
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+                for (int jj = 0; jj < 4; jj++) {
+                    const int j = (i & 1) ? 3 - jj : jj;
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[ks][j], fa[ks][i], acc[i][j], 0, 0, 0);
+                }
         // keeps the loop a loop: the operands change in a way the compiler cannot fold
-        asm volatile("" : "+v"(fa[0]), "+v"(fb[0]));
+        asm volatile("" : "+v"(fa[0][0]), "+v"(fb[0][0]));
     }
     float s = 0.0f;
 #pragma unroll
@@ -74,8 +82,10 @@ int launch_mfma_ceiling(void* stream, void* out, long workgroups, long k_steps, 
     if (workgroups <= 0 || k_steps <= 0 || workgroups > 0x7fffffffL || k_steps > 0x7fffffffL || !out)
         return (int)hipErrorInvalidValue;
     (void)hipGetLastError();
-    dev::mfma_ceiling_kernel<<<(unsigned)workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<float*>(out),
-                                                                                               (int)k_steps, 0.001f, random_operands);
+    if (random_operands)
+        dev::mfma_ceiling_kernel<true><<<(unsigned)workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<float*>(out), (int)k_steps, 0.001f);
+    else
+        dev::mfma_ceiling_kernel<false><<<(unsigned)workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<float*>(out), (int)k_steps, 0.001f);
     return (int)hipGetLastError();
 }
 

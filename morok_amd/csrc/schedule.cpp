@@ -948,8 +948,11 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
     // the B fragment goes in as the first operand: the tensor core then leaves four consecutive
     // columns of one row in a lane (result rows are written as vectors), same products, same order
     auto mfmas = [&](const std::vector<uint32_t>& af, const std::vector<uint32_t>& bf) {
+        // columns back and forth, so that consecutive tensor-core instructions always share one
+        // operand (fewer operand bits toggle; the part's clock under matrix load follows that)
         for (int i = 0; i < um; i++)
-            for (int j = 0; j < un; j++) {
+            for (int jj = 0; jj < un; jj++) {
+                const int j = (i & 1) ? un - 1 - jj : jj;
                 uint32_t slot = acc[i * un + j];
                 b.store(slot, b.add(Op::Wmma, cd, {bf[j], af[i], b.load(slot)}, 0, 0, 0, name));
             }
