@@ -990,19 +990,65 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
         mfmas(f1a, f1b);
     }
     b.end({r});
-    uint32_t row0 = b.iadd(b.iadd(b.imul(tm, BM), b.imul(wy, um * 16)), l16);
-    uint32_t col0 = b.iadd(b.iadd(b.imul(tn, BN), b.imul(wx, un * 16)), b.imul(lg, 4));
-    for (int i = 0; i < um; i++)
-        for (int j = 0; j < un; j++) {
-            uint32_t res = b.load(acc[i * un + j]);
-            std::vector<uint32_t> el;
-            for (int e = 0; e < 4; e++) {
-                uint32_t v = b.gep(res, e);
-                el.push_back(out != tc.dtype_out ? b.cast(v, out) : v);
+    // Result.  A lane holds, per 16x16 tile, four consecutive columns of one row.  When the result has
+    // the operands' 16-bit type the wave first lays its um*16 x un*16 block out in local memory
+    // (the tiles' stages are free after one more barrier; the first half of the waves uses the A
+    // stages, the second half the B stages; 16-byte pieces XOR-swizzled by the row) and then
+    // writes whole 16-byte pieces, un*32 contiguous bytes per row; otherwise every lane stores its
+    // four values directly.
+    const int RW = um * 16, CW = un * 16, pieces = CW / 8;  // per-wave block, 16-byte pieces per row
+    const bool staged = out == tc.dtype_in && W % 2 == 0 && pieces >= 2 && 64 % pieces == 0 &&
+                        (int64_t)BM * BN / 2 <= 128LL * std::min(BM, BN);
+    if (!staged) {
+        uint32_t row0 = b.iadd(b.iadd(b.imul(tm, BM), b.imul(wy, um * 16)), l16);
+        uint32_t col0 = b.iadd(b.iadd(b.imul(tn, BN), b.imul(wx, un * 16)), b.imul(lg, 4));
+        for (int i = 0; i < um; i++)
+            for (int j = 0; j < un; j++) {
+                uint32_t res = b.load(acc[i * un + j]);
+                std::vector<uint32_t> el;
+                for (int e = 0; e < 4; e++) {
+                    uint32_t v = b.gep(res, e);
+                    el.push_back(out != tc.dtype_out ? b.cast(v, out) : v);
+                }
+                uint32_t at = b.iadd(b.imul(b.iadd(row0, b.ci(i * 16)), N), b.iadd(col0, b.ci(j * 16)));
+                b.store(b.index(c, at), b.vectorize(el));
             }
-            uint32_t at = b.iadd(b.imul(b.iadd(row0, b.ci(i * 16)), N), b.iadd(col0, b.ci(j * 16)));
-            b.store(b.index(c, at), b.vectorize(el));
+    } else {
+        b.barrier();  // every wave has made its last fragment read
+        const int mask = std::min(8, pieces) - 1, rows_per_read = 64 / pieces, reads = RW / rows_per_read;
+        uint32_t low_half = bin(BinaryOp::Lt, wave, b.ci(W / 2));
+        // writes: row i*16 + l16, columns j*16 + lg*4 .. + 3 = piece 2j + lg/2, half lg%2
+        uint32_t w_sw = bin(BinaryOp::And, l16, b.ci(mask));
+        uint32_t w_base = b.iadd(b.imul(l16, CW), b.imul(b.imod(lg, 2), 4));
+        // reads: lane -> row lane / pieces (+ rows_per_read per step), piece lane % pieces
+        uint32_t r_row = b.idiv(lane, pieces), r_piece = b.imod(lane, pieces);
+        uint32_t g_row0 = b.iadd(b.iadd(b.imul(tm, BM), b.imul(wy, RW)), r_row);
+        uint32_t g_col = b.iadd(b.iadd(b.imul(tn, BN), b.imul(wx, CW)), b.imul(r_piece, 8));
+        for (int half = 0; half < 2; half++) {
+            b.if_(half == 0 ? low_half : b.unary(UnaryOp::Not, low_half));
+            uint32_t region = half == 0 ? sA : sB;
+            uint32_t base = b.imul(half == 0 ? wave : bin(BinaryOp::Sub, wave, b.ci(W / 2)), RW * CW);
+            for (int i = 0; i < um; i++)
+                for (int j = 0; j < un; j++) {
+                    uint32_t res = b.load(acc[i * un + j]);
+                    std::vector<uint32_t> el;
+                    for (int e = 0; e < 4; e++) el.push_back(b.cast(b.gep(res, e), out));
+                    // rows i*16 + l16: the swizzle key (row & mask) is l16 & mask whatever i
+                    uint32_t piece = bin(BinaryOp::Xor, b.iadd(b.idiv(lg, 2), b.ci(2 * j)), w_sw);
+                    uint32_t at = b.iadd(b.iadd(base, b.iadd(w_base, b.ci(i * 16 * CW))), b.imul(piece, 8));
+                    b.store(b.index(region, at), b.vectorize(el));
+                }
+            for (int t = 0; t < reads; t++) {
+                // row r_row + t * rows_per_read; rows_per_read is a multiple of 8 or divides 8: keep the key exact
+                uint32_t row = b.iadd(r_row, b.ci(t * rows_per_read));
+                uint32_t piece = bin(BinaryOp::Xor, r_piece, bin(BinaryOp::And, row, b.ci(mask)));
+                uint32_t v = b.load(b.index(region, b.iadd(b.iadd(base, b.imul(row, CW)), b.imul(piece, 8))), 8);
+                uint32_t at = b.iadd(b.imul(b.iadd(g_row0, b.ci(t * rows_per_read)), N), g_col);
+                b.store(b.index(c, at), v);
+            }
+            b.endif();
         }
+    }
     *k = b.finish();
     return kOk;
 }

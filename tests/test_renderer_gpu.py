@@ -367,6 +367,23 @@ def test_tc_matmul_direct_copy_choices_agree(dev, shape, opts):
     assert np.array_equal(run_fenced(synth.to_bf16(a1)), b[(np.arange(M) * 7) % K])
 
 
+def test_tc_matmul_direct_copy_f32_result(dev):
+    """An f32 result leaves the accumulators directly (no staging through local memory): the bits
+    of the register-only generated kernel with the same result type; f16 operands take the f16
+    transposing load."""
+    from morok_amd import sched
+
+    M, N, K = 256, 256, 192
+    a, b = synth.normal_bf16((M, K), 9, 51), synth.normal_bf16((K, N), 9, 52)
+    got = run(dev, sched.build_wmma_matmul_lds_opts(3, M, N, K, U.F32, (2, 2, 4, 4, 0, 2)), "r_tc_dma_f32", (M, N), np.float32, [a, b])
+    want = run(dev, sched.build_wmma_matmul(3, M, N, K, U.F32), "r_tc", (M, N), np.float32, [a, b])
+    assert np.array_equal(got, want)
+    ah, bh = synth.normal((M, K), 9, 53).astype(np.float16), synth.normal((K, N), 9, 54).astype(np.float16)
+    got = run(dev, sched.build_wmma_matmul_lds_opts(2, M, N, K, U.F16, (2, 4, 4, 2, 0, 2)), "r_tc_dma_h", (M, N), np.float16, [ah, bh])
+    want = run(dev, sched.build_wmma_matmul(2, M, N, K, U.F16), "r_tc_h", (M, N), np.float16, [ah, bh])
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("shape,opts", [((200, 136, 72), (2, 2, 4, 4, 0)), ((1, 8, 8), (1, 1, 1, 1, 0)), ((130, 264, 200), (2, 2, 2, 2, 2)),
                                         ((257, 256, 64), (4, 4, 4, 4, 0)), ((128, 128, 40), (2, 2, 4, 4, 0)), ((100, 128, 64), (1, 4, 4, 1, 2))])
 def test_tc_matmul_lds_padded_shapes(dev, shape, opts):

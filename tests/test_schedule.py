@@ -212,8 +212,10 @@ def test_wmma_matmul_lds_kernel_refuses_bad_choices(opts):
 def test_wmma_matmul_direct_copy_kernel_builds_and_compiles():
     """stages = 2: both tiles in two stages of local memory filled by direct global -> local copies
     (extension ops ASYNC_COPY / WAIT_ASYNC), B fragments through the transposing load (LOAD_TR),
-    one barrier per 64-deep K step plus the one that opens the loop, a flat grid whose workgroups
-    are mapped to tiles per XCD, and 8-byte vector stores of result rows."""
+    one barrier per 64-deep K step plus the one that opens the loop and the one in front of the
+    result staging, a flat grid whose workgroups are mapped to tiles per XCD; a 16-bit result is
+    staged through the (then free) tile stages and written as 16-byte pieces, an f32 result as
+    vectors of four straight from the accumulators."""
     import morok_amd
     from morok_amd import sched, uop as U
 
@@ -224,11 +226,13 @@ def test_wmma_matmul_direct_copy_kernel_builds_and_compiles():
     assert "__shared__ __bf16 local0[32768];" in src and "__shared__ __bf16 local1[32768];" in src   # 2 stages x 256 x 64 each
     copies_per_wave = (256 // 8 + 256 // 8) // 8
     assert src.count("global_load_lds_dwordx4") == 3 * copies_per_wave    # tiles 0 and 1 up front, tile r + 2 in the loop
-    assert src.count("__syncthreads();") == 2
+    assert src.count("__syncthreads();") == 3
     assert 's_waitcnt vmcnt(%d)' % copies_per_wave in src and src.count("s_waitcnt vmcnt(0)") == 1
     assert src.count("__builtin_amdgcn_ds_read_tr16_b64_v4bf16(") == 3 * 2 * 4   # 4 column tiles x (lo, hi) x (first half ahead, second, first)
     assert src.count("__WMMA_16_16_32_bfloat_float(") == 2 * 32 + 1
-    assert "*((mrk_bhalf4*)((data0 +" in src                               # result rows as vectors of four
+    assert "*((mrk_bhalf8*)((data0 +" in src and "*((mrk_bhalf4*)((data0 +" not in src   # 16-byte pieces of result rows
+    f32_out = U.render(sched.build_wmma_matmul_lds_opts(3, M, N, K, U.F32, (2, 4, 8, 4, 0, 2)), "r_tc_dma_f32").src
+    assert "*((mrk_float4*)((data0 +" in f32_out and f32_out.count("__syncthreads();") == 2
     assert "gidx0 % 8" in src                                              # the XCD regrouping
     morok_amd.compile_spec(spec)
     # a single K step has no loop-carried copies; half precision takes the f16 transposing load
