@@ -384,7 +384,10 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
                 *LDS_PTR(bf16x4, sC + ml * kCPitchT + nl * 2) = h;
             }
     if constexpr (kResidual) fetch_residual(kFirstBatch, kIts);
-    __syncthreads();
+    // a wave reads back only what it staged itself (the LDS serves a wave's requests in order),
+    // except for the gated epilogue, where gate and up blocks come from two waves
+    if constexpr (kSwiGLU) __syncthreads();
+    else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     if constexpr (kSwiGLU) {
         // waves (wm, 0) and (wm, 1) staged the gate and the up block of the same 128 rows x 128
         // columns; each of the two now combines 64 of those rows: 16 chunks of 8 columns per row
