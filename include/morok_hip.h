@@ -315,7 +315,10 @@ void mrk_hip_queue_destroy(mrk_queue* q);
  * local_max, upcast_max, tensor_cores (WMMA names in table order). */
 const char* mrk_hip_sched_caps(void);
 /* select_tensor_core (schedule/src/optimizer/tc.rs:126-168) over cdna4_tensor_cores()
- * (renderer.rs:724-733): scalar dtype tags as in morok_amd/csrc/uop.h; -1 if none matches. */
+ * (renderer.rs:724-733): scalar dtype tags as in morok_amd/csrc/uop.h; -1 if none matches.
+ * The table holds the reference's six entries in its order (indices 0-5: fp8e5m2, fp8e4m3, f16,
+ * bf16 as 16x16x32; f16, bf16 as 16x16x16) and, behind them, two that the reference does not
+ * have: f16 and bf16 as 32x32x16 (indices 6, 7), reachable by index only. */
 int mrk_hip_sched_tc_select(int in0_scalar, int in1_scalar, int acc_scalar);
 /* TensorCore fields (renderer.rs:358-417): dims (N, M, K), threads, elements per lane (A, B, C). */
 int mrk_hip_sched_tc_info(int tc_index, int dims[3], int* threads, int elements_per_thread[3]);

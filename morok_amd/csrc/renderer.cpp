@@ -381,22 +381,24 @@ bool wmma_wrapper(const std::string& name, Scalar operand, std::string* def) {
         const char* name;
         const char* builtin;
         const char* in_t;
-        int in_n;
+        int in_n, acc_n;
     };
     static const Entry table[] = {
-        {"WMMA_16_16_32_bfloat_float", "__builtin_amdgcn_mfma_f32_16x16x32_bf16", "__bf16", 8},
-        {"WMMA_16_16_32_half_float", "__builtin_amdgcn_mfma_f32_16x16x32_f16", "_Float16", 8},
-        {"WMMA_16_16_16_half_float", "__builtin_amdgcn_mfma_f32_16x16x16f16", "_Float16", 4},
-        {"WMMA_16_16_16_bfloat_float", "__builtin_amdgcn_mfma_f32_16x16x16bf16_1k", "__bf16", 4},
+        {"WMMA_16_16_32_bfloat_float", "__builtin_amdgcn_mfma_f32_16x16x32_bf16", "__bf16", 8, 4},
+        {"WMMA_16_16_32_half_float", "__builtin_amdgcn_mfma_f32_16x16x32_f16", "_Float16", 8, 4},
+        {"WMMA_16_16_16_half_float", "__builtin_amdgcn_mfma_f32_16x16x16f16", "_Float16", 4, 4},
+        {"WMMA_16_16_16_bfloat_float", "__builtin_amdgcn_mfma_f32_16x16x16bf16_1k", "__bf16", 4, 4},
+        {"WMMA_32_32_16_bfloat_float", "__builtin_amdgcn_mfma_f32_32x32x16_bf16", "__bf16", 8, 16},
+        {"WMMA_32_32_16_half_float", "__builtin_amdgcn_mfma_f32_32x32x16_f16", "_Float16", 8, 16},
     };
     for (const Entry& e : table) {
         if (name == e.name) {
             *def = fmt(
                 "typedef %s __%s_in __attribute__((ext_vector_type(%d)));\n"
-                "typedef float __%s_acc __attribute__((ext_vector_type(4)));\n"
+                "typedef float __%s_acc __attribute__((ext_vector_type(%d)));\n"
                 "static __device__ __forceinline__ __%s_acc __%s(__%s_in a, __%s_in b, __%s_acc c) {\n"
                 "  return %s(a, b, c, 0, 0, 0);\n}\n",
-                e.in_t, e.name, e.in_n, e.name, e.name, e.name, e.name, e.name, e.name, e.builtin);
+                e.in_t, e.name, e.in_n, e.name, e.acc_n, e.name, e.name, e.name, e.name, e.name, e.builtin);
             return true;
         }
     }
@@ -968,10 +970,18 @@ class HipRenderer final : public Renderer {
                 if (!g || g->op != Op::Param || !l || l->op != Op::DefineLocal)
                     return fail(kRenderError, "render: ASYNC_COPY copies from a PARAM to a DEFINE_LOCAL");
                 // M0 holds the wave's local-memory destination; the copy itself is invisible to the
-                // compiler's wait-count bookkeeping, WAIT_ASYNC is its only ordering
+                // compiler's wait-count bookkeeping, WAIT_ASYNC is its only ordering.  The destination
+                // is formed as the array's own local-memory offset plus an integer byte offset: cast
+                // back from a generic pointer it would carry a null check per copy.
+                std::string dst;
+                const UOp& li = node(u.src[1]);
+                if (li.op == Op::Index && li.src.size() == 2 && !li.sub && node(li.src[0]).op == Op::DefineLocal)
+                    dst = "(unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + ctx.get(li.src[0]) + ") + (unsigned)(" +
+                          ctx.get(li.src[1]) + ") * " + std::to_string(scalar_bytes(l->dtype.scalar) * l->dtype.vcount) + "u";
+                else
+                    dst = "(unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + S(1) + ")";
                 ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, off\" : : \"s\"(" +
-                                   "__builtin_amdgcn_readfirstlane((unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + S(1) +
-                                   "))), \"v\"((const char*)(" + S(0) + ")) : \"m0\", \"memory\");");
+                                   "__builtin_amdgcn_readfirstlane(" + dst + ")), \"v\"((const char*)(" + S(0) + ")) : \"m0\", \"memory\");");
                 return kOk;
             }
             case Op::WaitAsync:

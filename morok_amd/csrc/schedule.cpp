@@ -50,6 +50,24 @@ TensorCore cdna_161632(Scalar in, Scalar out) {
     return t;
 }
 
+// Not in the reference's tables: the 32x32x16 shape of gfx950, the one its matrix pipes sustain
+// the highest rate with (register-only streams: 1.70 PFLOP/s against 1.45 for 16x16x32, whose
+// instructions move a third more operand bytes per flop).  Lane l holds row / column l % 32 and the
+// 8 consecutive k of group l / 32 of A and B; accumulator register e of lane l is
+// C[8 * (e / 4) + 4 * (l / 32) + e % 4][l % 32].
+TensorCore cdna4_323216(Scalar in, Scalar out) {
+    TensorCore t;
+    t.dims = {32, 32, 16};
+    t.threads = 64;
+    t.elements_per_thread = {8, 8, 16};
+    t.dtype_in = in;
+    t.dtype_out = out;
+    t.opts = opts_from("l0 l0 l0 l0 l0 u1 u1 l1 u1 u1");
+    t.swizzle[0] = {sw({"u0", "u1", "l5", "u2", "u3", "r3"}), sw({"r0", "r1", "r2", "l0"}), sw({"l1", "l2", "l3", "l4"})};
+    t.swizzle[1] = {sw({"l0", "l1", "l2", "l3", "l4", "r3"}), sw({"r0", "r1", "r2", "u0"}), sw({"l5", "u1", "u2", "u3"})};
+    return t;
+}
+
 const char* tc_dtype_name(Scalar s) {  // tc.rs:677-688
     switch (s) {
         case Scalar::Float16: return "half";
@@ -90,6 +108,9 @@ std::vector<TensorCore> cdna4_tensor_cores() {  // renderer.rs:724-733, same ord
         cdna_161632(Scalar::BFloat16, Scalar::Float32),
         cdna_161616(Scalar::Float16, Scalar::Float32),
         cdna_161616(Scalar::BFloat16, Scalar::Float32),
+        // additions for gfx950, behind the reference's entries so that selection by dtype is unchanged
+        cdna4_323216(Scalar::Float16, Scalar::Float32),
+        cdna4_323216(Scalar::BFloat16, Scalar::Float32),
     };
 }
 
@@ -798,13 +819,15 @@ bool wmma_lds_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, 
 // per-lane sources; the swizzles are applied on the source side.
 static bool wmma_async_tile(const TensorCore& tc, const WmmaLdsOpts& o, int* bm, int* bn) {
     auto pow2_upto = [](int v, int hi) { return v >= 1 && v <= hi && (v & (v - 1)) == 0; };
-    if (tc.threads != 64 || tc.dims[0] != 16 || tc.dims[1] != 16 || tc.dims[2] != 32) return false;
+    const bool t16 = tc.dims[0] == 16 && tc.dims[1] == 16 && tc.dims[2] == 32, t32 = tc.dims[0] == 32 && tc.dims[1] == 32 && tc.dims[2] == 16;
+    if (tc.threads != 64 || (!t16 && !t32)) return false;
     if (tc.dtype_in != Scalar::BFloat16 && tc.dtype_in != Scalar::Float16) return false;
     if (!pow2_upto(o.waves_m, 8) || !pow2_upto(o.waves_n, 8) || o.waves_m * o.waves_n > 16) return false;
     if (!pow2_upto(o.up_m, 8) || !pow2_upto(o.up_n, 8)) return false;
-    if (o.unroll_k != 0 && o.unroll_k != 2) return false;
-    *bm = o.waves_m * o.up_m * 16;
-    *bn = o.waves_n * o.up_n * 16;
+    if (o.up_m * o.up_n * tc.elements_per_thread[2] > 256) return false;  // accumulator registers per lane
+    if (o.unroll_k != 0 && o.unroll_k != 64 / tc.dims[2]) return false;
+    *bm = o.waves_m * o.up_m * tc.dims[1];
+    *bn = o.waves_n * o.up_n * tc.dims[0];
     return true;
 }
 
@@ -829,21 +852,28 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
                      "tensor-core matmul (direct copies): shape %lldx%lldx%lld does not divide into the workgroup tile with a K step of 64, "
                      "or the tile does not fit two stages of local memory",
                      (long long)M, (long long)N, (long long)K);
-    // the lane <-> element maps this builder writes out by hand; checked against the table
-    for (int l = 0; l < 64; l++)
-        for (int e = 0; e < 8; e++) {
-            int mn, kk;
+    // TD x TD tiles, tk deep; a lane holds row / column l % TD and the 8 consecutive k of group l / TD
+    // of each operand; the accumulator of lane l is column l % TD and, in groups of four registers,
+    // rows q * (256 / TD) + 4 * (l / TD) + 0..3.  Written out by hand below, checked against the table here.
+    const int TD = tc.dims[0], tk = tc.dims[2], KG = 64 / TD, EC = tc.elements_per_thread[2];
+    if (tc.elements_per_thread[0] != 8 || tc.elements_per_thread[1] != 8 || EC != TD * TD / 64)
+        return fail(kInvalidArgument, "tensor-core matmul (direct copies): unexpected elements per lane");
+    for (int l = 0; l < 64; l++) {
+        for (int e = 0; e < 8; e++)
             for (int operand = 0; operand < 2; operand++) {
+                int mn, kk;
                 tc_operand_element(tc, operand, l, e, &mn, &kk);
-                if (mn != l % 16 || kk != 8 * (l / 16) + e) return fail(kInvalidArgument, "tensor-core matmul (direct copies): unexpected operand layout");
+                if (mn != l % TD || kk != 8 * (l / TD) + e) return fail(kInvalidArgument, "tensor-core matmul (direct copies): unexpected operand layout");
             }
-            if (e < 4) {
-                int m, n;
-                tc_acc_element(tc, l, e, &m, &n);
-                if (m != 4 * (l / 16) + e || n != l % 16) return fail(kInvalidArgument, "tensor-core matmul (direct copies): unexpected accumulator layout");
-            }
+        for (int e = 0; e < EC; e++) {
+            int m, n;
+            tc_acc_element(tc, l, e, &m, &n);
+            if (m != (e / 4) * (256 / TD) + 4 * (l / TD) + e % 4 || n != l % TD)
+                return fail(kInvalidArgument, "tensor-core matmul (direct copies): unexpected accumulator layout");
         }
+    }
     const int um = opts.up_m, un = opts.up_n, WM = opts.waves_m, WN = opts.waves_n, W = WM * WN;
+    const int KS = 64 / tk, HS = KS / 2;  // tensor-core K steps per 64-deep tile, per half of it
     const int64_t KT = K / 64, tiles_m = M / BM, tiles_n = N / BN, T = tiles_m * tiles_n;
     const int A_STAGE = BM * 64, B_STAGE = 64 * BN;  // elements
     const int CA = BM / 8 / W, CB = BN / 8 / W, PRB = BN / 8;
@@ -877,7 +907,8 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
         }
     }
     uint32_t wy = b.idiv(wave, WN), wx = b.imod(wave, WN);
-    uint32_t l16 = b.imod(lane, 16), lg = b.idiv(lane, 16);
+    uint32_t lr = b.imod(lane, TD), lgk = b.idiv(lane, TD);  // row / column inside a tile, k group
+    uint32_t i16 = b.imod(lane, 16);                         // lane inside its group of 16 (transposing loads)
     uint32_t sA = b.define_local(0, tc.dtype_in, 2LL * A_STAGE), sB = b.define_local(1, tc.dtype_in, 2LL * B_STAGE);
 
     // copies: per wave CA chunks of A and CB chunks of B per tile
@@ -906,73 +937,82 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
         for (int q = 0; q < CA; q++) b.async_copy(b.index(a, b.iadd(a_src[q], ka)), b.index(sA, b.iadd(a_dst[q], oa)));
         for (int q = 0; q < CB; q++) b.async_copy(b.index(bmat, b.iadd(b_src[q], kb)), b.index(sB, b.iadd(b_dst[q], ob)));
     };
-    // fragment addresses: lane-dependent base per k step (A) / per column tile (B) + constants
-    uint32_t a_sw = b.idiv(l16, 2);
-    uint32_t a_row = b.iadd(b.imul(wy, um * 16), l16);
-    uint32_t a_base[2], b_base[8];
-    for (int kk = 0; kk < 2; kk++)
-        a_base[kk] = b.iadd(b.imul(a_row, 64), b.imul(bin(BinaryOp::Xor, b.iadd(lg, b.ci(kk * 4)), a_sw), 8));
-    uint32_t b_kq = b.idiv(l16, 4);
+    // fragment addresses: lane-dependent base per K step (A) / per column tile (B) + constants.
+    // A, K step s: logical 16-byte piece s * KG + lgk of row wy*um*TD + i*TD + lr (swizzle key (lr >> 1) & 7).
+    // B, K step s: the 16 lanes of a group address rows k = s*tk + 8*lgk + i16/4 (+4 for the upper
+    // half) of granule (wx*un + j) * (TD/16) + (lr / 16), physically XORed with k & 3 = i16 / 4.
+    uint32_t a_sw = bin(BinaryOp::And, b.idiv(lr, 2), b.ci(7));
+    uint32_t a_row = b.iadd(b.imul(wy, um * TD), lr);
+    std::vector<uint32_t> a_base(KS), b_base(un);
+    for (int sst = 0; sst < KS; sst++)
+        a_base[sst] = b.iadd(b.imul(a_row, 64), b.imul(bin(BinaryOp::Xor, b.iadd(lgk, b.ci(sst * KG)), a_sw), 8));
+    uint32_t b_kq = b.idiv(i16, 4);
     for (int j = 0; j < un; j++) {
-        uint32_t gran = bin(BinaryOp::Xor, b.iadd(b.imul(wx, un), b.ci(j)), b_kq);
-        b_base[j] = b.iadd(b.imul(b.iadd(b.imul(lg, 8), b_kq), BN), b.iadd(b.imul(gran, 16), b.imul(b.imod(l16, 4), 4)));
+        uint32_t gl = b.iadd(b.imul(b.iadd(b.imul(wx, un), b.ci(j)), TD / 16), b.idiv(lr, 16));
+        uint32_t gran = bin(BinaryOp::Xor, gl, b_kq);
+        b_base[j] = b.iadd(b.imul(b.iadd(b.imul(lgk, 8), b_kq), BN), b.iadd(b.imul(gran, 16), b.imul(b.imod(i16, 4), 4)));
     }
-    auto read_a = [&](int kk, int i, uint32_t oa) {
-        return b.load(b.index(sA, b.iadd(b.iadd(a_base[kk], oa), b.ci(i * 16 * 64))), 8);
+    auto read_a = [&](int sst, int i, uint32_t oa) {
+        return b.load(b.index(sA, b.iadd(b.iadd(a_base[sst], oa), b.ci(i * TD * 64))), 8);
     };
-    auto read_b = [&](int kk, int j, uint32_t ob) {
+    auto read_b = [&](int sst, int j, uint32_t ob) {
         uint32_t at = b.iadd(b_base[j], ob);
-        uint32_t lo = b.load_tr(b.index(sB, b.iadd(at, b.ci(kk * 32 * BN))));
-        uint32_t hi = b.load_tr(b.index(sB, b.iadd(at, b.ci((kk * 32 + 4) * BN))));
+        uint32_t lo = b.load_tr(b.index(sB, b.iadd(at, b.ci(sst * tk * BN))));
+        uint32_t hi = b.load_tr(b.index(sB, b.iadd(at, b.ci((sst * tk + 4) * BN))));
         std::vector<uint32_t> el;
         for (int e = 0; e < 4; e++) el.push_back(b.gep(lo, e));
         for (int e = 0; e < 4; e++) el.push_back(b.gep(hi, e));
         return b.vectorize(el);
     };
-    // registers: accumulators (one object per tile) and the fragments of the first k step, which
-    // are read one half step ahead and so live across the loop edge
-    std::vector<uint32_t> acc(um * un), fa0(um), fb0(un);
+    // registers: accumulators (one object per tile) and the fragments of the first half of a
+    // tile's K steps, which are read half a step ahead and so live across the loop edge
+    std::vector<uint32_t> acc(um * un), fa0(HS * um), fb0(HS * un);
     int reg_id = 1;
     {
-        std::vector<uint32_t> z(4, b.cf(0.0, tc.dtype_out));
+        std::vector<uint32_t> z(EC, b.cf(0.0, tc.dtype_out));
         uint32_t zv = b.vectorize(z);
         for (int i = 0; i < um * un; i++) {
-            acc[i] = b.index(b.define_reg(reg_id++, tc.dtype_out, 1, 4), b.ci(0));
+            acc[i] = b.index(b.define_reg(reg_id++, tc.dtype_out, 1, EC), b.ci(0));
             b.store(acc[i], zv);
         }
-        for (int i = 0; i < um; i++) fa0[i] = b.index(b.define_reg(reg_id++, tc.dtype_in, 1, 8), b.ci(0));
-        for (int j = 0; j < un; j++) fb0[j] = b.index(b.define_reg(reg_id++, tc.dtype_in, 1, 8), b.ci(0));
+        for (size_t i = 0; i < fa0.size(); i++) fa0[i] = b.index(b.define_reg(reg_id++, tc.dtype_in, 1, 8), b.ci(0));
+        for (size_t j = 0; j < fb0.size(); j++) fb0[j] = b.index(b.define_reg(reg_id++, tc.dtype_in, 1, 8), b.ci(0));
     }
     const std::string name = wmma_name(tc);
-    const DType cd = KernelBuilder::scalar(tc.dtype_out, 4);
+    const DType cd = KernelBuilder::scalar(tc.dtype_out, EC);
     // the B fragment goes in as the first operand: the tensor core then leaves four consecutive
     // columns of one row in a lane (result rows are written as vectors), same products, same order
-    auto mfmas = [&](const std::vector<uint32_t>& af, const std::vector<uint32_t>& bf) {
+    auto mfmas = [&](const std::vector<uint32_t>& af, const std::vector<uint32_t>& bf) {  // [h * um + i], [h * un + j]
         // columns back and forth, so that consecutive tensor-core instructions always share one
         // operand (fewer operand bits toggle; the part's clock under matrix load follows that)
-        for (int i = 0; i < um; i++)
-            for (int jj = 0; jj < un; jj++) {
-                const int j = (i & 1) ? un - 1 - jj : jj;
-                uint32_t slot = acc[i * un + j];
-                b.store(slot, b.add(Op::Wmma, cd, {bf[j], af[i], b.load(slot)}, 0, 0, 0, name));
-            }
+        for (int h = 0; h < HS; h++)
+            for (int i = 0; i < um; i++)
+                for (int jj = 0; jj < un; jj++) {
+                    const int j = (i & 1) ? un - 1 - jj : jj;
+                    uint32_t slot = acc[i * un + j];
+                    b.store(slot, b.add(Op::Wmma, cd, {bf[h * un + j], af[h * um + i], b.load(slot)}, 0, 0, 0, name));
+                }
     };
     const int cpw = CA + CB;
     copy_tile(b.ci(0), b.ci(0));
     if (KT > 1) copy_tile(b.ci(1), b.ci(1));
     b.wait_async(KT > 1 ? cpw : 0);
     b.barrier();
-    for (int i = 0; i < um; i++) b.store(fa0[i], read_a(0, i, b.ci(0)));
-    for (int j = 0; j < un; j++) b.store(fb0[j], read_b(0, j, b.ci(0)));
+    for (int h = 0; h < HS; h++) {
+        for (int i = 0; i < um; i++) b.store(fa0[h * um + i], read_a(h, i, b.ci(0)));
+        for (int j = 0; j < un; j++) b.store(fb0[h * un + j], read_b(h, j, b.ci(0)));
+    }
     uint32_t r = b.range(KT, 0, AxisType::Reduce);
     {
         uint32_t st = b.imod(r, 2), sn = bin(BinaryOp::Sub, b.ci(1), st);
         uint32_t oa = b.imul(st, A_STAGE), ob = b.imul(st, B_STAGE), na = b.imul(sn, A_STAGE), nb = b.imul(sn, B_STAGE);
-        std::vector<uint32_t> f1a(um), f1b(un), f0a(um), f0b(un);
-        for (int i = 0; i < um; i++) f1a[i] = read_a(1, i, oa);
-        for (int j = 0; j < un; j++) f1b[j] = read_b(1, j, ob);
-        for (int i = 0; i < um; i++) f0a[i] = b.load(fa0[i]);
-        for (int j = 0; j < un; j++) f0b[j] = b.load(fb0[j]);
+        std::vector<uint32_t> f1a(HS * um), f1b(HS * un), f0a(HS * um), f0b(HS * un);
+        for (int h = 0; h < HS; h++) {
+            for (int i = 0; i < um; i++) f1a[h * um + i] = read_a(HS + h, i, oa);
+            for (int j = 0; j < un; j++) f1b[h * un + j] = read_b(HS + h, j, ob);
+        }
+        for (size_t i = 0; i < fa0.size(); i++) f0a[i] = b.load(fa0[i]);
+        for (size_t j = 0; j < fb0.size(); j++) f0b[j] = b.load(fb0[j]);
         mfmas(f0a, f0b);
         // tile r + 1 has landed in the other stage (issued half a step ago or earlier) and, behind
         // the barrier, nobody reads this stage any more
@@ -985,41 +1025,46 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             b.endif();
         }
         // first half of tile r + 1 (after the last tile: a stale stage, read and never used)
-        for (int i = 0; i < um; i++) b.store(fa0[i], read_a(0, i, na));
-        for (int j = 0; j < un; j++) b.store(fb0[j], read_b(0, j, nb));
+        for (int h = 0; h < HS; h++) {
+            for (int i = 0; i < um; i++) b.store(fa0[h * um + i], read_a(h, i, na));
+            for (int j = 0; j < un; j++) b.store(fb0[h * un + j], read_b(h, j, nb));
+        }
         mfmas(f1a, f1b);
     }
     b.end({r});
-    // Result.  A lane holds, per 16x16 tile, four consecutive columns of one row.  When the result has
-    // the operands' 16-bit type the wave first lays its um*16 x un*16 block out in local memory
+    // Result.  A lane holds, per tile, groups of four consecutive columns of one row.  When the result
+    // has the operands' 16-bit type the wave first lays its um*TD x un*TD block out in local memory
     // (the tiles' stages are free after one more barrier; the first half of the waves uses the A
     // stages, the second half the B stages; 16-byte pieces XOR-swizzled by the row) and then
-    // writes whole 16-byte pieces, un*32 contiguous bytes per row; otherwise every lane stores its
-    // four values directly.
-    const int RW = um * 16, CW = un * 16, pieces = CW / 8;  // per-wave block, 16-byte pieces per row
-    const bool staged = out == tc.dtype_in && W % 2 == 0 && pieces >= 2 && 64 % pieces == 0 &&
+    // writes whole 16-byte pieces, contiguous along each row; otherwise every lane stores its
+    // groups of four values directly.
+    const int RW = um * TD, CW = un * TD, pieces = CW / 8;  // per-wave block, 16-byte pieces per row
+    const int QG = EC / 4, qstride = 256 / TD;             // register groups per tile, columns between them
+    const bool staged = out == tc.dtype_in && W % 2 == 0 && pieces >= 2 && 64 % pieces == 0 && RW % (64 / pieces) == 0 &&
                         (int64_t)BM * BN / 2 <= 128LL * std::min(BM, BN);
     if (!staged) {
-        uint32_t row0 = b.iadd(b.iadd(b.imul(tm, BM), b.imul(wy, um * 16)), l16);
-        uint32_t col0 = b.iadd(b.iadd(b.imul(tn, BN), b.imul(wx, un * 16)), b.imul(lg, 4));
+        uint32_t row0 = b.iadd(b.iadd(b.imul(tm, BM), b.imul(wy, RW)), lr);
+        uint32_t col0 = b.iadd(b.iadd(b.imul(tn, BN), b.imul(wx, CW)), b.imul(lgk, 4));
         for (int i = 0; i < um; i++)
             for (int j = 0; j < un; j++) {
                 uint32_t res = b.load(acc[i * un + j]);
-                std::vector<uint32_t> el;
-                for (int e = 0; e < 4; e++) {
-                    uint32_t v = b.gep(res, e);
-                    el.push_back(out != tc.dtype_out ? b.cast(v, out) : v);
+                for (int q = 0; q < QG; q++) {
+                    std::vector<uint32_t> el;
+                    for (int e = 0; e < 4; e++) {
+                        uint32_t v = b.gep(res, 4 * q + e);
+                        el.push_back(out != tc.dtype_out ? b.cast(v, out) : v);
+                    }
+                    uint32_t at = b.iadd(b.imul(b.iadd(row0, b.ci(i * TD)), N), b.iadd(col0, b.ci(j * TD + q * qstride)));
+                    b.store(b.index(c, at), b.vectorize(el));
                 }
-                uint32_t at = b.iadd(b.imul(b.iadd(row0, b.ci(i * 16)), N), b.iadd(col0, b.ci(j * 16)));
-                b.store(b.index(c, at), b.vectorize(el));
             }
     } else {
         b.barrier();  // every wave has made its last fragment read
         const int mask = std::min(8, pieces) - 1, rows_per_read = 64 / pieces, reads = RW / rows_per_read;
         uint32_t low_half = bin(BinaryOp::Lt, wave, b.ci(W / 2));
-        // writes: row i*16 + l16, columns j*16 + lg*4 .. + 3 = piece 2j + lg/2, half lg%2
-        uint32_t w_sw = bin(BinaryOp::And, l16, b.ci(mask));
-        uint32_t w_base = b.iadd(b.imul(l16, CW), b.imul(b.imod(lg, 2), 4));
+        // writes: row i*TD + lr, columns j*TD + q*qstride + 4*lgk .. + 3: piece (j*TD + q*qstride) / 8 + lgk / 2, half lgk % 2
+        uint32_t w_sw = bin(BinaryOp::And, lr, b.ci(mask));
+        uint32_t w_base = b.iadd(b.imul(lr, CW), b.imul(b.imod(lgk, 2), 4));
         // reads: lane -> row lane / pieces (+ rows_per_read per step), piece lane % pieces
         uint32_t r_row = b.idiv(lane, pieces), r_piece = b.imod(lane, pieces);
         uint32_t g_row0 = b.iadd(b.iadd(b.imul(tm, BM), b.imul(wy, RW)), r_row);
@@ -1031,15 +1076,16 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             for (int i = 0; i < um; i++)
                 for (int j = 0; j < un; j++) {
                     uint32_t res = b.load(acc[i * un + j]);
-                    std::vector<uint32_t> el;
-                    for (int e = 0; e < 4; e++) el.push_back(b.cast(b.gep(res, e), out));
-                    // rows i*16 + l16: the swizzle key (row & mask) is l16 & mask whatever i
-                    uint32_t piece = bin(BinaryOp::Xor, b.iadd(b.idiv(lg, 2), b.ci(2 * j)), w_sw);
-                    uint32_t at = b.iadd(b.iadd(base, b.iadd(w_base, b.ci(i * 16 * CW))), b.imul(piece, 8));
-                    b.store(b.index(region, at), b.vectorize(el));
+                    for (int q = 0; q < QG; q++) {
+                        std::vector<uint32_t> el;
+                        for (int e = 0; e < 4; e++) el.push_back(b.cast(b.gep(res, 4 * q + e), out));
+                        // rows i*TD + lr: the swizzle key (row & mask) is lr & mask whatever i
+                        uint32_t piece = bin(BinaryOp::Xor, b.iadd(b.idiv(lgk, 2), b.ci((j * TD + q * qstride) / 8)), w_sw);
+                        uint32_t at = b.iadd(b.iadd(base, b.iadd(w_base, b.ci(i * TD * CW))), b.imul(piece, 8));
+                        b.store(b.index(region, at), b.vectorize(el));
+                    }
                 }
             for (int t = 0; t < reads; t++) {
-                // row r_row + t * rows_per_read; rows_per_read is a multiple of 8 or divides 8: keep the key exact
                 uint32_t row = b.iadd(r_row, b.ci(t * rows_per_read));
                 uint32_t piece = bin(BinaryOp::Xor, r_piece, bin(BinaryOp::And, row, b.ci(mask)));
                 uint32_t v = b.load(b.index(region, b.iadd(b.iadd(base, b.imul(row, CW)), b.imul(piece, 8))), 8);

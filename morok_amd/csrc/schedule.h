@@ -48,7 +48,7 @@ struct RendererCaps {
 // renderer.rs:290-303 with two corrections for the real part: gfx950 has 160 KB of LDS per
 // workgroup (the reference lists 65536) - everything else as upstream.
 RendererCaps amd_cdna4_caps();
-// renderer.rs:724-733 (fp8 entries omitted: no fp8 path is built here)
+// renderer.rs:724-733 entry for entry, then the 32x32x16 shape of gfx950 for f16 and bf16
 std::vector<TensorCore> cdna4_tensor_cores();
 // tc.rs:126-168: first table entry whose input and accumulator dtypes match; -1 if none.
 int select_tensor_core(const std::vector<TensorCore>& tcs, Scalar in0, Scalar in1, Scalar acc);

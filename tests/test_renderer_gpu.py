@@ -367,6 +367,30 @@ def test_tc_matmul_direct_copy_choices_agree(dev, shape, opts):
     assert np.array_equal(run_fenced(synth.to_bf16(a1)), b[(np.arange(M) * 7) % K])
 
 
+@pytest.mark.parametrize("shape,opts", [((512, 512, 256), (2, 4, 4, 2, 0, 2)), ((256, 256, 64), (2, 2, 2, 2, 0, 2)), ((512, 256, 192), (4, 2, 2, 4, 0, 2)),
+                                        ((256, 512, 128), (1, 4, 2, 1, 0, 2)), ((768, 384, 320), (2, 2, 4, 2, 0, 2))])
+def test_tc_matmul_32x32x16_tiles(dev, shape, opts):
+    """The 32x32x16 tensor-core entries (gfx950 additions behind the reference's table): the
+    register-only kernel and the direct-copy variant built from them agree bit for bit with each
+    other, with the 16x16x32 kernels (the matrix core adds the 16-deep and the 32-deep blocks of
+    products in the same order) and with the hand-written GEMM, which uses the same instruction."""
+    from morok_amd import ops, sched
+
+    M, N, K = shape
+    a, b = synth.normal_bf16((M, K), 9, 61), synth.normal_bf16((K, N), 9, 62)
+    plain32 = run(dev, sched.build_wmma_matmul(7, M, N, K, U.BF16), "r_tc32", (M, N), np.uint16, [a, b])
+    plain16 = run(dev, sched.build_wmma_matmul(3, M, N, K, U.BF16), "r_tc16", (M, N), np.uint16, [a, b])
+    dma32 = run(dev, sched.build_wmma_matmul_lds_opts(7, M, N, K, U.BF16, opts), "r_tc32_dma", (M, N), np.uint16, [a, b])
+    ba, bb, bc = (morok_amd.Buffer.from_numpy(a), morok_amd.Buffer.from_numpy(b), dev.buffer(M * N * 2))
+    ops.gemm_bf16(ba, bb, bc, M, N, K, dev.device_id)
+    hand = bc.copyout(np.uint16, (M, N))
+    assert np.array_equal(plain32, plain16) and np.array_equal(dma32, plain32) and np.array_equal(hand, plain32)
+    a1 = np.zeros((M, K), np.float32)
+    a1[np.arange(M), (np.arange(M) * 7) % K] = 1
+    one_hot = run(dev, sched.build_wmma_matmul_lds_opts(7, M, N, K, U.BF16, opts), "r_tc32_dma", (M, N), np.uint16, [synth.to_bf16(a1), b])
+    assert np.array_equal(one_hot, b[(np.arange(M) * 7) % K])
+
+
 def test_tc_matmul_direct_copy_f32_result(dev):
     """An f32 result leaves the accumulators directly (no staging through local memory): the bits
     of the register-only generated kernel with the same result type; f16 operands take the f16

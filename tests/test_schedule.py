@@ -18,8 +18,11 @@ def test_caps_match_reference_descriptor():
     assert c["shared_max"] == 163840  # gfx950 LDS per workgroup (the reference lists 65536)
     # cdna4_tensor_cores(), renderer.rs:724-733: fp8e5m2, fp8e4m3, f16, bf16 (16x16x32), f16, bf16 (16x16x16);
     # the reference's WMMA name table has no entry for the 8-bit floats (tc.rs:677-688: "unknown")
-    assert c["tensor_cores"] == ["WMMA_16_16_32_unknown_float", "WMMA_16_16_32_unknown_float", "WMMA_16_16_32_half_float",
-                                 "WMMA_16_16_32_bfloat_float", "WMMA_16_16_16_half_float", "WMMA_16_16_16_bfloat_float"]
+    assert c["tensor_cores"][:6] == ["WMMA_16_16_32_unknown_float", "WMMA_16_16_32_unknown_float", "WMMA_16_16_32_half_float",
+                                     "WMMA_16_16_32_bfloat_float", "WMMA_16_16_16_half_float", "WMMA_16_16_16_bfloat_float"]
+    # behind them, two entries the reference does not have: the 32x32x16 shape of gfx950 (selection by dtype
+    # still finds the reference's entries first)
+    assert c["tensor_cores"][6:] == ["WMMA_32_32_16_half_float", "WMMA_32_32_16_bfloat_float"]
 
 
 def test_tensor_core_selection():
@@ -38,27 +41,30 @@ def test_tensor_core_selection():
     assert dims == [16, 16, 16] and ept == [4, 4, 4]
     with pytest.raises(MorokHipError):
         sched.tc_info(11)
+    dims, threads, ept = sched.tc_info(7)
+    assert dims == [32, 32, 16] and threads == 64 and ept == [8, 8, 16]
 
 
-@pytest.mark.parametrize("tc", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tc", [0, 1, 2, 3, 4, 5, 6, 7])
 def test_swizzle_tables_equal_mfma_register_layout(tc):
-    """Layout of v_mfma_f32_16x16x{16,32}: lane l holds row/column l % 16 and the contiguous k
-    group l // 16 of A/B; accumulator element i of lane l is C[4 * (l // 16) + i][l % 16].
+    """Layout of v_mfma_f32_16x16x{16,32} and v_mfma_f32_32x32x16: with T the tile extent, lane l holds
+    row/column l % T and the contiguous k group l // T of A/B; accumulator register e of lane l is
+    C[(e // 4) * (256 // T) + 4 * (l // T) + e % 4][l % T] (16x16: 4 * (l // 16) + e).
     (The same formulas drive the one-hot MFMA test on the GPU.)"""
-    (_, _, K), _, (ea, eb, ec) = sched.tc_info(tc)
-    per = K // 4
-    assert ea == per and eb == per
+    (T, T2, K), _, (ea, eb, ec) = sched.tc_info(tc)
+    per = K * T // 64
+    assert T == T2 and ea == per and eb == per and ec == T * T // 64
     seen_a, seen_b, seen_c = set(), set(), set()
     for lane in range(64):
         for e in range(per):
-            assert sched.tc_element(tc, 0, lane, e) == (lane % 16, per * (lane // 16) + e)
-            assert sched.tc_element(tc, 1, lane, e) == (lane % 16, per * (lane // 16) + e)
+            assert sched.tc_element(tc, 0, lane, e) == (lane % T, per * (lane // T) + e)
+            assert sched.tc_element(tc, 1, lane, e) == (lane % T, per * (lane // T) + e)
             seen_a.add(sched.tc_element(tc, 0, lane, e))
             seen_b.add(sched.tc_element(tc, 1, lane, e))
         for e in range(ec):
-            assert sched.tc_element(tc, 2, lane, e) == (4 * (lane // 16) + e, lane % 16)
+            assert sched.tc_element(tc, 2, lane, e) == ((e // 4) * (256 // T) + 4 * (lane // T) + e % 4, lane % T)
             seen_c.add(sched.tc_element(tc, 2, lane, e))
-    assert len(seen_a) == 16 * K and len(seen_b) == 16 * K and len(seen_c) == 256  # every element exactly once
+    assert len(seen_a) == T * K and len(seen_b) == T * K and len(seen_c) == T * T  # every element exactly once
 
 
 # ---- the reference's gpudims unit tests
