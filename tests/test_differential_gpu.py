@@ -95,3 +95,36 @@ def test_generated_tensor_core_random_choices(dev, seed):
     c = synth.from_bf16(got[:M * N].reshape(M, N))
     ref = synth.from_bf16(a).astype(np.float64) @ synth.from_bf16(b).astype(np.float64)
     assert np.all(np.isfinite(c)) and np.abs(c - ref).max() <= 2e-2 * max(np.abs(ref).max(), 1e-6)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_generated_tensor_core_direct_copy_random_choices(dev, seed):
+    """Random workgroup shapes, tile counts and K depths of the direct-copy variant, both tile
+    shapes (16x16x32 and 32x32x16): the bits of the hand-written GEMM (which the register-only
+    kernels also produce), nothing written behind the result."""
+    rng = np.random.default_rng(7400 + seed)
+    tc = int(rng.choice([3, 7]))
+    while True:
+        opts = (int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4, 8])), int(rng.choice([1, 2, 4, 8])), 0, 2)
+        t = 16 if tc == 3 else 32
+        bm, bn = opts[0] * opts[2] * t, opts[1] * opts[3] * t
+        M, N, K = bm * int(rng.integers(1, 5)), bn * int(rng.integers(1, 5)), 64 * int(rng.integers(1, 7))
+        if M * N > 1 << 21:
+            continue
+        try:
+            kern = sched.build_wmma_matmul_lds_opts(tc, M, N, K, U.BF16, opts)
+            break
+        except morok_amd.MorokHipError:
+            continue
+    a, b = synth.normal_bf16((M, K), 7400 + seed, 0), synth.normal_bf16((K, N), 7400 + seed, 1)
+    ba, bb = morok_amd.Buffer.from_numpy(a, dev.device_id), morok_amd.Buffer.from_numpy(b, dev.device_id)
+    bc = morok_amd.Buffer.from_numpy(np.full(M * N + 512, NAN, np.uint16), dev.device_id)
+    k = morok_amd.Kernel.get_or_compile(kern, "r_tc_dma_random")
+    plan = morok_amd.ExecutionPlan()
+    plan.add_kernel(k, [plan.add_buffer(bc), plan.add_buffer(ba), plan.add_buffer(bb)])
+    plan.build().execute()
+    got = bc.copyout(np.uint16, (M * N + 512,))
+    assert np.all(got[M * N:] == NAN)
+    bh = dev.buffer(M * N * 2)
+    ops.gemm_bf16(ba, bb, bh, M, N, K, dev.device_id)
+    assert np.array_equal(got[:M * N].reshape(M, N), bh.copyout(np.uint16, (M, N))), (tc, opts, (M, N, K))
