@@ -682,6 +682,13 @@ struct KernelGen {
     // Nodes whose value this kernel has computed itself and holds in a register, whatever the
     // coordinates (a row's reduction inside the kernel that also consumes it).
     std::map<const TensorNode*, uint32_t> fixed;
+    // Flat upcast: when the kernel's output is walked as one flat run (its innermost axis does not
+    // divide into whole upcast groups, its element count does), the materialised tensors of the
+    // output's own shape that are reached through elementwise nodes only are read at the flat
+    // index itself: flat_base (a multiple of the width) + flat_off, one vector load per group.
+    std::set<const TensorNode*> flat_leaves;
+    uint32_t flat_base = 0;
+    int64_t flat_off = 0;
     const TensorNode* pick_cat = nullptr;
     int pick_part = -1;
     Cx probed_pos;
@@ -803,7 +810,7 @@ uint32_t emit(KernelGen& g, const TensorNode* n, const Coords& coords);
 uint32_t emit_load(KernelGen& g, const TensorNode* n, const Coords& coords) {
     KernelBuilder& b = g.b;
     uint32_t p = g.buffer_param(n->buffer, n->dtype, n->numel());
-    Cx flat = flatten(g, coords, n->shape);
+    Cx flat = g.flat_base && g.flat_leaves.count(n) ? Cx{g.flat_base, g.flat_off, true, g.width} : flatten(g, coords, n->shape);
     const int64_t per_load = std::min<int64_t>(g.width, 16 / std::max<int64_t>(1, static_cast<int64_t>(scalar_size(n->dtype))));
     // a group of per_load consecutive elements that starts on a multiple of per_load (and so lies
     // inside a buffer of a multiple of per_load elements) is one vector load
@@ -2026,6 +2033,19 @@ struct Scheduler {
         return finish_kernel(g, n, out, "rE_" + std::to_string(rows) + "_g" + std::to_string(C) + (width > 1 ? "_" + std::to_string(width) : ""));
     }
 
+    // Materialised tensors under `n` of shape `shape`: reached through elementwise nodes only
+    // (`direct`), or through at least one node that moves coordinates (`indirect`).
+    static void flat_candidates(const TensorNode* n, const std::vector<int64_t>& shape, bool pure, std::set<const TensorNode*>* direct,
+                                std::set<const TensorNode*>* indirect) {
+        if (n->buffer) {
+            (pure && n->shape == shape ? direct : indirect)->insert(n);
+            return;
+        }
+        const bool elementwise = n->kind == TKind::Unary || n->kind == TKind::Binary || n->kind == TKind::Where || n->kind == TKind::Cast ||
+                                 n->kind == TKind::Contiguous;
+        for (const TensorRef& c : n->src) flat_candidates(c.get(), shape, pure && elementwise && c->shape == shape, direct, indirect);
+    }
+
     int gen_elementwise(TensorNode* n, int64_t max_numel) {
         const int64_t N = n->numel();
         KernelGen g;
@@ -2043,6 +2063,28 @@ struct Scheduler {
                     width = w;
                     break;
                 }
+        // flat upcast: the innermost axis gives no (or a narrower) group but the element count does
+        // and some operand can be read flat (an odd vocabulary, [N, 3] points, a column vector)
+        bool flat = false;
+        const char* no_flat = std::getenv("MOROK_NO_FLAT_UPCAST");  // measurement switch
+        if (n->dtype != Scalar::Bool && N > 0 && !(no_flat && no_flat[0] && no_flat[0] != '0')) {
+            int64_t fw = 1;
+            for (int64_t w = up_bytes / static_cast<int64_t>(scalar_size(n->dtype)); w > 1; w /= 2)
+                if (N % w == 0) {
+                    fw = w;
+                    break;
+                }
+            if (fw > width) {
+                std::set<const TensorNode*> direct, indirect;
+                flat_candidates(n, n->shape, true, &direct, &indirect);
+                for (const TensorNode* d : direct)
+                    if (!indirect.count(d)) g.flat_leaves.insert(d);
+                if (!g.flat_leaves.empty()) {
+                    flat = true;
+                    width = fw;
+                }
+            }
+        }
         g.width = width;
         const int64_t items = N / width, block = gen_opts.local > 0 ? gen_opts.local : 256;
         uint32_t gx = workgroup_index(b, g.idx_t, workgroup_axes(items, n->shape.empty() ? 0 : n->shape.back() / width, block));
@@ -2068,7 +2110,7 @@ struct Scheduler {
         // all parts; instead the work-items are renumbered so that the 64 of a wave produce
         // outputs of one part only (R rows x the part's vectors), and each part gets its own
         // guarded region, which a wave of the other part skips altogether.
-        const TensorNode* cat = root_cat(n, width);
+        const TensorNode* cat = flat ? nullptr : root_cat(n, width);
         bool split = false;
         if (cat) {
             const int64_t P = static_cast<int64_t>(cat->src.size()), V = n->shape.back() / width, Vp = V / P;
@@ -2110,14 +2152,28 @@ struct Scheduler {
                 g.pick_part = -1;
             }
         }
-        if (!split) {
+        if (flat) {
+            // every element gets its own coordinates (for what cannot be read flat); operands of the
+            // output's shape ignore them and share one vector load per group
+            uint32_t base = b.imul(item, width);
+            g.flat_base = base;
+            std::vector<uint32_t> vals;
+            for (int64_t e = 0; e < width; e++) {
+                g.flat_off = e;
+                Coords ce = plain(unflatten(g, b.iadd(base, g.ci(e)), n->shape));
+                uint32_t v = n->kind == TKind::Contiguous ? emit(g, n->src[0].get(), ce) : emit_uncached(g, n, ce);
+                if (b.dtype(v).scalar != n->dtype) v = b.cast(v, n->dtype);
+                vals.push_back(v);
+            }
+            b.store(b.index(po, base), b.vectorize(vals));
+        } else if (!split) {
             uint32_t base = b.imul(item, width);
             Coords coords = plain(unflatten(g, base, n->shape));
             if (width > 1) coords.back().aligned = true;
             emit_group(coords, base);
         }
         b.endif();
-        return finish_kernel(g, n, out, "E_" + std::to_string(N) + (width > 1 ? "_" + std::to_string(width) : ""));
+        return finish_kernel(g, n, out, "E_" + std::to_string(N) + (width > 1 ? "_" + std::to_string(width) : "") + (flat ? "f" : ""));
     }
 
     int gen_reduce(TensorNode* n, int64_t max_numel) {

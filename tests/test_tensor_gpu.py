@@ -1236,3 +1236,50 @@ def test_beam_search_over_generated_kernels_keeps_values(T, tmp_path, monkeypatc
     for t, w in zip(graphs(), got):
         assert np.array_equal(t.to_numpy(), w)                          # same choices, same bits
         assert T.last_beam_search()[0] == 0 and T.last_beam_search()[1] >= 1
+
+
+# ---------------------------------------------------------------- flat upcast (odd innermost axes)
+@pytest.mark.parametrize("shape,dtype", [((1 << 16, 3), "f32"), ((1000, 333), "bf16"), ((64, 50257 // 7 * 8 + 1), "f32"), ((12, 5, 7, 2), "f32"),
+                                         ((4096, 1), "f32")])
+def test_flat_upcast_elementwise(T, shape, dtype):
+    """An innermost axis that does not divide into whole 16-byte groups (an odd vocabulary, [N, 3]
+    points, a column) while the element count does: the kernel walks its output as one flat run,
+    operands of the output's own shape are read with vector loads at the flat index, and operands
+    seen through movement ops (a broadcast row, a transposed square) keep their coordinates."""
+    from morok_amd import synth, uop
+
+    n = int(np.prod(shape))
+    if dtype == "bf16":
+        xb, yb = synth.normal_bf16(shape, 71, 0), synth.normal_bf16(shape, 71, 1)
+        x, y = synth.from_bf16(xb), synth.from_bf16(yb)
+        tx, ty = T.Tensor.from_numpy(xb, uop.BF16), T.Tensor.from_numpy(yb, uop.BF16)
+        got = synth.from_bf16(tx.try_mul(ty).try_add(tx).to_numpy())
+        want = synth.from_bf16(synth.to_bf16(x * y + x))
+    else:
+        x, y = synth.normal(shape, 71, 0), synth.normal(shape, 71, 1)
+        tx, ty = T.Tensor.from_numpy(x), T.Tensor.from_numpy(y)
+        got = tx.try_mul(ty).try_add(tx).to_numpy()
+        want = x * y + x
+    name = T.last_kernels()[0]
+    width = 16 // (2 if dtype == "bf16" else 4)
+    if shape[-1] % width and n % width == 0:
+        assert name.endswith("f") and name.startswith("E_%d_" % n), name       # flat, full width
+    if dtype == "f32":
+        assert np.array_equal(got, (x * y + x).astype(np.float32)) or np.allclose(got, want, rtol=1e-6, atol=0)
+        # a broadcast row stays on coordinates while x is read flat
+        row = synth.normal((1,) * (len(shape) - 1) + (shape[-1],), 71, 2)
+        got2 = tx.try_add(T.Tensor.from_numpy(row).try_expand(list(shape))).to_numpy()
+        assert np.array_equal(got2, x + row)
+    else:
+        assert np.array_equal(got, want)
+
+
+def test_flat_upcast_keeps_moved_operands_on_coordinates(T):
+    from morok_amd import synth
+
+    x, y = synth.normal((6, 6), 72, 0), synth.normal((6, 6), 72, 1)     # 36 elements: groups of 4, rows of 6
+    tx, ty = T.Tensor.from_numpy(x), T.Tensor.from_numpy(y)
+    got = tx.try_add(ty.try_permute([1, 0])).to_numpy()                   # same shape, but not the same positions
+    assert np.array_equal(got, x + y.T) and T.last_kernels()[0].endswith("f")
+    got = tx.try_add(tx.try_permute([1, 0])).to_numpy()                   # the same tensor both ways: no flat read at all
+    assert np.array_equal(got, x + x.T) and not T.last_kernels()[0].endswith("f")
