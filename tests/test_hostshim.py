@@ -792,6 +792,31 @@ def test_large_reductions_are_split_in_two_stages(T, shim):
     assert len(t.kernels()) == 1
 
 
+def test_column_reductions_and_flat_upcast_lowering(T, shim):
+    """Reductions that keep the contiguous axis run a work-item per output (split over the outermost
+    reduce axis when the outputs alone are too few); elementwise kernels over an innermost axis that
+    does not divide into 16-byte groups walk the output flat.  Every source compiles."""
+    T.set_fusion(False)
+    t = zeros(T, (8192, 4096)).max(0).realize()
+    assert t.kernels() == ["r_4096x64_128", "r_4096_64"]
+    assert all("global_load_lds" not in s and "__shared__" not in s for s in T.last_kernel_sources())
+    t = zeros(T, (129, 64)).sum(0).realize()             # an odd reduce extent is not split
+    assert t.kernels() == ["r_64_129"]
+    t = zeros(T, (4, 2048, 256)).sum(1).realize()        # a fold over a middle axis
+    assert len(t.kernels()) == 2 and t.kernels()[0].startswith("r_1024x")
+    t = zeros(T, (64, 8192)).sum(1).realize()            # the innermost axis is reduced: waves along the rows, as before
+    assert t.kernels() == ["r_64_g8192_l16"]
+    a, b = zeros(T, (1000, 333)), zeros(T, (1000, 333))
+    t = a.try_mul(b).try_add(a).realize()
+    assert t.kernels() == ["E_333000_4f"]
+    src = T.last_kernel_sources()[0]
+    assert src.count("*((mrk_float4*)") == 3              # two vector loads and the vector store
+    t = a.try_add(zeros(T, (1, 333)).try_expand([1000, 333])).realize()
+    assert t.kernels() == ["E_333000_4f"] and T.last_kernel_sources()[0].count("*((mrk_float4*)") == 2   # the broadcast row stays scalar
+    t = zeros(T, (333, 1000)).try_permute([1, 0]).contiguous().realize()
+    assert t.kernels() == ["E_333000"]                    # nothing to read flat: the scalar walk
+
+
 def test_grouped_reduce_through_local_memory(T, shim, monkeypatch):
     """GROUP / GROUPTOP (schedule/src/optimizer/heuristics.rs:370-392): kernels with at most 2048
     outputs let the waves of a workgroup share an output through local memory and a barrier."""
