@@ -1504,6 +1504,10 @@ struct Scheduler {
             for (TensorNode* d : deps)
                 if (d != R) MRK_TRY(materialize(d));
             for (TensorNode* d : deps_r) MRK_TRY(materialize(d));
+            if (const char* e = std::getenv("MOROK_BEAM")) {
+                const int beam = std::atoi(e);
+                if (beam > 0 && !dry) return beam_generated(n, max_numel, beam, R, row_block);
+            }
             return gen_row_fused(n, R, row_block, max_numel);
         }
         for (TensorNode* d : deps) MRK_TRY(materialize(d));
@@ -1521,13 +1525,17 @@ struct Scheduler {
     // like the matmul searches: UPCAST then LOCAL for an elementwise kernel, GROUP (waves per
     // output and segments) then LOCAL (outputs per workgroup) for a wave reduction.  The winner
     // is cached on disk under the hash of the kernel the fixed heuristics produce.
-    int beam_generated(TensorNode* n, int64_t max_numel, int width) {
-        const bool red = n->kind == TKind::Reduce;
+    int beam_generated(TensorNode* n, int64_t max_numel, int width, TensorNode* row_reduce = nullptr, int64_t row_block = 0) {
+        const bool red = n->kind == TKind::Reduce && !row_reduce;
+        auto generate = [&]() -> int {
+            if (row_reduce) return gen_row_fused(n, row_reduce, row_block, max_numel);
+            return red ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
+        };
         auto build = [&](const GenOpts& o, std::vector<DryKernel>* out) -> int {
             dry = true;
             gen_opts = o;
             dry_kernels.clear();
-            const int rc = red ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
+            const int rc = generate();
             dry = false;
             gen_opts = GenOpts();
             *out = std::move(dry_kernels);
@@ -1536,7 +1544,7 @@ struct Scheduler {
         };
         auto for_real = [&](const GenOpts& o) -> int {
             gen_opts = o;
-            const int rc = red ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
+            const int rc = generate();
             gen_opts = GenOpts();
             return rc;
         };
@@ -1623,7 +1631,16 @@ struct Scheduler {
             if (!time_one(GenOpts(), &ms)) return for_real(GenOpts());
             beam.emplace_back(ms, GenOpts());
         }
-        if (!red) {
+        if (row_reduce) {
+            // LOCAL: the work-items that share a row (the row stays in their registers)
+            for (int local : {64, 128, 256, 512, 1024}) {
+                GenOpts o;
+                o.local = local;
+                double ms;
+                if (time_one(o, &ms)) beam.emplace_back(ms, o);
+            }
+            keep_best(beam);
+        } else if (!red) {
             for (int up : {8, 4, 32}) {
                 GenOpts o;
                 o.upcast_bytes = up;
@@ -1981,6 +1998,11 @@ struct Scheduler {
                 break;
             }
         g.width = width;
+        if (gen_opts.local > 0) {  // a search's explicit choice; rows that do not split that way keep the heuristic
+            const int64_t cand = gen_opts.local, Vt = C / width;
+            if (cand % 64 || cand > 1024 || Vt % cand || Vt / cand > 8) return fail(kInvalidArgument, "row-resident kernel: the row does not split over that many work-items");
+            block = cand;
+        }
         const int64_t V = C / width, per_item = V / block, waves = block / 64;
         uint32_t row = workgroup_index(b, g.idx_t, {rows});
         if (!row) return last_status();

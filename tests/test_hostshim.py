@@ -527,6 +527,11 @@ def test_beam_search_over_generated_kernels(dev, shim, tmp_path, monkeypatch):
     small = T.Tensor.from_numpy(np.ones((16, 16), np.float32))
     small.try_mul(small).realize()
     assert T.last_beam_search() == (0, 0)
+    # a row-resident kernel: the work-items per row are searched
+    rows = T.Tensor.from_numpy(np.ones((256, 4096), np.float32))
+    rows.rms_norm(-1, 1e-6).realize()
+    timed, hits = T.last_beam_search()
+    assert timed >= 3 and hits == 0 and T.last_kernels() == ["rE_256_g4096_4"]
 
 
 def test_beam_search_uses_and_fills_the_disk_cache(dev, shim, tmp_path, monkeypatch):

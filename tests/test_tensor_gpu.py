@@ -1236,6 +1236,14 @@ def test_beam_search_over_generated_kernels_keeps_values(T, tmp_path, monkeypatc
     for t, w in zip(graphs(), got):
         assert np.array_equal(t.to_numpy(), w)                          # same choices, same bits
         assert T.last_beam_search()[0] == 0 and T.last_beam_search()[1] >= 1
+    # a row-resident kernel under the search: whatever workgroup size wins, rms_norm stays within
+    # the f32 tolerance of the unsearched kernel (the row sum changes its order only)
+    monkeypatch.delenv("MOROK_BEAM", raising=False)
+    base = Tensor.from_numpy(x).rms_norm(-1, 1e-6).to_numpy()
+    monkeypatch.setenv("MOROK_BEAM", "2")
+    searched = Tensor.from_numpy(x).rms_norm(-1, 1e-6).to_numpy()
+    assert T.last_kernels()[0].startswith("rE_768_g2048") and T.last_beam_search()[0] >= 3
+    assert np.abs(searched - base).max() <= 1e-5 * np.abs(base).max()
 
 
 # ---------------------------------------------------------------- flat upcast (odd innermost axes)
