@@ -472,7 +472,7 @@ int mrk_hip_gemm_bf16_swiglu(int device_id, const void* a, const void* w, void* 
  * statistics, P rounded to bf16 before the second product, bf16 output):
  * Tensor::scaled_dot_product_attention (tensor/src/transformer.rs:78-137) with is_causal as
  * given and no attn_mask / softcap.  q [B,H,Sq,D], k and v [B,H,Sk,D], o [B,H,Sq,D], row-major
- * bf16, D = 128 or 64 (other head dims: INVALID_ARGUMENT here, the composed graph through the tensor
+ * bf16, D = 256, 128 or 64 (other head dims: INVALID_ARGUMENT here, the composed graph through the tensor
  * API), scale > 0 (the reference default is 1/sqrt(D), transformer.rs:90-91).
  * Causal rule of the reference: key j is visible to query i iff j <= i (transformer.rs:103-109). */
 int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,

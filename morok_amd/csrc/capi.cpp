@@ -936,7 +936,7 @@ int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, con
                                 int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal) {
     if (batch < 0 || heads < 0 || sq < 0 || sk < 0) return fail(kInvalidArgument, "flash_attn_fwd: negative shape");
     if (batch == 0 || heads == 0 || sq == 0) return kOk;
-    if (d != 128 && d != 64) return failf(kInvalidArgument, "flash_attn_fwd: head_dim %lld is not supported (128 and 64 only)", (long long)d);
+    if (d != 256 && d != 128 && d != 64) return failf(kInvalidArgument, "flash_attn_fwd: head_dim %lld is not supported (256, 128 and 64 only)", (long long)d);
     if (sk == 0) return fail(kInvalidArgument, "flash_attn_fwd: empty key sequence (softmax over no keys is undefined)");
     if (!(scale > 0.0f)) return fail(kInvalidArgument, "flash_attn_fwd: scale must be positive");
     MRK_NONNULL(q);
@@ -956,7 +956,7 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
                                         const int64_t* strides) {
     if (batch < 0 || heads < 0 || sq < 0 || sk < 0) return fail(kInvalidArgument, "flash_attn_fwd_strided: negative shape");
     if (batch == 0 || heads == 0 || sq == 0) return kOk;
-    if (d != 128 && d != 64) return failf(kInvalidArgument, "flash_attn_fwd_strided: head_dim %lld is not supported (128 and 64 only)", (long long)d);
+    if (d != 256 && d != 128 && d != 64) return failf(kInvalidArgument, "flash_attn_fwd_strided: head_dim %lld is not supported (256, 128 and 64 only)", (long long)d);
     if (sk == 0) return fail(kInvalidArgument, "flash_attn_fwd_strided: empty key sequence (softmax over no keys is undefined)");
     if (!(scale > 0.0f)) return fail(kInvalidArgument, "flash_attn_fwd_strided: scale must be positive");
     MRK_NONNULL(q);

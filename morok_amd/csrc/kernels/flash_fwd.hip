@@ -71,7 +71,7 @@ template <int kD, bool kStrided>
 __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
                                                const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH, int Sq, int Sk,
                                                float scale_log2e, int causal, int q_tiles, int units, const FlashLayout& lay) {
-    static_assert(kD == 128 || kD == 64, "head dims with an instantiation: 128 and 64");
+    static_assert(kD == 256 || kD == 128 || kD == 64, "head dims with an instantiation: 256, 128 and 64");
     constexpr int kRow = kD * 2;          // bytes per K/V row in LDS: 256 (128)
     constexpr int kTile = kKT * kRow;     // 16 KB (8 KB)
     constexpr int kDS = kD / 16;          // 16-deep steps of the score product: 8 (4)
@@ -160,7 +160,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
             // serves 16 lanes x 16 B per cycle over 64 banks, so 16 consecutive rows must
             // land in 16 different chunk slots (128-byte rows: c16 ^ ((row >> 1) & 7), the
             // parity of the row selects the half of the banks)
-            const int ksw = kD == 128 ? (row & 15) : ((row >> 1) & 7);
+            const int ksw = kD >= 128 ? (row & 15) : ((row >> 1) & 7);
             const unsigned kvoff = (unsigned)key * k_row + ((c16 ^ ksw) << 4);
             dma(lds_base + stage * kTile + (wave * 16 + c * kRowsPerDma) * kRow, kvoff, Kh);
         }
@@ -218,7 +218,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     // lane-constant LDS offsets
     // K fragment (A operand): row = kb*32 + l%32, logical chunk 2*ds + l/32
     const int k_row_off = lq * kRow;
-    const int k_sw = kD == 128 ? (lq & 15) : ((lq >> 1) & 7);
+    const int k_sw = kD >= 128 ? (lq & 15) : ((lq >> 1) & 7);
     // V^T fragment via transposing read: 16-lane block b = l/16 covers d half (b & 1) and
     // key group g = b >> 1; inside the block lane j' = l%16 points at key row j'/4,
     // 8-byte unit j'%4 of the 32-byte granule.
@@ -308,7 +308,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         const float mb = m_run * scale_log2e;
 
         // ---- phase A: S(j+1) = K(j+1) Q^T on the matrix pipe, P(j) = exp2(S(j)*c - m*c) on
-        // the vector ALUs: each of the 16 (8) MFMAs is followed by the exponentials of two (four)
+        // the vector ALUs: each of the 16 (8; 32) MFMAs is followed by the exponentials of two (four; every second one by two)
         // score registers (the last iteration computes a tile nobody uses).  The fences keep the
         // compiler from regrouping the two instruction streams.
         float psum0 = 0.0f, psum1 = 0.0f;
@@ -323,7 +323,8 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
             for (int kb = 0; kb < 2; kb++)
                 kf[0][kb] = *LDS_PTR(bf16x8, sKn + kb * 32 * kRow + k_row_off + (((0 + lg) ^ k_sw) << 4));
             f32x8 p;
-            constexpr int kPairs = 8 / kDS;  // pairs of score registers per MFMA: 1 (2)
+            constexpr int kMfmaA = 2 * kDS;  // score MFMAs of this phase; the 16 pairs of score registers are spread over them:
+                                             // one per MFMA (D = 128), two (64), one after every second (256)
 #pragma unroll
             for (int ds = 0; ds < kDS; ds++) {
                 if (ds + 1 < kDS) {
@@ -336,8 +337,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
                 for (int kb = 0; kb < 2; kb++) {
                     nxt[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds & 1][kb], qf[ds], nxt[kb], 0, 0, 0);
 #pragma unroll
-                    for (int pr = 0; pr < kPairs; pr++) {
-                        const int idx = (ds * 2 + kb) * kPairs + pr;  // 0..15: score registers 2*idx, 2*idx+1
+                    for (int idx = (ds * 2 + kb) * 16 / kMfmaA; idx < (ds * 2 + kb + 1) * 16 / kMfmaA; idx++) {  // 0..15: score registers 2*idx, 2*idx+1
                         const int pk = idx >> 3, pe = (idx & 7) * 2;  // block, register inside the block
                         const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe], scale_log2e, -mb));
                         const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe + 1], scale_log2e, -mb));
@@ -481,6 +481,19 @@ __global__ __launch_bounds__(256, 2) void flash_fwd_d64_strided(const __bf16* __
     flash_fwd_body<64, true>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, lay);
 }
 
+// 512-byte rows: one workgroup's four tiles fill 128 KB of LDS, one workgroup per CU
+__global__ __launch_bounds__(256, 1) void flash_fwd_d256(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
+                                                         const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
+                                                         int Sq, int Sk, float scale_log2e, int causal, int q_tiles, int units) {
+    flash_fwd_body<256, false>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, FlashLayout{});
+}
+__global__ __launch_bounds__(256, 1) void flash_fwd_d256_strided(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
+                                                                 const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH,
+                                                                 int Sq, int Sk, float scale_log2e, int causal, int q_tiles,
+                                                                 int units, FlashLayout lay) {
+    flash_fwd_body<256, true>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, lay);
+}
+
 }  // namespace mrk::dev
 
 namespace mrk {
@@ -489,7 +502,7 @@ int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void
                           long D, float scale, int causal) {
     using namespace mrk::dev;
     if (BH <= 0 || Sq <= 0) return 0;
-    if ((D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
+    if ((D != 256 && D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
     if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
     const long q_tiles = (Sq + kQT - 1) / kQT;
     const long units = causal ? (q_tiles + 1) / 2 : q_tiles;
@@ -497,7 +510,7 @@ int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void
     if (blocks > 0x7fffffffL) return (int)hipErrorInvalidValue;
     (void)hipGetLastError();
     const float scale_log2e = scale * 1.4426950408889634f;
-    auto kernel = D == 128 ? flash_fwd_d128 : flash_fwd_d64;
+    auto kernel = D == 256 ? flash_fwd_d256 : D == 128 ? flash_fwd_d128 : flash_fwd_d64;
     kernel<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
         static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles, (int)units);
@@ -510,7 +523,7 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
     if (B < 0 || H < 0 || !strides) return (int)hipErrorInvalidValue;
     const long BH = B * H;
     if (BH == 0 || Sq <= 0) return 0;
-    if ((D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
+    if ((D != 256 && D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
     if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
     // strides: (batch, head, row) of q, k, v, o in elements.  Rows are read and written in
     // 16-byte pieces from 16-byte aligned addresses; row offsets inside a head are 32-bit
@@ -541,7 +554,7 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
     lay.heads = (int)H;
     (void)hipGetLastError();
     const float scale_log2e = scale * 1.4426950408889634f;
-    auto kernel = D == 128 ? flash_fwd_d128_strided : flash_fwd_d64_strided;
+    auto kernel = D == 256 ? flash_fwd_d256_strided : D == 128 ? flash_fwd_d128_strided : flash_fwd_d64_strided;
     kernel<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
         static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles, (int)units, lay);

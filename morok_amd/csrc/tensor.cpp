@@ -1213,7 +1213,7 @@ struct Scheduler {
                 const TensorNode* k = n->hint_inputs[1].get();
                 const TensorNode* v = n->hint_inputs[2].get();
                 return q->dtype == Scalar::BFloat16 && k->dtype == q->dtype && v->dtype == q->dtype &&
-                       q->shape.size() == 4 && (q->shape[3] == 128 || q->shape[3] == 64) && v->shape[3] == q->shape[3] && k->shape[2] > 0 &&
+                       q->shape.size() == 4 && (q->shape[3] == 256 || q->shape[3] == 128 || q->shape[3] == 64) && v->shape[3] == q->shape[3] && k->shape[2] > 0 &&
                        k->shape[0] == q->shape[0] && k->shape[1] == q->shape[1] && q->numel() > 0;
             }
             default: return false;

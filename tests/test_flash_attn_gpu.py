@@ -258,7 +258,7 @@ def test_flash_strided_refuses_what_it_cannot_address(dev):
         _strided(dev, bufs, [0, 0, 0, 0], [H * S * D, S * D, 2 * D] + good[3:], B, H, S, S, True)
 
 
-# ---------------------------------------------------------------- head dim 64
+# ---------------------------------------------------------------- head dims 64 and 256
 def _attn_d(dev, q, k, v, scale, causal, d):
     B, H, Sq, _ = q.shape
     Sk = k.shape[2]
@@ -273,67 +273,76 @@ def _inputs_d(B, H, Sq, Sk, d, seed):
             synth.normal_bf16((B, H, Sk, d), seed, 2))
 
 
+@pytest.mark.parametrize("d", [64, 256])
 @pytest.mark.parametrize("shape", [(1, 1, 1, 1), (1, 2, 64, 64), (2, 3, 80, 80), (1, 2, 129, 129), (1, 1, 300, 300),
                                    (2, 2, 512, 512), (1, 3, 33, 257), (1, 1, 257, 33), (1, 2, 1024, 1024)])
 @pytest.mark.parametrize("causal", [True, False])
-def test_flash_d64_parity_shapes(dev, oracle, shape, causal):
-    """The head-dim-64 instantiation of the same kernel body (128-byte rows in LDS, its own K
-    swizzle): the same cases as head dim 128 against the oracle, scale 1/sqrt(64)."""
+def test_flash_other_head_dims_parity_shapes(dev, oracle, shape, causal, d):
+    """The head-dim-64 and head-dim-256 instantiations of the same kernel body (128-byte rows in
+    LDS with their own K swizzle; 512-byte rows, one workgroup per CU, an exponential pair behind
+    every second score MFMA): the same cases as head dim 128 against the oracle, scale 1/sqrt(d)."""
     B, H, Sq, Sk = shape
-    q, k, v = _inputs_d(B, H, Sq, Sk, 64, seed=61)
-    _check(_attn_d(dev, q, k, v, 0.125, causal, 64), oracle.sdpa_bf16(q, k, v, 0.125, causal=causal))
+    q, k, v = _inputs_d(B, H, Sq, Sk, d, seed=61)
+    sc = float(d) ** -0.5
+    _check(_attn_d(dev, q, k, v, sc, causal, d), oracle.sdpa_bf16(q, k, v, sc, causal=causal))
 
 
-def test_flash_d64_special_cases_and_bounds(dev, oracle):
+@pytest.mark.parametrize("d", [64, 256])
+def test_flash_other_head_dims_special_cases_and_bounds(dev, oracle, d):
     B, H, S = 2, 2, 256
-    q, k, v = _inputs_d(B, H, S, S, 64, seed=62)
-    o = _attn_d(dev, q, k, v, 0.125, True, 64)
+    sc = float(d) ** -0.5
+    q, k, v = _inputs_d(B, H, S, S, d, seed=62)
+    o = _attn_d(dev, q, k, v, sc, True, d)
     assert np.array_equal(o[:, :, 0], v[:, :, 0])   # first causal row sees key 0 only
     # every d column is used: a one-hot V picks single columns of P's row sums (all ones)
-    ones = synth.to_bf16(np.ones((1, 1, 70, 64), np.float32))
-    eye_v = synth.to_bf16(np.tile(np.eye(64, dtype=np.float32), (2, 1))[:70][None, None])
-    o = synth.from_bf16(_attn_d(dev, ones, ones, eye_v, 0.125, False, 64))
-    want = np.tile(np.eye(64, dtype=np.float32), (2, 1))[:70].sum(0) / 70.0
+    rows = d + 6
+    ones = synth.to_bf16(np.ones((1, 1, rows, d), np.float32))
+    eye_rows = np.tile(np.eye(d, dtype=np.float32), (2, 1))[:rows]
+    o = synth.from_bf16(_attn_d(dev, ones, ones, synth.to_bf16(eye_rows[None, None]), sc, False, d))
+    want = eye_rows.sum(0) / float(rows)
     assert np.abs(o - want[None, None, None, :]).max() <= 2e-2 * want.max()
     # NaNs right behind every operand and the result (ragged last tiles)
     for Sq, Sk, causal in ((100, 100, True), (129, 257, False), (64, 33, True)):
-        q, k, v = _inputs_d(1, 2, Sq, Sk, 64, seed=63)
+        q, k, v = _inputs_d(1, 2, Sq, Sk, d, seed=63)
         nan = np.full(4096, 0x7FC0, np.uint16)
         bq, bk, bv = (morok_amd.Buffer.from_numpy(np.concatenate([t.reshape(-1), nan]), dev.device_id) for t in (q, k, v))
         bo = morok_amd.Buffer.from_numpy(np.full(q.size + 4096, 0x7FC0, np.uint16), dev.device_id)
-        ops.flash_attn_fwd_bf16(bq, bk, bv, bo, 1, 2, Sq, Sk, 64, 0.125, causal, dev.device_id)
+        ops.flash_attn_fwd_bf16(bq, bk, bv, bo, 1, 2, Sq, Sk, d, sc, causal, dev.device_id)
         out = bo.copyout(np.uint16)
-        _check(out[: q.size].reshape(q.shape), oracle.sdpa_bf16(q, k, v, 0.125, causal=causal))
+        _check(out[: q.size].reshape(q.shape), oracle.sdpa_bf16(q, k, v, sc, causal=causal))
         assert np.all(out[q.size:] == 0x7FC0)
 
 
-def test_flash_d64_views_and_tensor_api(dev, oracle):
-    """[B, S, H, 64] activations through the strided entry point, and head dim 64 through
+@pytest.mark.parametrize("d", [64, 256])
+def test_flash_other_head_dims_views_and_tensor_api(dev, oracle, d):
+    """[B, S, H, d] activations through the strided entry point, and head dims 64 / 256 through
     Tensor::scaled_dot_product_attention (one fused kernel instead of the composed graph)."""
     from morok_amd import tensor as T, uop
 
-    B, H, S, d = 2, 3, 200, 64
+    B, H, S = 2, 3, 200
+    sc = float(d) ** -0.5
     q, k, v = _inputs_d(B, H, S, S, d, seed=64)
     qs, ks, vs = (np.ascontiguousarray(t.transpose(0, 2, 1, 3)) for t in (q, k, v))
     strides = [S * H * d, d, H * d] * 4
     bq, bk, bv = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (qs, ks, vs))
     bo = morok_amd.Buffer.from_numpy(np.zeros_like(qs), dev.device_id)
-    ops.flash_attn_fwd_bf16_strided(bq, bk, bv, bo, B, H, S, S, d, 0.125, strides, [0, 0, 0, 0], True, dev.device_id)
+    ops.flash_attn_fwd_bf16_strided(bq, bk, bv, bo, B, H, S, S, d, sc, strides, [0, 0, 0, 0], True, dev.device_id)
     o = bo.copyout(np.uint16, qs.shape).transpose(0, 2, 1, 3)
-    assert np.array_equal(o, _attn_d(dev, q, k, v, 0.125, True, d))
+    assert np.array_equal(o, _attn_d(dev, q, k, v, sc, True, d))
     t = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(T.Tensor.from_numpy(k, uop.BF16),
                                                                       T.Tensor.from_numpy(v, uop.BF16), is_causal=True)
     got = t.to_numpy()
-    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("flash_fwd_bf16") and t.kernels()[0].endswith("_d64")
+    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("flash_fwd_bf16") and t.kernels()[0].endswith("_d%d" % d)
     assert np.array_equal(got, o)
-    _check(got, oracle.sdpa_bf16(q, k, v, 0.125, causal=True))
+    _check(got, oracle.sdpa_bf16(q, k, v, sc, causal=True))
 
 
+@pytest.mark.parametrize("d", [64, 256])
 @pytest.mark.parametrize("seed", range(8))
-def test_flash_d64_random_shapes(dev, oracle, seed):
+def test_flash_other_head_dims_random_shapes(dev, oracle, seed, d):
     rng = np.random.default_rng(5000 + seed)
     B, H = int(rng.integers(1, 3)), int(rng.integers(1, 4))
     Sq, Sk = int(rng.integers(1, 520)), int(rng.integers(1, 520))
-    q, k, v = _inputs_d(B, H, Sq, Sk, 64, seed=70 + seed)
-    scale = float(rng.choice([0.125, 0.05, 0.2]))
-    _check(_attn_d(dev, q, k, v, scale, bool(seed & 1), 64), oracle.sdpa_bf16(q, k, v, scale, causal=bool(seed & 1)))
+    q, k, v = _inputs_d(B, H, Sq, Sk, d, seed=70 + seed)
+    scale = float(rng.choice([0.125, 0.05, 0.2])) * (64.0 / d) ** 0.5
+    _check(_attn_d(dev, q, k, v, scale, bool(seed & 1), d), oracle.sdpa_bf16(q, k, v, scale, causal=bool(seed & 1)))

@@ -318,6 +318,8 @@ def test_tensor_fused_kernel_selection(T, shim):
     assert len(f.kernels()) == 1 and shim.mrk_shim_last_kernel() == b"flash_fwd_bf16"
     f64 = bf(1, 2, 64, 64).scaled_dot_product_attention(bf(1, 2, 64, 64), bf(1, 2, 64, 64), is_causal=True).realize()
     assert f64.kernels() == ["flash_fwd_bf16_2_64_64_d64"]   # head dim 64 has an instantiation of its own
+    f256 = bf(1, 2, 64, 256).scaled_dot_product_attention(bf(1, 2, 64, 256), bf(1, 2, 64, 256), is_causal=True).realize()
+    assert f256.kernels() == ["flash_fwd_bf16_2_64_64_d256"]  # and so has 256
     f96 = bf(1, 2, 64, 96).scaled_dot_product_attention(bf(1, 2, 64, 96), bf(1, 2, 64, 96), is_causal=True).realize()
     assert len(f96.kernels()) >= 4                   # other head dims: composed path
     m = zeros(T, (128, 40)).matmul(zeros(T, (40, 64))).realize()
