@@ -604,6 +604,25 @@ Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& val
     const int64_t head_dim = n_->shape[nd - 1];
     const double scale_val = scale > 0.0 ? scale : 1.0 / std::sqrt(static_cast<double>(head_dim));  // transformer.rs:90-91
     const Scalar sdt = n_->dtype;
+    // A head dim without a fused instantiation (80, 96, 192 ...) is padded with zero columns up to
+    // the next one that has (64, 128, 256): zero columns add exact zeros to every score, the
+    // padded columns of V give zero outputs that are cut off again, and the scale stays that of
+    // the real head dim.  Three padded copies instead of a materialised [Sq, Sk] score matrix.
+    if (nd == 4 && sdt == Scalar::BFloat16 && !attn_mask && !(softcap > 0.0) && head_dim > 0 && head_dim < 256 && head_dim != 64 &&
+        head_dim != 128 && key.shape()[3] == head_dim && value.shape()[3] == head_dim && key.dtype() == sdt && value.dtype() == sdt &&
+        n_->numel() > 0 && key.node()->numel() > 0) {
+        const int64_t padded = head_dim < 64 ? 64 : head_dim < 128 ? 128 : 256;
+        auto pad = [&](const Tensor& t) {
+            std::vector<int64_t> zs = t.shape();
+            zs[3] = padded - head_dim;
+            return Tensor::cat({t, Tensor::full(zs, 0.0, sdt, t.node()->device_id)}, 3);
+        };
+        Tensor out = pad(*this).scaled_dot_product_attention(pad(key), pad(value), scale_val, is_causal, nullptr, 0.0);
+        if (!out.valid()) return out;
+        std::vector<int64_t> b0(4, 0), e0 = out.shape();
+        e0[3] = head_dim;
+        return out.try_shrink(b0, e0);
+    }
     Tensor scores = matmul(key.try_transpose(-1, -2));
     scores = scores.try_mul(const_(scale_val, sdt, n_->device_id));
     if (is_causal) {

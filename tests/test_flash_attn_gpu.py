@@ -346,3 +346,22 @@ def test_flash_other_head_dims_random_shapes(dev, oracle, seed, d):
     q, k, v = _inputs_d(B, H, Sq, Sk, d, seed=70 + seed)
     scale = float(rng.choice([0.125, 0.05, 0.2])) * (64.0 / d) ** 0.5
     _check(_attn_d(dev, q, k, v, scale, bool(seed & 1), d), oracle.sdpa_bf16(q, k, v, scale, causal=bool(seed & 1)))
+
+
+@pytest.mark.parametrize("d,causal", [(96, True), (80, False), (40, True), (192, True), (8, False)])
+def test_head_dims_without_an_instantiation_are_padded(dev, oracle, d, causal):
+    """Tensor::scaled_dot_product_attention on a head dim with no fused instantiation: q, k, v are
+    padded with zero columns to the next one that has (zero columns add exact zeros to the scores,
+    the padded output columns are cut off), so the fused kernel runs and no [Sq, Sk] score matrix
+    is materialised; the scale is that of the real head dim."""
+    from morok_amd import tensor as T, uop
+
+    B, H, S = 2, 2, 300
+    q, k, v = _inputs_d(B, H, S, S, d, seed=81)
+    t = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(T.Tensor.from_numpy(k, uop.BF16),
+                                                                      T.Tensor.from_numpy(v, uop.BF16), is_causal=causal)
+    got = t.to_numpy()
+    names = t.kernels()
+    assert sum(nm.startswith("flash_fwd_bf16") for nm in names) == 1 and not any(nm.startswith("r_") for nm in names), names
+    assert got.shape == q.shape
+    _check(got, oracle.sdpa_bf16(q, k, v, float(d) ** -0.5, causal=causal))

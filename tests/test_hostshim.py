@@ -321,7 +321,11 @@ def test_tensor_fused_kernel_selection(T, shim):
     f256 = bf(1, 2, 64, 256).scaled_dot_product_attention(bf(1, 2, 64, 256), bf(1, 2, 64, 256), is_causal=True).realize()
     assert f256.kernels() == ["flash_fwd_bf16_2_64_64_d256"]  # and so has 256
     f96 = bf(1, 2, 64, 96).scaled_dot_product_attention(bf(1, 2, 64, 96), bf(1, 2, 64, 96), is_causal=True).realize()
-    assert len(f96.kernels()) >= 4                   # other head dims: composed path
+    # other head dims are padded with zero columns to the next instantiation: three padded copies, the
+    # fused kernel at 128, the cut back to 96 columns; no reduce kernels, no score matrix
+    assert sum(k.startswith("flash_fwd_bf16_2_64_64") for k in f96.kernels()) == 1 and not any(k.startswith("r_") for k in f96.kernels())
+    f300 = bf(1, 2, 64, 304).scaled_dot_product_attention(bf(1, 2, 64, 304), bf(1, 2, 64, 304), is_causal=True).realize()
+    assert len(f300.kernels()) >= 4 and any(k.startswith("r_") for k in f300.kernels())   # beyond 256: the composed graph
     m = zeros(T, (128, 40)).matmul(zeros(T, (40, 64))).realize()
     assert len(m.kernels()) == 1 and m.kernels()[0] == "r_128_64_40"  # scheduled f32 matmul
     # inputs that are lazy views get materialised first
