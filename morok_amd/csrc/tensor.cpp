@@ -1191,7 +1191,7 @@ struct Scheduler {
         *max_numel = std::max(*max_numel, n->numel());
         if (n->buffer) return;
         TensorNode* other = nullptr;
-        if (n != root && (is_boundary_kind(n) || fusable(n) ||
+        if (n != root && (is_boundary_kind(n) || fusable(n) || generated_tc(n) ||
                           residual_matmul(const_cast<TensorNode*>(n), &other) || swiglu_matmul(n))) {
             out.push_back(const_cast<TensorNode*>(n));
             return;
@@ -1285,12 +1285,15 @@ struct Scheduler {
         return found;
     }
     bool generated_tc(const TensorNode* n) const {
-        if (g_fusion || n->hint != HintKind::Matmul || n->numel() == 0) return false;
+        if (n->hint != HintKind::Matmul || n->numel() == 0) return false;
         const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
-        if (a->dtype != Scalar::BFloat16 || w->dtype != Scalar::BFloat16 || n->dtype != Scalar::BFloat16) return false;
+        const Scalar dt = n->dtype;
+        // bf16 has hand-written kernels (taken while they are switched on); half precision has none
+        if (dt == Scalar::BFloat16 ? g_fusion : dt != Scalar::Float16) return false;
+        if (a->dtype != dt || w->dtype != dt) return false;
         if (a->shape.size() != 2 || w->shape.size() != 2) return false;
         const auto tcs = cdna4_tensor_cores();
-        const int tc = select_tensor_core(tcs, Scalar::BFloat16, Scalar::BFloat16, Scalar::Float32);
+        const int tc = select_tensor_core(tcs, dt, dt, Scalar::Float32);
         WmmaLdsOpts o;
         return tc >= 0 && default_tc_opts(tcs[tc], a->shape[0], w->shape[1], a->shape[1], &o);
     }
@@ -1299,15 +1302,15 @@ struct Scheduler {
         const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
         const int64_t M = a->shape[0], K = a->shape[1], N = w->shape[1];
         const auto tcs = cdna4_tensor_cores();
-        const int tc = select_tensor_core(tcs, Scalar::BFloat16, Scalar::BFloat16, Scalar::Float32);
-        if (tc < 0) return fail(kRuntime, "no bf16 tensor core in the CDNA table");
+        const int tc = select_tensor_core(tcs, n->dtype, n->dtype, Scalar::Float32);
+        if (tc < 0) return fail(kRuntime, "no tensor core for this dtype in the CDNA table");
         WmmaLdsOpts opts;
         if (!default_tc_opts(tcs[tc], M, N, K, &opts)) return fail(kRuntime, "tensor-core matmul: no workgroup tile divides the shape");
         int beam = 0;
         if (const char* e = std::getenv("MOROK_BEAM")) beam = std::atoi(e);
         if (beam > 0) MRK_TRY(beam_search_wmma_matmul(*dev, tcs[tc], tc, M, N, K, beam, &opts, nullptr, nullptr, nullptr));
         LinearKernel k;
-        MRK_TRY(build_wmma_matmul_lds_kernel(tcs[tc], M, N, K, Scalar::BFloat16, opts, &k));
+        MRK_TRY(build_wmma_matmul_lds_kernel(tcs[tc], M, N, K, n->dtype, opts, &k));
         std::shared_ptr<CachedKernel> ck;
         bool cached = false;
         const std::string name = "r_tc_" + std::to_string(M) + "_" + std::to_string(N) + "_" + std::to_string(K);
@@ -1497,7 +1500,7 @@ struct Scheduler {
         if (n->kind == TKind::Reshape || n->kind == TKind::Contiguous) {
             TensorNode* s = n->src[0].get();
             TensorNode* other = nullptr;
-            if (s->buffer || is_boundary_kind(s) || fusable(s) || residual_matmul(s, &other) || swiglu_matmul(s)) {
+            if (s->buffer || is_boundary_kind(s) || fusable(s) || generated_tc(s) || residual_matmul(s, &other) || swiglu_matmul(s)) {
                 MRK_TRY(materialize(s));
                 n->buffer = s->buffer;
                 produced.push_back(n);

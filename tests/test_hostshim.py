@@ -328,6 +328,8 @@ def test_tensor_fused_kernel_selection(T, shim):
     assert len(f300.kernels()) >= 4 and any(k.startswith("r_") for k in f300.kernels())   # beyond 256: the composed graph
     m = zeros(T, (128, 40)).matmul(zeros(T, (40, 64))).realize()
     assert len(m.kernels()) == 1 and m.kernels()[0] == "r_128_64_40"  # scheduled f32 matmul
+    h = zeros(T, (256, 128), np.float16).matmul(zeros(T, (128, 192), np.float16)).realize()
+    assert h.kernels() == ["r_tc_256_192_128"] and "mfma_f32_16x16x32_f16" in T.last_kernel_sources()[0]   # half: the WMMA route
     # inputs that are lazy views get materialised first
     gt = bf(32, 64).try_transpose(0, 1).matmul(bf(32, 48)).realize()
     assert len(gt.kernels()) == 2

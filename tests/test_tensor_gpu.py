@@ -1291,3 +1291,26 @@ def test_flat_upcast_keeps_moved_operands_on_coordinates(T):
     assert np.array_equal(got, x + y.T) and T.last_kernels()[0].endswith("f")
     got = tx.try_add(tx.try_permute([1, 0])).to_numpy()                   # the same tensor both ways: no flat read at all
     assert np.array_equal(got, x + x.T) and not T.last_kernels()[0].endswith("f")
+
+
+@pytest.mark.parametrize("shape", [(256, 192, 128), (100, 40, 72), (512, 512, 256), (64, 64, 64)])
+def test_half_precision_matmul_takes_the_generated_tensor_core_kernel(T, shape):
+    """There is no hand-written f16 GEMM: Tensor::matmul on half operands lowers through the WMMA
+    route (f16 tensor core of the CDNA table, f32 accumulate, direct-copy variant where its tiles
+    divide the shape, the padded register-staged one elsewhere), as a kernel of its own also in the
+    middle of an expression."""
+    from morok_amd import synth
+
+    M, N, K = shape
+    a = synth.normal((M, K), 91, 0).astype(np.float16)
+    b = synth.normal((K, N), 91, 1).astype(np.float16)
+    ta, tb = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
+    c = ta.matmul(tb)
+    got = c.to_numpy()
+    assert c.kernels() == ["r_tc_%d_%d_%d" % (M, N, K)] and got.dtype == np.float16
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.abs(got - ref).max() <= 2e-3 * np.abs(ref).max()
+    both = ta.matmul(tb).try_add(ta.matmul(tb))
+    got2 = both.to_numpy()
+    assert sum(k.startswith("r_tc_") for k in both.kernels()) == 2
+    assert np.array_equal(got2, (got.astype(np.float32) * 2).astype(np.float16))
