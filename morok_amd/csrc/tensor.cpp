@@ -1517,20 +1517,25 @@ struct Scheduler {
         int64_t max_numel = 0;
         boundaries(n, n, seen, deps, &max_numel);
         int64_t row_block = 0;
-        if (TensorNode* R = row_reduce_dep(n, deps, &row_block)) {
-            // everything either kernel half reads has to exist: the other inputs of the elementwise
-            // part and the inputs of the reduction's own expression
-            std::set<const TensorNode*> seen_r;
-            std::vector<TensorNode*> deps_r;
-            boundaries(R, R, seen_r, deps_r, &max_numel);
+        const std::vector<TensorNode*> Rs = row_reduce_deps(n, deps, &row_block);
+        if (!Rs.empty()) {
+            // everything any part of the kernel reads has to exist: the other inputs of the elementwise
+            // part and the inputs of the reductions' own expressions
+            auto fused = [&](const TensorNode* d) { return std::find(Rs.begin(), Rs.end(), d) != Rs.end(); };
             for (TensorNode* d : deps)
-                if (d != R) MRK_TRY(materialize(d));
-            for (TensorNode* d : deps_r) MRK_TRY(materialize(d));
+                if (!fused(d)) MRK_TRY(materialize(d));
+            for (TensorNode* R : Rs) {
+                std::set<const TensorNode*> seen_r;
+                std::vector<TensorNode*> deps_r;
+                boundaries(R, R, seen_r, deps_r, &max_numel);
+                for (TensorNode* d : deps_r)
+                    if (!fused(d)) MRK_TRY(materialize(d));
+            }
             if (const char* e = std::getenv("MOROK_BEAM")) {
                 const int beam = std::atoi(e);
-                if (beam > 0 && !dry) return beam_generated(n, max_numel, beam, R, row_block);
+                if (beam > 0 && !dry) return beam_generated(n, max_numel, beam, &Rs, row_block);
             }
-            return gen_row_fused(n, R, row_block, max_numel);
+            return gen_row_fused(n, Rs, row_block, max_numel);
         }
         for (TensorNode* d : deps) MRK_TRY(materialize(d));
         if (const char* e = std::getenv("MOROK_BEAM")) {
@@ -1547,10 +1552,10 @@ struct Scheduler {
     // like the matmul searches: UPCAST then LOCAL for an elementwise kernel, GROUP (waves per
     // output and segments) then LOCAL (outputs per workgroup) for a wave reduction.  The winner
     // is cached on disk under the hash of the kernel the fixed heuristics produce.
-    int beam_generated(TensorNode* n, int64_t max_numel, int width, TensorNode* row_reduce = nullptr, int64_t row_block = 0) {
+    int beam_generated(TensorNode* n, int64_t max_numel, int width, const std::vector<TensorNode*>* row_reduce = nullptr, int64_t row_block = 0) {
         const bool red = n->kind == TKind::Reduce && !row_reduce;
         auto generate = [&]() -> int {
-            if (row_reduce) return gen_row_fused(n, row_reduce, row_block, max_numel);
+            if (row_reduce) return gen_row_fused(n, *row_reduce, row_block, max_numel);
             return red ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
         };
         auto build = [&](const GenOpts& o, std::vector<DryKernel>* out) -> int {
@@ -1965,25 +1970,66 @@ struct Scheduler {
     // does.  One workgroup then owns a row: it folds the row (wave reduction + local memory),
     // keeps the total in a register and produces the row's outputs from the values it already
     // loaded, so the row is read once and the reduction needs no kernel and no buffer of its own.
-    // Returns the reduce node, or null when the shape does not fit (the two-kernel path remains).
-    TensorNode* row_reduce_dep(const TensorNode* n, const std::vector<TensorNode*>& deps, int64_t* block_out) const {
+    // Returns the reduce nodes, or nothing when the shape does not fit (the separate kernels remain).
+    // Up to three such reductions may feed the kernel, one building on another (softmax: the row
+    // maximum, then the sum of exp(x - max); layer norm: the mean, then the variance of the centred
+    // row): they are returned in an order in which each one's own expression only needs earlier ones.
+    std::vector<TensorNode*> row_reduce_deps(const TensorNode* n, const std::vector<TensorNode*>& deps, int64_t* block_out) {
         const char* off = std::getenv("MOROK_NO_ROW_FUSION");
-        if (off && off[0] && off[0] != '0') return nullptr;
-        if (n->kind == TKind::Reduce || n->shape.empty() || n->dtype == Scalar::Bool || n->numel() == 0) return nullptr;
-        TensorNode* R = nullptr;
-        for (TensorNode* d : deps) {
-            if (d->buffer || d->kind != TKind::Reduce) continue;
-            if (R) return nullptr;  // one reduction per kernel
-            R = d;
-        }
-        if (!R || R->src.size() != 1 || R->arg.size() != 1) return nullptr;
-        const TensorNode* src = R->src[0].get();
+        if (off && off[0] && off[0] != '0') return {};
+        if (n->kind == TKind::Reduce || n->shape.empty() || n->dtype == Scalar::Bool || n->numel() == 0) return {};
         const int64_t last = static_cast<int64_t>(n->shape.size()) - 1;
-        if (src->shape != n->shape || R->arg[0] != last) return nullptr;
-        const ReduceOp op = static_cast<ReduceOp>(R->sub);
-        if (compute_dtype(R->dtype) != Scalar::Float32 || (op != ReduceOp::Add && op != ReduceOp::Max)) return nullptr;
-        auto u = uses.find(R);
-        if (u == uses.end() || u->second != 1) return nullptr;  // somebody else wants the reduction in memory
+        auto qualifies = [&](const TensorNode* R) {
+            if (R->buffer || R->kind != TKind::Reduce || R->src.size() != 1 || R->arg.size() != 1) return false;
+            if (R->src[0]->shape != n->shape || R->arg[0] != last) return false;
+            const ReduceOp op = static_cast<ReduceOp>(R->sub);
+            if (compute_dtype(R->dtype) != Scalar::Float32 || (op != ReduceOp::Add && op != ReduceOp::Max)) return false;
+            auto u = uses.find(R);
+            return u != uses.end() && u->second == 1;  // else somebody wants the reduction in memory
+        };
+        // the reductions directly under n, and the ones under those
+        std::vector<TensorNode*> found;
+        std::map<TensorNode*, std::vector<TensorNode*>> needs;  // reduction -> qualifying reductions its expression reads
+        std::vector<TensorNode*> todo;
+        for (TensorNode* d : deps)
+            if (!d->buffer && d->kind == TKind::Reduce) todo.push_back(d);
+        while (!todo.empty()) {
+            TensorNode* R = todo.back();
+            todo.pop_back();
+            if (std::find(found.begin(), found.end(), R) != found.end()) continue;
+            if (!qualifies(R)) {
+                // a reduction of another shape directly under n rules the fusion out; further down it is
+                // simply computed first, like any other input
+                if (std::find(deps.begin(), deps.end(), R) != deps.end()) return {};
+                continue;
+            }
+            found.push_back(R);
+            if (found.size() > 3) return {};
+            std::set<const TensorNode*> seen_r;
+            std::vector<TensorNode*> deps_r;
+            int64_t ignore = 0;
+            boundaries(R, R, seen_r, deps_r, &ignore);
+            for (TensorNode* d : deps_r)
+                if (!d->buffer && d->kind == TKind::Reduce && qualifies(d)) {
+                    needs[R].push_back(d);
+                    todo.push_back(d);
+                }
+        }
+        if (found.empty()) return {};
+        std::vector<TensorNode*> ordered;
+        while (ordered.size() < found.size()) {
+            bool progress = false;
+            for (TensorNode* R : found) {
+                if (std::find(ordered.begin(), ordered.end(), R) != ordered.end()) continue;
+                bool ready = true;
+                for (TensorNode* d : needs[R]) ready = ready && std::find(ordered.begin(), ordered.end(), d) != ordered.end();
+                if (ready) {
+                    ordered.push_back(R);
+                    progress = true;
+                }
+            }
+            if (!progress) return {};
+        }
         const int64_t C = n->shape.back(), rows = n->numel() / C;
         int64_t width = 1;
         for (int64_t w = 16 / static_cast<int64_t>(scalar_size(n->dtype)); w > 1; w /= 2)
@@ -1999,14 +2045,12 @@ struct Scheduler {
                 break;
             }
         // whole waves, at most 8 vectors per work-item (the row stays in registers), enough rows to fill the chip
-        if (!block || V / block > 8 || rows < 128) return nullptr;
+        if (!block || V / block > 8 || rows < 128) return {};
         *block_out = block;
-        return R;
+        return ordered;
     }
 
-    int gen_row_fused(TensorNode* n, TensorNode* R, int64_t block, int64_t max_numel) {
-        const TensorNode* src = R->src[0].get();
-        const ReduceOp op = static_cast<ReduceOp>(R->sub);
+    int gen_row_fused(TensorNode* n, const std::vector<TensorNode*>& Rs, int64_t block, int64_t max_numel) {
         const int64_t N = n->numel(), C = n->shape.back(), rows = N / C;
         KernelGen g;
         g.idx_t = max_numel >= (1LL << 31) ? Scalar::Int64 : Scalar::Int32;
@@ -2038,29 +2082,37 @@ struct Scheduler {
             coords[i] = plain(unflatten(g, base[i], n->shape));
             if (width > 1) coords[i].back().aligned = true;
         }
-        // ---- the row's reduction: per work-item, per wave, then across the waves through local memory
-        uint32_t acc = 0;
-        for (int64_t i = 0; i < per_item; i++)
-            for (int64_t e = 0; e < width; e++) {
-                Coords ce = coords[i];
-                ce.back().off = e;
-                uint32_t v = emit(g, src, ce);
-                if (b.dtype(v).scalar != Scalar::Float32) v = b.cast(v, Scalar::Float32);
-                acc = acc ? b.binary(op == ReduceOp::Add ? BinaryOp::Add : BinaryOp::Max, acc, v) : v;
+        // ---- the row's reductions, in dependency order: per work-item, per wave, then across the
+        // waves through local memory (an array of its own per reduction: no barrier is needed to
+        // reuse one).  A later reduction's expression finds the earlier totals in g.fixed and the
+        // values already computed for this row in the memo.
+        for (size_t ri = 0; ri < Rs.size(); ri++) {
+            TensorNode* R = Rs[ri];
+            const TensorNode* src = R->src[0].get();
+            const ReduceOp op = static_cast<ReduceOp>(R->sub);
+            uint32_t acc = 0;
+            for (int64_t i = 0; i < per_item; i++)
+                for (int64_t e = 0; e < width; e++) {
+                    Coords ce = coords[i];
+                    ce.back().off = e;
+                    uint32_t v = emit(g, src, ce);
+                    if (b.dtype(v).scalar != Scalar::Float32) v = b.cast(v, Scalar::Float32);
+                    acc = acc ? b.binary(op == ReduceOp::Add ? BinaryOp::Add : BinaryOp::Max, acc, v) : v;
+                }
+            uint32_t total = b.wave_reduce(op, acc);
+            if (waves > 1) {
+                uint32_t lds = b.define_local(static_cast<int>(ri), Scalar::Float32, waves);
+                uint32_t lane = b.imod(lx, 64), wave = b.idiv(lx, 64);
+                b.if_(b.binary(BinaryOp::Eq, lane, g.ci(0)));
+                b.store(b.index(lds, wave), total);
+                b.endif();
+                b.barrier();
+                total = b.load(b.index(lds, g.ci(0)));
+                for (int64_t w = 1; w < waves; w++)
+                    total = b.binary(op == ReduceOp::Add ? BinaryOp::Add : BinaryOp::Max, total, b.load(b.index(lds, g.ci(w))));
             }
-        uint32_t total = b.wave_reduce(op, acc);
-        if (waves > 1) {
-            uint32_t lds = b.define_local(0, Scalar::Float32, waves);
-            uint32_t lane = b.imod(lx, 64), wave = b.idiv(lx, 64);
-            b.if_(b.binary(BinaryOp::Eq, lane, g.ci(0)));
-            b.store(b.index(lds, wave), total);
-            b.endif();
-            b.barrier();
-            total = b.load(b.index(lds, g.ci(0)));
-            for (int64_t w = 1; w < waves; w++)
-                total = b.binary(op == ReduceOp::Add ? BinaryOp::Add : BinaryOp::Max, total, b.load(b.index(lds, g.ci(w))));
+            g.fixed[R] = R->dtype != Scalar::Float32 ? b.cast(total, compute_dtype(R->dtype)) : total;
         }
-        g.fixed[R] = R->dtype != Scalar::Float32 ? b.cast(total, compute_dtype(R->dtype)) : total;
         // ---- the row's outputs, from the loads the reduction already made
         for (int64_t i = 0; i < per_item; i++) {
             std::vector<uint32_t> vals;
@@ -2074,7 +2126,8 @@ struct Scheduler {
             if (width > 1) b.store(b.index(po, base[i]), b.vectorize(vals));
             else b.store(b.index(po, base[i]), vals[0]);
         }
-        return finish_kernel(g, n, out, "rE_" + std::to_string(rows) + "_g" + std::to_string(C) + (width > 1 ? "_" + std::to_string(width) : ""));
+        return finish_kernel(g, n, out, "rE_" + std::to_string(rows) + "_g" + std::to_string(C) + (width > 1 ? "_" + std::to_string(width) : "") +
+                                            (Rs.size() > 1 ? "_x" + std::to_string(Rs.size()) : ""));
     }
 
     // Materialised tensors under `n` of shape `shape`: reached through elementwise nodes only

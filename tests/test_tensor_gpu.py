@@ -1314,3 +1314,58 @@ def test_half_precision_matmul_takes_the_generated_tensor_core_kernel(T, shape):
     got2 = both.to_numpy()
     assert sum(k.startswith("r_tc_") for k in both.kernels()) == 2
     assert np.array_equal(got2, (got.astype(np.float32) * 2).astype(np.float16))
+
+
+# ---------------------------------------------------------------- row-resident kernels with chained reductions
+@pytest.mark.parametrize("rows,cols", [(256, 1024), (128, 8192), (1000, 512), (300, 2048)])
+def test_generated_softmax_family_is_one_kernel(T, oracle, rows, cols):
+    """softmax, log_softmax and a layer norm built from tensor ops are each an elementwise kernel fed
+    by two keepdim reductions over the last axis, the second building on the first: with the
+    hand-written softmax switched off (or for bf16, which it does not cover) they run as ONE
+    row-resident kernel: the row is loaded once, both totals stay in registers."""
+    from morok_amd import synth, uop
+
+    x = synth.normal((rows, cols), 95, 0, sigma=2.0)
+    T.set_fusion(False)
+    t = T.Tensor.from_numpy(x).softmax(-1)
+    got = t.to_numpy()
+    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("rE_%d_g%d" % (rows, cols)) and t.kernels()[0].endswith("_x2")
+    np.testing.assert_allclose(got, oracle.softmax_f32(x), rtol=1e-5, atol=1e-9)
+    ls = T.Tensor.from_numpy(x).log_softmax(-1)
+    got = ls.to_numpy()
+    assert len(ls.kernels()) == 1 and ls.kernels()[0].endswith("_x2")
+    x64 = x.astype(np.float64)
+    ref = x64 - x64.max(-1, keepdims=True)
+    ref = ref - np.log(np.exp(ref).sum(-1, keepdims=True))
+    assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max()
+    tx = T.Tensor.from_numpy(x)
+    xc = tx.try_sub(tx.mean(-1, keepdim=True))
+    ln = xc.try_mul(xc.try_mul(xc).mean(-1, keepdim=True).try_add(T.Tensor.const(1e-5)).try_rsqrt())
+    got = ln.to_numpy()
+    assert len(ln.kernels()) == 1 and ln.kernels()[0].endswith("_x2")
+    c64 = x64 - x64.mean(-1, keepdims=True)
+    ref = c64 / np.sqrt((c64 * c64).mean(-1, keepdims=True) + 1e-5)
+    assert np.abs(got - ref).max() <= 1e-4 * np.abs(ref).max()
+    T.set_fusion(True)
+    xb = synth.normal_bf16((rows, cols), 95, 1)
+    tb = T.Tensor.from_numpy(xb, uop.BF16).softmax(-1)
+    got = synth.from_bf16(tb.to_numpy())
+    assert len(tb.kernels()) == 1 and tb.kernels()[0].endswith("_x2")
+    ref = oracle.softmax_f32(synth.from_bf16(xb))
+    assert np.abs(got - ref).max() <= 2e-2 * ref.max()
+
+
+def test_chained_row_fusion_falls_back_when_a_total_is_needed_elsewhere(T):
+    from morok_amd import synth
+
+    x = synth.normal((256, 1024), 96, 0)
+    T.set_fusion(False)
+    tx = T.Tensor.from_numpy(x)
+    m = tx.max(-1, keepdim=True)
+    e = tx.try_sub(m).try_exp()
+    both = e.try_div(e.sum(-1, keepdim=True)).try_add(m.try_expand([256, 1024]))     # the maximum has a second reader
+    got = both.to_numpy()
+    x64 = x.astype(np.float64)
+    e64 = np.exp(x64 - x64.max(-1, keepdims=True))
+    ref = e64 / e64.sum(-1, keepdims=True) + x64.max(-1, keepdims=True)
+    assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max() and len(both.kernels()) >= 2
