@@ -289,7 +289,8 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     // is relative and the row sum is f32, so the result does not depend on the reference
     // point.  The first tile always rescales (m_run = -inf); key 0 is visible to every
     // query, so m_run is finite from then on.
-    auto body = [&](int j, f32x16 (&cur)[2], float mx_cur, f32x16 (&nxt)[2], float& mx_nxt, auto mask_next) {
+    auto body = [&](int j, f32x16 (&cur)[2], float mx_cur, f32x16 (&nxt)[2], float& mx_nxt, auto mask_next, auto last_tile) {
+        constexpr bool kLast = decltype(last_tile)::value;  // the wave's last tile: there is no S(j+1) to compute
         if (__builtin_amdgcn_ballot_w64(mx_cur > m_run + lazy_thresh) != 0) {
             const float m_new = fmaxf(m_run, mx_cur);
             const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
@@ -309,33 +310,38 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
 
         // ---- phase A: S(j+1) = K(j+1) Q^T on the matrix pipe, P(j) = exp2(S(j)*c - m*c) on
         // the vector ALUs: each of the 16 (8; 32) MFMAs is followed by the exponentials of two (four; every second one by two)
-        // score registers (the last iteration computes a tile nobody uses).  The fences keep the
+        // score registers (a wave's last tile has no successor: that instantiation runs the exponentials alone).  The fences keep the
         // compiler from regrouping the two instruction streams.
         float psum0 = 0.0f, psum1 = 0.0f;
         bf16x8 pb[2][2];
         {
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                for (int e = 0; e < 16; e++) nxt[kb][e] = 0.0f;
             bf16x8 kf[2][2];
+            if constexpr (!kLast) {
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-                kf[0][kb] = *LDS_PTR(bf16x8, sKn + kb * 32 * kRow + k_row_off + (((0 + lg) ^ k_sw) << 4));
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int e = 0; e < 16; e++) nxt[kb][e] = 0.0f;
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+                    kf[0][kb] = *LDS_PTR(bf16x8, sKn + kb * 32 * kRow + k_row_off + (((0 + lg) ^ k_sw) << 4));
+            }
             f32x8 p;
             constexpr int kMfmaA = 2 * kDS;  // score MFMAs of this phase; the 16 pairs of score registers are spread over them:
                                              // one per MFMA (D = 128), two (64), one after every second (256)
 #pragma unroll
             for (int ds = 0; ds < kDS; ds++) {
-                if (ds + 1 < kDS) {
+                if constexpr (!kLast) {
+                    if (ds + 1 < kDS) {
 #pragma unroll
-                    for (int kb = 0; kb < 2; kb++)
-                        kf[(ds + 1) & 1][kb] =
-                            *LDS_PTR(bf16x8, sKn + kb * 32 * kRow + k_row_off + (((2 * (ds + 1) + lg) ^ k_sw) << 4));
+                        for (int kb = 0; kb < 2; kb++)
+                            kf[(ds + 1) & 1][kb] =
+                                *LDS_PTR(bf16x8, sKn + kb * 32 * kRow + k_row_off + (((2 * (ds + 1) + lg) ^ k_sw) << 4));
+                    }
                 }
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++) {
-                    nxt[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds & 1][kb], qf[ds], nxt[kb], 0, 0, 0);
+                    if constexpr (!kLast)
+                        nxt[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ds & 1][kb], qf[ds], nxt[kb], 0, 0, 0);
 #pragma unroll
                     for (int idx = (ds * 2 + kb) * 16 / kMfmaA; idx < (ds * 2 + kb + 1) * 16 / kMfmaA; idx++) {  // 0..15: score registers 2*idx, 2*idx+1
                         const int pk = idx >> 3, pe = (idx & 7) * 2;  // block, register inside the block
@@ -375,7 +381,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
                 if (n + 2 < kNB) vf[(n + 2) % 3] = vfrag(n + 2);
                 const int kbt = n / kDB, db = n % kDB;
                 o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[n % 3], pb[kbt >> 1][kbt & 1], o[db], 0, 0, 0);
-                if (n >= kNB / 2) {  // the score MFMAs have drained by now: 4 (8) registers per slot
+                if (!kLast && n >= kNB / 2) {  // the score MFMAs have drained by now: 4 (8) registers per slot
                     constexpr int kSlotsPerKb = kNB / 4, kRegs = 16 / kSlotsPerKb;
                     const int kb = (n - kNB / 2) / kSlotsPerKb, e0 = ((n - kNB / 2) % kSlotsPerKb) * kRegs;
 #pragma unroll
@@ -394,7 +400,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        {
+        if constexpr (!kLast) {
             const float mx = fmaxf(mx0, mx1);
             // the other 16 keys of every 32 sit in lane l ^ 32
             mx_nxt = max_with_other_half(mx);
@@ -412,25 +418,57 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         // only keeps the barrier rhythm and copies its share of them for the other waves
         int nmine = ntiles;
         if (causal && (qw0 + 31) / kKT + 1 < nmine) nmine = (qw0 + 31) / kKT + 1;
-        const int jm = first_masked - 1 < nmine ? first_masked - 1 : nmine;  // iterations whose next tile is unmasked
-        for (; j + 1 < jm; j += 2) {
-            body(j, sa, mxa, sb, mxb, std::false_type{});
-            body(j + 1, sb, mxb, sa, mxa, std::false_type{});
-        }
-        if (j < jm) {
-            body(j, sa, mxa, sb, mxb, std::false_type{});
-            sa[0] = sb[0];
-            sa[1] = sb[1];
-            mxa = mxb;
+        constexpr std::false_type more{};
+        if constexpr (kD < 256) {
+            const int nl = nmine - 1;  // iterations that have a next tile; the wave's last one is a body of its own
+            const int jm = first_masked - 1 < nl ? first_masked - 1 : nl;  // iterations whose next tile is unmasked
+            for (; j + 1 < jm; j += 2) {
+                body(j, sa, mxa, sb, mxb, std::false_type{}, more);
+                body(j + 1, sb, mxb, sa, mxa, std::false_type{}, more);
+            }
+            if (j < jm) {
+                body(j, sa, mxa, sb, mxb, std::false_type{}, more);
+                sa[0] = sb[0];
+                sa[1] = sb[1];
+                mxa = mxb;
+                j++;
+            }
+            for (; j + 1 < nl; j += 2) {
+                body(j, sa, mxa, sb, mxb, std::true_type{}, more);
+                body(j + 1, sb, mxb, sa, mxa, std::true_type{}, more);
+            }
+            if (j < nl) {
+                body(j, sa, mxa, sb, mxb, std::true_type{}, more);
+                sa[0] = sb[0];
+                sa[1] = sb[1];
+                mxa = mxb;
+                j++;
+            }
+            body(j, sa, mxa, sb, mxb, std::false_type{}, std::true_type{});
             j++;
-        }
-        for (; j + 1 < nmine; j += 2) {
-            body(j, sa, mxa, sb, mxb, std::true_type{});
-            body(j + 1, sb, mxb, sa, mxa, std::true_type{});
-        }
-        if (j < nmine) {
-            body(j, sa, mxa, sb, mxb, std::true_type{});
-            j++;
+        } else {
+            // with 512-byte rows one more instantiation of the body would push the kernel over
+            // its register budget: the last tile runs the ordinary body and its S(j+1) goes unused
+            const int jm = first_masked - 1 < nmine ? first_masked - 1 : nmine;
+            for (; j + 1 < jm; j += 2) {
+                body(j, sa, mxa, sb, mxb, std::false_type{}, more);
+                body(j + 1, sb, mxb, sa, mxa, std::false_type{}, more);
+            }
+            if (j < jm) {
+                body(j, sa, mxa, sb, mxb, std::false_type{}, more);
+                sa[0] = sb[0];
+                sa[1] = sb[1];
+                mxa = mxb;
+                j++;
+            }
+            for (; j + 1 < nmine; j += 2) {
+                body(j, sa, mxa, sb, mxb, std::true_type{}, more);
+                body(j + 1, sb, mxb, sa, mxa, std::true_type{}, more);
+            }
+            if (j < nmine) {
+                body(j, sa, mxa, sb, mxb, std::true_type{}, more);
+                j++;
+            }
         }
         for (; j < ntiles; j++) {
             tile_barrier();
