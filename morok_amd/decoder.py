@@ -57,6 +57,9 @@ class DecoderBlock:
         self.cos_host, self.sin_host = cos, sin
         self.cos = Tensor.from_numpy(cos.reshape(1, 1, seq, self.dim // 2), device_id=device_id)
         self.sin = Tensor.from_numpy(sin.reshape(1, 1, seq, self.dim // 2), device_id=device_id)
+        # the same tables shaped for a token-major [batch, seq, heads, dim] operand
+        self.cos_tm = Tensor.from_numpy(cos.reshape(1, seq, 1, self.dim // 2), device_id=device_id)
+        self.sin_tm = Tensor.from_numpy(sin.reshape(1, seq, 1, self.dim // 2), device_id=device_id)
 
     def _heads(self, x):
         """[T, hidden] token-major -> [B, H, S, D] head-major (a view: no copy by itself)."""
@@ -74,13 +77,15 @@ class DecoderBlock:
             qkv = xn.matmul(w["Wqkv"])
             xv = qkv.try_shrink([(0, T), (2 * self.hidden, 3 * self.hidden)])
             # q and k lie side by side in the packed product: one rotary kernel over 2 * heads heads
-            # (the same per-head arithmetic), q and k are then the two halves of its result
+            # (the same per-head arithmetic).  Its result stays token-major (whole 2 * hidden rows
+            # in, whole rows out); q and k are head-major views of its two halves, which the
+            # attention kernel reads in place
             xqk = qkv.try_shrink([(0, T), (0, 2 * self.hidden)])
-            qk = xqk.try_reshape([self.batch, self.seq, 2 * self.heads, self.dim]).try_permute([0, 2, 1, 3])
-            qk = qk.apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16).contiguous()
-            full = [(0, self.batch), None, (0, self.seq), (0, self.dim)]
-            q = qk.try_shrink([r if r else (0, self.heads) for r in full])
-            k = qk.try_shrink([r if r else (self.heads, 2 * self.heads) for r in full])
+            qk = xqk.try_reshape([self.batch, self.seq, 2 * self.heads, self.dim])
+            qk = qk.apply_rotary_emb(self.cos_tm, self.sin_tm, False).cast(uop.BF16).contiguous()
+            full = [(0, self.batch), (0, self.seq), None, (0, self.dim)]
+            q = qk.try_shrink([r if r else (0, self.heads) for r in full]).try_permute([0, 2, 1, 3])
+            k = qk.try_shrink([r if r else (self.heads, 2 * self.heads) for r in full]).try_permute([0, 2, 1, 3])
         else:
             xq, xk, xv = xn.matmul(w["Wq"]), xn.matmul(w["Wk"]), xn.matmul(w["Wv"])
             q = self._heads(xq).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
