@@ -415,7 +415,7 @@ def bench_mfma_ceiling(m, dev, steps, warmup, cpu):
     smooth = _mfma_ceiling_tflops(m, dev, False)
     return {"metric": "MFMA-only ceiling TFLOP/s", "smooth_operands_value": smooth, "value": tf, "unit": "TFLOP/s", "ms_per_step": 2.0 * 4096 ** 3 / tf / 1e9,
             "dtype": "bf16", "config": {"workload": "calibration: 256 workgroups x 64 K steps of register-only "
-                                                    "v_mfma_f32_32x32x16_bf16 (the MFMA stream of the 4096^3 GEMM), hashed operand values"},
+                                                    "v_mfma_f32_16x16x32_bf16 (the MFMA stream of the 4096^3 GEMM), hashed operand values"},
             "roofline": {"bound": "mfma", "achieved": tf, "peak": BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                          "frac": tf / BF16_PEAK_TFLOPS, "traffic": 0, "traffic_source": "no memory operands",
                          "kernel": "mfma_ceiling_kernel", "algorithmic_flops_per_launch": 2.0 * 4096 ** 3}}

@@ -5,29 +5,31 @@
 // (tensor/src/matmul.rs:82-110: broadcast multiply then sum(-1) with the accumulator
 // promoted to f32, tensor/src/reduce.rs:101-117, cast back 665-691) after the tensor-core
 // rewrite (schedule/src/optimizer/tc.rs:36-94 strips the CAST around the product, so
-// exact bf16*bf16 products are accumulated in f32).  The reference names the instruction
-// shape in its CDNA table (schedule/src/optimizer/renderer.rs:549-558,724-733); this
-// hand-written kernel uses the 32x32x16 shape of the same family for more flops per LDS
-// byte.
+// exact bf16*bf16 products are accumulated in f32).  The instruction is the 16x16x32 shape the
+// reference names in its CDNA table (schedule/src/optimizer/renderer.rs:549-558,724-733): of
+// the two bf16 shapes of gfx950 it is the one the part sustains the higher clock on (it moves
+// less accumulator data per product than 32x32x16; 1.96 against 1.72 PFLOP/s from registers).
 //
 // Main kernel: 256x256 output tile per workgroup of 4 waves (2x2), each wave 128x128 =
-// 4x4 MFMA tiles (256 accumulator registers), K step 64.  Tiles travel global -> LDS
-// directly (global_load_lds, 16 B per lane, no register staging).  A is kept in LDS
+// 8x8 MFMA tiles (256 accumulator registers), K step 64 = two 32-deep sub-steps.  Tiles travel
+// global -> LDS directly (global_load_lds, 16 B per lane, no register staging).  A is kept in LDS
 // row-major with an XOR swizzle of its 16-byte chunks, B row-major (n contiguous) with
 // an XOR swizzle of its 32-byte granules and read through the transposing LDS load,
 // which hands each lane the 4 consecutive-k values of its column.  The MFMA is issued with
 // swapped operands (D' = B^T A^T) so each lane ends up with 4 consecutive n of one row,
-// which makes the epilogue 8-byte LDS writes and 16-byte coalesced global stores.
+// which makes the epilogue 8-byte LDS writes and 16-byte coalesced global stores.  A second
+// operand stored as B^T [N, K] (k contiguous: a Linear layer's weight) is staged and read
+// exactly like A instead.
 //
 // Pipeline.  The vector-memory path takes a 1 KB copy every ~16 cycles, so the 64 copies a
 // workgroup issues per K step need about half of the step's MFMA time; issued in one burst
 // they stall the waves' instruction streams behind them.  They are therefore spread evenly,
-// four per 16-MFMA phase and wave: the LDS holds two A stages and three B stages (160 KB, all
+// four per 32-MFMA phase and wave: the LDS holds two A stages and three B stages (160 KB, all
 // of it), the copies of B tile kt+2 go out during the first two phases of tile kt into the
 // stage tile kt-1 left, the one barrier of the step sits in the middle of it, and the copies
 // of A tile kt+2 follow in the last two phases into the stage tile kt has just left.  For the
 // barrier to sit there every fragment of tile kt must have been read by then: fragments are
-// read two phases ahead of their MFMAs into four register slots (one per 16-deep k-step).
+// read a sub-step ahead of their MFMAs into two register slots (one per 32-deep sub-step).
 //
 // Shapes.  M is arbitrary, N and K multiples of 8: edge tiles redirect out-of-range rows and
 // column chunks to the last valid one and mask their stores; a partial last K step is copied
@@ -86,7 +88,7 @@ __device__ __attribute__((aligned(16))) const unsigned g_zero16[4] = {0u, 0u, 0u
 // per-lane 64-bit addresses so that chunks beyond K can be redirected to g_zero16: zero
 // operands on both sides contribute nothing.  Every other step is copied as in the full case.
 //
-// kJ: 32-column MFMA tiles per wave.  kJ = 4: 256x256 workgroup tile, waves 2x2, each 128x128.
+// kJ: 32-column blocks (two MFMA tile columns each) per wave.  kJ = 4: 256x256 workgroup tile, waves 2x2, each 128x128.
 // kJ = 2: 128x256 workgroup tile, waves 1x4, each 128x64 (half the accumulators, an A stage of
 // half the size, the same B stages and pipeline) for shapes whose 256x256 tiles would leave
 // most compute units without work.
@@ -100,13 +102,17 @@ __device__ __attribute__((aligned(16))) const unsigned g_zero16[4] = {0u, 0u, 0u
 // C = bf16(float(bf16(A B)) + float(R)): the bits of the product kernel followed by an
 // elementwise add, without writing and re-reading the product.
 //
+// kBT: the second operand is stored as B^T [N, K] (k contiguous).  Its stage holds 256 n-rows of
+// 128 B, chunk-swizzled, copied and read like an A stage: one 16-byte read per fragment instead of
+// two transposing 8-byte reads.  Same products in the same order: the same bits as the [K, N] form.
+//
 // kSwiGLU (256-row tile only): B is [K, 2F] holding a gate matrix in its columns [0, F) and an up
 // matrix in [F, 2F) (N = 2F is B's row pitch); the workgroup's 256 tile columns are 128 gate
 // columns followed by the 128 up columns at the same offset, and the epilogue writes
 // C[M, F] = bf16(silu(float(bf16(A gate))) * float(bf16(A up))): the two products rounded to bf16
 // as separate kernels would leave them, then x * sigmoid(x) * y in f32 with one rounding, without
 // the 2F-wide product ever reaching memory.
-template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false, bool kSwiGLU = false>
+template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false, bool kSwiGLU = false, bool kBT = false>
 __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
                                                float* __restrict__ W = nullptr, int kt_per_split = 0,
@@ -118,7 +124,8 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     constexpr int kCWaveT = 128 * kCPitchT;
     constexpr int kSmemMainT = 2 * kAStageT + 3 * kBStageSw;
     constexpr int kSmemT = 4 * kCWaveT > kSmemMainT ? 4 * kCWaveT : kSmemMainT;
-    constexpr int kSlots = 4 * kJ;                // MFMAs per phase
+    constexpr int kI16 = 8, kJ16 = 2 * kJ;        // 16x16 MFMA tiles per wave: rows, columns
+    constexpr int kSlots = 4 * kJ16;              // MFMAs per phase (four tile rows x all tile columns)
     // A stage: kTM rows x 128 B, 16 B chunks XOR-swizzled by ((row >> 1) & 7);
     // B stage: 64 k-rows x 512 B, 32 B granules XOR-swizzled by (k & 3).
     __shared__ __attribute__((aligned(1024))) char smem[kSmemT];
@@ -157,6 +164,27 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         a_voff[q] = (unsigned)(((row - m0) * K + (chunk << 3)) * 2);
     }
     const int b_h = lane & 1, b_g = (lane & 31) >> 1, b_r = lane >> 5;
+    // kBT: B^T chunk q (1 KB = 8 n-rows of 128 B), copied and swizzled exactly like an A chunk;
+    // each wave moves the 64 rows wave*64 .. wave*64+63 of the stage.
+    unsigned bt_voff[kBT ? 8 : 1];
+    if constexpr (kBT) {
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const size_t lr = wave * 64 + q * 8 + (lane >> 3);  // row inside the 256-row stage
+            size_t row;
+            if (kSwiGLU) {
+                // stage rows 0..127 are gate rows of B^T, 128..255 the up rows at the same offset
+                const size_t F = (size_t)N / 2, half = lr >> 7;
+                row = n0 + (lr & 127);
+                row = (row < F ? row : F - 1) + half * F;
+            } else {
+                row = n0 + lr;
+                row = row < (size_t)N ? row : (size_t)N - 1;
+            }
+            const int chunk = (lane & 7) ^ ((q & 1) * 4 + (lane >> 4));
+            bt_voff[q] = (unsigned)(((row - n0) * K + (chunk << 3)) * 2);
+        }
+    }
     unsigned b_voff[2];
 #pragma unroll
     for (int par = 0; par < 2; par++) {
@@ -176,7 +204,8 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     const int KT = kSplitK ? (KT_all - kt0 < kt_per_split ? KT_all - kt0 : kt_per_split) : KT_all;
     const bool has_last = kt0 + KT == KT_all;  // the (possibly partial) last K step is in this range
     const char* a_tile = reinterpret_cast<const char*>(A + m0 * K) + (size_t)kt0 * kBK * 2;
-    const char* b_tile = reinterpret_cast<const char*>(B + n0) + (size_t)kt0 * kBK * N * 2;
+    const char* b_tile = kBT ? reinterpret_cast<const char*>(B + n0 * K) + (size_t)kt0 * kBK * 2
+                             : reinterpret_cast<const char*>(B + n0) + (size_t)kt0 * kBK * N * 2;
     const unsigned lds_a = (unsigned)(uintptr_t)LDS_PTR(char, sA0) + wave * (kAq * 1024);
     const unsigned lds_b = (unsigned)(uintptr_t)LDS_PTR(char, sB0) + wave * 8192;
     // One direct copy: 64 lanes x 16 B land at LDS [m0, m0 + 1 KB); the compiler is not told
@@ -203,6 +232,16 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         }
     };
     auto dma_b = [&](int q, int kt, int stage) {
+        if constexpr (kBT) {
+            if (kRaggedK && has_last && kt == KT - 1) {
+                const int chunk = (lane & 7) ^ ((q & 1) * 4 + (lane >> 4));
+                dma_from(lds_b + stage * kBStageSw + q * 1024,
+                         chunk * 8 < k_last ? b_tile + (size_t)kt * kBK * 2 + bt_voff[q] : zero16);
+            } else {
+                dma(lds_b + stage * kBStageSw + q * 1024, bt_voff[q], b_tile + (size_t)kt * kBK * 2);
+            }
+            return;
+        }
         if (kRaggedK && has_last && kt == KT - 1) {
             dma_from(lds_b + stage * kBStageSw + q * 1024,
                      wave * 16 + q * 2 + b_r < k_last ? b_tile + ((size_t)kt * kBK + q * 2) * N * 2 + b_voff[q & 1] : zero16);
@@ -211,26 +250,31 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         dma(lds_b + stage * kBStageSw + q * 1024, b_voff[q & 1], b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
     };
 
-    f32x16 acc[4][kJ];
+    f32x4 acc[kI16][kJ16];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < kI16; i++)
 #pragma unroll
-        for (int j = 0; j < kJ; j++)
+        for (int j = 0; j < kJ16; j++)
 #pragma unroll
-            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.0f;
+            for (int e = 0; e < 4; e++) acc[i][j][e] = 0.0f;
 
-    // lane-constant parts of the fragment addresses
-    const int a_base_l = (wm * 128 + (lane & 31)) * 128;  // + i*4096
-    int a_xo[4];
+    // lane-constant parts of the fragment addresses.  An operand fragment of the 16x16x32 MFMA is
+    // row (lane % 16) of a 16-row tile, k = 8 * (lane / 16) .. +7 of the 32-deep sub-step.
+    const int a_base_l = (wm * 128 + (lane & 15)) * 128;  // + i*2048
+    int a_xo[2];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) a_xo[ks] = ((ks * 2 + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4;
+    for (int ks = 0; ks < 2; ks++) a_xo[ks] = ((ks * 4 + (lane >> 4)) ^ ((lane >> 1) & 7)) << 4;
+    // B through the transposing read: 16-lane block b = lane / 16 covers k-rows 8b .. 8b+7 (two
+    // reads of four rows), lane j' of the block points at k-row j'/4, 8-byte unit j'%4 of the
+    // 32-byte granule (16 columns) of its tile column
     const int b_rr = (lane & 15) >> 2;
-    const int b_g0 = wn * (2 * kJ) + ((lane >> 4) & 1);  // first 16-column granule of this wave
-    const int b_row_l = (8 * (lane >> 5) + b_rr) * 512 + 8 * (lane & 3);  // + ks*16*512 + r*4*512
-    const int b_p0 = b_row_l + ((b_g0 ^ b_rr) << 5);                      // j = 0 (+128: j = 2)
-    const int b_p1 = b_row_l + (((b_g0 ^ b_rr) ^ 2) << 5);                // j = 1 (+128: j = 3)
+    const int b_row_l = (8 * (lane >> 4) + b_rr) * 512 + 8 * (lane & 3) + ((wn * kJ16) << 5);  // + ks*32*512 (+ 4*512: second read)
+    int b_p[4];  // tile column j: b_p[j & 3] + (j >> 2) * 128
+#pragma unroll
+    for (int q = 0; q < 4; q++) b_p[q] = b_row_l + ((q ^ b_rr) << 5);
+    const int bt_base_l = (wn * (kJ * 32) + (lane & 15)) * 128;  // kBT: + j*2048, chunk offset a_xo[ks]
 
-    bf16x8 fa[4][4], fb[4][kJ];  // fragment slot = k-step
+    bf16x8 fa[2][kI16], fb[2][kJ16];  // fragment slot = 32-deep sub-step
     // all but this wave's newest 8 copies (the B chunks issued since the last barrier) have
     // landed, its LDS reads are complete; then all waves meet
     auto tile_barrier = [&]() { asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
@@ -248,44 +292,61 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     // tile_barrier() covers them)
     if (kAq == 8) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(12) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    // B fragment of tile column j, sub-step base sB (a stage plus ks * 32 rows)
+    auto read_b = [&](const char* sB, int j, bf16x4* lo, bf16x4* hi) {
+        const int off = b_p[j & 3] + (j >> 2) * 128;
+        *lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off));
+        *hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off + 4 * 512));
+    };
+    {  // the fragments of sub-step 0 of tile 0
+        const char* sA = sA0 + a_base_l + a_xo[0];
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++) {
-        const char* sA = sA0 + a_base_l + a_xo[ks];
-        const char* sB = sB0 + ks * 16 * 512;
+        for (int i = 0; i < kI16; i++) fa[0][i] = *LDS_PTR(bf16x8, sA + i * 2048);
 #pragma unroll
-        for (int i = 0; i < 4; i++) fa[ks][i] = *LDS_PTR(bf16x8, sA + i * 4096);
-#pragma unroll
-        for (int j = 0; j < kJ; j++) {
-            const int off = ((j & 1) ? b_p1 : b_p0) + (j >> 1) * 128;
-            bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off));
-            bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sB + off + 4 * 512));
-            fb[ks][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        for (int j = 0; j < kJ16; j++) {
+            if constexpr (kBT) {
+                fb[0][j] = *LDS_PTR(bf16x8, sB0 + bt_base_l + a_xo[0] + j * 2048);
+            } else {
+                bf16x4 lo, hi;
+                read_b(sB0, j, &lo, &hi);
+                fb[0][j] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
         }
     }
 
-    // One phase = the 4 * kJ MFMAs of k-step p of the current tile (fragment slot p) with the
-    // other pipes' work slotted between them: the 4 + 2 * kJ LDS reads of the fragments needed two
-    // phases later (slot p ^ 2, from sAn / sBn) and chunk copies of tile kt2: phases 0-1 four of
-    // its B chunks each into B stage st2, phases 2-3 (after the barrier) kAq / 2 of its A chunks
-    // each into A stage `cur`.
+    // One phase = half of a 32-deep sub-step: phase p covers sub-step p / 2 (fragment slot p / 2)
+    // and tile rows 4 * (p % 2) .. +3 against every tile column, 4 * kJ16 MFMAs, with the other
+    // pipes' work slotted between them: the LDS reads of the other slot's fragments (the next
+    // sub-step; from sAn / sBn) for the same four tile rows and half of the tile columns, and
+    // chunk copies of tile kt2: phases 0-1 four of its B chunks each into B stage st2, phases 2-3
+    // (after the barrier) kAq / 2 of its A chunks each into A stage `cur`.  The columns loaded
+    // during the second phase of a sub-step are the ones the next sub-step multiplies last.
     auto phase = [&](auto p_c, auto cur_c, int kt2, int st2, const char* sAn, const char* sBn) {
         constexpr int p = decltype(p_c)::value, cur = decltype(cur_c)::value;
-        constexpr int slot = p, nslot = p ^ 2;
-        bf16x4 lo[kJ], hi[kJ];
+        constexpr int slot = p >> 1, nslot = slot ^ 1, h = p & 1;
+        constexpr int kHalfJ = kJ16 / 2;  // tile columns per half
+        bf16x4 lo[kHalfJ], hi[kHalfJ];
         constexpr int kBEvery = kSlots / 4, kAEvery = kSlots / (kAq / 2);  // slots between two copies
 #pragma unroll
         for (int n = 0; n < kSlots; n++) {
-            // back and forth over the columns: at a row change only the row operand changes, so
-            // consecutive instructions share one operand register set every time instead of three
-            // times in four (fewer operand bits toggle: about 1 % on the clock the part sustains)
-            const int mi = n / kJ, mj = (mi & 1) ? kJ - 1 - n % kJ : n % kJ;
-            acc[mi][mj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[slot][mj], fa[slot][mi], acc[mi][mj], 0, 0, 0);
-            if (n < 4) fa[nslot][n] = *LDS_PTR(bf16x8, sAn + n * 4096);
-            else if (n < 4 + 2 * kJ) {
-                const int j = (n - 4) >> 1;
-                const int off = ((j & 1) ? b_p1 : b_p0) + (j >> 1) * 128;
-                if ((n & 1) == 0) lo[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off));
-                else hi[j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off + 4 * 512));
+            // first the columns whose fragments arrived a sub-step ago, then the other half; back
+            // and forth over the columns and the rows, so that consecutive instructions share one
+            // operand register set (fewer operand bits toggle: about 1 % on the clock the part
+            // sustains)
+            const int jh = n / (kSlots / 2), r = n % (kSlots / 2), rr = r / kHalfJ, jj = r % kHalfJ;
+            const int mi = 4 * h + (jh ? 3 - rr : rr);
+            const int mj = jh * kHalfJ + ((rr & 1) ? kHalfJ - 1 - jj : jj);
+            // (written out so that the accumulator stays in place in the accumulation registers:
+            // through the builtin the compiler leaves this shape untied and copies tiles around)
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[mi][mj]) : "v"(fb[slot][mj]), "v"(fa[slot][mi]));
+            if (n < 4) fa[nslot][4 * h + n] = *LDS_PTR(bf16x8, sAn + (4 * h + n) * 2048);
+            else if constexpr (kBT) {
+                if (n < 4 + kHalfJ) fb[nslot][h * kHalfJ + n - 4] = *LDS_PTR(bf16x8, sBn + (h * kHalfJ + n - 4) * 2048);
+            } else if (n < 4 + 2 * kHalfJ) {
+                const int jl = (n - 4) >> 1, j = h * kHalfJ + jl;
+                const int off = b_p[j & 3] + (j >> 2) * 128;
+                if ((n & 1) == 0) lo[jl] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off));
+                else hi[jl] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off + 4 * 512));
             }
             if (p < 2) {
                 if (n % kBEvery == 1 % kBEvery) dma_b((p & 1) * 4 + n / kBEvery, kt2, st2);
@@ -294,8 +355,11 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        if constexpr (!kBT) {
 #pragma unroll
-        for (int j = 0; j < kJ; j++) fb[nslot][j] = __builtin_shufflevector(lo[j], hi[j], 0, 1, 2, 3, 4, 5, 6, 7);
+            for (int jl = 0; jl < kHalfJ; jl++)
+                fb[nslot][h * kHalfJ + jl] = __builtin_shufflevector(lo[jl], hi[jl], 0, 1, 2, 3, 4, 5, 6, 7);
+        }
         __builtin_amdgcn_sched_barrier(0);
     };
     using C0 = std::integral_constant<int, 0>;
@@ -308,15 +372,17 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         using C = std::integral_constant<int, cur>;
         const int kt2 = kt + 2 < KT ? kt + 2 : KT - 1;
         const char* sAc = sA0 + cur * kAStageT + a_base_l;
-        const char* sBc = sB0 + st * kBStageSw;
+        const char* sBc = sB0 + st * kBStageSw + (kBT ? bt_base_l : 0);
         const char* sAx = sA0 + (cur ^ 1) * kAStageT + a_base_l;
-        const char* sBx = sB0 + stn * kBStageSw;
-        phase(C0{}, C{}, kt2, st2, sAc + a_xo[2], sBc + 2 * 16 * 512);
-        phase(C1{}, C{}, kt2, st2, sAc + a_xo[3], sBc + 3 * 16 * 512);
+        const char* sBx = sB0 + stn * kBStageSw + (kBT ? bt_base_l : 0);
+        // sub-step ks of a B stage: 32 k-rows of 512 B further, or (kBT) the same chunk offset as A's
+        auto b_ks = [&](int ks) { return kBT ? a_xo[ks] : ks * 32 * 512; };
+        phase(C0{}, C{}, kt2, st2, sAc + a_xo[1], sBc + b_ks(1));
+        phase(C1{}, C{}, kt2, st2, sAc + a_xo[1], sBc + b_ks(1));
         // tile kt+1 has landed; nobody reads A stage cur any more
         tile_barrier();
-        phase(C2{}, C{}, kt2, st2, sAx + a_xo[0], sBx);
-        phase(C3{}, C{}, kt2, st2, sAx + a_xo[1], sBx + 1 * 16 * 512);
+        phase(C2{}, C{}, kt2, st2, sAx + a_xo[0], sBx + b_ks(0));
+        phase(C3{}, C{}, kt2, st2, sAx + a_xo[0], sBx + b_ks(0));
     };
     {
         int kt = 0, st = 0;
@@ -330,23 +396,23 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         if (kt < KT) iteration(C0{}, kt, st, nx(st), nx(nx(st)));
     }
     full_barrier();
+    // the last MFMAs' results must have left the matrix pipe before the vector ALUs read them
+    // (the compiler does not see the instructions above as matrix operations)
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
-    // Epilogue.  With swapped operands lane l of tile (i, j) holds, in registers 4g..4g+3,
-    // C[m = i*32 + l%32][n = j*32 + 8g + 4*(l/32) + 0..3].
+    // Epilogue.  With swapped operands lane l of tile (i, j) holds, in its four registers,
+    // C[m = i*16 + l%16][n = j*16 + 4*(l/16) + 0..3].
     if (kSplitK) {
         // f32 partials straight from the registers: 16 bytes per lane, rows and columns masked
         const size_t row0 = m0 + wm * 128, col0 = n0 + wn * (kJ * 32);
         float* Wt = W + ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * (size_t)M * N;
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < kI16; i++)
 #pragma unroll
-            for (int j = 0; j < kJ; j++)
-#pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const size_t row = row0 + i * 32 + (lane & 31), col = col0 + j * 32 + 8 * g + 4 * (lane >> 5);
-                    f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                    if (row < (size_t)M && col + 4 <= (size_t)N) *reinterpret_cast<f32x4*>(Wt + row * N + col) = v;
-                }
+            for (int j = 0; j < kJ16; j++) {
+                const size_t row = row0 + i * 16 + (lane & 15), col = col0 + j * 16 + 4 * (lane >> 4);
+                if (row < (size_t)M && col + 4 <= (size_t)N) *reinterpret_cast<f32x4*>(Wt + row * N + col) = acc[i][j];
+            }
         return;
     }
     char* sC = smem + wave * kCWaveT;
@@ -372,17 +438,14 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     };
     if constexpr (kResidual) fetch_residual(0, kFirstBatch);
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < kI16; i++)
 #pragma unroll
-        for (int j = 0; j < kJ; j++)
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                f32x4 v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-                bf16x4 h = __builtin_convertvector(v, bf16x4);
-                const int ml = i * 32 + (lane & 31);
-                const int nl = j * 32 + 8 * g + 4 * (lane >> 5);
-                *LDS_PTR(bf16x4, sC + ml * kCPitchT + nl * 2) = h;
-            }
+        for (int j = 0; j < kJ16; j++) {
+            bf16x4 h = __builtin_convertvector(acc[i][j], bf16x4);
+            const int ml = i * 16 + (lane & 15);
+            const int nl = j * 16 + 4 * (lane >> 4);
+            *LDS_PTR(bf16x4, sC + ml * kCPitchT + nl * 2) = h;
+        }
     if constexpr (kResidual) fetch_residual(kFirstBatch, kIts);
     // a wave reads back only what it staged itself (the LDS serves a wave's requests in order),
     // except for the gated epilogue, where gate and up blocks come from two waves
@@ -439,6 +502,13 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
                                                          __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
                                                          int tiles_n) {
     gemm_tile_body<false, 4>(A, B, C, M, N, K, tiles_m, tiles_n);
+}
+// B^T variants: the second operand is Bt[N, K] row-major (k contiguous, the layout of a Linear
+// layer's weight), C = A Bt^T.
+__global__ __launch_bounds__(256) void gemm_bf16_nt_tile256(const __bf16* __restrict__ A, const __bf16* __restrict__ Bt,
+                                                            __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
+                                                            int tiles_n) {
+    gemm_tile_body<false, 4, false, false, false, true>(A, Bt, C, M, N, K, tiles_m, tiles_n);
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_ragged_k(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ B, __bf16* __restrict__ C,
@@ -688,6 +758,13 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     // the tiled kernel addresses a tile's rows with 32-bit byte offsets from the tile origin:
     // 255 rows of A (K elements each) and 49 rows of B (N elements each) must stay below 4 GiB
     const bool offsets_fit = K <= (1L << 23) && N <= (1L << 25);
+    if (variant == 6) {  // B given as Bt[N, K]
+        if (!aligned || !offsets_fit || K <= 0 || K % kBK || N % 8) return (int)hipErrorInvalidValue;
+        const long tn = (N + kBN - 1) / kBN, tm = (M + kBM - 1) / kBM;
+        gemm_bf16_nt_tile256<<<dim3((unsigned)(tm * tn), (unsigned)batch), 256, 0, s>>>(
+            static_cast<const __bf16*>(A), static_cast<const __bf16*>(B), static_cast<__bf16*>(C), (int)M, (int)N, (int)K, (int)tm, (int)tn);
+        return (int)hipGetLastError();
+    }
     // any M; N and K in whole 16-byte chunks
     if (variant != 2 && aligned && offsets_fit && K > 0 && N % 8 == 0 && K % 8 == 0) {
         const long tn = (N + kBN - 1) / kBN;
