@@ -222,32 +222,33 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     };
     const int k_last = K - (KT_all - 1) * kBK;  // depth of the last K step: 64, or 8..56 when ragged
     const char* zero16 = reinterpret_cast<const char*>(g_zero16);
-    auto dma_a = [&](int q, int kt, int stage) {
+    // (stage_off: byte offset of the stage inside the A or B part of the LDS)
+    auto dma_a = [&](int q, int kt, unsigned stage_off) {
         if (kRaggedK && has_last && kt == KT - 1) {
             const int chunk = (lane & 7) ^ ((q & 1) * 4 + (lane >> 4));  // logical 8-deep k chunk of this lane
-            dma_from(lds_a + stage * kAStageT + q * 1024,
+            dma_from(lds_a + stage_off + q * 1024,
                      chunk * 8 < k_last ? a_tile + (size_t)kt * kBK * 2 + a_voff[q] : zero16);
         } else {
-            dma(lds_a + stage * kAStageT + q * 1024, a_voff[q], a_tile + (size_t)kt * kBK * 2);
+            dma(lds_a + stage_off + q * 1024, a_voff[q], a_tile + (size_t)kt * kBK * 2);
         }
     };
-    auto dma_b = [&](int q, int kt, int stage) {
+    auto dma_b = [&](int q, int kt, unsigned stage_off) {
         if constexpr (kBT) {
             if (kRaggedK && has_last && kt == KT - 1) {
                 const int chunk = (lane & 7) ^ ((q & 1) * 4 + (lane >> 4));
-                dma_from(lds_b + stage * kBStageSw + q * 1024,
+                dma_from(lds_b + stage_off + q * 1024,
                          chunk * 8 < k_last ? b_tile + (size_t)kt * kBK * 2 + bt_voff[q] : zero16);
             } else {
-                dma(lds_b + stage * kBStageSw + q * 1024, bt_voff[q], b_tile + (size_t)kt * kBK * 2);
+                dma(lds_b + stage_off + q * 1024, bt_voff[q], b_tile + (size_t)kt * kBK * 2);
             }
             return;
         }
         if (kRaggedK && has_last && kt == KT - 1) {
-            dma_from(lds_b + stage * kBStageSw + q * 1024,
+            dma_from(lds_b + stage_off + q * 1024,
                      wave * 16 + q * 2 + b_r < k_last ? b_tile + ((size_t)kt * kBK + q * 2) * N * 2 + b_voff[q & 1] : zero16);
             return;
         }
-        dma(lds_b + stage * kBStageSw + q * 1024, b_voff[q & 1], b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
+        dma(lds_b + stage_off + q * 1024, b_voff[q & 1], b_tile + ((size_t)kt * kBK + q * 2) * N * 2);
     };
 
     f32x4 acc[kI16][kJ16];
@@ -285,9 +286,9 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
 #pragma unroll
     for (int q = 0; q < 8; q++) dma_b(q, 0, 0);
 #pragma unroll
-    for (int q = 0; q < kAq; q++) dma_a(q, KT > 1 ? 1 : 0, 1);
+    for (int q = 0; q < kAq; q++) dma_a(q, KT > 1 ? 1 : 0, kAStageT);
 #pragma unroll
-    for (int q = 0; q < 8; q++) dma_b(q, KT > 1 ? 1 : 0, 1);
+    for (int q = 0; q < 8; q++) dma_b(q, KT > 1 ? 1 : 0, kBStageSw);
     // tile 0 has landed (the kAq + 8 copies of tile 1 may still be in flight; the first
     // tile_barrier() covers them)
     if (kAq == 8) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -314,19 +315,83 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         }
     }
 
+    // The accumulators as the matrix instructions below see them: initialised, and the writes of
+    // the initial zeros a few wait states back.
+    auto touch_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < kI16; i++)
+#pragma unroll
+            for (int j = 0; j < kJ16; j++) asm volatile("" : "+a"(acc[i][j]));
+    };
+    touch_acc();
+    asm volatile("s_nop 7" ::: "memory");
+
+    // Scalars carried from one K step to the next: the tile the copies of this step fetch
+    // (kt2 = min(kt + 2, KT - 1)), its source addresses, and the three B stages' byte offsets
+    // (tile kt, tile kt + 1, the stage being filled).  They are advanced at the end of a step, in
+    // issue slots nothing else uses, instead of being recomputed from kt at the top of the next.
+    struct Carried {
+        int kt2;
+        const char* a_src;  // A tile kt2 (row 0 of the workgroup tile)
+        const char* b_src;  // B tile kt2: k-row 0 of it ([K, N] form) or n-row 0 (B^T form)
+        unsigned sb_cur, sb_nxt, sb_fill;
+    } ls;
+    const unsigned b_step32 = kBT ? (unsigned)(kBK * 2) : (unsigned)kBK * (unsigned)N * 2u;  // bytes from one B tile to the next (N < 2^25)
+    unsigned adv = 0;
+    const size_t b_row2 = (size_t)N * 4;                                // [K, N] form: bytes from one 1 KB chunk (2 k-rows) to the next
+    ls.kt2 = KT > 2 ? 2 : KT - 1;
+    ls.a_src = a_tile + (size_t)ls.kt2 * kBK * 2;
+    ls.b_src = b_tile + (size_t)ls.kt2 * b_step32;
+    ls.sb_cur = 0, ls.sb_nxt = kBStageSw, ls.sb_fill = 2 * kBStageSw;
+
+    // The matrix instruction, written out so that the accumulator stays in place in the
+    // accumulation registers (through the builtin the compiler leaves this shape untied and copies
+    // tiles around) ...
+    auto mfma = [&](f32x4& c, const bf16x8& a, const bf16x8& b) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    };
+    // One direct copy with the LDS address formed in the instruction that writes M0 ...
+    auto dma_at = [&](unsigned lds_base, auto q_c, unsigned voff, const char* sbase) {
+        asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3"
+                     :
+                     : "s"(lds_base), "n"(decltype(q_c)::value * 1024), "v"(voff), "s"(sbase)
+                     : "m0", "scc");
+    };
+    // ... and the matrix instruction with one such copy behind it in one statement (the LDS address is formed
+    // in the instruction that writes M0), so that nothing else lands between them.
+    auto mfma_dma = [&](f32x4& c, const bf16x8& a, const bf16x8& b, unsigned lds_base, auto q_c, unsigned voff, const char* sbase) {
+        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\ts_add_u32 m0, %3, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %5, %6"
+                     : "+a"(c)
+                     : "v"(a), "v"(b), "s"(lds_base), "n"(decltype(q_c)::value * 1024), "v"(voff), "s"(sbase)
+                     : "m0", "scc");
+    };
+
     // One phase = half of a 32-deep sub-step: phase p covers sub-step p / 2 (fragment slot p / 2)
     // and tile rows 4 * (p % 2) .. +3 against every tile column, 4 * kJ16 MFMAs, with the other
     // pipes' work slotted between them: the LDS reads of the other slot's fragments (the next
     // sub-step; from sAn / sBn) for the same four tile rows and half of the tile columns, and
-    // chunk copies of tile kt2: phases 0-1 four of its B chunks each into B stage st2, phases 2-3
-    // (after the barrier) kAq / 2 of its A chunks each into A stage `cur`.  The columns loaded
-    // during the second phase of a sub-step are the ones the next sub-step multiplies last.
-    auto phase = [&](auto p_c, auto cur_c, int kt2, int st2, const char* sAn, const char* sBn) {
+    // chunk copies of tile kt2: phases 0-1 four of its B chunks each into the B stage being
+    // filled, phases 2-3 (after the barrier) kAq / 2 of its A chunks each into A stage `cur`.
+    // The columns loaded during the second phase of a sub-step are the ones the next sub-step
+    // multiplies last.  A wave issues one instruction every four cycles and an MFMA of this shape
+    // occupies the pipe for sixteen, so at most three other instructions fit behind an MFMA
+    // without delaying the next one: the reads take the first slots of a phase one by one, every
+    // copy (M0, the wait state, the load) a later slot of its own, its source address the slot
+    // before, and the carried scalars the tail of the last phase.
+    auto phase = [&](auto p_c, auto cur_c, const char* sAn, const char* sBn) {
         constexpr int p = decltype(p_c)::value, cur = decltype(cur_c)::value;
         constexpr int slot = p >> 1, nslot = slot ^ 1, h = p & 1;
         constexpr int kHalfJ = kJ16 / 2;  // tile columns per half
         bf16x4 lo[kHalfJ], hi[kHalfJ];
-        constexpr int kBEvery = kSlots / 4, kAEvery = kSlots / (kAq / 2);  // slots between two copies
+        constexpr int kCopies = p < 2 ? 4 : kAq / 2;                 // copies of this phase
+        constexpr int kFirst = 4 + kJ16;                             // first slot without a fragment read
+        constexpr int kTail = p == 3 ? 3 : p == 2 ? 1 : 0;           // last slots, kept for the carried scalars
+        constexpr int kEvery = (kSlots - kFirst - kTail) / kCopies;  // slots per copy (address, then copy)
+        static_assert(kEvery >= 2, "a copy needs two slots");
+        const unsigned lds_dst = p < 2 ? lds_b + ls.sb_fill : lds_a + cur * kAStageT;
+        const bool ragged_now = kRaggedK && has_last && ls.kt2 == KT - 1;  // this step copies the partial last tile
+        const char* src = p < 2 ? ls.b_src : ls.a_src;
+        if (p == 1 && !kBT) src += 4 * b_row2;
 #pragma unroll
         for (int n = 0; n < kSlots; n++) {
             // first the columns whose fragments arrived a sub-step ago, then the other half; back
@@ -336,9 +401,42 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
             const int jh = n / (kSlots / 2), r = n % (kSlots / 2), rr = r / kHalfJ, jj = r % kHalfJ;
             const int mi = 4 * h + (jh ? 3 - rr : rr);
             const int mj = jh * kHalfJ + ((rr & 1) ? kHalfJ - 1 - jj : jj);
-            // (written out so that the accumulator stays in place in the accumulation registers:
-            // through the builtin the compiler leaves this shape untied and copies tiles around)
-            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[mi][mj]) : "v"(fb[slot][mj]), "v"(fa[slot][mi]));
+            const bool copy_range = n >= kFirst && (n - kFirst) / kEvery < kCopies;
+            const int c = copy_range ? (n - kFirst) / kEvery : 0, part = copy_range ? (n - kFirst) % kEvery : -1;
+            const int q = (p & 1) * kCopies + c;  // chunk of the tile
+            // a copy slot: the MFMA and the copy as one statement; where a step may have to copy
+            // the partial last tile instead (kRaggedK) the choice is made at run time, and the MFMA
+            // stays outside that branch: an accumulator that flows through a branch would be moved
+            // by the compiler, which does not know that it has to wait for the matrix pipe first
+            auto with_q = [&](auto&& f) {
+                switch (q) {  // q is a constant of the unrolled loop
+                    case 0: f(std::integral_constant<int, 0>{}); break;
+                    case 1: f(std::integral_constant<int, 1>{}); break;
+                    case 2: f(std::integral_constant<int, 2>{}); break;
+                    case 3: f(std::integral_constant<int, 3>{}); break;
+                    case 4: f(std::integral_constant<int, 4>{}); break;
+                    case 5: f(std::integral_constant<int, 5>{}); break;
+                    case 6: f(std::integral_constant<int, 6>{}); break;
+                    default: f(std::integral_constant<int, 7>{}); break;
+                }
+            };
+            auto voff_of = [&](auto q_c) {
+                constexpr int qq = decltype(q_c)::value;
+                return p >= 2 ? a_voff[qq < kAq ? qq : 0] : kBT ? bt_voff[kBT ? qq : 0] : b_voff[qq & 1];
+            };
+            if (part == 1 && !kRaggedK) {
+                with_q([&](auto q_c) { mfma_dma(acc[mi][mj], fb[slot][mj], fa[slot][mi], lds_dst, q_c, voff_of(q_c), src); });
+            } else {
+                mfma(acc[mi][mj], fb[slot][mj], fa[slot][mi]);
+                if (part == 1) {
+                    if (ragged_now) {
+                        if (p < 2) dma_b(q, ls.kt2, ls.sb_fill);
+                        else dma_a(q, ls.kt2, cur * kAStageT);
+                    } else {
+                        with_q([&](auto q_c) { dma_at(lds_dst, q_c, voff_of(q_c), src); });
+                    }
+                }
+            }
             if (n < 4) fa[nslot][4 * h + n] = *LDS_PTR(bf16x8, sAn + (4 * h + n) * 2048);
             else if constexpr (kBT) {
                 if (n < 4 + kHalfJ) fb[nslot][h * kHalfJ + n - 4] = *LDS_PTR(bf16x8, sBn + (h * kHalfJ + n - 4) * 2048);
@@ -348,10 +446,33 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
                 if ((n & 1) == 0) lo[jl] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off));
                 else hi[jl] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(LDS_PTR(bf16x4, sBn + off + 4 * 512));
             }
-            if (p < 2) {
-                if (n % kBEvery == 1 % kBEvery) dma_b((p & 1) * 4 + n / kBEvery, kt2, st2);
-            } else {
-                if (n % kAEvery == 1) dma_a((p & 1) * (kAq / 2) + n / kAEvery, kt2, cur);
+            if (part == 0) {
+                // the chunk's source address, one slot ahead of the copy
+                if (p < 2 && !kBT && c > 0) src += b_row2;
+                asm volatile("" : "+s"(src));
+            }
+            // the scalars of the next K step, in the slots left over at the end
+            if (p == 2 && n == kSlots - 1) {
+                // (the copies of this step into the stage being filled went out in phases 0-1)
+                const unsigned t = ls.sb_cur;
+                ls.sb_cur = ls.sb_nxt;
+                ls.sb_nxt = ls.sb_fill;
+                ls.sb_fill = t;
+            }
+            if (p == 3 && n == kSlots - 3) {
+                // 1 while the copies have not reached the last tile (as a minimum: a comparison's
+                // result would take a detour through the vector unit to become a number)
+                adv = (unsigned)__builtin_elementwise_min(KT - 1 - ls.kt2, 1);
+                ls.kt2 += (int)adv;
+                asm volatile("" : "+s"(adv));
+            }
+            if (p == 3 && n == kSlots - 2) {
+                ls.a_src += adv * (unsigned)(kBK * 2);
+                asm volatile("" : "+s"(ls.a_src));
+            }
+            if (p == 3 && n == kSlots - 1) {
+                ls.b_src += adv * b_step32;  // (32-bit product: a tile-to-tile step stays below 4 GiB)
+                asm volatile("" : "+s"(ls.b_src));
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -366,39 +487,37 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     using C1 = std::integral_constant<int, 1>;
     using C2 = std::integral_constant<int, 2>;
     using C3 = std::integral_constant<int, 3>;
-    // tile kt: A in stage cur = kt & 1, B in stage st = kt % 3 (next tile's B in stn, the one after goes to st2)
-    auto iteration = [&](auto cur_c, int kt, int st, int stn, int st2) {
+    // tile kt: A in stage cur = kt & 1, B in the stage at ls.sb_cur (next tile's B at ls.sb_nxt, the one after goes to ls.sb_fill)
+    auto iteration = [&](auto cur_c) {
         constexpr int cur = decltype(cur_c)::value;
         using C = std::integral_constant<int, cur>;
-        const int kt2 = kt + 2 < KT ? kt + 2 : KT - 1;
         const char* sAc = sA0 + cur * kAStageT + a_base_l;
-        const char* sBc = sB0 + st * kBStageSw + (kBT ? bt_base_l : 0);
+        const char* sBc = sB0 + ls.sb_cur + (kBT ? bt_base_l : 0);
         const char* sAx = sA0 + (cur ^ 1) * kAStageT + a_base_l;
-        const char* sBx = sB0 + stn * kBStageSw + (kBT ? bt_base_l : 0);
+        const char* sBx = sB0 + ls.sb_nxt + (kBT ? bt_base_l : 0);
         // sub-step ks of a B stage: 32 k-rows of 512 B further, or (kBT) the same chunk offset as A's
         auto b_ks = [&](int ks) { return kBT ? a_xo[ks] : ks * 32 * 512; };
-        phase(C0{}, C{}, kt2, st2, sAc + a_xo[1], sBc + b_ks(1));
-        phase(C1{}, C{}, kt2, st2, sAc + a_xo[1], sBc + b_ks(1));
+        phase(C0{}, C{}, sAc + a_xo[1], sBc + b_ks(1));
+        phase(C1{}, C{}, sAc + a_xo[1], sBc + b_ks(1));
         // tile kt+1 has landed; nobody reads A stage cur any more
         tile_barrier();
-        phase(C2{}, C{}, kt2, st2, sAx + a_xo[0], sBx + b_ks(0));
-        phase(C3{}, C{}, kt2, st2, sAx + a_xo[0], sBx + b_ks(0));
+        phase(C2{}, C{}, sAx + a_xo[0], sBx + b_ks(0));
+        phase(C3{}, C{}, sAx + a_xo[0], sBx + b_ks(0));
     };
     {
-        int kt = 0, st = 0;
-        auto nx = [](int s) { return s == 2 ? 0 : s + 1; };
+        int kt = 0;
         for (; kt + 1 < KT; kt += 2) {
-            iteration(C0{}, kt, st, nx(st), nx(nx(st)));
-            st = nx(st);
-            iteration(C1{}, kt + 1, st, nx(st), nx(nx(st)));
-            st = nx(st);
+            iteration(C0{});
+            iteration(C1{});
         }
-        if (kt < KT) iteration(C0{}, kt, st, nx(st), nx(nx(st)));
+        if (kt < KT) iteration(C0{});
     }
     full_barrier();
-    // the last MFMAs' results must have left the matrix pipe before the vector ALUs read them
-    // (the compiler does not see the instructions above as matrix operations)
+    // the last MFMAs' results must have left the matrix pipe before the vector ALUs read them (the
+    // compiler does not see the instructions above as matrix operations); the empty statements
+    // behind the wait keep every later use of an accumulator behind it
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    touch_acc();
 
     // Epilogue.  With swapped operands lane l of tile (i, j) holds, in its four registers,
     // C[m = i*16 + l%16][n = j*16 + 4*(l/16) + 0..3].
@@ -445,8 +564,14 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
             const int ml = i * 16 + (lane & 15);
             const int nl = j * 16 + 4 * (lane >> 4);
             *LDS_PTR(bf16x4, sC + ml * kCPitchT + nl * 2) = h;
+            // (tile by tile: moved out of the accumulation registers all at once, the tile would
+            // not fit the vector registers next to the residual rows)
+            if (kResidual && (j & 1)) __builtin_amdgcn_sched_barrier(0);
         }
-    if constexpr (kResidual) fetch_residual(kFirstBatch, kIts);
+    if constexpr (kResidual) {
+        asm volatile("" ::: "memory");  // not before the accumulators have left their registers
+        fetch_residual(kFirstBatch, kIts);
+    }
     // a wave reads back only what it staged itself (the LDS serves a wave's requests in order),
     // except for the gated epilogue, where gate and up blocks come from two waves
     if constexpr (kSwiGLU) __syncthreads();
@@ -692,7 +817,7 @@ int launch_gemm_bf16_static_ws(void* stream, int device_id, const void* A, const
 
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch) {
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || batch > 65535) return false;
-    if (M > 0x7fffffffL || N > 0x7fffffffL || N % 8 || K % 8 || K > (1L << 23) || N > (1L << 25)) return false;
+    if (M > 0x7fffffffL || N > 0x7fffffffL || N % 8 || K % 8 || K > (1L << 23) || N >= (1L << 25)) return false;
     if (plan_split_k(M, N, K, batch).splits > 1) return false;  // split-K sums partials in another kernel
     const long tn = (N + mrk::dev::kBN - 1) / mrk::dev::kBN, tm128 = (M + 127) / 128;
     return tm128 * tn <= 0x7fffffffL;
@@ -724,7 +849,7 @@ int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const 
 
 bool gemm_bf16_swiglu_supported(long M, long F, long K) {
     if (M <= 0 || F <= 0 || K <= 0) return false;
-    if (M > 0x7fffffffL || F % 8 || K % 8 || K > (1L << 23) || 2 * F > (1L << 25)) return false;
+    if (M > 0x7fffffffL || F % 8 || K % 8 || K > (1L << 23) || 2 * F >= (1L << 25)) return false;
     const long tn = (F + 127) / 128, tm = (M + mrk::dev::kBM - 1) / mrk::dev::kBM;
     return tm * tn <= 0x7fffffffL;
 }
@@ -757,7 +882,7 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     const bool aligned = ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) % 16) == 0;
     // the tiled kernel addresses a tile's rows with 32-bit byte offsets from the tile origin:
     // 255 rows of A (K elements each) and 49 rows of B (N elements each) must stay below 4 GiB
-    const bool offsets_fit = K <= (1L << 23) && N <= (1L << 25);
+    const bool offsets_fit = K <= (1L << 23) && N < (1L << 25);
     if (variant == 6) {  // B given as Bt[N, K]
         if (!aligned || !offsets_fit || K <= 0 || K % kBK || N % 8) return (int)hipErrorInvalidValue;
         const long tn = (N + kBN - 1) / kBN, tm = (M + kBM - 1) / kBM;

@@ -65,8 +65,13 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ o
                     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fb[ks][j]), "v"(fa[ks][i]));
                 }
     }
-    // the last results must have left the matrix pipe before the vector ALUs read them
+    // the last results must have left the matrix pipe before the vector ALUs read them (the
+    // empty statements keep the reads behind the wait)
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+    for (int i = 0; i < 8; i++)
+#pragma unroll
+        for (int j = 0; j < 8; j++) asm volatile("" : "+a"(acc[i][j]));
     float s = 0.0f;
 #pragma unroll
     for (int i = 0; i < 8; i++)
