@@ -199,6 +199,10 @@ void mrk_hip_program_destroy(mrk_program* p);
  *                     (split-K for shapes with few output tiles; size from mrk_hip_gemm_bf16_workspace_bytes)
  *   "gemm_bf16_residual"  params = {M, N, K} or {M, N, K, batch}  buffers = {c, a, b, r}   (c = a b + r)
  *   "gemm_bf16_swiglu"    params = {M, F, K}                      buffers = {c, a, w}      (w = gate | up, [K, 2F])
+ *   "gemm_bf16_nt", "gemm_bf16_nt_residual", "gemm_bf16_nt_swiglu": the same three with the second operand
+ *                     stored transposed, [N, K] ([2F, K], gate rows first), as a Linear layer holds its
+ *                     weight (tensor/src/nn/linear.rs:9-14: y = x @ weight.T + bias); the same bits as
+ *                     the [K, N] kinds.  No split-K form: shapes with a workspace size > 0 are refused.
  *   "flash_fwd_bf16"  params = {B*H, Sq, Sk, D, causal, f32 bits of scale}   buffers = {o, q, k, v}
  *   "flash_fwd_bf16_strided"  params = {B, H, Sq, Sk, D, causal, f32 bits of scale, element offsets
  *                     of q k v o into their buffers (4), (batch, head, row) element strides of
@@ -431,6 +435,13 @@ int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int6
  * enough tiles by itself.  mrk_hip_gemm_bf16 takes that scratch from the device allocator by
  * itself; a "gemm_bf16" builtin Program takes it as its fourth buffer. */
 size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t batch);
+/* c[M,N] = a[M,K] * bt[N,K]^T: the product with the second operand as it is stored by a Linear
+ * layer (weight [out_features, in_features], tensor/src/nn/linear.rs:9-14, 39-41), read in place
+ * instead of through a transposed copy.  Same products in the same order as mrk_hip_gemm_bf16 on
+ * the transposed matrix, so the same bits.  N and K multiples of 8, 16-byte aligned operands, and
+ * enough output tiles that the split-K form would not be chosen (mrk_hip_gemm_bf16_workspace_bytes
+ * == 0); INVALID_ARGUMENT otherwise.  Builtin Program kind "gemm_bf16_nt". */
+int mrk_hip_gemm_bf16_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k);
 /* Same with an explicit kernel variant (0 choose by shape, 2 any-shape kernel, 3 / 4 tiled kernel
  * with the 256-row / 128-row tile); tuning/tests. */
 int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,

@@ -131,28 +131,45 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
-    if (k == "gemm_bf16_residual") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, b, r}
+    // the "_nt" kinds take the second operand as B^T [N, K] (a Linear layer's weight as it is stored)
+    if (k == "gemm_bf16_nt") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, bt}
         if (nparams < 3 || nparams > 4)
-            return failf(kInvalidArgument, "builtin 'gemm_bf16_residual' takes 3 or 4 parameters, got %zu", nparams);
+            return failf(kInvalidArgument, "builtin 'gemm_bf16_nt' takes 3 or 4 parameters, got %zu", nparams);
         while (p.size() < 4) p.push_back(1);
-        if (!gemm_bf16_residual_supported(p[0], p[1], p[2], p[3]))
-            return fail(kInvalidArgument, "gemm_bf16_residual: shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel)");
-        std::string name = "gemm_bf16_residual_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+        if (!gemm_bf16_nt_supported(p[0], p[1], p[2], p[3]))
+            return fail(kInvalidArgument, "gemm_bf16_nt: shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel)");
+        std::string name = "gemm_bf16_nt_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
         if (p[3] > 1) name += "_x" + std::to_string(p[3]);
-        out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
+        out->reset(new BuiltinProgram(device_id, stream, name, 3, p,
                                       [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
-                                          return launch_gemm_bf16_residual(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3]);
+                                          return launch_gemm_bf16(s, b[1], b[2], b[0], q[0], q[1], q[2], 0, q[3], nullptr, 0, true);
                                       }));
         return kOk;
     }
-    if (k == "gemm_bf16_swiglu") {  // {M, F, K}; buffers {c [M, F], a [M, K], w [K, 2F] = gate | up}
+    if (k == "gemm_bf16_residual" || k == "gemm_bf16_nt_residual") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, b, r}
+        const bool nt = k == "gemm_bf16_nt_residual";
+        if (nparams < 3 || nparams > 4)
+            return failf(kInvalidArgument, "builtin '%s' takes 3 or 4 parameters, got %zu", k.c_str(), nparams);
+        while (p.size() < 4) p.push_back(1);
+        if (!gemm_bf16_residual_supported(p[0], p[1], p[2], p[3]))
+            return failf(kInvalidArgument, "%s: shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel)", k.c_str());
+        std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+        if (p[3] > 1) name += "_x" + std::to_string(p[3]);
+        out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
+                                      [nt](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16_residual(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3], nt);
+                                      }));
+        return kOk;
+    }
+    if (k == "gemm_bf16_swiglu" || k == "gemm_bf16_nt_swiglu") {  // {M, F, K}; buffers {c [M, F], a [M, K], w [K, 2F] = gate | up ([2F, K]: _nt)}
+        const bool nt = k == "gemm_bf16_nt_swiglu";
         MRK_TRY(need(3));
-        if (!gemm_bf16_swiglu_supported(p[0], p[1], p[2]))
-            return fail(kInvalidArgument, "gemm_bf16_swiglu: shape not covered (M, F, K > 0; F and K multiples of 8)");
-        std::string name = "gemm_bf16_swiglu_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+        if (!gemm_bf16_swiglu_supported(p[0], p[1], p[2], nt))
+            return failf(kInvalidArgument, "%s: shape not covered (M, F, K > 0; F and K multiples of 8)", k.c_str());
+        std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
         out->reset(new BuiltinProgram(device_id, stream, name, 3, p,
-                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
-                                          return launch_gemm_bf16_swiglu(s, b[1], b[2], b[0], q[0], q[1], q[2]);
+                                      [nt](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16_swiglu(s, b[1], b[2], b[0], q[0], q[1], q[2], nt);
                                       }));
         return kOk;
     }

@@ -876,6 +876,22 @@ int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int6
     return mrk_hip_gemm_bf16_variant(device_id, a, b, c, m, n, k, 0);
 }
 
+int mrk_hip_gemm_bf16_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k) {
+    if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_nt: negative shape");
+    if (m == 0 || n == 0) return kOk;
+    MRK_NONNULL(a);
+    MRK_NONNULL(bt);
+    MRK_NONNULL(c);
+    if (!gemm_bf16_nt_supported(m, n, k, 1))
+        return fail(kInvalidArgument, "gemm_bf16_nt: shape not covered for a second operand stored [N, K] (N and K multiples of 8, "
+                                      "K > 0, enough output tiles that split-K is not used); transpose it and run mrk_hip_gemm_bf16");
+    std::shared_ptr<Device> dv;
+    MRK_TRY(get_device(device_id, &dv));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_gemm_bf16(dv->allocator->stream(), a, bt, c, m, n, k, 0, 1, nullptr, 0, true), "gemm_bf16_nt launch");
+    return kOk;
+}
+
 int mrk_hip_gemm_bf16_swiglu(int device_id, const void* a, const void* w, void* c, int64_t m, int64_t f, int64_t k) {
     if (m < 0 || f < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_swiglu: negative shape");
     if (m == 0 || f == 0) return kOk;

@@ -629,12 +629,30 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
     gemm_tile_body<false, 4>(A, B, C, M, N, K, tiles_m, tiles_n);
 }
 // B^T variants: the second operand is Bt[N, K] row-major (k contiguous, the layout of a Linear
-// layer's weight), C = A Bt^T.
-__global__ __launch_bounds__(256) void gemm_bf16_nt_tile256(const __bf16* __restrict__ A, const __bf16* __restrict__ Bt,
-                                                            __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
-                                                            int tiles_n) {
-    gemm_tile_body<false, 4, false, false, false, true>(A, Bt, C, M, N, K, tiles_m, tiles_n);
-}
+// layer's weight), C = A Bt^T; for the gated epilogue Bt is [2F, K], gate rows first.
+#define MRK_GEMM_NT_KERNEL(name, ...)                                                                                      \
+    __global__ __launch_bounds__(256) void name(const __bf16* __restrict__ A, const __bf16* __restrict__ Bt,              \
+                                                __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n) { \
+        gemm_tile_body<__VA_ARGS__>(A, Bt, C, M, N, K, tiles_m, tiles_n);                                                  \
+    }
+#define MRK_GEMM_NT_RESIDUAL_KERNEL(name, ...)                                                                          \
+    __global__ __launch_bounds__(256) void name(const __bf16* __restrict__ A, const __bf16* __restrict__ Bt,           \
+                                                const __bf16* __restrict__ R, __bf16* __restrict__ C, int M, int N,    \
+                                                int K, int tiles_m, int tiles_n) {                                     \
+        gemm_tile_body<__VA_ARGS__>(A, Bt, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);                                \
+    }
+MRK_GEMM_NT_KERNEL(gemm_bf16_nt_tile256, false, 4, false, false, false, true)
+MRK_GEMM_NT_KERNEL(gemm_bf16_nt_tile256_ragged_k, true, 4, false, false, false, true)
+MRK_GEMM_NT_KERNEL(gemm_bf16_nt_tile128, false, 2, false, false, false, true)
+MRK_GEMM_NT_KERNEL(gemm_bf16_nt_tile128_ragged_k, true, 2, false, false, false, true)
+MRK_GEMM_NT_KERNEL(gemm_bf16_nt_tile256_swiglu, false, 4, false, false, true, true)
+MRK_GEMM_NT_KERNEL(gemm_bf16_nt_tile256_swiglu_ragged_k, true, 4, false, false, true, true)
+MRK_GEMM_NT_RESIDUAL_KERNEL(gemm_bf16_nt_tile256_residual, false, 4, false, true, false, true)
+MRK_GEMM_NT_RESIDUAL_KERNEL(gemm_bf16_nt_tile256_residual_ragged_k, true, 4, false, true, false, true)
+MRK_GEMM_NT_RESIDUAL_KERNEL(gemm_bf16_nt_tile128_residual, false, 2, false, true, false, true)
+MRK_GEMM_NT_RESIDUAL_KERNEL(gemm_bf16_nt_tile128_residual_ragged_k, true, 2, false, true, false, true)
+#undef MRK_GEMM_NT_KERNEL
+#undef MRK_GEMM_NT_RESIDUAL_KERNEL
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_ragged_k(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ B, __bf16* __restrict__ C,
                                                                   int M, int N, int K, int tiles_m, int tiles_n) {
@@ -823,7 +841,13 @@ bool gemm_bf16_residual_supported(long M, long N, long K, long batch) {
     return tm128 * tn <= 0x7fffffffL;
 }
 
-int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch) {
+bool gemm_bf16_nt_supported(long M, long N, long K, long batch) {
+    // the tiled kernels only (no split-K, no any-shape kernel for this operand layout)
+    return gemm_bf16_residual_supported(M, N, K, batch);
+}
+
+int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch,
+                              bool b_transposed) {
     using namespace mrk::dev;
     if (M <= 0 || N <= 0 || batch <= 0) return 0;
     if (!gemm_bf16_residual_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
@@ -840,24 +864,27 @@ int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const 
     const __bf16* r = static_cast<const __bf16*>(R);
     __bf16* c = static_cast<__bf16*>(C);
     const bool ragged_k = K % kBK != 0;
-    if (small && !ragged_k) gemm_bf16_tile128_residual<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
-    else if (small) gemm_bf16_tile128_residual_ragged_k<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
-    else if (!ragged_k) gemm_bf16_tile256_residual<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
-    else gemm_bf16_tile256_residual_ragged_k<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+    auto kernel = b_transposed ? (small ? (ragged_k ? gemm_bf16_nt_tile128_residual_ragged_k : gemm_bf16_nt_tile128_residual)
+                                        : (ragged_k ? gemm_bf16_nt_tile256_residual_ragged_k : gemm_bf16_nt_tile256_residual))
+                               : (small ? (ragged_k ? gemm_bf16_tile128_residual_ragged_k : gemm_bf16_tile128_residual)
+                                        : (ragged_k ? gemm_bf16_tile256_residual_ragged_k : gemm_bf16_tile256_residual));
+    kernel<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
     return (int)hipGetLastError();
 }
 
-bool gemm_bf16_swiglu_supported(long M, long F, long K) {
+bool gemm_bf16_swiglu_supported(long M, long F, long K, bool b_transposed) {
     if (M <= 0 || F <= 0 || K <= 0) return false;
+    // [2F, K] form: the up rows are addressed F rows behind the gate rows with 32-bit byte offsets
+    if (b_transposed && (F + 256) * K * 2 >= (1L << 32)) return false;
     if (M > 0x7fffffffL || F % 8 || K % 8 || K > (1L << 23) || 2 * F >= (1L << 25)) return false;
     const long tn = (F + 127) / 128, tm = (M + mrk::dev::kBM - 1) / mrk::dev::kBM;
     return tm * tn <= 0x7fffffffL;
 }
 
-int launch_gemm_bf16_swiglu(void* stream, const void* A, const void* B, void* C, long M, long F, long K) {
+int launch_gemm_bf16_swiglu(void* stream, const void* A, const void* B, void* C, long M, long F, long K, bool b_transposed) {
     using namespace mrk::dev;
     if (M <= 0 || F <= 0) return 0;
-    if (!gemm_bf16_swiglu_supported(M, F, K)) return (int)hipErrorInvalidValue;
+    if (!gemm_bf16_swiglu_supported(M, F, K, b_transposed)) return (int)hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) % 16) return (int)hipErrorInvalidValue;
     hipStream_t s = static_cast<hipStream_t>(stream);
     (void)hipGetLastError();
@@ -866,13 +893,15 @@ int launch_gemm_bf16_swiglu(void* stream, const void* A, const void* B, void* C,
     const __bf16* a = static_cast<const __bf16*>(A);
     const __bf16* b = static_cast<const __bf16*>(B);
     __bf16* c = static_cast<__bf16*>(C);
-    if (K % kBK == 0) gemm_bf16_tile256_swiglu<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)(2 * F), (int)K, (int)tm, (int)tn);
-    else gemm_bf16_tile256_swiglu_ragged_k<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)(2 * F), (int)K, (int)tm, (int)tn);
+    const bool ragged_k = K % kBK != 0;
+    auto kernel = b_transposed ? (ragged_k ? gemm_bf16_nt_tile256_swiglu_ragged_k : gemm_bf16_nt_tile256_swiglu)
+                               : (ragged_k ? gemm_bf16_tile256_swiglu_ragged_k : gemm_bf16_tile256_swiglu);
+    kernel<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)(2 * F), (int)K, (int)tm, (int)tn);
     return (int)hipGetLastError();
 }
 
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
-                     long batch, void* workspace, size_t workspace_bytes) {
+                     long batch, void* workspace, size_t workspace_bytes, bool b_transposed) {
     using namespace mrk::dev;
     if (M <= 0 || N <= 0 || batch <= 0) return 0;
     if (batch > 65535) return (int)hipErrorInvalidValue;  // grid y extent
@@ -883,11 +912,17 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     // the tiled kernel addresses a tile's rows with 32-bit byte offsets from the tile origin:
     // 255 rows of A (K elements each) and 49 rows of B (N elements each) must stay below 4 GiB
     const bool offsets_fit = K <= (1L << 23) && N < (1L << 25);
-    if (variant == 6) {  // B given as Bt[N, K]
-        if (!aligned || !offsets_fit || K <= 0 || K % kBK || N % 8) return (int)hipErrorInvalidValue;
-        const long tn = (N + kBN - 1) / kBN, tm = (M + kBM - 1) / kBM;
-        gemm_bf16_nt_tile256<<<dim3((unsigned)(tm * tn), (unsigned)batch), 256, 0, s>>>(
-            static_cast<const __bf16*>(A), static_cast<const __bf16*>(B), static_cast<__bf16*>(C), (int)M, (int)N, (int)K, (int)tm, (int)tn);
+    if (b_transposed) {
+        // B given as Bt[N, K]: the tiled kernels, or nothing (variant 3 / 4 force a tile size)
+        if (!aligned || !gemm_bf16_nt_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
+        const long tn = (N + kBN - 1) / kBN, tm128 = (M + 127) / 128;
+        const bool small = variant == 4 || (variant != 3 && tm128 * tn * batch <= 256);
+        const long tm = small ? tm128 : (M + kBM - 1) / kBM;
+        const bool ragged_k = K % kBK != 0;
+        auto kernel = small ? (ragged_k ? gemm_bf16_nt_tile128_ragged_k : gemm_bf16_nt_tile128)
+                            : (ragged_k ? gemm_bf16_nt_tile256_ragged_k : gemm_bf16_nt_tile256);
+        kernel<<<dim3((unsigned)(tm * tn), (unsigned)batch), 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
+                                                                          static_cast<__bf16*>(C), (int)M, (int)N, (int)K, (int)tm, (int)tn);
         return (int)hipGetLastError();
     }
     // any M; N and K in whole 16-byte chunks

@@ -15,18 +15,25 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 // 128-row tile of the tiled kernel (where the shape allows the tiled kernel at all), 5 = as 0.  batch > 1: that many
 // independent products over matrices stored back to back (A [batch,M,K], B [batch,K,N],
 // C [batch,M,N]), one launch.
+// b_transposed: B is stored as B^T [N, K] (k contiguous: the layout of a Linear layer's weight;
+// [batch, N, K] for batch > 1).  Same products in the same order, so the same bits as the [K, N]
+// form.  Tiled kernels only: shapes outside gemm_bf16_nt_supported (N or K not a multiple of 8,
+// so few output tiles that split-K would be used) are refused with hipErrorInvalidValue.
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
-                     long batch = 1, void* workspace = nullptr, size_t workspace_bytes = 0);
+                     long batch = 1, void* workspace = nullptr, size_t workspace_bytes = 0, bool b_transposed = false);
+bool gemm_bf16_nt_supported(long M, long N, long K, long batch);
 // c = bf16(float(bf16(a b)) + float(r)) with r of c's shape, added in the product kernel's epilogue
 // (same bits as the product followed by an elementwise add).  Supported for the shapes the tiled
 // kernels take without split-K; gemm_bf16_residual_supported tells.
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch);
-int launch_gemm_bf16_residual(void* stream, const void* a, const void* b, const void* r, void* c, long M, long N, long K, long batch);
+int launch_gemm_bf16_residual(void* stream, const void* a, const void* b, const void* r, void* c, long M, long N, long K, long batch,
+                              bool b_transposed = false);
 // C[M, F] = bf16(silu(float(bf16(A Wg))) * float(bf16(A Wu))) for W = [Wg | Wu] stored side by side as
 // one [K, 2F] matrix: the gated-MLP pair of products with the gate applied in the product kernel's
 // epilogue, so that the [M, 2F] product never reaches memory.  F and K multiples of 8.
-bool gemm_bf16_swiglu_supported(long M, long F, long K);
-int launch_gemm_bf16_swiglu(void* stream, const void* a, const void* w, void* c, long M, long F, long K);
+// b_transposed: W is stored as [2F, K] (the rows of Wg^T, then the rows of Wu^T).
+bool gemm_bf16_swiglu_supported(long M, long F, long K, bool b_transposed = false);
+int launch_gemm_bf16_swiglu(void* stream, const void* a, const void* w, void* c, long M, long F, long K, bool b_transposed = false);
 // Bytes of f32 scratch with which launch_gemm_bf16 spreads the K loop of this shape over the
 // chip (split-K: partial products per K range, added up in a fixed order by a second kernel);
 // 0 when the shape has enough output tiles by itself.  Without the workspace the same shape

@@ -1381,12 +1381,47 @@ struct Scheduler {
         }
         return nullptr;
     }
+    // The second operand of a bf16 product given as the transpose of data that is in memory anyway
+    // (x @ w.T with w [N, K]: how a Linear layer multiplies, tensor/src/nn/linear.rs:39-41): the
+    // [N, K] node, which the "_nt" product kernels read in place; nullptr otherwise.
+    TensorNode* transposed_weight(const TensorNode* mm) const {
+        if (!g_fusion) return nullptr;
+        TensorNode* w = mm->hint_inputs[1].get();
+        if (w->buffer || w->kind != TKind::Permute || w->dtype != Scalar::BFloat16 || w->shape.size() != 2 || w->arg.size() != 2 ||
+            w->arg[0] != 1 || w->arg[1] != 0)
+            return nullptr;
+        TensorNode* wt = w->src[0].get();
+        const TensorNode* rb = wt;
+        while (!rb->buffer && rb->kind == TKind::Reshape) rb = rb->src[0].get();
+        return rb->buffer || is_boundary_kind(rb) || fusable(rb) ? wt : nullptr;
+    }
+    // Materialises a product's second operand and tells the layout the kernel will read it in:
+    // [K, N], or (where nt_ok says the shape has a kernel for it) the [N, K] data behind a transpose.
+    int weight_operand(TensorNode* mm, bool nt_ok, std::shared_ptr<Buffer>* buf, bool* nt) {
+        *nt = false;
+        TensorNode* wt = nt_ok ? transposed_weight(mm) : nullptr;
+        if (wt) {
+            MRK_TRY(materialize(wt));
+            if (wt->buffer->offset() % 16 == 0) {
+                *buf = wt->buffer;
+                *nt = true;
+                return kOk;
+            }
+        }
+        TensorNode* w = mm->hint_inputs[1].get();
+        MRK_TRY(materialize(w));
+        *buf = w->buffer;
+        return kOk;
+    }
     int materialize_swiglu_matmul(TensorNode* n, TensorNode* mm) {
-        for (const TensorRef& in : mm->hint_inputs) MRK_TRY(materialize(in.get()));
         int64_t M, N2, K, batch;
         matmul_extents(mm, &M, &N2, &K, &batch);
+        MRK_TRY(materialize(mm->hint_inputs[0].get()));
+        std::shared_ptr<Buffer> wbuf;
+        bool nt = false;
+        MRK_TRY(weight_operand(mm, gemm_bf16_swiglu_supported(M, N2 / 2, K, true), &wbuf, &nt));
         auto out = new_buffer(n);
-        MRK_TRY(builtin("gemm_bf16_swiglu", {M, N2 / 2, K}, {out, mm->hint_inputs[0]->buffer, mm->hint_inputs[1]->buffer}));
+        MRK_TRY(builtin(nt ? "gemm_bf16_nt_swiglu" : "gemm_bf16_swiglu", {M, N2 / 2, K}, {out, mm->hint_inputs[0]->buffer, wbuf}));
         n->buffer = out;
         produced.push_back(n);
         return kOk;
@@ -1400,13 +1435,16 @@ struct Scheduler {
         for (size_t i = 0; i + 2 < a->shape.size(); i++) (w->shape.size() == 2 ? *M : *batch) *= a->shape[i];
     }
     int materialize_residual_matmul(TensorNode* n, TensorNode* mm, TensorNode* r) {
-        for (const TensorRef& in : mm->hint_inputs) MRK_TRY(materialize(in.get()));
-        MRK_TRY(materialize(r));
         int64_t M, N, K, batch;
         matmul_extents(mm, &M, &N, &K, &batch);
+        MRK_TRY(materialize(mm->hint_inputs[0].get()));
+        std::shared_ptr<Buffer> wbuf;
+        bool nt = false;
+        MRK_TRY(weight_operand(mm, true, &wbuf, &nt));  // (the residual epilogue exists for exactly the shapes the B^T kernels take)
+        MRK_TRY(materialize(r));
         auto out = new_buffer(n);
         const std::vector<int64_t> params = batch == 1 ? std::vector<int64_t>{M, N, K} : std::vector<int64_t>{M, N, K, batch};
-        MRK_TRY(builtin("gemm_bf16_residual", params, {out, mm->hint_inputs[0]->buffer, mm->hint_inputs[1]->buffer, r->buffer}));
+        MRK_TRY(builtin(nt ? "gemm_bf16_nt_residual" : "gemm_bf16_residual", params, {out, mm->hint_inputs[0]->buffer, wbuf, r->buffer}));
         n->buffer = out;
         produced.push_back(n);
         return kOk;
@@ -1809,7 +1847,16 @@ struct Scheduler {
 
     int materialize_fused(TensorNode* n) {
         if (n->hint == HintKind::Sdpa) return materialize_attention(n, n, dense_strides(n->shape));
-        for (const TensorRef& in : n->hint_inputs) MRK_TRY(materialize(in.get()));
+        std::shared_ptr<Buffer> wbuf;  // a bf16 product's second operand, and its layout
+        bool nt = false;
+        if (n->hint == HintKind::Matmul && n->hint_inputs[0]->dtype == Scalar::BFloat16) {
+            int64_t M, N, K, batch;
+            matmul_extents(n, &M, &N, &K, &batch);
+            MRK_TRY(materialize(n->hint_inputs[0].get()));
+            MRK_TRY(weight_operand(n, gemm_bf16_workspace_bytes(M, N, K, batch) == 0 && gemm_bf16_nt_supported(M, N, K, batch), &wbuf, &nt));
+        } else {
+            for (const TensorRef& in : n->hint_inputs) MRK_TRY(materialize(in.get()));
+        }
         auto out = new_buffer(n);
         int rc = kOk;
         if (n->hint == HintKind::Softmax) {
@@ -1824,12 +1871,14 @@ struct Scheduler {
                 // few output tiles against a long K: scratch for split-K partials, an intermediate
                 // of the plan like any other (lazily allocated, placed by the memory planner)
                 const size_t ws = gemm_bf16_workspace_bytes(M, N, K, batch);
-                if (ws) {
+                if (nt) {
+                    rc = builtin("gemm_bf16_nt", {M, N, K}, {out, a->buffer, wbuf});
+                } else if (ws) {
                     auto scratch = std::make_shared<Buffer>(dev->allocator, ws, BufferOptions());
-                    rc = builtin("gemm_bf16", {M, N, K, batch, static_cast<int64_t>(ws)}, {out, a->buffer, w->buffer, scratch});
+                    rc = builtin("gemm_bf16", {M, N, K, batch, static_cast<int64_t>(ws)}, {out, a->buffer, wbuf, scratch});
                 } else {
-                    rc = batch == 1 ? builtin("gemm_bf16", {M, N, K}, {out, a->buffer, w->buffer})
-                                    : builtin("gemm_bf16", {M, N, K, batch}, {out, a->buffer, w->buffer});
+                    rc = batch == 1 ? builtin("gemm_bf16", {M, N, K}, {out, a->buffer, wbuf})
+                                    : builtin("gemm_bf16", {M, N, K, batch}, {out, a->buffer, wbuf});
                 }
             } else {
                 // MOROK_BEAM=<width> selects the LOCAL/UPCAST/UNROLL choices by timed search

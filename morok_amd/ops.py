@@ -33,6 +33,16 @@ def gemm_bf16(a, b, c, m, n, k, device_id=0, variant=0):
     check(lib.mrk_hip_gemm_bf16_variant(device_id, _p(a), _p(b), _p(c), m, n, k, variant))
 
 
+def gemm_bf16_nt(a, bt, c, m, n, k, device_id=0):
+    """c[m,n] = a[m,k] @ bt[n,k]^T: the second operand as a Linear layer stores its weight
+    ([out_features, in_features], k contiguous).  The same bits as gemm_bf16 on the transposed
+    matrix; tiled kernels only (n and k multiples of 8, no split-K shapes)."""
+    _need(a, m * k * 2, "gemm_bf16_nt a")
+    _need(bt, n * k * 2, "gemm_bf16_nt bt")
+    _need(c, m * n * 2, "gemm_bf16_nt c")
+    check(lib.mrk_hip_gemm_bf16_nt(device_id, _p(a), _p(bt), _p(c), m, n, k))
+
+
 def gemm_bf16_noalloc(a, b, c, m, n, k, device_id=0):
     """gemm_bf16 without any device allocation: split-K partials go to the library's fixed
     device scratch (for callers under graph capture or in loops that must not allocate)."""

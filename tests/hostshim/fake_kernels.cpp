@@ -10,9 +10,12 @@ int launch_softmax_f32(void* stream, const void*, void*, long, long, int) {
     return 0;
 }
 size_t gemm_bf16_workspace_bytes(long, long, long, long) { return 0; }
-int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, long, int, long, void*, size_t) {
-    mrk_shim_note_launch(stream, "gemm_bf16");
+int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, long, int, long, void*, size_t, bool b_transposed) {
+    mrk_shim_note_launch(stream, b_transposed ? "gemm_bf16_nt" : "gemm_bf16");
     return 0;
+}
+bool gemm_bf16_nt_supported(long M, long N, long K, long batch) {
+    return M > 0 && N > 0 && K > 0 && batch > 0 && N % 8 == 0 && K % 8 == 0;
 }
 int gemm_bf16_static_workspace_init(int) { return 0; }
 size_t gemm_bf16_static_workspace_capacity() { return size_t(32) << 20; }
@@ -23,13 +26,13 @@ int launch_gemm_bf16_static_ws(void* stream, int, const void*, const void*, void
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch) {
     return M > 0 && N > 0 && K > 0 && batch > 0 && N % 8 == 0 && K % 8 == 0;
 }
-int launch_gemm_bf16_residual(void* stream, const void*, const void*, const void*, void*, long, long, long, long) {
-    mrk_shim_note_launch(stream, "gemm_bf16_residual");
+int launch_gemm_bf16_residual(void* stream, const void*, const void*, const void*, void*, long, long, long, long, bool b_transposed) {
+    mrk_shim_note_launch(stream, b_transposed ? "gemm_bf16_nt_residual" : "gemm_bf16_residual");
     return 0;
 }
-bool gemm_bf16_swiglu_supported(long M, long F, long K) { return M > 0 && F > 0 && K > 0 && F % 8 == 0 && K % 8 == 0; }
-int launch_gemm_bf16_swiglu(void* stream, const void*, const void*, void*, long, long, long) {
-    mrk_shim_note_launch(stream, "gemm_bf16_swiglu");
+bool gemm_bf16_swiglu_supported(long M, long F, long K, bool) { return M > 0 && F > 0 && K > 0 && F % 8 == 0 && K % 8 == 0; }
+int launch_gemm_bf16_swiglu(void* stream, const void*, const void*, void*, long, long, long, bool b_transposed) {
+    mrk_shim_note_launch(stream, b_transposed ? "gemm_bf16_nt_swiglu" : "gemm_bf16_swiglu");
     return 0;
 }
 int launch_flash_fwd_bf16(void* stream, const void*, const void*, const void*, void*, long, long, long, long, float, int) {

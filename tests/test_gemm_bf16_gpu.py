@@ -288,3 +288,63 @@ def test_gemm_swiglu_epilogue_parity(dev, oracle, shape):
     fused = gu.try_shrink([(0, M), (0, F)]).silu().try_mul(gu.try_shrink([(0, M), (F, 2 * F)]))
     assert np.array_equal(fused.to_numpy(), got)
     assert [k for k in fused.kernels() if k.startswith("gemm_bf16_swiglu")], fused.kernels()
+
+
+# ---------------------------------------------------------------- second operand stored [N, K]
+# (a Linear layer's weight, tensor/src/nn/linear.rs:9-14: y = x @ weight.T + bias)
+@pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 256), (300, 520, 128), (1024, 1024, 1024), (1000, 776, 320),
+                                   (100, 264, 200), (256, 256, 72), (129, 8, 72), (2048, 512, 136), (37, 4096, 64)])
+def test_gemm_transposed_second_operand(dev, oracle, shape):
+    """a @ bt.T with bt [N, K] read in place: the same products in the same order as the
+    [K, N] form, so the same bits, on full, ragged-M/N and ragged-K shapes and with either tile
+    size; NaNs right behind a, bt and c show that no edge reads or writes past them."""
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 3, 20)
+    b = synth.normal_bf16((K, N), 3, 21)
+    bt = np.ascontiguousarray(b.T)
+    nan = np.full(8192, 0x7FC0, np.uint16)
+    ba = morok_amd.Buffer.from_numpy(np.concatenate([a.reshape(-1), nan]), dev.device_id)
+    bbt = morok_amd.Buffer.from_numpy(np.concatenate([bt.reshape(-1), nan]), dev.device_id)
+    bc = dev.buffer(M * N * 2 + 4096)
+    bc.copyin(np.full(M * N + 2048, 0x7FC0, np.uint16))
+    ops.gemm_bf16_nt(ba, bbt, bc, M, N, K, dev.device_id)
+    out = bc.copyout(np.uint16)
+    got = out[: M * N].reshape(M, N)
+    assert np.all(out[M * N:] == 0x7FC0)
+    _check(got, oracle.gemm_bf16(a, b), K)
+    assert np.array_equal(got, _gemm(dev, a, b, variant=3))
+    # and as a plan item
+    bc2 = dev.buffer(M * N * 2)
+    morok_amd.Program.builtin("gemm_bf16_nt", [M, N, K], dev.device_id).execute([bc2, ba, bbt])
+    assert np.array_equal(bc2.copyout(np.uint16, (M, N)), got)
+
+
+def test_gemm_transposed_second_operand_refusals(dev):
+    a, b, c = dev.buffer(4 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(4 * 1024 * 2)
+    with pytest.raises(morok_amd.MorokHipError):
+        ops.gemm_bf16_nt(a, b, c, 4, 1024, 4096, dev.device_id)   # few tiles, long K: the split-K shape
+    with pytest.raises(morok_amd.MorokHipError):
+        ops.gemm_bf16_nt(a, b, c, 4, 1020, 64, dev.device_id)     # N not a multiple of 8
+
+
+@pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 1024), (300, 264, 200), (1000, 520, 72)])
+def test_gemm_transposed_second_operand_epilogues(dev, shape):
+    """The residual and the gated epilogue over a [N, K] ([2F, K]) second operand, as plan items:
+    the bits of the same epilogues over the [K, N] form."""
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 7, 51)
+    b = synth.normal_bf16((K, N), 7, 52)
+    r = synth.normal_bf16((M, N), 7, 53)
+    ba, bb, bbt, br = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (a, b, np.ascontiguousarray(b.T), r))
+    c0, c1 = dev.buffer(M * N * 2), dev.buffer(M * N * 2)
+    morok_amd.Program.builtin("gemm_bf16_residual", [M, N, K], dev.device_id).execute([c0, ba, bb, br])
+    morok_amd.Program.builtin("gemm_bf16_nt_residual", [M, N, K], dev.device_id).execute([c1, ba, bbt, br])
+    assert np.array_equal(c0.copyout(np.uint16, (M, N)), c1.copyout(np.uint16, (M, N)))
+    F = N // 2
+    if F % 8 == 0:
+        w = synth.to_bf16(synth.normal((K, 2 * F), 11, 1, sigma=1.0 / np.sqrt(K)))
+        bw, bwt = morok_amd.Buffer.from_numpy(w, dev.device_id), morok_amd.Buffer.from_numpy(np.ascontiguousarray(w.T), dev.device_id)
+        g0, g1 = dev.buffer(M * F * 2), dev.buffer(M * F * 2)
+        morok_amd.Program.builtin("gemm_bf16_swiglu", [M, F, K], dev.device_id).execute([g0, ba, bw])
+        morok_amd.Program.builtin("gemm_bf16_nt_swiglu", [M, F, K], dev.device_id).execute([g1, ba, bwt])
+        assert np.array_equal(g0.copyout(np.uint16, (M, F)), g1.copyout(np.uint16, (M, F)))

@@ -435,6 +435,37 @@ def test_decoder_block_lowering(T, shim, fused, gemms):
     assert len(names) == (11 if fused else 16)   # fused: q and k also share one rotary kernel
 
 
+def test_linear_layout_weights_are_read_in_place(T, shim):
+    """x @ w.T with w [out, in] in memory (tensor/src/nn/linear.rs:39-41): the product kernels
+    take the weight as it is stored instead of a transposed copy, also under the residual and the
+    gated epilogue; shapes those kernels do not cover copy the transpose as before."""
+    bf = lambda shape: zeros(T, shape, np.uint16, uop.BF16)
+    x, w = bf((512, 256)), bf((768, 256))
+    y = x.linear(w)
+    assert y.shape == (512, 768) and y.realize().kernels() == ["gemm_bf16_nt_512_768_256"]
+    # the same through an explicit transpose, and with a bias (added by a kernel of its own)
+    assert x.matmul(w.try_transpose(0, 1)).realize().kernels() == ["gemm_bf16_nt_512_768_256"]
+    names = x.linear(w, bf((768,))).realize().kernels()
+    assert names[0] == "gemm_bf16_nt_512_768_256" and len(names) == 2
+    # residual epilogue
+    h = bf((512, 768))
+    assert h.try_add(x.linear(w)).realize().kernels() == ["gemm_bf16_nt_residual_512_768_256"]
+    # gated epilogue over a [2F, K] weight
+    w13 = bf((2 * 384, 256))
+    gu = x.linear(w13)
+    g = gu.try_shrink([(0, 512), (0, 384)]).silu().try_mul(gu.try_shrink([(0, 512), (384, 768)]))
+    assert g.realize().kernels() == ["gemm_bf16_nt_swiglu_512_384_256"]
+    # a weight that is not in memory as such (an expression) is computed in the layout the kernel reads
+    names = x.matmul(w.try_mul(2.0).cast(uop.BF16).try_transpose(0, 1)).realize().kernels()
+    assert names[-1] == "gemm_bf16_512_768_256" and len(names) == 2
+    # with fusion off nothing is matched
+    T.set_fusion(False)
+    try:
+        assert not any(k.startswith("gemm_bf16") for k in x.linear(w).realize().kernels())
+    finally:
+        T.set_fusion(True)
+
+
 def test_plan_graph_replay_records_once(T, shim):
     """execute_graph records the plan's launches once (nothing runs while recording), replays
     them with one graph launch per call, and drops the recording when variables are rebound or

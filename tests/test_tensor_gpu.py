@@ -951,6 +951,30 @@ def test_random_movement_chains_power_of_two_shapes(T, seed):
         np.testing.assert_array_equal(t.sum([ax]).to_numpy(), a.sum(ax))
 
 
+def test_linear_reads_the_weight_as_stored(T, oracle):
+    """x.linear(w) with w [out, in] (tensor/src/nn/linear.rs:39-41): one product kernel that reads
+    the weight in place, the bits of the product with the transposed copy, and within the GEMM
+    tolerance of the oracle; also under the residual add and with a ragged K."""
+    from morok_amd import synth, uop
+
+    T.set_fusion(True)
+    for (M, K, N) in ((512, 256, 768), (300, 200, 264)):
+        x, w, h = synth.normal_bf16((M, K), 9, 11), synth.normal_bf16((N, K), 9, 12), synth.normal_bf16((M, N), 9, 13)
+        tx, tw, th = (T.Tensor.from_numpy(t, uop.BF16) for t in (x, w, h))
+        y = tx.linear(tw)
+        got = y.to_numpy()
+        assert y.kernels() == [f"gemm_bf16_nt_{M}_{N}_{K}"]
+        wt = np.ascontiguousarray(w.T)
+        want = tx.matmul(T.Tensor.from_numpy(wt, uop.BF16)).to_numpy()
+        assert np.array_equal(got, want)
+        ref = synth.from_bf16(oracle.gemm_bf16(x, wt))
+        assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
+        r = th.try_add(tx.linear(tw))
+        got_r = r.to_numpy()
+        assert r.kernels() == [f"gemm_bf16_nt_residual_{M}_{N}_{K}"]
+        assert np.array_equal(got_r, synth.to_bf16(synth.from_bf16(got) + synth.from_bf16(h)))
+
+
 def test_matmul_bf16_residual_add_is_fused(T):
     """x + a @ w in bf16 with no other reader of the product: one kernel (the product kernel
     with the residual epilogue), on either side of the add and through contiguous(); the same
