@@ -364,7 +364,25 @@ std::string wmma_callee(const std::string& name, Scalar operand) {
     if (operand == Scalar::Fp8E5M2) return name + "_e5m2";
     return name;
 }
-bool wmma_wrapper(const std::string& name, Scalar operand, std::string* def) {
+// tied: the instruction written out with the accumulator in the accumulation registers and
+// result and accumulator in the same registers (16x16x32 bf16 / f16 only).  Through the builtin
+// the device compiler leaves this shape untied when the accumulators need those registers
+// (kernels with more than 128 declared registers per work-item, one wave per SIMD) and moves
+// whole tiles between the two register files on every step.
+bool wmma_wrapper(const std::string& name, Scalar operand, std::string* def, bool tied = false) {
+    if (tied) {
+        const char* mnemonic = name == "WMMA_16_16_32_bfloat_float" ? "v_mfma_f32_16x16x32_bf16"
+                               : name == "WMMA_16_16_32_half_float" ? "v_mfma_f32_16x16x32_f16" : nullptr;
+        if (!mnemonic) return false;
+        const char* in_t = name == "WMMA_16_16_32_bfloat_float" ? "__bf16" : "_Float16";
+        *def = fmt(
+            "typedef %s __%s_in __attribute__((ext_vector_type(8)));\n"
+            "typedef float __%s_acc __attribute__((ext_vector_type(4)));\n"
+            "static __device__ __forceinline__ __%s_acc __%s(__%s_in a, __%s_in b, __%s_acc c) {\n"
+            "  asm volatile(\"%s %%0, %%1, %%2, %%0\" : \"+a\"(c) : \"v\"(a), \"v\"(b));\n  return c;\n}\n",
+            in_t, name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str(), name.c_str(), mnemonic);
+        return true;
+    }
     if (operand == Scalar::Fp8E4M3 || operand == Scalar::Fp8E5M2) {
         if (name != "WMMA_16_16_32_unknown_float") return false;
         const std::string fn = wmma_callee(name, operand);
@@ -443,6 +461,25 @@ class Ctx {
     int depth = 1;
     std::map<std::string, int> counters;
     std::vector<std::pair<uint32_t, std::string>> pending_reduces;
+    // tensor-core instructions written as assembly (see wmma_wrapper): the register objects that
+    // hold their accumulators, (DEFINE_REG id, elements), and how many RANGEs are open
+    bool tied_wmma = false;
+    std::vector<std::pair<uint32_t, int64_t>> acc_regs;
+    std::unordered_set<uint32_t> acc_loads_with_other_users;
+    int range_depth = 0;
+    // The device compiler does not know such a statement as a matrix operation: the wait states it
+    // would insert between one and a vector instruction that reads or wrote the same registers
+    // are written out, and an empty statement per accumulator keeps its uses on the far side.
+    void settle_accumulators(int nops) {
+        for (int left = nops; left > 0; left -= 16)
+            body.push_back(indent() + fmt("asm volatile(\"s_nop %d\" ::: \"memory\");", (left > 16 ? 16 : left) - 1));
+        for (const auto& r : acc_regs) {
+            auto it = names.find(r.first);
+            if (it == names.end()) continue;
+            for (int64_t e = 0; e < r.second; e++)
+                body.push_back(indent() + fmt("asm volatile(\"\" : \"+a\"(%s[%" PRId64 "]));", it->second.c_str(), e));
+        }
+    }
 
     std::string indent() const { return std::string(static_cast<size_t>(depth) * 2, ' '); }
     std::string next(const std::string& prefix) { return prefix + std::to_string(counters[prefix]++); }
@@ -579,9 +616,52 @@ class HipRenderer final : public Renderer {
         // them between the halves on every trip of the K loop.  (One-wave workgroups measured
         // slower with the hint, so they go without.)
         const bool two_waves = !wmma_names.empty() && reg_bytes <= 128 * 4 && local[0] * local[1] * local[2] >= 256;
+        // more declared registers than half the file: the accumulators go to the accumulation
+        // registers, the 16x16x32 instruction is written out (see wmma_wrapper)
+        // (one wave per SIMD at most, and operands that reach the tensor core straight from local
+        // memory reads, as in the kernels with direct global -> local copies: a vector instruction
+        // that produced an operand just before would need wait states nothing inserts)
+        bool direct_copies = false;
+        for (const UOp& u : nodes) direct_copies = direct_copies || u.op == Op::AsyncCopy;
+        if (wmma_names.size() == 1 && reg_bytes > 128 * 4 && direct_copies && local[0] * local[1] * local[2] <= 256) {
+            std::string def;
+            ctx.tied_wmma = wmma_wrapper(wmma_names.begin()->first, wmma_names.begin()->second, &def, true);
+            // ... and only where an accumulator rests for at least eight instructions before the
+            // next one adds to it (also around the loop): nothing would make a dependent
+            // instruction wait for its predecessor's result
+            if (ctx.tied_wmma) {
+                auto nf = [&](uint32_t id) -> const UOp& { return *by_id.at(id); };
+                std::vector<uint32_t> order;  // register object (or the node itself) each WMMA accumulates into
+                for (const UOp& u : nodes)
+                    if (u.op == Op::Wmma && u.src.size() >= 3) {
+                        const UOp& c = *by_id.at(u.src[2]);
+                        const UOp* base = c.op == Op::Load && !c.src.empty() ? base_buffer_of(c.src[0], nf) : nullptr;
+                        order.push_back(base && base->op == Op::DefineReg ? base->id : u.src[2]);
+                    }
+                const size_t n = order.size();
+                for (size_t i = 0; i < n && ctx.tied_wmma; i++)
+                    for (size_t d = 1; d < 8 && d < n + 1; d++)
+                        if (order[(i + d) % n] == order[i]) ctx.tied_wmma = false;
+                if (n < 8) ctx.tied_wmma = false;
+            }
+        }
+        if (ctx.tied_wmma) {
+            std::set<uint32_t> seen_regs;
+            for (const UOp& u : nodes) {
+                if (u.op == Op::Store && u.src.size() >= 2 && by_id.at(u.src[1])->op == Op::Wmma) {
+                    auto nf = [&](uint32_t id) -> const UOp& { return *by_id.at(id); };
+                    const UOp* base = base_buffer_of(u.src[0], nf);
+                    if (base && base->op == Op::DefineReg && seen_regs.insert(base->id).second)
+                        ctx.acc_regs.push_back({base->id, base->dtype.ptr_size > 0 ? base->dtype.ptr_size : 1});
+                }
+                if (u.op != Op::Wmma)
+                    for (uint32_t sid : u.src)
+                        if (by_id.at(sid)->op == Op::Load) ctx.acc_loads_with_other_users.insert(sid);
+            }
+        }
         for (const auto& w : wmma_names) {
             std::string def;
-            if (!wmma_wrapper(w.first, w.second, &def)) return fail(kRenderError, "render: no gfx950 MFMA lowering for " + w.first);
+            if (!wmma_wrapper(w.first, w.second, &def, ctx.tied_wmma)) return fail(kRenderError, "render: no gfx950 MFMA lowering for " + w.first);
             pre.push_back(def);
         }
         if (uses_wave_reduce) pre.push_back(kWaveReducePreamble);
@@ -775,6 +855,9 @@ class HipRenderer final : public Renderer {
             case Op::Range: {  // ops.rs:303-316
                 MRK_TRY(need(1));
                 const std::string& var = ctx.get(u.id);
+                // the accumulators' initial values have been written a few wait states back
+                if (ctx.tied_wmma && ctx.range_depth == 0) ctx.settle_accumulators(8);
+                ctx.range_depth++;
                 ctx.body.push_back(ctx.indent() + fmt("for (%s %s = 0; %s < %s; %s++) {", c_scalar(u.dtype.scalar),
                                                       var.c_str(), var.c_str(), S(0).c_str(), var.c_str()));
                 ctx.depth++;
@@ -786,8 +869,11 @@ class HipRenderer final : public Renderer {
                     if (ctx.depth <= 1) return fail(kRenderError, "render: END without an open RANGE");
                     ctx.depth--;
                     ctx.body.push_back(ctx.indent() + "}");
+                    if (ctx.range_depth > 0) ctx.range_depth--;
                 }
                 ctx.pending_reduces.clear();
+                // the last results have left the matrix pipe before anything else reads them
+                if (ctx.tied_wmma && ctx.range_depth == 0) ctx.settle_accumulators(32);
                 return kOk;
             }
             case Op::If:
@@ -835,6 +921,13 @@ class HipRenderer final : public Renderer {
             case Op::Load: {  // ops.rs:186-215
                 MRK_TRY(need(1));
                 const UOp& ix = node(u.src[0]);
+                if (ctx.tied_wmma && ctx.range_depth > 0 && ctx.acc_loads_with_other_users.count(u.id)) {
+                    const UOp* base = base_buffer_of(u.src[0], node);
+                    for (const auto& r : ctx.acc_regs)
+                        if (base && base->id == r.first)
+                            return fail(kRenderError, "render: inside a loop an accumulator of written-out tensor-core instructions may only "
+                                                      "feed the next one (nothing waits for the matrix pipe there)");
+                }
                 std::string deref = u.dtype.vcount > 1 ? "*((" + c_value_type(u.dtype) + "*)(" + S(0) + "))" : "*(" + S(0) + ")";
                 std::string expr = deref;
                 if (ix.op == Op::Index && ix.sub) {
@@ -939,6 +1032,8 @@ class HipRenderer final : public Renderer {
             case Op::Wmma:  // ops.rs:404-411
                 MRK_TRY(need(3));
                 ctx.emit(u, "__" + wmma_callee(u.str, node(u.src[0]).dtype.scalar) + "(" + S(0) + ", " + S(1) + ", " + S(2) + ")", "wmma", true);
+                // written out, an instruction and what the kernel puts between it and the next one stay in that order
+                if (ctx.tied_wmma) ctx.body.push_back(ctx.indent() + "__builtin_amdgcn_sched_barrier(0);");
                 return kOk;
             case Op::Reduce: {  // ops.rs:342-361
                 MRK_TRY(need(1));
@@ -982,6 +1077,9 @@ class HipRenderer final : public Renderer {
                     dst = "(unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + S(1) + ")";
                 ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, off\" : : \"s\"(" +
                                    "__builtin_amdgcn_readfirstlane(" + dst + ")), \"v\"((const char*)(" + S(0) + ")) : \"m0\", \"memory\");");
+                // next to written-out tensor-core instructions the copy stays where the kernel puts it
+                // (a builder that spreads copies over a stretch of them means exactly that placement)
+                if (ctx.tied_wmma) ctx.body.push_back(ctx.indent() + "__builtin_amdgcn_sched_barrier(0);");
                 return kOk;
             }
             case Op::WaitAsync:

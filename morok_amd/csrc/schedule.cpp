@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstring>
+#include <functional>
 
 #include "error.h"
 
@@ -931,11 +932,13 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
         b_src[q] = b.iadd(b_tile0, b.iadd(b.imul(krow, N), col));
         b_dst[q] = b.imul(chunk, 512);
     }
-    auto copy_tile = [&](uint32_t kt, uint32_t stage) {  // kt, stage: nodes (uniform)
-        uint32_t ka = b.imul(kt, 64), kb = b.imul(kt, 64 * N);
-        uint32_t oa = b.imul(stage, A_STAGE), ob = b.imul(stage, B_STAGE);
-        for (int q = 0; q < CA; q++) b.async_copy(b.index(a, b.iadd(a_src[q], ka)), b.index(sA, b.iadd(a_dst[q], oa)));
-        for (int q = 0; q < CB; q++) b.async_copy(b.index(bmat, b.iadd(b_src[q], kb)), b.index(sB, b.iadd(b_dst[q], ob)));
+    // copy q (of CA + CB) of tile kt into stage `stage`; kt, stage: nodes (uniform)
+    auto copy_one = [&](int q, uint32_t kt, uint32_t stage) {
+        if (q < CA) b.async_copy(b.index(a, b.iadd(a_src[q], b.imul(kt, 64))), b.index(sA, b.iadd(a_dst[q], b.imul(stage, A_STAGE))));
+        else b.async_copy(b.index(bmat, b.iadd(b_src[q - CA], b.imul(kt, 64 * N))), b.index(sB, b.iadd(b_dst[q - CA], b.imul(stage, B_STAGE))));
+    };
+    auto copy_tile = [&](uint32_t kt, uint32_t stage) {
+        for (int q = 0; q < CA + CB; q++) copy_one(q, kt, stage);
     };
     // fragment addresses: lane-dependent base per K step (A) / per column tile (B) + constants.
     // A, K step s: logical 16-byte piece s * KG + lgk of row wy*um*TD + i*TD + lr (swizzle key (lr >> 1) & 7).
@@ -982,15 +985,20 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
     const DType cd = KernelBuilder::scalar(tc.dtype_out, EC);
     // the B fragment goes in as the first operand: the tensor core then leaves four consecutive
     // columns of one row in a lane (result rows are written as vectors), same products, same order
-    auto mfmas = [&](const std::vector<uint32_t>& af, const std::vector<uint32_t>& bf) {  // [h * um + i], [h * un + j]
+    // between(n): emitted behind tensor-core instruction n of the group
+    auto mfmas = [&](const std::vector<uint32_t>& af, const std::vector<uint32_t>& bf,  // [h * um + i], [h * un + j]
+                     const std::function<void(int)>& between = nullptr) {
         // columns back and forth, so that consecutive tensor-core instructions always share one
         // operand (fewer operand bits toggle; the part's clock under matrix load follows that)
+        int n = 0;
         for (int h = 0; h < HS; h++)
             for (int i = 0; i < um; i++)
                 for (int jj = 0; jj < un; jj++) {
                     const int j = (i & 1) ? un - 1 - jj : jj;
                     uint32_t slot = acc[i * un + j];
                     b.store(slot, b.add(Op::Wmma, cd, {bf[h * un + j], af[h * um + i], b.load(slot)}, 0, 0, 0, name));
+                    if (between) between(n);
+                    n++;
                 }
     };
     const int cpw = CA + CB;
@@ -1007,29 +1015,72 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
         uint32_t st = b.imod(r, 2), sn = bin(BinaryOp::Sub, b.ci(1), st);
         uint32_t oa = b.imul(st, A_STAGE), ob = b.imul(st, B_STAGE), na = b.imul(sn, A_STAGE), nb = b.imul(sn, B_STAGE);
         std::vector<uint32_t> f1a(HS * um), f1b(HS * un), f0a(HS * um), f0b(HS * un);
-        for (int h = 0; h < HS; h++) {
-            for (int i = 0; i < um; i++) f1a[h * um + i] = read_a(HS + h, i, oa);
-            for (int j = 0; j < un; j++) f1b[h * un + j] = read_b(HS + h, j, ob);
+        const int total = HS * um * un;  // tensor-core instructions per half step
+        if (W <= 4 && KT > 2) {
+            // One wave per SIMD: nothing fills the gaps a burst of local-memory reads or copies
+            // leaves in the wave's instruction stream, so every read and copy goes behind a
+            // tensor-core instruction of its own (the renderer keeps written-out tensor-core
+            // instructions and their neighbours in this order): the fragments of the second half
+            // behind the first half's instructions, the next tile's first-half fragments and the
+            // copies of tile r + 2 behind the second half's.  The last two steps copy the last
+            // tile again, into stages nobody reads any more, so that the loop has no branch.
+            std::vector<std::function<void()>> reads1, reads0;
+            for (int h = 0; h < HS; h++) {
+                for (int i = 0; i < um; i++) reads1.push_back([&, h, i] { f1a[h * um + i] = read_a(HS + h, i, oa); });
+                for (int j = 0; j < un; j++) reads1.push_back([&, h, j] { f1b[h * un + j] = read_b(HS + h, j, ob); });
+                for (int i = 0; i < um; i++) reads0.push_back([&, h, i] { b.store(fa0[h * um + i], read_a(h, i, na)); });
+                for (int j = 0; j < un; j++) reads0.push_back([&, h, j] { b.store(fb0[h * un + j], read_b(h, j, nb)); });
+            }
+            for (size_t i = 0; i < fa0.size(); i++) f0a[i] = b.load(fa0[i]);
+            for (size_t j = 0; j < fb0.size(); j++) f0b[j] = b.load(fb0[j]);
+            size_t done1 = 0;
+            mfmas(f0a, f0b, [&](int n) {
+                if (done1 < reads1.size()) reads1[done1++]();
+                if (n == total - 1)
+                    while (done1 < reads1.size()) reads1[done1++]();
+            });
+            // tile r + 1 has landed in the other stage and, behind the barrier, nobody reads this
+            // stage any more
+            b.wait_async(0);
+            b.barrier();
+            uint32_t kt2 = bin(BinaryOp::Sub, b.ci(KT - 1), bin(BinaryOp::Max, bin(BinaryOp::Sub, b.ci(KT - 3), r), b.ci(0)));
+            size_t done0 = 0;
+            int issued = 0;
+            const int left = std::max(1, total - (int)reads0.size());
+            const int every = std::max(1, left / cpw);
+            mfmas(f1a, f1b, [&](int n) {
+                if (done0 < reads0.size()) reads0[done0++]();
+                else if ((n - (int)reads0.size()) % every == 0 && issued < cpw) copy_one(issued++, kt2, st);
+                if (n == total - 1) {
+                    while (done0 < reads0.size()) reads0[done0++]();
+                    while (issued < cpw) copy_one(issued++, kt2, st);
+                }
+            });
+        } else {
+            for (int h = 0; h < HS; h++) {
+                for (int i = 0; i < um; i++) f1a[h * um + i] = read_a(HS + h, i, oa);
+                for (int j = 0; j < un; j++) f1b[h * un + j] = read_b(HS + h, j, ob);
+            }
+            for (size_t i = 0; i < fa0.size(); i++) f0a[i] = b.load(fa0[i]);
+            for (size_t j = 0; j < fb0.size(); j++) f0b[j] = b.load(fb0[j]);
+            mfmas(f0a, f0b);
+            // tile r + 1 has landed in the other stage (issued half a step ago or earlier) and, behind
+            // the barrier, nobody reads this stage any more
+            b.wait_async(0);
+            b.barrier();
+            if (KT > 2) {
+                uint32_t r2 = b.iadd(r, b.ci(2));
+                b.if_(bin(BinaryOp::Lt, r2, b.ci(KT)));
+                copy_tile(r2, st);
+                b.endif();
+            }
+            // first half of tile r + 1 (after the last tile: a stale stage, read and never used)
+            for (int h = 0; h < HS; h++) {
+                for (int i = 0; i < um; i++) b.store(fa0[h * um + i], read_a(h, i, na));
+                for (int j = 0; j < un; j++) b.store(fb0[h * un + j], read_b(h, j, nb));
+            }
+            mfmas(f1a, f1b);
         }
-        for (size_t i = 0; i < fa0.size(); i++) f0a[i] = b.load(fa0[i]);
-        for (size_t j = 0; j < fb0.size(); j++) f0b[j] = b.load(fb0[j]);
-        mfmas(f0a, f0b);
-        // tile r + 1 has landed in the other stage (issued half a step ago or earlier) and, behind
-        // the barrier, nobody reads this stage any more
-        b.wait_async(0);
-        b.barrier();
-        if (KT > 2) {
-            uint32_t r2 = b.iadd(r, b.ci(2));
-            b.if_(bin(BinaryOp::Lt, r2, b.ci(KT)));
-            copy_tile(r2, st);
-            b.endif();
-        }
-        // first half of tile r + 1 (after the last tile: a stale stage, read and never used)
-        for (int h = 0; h < HS; h++) {
-            for (int i = 0; i < um; i++) b.store(fa0[h * um + i], read_a(h, i, na));
-            for (int j = 0; j < un; j++) b.store(fb0[h * un + j], read_b(h, j, nb));
-        }
-        mfmas(f1a, f1b);
     }
     b.end({r});
     // Result.  A lane holds, per tile, groups of four consecutive columns of one row.  When the result

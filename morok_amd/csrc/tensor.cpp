@@ -1252,7 +1252,7 @@ struct Scheduler {
         // global -> local copies (faster at every shape measured: 4096^3 1.26 against 1.08 PF,
         // 2048^3 0.76 against 0.49, 1024^3 0.30 against 0.23): the largest tile that still fills
         // the chip (one 256 x 256 workgroup or two smaller ones per CU), else the smallest
-        static const int direct[][5] = {{2, 4, 8, 4, 256}, {2, 2, 4, 4, 512}, {2, 2, 4, 2, 512}, {2, 2, 2, 2, 0}};
+        static const int direct[][5] = {{2, 2, 8, 8, 256}, {2, 4, 8, 4, 256}, {2, 2, 4, 4, 512}, {2, 2, 4, 2, 512}, {2, 2, 2, 2, 0}};
         for (auto& c : direct) {
             WmmaLdsOpts t{c[0], c[1], c[2], c[3], 0, 2};
             if (!wmma_lds_opts_valid(tc, t, M, N, K)) continue;

@@ -248,6 +248,40 @@ def test_wmma_matmul_direct_copy_kernel_builds_and_compiles():
     half = U.render(sched.build_wmma_matmul_lds_opts(2, 128, 128, 128, U.F16, (2, 2, 4, 4, 0, 2)), "r_tc_dma_h")
     assert "__builtin_amdgcn_ds_read_tr16_b64_v4f16(" in half.src
     morok_amd.compile_spec(half)
+    # builtin form for the kernels above (their accumulators fit half of the register file)
+    assert "__builtin_amdgcn_mfma_f32_16x16x32_bf16(" in src and "v_mfma_f32_16x16x32_bf16 %0" not in src
+
+
+def test_wmma_matmul_direct_copy_one_wave_per_simd_is_written_out():
+    """Four waves with 8 x 8 tiles each (256 accumulator registers, one wave per SIMD): the tensor-core
+    instruction is written out with its accumulator tied in place in the accumulation registers,
+    the waits the device compiler would insert around it are explicit (in front of the loop for the
+    initial values, behind it for the last results, each followed by one empty statement per
+    accumulator), every local-memory read and copy of the loop sits behind a tensor-core instruction
+    of its own, and the loop has no branch (the last two steps copy the last tile again)."""
+    import morok_amd
+    from morok_amd import sched, uop as U
+
+    M, N, K = 512, 512, 256
+    spec = U.render(sched.build_wmma_matmul_lds_opts(3, M, N, K, U.BF16, (2, 2, 8, 8, 0, 2)), "r_tc_dma4")
+    src = spec.src
+    assert spec.sizes() == ([4, 1, 1], [64, 4, 1])
+    assert 'asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));' in src
+    assert "__builtin_amdgcn_mfma_f32_16x16x32_bf16(" not in src
+    loop = src[src.index("for (int ridx0"):]
+    loop = loop[:loop.index("\n  }\n")]
+    assert "if (" not in loop and loop.count("global_load_lds_dwordx4") == 16 and loop.count("__WMMA_16_16_32_bfloat_float(") == 128
+    # no two reads or copies without a tensor-core instruction between them
+    kinds = [("w" if "__WMMA_" in l else "m" if ("global_load_lds" in l or "ds_read_tr16" in l) else "") for l in loop.split("\n")]
+    seq = "".join(kinds)
+    assert "mmm" not in seq.replace("w", "|").replace("||", "|")  # (a B fragment is two transposing reads)
+    before, after = src[:src.index("for (int ridx0")], src[src.index("for (int ridx0"):]
+    assert before.count('asm volatile("" : "+a"(') == 64 and 'asm volatile("s_nop 7"' in before
+    assert after.count('asm volatile("" : "+a"(') == 64 and after.count('asm volatile("s_nop 15"') == 2
+    morok_amd.compile_spec(spec)
+    half = U.render(sched.build_wmma_matmul_lds_opts(2, M, N, K, U.F16, (2, 2, 8, 8, 0, 2)), "r_tc_dma4_h")
+    assert "v_mfma_f32_16x16x32_f16 %0" in half.src
+    morok_amd.compile_spec(half)
 
 
 def test_tc_matmul_direct_copy_refuses_what_it_cannot_tile():
