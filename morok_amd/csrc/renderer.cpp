@@ -1075,8 +1075,19 @@ class HipRenderer final : public Renderer {
                           ctx.get(li.src[1]) + ") * " + std::to_string(scalar_bytes(l->dtype.scalar) * l->dtype.vcount) + "u";
                 else
                     dst = "(unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + S(1) + ")";
-                ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, off\" : : \"s\"(" +
-                                   "__builtin_amdgcn_readfirstlane(" + dst + ")), \"v\"((const char*)(" + S(0) + ")) : \"m0\", \"memory\");");
+                // source: the buffer's (scalar) base plus a 32-bit byte offset per lane where the buffer
+                // is known to be smaller than 4 GiB (two vector instructions fewer per copy than a
+                // 64-bit address per lane), else the full address
+                const UOp& gi = node(u.src[0]);
+                const int64_t gbytes = static_cast<int64_t>(scalar_bytes(g->dtype.scalar)) * g->dtype.vcount;
+                if (gi.op == Op::Index && gi.src.size() == 2 && !gi.sub && node(gi.src[0]).op == Op::Param && g->dtype.ptr_size > 0 &&
+                    g->dtype.ptr_size * gbytes <= (int64_t(1) << 32))
+                    ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, %2\" : : \"s\"(" +
+                                       "__builtin_amdgcn_readfirstlane(" + dst + ")), \"v\"((unsigned)(" + ctx.get(gi.src[1]) + ") * " +
+                                       std::to_string(gbytes) + "u), \"s\"(" + ctx.get(gi.src[0]) + ") : \"m0\", \"memory\");");
+                else
+                    ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, off\" : : \"s\"(" +
+                                       "__builtin_amdgcn_readfirstlane(" + dst + ")), \"v\"((const char*)(" + S(0) + ")) : \"m0\", \"memory\");");
                 // next to written-out tensor-core instructions the copy stays where the kernel puts it
                 // (a builder that spreads copies over a stretch of them means exactly that placement)
                 if (ctx.tied_wmma) ctx.body.push_back(ctx.indent() + "__builtin_amdgcn_sched_barrier(0);");
