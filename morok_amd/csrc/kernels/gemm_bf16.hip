@@ -539,6 +539,41 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     constexpr int kChunks = kJ * 4;          // 16-byte chunks per row of the wave's tile
     constexpr int kRowsPerIt = 64 / kChunks;  // rows one store instruction covers
     constexpr int kIts = 128 / kRowsPerIt;
+    if constexpr (!kResidual && !kSwiGLU) {
+        // The plain product: 16 rows at a time.  A wave reads back only what it staged itself, and
+        // the LDS serves a wave's requests in order, so the rows of tile row i are read back and
+        // stored while tile row i + 1 is being converted and staged: the stores start one tile row
+        // after the loop ends instead of after the whole staging.
+        constexpr int kPerRow = 16 / kRowsPerIt;  // store instructions per tile row
+        const int lr = lane / kChunks, lc = lane % kChunks;  // the lane's row inside a store, its 16-byte chunk
+        const int rows_here = row0 >= (size_t)M ? 0 : (size_t)M - row0 < 128 ? (int)((size_t)M - row0) : 128;  // rows of the wave's tile inside C
+        const bool col_ok = col0 + lc * 8 + 8 <= (size_t)N;
+        __bf16* Cl = C + (row0 + lr) * N + col0 + lc * 8;
+        const char* sCl = sC + lr * kCPitchT + lc * 16;
+        auto stage_row = [&](int i) {
+#pragma unroll
+            for (int j = 0; j < kJ16; j++) {
+                bf16x4 h = __builtin_convertvector(acc[i][j], bf16x4);
+                *LDS_PTR(bf16x4, sC + (i * 16 + (lane & 15)) * kCPitchT + (j * 16 + 4 * (lane >> 4)) * 2) = h;
+            }
+        };
+        stage_row(0);
+#pragma unroll
+        for (int i = 0; i < kI16; i++) {
+            u32x4 v[kPerRow];
+#pragma unroll
+            for (int t = 0; t < kPerRow; t++) v[t] = *LDS_PTR(u32x4, sCl + (i * 16 + t * kRowsPerIt) * kCPitchT);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i + 1 < kI16) stage_row(i + 1);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < kPerRow; t++) {
+                const int r = i * 16 + t * kRowsPerIt;
+                if (col_ok && r + lr < rows_here) *reinterpret_cast<u32x4*>(Cl + (size_t)r * N) = v[t];
+            }
+        }
+        return;
+    }
     constexpr int kFirstBatch = kIts / 4;  // as many as fit the register file next to the live accumulators
     // the residual rows this lane will add are fetched ahead, in two batches, so that their latency
     // overlaps the staging of the accumulators instead of sitting in front of every store
