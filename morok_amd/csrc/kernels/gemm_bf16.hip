@@ -504,6 +504,25 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         phase(C2{}, C{}, sAx + a_xo[0], sBx + b_ks(0));
         phase(C3{}, C{}, sAx + a_xo[0], sBx + b_ks(0));
     };
+    // What the epilogue of the plain and the residual product needs, ahead of the loop's end: lane l
+    // stores (and fetches from R) 16-byte chunk l % kChunks of row it * kRowsPerIt + l / kChunks of
+    // the wave's 128-row tile, for it = 0 .. kIts-1.
+    const size_t row0 = m0 + wm * 128, col0 = n0 + wn * (kJ * 32);
+    constexpr int kChunks = kJ * 4;          // 16-byte chunks per row of the wave's tile
+    constexpr int kRowsPerIt = 64 / kChunks;  // rows one store instruction covers
+    constexpr int kIts = 128 / kRowsPerIt;
+    const int lr = lane / kChunks, lc = lane % kChunks;
+    const int rows_here = row0 >= (size_t)M ? 0 : (size_t)M - row0 < 128 ? (int)((size_t)M - row0) : 128;  // rows of the wave's tile inside C
+    const bool col_ok = col0 + lc * 8 + 8 <= (size_t)N;
+    u32x4 res[kResidual ? kIts : 1];
+    auto fetch_residual = [&](int first, int last) {
+        const __bf16* Rl = R + (row0 + lr) * N + col0 + lc * 8;
+#pragma unroll
+        for (int it = first; it < last; it++) {
+            res[it] = u32x4{0u, 0u, 0u, 0u};
+            if (col_ok && it * kRowsPerIt + lr < rows_here) res[it] = *reinterpret_cast<const u32x4*>(Rl + (size_t)(it * kRowsPerIt) * N);
+        }
+    };
     {
         int kt = 0;
         for (; kt + 1 < KT; kt += 2) {
@@ -512,6 +531,11 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         }
         if (kt < KT) iteration(C0{});
     }
+    // The residual rows are on their way while the accumulators are converted and staged: the
+    // fragment registers of the loop are free from here on.  (Fetching half of them before the
+    // last two K steps instead measured the same: the loop's waits on its own copies count
+    // vector-memory operations in order, so they wait for the residual rows as well.)
+    if constexpr (kResidual) fetch_residual(0, kIts);
     full_barrier();
     // the last MFMAs' results must have left the matrix pipe before the vector ALUs read them (the
     // compiler does not see the instructions above as matrix operations); the empty statements
@@ -523,7 +547,6 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     // C[m = i*16 + l%16][n = j*16 + 4*(l/16) + 0..3].
     if (kSplitK) {
         // f32 partials straight from the registers: 16 bytes per lane, rows and columns masked
-        const size_t row0 = m0 + wm * 128, col0 = n0 + wn * (kJ * 32);
         float* Wt = W + ((size_t)blockIdx.z * gridDim.y + blockIdx.y) * (size_t)M * N;
 #pragma unroll
         for (int i = 0; i < kI16; i++)
@@ -535,19 +558,12 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         return;
     }
     char* sC = smem + wave * kCWaveT;
-    const size_t row0 = m0 + wm * 128, col0 = n0 + wn * (kJ * 32);
-    constexpr int kChunks = kJ * 4;          // 16-byte chunks per row of the wave's tile
-    constexpr int kRowsPerIt = 64 / kChunks;  // rows one store instruction covers
-    constexpr int kIts = 128 / kRowsPerIt;
-    if constexpr (!kResidual && !kSwiGLU) {
-        // The plain product: 16 rows at a time.  A wave reads back only what it staged itself, and
-        // the LDS serves a wave's requests in order, so the rows of tile row i are read back and
-        // stored while tile row i + 1 is being converted and staged: the stores start one tile row
-        // after the loop ends instead of after the whole staging.
+    if constexpr (!kSwiGLU) {
+        // The plain and the residual product: 16 rows at a time.  A wave reads back only what it
+        // staged itself, and the LDS serves a wave's requests in order, so the rows of tile row i
+        // are read back and stored while tile row i + 1 is being converted and staged: the stores
+        // start one tile row after the loop ends instead of after the whole staging.
         constexpr int kPerRow = 16 / kRowsPerIt;  // store instructions per tile row
-        const int lr = lane / kChunks, lc = lane % kChunks;  // the lane's row inside a store, its 16-byte chunk
-        const int rows_here = row0 >= (size_t)M ? 0 : (size_t)M - row0 < 128 ? (int)((size_t)M - row0) : 128;  // rows of the wave's tile inside C
-        const bool col_ok = col0 + lc * 8 + 8 <= (size_t)N;
         __bf16* Cl = C + (row0 + lr) * N + col0 + lc * 8;
         const char* sCl = sC + lr * kCPitchT + lc * 16;
         auto stage_row = [&](int i) {
@@ -569,28 +585,16 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
 #pragma unroll
             for (int t = 0; t < kPerRow; t++) {
                 const int r = i * 16 + t * kRowsPerIt;
+                if constexpr (kResidual) {
+                    const f32x8 sum = __builtin_convertvector(__builtin_bit_cast(bf16x8, v[t]), f32x8) +
+                                      __builtin_convertvector(__builtin_bit_cast(bf16x8, res[i * kPerRow + t]), f32x8);
+                    v[t] = __builtin_bit_cast(u32x4, __builtin_convertvector(sum, bf16x8));
+                }
                 if (col_ok && r + lr < rows_here) *reinterpret_cast<u32x4*>(Cl + (size_t)r * N) = v[t];
             }
         }
         return;
     }
-    constexpr int kFirstBatch = kIts / 4;  // as many as fit the register file next to the live accumulators
-    // the residual rows this lane will add are fetched ahead, in two batches, so that their latency
-    // overlaps the staging of the accumulators instead of sitting in front of every store
-    // (a quarter of them while the accumulators are still live, the rest once they are staged:
-    // more at once would not fit the register file next to the accumulators)
-    u32x4 res[kResidual ? kIts : 1];
-    auto fetch_residual = [&](int first, int last) {
-#pragma unroll
-        for (int it = first; it < last; it++) {
-            const int r = it * kRowsPerIt + lane / kChunks;
-            const int ch = lane % kChunks;
-            res[it] = u32x4{0u, 0u, 0u, 0u};
-            if (row0 + r < (size_t)M && col0 + ch * 8 + 8 <= (size_t)N)
-                res[it] = *reinterpret_cast<const u32x4*>(R + (row0 + r) * N + col0 + ch * 8);
-        }
-    };
-    if constexpr (kResidual) fetch_residual(0, kFirstBatch);
 #pragma unroll
     for (int i = 0; i < kI16; i++)
 #pragma unroll
@@ -599,21 +603,12 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
             const int ml = i * 16 + (lane & 15);
             const int nl = j * 16 + 4 * (lane >> 4);
             *LDS_PTR(bf16x4, sC + ml * kCPitchT + nl * 2) = h;
-            // (tile by tile: moved out of the accumulation registers all at once, the tile would
-            // not fit the vector registers next to the residual rows)
-            if (kResidual && (j & 1)) __builtin_amdgcn_sched_barrier(0);
         }
-    if constexpr (kResidual) {
-        asm volatile("" ::: "memory");  // not before the accumulators have left their registers
-        fetch_residual(kFirstBatch, kIts);
-    }
-    // a wave reads back only what it staged itself (the LDS serves a wave's requests in order),
-    // except for the gated epilogue, where gate and up blocks come from two waves
-    if constexpr (kSwiGLU) __syncthreads();
-    else asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    // The gated epilogue: waves (wm, 0) and (wm, 1) staged the gate and the up block of the same
+    // 128 rows x 128 columns; each of the two now combines 64 of those rows: 16 chunks of 8 columns
+    // per row.
     if constexpr (kSwiGLU) {
-        // waves (wm, 0) and (wm, 1) staged the gate and the up block of the same 128 rows x 128
-        // columns; each of the two now combines 64 of those rows: 16 chunks of 8 columns per row
+        __syncthreads();
         const size_t F = (size_t)N / 2;
         const char* sG = smem + (wm * 2 + 0) * kCWaveT;
         const char* sU = smem + (wm * 2 + 1) * kCWaveT;
@@ -632,28 +627,6 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
             }
             const u32x4 v = __builtin_bit_cast(u32x4, __builtin_convertvector(y, bf16x8));
             if (row0 + r < (size_t)M && n0 + ch * 8 + 8 <= F) *reinterpret_cast<u32x4*>(C + (row0 + r) * F + n0 + ch * 8) = v;
-        }
-        return;
-    }
-    __bf16* Cg = C + row0 * N + col0;
-    if constexpr (kResidual) {
-#pragma unroll
-        for (int it = 0; it < kIts; it++) {
-            const int r = it * kRowsPerIt + lane / kChunks;
-            const int ch = lane % kChunks;
-            u32x4 v = *LDS_PTR(u32x4, sC + r * kCPitchT + ch * 16);
-            const f32x8 sum = __builtin_convertvector(__builtin_bit_cast(bf16x8, v), f32x8) +
-                              __builtin_convertvector(__builtin_bit_cast(bf16x8, res[it]), f32x8);
-            v = __builtin_bit_cast(u32x4, __builtin_convertvector(sum, bf16x8));
-            if (row0 + r < (size_t)M && col0 + ch * 8 + 8 <= (size_t)N) *reinterpret_cast<u32x4*>(Cg + (size_t)r * N + ch * 8) = v;
-        }
-    } else {
-#pragma unroll 4
-        for (int it = 0; it < kIts; it++) {
-            const int r = it * kRowsPerIt + lane / kChunks;
-            const int ch = lane % kChunks;
-            u32x4 v = *LDS_PTR(u32x4, sC + r * kCPitchT + ch * 16);
-            if (row0 + r < (size_t)M && col0 + ch * 8 + 8 <= (size_t)N) *reinterpret_cast<u32x4*>(Cg + (size_t)r * N + ch * 8) = v;
         }
     }
 }
