@@ -212,7 +212,10 @@ def test_gemm_split_k_not_used_for_large_shapes():
         assert lib.mrk_hip_gemm_bf16_workspace_bytes(*shape, 1) == 0, shape
 
 
-@pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 4096), (300, 264, 200), (128, 4096, 136), (1000, 520, 72), (257, 8, 8)])
+# (2148, 4096, 64) and (2148, 4104, 72) are large enough for the 256-row tile and end in a tile
+# whose lower two waves lie entirely below row M.
+@pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 4096), (300, 264, 200), (128, 4096, 136), (1000, 520, 72), (257, 8, 8),
+                                   (2148, 4096, 64), (2148, 4104, 72)])
 def test_gemm_residual_epilogue(dev, oracle, shape):
     """c = a b + r with r added in the product kernel's epilogue: the bits of the plain
     product followed by an f32 add and one more rounding (the oracle's product, then numpy),
