@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <functional>
 #include <map>
 #include <mutex>
 #include <set>
@@ -2079,6 +2080,58 @@ struct Scheduler {
             }
             if (!progress) return {};
         }
+        // The kernel hands a reduction's consumer the total of the workgroup's own row whatever
+        // coordinates the consumer asks for, so every path from the output (and from a later
+        // reduction's expression) down to a fused reduction must keep the row: elementwise nodes
+        // of the output's shape, one expand of the keepdim shape, and below it elementwise nodes
+        // and reshapes that only add or drop axes of extent 1.  A transpose, shrink, cat, gather
+        // or any other expand on such a path (x + rowsum.T) keeps the separate reduce kernel.
+        std::vector<int64_t> kshape = n->shape;
+        kshape.back() = 1;
+        auto strip1 = [](const std::vector<int64_t>& s) {
+            std::vector<int64_t> r;
+            for (int64_t d : s)
+                if (d != 1) r.push_back(d);
+            return r;
+        };
+        const std::vector<int64_t> kstripped = strip1(kshape);
+        std::map<const TensorNode*, bool> reach_memo;
+        std::function<bool(const TensorNode*)> reaches = [&](const TensorNode* m) -> bool {
+            if (std::find(found.begin(), found.end(), m) != found.end()) return true;
+            if (m->buffer || m->kind == TKind::Reduce) return false;
+            auto it = reach_memo.find(m);
+            if (it != reach_memo.end()) return it->second;
+            bool r = false;
+            for (const TensorRef& c : m->src) r = r || reaches(c.get());
+            return reach_memo[m] = r;
+        };
+        std::map<std::pair<const TensorNode*, bool>, bool> ok_memo;
+        std::function<bool(const TensorNode*, bool)> keeps_row = [&](const TensorNode* m, bool full) -> bool {
+            if (std::find(found.begin(), found.end(), m) != found.end()) return !full && m->shape == kshape;
+            if (!reaches(m)) return true;  // read at the coordinates it is asked for, like any operand
+            auto it = ok_memo.find({m, full});
+            if (it != ok_memo.end()) return it->second;
+            bool ok = false;
+            switch (m->kind) {
+                case TKind::Unary:
+                case TKind::Binary:
+                case TKind::Where:
+                case TKind::Cast:
+                case TKind::Contiguous:
+                    ok = true;
+                    for (const TensorRef& c : m->src) ok = ok && c->shape == m->shape && keeps_row(c.get(), full);
+                    break;
+                case TKind::Expand: ok = full && m->shape == n->shape && m->src[0]->shape == kshape && keeps_row(m->src[0].get(), false); break;
+                case TKind::Reshape:
+                    ok = !full && strip1(m->shape) == kstripped && strip1(m->src[0]->shape) == kstripped && keeps_row(m->src[0].get(), false);
+                    break;
+                default: break;
+            }
+            return ok_memo[{m, full}] = ok;
+        };
+        if (!keeps_row(n, true)) return {};
+        for (TensorNode* R : ordered)
+            if (!keeps_row(R->src[0].get(), true)) return {};
         const int64_t C = n->shape.back(), rows = n->numel() / C;
         int64_t width = 1;
         for (int64_t w = 16 / static_cast<int64_t>(scalar_size(n->dtype)); w > 1; w /= 2)

@@ -573,6 +573,38 @@ def test_beam_search_over_generated_kernels(dev, shim, tmp_path, monkeypatch):
     assert timed >= 3 and hits == 0 and T.last_kernels() == ["rE_256_g4096_4"]
 
 
+def test_row_resident_fusion_needs_a_path_that_keeps_the_row(T):
+    """A keepdim reduction reaches the fused kernel's consumer as the workgroup's own row total,
+    so it may only be fused when every path to it keeps the row coordinate: a transpose, a
+    shrink or a reshape that moves the reduced axis in between must keep the separate kernel."""
+    def names(t):
+        t.realize()
+        return T.last_kernels()
+
+    x = zeros(T, (256, 256))
+    same_row = x.try_add(x.sum(1, keepdim=True).try_expand([256, 256]))
+    assert names(same_row) == ["rE_256_g256_4"]
+    squeezed = x.try_mul(x.sum(1).try_reshape([256, 1]).try_expand([256, 256]))      # drop and re-add the axis of extent 1
+    assert names(squeezed) == ["rE_256_g256_4"]
+    other_row = x.try_add(x.sum(1, keepdim=True).try_transpose(0, 1).try_expand([256, 256]))   # x[i, j] + rowsum[j]
+    assert not any(k.startswith("rE_") for k in names(other_row)) and len(T.last_kernels()) == 2
+    as_columns = x.try_add(x.sum(1).try_reshape([1, 256]).try_expand([256, 256]))
+    assert not any(k.startswith("rE_") for k in names(as_columns))
+    b = zeros(T, (128, 128, 64))
+    batch_swapped = b.try_add(b.sum(2, keepdim=True).try_permute([1, 0, 2]).try_expand([128, 128, 64]))
+    assert not any(k.startswith("rE_") for k in names(batch_swapped))
+    y = zeros(T, (512, 256))
+    shifted = y.try_shrink([(0, 256), (0, 256)]).try_add(y.sum(1, keepdim=True).try_shrink([(256, 512), (0, 1)]).try_expand([256, 256]))
+    assert not any(k.startswith("rE_") for k in names(shifted))
+    # the second reduction of a chain must keep the row as well
+    m = x.max(1, keepdim=True)
+    chain = x.try_sub(m.try_transpose(0, 1).try_expand([256, 256])).try_exp()
+    bad_chain = chain.try_div(chain.sum(1, keepdim=True).try_expand([256, 256]))
+    assert not any(k.endswith("_x2") for k in names(bad_chain))
+    good = names(zeros(T, (256, 1024), np.uint16, uop.BF16).softmax(-1))
+    assert len(good) == 1 and good[0].startswith("rE_") and good[0].endswith("_x2")
+
+
 def test_beam_search_uses_and_fills_the_disk_cache(dev, shim, tmp_path, monkeypatch):
     from morok_amd import sched
 

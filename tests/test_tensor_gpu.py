@@ -1393,3 +1393,36 @@ def test_chained_row_fusion_falls_back_when_a_total_is_needed_elsewhere(T):
     e64 = np.exp(x64 - x64.max(-1, keepdims=True))
     ref = e64 / e64.sum(-1, keepdims=True) + x64.max(-1, keepdims=True)
     assert np.abs(got - ref).max() <= 1e-5 * np.abs(ref).max() and len(both.kernels()) >= 2
+
+
+def test_row_fusion_is_refused_when_the_reduction_is_read_at_other_rows(T):
+    """x[i, j] + rowsum[j] (the row totals transposed), a batch permute of them and a shifted slice
+    of them over square shapes: the consumer does not read its own row's total, so these must not
+    become the row-resident kernel; values against float64."""
+    from morok_amd import synth
+
+    x = synth.normal((256, 256), 97, 0)
+    x64 = x.astype(np.float64)
+    tx = T.Tensor.from_numpy(x)
+    rs = tx.sum(1, keepdim=True)
+    same = tx.try_add(rs.try_expand([256, 256]))
+    got = same.to_numpy()
+    assert same.kernels() == ["rE_256_g256_4"]
+    np.testing.assert_allclose(got, x64 + x64.sum(1, keepdims=True), rtol=1e-4, atol=1e-4)
+    other = tx.try_add(tx.sum(1, keepdim=True).try_transpose(0, 1).try_expand([256, 256]))
+    got = other.to_numpy()
+    assert not any(k.startswith("rE_") for k in other.kernels())
+    np.testing.assert_allclose(got, x64 + x64.sum(1)[None, :], rtol=1e-4, atol=1e-4)
+    b = synth.normal((128, 128, 64), 97, 1)
+    b64 = b.astype(np.float64)
+    tb = T.Tensor.from_numpy(b)
+    sw = tb.try_mul(tb.max(2, keepdim=True).try_permute([1, 0, 2]).try_expand([128, 128, 64]))
+    got = sw.to_numpy()
+    assert not any(k.startswith("rE_") for k in sw.kernels())
+    np.testing.assert_allclose(got, b64 * b64.max(2, keepdims=True).transpose(1, 0, 2), rtol=1e-5, atol=1e-6)
+    y = synth.normal((512, 256), 97, 2)
+    y64 = y.astype(np.float64)
+    ty = T.Tensor.from_numpy(y)
+    sh = ty.try_shrink([(0, 256), (0, 256)]).try_add(ty.sum(1, keepdim=True).try_shrink([(256, 512), (0, 1)]).try_expand([256, 256]))
+    got = sh.to_numpy()
+    np.testing.assert_allclose(got, y64[:256] + y64.sum(1, keepdims=True)[256:], rtol=1e-4, atol=1e-4)
