@@ -38,7 +38,7 @@ MIB = 1 << 20
 # kernel, and only when that summary names the kernel this run launched; otherwise null.
 PROFILE_OF = {"softmax": "softmax_rows_in_regs_8192x8192_f32.txt", "gemm": "gemm_bf16_tile256_4096cubed.txt",
               "flash": "flash_fwd_d128_causal_8x32x4096x128.txt", "decoder": "decoder_block_4x2048_h4096.txt",
-              "generated_tc": "generated_tensor_core_gemm_4096cubed.txt"}
+              "generated_tc": "generated_tensor_core_gemm_4096cubed.txt", "matmul_f32": "generated_f32_matmul_1024cubed.txt"}
 
 
 def _profiled_traffic(workload, kernel):
@@ -359,9 +359,8 @@ def bench_matmul_f32(m, dev, steps, warmup, cpu):
         "config": {"workload": "f32 matmul 1024^3 via the lazy tensor API, generated kernel (configs[0])"},
         # a generated kernel of vector-ALU fused multiply-adds (no matrix instructions exist for
         # f32 operands in the vocabulary): priced against the part's published vector fp32 rate
-        "roofline": {"bound": "valu_fp32", "achieved": tf, "peak": 157.3, "unit": "TFLOP/s", "frac": tf / 157.3,
-                     "traffic": None, "traffic_source": "not profiled (plumbing config)", "kernel": plan.kernel_name(0),
-                     "algorithmic_flops_per_launch": flops},
+        "roofline": dict(_roofline("matmul_f32", "valu_fp32", tf, 157.3, "TFLOP/s", plan.kernel_name(0)),
+                         algorithmic_flops_per_launch=flops),
     }
     rec.update(stats)
     if cpu:

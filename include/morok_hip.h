@@ -474,7 +474,12 @@ int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, cons
  * (x.matmul(w)[:, :F]).silu() * x.matmul(w)[:, F:] computes (Tensor::matmul, tensor/src/matmul.rs:82-110;
  * Tensor::silu / swish, tensor/src/activation.rs:309-318; the products rounded to bf16 first, then
  * x * sigmoid(x) * y in f32 and one rounding), with the gate applied in the product kernel's
- * epilogue so that the [M, 2F] product is never written.  F and K multiples of 8, K > 0;
+ * epilogue so that the [M, 2F] product is never written.  The epilogue evaluates sigmoid(x) as
+ * rcp(1 + exp2(-x log2 e)) with the hardware reciprocal (1 ulp in f32) where the separate
+ * elementwise kernel divides exactly, so about 2 % of the results differ from the unfused
+ * sequence by one bf16 ulp: fusing changes output bits within that bound.  No test of the
+ * reference covers the gated product (parity unpinned by reference tests; pinned against
+ * float64 and the oracle within 2e-2).  F and K multiples of 8, K > 0;
  * INVALID_ARGUMENT otherwise.  Builtin Program kind "gemm_bf16_swiglu", params {M, F, K},
  * buffers {c, a, w}. */
 int mrk_hip_gemm_bf16_swiglu(int device_id, const void* a, const void* w, void* c, int64_t m, int64_t f, int64_t k);
@@ -642,6 +647,10 @@ double mrk_hip_tensor_last_elapsed_ms(void);
  * Intermediates share blocks by liveness; MOROK_NO_MEMORY_PLANNER=1 turns that off. */
 size_t mrk_hip_tensor_last_buffers_reused(void);
 size_t mrk_hip_tensor_last_memory_saved(void);
+/* Device bytes the intermediates of that plan occupy: the planner's pool after reuse, or one
+ * block per intermediate with the planner off (MemoryPlannerResult::memory_planned,
+ * tensor/src/memory_planner.rs:84-96). */
+size_t mrk_hip_tensor_last_intermediate_bytes(void);
 /* With MOROK_BEAM=<width> in the environment, realize / prepare searches the choices of every
  * generated elementwise and reduce kernel of at least 65536 elements of work as well
  * (tensor/src/realize.rs:1190-1242, schedule/src/optimizer/beam.rs:36-120): UPCAST then LOCAL for

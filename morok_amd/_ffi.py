@@ -237,6 +237,7 @@ _SIGS = {
     "mrk_hip_tensor_last_elapsed_ms": (C.c_double, []),
     "mrk_hip_tensor_last_buffers_reused": (C.c_size_t, []),
     "mrk_hip_tensor_last_memory_saved": (C.c_size_t, []),
+    "mrk_hip_tensor_last_intermediate_bytes": (C.c_size_t, []),
     "mrk_hip_tensor_last_beam_candidates": (C.c_size_t, []),
     "mrk_hip_tensor_last_beam_cache_hits": (C.c_size_t, []),
 }

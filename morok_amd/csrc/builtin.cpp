@@ -176,7 +176,7 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
     if (k == "flash_fwd_bf16") {
         MRK_TRY(need(6));
         if (p[0] < 0 || p[1] < 0 || p[2] <= 0 || (p[3] != 256 && p[3] != 128 && p[3] != 64))
-            return fail(kInvalidArgument, "flash_fwd_bf16: bad shape (params BH, Sq, Sk, D = 128 or 64, causal, scale bits)");
+            return fail(kInvalidArgument, "flash_fwd_bf16: bad shape (params BH, Sq, Sk, D = 256, 128 or 64, causal, scale bits)");
         std::string name = "flash_fwd_bf16_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]) + (p[3] != 128 ? "_d" + std::to_string(p[3]) : "");
         out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
                                       [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
@@ -193,7 +193,7 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
         // buffers (4), then (batch, head, row) element strides of q k v o (12)
         MRK_TRY(need(23));
         if (p[0] < 0 || p[1] < 0 || p[2] < 0 || p[3] <= 0 || (p[4] != 256 && p[4] != 128 && p[4] != 64))
-            return fail(kInvalidArgument, "flash_fwd_bf16_strided: bad shape (params B, H, Sq, Sk, D = 128 or 64, causal, scale bits, 4 offsets, 12 strides)");
+            return fail(kInvalidArgument, "flash_fwd_bf16_strided: bad shape (params B, H, Sq, Sk, D = 256, 128 or 64, causal, scale bits, 4 offsets, 12 strides)");
         for (int i = 7; i < 23; i++)
             if (p[i] < 0 || p[i] % 8) return fail(kInvalidArgument, "flash_fwd_bf16_strided: offsets and strides must be non-negative multiples of 8 elements");
         std::string name = "flash_fwd_bf16_strided_" + std::to_string(p[0] * p[1]) + "_" + std::to_string(p[2]) + "_" + std::to_string(p[3]) + (p[4] != 128 ? "_d" + std::to_string(p[4]) : "");

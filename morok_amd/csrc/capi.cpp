@@ -1351,6 +1351,7 @@ size_t mrk_hip_tensor_last_cached_count(void) { return last_realize_stats().cach
 double mrk_hip_tensor_last_elapsed_ms(void) { return last_realize_stats().elapsed_ms; }
 size_t mrk_hip_tensor_last_buffers_reused(void) { return last_realize_stats().buffers_reused; }
 size_t mrk_hip_tensor_last_memory_saved(void) { return last_realize_stats().memory_saved; }
+size_t mrk_hip_tensor_last_intermediate_bytes(void) { return last_realize_stats().intermediate_bytes; }
 size_t mrk_hip_tensor_last_beam_candidates(void) { return last_realize_stats().beam_candidates; }
 size_t mrk_hip_tensor_last_beam_cache_hits(void) { return last_realize_stats().beam_cache_hits; }
 

@@ -71,7 +71,7 @@ int launch_copy(void* stream, const void* in, void* out, size_t bytes);
 
 
 // MFMA-only calibration kernel: `workgroups` workgroups of four waves, each wave issuing
-// k_steps x 64 v_mfma_f32_32x32x16_bf16 from registers (the instruction stream of one
+// k_steps x 128 v_mfma_f32_16x16x32_bf16 from registers (the instruction stream of one
 // 256 x 256 x 64*k_steps GEMM tile without its memory traffic): 2 * 256 * 256 * 64 * k_steps
 // flops per workgroup.  `out` (>= 4 bytes) is never written in practice.
 // random_operands: 0 = smooth small operand values, 1 = hashed values in [-1.7, 1.7) like a product of

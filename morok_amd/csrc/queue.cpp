@@ -14,12 +14,12 @@ HardwareQueue::~HardwareQueue() {
     if (stream_) {
         ffi::set_device(device_id_);
         ffi::stream_synchronize(stream_);
-        retire(true);
+        retire(true, /*after_synchronize=*/true);
         ffi::stream_destroy(stream_);
     }
 }
 
-void HardwareQueue::retire(bool all) {
+void HardwareQueue::retire(bool all, bool after_synchronize) {
     while (!in_flight_.empty()) {
         InFlight& f = in_flight_.front();
         if (!all && f.done && ffi::event_query(f.done) != 0) {  // batches complete in order
@@ -28,7 +28,8 @@ void HardwareQueue::retire(bool all) {
         }
         // the blocks may return to the allocator's cache now: device-stream work queued from
         // here on starts after this batch (a no-op when the event has already fired)
-        if (f.done && device_stream_) ffi::stream_wait_event(device_stream_, f.done);
+        // (nothing to order after a full synchronize of the queue's stream: every batch has finished)
+        if (f.done && device_stream_ && !after_synchronize) ffi::stream_wait_event(device_stream_, f.done);
         f.batch.clear();
         if (f.done) ffi::event_destroy(f.done);
         if (f.ready) ffi::event_destroy(f.ready);
@@ -41,7 +42,8 @@ int HardwareQueue::init() {
     MRK_HIP(ffi::stream_create(&stream_), "hipStreamCreate");
     std::shared_ptr<Device> dev;
     MRK_TRY(DeviceFactoryRegistry::global().device("HIP", device_id_, &dev));
-    device_stream_ = dev->allocator->stream();
+    device_allocator_ = dev->allocator;  // keeps the stream below alive for as long as this queue exists
+    device_stream_ = device_allocator_->stream();
     return kOk;
 }
 

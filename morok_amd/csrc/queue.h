@@ -73,11 +73,12 @@ class HardwareQueue {
     };
     // drops the batches whose completion event has fired (all of them when `all`, after the
     // caller has synchronized the stream)
-    void retire(bool all);
+    void retire(bool all, bool after_synchronize = false);
     int issue(std::vector<Command>& batch, uint64_t wait_timeout_ms);
     int device_id_;
     bool copy_queue_;
     ffi::Stream stream_ = nullptr;
+    std::shared_ptr<Allocator> device_allocator_;  // owner of device_stream_
     ffi::Stream device_stream_ = nullptr;  // the allocator's stream of this device
     std::vector<Command> cmds_;
     std::deque<InFlight> in_flight_;

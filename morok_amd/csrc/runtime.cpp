@@ -8,6 +8,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <functional>
+#include <set>
 #include <thread>
 
 #include "schedule.h"
@@ -164,6 +165,22 @@ int ExecutionPlan::plan_memory() {
 
 int ExecutionPlan::build() {
     if (plan_memory_ && !memory_planned_ && !outputs_.empty()) MRK_TRY(plan_memory());
+    if (!memory_planned_ && !census_done_) {
+        census_done_ = true;
+        // without the planner every intermediate keeps a block of its own: the same census
+        // (not yet allocated, not an output, whole, device memory), sizes rounded the same way
+        mem_stats_.memory_planned = 0;
+        std::vector<bool> used(buffers_.size(), false);
+        for (const PreparedKernel& pk : kernels_)
+            for (size_t i : pk.buffer_indices) used[i] = true;
+        std::set<const Buffer*> counted;
+        for (size_t i = 0; i < buffers_.size(); i++) {
+            const Buffer& b = *buffers_[i];
+            const bool is_output = std::find(outputs_.begin(), outputs_.end(), i) != outputs_.end();
+            if (used[i] && !b.is_allocated() && !is_output && b.is_whole() && !b.options().cpu_accessible && counted.insert(&b).second)
+                mem_stats_.memory_planned += (b.size() + 0xfff) / 0x1000 * 0x1000;
+        }
+    }
     for (auto& b : buffers_) MRK_TRY(b->ensure_allocated());  // tensor/src/realize.rs:974-981
     for (auto& pk : kernels_) {
         pk.buffer_ptrs.clear();

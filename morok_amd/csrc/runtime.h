@@ -72,7 +72,7 @@ struct MemoryPlanStats {
     size_t planned = 0;         // intermediates that took part
     size_t buffers_reused = 0;  // of those, how many were given an already used block
     size_t memory_saved = 0;    // bytes not allocated thanks to reuse
-    size_t memory_planned = 0;  // bytes the planned intermediates occupy after reuse
+    size_t memory_planned = 0;  // bytes the intermediates occupy (after reuse when the planner ran; one block each otherwise)
 };
 
 class ExecutionPlan {
@@ -124,7 +124,7 @@ class ExecutionPlan {
     ffi::GraphExec graph_exec_ = nullptr;
     int device_id_;
     bool built_ = false;
-    bool plan_memory_ = false, memory_planned_ = false;
+    bool plan_memory_ = false, memory_planned_ = false, census_done_ = false;
     MemoryPlanStats mem_stats_;
     std::vector<PreparedKernel> kernels_;
     std::vector<std::shared_ptr<Buffer>> buffers_;

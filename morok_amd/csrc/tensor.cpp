@@ -1400,7 +1400,10 @@ struct Scheduler {
     // [K, N], or (where nt_ok says the shape has a kernel for it) the [N, K] data behind a transpose.
     int weight_operand(TensorNode* mm, bool nt_ok, std::shared_ptr<Buffer>* buf, bool* nt) {
         *nt = false;
-        TensorNode* wt = nt_ok ? transposed_weight(mm) : nullptr;
+        // the B^T kernels have no any-alignment fallback: the first operand (materialised by the
+        // caller; the output is always a fresh buffer) must start on a 16-byte boundary as well
+        const std::shared_ptr<Buffer>& ab = mm->hint_inputs[0]->buffer;
+        TensorNode* wt = nt_ok && ab && ab->offset() % 16 == 0 ? transposed_weight(mm) : nullptr;
         if (wt) {
             MRK_TRY(materialize(wt));
             if (wt->buffer->offset() % 16 == 0) {
@@ -2647,6 +2650,7 @@ int prepare_locked(const TensorRef& root, std::unique_ptr<ExecutionPlan>* out, s
     if (kept) kept->insert(kept->end(), s.produced_host.begin(), s.produced_host.end());
     s.stats.buffers_reused = s.plan->memory_plan().buffers_reused;
     s.stats.memory_saved = s.plan->memory_plan().memory_saved;
+    s.stats.intermediate_bytes = s.plan->memory_plan().memory_planned;
     s.stats.elapsed_ms = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
     g_stats = s.stats;
     *out = std::move(s.plan);

@@ -77,6 +77,7 @@ struct RealizeStats {
     size_t cached_kernels = 0;
     size_t buffers_reused = 0;  // memory planner (tensor/src/memory_planner.rs:84-96)
     size_t memory_saved = 0;
+    size_t intermediate_bytes = 0;  // device bytes the plan's intermediates occupy
     size_t beam_candidates = 0;  // generated-kernel candidates compiled and timed (MOROK_BEAM)
     size_t beam_cache_hits = 0;  // generated kernels whose choices came from the on-disk cache
     double elapsed_ms = 0.0;

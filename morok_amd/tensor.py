@@ -51,6 +51,12 @@ def last_memory_plan():
     return lib.mrk_hip_tensor_last_buffers_reused(), lib.mrk_hip_tensor_last_memory_saved()
 
 
+def last_intermediate_bytes():
+    """Device bytes the intermediates of the last realize / prepare occupy (the planner's pool after
+    reuse, or one block per intermediate with MOROK_NO_MEMORY_PLANNER=1)."""
+    return lib.mrk_hip_tensor_last_intermediate_bytes()
+
+
 def last_beam_search():
     """(candidates compiled and timed, kernels answered by the disk cache) for the generated
     elementwise / reduce kernels of the last realize / prepare under MOROK_BEAM."""

@@ -84,3 +84,37 @@ def test_decoder_block_full_size_properties(dev):
     cfg1 = dict(cfg, batch=1)
     _, out4, _ = run_block(cfg1, tok[: cfg["seq"]], w)
     assert np.array_equal(out4.to_numpy(), a4[0])
+
+
+def test_memory_planner_on_and_off_give_the_same_bits_in_less_memory(dev, oracle, monkeypatch):
+    """tensor/src/memory_planner.rs:1-45 on the device: the decoder block with the planner
+    (intermediates share blocks by liveness) and without it (MOROK_NO_MEMORY_PLANNER=1, every
+    intermediate keeps a block of its own) must give identical bits, the planned run must reuse
+    blocks and hold strictly fewer intermediate bytes, and both must match the oracle."""
+    from morok_amd import decoder, synth, tensor
+
+    cfg = dict(batch=1, seq=192, hidden=512, heads=4, ffn=1280, vocab=777, eps=1e-6)
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], cfg["vocab"], seed=3)
+    tok = synth.randint((cfg["batch"] * cfg["seq"],), 3, 1, cfg["vocab"])
+    monkeypatch.delenv("MOROK_NO_MEMORY_PLANNER", raising=False)
+    blk, out, kernels = run_block(cfg, tok, w)
+    planned = out.to_numpy()
+    reused, saved = tensor.last_memory_plan()
+    planned_bytes = tensor.last_intermediate_bytes()
+    assert reused >= 2 and saved > 0 and planned_bytes > 0
+    monkeypatch.setenv("MOROK_NO_MEMORY_PLANNER", "1")
+    _, out2, kernels2 = run_block(cfg, tok, w)
+    unplanned = out2.to_numpy()
+    assert tensor.last_memory_plan() == (0, 0)
+    unplanned_bytes = tensor.last_intermediate_bytes()
+    assert kernels2 == kernels
+    assert np.array_equal(planned, unplanned)
+    assert planned_bytes < unplanned_bytes and unplanned_bytes - planned_bytes == saved
+    ref = oracle.decoder_block_bf16(tok, w, blk.cos_host, blk.sin_host, cfg["batch"], cfg["seq"], cfg["hidden"],
+                                    cfg["heads"], cfg["ffn"], cfg["eps"])
+    assert rel_err(planned, ref) <= 2e-2
+    # a block really is shared: run again with the planner and poison nothing -- the second
+    # planned run reuses the cached blocks of the first and still gives the same bits
+    monkeypatch.delenv("MOROK_NO_MEMORY_PLANNER")
+    _, out3, _ = run_block(cfg, tok, w)
+    assert np.array_equal(out3.to_numpy(), planned)

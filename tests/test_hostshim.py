@@ -698,6 +698,7 @@ def test_memory_planner_reuses_intermediates(T, shim, monkeypatch):
     base = shim.mrk_shim_bytes_in_use()
     out = blk.forward(tok).realize()
     reused, saved = tensor.last_memory_plan()
+    pool_bytes = tensor.last_intermediate_bytes()
     planned_bytes = shim.mrk_shim_bytes_in_use() - base
     assert reused >= 4 and saved >= 3 * 128 * 256 * 2
     del out
@@ -708,6 +709,7 @@ def test_memory_planner_reuses_intermediates(T, shim, monkeypatch):
     assert tensor.last_memory_plan() == (0, 0)
     unplanned_bytes = shim.mrk_shim_bytes_in_use() - base
     assert planned_bytes < unplanned_bytes and unplanned_bytes - planned_bytes >= saved // 2
+    assert tensor.last_intermediate_bytes() == pool_bytes + saved       # one block per intermediate
     del out2
 
 

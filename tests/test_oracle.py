@@ -508,6 +508,41 @@ def test_add_bf16_definition(oracle):
     assert synth.from_bf16(oracle.add_bf16(x, synth.to_bf16(np.float32([-1.0]))))[0] == np.float32(2.0 ** -7)
 
 
+def test_bf16_conversions_round_to_nearest_even_over_every_code(oracle):
+    """orc_bf16_to_f32 over all 65536 codes is the code shifted into the upper half of a
+    float32; orc_f32_to_bf16 is pinned without restating its bit trick: for every finite bf16
+    value v with successor w, everything strictly below the midpoint rounds to v, everything
+    above to w, and the midpoint itself to whichever of the two has an even mantissa (computed
+    in float64, where v, w and their midpoint are exact); NaN stays NaN, the largest float32
+    values round to infinity."""
+    codes = np.arange(65536, dtype=np.uint16)
+    f = np.empty(65536, np.float32)
+    oracle.lib.orc_bf16_to_f32(codes.ctypes.data_as(C.c_void_p), f.ctypes.data_as(C.c_void_p), C.c_long(65536))
+    assert np.array_equal(f.view(np.uint32), codes.astype(np.uint32) << 16)
+
+    def to_bf16(x):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty(x.shape, np.uint16)
+        oracle.lib.orc_f32_to_bf16(x.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p), C.c_long(x.size))
+        return out
+
+    assert np.array_equal(to_bf16(f[np.isfinite(f)]), codes[np.isfinite(f)])        # exact values keep their code
+    pos = codes[(codes < 0x7f7f)]                                                    # positive finite, successor finite
+    v, w = f[pos].astype(np.float64), f[pos + 1].astype(np.float64)
+    mid = (v + w) / 2                                                                # exact: one more mantissa bit
+    below = np.nextafter(mid.astype(np.float32), np.float32(0)).astype(np.float32)
+    above = np.nextafter(mid.astype(np.float32), np.float32(np.inf)).astype(np.float32)
+    assert np.array_equal(mid.astype(np.float32).astype(np.float64), mid)
+    assert np.array_equal(to_bf16(below), pos) and np.array_equal(to_bf16(above), pos + 1)
+    even = np.where(pos % 2 == 0, pos, pos + 1)
+    assert np.array_equal(to_bf16(mid.astype(np.float32)), even)
+    assert np.array_equal(to_bf16(-mid.astype(np.float32)), even | 0x8000)           # sign symmetric
+    big = np.float32([3.4e38, -3.4e38, np.inf, -np.inf])
+    assert np.array_equal(to_bf16(big), np.uint16([0x7f80, 0xff80, 0x7f80, 0xff80]))
+    nan = to_bf16(np.float32([np.nan]))[0]
+    assert (nan & 0x7f80) == 0x7f80 and (nan & 0x7f) != 0
+
+
 def test_heads_to_tokens_and_rope_heads_layout(oracle):
     """Index checks with distinct values per position: [B,H,S,D] -> [B*S, H*D] and the
     token-major -> head-major move of orc_rope_heads_bf16 (apply=0: a pure permutation;
