@@ -955,6 +955,9 @@ int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, con
     if (d != 256 && d != 128 && d != 64) return failf(kInvalidArgument, "flash_attn_fwd: head_dim %lld is not supported (256, 128 and 64 only)", (long long)d);
     if (sk == 0) return fail(kInvalidArgument, "flash_attn_fwd: empty key sequence (softmax over no keys is undefined)");
     if (!(scale > 0.0f)) return fail(kInvalidArgument, "flash_attn_fwd: scale must be positive");
+    if (!flash_fwd_rows_addressable(sq, d * 2, d) || !flash_fwd_rows_addressable(sk, d * 2, d))
+        return failf(kInvalidArgument, "flash_attn_fwd: the rows of one (batch, head) must end below 4 GiB (row offsets are 32-bit): "
+                                       "at head_dim %lld at most %lld rows", (long long)d, (long long)((0xffffffffLL - d * 2) / (d * 2) + 1));
     MRK_NONNULL(q);
     MRK_NONNULL(k);
     MRK_NONNULL(v);
@@ -989,6 +992,11 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
     }
     if (st[11] < d || (heads > 1 && st[10] == 0) || (batch > 1 && st[9] == 0))
         return fail(kInvalidArgument, "flash_attn_fwd_strided: output rows, heads and batches must not overlap");
+    const int64_t row_counts[4] = {sq, sk, sk, sq};
+    for (int t = 0; t < 4; t++)
+        if (st[3 * t + 2] > (1L << 30) || !flash_fwd_rows_addressable(row_counts[t], st[3 * t + 2] * 2, d))
+            return failf(kInvalidArgument, "flash_attn_fwd_strided: operand %d: the rows of one (batch, head) must end below 4 GiB "
+                                           "(row offsets are 32-bit)", t);
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");

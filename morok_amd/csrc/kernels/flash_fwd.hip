@@ -542,6 +542,8 @@ int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void
     if (BH <= 0 || Sq <= 0) return 0;
     if ((D != 256 && D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
     if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
+    // row offsets inside a head are formed in 32 bits (row * row bytes): the last row must end below 4 GiB
+    if (!flash_fwd_rows_addressable(Sq, D * 2, D) || !flash_fwd_rows_addressable(Sk, D * 2, D)) return (int)hipErrorInvalidValue;
     const long q_tiles = (Sq + kQT - 1) / kQT;
     const long units = causal ? (q_tiles + 1) / 2 : q_tiles;
     const long blocks = BH * units;
@@ -572,7 +574,7 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
         const long sb = strides[3 * t], sh = strides[3 * t + 1], sr = strides[3 * t + 2];
         if (sb < 0 || sh < 0 || sr < 0 || sb % 8 || sh % 8 || sr % 8) return (int)hipErrorInvalidValue;
         if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16) return (int)hipErrorInvalidValue;
-        if (sr > (1L << 30) || (rows[t] - 1) * sr * 2 + D * 2 > 0xffffffffL) return (int)hipErrorInvalidValue;
+        if (sr > (1L << 30) || !flash_fwd_rows_addressable(rows[t], sr * 2, D)) return (int)hipErrorInvalidValue;
         // the output must not alias itself: distinct rows, heads and batches at distinct places
         if (t == 3 && (sr < D || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
         dense = dense && sr == D && sh == rows[t] * D && sb == H * rows[t] * D;

@@ -49,7 +49,12 @@ int gemm_bf16_static_workspace_init(int device_id);
 size_t gemm_bf16_static_workspace_capacity();
 int launch_gemm_bf16_static_ws(void* stream, int device_id, const void* A, const void* B, void* C, long M, long N, long K);
 
-// O = softmax(Q K^T * scale [causal]) V; Q [BH,Sq,D], K/V [BH,Sk,D], O [BH,Sq,D] bf16, D = 128,
+// The attention kernels form the byte offset of a row inside one (batch, head) in 32 bits:
+// `rows` rows of `row_bytes` each (D elements of them used) must end below 4 GiB.
+inline bool flash_fwd_rows_addressable(long rows, long row_bytes, long D) {
+    return rows <= 0 || (rows - 1) * row_bytes + D * 2 <= 0xffffffffL;
+}
+// O = softmax(Q K^T * scale [causal]) V; Q [BH,Sq,D], K/V [BH,Sk,D], O [BH,Sq,D] bf16, D = 256, 128 or 64,
 // scale > 0.  Causal: key j visible to query i iff j <= i.
 int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
                           long D, float scale, int causal);

@@ -843,6 +843,26 @@ def test_ops_refuse_undersized_buffers(dev, shim):
     assert shim.mrk_shim_last_kernel() == b"softmax_f32"
 
 
+def test_flash_attention_refuses_heads_whose_rows_pass_4_gib(dev, shim):
+    """The attention kernels form row offsets inside one (batch, head) in 32 bits: a dense head
+    of 512-byte rows (head_dim 256) holds at most 2^23 - 1 rows, one of 256-byte rows 2^24 - 1; a strided
+    operand's last row must end below 4 GiB as well.  Refused before anything is launched."""
+    n = shim.mrk_shim_launches()
+    one = C.c_void_p(16)
+    rows = 1 << 23
+    assert shim.mrk_hip_flash_attn_fwd_bf16(0, one, one, one, one, 1, 1, 128, rows, 256, C.c_float(1.0), 0) == 11
+    assert b"4 GiB" in shim.mrk_hip_last_error()
+    assert shim.mrk_hip_flash_attn_fwd_bf16(0, one, one, one, one, 1, 1, rows, 128, 256, C.c_float(1.0), 0) == 11
+    assert shim.mrk_hip_flash_attn_fwd_bf16(0, one, one, one, one, 1, 1, 128, rows - 1, 256, C.c_float(1.0), 0) == 0
+    assert shim.mrk_hip_flash_attn_fwd_bf16(0, one, one, one, one, 1, 1, 128, rows, 128, C.c_float(1.0), 0) == 0
+    st = (C.c_int64 * 12)(*([0, 0, 128] * 4))
+    st[5] = 1 << 20                                   # key rows 2 MiB apart: 4096 of them pass 4 GiB
+    assert shim.mrk_hip_flash_attn_fwd_bf16_strided(0, one, one, one, one, 1, 1, 128, 4096, 128, C.c_float(1.0), 0, st) == 11
+    assert b"operand 1" in shim.mrk_hip_last_error()
+    assert shim.mrk_hip_flash_attn_fwd_bf16_strided(0, one, one, one, one, 1, 1, 128, 2048, 128, C.c_float(1.0), 0, st) == 0
+    assert shim.mrk_shim_launches() == n + 3
+
+
 def test_tensor_from_buffer_view_alignment(T, dev):
     b = dev.buffer(1024).ensure_allocated()
     t = T.Tensor.from_buffer(b.view(64, 256), (64,), uop.F32)
