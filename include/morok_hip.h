@@ -504,6 +504,25 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
                                         int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal,
                                         const int64_t* strides);
 
+/* The same attention with attn_mask and / or softcap inside the fused kernel
+ * (Tensor::scaled_dot_product_attention, tensor/src/transformer.rs:112-132), in the reference's
+ * order: scale, causal where(-inf), mask, softcap, softmax.  `strides` as in the call above, or
+ * NULL for dense [batch, heads, rows, d] operands.  mask_kind 0: none (mask, mask_strides unused);
+ * 1: Bool, one byte per element, nonzero = attend, false adds -inf (transformer.rs:114-121);
+ * 2: additive bf16 (transformer.rs:122-124).  The mask is a [batch, heads, sq, sk] view with
+ * contiguous keys; mask_strides holds its element strides per batch, head and query row (0 =
+ * broadcast over that axis), each a multiple of 4, and sk must be a multiple of 4 when a mask is
+ * given.  softcap 0: none; > 0: scores become softcap * tanh(score / softcap) AFTER the masks
+ * (transformer.rs:128-132), so a masked score (causal ones included) becomes -softcap and still
+ * takes part in the softmax, exactly as the reference's graph computes it; the kernel then visits
+ * every key tile.  A row whose keys are all masked out (no softcap) is NaN, as softmax over -inf
+ * only is.  Without mask and softcap this is mrk_hip_flash_attn_fwd_bf16_strided.
+ * Builtin Program kind "flash_fwd_bf16_ext" (29 params, buffers {o, q, k, v, mask}). */
+int mrk_hip_flash_attn_fwd_bf16_ex(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
+                                   int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal,
+                                   const int64_t* strides, const void* mask, int mask_kind, const int64_t* mask_strides,
+                                   float softcap);
+
 /* =====================================================================================
  * Synthetic inputs for benchmarks (no counterpart in the reference, whose tensor API has no
  * RNG, tensor/src/nn/mod.rs:304): counter-based SplitMix64 values written on the device.

@@ -157,6 +157,9 @@ _SIGS = {
     "mrk_hip_flash_attn_fwd_bf16_strided": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
                                                       C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_int,
                                                       C.POINTER(C.c_int64)]),
+    "mrk_hip_flash_attn_fwd_bf16_ex": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                                 C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_int,
+                                                 C.POINTER(C.c_int64), C.c_void_p, C.c_int, C.POINTER(C.c_int64), C.c_float]),
     "mrk_hip_fill": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_uint64, C.c_uint64, C.c_float,
                                C.c_float]),
     "mrk_hip_mfma_ceiling": (C.c_int, [C.c_int, C.c_void_p, C.c_int64, C.c_int64, C.c_int]),

@@ -1005,6 +1005,56 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
     return kOk;
 }
 
+int mrk_hip_flash_attn_fwd_bf16_ex(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch, int64_t heads,
+                                   int64_t sq, int64_t sk, int64_t d, float scale, int causal, const int64_t* strides, const void* mask,
+                                   int mask_kind, const int64_t* mask_strides, float softcap) {
+    if (batch < 0 || heads < 0 || sq < 0 || sk < 0) return fail(kInvalidArgument, "flash_attn_fwd_ex: negative shape");
+    if (mask_kind < 0 || mask_kind > 2) return fail(kInvalidArgument, "flash_attn_fwd_ex: mask_kind must be 0 (none), 1 (Bool bytes) or 2 (additive bf16)");
+    if (!(softcap >= 0.0f)) return fail(kInvalidArgument, "flash_attn_fwd_ex: softcap must be 0 (none) or positive");
+    if (batch == 0 || heads == 0 || sq == 0) return kOk;
+    if (d != 256 && d != 128 && d != 64) return failf(kInvalidArgument, "flash_attn_fwd_ex: head_dim %lld is not supported (256, 128 and 64 only)", (long long)d);
+    if (sk == 0) return fail(kInvalidArgument, "flash_attn_fwd_ex: empty key sequence (softmax over no keys is undefined)");
+    if (!(scale > 0.0f)) return fail(kInvalidArgument, "flash_attn_fwd_ex: scale must be positive");
+    MRK_NONNULL(q);
+    MRK_NONNULL(k);
+    MRK_NONNULL(v);
+    MRK_NONNULL(o);
+    long st[12];
+    const int64_t row_counts[4] = {sq, sk, sk, sq};
+    for (int t = 0; t < 4; t++) {  // no strides: dense [batch, heads, rows, d]
+        st[3 * t] = strides ? strides[3 * t] : heads * row_counts[t] * d;
+        st[3 * t + 1] = strides ? strides[3 * t + 1] : row_counts[t] * d;
+        st[3 * t + 2] = strides ? strides[3 * t + 2] : d;
+    }
+    for (int i = 0; i < 12; i++)
+        if (st[i] < 0 || st[i] % 8)
+            return failf(kInvalidArgument, "flash_attn_fwd_ex: stride %d (%ld) must be a non-negative multiple of 8 elements", i, st[i]);
+    if (st[11] < d || (heads > 1 && st[10] == 0) || (batch > 1 && st[9] == 0))
+        return fail(kInvalidArgument, "flash_attn_fwd_ex: output rows, heads and batches must not overlap");
+    for (int t = 0; t < 4; t++)
+        if (st[3 * t + 2] > (1L << 30) || !flash_fwd_rows_addressable(row_counts[t], st[3 * t + 2] * 2, d))
+            return failf(kInvalidArgument, "flash_attn_fwd_ex: operand %d: the rows of one (batch, head) must end below 4 GiB "
+                                           "(row offsets are 32-bit)", t);
+    long mst[3] = {0, 0, 0};
+    if (mask_kind != 0) {
+        MRK_NONNULL(mask);
+        MRK_NONNULL(mask_strides);
+        if (sk % 4) return failf(kInvalidArgument, "flash_attn_fwd_ex: with a mask the key count (%lld) must be a multiple of 4", (long long)sk);
+        if (reinterpret_cast<uintptr_t>(mask) % (mask_kind == 2 ? 8 : 4)) return fail(kInvalidArgument, "flash_attn_fwd_ex: the mask must start on a multiple of 4 elements");
+        for (int i = 0; i < 3; i++) {
+            if (mask_strides[i] < 0 || mask_strides[i] % 4)
+                return failf(kInvalidArgument, "flash_attn_fwd_ex: mask stride %d (%lld) must be a non-negative multiple of 4 elements", i, (long long)mask_strides[i]);
+            mst[i] = static_cast<long>(mask_strides[i]);
+        }
+    }
+    std::shared_ptr<Device> dv;
+    MRK_TRY(get_device(device_id, &dv));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_flash_fwd_bf16_ext(dv->allocator->stream(), q, k, v, o, batch, heads, sq, sk, d, scale, causal ? 1 : 0, st, mask, mask_kind, mst, softcap),
+            "flash_attn_fwd_ex launch");
+    return kOk;
+}
+
 int mrk_hip_fill(int device_id, void* out, size_t n, int dtype, int mode, uint64_t seed, uint64_t tensor_id, float a,
                  float b) {
     if (n == 0) return kOk;

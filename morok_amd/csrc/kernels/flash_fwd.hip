@@ -7,8 +7,14 @@
 // tensor (tensor/src/test/unit/fusion.rs:90-104).  Causal rule as in the reference:
 // key j is visible to query i iff j <= i (tril(0) over [Sq, Sk], transformer.rs:103-109).
 //
-// Layout: Q [BH, Sq, D], K [BH, Sk, D], V [BH, Sk, D], O [BH, Sq, D], row-major, D = 128 or 64
+// Layout: Q [BH, Sq, D], K [BH, Sk, D], V [BH, Sk, D], O [BH, Sq, D], row-major, D = 256, 128 or 64
 // (one instantiation of the same body per head dim; the comments below give the D = 128 numbers).
+//
+// attn_mask and softcap (transformer.rs:112-132) run in instantiations of their own
+// (flash_fwd_ext_*), in the reference's order: scale, causal where(-inf), mask (Bool: true =
+// attend, else -inf added; float: added), then cap * tanh(score / cap).  The reference caps
+// after masking, so under a softcap a masked score becomes -cap instead of -inf and still takes
+// part in the softmax: those kernels visit every key tile and apply the causal rule per element.
 //
 // Work split: one workgroup = 128 queries of one (batch, head); 4 waves x 32 queries.
 // K and V tiles of 64 keys travel global -> LDS directly (global_load_lds), two stages.
@@ -62,16 +68,33 @@ struct FlashLayout {
     int heads;
 };
 
+// attn_mask / softcap of the extended kernels.  The mask is a [batch, head, query, key] view
+// with contiguous keys: element strides per batch, head and query row (0 = broadcast).
+struct FlashExt {
+    const void* mask;
+    long long batch, head, row;
+    float cap;        // softcap in score units (> 0 when the kernel applies one)
+    int causal_elem;  // apply the causal rule per element while every key tile is visited
+};
+
 // kD: head dim, 128 or 64.  Rows of K and V are kD * 2 bytes in LDS (256 or 128): with 256-byte
 // rows one row spans all 64 banks and the swizzles spread 16 consecutive rows over the 16-byte
 // chunks; with 128-byte rows two consecutive rows span the banks, so the K swizzle uses
 // (row >> 1) & 7 over the 8 chunks of a row and the V granule swizzle (row & 3 over 32-byte
 // granules) needs no change.
-template <int kD, bool kStrided>
+// kMask: 0 none, 1 Bool (one byte per element, nonzero = attend), 2 additive bf16.  kCap: softcap.
+template <int kD, bool kStrided, int kMask = 0, bool kCap = false>
 __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,
                                                const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH, int Sq, int Sk,
-                                               float scale_log2e, int causal, int q_tiles, int units, const FlashLayout& lay) {
+                                               float scale_log2e, int causal, int q_tiles, int units, const FlashLayout& lay,
+                                               const FlashExt& ext = FlashExt{}) {
     static_assert(kD == 256 || kD == 128 || kD == 64, "head dims with an instantiation: 256, 128 and 64");
+    static_assert(kStrided || (kMask == 0 && !kCap), "the extended kernels take their operands as views");
+    // The extended kernels turn every score into its final value in exp2 units (scale, masks,
+    // softcap, log2 e) as soon as the score product has drained; from there on the online softmax
+    // is the plain kernel's with a scale of one.
+    constexpr bool kExt = kMask != 0 || kCap;
+    const float sc = kExt ? 1.0f : scale_log2e;
     constexpr int kRow = kD * 2;          // bytes per K/V row in LDS: 256 (128)
     constexpr int kTile = kKT * kRow;     // 16 KB (8 KB)
     constexpr int kDS = kD / 16;          // 16-deep steps of the score product: 8 (4)
@@ -104,8 +127,11 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     const __bf16 *Qh, *Kh_, *Vh_;
     __bf16* Oh;
     unsigned q_row, k_row, v_row, o_row;  // bytes between consecutive rows
+    const char* mask_row = nullptr;  // the mask of this (batch, head)
     if constexpr (kStrided) {
         const int bb = bh / lay.heads, hh = bh - bb * lay.heads;
+        if constexpr (kMask != 0)
+            mask_row = static_cast<const char*>(ext.mask) + (bb * ext.batch + hh * ext.head) * (kMask == 2 ? 2 : 1);
         Qh = Q + bb * lay.q.batch + hh * lay.q.head;
         Kh_ = K + bb * lay.k.batch + hh * lay.k.head;
         Vh_ = V + bb * lay.v.batch + hh * lay.v.head;
@@ -213,7 +239,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         for (int e = 0; e < 16; e++) o[db][e] = 0.0f;
     float m_run = -INFINITY;  // running max of raw scores (before scale)
     float l_run = 0.0f;       // this lane's partial row sum
-    const float lazy_thresh = 8.0f / scale_log2e;  // kLazy = 8: probabilities stay below 256
+    const float lazy_thresh = 8.0f / sc;  // kLazy = 8: probabilities stay below 256
 
     // lane-constant LDS offsets
     // K fragment (A operand): row = kb*32 + l%32, logical chunk 2*ds + l/32
@@ -232,6 +258,51 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     if (causal && qw0 / kKT < first_masked) first_masked = qw0 / kKT;
     const int qidx = qw0 + lq;
     const int lim = causal ? (qidx < Sk - 1 ? qidx : Sk - 1) : Sk - 1;  // last visible key
+    // ---- extended kernels: mask values of a tile and the score transform
+    // A lane's 32 scores of a tile are eight groups of four consecutive keys (block kb, group g:
+    // keys key0 + kb*32 + 8*g + 4*(l/32) + 0..3); the mask values of a group are one 8-byte
+    // (bf16) or 4-byte (Bool) load.  Groups past the last key re-read the last group (Sk is a
+    // multiple of 4 here) and are masked as non-existent keys afterwards.
+    using MaskGroup = std::conditional_t<kMask == 2, bf16x4, unsigned>;
+    struct MaskTile {
+        MaskGroup g[2][4];
+    };
+    const char* mask_q = nullptr;  // this lane's query row of the mask (of this pass)
+    if constexpr (kMask != 0) mask_q = mask_row + (long long)(qidx < Sq ? qidx : Sq - 1) * ext.row * (kMask == 2 ? 2 : 1);
+    auto load_mask = [&](int key0, MaskTile& mt) {
+        if constexpr (kMask != 0) {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    int key = key0 + kb * 32 + 8 * g + 4 * lg;
+                    key = key < Sk - 4 ? key : Sk - 4;
+                    mt.g[kb][g] = *reinterpret_cast<const MaskGroup*>(mask_q + (long long)key * (kMask == 2 ? 2 : 1));
+                }
+        }
+    };
+    const int lim_causal = ext.causal_elem ? qidx : 0x7fffffff;  // reference mask: -inf before the softcap
+    constexpr float kLog2e = 1.4426950408889634f;
+    const float cap_out = kCap ? ext.cap * kLog2e : 0.0f;  // the cap in exp2 units
+    const float cap_in = kCap ? 2.0f / ext.cap : 0.0f;
+    // raw score (sum of q k) of key `key` -> final score in exp2 units
+    auto ext_score = [&](float s, int key, const MaskTile& mt, int kb, int e) -> float {
+        float t = s * scale_log2e;  // scaled score, in exp2 units for now
+        if (key > lim_causal) t = -INFINITY;
+        if constexpr (kMask == 1) {
+            if (((mt.g[kb][e >> 2] >> (8 * (e & 3))) & 0xffu) == 0) t = -INFINITY;
+        } else if constexpr (kMask == 2) {
+            t += (float)mt.g[kb][e >> 2][e & 3] * kLog2e;
+        }
+        if constexpr (kCap) {
+            // cap * tanh(x / cap) with tanh(y) = 1 - 2 / (exp(2 y) + 1) and x = t / log2 e, so
+            // exp(2 x / cap) = exp2(2 t / cap); x = -inf gives -cap, x = +inf gives cap
+            const float z = __builtin_amdgcn_exp2f(t * cap_in);
+            t = cap_out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(z + 1.0f));
+        }
+        if (key > Sk - 1) t = -INFINITY;  // keys that do not exist
+        return t;
+    };
 
     // S^T = K Q^T for one tile (K fragments fetched one d-step ahead of their MFMAs),
     // then the mask and the row maximum.  Register e of block kb is key
@@ -259,7 +330,15 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         }
     };
     auto mask_and_max = [&](f32x16 (&st)[2], int key0, bool mask) -> float {
-        if (mask) {
+        if constexpr (kExt) {
+            MaskTile mt;
+            load_mask(key0, mt);
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int e = 0; e < 16; e++)
+                    st[kb][e] = ext_score(st[kb][e], key0 + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3), mt, kb, e);
+        } else if (mask) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
@@ -293,7 +372,8 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         constexpr bool kLast = decltype(last_tile)::value;  // the wave's last tile: there is no S(j+1) to compute
         if (__builtin_amdgcn_ballot_w64(mx_cur > m_run + lazy_thresh) != 0) {
             const float m_new = fmaxf(m_run, mx_cur);
-            const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * scale_log2e);
+            // (a row with nothing visible yet keeps -inf: its empty accumulators are left as they are)
+            const float alpha = kExt && m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * sc);
             m_run = m_new;
             l_run *= alpha;
 #pragma unroll
@@ -306,7 +386,8 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         seq_v(g + 1);
         const char* sKn = smem + ((g + 1) & 1) * kTile;
         const char* sV = smem + 2 * kTile + (g & 1) * kTile;
-        const float mb = m_run * scale_log2e;
+        // (a row whose keys so far are all masked has m_run = -inf: its probabilities must come out as 0, not NaN)
+        const float mb = kExt && m_run == -INFINITY ? 0.0f : m_run * sc;
 
         // ---- phase A: S(j+1) = K(j+1) Q^T on the matrix pipe, P(j) = exp2(S(j)*c - m*c) on
         // the vector ALUs: each of the 16 (8; 32) MFMAs is followed by the exponentials of two (four; every second one by two)
@@ -345,8 +426,8 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
 #pragma unroll
                     for (int idx = (ds * 2 + kb) * 16 / kMfmaA; idx < (ds * 2 + kb + 1) * 16 / kMfmaA; idx++) {  // 0..15: score registers 2*idx, 2*idx+1
                         const int pk = idx >> 3, pe = (idx & 7) * 2;  // block, register inside the block
-                        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe], scale_log2e, -mb));
-                        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe + 1], scale_log2e, -mb));
+                        const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe], sc, -mb));
+                        const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(cur[pk][pe + 1], sc, -mb));
                         psum0 += p0;
                         psum1 += p1;
                         p[pe & 7] = p0;
@@ -365,6 +446,8 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         float mx0 = -INFINITY, mx1 = -INFINITY;
         {
             constexpr int kNB = 4 * kDB;  // MFMAs of this phase: 16 (8)
+            MaskTile mt;  // the next tile's mask values: requested here, used in the second half of the phase
+            if constexpr (kExt && !kLast) load_mask((j + 1) * kKT, mt);
             auto vfrag = [&](int n) {  // n = (kb*2 + t)*kDB + db
                 const int kbt = n / kDB, db = n % kDB;
                 const int off = (kbt * 16) * kRow + v_row_off + (((db * 2 + v_half) ^ v_rr) << 5);
@@ -386,7 +469,9 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
                     const int kb = (n - kNB / 2) / kSlotsPerKb, e0 = ((n - kNB / 2) % kSlotsPerKb) * kRegs;
 #pragma unroll
                     for (int e = e0; e < e0 + kRegs; e++) {
-                        if (decltype(mask_next)::value) {
+                        if constexpr (kExt) {
+                            nxt[kb][e] = ext_score(nxt[kb][e], key0n + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3), mt, kb, e);
+                        } else if (decltype(mask_next)::value) {
                             const int key = key0n + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3);
                             if (key > lim) nxt[kb][e] = -INFINITY;
                         }
@@ -421,7 +506,8 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         constexpr std::false_type more{};
         if constexpr (kD < 256) {
             const int nl = nmine - 1;  // iterations that have a next tile; the wave's last one is a body of its own
-            const int jm = first_masked - 1 < nl ? first_masked - 1 : nl;  // iterations whose next tile is unmasked
+            // iterations whose next tile is unmasked (none in the extended kernels: every tile is transformed)
+            const int jm = kExt ? 0 : (first_masked - 1 < nl ? first_masked - 1 : nl);
             for (; j + 1 < jm; j += 2) {
                 body(j, sa, mxa, sb, mxb, std::false_type{}, more);
                 body(j + 1, sb, mxb, sa, mxa, std::false_type{}, more);
@@ -449,7 +535,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         } else {
             // with 512-byte rows one more instantiation of the body would push the kernel over
             // its register budget: the last tile runs the ordinary body and its S(j+1) goes unused
-            const int jm = first_masked - 1 < nmine ? first_masked - 1 : nmine;
+            const int jm = kExt ? 0 : (first_masked - 1 < nmine ? first_masked - 1 : nmine);
             for (; j + 1 < jm; j += 2) {
                 body(j, sa, mxa, sb, mxb, std::false_type{}, more);
                 body(j + 1, sb, mxb, sa, mxa, std::false_type{}, more);
@@ -532,6 +618,31 @@ __global__ __launch_bounds__(256, 1) void flash_fwd_d256_strided(const __bf16* _
     flash_fwd_body<256, true>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, lay);
 }
 
+// attn_mask / softcap instantiations; operands always as views
+#define MRK_FLASH_EXT_KERNEL(NAME, D, WG, MASK, CAP)                                                                            \
+    __global__ __launch_bounds__(256, WG) void NAME(const __bf16* __restrict__ Q, const __bf16* __restrict__ K,                   \
+                                                    const __bf16* __restrict__ V, __bf16* __restrict__ O, int BH, int Sq, int Sk, \
+                                                    float scale_log2e, int causal, int q_tiles, int units, FlashLayout lay,       \
+                                                    FlashExt ext) {                                                               \
+        flash_fwd_body<D, true, MASK, CAP>(Q, K, V, O, BH, Sq, Sk, scale_log2e, causal, q_tiles, units, lay, ext);                \
+    }
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d128_bool, 128, 2, 1, false)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d128_add, 128, 2, 2, false)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d128_cap, 128, 2, 0, true)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d128_bool_cap, 128, 2, 1, true)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d128_add_cap, 128, 2, 2, true)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d64_bool, 64, 2, 1, false)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d64_add, 64, 2, 2, false)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d64_cap, 64, 2, 0, true)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d64_bool_cap, 64, 2, 1, true)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d64_add_cap, 64, 2, 2, true)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d256_bool, 256, 1, 1, false)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d256_add, 256, 1, 2, false)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d256_cap, 256, 1, 0, true)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d256_bool_cap, 256, 1, 1, true)
+MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d256_add_cap, 256, 1, 2, true)
+#undef MRK_FLASH_EXT_KERNEL
+
 }  // namespace mrk::dev
 
 namespace mrk {
@@ -598,6 +709,69 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
     kernel<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v),
         static_cast<__bf16*>(o), (int)BH, (int)Sq, (int)Sk, scale_log2e, causal, (int)q_tiles, (int)units, lay);
+    return (int)hipGetLastError();
+}
+
+int launch_flash_fwd_bf16_ext(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk,
+                              long D, float scale, int causal, const long* strides, const void* mask, int mask_kind,
+                              const long* mask_strides, float softcap) {
+    using namespace mrk::dev;
+    if (B < 0 || H < 0 || !strides) return (int)hipErrorInvalidValue;
+    if (mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && (!mask || !mask_strides)) || !(softcap >= 0.0f)) return (int)hipErrorInvalidValue;
+    if (mask_kind == 0 && !(softcap > 0.0f)) return launch_flash_fwd_bf16_strided(stream, q, k, v, o, B, H, Sq, Sk, D, scale, causal, strides);
+    const long BH = B * H;
+    if (BH == 0 || Sq <= 0) return 0;
+    if ((D != 256 && D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
+    if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
+    const void* ptrs[4] = {q, k, v, o};
+    const long rows[4] = {Sq, Sk, Sk, Sq};
+    for (int t = 0; t < 4; t++) {
+        const long sb = strides[3 * t], sh = strides[3 * t + 1], sr = strides[3 * t + 2];
+        if (sb < 0 || sh < 0 || sr < 0 || sb % 8 || sh % 8 || sr % 8) return (int)hipErrorInvalidValue;
+        if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16) return (int)hipErrorInvalidValue;
+        if (sr > (1L << 30) || !flash_fwd_rows_addressable(rows[t], sr * 2, D)) return (int)hipErrorInvalidValue;
+        if (t == 3 && (sr < D || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
+    }
+    FlashExt ext{};
+    if (mask_kind != 0) {
+        // a lane reads the mask in groups of four keys: rows, heads and batches start on multiples of
+        // four elements, and so does the end of a row
+        const long esize = mask_kind == 2 ? 2 : 1;
+        if (Sk % 4 || reinterpret_cast<uintptr_t>(mask) % (4 * esize)) return (int)hipErrorInvalidValue;
+        for (int i = 0; i < 3; i++)
+            if (mask_strides[i] < 0 || mask_strides[i] % 4) return (int)hipErrorInvalidValue;
+        ext.mask = mask;
+        ext.batch = mask_strides[0], ext.head = mask_strides[1], ext.row = mask_strides[2];
+    }
+    const bool cap = softcap > 0.0f;
+    ext.cap = softcap;
+    ext.causal_elem = causal ? 1 : 0;
+    // under a softcap a causally masked score becomes -cap and still counts: every key tile is visited
+    const int causal_tiles = causal && !cap;
+    const long q_tiles = (Sq + kQT - 1) / kQT;
+    const long units = causal_tiles ? (q_tiles + 1) / 2 : q_tiles;
+    const long blocks = BH * units;
+    if (blocks > 0x7fffffffL) return (int)hipErrorInvalidValue;
+    FlashLayout lay;
+    RowLayout* rl[4] = {&lay.q, &lay.k, &lay.v, &lay.o};
+    for (int t = 0; t < 4; t++) {
+        rl[t]->batch = strides[3 * t];
+        rl[t]->head = strides[3 * t + 1];
+        rl[t]->row_bytes = (unsigned)(strides[3 * t + 2] * 2);
+    }
+    lay.heads = (int)H;
+    (void)hipGetLastError();
+    const float scale_log2e = scale * 1.4426950408889634f;
+    using Kernel = void (*)(const __bf16*, const __bf16*, const __bf16*, __bf16*, int, int, int, float, int, int, int, FlashLayout, FlashExt);
+    // [head dim][mask kind][cap]
+    static const Kernel table[3][3][2] = {
+        {{nullptr, flash_fwd_ext_d64_cap}, {flash_fwd_ext_d64_bool, flash_fwd_ext_d64_bool_cap}, {flash_fwd_ext_d64_add, flash_fwd_ext_d64_add_cap}},
+        {{nullptr, flash_fwd_ext_d128_cap}, {flash_fwd_ext_d128_bool, flash_fwd_ext_d128_bool_cap}, {flash_fwd_ext_d128_add, flash_fwd_ext_d128_add_cap}},
+        {{nullptr, flash_fwd_ext_d256_cap}, {flash_fwd_ext_d256_bool, flash_fwd_ext_d256_bool_cap}, {flash_fwd_ext_d256_add, flash_fwd_ext_d256_add_cap}}};
+    const Kernel kernel = table[D == 64 ? 0 : D == 128 ? 1 : 2][mask_kind][cap ? 1 : 0];
+    kernel<<<(unsigned)blocks, 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const __bf16*>(q), static_cast<const __bf16*>(k), static_cast<const __bf16*>(v), static_cast<__bf16*>(o), (int)BH,
+        (int)Sq, (int)Sk, scale_log2e, causal_tiles, (int)q_tiles, (int)units, lay, ext);
     return (int)hipGetLastError();
 }
 

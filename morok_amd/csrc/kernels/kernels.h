@@ -65,6 +65,18 @@ int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void
 int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq,
                                   long Sk, long D, float scale, int causal, const long* strides);
 
+// The same attention with an attn_mask and / or a softcap (transformer.rs:112-132), operands as
+// views like the strided launcher.  mask_kind 0: none; 1: Bool, one byte per element, nonzero =
+// attend; 2: additive bf16.  mask_strides: element strides of the mask per batch, head and query
+// row (0 broadcasts; keys are contiguous), multiples of 4, and Sk a multiple of 4.  softcap 0:
+// none; else scores become softcap * tanh(score / softcap) after masking, so masked scores
+// (causal ones included) turn into -softcap and still take part, as in the reference.  A row
+// whose keys are all masked out (no softcap) comes out as NaN, as the reference's softmax does.
+// Without mask and softcap this is launch_flash_fwd_bf16_strided.
+int launch_flash_fwd_bf16_ext(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk,
+                              long D, float scale, int causal, const long* strides, const void* mask, int mask_kind,
+                              const long* mask_strides, float softcap);
+
 // Synthetic benchmark inputs. dtype 0 = f32, 1 = bf16; mode 0 = uniform [a, b), 1 = normal(0, a).
 int launch_fill(void* stream, void* out, size_t n, int dtype, int mode, unsigned long long seed,
                 unsigned long long tensor_id, float a, float b);

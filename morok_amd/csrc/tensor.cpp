@@ -609,7 +609,7 @@ Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& val
     // the next one that has (64, 128, 256): zero columns add exact zeros to every score, the
     // padded columns of V give zero outputs that are cut off again, and the scale stays that of
     // the real head dim.  Three padded copies instead of a materialised [Sq, Sk] score matrix.
-    if (nd == 4 && sdt == Scalar::BFloat16 && !attn_mask && !(softcap > 0.0) && head_dim > 0 && head_dim < 256 && head_dim != 64 &&
+    if (nd == 4 && sdt == Scalar::BFloat16 && head_dim > 0 && head_dim < 256 && head_dim != 64 &&
         head_dim != 128 && key.shape()[3] == head_dim && value.shape()[3] == head_dim && key.dtype() == sdt && value.dtype() == sdt &&
         n_->numel() > 0 && key.node()->numel() > 0) {
         const int64_t padded = head_dim < 64 ? 64 : head_dim < 128 ? 128 : 256;
@@ -618,7 +618,7 @@ Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& val
             zs[3] = padded - head_dim;
             return Tensor::cat({t, Tensor::full(zs, 0.0, sdt, t.node()->device_id)}, 3);
         };
-        Tensor out = pad(*this).scaled_dot_product_attention(pad(key), pad(value), scale_val, is_causal, nullptr, 0.0);
+        Tensor out = pad(*this).scaled_dot_product_attention(pad(key), pad(value), scale_val, is_causal, attn_mask, softcap);
         if (!out.valid()) return out;
         std::vector<int64_t> b0(4, 0), e0 = out.shape();
         e0[3] = head_dim;
@@ -653,11 +653,15 @@ Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& val
     }
     Tensor out = scores.softmax(-1).matmul(value);
     if (!out.valid()) return out;
-    if (attn_mask || softcap > 0.0) return out;  // the fused kernel covers neither: composed graph
+    // the fused kernel takes a Bool or an additive mask of the scores' own dtype; any other mask
+    // dtype changes the dtype of the scores themselves and stays the composed graph
+    if (attn_mask && attn_mask->dtype() != Scalar::Bool && attn_mask->dtype() != sdt) return out;
     out.node()->hint = HintKind::Sdpa;
     out.node()->hint_inputs = {n_, key.node(), value.node()};
+    if (attn_mask) out.node()->hint_inputs.push_back(attn_mask->node());
     out.node()->hint_scale = scale_val;
     out.node()->hint_causal = is_causal;
+    out.node()->hint_softcap = softcap > 0.0 ? softcap : 0.0;
     return out;
 }
 
@@ -1232,9 +1236,24 @@ struct Scheduler {
                 const TensorNode* q = n->hint_inputs[0].get();
                 const TensorNode* k = n->hint_inputs[1].get();
                 const TensorNode* v = n->hint_inputs[2].get();
-                return q->dtype == Scalar::BFloat16 && k->dtype == q->dtype && v->dtype == q->dtype &&
-                       q->shape.size() == 4 && (q->shape[3] == 256 || q->shape[3] == 128 || q->shape[3] == 64) && v->shape[3] == q->shape[3] && k->shape[2] > 0 &&
-                       k->shape[0] == q->shape[0] && k->shape[1] == q->shape[1] && q->numel() > 0;
+                if (!(q->dtype == Scalar::BFloat16 && k->dtype == q->dtype && v->dtype == q->dtype &&
+                      q->shape.size() == 4 && (q->shape[3] == 256 || q->shape[3] == 128 || q->shape[3] == 64) && v->shape[3] == q->shape[3] && k->shape[2] > 0 &&
+                      k->shape[0] == q->shape[0] && k->shape[1] == q->shape[1] && q->numel() > 0))
+                    return false;
+                if (n->hint_inputs.size() > 3) {
+                    // attn_mask inside the kernel: Bool or bf16, broadcastable to [B, H, Sq, Sk] with the
+                    // key axis in full, read in groups of four keys
+                    const TensorNode* m = n->hint_inputs[3].get();
+                    const int64_t full[4] = {q->shape[0], q->shape[1], q->shape[2], k->shape[2]};
+                    if ((m->dtype != Scalar::Bool && m->dtype != Scalar::BFloat16) || m->shape.empty() || m->shape.size() > 4 ||
+                        m->shape.back() != full[3] || full[3] % 4)
+                        return false;
+                    for (size_t i = 0; i < m->shape.size(); i++) {
+                        const int64_t want = full[4 - m->shape.size() + i];
+                        if (m->shape[i] != want && m->shape[i] != 1) return false;
+                    }
+                }
+                return true;
             }
             default: return false;
         }
@@ -1832,12 +1851,49 @@ struct Scheduler {
         }
         strides.insert(strides.end(), out_strides.begin(), out_strides.begin() + 3);
         dense = dense && out_strides == dense_strides(att->shape);
+        // attn_mask: read in place where it is a view of data in memory with contiguous keys whose
+        // offset and strides are multiples of four elements; else materialised in its own shape
+        const bool has_mask = att->hint_inputs.size() > 3;
+        int64_t mask_offset = 0, mask_strides[3] = {0, 0, 0};
+        std::shared_ptr<Buffer> mask_buf;
+        if (has_mask) {
+            TensorNode* m = att->hint_inputs[3].get();
+            const size_t mr = m->shape.size();
+            std::vector<int64_t> mst;
+            StridedView v;
+            bool ok = !m->buffer && strided_view(m, &v) && v.base != m && v.strides.size() == mr && v.offset % 4 == 0 &&
+                      (v.base->buffer || is_boundary_kind(v.base) || fusable(v.base)) && (m->shape.back() == 1 || v.strides.back() == 1);
+            if (ok)
+                for (size_t a = 0; a + 1 < mr; a++) ok = ok && (m->shape[a] == 1 || (v.strides[a] >= 0 && v.strides[a] % 4 == 0));
+            if (ok) {
+                MRK_TRY(materialize(v.base));
+                mask_buf = v.base->buffer;
+                mask_offset = v.offset;
+                mst = v.strides;
+            } else {
+                MRK_TRY(materialize(m));
+                mask_buf = m->buffer;
+                mst = dense_strides(m->shape);
+            }
+            for (size_t a = 0; a + 1 < mr; a++) mask_strides[4 - mr + a] = m->shape[a] == 1 ? 0 : mst[a];
+        }
         auto out = new_buffer(dst);
         bufs[0] = out;
         float scale = static_cast<float>(att->hint_scale);
         uint32_t bits;
         std::memcpy(&bits, &scale, 4);
-        if (dense) {
+        if (has_mask || att->hint_softcap > 0.0) {
+            float cap = static_cast<float>(att->hint_softcap);
+            uint32_t cap_bits;
+            std::memcpy(&cap_bits, &cap, 4);
+            const int64_t kind = !has_mask ? 0 : att->hint_inputs[3]->dtype == Scalar::Bool ? 1 : 2;
+            params = {B, H, Sq, Sk, D, att->hint_causal ? 1 : 0, static_cast<int64_t>(bits), att->hint_softcap > 0.0 ? static_cast<int64_t>(cap_bits) : 0,
+                      kind, offsets[0], offsets[1], offsets[2], 0, mask_offset};
+            params.insert(params.end(), strides.begin(), strides.end());
+            params.insert(params.end(), mask_strides, mask_strides + 3);
+            bufs.push_back(has_mask ? mask_buf : bufs[1]);
+            MRK_TRY(builtin("flash_fwd_bf16_ext", params, bufs));
+        } else if (dense) {
             MRK_TRY(builtin("flash_fwd_bf16", {B * H, Sq, Sk, D, att->hint_causal ? 1 : 0, static_cast<int64_t>(bits)}, bufs));
         } else {
             params = {B, H, Sq, Sk, D, att->hint_causal ? 1 : 0, static_cast<int64_t>(bits), offsets[0], offsets[1], offsets[2], 0};

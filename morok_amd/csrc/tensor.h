@@ -62,6 +62,7 @@ struct TensorNode {
     std::vector<TensorRef> hint_inputs;
     double hint_scale = 0.0;
     bool hint_causal = false;
+    double hint_softcap = 0.0;  // Sdpa: 0 = none; hint_inputs[3] is the attn_mask when there is one
 
     int64_t numel() const {
         int64_t n = 1;

@@ -104,6 +104,40 @@ def flash_attn_fwd_bf16_strided(q, k, v, o, batch, heads, sq, sk, d, scale, stri
                                                   scale, int(causal), arr))
 
 
+def flash_attn_fwd_bf16_ex(q, k, v, o, batch, heads, sq, sk, d, scale, causal=False, mask=None, mask_kind=0,
+                           mask_strides=(0, 0, 0), softcap=0.0, strides=None, device_id=0):
+    """The fused SDPA forward with attn_mask and / or softcap inside the kernel
+    (tensor/src/transformer.rs:112-132).  mask_kind 1: Bool bytes (nonzero = attend), 2: additive
+    bf16; mask_strides = element strides of the mask per batch, head and query row (0 broadcasts),
+    keys contiguous.  `strides`: as flash_attn_fwd_bf16_strided, or None for dense operands."""
+    if strides is None:
+        _need(q, batch * heads * sq * d * 2, "attention Q")
+        _need(o, batch * heads * sq * d * 2, "attention O")
+        _need(k, batch * heads * sk * d * 2, "attention K")
+        _need(v, batch * heads * sk * d * 2, "attention V")
+        arr = None
+    else:
+        strides = [int(x) for x in strides]
+        if len(strides) != 12:
+            raise ValueError("flash_attn_fwd_bf16_ex takes 12 strides")
+        for i, (b, rows, what) in enumerate(((q, sq, "attention Q"), (k, sk, "attention K"), (v, sk, "attention V"),
+                                             (o, sq, "attention O"))):
+            sb, sh, sr = strides[3 * i:3 * i + 3]
+            if batch and heads and rows:
+                _need(b, ((batch - 1) * sb + (heads - 1) * sh + (rows - 1) * sr + d) * 2, what)
+        arr = (C.c_int64 * 12)(*strides)
+    marr = None
+    if mask_kind:
+        if mask is None or len(mask_strides) != 3:
+            raise ValueError("flash_attn_fwd_bf16_ex: a mask kind needs a mask and 3 mask strides")
+        mb, mh, mr = (int(x) for x in mask_strides)
+        if batch and heads and sq:
+            _need(mask, ((batch - 1) * mb + (heads - 1) * mh + (sq - 1) * mr + sk) * (2 if mask_kind == 2 else 1), "attention mask")
+        marr = (C.c_int64 * 3)(mb, mh, mr)
+    check(lib.mrk_hip_flash_attn_fwd_bf16_ex(device_id, _p(q), _p(k), _p(v), _p(o), batch, heads, sq, sk, d, scale, int(causal),
+                                             arr, _p(mask) if mask_kind else None, int(mask_kind), marr, float(softcap)))
+
+
 def fill_normal(buf, n, sigma=1.0, seed=0, tensor_id=0, bf16=False, device_id=0):
     """Device-side synthetic normal(0, sigma) values (benchmark inputs)."""
     _need(buf, n * (2 if bf16 else 4), "fill")

@@ -316,7 +316,8 @@ class Tensor:
 
     def scaled_dot_product_attention(self, key, value, scale=None, is_causal=False, attn_mask=None, softcap=None):
         """transformer.rs:78-137.  attn_mask: Bool (True = attend) or additive, broadcastable to
-        [.., Sq, Sk]; softcap: cap * tanh(scores / cap).  Either of them selects the composed graph."""
+        [.., Sq, Sk]; softcap: cap * tanh(scores / cap), applied after the masks.  bf16 operands with a
+        Bool or bf16 mask run inside the fused attention kernel."""
         if attn_mask is None and not softcap:
             return self._new(lib.mrk_hip_tensor_sdpa, key._h, value._h, float(scale) if scale else 0.0, int(is_causal))
         return self._new(lib.mrk_hip_tensor_sdpa_ex, key._h, value._h, attn_mask._h if attn_mask is not None else None,

@@ -24,6 +24,7 @@
  *   orc_rope_*            pinned: the reference's three closed-form cases
  *   orc_embedding_*       pinned: the reference's row-gather cases (bit exact)
  *   orc_sdpa_*            pinned: causal row 0 == V[0], uniform-K running mean, S=1, float64 SDPA
+ *   orc_sdpa_bf16_ex      attn_mask / softcap: unpinned by reference tests; closed forms, identities with the causal path, float64
  *   orc_gemm_bf16         parity unpinned by reference tests (no bf16 matmul test upstream);
  *                         pinned by definition on bf16-rounded inputs vs float64, identity/ones cases
  *   orc_silu_mul_*, orc_decoder_block_bf16
@@ -275,6 +276,61 @@ void orc_sdpa_bf16(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O,
         float* s = (float*)malloc(sizeof(float) * (size_t)(Sk + D + 1));
         sdpa_bf16_head(Q + (size_t)bh * Sq * D, K + (size_t)bh * Sk * D, V + (size_t)bh * Sk * D,
                        O + (size_t)bh * Sq * D, Sq, Sk, D, scale, causal, policy, s, s + Sk);
+        free(s);
+    }
+}
+/* The same attention with attn_mask and softcap, in the order of tensor/src/transformer.rs:96-132
+ * (parity policy 0: f32 scores and statistics):
+ *   s = (q . k) * scale
+ *   causal:  s = -inf where j > i                                   (103-109)
+ *   mask:    Bool (kind 1, one byte, nonzero = attend): s += attend ? 0 : -inf;   (112-121)
+ *            float (kind 2, bf16): s += mask                                      (122-124)
+ *   softcap: s = tanh(s / cap) * cap, applied AFTER the masks          (128-132), so a masked
+ *            score becomes -cap and still takes part in the softmax
+ *   softmax over all Sk keys, P rounded to bf16 before P V, division by the f32 row sum last.
+ * A row with every key masked out (no softcap) is NaN, as softmax over -inf only is.
+ * mask_strides: element strides of the mask per batch, head and query row (0 broadcasts);
+ * keys are contiguous.  No test of the reference holds values for masks or softcap ("all
+ * outputs finite" is its only softcap check): these options are pinned by closed forms, by
+ * identities with the causal path and against float64 in tests/test_oracle.py. */
+void orc_sdpa_bf16_ex(const bf16_t* Q, const bf16_t* K, const bf16_t* V, bf16_t* O, int B, int H, int Sq, int Sk, int D,
+                      float scale, int causal, const void* mask, int mask_kind, const long* mask_strides, float softcap,
+                      int threads) {
+    if (threads < 1) threads = 1;
+#pragma omp parallel for num_threads(threads) schedule(dynamic, 1)
+    for (int bh = 0; bh < B * H; bh++) {
+        const int b = bh / H, h = bh % H;
+        float* s = (float*)malloc(sizeof(float) * (size_t)(Sk + D + 1));
+        float* acc = s + Sk;
+        const bf16_t *Qh = Q + (size_t)bh * Sq * D, *Kh = K + (size_t)bh * Sk * D, *Vh = V + (size_t)bh * Sk * D;
+        bf16_t* Oh = O + (size_t)bh * Sq * D;
+        for (int i = 0; i < Sq; i++) {
+            const long mrow = mask_kind ? b * mask_strides[0] + h * mask_strides[1] + i * mask_strides[2] : 0;
+            float m = -INFINITY;
+            for (int j = 0; j < Sk; j++) {
+                float a = 0.0f;
+                for (int d = 0; d < D; d++) a = fmaf(bf16_to_f32(Qh[(size_t)i * D + d]), bf16_to_f32(Kh[(size_t)j * D + d]), a);
+                a *= scale;
+                if (causal && j > i) a = -INFINITY;
+                if (mask_kind == 1) a += ((const uint8_t*)mask)[mrow + j] ? 0.0f : -INFINITY;
+                else if (mask_kind == 2) a += bf16_to_f32(((const bf16_t*)mask)[mrow + j]);
+                if (softcap > 0.0f) a = tanhf(a / softcap) * softcap;
+                s[j] = a;
+                m = fmaxf(m, a);
+            }
+            float l = 0.0f;
+            for (int j = 0; j < Sk; j++) {
+                float e = expf(s[j] - m);
+                l += e;
+                s[j] = bf16_to_f32(f32_to_bf16(e));
+            }
+            for (int d = 0; d < D; d++) acc[d] = 0.0f;
+            for (int j = 0; j < Sk; j++) {
+                float p = s[j];
+                for (int d = 0; d < D; d++) acc[d] = fmaf(p, bf16_to_f32(Vh[(size_t)j * D + d]), acc[d]);
+            }
+            for (int d = 0; d < D; d++) Oh[(size_t)i * D + d] = f32_to_bf16(acc[d] / l);
+        }
         free(s);
     }
 }

@@ -74,6 +74,28 @@ class Oracle:
                                C.c_int(threads or self.max_threads))
         return o
 
+    def sdpa_bf16_ex(self, q, k, v, scale, causal=False, mask=None, softcap=0.0, threads=None):
+        """attn_mask (bool or bf16-as-uint16 array broadcastable to [B, H, Sq, Sk] with the key axis
+        full) and softcap, in the reference's order (tensor/src/transformer.rs:96-132)."""
+        B, H, Sq, D = q.shape
+        Sk = k.shape[2]
+        q, k, v = (np.ascontiguousarray(t_) for t_ in (q, k, v))
+        o = np.empty_like(q)
+        kind, mptr, strides = 0, None, (C.c_long * 3)(0, 0, 0)
+        if mask is not None:
+            mask = np.ascontiguousarray(mask)
+            kind = 1 if mask.dtype == np.bool_ else 2
+            assert kind == 1 or mask.dtype == np.uint16
+            shape = (1,) * (4 - mask.ndim) + mask.shape
+            assert shape[3] == Sk and all(s_ in (1, full) for s_, full in zip(shape[:3], (B, H, Sq)))
+            dense = [shape[1] * shape[2] * shape[3], shape[2] * shape[3], shape[3]]
+            strides = (C.c_long * 3)(*[0 if shape[i] == 1 else dense[i] for i in range(3)])
+            mptr = _ptr(mask.view(np.uint8) if kind == 1 else mask)
+        self.lib.orc_sdpa_bf16_ex(_ptr(q), _ptr(k), _ptr(v), _ptr(o), C.c_int(B), C.c_int(H), C.c_int(Sq), C.c_int(Sk),
+                                  C.c_int(D), C.c_float(scale), C.c_int(int(causal)), mptr, C.c_int(kind), strides,
+                                  C.c_float(softcap), C.c_int(threads or self.max_threads))
+        return o
+
     def sdpa_bf16_rows(self, q, k, v, scale, causal=True, threads=None):
         Sq, D = q.shape
         Sk = k.shape[0]

@@ -365,3 +365,114 @@ def test_head_dims_without_an_instantiation_are_padded(dev, oracle, d, causal):
     assert sum(nm.startswith("flash_fwd_bf16") for nm in names) == 1 and not any(nm.startswith("r_") for nm in names), names
     assert got.shape == q.shape
     _check(got, oracle.sdpa_bf16(q, k, v, float(d) ** -0.5, causal=causal))
+
+
+# ---------------------------------------------------------------- attn_mask and softcap inside the kernel
+def _mask_for(kind, layout, B, H, Sq, Sk, seed):
+    """(host array for the oracle, element strides per batch / head / row) of a mask broadcastable to
+    [B, H, Sq, Sk]: Bool with ~60 % of the keys kept (key 0 always, so no row is empty) or additive bf16."""
+    shape = {"qk": (Sq, Sk), "b11k": (B, 1, 1, Sk), "bhqk": (B, H, Sq, Sk), "1hqk": (1, H, Sq, Sk)}[layout]
+    if kind == "bool":
+        m = synth.uniform(shape, seed, 8) < 0.2
+        m[..., 0] = True
+    else:
+        m = synth.to_bf16((synth.normal(shape, seed, 9) * 2.0).astype(np.float32))
+    full = (1,) * (4 - len(shape)) + shape
+    dense = [full[1] * full[2] * full[3], full[2] * full[3], full[3]]
+    return m, [0 if full[i] == 1 else dense[i] for i in range(3)]
+
+
+def _attn_ex(dev, q, k, v, scale, causal, mask, mstrides, cap, d, via_program=False):
+    B, H, Sq, _ = q.shape
+    Sk = k.shape[2]
+    bq, bk, bv = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (q, k, v))
+    bo = dev.buffer(q.nbytes)
+    kind = 0 if mask is None else 1 if mask.dtype == np.bool_ else 2
+    bm = morok_amd.Buffer.from_numpy(mask.view(np.uint8) if kind == 1 else mask, dev.device_id) if kind else None
+    if via_program:
+        bits = lambda x: int(np.float32(x).view(np.uint32))
+        dense = lambda rows: [H * rows * d, rows * d, d]
+        params = [B, H, Sq, Sk, d, int(causal), bits(scale), bits(cap) if cap else 0, kind, 0, 0, 0, 0, 0,
+                  *dense(Sq), *dense(Sk), *dense(Sk), *dense(Sq), *(mstrides if kind else [0, 0, 0])]
+        prog = morok_amd.Program.builtin("flash_fwd_bf16_ext", params, dev.device_id)
+        prog.execute([bo, bq, bk, bv, bm if kind else bq])
+    else:
+        ops.flash_attn_fwd_bf16_ex(bq, bk, bv, bo, B, H, Sq, Sk, d, scale, causal, bm, kind, mstrides if kind else (0, 0, 0), cap,
+                                   device_id=dev.device_id)
+    return bo.copyout(np.uint16, q.shape)
+
+
+@pytest.mark.parametrize("d", [128, 64, 256])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("kind,layout,cap", [(kind, layout, cap) for cap in (0.0, 1.5, 30.0)
+                                             for kind, layout in (("none", None), ("bool", "qk"), ("bool", "b11k"), ("add", "bhqk"), ("add", "1hqk"))
+                                             if kind != "none" or cap > 0.0])     # (no option at all is the plain kernel, covered above)
+def test_flash_mask_and_softcap_vs_oracle(dev, oracle, d, causal, kind, layout, cap):
+    """attn_mask (Bool / additive, several broadcast layouts) and softcap inside the fused kernel
+    against the oracle's restatement of transformer.rs:96-132, ragged query and key counts, all
+    three head dims; <= 2e-2 of the largest reference magnitude."""
+    B, H, Sq, Sk = 2, 2, 200, 260
+    q, k, v = (synth.normal_bf16((B, H, s, d), 41, i) for i, s in enumerate((Sq, Sk, Sk)))
+    mask, mst = (None, None) if kind == "none" else _mask_for(kind, layout, B, H, Sq, Sk, 41)
+    scale = 1.0 / np.sqrt(d)
+    got = _attn_ex(dev, q, k, v, scale, causal, mask, mst, cap, d, via_program=(d == 128 and causal))
+    ref = oracle.sdpa_bf16_ex(q, k, v, scale, causal=causal, mask=mask, softcap=cap)
+    _check(got, ref)
+
+
+def test_flash_mask_identities_and_empty_rows(dev, oracle):
+    """A Bool tril mask, an additive mask that is -inf above the diagonal and is_causal agree with the
+    plain causal kernel to the tolerance; an all-true mask is the plain kernel; a row with no key left
+    is NaN and leaves the other rows alone; a key-padding mask equals attention over the kept keys."""
+    B, H, S, d = 1, 2, 256, 128
+    q, k, v = _inputs(B, H, S, S, seed=43)
+    tril = np.tril(np.ones((S, S), bool))
+    plain_causal = _attn(dev, q, k, v, SCALE, True)
+    _check(_attn_ex(dev, q, k, v, SCALE, False, tril, [0, 0, S], 0.0, d), plain_causal)
+    neg = synth.to_bf16(np.where(tril, 0.0, -np.inf).astype(np.float32))
+    _check(_attn_ex(dev, q, k, v, SCALE, False, neg, [0, 0, S], 0.0, d), plain_causal)
+    _check(_attn_ex(dev, q, k, v, SCALE, True, tril, [0, 0, S], 0.0, d), plain_causal)       # both at once
+    _check(_attn_ex(dev, q, k, v, SCALE, False, np.ones((S, S), bool), [0, 0, S], 0.0, d), _attn(dev, q, k, v, SCALE, False))
+    none = np.ones((S, S), bool)
+    none[70] = False
+    none[:, :64] |= False
+    got = synth.from_bf16(_attn_ex(dev, q, k, v, SCALE, False, none, [0, 0, S], 0.0, d))
+    ref = synth.from_bf16(oracle.sdpa_bf16_ex(q, k, v, SCALE, mask=none))
+    assert np.isnan(got[:, :, 70]).all() and np.isnan(ref[:, :, 70]).all()
+    keep = np.delete(np.arange(S), 70)
+    assert np.abs(got[:, :, keep] - ref[:, :, keep]).max() <= 2e-2 * np.abs(ref[:, :, keep]).max()
+    # rows whose first key tiles are fully masked (a sliding window): the running maximum starts at -inf
+    win = np.zeros((S, S), bool)
+    for i in range(S):
+        win[i, max(0, i - 20): i + 1] = True
+    _check(_attn_ex(dev, q, k, v, SCALE, False, win, [0, 0, S], 0.0, d), oracle.sdpa_bf16_ex(q, k, v, SCALE, mask=win))
+    pad = np.ones((B, 1, 1, S), bool)
+    pad[..., 200:] = False
+    _check(_attn_ex(dev, q, k, v, SCALE, False, pad, [S, 0, 0], 0.0, d),
+           oracle.sdpa_bf16(q, k[:, :, :200], v[:, :, :200], SCALE, causal=False))
+
+
+def test_flash_softcap_masked_scores_become_minus_cap(dev, oracle):
+    """The reference caps after masking: with zero queries and keys every score is 0, a causally
+    masked one -cap, so row i is the mean of v[0..i] and exp(-cap) times the rest."""
+    S, d, cap = 128, 128, 0.75
+    z = np.zeros((1, 1, S, d), np.uint16)
+    v = synth.normal_bf16((1, 1, S, d), 44, 2)
+    got = synth.from_bf16(_attn_ex(dev, z, z, v, 1.0, True, None, None, cap, d))
+    vf = synth.from_bf16(v).astype(np.float64)[0, 0]
+    w = np.where(np.tril(np.ones((S, S), bool)), 1.0, np.exp(-cap))
+    ref = (w @ vf) / w.sum(1, keepdims=True)
+    assert np.abs(got[0, 0] - ref).max() <= 2e-2 * np.abs(ref).max()
+    _check(_attn_ex(dev, z, z, v, 1.0, True, None, None, cap, d), oracle.sdpa_bf16_ex(z, z, v, 1.0, causal=True, softcap=cap))
+
+
+def test_flash_ex_argument_errors(dev):
+    b = dev.buffer(4 * 128 * 2 * 8).ensure_allocated()
+    with pytest.raises(MorokHipError):   # key count not a multiple of 4 with a mask
+        ops.flash_attn_fwd_bf16_ex(b, b, b, b, 1, 1, 4, 6, 128, 1.0, False, b, 1, (0, 0, 8), 0.0)
+    with pytest.raises(MorokHipError):   # mask stride not a multiple of 4
+        ops.flash_attn_fwd_bf16_ex(b, b, b, b, 1, 1, 4, 8, 128, 1.0, False, b, 1, (0, 0, 6), 0.0)
+    with pytest.raises(MorokHipError):   # negative softcap
+        ops.flash_attn_fwd_bf16_ex(b, b, b, b, 1, 1, 4, 8, 128, 1.0, False, None, 0, (0, 0, 0), -1.0)
+    with pytest.raises(MorokHipError):   # unknown mask kind
+        ops.flash_attn_fwd_bf16_ex(b, b, b, b, 1, 1, 4, 8, 128, 1.0, False, b, 3, (0, 0, 8), 0.0)

@@ -210,6 +210,89 @@ def test_sdpa_bf16_vs_float64_and_special_cases(oracle):
     assert np.abs(lit - pol).max() < 6e-2 * np.abs(pol).max()
 
 
+def _sdpa64_ex(q, k, v, scale, causal, mask_add=None, cap=0.0):
+    """float64 restatement of transformer.rs:96-132: scale, causal where(-inf), additive mask, softcap
+    AFTER the masks, softmax over every key."""
+    q, k, v = (t.astype(np.float64) for t in (q, k, v))
+    s = np.einsum("bhqd,bhkd->bhqk", q, k) * scale
+    if causal:
+        sq, sk = s.shape[-2:]
+        s = np.where(np.tril(np.ones((sq, sk), bool)), s, -np.inf)
+    if mask_add is not None:
+        s = s + mask_add
+    if cap > 0:
+        s = np.tanh(s / cap) * cap
+    with np.errstate(invalid="ignore"):
+        p = np.exp(s - s.max(-1, keepdims=True))
+        p /= p.sum(-1, keepdims=True)
+    return np.einsum("bhqk,bhkd->bhqd", p, v)
+
+
+def test_sdpa_mask_and_softcap_closed_forms_identities_and_float64(oracle):
+    """orc_sdpa_bf16_ex has no values to match in the reference's tests (its softcap test only asks
+    for finite outputs), so it is pinned here: the reference's softcap case in closed form, masks
+    that must reproduce the causal path bit for bit, the -cap (not -inf) a masked score turns into
+    under a softcap, a fully masked row, and float64 on random inputs for every combination."""
+    g = GOLD["sdpa_softcap_finite"]
+    q = synth.to_bf16(np.array(g["q"], np.float32))
+    v = synth.to_bf16(np.array(g["v"], np.float32))
+    o = synth.from_bf16(oracle.sdpa_bf16_ex(q, q, v, 1.0 / np.sqrt(2.0), softcap=g["softcap"]))
+    assert np.isfinite(o).all()
+    # scores 70.7 / 0 -> tanh(70.7) = 1, tanh(0) = 0 -> softmax([1, 0]) = [e, 1] / (e + 1)
+    w = np.e / (np.e + 1.0)
+    assert np.abs(o - np.array([[[[w, 1 - w], [1 - w, w]]]])).max() < 4e-3          # bf16 output rounding
+    B, H, Sq, Sk, D = 2, 3, 40, 56, 32
+    qb, kb, vb = (synth.normal_bf16((B, H, s_, D), 31, i) for i, s_ in enumerate((Sq, Sk, Sk)))
+    qf, kf, vf = (synth.from_bf16(t) for t in (qb, kb, vb))
+    scale = 1.0 / np.sqrt(D)
+    plain = oracle.sdpa_bf16_ex(qb, kb, vb, scale)
+    sq_k = oracle.sdpa_bf16(qb[:, :, :, :], kb[:, :, :Sq], vb[:, :, :Sq], scale, causal=True)
+    tril = np.tril(np.ones((Sq, Sq), bool))
+    # identities, bit for bit: no options = the plain function; a True mask and a zero mask change nothing;
+    # a Bool tril mask and an additive -inf-above-the-diagonal mask are the causal path
+    assert np.array_equal(plain, oracle.sdpa_bf16(qb, kb, vb, scale, causal=False))
+    assert np.array_equal(plain, oracle.sdpa_bf16_ex(qb, kb, vb, scale, mask=np.ones((Sq, Sk), bool)))
+    assert np.array_equal(plain, oracle.sdpa_bf16_ex(qb, kb, vb, scale, mask=np.zeros((B, 1, Sq, Sk), np.uint16)))
+    assert np.array_equal(sq_k, oracle.sdpa_bf16_ex(qb, kb[:, :, :Sq], vb[:, :, :Sq], scale, causal=True))
+    assert np.array_equal(sq_k, oracle.sdpa_bf16_ex(qb, kb[:, :, :Sq], vb[:, :, :Sq], scale, mask=tril))
+    neg = synth.to_bf16(np.where(tril, 0.0, -np.inf).astype(np.float32))
+    assert np.array_equal(sq_k, oracle.sdpa_bf16_ex(qb, kb[:, :, :Sq], vb[:, :, :Sq], scale, mask=neg))
+    # per-batch key padding mask [B, 1, 1, Sk] = attention over the kept keys only
+    keep = np.ones((B, 1, 1, Sk), bool)
+    keep[0, :, :, 40:] = False
+    keep[1, :, :, :7] = False
+    got = oracle.sdpa_bf16_ex(qb, kb, vb, scale, mask=keep)
+    assert np.array_equal(got[0], oracle.sdpa_bf16(qb[:1], kb[:1, :, :40], vb[:1, :, :40], scale, causal=False)[0])
+    assert np.array_equal(got[1], oracle.sdpa_bf16(qb[1:], kb[1:, :, 7:], vb[1:, :, 7:], scale, causal=False)[0])
+    # a row with no key left is NaN (softmax over -inf only); the other rows are untouched
+    none = np.ones((Sq, Sk), bool)
+    none[5] = False
+    got = synth.from_bf16(oracle.sdpa_bf16_ex(qb, kb, vb, scale, mask=none))
+    assert np.isnan(got[:, :, 5]).all() and np.array_equal(np.delete(got, 5, 2), np.delete(synth.from_bf16(plain), 5, 2))
+    # softcap after the masks: with two keys, zero queries and key 1 masked, the scores are [0, -cap],
+    # so row 0 is (v0 + exp(-cap) v1) / (1 + exp(-cap)), not v0
+    z = np.zeros((1, 1, 2, 8), np.uint16)
+    v2 = synth.to_bf16(np.array([[1.0] * 8, [3.0] * 8], np.float32).reshape(1, 1, 2, 8))
+    for cap in (0.5, 2.0):
+        got = synth.from_bf16(oracle.sdpa_bf16_ex(z, z, v2, 1.0, causal=True, softcap=cap))
+        e = np.exp(-cap)
+        assert abs(got[0, 0, 0, 0] - (1.0 + 3.0 * e) / (1.0 + e)) < 1e-2 and abs(got[0, 0, 1, 0] - 2.0) < 1e-2
+    # float64 on random inputs, every combination
+    add = synth.from_bf16(synth.normal_bf16((B, H, Sq, Sk), 31, 7)).astype(np.float64) * 2.0
+    addb = synth.to_bf16(add.astype(np.float32))
+    add = synth.from_bf16(addb).astype(np.float64)
+    boolm = synth.uniform((H, Sq, Sk), 31, 8) < 0.6
+    boolm[..., 0] = True                                                           # no empty rows
+    for causal in (False, True):
+        for cap in (0.0, 1.5, 30.0):
+            for kind in ("none", "bool", "add"):
+                m = None if kind == "none" else boolm if kind == "bool" else addb
+                m64 = None if kind == "none" else np.where(boolm, 0.0, -np.inf)[None] if kind == "bool" else add
+                got = synth.from_bf16(oracle.sdpa_bf16_ex(qb, kb, vb, scale, causal=causal, mask=m, softcap=cap))
+                ref = _sdpa64_ex(qf, kf, vf, scale, causal, m64, cap)
+                assert np.abs(got - ref).max() < 2e-2 * np.abs(ref).max(), (causal, cap, kind)
+
+
 # ------------------------------------------------------------------ C5 pieces
 def test_rms_norm_reference_cases(oracle):
     g = GOLD["rms_norm_basic"]

@@ -445,22 +445,85 @@ def test_sdpa_attn_mask(T, fusion, kind):
     assert not any(n.startswith("flash_fwd") for n in t.kernels())
 
 
-def test_sdpa_bf16_with_mask_takes_the_composed_graph(T):
-    """bf16 operands with a mask: the fused kernel does not apply, the composed graph still
-    computes the masked attention (bf16 scores: loose tolerance)."""
+def test_sdpa_bf16_with_mask_and_softcap_is_the_fused_kernel(T, oracle):
+    """tensor/src/transformer.rs:112-132 inside the fused kernel: a Bool mask, an additive bf16
+    mask (as a broadcast [B, 1, 1, Sk] view and as a slice of a larger tensor) and a softcap each
+    run as ONE flash_fwd kernel, <= 2e-2 against the oracle; the same graphs with the hand-written
+    kernels switched off (the composed graph, bf16 scores) agree with it loosely."""
     from morok_amd import synth, uop
 
     rng = np.random.default_rng(62)
-    B, H, S, D = 1, 2, 64, 128
+    B, H, S, D = 2, 2, 192, 128
     q, k, v = (synth.to_bf16(rng.standard_normal((B, H, S, D)).astype(np.float32)) for _ in range(3))
+    tq, tk, tv = (T.Tensor.from_numpy(a, uop.BF16) for a in (q, k, v))
+    scale = 1 / np.sqrt(D)
     mask = rng.random((S, S)) < 0.7
     mask[:, 0] = True
-    t = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(T.Tensor.from_numpy(k, uop.BF16), T.Tensor.from_numpy(v, uop.BF16),
-                                                                      attn_mask=T.Tensor.from_numpy(mask))
+    t = tq.scaled_dot_product_attention(tk, tv, attn_mask=T.Tensor.from_numpy(mask))
+    got = t.to_numpy()
+    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("flash_fwd_bf16_ext_bool"), t.kernels()
+    ref = synth.from_bf16(oracle.sdpa_bf16_ex(q, k, v, scale, mask=mask))
+    assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
+    # causal + key padding mask [B, 1, 1, S] + softcap, the mask an expand of a [B, S] tensor
+    pad = np.ones((B, S), bool)
+    pad[0, 150:] = False
+    pad[1, 3:40] = False
+    tm = T.Tensor.from_numpy(pad).try_reshape([B, 1, 1, S])
+    t = tq.scaled_dot_product_attention(tk, tv, is_causal=True, attn_mask=tm, softcap=20.0)
+    got = t.to_numpy()
+    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("flash_fwd_bf16_ext_bool_cap"), t.kernels()
+    ref = synth.from_bf16(oracle.sdpa_bf16_ex(q, k, v, scale, causal=True, mask=pad.reshape(B, 1, 1, S), softcap=20.0))
+    assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
+    # additive bf16 mask that is a slice of a larger tensor in memory: read in place
+    big = synth.to_bf16((rng.standard_normal((H, S + 8, S + 64)) * 2).astype(np.float32))
+    tm = T.Tensor.from_numpy(big, uop.BF16).try_shrink([(0, H), (8, S + 8), (64, S + 64)])
+    t = tq.scaled_dot_product_attention(tk, tv, attn_mask=tm)
+    got = t.to_numpy()
+    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("flash_fwd_bf16_ext_add"), t.kernels()
+    ref = synth.from_bf16(oracle.sdpa_bf16_ex(q, k, v, scale, mask=np.ascontiguousarray(big[:, 8:, 64:])))
+    assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
+    # softcap alone
+    t = tq.scaled_dot_product_attention(tk, tv, softcap=1.5)
+    got = t.to_numpy()
+    assert len(t.kernels()) == 1 and t.kernels()[0].startswith("flash_fwd_bf16_ext_cap"), t.kernels()
+    ref = synth.from_bf16(oracle.sdpa_bf16_ex(q, k, v, scale, softcap=1.5))
+    assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
+    # an f32 mask changes the dtype of the scores: composed graph, as before; so does a key count
+    # that is not a multiple of four
+    T.set_fusion(False)
+    try:
+        t = tq.scaled_dot_product_attention(tk, tv, attn_mask=T.Tensor.from_numpy(mask), softcap=1.5)
+        loose = synth.from_bf16(t.to_numpy())
+        assert not any(n.startswith("flash_fwd") for n in t.kernels())
+    finally:
+        T.set_fusion(True)
+    ref = synth.from_bf16(oracle.sdpa_bf16_ex(q, k, v, scale, mask=mask, softcap=1.5))
+    assert np.abs(loose - ref).max() <= 6e-2 * np.abs(ref).max()
+    k3, v3 = k[:, :, :190], v[:, :, :190]
+    t = tq.scaled_dot_product_attention(T.Tensor.from_numpy(k3, uop.BF16), T.Tensor.from_numpy(v3, uop.BF16),
+                                        attn_mask=T.Tensor.from_numpy(mask[:, :190]))
     got = synth.from_bf16(t.to_numpy())
     assert not any(n.startswith("flash_fwd") for n in t.kernels())
-    want = _np_sdpa(synth.from_bf16(q), synth.from_bf16(k), synth.from_bf16(v), 1 / np.sqrt(D), mask=mask)
-    assert np.abs(got - want).max() <= 5e-2 * np.abs(want).max()
+    ref = synth.from_bf16(oracle.sdpa_bf16_ex(q, k3, v3, scale, mask=np.ascontiguousarray(mask[:, :190])))
+    assert np.abs(got - ref).max() <= 6e-2 * np.abs(ref).max()
+
+
+def test_sdpa_padded_head_dim_with_mask_and_softcap(T, oracle):
+    """A head dim without an instantiation (96) is zero-padded to 128 by the graph builder; mask and
+    softcap ride along into the fused kernel."""
+    from morok_amd import synth, uop
+
+    rng = np.random.default_rng(63)
+    B, H, S, D = 1, 2, 128, 96
+    q, k, v = (synth.to_bf16(rng.standard_normal((B, H, S, D)).astype(np.float32)) for _ in range(3))
+    mask = rng.random((B, H, S, S)) < 0.5
+    mask[..., 0] = True
+    t = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(T.Tensor.from_numpy(k, uop.BF16), T.Tensor.from_numpy(v, uop.BF16),
+                                                                      attn_mask=T.Tensor.from_numpy(mask), softcap=5.0)
+    got = synth.from_bf16(t.to_numpy())
+    assert sum(n.startswith("flash_fwd_bf16_ext") for n in t.kernels()) == 1
+    ref = synth.from_bf16(oracle.sdpa_bf16_ex(q, k, v, 1 / np.sqrt(D), mask=mask, softcap=5.0))
+    assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max()
 
 
 def test_sdpa_bf16_uses_flash(T, oracle):
