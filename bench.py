@@ -160,7 +160,7 @@ def _mfma_ceiling_tflops(m, dev, random_operands=True):
     and sustains a lower clock the more the operand bits toggle."""
     from morok_amd import ops
 
-    key = "random" if random_operands else "smooth"
+    key = "f16" if random_operands == "f16" else "random" if random_operands else "smooth"
     if key not in _CEILING:
         scratch = dev.buffer(256).ensure_allocated()
         ms, _ = _launch_stats(m, lambda: ops.mfma_ceiling(scratch, 256, 64, random_operands=random_operands), 50, 5)
@@ -250,6 +250,48 @@ def bench_gemm(m, dev, steps, warmup, cpu):
                                        "product path", "ratio": tf / vendor}
     if cpu:
         rec["cpu_baseline"] = _gemm_cpu_baseline(M, N, K)
+    return rec
+
+
+def bench_gemm_f16(m, dev, steps, warmup, cpu):
+    """The 4096^3 product in IEEE half precision through the same caller path: the f16 instantiation of
+    the hand-written kernel (v_mfma_f32_16x16x32_f16), inputs normal(0,1) * 0.25 rounded to f16."""
+    import numpy as np
+
+    from morok_amd import synth, tensor, uop
+
+    M = N = K = 4096
+    a = (synth.normal((M, K), 3, 0) * np.float32(0.25)).astype(np.float16)
+    b = synth.normal((K, N), 3, 1).astype(np.float16)
+    ba, bb = m.Buffer.from_numpy(a.view(np.uint16)), m.Buffer.from_numpy(b.view(np.uint16))
+    c = tensor.Tensor.from_buffer(ba, (M, K), uop.F16).matmul(tensor.Tensor.from_buffer(bb, (K, N), uop.F16))
+    plan = c.prepare()
+    program = plan.kernel_name(0)
+    if not program.startswith("gemm_f16"):
+        raise RuntimeError("Tensor::matmul did not select the hand-written f16 GEMM: " + program)
+    ms, stats = _launch_stats(m, plan.execute, steps, warmup)
+    flops = 2.0 * M * N * K
+    tf = flops / (ms * 1e-3) / 1e12
+    rec = {
+        "metric": "f16 GEMM TFLOP/s", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "f16",
+        "config": {"workload": "f16 GEMM M=N=K=4096, f32 accumulate, f16 out, via Tensor::matmul -> prepare -> execute"},
+        # the dense f16 MFMA peak is the bf16 one
+        "roofline": _roofline("gemm_f16", "mfma", tf, BF16_PEAK_TFLOPS, "TFLOP/s", "gemm_f16_tile256", algorithmic_flops_per_launch=flops),
+        "plan_item": program,
+    }
+    rec.update(stats)
+    if REFERENCE_LEGS:
+        # register-only stream of the f16 instruction on the same values, and of the bf16 one beside it
+        ceiling = _mfma_ceiling_tflops(m, dev, "f16")
+        rec["roofline"].update(mfma_only_ceiling=ceiling, frac_of_ceiling=tf / ceiling, mfma_only_ceiling_bf16_instruction=_mfma_ceiling_tflops(m, dev))
+    if cpu:
+        from tests.oracle_lib import Oracle
+
+        orc = Oracle()
+        rows = 256
+        sec = _cpu_time(lambda: orc.gemm_f16(a[:rows], b))
+        rec["cpu_baseline"] = {"value": 2.0 * rows * N * K / sec / 1e12, "unit": "TFLOP/s", "cores": orc.max_threads, "kind": "port",
+                               "sample": f"{rows} of the {M} output rows (K=N=4096), f32-accumulate f16 matmul, min of 3 after 1 warm-up"}
     return rec
 
 
@@ -478,7 +520,7 @@ def bench_copy(m, dev, steps, warmup, cpu):
 
 WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "decoder": bench_decoder,
              "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling,
-             "group_reduce": bench_group_reduce}
+             "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16}
 PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc"]
 
 

@@ -442,6 +442,14 @@ size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_
  * enough output tiles that the split-K form would not be chosen (mrk_hip_gemm_bf16_workspace_bytes
  * == 0); INVALID_ARGUMENT otherwise.  Builtin Program kind "gemm_bf16_nt". */
 int mrk_hip_gemm_bf16_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k);
+/* The same two products on IEEE half precision (f16) operands and result, f32 accumulate: the f16
+ * 16x16x32 entry of the reference's CDNA4 tensor-core table
+ * (schedule/src/optimizer/renderer.rs:724-733, listed ahead of the bf16 one) as a hand-written
+ * kernel; what Tensor::matmul computes for f16 inputs (tensor/src/matmul.rs:82-110 with the
+ * tensor-core rewrite).  Same shapes, fallbacks and argument rules as the bf16 entry points; the
+ * fused residual / gated epilogues are bf16 only.  Builtin Program kinds "gemm_f16", "gemm_f16_nt". */
+int mrk_hip_gemm_f16(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k);
+int mrk_hip_gemm_f16_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k);
 /* Same with an explicit kernel variant (0 choose by shape, 2 any-shape kernel, 3 / 4 tiled kernel
  * with the 256-row / 128-row tile); tuning/tests. */
 int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
@@ -539,7 +547,8 @@ int mrk_hip_copy_kernel(int device_id, const void* src, void* dst, size_t bytes)
  * workgroup.  The rate it sustains is the ceiling GEMM kernels are compared with next to the
  * published peak.  random_operands: 0 = smooth small operand values, 1 = hashed values in
  * [-1.7, 1.7) as in a product of random matrices (the pipes' power draw, and with it the sustained
- * clock, depends on how much the operand bits toggle).  `scratch`: any device allocation of >= 4 bytes. */
+ * clock, depends on how much the operand bits toggle), 2 = the same hashed values rounded to IEEE
+ * half precision and issued as the f16 instruction.  `scratch`: any device allocation of >= 4 bytes. */
 int mrk_hip_mfma_ceiling(int device_id, void* scratch, int64_t workgroups, int64_t k_steps, int random_operands);
 /* int32 values uniform over [0, high). */
 int mrk_hip_fill_randint(int device_id, void* out, size_t n, uint64_t seed, uint64_t tensor_id, int high);

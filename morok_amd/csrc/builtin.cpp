@@ -108,41 +108,44 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
-    if (k == "gemm_bf16") {  // {M, N, K}, {M, N, K, batch} or {M, N, K, batch, workspace bytes}
+    // "gemm_f16" / "gemm_f16_nt": the same kernels on IEEE half precision operands and result
+    if (k == "gemm_bf16" || k == "gemm_f16") {  // {M, N, K}, {M, N, K, batch} or {M, N, K, batch, workspace bytes}
+        const bool f16 = k == "gemm_f16";
         if (nparams < 3 || nparams > 5)
-            return failf(kInvalidArgument, "builtin 'gemm_bf16' takes 3 to 5 parameters, got %zu", nparams);
+            return failf(kInvalidArgument, "builtin '%s' takes 3 to 5 parameters, got %zu", k.c_str(), nparams);
         while (p.size() < 4) p.push_back(1);
         if (p.size() < 5) p.push_back(0);
         if (p[0] < 0 || p[1] < 0 || p[2] < 0 || p[3] < 1 || p[3] > 65535 || p[4] < 0)
-            return fail(kInvalidArgument, "gemm_bf16: bad shape (M, N, K >= 0, 1 <= batch <= 65535, workspace >= 0)");
-        std::string name = "gemm_bf16_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+            return fail(kInvalidArgument, k + ": bad shape (M, N, K >= 0, 1 <= batch <= 65535, workspace >= 0)");
+        std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
         if (p[3] > 1) name += "_x" + std::to_string(p[3]);
         if (p[4] > 0) {  // a fourth buffer of p[4] bytes: scratch for the split-K partial results
             out->reset(new BuiltinProgram(device_id, stream, name + "_splitk", 4, p,
-                                          [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          [f16](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
                                               return launch_gemm_bf16(s, b[1], b[2], b[0], q[0], q[1], q[2], 0, q[3], b[3],
-                                                                      static_cast<size_t>(q[4]));
+                                                                      static_cast<size_t>(q[4]), false, f16);
                                           }));
             return kOk;
         }
         out->reset(new BuiltinProgram(device_id, stream, name, 3, p,
-                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
-                                          return launch_gemm_bf16(s, b[1], b[2], b[0], q[0], q[1], q[2], 0, q[3]);
+                                      [f16](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16(s, b[1], b[2], b[0], q[0], q[1], q[2], 0, q[3], nullptr, 0, false, f16);
                                       }));
         return kOk;
     }
     // the "_nt" kinds take the second operand as B^T [N, K] (a Linear layer's weight as it is stored)
-    if (k == "gemm_bf16_nt") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, bt}
+    if (k == "gemm_bf16_nt" || k == "gemm_f16_nt") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, bt}
+        const bool f16 = k == "gemm_f16_nt";
         if (nparams < 3 || nparams > 4)
-            return failf(kInvalidArgument, "builtin 'gemm_bf16_nt' takes 3 or 4 parameters, got %zu", nparams);
+            return failf(kInvalidArgument, "builtin '%s' takes 3 or 4 parameters, got %zu", k.c_str(), nparams);
         while (p.size() < 4) p.push_back(1);
         if (!gemm_bf16_nt_supported(p[0], p[1], p[2], p[3]))
-            return fail(kInvalidArgument, "gemm_bf16_nt: shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel)");
-        std::string name = "gemm_bf16_nt_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+            return fail(kInvalidArgument, k + ": shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel)");
+        std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
         if (p[3] > 1) name += "_x" + std::to_string(p[3]);
         out->reset(new BuiltinProgram(device_id, stream, name, 3, p,
-                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
-                                          return launch_gemm_bf16(s, b[1], b[2], b[0], q[0], q[1], q[2], 0, q[3], nullptr, 0, true);
+                                      [f16](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16(s, b[1], b[2], b[0], q[0], q[1], q[2], 0, q[3], nullptr, 0, true, f16);
                                       }));
         return kOk;
     }

@@ -845,9 +845,8 @@ int mrk_hip_softmax_f32(int device_id, const void* x, void* y, int64_t rows, int
     return mrk_hip_softmax_f32_variant(device_id, x, y, rows, cols, 0);
 }
 
-int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
-                               int variant) {
-    if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16: negative shape");
+static int gemm_16bit(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k, int variant, bool f16) {
+    if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, f16 ? "gemm_f16: negative shape" : "gemm_bf16: negative shape");
     if (m == 0 || n == 0) return kOk;
     MRK_NONNULL(c);
     if (k > 0) {
@@ -864,10 +863,17 @@ int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void*
     RawBuffer scratch;
     BufferOptions so;
     if (ws) MRK_TRY(d->allocator->alloc(ws, so, &scratch));
-    int rc = launch_gemm_bf16(d->allocator->stream(), a, b, c, m, n, k, variant, 1, ws ? scratch.ptr : nullptr, ws);
+    int rc = launch_gemm_bf16(d->allocator->stream(), a, b, c, m, n, k, variant, 1, ws ? scratch.ptr : nullptr, ws, false, f16);
     if (ws) d->allocator->free(scratch, so);
-    MRK_HIP(rc, "gemm_bf16 launch");
+    MRK_HIP(rc, f16 ? "gemm_f16 launch" : "gemm_bf16 launch");
     return kOk;
+}
+int mrk_hip_gemm_bf16_variant(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k,
+                               int variant) {
+    return gemm_16bit(device_id, a, b, c, m, n, k, variant, false);
+}
+int mrk_hip_gemm_f16(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k) {
+    return gemm_16bit(device_id, a, b, c, m, n, k, 0, true);
 }
 size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t batch) {
     return gemm_bf16_workspace_bytes(m, n, k, batch);
@@ -876,7 +882,14 @@ int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int6
     return mrk_hip_gemm_bf16_variant(device_id, a, b, c, m, n, k, 0);
 }
 
+static int gemm_16bit_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k, bool f16);
 int mrk_hip_gemm_bf16_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k) {
+    return gemm_16bit_nt(device_id, a, bt, c, m, n, k, false);
+}
+int mrk_hip_gemm_f16_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k) {
+    return gemm_16bit_nt(device_id, a, bt, c, m, n, k, true);
+}
+static int gemm_16bit_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k, bool f16) {
     if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_nt: negative shape");
     if (m == 0 || n == 0) return kOk;
     MRK_NONNULL(a);
@@ -888,7 +901,7 @@ int mrk_hip_gemm_bf16_nt(int device_id, const void* a, const void* bt, void* c, 
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_gemm_bf16(dv->allocator->stream(), a, bt, c, m, n, k, 0, 1, nullptr, 0, true), "gemm_bf16_nt launch");
+    MRK_HIP(launch_gemm_bf16(dv->allocator->stream(), a, bt, c, m, n, k, 0, 1, nullptr, 0, true, f16), "gemm_bf16_nt launch");
     return kOk;
 }
 
@@ -1095,7 +1108,7 @@ int mrk_hip_mfma_ceiling(int device_id, void* scratch, int64_t workgroups, int64
     std::shared_ptr<Device> d;
     MRK_TRY(get_device(device_id, &d));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_mfma_ceiling(d->allocator->stream(), scratch, workgroups, k_steps, random_operands != 0), "mfma_ceiling launch");
+    MRK_HIP(launch_mfma_ceiling(d->allocator->stream(), scratch, workgroups, k_steps, random_operands), "mfma_ceiling launch");
     return kOk;
 }
 

@@ -112,11 +112,25 @@ __device__ __attribute__((aligned(16))) const unsigned g_zero16[4] = {0u, 0u, 0u
 // C[M, F] = bf16(silu(float(bf16(A gate))) * float(bf16(A up))): the two products rounded to bf16
 // as separate kernels would leave them, then x * sigmoid(x) * y in f32 with one rounding, without
 // the 2F-wide product ever reaching memory.
-template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false, bool kSwiGLU = false, bool kBT = false>
+//
+// kF16: the operands and the result are IEEE half precision instead of bf16
+// (v_mfma_f32_16x16x32_f16: the f16 entry of the reference's CDNA4 table,
+// schedule/src/optimizer/renderer.rs:724-733).  Both are 16-bit elements, so copies, LDS layout,
+// fragment reads and stores are the same bytes; only the matrix instruction and the conversion of
+// the f32 accumulators differ.  The element pointers stay typed as 16-bit carriers.
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+template <bool kF16>
+__device__ __forceinline__ bf16x4 round_to_elem(const f32x4& v) {
+    if constexpr (kF16) return __builtin_bit_cast(bf16x4, __builtin_convertvector(v, f16x4));
+    else return __builtin_convertvector(v, bf16x4);
+}
+template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false, bool kSwiGLU = false, bool kBT = false, bool kF16 = false>
 __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
                                                float* __restrict__ W = nullptr, int kt_per_split = 0,
                                                const __bf16* __restrict__ R = nullptr) {
+    static_assert(!kF16 || (!kResidual && !kSwiGLU), "the fused epilogues exist for bf16 only");
     constexpr int kTM = kJ == 4 ? 256 : 128;      // rows of the workgroup tile
     constexpr int kAq = kTM / 32;                 // 1 KB A chunks (8 rows) each wave copies per K step
     constexpr int kAStageT = kTM * kBK * 2;       // bytes of an A stage
@@ -348,7 +362,8 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     // accumulation registers (through the builtin the compiler leaves this shape untied and copies
     // tiles around) ...
     auto mfma = [&](f32x4& c, const bf16x8& a, const bf16x8& b) {
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+        if constexpr (kF16) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+        else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     };
     // One direct copy with the LDS address formed in the instruction that writes M0 ...
     auto dma_at = [&](unsigned lds_base, auto q_c, unsigned voff, const char* sbase) {
@@ -360,10 +375,16 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     // ... and the matrix instruction with one such copy behind it in one statement (the LDS address is formed
     // in the instruction that writes M0), so that nothing else lands between them.
     auto mfma_dma = [&](f32x4& c, const bf16x8& a, const bf16x8& b, unsigned lds_base, auto q_c, unsigned voff, const char* sbase) {
-        asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\ts_add_u32 m0, %3, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %5, %6"
-                     : "+a"(c)
-                     : "v"(a), "v"(b), "s"(lds_base), "n"(decltype(q_c)::value * 1024), "v"(voff), "s"(sbase)
-                     : "m0", "scc");
+        if constexpr (kF16)
+            asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0\n\ts_add_u32 m0, %3, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %5, %6"
+                         : "+a"(c)
+                         : "v"(a), "v"(b), "s"(lds_base), "n"(decltype(q_c)::value * 1024), "v"(voff), "s"(sbase)
+                         : "m0", "scc");
+        else
+            asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0\n\ts_add_u32 m0, %3, %4\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %5, %6"
+                         : "+a"(c)
+                         : "v"(a), "v"(b), "s"(lds_base), "n"(decltype(q_c)::value * 1024), "v"(voff), "s"(sbase)
+                         : "m0", "scc");
     };
 
     // One phase = half of a 32-deep sub-step: phase p covers sub-step p / 2 (fragment slot p / 2)
@@ -569,7 +590,7 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         auto stage_row = [&](int i) {
 #pragma unroll
             for (int j = 0; j < kJ16; j++) {
-                bf16x4 h = __builtin_convertvector(acc[i][j], bf16x4);
+                bf16x4 h = round_to_elem<kF16>(acc[i][j]);
                 *LDS_PTR(bf16x4, sC + (i * 16 + (lane & 15)) * kCPitchT + (j * 16 + 4 * (lane >> 4)) * 2) = h;
             }
         };
@@ -659,8 +680,27 @@ MRK_GEMM_NT_RESIDUAL_KERNEL(gemm_bf16_nt_tile256_residual, false, 4, false, true
 MRK_GEMM_NT_RESIDUAL_KERNEL(gemm_bf16_nt_tile256_residual_ragged_k, true, 4, false, true, false, true)
 MRK_GEMM_NT_RESIDUAL_KERNEL(gemm_bf16_nt_tile128_residual, false, 2, false, true, false, true)
 MRK_GEMM_NT_RESIDUAL_KERNEL(gemm_bf16_nt_tile128_residual_ragged_k, true, 2, false, true, false, true)
+// half-precision instantiations (plain product; [K, N] and [N, K] second operand)
+MRK_GEMM_NT_KERNEL(gemm_f16_tile256, false, 4, false, false, false, false, true)
+MRK_GEMM_NT_KERNEL(gemm_f16_tile256_ragged_k, true, 4, false, false, false, false, true)
+MRK_GEMM_NT_KERNEL(gemm_f16_tile128, false, 2, false, false, false, false, true)
+MRK_GEMM_NT_KERNEL(gemm_f16_tile128_ragged_k, true, 2, false, false, false, false, true)
+MRK_GEMM_NT_KERNEL(gemm_f16_nt_tile256, false, 4, false, false, false, true, true)
+MRK_GEMM_NT_KERNEL(gemm_f16_nt_tile256_ragged_k, true, 4, false, false, false, true, true)
+MRK_GEMM_NT_KERNEL(gemm_f16_nt_tile128, false, 2, false, false, false, true, true)
+MRK_GEMM_NT_KERNEL(gemm_f16_nt_tile128_ragged_k, true, 2, false, false, false, true, true)
 #undef MRK_GEMM_NT_KERNEL
 #undef MRK_GEMM_NT_RESIDUAL_KERNEL
+__global__ __launch_bounds__(256) void gemm_f16_tile128_splitk(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                               float* __restrict__ W, int M, int N, int K, int tiles_m,
+                                                               int tiles_n, int kt_per_split) {
+    gemm_tile_body<false, 2, true, false, false, false, true>(A, B, nullptr, M, N, K, tiles_m, tiles_n, W, kt_per_split);
+}
+__global__ __launch_bounds__(256) void gemm_f16_tile128_splitk_ragged_k(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                                        float* __restrict__ W, int M, int N, int K, int tiles_m,
+                                                                        int tiles_n, int kt_per_split) {
+    gemm_tile_body<true, 2, true, false, false, false, true>(A, B, nullptr, M, N, K, tiles_m, tiles_n, W, kt_per_split);
+}
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_ragged_k(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ B, __bf16* __restrict__ C,
                                                                   int M, int N, int K, int tiles_m, int tiles_n) {
@@ -722,6 +762,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile128_splitk_ragged_k(const _
 }
 // C[i] = bf16(W[0][i] + W[1][i] + ... + W[splits-1][i]), 8 elements per work-item, partials added
 // in the order of their K ranges so the result does not depend on timing.
+template <bool kF16>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce(const float* __restrict__ W, __bf16* __restrict__ C, long total,
                                                           int splits) {
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
@@ -732,13 +773,14 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce(const float* __restric
         lo += p[0];
         hi += p[1];
     }
-    bf16x4 l = __builtin_convertvector(lo, bf16x4), h = __builtin_convertvector(hi, bf16x4);
+    bf16x4 l = round_to_elem<kF16>(lo), h = round_to_elem<kF16>(hi);
     *reinterpret_cast<bf16x8*>(C + i) = __builtin_shufflevector(l, h, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
 // Any shape: one wave per 32x32 output tile, operands fetched straight from global memory
 // with bounds checks (zero fill), no LDS.  Correct for every M, N, K; used when the shape
 // does not fit the tiled kernel.
+template <bool kF16>
 __global__ __launch_bounds__(256) void gemm_bf16_generic(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                          __bf16* __restrict__ C, int M, int N, int K, int tiles_n,
                                                          long total_tiles) {
@@ -762,13 +804,17 @@ __global__ __launch_bounds__(256) void gemm_bf16_generic(const __bf16* __restric
             a[e] = (m < M && k < K) ? A[m * K + k] : (__bf16)0.0f;
             b[e] = (n < N && k < K) ? B[(long)k * N + n] : (__bf16)0.0f;
         }
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
+        if constexpr (kF16) acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
+        else acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc, 0, 0, 0);
     }
     // lane l register e: row 8*(e/4) + 4*(l/32) + e%4, column l%32
 #pragma unroll
     for (int e = 0; e < 16; e++) {
         const long r = m0 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-        if (r < M && n < N) C[r * N + n] = (__bf16)acc[e];
+        if (r < M && n < N) {
+            if constexpr (kF16) C[r * N + n] = __builtin_bit_cast(__bf16, (_Float16)acc[e]);
+            else C[r * N + n] = (__bf16)acc[e];
+        }
     }
 }
 
@@ -909,7 +955,7 @@ int launch_gemm_bf16_swiglu(void* stream, const void* A, const void* B, void* C,
 }
 
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
-                     long batch, void* workspace, size_t workspace_bytes, bool b_transposed) {
+                     long batch, void* workspace, size_t workspace_bytes, bool b_transposed, bool f16) {
     using namespace mrk::dev;
     if (M <= 0 || N <= 0 || batch <= 0) return 0;
     if (batch > 65535) return (int)hipErrorInvalidValue;  // grid y extent
@@ -927,8 +973,10 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
         const bool small = variant == 4 || (variant != 3 && tm128 * tn * batch <= 256);
         const long tm = small ? tm128 : (M + kBM - 1) / kBM;
         const bool ragged_k = K % kBK != 0;
-        auto kernel = small ? (ragged_k ? gemm_bf16_nt_tile128_ragged_k : gemm_bf16_nt_tile128)
-                            : (ragged_k ? gemm_bf16_nt_tile256_ragged_k : gemm_bf16_nt_tile256);
+        auto kernel = f16 ? (small ? (ragged_k ? gemm_f16_nt_tile128_ragged_k : gemm_f16_nt_tile128)
+                                   : (ragged_k ? gemm_f16_nt_tile256_ragged_k : gemm_f16_nt_tile256))
+                          : (small ? (ragged_k ? gemm_bf16_nt_tile128_ragged_k : gemm_bf16_nt_tile128)
+                                   : (ragged_k ? gemm_bf16_nt_tile256_ragged_k : gemm_bf16_nt_tile256));
         kernel<<<dim3((unsigned)(tm * tn), (unsigned)batch), 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
                                                                           static_cast<__bf16*>(C), (int)M, (int)N, (int)K, (int)tm, (int)tn);
         return (int)hipGetLastError();
@@ -946,12 +994,12 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
             float* w = static_cast<float*>(workspace);
             const __bf16* a = static_cast<const __bf16*>(A);
             const __bf16* b = static_cast<const __bf16*>(B);
-            if (K % kBK == 0)
-                gemm_bf16_tile128_splitk<<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)tm128, (int)tn, (int)sp.kt_per_split);
-            else
-                gemm_bf16_tile128_splitk_ragged_k<<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)tm128, (int)tn, (int)sp.kt_per_split);
+            auto split_kernel = f16 ? (K % kBK == 0 ? gemm_f16_tile128_splitk : gemm_f16_tile128_splitk_ragged_k)
+                                    : (K % kBK == 0 ? gemm_bf16_tile128_splitk : gemm_bf16_tile128_splitk_ragged_k);
+            split_kernel<<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)tm128, (int)tn, (int)sp.kt_per_split);
             const long total = batch * M * N;
-            gemm_splitk_reduce<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>(w, static_cast<__bf16*>(C), total, (int)sp.splits);
+            auto reduce_kernel = f16 ? gemm_splitk_reduce<true> : gemm_splitk_reduce<false>;
+            reduce_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>(w, static_cast<__bf16*>(C), total, (int)sp.splits);
             return (int)hipGetLastError();
         }
         // variant 0: the 128-row tile when all its workgroups are resident at once (at most one per
@@ -964,16 +1012,18 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
         const __bf16* b = static_cast<const __bf16*>(B);
         __bf16* c = static_cast<__bf16*>(C);
         const bool ragged_k = K % kBK != 0;
-        if (small && !ragged_k) gemm_bf16_tile128<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
-        else if (small) gemm_bf16_tile128_ragged_k<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
-        else if (!ragged_k) gemm_bf16_tile256<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
-        else gemm_bf16_tile256_ragged_k<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+        auto kernel = f16 ? (small ? (ragged_k ? gemm_f16_tile128_ragged_k : gemm_f16_tile128)
+                                   : (ragged_k ? gemm_f16_tile256_ragged_k : gemm_f16_tile256))
+                          : (small ? (ragged_k ? gemm_bf16_tile128_ragged_k : gemm_bf16_tile128)
+                                   : (ragged_k ? gemm_bf16_tile256_ragged_k : gemm_bf16_tile256));
+        kernel<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
     } else {
         const long tm = (M + 31) / 32, tn = (N + 31) / 32;
         const long total = tm * tn;
         const long blocks = (total + 3) / 4;
         if (blocks > 0x7fffffffL) return (int)hipErrorInvalidValue;
-        gemm_bf16_generic<<<dim3((unsigned)blocks, (unsigned)batch), 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
+        auto generic = f16 ? gemm_bf16_generic<true> : gemm_bf16_generic<false>;
+        generic<<<dim3((unsigned)blocks, (unsigned)batch), 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
                                                            static_cast<__bf16*>(C), (int)M, (int)N, (int)K, (int)tn,
                                                            total);
     }

@@ -19,8 +19,11 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 // [batch, N, K] for batch > 1).  Same products in the same order, so the same bits as the [K, N]
 // form.  Tiled kernels only: shapes outside gemm_bf16_nt_supported (N or K not a multiple of 8,
 // so few output tiles that split-K would be used) are refused with hipErrorInvalidValue.
+// f16: operands and result are IEEE half precision instead of bf16 (the same kernels around
+// v_mfma_f32_16x16x32_f16; plain product only, the fused epilogues are bf16).
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
-                     long batch = 1, void* workspace = nullptr, size_t workspace_bytes = 0, bool b_transposed = false);
+                     long batch = 1, void* workspace = nullptr, size_t workspace_bytes = 0, bool b_transposed = false,
+                     bool f16 = false);
 bool gemm_bf16_nt_supported(long M, long N, long K, long batch);
 // c = bf16(float(bf16(a b)) + float(r)) with r of c's shape, added in the product kernel's epilogue
 // (same bits as the product followed by an elementwise add).  Supported for the shapes the tiled
@@ -92,7 +95,8 @@ int launch_copy(void* stream, const void* in, void* out, size_t bytes);
 // 256 x 256 x 64*k_steps GEMM tile without its memory traffic): 2 * 256 * 256 * 64 * k_steps
 // flops per workgroup.  `out` (>= 4 bytes) is never written in practice.
 // random_operands: 0 = smooth small operand values, 1 = hashed values in [-1.7, 1.7) like a product of
-// random matrices (operand bit toggling costs power, and the sustained clock follows the power).
+// random matrices (operand bit toggling costs power, and the sustained clock follows the power),
+// 2 = the same hashed values rounded to IEEE half precision, issued as v_mfma_f32_16x16x32_f16.
 int launch_mfma_ceiling(void* stream, void* out, long workgroups, long k_steps, int random_operands);
 
 }  // namespace mrk

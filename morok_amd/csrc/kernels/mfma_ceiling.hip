@@ -22,7 +22,9 @@ typedef float cal_f32x4 __attribute__((ext_vector_type(4)));
 // random matrices are.  The matrix pipes' power draw, and with it the clock the part sustains,
 // depends on how much the operand bits toggle.
 // (a template parameter, so that the set-up in front of the loop is straight-line code)
-template <bool random_operands>
+// half: the same stream of v_mfma_f32_16x16x32_f16 on the same values rounded to IEEE half
+// precision (eleven significant bits per operand instead of eight).
+template <bool random_operands, bool half = false>
 __global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ out, int k_steps, float seed) {
     const int lane = threadIdx.x & 63;
     cal_f32x4 acc[8][8];
@@ -46,8 +48,14 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ o
                 x ^= x >> 13;
                 unsigned y = x * 3266489917u;
                 y ^= y >> 16;
-                fa[ks][i][e] = (__bf16)(((float)(x >> 8) / 8388608.0f - 1.0f) * 1.7f);
-                fb[ks][i][e] = (__bf16)(((float)(y >> 8) / 8388608.0f - 1.0f) * 1.7f);
+                const float va = ((float)(x >> 8) / 8388608.0f - 1.0f) * 1.7f, vb = ((float)(y >> 8) / 8388608.0f - 1.0f) * 1.7f;
+                if (half) {
+                    fa[ks][i][e] = __builtin_bit_cast(__bf16, (_Float16)va);
+                    fb[ks][i][e] = __builtin_bit_cast(__bf16, (_Float16)vb);
+                } else {
+                    fa[ks][i][e] = (__bf16)va;
+                    fb[ks][i][e] = (__bf16)vb;
+                }
             } else {
                 fa[ks][i][e] = (__bf16)(seed * (float)(lane + e + i));
                 fb[ks][i][e] = (__bf16)(seed * (float)(lane - e - i));
@@ -62,7 +70,8 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(float* __restrict__ o
                 for (int jj = 0; jj < 8; jj++) {
                     const int j = (i & 1) ? 7 - jj : jj;
                     // written out, with the accumulator tied in place, as in the GEMM kernel
-                    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fb[ks][j]), "v"(fa[ks][i]));
+                    if (half) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fb[ks][j]), "v"(fa[ks][i]));
+                    else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fb[ks][j]), "v"(fa[ks][i]));
                 }
     }
     // the last results must have left the matrix pipe before the vector ALUs read them (the
@@ -90,7 +99,9 @@ int launch_mfma_ceiling(void* stream, void* out, long workgroups, long k_steps, 
     if (workgroups <= 0 || k_steps <= 0 || workgroups > 0x7fffffffL || k_steps > 0x7fffffffL || !out)
         return (int)hipErrorInvalidValue;
     (void)hipGetLastError();
-    if (random_operands)
+    if (random_operands == 2)
+        dev::mfma_ceiling_kernel<true, true><<<(unsigned)workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<float*>(out), (int)k_steps, 0.001f);
+    else if (random_operands)
         dev::mfma_ceiling_kernel<true><<<(unsigned)workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<float*>(out), (int)k_steps, 0.001f);
     else
         dev::mfma_ceiling_kernel<false><<<(unsigned)workgroups, 256, 0, static_cast<hipStream_t>(stream)>>>(static_cast<float*>(out), (int)k_steps, 0.001f);

@@ -464,6 +464,11 @@ class Ctx {
     // tensor-core instructions written as assembly (see wmma_wrapper): the register objects that
     // hold their accumulators, (DEFINE_REG id, elements), and how many RANGEs are open
     bool tied_wmma = false;
+    // workgroups whose x extent is a whole number of wavefronts: threadIdx.y / .z are the same for
+    // the 64 lanes of a wave (declared through readfirstlane, so the compiler keeps what derives
+    // from them in scalar registers)
+    bool wave_uniform_yz = false;
+    std::unordered_map<uint32_t, bool> uniform_memo;
     std::vector<std::pair<uint32_t, int64_t>> acc_regs;
     std::unordered_set<uint32_t> acc_loads_with_other_users;
     int range_depth = 0;
@@ -584,6 +589,7 @@ class HipRenderer final : public Renderer {
             return fail(kRenderError, "render: workgroup larger than 1024 work-items");
 
         Ctx ctx;
+        ctx.wave_uniform_yz = local[0] % 64 == 0 && local[1] * local[2] > 1;
         for (const UOp& u : nodes)
             for (uint32_t s : u.src) ctx.refs[s]++;
         ctx.escaping = scope_escaping(nodes, ctx.refs);
@@ -809,6 +815,48 @@ class HipRenderer final : public Renderer {
         }
     }
 
+    // Whether every lane of a wavefront computes the same value for this node: constants, kernel
+    // variables, workgroup ids, loop counters, the y / z work-item ids of workgroups whose x extent
+    // is a whole number of waves, and integer arithmetic over those.
+    template <class NodeFn>
+    bool wave_uniform(uint32_t id, NodeFn& node, Ctx& ctx) {
+        auto it = ctx.uniform_memo.find(id);
+        if (it != ctx.uniform_memo.end()) return it->second;
+        const UOp& n = node(id);
+        bool r = false;
+        switch (n.op) {
+            case Op::Const:
+            case Op::DefineVar:
+            case Op::Range: r = true; break;
+            case Op::Special: r = n.str[0] == 'g' || (n.str[4] != '0' && ctx.wave_uniform_yz); break;
+            case Op::Unary:
+            case Op::Binary:
+            case Op::Where:
+            case Op::MulAcc:
+            case Op::Cast:
+                r = !n.src.empty() && n.dtype.vcount <= 1;
+                for (uint32_t s : n.src) r = r && wave_uniform(s, node, ctx);
+                break;
+            default: break;
+        }
+        return ctx.uniform_memo[id] = r;
+    }
+    // The terms of an integer sum (a tree of ADDs), split into wave-uniform ones and the rest.
+    template <class NodeFn>
+    // A sum with per-lane terms is taken apart only where it is inlined into its consumer anyway
+    // (single use); a wave-uniform sum (`whole_uniform`) always: its terms live in scalar registers
+    // whether or not the sum itself has a name.
+    void split_sum(uint32_t id, NodeFn& node, Ctx& ctx, std::vector<uint32_t>* uniform, std::vector<uint32_t>* varying, bool whole_uniform = false) {
+        const UOp& n = node(id);
+        if (n.op == Op::Binary && static_cast<BinaryOp>(n.sub) == BinaryOp::Add && n.src.size() == 2 && n.dtype.vcount <= 1 &&
+            (whole_uniform || (!wave_uniform(id, node, ctx) && ctx.refs[id] <= 1))) {
+            split_sum(n.src[0], node, ctx, uniform, varying, whole_uniform);
+            split_sum(n.src[1], node, ctx, uniform, varying, whole_uniform);
+            return;
+        }
+        (wave_uniform(id, node, ctx) ? uniform : varying)->push_back(id);
+    }
+
     template <class NodeFn>
     int render_uop(const UOp& u, NodeFn& node, Ctx& ctx) {
         auto S = [&](size_t i) -> const std::string& { return ctx.get(u.src[i]); };
@@ -847,8 +895,12 @@ class HipRenderer final : public Renderer {
                 const char* builtin = u.str[0] == 'g' ? "blockIdx" : "threadIdx";
                 const char axis = "xyz"[u.str[4] - '0'];
                 const int64_t extent = node(u.src[0]).arg_i;
-                ctx.body.push_back(ctx.indent() + fmt("const %s %s = %s.%c; /* %" PRId64 " */", c_scalar(u.dtype.scalar),
-                                                      u.str.c_str(), builtin, axis, extent));
+                if (u.str[0] == 'l' && axis != 'x' && ctx.wave_uniform_yz)
+                    ctx.body.push_back(ctx.indent() + fmt("const %s %s = __builtin_amdgcn_readfirstlane(%s.%c); /* %" PRId64 ", the same for a whole wave */",
+                                                          c_scalar(u.dtype.scalar), u.str.c_str(), builtin, axis, extent));
+                else
+                    ctx.body.push_back(ctx.indent() + fmt("const %s %s = %s.%c; /* %" PRId64 " */", c_scalar(u.dtype.scalar),
+                                                          u.str.c_str(), builtin, axis, extent));
                 ctx.names[u.id] = u.str;
                 return kOk;
             }
@@ -1068,26 +1120,58 @@ class HipRenderer final : public Renderer {
                 // compiler's wait-count bookkeeping, WAIT_ASYNC is its only ordering.  The destination
                 // is formed as the array's own local-memory offset plus an integer byte offset: cast
                 // back from a generic pointer it would carry a null check per copy.
-                std::string dst;
+                auto sum_of = [&](const std::vector<uint32_t>& terms) {
+                    std::string e;
+                    for (uint32_t t : terms) e += (e.empty() ? "" : " + ") + ctx.get(t);
+                    return e.empty() ? std::string("0") : "(" + e + ")";
+                };
                 const UOp& li = node(u.src[1]);
-                if (li.op == Op::Index && li.src.size() == 2 && !li.sub && node(li.src[0]).op == Op::DefineLocal)
-                    dst = "(unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + ctx.get(li.src[0]) + ") + (unsigned)(" +
-                          ctx.get(li.src[1]) + ") * " + std::to_string(scalar_bytes(l->dtype.scalar) * l->dtype.vcount) + "u";
-                else
-                    dst = "(unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + S(1) + ")";
-                // source: the buffer's (scalar) base plus a 32-bit byte offset per lane where the buffer
-                // is known to be smaller than 4 GiB (two vector instructions fewer per copy than a
-                // 64-bit address per lane), else the full address
                 const UOp& gi = node(u.src[0]);
+                const int64_t lbytes = static_cast<int64_t>(scalar_bytes(l->dtype.scalar)) * l->dtype.vcount;
                 const int64_t gbytes = static_cast<int64_t>(scalar_bytes(g->dtype.scalar)) * g->dtype.vcount;
-                if (gi.op == Op::Index && gi.src.size() == 2 && !gi.sub && node(gi.src[0]).op == Op::Param && g->dtype.ptr_size > 0 &&
-                    g->dtype.ptr_size * gbytes <= (int64_t(1) << 32))
-                    ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, %2\" : : \"s\"(" +
-                                       "__builtin_amdgcn_readfirstlane(" + dst + ")), \"v\"((unsigned)(" + ctx.get(gi.src[1]) + ") * " +
-                                       std::to_string(gbytes) + "u), \"s\"(" + ctx.get(gi.src[0]) + ") : \"m0\", \"memory\");");
-                else
-                    ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, off\" : : \"s\"(" +
-                                       "__builtin_amdgcn_readfirstlane(" + dst + ")), \"v\"((const char*)(" + S(0) + ")) : \"m0\", \"memory\");");
+                const bool plain_dst = li.op == Op::Index && li.src.size() == 2 && !li.sub && node(li.src[0]).op == Op::DefineLocal;
+                const bool plain_src = gi.op == Op::Index && gi.src.size() == 2 && !gi.sub && node(gi.src[0]).op == Op::Param && g->dtype.ptr_size > 0 &&
+                                       g->dtype.ptr_size * gbytes <= (int64_t(1) << 32);
+                if (plain_dst && plain_src && wave_uniform(li.src[1], node, ctx)) {
+                    // The form of the hand-written kernels: the destination is wave-uniform, so M0 is written
+                    // by the one scalar addition that forms it (the array's base plus the terms that do not
+                    // change from copy to copy on one side, the rest on the other); the source is the
+                    // buffer's base advanced by the wave-uniform terms of the index in scalar registers
+                    // plus the remaining per-lane terms as a 32-bit byte offset, which the compiler hoists
+                    // out of the loop when they do not depend on it.
+                    std::vector<uint32_t> du, dv, su, sv;
+                    split_sum(li.src[1], node, ctx, &du, &dv, true);
+                    split_sum(gi.src[1], node, ctx, &su, &sv);
+                    std::vector<uint32_t> d_first(du.begin(), du.begin() + (du.size() + 1) / 2), d_rest(du.begin() + (du.size() + 1) / 2, du.end());
+                    const std::string m0_a = "(unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + ctx.get(li.src[0]) + ") + (unsigned)" +
+                                             sum_of(d_first) + " * " + std::to_string(lbytes) + "u";
+                    const std::string m0_b = "(unsigned)" + sum_of(d_rest) + " * " + std::to_string(lbytes) + "u";
+                    const std::string src_ops = "\"v\"((unsigned)" + sum_of(sv) + " * " + std::to_string(gbytes) + "u), \"s\"(" + ctx.get(gi.src[0]) + " + " +
+                                                sum_of(su) + ")";
+                    if (d_rest.empty())
+                        ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, %2\" : : \"s\"(" + m0_a +
+                                           "), " + src_ops + " : \"m0\", \"memory\");");
+                    else
+                        ctx.body.push_back(ctx.indent() + "asm volatile(\"s_add_u32 m0, %0, %1\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %2, %3\" : : \"s\"(" + m0_a +
+                                           "), \"s\"(" + m0_b + "), " + src_ops + " : \"m0\", \"scc\", \"memory\");");
+                } else {
+                    std::string dst;
+                    if (plain_dst)
+                        dst = "(unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + ctx.get(li.src[0]) + ") + (unsigned)(" +
+                              ctx.get(li.src[1]) + ") * " + std::to_string(lbytes) + "u";
+                    else
+                        dst = "(unsigned)(unsigned long long)(__attribute__((address_space(3))) char*)(" + S(1) + ")";
+                    // source: the buffer's (scalar) base plus a 32-bit byte offset per lane where the buffer
+                    // is known to be smaller than 4 GiB (two vector instructions fewer per copy than a
+                    // 64-bit address per lane), else the full address
+                    if (plain_src)
+                        ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, %2\" : : \"s\"(" +
+                                           "__builtin_amdgcn_readfirstlane(" + dst + ")), \"v\"((unsigned)(" + ctx.get(gi.src[1]) + ") * " +
+                                           std::to_string(gbytes) + "u), \"s\"(" + ctx.get(gi.src[0]) + ") : \"m0\", \"memory\");");
+                    else
+                        ctx.body.push_back(ctx.indent() + "asm volatile(\"s_mov_b32 m0, %0\\n\\ts_nop 0\\n\\tglobal_load_lds_dwordx4 %1, off\" : : \"s\"(" +
+                                           "__builtin_amdgcn_readfirstlane(" + dst + ")), \"v\"((const char*)(" + S(0) + ")) : \"m0\", \"memory\");");
+                }
                 // next to written-out tensor-core instructions the copy stays where the kernel puts it
                 // (a builder that spreads copies over a stretch of them means exactly that placement)
                 if (ctx.tied_wmma) ctx.body.push_back(ctx.indent() + "__builtin_amdgcn_sched_barrier(0);");

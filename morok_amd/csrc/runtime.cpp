@@ -699,12 +699,13 @@ int beam_search_wmma_matmul(const Device& dev, const TensorCore& tc, int tc_inde
             o.waves_m = sh[0], o.waves_n = sh[1], o.up_m = sh[2], o.up_n = sh[3];
             seeds.push_back(o);
         }
-        for (WmmaLdsOpts o : seeds) {
-            o.unroll_k = 0;
-            o.stages = 2;
-            double ms;
-            if (time_one(o, &ms)) next.emplace_back(ms, o);
-        }
+        for (WmmaLdsOpts o : seeds)
+            for (int stages : {2, 3}) {
+                o.unroll_k = 0;
+                o.stages = stages;
+                double ms;
+                if (time_one(o, &ms)) next.emplace_back(ms, o);
+            }
         beam = next;
         keep_best(beam);
     }

@@ -772,7 +772,7 @@ int build_wmma_matmul_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t
 static bool wmma_async_tile(const TensorCore& tc, const WmmaLdsOpts& o, int* bm, int* bn);
 
 bool wmma_lds_tile(const TensorCore& tc, const WmmaLdsOpts& o, int64_t K, int* bm, int* bn, int* bk) {
-    if (o.stages == 2) {
+    if (o.stages == 2 || o.stages == 3) {
         *bk = 64;
         return wmma_async_tile(tc, o, bm, bn);
     }
@@ -795,7 +795,7 @@ bool wmma_lds_tile(const TensorCore& tc, const WmmaLdsOpts& o, int64_t K, int* b
 static bool wmma_async_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, int64_t N, int64_t K);
 
 bool wmma_lds_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, int64_t M, int64_t N, int64_t K) {
-    if (o.stages == 2) return wmma_async_opts_valid(tc, o, M, N, K);
+    if (o.stages == 2 || o.stages == 3) return wmma_async_opts_valid(tc, o, M, N, K);
     if (o.stages != 0) return false;
     if (tc.dtype_in != Scalar::BFloat16 && tc.dtype_in != Scalar::Float16) return false;  // 8 elements per 16-byte copy
     int BM, BN, BK;
@@ -841,7 +841,9 @@ static bool wmma_async_opts_valid(const TensorCore& tc, const WmmaLdsOpts& o, in
     if (BN < 64 || BN > 512) return false;              // whole granule groups per row, at most one row per copy
     if ((BM / 8) % W || (BN / 8) % W) return false;     // every wave copies the same number of 1 KB chunks
     if ((BM / 8 + BN / 8) / W > 32) return false;
-    if (2 * (BM + BN) * 64 * 2 > 160 * 1024) return false;  // two stages of both tiles in 160 KB
+    // two stages of the A tile and two (stages = 2) or three (stages = 3) of the B tile in 160 KB
+    if ((2 * BM + (o.stages == 3 ? 3 : 2) * BN) * 64 * 2 > 160 * 1024) return false;
+    if (o.stages == 3 && (W > 4 || K / 64 <= 2)) return false;  // the three-stage schedule exists for the one-wave-per-SIMD form only
     return true;
 }
 
@@ -877,6 +879,12 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
     const int KS = 64 / tk, HS = KS / 2;  // tensor-core K steps per 64-deep tile, per half of it
     const int64_t KT = K / 64, tiles_m = M / BM, tiles_n = N / BN, T = tiles_m * tiles_n;
     const int A_STAGE = BM * 64, B_STAGE = 64 * BN;  // elements
+    // stages = 3: a third stage of the B tile, as in the hand-written kernel.  The copies of tile
+    // r + 2 then split over the whole step: its B chunks go out behind the first half's
+    // tensor-core instructions (into the stage tile r - 1 left one barrier ago), its A chunks
+    // behind the second half's (into the stage tile r has just left), so that the vector-memory
+    // path sees a copy every few instructions instead of all of a tile's copies in half a step.
+    const int BST = opts.stages == 3 ? 3 : 2;
     const int CA = BM / 8 / W, CB = BN / 8 / W, PRB = BN / 8;
     KernelBuilder b;
     b.enable_cse();
@@ -910,7 +918,7 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
     uint32_t wy = b.idiv(wave, WN), wx = b.imod(wave, WN);
     uint32_t lr = b.imod(lane, TD), lgk = b.idiv(lane, TD);  // row / column inside a tile, k group
     uint32_t i16 = b.imod(lane, 16);                         // lane inside its group of 16 (transposing loads)
-    uint32_t sA = b.define_local(0, tc.dtype_in, 2LL * A_STAGE), sB = b.define_local(1, tc.dtype_in, 2LL * B_STAGE);
+    uint32_t sA = b.define_local(0, tc.dtype_in, 2LL * A_STAGE), sB = b.define_local(1, tc.dtype_in, (int64_t)BST * B_STAGE);
 
     // copies: per wave CA chunks of A and CB chunks of B per tile
     std::vector<uint32_t> a_src(CA), a_dst(CA), b_src(CB), b_dst(CB);
@@ -933,9 +941,10 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
         b_dst[q] = b.imul(chunk, 512);
     }
     // copy q (of CA + CB) of tile kt into stage `stage`; kt, stage: nodes (uniform)
-    auto copy_one = [&](int q, uint32_t kt, uint32_t stage) {
+    // (stage_b: the B stage when it differs from the A stage; 0 = the same)
+    auto copy_one = [&](int q, uint32_t kt, uint32_t stage, uint32_t stage_b = 0) {
         if (q < CA) b.async_copy(b.index(a, b.iadd(a_src[q], b.imul(kt, 64))), b.index(sA, b.iadd(a_dst[q], b.imul(stage, A_STAGE))));
-        else b.async_copy(b.index(bmat, b.iadd(b_src[q - CA], b.imul(kt, 64 * N))), b.index(sB, b.iadd(b_dst[q - CA], b.imul(stage, B_STAGE))));
+        else b.async_copy(b.index(bmat, b.iadd(b_src[q - CA], b.imul(kt, 64 * N))), b.index(sB, b.iadd(b_dst[q - CA], b.imul(stage_b ? stage_b : stage, B_STAGE))));
     };
     auto copy_tile = [&](uint32_t kt, uint32_t stage) {
         for (int q = 0; q < CA + CB; q++) copy_one(q, kt, stage);
@@ -1013,7 +1022,10 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
     uint32_t r = b.range(KT, 0, AxisType::Reduce);
     {
         uint32_t st = b.imod(r, 2), sn = bin(BinaryOp::Sub, b.ci(1), st);
-        uint32_t oa = b.imul(st, A_STAGE), ob = b.imul(st, B_STAGE), na = b.imul(sn, A_STAGE), nb = b.imul(sn, B_STAGE);
+        // B stages of tile r, r + 1 and (three stages) the one tile r + 2 goes to
+        uint32_t sb0 = BST == 3 ? b.imod(r, 3) : st, sb1 = BST == 3 ? b.imod(b.iadd(r, b.ci(1)), 3) : sn;
+        uint32_t sb2 = BST == 3 ? b.imod(b.iadd(r, b.ci(2)), 3) : st;
+        uint32_t oa = b.imul(st, A_STAGE), ob = b.imul(sb0, B_STAGE), na = b.imul(sn, A_STAGE), nb = b.imul(sb1, B_STAGE);
         std::vector<uint32_t> f1a(HS * um), f1b(HS * un), f0a(HS * um), f0b(HS * un);
         const int total = HS * um * un;  // tensor-core instructions per half step
         if (W <= 4 && KT > 2) {
@@ -1033,27 +1045,35 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             }
             for (size_t i = 0; i < fa0.size(); i++) f0a[i] = b.load(fa0[i]);
             for (size_t j = 0; j < fb0.size(); j++) f0b[j] = b.load(fb0[j]);
+            uint32_t kt2 = bin(BinaryOp::Sub, b.ci(KT - 1), bin(BinaryOp::Max, bin(BinaryOp::Sub, b.ci(KT - 3), r), b.ci(0)));
             size_t done1 = 0;
+            int issued_b = 0;
+            const int left1 = std::max(1, total - (int)reads1.size());
+            const int every1 = std::max(1, left1 / std::max(1, CB));
             mfmas(f0a, f0b, [&](int n) {
                 if (done1 < reads1.size()) reads1[done1++]();
-                if (n == total - 1)
+                else if (BST == 3 && (n - (int)reads1.size()) % every1 == 0 && issued_b < CB) copy_one(CA + issued_b++, kt2, st, sb2);
+                if (n == total - 1) {
                     while (done1 < reads1.size()) reads1[done1++]();
+                    while (BST == 3 && issued_b < CB) copy_one(CA + issued_b++, kt2, st, sb2);
+                }
             });
-            // tile r + 1 has landed in the other stage and, behind the barrier, nobody reads this
-            // stage any more
-            b.wait_async(0);
+            // tile r + 1 has landed in the other stage (with three stages the B chunks of tile r + 2,
+            // the newest copies, may still be on their way) and, behind the barrier, nobody reads
+            // this A stage any more
+            b.wait_async(BST == 3 ? CB : 0);
             b.barrier();
-            uint32_t kt2 = bin(BinaryOp::Sub, b.ci(KT - 1), bin(BinaryOp::Max, bin(BinaryOp::Sub, b.ci(KT - 3), r), b.ci(0)));
             size_t done0 = 0;
             int issued = 0;
+            const int second = BST == 3 ? CA : cpw;  // copies behind the second half: A only, or the whole tile
             const int left = std::max(1, total - (int)reads0.size());
-            const int every = std::max(1, left / cpw);
+            const int every = std::max(1, left / second);
             mfmas(f1a, f1b, [&](int n) {
                 if (done0 < reads0.size()) reads0[done0++]();
-                else if ((n - (int)reads0.size()) % every == 0 && issued < cpw) copy_one(issued++, kt2, st);
+                else if ((n - (int)reads0.size()) % every == 0 && issued < second) copy_one(issued++, kt2, st);
                 if (n == total - 1) {
                     while (done0 < reads0.size()) reads0[done0++]();
-                    while (issued < cpw) copy_one(issued++, kt2, st);
+                    while (issued < second) copy_one(issued++, kt2, st);
                 }
             });
         } else {
@@ -1152,8 +1172,9 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
 
 int build_wmma_matmul_lds_kernel(const TensorCore& tc, int64_t M, int64_t N, int64_t K, Scalar out, const WmmaLdsOpts& opts,
                                  LinearKernel* k) {
-    if (opts.stages == 2) return build_wmma_matmul_async_kernel(tc, M, N, K, out, opts, k);
-    if (opts.stages != 0) return fail(kInvalidArgument, "tensor-core matmul (LDS): stages must be 0 (through registers) or 2 (direct copies)");
+    if (opts.stages == 2 || opts.stages == 3) return build_wmma_matmul_async_kernel(tc, M, N, K, out, opts, k);
+    if (opts.stages != 0)
+        return fail(kInvalidArgument, "tensor-core matmul (LDS): stages must be 0 (through registers), 2 (direct copies) or 3 (direct copies, a third stage of the second operand)");
     const int tn = tc.dims[0], tm = tc.dims[1], tk = tc.dims[2];
     if (tc.threads != 64 || tm != 16 || tn != 16) return fail(kInvalidArgument, "tensor-core matmul (LDS): only 64-lane 16x16 tensor cores are lowered");
     int BM, BN, BK;

@@ -240,7 +240,10 @@ struct WmmaLdsOpts {
     // local memory filled by direct global -> local copies (ASYNC_COPY / WAIT_ASYNC), B fragments
     // read with the transposing load (LOAD_TR), one barrier per 64-deep K step, workgroups
     // mapped to tiles in compact blocks per XCD, result rows written as 8-byte vectors.  Needs a
-    // 16x16x32 tensor core, M, N, K divisible by the tile and a K step of 64.
+    // 16x16x32 tensor core, M, N, K divisible by the tile and a K step of 64.  3: the same with a
+    // third stage of the second operand's tile (workgroups of at most four waves, more than two K
+    // steps): the copies of tile r + 2 are spread over the whole of step r, B chunks behind the
+    // first half's tensor-core instructions, A chunks behind the second half's.
     int stages = 0;
 };
 // Extents of the workgroup tile these choices give (false if the choices are not buildable at all)

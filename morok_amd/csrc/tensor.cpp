@@ -1214,10 +1214,10 @@ struct Scheduler {
             case HintKind::Matmul: {
                 const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
                 if (a->dtype != w->dtype) return false;
-                if (a->dtype == Scalar::BFloat16) {
+                if (a->dtype == Scalar::BFloat16 || a->dtype == Scalar::Float16) {  // the hand-written 16-bit products
                     // [..., M, K] x [K, N] is one product over the flattened leading axes;
                     // equal leading axes on both sides are that many products in one launch
-                    if (n->dtype != Scalar::BFloat16 || n->numel() == 0 || a->shape.size() < 2) return false;
+                    if (n->dtype != a->dtype || n->numel() == 0 || a->shape.size() < 2) return false;
                     if (w->shape.size() == 2) return true;
                     if (w->shape.size() != a->shape.size()) return false;
                     int64_t batch = 1;
@@ -1274,7 +1274,8 @@ struct Scheduler {
         // the chip (one 256 x 256 workgroup or two smaller ones per CU), else the smallest
         static const int direct[][5] = {{2, 2, 8, 8, 256}, {2, 4, 8, 4, 256}, {2, 2, 4, 4, 512}, {2, 2, 4, 2, 512}, {2, 2, 2, 2, 0}};
         for (auto& c : direct) {
-            WmmaLdsOpts t{c[0], c[1], c[2], c[3], 0, 2};
+            WmmaLdsOpts t{c[0], c[1], c[2], c[3], 0, 3};  // a third B stage where the schedule and the 160 KB allow it
+            if (!wmma_lds_opts_valid(tc, t, M, N, K)) t.stages = 2;
             if (!wmma_lds_opts_valid(tc, t, M, N, K)) continue;
             int bm, bn, bk;
             wmma_lds_tile(tc, t, K, &bm, &bn, &bk);
@@ -1308,8 +1309,8 @@ struct Scheduler {
         if (n->hint != HintKind::Matmul || n->numel() == 0) return false;
         const TensorNode *a = n->hint_inputs[0].get(), *w = n->hint_inputs[1].get();
         const Scalar dt = n->dtype;
-        // bf16 has hand-written kernels (taken while they are switched on); half precision has none
-        if (dt == Scalar::BFloat16 ? g_fusion : dt != Scalar::Float16) return false;
+        // both 16-bit float types have hand-written kernels, taken while those are switched on
+        if ((dt != Scalar::BFloat16 && dt != Scalar::Float16) || g_fusion) return false;
         if (a->dtype != dt || w->dtype != dt) return false;
         if (a->shape.size() != 2 || w->shape.size() != 2) return false;
         const auto tcs = cdna4_tensor_cores();
@@ -1407,7 +1408,8 @@ struct Scheduler {
     TensorNode* transposed_weight(const TensorNode* mm) const {
         if (!g_fusion) return nullptr;
         TensorNode* w = mm->hint_inputs[1].get();
-        if (w->buffer || w->kind != TKind::Permute || w->dtype != Scalar::BFloat16 || w->shape.size() != 2 || w->arg.size() != 2 ||
+        if (w->buffer || w->kind != TKind::Permute || (w->dtype != Scalar::BFloat16 && w->dtype != Scalar::Float16) || w->shape.size() != 2 ||
+            w->arg.size() != 2 ||
             w->arg[0] != 1 || w->arg[1] != 0)
             return nullptr;
         TensorNode* wt = w->src[0].get();
@@ -1909,7 +1911,7 @@ struct Scheduler {
         if (n->hint == HintKind::Sdpa) return materialize_attention(n, n, dense_strides(n->shape));
         std::shared_ptr<Buffer> wbuf;  // a bf16 product's second operand, and its layout
         bool nt = false;
-        if (n->hint == HintKind::Matmul && n->hint_inputs[0]->dtype == Scalar::BFloat16) {
+        if (n->hint == HintKind::Matmul && (n->hint_inputs[0]->dtype == Scalar::BFloat16 || n->hint_inputs[0]->dtype == Scalar::Float16)) {
             int64_t M, N, K, batch;
             matmul_extents(n, &M, &N, &K, &batch);
             MRK_TRY(materialize(n->hint_inputs[0].get()));
@@ -1927,18 +1929,18 @@ struct Scheduler {
             const int64_t K = a->shape.back(), N = w->shape.back();
             int64_t M = a->shape[a->shape.size() - 2], batch = 1;
             for (size_t i = 0; i + 2 < a->shape.size(); i++) (w->shape.size() == 2 ? M : batch) *= a->shape[i];
-            if (a->dtype == Scalar::BFloat16) {
+            if (a->dtype == Scalar::BFloat16 || a->dtype == Scalar::Float16) {
                 // few output tiles against a long K: scratch for split-K partials, an intermediate
                 // of the plan like any other (lazily allocated, placed by the memory planner)
                 const size_t ws = gemm_bf16_workspace_bytes(M, N, K, batch);
+                const std::string kind = a->dtype == Scalar::Float16 ? "gemm_f16" : "gemm_bf16";
                 if (nt) {
-                    rc = builtin("gemm_bf16_nt", {M, N, K}, {out, a->buffer, wbuf});
+                    rc = builtin((kind + "_nt").c_str(), {M, N, K}, {out, a->buffer, wbuf});
                 } else if (ws) {
                     auto scratch = std::make_shared<Buffer>(dev->allocator, ws, BufferOptions());
-                    rc = builtin("gemm_bf16", {M, N, K, batch, static_cast<int64_t>(ws)}, {out, a->buffer, wbuf, scratch});
+                    rc = builtin(kind.c_str(), {M, N, K, batch, static_cast<int64_t>(ws)}, {out, a->buffer, wbuf, scratch});
                 } else {
-                    rc = batch == 1 ? builtin("gemm_bf16", {M, N, K}, {out, a->buffer, wbuf})
-                                    : builtin("gemm_bf16", {M, N, K, batch}, {out, a->buffer, wbuf});
+                    rc = batch == 1 ? builtin(kind.c_str(), {M, N, K}, {out, a->buffer, wbuf}) : builtin(kind.c_str(), {M, N, K, batch}, {out, a->buffer, wbuf});
                 }
             } else {
                 // MOROK_BEAM=<width> selects the LOCAL/UPCAST/UNROLL choices by timed search

@@ -43,6 +43,23 @@ def gemm_bf16_nt(a, bt, c, m, n, k, device_id=0):
     check(lib.mrk_hip_gemm_bf16_nt(device_id, _p(a), _p(bt), _p(c), m, n, k))
 
 
+def gemm_f16(a, b, c, m, n, k, device_id=0):
+    """c[m,n] = a[m,k] @ b[k,n] on IEEE half precision operands, f32 accumulate, f16 result: the
+    hand-written tiled kernels around v_mfma_f32_16x16x32_f16 (Tensor::matmul on f16)."""
+    _need(a, m * k * 2, "gemm A")
+    _need(b, k * n * 2, "gemm B")
+    _need(c, m * n * 2, "gemm C")
+    check(lib.mrk_hip_gemm_f16(device_id, _p(a), _p(b), _p(c), m, n, k))
+
+
+def gemm_f16_nt(a, bt, c, m, n, k, device_id=0):
+    """c[m,n] = a[m,k] @ bt[n,k]^T on f16 operands (second operand as a Linear layer stores it)."""
+    _need(a, m * k * 2, "gemm_f16_nt a")
+    _need(bt, n * k * 2, "gemm_f16_nt bt")
+    _need(c, m * n * 2, "gemm_f16_nt c")
+    check(lib.mrk_hip_gemm_f16_nt(device_id, _p(a), _p(bt), _p(c), m, n, k))
+
+
 def gemm_bf16_noalloc(a, b, c, m, n, k, device_id=0):
     """gemm_bf16 without any device allocation: split-K partials go to the library's fixed
     device scratch (for callers under graph capture or in loops that must not allocate)."""
@@ -165,4 +182,4 @@ def mfma_ceiling(scratch, workgroups, k_steps, device_id=0, random_operands=True
     """MFMA-only calibration kernel: the matrix-instruction stream of `workgroups` 256x256 GEMM
     tiles of depth 64 * k_steps, from registers (2 * 256 * 256 * 64 * k_steps flops each)."""
     _need(scratch, 4, "mfma_ceiling scratch")
-    check(lib.mrk_hip_mfma_ceiling(device_id, _p(scratch), workgroups, k_steps, int(random_operands)))
+    check(lib.mrk_hip_mfma_ceiling(device_id, _p(scratch), workgroups, k_steps, 2 if random_operands == "f16" else int(random_operands)))

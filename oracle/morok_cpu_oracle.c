@@ -25,6 +25,8 @@
  *   orc_embedding_*       pinned: the reference's row-gather cases (bit exact)
  *   orc_sdpa_*            pinned: causal row 0 == V[0], uniform-K running mean, S=1, float64 SDPA
  *   orc_sdpa_bf16_ex      attn_mask / softcap: unpinned by reference tests; closed forms, identities with the causal path, float64
+ *   orc_gemm_f16          parity unpinned by reference tests (no f16 matmul test upstream); conversions pinned over every
+ *                         code against numpy's IEEE half, the product by definition vs float64
  *   orc_gemm_bf16         parity unpinned by reference tests (no bf16 matmul test upstream);
  *                         pinned by definition on bf16-rounded inputs vs float64, identity/ones cases
  *   orc_silu_mul_*, orc_decoder_block_bf16
@@ -201,6 +203,73 @@ void orc_gemm_bf16(const bf16_t* A, const bf16_t* B, bf16_t* C, int M, int N, in
     for (int t = 0; t < threads; t++) {
         float* acc = (float*)malloc(sizeof(float) * (size_t)(N > 0 ? N : 1));
         gemm_bf16_slice(A, B, C, M, N, K, literal, t, threads, acc);
+        free(acc);
+    }
+}
+
+/* The same product on IEEE half precision operands (Tensor::matmul on f16 inputs with the
+ * tensor-core rewrite, schedule/src/optimizer/renderer.rs:724-733: f16 x f16 products, exact in
+ * f32, accumulated in f32 along k, the result rounded once to f16, ties to even, subnormals
+ * kept).  No matmul test of the reference uses f16: pinned by definition against float64 and
+ * the conversions over every code in tests/test_oracle.py. */
+typedef uint16_t f16_t;
+static inline float f16_to_f32(f16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16, exp = (h >> 10) & 0x1fu, man = h & 0x3ffu, u;
+    if (exp == 0) {
+        if (man == 0) {
+            u = sign;
+        } else { /* subnormal: man * 2^-24, exact in f32 */
+            float f = (float)man * 5.9604644775390625e-08f;
+            memcpy(&u, &f, 4);
+            u |= sign;
+        }
+    } else if (exp == 31) {
+        u = sign | 0x7f800000u | (man << 13);
+    } else {
+        u = sign | ((exp + 112u) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+static inline f16_t f32_to_f16(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (f16_t)(sign | 0x7e00u);  /* NaN */
+    if (a >= 0x47800000u) return (f16_t)(sign | 0x7c00u); /* >= 65536 (and inf): inf; 65520..65536 handled below */
+    if (a < 0x38800000u) {                                 /* below the smallest normal 2^-14: fixed point in units of 2^-24 */
+        float mag;
+        memcpy(&mag, &a, 4);
+        /* mag * 2^24 is exact; rintf rounds half to even in the default rounding mode */
+        return (f16_t)(sign | (uint16_t)rintf(mag * 16777216.0f));
+    }
+    /* normal range: round the 13 dropped mantissa bits to nearest even; a carry may run into the
+     * exponent, which is exactly the next binade (or infinity from 65520 on) */
+    uint32_t r = a - 0x38000000u; /* rebias exponent 127 -> 15 */
+    const uint32_t lsb = (r >> 13) & 1u;
+    r += 0xfffu + lsb;
+    return (f16_t)(sign | (uint16_t)(r >> 13));
+}
+void orc_f16_to_f32(const f16_t* in, float* out, long n) {
+    for (long i = 0; i < n; i++) out[i] = f16_to_f32(in[i]);
+}
+void orc_f32_to_f16(const float* in, f16_t* out, long n) {
+    for (long i = 0; i < n; i++) out[i] = f32_to_f16(in[i]);
+}
+void orc_gemm_f16(const f16_t* A, const f16_t* B, f16_t* C, int M, int N, int K, int threads) {
+    if (threads < 1) threads = 1;
+#pragma omp parallel for num_threads(threads) schedule(static, 1)
+    for (int m = 0; m < M; m++) {
+        float* acc = (float*)malloc(sizeof(float) * (size_t)(N > 0 ? N : 1));
+        for (int n = 0; n < N; n++) acc[n] = 0.0f;
+        for (int k = 0; k < K; k++) {
+            const float a = f16_to_f32(A[(size_t)m * K + k]);
+            const f16_t* b = B + (size_t)k * N;
+            for (int n = 0; n < N; n++) acc[n] = fmaf(a, f16_to_f32(b[n]), acc[n]);
+        }
+        for (int n = 0; n < N; n++) C[(size_t)m * N + n] = f32_to_f16(acc[n]);
         free(acc);
     }
 }

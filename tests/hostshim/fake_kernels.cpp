@@ -10,8 +10,8 @@ int launch_softmax_f32(void* stream, const void*, void*, long, long, int) {
     return 0;
 }
 size_t gemm_bf16_workspace_bytes(long, long, long, long) { return 0; }
-int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, long, int, long, void*, size_t, bool b_transposed) {
-    mrk_shim_note_launch(stream, b_transposed ? "gemm_bf16_nt" : "gemm_bf16");
+int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, long, int, long, void*, size_t, bool b_transposed, bool f16) {
+    mrk_shim_note_launch(stream, f16 ? (b_transposed ? "gemm_f16_nt" : "gemm_f16") : b_transposed ? "gemm_bf16_nt" : "gemm_bf16");
     return 0;
 }
 bool gemm_bf16_nt_supported(long M, long N, long K, long batch) {

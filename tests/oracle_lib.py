@@ -64,6 +64,15 @@ class Oracle:
                                C.c_int(t))
         return c
 
+    def gemm_f16(self, a, b, threads=None):
+        """a [M, K], b [K, N] numpy float16 -> float16 [M, N] (f32 accumulate along k, one rounding)."""
+        M, K = a.shape
+        N = b.shape[1]
+        a, b = np.ascontiguousarray(a, np.float16), np.ascontiguousarray(b, np.float16)
+        c = np.empty((M, N), np.float16)
+        self.lib.orc_gemm_f16(_ptr(a), _ptr(b), _ptr(c), C.c_int(M), C.c_int(N), C.c_int(K), C.c_int(threads or self.max_threads))
+        return c
+
     def sdpa_bf16(self, q, k, v, scale, causal=True, policy=0, threads=None):
         B, H, Sq, D = q.shape
         Sk = k.shape[2]

@@ -329,7 +329,13 @@ def test_tensor_fused_kernel_selection(T, shim):
     m = zeros(T, (128, 40)).matmul(zeros(T, (40, 64))).realize()
     assert len(m.kernels()) == 1 and m.kernels()[0] == "r_128_64_40"  # scheduled f32 matmul
     h = zeros(T, (256, 128), np.float16).matmul(zeros(T, (128, 192), np.float16)).realize()
-    assert h.kernels() == ["r_tc_256_192_128"] and "mfma_f32_16x16x32_f16" in T.last_kernel_sources()[0]   # half: the WMMA route
+    assert h.kernels() == ["gemm_f16_256_192_128"] and shim.mrk_shim_last_kernel() == b"gemm_f16"     # half: hand-written too
+    hw = zeros(T, (192, 128), np.float16)
+    assert zeros(T, (512, 128), np.float16).linear(hw).realize().kernels() == ["gemm_f16_nt_512_192_128"]
+    T.set_fusion(False)
+    h = zeros(T, (256, 128), np.float16).matmul(zeros(T, (128, 192), np.float16)).realize()
+    assert h.kernels() == ["r_tc_256_192_128"] and "mfma_f32_16x16x32_f16" in T.last_kernel_sources()[0]   # switched off: the WMMA route
+    T.set_fusion(True)
     # inputs that are lazy views get materialised first
     gt = bf(32, 64).try_transpose(0, 1).matmul(bf(32, 48)).realize()
     assert len(gt.kernels()) == 2

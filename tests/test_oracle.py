@@ -626,6 +626,51 @@ def test_bf16_conversions_round_to_nearest_even_over_every_code(oracle):
     assert (nan & 0x7f80) == 0x7f80 and (nan & 0x7f) != 0
 
 
+def test_f16_conversions_over_every_code_and_gemm_f16_by_definition(oracle):
+    """orc_f16_to_f32 against numpy's IEEE half over all 65536 codes (subnormals, infinities, NaN);
+    orc_f32_to_f16 against numpy's float32 -> float16 rounding on every midpoint between neighbouring
+    halves, its two float32 neighbours, the overflow boundary 65520 and random values; orc_gemm_f16
+    against the float64 product of the same f16 inputs and against cases with exact answers."""
+    codes = np.arange(65536, dtype=np.uint16)
+    f = np.empty(65536, np.float32)
+    oracle.lib.orc_f16_to_f32(codes.ctypes.data_as(C.c_void_p), f.ctypes.data_as(C.c_void_p), C.c_long(65536))
+    want = codes.view(np.float16).astype(np.float32)
+    assert np.array_equal(f.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.isnan(f[np.isnan(want)]).all()
+
+    def to_f16(x):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty(x.shape, np.uint16)
+        oracle.lib.orc_f32_to_f16(x.ctypes.data_as(C.c_void_p), out.ctypes.data_as(C.c_void_p), C.c_long(x.size))
+        return out
+
+    fin = np.isfinite(want)
+    assert np.array_equal(to_f16(want[fin]), codes[fin])
+    pos = codes[codes < 0x7bff]
+    v, w = want[pos].astype(np.float64), want[pos + 1].astype(np.float64)
+    mid = ((v + w) / 2).astype(np.float32)
+    trial = np.concatenate([mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(np.inf)), -mid,
+                            np.float32([65504.0, 65519.99, 65520.0, 65536.0, 1e9, -65520.0, np.inf, 0.0, -0.0, 1e-10, 2.0 ** -25, 2.0 ** -24 * 1.5]),
+                            synth.normal((20000,), 97, 0) * np.float32(100.0), synth.normal((20000,), 97, 1) * np.float32(1e-5)])
+    with np.errstate(over="ignore"):
+        assert np.array_equal(to_f16(trial), trial.astype(np.float16).view(np.uint16))
+    nan = to_f16(np.float32([np.nan]))[0]
+    assert (nan & 0x7c00) == 0x7c00 and (nan & 0x3ff) != 0
+    M, N, K = 37, 29, 200
+    a = synth.normal((M, K), 97, 2).astype(np.float16)
+    b = synth.normal((K, N), 97, 3).astype(np.float16)
+    got = oracle.gemm_f16(a, b).astype(np.float64)
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.abs(got - ref).max() <= 1.5e-3 * np.abs(ref).max()           # one f16 rounding (2^-11) + f32 accumulation
+    eye = np.eye(K, dtype=np.float16)
+    assert np.array_equal(oracle.gemm_f16(a, eye), a)                       # identity: exact
+    ones = np.ones((K, N), np.float16)
+    small = (synth.uniform((M, K), 97, 4) * 8).astype(np.int32).astype(np.float16)   # small integers: sums exact
+    assert np.array_equal(oracle.gemm_f16(small, ones).astype(np.float64), small.astype(np.float64).sum(1, keepdims=True).repeat(N, 1))
+    # transposed operand order matters: a dropped transpose or a swapped index fails here
+    assert not np.allclose(oracle.gemm_f16(a[:29, :29], b[:29, :29].T.copy()).astype(np.float64), ref[:29, :29], atol=1e-2)
+
+
 def test_heads_to_tokens_and_rope_heads_layout(oracle):
     """Index checks with distinct values per position: [B,H,S,D] -> [B*S, H*D] and the
     token-major -> head-major move of orc_rope_heads_bf16 (apply=0: a pure permutation;

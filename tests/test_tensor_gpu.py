@@ -1381,11 +1381,12 @@ def test_flat_upcast_keeps_moved_operands_on_coordinates(T):
 
 
 @pytest.mark.parametrize("shape", [(256, 192, 128), (100, 40, 72), (512, 512, 256), (64, 64, 64)])
-def test_half_precision_matmul_takes_the_generated_tensor_core_kernel(T, shape):
-    """There is no hand-written f16 GEMM: Tensor::matmul on half operands lowers through the WMMA
-    route (f16 tensor core of the CDNA table, f32 accumulate, direct-copy variant where its tiles
-    divide the shape, the padded register-staged one elsewhere), as a kernel of its own also in the
-    middle of an expression."""
+def test_half_precision_matmul_hand_written_and_generated(T, oracle, shape):
+    """Tensor::matmul on half operands: the hand-written f16 kernels (gemm_f16: the tiled body around
+    v_mfma_f32_16x16x32_f16), and with them switched off the WMMA route (f16 tensor core of the CDNA
+    table, f32 accumulate, direct-copy variant where its tiles divide the shape, the padded
+    register-staged one elsewhere), as a kernel of its own also in the middle of an expression.
+    Both against the oracle, and with the same bits as each other."""
     from morok_amd import synth
 
     M, N, K = shape
@@ -1393,10 +1394,20 @@ def test_half_precision_matmul_takes_the_generated_tensor_core_kernel(T, shape):
     b = synth.normal((K, N), 91, 1).astype(np.float16)
     ta, tb = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
     c = ta.matmul(tb)
+    hand = c.to_numpy()
+    assert c.kernels() == ["gemm_f16_%d_%d_%d" % (M, N, K)] and hand.dtype == np.float16
+    ref = oracle.gemm_f16(a, b).astype(np.float64)
+    assert np.abs(hand - ref).max() <= 2e-2 * np.abs(ref).max() and np.abs(hand - ref).max() <= 2e-3 * np.abs(ref).max()
+    lin = ta.linear(T.Tensor.from_numpy(np.ascontiguousarray(b.T)))      # x @ w.T with w stored [N, K]
+    got = lin.to_numpy()
+    if K % 8 == 0 and N % 8 == 0:
+        assert lin.kernels()[-1].startswith("gemm_f16")
+    assert np.abs(got - ref).max() <= 2e-3 * np.abs(ref).max()
+    T.set_fusion(False)
+    c = ta.matmul(tb)
     got = c.to_numpy()
     assert c.kernels() == ["r_tc_%d_%d_%d" % (M, N, K)] and got.dtype == np.float16
-    ref = a.astype(np.float64) @ b.astype(np.float64)
-    assert np.abs(got - ref).max() <= 2e-3 * np.abs(ref).max()
+    assert np.array_equal(got.view(np.uint16), hand.view(np.uint16))
     both = ta.matmul(tb).try_add(ta.matmul(tb))
     got2 = both.to_numpy()
     assert sum(k.startswith("r_tc_") for k in both.kernels()) == 2
