@@ -46,6 +46,15 @@ int KernelCache::get_or_compile(uint64_t ast_hash, const std::string& device, co
     return kOk;
 }
 
+bool KernelCache::lookup(uint64_t ast_hash, const std::string& device, std::shared_ptr<CachedKernel>* out) {
+    const std::string key = std::to_string(ast_hash) + "@" + device;
+    std::lock_guard<std::mutex> lock(mu_);
+    auto it = map_.find(key);
+    if (it == map_.end()) return false;
+    *out = it->second;
+    return true;
+}
+
 size_t KernelCache::size() {
     std::lock_guard<std::mutex> lock(mu_);
     return map_.size();
@@ -59,12 +68,20 @@ void KernelCache::clear_all() {
     }
 }
 
+// the cache key also covers the compiler backend (tensor/src/realize.rs:1052-1054)
+static uint64_t linear_kernel_key(const Device& dev, const LinearKernel& k) {
+    return k.content_hash ^ fnv1a64(reinterpret_cast<const uint8_t*>(dev.compiler->cache_key()), std::strlen(dev.compiler->cache_key()));
+}
+
+bool lookup_linear_kernel(const Device& dev, const LinearKernel& k, std::shared_ptr<CachedKernel>* out) {
+    const std::string device = std::string(Device::base_device_key()) + ":" + std::to_string(dev.device_id);
+    return KernelCache::global().lookup(linear_kernel_key(dev, k), device, out);
+}
+
 int get_or_compile_linear_kernel(const Device& dev, const LinearKernel& k, const char* name,
                                  std::shared_ptr<CachedKernel>* out, bool* was_cached) {
     const std::string device = std::string(Device::base_device_key()) + ":" + std::to_string(dev.device_id);
-    // the cache key also covers the compiler backend (tensor/src/realize.rs:1052-1054)
-    const uint64_t key = k.content_hash ^ fnv1a64(reinterpret_cast<const uint8_t*>(dev.compiler->cache_key()),
-                                                  std::strlen(dev.compiler->cache_key()));
+    const uint64_t key = linear_kernel_key(dev, k);
     return KernelCache::global().get_or_compile(
         key, device,
         [&](std::shared_ptr<CachedKernel>* fresh) -> int {

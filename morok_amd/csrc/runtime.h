@@ -36,6 +36,8 @@ class KernelCache {
     using CompileFn = std::function<int(std::shared_ptr<CachedKernel>*)>;
     int get_or_compile(uint64_t ast_hash, const std::string& device, const CompileFn& compile_fn,
                        std::shared_ptr<CachedKernel>* out, bool* was_cached = nullptr);
+    // the cached kernel, if there is one (no compile)
+    bool lookup(uint64_t ast_hash, const std::string& device, std::shared_ptr<CachedKernel>* out);
     size_t size();
     void clear_all();  // kernel_cache.rs:124-130
 
@@ -48,6 +50,8 @@ class KernelCache {
 // what prepare_execution_plan does per kernel (tensor/src/realize.rs:1052-1070).
 int get_or_compile_linear_kernel(const Device& dev, const LinearKernel& k, const char* name,
                                  std::shared_ptr<CachedKernel>* out, bool* was_cached = nullptr);
+// The cache lookup alone: true and the kernel when this device already holds it.
+bool lookup_linear_kernel(const Device& dev, const LinearKernel& k, std::shared_ptr<CachedKernel>* out);
 
 // execution_plan.rs:50-82
 struct PreparedKernel {

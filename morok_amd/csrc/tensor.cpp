@@ -1167,6 +1167,29 @@ struct Scheduler {
         size_t bytes = static_cast<size_t>(n->numel()) * scalar_size(n->dtype);
         return std::make_shared<Buffer>(dev->allocator, bytes ? bytes : 1, o);
     }
+    // Kernels this schedule needs that the cache does not hold yet.  With `deferred` set they are
+    // not compiled here (the caller holds the graph lock): the schedule goes on with a placeholder
+    // and is thrown away, the caller compiles them with the lock released and schedules again.
+    // `fresh` names the kernels compiled that way, so that the second pass still reports them as
+    // newly compiled.
+    struct PendingKernel {
+        LinearKernel k;
+        std::string name;
+    };
+    std::vector<PendingKernel>* deferred = nullptr;
+    const std::set<uint64_t>* fresh = nullptr;
+    int compile_kernel(const LinearKernel& k, const char* name, std::shared_ptr<CachedKernel>* ck, bool* cached) {
+        if (deferred && !lookup_linear_kernel(*dev, k, ck)) {
+            deferred->push_back({k, name});
+            *ck = std::make_shared<CachedKernel>();
+            (*ck)->entry_point = name;
+            *cached = false;
+            return kOk;
+        }
+        MRK_TRY(get_or_compile_linear_kernel(*dev, k, name, ck, cached));
+        if (fresh && fresh->count(k.content_hash)) *cached = false;
+        return kOk;
+    }
     int builtin(const char* kind, const std::vector<int64_t>& params, const std::vector<std::shared_ptr<Buffer>>& bufs) {
         std::string key = std::string("builtin:") + kind;
         for (int64_t p : params) key += ":" + std::to_string(p);
@@ -1274,8 +1297,9 @@ struct Scheduler {
         // the chip (one 256 x 256 workgroup or two smaller ones per CU), else the smallest
         static const int direct[][5] = {{2, 2, 8, 8, 256}, {2, 4, 8, 4, 256}, {2, 2, 4, 4, 512}, {2, 2, 4, 2, 512}, {2, 2, 2, 2, 0}};
         for (auto& c : direct) {
-            WmmaLdsOpts t{c[0], c[1], c[2], c[3], 0, 3};  // a third B stage where the schedule and the 160 KB allow it
-            if (!wmma_lds_opts_valid(tc, t, M, N, K)) t.stages = 2;
+            // (stages = 3, a third stage of the second operand with the copies spread over the whole step,
+            // measured the same or 1 % slower at 4096^3: the beam search tries it, the heuristic does not)
+            WmmaLdsOpts t{c[0], c[1], c[2], c[3], 0, 2};
             if (!wmma_lds_opts_valid(tc, t, M, N, K)) continue;
             int bm, bn, bk;
             wmma_lds_tile(tc, t, K, &bm, &bn, &bk);
@@ -1335,7 +1359,7 @@ struct Scheduler {
         std::shared_ptr<CachedKernel> ck;
         bool cached = false;
         const std::string name = "r_tc_" + std::to_string(M) + "_" + std::to_string(N) + "_" + std::to_string(K);
-        MRK_TRY(get_or_compile_linear_kernel(*dev, k, name.c_str(), &ck, &cached));
+        MRK_TRY(compile_kernel(k, name.c_str(), &ck, &cached));
         auto out = new_buffer(n);
         MRK_TRY(add_kernel(ck, {out, a->buffer, w->buffer}, cached));
         n->buffer = out;
@@ -1963,7 +1987,7 @@ struct Scheduler {
                 std::shared_ptr<CachedKernel> ck;
                 bool cached = false;
                 const std::string name = "r_" + std::to_string(M) + "_" + std::to_string(N) + "_" + std::to_string(K);
-                MRK_TRY(get_or_compile_linear_kernel(*dev, k, name.c_str(), &ck, &cached));
+                MRK_TRY(compile_kernel(k, name.c_str(), &ck, &cached));
                 rc = add_kernel(ck, {out, a->buffer, w->buffer}, cached);
             }
         }
@@ -2005,7 +2029,7 @@ struct Scheduler {
         }
         std::shared_ptr<CachedKernel> ck;
         bool cached = false;
-        MRK_TRY(get_or_compile_linear_kernel(*dev, k, name.c_str(), &ck, &cached));
+        MRK_TRY(compile_kernel(k, name.c_str(), &ck, &cached));
         std::vector<std::shared_ptr<Buffer>> bufs{out};
         bufs.insert(bufs.end(), g.inputs.begin(), g.inputs.end());
         return add_kernel(ck, bufs, cached);
@@ -2665,10 +2689,14 @@ static std::recursive_mutex g_graph_mutex;
 namespace {
 // Schedules `root`.  On success `kept` lists the nodes (root included) that keep a buffer whose
 // contents exist only after the plan has run; on failure no node keeps one.
-int prepare_locked(const TensorRef& root, std::unique_ptr<ExecutionPlan>* out, std::vector<TensorNode*>* kept) {
+constexpr int kCompileFirst = -77001;  // internal: the schedule found kernels to compile; nothing was kept
+int prepare_locked(const TensorRef& root, std::unique_ptr<ExecutionPlan>* out, std::vector<TensorNode*>* kept,
+                   std::vector<Scheduler::PendingKernel>* deferred = nullptr, const std::set<uint64_t>* fresh = nullptr) {
     g_stats = RealizeStats();
     auto t0 = std::chrono::steady_clock::now();
     Scheduler s;
+    s.deferred = deferred;
+    s.fresh = fresh;
     // every exit that is not the successful one returns the touched nodes to their lazy state
     struct Rollback {
         Scheduler& s;
@@ -2693,6 +2721,7 @@ int prepare_locked(const TensorRef& root, std::unique_ptr<ExecutionPlan>* out, s
         if (!root->buffer) MRK_TRY(s.materialize(root.get()));
         s.plan->set_outputs({s.plan->add_buffer(root->buffer)});
     }
+    if (deferred && !deferred->empty()) return kCompileFirst;  // (the rollback returns every touched node to its lazy state)
     // Intermediates share blocks by liveness (tensor/src/memory_planner.rs); their contents do
     // not outlive the plan's execution, so their nodes go back to being lazy: only the root
     // keeps its buffer.  MOROK_NO_MEMORY_PLANNER=1 keeps every intermediate resident.
@@ -2714,17 +2743,51 @@ int prepare_locked(const TensorRef& root, std::unique_ptr<ExecutionPlan>* out, s
     *out = std::move(s.plan);
     return kOk;
 }
+// Schedules `root` with the graph lock held by `lock` on entry and on return, but released while
+// kernels are compiled: a first pass under the lock only collects what the kernel cache lacks and
+// rolls the graph back, the compiles (the slow part: hiprtc) run unlocked, so realizations of
+// other tensors proceed meanwhile (as the reference's get_or_compile_kernel lets compiles race,
+// runtime/src/kernel_cache.rs:95-117), and a second pass under the lock builds the plan from the
+// cache.  A graph that needs no new kernel takes one pass.  Under MOROK_BEAM the search times its
+// candidates on the device and everything stays under the lock.
+int prepare_compiling_unlocked(const TensorRef& root, std::unique_lock<std::recursive_mutex>& lock, std::unique_ptr<ExecutionPlan>* out,
+                               std::vector<TensorNode*>* kept) {
+    int beam = 0;
+    if (const char* e = std::getenv("MOROK_BEAM")) beam = std::atoi(e);
+    if (beam > 0) return prepare_locked(root, out, kept);
+    std::vector<Scheduler::PendingKernel> pending;
+    int rc = prepare_locked(root, out, kept, &pending);
+    if (rc != kCompileFirst) return rc;
+    const bool to_cpu = root->device_id == kCpuDevice && root->kind == TKind::Copy;
+    const int device_id = to_cpu ? root->src[0]->device_id : root->device_id;
+    std::shared_ptr<Device> dev;
+    MRK_TRY(DeviceFactoryRegistry::global().device("HIP", device_id, &dev));
+    std::set<uint64_t> fresh;
+    lock.unlock();
+    rc = kOk;
+    for (const Scheduler::PendingKernel& p : pending) {
+        std::shared_ptr<CachedKernel> ck;
+        bool cached = false;
+        rc = get_or_compile_linear_kernel(*dev, p.k, p.name.c_str(), &ck, &cached);
+        if (rc != kOk) break;
+        if (!cached) fresh.insert(p.k.content_hash);
+    }
+    lock.lock();
+    if (rc != kOk) return rc;
+    if (kept) kept->clear();
+    return prepare_locked(root, out, kept, nullptr, &fresh);
+}
 }  // namespace
 
 int Tensor::prepare(std::unique_ptr<ExecutionPlan>* out) const {
     if (!n_) return fail(kInvalidArgument, "prepare: invalid tensor");
-    std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
-    return prepare_locked(n_, out, nullptr);
+    std::unique_lock<std::recursive_mutex> lock(g_graph_mutex);
+    return prepare_compiling_unlocked(n_, lock, out, nullptr);
 }
 
 int Tensor::realize() const {
     if (!n_) return fail(kInvalidArgument, "realize: invalid tensor");
-    std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
+    std::unique_lock<std::recursive_mutex> lock(g_graph_mutex);
     if (n_->buffer || (n_->device_id == kCpuDevice && n_->host)) {
         g_stats = RealizeStats();
         return kOk;
@@ -2732,7 +2795,7 @@ int Tensor::realize() const {
     auto t0 = std::chrono::steady_clock::now();
     std::unique_ptr<ExecutionPlan> plan;
     std::vector<TensorNode*> kept;
-    MRK_TRY(prepare_locked(n_, &plan, &kept));
+    MRK_TRY(prepare_compiling_unlocked(n_, lock, &plan, &kept));
     // The plan is enqueued before the lock is released: whoever sees the root's buffer next
     // queues its reads behind these kernels on the device's in-order stream.
     int rc = plan->execute();
@@ -2758,17 +2821,20 @@ int Tensor::to_bytes(void* dst, size_t nbytes) const {
     std::shared_ptr<Buffer> buf;
     std::shared_ptr<std::vector<uint8_t>> host;
     int host_from = kCpuDevice;
-    {
-        std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
-        if (n_->device_id == kCpuDevice) {
-            if (!n_->host) MRK_TRY(realize());
-            host = n_->host;
-            host_from = n_->host_from;
-        } else {
-            if (!n_->buffer) MRK_TRY(realize());
-            buf = n_->buffer;
+    for (int attempt = 0; attempt < 2 && !buf && !host; attempt++) {
+        {
+            std::lock_guard<std::recursive_mutex> lock(g_graph_mutex);
+            if (n_->device_id == kCpuDevice) {
+                host = n_->host;
+                host_from = n_->host_from;
+            } else {
+                buf = n_->buffer;
+            }
         }
+        // realize takes the lock itself (and lets go of it while kernels compile)
+        if (!buf && !host && attempt == 0) MRK_TRY(realize());
     }
+    if (!buf && !host) return fail(kRuntime, "to_vec: the tensor has no data after realize");
     const size_t expect = static_cast<size_t>(n_->numel()) * scalar_size(n_->dtype);
     if (nbytes != expect) return failf(kSizeMismatch, "size mismatch: expected %zu, got %zu", expect, nbytes);
     if (expect == 0) return kOk;

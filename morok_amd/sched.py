@@ -107,7 +107,8 @@ def build_wmma_matmul_lds(tc_index, m, n, k, out_scalar):
 
 def build_wmma_matmul_lds_opts(tc_index, m, n, k, out_scalar, opts):
     """The same with explicit (waves_m, waves_n, tiles_m per wave, tiles_n per wave, K steps per
-    barrier pair; 0 = by K[, stages: 0 = through registers, 2 = direct global -> local copies])."""
+    barrier pair; 0 = by K[, stages: 0 = through registers, 2 = direct global -> local copies, 3 = the
+    same with a third stage of the second operand (at most four waves, more than two K steps)])."""
     opts = list(opts) + [0] * (6 - len(opts))
     arr = (C.c_int * 6)(*opts)
     return _take(lib.mrk_hip_sched_build_wmma_matmul_lds_opts, tc_index, m, n, k, out_scalar, arr)

@@ -56,6 +56,42 @@ static int shared_subgraph() {
     for (mrk_tensor* p : {t, u, mid}) mrk_hip_tensor_release(p);
     return 0;
 }
+// Four threads realize graphs that share nothing and whose kernels nobody has compiled yet (every
+// thread and round has a shape of its own): the graph lock is released while a thread compiles, so
+// the compiles of unrelated graphs overlap and the schedules interleave around them.
+static int unrelated_graphs_compile_concurrently() {
+    int rcs[4] = {0, 0, 0, 0};
+    std::vector<std::thread> th;
+    for (int i = 0; i < 4; i++)
+        th.emplace_back([i, &rcs] {
+            rcs[i] = [&]() -> int {
+                for (int r = 0; r < 3; r++) {
+                    int64_t shp[2] = {16 + 8 * i + r, 24 + 4 * r + i};
+                    std::vector<float> x(shp[0] * shp[1], 0.25f);
+                    mrk_tensor *t = nullptr, *u = nullptr, *root = nullptr;
+                    CK(mrk_hip_tensor_from_bytes(0, x.data(), x.size() * 4, shp, 2, 11 /*f32*/, &t));
+                    CK(mrk_hip_tensor_binary(t, 2 /*mul*/, t, &u));
+                    int64_t ax[1] = {1};
+                    CK(mrk_hip_tensor_reduce(u, 0 /*add*/, ax, 1, 0, 1, &root));
+                    if (r == 1) {
+                        mrk_plan* plan = nullptr;
+                        CK(mrk_hip_tensor_prepare(root, &plan));
+                        CK(mrk_hip_plan_execute(plan));
+                        mrk_hip_plan_release(plan);
+                    }
+                    std::vector<float> out(shp[0]);
+                    CK(mrk_hip_tensor_to_bytes(root, out.data(), out.size() * 4));
+                    CK(mrk_hip_tensor_realize(root));   // already realized: no second schedule
+                    for (mrk_tensor* p : {t, u, root}) mrk_hip_tensor_release(p);
+                }
+                return 0;
+            }();
+        });
+    for (auto& thr : th) thr.join();
+    for (int rc : rcs)
+        if (rc) return 1;
+    return 0;
+}
 int main() {
     if (mrk_hip_device_create(0)) return 1;
     std::vector<std::thread> th; int rcs[4] = {0,0,0,0};
@@ -63,6 +99,7 @@ int main() {
     for (auto& t : th) t.join();
     for (int i = 0; i < 4; i++) if (rcs[i]) return 1;
     if (shared_subgraph()) return 1;
+    if (unrelated_graphs_compile_concurrently()) return 1;
     printf("threads ok\n");
     return 0;
 }

@@ -105,7 +105,8 @@ def test_generated_tensor_core_direct_copy_random_choices(dev, seed):
     rng = np.random.default_rng(7400 + seed)
     tc = int(rng.choice([3, 7]))
     while True:
-        opts = (int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4, 8])), int(rng.choice([1, 2, 4, 8])), 0, 2)
+        opts = (int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4])), int(rng.choice([1, 2, 4, 8])), int(rng.choice([1, 2, 4, 8])), 0,
+                2 + seed % 2)   # two stages of both tiles, or a third one of the second operand's
         t = 16 if tc == 3 else 32
         bm, bn = opts[0] * opts[2] * t, opts[1] * opts[3] * t
         M, N, K = bm * int(rng.integers(1, 5)), bn * int(rng.integers(1, 5)), 64 * int(rng.integers(1, 7))

@@ -329,7 +329,10 @@ def test_tc_apply_matmul_fp8(dev, oracle, tc, kind, one, shape):
                                         ((128, 192, 128), (1, 4, 4, 1, 0, 2)), ((512, 512, 192), (4, 4, 4, 4, 0, 2)),
                                         ((512, 256, 320), (2, 2, 8, 8, 0, 2)), ((256, 512, 256), (2, 4, 8, 4, 0, 2)),
                                         ((192, 128, 448), (1, 1, 4, 4, 0, 2)), ((768, 256, 128), (2, 2, 8, 4, 2, 2)),
-                                        ((256, 1024, 128), (4, 2, 4, 8, 0, 2)), ((1536, 768, 64), (2, 2, 8, 8, 0, 2))])
+                                        ((256, 1024, 128), (4, 2, 4, 8, 0, 2)), ((1536, 768, 64), (2, 2, 8, 8, 0, 2)),
+                                        # a third stage of the second operand's tile (copies spread over the whole step)
+                                        ((512, 256, 320), (2, 2, 8, 8, 0, 3)), ((256, 512, 192), (2, 2, 8, 8, 0, 3)), ((256, 256, 256), (1, 4, 8, 2, 0, 3)),
+                                        ((384, 128, 448), (1, 1, 4, 4, 0, 3)), ((768, 512, 1024), (2, 2, 8, 4, 0, 3))])
 def test_tc_matmul_direct_copy_choices_agree(dev, shape, opts):
     """The variant whose tiles arrive by direct global -> local copies (two stages, transposing B
     reads, operands swapped at the tensor core, tiles assigned per XCD) computes the same products
