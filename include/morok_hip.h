@@ -492,6 +492,21 @@ int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, cons
  * buffers {c, a, w}. */
 int mrk_hip_gemm_bf16_swiglu(int device_id, const void* a, const void* w, void* c, int64_t m, int64_t f, int64_t k);
 
+/* A packed projection with the rotary embedding in its epilogue: for w [K, N] whose first `split`
+ * columns are attention heads of 128 columns each (Wq | Wk of a fused QKV projection; split a
+ * multiple of 256), c_rot[M, split] = apply_rotary_emb(bf16(a w)[:, :split] seen as heads, cos, sin)
+ * in the reference's non-interleaved form (tensor/src/transformer.rs:32-69: x1 cos - x2 sin |
+ * x1 sin + x2 cos over the two halves of a head), computed in f32 on the rounded product and
+ * rounded once, as Tensor::matmul followed by apply_rotary_emb and a cast computes it; row r has
+ * position r % seq, cos / sin are [seq, 64] f32.  The remaining columns go, unrotated, to
+ * c_rest[M, N - split] (NULL when split == N).  The rotated product is never written and read
+ * again in between.  K a multiple of 64, N of 8, cos / sin 32-byte aligned; INVALID_ARGUMENT
+ * otherwise.  Builtin Program kind "gemm_bf16_rope", params {M, N, K, split, seq}, buffers
+ * {c_rot, a, w, c_rest, cos, sin}.  The reference holds no value test of this composition: parity
+ * unpinned by reference tests, pinned against the oracle's product followed by its rotary stage. */
+int mrk_hip_gemm_bf16_rope(int device_id, const void* a, const void* b, const void* cos, const void* sin, void* c_rot, void* c_rest,
+                           int64_t m, int64_t n, int64_t k, int64_t split, int64_t seq);
+
 /* Scaled dot-product attention forward in one kernel (online softmax, f32 scores and
  * statistics, P rounded to bf16 before the second product, bf16 output):
  * Tensor::scaled_dot_product_attention (tensor/src/transformer.rs:78-137) with is_causal as

@@ -154,6 +154,8 @@ _SIGS = {
                                             C.c_int64, C.c_int]),
     "mrk_hip_gemm_bf16_residual": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
                                              C.c_int64]),
+    "mrk_hip_gemm_bf16_rope": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
+                                         C.c_int64, C.c_int64, C.c_int64, C.c_int64]),
     "mrk_hip_flash_attn_fwd_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
                                               C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_int]),
     "mrk_hip_flash_attn_fwd_bf16_strided": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,

@@ -905,6 +905,26 @@ static int gemm_16bit_nt(int device_id, const void* a, const void* bt, void* c, 
     return kOk;
 }
 
+int mrk_hip_gemm_bf16_rope(int device_id, const void* a, const void* b, const void* cos, const void* sin, void* c_rot, void* c_rest,
+                           int64_t m, int64_t n, int64_t k, int64_t split, int64_t seq) {
+    if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_rope: negative shape");
+    if (m == 0 || n == 0) return kOk;
+    MRK_NONNULL(a);
+    MRK_NONNULL(b);
+    MRK_NONNULL(cos);
+    MRK_NONNULL(sin);
+    MRK_NONNULL(c_rot);
+    if (!gemm_bf16_rope_supported(m, n, k, split, seq))
+        return fail(kInvalidArgument, "gemm_bf16_rope: shape not covered by the rotary epilogue (K a multiple of 64, N of 8, split a multiple of "
+                                      "256 within N, seq > 0); run mrk_hip_gemm_bf16 and rotate separately");
+    if (split < n) MRK_NONNULL(c_rest);
+    std::shared_ptr<Device> dv;
+    MRK_TRY(get_device(device_id, &dv));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_gemm_bf16_rope(dv->allocator->stream(), a, b, c_rot, c_rest, m, n, k, split, cos, sin, seq), "gemm_bf16_rope launch");
+    return kOk;
+}
+
 int mrk_hip_gemm_bf16_swiglu(int device_id, const void* a, const void* w, void* c, int64_t m, int64_t f, int64_t k) {
     if (m < 0 || f < 0 || k < 0) return fail(kInvalidArgument, "gemm_bf16_swiglu: negative shape");
     if (m == 0 || f == 0) return kOk;

@@ -125,12 +125,30 @@ __device__ __forceinline__ bf16x4 round_to_elem(const f32x4& v) {
     if constexpr (kF16) return __builtin_bit_cast(bf16x4, __builtin_convertvector(v, f16x4));
     else return __builtin_convertvector(v, bf16x4);
 }
-template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false, bool kSwiGLU = false, bool kBT = false, bool kF16 = false>
+//
+// kRope (256-row tile only): the product of a packed projection whose first `split` columns are
+// attention heads of 128 columns each (q | k of a fused QKV product).  The epilogue applies the
+// rotary embedding (non-interleaved form, tensor/src/transformer.rs:32-69) to those heads on the
+// bf16-rounded product, as the separate kernel would: with x1 = columns 0..63 and x2 = columns
+// 64..127 of a head, out = [x1 cos - x2 sin | x1 sin + x2 cos] in f32 and one rounding, cos / sin
+// [seq, 64] f32 indexed by the row's position (row % seq).  A wave's 128 columns are exactly one
+// head, so both halves of a pair sit in the tile row the wave has just staged.  The rotated
+// columns go to C with a row pitch of `split`; the columns behind them (v) go, unrotated, to a
+// second matrix of their own with a row pitch of N - split.
+struct RopeEpilogue {
+    const float* cos;
+    const float* sin;
+    __bf16* rest;  // [M, N - split]: the columns from `split` on
+    int seq, split;
+};
+template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false, bool kSwiGLU = false, bool kBT = false, bool kF16 = false,
+          bool kRope = false>
 __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
                                                float* __restrict__ W = nullptr, int kt_per_split = 0,
-                                               const __bf16* __restrict__ R = nullptr) {
-    static_assert(!kF16 || (!kResidual && !kSwiGLU), "the fused epilogues exist for bf16 only");
+                                               const __bf16* __restrict__ R = nullptr, const RopeEpilogue& rope = RopeEpilogue{}) {
+    static_assert(!kF16 || (!kResidual && !kSwiGLU && !kRope), "the fused epilogues exist for bf16 only");
+    static_assert(!kRope || (kJ == 4 && !kSplitK && !kResidual && !kSwiGLU), "the rotary epilogue exists for the plain 256-row tile only");
     constexpr int kTM = kJ == 4 ? 256 : 128;      // rows of the workgroup tile
     constexpr int kAq = kTM / 32;                 // 1 KB A chunks (8 rows) each wave copies per K step
     constexpr int kAStageT = kTM * kBK * 2;       // bytes of an A stage
@@ -585,7 +603,10 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
         // are read back and stored while tile row i + 1 is being converted and staged: the stores
         // start one tile row after the loop ends instead of after the whole staging.
         constexpr int kPerRow = 16 / kRowsPerIt;  // store instructions per tile row
-        __bf16* Cl = C + (row0 + lr) * N + col0 + lc * 8;
+        // (rotary epilogue: the tile's columns lie either all in front of `split` or all behind it)
+        const bool rotate = kRope && n0 < (size_t)rope.split;
+        const size_t ldc = !kRope ? (size_t)N : rotate ? (size_t)rope.split : (size_t)(N - rope.split);
+        __bf16* Cl = (!kRope || rotate ? C + col0 : rope.rest + (col0 - rope.split)) + (row0 + lr) * ldc + lc * 8;
         const char* sCl = sC + lr * kCPitchT + lc * 16;
         auto stage_row = [&](int i) {
 #pragma unroll
@@ -611,7 +632,22 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
                                       __builtin_convertvector(__builtin_bit_cast(bf16x8, res[i * kPerRow + t]), f32x8);
                     v[t] = __builtin_bit_cast(u32x4, __builtin_convertvector(sum, bf16x8));
                 }
-                if (col_ok && r + lr < rows_here) *reinterpret_cast<u32x4*>(Cl + (size_t)r * N) = v[t];
+                if constexpr (kRope) {
+                    if (rotate) {
+                        // this lane's 8 columns of a head, their partners 64 columns away (chunk lc ^ 8 of the
+                        // same staged row), and the 8 angles of the row's position
+                        const u32x4 pv = *LDS_PTR(u32x4, sC + (r + lr) * kCPitchT + (lc ^ 8) * 16);
+                        const f32x8 x = __builtin_convertvector(__builtin_bit_cast(bf16x8, v[t]), f32x8);
+                        const f32x8 y = __builtin_convertvector(__builtin_bit_cast(bf16x8, pv), f32x8);
+                        const size_t pos = (row0 + r + lr) % (size_t)rope.seq;
+                        const f32x8 cs = *reinterpret_cast<const f32x8*>(rope.cos + pos * 64 + (lc & 7) * 8);
+                        f32x8 sn = *reinterpret_cast<const f32x8*>(rope.sin + pos * 64 + (lc & 7) * 8);
+                        if (lc < 8) sn = -sn;  // first half: x1 cos - x2 sin; second half: x2 cos + x1 sin
+                        const f32x8 o = x * cs + y * sn;
+                        v[t] = __builtin_bit_cast(u32x4, __builtin_convertvector(o, bf16x8));
+                    }
+                }
+                if (col_ok && r + lr < rows_here) *reinterpret_cast<u32x4*>(Cl + (size_t)r * ldc) = v[t];
             }
         }
         return;
@@ -700,6 +736,11 @@ __global__ __launch_bounds__(256) void gemm_f16_tile128_splitk_ragged_k(const __
                                                                         float* __restrict__ W, int M, int N, int K, int tiles_m,
                                                                         int tiles_n, int kt_per_split) {
     gemm_tile_body<true, 2, true, false, false, false, true>(A, B, nullptr, M, N, K, tiles_m, tiles_n, W, kt_per_split);
+}
+__global__ __launch_bounds__(256) void gemm_bf16_tile256_rope(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                              __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+                                                              RopeEpilogue rope) {
+    gemm_tile_body<false, 4, false, false, false, false, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, nullptr, rope);
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_ragged_k(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ B, __bf16* __restrict__ C,
@@ -951,6 +992,28 @@ int launch_gemm_bf16_swiglu(void* stream, const void* A, const void* B, void* C,
     auto kernel = b_transposed ? (ragged_k ? gemm_bf16_nt_tile256_swiglu_ragged_k : gemm_bf16_nt_tile256_swiglu)
                                : (ragged_k ? gemm_bf16_tile256_swiglu_ragged_k : gemm_bf16_tile256_swiglu);
     kernel<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)(2 * F), (int)K, (int)tm, (int)tn);
+    return (int)hipGetLastError();
+}
+
+bool gemm_bf16_rope_supported(long M, long N, long K, long split, long seq) {
+    using namespace mrk::dev;
+    return M > 0 && N > 0 && K > 0 && seq > 0 && K % kBK == 0 && N % 8 == 0 && split > 0 && split <= N && split % kBN == 0 &&
+           M <= 0x7fffffffL && N < (1L << 25) && K <= (1L << 23) && ((M + kBM - 1) / kBM) * ((N + kBN - 1) / kBN) <= 0x7fffffffL;
+}
+
+int launch_gemm_bf16_rope(void* stream, const void* A, const void* B, void* C_rot, void* C_rest, long M, long N, long K, long split,
+                          const void* cos, const void* sin, long seq) {
+    using namespace mrk::dev;
+    if (!gemm_bf16_rope_supported(M, N, K, split, seq) || !A || !B || !C_rot || !cos || !sin || (split < N && !C_rest))
+        return (int)hipErrorInvalidValue;
+    const uintptr_t all = reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C_rot) |
+                          reinterpret_cast<uintptr_t>(C_rest) | reinterpret_cast<uintptr_t>(cos) | reinterpret_cast<uintptr_t>(sin);
+    if (all % 16 || reinterpret_cast<uintptr_t>(cos) % 32 || reinterpret_cast<uintptr_t>(sin) % 32) return (int)hipErrorInvalidValue;
+    (void)hipGetLastError();
+    const long tm = (M + kBM - 1) / kBM, tn = (N + kBN - 1) / kBN;
+    RopeEpilogue rope{static_cast<const float*>(cos), static_cast<const float*>(sin), static_cast<__bf16*>(C_rest), (int)seq, (int)split};
+    gemm_bf16_tile256_rope<<<dim3((unsigned)(tm * tn)), 256, 0, static_cast<hipStream_t>(stream)>>>(
+        static_cast<const __bf16*>(A), static_cast<const __bf16*>(B), static_cast<__bf16*>(C_rot), (int)M, (int)N, (int)K, (int)tm, (int)tn, rope);
     return (int)hipGetLastError();
 }
 

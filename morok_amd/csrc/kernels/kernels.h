@@ -37,6 +37,15 @@ int launch_gemm_bf16_residual(void* stream, const void* a, const void* b, const 
 // b_transposed: W is stored as [2F, K] (the rows of Wg^T, then the rows of Wu^T).
 bool gemm_bf16_swiglu_supported(long M, long F, long K, bool b_transposed = false);
 int launch_gemm_bf16_swiglu(void* stream, const void* a, const void* w, void* c, long M, long F, long K, bool b_transposed = false);
+// A packed projection whose first `split` columns are attention heads of 128 columns (q | k of a
+// fused QKV product, split a multiple of 256) with the rotary embedding applied in the product
+// kernel's epilogue: c_rot [M, split] = rope(bf16(a b)[:, :split]) (non-interleaved halves, cos /
+// sin [seq, 64] f32, 32-byte aligned, position = row % seq; f32 arithmetic on the rounded product,
+// one rounding), c_rest [M, N - split] = bf16(a b)[:, split:] (may be null when split == N).
+// K a multiple of 64, N of 8.
+bool gemm_bf16_rope_supported(long M, long N, long K, long split, long seq);
+int launch_gemm_bf16_rope(void* stream, const void* a, const void* b, void* c_rot, void* c_rest, long M, long N, long K, long split,
+                          const void* cos, const void* sin, long seq);
 // Bytes of f32 scratch with which launch_gemm_bf16 spreads the K loop of this shape over the
 // chip (split-K: partial products per K range, added up in a fixed order by a second kernel);
 // 0 when the shape has enough output tiles by itself.  Without the workspace the same shape

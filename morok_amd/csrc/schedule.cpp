@@ -1019,9 +1019,14 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
         for (int i = 0; i < um; i++) b.store(fa0[h * um + i], read_a(h, i, b.ci(0)));
         for (int j = 0; j < un; j++) b.store(fb0[h * un + j], read_b(h, j, b.ci(0)));
     }
-    uint32_t r = b.range(KT, 0, AxisType::Reduce);
-    {
-        uint32_t st = b.imod(r, 2), sn = bin(BinaryOp::Sub, b.ci(1), st);
+    // One wave per SIMD and an even number of steps: the loop runs two steps per trip, so that the
+    // stage of a step is a constant and the fragment reads address it through their immediate
+    // offsets instead of one vector addition each.
+    const bool two_per_trip = W <= 4 && KT > 2 && KT % 2 == 0 && BST == 2;
+    uint32_t r_outer = b.range(two_per_trip ? KT / 2 : KT, 0, AxisType::Reduce);
+    for (int trip_step = 0; trip_step < (two_per_trip ? 2 : 1); trip_step++) {
+        uint32_t r = two_per_trip ? b.iadd(b.imul(r_outer, 2), b.ci(trip_step)) : r_outer;
+        uint32_t st = two_per_trip ? b.ci(trip_step) : b.imod(r, 2), sn = two_per_trip ? b.ci(1 - trip_step) : bin(BinaryOp::Sub, b.ci(1), st);
         // B stages of tile r, r + 1 and (three stages) the one tile r + 2 goes to
         uint32_t sb0 = BST == 3 ? b.imod(r, 3) : st, sb1 = BST == 3 ? b.imod(b.iadd(r, b.ci(1)), 3) : sn;
         uint32_t sb2 = BST == 3 ? b.imod(b.iadd(r, b.ci(2)), 3) : st;
@@ -1102,7 +1107,7 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             mfmas(f1a, f1b);
         }
     }
-    b.end({r});
+    b.end({r_outer});
     // Result.  A lane holds, per tile, groups of four consecutive columns of one row.  When the result
     // has the operands' 16-bit type the wave first lays its um*TD x un*TD block out in local memory
     // (the tiles' stages are free after one more barrier; the first half of the waves uses the A
@@ -1144,7 +1149,10 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             b.if_(half == 0 ? low_half : b.unary(UnaryOp::Not, low_half));
             uint32_t region = half == 0 ? sA : sB;
             uint32_t base = b.imul(half == 0 ? wave : bin(BinaryOp::Sub, wave, b.ci(W / 2)), RW * CW);
-            for (int i = 0; i < um; i++)
+            // A wave reads back only what it staged itself and local memory serves a wave's requests
+            // in order, so the rows of tile row i - 1 are read back and stored while tile row i is
+            // being converted and staged: the stores start one tile row after the loop ends.
+            auto stage_tile_row = [&](int i) {
                 for (int j = 0; j < un; j++) {
                     uint32_t res = b.load(acc[i * un + j]);
                     for (int q = 0; q < QG; q++) {
@@ -1156,13 +1164,22 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
                         b.store(b.index(region, at), b.vectorize(el));
                     }
                 }
-            for (int t = 0; t < reads; t++) {
+            };
+            auto store_rows = [&](int t) {
                 uint32_t row = b.iadd(r_row, b.ci(t * rows_per_read));
                 uint32_t piece = bin(BinaryOp::Xor, r_piece, bin(BinaryOp::And, row, b.ci(mask)));
                 uint32_t v = b.load(b.index(region, b.iadd(b.iadd(base, b.imul(row, CW)), b.imul(piece, 8))), 8);
                 uint32_t at = b.iadd(b.imul(b.iadd(g_row0, b.ci(t * rows_per_read)), N), g_col);
                 b.store(b.index(c, at), v);
+            };
+            const bool by_tile_row = TD % rows_per_read == 0;  // whole read steps per tile row
+            int stored = 0;
+            for (int i = 0; i < um; i++) {
+                stage_tile_row(i);
+                if (by_tile_row && i > 0)
+                    for (; stored < i * TD / rows_per_read; stored++) store_rows(stored);
             }
+            for (; stored < reads; stored++) store_rows(stored);
             b.endif();
         }
     }

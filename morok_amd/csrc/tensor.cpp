@@ -594,7 +594,12 @@ Tensor Tensor::apply_rotary_emb(const Tensor& cos, const Tensor& sin, bool inter
         fs.back() = last;
         return st.try_reshape(fs);
     }
-    return cat({real, imag}, -1);
+    Tensor out = cat({real, imag}, -1);
+    if (out.valid()) {  // what this subgraph computes, for the scheduler (a product kernel can apply it in its epilogue)
+        out.node()->hint = HintKind::Rope;
+        out.node()->hint_inputs = {n_, cos.node(), sin.node()};
+    }
+    return out;
 }
 
 Tensor Tensor::scaled_dot_product_attention(const Tensor& key, const Tensor& value, double scale, bool is_causal,
@@ -1140,6 +1145,7 @@ struct Scheduler {
     std::vector<TensorNode*> produced_host;  // CPU nodes this realization gave host memory (device -> CPU copies)
     std::unordered_map<const TensorNode*, int> uses;  // consumers of a node within the realised graph
 
+    std::unordered_map<const TensorNode*, std::vector<TensorNode*>> matmul_readers;  // who reads each product node
     void count_uses(const TensorNode* root) {
         std::vector<const TensorNode*> stack{root};
         std::set<const TensorNode*> seen{root};
@@ -1148,6 +1154,7 @@ struct Scheduler {
             stack.pop_back();
             for (const TensorRef& c : n->src) {
                 uses[c.get()]++;
+                if (c->hint == HintKind::Matmul) matmul_readers[c.get()].push_back(const_cast<TensorNode*>(n));
                 if (seen.insert(c.get()).second) stack.push_back(c.get());
             }
         }
@@ -1231,6 +1238,7 @@ struct Scheduler {
         if (!g_fusion || n->hint == HintKind::None) return false;
         switch (n->hint) {
             case HintKind::Swish: return false;  // no kernel of its own: only matched as part of swiglu_matmul
+            case HintKind::Rope: return false;   // likewise: only matched as the epilogue of a packed projection (rope_matmul)
             case HintKind::Softmax:
                 return n->dtype == Scalar::Float32 && !n->shape.empty() &&
                        n->arg[0] == static_cast<int64_t>(n->shape.size()) - 1 && n->numel() > 0;
@@ -1569,6 +1577,78 @@ struct Scheduler {
         return kOk;
     }
 
+    // contiguous(cast_bf16(apply_rotary_emb(reshape(p[:, :split], [B, S, heads, 128]), cos, sin))) over a packed
+    // bf16 projection p = a @ w whose only other reader is the slice p[:, split:] (q | k and v of a fused
+    // QKV product): the product kernel rotates the heads in its epilogue and writes the two parts to
+    // buffers of their own, so the packed product is never written and read again.  Returns the
+    // product node and the node of the unrotated slice (nullptr when split == N).
+    TensorNode* rope_matmul(TensorNode* n, TensorNode** rest, int64_t* split_out, int64_t* seq_out) const {
+        if (!g_fusion || n->kind != TKind::Contiguous || n->dtype != Scalar::BFloat16 || n->numel() == 0) return nullptr;
+        auto used_once = [&](const TensorNode* t) {
+            auto u = uses.find(t);
+            return u != uses.end() && u->second == 1;
+        };
+        const TensorNode* c = n->src[0].get();
+        if (c->buffer || c->kind != TKind::Cast || !used_once(c)) return nullptr;
+        const TensorNode* rp = c->src[0].get();
+        if (rp->buffer || rp->hint != HintKind::Rope || rp->hint_inputs.size() != 3 || !used_once(rp)) return nullptr;
+        const TensorNode* x = rp->hint_inputs[0].get();  // [B, S, heads, 128], read by the two half slices only
+        const TensorNode *cs = rp->hint_inputs[1].get(), *sn = rp->hint_inputs[2].get();
+        if (x->buffer || x->kind != TKind::Reshape || x->shape.size() != 4 || x->shape[3] != 128 || x->dtype != Scalar::BFloat16) return nullptr;
+        auto ux = uses.find(x);
+        if (ux == uses.end() || ux->second != 2) return nullptr;
+        const int64_t S = x->shape[1];
+        for (const TensorNode* t : {cs, sn})  // tables [1, S, 1, 64] f32, in memory
+            if (!t->buffer || t->dtype != Scalar::Float32 || t->shape != std::vector<int64_t>{1, S, 1, 64} || t->buffer->offset() % 32) return nullptr;
+        const TensorNode* sl = x->src[0].get();  // p[:, :split]
+        if (sl->buffer || sl->kind != TKind::Shrink || !used_once(sl) || sl->shape.size() != 2) return nullptr;
+        TensorNode* mm = sl->src[0].get();
+        if (mm->buffer || mm->hint != HintKind::Matmul || !fusable(mm) || mm->dtype != Scalar::BFloat16 || mm->shape.size() != 2) return nullptr;
+        if (mm->hint_inputs[0]->shape.size() != 2 || mm->hint_inputs[1]->shape.size() != 2 || transposed_weight(mm)) return nullptr;
+        const int64_t M = mm->shape[0], N = mm->shape[1], K = mm->hint_inputs[0]->shape[1], split = sl->shape[1];
+        if (sl->shape[0] != M || sl->arg.size() != 2 || sl->arg[0] != 0 || sl->arg[1] != 0) return nullptr;
+        if (x->shape[0] * S != M || x->shape[2] * 128 != split || !gemm_bf16_rope_supported(M, N, K, split, S)) return nullptr;
+        // the product's readers: this slice and, when there are columns left, exactly the slice of all of them
+        auto readers = matmul_readers.find(mm);
+        if (readers == matmul_readers.end()) return nullptr;
+        TensorNode* other = nullptr;
+        for (TensorNode* r : readers->second)
+            if (r != sl) {
+                if (other && other != r) return nullptr;
+                other = r;
+            }
+        if (split == N) {
+            if (other) return nullptr;
+        } else {
+            if (!other || other->buffer || other->kind != TKind::Shrink || other->shape != std::vector<int64_t>{M, N - split} || other->arg.size() != 2 ||
+                other->arg[0] != 0 || other->arg[1] != split)
+                return nullptr;
+        }
+        *rest = other;
+        *split_out = split;
+        *seq_out = S;
+        return mm;
+    }
+    int materialize_rope_matmul(TensorNode* n, TensorNode* mm, TensorNode* rest, int64_t split, int64_t seq) {
+        const TensorNode* rp = n->src[0]->src[0].get();
+        int64_t M, N, K, batch;
+        matmul_extents(mm, &M, &N, &K, &batch);
+        MRK_TRY(materialize(mm->hint_inputs[0].get()));
+        MRK_TRY(materialize(mm->hint_inputs[1].get()));
+        const std::shared_ptr<Buffer>&a = mm->hint_inputs[0]->buffer, &w = mm->hint_inputs[1]->buffer;
+        if (a->offset() % 16 || w->offset() % 16) return fail(kRuntime, "rope_matmul: unaligned operand");  // (views of whole tensors start aligned)
+        auto out = new_buffer(n);
+        std::shared_ptr<Buffer> rest_buf = rest ? new_buffer(rest) : out;
+        MRK_TRY(builtin("gemm_bf16_rope", {M, N, K, split, seq}, {out, a, w, rest_buf, rp->hint_inputs[1]->buffer, rp->hint_inputs[2]->buffer}));
+        n->buffer = out;
+        produced.push_back(n);
+        if (rest) {
+            rest->buffer = rest_buf;
+            produced.push_back(rest);
+        }
+        return kOk;
+    }
+
     int materialize(TensorNode* n) {
         if (n->buffer) return kOk;
         if (n->kind == TKind::Copy) return materialize_copy(n);
@@ -1577,6 +1657,8 @@ struct Scheduler {
             TensorNode* other = nullptr;
             if (TensorNode* mm = residual_matmul(n, &other)) return materialize_residual_matmul(n, mm, other);
             if (TensorNode* mm = swiglu_matmul(n)) return materialize_swiglu_matmul(n, mm);
+            int64_t split = 0, seq = 0;
+            if (TensorNode* mm = rope_matmul(n, &other, &split, &seq)) return materialize_rope_matmul(n, mm, other, split, seq);
         }
         {
             std::vector<int64_t> out_strides;

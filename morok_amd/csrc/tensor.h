@@ -37,7 +37,7 @@ enum class TKind : uint8_t {
 // Device id of data that lives in host memory (DeviceSpec::Cpu); HIP devices are 0, 1, ...
 constexpr int kCpuDevice = -1;
 
-enum class HintKind : uint8_t { None, Softmax, Matmul, Sdpa, Swish };
+enum class HintKind : uint8_t { None, Softmax, Matmul, Sdpa, Swish, Rope };
 
 struct TensorNode;
 using TensorRef = std::shared_ptr<TensorNode>;

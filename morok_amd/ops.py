@@ -88,6 +88,21 @@ def gemm_bf16_residual(a, b, r, c, m, n, k, device_id=0):
     check(lib.mrk_hip_gemm_bf16_residual(device_id, _p(a), _p(b), _p(r), _p(c), m, n, k))
 
 
+def gemm_bf16_rope(a, b, cos, sin, c_rot, c_rest, m, n, k, split, seq, device_id=0):
+    """c_rot[m, split] = rotary embedding (heads of 128 columns, non-interleaved, position = row % seq,
+    cos / sin [seq, 64] f32) of the first `split` columns of a[m,k] @ b[k,n]; c_rest[m, n - split] =
+    the remaining columns, unrotated.  One kernel: the rotation runs in the product's epilogue."""
+    _need(a, m * k * 2, "gemm A")
+    _need(b, k * n * 2, "gemm B")
+    _need(cos, seq * 64 * 4, "rope cos")
+    _need(sin, seq * 64 * 4, "rope sin")
+    _need(c_rot, m * split * 2, "gemm C (rotated part)")
+    if split < n:
+        _need(c_rest, m * (n - split) * 2, "gemm C (rest)")
+    check(lib.mrk_hip_gemm_bf16_rope(device_id, _p(a), _p(b), _p(cos), _p(sin), _p(c_rot), _p(c_rest) if split < n else None, m, n, k,
+                                     split, seq))
+
+
 def flash_attn_fwd_bf16(q, k, v, o, batch, heads, sq, sk, d, scale, causal=True, device_id=0):
     """Fused SDPA forward (Tensor::scaled_dot_product_attention, tensor/src/transformer.rs:78-137)."""
     _need(q, batch * heads * sq * d * 2, "attention Q")

@@ -351,3 +351,51 @@ def test_gemm_transposed_second_operand_epilogues(dev, shape):
         morok_amd.Program.builtin("gemm_bf16_swiglu", [M, F, K], dev.device_id).execute([g0, ba, bw])
         morok_amd.Program.builtin("gemm_bf16_nt_swiglu", [M, F, K], dev.device_id).execute([g1, ba, bwt])
         assert np.array_equal(g0.copyout(np.uint16, (M, F)), g1.copyout(np.uint16, (M, F)))
+
+
+@pytest.mark.parametrize("shape", [(256, 768, 128, 512, 64), (512, 1536, 256, 1024, 128), (300, 512, 192, 512, 100), (1000, 1288, 320, 768, 77),
+                                   (256, 512, 64, 256, 256), (256, 512, 128, 512, 32)])
+def test_gemm_rotary_epilogue(dev, oracle, shape):
+    """The packed projection with the rotary embedding of its first `split` columns (heads of 128) in
+    the product's epilogue: against the oracle's product followed by its rotary stage on the
+    bf16-rounded product (f32 arithmetic, one rounding) and against the plain product for the
+    unrotated rest; rows past a multiple of 256, a rest that is not a multiple of 256 columns and
+    positions that wrap (row % seq) included; NaNs behind both results show nothing is written past them."""
+    M, N, K, split, seq = shape
+    a = synth.normal_bf16((M, K), 3, 30)
+    b = synth.normal_bf16((K, N), 3, 31)
+    ang = synth.uniform((seq, 64), 3, 32) * np.float32(3.0)
+    cos, sin = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    ba, bb = morok_amd.Buffer.from_numpy(a, dev.device_id), morok_amd.Buffer.from_numpy(b, dev.device_id)
+    bcos, bsin = morok_amd.Buffer.from_numpy(cos, dev.device_id), morok_amd.Buffer.from_numpy(sin, dev.device_id)
+    rest = N - split
+    brot = morok_amd.Buffer.from_numpy(np.full(M * split + 2048, 0x7FC0, np.uint16), dev.device_id)
+    brest = morok_amd.Buffer.from_numpy(np.full(M * rest + 2048, 0x7FC0, np.uint16), dev.device_id)
+    ops.gemm_bf16_rope(ba, bb, bcos, bsin, brot, brest, M, N, K, split, seq, dev.device_id)
+    rot_all, rest_all = brot.copyout(np.uint16), brest.copyout(np.uint16)
+    assert np.all(rot_all[M * split:] == 0x7FC0) and np.all(rest_all[M * rest:] == 0x7FC0)
+    got_rot, got_rest = rot_all[: M * split].reshape(M, split), rest_all[: M * rest].reshape(M, rest)
+    plain = _gemm(dev, a, b)
+    assert np.array_equal(got_rest, plain[:, split:])                        # the unrotated columns: the plain product's bits
+    heads = split // 128
+    x = synth.from_bf16(plain[:, :split]).reshape(M, heads, 128)             # the bf16-rounded product, as the separate kernel reads it
+    pos = np.arange(M) % seq
+    want = oracle.rope_f32(x, cos[pos][:, None, :], sin[pos][:, None, :], False).reshape(M, split)
+    gf = synth.from_bf16(got_rot)
+    assert np.all(np.isfinite(gf))
+    # the same arithmetic up to the contraction of a multiply-add: within one bf16 rounding of the f32 result
+    assert np.all(np.abs(gf - want) <= np.abs(want) * 2.0 ** -7 + 1e-6 * np.abs(x).max())
+    ref_prod = synth.from_bf16(oracle.gemm_bf16(a, b))[:, :split].reshape(M, heads, 128)
+    ref = oracle.rope_f32(ref_prod, cos[pos][:, None, :], sin[pos][:, None, :], False).reshape(M, split)
+    assert np.abs(gf - ref).max() <= 2e-2 * np.abs(ref).max()
+    # as a plan item
+    brot2, brest2 = dev.buffer(M * split * 2), dev.buffer(max(M * rest * 2, 2))
+    morok_amd.Program.builtin("gemm_bf16_rope", [M, N, K, split, seq], dev.device_id).execute([brot2, ba, bb, brest2, bcos, bsin])
+    assert np.array_equal(brot2.copyout(np.uint16, (M, split)), got_rot)
+
+
+def test_gemm_rotary_epilogue_refusals(dev):
+    b = dev.buffer(1 << 20).ensure_allocated()
+    for (m, n, k, split, seq) in [(64, 512, 72, 256, 8), (64, 512, 64, 128, 8), (64, 512, 64, 768, 8), (64, 508, 64, 256, 8), (64, 512, 64, 256, 0)]:
+        with pytest.raises(morok_amd.MorokHipError):
+            ops.gemm_bf16_rope(b, b, b, b, b, b, m, n, k, split, seq, dev.device_id)

@@ -438,7 +438,9 @@ def test_decoder_block_lowering(T, shim, fused, gemms):
     assert sum(k.startswith("gemm_bf16_residual") for k in names) == 2
     # with gate and up stored side by side, silu(gate) * up happens in the epilogue of their product
     assert sum(k.startswith("gemm_bf16_swiglu") for k in names) == (1 if fused else 0)
-    assert len(names) == (11 if fused else 16)   # fused: q and k also share one rotary kernel
+    # fused: q | k are rotated in the epilogue of the packed QKV product (no rotary kernel of its own)
+    assert sum(k.startswith("gemm_bf16_rope") for k in names) == (1 if fused else 0)
+    assert len(names) == (10 if fused else 16)
 
 
 def test_linear_layout_weights_are_read_in_place(T, shim):
