@@ -615,12 +615,48 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
                 *LDS_PTR(bf16x4, sC + (i * 16 + (lane & 15)) * kCPitchT + (j * 16 + 4 * (lane >> 4)) * 2) = h;
             }
         };
+        // Rotary epilogue: the angles of a tile row (four store steps: eight cos and eight sin values each)
+        // are requested one tile row ahead; the row's position advances by the rows of a store step,
+        // wrapping at seq, so the only division is the one that finds the first position.
+        f32x8 cs_nxt[kRope ? kPerRow : 1], sn_nxt[kRope ? kPerRow : 1], cs_cur[kRope ? kPerRow : 1], sn_cur[kRope ? kPerRow : 1];
+        unsigned rope_pos = 0;
+        auto fetch_angles = [&]() {
+            if constexpr (kRope) {
+                const unsigned seq = (unsigned)rope.seq;
+#pragma unroll
+                for (int t = 0; t < kPerRow; t++) {
+                    cs_nxt[t] = *reinterpret_cast<const f32x8*>(rope.cos + (size_t)rope_pos * 64 + (lc & 7) * 8);
+                    sn_nxt[t] = *reinterpret_cast<const f32x8*>(rope.sin + (size_t)rope_pos * 64 + (lc & 7) * 8);
+                    rope_pos += kRowsPerIt;
+                    if (seq < (unsigned)kRowsPerIt) rope_pos %= seq;
+                    else if (rope_pos >= seq) rope_pos -= seq;
+                }
+            }
+        };
+        if constexpr (kRope) {
+            if (rotate) {
+                rope_pos = (unsigned)((row0 + lr) % (size_t)rope.seq);
+                fetch_angles();
+            }
+        }
         stage_row(0);
 #pragma unroll
         for (int i = 0; i < kI16; i++) {
-            u32x4 v[kPerRow];
+            u32x4 v[kPerRow], pv[kRope ? kPerRow : 1];
 #pragma unroll
             for (int t = 0; t < kPerRow; t++) v[t] = *LDS_PTR(u32x4, sCl + (i * 16 + t * kRowsPerIt) * kCPitchT);
+            if constexpr (kRope) {
+                if (rotate) {
+                    // the partners 64 columns away: chunk lc ^ 8 of the same staged rows
+#pragma unroll
+                    for (int t = 0; t < kPerRow; t++) {
+                        pv[t] = *LDS_PTR(u32x4, sC + (i * 16 + t * kRowsPerIt + lr) * kCPitchT + (lc ^ 8) * 16);
+                        cs_cur[t] = cs_nxt[t];
+                        sn_cur[t] = sn_nxt[t];
+                    }
+                    if (i + 1 < kI16) fetch_angles();
+                }
+            }
             __builtin_amdgcn_sched_barrier(0);
             if (i + 1 < kI16) stage_row(i + 1);
             __builtin_amdgcn_sched_barrier(0);
@@ -634,16 +670,11 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
                 }
                 if constexpr (kRope) {
                     if (rotate) {
-                        // this lane's 8 columns of a head, their partners 64 columns away (chunk lc ^ 8 of the
-                        // same staged row), and the 8 angles of the row's position
-                        const u32x4 pv = *LDS_PTR(u32x4, sC + (r + lr) * kCPitchT + (lc ^ 8) * 16);
+                        // this lane's 8 columns of a head, their partners, and the 8 angles of the row's position
                         const f32x8 x = __builtin_convertvector(__builtin_bit_cast(bf16x8, v[t]), f32x8);
-                        const f32x8 y = __builtin_convertvector(__builtin_bit_cast(bf16x8, pv), f32x8);
-                        const size_t pos = (row0 + r + lr) % (size_t)rope.seq;
-                        const f32x8 cs = *reinterpret_cast<const f32x8*>(rope.cos + pos * 64 + (lc & 7) * 8);
-                        f32x8 sn = *reinterpret_cast<const f32x8*>(rope.sin + pos * 64 + (lc & 7) * 8);
-                        if (lc < 8) sn = -sn;  // first half: x1 cos - x2 sin; second half: x2 cos + x1 sin
-                        const f32x8 o = x * cs + y * sn;
+                        const f32x8 y = __builtin_convertvector(__builtin_bit_cast(bf16x8, pv[t]), f32x8);
+                        const f32x8 sn = lc < 8 ? -sn_cur[t] : sn_cur[t];  // first half: x1 cos - x2 sin; second half: x2 cos + x1 sin
+                        const f32x8 o = x * cs_cur[t] + y * sn;
                         v[t] = __builtin_bit_cast(u32x4, __builtin_convertvector(o, bf16x8));
                     }
                 }
