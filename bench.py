@@ -335,6 +335,54 @@ def bench_flash(m, dev, steps, warmup, cpu):
     return rec
 
 
+def bench_flash_options(m, dev, steps, warmup, cpu):
+    """The attention of configs[3] with the options of tensor/src/transformer.rs:112-132 inside the fused
+    kernel: a key-padding Bool mask [B, 1, 1, S] together with the causal rule, and (second figure) an additive
+    bf16 mask [S, S] with a softcap, which makes the kernel visit every key tile."""
+    import numpy as np
+
+    from morok_amd import ops, synth
+
+    B, H, S, D = 8, 32, 4096, 128
+    n = B * H * S * D
+    bq, bk, bv, bo = (dev.buffer(n * 2).ensure_allocated() for _ in range(4))
+    for i, b in enumerate((bq, bk, bv)):
+        ops.fill_normal(b, n, seed=4, tensor_id=i, bf16=True)
+    pad = np.ones((B, S), np.uint8)
+    for bi in range(B):
+        pad[bi, S - 128 * bi:] = 0            # the last 128 * b keys of batch b are padding
+    bpad = m.Buffer.from_numpy(pad)
+    badd = dev.buffer(S * S * 2).ensure_allocated()
+    ops.fill_normal(badd, S * S, seed=4, tensor_id=9, bf16=True)
+    scale = 1.0 / np.sqrt(D)
+    steps = max(1, min(steps, 20))
+    ms, stats = _launch_stats(m, lambda: ops.flash_attn_fwd_bf16_ex(bq, bk, bv, bo, B, H, S, S, D, scale, True, bpad, 1, (S, 0, 0), 0.0), steps, warmup)
+    flops = 0.5 * 4.0 * B * H * S * S * D
+    tf = flops / (ms * 1e-3) / 1e12
+    rec = {
+        "metric": "flash-attn fwd TFLOP/s (causal + Bool key-padding mask)", "value": tf, "unit": "TFLOP/s", "ms_per_step": ms, "dtype": "bf16",
+        "steps": steps,
+        "config": {"workload": "causal flash-attention fwd with a Bool key-padding mask [8,1,1,4096], bf16 [8,32,4096,128]"},
+        "roofline": _roofline("flash_options", "mfma", tf, BF16_PEAK_TFLOPS, "TFLOP/s", "flash_fwd_ext_d128_bool", algorithmic_flops_per_launch=flops),
+    }
+    rec.update(stats)
+    ms2, _ = _launch_stats(m, lambda: ops.flash_attn_fwd_bf16_ex(bq, bk, bv, bo, B, H, S, S, D, scale, False, badd, 2, (0, 0, S), 30.0), steps, warmup)
+    rec["additive_mask_softcap"] = {"ms_per_step": ms2, "value": 4.0 * B * H * S * S * D / (ms2 * 1e-3) / 1e12, "unit": "TFLOP/s",
+                                    "kernel": "flash_fwd_ext_d128_add_cap", "workload": "every key tile: additive bf16 mask [4096,4096] + softcap 30"}
+    if cpu:
+        from tests.oracle_lib import Oracle
+
+        orc = Oracle()
+        sl, Sc = 16, 1024
+        q, k, v = (synth.normal_bf16((1, sl, Sc, D), 4, i) for i in range(3))
+        mask = np.ones((1, 1, 1, Sc), bool)
+        mask[..., Sc - 128:] = False
+        sec = _cpu_time(lambda: orc.sdpa_bf16_ex(q, k, v, scale, causal=True, mask=mask))
+        rec["cpu_baseline"] = {"value": 0.5 * 4.0 * sl * Sc * Sc * D / sec / 1e12, "unit": "TFLOP/s", "cores": orc.max_threads, "kind": "port",
+                               "sample": f"{sl} (batch, head) slices at S={Sc}, D=128, causal + key-padding mask (the oracle visits every key), min of 3 after 1 warm-up"}
+    return rec
+
+
 def bench_decoder(m, dev, steps, warmup, cpu):
     """configs[4]: decoder transformer block from the tensor API, bf16, hidden 4096, 32 heads x 128,
     SwiGLU 11008, RMSNorm eps 1e-6, RoPE theta 1e4, batch 4 x seq 2048 prefill, vocab 32000."""
@@ -520,7 +568,7 @@ def bench_copy(m, dev, steps, warmup, cpu):
 
 WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "decoder": bench_decoder,
              "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling,
-             "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16}
+             "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16, "flash_options": bench_flash_options}
 PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc"]
 
 
@@ -566,7 +614,7 @@ def main():
         if "cpu_baseline" in r:
             r["cpu_baseline"]["cpu_model"] = cpu_model
             r["cpu_baseline"]["host_cores"] = os.cpu_count()
-    for k in ("median_ms", "min_ms", "plan_item", "direct_abi_ms_per_step", "vendor_reference"):
+    for k in ("median_ms", "min_ms", "plan_item", "direct_abi_ms_per_step", "vendor_reference", "additive_mask_softcap"):
         if k in primary:
             line[k] = primary[k]
     if "cpu_baseline" in primary:

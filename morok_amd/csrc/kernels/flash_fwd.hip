@@ -255,7 +255,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     // first tile that needs masking for this wave: the causal diagonal (a tile is clear of
     // it iff its last key <= the wave's first query) or the ragged tail of the keys
     int first_masked = (Sk % kKT) ? Sk / kKT : ntiles;
-    if (causal && qw0 / kKT < first_masked) first_masked = qw0 / kKT;
+    if ((causal || (kExt && ext.causal_elem)) && qw0 / kKT < first_masked) first_masked = qw0 / kKT;
     const int qidx = qw0 + lq;
     const int lim = causal ? (qidx < Sk - 1 ? qidx : Sk - 1) : Sk - 1;  // last visible key
     // ---- extended kernels: mask values of a tile and the score transform
@@ -286,9 +286,12 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
     const float cap_out = kCap ? ext.cap * kLog2e : 0.0f;  // the cap in exp2 units
     const float cap_in = kCap ? 2.0f / ext.cap : 0.0f;
     // raw score (sum of q k) of key `key` -> final score in exp2 units
-    auto ext_score = [&](float s, int key, const MaskTile& mt, int kb, int e) -> float {
+    // `limits`: the tile touches the causal diagonal or the end of the keys (the others skip the compares)
+    auto ext_score = [&](float s, int key, const MaskTile& mt, int kb, int e, bool limits) -> float {
         float t = s * scale_log2e;  // scaled score, in exp2 units for now
-        if (key > lim_causal) t = -INFINITY;
+        // without a softcap -inf before or after the mask is the same thing: one compare against the
+        // smaller limit; with one the causal limit applies here and the end of the keys after the cap
+        if (limits && key > (kCap ? lim_causal : (lim_causal < Sk - 1 ? lim_causal : Sk - 1))) t = -INFINITY;
         if constexpr (kMask == 1) {
             if (((mt.g[kb][e >> 2] >> (8 * (e & 3))) & 0xffu) == 0) t = -INFINITY;
         } else if constexpr (kMask == 2) {
@@ -300,7 +303,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
             const float z = __builtin_amdgcn_exp2f(t * cap_in);
             t = cap_out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(z + 1.0f));
         }
-        if (key > Sk - 1) t = -INFINITY;  // keys that do not exist
+        if (kCap && limits && key > Sk - 1) t = -INFINITY;  // keys that do not exist
         return t;
     };
 
@@ -337,7 +340,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                 for (int e = 0; e < 16; e++)
-                    st[kb][e] = ext_score(st[kb][e], key0 + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3), mt, kb, e);
+                    st[kb][e] = ext_score(st[kb][e], key0 + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3), mt, kb, e, mask);
         } else if (mask) {
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
@@ -470,7 +473,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
 #pragma unroll
                     for (int e = e0; e < e0 + kRegs; e++) {
                         if constexpr (kExt) {
-                            nxt[kb][e] = ext_score(nxt[kb][e], key0n + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3), mt, kb, e);
+                            nxt[kb][e] = ext_score(nxt[kb][e], key0n + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3), mt, kb, e, decltype(mask_next)::value);
                         } else if (decltype(mask_next)::value) {
                             const int key = key0n + kb * 32 + 8 * (e >> 2) + 4 * lg + (e & 3);
                             if (key > lim) nxt[kb][e] = -INFINITY;
@@ -506,8 +509,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         constexpr std::false_type more{};
         if constexpr (kD < 256) {
             const int nl = nmine - 1;  // iterations that have a next tile; the wave's last one is a body of its own
-            // iterations whose next tile is unmasked (none in the extended kernels: every tile is transformed)
-            const int jm = kExt ? 0 : (first_masked - 1 < nl ? first_masked - 1 : nl);
+            const int jm = first_masked - 1 < nl ? first_masked - 1 : nl;  // iterations whose next tile is unmasked
             for (; j + 1 < jm; j += 2) {
                 body(j, sa, mxa, sb, mxb, std::false_type{}, more);
                 body(j + 1, sb, mxb, sa, mxa, std::false_type{}, more);
@@ -535,7 +537,7 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         } else {
             // with 512-byte rows one more instantiation of the body would push the kernel over
             // its register budget: the last tile runs the ordinary body and its S(j+1) goes unused
-            const int jm = kExt ? 0 : (first_masked - 1 < nmine ? first_masked - 1 : nmine);
+            const int jm = first_masked - 1 < nmine ? first_masked - 1 : nmine;
             for (; j + 1 < jm; j += 2) {
                 body(j, sa, mxa, sb, mxb, std::false_type{}, more);
                 body(j + 1, sb, mxb, sa, mxa, std::false_type{}, more);
