@@ -103,7 +103,9 @@ def test_wmma_lowers_to_mfma():
 
 def test_local_memory_extension_ops_render():
     spec = U.render(KL.async_copy_transposing_load(), "tr")
-    assert "global_load_lds_dwordx4" in spec.src and "s_mov_b32 m0" in spec.src and "readfirstlane" in spec.src
+    # a wave-uniform destination: M0 straight from a scalar expression, the source as the buffer's scalar
+    # base plus the per-lane terms as a 32-bit offset
+    assert "global_load_lds_dwordx4" in spec.src and "s_mov_b32 m0" in spec.src and '"s"(data1 + 0)' in spec.src
     assert 's_waitcnt vmcnt(0)' in spec.src
     assert "__builtin_amdgcn_ds_read_tr16_b64_v4bf16(" in spec.src
     morok_amd.compile_spec(spec)

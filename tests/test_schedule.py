@@ -270,7 +270,9 @@ def test_wmma_matmul_direct_copy_one_wave_per_simd_is_written_out():
     assert "__builtin_amdgcn_mfma_f32_16x16x32_bf16(" not in src
     loop = src[src.index("for (int ridx0"):]
     loop = loop[:loop.index("\n  }\n")]
-    assert "if (" not in loop and loop.count("global_load_lds_dwordx4") == 16 and loop.count("__WMMA_16_16_32_bfloat_float(") == 128
+    # each trip of the loop holds two K steps (one per stage), so stage offsets are constants
+    assert "ridx0 < 2;" in loop
+    assert "if (" not in loop and loop.count("global_load_lds_dwordx4") == 32 and loop.count("__WMMA_16_16_32_bfloat_float(") == 256
     # no two reads or copies without a tensor-core instruction between them
     kinds = [("w" if "__WMMA_" in l else "m" if ("global_load_lds" in l or "ds_read_tr16" in l) else "") for l in loop.split("\n")]
     seq = "".join(kinds)
@@ -293,7 +295,8 @@ def test_tc_matmul_direct_copy_refuses_what_it_cannot_tile():
                         ((512, 512, 256), (2, 2, 2, 2, 1, 2)),     # the K step is 64 deep
                         ((512, 512, 256), (1, 1, 2, 2, 0, 2)),     # 32 columns: no whole granule group
                         ((1024, 1024, 256), (4, 4, 8, 8, 0, 2)),   # two stages of 512 x 512 exceed local memory
-                        ((512, 512, 256), (2, 2, 2, 2, 0, 3))):    # no such variant
+                        ((512, 512, 128), (2, 2, 2, 2, 0, 3)),     # three stages need more than two K steps
+                        ((512, 512, 256), (2, 2, 2, 2, 0, 4))):    # no such variant
         with pytest.raises(morok_amd.MorokHipError):
             sched.build_wmma_matmul_lds_opts(3, *shape, U.BF16, opts)
     with pytest.raises(morok_amd.MorokHipError):
