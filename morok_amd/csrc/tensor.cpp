@@ -1226,12 +1226,44 @@ struct Scheduler {
         *max_numel = std::max(*max_numel, n->numel());
         if (n->buffer) return;
         TensorNode* other = nullptr;
-        if (n != root && (is_boundary_kind(n) || fusable(n) || generated_tc(n) ||
-                          residual_matmul(const_cast<TensorNode*>(n), &other) || swiglu_matmul(n))) {
+        if (n != root && !side_inline.count(n) &&
+            (is_boundary_kind(n) || fusable(n) || generated_tc(n) || residual_matmul(const_cast<TensorNode*>(n), &other) || swiglu_matmul(n))) {
             out.push_back(const_cast<TensorNode*>(n));
             return;
         }
         for (const TensorRef& s : n->src) boundaries(s.get(), root, seen, out, max_numel);
+    }
+    // Tensors the row-resident kernel being generated computes in passing and also writes out
+    // (its side outputs): boundaries() looks through them, emit() evaluates them in place.
+    std::set<const TensorNode*> side_inline;
+
+    // An input of a row-resident kernel rooted at `n` that this kernel can produce itself: an
+    // elementwise expression the caller wants in memory (`contiguous()`) that nobody has computed
+    // yet, of the kernel's own shape and element size, so that every work-item holds exactly the
+    // elements it would otherwise load (an embedding lookup in front of the first normalisation
+    // of a decoder block: the looked-up rows are written for the residual and normalised without
+    // being read back).  Anything with a kernel of its own kind (a product, an attention, a copy
+    // between devices, a reshape of data in memory) keeps it.
+    bool side_output_candidate(const TensorNode* d, const TensorNode* n) {
+        if (d->buffer || d->kind != TKind::Contiguous || d->hint != HintKind::None || d->shape != n->shape || d->numel() == 0) return false;
+        if (d->dtype == Scalar::Bool || scalar_size(d->dtype) != scalar_size(n->dtype)) return false;
+        const TensorNode* s = d->src[0].get();
+        TensorNode* other = nullptr;
+        if (s->buffer || is_boundary_kind(s) || fusable(s) || generated_tc(s) || residual_matmul(const_cast<TensorNode*>(s), &other) || swiglu_matmul(s)) return false;
+        {
+            TensorNode* rest = nullptr;
+            int64_t split = 0, seq = 0;
+            std::vector<int64_t> out_strides;
+            if (rope_matmul(const_cast<TensorNode*>(d), &rest, &split, &seq) || attention_under(const_cast<TensorNode*>(d), &out_strides)) return false;
+        }
+        // no reduction of the row's own may hide under it (it would have to be fused as well)
+        std::set<const TensorNode*> seen;
+        std::vector<TensorNode*> deps;
+        int64_t ignore = 0;
+        boundaries(d, d, seen, deps, &ignore);
+        for (const TensorNode* x : deps)
+            if (!x->buffer && x->kind == TKind::Reduce) return false;
+        return true;
     }
 
     bool fusable(const TensorNode* n) const {
@@ -1688,23 +1720,56 @@ struct Scheduler {
         int64_t row_block = 0;
         const std::vector<TensorNode*> Rs = row_reduce_deps(n, deps, &row_block);
         if (!Rs.empty()) {
+            std::vector<TensorNode*> sides;
+            {
+                const char* off = std::getenv("MOROK_NO_SIDE_OUTPUTS");  // measurement switch
+                const bool enabled = !(off && off[0] && off[0] != '0');
+                for (TensorNode* d : deps)
+                    if (enabled && sides.size() < 2 && side_output_candidate(d, n)) sides.push_back(d);
+                for (TensorNode* R : Rs) {  // the reductions' expressions may read such a tensor as well
+                    if (!enabled) break;
+                    std::set<const TensorNode*> seen_r;
+                    std::vector<TensorNode*> deps_r;
+                    int64_t ignore = 0;
+                    boundaries(R, R, seen_r, deps_r, &ignore);
+                    for (TensorNode* d : deps_r)
+                        if (sides.size() < 2 && std::find(sides.begin(), sides.end(), d) == sides.end() && side_output_candidate(d, n)) sides.push_back(d);
+                }
+            }
+            struct ClearSides {
+                std::set<const TensorNode*>& s;
+                ~ClearSides() { s.clear(); }
+            } clear_sides{side_inline};
+            if (!sides.empty()) {
+                side_inline.insert(sides.begin(), sides.end());
+                seen.clear();
+                deps.clear();
+                boundaries(n, n, seen, deps, &max_numel);
+            }
             // everything any part of the kernel reads has to exist: the other inputs of the elementwise
             // part and the inputs of the reductions' own expressions
             auto fused = [&](const TensorNode* d) { return std::find(Rs.begin(), Rs.end(), d) != Rs.end(); };
+            auto input = [&](TensorNode* d) {  // the kernels of this kernel's inputs are scheduled on their own terms
+                std::set<const TensorNode*> mine;
+                mine.swap(side_inline);
+                const int rc = materialize(d);
+                mine.swap(side_inline);
+                return rc;
+            };
             for (TensorNode* d : deps)
-                if (!fused(d)) MRK_TRY(materialize(d));
+                if (!fused(d)) MRK_TRY(input(d));
             for (TensorNode* R : Rs) {
                 std::set<const TensorNode*> seen_r;
                 std::vector<TensorNode*> deps_r;
                 boundaries(R, R, seen_r, deps_r, &max_numel);
                 for (TensorNode* d : deps_r)
-                    if (!fused(d)) MRK_TRY(materialize(d));
+                    if (!fused(d)) MRK_TRY(input(d));
             }
             if (const char* e = std::getenv("MOROK_BEAM")) {
                 const int beam = std::atoi(e);
-                if (beam > 0 && !dry) return beam_generated(n, max_numel, beam, &Rs, row_block);
+                if (beam > 0 && !dry) return beam_generated(n, max_numel, beam, &Rs, row_block, &sides);
             }
-            return gen_row_fused(n, Rs, row_block, max_numel);
+            return gen_row_fused(n, Rs, row_block, max_numel, sides);
         }
         for (TensorNode* d : deps) MRK_TRY(materialize(d));
         if (const char* e = std::getenv("MOROK_BEAM")) {
@@ -1721,10 +1786,11 @@ struct Scheduler {
     // like the matmul searches: UPCAST then LOCAL for an elementwise kernel, GROUP (waves per
     // output and segments) then LOCAL (outputs per workgroup) for a wave reduction.  The winner
     // is cached on disk under the hash of the kernel the fixed heuristics produce.
-    int beam_generated(TensorNode* n, int64_t max_numel, int width, const std::vector<TensorNode*>* row_reduce = nullptr, int64_t row_block = 0) {
+    int beam_generated(TensorNode* n, int64_t max_numel, int width, const std::vector<TensorNode*>* row_reduce = nullptr, int64_t row_block = 0,
+                       const std::vector<TensorNode*>* sides = nullptr) {
         const bool red = n->kind == TKind::Reduce && !row_reduce;
         auto generate = [&]() -> int {
-            if (row_reduce) return gen_row_fused(n, *row_reduce, row_block, max_numel);
+            if (row_reduce) return gen_row_fused(n, *row_reduce, row_block, max_numel, sides ? *sides : std::vector<TensorNode*>());
             return red ? gen_reduce(n, max_numel) : gen_elementwise(n, max_numel);
         };
         auto build = [&](const GenOpts& o, std::vector<DryKernel>* out) -> int {
@@ -2319,7 +2385,7 @@ struct Scheduler {
         return ordered;
     }
 
-    int gen_row_fused(TensorNode* n, const std::vector<TensorNode*>& Rs, int64_t block, int64_t max_numel) {
+    int gen_row_fused(TensorNode* n, const std::vector<TensorNode*>& Rs, int64_t block, int64_t max_numel, const std::vector<TensorNode*>& sides = {}) {
         const int64_t N = n->numel(), C = n->shape.back(), rows = N / C;
         KernelGen g;
         g.idx_t = max_numel >= (1LL << 31) ? Scalar::Int64 : Scalar::Int32;
@@ -2395,8 +2461,35 @@ struct Scheduler {
             if (width > 1) b.store(b.index(po, base[i]), b.vectorize(vals));
             else b.store(b.index(po, base[i]), vals[0]);
         }
-        return finish_kernel(g, n, out, "rE_" + std::to_string(rows) + "_g" + std::to_string(C) + (width > 1 ? "_" + std::to_string(width) : "") +
-                                            (Rs.size() > 1 ? "_x" + std::to_string(Rs.size()) : ""));
+        // ---- side outputs: inputs of the row that this kernel computed in passing (the values are
+        // the ones the reductions and the outputs used: same memo entries), written where a kernel of
+        // their own would have put them
+        std::vector<std::pair<TensorNode*, std::shared_ptr<Buffer>>> side_bufs;
+        for (TensorNode* d : sides) {
+            if (d->buffer) continue;  // another input of this kernel needed it first: it is in memory, and was read from there
+            side_bufs.emplace_back(d, new_buffer(d));
+            uint32_t ps = g.buffer_param(side_bufs.back().second, d->dtype, N);
+            for (int64_t i = 0; i < per_item; i++) {
+                std::vector<uint32_t> vals;
+                for (int64_t e = 0; e < width; e++) {
+                    Coords ce = coords[i];
+                    ce.back().off = e;
+                    uint32_t v = emit(g, d, ce);
+                    if (b.dtype(v).scalar != d->dtype) v = b.cast(v, d->dtype);
+                    vals.push_back(v);
+                }
+                if (width > 1) b.store(b.index(ps, base[i]), b.vectorize(vals));
+                else b.store(b.index(ps, base[i]), vals[0]);
+            }
+        }
+        MRK_TRY(finish_kernel(g, n, out, "rE_" + std::to_string(rows) + "_g" + std::to_string(C) + (width > 1 ? "_" + std::to_string(width) : "") +
+                                             (Rs.size() > 1 ? "_x" + std::to_string(Rs.size()) : "") + (side_bufs.empty() ? "" : "_s" + std::to_string(side_bufs.size()))));
+        if (!dry)
+            for (auto& sb : side_bufs) {
+                sb.first->buffer = sb.second;
+                produced.push_back(sb.first);
+            }
+        return kOk;
     }
 
     // Materialised tensors under `n` of shape `shape`: reached through elementwise nodes only

@@ -443,6 +443,35 @@ def test_decoder_block_lowering(T, shim, fused, gemms):
     assert len(names) == (10 if fused else 16)
 
 
+def test_decoder_block_first_norm_writes_the_embedding_rows(T, shim):
+    """With rows wide enough for the row-resident kernel (hidden 512: 64 work-items of 8 elements),
+    the embedding lookup the caller asked to have in memory (`contiguous()`, the residual reads it
+    later) is computed by the first RMSNorm kernel itself and written as that kernel's second
+    output: 7 kernels in all (norm, QKV + rotary, attention, Wo + residual, norm, gated product,
+    W2 + residual); switched off, the lookup is a kernel of its own again."""
+    import os
+
+    from morok_amd import decoder, synth
+
+    cfg = dict(batch=2, seq=64, hidden=512, heads=4, ffn=1024)
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], 100, seed=1)
+
+    def lower():
+        blk = decoder.DecoderBlock(w, cfg["batch"], cfg["seq"], cfg["hidden"], cfg["heads"], cfg["ffn"])
+        return blk.forward(T.Tensor.from_numpy(synth.randint((128,), 1, 1, 100))).realize().kernels()
+
+    names = lower()
+    assert len(names) == 7, names
+    assert names[0] == "rE_128_g512_8_s1" and sum(k.startswith("rE_128_g512_8") for k in names) == 2
+    assert not any(k.startswith("E_") for k in names)
+    os.environ["MOROK_NO_SIDE_OUTPUTS"] = "1"
+    try:
+        names = lower()
+    finally:
+        del os.environ["MOROK_NO_SIDE_OUTPUTS"]
+    assert len(names) == 8 and names[0].startswith("E_") and names[1] == "rE_128_g512_8"
+
+
 def test_linear_layout_weights_are_read_in_place(T, shim):
     """x @ w.T with w [out, in] in memory (tensor/src/nn/linear.rs:39-41): the product kernels
     take the weight as it is stored instead of a transposed copy, also under the residual and the

@@ -1282,6 +1282,71 @@ def test_row_resident_norm_kernels(T, oracle, rows, cols, monkeypatch):
     assert np.array_equal(sm.to_numpy(), x - x.max(1, keepdims=True)) and len(sm.kernels()) == 1
 
 
+@pytest.mark.parametrize("rows,cols,vocab", [(256, 4096, 1000), (130, 512, 37), (1024, 1024, 5)])
+def test_row_resident_kernel_writes_the_rows_it_looked_up(T, rows, cols, vocab, monkeypatch):
+    """An embedding lookup the caller wants in memory (`contiguous()`) in front of a row-resident
+    normalisation: the normalisation's kernel looks the rows up itself and writes them as a second
+    output.  Both results carry the bits of the two-kernel path, the looked-up tensor is usable
+    afterwards (read back, and as an operand of a later kernel)."""
+    from morok_amd import synth, uop
+
+    emb = synth.normal_bf16((vocab, cols), 83, 0)
+    tok = synth.randint((rows,), 83, 1, vocab)
+    wb = synth.to_bf16(1.0 + synth.normal((cols,), 83, 2, sigma=0.1))
+
+    def run():
+        h = T.Tensor.from_numpy(emb, uop.BF16).embedding(T.Tensor.from_numpy(tok)).contiguous()
+        xn = h.rms_norm(-1, 1e-6).try_mul(T.Tensor.from_numpy(wb, uop.BF16)).cast(uop.BF16)
+        a = xn.to_numpy()
+        names = list(xn.kernels())
+        later = h.try_add(xn).to_numpy()          # h is read from memory here
+        return a, h.to_numpy(), later, names, list(T.last_kernels())
+
+    a, h, later, names, later_names = run()
+    assert names == ["rE_%d_g%d_8_s1" % (rows, cols)], names
+    assert len(later_names) == 1 and later_names[0].startswith("E_")
+    assert np.array_equal(h, emb[tok])
+    monkeypatch.setenv("MOROK_NO_SIDE_OUTPUTS", "1")
+    a2, h2, later2, names2, _ = run()
+    monkeypatch.delenv("MOROK_NO_SIDE_OUTPUTS")
+    assert len(names2) == 2 and names2[0].startswith("E_")
+    assert np.array_equal(a, a2) and np.array_equal(h, h2) and np.array_equal(later, later2)
+
+
+def test_side_output_is_left_alone_when_it_does_not_fit(T):
+    """A lookup of another element size than the row kernel's output (f32 rows under a bf16
+    normalisation) and one that another input of the same kernel needs first keep their own kernels."""
+    from morok_amd import synth, uop
+
+    emb = synth.normal((50, 1024), 84, 0)
+    tok = synth.randint((256,), 84, 1, 50)
+    h = T.Tensor.from_numpy(emb).embedding(T.Tensor.from_numpy(tok)).contiguous()
+    xn = h.rms_norm(-1, 1e-6).cast(uop.BF16)
+    xn.realize()
+    assert [k.split("_")[0] for k in xn.kernels()] == ["E", "rE"]
+    assert np.array_equal(h.to_numpy(), emb[tok])
+    # another input of the row kernel (bf16: not a side output of an f32 row) reads the lookup: it is computed
+    # first, the row kernel loads it
+    x = emb[tok]
+    ref = x / np.sqrt((x.astype(np.float64) ** 2).mean(1, keepdims=True) + 1e-6) + 2 * x
+    h = T.Tensor.from_numpy(emb).embedding(T.Tensor.from_numpy(tok)).contiguous()
+    g = h.try_mul(2.0).cast(uop.BF16).contiguous()
+    y = h.rms_norm(-1, 1e-6).try_add(g.cast(uop.F32))
+    got = y.to_numpy()
+    assert [k.split("_")[0] for k in y.kernels()] == ["E", "E", "rE"] and not y.kernels()[-1].endswith("_s1"), y.kernels()
+    g_ref = synth.from_bf16(synth.to_bf16(2 * x))
+    np.testing.assert_allclose(got, ref - 2 * x + g_ref, rtol=1e-5, atol=1e-5)
+    assert np.array_equal(h.to_numpy(), x) and np.array_equal(synth.from_bf16(g.to_numpy()), g_ref)
+    # two tensors of the row's own kind: both are written by the one kernel
+    h = T.Tensor.from_numpy(emb).embedding(T.Tensor.from_numpy(tok)).contiguous()
+    g = h.try_mul(2.0).contiguous()
+    y = h.rms_norm(-1, 1e-6).try_add(g)
+    got = y.to_numpy()
+    assert len(y.kernels()) == 1 and y.kernels()[0].endswith("_s2"), y.kernels()
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5)
+    assert np.array_equal(h.to_numpy(), x) and np.array_equal(g.to_numpy(), 2 * x)
+
+
 def test_beam_search_over_generated_kernels_keeps_values(T, tmp_path, monkeypatch):
     """Under MOROK_BEAM the choices of generated elementwise and reduce kernels are searched on the
     device (candidates timed on scratch buffers of the real sizes); whatever wins, elementwise
