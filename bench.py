@@ -38,7 +38,8 @@ MIB = 1 << 20
 # kernel, and only when that summary names the kernel this run launched; otherwise null.
 PROFILE_OF = {"softmax": "softmax_rows_in_regs_8192x8192_f32.txt", "gemm": "gemm_bf16_tile256_4096cubed.txt",
               "flash": "flash_fwd_d128_causal_8x32x4096x128.txt", "decoder": "decoder_block_4x2048_h4096.txt",
-              "generated_tc": "generated_tensor_core_gemm_4096cubed.txt", "matmul_f32": "generated_f32_matmul_1024cubed.txt"}
+              "generated_tc": "generated_tensor_core_gemm_4096cubed.txt", "matmul_f32": "generated_f32_matmul_1024cubed.txt",
+              "gemm_f16": "gemm_f16_tile256_4096cubed.txt", "flash_options": "flash_fwd_ext_d128_8x32x4096x128.txt"}
 
 
 def _profiled_traffic(workload, kernel):
