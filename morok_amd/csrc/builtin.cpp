@@ -134,15 +134,25 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
         return kOk;
     }
     // the "_nt" kinds take the second operand as B^T [N, K] (a Linear layer's weight as it is stored)
-    if (k == "gemm_bf16_nt" || k == "gemm_f16_nt") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, bt}
+    if (k == "gemm_bf16_nt" || k == "gemm_f16_nt") {  // {M, N, K}, {M, N, K, batch} or {M, N, K, batch, workspace bytes}; buffers {c, a, bt[, scratch]}
         const bool f16 = k == "gemm_f16_nt";
-        if (nparams < 3 || nparams > 4)
-            return failf(kInvalidArgument, "builtin '%s' takes 3 or 4 parameters, got %zu", k.c_str(), nparams);
+        if (nparams < 3 || nparams > 5)
+            return failf(kInvalidArgument, "builtin '%s' takes 3 to 5 parameters, got %zu", k.c_str(), nparams);
         while (p.size() < 4) p.push_back(1);
+        if (p.size() < 5) p.push_back(0);
+        if (p[4] < 0) return fail(kInvalidArgument, k + ": negative workspace size");
         if (!gemm_bf16_nt_supported(p[0], p[1], p[2], p[3]))
-            return fail(kInvalidArgument, k + ": shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel)");
+            return fail(kInvalidArgument, k + ": shape not covered (K a multiple of 8; at most 16 rows, or N a multiple of 8)");
         std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
         if (p[3] > 1) name += "_x" + std::to_string(p[3]);
+        if (p[4] > 0) {  // a fourth buffer of p[4] bytes: scratch for the split-K partial results
+            out->reset(new BuiltinProgram(device_id, stream, name + "_splitk", 4, p,
+                                          [f16](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                              return launch_gemm_bf16(s, b[1], b[2], b[0], q[0], q[1], q[2], 0, q[3], b[3],
+                                                                      static_cast<size_t>(q[4]), true, f16);
+                                          }));
+            return kOk;
+        }
         out->reset(new BuiltinProgram(device_id, stream, name, 3, p,
                                       [f16](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
                                           return launch_gemm_bf16(s, b[1], b[2], b[0], q[0], q[1], q[2], 0, q[3], nullptr, 0, true, f16);

@@ -896,12 +896,19 @@ static int gemm_16bit_nt(int device_id, const void* a, const void* bt, void* c, 
     MRK_NONNULL(bt);
     MRK_NONNULL(c);
     if (!gemm_bf16_nt_supported(m, n, k, 1))
-        return fail(kInvalidArgument, "gemm_bf16_nt: shape not covered for a second operand stored [N, K] (N and K multiples of 8, "
-                                      "K > 0, enough output tiles that split-K is not used); transpose it and run mrk_hip_gemm_bf16");
+        return fail(kInvalidArgument, "gemm_bf16_nt: shape not covered for a second operand stored [N, K] (K a multiple of 8, K > 0; "
+                                      "at most 16 rows, or N a multiple of 8); transpose it and run mrk_hip_gemm_bf16");
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_gemm_bf16(dv->allocator->stream(), a, bt, c, m, n, k, 0, 1, nullptr, 0, true, f16), "gemm_bf16_nt launch");
+    // few output tiles against a long K, more than two rows: scratch for split-K partials, as for the [K, N] form
+    const size_t ws = m > 2 ? gemm_bf16_workspace_bytes(m, n, k, 1) : 0;
+    RawBuffer scratch;
+    BufferOptions so;
+    if (ws) MRK_TRY(dv->allocator->alloc(ws, so, &scratch));
+    int rc = launch_gemm_bf16(dv->allocator->stream(), a, bt, c, m, n, k, 0, 1, ws ? scratch.ptr : nullptr, ws, true, f16);
+    if (ws) dv->allocator->free(scratch, so);
+    MRK_HIP(rc, "gemm_bf16_nt launch");
     return kOk;
 }
 

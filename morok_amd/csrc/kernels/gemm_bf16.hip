@@ -768,6 +768,17 @@ __global__ __launch_bounds__(256) void gemm_f16_tile128_splitk_ragged_k(const __
                                                                         int tiles_n, int kt_per_split) {
     gemm_tile_body<true, 2, true, false, false, false, true>(A, B, nullptr, M, N, K, tiles_m, tiles_n, W, kt_per_split);
 }
+// split-K over a second operand stored [N, K]
+#define MRK_GEMM_NT_SPLITK_KERNEL(name, ragged, f16)                                                                                   \
+    __global__ __launch_bounds__(256) void name(const __bf16* __restrict__ A, const __bf16* __restrict__ B, float* __restrict__ W, int M, \
+                                                int N, int K, int tiles_m, int tiles_n, int kt_per_split) {                             \
+        gemm_tile_body<ragged, 2, true, false, false, true, f16>(A, B, nullptr, M, N, K, tiles_m, tiles_n, W, kt_per_split);            \
+    }
+MRK_GEMM_NT_SPLITK_KERNEL(gemm_bf16_nt_tile128_splitk, false, false)
+MRK_GEMM_NT_SPLITK_KERNEL(gemm_bf16_nt_tile128_splitk_ragged_k, true, false)
+MRK_GEMM_NT_SPLITK_KERNEL(gemm_f16_nt_tile128_splitk, false, true)
+MRK_GEMM_NT_SPLITK_KERNEL(gemm_f16_nt_tile128_splitk_ragged_k, true, true)
+#undef MRK_GEMM_NT_SPLITK_KERNEL
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_rope(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                               __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
                                                               RopeEpilogue rope) {
@@ -967,9 +978,20 @@ bool gemm_bf16_residual_supported(long M, long N, long K, long batch) {
     return tm128 * tn <= 0x7fffffffL;
 }
 
+namespace {
+// shapes the tiled kernels address (any M; N and K in whole 16-byte chunks; 32-bit offsets inside a tile)
+bool tiled_shape(long M, long N, long K, long batch) {
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || batch > 65535) return false;
+    if (M > 0x7fffffffL || N > 0x7fffffffL || N % 8 || K % 8 || K > (1L << 23) || N >= (1L << 25)) return false;
+    const long tn = (N + mrk::dev::kBN - 1) / mrk::dev::kBN, tm128 = (M + 127) / 128;
+    return tm128 * tn <= 0x7fffffffL;
+}
+}  // namespace
+
 bool gemm_bf16_nt_supported(long M, long N, long K, long batch) {
-    // the tiled kernels only (no split-K, no any-shape kernel for this operand layout)
-    return gemm_bf16_residual_supported(M, N, K, batch);
+    // the tiled kernels (no any-shape kernel for this operand layout), or the streaming kernel for a
+    // handful of rows
+    return tiled_shape(M, N, K, batch) || gemm_nt_skinny_supported(M, N, K, batch);
 }
 
 int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch,
@@ -1063,7 +1085,32 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
     if (b_transposed) {
         // B given as Bt[N, K]: the tiled kernels, or nothing (variant 3 / 4 force a tile size)
         if (!aligned || !gemm_bf16_nt_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
+        const bool choose = variant == 0 || variant == 5;  // 3 / 4 force a tile where the shape has one
+        const bool tiled = tiled_shape(M, N, K, batch);
+        // one or two rows: one pass over the weight on the vector ALUs streams it faster than any tile
+        if (gemm_nt_skinny_supported(M, N, K, batch) && (!tiled || (choose && M <= 2)))
+            return launch_gemm_nt_skinny(stream, A, B, C, M, N, K, batch, f16);
         const long tn = (N + kBN - 1) / kBN, tm128 = (M + 127) / 128;
+        const SplitPlan sp = choose ? plan_split_k(M, N, K, batch) : SplitPlan();
+        if (sp.splits > 1) {
+            // few output tiles against a long K: the K loop spread over the chip when the caller
+            // brought the workspace for the partial results; without one, up to 16 rows stream
+            // (anything else runs the plain tiled kernel on the few workgroups it has)
+            if (workspace && workspace_bytes >= (size_t)sp.splits * batch * M * N * sizeof(float) &&
+                reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && batch * sp.splits <= 65535) {
+                const dim3 grid((unsigned)(tm128 * tn), (unsigned)batch, (unsigned)sp.splits);
+                float* w = static_cast<float*>(workspace);
+                auto split_kernel = f16 ? (K % kBK == 0 ? gemm_f16_nt_tile128_splitk : gemm_f16_nt_tile128_splitk_ragged_k)
+                                        : (K % kBK == 0 ? gemm_bf16_nt_tile128_splitk : gemm_bf16_nt_tile128_splitk_ragged_k);
+                split_kernel<<<grid, 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B), w, (int)M, (int)N, (int)K,
+                                                  (int)tm128, (int)tn, (int)sp.kt_per_split);
+                const long total = batch * M * N;
+                auto reduce_kernel = f16 ? gemm_splitk_reduce<true> : gemm_splitk_reduce<false>;
+                reduce_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>(w, static_cast<__bf16*>(C), total, (int)sp.splits);
+                return (int)hipGetLastError();
+            }
+            if (gemm_nt_skinny_supported(M, N, K, batch)) return launch_gemm_nt_skinny(stream, A, B, C, M, N, K, batch, f16);
+        }
         const bool small = variant == 4 || (variant != 3 && tm128 * tn * batch <= 256);
         const long tm = small ? tm128 : (M + kBM - 1) / kBM;
         const bool ragged_k = K % kBK != 0;

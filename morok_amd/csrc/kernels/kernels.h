@@ -17,14 +17,23 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 // C [batch,M,N]), one launch.
 // b_transposed: B is stored as B^T [N, K] (k contiguous: the layout of a Linear layer's weight;
 // [batch, N, K] for batch > 1).  Same products in the same order, so the same bits as the [K, N]
-// form.  Tiled kernels only: shapes outside gemm_bf16_nt_supported (N or K not a multiple of 8,
-// so few output tiles that split-K would be used) are refused with hipErrorInvalidValue.
+// form (split-K included, given the workspace).  One or two rows, and up to 16 where the tiled
+// kernels do not apply (N not a multiple of 8, split-K shape without a workspace), take the
+// streaming kernel below, whose sums run in another order.  Shapes outside
+// gemm_bf16_nt_supported (K not a multiple of 8; N not a multiple of 8 with more than 16 rows)
+// are refused with hipErrorInvalidValue.
 // f16: operands and result are IEEE half precision instead of bf16 (the same kernels around
 // v_mfma_f32_16x16x32_f16; plain product only, the fused epilogues are bf16).
 int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
                      long batch = 1, void* workspace = nullptr, size_t workspace_bytes = 0, bool b_transposed = false,
                      bool f16 = false);
 bool gemm_bf16_nt_supported(long M, long N, long K, long batch);
+// C[M, N] = A[M, K] @ Bt[N, K]^T for M <= 16 (a decode step against a Linear layer's weight): one
+// pass over the weight with packed dot products, no matrix pipe, no scratch memory.  K a multiple
+// of 8, any N; bf16 or (f16) IEEE half operands and result, f32 accumulation.  Summation order
+// differs from the tiled kernels', so results agree with them to rounding, not bit for bit.
+bool gemm_nt_skinny_supported(long M, long N, long K, long batch);
+int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16);
 // c = bf16(float(bf16(a b)) + float(r)) with r of c's shape, added in the product kernel's epilogue
 // (same bits as the product followed by an elementwise add).  Supported for the shapes the tiled
 // kernels take without split-K; gemm_bf16_residual_supported tells.

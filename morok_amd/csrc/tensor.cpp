@@ -2087,7 +2087,7 @@ struct Scheduler {
             int64_t M, N, K, batch;
             matmul_extents(n, &M, &N, &K, &batch);
             MRK_TRY(materialize(n->hint_inputs[0].get()));
-            MRK_TRY(weight_operand(n, gemm_bf16_workspace_bytes(M, N, K, batch) == 0 && gemm_bf16_nt_supported(M, N, K, batch), &wbuf, &nt));
+            MRK_TRY(weight_operand(n, gemm_bf16_nt_supported(M, N, K, batch), &wbuf, &nt));
         } else {
             for (const TensorRef& in : n->hint_inputs) MRK_TRY(materialize(in.get()));
         }
@@ -2106,7 +2106,10 @@ struct Scheduler {
                 // of the plan like any other (lazily allocated, placed by the memory planner)
                 const size_t ws = gemm_bf16_workspace_bytes(M, N, K, batch);
                 const std::string kind = a->dtype == Scalar::Float16 ? "gemm_f16" : "gemm_bf16";
-                if (nt) {
+                if (nt && ws && M > 2) {  // (one or two rows stream the weight in one pass and need no scratch)
+                    auto scratch = std::make_shared<Buffer>(dev->allocator, ws, BufferOptions());
+                    rc = builtin((kind + "_nt").c_str(), {M, N, K, 1, static_cast<int64_t>(ws)}, {out, a->buffer, wbuf, scratch});
+                } else if (nt) {
                     rc = builtin((kind + "_nt").c_str(), {M, N, K}, {out, a->buffer, wbuf});
                 } else if (ws) {
                     auto scratch = std::make_shared<Buffer>(dev->allocator, ws, BufferOptions());

@@ -17,6 +17,11 @@ int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, 
 bool gemm_bf16_nt_supported(long M, long N, long K, long batch) {
     return M > 0 && N > 0 && K > 0 && batch > 0 && N % 8 == 0 && K % 8 == 0;
 }
+bool gemm_nt_skinny_supported(long M, long N, long K, long batch) { return M >= 1 && M <= 16 && N >= 1 && K >= 8 && K % 8 == 0 && batch >= 1; }
+int launch_gemm_nt_skinny(void* stream, const void*, const void*, void*, long, long, long, long, bool f16) {
+    mrk_shim_note_launch(stream, f16 ? "gemm_f16_nt" : "gemm_bf16_nt");
+    return 0;
+}
 int gemm_bf16_static_workspace_init(int) { return 0; }
 size_t gemm_bf16_static_workspace_capacity() { return size_t(32) << 20; }
 int launch_gemm_bf16_static_ws(void* stream, int, const void*, const void*, void*, long, long, long) {

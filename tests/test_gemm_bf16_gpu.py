@@ -323,11 +323,38 @@ def test_gemm_transposed_second_operand(dev, oracle, shape):
 
 
 def test_gemm_transposed_second_operand_refusals(dev):
-    a, b, c = dev.buffer(4 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(4 * 1024 * 2)
+    a, b, c = dev.buffer(32 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(32 * 1024 * 2)
     with pytest.raises(morok_amd.MorokHipError):
-        ops.gemm_bf16_nt(a, b, c, 4, 1024, 4096, dev.device_id)   # few tiles, long K: the split-K shape
+        ops.gemm_bf16_nt(a, b, c, 32, 1024, 4092, dev.device_id)  # K not a multiple of 8
     with pytest.raises(morok_amd.MorokHipError):
-        ops.gemm_bf16_nt(a, b, c, 4, 1020, 64, dev.device_id)     # N not a multiple of 8
+        ops.gemm_bf16_nt(a, b, c, 32, 1020, 64, dev.device_id)    # N not a multiple of 8 with more than 16 rows
+
+
+@pytest.mark.parametrize("shape", [(32, 1024, 4096), (64, 4096, 4096), (17, 520, 2048), (100, 264, 4104), (3, 4096, 4096), (128, 512, 8192)])
+def test_gemm_transposed_second_operand_split_k(dev, oracle, shape):
+    """Few output tiles against a long K with the weight stored [N, K]: the K loop is spread over the
+    chip as for the [K, N] form (same K ranges, same order inside a range: the same bits), through the
+    ABI (which brings the scratch itself) and as a plan item with a scratch buffer."""
+    M, N, K = shape
+    ws = morok_amd._ffi.lib.mrk_hip_gemm_bf16_workspace_bytes(M, N, K, 1)
+    assert ws > 0
+    a = synth.normal_bf16((M, K), 3, 30)
+    b = synth.normal_bf16((K, N), 3, 31)
+    bt = np.ascontiguousarray(b.T)
+    nan = np.full(8192, 0x7FC0, np.uint16)
+    ba = morok_amd.Buffer.from_numpy(np.concatenate([a.reshape(-1), nan]), dev.device_id)
+    bbt = morok_amd.Buffer.from_numpy(np.concatenate([bt.reshape(-1), nan]), dev.device_id)
+    bc = dev.buffer(M * N * 2 + 4096)
+    bc.copyin(np.full(M * N + 2048, 0x7FC0, np.uint16))
+    ops.gemm_bf16_nt(ba, bbt, bc, M, N, K, dev.device_id)
+    out = bc.copyout(np.uint16)
+    got = out[: M * N].reshape(M, N)
+    assert np.all(out[M * N:] == 0x7FC0)
+    _check(got, oracle.gemm_bf16(a, b), K)
+    assert np.array_equal(got, _gemm(dev, a, b))
+    bc2, scratch = dev.buffer(M * N * 2), dev.buffer(ws)
+    morok_amd.Program.builtin("gemm_bf16_nt", [M, N, K, 1, ws], dev.device_id).execute([bc2, ba, bbt, scratch])
+    assert np.array_equal(bc2.copyout(np.uint16, (M, N)), got)
 
 
 @pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 1024), (300, 264, 200), (1000, 520, 72)])

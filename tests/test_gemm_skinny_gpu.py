@@ -1,0 +1,143 @@
+"""A handful of rows against a Linear layer's weight as it is stored ([out_features, in_features],
+tensor/src/nn/linear.rs:9-14,39-41: y = x @ weight.T): the streaming kernel behind
+mrk_hip_gemm_bf16_nt / mrk_hip_gemm_f16_nt for M <= 16, against the CPU oracle (exact products, f32
+accumulate, one rounding) on identical seeded inputs.  Tolerance from the north star: <= 2e-2 max
+relative error (max|gpu - ref| / max|ref|) plus the elementwise bound of the tiled kernels' tests
+(the result's own rounding plus summation-order noise); against the tiled kernel on the transposed
+weight the results may differ by one rounding of the result."""
+import numpy as np
+import pytest
+
+import morok_amd
+from morok_amd import ops, synth
+
+pytestmark = pytest.mark.gpu
+
+@pytest.fixture()
+def T(dev):
+    from morok_amd import tensor
+
+    yield tensor
+    tensor.set_fusion(True)
+
+
+SHAPES = [(1, 4096, 4096), (1, 8, 8), (2, 1020, 64), (3, 37, 520), (4, 1024, 4096), (5, 4099, 512), (7, 256, 11008),
+          (8, 2048, 2048), (9, 130, 1032), (13, 515, 264), (16, 4096, 1024), (16, 3, 8)]
+
+
+def _check(cf, rf, K, ulp):
+    assert np.all(np.isfinite(cf))
+    scale = np.abs(rf).max()
+    assert np.abs(cf - rf).max() <= 2e-2 * scale
+    assert np.all(np.abs(cf - rf) <= np.abs(rf) * ulp + 1e-5 * np.sqrt(K) * max(scale / np.sqrt(K), 1.0))
+
+
+def _run(dev, a16, bt16, nan, f16):
+    """a16 [M, K], bt16 [N, K] as uint16 bit patterns; NaNs right behind every operand and the result."""
+    M, K = a16.shape
+    N = bt16.shape[0]
+    pad = np.full(4096, nan, np.uint16)
+    ba = morok_amd.Buffer.from_numpy(np.concatenate([a16.reshape(-1), pad]), dev.device_id)
+    bb = morok_amd.Buffer.from_numpy(np.concatenate([bt16.reshape(-1), pad]), dev.device_id)
+    bc = dev.buffer((M * N + 2048) * 2)
+    bc.copyin(np.full(M * N + 2048, nan, np.uint16))
+    # as a plan item without a scratch buffer: every shape of this file then takes the streaming kernel (one or
+    # two rows; N not a multiple of 8; few tiles against a long K, where the ABI call would bring scratch for split-K)
+    morok_amd.Program.builtin("gemm_f16_nt" if f16 else "gemm_bf16_nt", [M, N, K], dev.device_id).execute([bc, ba, bb])
+    out = bc.copyout(np.uint16)
+    assert np.all(out[M * N:] == nan)            # nothing written past the result
+    return out[: M * N].reshape(M, N), ba, bb
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_skinny_bf16_vs_oracle_and_tiled_kernel(dev, oracle, shape):
+    M, N, K = shape
+    a = synth.normal_bf16((M, K), 13, 0)
+    b = synth.normal_bf16((K, N), 13, 1)
+    bt = np.ascontiguousarray(b.T)
+    got, ba, bb = _run(dev, a, bt, 0x7FC0, False)
+    ref = oracle.gemm_bf16(a, b)
+    _check(synth.from_bf16(got), synth.from_bf16(ref), K, 2**-7)
+    # the tiled kernel on the [K, N] copy sums in another order: the same values up to the result's rounding
+    bb2 = morok_amd.Buffer.from_numpy(b, dev.device_id)
+    bc2 = dev.buffer(M * N * 2)
+    ops.gemm_bf16(ba, bb2, bc2, M, N, K, dev.device_id)
+    tiled = synth.from_bf16(bc2.copyout(np.uint16, (M, N)))
+    g = synth.from_bf16(got)
+    assert np.all(np.abs(g - tiled) <= np.abs(tiled) * 2**-7 + 2e-5 * np.sqrt(K) * max(np.abs(tiled).max() / np.sqrt(K), 1.0))
+    # again: the same bits every time (no atomics, fixed summation order)
+    bc3 = dev.buffer(M * N * 2)
+    morok_amd.Program.builtin("gemm_bf16_nt", [M, N, K], dev.device_id).execute([bc3, ba, bb])
+    assert np.array_equal(bc3.copyout(np.uint16, (M, N)), got)
+    # through the ABI (one or two rows: the same kernel; more: split-K over the tiled kernels where the shape has tiles)
+    ops.gemm_bf16_nt(ba, bb, bc3, M, N, K, dev.device_id)
+    abi = bc3.copyout(np.uint16, (M, N))
+    if M <= 2 or N % 8:
+        assert np.array_equal(abi, got)
+    else:
+        assert np.array_equal(abi, bc2.copyout(np.uint16, (M, N)))     # the bits of the [K, N] form
+
+
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (3, 37, 520), (8, 2048, 2048), (16, 1000, 1032), (6, 4099, 64)])
+def test_skinny_f16_vs_oracle(dev, oracle, shape):
+    M, N, K = shape
+    a = synth.normal((M, K), 13, 2).astype(np.float16)
+    b = synth.normal((K, N), 13, 3).astype(np.float16)
+    bt = np.ascontiguousarray(b.T)
+    got, _, _ = _run(dev, a.view(np.uint16), bt.view(np.uint16), 0x7E00, True)
+    ref = oracle.gemm_f16(a, b)
+    _check(got.view(np.float16).astype(np.float32), ref.astype(np.float32), K, 2**-10)
+
+
+def test_skinny_exact_cases(dev):
+    """Values whose sums are exact in f32 whatever the order: small integers.  Every output must be the
+    integer dot product, for every row count the kernel is instantiated for and the ones between."""
+    rng = np.random.default_rng(5)
+    for M in range(1, 17):
+        N, K = 260 + M, 1544
+        a = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+        bt = rng.integers(-4, 5, size=(N, K)).astype(np.float32)
+        got, _, _ = _run(dev, synth.to_bf16(a), synth.to_bf16(bt), 0x7FC0, False)
+        want = a.astype(np.int64) @ bt.astype(np.int64).T            # |sum| <= 16 * 1544 < 2^15: but bf16 keeps 8 bits
+        assert np.array_equal(got, synth.to_bf16(want.astype(np.float32)))
+
+
+def test_skinny_batched_plan_item(dev, oracle):
+    """{M, N, K, batch}: that many products over operands stored back to back."""
+    M, N, K, B = 4, 520, 1024, 3
+    a = synth.normal_bf16((B, M, K), 13, 4)
+    bt = synth.normal_bf16((B, N, K), 13, 5)
+    ba, bb = morok_amd.Buffer.from_numpy(a, dev.device_id), morok_amd.Buffer.from_numpy(bt, dev.device_id)
+    bc = dev.buffer(B * M * N * 2)
+    morok_amd.Program.builtin("gemm_bf16_nt", [M, N, K, B], dev.device_id).execute([bc, ba, bb])
+    got = bc.copyout(np.uint16, (B, M, N))
+    for i in range(B):
+        ref = oracle.gemm_bf16(a[i], np.ascontiguousarray(bt[i].T))
+        _check(synth.from_bf16(got[i]), synth.from_bf16(ref), K, 2**-7)
+
+
+def test_skinny_refusals(dev):
+    a, b, c = dev.buffer(64 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(64 * 1024 * 2)
+    with pytest.raises(morok_amd.MorokHipError):
+        ops.gemm_bf16_nt(a, b, c, 4, 1024, 4092, dev.device_id)    # K not a multiple of 8
+    with pytest.raises(morok_amd.MorokHipError):
+        ops.gemm_bf16_nt(a, b, c, 17, 1020, 4096, dev.device_id)   # more than 16 rows and N not a multiple of 8
+
+
+def test_linear_decode_step_is_one_kernel(T, oracle):
+    """x [1, K] (and a batch of 8) through Tensor.linear with the weight as stored: one product that
+    reads the weight in place, no transposed copy (one row streams it in one pass, eight rows take the
+    tiled kernels with the K loop spread over the chip)."""
+    from morok_amd import uop
+
+    T.set_fusion(True)
+    K, N = 2048, 3072
+    w = synth.normal_bf16((N, K), 13, 6)
+    tw = T.Tensor.from_numpy(w, uop.BF16)
+    for M in (1, 8):
+        x = synth.normal_bf16((M, K), 13, 7)
+        y = T.Tensor.from_numpy(x, uop.BF16).linear(tw)
+        got = y.to_numpy()
+        assert y.kernels() == [f"gemm_bf16_nt_{M}_{N}_{K}" + ("" if M == 1 else "_splitk")]
+        ref = oracle.gemm_bf16(x, np.ascontiguousarray(w.T))
+        _check(synth.from_bf16(got), synth.from_bf16(ref), K, 2**-7)
