@@ -437,10 +437,15 @@ int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int6
 size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t batch);
 /* c[M,N] = a[M,K] * bt[N,K]^T: the product with the second operand as it is stored by a Linear
  * layer (weight [out_features, in_features], tensor/src/nn/linear.rs:9-14, 39-41), read in place
- * instead of through a transposed copy.  Same products in the same order as mrk_hip_gemm_bf16 on
- * the transposed matrix, so the same bits.  N and K multiples of 8, 16-byte aligned operands, and
- * enough output tiles that the split-K form would not be chosen (mrk_hip_gemm_bf16_workspace_bytes
- * == 0); INVALID_ARGUMENT otherwise.  Builtin Program kind "gemm_bf16_nt". */
+ * instead of through a transposed copy.  K a multiple of 8, 16-byte aligned operands.  More than
+ * two rows with N a multiple of 8: the tiled kernels, the same products in the same order as
+ * mrk_hip_gemm_bf16 on the transposed matrix, so the same bits (split-K shapes included; the
+ * scratch comes from the device allocator).  One or two rows (a decode step), and up to 16 rows
+ * with any N: one streaming pass over the weight with packed dot products, f32 accumulation in
+ * another order (results agree with the tiled kernels to the rounding of the result).  More than
+ * 16 rows with N not a multiple of 8, or K not a multiple of 8: INVALID_ARGUMENT.  Builtin Program
+ * kind "gemm_bf16_nt" ({M, N, K[, batch[, workspace bytes]]}; without a workspace a split-K shape
+ * of up to 16 rows streams, a larger one runs the plain tiled kernel). */
 int mrk_hip_gemm_bf16_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k);
 /* The same two products on IEEE half precision (f16) operands and result, f32 accumulate: the f16
  * 16x16x32 entry of the reference's CDNA4 tensor-core table
