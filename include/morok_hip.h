@@ -438,9 +438,9 @@ size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_
 /* c[M,N] = a[M,K] * bt[N,K]^T: the product with the second operand as it is stored by a Linear
  * layer (weight [out_features, in_features], tensor/src/nn/linear.rs:9-14, 39-41), read in place
  * instead of through a transposed copy.  K a multiple of 8, 16-byte aligned operands.  More than
- * two rows with N a multiple of 8: the tiled kernels, the same products in the same order as
+ * eight rows with N a multiple of 8: the tiled kernels, the same products in the same order as
  * mrk_hip_gemm_bf16 on the transposed matrix, so the same bits (split-K shapes included; the
- * scratch comes from the device allocator).  One or two rows (a decode step), and up to 16 rows
+ * scratch comes from the device allocator).  Up to eight rows (a decode step), and up to 16 rows
  * with any N: one streaming pass over the weight with packed dot products, f32 accumulation in
  * another order (results agree with the tiled kernels to the rounding of the result).  More than
  * 16 rows with N not a multiple of 8, or K not a multiple of 8: INVALID_ARGUMENT.  Builtin Program

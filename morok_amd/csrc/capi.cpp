@@ -901,8 +901,8 @@ static int gemm_16bit_nt(int device_id, const void* a, const void* bt, void* c, 
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    // few output tiles against a long K, more than two rows: scratch for split-K partials, as for the [K, N] form
-    const size_t ws = m > 2 ? gemm_bf16_workspace_bytes(m, n, k, 1) : 0;
+    // few output tiles against a long K, more than eight rows: scratch for split-K partials, as for the [K, N] form
+    const size_t ws = m > 8 ? gemm_bf16_workspace_bytes(m, n, k, 1) : 0;
     RawBuffer scratch;
     BufferOptions so;
     if (ws) MRK_TRY(dv->allocator->alloc(ws, so, &scratch));

@@ -1087,8 +1087,8 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
         if (!aligned || !gemm_bf16_nt_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
         const bool choose = variant == 0 || variant == 5;  // 3 / 4 force a tile where the shape has one
         const bool tiled = tiled_shape(M, N, K, batch);
-        // one or two rows: one pass over the weight on the vector ALUs streams it faster than any tile
-        if (gemm_nt_skinny_supported(M, N, K, batch) && (!tiled || (choose && M <= 2)))
+        // up to eight rows: one pass over the weight on the vector ALUs streams it faster than any tile
+        if (gemm_nt_skinny_supported(M, N, K, batch) && (!tiled || (choose && M <= 8)))
             return launch_gemm_nt_skinny(stream, A, B, C, M, N, K, batch, f16);
         const long tn = (N + kBN - 1) / kBN, tm128 = (M + 127) / 128;
         const SplitPlan sp = choose ? plan_split_k(M, N, K, batch) : SplitPlan();

@@ -2,14 +2,15 @@
 // layer keeps it ([out_features, in_features], tensor/src/nn/linear.rs:9-14,39-41): the decode step
 // of a language model.  The product is a stream over the weight: 2 * N * K bytes against 2 * M * N * K
 // flops, HBM-bound for these M, so nothing is tiled for the matrix pipes.  A workgroup of four waves
-// owns four weight rows; the waves take the 512-element chunks of K in turn, a lane loads 16 bytes
-// of each of the four rows (a wave reads 1 KB of one row per instruction) and of each row of A
-// (cache hits: every workgroup reads the same few KB), and multiplies with packed two-element
-// dot products (v_dot2c_f32_bf16 / _f16: exact products, f32 accumulation).  The lanes' partial sums
-// are folded with a transposing butterfly (after step s a lane keeps half of the values it held,
-// summed with its partner's: M * 4 values take M * 4 - 1 exchanges in all, not 6 each), the four
-// waves' results meet in LDS, wave 0 adds them in a fixed order and writes the outputs.  One launch,
-// no scratch memory, no atomics: results do not depend on scheduling.
+// owns four or eight weight rows; the waves take the 512-element chunks of K in turn, a lane loads
+// 16 bytes of each of the rows (a wave reads 1 KB of one row per instruction) and of each row of A
+// (cache hits: every workgroup reads the same few KB, each starting at another chunk so that they
+// do not all queue on the same L2 channel), and multiplies with packed two-element dot products
+// (v_dot2c_f32_bf16 / _f16: exact products, f32 accumulation).  The lanes' partial sums are folded
+// with a transposing butterfly (after step s a lane keeps half of the values it held, summed with
+// its partner's: V values take V - 1 exchanges in all, not 6 each), the four waves' results meet in
+// LDS, wave 0 adds them in a fixed order and writes the outputs.  One launch, no scratch memory, no
+// atomics: results do not depend on scheduling.
 #include <hip/hip_runtime.h>
 
 #include "kernels.h"
@@ -21,7 +22,6 @@ typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
-constexpr int kRowsPerGroup = 4;  // weight rows of a workgroup
 constexpr int kChunk = 512;       // elements of K one wave covers per step (64 lanes x 8)
 
 template <bool kF16>
@@ -62,8 +62,8 @@ __device__ __forceinline__ void fold_lanes(float* acc, int lane) {
 }  // namespace
 
 // kM: rows of A the kernel holds accumulators for (M <= kM; rows beyond M repeat row M - 1 and are
-// not written).  grid = (ceil(N / 4), batch).
-template <int kM, bool kF16>
+// not written); kRowsPerGroup: weight rows of a workgroup.  grid = (ceil(N / kRowsPerGroup), batch).
+template <int kM, int kRowsPerGroup, bool kF16>
 __global__ __launch_bounds__(256) void gemm_nt_skinny(const unsigned short* __restrict__ A, const unsigned short* __restrict__ Bt,
                                                        unsigned short* __restrict__ C, int M, int N, int K) {
     constexpr int kV = kM * kRowsPerGroup;  // values a lane accumulates
@@ -86,8 +86,16 @@ __global__ __launch_bounds__(256) void gemm_nt_skinny(const unsigned short* __re
     float acc[kV];
 #pragma unroll
     for (int v = 0; v < kV; v++) acc[v] = 0.0f;
-    const int groups = K >> 3;  // 16-byte groups per row
-    for (int g = wave * 64 + lane; g < groups; g += 4 * 64) {
+    // The waves take the chunks in turn, every workgroup starting at another one: at any moment the
+    // workgroups then read different parts of A (rows of A lie a multiple of 4 KB apart for the usual K,
+    // i.e. in the same L2 channel, and workgroups in step would all queue on that one channel).
+    const int chunks = (K + kChunk - 1) / kChunk;
+    const int first = (int)(blockIdx.x % (unsigned)chunks);
+    for (int c = wave; c < chunks; c += 4) {
+        int cc = c + first;
+        if (cc >= chunks) cc -= chunks;
+        const int g = cc * 64 + lane;  // 16-byte group of the row
+        if (g >= (K >> 3)) continue;
         u32x4 w[kRowsPerGroup], x[kM];
 #pragma unroll
         for (int r = 0; r < kRowsPerGroup; r++) w[r] = __builtin_nontemporal_load(w_row[r] + g);
@@ -139,7 +147,7 @@ namespace mrk {
 
 bool gemm_nt_skinny_supported(long M, long N, long K, long batch) {
     return M >= 1 && M <= 16 && N >= 1 && K >= 8 && K % 8 == 0 && K <= 0x7fffffffL && N <= 0x7fffffffL && batch >= 1 && batch <= 65535 &&
-           (N + 3) / 4 <= 0x7fffffffL;
+           true;
 }
 
 int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16) {
@@ -147,21 +155,23 @@ int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, 
     if (!gemm_nt_skinny_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) % 16 || reinterpret_cast<uintptr_t>(C) % 2) return (int)hipErrorInvalidValue;
     (void)hipGetLastError();
-    const dim3 grid((unsigned)((N + 3) / 4), (unsigned)batch);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const unsigned short* a = static_cast<const unsigned short*>(A);
     const unsigned short* b = static_cast<const unsigned short*>(Bt);
     unsigned short* c = static_cast<unsigned short*>(C);
-#define MRK_SKINNY(KM)                                                                             \
-    do {                                                                                           \
-        if (f16) gemm_nt_skinny<KM, true><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K);   \
-        else gemm_nt_skinny<KM, false><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K);      \
+    // more weight rows per workgroup where the accumulators allow it: every workgroup reads all of A,
+    // so A's share of the traffic is M / rows
+#define MRK_SKINNY(KM, KR)                                                                                  \
+    do {                                                                                                    \
+        const dim3 grid((unsigned)((N + KR - 1) / KR), (unsigned)batch);                                    \
+        if (f16) gemm_nt_skinny<KM, KR, true><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K);        \
+        else gemm_nt_skinny<KM, KR, false><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K);           \
     } while (0)
-    if (M == 1) MRK_SKINNY(1);
-    else if (M == 2) MRK_SKINNY(2);
-    else if (M <= 4) MRK_SKINNY(4);
-    else if (M <= 8) MRK_SKINNY(8);
-    else MRK_SKINNY(16);
+    if (M == 1) MRK_SKINNY(1, 4);
+    else if (M == 2) MRK_SKINNY(2, 4);
+    else if (M <= 4) MRK_SKINNY(4, 8);
+    else if (M <= 8) MRK_SKINNY(8, 8);
+    else MRK_SKINNY(16, 4);
 #undef MRK_SKINNY
     return (int)hipGetLastError();
 }

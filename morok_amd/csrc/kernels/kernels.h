@@ -17,7 +17,7 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 // C [batch,M,N]), one launch.
 // b_transposed: B is stored as B^T [N, K] (k contiguous: the layout of a Linear layer's weight;
 // [batch, N, K] for batch > 1).  Same products in the same order, so the same bits as the [K, N]
-// form (split-K included, given the workspace).  One or two rows, and up to 16 where the tiled
+// form (split-K included, given the workspace).  Up to eight rows, and up to 16 where the tiled
 // kernels do not apply (N not a multiple of 8, split-K shape without a workspace), take the
 // streaming kernel below, whose sums run in another order.  Shapes outside
 // gemm_bf16_nt_supported (K not a multiple of 8; N not a multiple of 8 with more than 16 rows)

@@ -2106,7 +2106,7 @@ struct Scheduler {
                 // of the plan like any other (lazily allocated, placed by the memory planner)
                 const size_t ws = gemm_bf16_workspace_bytes(M, N, K, batch);
                 const std::string kind = a->dtype == Scalar::Float16 ? "gemm_f16" : "gemm_bf16";
-                if (nt && ws && M > 2) {  // (one or two rows stream the weight in one pass and need no scratch)
+                if (nt && ws && M > 8) {  // (up to eight rows stream the weight in one pass and need no scratch)
                     auto scratch = std::make_shared<Buffer>(dev->allocator, ws, BufferOptions());
                     rc = builtin((kind + "_nt").c_str(), {M, N, K, 1, static_cast<int64_t>(ws)}, {out, a->buffer, wbuf, scratch});
                 } else if (nt) {

@@ -41,8 +41,8 @@ def _run(dev, a16, bt16, nan, f16):
     bb = morok_amd.Buffer.from_numpy(np.concatenate([bt16.reshape(-1), pad]), dev.device_id)
     bc = dev.buffer((M * N + 2048) * 2)
     bc.copyin(np.full(M * N + 2048, nan, np.uint16))
-    # as a plan item without a scratch buffer: every shape of this file then takes the streaming kernel (one or
-    # two rows; N not a multiple of 8; few tiles against a long K, where the ABI call would bring scratch for split-K)
+    # as a plan item without a scratch buffer: every shape of this file then takes the streaming kernel (up to
+    # eight rows; N not a multiple of 8; few tiles against a long K, where the ABI call would bring scratch for split-K)
     morok_amd.Program.builtin("gemm_f16_nt" if f16 else "gemm_bf16_nt", [M, N, K], dev.device_id).execute([bc, ba, bb])
     out = bc.copyout(np.uint16)
     assert np.all(out[M * N:] == nan)            # nothing written past the result
@@ -69,10 +69,10 @@ def test_skinny_bf16_vs_oracle_and_tiled_kernel(dev, oracle, shape):
     bc3 = dev.buffer(M * N * 2)
     morok_amd.Program.builtin("gemm_bf16_nt", [M, N, K], dev.device_id).execute([bc3, ba, bb])
     assert np.array_equal(bc3.copyout(np.uint16, (M, N)), got)
-    # through the ABI (one or two rows: the same kernel; more: split-K over the tiled kernels where the shape has tiles)
+    # through the ABI (up to eight rows: the same kernel; more: split-K over the tiled kernels where the shape has tiles)
     ops.gemm_bf16_nt(ba, bb, bc3, M, N, K, dev.device_id)
     abi = bc3.copyout(np.uint16, (M, N))
-    if M <= 2 or N % 8:
+    if M <= 8 or N % 8:
         assert np.array_equal(abi, got)
     else:
         assert np.array_equal(abi, bc2.copyout(np.uint16, (M, N)))     # the bits of the [K, N] form
@@ -125,8 +125,8 @@ def test_skinny_refusals(dev):
 
 
 def test_linear_decode_step_is_one_kernel(T, oracle):
-    """x [1, K] (and a batch of 8) through Tensor.linear with the weight as stored: one product that
-    reads the weight in place, no transposed copy (one row streams it in one pass, eight rows take the
+    """x [1, K] (and batches of 8 and 12) through Tensor.linear with the weight as stored: one product that
+    reads the weight in place, no transposed copy (up to eight rows stream it in one pass, twelve take the
     tiled kernels with the K loop spread over the chip)."""
     from morok_amd import uop
 
@@ -134,10 +134,10 @@ def test_linear_decode_step_is_one_kernel(T, oracle):
     K, N = 2048, 3072
     w = synth.normal_bf16((N, K), 13, 6)
     tw = T.Tensor.from_numpy(w, uop.BF16)
-    for M in (1, 8):
+    for M in (1, 8, 12):
         x = synth.normal_bf16((M, K), 13, 7)
         y = T.Tensor.from_numpy(x, uop.BF16).linear(tw)
         got = y.to_numpy()
-        assert y.kernels() == [f"gemm_bf16_nt_{M}_{N}_{K}" + ("" if M == 1 else "_splitk")]
+        assert y.kernels() == [f"gemm_bf16_nt_{M}_{N}_{K}" + ("" if M <= 8 else "_splitk")]
         ref = oracle.gemm_bf16(x, np.ascontiguousarray(w.T))
         _check(synth.from_bf16(got), synth.from_bf16(ref), K, 2**-7)
