@@ -1347,6 +1347,70 @@ def test_side_output_is_left_alone_when_it_does_not_fit(T):
     assert np.array_equal(h.to_numpy(), x) and np.array_equal(g.to_numpy(), 2 * x)
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_row_kernels_with_side_outputs(T, seed, monkeypatch):
+    """Random elementwise chains with `contiguous()` at random places in front of a row statistic
+    (sum or max over the last axis, consumed by the same rows), on small integers so that every value
+    is exact: the result and every tensor the caller asked to have in memory equal numpy's, whether
+    the row kernel writes them itself or they get kernels of their own, and both ways give the same
+    kernels' worth of values."""
+    rng = np.random.default_rng(4000 + seed)
+    rows, cols = int(rng.choice([128, 256, 300, 512])), int(rng.choice([256, 512, 1024, 2048]))
+    if seed % 4 == 3:
+        rows = cols = 512                                     # square: one operand is read transposed
+    x = rng.integers(-3, 4, size=(rows, cols)).astype(np.float32)
+
+    def build():
+        a, t = x, T.Tensor.from_numpy(x)
+        kept = []
+        r = np.random.default_rng(5000 + seed)
+        for _ in range(int(r.integers(1, 4))):
+            kind = r.choice(["add", "mul", "neg", "contig", "contig"])
+            if kind == "add":
+                a, t = a + 2.0, t.try_add(T.Tensor.const(2.0))
+            elif kind == "mul":
+                a, t = a * 2.0, t.try_mul(T.Tensor.const(2.0))
+            elif kind == "neg":
+                a, t = -a, t.try_mul(T.Tensor.const(-1.0))
+            else:
+                a, t = a.copy(), t.contiguous()
+                kept.append((a, t))
+        a, t = a.copy(), t.contiguous()
+        kept.append((a, t))
+        if r.integers(0, 2):
+            a2, t2 = a * a, t.try_mul(t).contiguous()         # a second tensor of the row's kind, built on the first
+            kept.append((a2, t2))
+        else:
+            a2, t2 = a, t
+        if r.integers(0, 2):
+            stat_a, stat_t = a2.sum(1, keepdims=True), t2.sum(1, keepdim=True)
+        else:
+            stat_a, stat_t = a2.max(1, keepdims=True), t2.max(1, keepdim=True)
+        if rows == cols:
+            ya, yt = a.T + stat_a, t.try_permute([1, 0]).try_add(stat_t)
+        else:
+            ya, yt = a2 - stat_a + a, t2.try_sub(stat_t).try_add(t)
+        return ya, yt, kept
+
+    ya, yt, kept = build()
+    got = yt.to_numpy()
+    names = list(yt.kernels())
+    np.testing.assert_array_equal(got, ya)
+    for a, t in kept:
+        np.testing.assert_array_equal(t.to_numpy(), a)
+    assert names[-1].startswith("rE_"), names
+    monkeypatch.setenv("MOROK_NO_SIDE_OUTPUTS", "1")
+    ya2, yt2, kept2 = build()
+    np.testing.assert_array_equal(yt2.to_numpy(), ya)
+    names2 = list(yt2.kernels())
+    for a, t in kept2:
+        np.testing.assert_array_equal(t.to_numpy(), a)
+    monkeypatch.delenv("MOROK_NO_SIDE_OUTPUTS")
+    assert len(names) <= len(names2)
+    if "_s" in names[-1].split("_g")[-1]:
+        assert len(names) < len(names2)                       # every side output saved a kernel
+
+
 def test_beam_search_over_generated_kernels_keeps_values(T, tmp_path, monkeypatch):
     """Under MOROK_BEAM the choices of generated elementwise and reduce kernels are searched on the
     device (candidates timed on scratch buffers of the real sizes); whatever wins, elementwise
