@@ -39,7 +39,8 @@ MIB = 1 << 20
 PROFILE_OF = {"softmax": "softmax_rows_in_regs_8192x8192_f32.txt", "gemm": "gemm_bf16_tile256_4096cubed.txt",
               "flash": "flash_fwd_d128_causal_8x32x4096x128.txt", "decoder": "decoder_block_4x2048_h4096.txt",
               "generated_tc": "generated_tensor_core_gemm_4096cubed.txt", "matmul_f32": "generated_f32_matmul_1024cubed.txt",
-              "gemm_f16": "gemm_f16_tile256_4096cubed.txt", "flash_options": "flash_fwd_ext_d128_8x32x4096x128.txt"}
+              "gemm_f16": "gemm_f16_tile256_4096cubed.txt", "flash_options": "flash_fwd_ext_d128_8x32x4096x128.txt",
+              "linear_decode": "gemm_nt_skinny_1x12288x4096_x8.txt"}
 
 
 def _profiled_traffic(workload, kernel):
@@ -550,6 +551,54 @@ def bench_group_reduce(m, dev, steps, warmup, cpu):
     return rec
 
 
+def bench_linear_decode(m, dev, steps, warmup, cpu):
+    """One token through eight Linear layers (x [1, 4096] @ W.T, W [12288, 4096] bf16 as `nn::Linear` stores
+    it): the streaming kernel for a handful of rows.  HBM-bound; the eight weights (96 MiB each) are
+    different buffers visited in turn, so no launch finds its weight in the 256 MiB last-level cache.
+    A step is the eight launches; the rate counts every byte a launch has to move."""
+    import numpy as np
+
+    from morok_amd import ops, synth
+
+    layers, M, N, K = 8, 1, 12288, 4096
+    bx = dev.buffer(M * K * 2).ensure_allocated()
+    ops.fill_normal(bx, M * K, seed=7, tensor_id=0, bf16=True)
+    ws, ys = [], []
+    for i in range(layers):
+        w = dev.buffer(N * K * 2).ensure_allocated()
+        ops.fill_normal(w, N * K, seed=7, tensor_id=1 + i, bf16=True)
+        ws.append(w)
+        ys.append(dev.buffer(M * N * 2).ensure_allocated())
+
+    def step():
+        for w, y in zip(ws, ys):
+            ops.gemm_bf16_nt(bx, w, y, M, N, K)
+
+    ms, stats = _launch_stats(m, step, max(1, min(steps, 20)), warmup)
+    algo_bytes = 2 * (N * K + M * K + M * N)  # per launch
+    gbs = layers * algo_bytes / (ms * 1e-3) / 1e9
+    rec = {"metric": "linear decode HBM GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "bf16", **stats,
+           "config": {"workload": "1 token x 8 Linear layers [12288, 4096] bf16, weights stored [out, in], one streaming launch each"},
+           "launches_per_step": layers, "us_per_launch": ms * 1e3 / layers,
+           "roofline": _roofline("linear_decode", "hbm", gbs, HBM_PEAK_GBS, "GB/s", "gemm_nt_skinny<1,2,false>",
+                                 algorithmic_bytes_per_launch=algo_bytes)}
+    if cpu:
+        from tests.oracle_lib import Oracle
+
+        orc = Oracle()
+        x = bx.copyout(np.uint16, (M, K))
+        rows = 2048                                        # a slice of one weight: the oracle's bf16 product, all host threads
+        wt = ws[0].copyout(np.uint16, (N, K))[:rows]
+        b = np.ascontiguousarray(wt.T)
+        sec = _cpu_time(lambda: orc.gemm_bf16(x, b))
+        got = synth.from_bf16(ys[0].copyout(np.uint16, (M, N))[:, :rows])
+        ref = synth.from_bf16(orc.gemm_bf16(x, b))
+        rec["max_rel_err_vs_cpu"] = float(np.abs(got - ref).max() / np.abs(ref).max())
+        rec["cpu_baseline"] = {"value": 2 * (rows * K + K + rows) / sec / 1e9, "unit": "GB/s", "cores": orc.thread_count(M * rows * K, M),
+                               "kind": "port", "sample": f"{rows} of the 12288 weight rows of one layer, f32-accumulate bf16 product, min of 3 after 1 warm-up"}
+    return rec
+
+
 def bench_copy(m, dev, steps, warmup, cpu):
     """Calibration only: 256 MiB streaming copy kernel (known traffic 2 x 256 MiB per launch)."""
     from morok_amd import ops
@@ -569,7 +618,8 @@ def bench_copy(m, dev, steps, warmup, cpu):
 
 WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "decoder": bench_decoder,
              "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling,
-             "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16, "flash_options": bench_flash_options}
+             "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16, "flash_options": bench_flash_options,
+             "linear_decode": bench_linear_decode}
 PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc"]
 
 
