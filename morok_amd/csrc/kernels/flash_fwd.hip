@@ -385,6 +385,9 @@ __device__ __forceinline__ void flash_fwd_body(const __bf16* __restrict__ Q, con
         // K(j+1) and V(j) have landed; every wave is done with K(j) and V(j-1)
         tile_barrier();
         const int g = base + j;
+        // (the copies go out at the highest priority of the iteration: the sooner all four waves have issued theirs,
+        // the longer the tiles have to land; +0.9 % over issuing them at the previous phase's priority)
+        __builtin_amdgcn_s_setprio(2);
         seq_k(g + 2);
         seq_v(g + 1);
         const char* sKn = smem + ((g + 1) & 1) * kTile;
