@@ -942,6 +942,8 @@ SplitPlan plan_split_k(long M, long N, long K, long batch) {
 
 size_t gemm_bf16_workspace_bytes(long M, long N, long K, long batch) {
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
+    long ks = 0, kr = 0;
+    if (gemm_kn_skinny_plan(M, N, K, batch, &ks, &kr)) return (size_t)ks * M * N * sizeof(float);  // a handful of rows: streamed
     const SplitPlan p = plan_split_k(M, N, K, batch);
     return p.splits > 1 ? (size_t)p.splits * batch * M * N * sizeof(float) : 0;
 }
@@ -1121,6 +1123,14 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
         kernel<<<dim3((unsigned)(tm * tn), (unsigned)batch), 256, 0, s>>>(static_cast<const __bf16*>(A), static_cast<const __bf16*>(B),
                                                                           static_cast<__bf16*>(C), (int)M, (int)N, (int)K, (int)tm, (int)tn);
         return (int)hipGetLastError();
+    }
+    // up to eight rows: one streaming pass over the weight into f32 partial sums, then their sum
+    {
+        long ks = 0, kr = 0;
+        if ((variant == 0 || variant == 5) && aligned && gemm_kn_skinny_plan(M, N, K, batch, &ks, &kr) && workspace &&
+            workspace_bytes >= (size_t)ks * M * N * sizeof(float) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+            return launch_gemm_kn_skinny(stream, A, B, C, workspace, M, N, K, ks, kr, f16);
+        }
     }
     // any M; N and K in whole 16-byte chunks
     if (variant != 2 && aligned && offsets_fit && K > 0 && N % 8 == 0 && K % 8 == 0) {

@@ -142,6 +142,136 @@ __global__ __launch_bounds__(256) void gemm_nt_skinny(const unsigned short* __re
     }
 }
 
+
+// C[M, N] = A[M, K] @ B[K, N] for up to eight rows with the weight stored [K, N]: the first of two
+// kernels, which streams the weight once and leaves f32 partial sums (the tiled kernels' split-K
+// reduction adds them up and rounds).  A lane owns eight consecutive columns, a wave 512; the
+// workgroups split K (blockIdx.y: rows_per_group consecutive k-rows each, a multiple of 32) and a
+// workgroup's four waves split its rows into four consecutive runs.  A wave reads 1 KB of one
+// k-row per instruction, eight rows per step; two rows' columns are interleaved into (k, k + 1)
+// pairs (v_perm_b32) and multiplied with the matching pair of A, which is wave-uniform and comes
+// through scalar loads, by the packed dot product.  The waves' sums meet in LDS and the workgroup
+// writes one f32 partial row block W[blockIdx.y][m][its 512 columns].
+template <int kM, bool kF16>
+__global__ __launch_bounds__(256) void gemm_kn_skinny_partial(const unsigned short* __restrict__ A, const unsigned short* __restrict__ B,
+                                                               float* __restrict__ W, int M, int N, int K, int rows_per_group) {
+    __shared__ float red[4][kM][512];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long col0 = (long)blockIdx.x * 512 + lane * 8;
+    const bool active = col0 < N;                              // N is a multiple of 8: a lane's columns are all inside or all outside
+    const long col = active ? col0 : 0;
+    const int k_begin = blockIdx.y * rows_per_group;
+    const int k_end = k_begin + rows_per_group < K ? k_begin + rows_per_group : K;
+    const int per_wave = rows_per_group >> 2;                  // a multiple of 8
+    int k = k_begin + wave * per_wave;
+    int kw_end = k + per_wave;
+    kw_end = kw_end < k_end ? kw_end : k_end;                  // (K is a multiple of 8, so runs end on even rows)
+    const unsigned* a32[kM];                                   // rows of A as (k, k + 1) pairs
+#pragma unroll
+    for (int m = 0; m < kM; m++) a32[m] = reinterpret_cast<const unsigned*>(A + (size_t)(m < M ? m : M - 1) * K);
+    float acc[kM][8];
+#pragma unroll
+    for (int m = 0; m < kM; m++)
+#pragma unroll
+        for (int c = 0; c < 8; c++) acc[m][c] = 0.0f;
+    // two k-rows' eight columns -> eight (k, k + 1) pairs, multiplied with A's pair of every row
+    auto pair_rows = [&](const u32x4& lo, const u32x4& hi, int kk) {
+        unsigned pr[8];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            pr[2 * i] = __builtin_amdgcn_perm(hi[i], lo[i], 0x05040100u);
+            pr[2 * i + 1] = __builtin_amdgcn_perm(hi[i], lo[i], 0x07060302u);
+        }
+#pragma unroll
+        for (int m = 0; m < kM; m++) {
+            const unsigned xp = a32[m][kk >> 1];               // wave-uniform
+#pragma unroll
+            for (int c = 0; c < 8; c++) acc[m][c] = dot2<kF16>(xp, pr[c], acc[m][c]);
+        }
+    };
+    const u32x4* b_col = reinterpret_cast<const u32x4*>(B + col);  // + k * N / 8 per row
+    const size_t row_stride = (size_t)N >> 3;                        // in 16-byte words
+    for (; k + 8 <= kw_end; k += 8) {
+        // the step's four pairs of every row of A in one scalar load each (k is a multiple of 8 here: 16-byte aligned)
+        u32x4 xq[kM];
+#pragma unroll
+        for (int m = 0; m < kM; m++) xq[m] = *reinterpret_cast<const u32x4*>(a32[m] + (k >> 1));
+        u32x4 r[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) r[j] = __builtin_nontemporal_load(b_col + (size_t)(k + j) * row_stride);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            unsigned pr[8];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                pr[2 * i] = __builtin_amdgcn_perm(r[2 * j + 1][i], r[2 * j][i], 0x05040100u);
+                pr[2 * i + 1] = __builtin_amdgcn_perm(r[2 * j + 1][i], r[2 * j][i], 0x07060302u);
+            }
+#pragma unroll
+            for (int m = 0; m < kM; m++)
+#pragma unroll
+                for (int c = 0; c < 8; c++) acc[m][c] = dot2<kF16>(xq[m][j], pr[c], acc[m][c]);
+        }
+    }
+    for (; k + 2 <= kw_end; k += 2) {
+        const u32x4 lo = __builtin_nontemporal_load(b_col + (size_t)k * row_stride);
+        const u32x4 hi = __builtin_nontemporal_load(b_col + (size_t)(k + 1) * row_stride);
+        pair_rows(lo, hi, k);
+    }
+#pragma unroll
+    for (int m = 0; m < kM; m++)
+#pragma unroll
+        for (int c = 0; c < 8; c += 4)
+            *reinterpret_cast<float4*>(&red[wave][m][lane * 8 + c]) = make_float4(acc[m][c], acc[m][c + 1], acc[m][c + 2], acc[m][c + 3]);
+    __syncthreads();
+    // 256 work-items add the four waves' sums: element e = m * 512 + column, two columns apart per step
+    for (int e = threadIdx.x; e < kM * 512; e += 256) {
+        const int m = e >> 9, c = e & 511;
+        const long n = (long)blockIdx.x * 512 + c;
+        if (m < M && n < N) W[((size_t)blockIdx.y * M + m) * N + n] = ((red[0][m][c] + red[1][m][c]) + red[2][m][c]) + red[3][m][c];
+    }
+}
+
+
+// C[i] = round(W[0][i] + W[1][i] + ... + W[splits - 1][i]) for the partial sums above, which come in many
+// more slices than the tiled kernels' split-K leaves (up to 128): a workgroup folds 64 outputs, 32
+// work-items per group of eight outputs each taking every 32nd slice, then one of them adds the 32
+// sums in order.  The order is fixed, so the result does not depend on timing.
+template <bool kF16>
+__global__ __launch_bounds__(256) void gemm_kn_skinny_reduce(const float* __restrict__ W, unsigned short* __restrict__ C, long total, int splits) {
+    __shared__ float4 red[32][8][2];
+    const int eg = threadIdx.x & 7, sl = threadIdx.x >> 3;
+    const long i = ((long)blockIdx.x * 8 + eg) * 8;
+    float4 lo = make_float4(0.f, 0.f, 0.f, 0.f), hi = lo;
+    if (i < total)
+        for (int s = sl; s < splits; s += 32) {
+            const float4* p = reinterpret_cast<const float4*>(W + (size_t)s * total + i);
+            const float4 a = p[0], b = p[1];
+            lo.x += a.x, lo.y += a.y, lo.z += a.z, lo.w += a.w;
+            hi.x += b.x, hi.y += b.y, hi.z += b.z, hi.w += b.w;
+        }
+    red[sl][eg][0] = lo;
+    red[sl][eg][1] = hi;
+    __syncthreads();
+    if (sl == 0 && i < total) {
+        for (int l = 1; l < 32; l++) {
+            const float4 a = red[l][eg][0], b = red[l][eg][1];
+            lo.x += a.x, lo.y += a.y, lo.z += a.z, lo.w += a.w;
+            hi.x += b.x, hi.y += b.y, hi.z += b.z, hi.w += b.w;
+        }
+        const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+        unsigned short o[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            if constexpr (kF16) o[e] = __builtin_bit_cast(unsigned short, (_Float16)v[e]);
+            else o[e] = round_bf16(v[e]);
+        }
+        u32x4 pk = {(unsigned)o[0] | ((unsigned)o[1] << 16), (unsigned)o[2] | ((unsigned)o[3] << 16), (unsigned)o[4] | ((unsigned)o[5] << 16),
+                    (unsigned)o[6] | ((unsigned)o[7] << 16)};
+        *reinterpret_cast<u32x4*>(C + i) = pk;
+    }
+}
+
 }  // namespace mrk::dev
 
 namespace mrk {
@@ -174,6 +304,59 @@ int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, 
     else if (M <= 8) MRK_SKINNY(8, 8);
     else MRK_SKINNY(16, 4);
 #undef MRK_SKINNY
+    return (int)hipGetLastError();
+}
+
+// Plan of the [K, N] form for one or two rows: K split into `splits` groups of `rows_per_group` rows
+// (a multiple of 32), enough of them to fill the chip with workgroups of 512 columns, few enough
+// that the f32 partial sums stay a small part of the weight's bytes (and within 32 MiB).
+bool gemm_kn_skinny_plan(long M, long N, long K, long batch, long* splits, long* rows_per_group) {
+    // One or two rows, up to 24576 columns: measured against split-K over the tiled kernels, 9.3 against 12.5 us at
+    // 1 x 4096 x 4096, 18.8 against 20.1 at N = 12288, 34 against 39 at N = 22016, 18.3 against 21.8 at 4096 x 11008;
+    // with 32000 columns (46.6 against 42.9 us) and with four or eight rows (the partial sums' traffic and the
+    // workgroups' LDS footprint grow with the rows) the tiles win.  The kernel itself takes up to eight rows.
+    if (M < 1 || M > 2 || batch != 1 || N < 8 || N > 24576 || N % 8 || K < 256 || K % 8 || K > 0x7fffffffL) return false;
+    const long col_groups = (N + 511) / 512;
+    long want = (2048 + col_groups - 1) / col_groups;
+    const long by_traffic = K / (16 * M) > 0 ? K / (16 * M) : 1;          // 2 * S * M * N * 4 <= K * N * 2 / 4
+    const long by_bytes = (32L << 20) / (M * N * 4) > 0 ? (32L << 20) / (M * N * 4) : 1;
+    want = want < by_traffic ? want : by_traffic;
+    want = want < by_bytes ? want : by_bytes;
+    want = want < K / 32 ? want : K / 32;
+    if (want < 2) return false;
+    long rows = ((K + want - 1) / want + 31) / 32 * 32;
+    const long s = (K + rows - 1) / rows;
+    if (s < 2 || s > 65535) return false;
+    *splits = s;
+    *rows_per_group = rows;
+    return true;
+}
+
+int launch_gemm_kn_skinny(void* stream, const void* A, const void* B, void* C, void* W, long M, long N, long K, long splits, long rows_per_group,
+                          bool f16) {
+    using namespace mrk::dev;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(C)) % 16)
+        return (int)hipErrorInvalidValue;
+    (void)hipGetLastError();
+    const dim3 grid((unsigned)((N + 511) / 512), (unsigned)splits);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned short* a = static_cast<const unsigned short*>(A);
+    const unsigned short* b = static_cast<const unsigned short*>(B);
+    float* w = static_cast<float*>(W);
+#define MRK_KN(KM)                                                                                                  \
+    do {                                                                                                            \
+        if (f16) gemm_kn_skinny_partial<KM, true><<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)rows_per_group);  \
+        else gemm_kn_skinny_partial<KM, false><<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)rows_per_group);     \
+    } while (0)
+    if (M == 1) MRK_KN(1);
+    else if (M == 2) MRK_KN(2);
+    else if (M <= 4) MRK_KN(4);
+    else MRK_KN(8);
+#undef MRK_KN
+    const long total = M * N;  // (a multiple of 8)
+    const unsigned blocks = (unsigned)((total + 63) / 64);
+    if (f16) gemm_kn_skinny_reduce<true><<<blocks, 256, 0, s>>>(w, static_cast<unsigned short*>(C), total, (int)splits);
+    else gemm_kn_skinny_reduce<false><<<blocks, 256, 0, s>>>(w, static_cast<unsigned short*>(C), total, (int)splits);
     return (int)hipGetLastError();
 }
 

@@ -34,6 +34,13 @@ bool gemm_bf16_nt_supported(long M, long N, long K, long batch);
 // differs from the tiled kernels', so results agree with them to rounding, not bit for bit.
 bool gemm_nt_skinny_supported(long M, long N, long K, long batch);
 int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16);
+// The [K, N] form for one or two rows (N <= 24576 and K multiples of 8, K >= 256, one product): the weight is
+// streamed once into `splits` f32 partial results W[splits][M][N], which a second kernel adds up in a
+// fixed order and rounds into C; gemm_kn_skinny_plan chooses the split and tells whether the shape is
+// taken this way.  gemm_bf16_workspace_bytes reports splits * M * N * 4 for such shapes.
+bool gemm_kn_skinny_plan(long M, long N, long K, long batch, long* splits, long* rows_per_group);
+int launch_gemm_kn_skinny(void* stream, const void* A, const void* B, void* C, void* W, long M, long N, long K, long splits, long rows_per_group,
+                          bool f16);
 // c = bf16(float(bf16(a b)) + float(r)) with r of c's shape, added in the product kernel's epilogue
 // (same bits as the product followed by an elementwise add).  Supported for the shapes the tiled
 // kernels take without split-K; gemm_bf16_residual_supported tells.

@@ -22,6 +22,11 @@ int launch_gemm_nt_skinny(void* stream, const void*, const void*, void*, long, l
     mrk_shim_note_launch(stream, f16 ? "gemm_f16_nt" : "gemm_bf16_nt");
     return 0;
 }
+bool gemm_kn_skinny_plan(long, long, long, long, long*, long*) { return false; }
+int launch_gemm_kn_skinny(void* stream, const void*, const void*, void*, void*, long, long, long, long, long, bool) {
+    mrk_shim_note_launch(stream, "gemm_bf16");
+    return 0;
+}
 int gemm_bf16_static_workspace_init(int) { return 0; }
 size_t gemm_bf16_static_workspace_capacity() { return size_t(32) << 20; }
 int launch_gemm_bf16_static_ws(void* stream, int, const void*, const void*, void*, long, long, long) {

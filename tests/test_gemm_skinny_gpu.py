@@ -141,3 +141,86 @@ def test_linear_decode_step_is_one_kernel(T, oracle):
         assert y.kernels() == [f"gemm_bf16_nt_{M}_{N}_{K}" + ("" if M <= 8 else "_splitk")]
         ref = oracle.gemm_bf16(x, np.ascontiguousarray(w.T))
         _check(synth.from_bf16(got), synth.from_bf16(ref), K, 2**-7)
+
+
+# ---------------------------------------------------------------- the same rows against a weight stored [K, N]
+KN_SHAPES = [(1, 4096, 4096), (2, 520, 1024), (1, 264, 4104), (2, 12288, 4096), (1, 1024, 256), (2, 256, 11008), (1, 4104, 520),
+             (2, 8, 4096), (1, 2048, 2048), (2, 24576, 512)]
+
+
+@pytest.mark.parametrize("shape", KN_SHAPES)
+def test_skinny_kn_form_vs_oracle_and_tiled_kernel(dev, oracle, shape):
+    """One or two rows through mrk_hip_gemm_bf16 ([K, N] weight): one streaming pass into f32 partial sums
+    plus their sum.  Against the oracle, against the tiled kernel (another summation order), the
+    same bits on every run, through the ABI (allocator scratch) and as a plan item with a scratch buffer;
+    NaNs right behind the operands and the result show that nothing reads or writes past them."""
+    from morok_amd._ffi import lib
+
+    M, N, K = shape
+    ws = lib.mrk_hip_gemm_bf16_workspace_bytes(M, N, K, 1)
+    assert ws > 0 and ws % (M * N * 4) == 0
+    a = synth.normal_bf16((M, K), 13, 8)
+    b = synth.normal_bf16((K, N), 13, 9)
+    pad = np.full(4096, 0x7FC0, np.uint16)
+    ba = morok_amd.Buffer.from_numpy(np.concatenate([a.reshape(-1), pad]), dev.device_id)
+    bb = morok_amd.Buffer.from_numpy(np.concatenate([b.reshape(-1), pad]), dev.device_id)
+    bc = dev.buffer((M * N + 2048) * 2)
+    bc.copyin(np.full(M * N + 2048, 0x7FC0, np.uint16))
+    ops.gemm_bf16(ba, bb, bc, M, N, K, dev.device_id)
+    out = bc.copyout(np.uint16)
+    assert np.all(out[M * N:] == 0x7FC0)
+    got = out[: M * N].reshape(M, N)
+    ref = oracle.gemm_bf16(a, b)
+    _check(synth.from_bf16(got), synth.from_bf16(ref), K, 2**-7)
+    bc2 = dev.buffer(M * N * 2)
+    ops.gemm_bf16(ba, bb, bc2, M, N, K, dev.device_id, 4)          # the tiled kernel, unsplit
+    tiled = synth.from_bf16(bc2.copyout(np.uint16, (M, N)))
+    g = synth.from_bf16(got)
+    assert np.all(np.abs(g - tiled) <= np.abs(tiled) * 2**-7 + 2e-5 * np.sqrt(K) * max(np.abs(tiled).max() / np.sqrt(K), 1.0))
+    ops.gemm_bf16(ba, bb, bc2, M, N, K, dev.device_id)
+    assert np.array_equal(bc2.copyout(np.uint16, (M, N)), got)
+    bw = dev.buffer(ws + 4096)
+    bw.copyin(np.full((ws + 4096) // 4, np.nan, np.float32))
+    prog = morok_amd.Program.builtin("gemm_bf16", [M, N, K, 1, ws], dev.device_id)
+    prog.execute([bc2, ba, bb, bw])
+    assert np.array_equal(bc2.copyout(np.uint16, (M, N)), got)
+    assert np.all(np.isnan(bw.copyout(np.float32)[ws // 4:]))     # the partial sums stay inside the scratch asked for
+
+
+def test_skinny_kn_form_f16_and_exact(dev, oracle):
+    M, N, K = 4, 1032, 2048
+    a = synth.normal((M, K), 13, 10).astype(np.float16)
+    b = synth.normal((K, N), 13, 11).astype(np.float16)
+    ba, bb = morok_amd.Buffer.from_numpy(a.view(np.uint16), dev.device_id), morok_amd.Buffer.from_numpy(b.view(np.uint16), dev.device_id)
+    bc = dev.buffer(M * N * 2)
+    ops.gemm_f16(ba, bb, bc, M, N, K, dev.device_id)
+    got = bc.copyout(np.uint16, (M, N)).view(np.float16).astype(np.float32)
+    _check(got, oracle.gemm_f16(a, b).astype(np.float32), K, 2**-10)
+    # small integers: every sum is exact in f32 whatever the order (one or two rows stream, more take the tiles)
+    rng = np.random.default_rng(6)
+    for M in range(1, 9):
+        N, K = 520 + 8 * M, 1288
+        ai = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+        bi = rng.integers(-4, 5, size=(K, N)).astype(np.float32)
+        ba, bb = morok_amd.Buffer.from_numpy(synth.to_bf16(ai), dev.device_id), morok_amd.Buffer.from_numpy(synth.to_bf16(bi), dev.device_id)
+        bc = dev.buffer(M * N * 2)
+        ops.gemm_bf16(ba, bb, bc, M, N, K, dev.device_id)
+        want = ai.astype(np.int64) @ bi.astype(np.int64)
+        assert np.array_equal(bc.copyout(np.uint16, (M, N)), synth.to_bf16(want.astype(np.float32)))
+
+
+def test_matmul_decode_step_kn_weight(T, oracle):
+    """x [M, K] @ w [K, N] through Tensor.matmul for a handful of rows: one plan item with scratch placed by
+    the plan (one row: the streaming pair of kernels; eight: split-K over the tiles)."""
+    from morok_amd import uop
+
+    T.set_fusion(True)
+    K, N = 2048, 3072
+    w = synth.normal_bf16((K, N), 13, 12)
+    tw = T.Tensor.from_numpy(w, uop.BF16)
+    for M in (1, 8):
+        x = synth.normal_bf16((M, K), 13, 13)
+        y = T.Tensor.from_numpy(x, uop.BF16).matmul(tw)
+        got = y.to_numpy()
+        assert y.kernels() == [f"gemm_bf16_{M}_{N}_{K}_splitk"]
+        _check(synth.from_bf16(got), synth.from_bf16(oracle.gemm_bf16(x, w)), K, 2**-7)
