@@ -1042,12 +1042,30 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             // copies of tile r + 2 behind the second half's.  The last two steps copy the last
             // tile again, into stages nobody reads any more, so that the loop has no branch.
             std::vector<std::function<void()>> reads1, reads0;
+            // The reads of a group go out in two bursts, behind the first instructions of each half of the group
+            // (rows 0 .. um/2-1 and columns 0 .. un/2-1 first, the rest half a group later, still ahead of their
+            // first use): the four waves run in step behind a barrier, and one burst of all of a half step's
+            // reads queues longer on the LDS than two of half the size (+1 % at 4096^3).
+            const bool split_reads = BST == 2 && um % 2 == 0 && un % 2 == 0;
             for (int h = 0; h < HS; h++) {
+                if (split_reads) {
+                    for (int part = 0; part < 2; part++) {
+                        for (int i = part * um / 2; i < (part + 1) * um / 2; i++) reads1.push_back([&, h, i] { f1a[h * um + i] = read_a(HS + h, i, oa); });
+                        for (int j = part * un / 2; j < (part + 1) * un / 2; j++) reads1.push_back([&, h, j] { f1b[h * un + j] = read_b(HS + h, j, ob); });
+                    }
+                    for (int part = 0; part < 2; part++) {
+                        for (int i = part * um / 2; i < (part + 1) * um / 2; i++) reads0.push_back([&, h, i] { b.store(fa0[h * um + i], read_a(h, i, na)); });
+                        for (int j = part * un / 2; j < (part + 1) * un / 2; j++) reads0.push_back([&, h, j] { b.store(fb0[h * un + j], read_b(h, j, nb)); });
+                    }
+                    continue;
+                }
                 for (int i = 0; i < um; i++) reads1.push_back([&, h, i] { f1a[h * um + i] = read_a(HS + h, i, oa); });
                 for (int j = 0; j < un; j++) reads1.push_back([&, h, j] { f1b[h * un + j] = read_b(HS + h, j, ob); });
                 for (int i = 0; i < um; i++) reads0.push_back([&, h, i] { b.store(fa0[h * um + i], read_a(h, i, na)); });
                 for (int j = 0; j < un; j++) reads0.push_back([&, h, j] { b.store(fb0[h * un + j], read_b(h, j, nb)); });
             }
+            // slot of read closure c when the reads are split over the two halves of the group
+            auto slot_of = [&](int c, int nreads) { return c < nreads / 2 ? c : total / 2 + (c - nreads / 2); };
             for (size_t i = 0; i < fa0.size(); i++) f0a[i] = b.load(fa0[i]);
             for (size_t j = 0; j < fb0.size(); j++) f0b[j] = b.load(fb0[j]);
             uint32_t kt2 = bin(BinaryOp::Sub, b.ci(KT - 1), bin(BinaryOp::Max, bin(BinaryOp::Sub, b.ci(KT - 3), r), b.ci(0)));
@@ -1056,6 +1074,11 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             const int left1 = std::max(1, total - (int)reads1.size());
             const int every1 = std::max(1, left1 / std::max(1, CB));
             mfmas(f0a, f0b, [&](int n) {
+                if (split_reads) {
+                    if (done1 < reads1.size() && n == slot_of((int)done1, (int)reads1.size())) reads1[done1++]();
+                    if (n == total - 1) while (done1 < reads1.size()) reads1[done1++]();
+                    return;
+                }
                 if (done1 < reads1.size()) reads1[done1++]();
                 else if (BST == 3 && (n - (int)reads1.size()) % every1 == 0 && issued_b < CB) copy_one(CA + issued_b++, kt2, st, sb2);
                 if (n == total - 1) {
@@ -1074,6 +1097,21 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             const int left = std::max(1, total - (int)reads0.size());
             const int every = std::max(1, left / second);
             mfmas(f1a, f1b, [&](int n) {
+                if (split_reads) {
+                    const int nr = (int)reads0.size();
+                    if (done0 < reads0.size() && n == slot_of((int)done0, nr)) reads0[done0++]();
+                    else {
+                        // copies in the slots without a read: every third of them
+                        const bool read_slot = n < nr / 2 || (n >= total / 2 && n < total / 2 + nr / 2);
+                        const int free_index = n < total / 2 ? n - nr / 2 : n - nr;
+                        if (!read_slot && free_index % 3 == 0 && issued < second) copy_one(issued++, kt2, st);
+                    }
+                    if (n == total - 1) {
+                        while (done0 < reads0.size()) reads0[done0++]();
+                        while (issued < second) copy_one(issued++, kt2, st);
+                    }
+                    return;
+                }
                 if (done0 < reads0.size()) reads0[done0++]();
                 else if ((n - (int)reads0.size()) % every == 0 && issued < second) copy_one(issued++, kt2, st);
                 if (n == total - 1) {
