@@ -1022,7 +1022,7 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
     // One wave per SIMD and an even number of steps: the loop runs two steps per trip, so that the
     // stage of a step is a constant and the fragment reads address it through their immediate
     // offsets instead of one vector addition each.
-    const bool two_per_trip = W <= 4 && KT > 2 && KT % 2 == 0 && BST == 2;
+    const bool two_per_trip = W <= 4 && KT > 2 && KT % 2 == 0;
     uint32_t r_outer = b.range(two_per_trip ? KT / 2 : KT, 0, AxisType::Reduce);
     for (int trip_step = 0; trip_step < (two_per_trip ? 2 : 1); trip_step++) {
         uint32_t r = two_per_trip ? b.iadd(b.imul(r_outer, 2), b.ci(trip_step)) : r_outer;
@@ -1101,10 +1101,11 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
                     const int nr = (int)reads0.size();
                     if (done0 < reads0.size() && n == slot_of((int)done0, nr)) reads0[done0++]();
                     else {
-                        // copies in the slots without a read: every third of them
+                        // copies in the slots without a read, spread evenly over them
                         const bool read_slot = n < nr / 2 || (n >= total / 2 && n < total / 2 + nr / 2);
                         const int free_index = n < total / 2 ? n - nr / 2 : n - nr;
-                        if (!read_slot && free_index % 3 == 0 && issued < second) copy_one(issued++, kt2, st);
+                        const int spacing = std::max(1, (total - nr) / std::max(1, second));
+                        if (!read_slot && free_index % spacing == 0 && issued < second) copy_one(issued++, kt2, st);
                     }
                     if (n == total - 1) {
                         while (done0 < reads0.size()) reads0[done0++]();
