@@ -224,3 +224,32 @@ def test_matmul_decode_step_kn_weight(T, oracle):
         got = y.to_numpy()
         assert y.kernels() == [f"gemm_bf16_{M}_{N}_{K}_splitk"]
         _check(synth.from_bf16(got), synth.from_bf16(oracle.gemm_bf16(x, w)), K, 2**-7)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_skinny_random_shapes_exact(dev, seed):
+    """Random small shapes on small-integer data, where every sum is exact in f32 whatever its order: the
+    [N, K] form for 1-16 rows (any N, K a multiple of 8) and the [K, N] form for 1-8 rows (N, K multiples of 8)
+    must give the integer products exactly, whichever kernel the shape selects."""
+    rng = np.random.default_rng(7000 + seed)
+    for _ in range(12):
+        M = int(rng.integers(1, 17))
+        N = int(rng.integers(1, 700))
+        K = 8 * int(rng.integers(1, 300))
+        a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+        bt = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+        want = synth.to_bf16((a.astype(np.int64) @ bt.astype(np.int64).T).astype(np.float32))
+        ba, bb = morok_amd.Buffer.from_numpy(synth.to_bf16(a), dev.device_id), morok_amd.Buffer.from_numpy(synth.to_bf16(bt), dev.device_id)
+        bc = dev.buffer(M * N * 2)
+        morok_amd.Program.builtin("gemm_bf16_nt", [M, N, K], dev.device_id).execute([bc, ba, bb])
+        assert np.array_equal(bc.copyout(np.uint16, (M, N)), want), (M, N, K)
+        if M <= 8:
+            N8 = 8 * int(rng.integers(1, 200))
+            K2 = 8 * int(rng.integers(32, 400))
+            a2 = rng.integers(-3, 4, size=(M, K2)).astype(np.float32)
+            b2 = rng.integers(-3, 4, size=(K2, N8)).astype(np.float32)
+            want2 = synth.to_bf16((a2.astype(np.int64) @ b2.astype(np.int64)).astype(np.float32))
+            ba2, bb2 = morok_amd.Buffer.from_numpy(synth.to_bf16(a2), dev.device_id), morok_amd.Buffer.from_numpy(synth.to_bf16(b2), dev.device_id)
+            bc2 = dev.buffer(M * N8 * 2)
+            ops.gemm_bf16(ba2, bb2, bc2, M, N8, K2, dev.device_id)
+            assert np.array_equal(bc2.copyout(np.uint16, (M, N8)), want2), (M, N8, K2)
