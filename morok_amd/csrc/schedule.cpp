@@ -1046,7 +1046,7 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             // (rows 0 .. um/2-1 and columns 0 .. un/2-1 first, the rest half a group later, still ahead of their
             // first use): the four waves run in step behind a barrier, and one burst of all of a half step's
             // reads queues longer on the LDS than two of half the size (+1 % at 4096^3).
-            const bool split_reads = BST == 2 && um % 2 == 0 && un % 2 == 0;
+            const bool split_reads = um % 2 == 0 && un % 2 == 0;
             for (int h = 0; h < HS; h++) {
                 if (split_reads) {
                     for (int part = 0; part < 2; part++) {
@@ -1075,8 +1075,19 @@ static int build_wmma_matmul_async_kernel(const TensorCore& tc, int64_t M, int64
             const int every1 = std::max(1, left1 / std::max(1, CB));
             mfmas(f0a, f0b, [&](int n) {
                 if (split_reads) {
-                    if (done1 < reads1.size() && n == slot_of((int)done1, (int)reads1.size())) reads1[done1++]();
-                    if (n == total - 1) while (done1 < reads1.size()) reads1[done1++]();
+                    const int nr = (int)reads1.size();
+                    if (done1 < reads1.size() && n == slot_of((int)done1, nr)) reads1[done1++]();
+                    else if (BST == 3) {
+                        // three stages: the B chunks of tile r + 2 in the slots without a read, spread evenly
+                        const bool read_slot = n < nr / 2 || (n >= total / 2 && n < total / 2 + nr / 2);
+                        const int free_index = n < total / 2 ? n - nr / 2 : n - nr;
+                        const int spacing = std::max(1, (total - nr) / std::max(1, CB));
+                        if (!read_slot && free_index % spacing == 0 && issued_b < CB) copy_one(CA + issued_b++, kt2, st, sb2);
+                    }
+                    if (n == total - 1) {
+                        while (done1 < reads1.size()) reads1[done1++]();
+                        while (BST == 3 && issued_b < CB) copy_one(CA + issued_b++, kt2, st, sb2);
+                    }
                     return;
                 }
                 if (done1 < reads1.size()) reads1[done1++]();
