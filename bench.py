@@ -40,7 +40,7 @@ PROFILE_OF = {"softmax": "softmax_rows_in_regs_8192x8192_f32.txt", "gemm": "gemm
               "flash": "flash_fwd_d128_causal_8x32x4096x128.txt", "decoder": "decoder_block_4x2048_h4096.txt",
               "generated_tc": "generated_tensor_core_gemm_4096cubed.txt", "matmul_f32": "generated_f32_matmul_1024cubed.txt",
               "gemm_f16": "gemm_f16_tile256_4096cubed.txt", "flash_options": "flash_fwd_ext_d128_8x32x4096x128.txt",
-              "linear_decode": "gemm_nt_skinny_1x12288x4096_x8.txt"}
+              "linear_decode": "gemm_nt_skinny_1x12288x4096_x8.txt", "linear_decode_16": "gemm_nt_rows_16x12288x4096_x8.txt"}
 
 
 def _profiled_traffic(workload, kernel):
@@ -553,14 +553,24 @@ def bench_group_reduce(m, dev, steps, warmup, cpu):
 
 def bench_linear_decode(m, dev, steps, warmup, cpu):
     """One token through eight Linear layers (x [1, 4096] @ W.T, W [12288, 4096] bf16 as `nn::Linear` stores
-    it): the streaming kernel for a handful of rows.  HBM-bound; the eight weights (96 MiB each) are
+    it): the streaming kernel for one and two rows.  HBM-bound; the eight weights (96 MiB each) are
     different buffers visited in turn, so no launch finds its weight in the 256 MiB last-level cache.
     A step is the eight launches; the rate counts every byte a launch has to move."""
+    return _linear_decode(m, dev, steps, warmup, cpu, 1, "linear_decode", "gemm_nt_skinny<1,2,false>")
+
+
+def bench_linear_decode_16(m, dev, steps, warmup, cpu):
+    """The same with 16 tokens in flight (x [16, 4096]): the streaming kernel for 3 to 64 rows, which feeds the
+    matrix pipes from 16-row blocks staged through LDS."""
+    return _linear_decode(m, dev, steps, warmup, cpu, 16, "linear_decode_16", "gemm_nt_rows<1,3,8,false>")
+
+
+def _linear_decode(m, dev, steps, warmup, cpu, M, workload, kernel):
     import numpy as np
 
     from morok_amd import ops, synth
 
-    layers, M, N, K = 8, 1, 12288, 4096
+    layers, N, K = 8, 12288, 4096
     bx = dev.buffer(M * K * 2).ensure_allocated()
     ops.fill_normal(bx, M * K, seed=7, tensor_id=0, bf16=True)
     ws, ys = [], []
@@ -578,10 +588,9 @@ def bench_linear_decode(m, dev, steps, warmup, cpu):
     algo_bytes = 2 * (N * K + M * K + M * N)  # per launch
     gbs = layers * algo_bytes / (ms * 1e-3) / 1e9
     rec = {"metric": "linear decode HBM GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "bf16", **stats,
-           "config": {"workload": "1 token x 8 Linear layers [12288, 4096] bf16, weights stored [out, in], one streaming launch each"},
+           "config": {"workload": "%d token%s x 8 Linear layers [12288, 4096] bf16, weights stored [out, in], one streaming launch each" % (M, "" if M == 1 else "s")},
            "launches_per_step": layers, "us_per_launch": ms * 1e3 / layers,
-           "roofline": _roofline("linear_decode", "hbm", gbs, HBM_PEAK_GBS, "GB/s", "gemm_nt_skinny<1,2,false>",
-                                 algorithmic_bytes_per_launch=algo_bytes)}
+           "roofline": _roofline(workload, "hbm", gbs, HBM_PEAK_GBS, "GB/s", kernel, algorithmic_bytes_per_launch=algo_bytes)}
     if cpu:
         from tests.oracle_lib import Oracle
 
@@ -619,7 +628,7 @@ def bench_copy(m, dev, steps, warmup, cpu):
 WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "decoder": bench_decoder,
              "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling,
              "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16, "flash_options": bench_flash_options,
-             "linear_decode": bench_linear_decode}
+             "linear_decode": bench_linear_decode, "linear_decode_16": bench_linear_decode_16}
 PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc"]
 
 

@@ -142,7 +142,7 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
         if (p.size() < 5) p.push_back(0);
         if (p[4] < 0) return fail(kInvalidArgument, k + ": negative workspace size");
         if (!gemm_bf16_nt_supported(p[0], p[1], p[2], p[3]))
-            return fail(kInvalidArgument, k + ": shape not covered (K a multiple of 8; at most 16 rows, or N a multiple of 8)");
+            return fail(kInvalidArgument, k + ": shape not covered (K a multiple of 8; at most 64 rows, or N a multiple of 8)");
         std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
         if (p[3] > 1) name += "_x" + std::to_string(p[3]);
         if (p[4] > 0) {  // a fourth buffer of p[4] bytes: scratch for the split-K partial results

@@ -897,12 +897,12 @@ static int gemm_16bit_nt(int device_id, const void* a, const void* bt, void* c, 
     MRK_NONNULL(c);
     if (!gemm_bf16_nt_supported(m, n, k, 1))
         return fail(kInvalidArgument, "gemm_bf16_nt: shape not covered for a second operand stored [N, K] (K a multiple of 8, K > 0; "
-                                      "at most 16 rows, or N a multiple of 8); transpose it and run mrk_hip_gemm_bf16");
+                                      "at most 64 rows, or N a multiple of 8); transpose it and run mrk_hip_gemm_bf16");
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    // few output tiles against a long K, more than eight rows: scratch for split-K partials, as for the [K, N] form
-    const size_t ws = m > 8 ? gemm_bf16_workspace_bytes(m, n, k, 1) : 0;
+    // few output tiles against a long K, more than 64 rows: scratch for split-K partials, as for the [K, N] form
+    const size_t ws = gemm_bf16_nt_workspace_bytes(m, n, k, 1);
     RawBuffer scratch;
     BufferOptions so;
     if (ws) MRK_TRY(dv->allocator->alloc(ws, so, &scratch));

@@ -991,9 +991,16 @@ bool tiled_shape(long M, long N, long K, long batch) {
 }  // namespace
 
 bool gemm_bf16_nt_supported(long M, long N, long K, long batch) {
-    // the tiled kernels (no any-shape kernel for this operand layout), or the streaming kernel for a
+    // the tiled kernels (no any-shape kernel for this operand layout), or the streaming kernels for a
     // handful of rows
-    return tiled_shape(M, N, K, batch) || gemm_nt_skinny_supported(M, N, K, batch);
+    return tiled_shape(M, N, K, batch) || gemm_nt_skinny_supported(M, N, K, batch) || gemm_nt_rows_supported(M, N, K, batch);
+}
+
+size_t gemm_bf16_nt_workspace_bytes(long M, long N, long K, long batch) {
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
+    if (gemm_nt_skinny_supported(M, N, K, batch) || gemm_nt_rows_supported(M, N, K, batch)) return 0;  // streamed in one launch
+    const SplitPlan p = plan_split_k(M, N, K, batch);
+    return p.splits > 1 ? (size_t)p.splits * batch * M * N * sizeof(float) : 0;
 }
 
 int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch,
@@ -1089,15 +1096,18 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
         if (!aligned || !gemm_bf16_nt_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
         const bool choose = variant == 0 || variant == 5;  // 3 / 4 force a tile where the shape has one
         const bool tiled = tiled_shape(M, N, K, batch);
-        // up to eight rows: one pass over the weight on the vector ALUs streams it faster than any tile
-        if (gemm_nt_skinny_supported(M, N, K, batch) && (!tiled || (choose && M <= 8)))
-            return launch_gemm_nt_skinny(stream, A, B, C, M, N, K, batch, f16);
+        // up to 64 rows: one pass over the weight streams it faster than any tile (one or two rows on the
+        // vector ALUs, more on the matrix pipes with 16-row blocks staged through LDS)
+        if (choose || !tiled) {
+            if (gemm_nt_skinny_supported(M, N, K, batch)) return launch_gemm_nt_skinny(stream, A, B, C, M, N, K, batch, f16);
+            if (gemm_nt_rows_supported(M, N, K, batch)) return launch_gemm_nt_rows(stream, A, B, C, M, N, K, batch, f16);
+        }
         const long tn = (N + kBN - 1) / kBN, tm128 = (M + 127) / 128;
         const SplitPlan sp = choose ? plan_split_k(M, N, K, batch) : SplitPlan();
         if (sp.splits > 1) {
             // few output tiles against a long K: the K loop spread over the chip when the caller
-            // brought the workspace for the partial results; without one, up to 16 rows stream
-            // (anything else runs the plain tiled kernel on the few workgroups it has)
+            // brought the workspace for the partial results
+            // (without one the plain tiled kernel runs on the few workgroups it has)
             if (workspace && workspace_bytes >= (size_t)sp.splits * batch * M * N * sizeof(float) &&
                 reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && batch * sp.splits <= 65535) {
                 const dim3 grid((unsigned)(tm128 * tn), (unsigned)batch, (unsigned)sp.splits);
@@ -1111,7 +1121,6 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
                 reduce_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>(w, static_cast<__bf16*>(C), total, (int)sp.splits);
                 return (int)hipGetLastError();
             }
-            if (gemm_nt_skinny_supported(M, N, K, batch)) return launch_gemm_nt_skinny(stream, A, B, C, M, N, K, batch, f16);
         }
         const bool small = variant == 4 || (variant != 3 && tm128 * tn * batch <= 256);
         const long tm = small ? tm128 : (M + kBM - 1) / kBM;

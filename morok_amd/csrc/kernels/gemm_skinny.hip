@@ -1,8 +1,10 @@
-// C[M, N] = A[M, K] @ Bt[N, K]^T for a handful of rows (M <= 16) against a weight stored as a Linear
+// C[M, N] = A[M, K] @ Bt[N, K]^T for a handful of rows (M <= 64) against a weight stored as a Linear
 // layer keeps it ([out_features, in_features], tensor/src/nn/linear.rs:9-14,39-41): the decode step
 // of a language model.  The product is a stream over the weight: 2 * N * K bytes against 2 * M * N * K
-// flops, HBM-bound for these M, so nothing is tiled for the matrix pipes.  A workgroup of four waves
-// owns two to eight weight rows; the waves take the 512-element chunks of K in turn, a lane loads
+// flops, HBM-bound for these M.  Two kernels: gemm_nt_skinny for one and two rows on the vector ALUs,
+// gemm_nt_rows for 3 to 64 rows on the matrix pipes (further down, with the [K, N] form for one and two rows).
+// gemm_nt_skinny: a workgroup of four waves
+// owns two or four weight rows; the waves take the 512-element chunks of K in turn, a lane loads
 // 16 bytes of each of the rows (a wave reads 1 KB of one row per instruction) and of each row of A
 // (cache hits: every workgroup reads the same few KB, each starting at another chunk so that they
 // do not all queue on the same L2 channel), and multiplies with packed two-element dot products
@@ -10,7 +12,9 @@
 // with a transposing butterfly (after step s a lane keeps half of the values it held, summed with
 // its partner's: V values take V - 1 exchanges in all, not 6 each), the four waves' results meet in
 // LDS, wave 0 adds them in a fixed order and writes the outputs.  One launch, no scratch memory, no
-// atomics: results do not depend on scheduling.
+// atomics: results do not depend on scheduling.  (A lane needs its own 16 bytes of every row of A per
+// 16 bytes of a weight row, so the cache traffic grows with M: 6.2 TB/s of weight for one row, 5.9 for
+// two, 4.5 for eight, which is where the matrix-pipe kernel takes over.)
 #include <hip/hip_runtime.h>
 
 #include "kernels.h"
@@ -138,6 +142,168 @@ __global__ __launch_bounds__(256) void gemm_nt_skinny(const unsigned short* __re
             if constexpr (kF16) out = __builtin_bit_cast(unsigned short, (_Float16)s);
             else out = round_bf16(s);
             C[(size_t)m * N + n0 + r] = out;
+        }
+    }
+}
+
+
+// The same product for 3 to 64 rows of A, on the matrix pipes.  v_mfma_f32_16x16x32 takes, per lane, eight
+// consecutive k of one row of each operand (lane l: row l % 16, k 8 * (l / 16) ...), i.e. 16 rows with 64 bytes
+// each per instruction if it were loaded straight from memory; the vector-memory path serves such row gathers at
+// a fraction of its rate for consecutive bytes.  So both operands go through LDS: a wave copies its chunk (64
+// elements of K) of 16-row blocks with direct global -> LDS loads, 1 KB per instruction = eight rows of 128
+// bytes, the weight's with the non-temporal hint (it is read once; A stays in L2), and reads the fragments back
+// with ds_read_b128.  The 16-byte pieces of a row are stored swizzled by the row (piece p of row r at position
+// p ^ ((r >> 1) & 7): the 16 rows a fragment read touches then fall into 16 different bank groups).  The region
+// is private to the wave, so the loop has no barrier; the waves of a workgroup take the chunks of K in turn
+// (every workgroup starting at another one, as above), each holds kRT x kMT accumulator blocks for the
+// workgroup's 16 * kRT weight rows, and their sums meet in LDS at the end and are added in a fixed order.
+// What bounds the rate is the number of weight bytes in flight per CU, which is what the LDS holds: with one
+// chunk per wave in flight, 8 or 16 waves per workgroup and enough workgroups resident the weight streams at
+// 5.6-6.5 TB/s for up to 32 rows of A.  kMT: 16-row blocks of A (M <= 16 * kMT; rows beyond M repeat row M - 1
+// and are not written); kRT: 16-row blocks of the weight per workgroup.  grid = (ceil(N / (16 kRT)), batch).
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+#define MRK_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+template <int kMT, int kRT, int kWaves, bool kF16>
+__global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short* __restrict__ A, const unsigned short* __restrict__ Bt,
+                                                             unsigned short* __restrict__ C, int M, int N, int K) {
+    constexpr int kSteps = 2;                      // 32-deep matrix steps per chunk
+    constexpr int kPieces = 4 * kSteps;            // 16-byte pieces of a row per chunk
+    constexpr int kRowsPerCopy = 64 / kPieces;     // rows one copy instruction covers
+    constexpr int kCopies = 16 / kRowsPerCopy;     // copy instructions per 16-row block
+    constexpr int kBlockBytes = 16 * kPieces * 16; // one block's chunk in LDS
+    constexpr int kWaveBytes = (kRT + kMT) * kBlockBytes;
+    constexpr int kTiles = kRT * kMT;
+    constexpr int kSumBytes = kWaves * kTiles * 1024;
+    constexpr int kLds = kWaves * kWaveBytes > kSumBytes ? kWaves * kWaveBytes : kSumBytes;
+    static_assert(kLds <= 160 * 1024, "LDS");
+    __shared__ __attribute__((aligned(1024))) char smem[kLds];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int li = lane & 15, g = lane >> 4;
+    const long n0 = (long)blockIdx.x * (16 * kRT);
+    A += (size_t)blockIdx.y * M * K;
+    Bt += (size_t)blockIdx.y * N * K;
+    C += (size_t)blockIdx.y * M * N;
+    const char* w_base = reinterpret_cast<const char*>(Bt + (size_t)n0 * K);
+    const char* a_base = reinterpret_cast<const char*>(A);
+    const unsigned lds_wave = (unsigned)(uintptr_t)MRK_LDS_PTR(char, smem) + wave * kWaveBytes;
+    // copy side: lane -> (row of the copy, position in the row); byte offsets of its rows from the bases
+    const int pos = lane % kPieces, rsub = lane / kPieces;
+    unsigned w_off[kRT][kCopies], a_off[kMT][kCopies], piece_of[kCopies];
+#pragma unroll
+    for (int i = 0; i < kCopies; i++) {
+        const int r = i * kRowsPerCopy + rsub;
+        piece_of[i] = (unsigned)(pos ^ ((r >> 1) & 7));
+#pragma unroll
+        for (int t = 0; t < kRT; t++) {
+            long n = n0 + t * 16 + r;
+            n = n < N ? n : N - 1;  // a row past the end repeats the last one (not written)
+            w_off[t][i] = (unsigned)(n - n0) * (unsigned)K * 2u;
+        }
+#pragma unroll
+        for (int t = 0; t < kMT; t++) {
+            int m = t * 16 + r;
+            m = m < M ? m : M - 1;
+            a_off[t][i] = (unsigned)m * (unsigned)K * 2u;
+        }
+    }
+    f32x4 acc[kRT][kMT];
+#pragma unroll
+    for (int r = 0; r < kRT; r++)
+#pragma unroll
+        for (int m = 0; m < kMT; m++) acc[r][m] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // read side: row li of a block, piece 4 s + g of the chunk at position (4 s + g) ^ key(li)
+    const unsigned rd_row = lds_wave + li * (kPieces * 16);
+    const unsigned gx = (unsigned)(g ^ ((li >> 1) & 7));
+    const int pieces = K >> 3;
+    const int chunks = (pieces + kPieces - 1) / kPieces;
+    const int first = (int)(blockIdx.x % (unsigned)chunks);
+    for (int c = wave; c < chunks; c += kWaves) {
+        int cc = c + first;
+        if (cc >= chunks) cc -= chunks;
+        const int p0 = cc * kPieces;
+        const bool full = p0 + kPieces <= pieces;  // else the last chunk of a K that is no multiple of 64
+        // (the previous chunk's fragment reads have all been consumed by matrix instructions; the wait makes that
+        // explicit before the copies may overwrite them)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < kCopies; i++) {
+            unsigned piece = (unsigned)p0 + piece_of[i];
+            if (!full) piece = piece < (unsigned)pieces ? piece : (unsigned)pieces - 1u;  // any valid piece: zeroed below
+#pragma unroll
+            for (int t = 0; t < kRT; t++)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                             :
+                             : "s"(lds_wave + t * kBlockBytes + i * 1024), "v"(w_off[t][i] + piece * 16u), "s"(w_base)
+                             : "m0", "memory");
+#pragma unroll
+            for (int t = 0; t < kMT; t++)
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                             :
+                             : "s"(lds_wave + (kRT + t) * kBlockBytes + i * 1024), "v"(a_off[t][i] + piece * 16u), "s"(a_base)
+                             : "m0", "memory");
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            const unsigned po = (((unsigned)(4 * s)) ^ gx) * 16u;
+            const bool in = full || p0 + 4 * s + g < pieces;
+            u32x4 x[kMT];
+#pragma unroll
+            for (int t = 0; t < kMT; t++) {
+                x[t] = *MRK_LDS_PTR(u32x4, rd_row + (kRT + t) * kBlockBytes + po);
+                if (!full) x[t] = in ? x[t] : u32x4{0u, 0u, 0u, 0u};
+            }
+#pragma unroll
+            for (int r = 0; r < kRT; r++) {
+                u32x4 w = *MRK_LDS_PTR(u32x4, rd_row + r * kBlockBytes + po);
+                if (!full) w = in ? w : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int t = 0; t < kMT; t++) {
+                    if constexpr (kF16)
+                        acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w), __builtin_bit_cast(f16x8, x[t]), acc[r][t], 0, 0, 0);
+                    else
+                        acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x[t]), acc[r][t], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // the waves' partial blocks meet in LDS (over the copy regions, hence the first barrier); a lane of the matrix
+    // result holds four consecutive weight rows for one row of A, i.e. four consecutive elements of a row of C
+    __syncthreads();
+    f32x4* partial = reinterpret_cast<f32x4*>(smem);  // [kWaves][kTiles][64]
+#pragma unroll
+    for (int r = 0; r < kRT; r++)
+#pragma unroll
+        for (int m = 0; m < kMT; m++) partial[(wave * kTiles + r * kMT + m) * 64 + lane] = acc[r][m];
+    __syncthreads();
+    const bool vec = (N & 3) == 0;
+    for (int e = threadIdx.x; e < kTiles * 64; e += kWaves * 64) {
+        const int tile = e >> 6, l = e & 63;
+        f32x4 s = partial[tile * 64 + l];
+#pragma unroll
+        for (int w = 1; w < kWaves; w++) s += partial[(w * kTiles + tile) * 64 + l];
+        const int r = tile / kMT, m = (tile % kMT) * 16 + (l & 15);
+        const long n = n0 + r * 16 + 4 * (l >> 4);
+        if (m >= M || n >= N) continue;
+        unsigned short o[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            if constexpr (kF16) o[i] = __builtin_bit_cast(unsigned short, (_Float16)s[i]);
+            else o[i] = round_bf16(s[i]);
+        }
+        unsigned short* dst = C + (size_t)m * N + n;
+        if (vec) {
+            *reinterpret_cast<u32x2*>(dst) = u32x2{(unsigned)o[0] | ((unsigned)o[1] << 16), (unsigned)o[2] | ((unsigned)o[3] << 16)};
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (n + i < N) dst[i] = o[i];
         }
     }
 }
@@ -277,8 +443,7 @@ __global__ __launch_bounds__(256) void gemm_kn_skinny_reduce(const float* __rest
 namespace mrk {
 
 bool gemm_nt_skinny_supported(long M, long N, long K, long batch) {
-    return M >= 1 && M <= 16 && N >= 1 && K >= 8 && K % 8 == 0 && K <= 0x7fffffffL && N <= 0x7fffffffL && batch >= 1 && batch <= 65535 &&
-           true;
+    return M >= 1 && M <= 2 && N >= 1 && K >= 8 && K % 8 == 0 && K <= 0x7fffffffL && N <= 0x7fffffffL && batch >= 1 && batch <= 65535;
 }
 
 int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16) {
@@ -290,20 +455,82 @@ int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, 
     const unsigned short* a = static_cast<const unsigned short*>(A);
     const unsigned short* b = static_cast<const unsigned short*>(Bt);
     unsigned short* c = static_cast<unsigned short*>(C);
-    // more weight rows per workgroup where the accumulators allow it: every workgroup reads all of A,
-    // so A's share of the traffic is M / rows
+    // (one row: two weight rows per workgroup stream fastest, 6.2 against 6.0 TB/s with four; every workgroup reads
+    // all of A, so with two rows four weight rows per workgroup halve A's share of the traffic)
 #define MRK_SKINNY(KM, KR)                                                                                  \
     do {                                                                                                    \
         const dim3 grid((unsigned)((N + KR - 1) / KR), (unsigned)batch);                                    \
         if (f16) gemm_nt_skinny<KM, KR, true><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K);        \
         else gemm_nt_skinny<KM, KR, false><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K);           \
     } while (0)
-    if (M == 1) MRK_SKINNY(1, 2);  // (one row: two weight rows per workgroup stream fastest, 6.2 against 6.0 TB/s with four)
-    else if (M == 2) MRK_SKINNY(2, 4);
-    else if (M <= 4) MRK_SKINNY(4, 8);
-    else if (M <= 8) MRK_SKINNY(8, 8);
-    else MRK_SKINNY(16, 4);
+    if (M == 1) MRK_SKINNY(1, 2);
+    else MRK_SKINNY(2, 4);
 #undef MRK_SKINNY
+    return (int)hipGetLastError();
+}
+
+// 3 to 64 rows on the matrix pipes (gemm_nt_rows).  Byte offsets inside a workgroup's rows are 32-bit.
+bool gemm_nt_rows_supported(long M, long N, long K, long batch) {
+    return M >= 1 && M <= 64 && N >= 1 && N <= 0x7fffffffL && K >= 8 && K % 8 == 0 && K <= (1L << 23) && batch >= 1 && batch <= 65535;
+}
+
+namespace {
+// Weight blocks (16 rows) per workgroup.  More of them spread the traffic of A (every workgroup reads all of it:
+// kMT / kRT of the weight's bytes) over more weight rows; what costs more is an uneven spread over the 256 CUs:
+// the memory system serves the CUs about evenly, so the launch lasts as long as the CU with the most workgroups
+// needs (344 workgroups, i.e. two on 88 CUs and one on the rest, measured 15 % slower than 230 or 459).
+int rows_blocks_per_group(long N, int mt) {
+    const long tiles = (N + 15) / 16;
+    int best = 1;
+    double best_score = -1.0;
+    for (int rt : {6, 4, 3, 2, 1}) {
+        if (rt * mt > 18) continue;  // (not instantiated: the partial sums of 8 waves would not fit the LDS)
+        const long groups = (tiles + rt - 1) / rt;
+        const long per_cu = (groups + 255) / 256;
+        const double even = (double)groups / (double)(256 * per_cu);
+        const double score = even / (1.0 + 0.25 * mt / rt);
+        if (score > best_score) best_score = score, best = rt;
+    }
+    return best;
+}
+}  // namespace
+
+int launch_gemm_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16) {
+    using namespace mrk::dev;
+    if (!gemm_nt_rows_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) % 16 || reinterpret_cast<uintptr_t>(C) % 8) return (int)hipErrorInvalidValue;
+    (void)hipGetLastError();
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned short* a = static_cast<const unsigned short*>(A);
+    const unsigned short* b = static_cast<const unsigned short*>(Bt);
+    unsigned short* c = static_cast<unsigned short*>(C);
+    const int mt = (int)((M + 15) / 16);
+    const int rt = rows_blocks_per_group(N, mt);
+#define MRK_ROWS(MT, RT, WV)                                                                              \
+    do {                                                                                                  \
+        const dim3 grid((unsigned)((N + 16 * RT - 1) / (16 * RT)), (unsigned)batch);                      \
+        if (f16) gemm_nt_rows<MT, RT, WV, true><<<grid, WV * 64, 0, s>>>(a, b, c, (int)M, (int)N, (int)K); \
+        else gemm_nt_rows<MT, RT, WV, false><<<grid, WV * 64, 0, s>>>(a, b, c, (int)M, (int)N, (int)K);    \
+    } while (0)
+#define MRK_ROWS_UP_TO_4(MT)                  \
+    do {                                      \
+        if (rt == 1) MRK_ROWS(MT, 1, 16);     \
+        else if (rt == 2) MRK_ROWS(MT, 2, 8); \
+        else if (rt == 3) MRK_ROWS(MT, 3, 8); \
+        else MRK_ROWS(MT, 4, 8);              \
+    } while (0)
+#define MRK_ROWS_MT(MT)                      \
+    do {                                     \
+        if (rt == 6) MRK_ROWS(MT, 6, 8);     \
+        else MRK_ROWS_UP_TO_4(MT);           \
+    } while (0)
+    if (mt == 1) MRK_ROWS_MT(1);
+    else if (mt == 2) MRK_ROWS_MT(2);
+    else if (mt == 3) MRK_ROWS_MT(3);
+    else MRK_ROWS_UP_TO_4(4);  // (six blocks of 4 x 16 rows: not instantiated, rows_blocks_per_group never asks for it)
+#undef MRK_ROWS_UP_TO_4
+#undef MRK_ROWS_MT
+#undef MRK_ROWS
     return (int)hipGetLastError();
 }
 

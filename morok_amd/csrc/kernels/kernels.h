@@ -17,10 +17,9 @@ int launch_softmax_f32(void* stream, const void* x, void* y, long rows, long col
 // C [batch,M,N]), one launch.
 // b_transposed: B is stored as B^T [N, K] (k contiguous: the layout of a Linear layer's weight;
 // [batch, N, K] for batch > 1).  Same products in the same order, so the same bits as the [K, N]
-// form (split-K included, given the workspace).  Up to eight rows, and up to 16 where the tiled
-// kernels do not apply (N not a multiple of 8, split-K shape without a workspace), take the
-// streaming kernel below, whose sums run in another order.  Shapes outside
-// gemm_bf16_nt_supported (K not a multiple of 8; N not a multiple of 8 with more than 16 rows)
+// form (split-K included, given the workspace).  Up to 64 rows with K a multiple of 8 take the
+// streaming kernels below (any N, no workspace), whose sums run in another order.  Shapes outside
+// gemm_bf16_nt_supported (K not a multiple of 8; N not a multiple of 8 with more than 64 rows)
 // are refused with hipErrorInvalidValue.
 // f16: operands and result are IEEE half precision instead of bf16 (the same kernels around
 // v_mfma_f32_16x16x32_f16; plain product only, the fused epilogues are bf16).
@@ -28,12 +27,20 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
                      long batch = 1, void* workspace = nullptr, size_t workspace_bytes = 0, bool b_transposed = false,
                      bool f16 = false);
 bool gemm_bf16_nt_supported(long M, long N, long K, long batch);
-// C[M, N] = A[M, K] @ Bt[N, K]^T for M <= 16 (a decode step against a Linear layer's weight): one
+// Scratch bytes launch_gemm_bf16 wants for the Bt[N, K] form: 0 for up to 64 rows (streamed), else the split-K
+// plan's as for the [K, N] form.
+size_t gemm_bf16_nt_workspace_bytes(long M, long N, long K, long batch);
+// C[M, N] = A[M, K] @ Bt[N, K]^T for one or two rows (a decode step against a Linear layer's weight): one
 // pass over the weight with packed dot products, no matrix pipe, no scratch memory.  K a multiple
 // of 8, any N; bf16 or (f16) IEEE half operands and result, f32 accumulation.  Summation order
 // differs from the tiled kernels', so results agree with them to rounding, not bit for bit.
 bool gemm_nt_skinny_supported(long M, long N, long K, long batch);
 int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16);
+// The same for up to 64 rows on the matrix pipes: 16-row blocks of both operands go through LDS (direct
+// copies, fragments read back), the waves of a workgroup split K and add their sums in a fixed order.  One
+// launch, no scratch memory.  K a multiple of 8 (at most 2^23), any N.
+bool gemm_nt_rows_supported(long M, long N, long K, long batch);
+int launch_gemm_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16);
 // The [K, N] form for one or two rows (N <= 24576 and K multiples of 8, K >= 256, one product): the weight is
 // streamed once into `splits` f32 partial results W[splits][M][N], which a second kernel adds up in a
 // fixed order and rounds into C; gemm_kn_skinny_plan chooses the split and tells whether the shape is

@@ -2104,9 +2104,10 @@ struct Scheduler {
             if (a->dtype == Scalar::BFloat16 || a->dtype == Scalar::Float16) {
                 // few output tiles against a long K: scratch for split-K partials, an intermediate
                 // of the plan like any other (lazily allocated, placed by the memory planner)
-                const size_t ws = gemm_bf16_workspace_bytes(M, N, K, batch);
+                // (up to 64 rows against an [N, K] weight stream it in one pass and need no scratch)
+                const size_t ws = nt ? gemm_bf16_nt_workspace_bytes(M, N, K, batch) : gemm_bf16_workspace_bytes(M, N, K, batch);
                 const std::string kind = a->dtype == Scalar::Float16 ? "gemm_f16" : "gemm_bf16";
-                if (nt && ws && M > 8) {  // (up to eight rows stream the weight in one pass and need no scratch)
+                if (nt && ws) {
                     auto scratch = std::make_shared<Buffer>(dev->allocator, ws, BufferOptions());
                     rc = builtin((kind + "_nt").c_str(), {M, N, K, 1, static_cast<int64_t>(ws)}, {out, a->buffer, wbuf, scratch});
                 } else if (nt) {

@@ -10,6 +10,7 @@ int launch_softmax_f32(void* stream, const void*, void*, long, long, int) {
     return 0;
 }
 size_t gemm_bf16_workspace_bytes(long, long, long, long) { return 0; }
+size_t gemm_bf16_nt_workspace_bytes(long, long, long, long) { return 0; }
 int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, long, int, long, void*, size_t, bool b_transposed, bool f16) {
     mrk_shim_note_launch(stream, f16 ? (b_transposed ? "gemm_f16_nt" : "gemm_f16") : b_transposed ? "gemm_bf16_nt" : "gemm_bf16");
     return 0;
@@ -17,8 +18,13 @@ int launch_gemm_bf16(void* stream, const void*, const void*, void*, long, long, 
 bool gemm_bf16_nt_supported(long M, long N, long K, long batch) {
     return M > 0 && N > 0 && K > 0 && batch > 0 && N % 8 == 0 && K % 8 == 0;
 }
-bool gemm_nt_skinny_supported(long M, long N, long K, long batch) { return M >= 1 && M <= 16 && N >= 1 && K >= 8 && K % 8 == 0 && batch >= 1; }
+bool gemm_nt_skinny_supported(long M, long N, long K, long batch) { return M >= 1 && M <= 2 && N >= 1 && K >= 8 && K % 8 == 0 && batch >= 1; }
 int launch_gemm_nt_skinny(void* stream, const void*, const void*, void*, long, long, long, long, bool f16) {
+    mrk_shim_note_launch(stream, f16 ? "gemm_f16_nt" : "gemm_bf16_nt");
+    return 0;
+}
+bool gemm_nt_rows_supported(long M, long N, long K, long batch) { return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && batch >= 1; }
+int launch_gemm_nt_rows(void* stream, const void*, const void*, void*, long, long, long, long, bool f16) {
     mrk_shim_note_launch(stream, f16 ? "gemm_f16_nt" : "gemm_bf16_nt");
     return 0;
 }

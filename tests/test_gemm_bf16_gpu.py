@@ -296,7 +296,7 @@ def test_gemm_swiglu_epilogue_parity(dev, oracle, shape):
 # ---------------------------------------------------------------- second operand stored [N, K]
 # (a Linear layer's weight, tensor/src/nn/linear.rs:9-14: y = x @ weight.T + bias)
 @pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 256), (300, 520, 128), (1024, 1024, 1024), (1000, 776, 320),
-                                   (100, 264, 200), (256, 256, 72), (129, 8, 72), (2048, 512, 136), (37, 4096, 64)])
+                                   (100, 264, 200), (256, 256, 72), (129, 8, 72), (2048, 512, 136), (137, 4096, 64)])
 def test_gemm_transposed_second_operand(dev, oracle, shape):
     """a @ bt.T with bt [N, K] read in place: the same products in the same order as the
     [K, N] form, so the same bits, on full, ragged-M/N and ragged-K shapes and with either tile
@@ -323,16 +323,16 @@ def test_gemm_transposed_second_operand(dev, oracle, shape):
 
 
 def test_gemm_transposed_second_operand_refusals(dev):
-    a, b, c = dev.buffer(32 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(32 * 1024 * 2)
+    a, b, c = dev.buffer(72 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(72 * 1024 * 2)
     with pytest.raises(morok_amd.MorokHipError):
         ops.gemm_bf16_nt(a, b, c, 32, 1024, 4092, dev.device_id)  # K not a multiple of 8
     with pytest.raises(morok_amd.MorokHipError):
-        ops.gemm_bf16_nt(a, b, c, 32, 1020, 64, dev.device_id)    # N not a multiple of 8 with more than 16 rows
+        ops.gemm_bf16_nt(a, b, c, 72, 1020, 64, dev.device_id)    # N not a multiple of 8 with more than 64 rows
 
 
-@pytest.mark.parametrize("shape", [(32, 1024, 4096), (64, 4096, 4096), (17, 520, 2048), (100, 264, 4104), (9, 4096, 4096), (128, 512, 8192)])
+@pytest.mark.parametrize("shape", [(72, 1024, 4096), (96, 4096, 4096), (65, 520, 2048), (100, 264, 4104), (80, 4096, 8192), (128, 512, 8192)])
 def test_gemm_transposed_second_operand_split_k(dev, oracle, shape):
-    """Few output tiles against a long K with the weight stored [N, K]: the K loop is spread over the
+    """Few output tiles against a long K with the weight stored [N, K] and more than 64 rows: the K loop is spread over the
     chip as for the [K, N] form (same K ranges, same order inside a range: the same bits), through the
     ABI (which brings the scratch itself) and as a plan item with a scratch buffer."""
     M, N, K = shape

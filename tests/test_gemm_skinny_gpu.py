@@ -1,6 +1,7 @@
 """A handful of rows against a Linear layer's weight as it is stored ([out_features, in_features],
-tensor/src/nn/linear.rs:9-14,39-41: y = x @ weight.T): the streaming kernel behind
-mrk_hip_gemm_bf16_nt / mrk_hip_gemm_f16_nt for M <= 16, against the CPU oracle (exact products, f32
+tensor/src/nn/linear.rs:9-14,39-41: y = x @ weight.T): the streaming kernels behind
+mrk_hip_gemm_bf16_nt / mrk_hip_gemm_f16_nt for M <= 64 (one and two rows on the vector ALUs, 3 to 64 on the
+matrix pipes), against the CPU oracle (exact products, f32
 accumulate, one rounding) on identical seeded inputs.  Tolerance from the north star: <= 2e-2 max
 relative error (max|gpu - ref| / max|ref|) plus the elementwise bound of the tiled kernels' tests
 (the result's own rounding plus summation-order noise); against the tiled kernel on the transposed
@@ -22,7 +23,10 @@ def T(dev):
 
 
 SHAPES = [(1, 4096, 4096), (1, 8, 8), (2, 1020, 64), (3, 37, 520), (4, 1024, 4096), (5, 4099, 512), (7, 256, 11008),
-          (8, 2048, 2048), (9, 130, 1032), (13, 515, 264), (16, 4096, 1024), (16, 3, 8)]
+          (8, 2048, 2048), (9, 130, 1032), (13, 515, 264), (16, 4096, 1024), (16, 3, 8),
+          # every block count of A (1-4) and of the weight (1, 2, 3, 4, 6 blocks per workgroup), K with a partial chunk
+          (17, 8192, 1096), (24, 12288, 512), (32, 16384, 264), (33, 22016, 256), (40, 5000, 1032), (48, 24576, 128),
+          (49, 4096, 4096), (64, 16384, 520), (64, 77, 40), (61, 12288, 64), (3, 22016, 72), (20, 1, 8)]
 
 
 def _check(cf, rf, K, ulp):
@@ -41,8 +45,7 @@ def _run(dev, a16, bt16, nan, f16):
     bb = morok_amd.Buffer.from_numpy(np.concatenate([bt16.reshape(-1), pad]), dev.device_id)
     bc = dev.buffer((M * N + 2048) * 2)
     bc.copyin(np.full(M * N + 2048, nan, np.uint16))
-    # as a plan item without a scratch buffer: every shape of this file then takes the streaming kernel (up to
-    # eight rows; N not a multiple of 8; few tiles against a long K, where the ABI call would bring scratch for split-K)
+    # as a plan item: up to 64 rows take the streaming kernels and no scratch buffer
     morok_amd.Program.builtin("gemm_f16_nt" if f16 else "gemm_bf16_nt", [M, N, K], dev.device_id).execute([bc, ba, bb])
     out = bc.copyout(np.uint16)
     assert np.all(out[M * N:] == nan)            # nothing written past the result
@@ -69,16 +72,13 @@ def test_skinny_bf16_vs_oracle_and_tiled_kernel(dev, oracle, shape):
     bc3 = dev.buffer(M * N * 2)
     morok_amd.Program.builtin("gemm_bf16_nt", [M, N, K], dev.device_id).execute([bc3, ba, bb])
     assert np.array_equal(bc3.copyout(np.uint16, (M, N)), got)
-    # through the ABI (up to eight rows: the same kernel; more: split-K over the tiled kernels where the shape has tiles)
+    # through the ABI: the same kernel
     ops.gemm_bf16_nt(ba, bb, bc3, M, N, K, dev.device_id)
-    abi = bc3.copyout(np.uint16, (M, N))
-    if M <= 8 or N % 8:
-        assert np.array_equal(abi, got)
-    else:
-        assert np.array_equal(abi, bc2.copyout(np.uint16, (M, N)))     # the bits of the [K, N] form
+    assert np.array_equal(bc3.copyout(np.uint16, (M, N)), got)
 
 
-@pytest.mark.parametrize("shape", [(1, 4096, 4096), (3, 37, 520), (8, 2048, 2048), (16, 1000, 1032), (6, 4099, 64)])
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (3, 37, 520), (8, 2048, 2048), (16, 1000, 1032), (6, 4099, 64), (2, 515, 264),
+                                   (24, 12288, 520), (40, 16384, 128), (64, 4100, 1032), (33, 32000, 64)])
 def test_skinny_f16_vs_oracle(dev, oracle, shape):
     M, N, K = shape
     a = synth.normal((M, K), 13, 2).astype(np.float16)
@@ -93,7 +93,7 @@ def test_skinny_exact_cases(dev):
     """Values whose sums are exact in f32 whatever the order: small integers.  Every output must be the
     integer dot product, for every row count the kernel is instantiated for and the ones between."""
     rng = np.random.default_rng(5)
-    for M in range(1, 17):
+    for M in list(range(1, 18)) + [31, 32, 33, 47, 48, 49, 63, 64]:
         N, K = 260 + M, 1544
         a = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
         bt = rng.integers(-4, 5, size=(N, K)).astype(np.float32)
@@ -104,7 +104,11 @@ def test_skinny_exact_cases(dev):
 
 def test_skinny_batched_plan_item(dev, oracle):
     """{M, N, K, batch}: that many products over operands stored back to back."""
-    M, N, K, B = 4, 520, 1024, 3
+    for M, N, K, B in ((4, 520, 1024, 3), (2, 130, 512, 2), (20, 4100, 264, 3)):
+        _batched(dev, oracle, M, N, K, B)
+
+
+def _batched(dev, oracle, M, N, K, B):
     a = synth.normal_bf16((B, M, K), 13, 4)
     bt = synth.normal_bf16((B, N, K), 13, 5)
     ba, bb = morok_amd.Buffer.from_numpy(a, dev.device_id), morok_amd.Buffer.from_numpy(bt, dev.device_id)
@@ -117,16 +121,16 @@ def test_skinny_batched_plan_item(dev, oracle):
 
 
 def test_skinny_refusals(dev):
-    a, b, c = dev.buffer(64 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(64 * 1024 * 2)
+    a, b, c = dev.buffer(72 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(72 * 1024 * 2)
     with pytest.raises(morok_amd.MorokHipError):
         ops.gemm_bf16_nt(a, b, c, 4, 1024, 4092, dev.device_id)    # K not a multiple of 8
     with pytest.raises(morok_amd.MorokHipError):
-        ops.gemm_bf16_nt(a, b, c, 17, 1020, 4096, dev.device_id)   # more than 16 rows and N not a multiple of 8
+        ops.gemm_bf16_nt(a, b, c, 65, 1020, 4096, dev.device_id)   # more than 64 rows and N not a multiple of 8
 
 
 def test_linear_decode_step_is_one_kernel(T, oracle):
-    """x [1, K] (and batches of 8 and 12) through Tensor.linear with the weight as stored: one product that
-    reads the weight in place, no transposed copy (up to eight rows stream it in one pass, twelve take the
+    """x [1, K] (and batches of 8, 12 and 64) through Tensor.linear with the weight as stored: one product that
+    reads the weight in place, no transposed copy, no scratch (up to 64 rows stream it in one pass; 80 take the
     tiled kernels with the K loop spread over the chip)."""
     from morok_amd import uop
 
@@ -134,11 +138,11 @@ def test_linear_decode_step_is_one_kernel(T, oracle):
     K, N = 2048, 3072
     w = synth.normal_bf16((N, K), 13, 6)
     tw = T.Tensor.from_numpy(w, uop.BF16)
-    for M in (1, 8, 12):
+    for M in (1, 8, 12, 64, 80):
         x = synth.normal_bf16((M, K), 13, 7)
         y = T.Tensor.from_numpy(x, uop.BF16).linear(tw)
         got = y.to_numpy()
-        assert y.kernels() == [f"gemm_bf16_nt_{M}_{N}_{K}" + ("" if M <= 8 else "_splitk")]
+        assert y.kernels() == [f"gemm_bf16_nt_{M}_{N}_{K}" + ("" if M <= 64 else "_splitk")]
         ref = oracle.gemm_bf16(x, np.ascontiguousarray(w.T))
         _check(synth.from_bf16(got), synth.from_bf16(ref), K, 2**-7)
 
