@@ -439,14 +439,16 @@ size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_
 /* c[M,N] = a[M,K] * bt[N,K]^T: the product with the second operand as it is stored by a Linear
  * layer (weight [out_features, in_features], tensor/src/nn/linear.rs:9-14, 39-41), read in place
  * instead of through a transposed copy.  K a multiple of 8, 16-byte aligned operands.  More than
- * eight rows with N a multiple of 8: the tiled kernels, the same products in the same order as
+ * 64 rows with N a multiple of 8: the tiled kernels, the same products in the same order as
  * mrk_hip_gemm_bf16 on the transposed matrix, so the same bits (split-K shapes included; the
- * scratch comes from the device allocator).  Up to eight rows (a decode step), and up to 16 rows
- * with any N: one streaming pass over the weight with packed dot products, f32 accumulation in
- * another order (results agree with the tiled kernels to the rounding of the result).  More than
- * 16 rows with N not a multiple of 8, or K not a multiple of 8: INVALID_ARGUMENT.  Builtin Program
- * kind "gemm_bf16_nt" ({M, N, K[, batch[, workspace bytes]]}; without a workspace a split-K shape
- * of up to 16 rows streams, a larger one runs the plain tiled kernel). */
+ * scratch comes from the device allocator).  Up to 64 rows (a decode step, a batch of them) with
+ * any N: one streaming pass over the weight, no scratch: one or two rows with packed dot products
+ * on the vector ALUs, 3 to 64 on the matrix pipes from 16-row blocks staged through LDS; f32
+ * accumulation in another order than the tiled kernels' (results agree with them to the rounding
+ * of the result), the same bits on every run.  More than 64 rows with N not a multiple of 8, or K
+ * not a multiple of 8: INVALID_ARGUMENT.  Builtin Program kind "gemm_bf16_nt"
+ * ({M, N, K[, batch[, workspace bytes]]}; the workspace is used by split-K shapes of more than 64
+ * rows, which without one run the plain tiled kernel). */
 int mrk_hip_gemm_bf16_nt(int device_id, const void* a, const void* bt, void* c, int64_t m, int64_t n, int64_t k);
 /* The same two products on IEEE half precision (f16) operands and result, f32 accumulate: the f16
  * 16x16x32 entry of the reference's CDNA4 tensor-core table
