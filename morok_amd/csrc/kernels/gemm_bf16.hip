@@ -925,14 +925,18 @@ SplitPlan plan_split_k(long M, long N, long K, long batch) {
     SplitPlan p;
     const long tiles = ((M + 127) / 128) * ((N + 255) / 256) * batch;
     const long kt_all = (K + 63) / 64;
-    if (K % 8 != 0 || N % 8 != 0 || tiles > 64 || kt_all < 8) return p;  // at most a quarter of the CUs busy
+    // at most a quarter of the CUs busy; with up to 64 rows (the weight is streamed once, the partial results are
+    // small) up to half of them, and then two or three ranges already pay (16 x 22016 x 4096: 86 tiles)
+    const bool few_rows = M <= 64;
+    if (K % 8 != 0 || N % 8 != 0 || tiles > (few_rows ? 128 : 64) || kt_all < 8) return p;
     long want = 256 / tiles;                 // ranges that would put one workgroup on every CU
     if (want > kt_all / 2) want = kt_all / 2;  // at least two K steps per range
     // the partial results are written and read back once per range: worth it only while that
     // traffic stays below what the operands themselves move
     const double operand_bytes = 2.0 * batch * ((double)M * K + (double)K * N);
-    while (want >= 4 && 2.0 * want * batch * M * N * 4.0 > operand_bytes) want--;
-    if (want < 4) return p;
+    const long least = few_rows ? 2 : 4;
+    while (want >= least && 2.0 * want * batch * M * N * 4.0 > operand_bytes) want--;
+    if (want < least) return p;
     p.kt_per_split = (kt_all + want - 1) / want;
     p.splits = (kt_all + p.kt_per_split - 1) / p.kt_per_split;
     if (p.splits < 2) p.splits = 1;

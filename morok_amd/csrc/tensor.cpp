@@ -1407,6 +1407,14 @@ struct Scheduler {
         return kOk;
     }
 
+    // A product with so few rows that it is not run as one pass of output tiles: the K loop spread over the chip
+    // (scratch and a second kernel), or the weight streamed for a handful of rows.  The tiled kernels' fused
+    // epilogues would hold such a product on the few workgroups its tiles make (measured at 4 x 22016 x 4096 with
+    // the gate: 70 us against 30 us for the streamed product plus an elementwise kernel), so they are not matched.
+    bool spread_or_streamed(const TensorNode* mm, int64_t M, int64_t N, int64_t K, int64_t batch) const {
+        if (gemm_bf16_workspace_bytes(M, N, K, batch)) return true;
+        return transposed_weight(mm) && (gemm_nt_skinny_supported(M, N, K, batch) || gemm_nt_rows_supported(M, N, K, batch));
+    }
     // x + (a @ w) in bf16 where nothing else reads the product: the product kernel adds x in its
     // epilogue (same bits as the product followed by the add).  Returns the product node and the
     // other operand.
@@ -1428,7 +1436,7 @@ struct Scheduler {
             if (!(rb->buffer || is_boundary_kind(rb) || fusable(rb))) continue;
             int64_t M, N, K, batch;
             matmul_extents(mm, &M, &N, &K, &batch);
-            if (!gemm_bf16_residual_supported(M, N, K, batch) || gemm_bf16_workspace_bytes(M, N, K, batch)) continue;
+            if (!gemm_bf16_residual_supported(M, N, K, batch) || spread_or_streamed(mm, M, N, K, batch)) continue;
             *other = r;
             return mm;
         }
@@ -1461,7 +1469,7 @@ struct Scheduler {
             if (!used(mm, 2) || !used(gate, 2) || !used(up, 1) || !used(sw, 1)) continue;
             int64_t Mx, N2, K, batch;
             matmul_extents(mm, &Mx, &N2, &K, &batch);
-            if (batch != 1 || Mx != M || N2 != 2 * F || !gemm_bf16_swiglu_supported(M, F, K)) continue;
+            if (batch != 1 || Mx != M || N2 != 2 * F || !gemm_bf16_swiglu_supported(M, F, K) || spread_or_streamed(mm, M, N2, K, 1)) continue;
             return mm;
         }
         return nullptr;
@@ -1639,7 +1647,8 @@ struct Scheduler {
         if (mm->hint_inputs[0]->shape.size() != 2 || mm->hint_inputs[1]->shape.size() != 2 || transposed_weight(mm)) return nullptr;
         const int64_t M = mm->shape[0], N = mm->shape[1], K = mm->hint_inputs[0]->shape[1], split = sl->shape[1];
         if (sl->shape[0] != M || sl->arg.size() != 2 || sl->arg[0] != 0 || sl->arg[1] != 0) return nullptr;
-        if (x->shape[0] * S != M || x->shape[2] * 128 != split || !gemm_bf16_rope_supported(M, N, K, split, S)) return nullptr;
+        if (x->shape[0] * S != M || x->shape[2] * 128 != split || !gemm_bf16_rope_supported(M, N, K, split, S) || gemm_bf16_workspace_bytes(M, N, K, 1))
+            return nullptr;
         // the product's readers: this slice and, when there are columns left, exactly the slice of all of them
         auto readers = matmul_readers.find(mm);
         if (readers == matmul_readers.end()) return nullptr;

@@ -56,6 +56,30 @@ def test_decoder_block_vs_oracle(dev, oracle, cfg):
     assert rel_err(out7.to_numpy(), ref) <= 2e-2
 
 
+@pytest.mark.parametrize("cfg", [
+    dict(batch=2, seq=8, hidden=4096, heads=32, ffn=11008, vocab=32000, eps=1e-6),
+    dict(batch=1, seq=40, hidden=1024, heads=8, ffn=2816, vocab=500, eps=1e-6),
+], ids=["h4096_16tokens", "h1024_40tokens"])
+def test_decoder_block_few_tokens(dev, oracle, cfg):
+    """A handful of tokens: every product has few output tiles against a long K, so it is spread along K (or
+    streamed) instead of run as one pass of tiles, and the fused epilogues, which exist for the tiled
+    kernels only, are not matched: the gate and the residual adds run as generated kernels."""
+    from morok_amd import decoder, synth
+
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], cfg["vocab"], seed=4)
+    T = cfg["batch"] * cfg["seq"]
+    tok = synth.randint((T,), 4, 1, cfg["vocab"])
+    blk, out, kernels = run_block(cfg, tok, w)
+    got = out.to_numpy()
+    ref = oracle.decoder_block_bf16(tok, w, blk.cos_host, blk.sin_host, cfg["batch"], cfg["seq"], cfg["hidden"],
+                                    cfg["heads"], cfg["ffn"], cfg["eps"])
+    assert rel_err(got, ref) <= 2e-2
+    assert sum(k.startswith("gemm_bf16") for k in kernels) == 4
+    assert sum(k.startswith("flash_fwd") for k in kernels) == 1
+    if cfg["hidden"] == 4096:
+        assert all(k.endswith("_splitk") for k in kernels if k.startswith("gemm_bf16")), kernels
+
+
 def test_decoder_block_full_size_properties(dev):
     """hidden 4096, 32 heads, SwiGLU 11008, batch 4 x seq 2048: too large for the CPU oracle in
     a test, so checked through properties that hold at any size: determinism, independence of
