@@ -947,7 +947,9 @@ SplitPlan plan_split_k(long M, long N, long K, long batch) {
 size_t gemm_bf16_workspace_bytes(long M, long N, long K, long batch) {
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return 0;
     long ks = 0, kr = 0;
-    if (gemm_kn_skinny_plan(M, N, K, batch, &ks, &kr)) return (size_t)ks * M * N * sizeof(float);  // a handful of rows: streamed
+    // a handful of rows: streamed (one row on the vector ALUs where that kernel's plan takes the shape, more on the matrix pipes)
+    if (gemm_kn_skinny_plan(M, N, K, batch, &ks, &kr)) return (size_t)ks * M * N * sizeof(float);
+    if (gemm_kn_rows_plan(M, N, K, batch, &ks, &kr)) return ks > 1 ? (size_t)ks * M * N * sizeof(float) : 0;
     const SplitPlan p = plan_split_k(M, N, K, batch);
     return p.splits > 1 ? (size_t)p.splits * batch * M * N * sizeof(float) : 0;
 }
@@ -1137,12 +1139,16 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
                                                                           static_cast<__bf16*>(C), (int)M, (int)N, (int)K, (int)tm, (int)tn);
         return (int)hipGetLastError();
     }
-    // up to eight rows: one streaming pass over the weight into f32 partial sums, then their sum
+    // up to 16 rows: one streaming pass over the weight into f32 partial sums, then their sum
     {
         long ks = 0, kr = 0;
         if ((variant == 0 || variant == 5) && aligned && gemm_kn_skinny_plan(M, N, K, batch, &ks, &kr) && workspace &&
             workspace_bytes >= (size_t)ks * M * N * sizeof(float) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
             return launch_gemm_kn_skinny(stream, A, B, C, workspace, M, N, K, ks, kr, f16);
+        }
+        if ((variant == 0 || variant == 5) && aligned && gemm_kn_rows_plan(M, N, K, batch, &ks, &kr) &&
+            (ks == 1 || (workspace && workspace_bytes >= (size_t)ks * M * N * sizeof(float) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0))) {
+            return launch_gemm_kn_rows(stream, A, B, C, workspace, M, N, K, ks, kr, f16);
         }
     }
     // any M; N and K in whole 16-byte chunks

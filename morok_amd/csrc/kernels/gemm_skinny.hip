@@ -163,6 +163,7 @@ __global__ __launch_bounds__(256) void gemm_nt_skinny(const unsigned short* __re
 // 5.6-6.5 TB/s for up to 32 rows of A.  kMT: 16-row blocks of A (M <= 16 * kMT; rows beyond M repeat row M - 1
 // and are not written); kRT: 16-row blocks of the weight per workgroup.  grid = (ceil(N / (16 kRT)), batch).
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
@@ -309,7 +310,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
 }
 
 
-// C[M, N] = A[M, K] @ B[K, N] for up to eight rows with the weight stored [K, N]: the first of two
+// C[M, N] = A[M, K] @ B[K, N] for one row (the template takes up to eight) with the weight stored [K, N]: the first of two
 // kernels, which streams the weight once and leaves f32 partial sums (the tiled kernels' split-K
 // reduction adds them up and rounds).  A lane owns eight consecutive columns, a wave 512; the
 // workgroups split K (blockIdx.y: rows_per_group consecutive k-rows each, a multiple of 32) and a
@@ -399,6 +400,143 @@ __global__ __launch_bounds__(256) void gemm_kn_skinny_partial(const unsigned sho
 }
 
 
+// 2 to 16 rows (to 64 against a narrow weight) against a weight stored [K, N], on the matrix pipes: the matrix instruction wants eight consecutive k
+// of one weight column per lane, and in this layout consecutive bytes are consecutive columns, so the weight goes
+// through LDS and comes back through the transposing read.  A workgroup of eight waves owns 64 * kCB columns and
+// (blockIdx.y) a range of K; the waves take the range's 32-row chunks in turn.  A wave copies its chunk with direct
+// global -> LDS loads (1 KB per instruction = eight k-rows x 128 bytes, non-temporal), the 32-byte granules (16
+// columns) of a k-row stored at granule ^ f(k-row) with f = bit 1 | bit 3 << 1 of the row, so that the rows a
+// transposing read touches in one pass fall into different banks; ds_read_b64_tr_b16 then hands lane j of a
+// 16-lane block column j's four k (two reads: eight), which is the matrix instruction's operand.  A's fragment
+// (16 rows x 64 bytes, cache hits) is loaded straight from memory.  The region is private to the wave: no barrier
+// in the loop.  The waves' sums meet in LDS; the workgroup writes f32 partial sums W[blockIdx.y][M][N] for
+// gemm_kn_rows_reduce, or with a single K range the rounded result.
+template <int kMT, int kCB, bool kF16>
+__global__ __launch_bounds__(512) void gemm_kn_rows(const unsigned short* __restrict__ A, const unsigned short* __restrict__ B,
+                                                    unsigned short* __restrict__ C, float* __restrict__ W, int M, int N, int K, int k_per_split) {
+    constexpr int kWaves = 8;
+    constexpr int kBlockBytes = 32 * 128;  // 32 k-rows x 64 columns
+    constexpr int kWaveBytes = kCB * kBlockBytes;
+    constexpr int kTiles = kCB * 4 * kMT;  // 16 x 16 accumulator blocks per wave
+    constexpr int kSumBytes = kWaves * kTiles * 1024;
+    constexpr int kLds = kWaves * kWaveBytes > kSumBytes ? kWaves * kWaveBytes : kSumBytes;
+    __shared__ __attribute__((aligned(1024))) char smem[kLds];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long n0 = (long)blockIdx.x * (64 * kCB);
+    const int k_begin = blockIdx.y * k_per_split;
+    const int k_end = k_begin + k_per_split < K ? k_begin + k_per_split : K;
+    const unsigned lds_wave = (unsigned)(uintptr_t)MRK_LDS_PTR(char, smem) + wave * kWaveBytes;
+    // copy side: copy i of a block covers k-rows 8 i .. 8 i + 7; lane -> k-row 8 i + lane / 8, position lane % 8 of the row
+    const int prow = lane >> 3, ppos = lane & 7;
+    unsigned b_off[kCB][4];  // byte offset from (the chunk's first k-row, column n0)
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int kr = 8 * i + prow;
+        const int f = ((kr >> 1) & 1) | (((kr >> 3) & 1) << 1);
+        const int q = (((ppos >> 1) ^ f) << 1) | (ppos & 1);  // 16-byte piece of the row this lane fetches
+#pragma unroll
+        for (int c = 0; c < kCB; c++) {
+            long col = n0 + c * 64 + q * 8;
+            col = col < N ? col : N - 8;  // a piece past the end repeats the last one (not written)
+            b_off[c][i] = (unsigned)kr * (unsigned)N * 2u + (unsigned)(col - n0) * 2u;
+        }
+    }
+    // read side: 16-lane block blk covers k-rows 8 blk .. 8 blk + 7 in two reads of four; lane jl of the block points
+    // at k-row jl / 4 of the four, 8-byte unit jl % 4 of the column block's granule
+    const int jl = lane & 15, blk = lane >> 4;
+    const int fr = ((jl >> 3) & 1) | ((blk & 1) << 1);
+    unsigned rd[4];
+#pragma unroll
+    for (int c4 = 0; c4 < 4; c4++) rd[c4] = lds_wave + (8 * blk + (jl >> 2)) * 128 + ((c4 ^ fr) << 5) + (jl & 3) * 8;
+    const u32x4* a_row[kMT];
+#pragma unroll
+    for (int t = 0; t < kMT; t++) {
+        const int m = t * 16 + jl;
+        a_row[t] = reinterpret_cast<const u32x4*>(A + (size_t)(m < M ? m : M - 1) * K);
+    }
+    f32x4 acc[kCB * 4][kMT];
+#pragma unroll
+    for (int c = 0; c < kCB * 4; c++)
+#pragma unroll
+        for (int t = 0; t < kMT; t++) acc[c][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int chunks = (k_end - k_begin + 31) / 32;
+    const int first = (int)(blockIdx.x % (unsigned)chunks);
+    for (int ci = wave; ci < chunks; ci += kWaves) {
+        int cc = ci + first;
+        if (cc >= chunks) cc -= chunks;
+        const int k0 = k_begin + cc * 32;
+        const bool full = k0 + 32 <= k_end;  // else the last chunk of a range that is no multiple of 32 (it is one of 8)
+        const char* base = reinterpret_cast<const char*>(B) + ((size_t)k0 * N + n0) * 2;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int c = 0; c < kCB; c++) {
+                unsigned off = b_off[c][i];
+                if (!full) {  // a k-row past the end repeats the range's last one (zeroed below)
+                    const int kr = 8 * i + prow;
+                    if (k0 + kr >= k_end) off -= (unsigned)(k0 + kr - (k_end - 1)) * (unsigned)N * 2u;
+                }
+                asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                             :
+                             : "s"(lds_wave + c * kBlockBytes + i * 1024), "v"(off), "s"(base)
+                             : "m0", "memory");
+            }
+        }
+        const bool in = full || k0 + 8 * blk < k_end;
+        u32x4 x[kMT];
+#pragma unroll
+        for (int t = 0; t < kMT; t++) {
+            x[t] = a_row[t][(k0 >> 3) + (in ? blk : 0)];
+            if (!full) x[t] = in ? x[t] : u32x4{0u, 0u, 0u, 0u};
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int c = 0; c < kCB; c++)
+#pragma unroll
+            for (int c4 = 0; c4 < 4; c4++) {
+                const bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(MRK_LDS_PTR(bf16x4, rd[c4] + c * kBlockBytes));
+                const bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(MRK_LDS_PTR(bf16x4, rd[c4] + c * kBlockBytes + 4 * 128));
+                u32x4 w = __builtin_bit_cast(u32x4, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                if (!full) w = in ? w : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+                for (int t = 0; t < kMT; t++) {
+                    f32x4& d = acc[c * 4 + c4][t];
+                    if constexpr (kF16) d = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, w), __builtin_bit_cast(f16x8, x[t]), d, 0, 0, 0);
+                    else d = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, w), __builtin_bit_cast(bf16x8, x[t]), d, 0, 0, 0);
+                }
+            }
+    }
+    __syncthreads();
+    f32x4* partial = reinterpret_cast<f32x4*>(smem);  // [kWaves][kTiles][64]
+#pragma unroll
+    for (int c = 0; c < kCB * 4; c++)
+#pragma unroll
+        for (int t = 0; t < kMT; t++) partial[(wave * kTiles + c * kMT + t) * 64 + lane] = acc[c][t];
+    __syncthreads();
+    for (int e = threadIdx.x; e < kTiles * 64; e += kWaves * 64) {
+        const int tile = e >> 6, l = e & 63;
+        f32x4 s = partial[tile * 64 + l];
+#pragma unroll
+        for (int w = 1; w < kWaves; w++) s += partial[(w * kTiles + tile) * 64 + l];
+        const int c = tile / kMT, m = (tile % kMT) * 16 + (l & 15);
+        const long n = n0 + c * 16 + 4 * (l >> 4);
+        if (m >= M || n >= N) continue;  // N is a multiple of 8: a lane's four columns are all inside or all outside
+        if (W) {
+            *reinterpret_cast<f32x4*>(W + ((size_t)blockIdx.y * M + m) * N + n) = s;
+        } else {
+            unsigned short o[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if constexpr (kF16) o[i] = __builtin_bit_cast(unsigned short, (_Float16)s[i]);
+                else o[i] = round_bf16(s[i]);
+            }
+            *reinterpret_cast<u32x2*>(C + (size_t)m * N + n) = u32x2{(unsigned)o[0] | ((unsigned)o[1] << 16), (unsigned)o[2] | ((unsigned)o[3] << 16)};
+        }
+    }
+}
+
+
 // C[i] = round(W[0][i] + W[1][i] + ... + W[splits - 1][i]) for the partial sums above, which come in many
 // more slices than the tiled kernels' split-K leaves (up to 128): a workgroup folds 64 outputs, 32
 // work-items per group of eight outputs each taking every 32nd slice, then one of them adds the 32
@@ -436,6 +574,24 @@ __global__ __launch_bounds__(256) void gemm_kn_skinny_reduce(const float* __rest
                     (unsigned)o[6] | ((unsigned)o[7] << 16)};
         *reinterpret_cast<u32x4*>(C + i) = pk;
     }
+}
+
+
+// C[i] = round(W[0][i] + ... + W[splits - 1][i]) for the few ranges gemm_kn_rows leaves (at most a few dozen):
+// a work-item adds its four outputs' partial sums in the order of the ranges.
+template <bool kF16>
+__global__ __launch_bounds__(256) void gemm_kn_rows_reduce(const float* __restrict__ W, unsigned short* __restrict__ C, long total, int splits) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= total) return;
+    f32x4 s = *reinterpret_cast<const f32x4*>(W + i);
+    for (int k = 1; k < splits; k++) s += *reinterpret_cast<const f32x4*>(W + (size_t)k * total + i);
+    unsigned short o[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        if constexpr (kF16) o[j] = __builtin_bit_cast(unsigned short, (_Float16)s[j]);
+        else o[j] = round_bf16(s[j]);
+    }
+    *reinterpret_cast<u32x2*>(C + i) = u32x2{(unsigned)o[0] | ((unsigned)o[1] << 16), (unsigned)o[2] | ((unsigned)o[3] << 16)};
 }
 
 }  // namespace mrk::dev
@@ -534,15 +690,15 @@ int launch_gemm_nt_rows(void* stream, const void* A, const void* Bt, void* C, lo
     return (int)hipGetLastError();
 }
 
-// Plan of the [K, N] form for one or two rows: K split into `splits` groups of `rows_per_group` rows
+// Plan of the [K, N] form for one row on the vector ALUs: K split into `splits` groups of `rows_per_group` rows
 // (a multiple of 32), enough of them to fill the chip with workgroups of 512 columns, few enough
 // that the f32 partial sums stay a small part of the weight's bytes (and within 32 MiB).
 bool gemm_kn_skinny_plan(long M, long N, long K, long batch, long* splits, long* rows_per_group) {
-    // One or two rows, up to 24576 columns: measured against split-K over the tiled kernels, 9.3 against 12.5 us at
-    // 1 x 4096 x 4096, 18.8 against 20.1 at N = 12288, 34 against 39 at N = 22016, 18.3 against 21.8 at 4096 x 11008;
-    // with 32000 columns (46.6 against 42.9 us) and with four or eight rows (the partial sums' traffic and the
-    // workgroups' LDS footprint grow with the rows) the tiles win.  The kernel itself takes up to eight rows.
-    if (M < 1 || M > 2 || batch != 1 || N < 8 || N > 24576 || N % 8 || K < 256 || K % 8 || K > 0x7fffffffL) return false;
+    // One row, up to 24576 columns: measured against split-K over the tiled kernels, 9.3 against 12.5 us at
+    // 1 x 4096 x 4096, 18.8 against 20.1 at N = 12288, 34 against 39 at N = 22016, 18.3 against 21.8 at 4096 x 11008
+    // (with 32000 columns 46.6 against 42.9 us).  Two and more rows, and one row against wider weights, take the
+    // matrix-pipe kernel (gemm_kn_rows_plan), which measured faster from two rows on.
+    if (M != 1 || batch != 1 || N < 8 || N > 24576 || N % 8 || K < 256 || K % 8 || K > 0x7fffffffL) return false;
     const long col_groups = (N + 511) / 512;
     long want = (2048 + col_groups - 1) / col_groups;
     const long by_traffic = K / (16 * M) > 0 ? K / (16 * M) : 1;          // 2 * S * M * N * 4 <= K * N * 2 / 4
@@ -575,15 +731,66 @@ int launch_gemm_kn_skinny(void* stream, const void* A, const void* B, void* C, v
         if (f16) gemm_kn_skinny_partial<KM, true><<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)rows_per_group);  \
         else gemm_kn_skinny_partial<KM, false><<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)rows_per_group);     \
     } while (0)
-    if (M == 1) MRK_KN(1);
-    else if (M == 2) MRK_KN(2);
-    else if (M <= 4) MRK_KN(4);
-    else MRK_KN(8);
+    MRK_KN(1);
 #undef MRK_KN
     const long total = M * N;  // (a multiple of 8)
     const unsigned blocks = (unsigned)((total + 63) / 64);
     if (f16) gemm_kn_skinny_reduce<true><<<blocks, 256, 0, s>>>(w, static_cast<unsigned short*>(C), total, (int)splits);
     else gemm_kn_skinny_reduce<false><<<blocks, 256, 0, s>>>(w, static_cast<unsigned short*>(C), total, (int)splits);
+    return (int)hipGetLastError();
+}
+
+
+// Plan of the [K, N] form for up to 16 rows (one row: where gemm_kn_skinny_plan does not take it), and up to 64 rows against a weight of at most 4096 columns and 8192 rows,
+// where the tiled kernels have the fewest tiles to spread (gemm_kn_rows): column groups of 128 (64 for a narrow weight),
+// K split into enough ranges (multiples of 32 rows) for about one workgroup per CU, few enough that the f32 partial sums
+// stay a small part of the weight's bytes.  splits == 1: one launch, no scratch.
+bool gemm_kn_rows_plan(long M, long N, long K, long batch, long* splits, long* k_per_split) {
+    if (M < 1 || M > 64 || batch != 1 || N < 8 || N % 8 || N > (1L << 24) || K < 256 || K % 8 || K > (1L << 23)) return false;
+    if (M > 16 && (N > 4096 || K > 8192)) return false;
+    const long groups = N >= 8192 ? (N + 127) / 128 : (N + 63) / 64;
+    long want = 256 / groups;
+    const long by_traffic = K / (16 * M), by_rows = K / 256;
+    want = want < by_traffic ? want : by_traffic;
+    want = want < by_rows ? want : by_rows;
+    if (want < 1) want = 1;
+    const long per = ((K + want - 1) / want + 31) / 32 * 32;
+    const long s = (K + per - 1) / per;
+    if (s > 65535 || s * M * N * 4 > (32L << 20)) return false;
+    *splits = s;
+    *k_per_split = per;
+    return true;
+}
+
+int launch_gemm_kn_rows(void* stream, const void* A, const void* B, void* C, void* W, long M, long N, long K, long splits, long k_per_split,
+                        bool f16) {
+    using namespace mrk::dev;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(C)) % 16)
+        return (int)hipErrorInvalidValue;
+    if (splits > 1 && !W) return (int)hipErrorInvalidValue;
+    (void)hipGetLastError();
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned short* a = static_cast<const unsigned short*>(A);
+    const unsigned short* b = static_cast<const unsigned short*>(B);
+    unsigned short* c = static_cast<unsigned short*>(C);
+    float* w = splits > 1 ? static_cast<float*>(W) : nullptr;
+#define MRK_KN_ROWS(MT, CB)                                                                                              \
+    do {                                                                                                                 \
+        const dim3 grid((unsigned)((N + 64 * CB - 1) / (64 * CB)), (unsigned)splits);                                    \
+        if (f16) gemm_kn_rows<MT, CB, true><<<grid, 512, 0, s>>>(a, b, c, w, (int)M, (int)N, (int)K, (int)k_per_split);   \
+        else gemm_kn_rows<MT, CB, false><<<grid, 512, 0, s>>>(a, b, c, w, (int)M, (int)N, (int)K, (int)k_per_split);      \
+    } while (0)
+    if (M > 32) MRK_KN_ROWS(4, 1);
+    else if (M > 16) MRK_KN_ROWS(2, 1);
+    else if (N >= 8192) MRK_KN_ROWS(1, 2);
+    else MRK_KN_ROWS(1, 1);
+#undef MRK_KN_ROWS
+    if (splits > 1) {
+        const long total = M * N;  // (a multiple of 8)
+        const unsigned blocks = (unsigned)((total / 4 + 255) / 256);
+        if (f16) gemm_kn_rows_reduce<true><<<blocks, 256, 0, s>>>(w, c, total, (int)splits);
+        else gemm_kn_rows_reduce<false><<<blocks, 256, 0, s>>>(w, c, total, (int)splits);
+    }
     return (int)hipGetLastError();
 }
 

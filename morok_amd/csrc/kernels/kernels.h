@@ -41,13 +41,20 @@ int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, 
 // launch, no scratch memory.  K a multiple of 8 (at most 2^23), any N.
 bool gemm_nt_rows_supported(long M, long N, long K, long batch);
 int launch_gemm_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16);
-// The [K, N] form for one or two rows (N <= 24576 and K multiples of 8, K >= 256, one product): the weight is
+// The [K, N] form for one row (N <= 24576 and K multiples of 8, K >= 256, one product): the weight is
 // streamed once into `splits` f32 partial results W[splits][M][N], which a second kernel adds up in a
 // fixed order and rounds into C; gemm_kn_skinny_plan chooses the split and tells whether the shape is
 // taken this way.  gemm_bf16_workspace_bytes reports splits * M * N * 4 for such shapes.
 bool gemm_kn_skinny_plan(long M, long N, long K, long batch, long* splits, long* rows_per_group);
 int launch_gemm_kn_skinny(void* stream, const void* A, const void* B, void* C, void* W, long M, long N, long K, long splits, long rows_per_group,
                           bool f16);
+// The [K, N] form for up to 16 rows (up to 64 against a weight of at most 4096 columns and 8192 rows) on the matrix
+// pipes (weight blocks through LDS and the transposing read), with the
+// same split into f32 partial sums W[splits][M][N] and the same second kernel; with splits == 1 one launch writes C
+// and W is not used.  N and K multiples of 8, K >= 256, one product.
+bool gemm_kn_rows_plan(long M, long N, long K, long batch, long* splits, long* k_per_split);
+int launch_gemm_kn_rows(void* stream, const void* A, const void* B, void* C, void* W, long M, long N, long K, long splits, long k_per_split,
+                        bool f16);
 // c = bf16(float(bf16(a b)) + float(r)) with r of c's shape, added in the product kernel's epilogue
 // (same bits as the product followed by an elementwise add).  Supported for the shapes the tiled
 // kernels take without split-K; gemm_bf16_residual_supported tells.

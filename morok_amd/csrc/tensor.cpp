@@ -1412,7 +1412,8 @@ struct Scheduler {
     // epilogues would hold such a product on the few workgroups its tiles make (measured at 4 x 22016 x 4096 with
     // the gate: 70 us against 30 us for the streamed product plus an elementwise kernel), so they are not matched.
     bool spread_or_streamed(const TensorNode* mm, int64_t M, int64_t N, int64_t K, int64_t batch) const {
-        if (gemm_bf16_workspace_bytes(M, N, K, batch)) return true;
+        long splits = 0, per = 0;
+        if (gemm_bf16_workspace_bytes(M, N, K, batch) || gemm_kn_rows_plan(M, N, K, batch, &splits, &per)) return true;
         return transposed_weight(mm) && (gemm_nt_skinny_supported(M, N, K, batch) || gemm_nt_rows_supported(M, N, K, batch));
     }
     // x + (a @ w) in bf16 where nothing else reads the product: the product kernel adds x in its
@@ -1647,7 +1648,7 @@ struct Scheduler {
         if (mm->hint_inputs[0]->shape.size() != 2 || mm->hint_inputs[1]->shape.size() != 2 || transposed_weight(mm)) return nullptr;
         const int64_t M = mm->shape[0], N = mm->shape[1], K = mm->hint_inputs[0]->shape[1], split = sl->shape[1];
         if (sl->shape[0] != M || sl->arg.size() != 2 || sl->arg[0] != 0 || sl->arg[1] != 0) return nullptr;
-        if (x->shape[0] * S != M || x->shape[2] * 128 != split || !gemm_bf16_rope_supported(M, N, K, split, S) || gemm_bf16_workspace_bytes(M, N, K, 1))
+        if (x->shape[0] * S != M || x->shape[2] * 128 != split || !gemm_bf16_rope_supported(M, N, K, split, S) || spread_or_streamed(mm, M, N, K, 1))
             return nullptr;
         // the product's readers: this slice and, when there are columns left, exactly the slice of all of them
         auto readers = matmul_readers.find(mm);

@@ -29,6 +29,11 @@ int launch_gemm_nt_rows(void* stream, const void*, const void*, void*, long, lon
     return 0;
 }
 bool gemm_kn_skinny_plan(long, long, long, long, long*, long*) { return false; }
+bool gemm_kn_rows_plan(long, long, long, long, long*, long*) { return false; }
+int launch_gemm_kn_rows(void* stream, const void*, const void*, void*, void*, long, long, long, long, long, bool) {
+    mrk_shim_note_launch(stream, "gemm_bf16");
+    return 0;
+}
 int launch_gemm_kn_skinny(void* stream, const void*, const void*, void*, void*, long, long, long, long, long, bool) {
     mrk_shim_note_launch(stream, "gemm_bf16");
     return 0;

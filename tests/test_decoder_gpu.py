@@ -76,8 +76,7 @@ def test_decoder_block_few_tokens(dev, oracle, cfg):
     assert rel_err(got, ref) <= 2e-2
     assert sum(k.startswith("gemm_bf16") for k in kernels) == 4
     assert sum(k.startswith("flash_fwd") for k in kernels) == 1
-    if cfg["hidden"] == 4096:
-        assert all(k.endswith("_splitk") for k in kernels if k.startswith("gemm_bf16")), kernels
+    assert not any(tag in k for k in kernels for tag in ("swiglu", "residual", "rope")), kernels
 
 
 def test_decoder_block_full_size_properties(dev):

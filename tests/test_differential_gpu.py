@@ -127,5 +127,5 @@ def test_generated_tensor_core_direct_copy_random_choices(dev, seed):
     got = bc.copyout(np.uint16, (M * N + 512,))
     assert np.all(got[M * N:] == NAN)
     bh = dev.buffer(M * N * 2)
-    ops.gemm_bf16(ba, bb, bh, M, N, K, dev.device_id)
+    ops.gemm_bf16(ba, bb, bh, M, N, K, dev.device_id, 4)       # the tiled kernel (a handful of rows would otherwise be streamed)
     assert np.array_equal(got[:M * N].reshape(M, N), bh.copyout(np.uint16, (M, N))), (tc, opts, (M, N, K))

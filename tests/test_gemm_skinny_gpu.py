@@ -148,13 +148,13 @@ def test_linear_decode_step_is_one_kernel(T, oracle):
 
 
 # ---------------------------------------------------------------- the same rows against a weight stored [K, N]
-KN_SHAPES = [(1, 4096, 4096), (2, 520, 1024), (1, 264, 4104), (2, 12288, 4096), (1, 1024, 256), (2, 256, 11008), (1, 4104, 520),
-             (2, 8, 4096), (1, 2048, 2048), (2, 24576, 512)]
+KN_SHAPES = [(1, 4096, 4096), (1, 520, 1024), (1, 264, 4104), (1, 12288, 4096), (1, 1024, 256), (1, 256, 11008), (1, 4104, 520),
+             (1, 8, 4096), (1, 2048, 2048), (1, 24576, 512)]
 
 
 @pytest.mark.parametrize("shape", KN_SHAPES)
 def test_skinny_kn_form_vs_oracle_and_tiled_kernel(dev, oracle, shape):
-    """One or two rows through mrk_hip_gemm_bf16 ([K, N] weight): one streaming pass into f32 partial sums
+    """One row through mrk_hip_gemm_bf16 ([K, N] weight): one streaming pass on the vector ALUs into f32 partial sums
     plus their sum.  Against the oracle, against the tiled kernel (another summation order), the
     same bits on every run, through the ABI (allocator scratch) and as a plan item with a scratch buffer;
     NaNs right behind the operands and the result show that nothing reads or writes past them."""
@@ -191,6 +191,53 @@ def test_skinny_kn_form_vs_oracle_and_tiled_kernel(dev, oracle, shape):
     assert np.all(np.isnan(bw.copyout(np.float32)[ws // 4:]))     # the partial sums stay inside the scratch asked for
 
 
+ROWS_KN_SHAPES = [(3, 4096, 4096), (16, 12288, 4096), (8, 520, 1024), (5, 264, 4104), (16, 22016, 512), (12, 8, 4096),
+                  (16, 32000, 256), (4, 1024, 264), (7, 8200, 2056), (9, 4096, 11008), (16, 72, 296),
+                  # two rows; one row against more than 24576 columns; 17 to 64 rows against a narrow weight
+                  (2, 520, 1024), (2, 12288, 4096), (2, 256, 11008), (2, 8, 4096), (2, 24576, 512), (1, 32000, 1024),
+                  (17, 4096, 4096), (33, 1032, 8192), (48, 264, 2056), (64, 4096, 4096), (40, 4096, 296)]
+
+
+@pytest.mark.parametrize("shape", ROWS_KN_SHAPES)
+def test_rows_kn_form_vs_oracle_and_tiled_kernel(dev, oracle, shape):
+    """2 to 16 rows (to 64 against a narrow weight) through mrk_hip_gemm_bf16 ([K, N] weight): the weight streamed once through LDS and the
+    transposing read onto the matrix pipes, f32 partial sums per K range plus their sum (or one launch when one
+    range is enough).  Against the oracle, against the tiled kernel (another summation order), the same bits
+    on every run, through the ABI and as a plan item; NaNs right behind the operands, the result and the scratch."""
+    from morok_amd._ffi import lib
+
+    M, N, K = shape
+    ws = lib.mrk_hip_gemm_bf16_workspace_bytes(M, N, K, 1)
+    assert ws % (M * N * 4) == 0 and ws <= 32 << 20
+    a = synth.normal_bf16((M, K), 13, 14)
+    b = synth.normal_bf16((K, N), 13, 15)
+    pad = np.full(4096, 0x7FC0, np.uint16)
+    ba = morok_amd.Buffer.from_numpy(np.concatenate([a.reshape(-1), pad]), dev.device_id)
+    bb = morok_amd.Buffer.from_numpy(np.concatenate([b.reshape(-1), pad]), dev.device_id)
+    bc = dev.buffer((M * N + 2048) * 2)
+    bc.copyin(np.full(M * N + 2048, 0x7FC0, np.uint16))
+    ops.gemm_bf16(ba, bb, bc, M, N, K, dev.device_id)
+    out = bc.copyout(np.uint16)
+    assert np.all(out[M * N:] == 0x7FC0)
+    got = out[: M * N].reshape(M, N)
+    _check(synth.from_bf16(got), synth.from_bf16(oracle.gemm_bf16(a, b)), K, 2**-7)
+    bc2 = dev.buffer(M * N * 2)
+    ops.gemm_bf16(ba, bb, bc2, M, N, K, dev.device_id, 4)          # the tiled kernel, unsplit
+    tiled = synth.from_bf16(bc2.copyout(np.uint16, (M, N)))
+    g = synth.from_bf16(got)
+    assert np.all(np.abs(g - tiled) <= np.abs(tiled) * 2**-7 + 2e-5 * np.sqrt(K) * max(np.abs(tiled).max() / np.sqrt(K), 1.0))
+    ops.gemm_bf16(ba, bb, bc2, M, N, K, dev.device_id)
+    assert np.array_equal(bc2.copyout(np.uint16, (M, N)), got)
+    if ws:
+        bw = dev.buffer(ws + 4096)
+        bw.copyin(np.full((ws + 4096) // 4, np.nan, np.float32))
+        morok_amd.Program.builtin("gemm_bf16", [M, N, K, 1, ws], dev.device_id).execute([bc2, ba, bb, bw])
+        assert np.all(np.isnan(bw.copyout(np.float32)[ws // 4:]))     # the partial sums stay inside the scratch asked for
+    else:
+        morok_amd.Program.builtin("gemm_bf16", [M, N, K], dev.device_id).execute([bc2, ba, bb])
+    assert np.array_equal(bc2.copyout(np.uint16, (M, N)), got)
+
+
 def test_skinny_kn_form_f16_and_exact(dev, oracle):
     M, N, K = 4, 1032, 2048
     a = synth.normal((M, K), 13, 10).astype(np.float16)
@@ -200,9 +247,9 @@ def test_skinny_kn_form_f16_and_exact(dev, oracle):
     ops.gemm_f16(ba, bb, bc, M, N, K, dev.device_id)
     got = bc.copyout(np.uint16, (M, N)).view(np.float16).astype(np.float32)
     _check(got, oracle.gemm_f16(a, b).astype(np.float32), K, 2**-10)
-    # small integers: every sum is exact in f32 whatever the order (one or two rows stream, more take the tiles)
+    # small integers: every sum is exact in f32 whatever the order (up to 16 rows stream, more take the tiles)
     rng = np.random.default_rng(6)
-    for M in range(1, 9):
+    for M in list(range(1, 18)) + [33]:
         N, K = 520 + 8 * M, 1288
         ai = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
         bi = rng.integers(-4, 5, size=(K, N)).astype(np.float32)
@@ -215,7 +262,7 @@ def test_skinny_kn_form_f16_and_exact(dev, oracle):
 
 def test_matmul_decode_step_kn_weight(T, oracle):
     """x [M, K] @ w [K, N] through Tensor.matmul for a handful of rows: one plan item with scratch placed by
-    the plan (one row: the streaming pair of kernels; eight: split-K over the tiles)."""
+    the plan (the streaming kernels: one row on the vector ALUs, eight on the matrix pipes; K split over the chip)."""
     from morok_amd import uop
 
     T.set_fusion(True)
