@@ -431,9 +431,10 @@ int mrk_hip_softmax_f32_variant(int device_id, const void* x, void* y, int64_t r
  * K % 64 == 0 take the LDS-tiled kernel. */
 int mrk_hip_gemm_bf16(int device_id, const void* a, const void* b, void* c, int64_t m, int64_t n, int64_t k);
 /* Bytes of f32 scratch with which the product of this shape is spread over the chip along K
- * (few output tiles, long K: a handful of rows against a weight matrix; one or two rows stream
- * the weight into more, smaller partial sums than the tiled kernels); 0 when the shape has
- * enough tiles by itself.  mrk_hip_gemm_bf16 takes that scratch from the device allocator by
+ * (few output tiles, long K: a handful of rows against a weight matrix; up to 16 rows, and up to
+ * 64 against a weight of at most 4096 columns, stream the weight once into partial sums instead
+ * of running the tiled kernels); 0 when the shape has enough tiles by itself or one streaming
+ * launch does.  mrk_hip_gemm_bf16 takes that scratch from the device allocator by
  * itself; a "gemm_bf16" builtin Program takes it as its fourth buffer. */
 size_t mrk_hip_gemm_bf16_workspace_bytes(int64_t m, int64_t n, int64_t k, int64_t batch);
 /* c[M,N] = a[M,K] * bt[N,K]^T: the product with the second operand as it is stored by a Linear
