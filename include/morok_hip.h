@@ -198,8 +198,9 @@ void mrk_hip_program_destroy(mrk_program* p);
  *                     params = {M, N, K, batch, workspace bytes}    buffers = {c, a, b, workspace}
  *                     (split-K for shapes with few output tiles; size from mrk_hip_gemm_bf16_workspace_bytes)
  *   "gemm_bf16_residual"  params = {M, N, K} or {M, N, K, batch}  buffers = {c, a, b, r}   (c = a b + r)
+ *   "gemm_bf16_bias"      params = {M, N, K} or {M, N, K, batch}  buffers = {c, a, b, bias} (c = a b + bias, bias [N])
  *   "gemm_bf16_swiglu"    params = {M, F, K}                      buffers = {c, a, w}      (w = gate | up, [K, 2F])
- *   "gemm_bf16_nt", "gemm_bf16_nt_residual", "gemm_bf16_nt_swiglu": the same three with the second operand
+ *   "gemm_bf16_nt", "gemm_bf16_nt_residual", "gemm_bf16_nt_bias", "gemm_bf16_nt_swiglu": the same with the second operand
  *                     stored transposed, [N, K] ([2F, K], gate rows first), as a Linear layer holds its
  *                     weight (tensor/src/nn/linear.rs:9-14: y = x @ weight.T + bias); the same bits as
  *                     the [K, N] kinds.  No split-K form: shapes with a workspace size > 0 are refused.
@@ -485,6 +486,15 @@ size_t mrk_hip_gemm_bf16_noalloc_capacity(void);
  * multiple of 8, K = 0, or so few output tiles that split-K is used). */
 int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, const void* r, void* c, int64_t m, int64_t n,
                                int64_t k);
+/* y[M, N] = x[M, K] * w[N, K]^T + bias[N]: a Linear layer's forward pass on its parameters as it stores them
+ * (tensor/src/nn/linear.rs:9-14 weight [out_features, in_features] and bias [out_features]; :39-41
+ * x.linear(weight, bias) = x @ weight.T + bias), bf16 operands and result, f32 accumulation.  The bias is added in
+ * the product kernel's epilogue: y = bf16(float(bf16(x w^T)) + float(bias)), the bits of the product followed by
+ * the elementwise add.  bias may be NULL (the plain product, mrk_hip_gemm_bf16_nt).  Shapes as for
+ * mrk_hip_gemm_bf16_nt; up to 64 rows run the streaming kernels, more rows the tiled kernels (a shape that the plain
+ * product would spread along K runs unsplit here, on the workgroups its tiles make).  Builtin Program kinds
+ * "gemm_bf16_nt_bias" and, for a weight stored [K, N], "gemm_bf16_bias" ({M, N, K[, batch]}, buffers {y, x, w, bias}). */
+int mrk_hip_linear_bf16(int device_id, const void* x, const void* w, const void* bias, void* y, int64_t m, int64_t n, int64_t k);
 
 /* Gated-MLP pair of products: c[M, F] = bf16(silu(float(bf16(a wg))) * float(bf16(a wu))) with
  * w = [wg | wu] stored side by side as one row-major [K, 2F] matrix: what

@@ -154,6 +154,7 @@ _SIGS = {
                                             C.c_int64, C.c_int]),
     "mrk_hip_gemm_bf16_residual": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
                                              C.c_int64]),
+    "mrk_hip_linear_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64]),
     "mrk_hip_gemm_bf16_rope": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,
                                          C.c_int64, C.c_int64, C.c_int64, C.c_int64]),
     "mrk_hip_flash_attn_fwd_bf16": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64,

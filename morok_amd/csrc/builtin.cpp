@@ -159,6 +159,22 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
+    if (k == "gemm_bf16_bias" || k == "gemm_bf16_nt_bias") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, b, bias [N]}
+        const bool nt = k == "gemm_bf16_nt_bias";
+        if (nparams != 3 && nparams != 4)
+            return failf(kInvalidArgument, "builtin '%s' takes 3 or 4 parameters, got %zu", k.c_str(), nparams);
+        if (p.size() < 4) p.push_back(1);
+        if (!gemm_bf16_bias_launchable(p[0], p[1], p[2], p[3], nt))
+            return fail(kInvalidArgument, k + ": shape not covered (N and K multiples of 8, or up to 64 rows against an [N, K] operand with K a "
+                                              "multiple of 8)");
+        std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
+        if (p[3] > 1) name += "_x" + std::to_string(p[3]);
+        out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
+                                      [nt](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16_bias(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3], nt);
+                                      }));
+        return kOk;
+    }
     if (k == "gemm_bf16_residual" || k == "gemm_bf16_nt_residual") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, b, r}
         const bool nt = k == "gemm_bf16_nt_residual";
         if (nparams < 3 || nparams > 4)

@@ -988,6 +988,23 @@ int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, cons
     return kOk;
 }
 
+int mrk_hip_linear_bf16(int device_id, const void* x, const void* w, const void* bias, void* y, int64_t m, int64_t n, int64_t k) {
+    if (!bias) return mrk_hip_gemm_bf16_nt(device_id, x, w, y, m, n, k);
+    if (m < 0 || n < 0 || k < 0) return fail(kInvalidArgument, "linear_bf16: negative shape");
+    if (m == 0 || n == 0) return kOk;
+    MRK_NONNULL(x);
+    MRK_NONNULL(w);
+    MRK_NONNULL(y);
+    if (!gemm_bf16_nt_supported(m, n, k, 1))
+        return fail(kInvalidArgument, "linear_bf16: shape not covered (in_features a multiple of 8 and > 0; at most 64 rows, or "
+                                      "out_features a multiple of 8)");
+    std::shared_ptr<Device> dv;
+    MRK_TRY(get_device(device_id, &dv));
+    MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
+    MRK_HIP(launch_gemm_bf16_bias(dv->allocator->stream(), x, w, bias, y, m, n, k, 1, true), "linear_bf16 launch");
+    return kOk;
+}
+
 int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
                                 int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal) {
     if (batch < 0 || heads < 0 || sq < 0 || sk < 0) return fail(kInvalidArgument, "flash_attn_fwd: negative shape");

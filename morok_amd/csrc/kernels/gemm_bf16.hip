@@ -146,7 +146,8 @@ template <bool kRaggedK, int kJ, bool kSplitK = false, bool kResidual = false, b
 __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
                                                float* __restrict__ W = nullptr, int kt_per_split = 0,
-                                               const __bf16* __restrict__ R = nullptr, const RopeEpilogue& rope = RopeEpilogue{}) {
+                                               const __bf16* __restrict__ R = nullptr, const RopeEpilogue& rope = RopeEpilogue{},
+                                               int ldr = -1) {
     static_assert(!kF16 || (!kResidual && !kSwiGLU && !kRope), "the fused epilogues exist for bf16 only");
     static_assert(!kRope || (kJ == 4 && !kSplitK && !kResidual && !kSwiGLU), "the rotary epilogue exists for the plain 256-row tile only");
     constexpr int kTM = kJ == 4 ? 256 : 128;      // rows of the workgroup tile
@@ -167,7 +168,9 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     A += (size_t)blockIdx.y * M * K;
     B += (size_t)blockIdx.y * K * N;
     if (!kSplitK) C += (size_t)blockIdx.y * M * N;
-    if (kResidual) R += (size_t)blockIdx.y * M * N;
+    // row pitch of R in elements: N for a matrix of C's shape, 0 for one row added to every row of C (a bias)
+    const size_t r_pitch = ldr < 0 ? (size_t)N : (size_t)ldr;
+    if (kResidual) R += (size_t)blockIdx.y * M * r_pitch;
     int tile_m, tile_n;
     tile_of_block(blockIdx.x, tiles_m, tiles_n, &tile_m, &tile_n);
     static_assert(!kSwiGLU || (kJ == 4 && !kSplitK && !kResidual), "the gated epilogue exists for the 256-row tile only");
@@ -555,11 +558,11 @@ __device__ __forceinline__ void gemm_tile_body(const __bf16* __restrict__ A, con
     const bool col_ok = col0 + lc * 8 + 8 <= (size_t)N;
     u32x4 res[kResidual ? kIts : 1];
     auto fetch_residual = [&](int first, int last) {
-        const __bf16* Rl = R + (row0 + lr) * N + col0 + lc * 8;
+        const __bf16* Rl = R + (row0 + lr) * r_pitch + col0 + lc * 8;
 #pragma unroll
         for (int it = first; it < last; it++) {
             res[it] = u32x4{0u, 0u, 0u, 0u};
-            if (col_ok && it * kRowsPerIt + lr < rows_here) res[it] = *reinterpret_cast<const u32x4*>(Rl + (size_t)(it * kRowsPerIt) * N);
+            if (col_ok && it * kRowsPerIt + lr < rows_here) res[it] = *reinterpret_cast<const u32x4*>(Rl + (size_t)(it * kRowsPerIt) * r_pitch);
         }
     };
     {
@@ -734,8 +737,8 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256(const __bf16* __restric
 #define MRK_GEMM_NT_RESIDUAL_KERNEL(name, ...)                                                                          \
     __global__ __launch_bounds__(256) void name(const __bf16* __restrict__ A, const __bf16* __restrict__ Bt,           \
                                                 const __bf16* __restrict__ R, __bf16* __restrict__ C, int M, int N,    \
-                                                int K, int tiles_m, int tiles_n) {                                     \
-        gemm_tile_body<__VA_ARGS__>(A, Bt, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);                                \
+                                                int K, int tiles_m, int tiles_n, int ldr) {                            \
+        gemm_tile_body<__VA_ARGS__>(A, Bt, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R, RopeEpilogue{}, ldr);           \
     }
 MRK_GEMM_NT_KERNEL(gemm_bf16_nt_tile256, false, 4, false, false, false, true)
 MRK_GEMM_NT_KERNEL(gemm_bf16_nt_tile256_ragged_k, true, 4, false, false, false, true)
@@ -791,14 +794,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256_ragged_k(const __bf16* 
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_residual(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                                   const __bf16* __restrict__ R, __bf16* __restrict__ C, int M,
-                                                                  int N, int K, int tiles_m, int tiles_n) {
-    gemm_tile_body<false, 4, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);
+                                                                  int N, int K, int tiles_m, int tiles_n, int ldr) {
+    gemm_tile_body<false, 4, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R, RopeEpilogue{}, ldr);
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_residual_ragged_k(const __bf16* __restrict__ A,
                                                                            const __bf16* __restrict__ B,
                                                                            const __bf16* __restrict__ R, __bf16* __restrict__ C,
-                                                                           int M, int N, int K, int tiles_m, int tiles_n) {
-    gemm_tile_body<true, 4, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);
+                                                                           int M, int N, int K, int tiles_m, int tiles_n, int ldr) {
+    gemm_tile_body<true, 4, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R, RopeEpilogue{}, ldr);
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_swiglu(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                                 __bf16* __restrict__ C, int M, int N2, int K, int tiles_m,
@@ -812,14 +815,14 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256_swiglu_ragged_k(const _
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile128_residual(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                                   const __bf16* __restrict__ R, __bf16* __restrict__ C, int M,
-                                                                  int N, int K, int tiles_m, int tiles_n) {
-    gemm_tile_body<false, 2, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);
+                                                                  int N, int K, int tiles_m, int tiles_n, int ldr) {
+    gemm_tile_body<false, 2, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R, RopeEpilogue{}, ldr);
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile128_residual_ragged_k(const __bf16* __restrict__ A,
                                                                            const __bf16* __restrict__ B,
                                                                            const __bf16* __restrict__ R, __bf16* __restrict__ C,
-                                                                           int M, int N, int K, int tiles_m, int tiles_n) {
-    gemm_tile_body<true, 2, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R);
+                                                                           int M, int N, int K, int tiles_m, int tiles_n, int ldr) {
+    gemm_tile_body<true, 2, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, R, RopeEpilogue{}, ldr);
 }
 __global__ __launch_bounds__(256) void gemm_bf16_tile128(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
                                                          __bf16* __restrict__ C, int M, int N, int K, int tiles_m,
@@ -1010,10 +1013,11 @@ size_t gemm_bf16_nt_workspace_bytes(long M, long N, long K, long batch) {
 }
 
 int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch,
-                              bool b_transposed) {
+                              bool b_transposed, bool r_is_row) {
     using namespace mrk::dev;
     if (M <= 0 || N <= 0 || batch <= 0) return 0;
-    if (!gemm_bf16_residual_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
+    // every shape the tiled kernels address; gemm_bf16_residual_supported is narrower (it leaves out what split-K runs faster)
+    if (!tiled_shape(M, N, K, batch)) return (int)hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(R)) % 16)
         return (int)hipErrorInvalidValue;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1031,8 +1035,29 @@ int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const 
                                         : (ragged_k ? gemm_bf16_nt_tile256_residual_ragged_k : gemm_bf16_nt_tile256_residual))
                                : (small ? (ragged_k ? gemm_bf16_tile128_residual_ragged_k : gemm_bf16_tile128_residual)
                                         : (ragged_k ? gemm_bf16_tile256_residual_ragged_k : gemm_bf16_tile256_residual));
-    kernel<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
+    kernel<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn, r_is_row ? 0 : -1);
     return (int)hipGetLastError();
+}
+
+bool gemm_bf16_bias_supported(long M, long N, long K, long batch, bool b_transposed) {
+    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return false;
+    if (b_transposed && gemm_nt_bias_streamed(M, N, K, batch)) return true;
+    long ks = 0, kr = 0;
+    if (!b_transposed && (gemm_kn_skinny_plan(M, N, K, batch, &ks, &kr) || gemm_kn_rows_plan(M, N, K, batch, &ks, &kr))) return false;
+    return gemm_bf16_residual_supported(M, N, K, batch);
+}
+
+bool gemm_bf16_bias_launchable(long M, long N, long K, long batch, bool b_transposed) {
+    return (b_transposed && gemm_nt_bias_streamed(M, N, K, batch)) || tiled_shape(M, N, K, batch);
+}
+
+int launch_gemm_bf16_bias(void* stream, const void* a, const void* b, const void* bias, void* c, long M, long N, long K, long batch,
+                          bool b_transposed) {
+    if (M <= 0 || N <= 0 || batch <= 0) return 0;
+    if (!bias) return (int)hipErrorInvalidValue;
+    if (b_transposed && gemm_nt_bias_streamed(M, N, K, batch)) return launch_gemm_nt_bias_streamed(stream, a, b, bias, c, M, N, K, false);
+    // (a shape outside gemm_bf16_bias_supported that the tiled kernels address still runs here, on the workgroups its tiles make)
+    return launch_gemm_bf16_residual(stream, a, b, bias, c, M, N, K, batch, b_transposed, true);
 }
 
 bool gemm_bf16_swiglu_supported(long M, long F, long K, bool b_transposed) {

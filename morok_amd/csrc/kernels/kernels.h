@@ -57,10 +57,23 @@ int launch_gemm_kn_rows(void* stream, const void* A, const void* B, void* C, voi
                         bool f16);
 // c = bf16(float(bf16(a b)) + float(r)) with r of c's shape, added in the product kernel's epilogue
 // (same bits as the product followed by an elementwise add).  Supported for the shapes the tiled
-// kernels take without split-K; gemm_bf16_residual_supported tells.
+// kernels take without split-K; gemm_bf16_residual_supported tells.  r_is_row: r is one row [N] added to every row
+// of c (a Linear layer's bias, tensor/src/nn/linear.rs:39-41) instead of a matrix of c's shape.
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch);
 int launch_gemm_bf16_residual(void* stream, const void* a, const void* b, const void* r, void* c, long M, long N, long K, long batch,
-                              bool b_transposed = false);
+                              bool b_transposed = false, bool r_is_row = false);
+// y[M, N] = bf16(float(bf16(x wt^T)) + float(bias)) with wt [N, K] and bias [N] as a Linear layer holds them, for the
+// shapes the streaming kernels take (up to 64 rows, K a multiple of 8, one product): the bias is added where the
+// kernel writes its result.  Same bits as the product followed by the add.
+// The product with a bias row, whichever kernel takes the shape: the streaming kernels (second operand [N, K], up to 64
+// rows) or the tiled kernels' residual epilogue with a row pitch of zero.  gemm_bf16_bias_supported tells; shapes that
+// would be spread along K ([K, N] with few rows, more than 64 rows with few tiles) are not covered.
+bool gemm_bf16_bias_supported(long M, long N, long K, long batch, bool b_transposed);
+bool gemm_bf16_bias_launchable(long M, long N, long K, long batch, bool b_transposed);  // every shape launch_gemm_bf16_bias runs
+int launch_gemm_bf16_bias(void* stream, const void* a, const void* b, const void* bias, void* c, long M, long N, long K, long batch,
+                          bool b_transposed);
+bool gemm_nt_bias_streamed(long M, long N, long K, long batch);
+int launch_gemm_nt_bias_streamed(void* stream, const void* A, const void* Bt, const void* bias, void* C, long M, long N, long K, bool f16);
 // C[M, F] = bf16(silu(float(bf16(A Wg))) * float(bf16(A Wu))) for W = [Wg | Wu] stored side by side as
 // one [K, 2F] matrix: the gated-MLP pair of products with the gate applied in the product kernel's
 // epilogue, so that the [M, 2F] product never reaches memory.  F and K multiples of 8.

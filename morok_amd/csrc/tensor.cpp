@@ -1419,7 +1419,8 @@ struct Scheduler {
     // x + (a @ w) in bf16 where nothing else reads the product: the product kernel adds x in its
     // epilogue (same bits as the product followed by the add).  Returns the product node and the
     // other operand.
-    TensorNode* residual_matmul(TensorNode* n, TensorNode** other) const {
+    TensorNode* residual_matmul(TensorNode* n, TensorNode** other, bool* is_row = nullptr) const {
+        if (is_row) *is_row = false;
         if (!g_fusion || n->kind != TKind::Binary || static_cast<BinaryOp>(n->sub) != BinaryOp::Add || n->dtype != Scalar::BFloat16 ||
             n->numel() == 0 || n->src.size() != 2)
             return nullptr;
@@ -1430,13 +1431,25 @@ struct Scheduler {
             auto u = uses.find(mm);
             if (u == uses.end() || u->second != 1) continue;
             if (r->dtype != Scalar::BFloat16 || r->shape != n->shape || mm->shape != n->shape) continue;
-            // only an operand that is in memory anyway: a lazy expression (a broadcast bias, x * 2)
+            int64_t M, N, K, batch;
+            matmul_extents(mm, &M, &N, &K, &batch);
+            // a bias (x @ w + b, tensor/src/nn/linear.rs:39-41): one row [N] that is in memory, broadcast over the
+            // rows (reshape to [1, .., 1, N], expand); the kernel adds it with a row pitch of zero
+            // (with a single row the expand is the identity and there is no such node)
+            if (!r->buffer && (r->kind == TKind::Expand || (M * batch == 1 && r->kind == TKind::Reshape))) {
+                TensorNode* b = r->kind == TKind::Expand ? r->src[0].get() : r;
+                while (!b->buffer && b->kind == TKind::Reshape) b = b->src[0].get();
+                if (!b->buffer || b->dtype != Scalar::BFloat16 || b->numel() != N || n->shape.back() != N || b->buffer->offset() % 16) continue;
+                if (!gemm_bf16_bias_supported(M, N, K, batch, transposed_weight(mm) != nullptr)) continue;
+                *other = b;
+                if (is_row) *is_row = true;
+                return mm;
+            }
+            // only an operand that is in memory anyway: a lazy expression (x * 2)
             // is cheaper evaluated inside the add than written out first
             const TensorNode* rb = r;
             while (!rb->buffer && rb->kind == TKind::Reshape) rb = rb->src[0].get();
             if (!(rb->buffer || is_boundary_kind(rb) || fusable(rb))) continue;
-            int64_t M, N, K, batch;
-            matmul_extents(mm, &M, &N, &K, &batch);
             if (!gemm_bf16_residual_supported(M, N, K, batch) || spread_or_streamed(mm, M, N, K, batch)) continue;
             *other = r;
             return mm;
@@ -1532,7 +1545,7 @@ struct Scheduler {
         *batch = 1;
         for (size_t i = 0; i + 2 < a->shape.size(); i++) (w->shape.size() == 2 ? *M : *batch) *= a->shape[i];
     }
-    int materialize_residual_matmul(TensorNode* n, TensorNode* mm, TensorNode* r) {
+    int materialize_residual_matmul(TensorNode* n, TensorNode* mm, TensorNode* r, bool is_row) {
         int64_t M, N, K, batch;
         matmul_extents(mm, &M, &N, &K, &batch);
         MRK_TRY(materialize(mm->hint_inputs[0].get()));
@@ -1542,7 +1555,8 @@ struct Scheduler {
         MRK_TRY(materialize(r));
         auto out = new_buffer(n);
         const std::vector<int64_t> params = batch == 1 ? std::vector<int64_t>{M, N, K} : std::vector<int64_t>{M, N, K, batch};
-        MRK_TRY(builtin(nt ? "gemm_bf16_nt_residual" : "gemm_bf16_residual", params, {out, mm->hint_inputs[0]->buffer, wbuf, r->buffer}));
+        const std::string kind = std::string(nt ? "gemm_bf16_nt_" : "gemm_bf16_") + (is_row ? "bias" : "residual");
+        MRK_TRY(builtin(kind.c_str(), params, {out, mm->hint_inputs[0]->buffer, wbuf, r->buffer}));
         n->buffer = out;
         produced.push_back(n);
         return kOk;
@@ -1697,7 +1711,8 @@ struct Scheduler {
         if (n->numel() > 0 && fusable(n)) return materialize_fused(n);
         {
             TensorNode* other = nullptr;
-            if (TensorNode* mm = residual_matmul(n, &other)) return materialize_residual_matmul(n, mm, other);
+            bool is_row = false;
+            if (TensorNode* mm = residual_matmul(n, &other, &is_row)) return materialize_residual_matmul(n, mm, other, is_row);
             if (TensorNode* mm = swiglu_matmul(n)) return materialize_swiglu_matmul(n, mm);
             int64_t split = 0, seq = 0;
             if (TensorNode* mm = rope_matmul(n, &other, &split, &seq)) return materialize_rope_matmul(n, mm, other, split, seq);

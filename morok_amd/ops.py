@@ -78,6 +78,17 @@ def gemm_bf16_swiglu(a, w, c, m, f, k, device_id=0):
     check(lib.mrk_hip_gemm_bf16_swiglu(device_id, _p(a), _p(w), _p(c), m, f, k))
 
 
+def linear_bf16(x, w, bias, y, m, n, k, device_id=0):
+    """y[m, n] = x[m, k] @ w[n, k].T + bias[n] with the weight and bias as a Linear layer stores them; bias may be
+    None.  The bias is added in the product kernel's epilogue (the bits of the product followed by the add)."""
+    _need(x, m * k * 2, "linear_bf16 x")
+    _need(w, n * k * 2, "linear_bf16 w")
+    _need(y, m * n * 2, "linear_bf16 y")
+    if bias is not None:
+        _need(bias, n * 2, "linear_bf16 bias")
+    check(lib.mrk_hip_linear_bf16(device_id, _p(x), _p(w), _p(bias) if bias is not None else None, _p(y), m, n, k))
+
+
 def gemm_bf16_residual(a, b, r, c, m, n, k, device_id=0):
     """c[m,n] = a[m,k] @ b[k,n] + r[m,n]: the residual added in the product kernel's epilogue,
     same bits as gemm_bf16 followed by an elementwise add."""

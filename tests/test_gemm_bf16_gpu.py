@@ -357,6 +357,70 @@ def test_gemm_transposed_second_operand_split_k(dev, oracle, shape):
     assert np.array_equal(bc2.copyout(np.uint16, (M, N)), got)
 
 
+LINEAR_SHAPES = [(256, 256, 64), (512, 768, 256), (300, 520, 128), (1000, 776, 320), (2048, 512, 136),   # tiled kernels
+                 (1, 4096, 4096), (2, 1020, 64), (5, 37, 520), (16, 4096, 1024), (33, 515, 264), (64, 12288, 512)]  # streamed
+
+
+@pytest.mark.parametrize("shape", LINEAR_SHAPES)
+def test_linear_forward_with_bias(dev, oracle, shape):
+    """y = x @ w.T + bias with w [out, in] and bias [out] as nn::Linear holds them (tensor/src/nn/linear.rs:9-14,
+    39-41), the bias added in the product kernel's epilogue: the bits of the product (same kernel family, no bias)
+    followed by the elementwise add in bf16, within the GEMM tolerance of the oracle; NaNs right behind every
+    operand and the result; bias = None is the plain product."""
+    M, N, K = shape
+    x = synth.normal_bf16((M, K), 3, 40)
+    w = synth.normal_bf16((N, K), 3, 41)
+    bias = synth.normal_bf16((N,), 3, 42)
+    nan = np.full(8192, 0x7FC0, np.uint16)
+    bx = morok_amd.Buffer.from_numpy(np.concatenate([x.reshape(-1), nan]), dev.device_id)
+    bw = morok_amd.Buffer.from_numpy(np.concatenate([w.reshape(-1), nan]), dev.device_id)
+    bb = morok_amd.Buffer.from_numpy(np.concatenate([bias, nan]), dev.device_id)
+    by = dev.buffer(M * N * 2 + 4096)
+    by.copyin(np.full(M * N + 2048, 0x7FC0, np.uint16))
+    ops.linear_bf16(bx, bw, bb, by, M, N, K, dev.device_id)
+    out = by.copyout(np.uint16)
+    got = out[: M * N].reshape(M, N)
+    assert np.all(out[M * N:] == 0x7FC0)
+    bp = dev.buffer(M * N * 2)
+    ops.linear_bf16(bx, bw, None, bp, M, N, K, dev.device_id)
+    prod = bp.copyout(np.uint16, (M, N))
+    bp2 = dev.buffer(M * N * 2)
+    ops.gemm_bf16_nt(bx, bw, bp2, M, N, K, dev.device_id)
+    assert np.array_equal(prod, bp2.copyout(np.uint16, (M, N)))
+    want = synth.to_bf16(synth.from_bf16(prod) + synth.from_bf16(bias)[None, :])
+    assert np.array_equal(got, want)
+    ref = synth.from_bf16(oracle.gemm_bf16(x, np.ascontiguousarray(w.T))) + synth.from_bf16(bias)[None, :]
+    assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
+    # as plan items, for either layout of the weight
+    by2 = dev.buffer(M * N * 2)
+    morok_amd.Program.builtin("gemm_bf16_nt_bias", [M, N, K], dev.device_id).execute([by2, bx, bw, bb])
+    assert np.array_equal(by2.copyout(np.uint16, (M, N)), got)
+    if N % 8 == 0:
+        bwt = morok_amd.Buffer.from_numpy(np.ascontiguousarray(w.T), dev.device_id)
+        morok_amd.Program.builtin("gemm_bf16_bias", [M, N, K], dev.device_id).execute([by2, bx, bwt, bb])
+        kn = synth.from_bf16(by2.copyout(np.uint16, (M, N)))
+        if M > 64:
+            assert np.array_equal(by2.copyout(np.uint16, (M, N)), got)      # the tiled kernels: the same bits in either layout
+        else:
+            assert np.abs(kn - ref).max() <= 2e-2 * np.abs(ref).max()
+
+
+def test_linear_forward_with_bias_few_tiles_and_refusals(dev, oracle):
+    """More than 64 rows with few output tiles against a long K (the plain product would be spread along K): the
+    bias form runs unsplit; K not a multiple of 8 is refused."""
+    M, N, K = 100, 264, 4104
+    x, w, bias = synth.normal_bf16((M, K), 3, 43), synth.normal_bf16((N, K), 3, 44), synth.normal_bf16((N,), 3, 45)
+    bx, bw, bb = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (x, w, bias))
+    by = dev.buffer(M * N * 2)
+    ops.linear_bf16(bx, bw, bb, by, M, N, K, dev.device_id)
+    ref = synth.from_bf16(oracle.gemm_bf16(x, np.ascontiguousarray(w.T))) + synth.from_bf16(bias)[None, :]
+    assert np.abs(synth.from_bf16(by.copyout(np.uint16, (M, N))) - ref).max() <= 2e-2 * np.abs(ref).max()
+    with pytest.raises(morok_amd.MorokHipError):
+        ops.linear_bf16(bx, bw, bb, by, M, N, 4100, dev.device_id)
+    with pytest.raises(morok_amd.MorokHipError):
+        ops.linear_bf16(bx, bw, bb, by, M, 260, K, dev.device_id)       # more than 64 rows and N not a multiple of 8
+
+
 @pytest.mark.parametrize("shape", [(256, 256, 64), (512, 768, 1024), (300, 264, 200), (1000, 520, 72)])
 def test_gemm_transposed_second_operand_epilogues(dev, shape):
     """The residual and the gated epilogue over a [N, K] ([2F, K]) second operand, as plan items:

@@ -480,9 +480,15 @@ def test_linear_layout_weights_are_read_in_place(T, shim):
     x, w = bf((512, 256)), bf((768, 256))
     y = x.linear(w)
     assert y.shape == (512, 768) and y.realize().kernels() == ["gemm_bf16_nt_512_768_256"]
-    # the same through an explicit transpose, and with a bias (added by a kernel of its own)
+    # the same through an explicit transpose, and with a bias (added in the product kernel's epilogue; a bias that
+    # is an expression, or a product with a second reader, is added by a kernel of its own)
     assert x.matmul(w.try_transpose(0, 1)).realize().kernels() == ["gemm_bf16_nt_512_768_256"]
-    names = x.linear(w, bf((768,))).realize().kernels()
+    assert x.linear(w, bf((768,))).realize().kernels() == ["gemm_bf16_nt_bias_512_768_256"]
+    assert x.matmul(bf((256, 768))).try_add(bf((768,))).realize().kernels() == ["gemm_bf16_bias_512_768_256"]
+    names = x.linear(w, bf((768,)).try_mul(2.0).cast(uop.BF16)).realize().kernels()
+    assert names[0] == "gemm_bf16_nt_512_768_256" and len(names) == 2
+    p = x.linear(w)
+    names = p.try_add(bf((768,))).try_mul(p).realize().kernels()
     assert names[0] == "gemm_bf16_nt_512_768_256" and len(names) == 2
     # residual epilogue
     h = bf((512, 768))

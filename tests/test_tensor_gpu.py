@@ -1038,6 +1038,23 @@ def test_linear_reads_the_weight_as_stored(T, oracle):
         assert np.array_equal(got_r, synth.to_bf16(synth.from_bf16(got) + synth.from_bf16(h)))
 
 
+def test_linear_with_bias_is_one_kernel(T, oracle):
+    """x.linear(w, bias) in bf16 with the parameters in memory (tensor/src/nn/linear.rs:39-41): one product kernel
+    that adds the bias in its epilogue, for a prefill-sized and a decode-sized x; the bits of the unfused graph."""
+    from morok_amd import synth, uop
+
+    for (M, K, N) in ((300, 200, 264), (8, 1024, 520), (1, 512, 4100)):
+        x, w, b = synth.normal_bf16((M, K), 9, 21), synth.normal_bf16((N, K), 9, 22), synth.normal_bf16((N,), 9, 23)
+        T.set_fusion(True)
+        y = T.Tensor.from_numpy(x, uop.BF16).linear(T.Tensor.from_numpy(w, uop.BF16), T.Tensor.from_numpy(b, uop.BF16))
+        got = y.to_numpy()
+        assert y.kernels() == [f"gemm_bf16_nt_bias_{M}_{N}_{K}"]
+        ref = synth.from_bf16(oracle.gemm_bf16(x, np.ascontiguousarray(w.T))) + synth.from_bf16(b)[None, :]
+        assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
+        p = T.Tensor.from_numpy(x, uop.BF16).linear(T.Tensor.from_numpy(w, uop.BF16)).to_numpy()
+        assert np.array_equal(got, synth.to_bf16(synth.from_bf16(p) + synth.from_bf16(b)[None, :]))
+
+
 def test_matmul_bf16_residual_add_is_fused(T):
     """x + a @ w in bf16 with no other reader of the product: one kernel (the product kernel
     with the residual epilogue), on either side of the add and through contiguous(); the same
