@@ -180,8 +180,9 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
         if (nparams < 3 || nparams > 4)
             return failf(kInvalidArgument, "builtin '%s' takes 3 or 4 parameters, got %zu", k.c_str(), nparams);
         while (p.size() < 4) p.push_back(1);
-        if (!gemm_bf16_residual_supported(p[0], p[1], p[2], p[3]))
-            return failf(kInvalidArgument, "%s: shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel)", k.c_str());
+        if (!gemm_bf16_residual_supported(p[0], p[1], p[2], p[3]) && !(nt && gemm_nt_bias_streamed(p[0], p[1], p[2], p[3])))
+            return failf(kInvalidArgument, "%s: shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel%s)", k.c_str(),
+                         nt ? "; or up to 64 rows with K a multiple of 8" : "");
         std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
         if (p[3] > 1) name += "_x" + std::to_string(p[3]);
         out->reset(new BuiltinProgram(device_id, stream, name, 4, p,

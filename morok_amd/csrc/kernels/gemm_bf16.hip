@@ -1016,6 +1016,9 @@ int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const 
                               bool b_transposed, bool r_is_row) {
     using namespace mrk::dev;
     if (M <= 0 || N <= 0 || batch <= 0) return 0;
+    // a handful of rows against an [N, K] weight: the streaming kernels add R where they write their result
+    if (b_transposed && gemm_nt_bias_streamed(M, N, K, batch))
+        return launch_gemm_nt_bias_streamed(stream, A, B, R, C, M, N, K, false, r_is_row);
     // every shape the tiled kernels address; gemm_bf16_residual_supported is narrower (it leaves out what split-K runs faster)
     if (!tiled_shape(M, N, K, batch)) return (int)hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(R)) % 16)

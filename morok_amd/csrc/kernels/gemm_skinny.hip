@@ -40,17 +40,18 @@ __device__ __forceinline__ unsigned short round_bf16(float f) {
     u += 0x7fffu + ((u >> 16) & 1u);
     return (unsigned short)(u >> 16);
 }
-// The element a kernel writes: the sum rounded to the result's type; with a bias (one element per column, of the
-// result's type) that rounded value plus the bias, rounded again (the bits of the product followed by the add).
+// The element a kernel writes: the sum rounded to the result's type; with an addend (a bias row or a matrix of the
+// result's shape, of the result's type) that rounded value plus the addend, rounded again (the bits of the product
+// followed by the add).  `add` points at the addend's row, or is null.
 template <bool kF16>
-__device__ __forceinline__ unsigned short round_out(float s, const unsigned short* bias, long n) {
+__device__ __forceinline__ unsigned short round_out(float s, const unsigned short* add, long n) {
     if constexpr (kF16) {
         _Float16 h = (_Float16)s;
-        if (bias) h = (_Float16)((float)h + (float)__builtin_bit_cast(_Float16, bias[n]));
+        if (add) h = (_Float16)((float)h + (float)__builtin_bit_cast(_Float16, add[n]));
         return __builtin_bit_cast(unsigned short, h);
     } else {
         unsigned short h = round_bf16(s);
-        if (bias) h = round_bf16(__builtin_bit_cast(float, (unsigned)h << 16) + __builtin_bit_cast(float, (unsigned)bias[n] << 16));
+        if (add) h = round_bf16(__builtin_bit_cast(float, (unsigned)h << 16) + __builtin_bit_cast(float, (unsigned)add[n] << 16));
         return h;
     }
 }
@@ -84,7 +85,7 @@ __device__ __forceinline__ void fold_lanes(float* acc, int lane) {
 template <int kM, int kRowsPerGroup, bool kF16>
 __global__ __launch_bounds__(256) void gemm_nt_skinny(const unsigned short* __restrict__ A, const unsigned short* __restrict__ Bt,
                                                        unsigned short* __restrict__ C, int M, int N, int K,
-                                                       const unsigned short* __restrict__ bias) {
+                                                       const unsigned short* __restrict__ add, long add_pitch) {
     constexpr int kV = kM * kRowsPerGroup;  // values a lane accumulates
     __shared__ float partial[4][kV];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(256) void gemm_nt_skinny(const unsigned short* __re
         const float s = ((partial[0][lane] + partial[1][lane]) + partial[2][lane]) + partial[3][lane];
         const int m = lane / kRowsPerGroup, r = lane % kRowsPerGroup;
         if (m < M && n0 + r < N) {
-            C[(size_t)m * N + n0 + r] = round_out<kF16>(s, bias, n0 + r);
+            C[(size_t)m * N + n0 + r] = round_out<kF16>(s, add ? add + (size_t)m * add_pitch : nullptr, n0 + r);
         }
     }
 }
@@ -185,7 +186,7 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 template <int kMT, int kRT, int kWaves, bool kF16>
 __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short* __restrict__ A, const unsigned short* __restrict__ Bt,
                                                              unsigned short* __restrict__ C, int M, int N, int K,
-                                                             const unsigned short* __restrict__ bias) {
+                                                             const unsigned short* __restrict__ add, long add_pitch) {
     constexpr int kSteps = 2;                      // 32-deep matrix steps per chunk
     constexpr int kPieces = 4 * kSteps;            // 16-byte pieces of a row per chunk
     constexpr int kRowsPerCopy = 64 / kPieces;     // rows one copy instruction covers
@@ -307,7 +308,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
         if (m >= M || n >= N) continue;
         unsigned short o[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) o[i] = round_out<kF16>(s[i], n + i < N ? bias : nullptr, n + i);
+        for (int i = 0; i < 4; i++) o[i] = round_out<kF16>(s[i], add && n + i < N ? add + (size_t)m * add_pitch : nullptr, n + i);
         unsigned short* dst = C + (size_t)m * N + n;
         if (vec) {
             *reinterpret_cast<u32x2*>(dst) = u32x2{(unsigned)o[0] | ((unsigned)o[1] << 16), (unsigned)o[2] | ((unsigned)o[3] << 16)};
@@ -613,9 +614,11 @@ bool gemm_nt_skinny_supported(long M, long N, long K, long batch) {
 }
 
 namespace {
-int launch_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16, const void* bias) {
+int launch_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16, const void* add,
+                     long add_pitch) {
     using namespace mrk::dev;
-    const unsigned short* bs = static_cast<const unsigned short*>(bias);
+    const unsigned short* bs = static_cast<const unsigned short*>(add);
+    const long bp = add_pitch;
     if (!gemm_nt_skinny_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) % 16 || reinterpret_cast<uintptr_t>(C) % 2) return (int)hipErrorInvalidValue;
     (void)hipGetLastError();
@@ -628,8 +631,8 @@ int launch_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long 
 #define MRK_SKINNY(KM, KR)                                                                                  \
     do {                                                                                                    \
         const dim3 grid((unsigned)((N + KR - 1) / KR), (unsigned)batch);                                    \
-        if (f16) gemm_nt_skinny<KM, KR, true><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, bs);    \
-        else gemm_nt_skinny<KM, KR, false><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, bs);       \
+        if (f16) gemm_nt_skinny<KM, KR, true><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, bs, bp); \
+        else gemm_nt_skinny<KM, KR, false><<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, bs, bp);    \
     } while (0)
     if (M == 1) MRK_SKINNY(1, 2);
     else MRK_SKINNY(2, 4);
@@ -639,7 +642,7 @@ int launch_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long 
 }  // namespace
 
 int launch_gemm_nt_skinny(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16) {
-    return launch_nt_skinny(stream, A, Bt, C, M, N, K, batch, f16, nullptr);
+    return launch_nt_skinny(stream, A, Bt, C, M, N, K, batch, f16, nullptr, 0);
 }
 
 // 3 to 64 rows on the matrix pipes (gemm_nt_rows).  Byte offsets inside a workgroup's rows are 32-bit.
@@ -669,9 +672,11 @@ int rows_blocks_per_group(long N, int mt) {
 }  // namespace
 
 namespace {
-int launch_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16, const void* bias) {
+int launch_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16, const void* add,
+                   long add_pitch) {
     using namespace mrk::dev;
-    const unsigned short* bs = static_cast<const unsigned short*>(bias);
+    const unsigned short* bs = static_cast<const unsigned short*>(add);
+    const long bp = add_pitch;
     if (!gemm_nt_rows_supported(M, N, K, batch)) return (int)hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) % 16 || reinterpret_cast<uintptr_t>(C) % 8) return (int)hipErrorInvalidValue;
     (void)hipGetLastError();
@@ -684,8 +689,8 @@ int launch_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M,
 #define MRK_ROWS(MT, RT, WV)                                                                              \
     do {                                                                                                  \
         const dim3 grid((unsigned)((N + 16 * RT - 1) / (16 * RT)), (unsigned)batch);                      \
-        if (f16) gemm_nt_rows<MT, RT, WV, true><<<grid, WV * 64, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, bs); \
-        else gemm_nt_rows<MT, RT, WV, false><<<grid, WV * 64, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, bs);    \
+        if (f16) gemm_nt_rows<MT, RT, WV, true><<<grid, WV * 64, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, bs, bp); \
+        else gemm_nt_rows<MT, RT, WV, false><<<grid, WV * 64, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, bs, bp); \
     } while (0)
 #define MRK_ROWS_UP_TO_4(MT)                  \
     do {                                      \
@@ -711,17 +716,19 @@ int launch_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M,
 }  // namespace
 
 int launch_gemm_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16) {
-    return launch_nt_rows(stream, A, Bt, C, M, N, K, batch, f16, nullptr);
+    return launch_nt_rows(stream, A, Bt, C, M, N, K, batch, f16, nullptr, 0);
 }
 
 bool gemm_nt_bias_streamed(long M, long N, long K, long batch) {
     return batch == 1 && (gemm_nt_skinny_supported(M, N, K, 1) || gemm_nt_rows_supported(M, N, K, 1));
 }
 
-int launch_gemm_nt_bias_streamed(void* stream, const void* A, const void* Bt, const void* bias, void* C, long M, long N, long K, bool f16) {
-    if (!bias || reinterpret_cast<uintptr_t>(bias) % 2) return (int)hipErrorInvalidValue;
-    if (gemm_nt_skinny_supported(M, N, K, 1)) return launch_nt_skinny(stream, A, Bt, C, M, N, K, 1, f16, bias);
-    return launch_nt_rows(stream, A, Bt, C, M, N, K, 1, f16, bias);
+int launch_gemm_nt_bias_streamed(void* stream, const void* A, const void* Bt, const void* add, void* C, long M, long N, long K, bool f16,
+                                 bool add_is_row) {
+    if (!add || reinterpret_cast<uintptr_t>(add) % 2) return (int)hipErrorInvalidValue;
+    const long pitch = add_is_row ? 0 : N;
+    if (gemm_nt_skinny_supported(M, N, K, 1)) return launch_nt_skinny(stream, A, Bt, C, M, N, K, 1, f16, add, pitch);
+    return launch_nt_rows(stream, A, Bt, C, M, N, K, 1, f16, add, pitch);
 }
 
 // Plan of the [K, N] form for one row on the vector ALUs: K split into `splits` groups of `rows_per_group` rows

@@ -62,18 +62,20 @@ int launch_gemm_kn_rows(void* stream, const void* A, const void* B, void* C, voi
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch);
 int launch_gemm_bf16_residual(void* stream, const void* a, const void* b, const void* r, void* c, long M, long N, long K, long batch,
                               bool b_transposed = false, bool r_is_row = false);
-// y[M, N] = bf16(float(bf16(x wt^T)) + float(bias)) with wt [N, K] and bias [N] as a Linear layer holds them, for the
-// shapes the streaming kernels take (up to 64 rows, K a multiple of 8, one product): the bias is added where the
-// kernel writes its result.  Same bits as the product followed by the add.
 // The product with a bias row, whichever kernel takes the shape: the streaming kernels (second operand [N, K], up to 64
-// rows) or the tiled kernels' residual epilogue with a row pitch of zero.  gemm_bf16_bias_supported tells; shapes that
-// would be spread along K ([K, N] with few rows, more than 64 rows with few tiles) are not covered.
+// rows) or the tiled kernels' residual epilogue with a row pitch of zero.  gemm_bf16_bias_supported tells where that is
+// the fast route (shapes that would be spread along K are left out: [K, N] with few rows, more than 64 rows with few
+// tiles); gemm_bf16_bias_launchable every shape launch_gemm_bf16_bias runs.
 bool gemm_bf16_bias_supported(long M, long N, long K, long batch, bool b_transposed);
-bool gemm_bf16_bias_launchable(long M, long N, long K, long batch, bool b_transposed);  // every shape launch_gemm_bf16_bias runs
+bool gemm_bf16_bias_launchable(long M, long N, long K, long batch, bool b_transposed);
 int launch_gemm_bf16_bias(void* stream, const void* a, const void* b, const void* bias, void* c, long M, long N, long K, long batch,
                           bool b_transposed);
+// y[M, N] = bf16(float(bf16(x wt^T)) + float(add)) with wt [N, K] as a Linear layer holds it and `add` either one row
+// [N] (its bias) or a matrix [M, N] (a residual), for the shapes the streaming kernels take (up to 64 rows, K a
+// multiple of 8, one product): added where the kernel writes its result.  Same bits as the product followed by the add.
 bool gemm_nt_bias_streamed(long M, long N, long K, long batch);
-int launch_gemm_nt_bias_streamed(void* stream, const void* A, const void* Bt, const void* bias, void* C, long M, long N, long K, bool f16);
+int launch_gemm_nt_bias_streamed(void* stream, const void* A, const void* Bt, const void* add, void* C, long M, long N, long K, bool f16,
+                                 bool add_is_row = true);
 // C[M, F] = bf16(silu(float(bf16(A Wg))) * float(bf16(A Wu))) for W = [Wg | Wu] stored side by side as
 // one [K, 2F] matrix: the gated-MLP pair of products with the gate applied in the product kernel's
 // epilogue, so that the [M, 2F] product never reaches memory.  F and K multiples of 8.

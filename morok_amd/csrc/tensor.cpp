@@ -1450,7 +1450,9 @@ struct Scheduler {
             const TensorNode* rb = r;
             while (!rb->buffer && rb->kind == TKind::Reshape) rb = rb->src[0].get();
             if (!(rb->buffer || is_boundary_kind(rb) || fusable(rb))) continue;
-            if (!gemm_bf16_residual_supported(M, N, K, batch) || spread_or_streamed(mm, M, N, K, batch)) continue;
+            // (a handful of rows against an [N, K] weight: the streaming kernels add the operand where they write their result)
+            const bool streamed = transposed_weight(mm) && gemm_nt_bias_streamed(M, N, K, batch);
+            if (!streamed && (!gemm_bf16_residual_supported(M, N, K, batch) || spread_or_streamed(mm, M, N, K, batch))) continue;
             *other = r;
             return mm;
         }

@@ -120,6 +120,41 @@ def _batched(dev, oracle, M, N, K, B):
         _check(synth.from_bf16(got[i]), synth.from_bf16(ref), K, 2**-7)
 
 
+@pytest.mark.parametrize("shape", [(1, 4096, 4096), (2, 1020, 64), (5, 37, 520), (16, 4096, 1024), (33, 515, 264), (64, 12288, 512)])
+def test_streamed_residual_add(dev, shape):
+    """h + x @ w.T for a handful of rows, as the plan item the scheduler picks ("gemm_bf16_nt_residual"): the
+    streaming kernels add h where they write their result, with the bits of the product followed by the add."""
+    M, N, K = shape
+    x, w, h = synth.normal_bf16((M, K), 13, 30), synth.normal_bf16((N, K), 13, 31), synth.normal_bf16((M, N), 13, 32)
+    bx, bw, bh = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (x, w, h))
+    by = dev.buffer((M * N + 2048) * 2)
+    by.copyin(np.full(M * N + 2048, 0x7FC0, np.uint16))
+    morok_amd.Program.builtin("gemm_bf16_nt_residual", [M, N, K], dev.device_id).execute([by, bx, bw, bh])
+    out = by.copyout(np.uint16)
+    assert np.all(out[M * N:] == 0x7FC0)
+    bp = dev.buffer(M * N * 2)
+    ops.gemm_bf16_nt(bx, bw, bp, M, N, K, dev.device_id)
+    want = synth.to_bf16(synth.from_bf16(bp.copyout(np.uint16, (M, N))) + synth.from_bf16(h))
+    assert np.array_equal(out[: M * N].reshape(M, N), want)
+
+
+def test_linear_decode_with_residual_is_one_kernel(T, oracle):
+    """h + x.linear(w) over 8 rows: one streaming kernel (no elementwise kernel behind it), the bits of the unfused pair."""
+    from morok_amd import uop
+
+    M, K, N = 8, 1024, 3072
+    x, w, h = synth.normal_bf16((M, K), 13, 33), synth.normal_bf16((N, K), 13, 34), synth.normal_bf16((M, N), 13, 35)
+    tx, tw, th = (T.Tensor.from_numpy(t, uop.BF16) for t in (x, w, h))
+    T.set_fusion(True)
+    r = th.try_add(tx.linear(tw))
+    got = r.to_numpy()
+    assert r.kernels() == [f"gemm_bf16_nt_residual_{M}_{N}_{K}"]
+    p = tx.linear(tw).to_numpy()
+    assert np.array_equal(got, synth.to_bf16(synth.from_bf16(p) + synth.from_bf16(h)))
+    ref = synth.from_bf16(oracle.gemm_bf16(x, np.ascontiguousarray(w.T))) + synth.from_bf16(h)
+    assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
+
+
 def test_skinny_refusals(dev):
     a, b, c = dev.buffer(72 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(72 * 1024 * 2)
     with pytest.raises(morok_amd.MorokHipError):
