@@ -314,13 +314,14 @@ def test_matmul_decode_step_kn_weight(T, oracle):
 
 @pytest.mark.parametrize("seed", range(6))
 def test_skinny_random_shapes_exact(dev, seed):
-    """Random small shapes on small-integer data, where every sum is exact in f32 whatever its order: the
-    [N, K] form for 1-16 rows (any N, K a multiple of 8) and the [K, N] form for 1-8 rows (N, K multiples of 8)
-    must give the integer products exactly, whichever kernel the shape selects."""
+    """Random shapes on small-integer data, where every sum is exact in f32 whatever its order: the
+    [N, K] form for 1-64 rows (any N, K a multiple of 8; now and then with a bias row or a residual matrix of small
+    integers, whose sum with the product is exact as well) and the [K, N] form for 1-64 rows (N, K multiples of 8)
+    must give the integer results exactly, whichever kernel the shape selects."""
     rng = np.random.default_rng(7000 + seed)
-    for _ in range(12):
-        M = int(rng.integers(1, 17))
-        N = int(rng.integers(1, 700))
+    for it in range(12):
+        M = int(rng.integers(1, 65)) if it % 3 else int(rng.integers(1, 17))
+        N = int(rng.integers(1, 700)) if it % 4 else int(rng.integers(1, 400)) * 16 + int(rng.integers(0, 16))
         K = 8 * int(rng.integers(1, 300))
         a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
         bt = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
@@ -329,13 +330,20 @@ def test_skinny_random_shapes_exact(dev, seed):
         bc = dev.buffer(M * N * 2)
         morok_amd.Program.builtin("gemm_bf16_nt", [M, N, K], dev.device_id).execute([bc, ba, bb])
         assert np.array_equal(bc.copyout(np.uint16, (M, N)), want), (M, N, K)
-        if M <= 8:
-            N8 = 8 * int(rng.integers(1, 200))
-            K2 = 8 * int(rng.integers(32, 400))
-            a2 = rng.integers(-3, 4, size=(M, K2)).astype(np.float32)
-            b2 = rng.integers(-3, 4, size=(K2, N8)).astype(np.float32)
-            want2 = synth.to_bf16((a2.astype(np.int64) @ b2.astype(np.int64)).astype(np.float32))
-            ba2, bb2 = morok_amd.Buffer.from_numpy(synth.to_bf16(a2), dev.device_id), morok_amd.Buffer.from_numpy(synth.to_bf16(b2), dev.device_id)
-            bc2 = dev.buffer(M * N8 * 2)
-            ops.gemm_bf16(ba2, bb2, bc2, M, N8, K2, dev.device_id)
-            assert np.array_equal(bc2.copyout(np.uint16, (M, N8)), want2), (M, N8, K2)
+        if it % 2:
+            # |product| <= 9 K and the addend keep the sum an integer below 2^24; the result is rounded once more to bf16
+            row = bool(rng.integers(0, 2))
+            add = rng.integers(-3, 4, size=(N,) if row else (M, N)).astype(np.float32)
+            badd = morok_amd.Buffer.from_numpy(synth.to_bf16(add), dev.device_id)
+            morok_amd.Program.builtin("gemm_bf16_nt_bias" if row else "gemm_bf16_nt_residual", [M, N, K], dev.device_id).execute([bc, ba, bb, badd])
+            want_add = synth.to_bf16(synth.from_bf16(want) + add)
+            assert np.array_equal(bc.copyout(np.uint16, (M, N)), want_add), (M, N, K, row)
+        N8 = 8 * int(rng.integers(1, 200))
+        K2 = 8 * int(rng.integers(32, 400))
+        a2 = rng.integers(-3, 4, size=(M, K2)).astype(np.float32)
+        b2 = rng.integers(-3, 4, size=(K2, N8)).astype(np.float32)
+        want2 = synth.to_bf16((a2.astype(np.int64) @ b2.astype(np.int64)).astype(np.float32))
+        ba2, bb2 = morok_amd.Buffer.from_numpy(synth.to_bf16(a2), dev.device_id), morok_amd.Buffer.from_numpy(synth.to_bf16(b2), dev.device_id)
+        bc2 = dev.buffer(M * N8 * 2)
+        ops.gemm_bf16(ba2, bb2, bc2, M, N8, K2, dev.device_id)
+        assert np.array_equal(bc2.copyout(np.uint16, (M, N8)), want2), (M, N8, K2)
