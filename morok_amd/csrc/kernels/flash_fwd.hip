@@ -697,7 +697,8 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
         if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16) return (int)hipErrorInvalidValue;
         if (sr > (1L << 30) || !flash_fwd_rows_addressable(rows[t], sr * 2, D)) return (int)hipErrorInvalidValue;
         // the output must not alias itself: distinct rows, heads and batches at distinct places
-        if (t == 3 && (sr < D || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
+        // (the stride of an axis of extent one is never multiplied by anything but zero: any value will do)
+        if (t == 3 && ((Sq > 1 && sr < D) || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
         dense = dense && sr == D && sh == rows[t] * D && sb == H * rows[t] * D;
     }
     if (dense) return launch_flash_fwd_bf16(stream, q, k, v, o, BH, Sq, Sk, D, scale, causal);
@@ -740,7 +741,8 @@ int launch_flash_fwd_bf16_ext(void* stream, const void* q, const void* k, const 
         if (sb < 0 || sh < 0 || sr < 0 || sb % 8 || sh % 8 || sr % 8) return (int)hipErrorInvalidValue;
         if (reinterpret_cast<uintptr_t>(ptrs[t]) % 16) return (int)hipErrorInvalidValue;
         if (sr > (1L << 30) || !flash_fwd_rows_addressable(rows[t], sr * 2, D)) return (int)hipErrorInvalidValue;
-        if (t == 3 && (sr < D || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
+        // (the stride of an axis of extent one is never multiplied by anything but zero: any value will do)
+        if (t == 3 && ((Sq > 1 && sr < D) || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
     }
     FlashExt ext{};
     if (mask_kind != 0) {

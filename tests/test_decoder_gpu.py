@@ -59,7 +59,8 @@ def test_decoder_block_vs_oracle(dev, oracle, cfg):
 @pytest.mark.parametrize("cfg", [
     dict(batch=2, seq=8, hidden=4096, heads=32, ffn=11008, vocab=32000, eps=1e-6),
     dict(batch=1, seq=40, hidden=1024, heads=8, ffn=2816, vocab=500, eps=1e-6),
-], ids=["h4096_16tokens", "h1024_40tokens"])
+    dict(batch=5, seq=1, hidden=256, heads=2, ffn=512, vocab=300, eps=1e-6),      # one position per sequence: every stride of the sequence axis is moot
+], ids=["h4096_16tokens", "h1024_40tokens", "h256_seq1"])
 def test_decoder_block_few_tokens(dev, oracle, cfg):
     """A handful of tokens: every product has few output tiles against a long K, so it is spread along K (or
     streamed) instead of run as one pass of tiles, and the fused epilogues, which exist for the tiled
