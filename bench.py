@@ -629,7 +629,7 @@ WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash,
              "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling,
              "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16, "flash_options": bench_flash_options,
              "linear_decode": bench_linear_decode, "linear_decode_16": bench_linear_decode_16}
-PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc"]
+PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc", "linear_decode", "linear_decode_16"]
 
 
 def main():
