@@ -521,7 +521,8 @@ int mrk_hip_gemm_bf16_swiglu(int device_id, const void* a, const void* w, void* 
  * c_rest[M, N - split] (NULL when split == N).  The rotated product is never written and read
  * again in between.  K a multiple of 64, N of 8, cos / sin 32-byte aligned; INVALID_ARGUMENT
  * otherwise.  Builtin Program kind "gemm_bf16_rope", params {M, N, K, split, seq}, buffers
- * {c_rot, a, w, c_rest, cos, sin}.  The reference holds no value test of this composition: parity
+ * {c_rot, a, w, c_rest, cos, sin}; "gemm_bf16_nt_rope" is the same over a weight stored [N, K]
+ * (a Linear layer's), with the same bits.  The reference holds no value test of this composition: parity
  * unpinned by reference tests, pinned against the oracle's product followed by its rotary stage. */
 int mrk_hip_gemm_bf16_rope(int device_id, const void* a, const void* b, const void* cos, const void* sin, void* c_rot, void* c_rest,
                            int64_t m, int64_t n, int64_t k, int64_t split, int64_t seq);

@@ -203,16 +203,17 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
-    if (k == "gemm_bf16_rope") {
+    if (k == "gemm_bf16_rope" || k == "gemm_bf16_nt_rope") {
+        const bool nt = k == "gemm_bf16_nt_rope";  // (b stored [N, K])
         // {M, N, K, split, seq}; buffers {c_rot [M, split], a [M, K], b [K, N], c_rest [M, N - split], cos [seq, 64] f32, sin}:
         // the product with the rotary embedding of its first `split` columns (heads of 128) in the epilogue
         MRK_TRY(need(5));
         if (!gemm_bf16_rope_supported(p[0], p[1], p[2], p[3], p[4]))
-            return fail(kInvalidArgument, "gemm_bf16_rope: shape not covered (K a multiple of 64, N of 8, split a multiple of 256 within N, seq > 0)");
-        std::string name = "gemm_bf16_rope_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]) + "_s" + std::to_string(p[3]);
+            return fail(kInvalidArgument, k + ": shape not covered (K a multiple of 64, N of 8, split a multiple of 256 within N, seq > 0)");
+        std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]) + "_s" + std::to_string(p[3]);
         out->reset(new BuiltinProgram(device_id, stream, name, 6, p,
-                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
-                                          return launch_gemm_bf16_rope(s, b[1], b[2], b[0], b[3], q[0], q[1], q[2], q[3], b[4], b[5], q[4]);
+                                      [nt](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16_rope(s, b[1], b[2], b[0], b[3], q[0], q[1], q[2], q[3], b[4], b[5], q[4], nt);
                                       }));
         return kOk;
     }

@@ -787,6 +787,11 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile256_rope(const __bf16* __re
                                                               RopeEpilogue rope) {
     gemm_tile_body<false, 4, false, false, false, false, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, nullptr, rope);
 }
+__global__ __launch_bounds__(256) void gemm_bf16_nt_tile256_rope(const __bf16* __restrict__ A, const __bf16* __restrict__ B,
+                                                              __bf16* __restrict__ C, int M, int N, int K, int tiles_m, int tiles_n,
+                                                              RopeEpilogue rope) {
+    gemm_tile_body<false, 4, false, false, false, true, false, true>(A, B, C, M, N, K, tiles_m, tiles_n, nullptr, 0, nullptr, rope);
+}
 __global__ __launch_bounds__(256) void gemm_bf16_tile256_ragged_k(const __bf16* __restrict__ A,
                                                                   const __bf16* __restrict__ B, __bf16* __restrict__ C,
                                                                   int M, int N, int K, int tiles_m, int tiles_n) {
@@ -1098,7 +1103,7 @@ bool gemm_bf16_rope_supported(long M, long N, long K, long split, long seq) {
 }
 
 int launch_gemm_bf16_rope(void* stream, const void* A, const void* B, void* C_rot, void* C_rest, long M, long N, long K, long split,
-                          const void* cos, const void* sin, long seq) {
+                          const void* cos, const void* sin, long seq, bool b_transposed) {
     using namespace mrk::dev;
     if (!gemm_bf16_rope_supported(M, N, K, split, seq) || !A || !B || !C_rot || !cos || !sin || (split < N && !C_rest))
         return (int)hipErrorInvalidValue;
@@ -1108,7 +1113,8 @@ int launch_gemm_bf16_rope(void* stream, const void* A, const void* B, void* C_ro
     (void)hipGetLastError();
     const long tm = (M + kBM - 1) / kBM, tn = (N + kBN - 1) / kBN;
     RopeEpilogue rope{static_cast<const float*>(cos), static_cast<const float*>(sin), static_cast<__bf16*>(C_rest), (int)seq, (int)split};
-    gemm_bf16_tile256_rope<<<dim3((unsigned)(tm * tn)), 256, 0, static_cast<hipStream_t>(stream)>>>(
+    auto kernel = b_transposed ? gemm_bf16_nt_tile256_rope : gemm_bf16_tile256_rope;
+    kernel<<<dim3((unsigned)(tm * tn)), 256, 0, static_cast<hipStream_t>(stream)>>>(
         static_cast<const __bf16*>(A), static_cast<const __bf16*>(B), static_cast<__bf16*>(C_rot), (int)M, (int)N, (int)K, (int)tm, (int)tn, rope);
     return (int)hipGetLastError();
 }

@@ -90,7 +90,7 @@ int launch_gemm_bf16_swiglu(void* stream, const void* a, const void* w, void* c,
 // K a multiple of 64, N of 8.
 bool gemm_bf16_rope_supported(long M, long N, long K, long split, long seq);
 int launch_gemm_bf16_rope(void* stream, const void* a, const void* b, void* c_rot, void* c_rest, long M, long N, long K, long split,
-                          const void* cos, const void* sin, long seq);
+                          const void* cos, const void* sin, long seq, bool b_transposed = false);
 // Bytes of f32 scratch with which launch_gemm_bf16 spreads the K loop of this shape over the
 // chip (split-K: partial products per K range, added up in a fixed order by a second kernel);
 // 0 when the shape has enough output tiles by itself.  Without the workspace the same shape

@@ -1661,7 +1661,7 @@ struct Scheduler {
         if (sl->buffer || sl->kind != TKind::Shrink || !used_once(sl) || sl->shape.size() != 2) return nullptr;
         TensorNode* mm = sl->src[0].get();
         if (mm->buffer || mm->hint != HintKind::Matmul || !fusable(mm) || mm->dtype != Scalar::BFloat16 || mm->shape.size() != 2) return nullptr;
-        if (mm->hint_inputs[0]->shape.size() != 2 || mm->hint_inputs[1]->shape.size() != 2 || transposed_weight(mm)) return nullptr;
+        if (mm->hint_inputs[0]->shape.size() != 2 || mm->hint_inputs[1]->shape.size() != 2) return nullptr;
         const int64_t M = mm->shape[0], N = mm->shape[1], K = mm->hint_inputs[0]->shape[1], split = sl->shape[1];
         if (sl->shape[0] != M || sl->arg.size() != 2 || sl->arg[0] != 0 || sl->arg[1] != 0) return nullptr;
         if (x->shape[0] * S != M || x->shape[2] * 128 != split || !gemm_bf16_rope_supported(M, N, K, split, S) || spread_or_streamed(mm, M, N, K, 1))
@@ -1692,12 +1692,15 @@ struct Scheduler {
         int64_t M, N, K, batch;
         matmul_extents(mm, &M, &N, &K, &batch);
         MRK_TRY(materialize(mm->hint_inputs[0].get()));
-        MRK_TRY(materialize(mm->hint_inputs[1].get()));
-        const std::shared_ptr<Buffer>&a = mm->hint_inputs[0]->buffer, &w = mm->hint_inputs[1]->buffer;
+        const std::shared_ptr<Buffer>& a = mm->hint_inputs[0]->buffer;
+        std::shared_ptr<Buffer> w;
+        bool nt = false;
+        MRK_TRY(weight_operand(mm, true, &w, &nt));  // (a weight stored [N, K] is read in place)
         if (a->offset() % 16 || w->offset() % 16) return fail(kRuntime, "rope_matmul: unaligned operand");  // (views of whole tensors start aligned)
         auto out = new_buffer(n);
         std::shared_ptr<Buffer> rest_buf = rest ? new_buffer(rest) : out;
-        MRK_TRY(builtin("gemm_bf16_rope", {M, N, K, split, seq}, {out, a, w, rest_buf, rp->hint_inputs[1]->buffer, rp->hint_inputs[2]->buffer}));
+        MRK_TRY(builtin(nt ? "gemm_bf16_nt_rope" : "gemm_bf16_rope", {M, N, K, split, seq},
+                        {out, a, w, rest_buf, rp->hint_inputs[1]->buffer, rp->hint_inputs[2]->buffer}));
         n->buffer = out;
         produced.push_back(n);
         if (rest) {

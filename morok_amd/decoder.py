@@ -40,19 +40,27 @@ class DecoderBlock:
     """Holds the device-resident weights and builds the lazy graph of one forward pass."""
 
     def __init__(self, weights, batch, seq, hidden, heads, ffn, eps=1e-6, theta=10000.0, device_id=0,
-                 fuse_projections=True):
+                 fuse_projections=True, linear_layout=False):
         """fuse_projections: store Wq|Wk|Wv and W1|W3 side by side and run each group as one
         product (same dot products, so the same bits): one launch instead of three / two, and the
         gate+up product at hidden 4096 / ffn 11008 fills whole rounds of output tiles over the
-        compute units where two separate products each leave the last round two thirds empty."""
+        compute units where two separate products each leave the last round two thirds empty.
+        linear_layout: hold every projection as `nn::Linear` does, [out_features, in_features]
+        (tensor/src/nn/linear.rs:9-14), and multiply with `linear` (x @ w.T): the same dot products; the kernels
+        read the weight in place, and a handful of tokens stream it once."""
         assert hidden % heads == 0
         self.batch, self.seq, self.hidden, self.heads, self.ffn, self.eps = batch, seq, hidden, heads, ffn, eps
         self.dim = hidden // heads
-        self.w = {k: Tensor.from_numpy(np.ascontiguousarray(weights[k]), uop.BF16, device_id) for k in WEIGHT_NAMES}
+        self.linear_layout = bool(linear_layout)
+        projections = ("Wq", "Wk", "Wv", "Wo", "W1", "W2", "W3")
+        stored = {k: (np.ascontiguousarray(weights[k].T) if self.linear_layout and k in projections else np.ascontiguousarray(weights[k]))
+                  for k in WEIGHT_NAMES}
+        self.w = {k: Tensor.from_numpy(stored[k], uop.BF16, device_id) for k in WEIGHT_NAMES}
         self.fused = bool(fuse_projections)
         if self.fused:
-            self.w["Wqkv"] = Tensor.cat([self.w["Wq"], self.w["Wk"], self.w["Wv"]], 1).realize()
-            self.w["W13"] = Tensor.cat([self.w["W1"], self.w["W3"]], 1).realize()
+            axis = 0 if self.linear_layout else 1
+            self.w["Wqkv"] = Tensor.cat([self.w["Wq"], self.w["Wk"], self.w["Wv"]], axis).realize()
+            self.w["W13"] = Tensor.cat([self.w["W1"], self.w["W3"]], axis).realize()
         cos, sin = rope_tables(seq, self.dim, theta)
         self.cos_host, self.sin_host = cos, sin
         self.cos = Tensor.from_numpy(cos.reshape(1, 1, seq, self.dim // 2), device_id=device_id)
@@ -65,6 +73,10 @@ class DecoderBlock:
         """[T, hidden] token-major -> [B, H, S, D] head-major (a view: no copy by itself)."""
         return x.try_reshape([self.batch, self.seq, self.heads, self.dim]).try_permute([0, 2, 1, 3])
 
+    def _proj(self, x, name):
+        """x @ W for the projection `name`, in whichever layout the block holds it."""
+        return x.linear(self.w[name]) if self.linear_layout else x.matmul(self.w[name])
+
     def _norm(self, x, weight):
         return x.rms_norm(-1, self.eps).try_mul(weight).cast(uop.BF16)
 
@@ -74,7 +86,7 @@ class DecoderBlock:
         h = w["emb"].embedding(tokens).contiguous()
         xn = self._norm(h, w["w_an"])
         if self.fused:
-            qkv = xn.matmul(w["Wqkv"])
+            qkv = self._proj(xn, "Wqkv")
             xv = qkv.try_shrink([(0, T), (2 * self.hidden, 3 * self.hidden)])
             # q and k lie side by side in the packed product: one rotary kernel over 2 * heads heads
             # (the same per-head arithmetic).  Its result stays token-major (whole 2 * hidden rows
@@ -87,17 +99,17 @@ class DecoderBlock:
             q = qk.try_shrink([r if r else (0, self.heads) for r in full]).try_permute([0, 2, 1, 3])
             k = qk.try_shrink([r if r else (self.heads, 2 * self.heads) for r in full]).try_permute([0, 2, 1, 3])
         else:
-            xq, xk, xv = xn.matmul(w["Wq"]), xn.matmul(w["Wk"]), xn.matmul(w["Wv"])
+            xq, xk, xv = self._proj(xn, "Wq"), self._proj(xn, "Wk"), self._proj(xn, "Wv")
             q = self._heads(xq).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
             k = self._heads(xk).apply_rotary_emb(self.cos, self.sin, False).cast(uop.BF16)
         v = self._heads(xv)
         a = q.scaled_dot_product_attention(k, v, is_causal=True)
         a = a.try_permute([0, 2, 1, 3]).try_reshape([T, self.hidden])
-        h2 = h.try_add(a.matmul(w["Wo"])).contiguous()
+        h2 = h.try_add(self._proj(a, "Wo")).contiguous()
         xn2 = self._norm(h2, w["w_fn"])
         if self.fused:
-            gu = xn2.matmul(w["W13"])
+            gu = self._proj(xn2, "W13")
             g = gu.try_shrink([(0, T), (0, self.ffn)]).silu().try_mul(gu.try_shrink([(0, T), (self.ffn, 2 * self.ffn)]))
         else:
-            g = xn2.matmul(w["W1"]).silu().try_mul(xn2.matmul(w["W3"]))
-        return h2.try_add(g.matmul(w["W2"]))
+            g = self._proj(xn2, "W1").silu().try_mul(self._proj(xn2, "W3"))
+        return h2.try_add(self._proj(g, "W2"))

@@ -66,8 +66,8 @@ int launch_gemm_bf16_swiglu(void* stream, const void*, const void*, void*, long,
 bool gemm_bf16_rope_supported(long M, long N, long K, long split, long seq) {
     return M > 0 && N > 0 && K > 0 && seq > 0 && K % 64 == 0 && N % 8 == 0 && split > 0 && split <= N && split % 256 == 0;
 }
-int launch_gemm_bf16_rope(void* stream, const void*, const void*, void*, void*, long, long, long, long, const void*, const void*, long) {
-    mrk_shim_note_launch(stream, "gemm_bf16_rope");
+int launch_gemm_bf16_rope(void* stream, const void*, const void*, void*, void*, long, long, long, long, const void*, const void*, long, bool b_transposed) {
+    mrk_shim_note_launch(stream, b_transposed ? "gemm_bf16_nt_rope" : "gemm_bf16_rope");
     return 0;
 }
 int launch_flash_fwd_bf16(void* stream, const void*, const void*, const void*, void*, long, long, long, long, float, int) {

@@ -6,11 +6,11 @@ import pytest
 pytestmark = pytest.mark.gpu
 
 
-def run_block(cfg, tokens, weights, fused=True):
+def run_block(cfg, tokens, weights, fused=True, linear_layout=False):
     from morok_amd import decoder, tensor, uop
 
     blk = decoder.DecoderBlock(weights, cfg["batch"], cfg["seq"], cfg["hidden"], cfg["heads"], cfg["ffn"], cfg["eps"],
-                               fuse_projections=fused)
+                               fuse_projections=fused, linear_layout=linear_layout)
     out = blk.forward(tensor.Tensor.from_numpy(tokens.astype(np.int32)))
     out.realize()
     return blk, out, out.kernels()
@@ -78,6 +78,36 @@ def test_decoder_block_few_tokens(dev, oracle, cfg):
     assert sum(k.startswith("gemm_bf16") for k in kernels) == 4
     assert sum(k.startswith("flash_fwd") for k in kernels) == 1
     assert not any(tag in k for k in kernels for tag in ("swiglu", "residual", "rope")), kernels
+
+
+@pytest.mark.parametrize("cfg", [
+    dict(batch=1, seq=256, hidden=4096, heads=32, ffn=11008, vocab=32000, eps=1e-6),
+    dict(batch=2, seq=8, hidden=4096, heads=32, ffn=11008, vocab=32000, eps=1e-6),
+    dict(batch=3, seq=1, hidden=512, heads=4, ffn=1280, vocab=777, eps=1e-6),
+], ids=["h4096_seq256", "h4096_16tokens", "h512_seq1"])
+def test_decoder_block_with_linear_layout_weights(dev, oracle, cfg):
+    """Every projection held as nn::Linear holds it ([out_features, in_features], tensor/src/nn/linear.rs:9-14)
+    and applied with `linear`: the kernels read the weights in place.  A prefill-sized run keeps the fused
+    epilogues (rotary, residual, gate) and gives the bits of the [K, N] block (the same products in the same
+    order); a handful of tokens streams every weight once, with the residual adds inside the streaming kernels."""
+    from morok_amd import decoder, synth
+
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], cfg["vocab"], seed=6)
+    T = cfg["batch"] * cfg["seq"]
+    tok = synth.randint((T,), 6, 1, cfg["vocab"])
+    blk, out, kernels = run_block(cfg, tok, w, linear_layout=True)
+    got = out.to_numpy()
+    ref = oracle.decoder_block_bf16(tok, w, blk.cos_host, blk.sin_host, cfg["batch"], cfg["seq"], cfg["hidden"],
+                                    cfg["heads"], cfg["ffn"], cfg["eps"])
+    assert rel_err(got, ref) <= 2e-2
+    products = [k for k in kernels if k.startswith("gemm_bf16")]
+    assert len(products) == 4 and all(k.startswith("gemm_bf16_nt") for k in products), kernels
+    if T >= 256:
+        assert any("rope" in k for k in products) and any("swiglu" in k for k in products), kernels
+        _, out_kn, _ = run_block(cfg, tok, w)
+        assert np.array_equal(got, out_kn.to_numpy())
+    else:
+        assert sum("residual" in k for k in products) == 2 and not any("swiglu" in k or "rope" in k for k in products), kernels
 
 
 def test_decoder_block_full_size_properties(dev):

@@ -483,6 +483,12 @@ def test_gemm_rotary_epilogue(dev, oracle, shape):
     brot2, brest2 = dev.buffer(M * split * 2), dev.buffer(max(M * rest * 2, 2))
     morok_amd.Program.builtin("gemm_bf16_rope", [M, N, K, split, seq], dev.device_id).execute([brot2, ba, bb, brest2, bcos, bsin])
     assert np.array_equal(brot2.copyout(np.uint16, (M, split)), got_rot)
+    # with the weight stored [N, K] (a Linear layer's): the same products in the same order, so the same bits
+    bbt = morok_amd.Buffer.from_numpy(np.ascontiguousarray(b.T), dev.device_id)
+    brot3 = morok_amd.Buffer.from_numpy(np.full(M * split + 2048, 0x7FC0, np.uint16), dev.device_id)
+    brest3 = morok_amd.Buffer.from_numpy(np.full(M * rest + 2048, 0x7FC0, np.uint16), dev.device_id)
+    morok_amd.Program.builtin("gemm_bf16_nt_rope", [M, N, K, split, seq], dev.device_id).execute([brot3, ba, bbt, brest3, bcos, bsin])
+    assert np.array_equal(brot3.copyout(np.uint16), rot_all) and np.array_equal(brest3.copyout(np.uint16), rest_all)
 
 
 def test_gemm_rotary_epilogue_refusals(dev):
