@@ -2413,8 +2413,11 @@ struct Scheduler {
                 block = c;
                 break;
             }
-        // whole waves, at most 8 vectors per work-item (the row stays in registers), enough rows to fill the chip
-        if (!block || V / block > 8 || rows < 128) return {};
+        // whole waves, at most 8 vectors per work-item (the row stays in registers), enough rows to fill the chip; a
+        // handful of short rows (a decode step's activations: up to 1 MiB in all) is bound by launches, not by the
+        // chip, and one kernel instead of a reduction and an elementwise kernel is the faster form there
+        const bool tiny = n->numel() * static_cast<int64_t>(scalar_size(n->dtype)) <= (1 << 20);
+        if (!block || V / block > 8 || (rows < 128 && !tiny)) return {};
         *block_out = block;
         return ordered;
     }
