@@ -432,6 +432,52 @@ def bench_decoder(m, dev, steps, warmup, cpu):
     return rec
 
 
+def bench_decoder_decode(m, dev, steps, warmup, cpu):
+    """The same block over 16 tokens (16 sequences, one position each), weights held as `nn::Linear` holds them
+    ([out, in]): every weight is streamed once per step, so the step is bound by HBM, and the rate counts the
+    weights' bytes.  Eight blocks with different weights run in turn so that none is found in the last-level cache."""
+    import numpy as np
+
+    from morok_amd import decoder, synth, tensor
+
+    B, S, hidden, heads, ffn, vocab, layers = 16, 1, 4096, 32, 11008, 32000, 8
+    plans = []
+    for i in range(layers):
+        w = decoder.synthetic_weights(hidden, ffn, vocab, seed=20 + i)
+        blk = decoder.DecoderBlock(w, B, S, hidden, heads, ffn, eps=1e-6, theta=10000.0, linear_layout=True)
+        tok = tensor.Tensor.from_numpy(synth.randint((B * S,), 5, 1, vocab))
+        plans.append((blk, blk.forward(tok).prepare()))
+
+    def step():
+        for _, p in plans:
+            p.execute()
+
+    ms, stats = _launch_stats(m, step, max(1, min(steps, 20)), warmup)
+    prof = plans[0][1].execute_profiled()
+    weight_bytes = 2 * hidden * (4 * hidden + 3 * ffn)          # per block
+    gbs = layers * weight_bytes / (ms * 1e-3) / 1e9
+    rec = {"metric": "decoder block decode HBM GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "bf16", **stats,
+           "config": {"workload": "decoder block via tensor API over 16 tokens (16 sequences x 1 position), weights [out, in]: "
+                                  "hidden 4096, 32x128 heads, SwiGLU 11008; 8 blocks with different weights per step"},
+           "blocks_per_step": layers, "us_per_block": ms * 1e3 / layers, "tokens_per_s": B * S * layers / (ms * 1e-3), "kernels": len(prof),
+           "gemm_us": 1e3 * sum(t for n, t in prof if n.startswith("gemm_bf16")), "other_us": 1e3 * sum(t for n, t in prof if not n.startswith("gemm_bf16")),
+           "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
+                        "traffic_source": "per-kernel figures in profiles/" + PROFILE_OF["linear_decode_16"],
+                        "kernel": "gemm_nt_rows (4 of the %d kernels)" % len(prof), "algorithmic_bytes_per_launch": weight_bytes}}
+    if cpu:
+        from tests.oracle_lib import Oracle
+
+        orc = Oracle()
+        w = decoder.synthetic_weights(hidden, ffn, vocab, seed=20)
+        stok = synth.randint((B * S,), 5, 1, vocab)
+        cos, sin = decoder.rope_tables(S, hidden // heads)
+        t = orc.max_threads
+        sec = _cpu_time(lambda: orc.decoder_block_bf16(stok, w, cos, sin, B, S, hidden, heads, ffn, 1e-6, threads=t))
+        rec["cpu_baseline"] = {"value": weight_bytes / sec / 1e9, "unit": "GB/s", "cores": t, "kind": "port",
+                               "sample": f"one block over the same 16 tokens, {t} threads, min of 3 after 1 warm-up"}
+    return rec
+
+
 def bench_matmul_f32(m, dev, steps, warmup, cpu):
     """configs[0]: f32 matmul through Tensor::matmul, A[1024x1024] @ B[1024x1024], uniform(-1,1), seed 1
     (plumbing + correctness: lazy graph -> schedule -> render -> hiprtc -> launch)."""
@@ -628,7 +674,8 @@ def bench_copy(m, dev, steps, warmup, cpu):
 WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash, "decoder": bench_decoder,
              "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling,
              "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16, "flash_options": bench_flash_options,
-             "linear_decode": bench_linear_decode, "linear_decode_16": bench_linear_decode_16}
+             "linear_decode": bench_linear_decode, "linear_decode_16": bench_linear_decode_16,
+             "decoder_decode": bench_decoder_decode}
 PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc", "linear_decode", "linear_decode_16"]
 
 
