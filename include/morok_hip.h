@@ -482,8 +482,12 @@ size_t mrk_hip_gemm_bf16_noalloc_capacity(void);
 /* c = bf16(float(bf16(a b)) + float(r)): the product above with a bf16 matrix r of c's shape added
  * in the kernel's epilogue - the bits of mrk_hip_gemm_bf16 followed by an elementwise add
  * (Tensor::matmul + try_add, tensor/src/matmul.rs:82-110), without the round trip of the product
- * through memory.  INVALID_ARGUMENT for shapes the fused epilogue does not cover (N or K not a
- * multiple of 8, K = 0, or so few output tiles that split-K is used). */
+ * through memory.  The product takes the route mrk_hip_gemm_bf16 takes and r joins where its result is
+ * written: the tiled kernels' epilogue, the sum of the partial results of a product spread along K (scratch
+ * from the device allocator), the streaming kernels for a handful of rows.  INVALID_ARGUMENT for shapes
+ * outside the tiled kernels' (N or K not a multiple of 8, K = 0).  Builtin Program kinds
+ * "gemm_bf16_residual" / "gemm_bf16_nt_residual" / "gemm_bf16_bias" / "gemm_bf16_nt_bias" take
+ * {M, N, K[, batch[, workspace bytes]]} and buffers {c, a, b, r[, scratch]}. */
 int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, const void* r, void* c, int64_t m, int64_t n,
                                int64_t k);
 /* y[M, N] = x[M, K] * w[N, K]^T + bias[N]: a Linear layer's forward pass on its parameters as it stores them

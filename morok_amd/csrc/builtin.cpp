@@ -159,35 +159,31 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
-    if (k == "gemm_bf16_bias" || k == "gemm_bf16_nt_bias") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, b, bias [N]}
-        const bool nt = k == "gemm_bf16_nt_bias";
-        if (nparams != 3 && nparams != 4)
-            return failf(kInvalidArgument, "builtin '%s' takes 3 or 4 parameters, got %zu", k.c_str(), nparams);
-        if (p.size() < 4) p.push_back(1);
-        if (!gemm_bf16_bias_launchable(p[0], p[1], p[2], p[3], nt))
-            return fail(kInvalidArgument, k + ": shape not covered (N and K multiples of 8, or up to 64 rows against an [N, K] operand with K a "
-                                              "multiple of 8)");
-        std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
-        if (p[3] > 1) name += "_x" + std::to_string(p[3]);
-        out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
-                                      [nt](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
-                                          return launch_gemm_bf16_bias(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3], nt);
-                                      }));
-        return kOk;
-    }
-    if (k == "gemm_bf16_residual" || k == "gemm_bf16_nt_residual") {  // {M, N, K} or {M, N, K, batch}; buffers {c, a, b, r}
-        const bool nt = k == "gemm_bf16_nt_residual";
-        if (nparams < 3 || nparams > 4)
-            return failf(kInvalidArgument, "builtin '%s' takes 3 or 4 parameters, got %zu", k.c_str(), nparams);
+    // c = a b + r in the product's own kernels: r a matrix of c's shape ("_residual") or one row [N] ("_bias");
+    // {M, N, K}, {M, N, K, batch} or {M, N, K, batch, workspace bytes}; buffers {c, a, b, r[, scratch]}
+    if (k == "gemm_bf16_bias" || k == "gemm_bf16_nt_bias" || k == "gemm_bf16_residual" || k == "gemm_bf16_nt_residual") {
+        const bool nt = k.find("_nt_") != std::string::npos, row = k.find("_bias") != std::string::npos;
+        if (nparams < 3 || nparams > 5)
+            return failf(kInvalidArgument, "builtin '%s' takes 3 to 5 parameters, got %zu", k.c_str(), nparams);
         while (p.size() < 4) p.push_back(1);
-        if (!gemm_bf16_residual_supported(p[0], p[1], p[2], p[3]) && !(nt && gemm_nt_bias_streamed(p[0], p[1], p[2], p[3])))
-            return failf(kInvalidArgument, "%s: shape not covered (N and K multiples of 8, enough output tiles for the plain tiled kernel%s)", k.c_str(),
+        if (p.size() < 5) p.push_back(0);
+        if (p[4] < 0) return fail(kInvalidArgument, k + ": negative workspace size");
+        if (!gemm_bf16_bias_launchable(p[0], p[1], p[2], p[3], nt))
+            return failf(kInvalidArgument, "%s: shape not covered (N and K multiples of 8%s)", k.c_str(),
                          nt ? "; or up to 64 rows with K a multiple of 8" : "");
         std::string name = k + "_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]);
         if (p[3] > 1) name += "_x" + std::to_string(p[3]);
+        if (p[4] > 0) {  // a fifth buffer of p[4] bytes: scratch for the partial results of a product spread along K
+            out->reset(new BuiltinProgram(device_id, stream, name + "_splitk", 5, p,
+                                          [nt, row](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                              return launch_gemm_bf16_residual(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3], nt, row, b[4],
+                                                                               static_cast<size_t>(q[4]));
+                                          }));
+            return kOk;
+        }
         out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
-                                      [nt](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
-                                          return launch_gemm_bf16_residual(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3], nt);
+                                      [nt, row](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+                                          return launch_gemm_bf16_residual(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3], nt, row);
                                       }));
         return kOk;
     }

@@ -979,12 +979,19 @@ int mrk_hip_gemm_bf16_residual(int device_id, const void* a, const void* b, cons
     MRK_NONNULL(r);
     MRK_NONNULL(c);
     if (!gemm_bf16_residual_supported(m, n, k, 1))
-        return fail(kInvalidArgument, "gemm_bf16_residual: shape not covered by the fused epilogue (N and K multiples of 8, K > 0, "
-                                      "enough output tiles that split-K is not used); run mrk_hip_gemm_bf16 and add separately");
+        return fail(kInvalidArgument, "gemm_bf16_residual: shape not covered by the fused epilogue (N and K multiples of 8, K > 0); "
+                                      "run mrk_hip_gemm_bf16 and add separately");
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_gemm_bf16_residual(dv->allocator->stream(), a, b, r, c, m, n, k, 1), "gemm_bf16_residual launch");
+    // few output tiles against a long K: scratch for the partial results, as for the plain product
+    const size_t ws = gemm_bf16_workspace_bytes(m, n, k, 1);
+    RawBuffer scratch;
+    BufferOptions so;
+    if (ws) MRK_TRY(dv->allocator->alloc(ws, so, &scratch));
+    int rc = launch_gemm_bf16_residual(dv->allocator->stream(), a, b, r, c, m, n, k, 1, false, false, ws ? scratch.ptr : nullptr, ws);
+    if (ws) dv->allocator->free(scratch, so);
+    MRK_HIP(rc, "gemm_bf16_residual launch");
     return kOk;
 }
 
@@ -1001,7 +1008,13 @@ int mrk_hip_linear_bf16(int device_id, const void* x, const void* w, const void*
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_gemm_bf16_bias(dv->allocator->stream(), x, w, bias, y, m, n, k, 1, true), "linear_bf16 launch");
+    const size_t ws = gemm_bf16_nt_workspace_bytes(m, n, k, 1);
+    RawBuffer scratch;
+    BufferOptions so;
+    if (ws) MRK_TRY(dv->allocator->alloc(ws, so, &scratch));
+    int rc = launch_gemm_bf16_bias(dv->allocator->stream(), x, w, bias, y, m, n, k, 1, true, ws ? scratch.ptr : nullptr, ws);
+    if (ws) dv->allocator->free(scratch, so);
+    MRK_HIP(rc, "linear_bf16 launch");
     return kOk;
 }
 

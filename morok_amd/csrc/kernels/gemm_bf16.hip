@@ -852,10 +852,12 @@ __global__ __launch_bounds__(256) void gemm_bf16_tile128_splitk_ragged_k(const _
     gemm_tile_body<true, 2, true>(A, B, nullptr, M, N, K, tiles_m, tiles_n, W, kt_per_split);
 }
 // C[i] = bf16(W[0][i] + W[1][i] + ... + W[splits-1][i]), 8 elements per work-item, partials added
-// in the order of their K ranges so the result does not depend on timing.
+// in the order of their K ranges so the result does not depend on timing.  R, when given, is added to the rounded
+// sum and the result rounded again (the bits of the product followed by an elementwise add): a matrix of C's shape
+// (r_period 0) or one row repeated every r_period elements (a bias).
 template <bool kF16>
 __global__ __launch_bounds__(256) void gemm_splitk_reduce(const float* __restrict__ W, __bf16* __restrict__ C, long total,
-                                                          int splits) {
+                                                          int splits, const __bf16* __restrict__ R, long r_period) {
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
     if (i >= total) return;
     f32x4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = lo;
@@ -865,6 +867,15 @@ __global__ __launch_bounds__(256) void gemm_splitk_reduce(const float* __restric
         hi += p[1];
     }
     bf16x4 l = round_to_elem<kF16>(lo), h = round_to_elem<kF16>(hi);
+    if (R) {
+        const bf16x8 r = *reinterpret_cast<const bf16x8*>(R + (r_period ? i % r_period : i));
+        auto widen = [](const bf16x4& v) {
+            if constexpr (kF16) return __builtin_convertvector(__builtin_bit_cast(f16x4, v), f32x4);
+            else return __builtin_convertvector(v, f32x4);
+        };
+        l = round_to_elem<kF16>(widen(l) + widen(__builtin_shufflevector(r, r, 0, 1, 2, 3)));
+        h = round_to_elem<kF16>(widen(h) + widen(__builtin_shufflevector(r, r, 4, 5, 6, 7)));
+    }
     *reinterpret_cast<bf16x8*>(C + i) = __builtin_shufflevector(l, h, 0, 1, 2, 3, 4, 5, 6, 7);
 }
 
@@ -986,13 +997,7 @@ int launch_gemm_bf16_static_ws(void* stream, int device_id, const void* A, const
     return launch_gemm_bf16(stream, A, B, C, M, N, K, 0, 1, need ? ws : nullptr, need);
 }
 
-bool gemm_bf16_residual_supported(long M, long N, long K, long batch) {
-    if (M <= 0 || N <= 0 || K <= 0 || batch <= 0 || batch > 65535) return false;
-    if (M > 0x7fffffffL || N > 0x7fffffffL || N % 8 || K % 8 || K > (1L << 23) || N >= (1L << 25)) return false;
-    if (plan_split_k(M, N, K, batch).splits > 1) return false;  // split-K sums partials in another kernel
-    const long tn = (N + mrk::dev::kBN - 1) / mrk::dev::kBN, tm128 = (M + 127) / 128;
-    return tm128 * tn <= 0x7fffffffL;
-}
+bool gemm_bf16_residual_supported(long M, long N, long K, long batch);  // (defined behind tiled_shape)
 
 namespace {
 // shapes the tiled kernels address (any M; N and K in whole 16-byte chunks; 32-bit offsets inside a tile)
@@ -1003,6 +1008,8 @@ bool tiled_shape(long M, long N, long K, long batch) {
     return tm128 * tn <= 0x7fffffffL;
 }
 }  // namespace
+
+bool gemm_bf16_residual_supported(long M, long N, long K, long batch) { return tiled_shape(M, N, K, batch); }
 
 bool gemm_bf16_nt_supported(long M, long N, long K, long batch) {
     // the tiled kernels (no any-shape kernel for this operand layout), or the streaming kernels for a
@@ -1017,21 +1024,22 @@ size_t gemm_bf16_nt_workspace_bytes(long M, long N, long K, long batch) {
     return p.splits > 1 ? (size_t)p.splits * batch * M * N * sizeof(float) : 0;
 }
 
-int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch,
-                              bool b_transposed, bool r_is_row) {
+int launch_gemm_16bit(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant, long batch, void* workspace,
+                      size_t workspace_bytes, bool b_transposed, bool f16, const void* add, bool add_is_row);
+
+namespace {
+// the tiled kernels with the residual epilogue (one pass of output tiles; variant 3 / 4 force the tile)
+int launch_tiled_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch,
+                          bool b_transposed, bool r_is_row, int variant) {
     using namespace mrk::dev;
     if (M <= 0 || N <= 0 || batch <= 0) return 0;
-    // a handful of rows against an [N, K] weight: the streaming kernels add R where they write their result
-    if (b_transposed && gemm_nt_bias_streamed(M, N, K, batch))
-        return launch_gemm_nt_bias_streamed(stream, A, B, R, C, M, N, K, false, r_is_row);
-    // every shape the tiled kernels address; gemm_bf16_residual_supported is narrower (it leaves out what split-K runs faster)
     if (!tiled_shape(M, N, K, batch)) return (int)hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C) | reinterpret_cast<uintptr_t>(R)) % 16)
         return (int)hipErrorInvalidValue;
     hipStream_t s = static_cast<hipStream_t>(stream);
     (void)hipGetLastError();
     const long tn = (N + kBN - 1) / kBN, tm128 = (M + 127) / 128;
-    const bool small = tm128 * tn * batch <= 256;
+    const bool small = variant == 4 || (variant != 3 && tm128 * tn * batch <= 256);
     const long tm = small ? tm128 : (M + kBM - 1) / kBM;
     const dim3 grid((unsigned)(tm * tn), (unsigned)batch);
     const __bf16* a = static_cast<const __bf16*>(A);
@@ -1046,26 +1054,24 @@ int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const 
     kernel<<<grid, 256, 0, s>>>(a, b, r, c, (int)M, (int)N, (int)K, (int)tm, (int)tn, r_is_row ? 0 : -1);
     return (int)hipGetLastError();
 }
+}  // namespace
+
+int launch_gemm_bf16_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch,
+                              bool b_transposed, bool r_is_row, void* workspace, size_t workspace_bytes) {
+    if (!R) return (int)hipErrorInvalidValue;
+    return launch_gemm_16bit(stream, A, B, C, M, N, K, 0, batch, workspace, workspace_bytes, b_transposed, false, R, r_is_row);
+}
 
 bool gemm_bf16_bias_supported(long M, long N, long K, long batch, bool b_transposed) {
     if (M <= 0 || N <= 0 || K <= 0 || batch <= 0) return false;
-    if (b_transposed && gemm_nt_bias_streamed(M, N, K, batch)) return true;
-    long ks = 0, kr = 0;
-    if (!b_transposed && (gemm_kn_skinny_plan(M, N, K, batch, &ks, &kr) || gemm_kn_rows_plan(M, N, K, batch, &ks, &kr))) return false;
-    return gemm_bf16_residual_supported(M, N, K, batch);
-}
-
-bool gemm_bf16_bias_launchable(long M, long N, long K, long batch, bool b_transposed) {
     return (b_transposed && gemm_nt_bias_streamed(M, N, K, batch)) || tiled_shape(M, N, K, batch);
 }
 
+bool gemm_bf16_bias_launchable(long M, long N, long K, long batch, bool b_transposed) { return gemm_bf16_bias_supported(M, N, K, batch, b_transposed); }
+
 int launch_gemm_bf16_bias(void* stream, const void* a, const void* b, const void* bias, void* c, long M, long N, long K, long batch,
-                          bool b_transposed) {
-    if (M <= 0 || N <= 0 || batch <= 0) return 0;
-    if (!bias) return (int)hipErrorInvalidValue;
-    if (b_transposed && gemm_nt_bias_streamed(M, N, K, batch)) return launch_gemm_nt_bias_streamed(stream, a, b, bias, c, M, N, K, false);
-    // (a shape outside gemm_bf16_bias_supported that the tiled kernels address still runs here, on the workgroups its tiles make)
-    return launch_gemm_bf16_residual(stream, a, b, bias, c, M, N, K, batch, b_transposed, true);
+                          bool b_transposed, void* workspace, size_t workspace_bytes) {
+    return launch_gemm_bf16_residual(stream, a, b, bias, c, M, N, K, batch, b_transposed, true, workspace, workspace_bytes);
 }
 
 bool gemm_bf16_swiglu_supported(long M, long F, long K, bool b_transposed) {
@@ -1119,10 +1125,20 @@ int launch_gemm_bf16_rope(void* stream, const void* A, const void* B, void* C_ro
     return (int)hipGetLastError();
 }
 
-int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant,
-                     long batch, void* workspace, size_t workspace_bytes, bool b_transposed, bool f16) {
+namespace {
+int launch_tiled_residual(void* stream, const void* A, const void* B, const void* R, void* C, long M, long N, long K, long batch,
+                          bool b_transposed, bool r_is_row, int variant);
+}
+
+// The product, with `add` (a matrix of C's shape or, add_is_row, one row [N]; bf16) added to the rounded result by
+// whichever kernel writes it: the streaming kernels, the split-K reduction or the tiled kernels' residual epilogue.
+int launch_gemm_16bit(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant, long batch, void* workspace,
+                      size_t workspace_bytes, bool b_transposed, bool f16, const void* add, bool add_is_row) {
     using namespace mrk::dev;
     if (M <= 0 || N <= 0 || batch <= 0) return 0;
+    if (add && reinterpret_cast<uintptr_t>(add) % 16) return (int)hipErrorInvalidValue;
+    const __bf16* addp = static_cast<const __bf16*>(add);
+    const long add_period = add_is_row ? N : 0;
     if (batch > 65535) return (int)hipErrorInvalidValue;  // grid y extent
     if (M > 0x7fffffffL || N > 0x7fffffffL || K > 0x7fffffffL || K < 0) return (int)hipErrorInvalidValue;
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -1139,9 +1155,14 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
         // up to 64 rows: one pass over the weight streams it faster than any tile (one or two rows on the
         // vector ALUs, more on the matrix pipes with 16-row blocks staged through LDS)
         if (choose || !tiled) {
-            if (gemm_nt_skinny_supported(M, N, K, batch)) return launch_gemm_nt_skinny(stream, A, B, C, M, N, K, batch, f16);
-            if (gemm_nt_rows_supported(M, N, K, batch)) return launch_gemm_nt_rows(stream, A, B, C, M, N, K, batch, f16);
+            if (add) {
+                if (gemm_nt_bias_streamed(M, N, K, batch)) return launch_gemm_nt_bias_streamed(stream, A, B, add, C, M, N, K, f16, add_is_row);
+            } else {
+                if (gemm_nt_skinny_supported(M, N, K, batch)) return launch_gemm_nt_skinny(stream, A, B, C, M, N, K, batch, f16);
+                if (gemm_nt_rows_supported(M, N, K, batch)) return launch_gemm_nt_rows(stream, A, B, C, M, N, K, batch, f16);
+            }
         }
+        if (!tiled) return (int)hipErrorInvalidValue;
         const long tn = (N + kBN - 1) / kBN, tm128 = (M + 127) / 128;
         const SplitPlan sp = choose ? plan_split_k(M, N, K, batch) : SplitPlan();
         if (sp.splits > 1) {
@@ -1158,10 +1179,11 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
                                                   (int)tm128, (int)tn, (int)sp.kt_per_split);
                 const long total = batch * M * N;
                 auto reduce_kernel = f16 ? gemm_splitk_reduce<true> : gemm_splitk_reduce<false>;
-                reduce_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>(w, static_cast<__bf16*>(C), total, (int)sp.splits);
+                reduce_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>(w, static_cast<__bf16*>(C), total, (int)sp.splits, addp, add_period);
                 return (int)hipGetLastError();
             }
         }
+        if (add) return f16 ? (int)hipErrorInvalidValue : launch_tiled_residual(stream, A, B, add, C, M, N, K, batch, true, add_is_row, variant);
         const bool small = variant == 4 || (variant != 3 && tm128 * tn * batch <= 256);
         const long tm = small ? tm128 : (M + kBM - 1) / kBM;
         const bool ragged_k = K % kBK != 0;
@@ -1178,11 +1200,11 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
         long ks = 0, kr = 0;
         if ((variant == 0 || variant == 5) && aligned && gemm_kn_skinny_plan(M, N, K, batch, &ks, &kr) && workspace &&
             workspace_bytes >= (size_t)ks * M * N * sizeof(float) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
-            return launch_gemm_kn_skinny(stream, A, B, C, workspace, M, N, K, ks, kr, f16);
+            return launch_gemm_kn_skinny(stream, A, B, C, workspace, M, N, K, ks, kr, f16, add, add_is_row);
         }
         if ((variant == 0 || variant == 5) && aligned && gemm_kn_rows_plan(M, N, K, batch, &ks, &kr) &&
             (ks == 1 || (workspace && workspace_bytes >= (size_t)ks * M * N * sizeof(float) && reinterpret_cast<uintptr_t>(workspace) % 16 == 0))) {
-            return launch_gemm_kn_rows(stream, A, B, C, workspace, M, N, K, ks, kr, f16);
+            return launch_gemm_kn_rows(stream, A, B, C, workspace, M, N, K, ks, kr, f16, add, add_is_row);
         }
     }
     // any M; N and K in whole 16-byte chunks
@@ -1203,11 +1225,12 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
             split_kernel<<<grid, 256, 0, s>>>(a, b, w, (int)M, (int)N, (int)K, (int)tm128, (int)tn, (int)sp.kt_per_split);
             const long total = batch * M * N;
             auto reduce_kernel = f16 ? gemm_splitk_reduce<true> : gemm_splitk_reduce<false>;
-            reduce_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>(w, static_cast<__bf16*>(C), total, (int)sp.splits);
+            reduce_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, s>>>(w, static_cast<__bf16*>(C), total, (int)sp.splits, addp, add_period);
             return (int)hipGetLastError();
         }
         // variant 0: the 128-row tile when all its workgroups are resident at once (at most one per
         // compute unit): twice the workgroups of the 256-row tile for the same work.  3 / 4 force one.
+        if (add) return f16 ? (int)hipErrorInvalidValue : launch_tiled_residual(stream, A, B, add, C, M, N, K, batch, false, add_is_row, variant);
         const bool small = variant == 4 || (variant != 3 && tm128 * tn * batch <= 256);
         const long tm = small ? tm128 : (M + kBM - 1) / kBM;
         if (tm * tn > 0x7fffffffL) return (int)hipErrorInvalidValue;
@@ -1222,6 +1245,7 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
                                    : (ragged_k ? gemm_bf16_tile256_ragged_k : gemm_bf16_tile256));
         kernel<<<grid, 256, 0, s>>>(a, b, c, (int)M, (int)N, (int)K, (int)tm, (int)tn);
     } else {
+        if (add) return (int)hipErrorInvalidValue;  // (the any-shape kernel has no epilogue)
         const long tm = (M + 31) / 32, tn = (N + 31) / 32;
         const long total = tm * tn;
         const long blocks = (total + 3) / 4;
@@ -1232,6 +1256,11 @@ int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M
                                                            total);
     }
     return (int)hipGetLastError();
+}
+
+int launch_gemm_bf16(void* stream, const void* A, const void* B, void* C, long M, long N, long K, int variant, long batch, void* workspace,
+                     size_t workspace_bytes, bool b_transposed, bool f16) {
+    return launch_gemm_16bit(stream, A, B, C, M, N, K, variant, batch, workspace, workspace_bytes, b_transposed, f16, nullptr, false);
 }
 
 }  // namespace mrk

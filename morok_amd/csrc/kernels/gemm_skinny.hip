@@ -424,7 +424,8 @@ __global__ __launch_bounds__(256) void gemm_kn_skinny_partial(const unsigned sho
 // gemm_kn_rows_reduce, or with a single K range the rounded result.
 template <int kMT, int kCB, bool kF16>
 __global__ __launch_bounds__(512) void gemm_kn_rows(const unsigned short* __restrict__ A, const unsigned short* __restrict__ B,
-                                                    unsigned short* __restrict__ C, float* __restrict__ W, int M, int N, int K, int k_per_split) {
+                                                    unsigned short* __restrict__ C, float* __restrict__ W, int M, int N, int K, int k_per_split,
+                                                    const unsigned short* __restrict__ add, long add_pitch) {
     constexpr int kWaves = 8;
     constexpr int kBlockBytes = 32 * 128;  // 32 k-rows x 64 columns
     constexpr int kWaveBytes = kCB * kBlockBytes;
@@ -536,12 +537,10 @@ __global__ __launch_bounds__(512) void gemm_kn_rows(const unsigned short* __rest
         if (W) {
             *reinterpret_cast<f32x4*>(W + ((size_t)blockIdx.y * M + m) * N + n) = s;
         } else {
+            const unsigned short* ad = add ? add + (size_t)m * add_pitch : nullptr;  // (the addend's row: pitch 0 for a bias)
             unsigned short o[4];
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                if constexpr (kF16) o[i] = __builtin_bit_cast(unsigned short, (_Float16)s[i]);
-                else o[i] = round_bf16(s[i]);
-            }
+            for (int i = 0; i < 4; i++) o[i] = round_out<kF16>(s[i], ad, n + i);
             *reinterpret_cast<u32x2*>(C + (size_t)m * N + n) = u32x2{(unsigned)o[0] | ((unsigned)o[1] << 16), (unsigned)o[2] | ((unsigned)o[3] << 16)};
         }
     }
@@ -553,7 +552,8 @@ __global__ __launch_bounds__(512) void gemm_kn_rows(const unsigned short* __rest
 // work-items per group of eight outputs each taking every 32nd slice, then one of them adds the 32
 // sums in order.  The order is fixed, so the result does not depend on timing.
 template <bool kF16>
-__global__ __launch_bounds__(256) void gemm_kn_skinny_reduce(const float* __restrict__ W, unsigned short* __restrict__ C, long total, int splits) {
+__global__ __launch_bounds__(256) void gemm_kn_skinny_reduce(const float* __restrict__ W, unsigned short* __restrict__ C, long total, int splits,
+                                                             const unsigned short* __restrict__ add, long add_period) {
     __shared__ float4 red[32][8][2];
     const int eg = threadIdx.x & 7, sl = threadIdx.x >> 3;
     const long i = ((long)blockIdx.x * 8 + eg) * 8;
@@ -576,11 +576,10 @@ __global__ __launch_bounds__(256) void gemm_kn_skinny_reduce(const float* __rest
         }
         const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
         unsigned short o[8];
+        // (the addend: a matrix of the result's shape, add_period 0, or one row repeated every add_period elements)
+        const unsigned short* ad = add ? add + (add_period ? i % add_period : i) : nullptr;
 #pragma unroll
-        for (int e = 0; e < 8; e++) {
-            if constexpr (kF16) o[e] = __builtin_bit_cast(unsigned short, (_Float16)v[e]);
-            else o[e] = round_bf16(v[e]);
-        }
+        for (int e = 0; e < 8; e++) o[e] = round_out<kF16>(v[e], ad, e);
         u32x4 pk = {(unsigned)o[0] | ((unsigned)o[1] << 16), (unsigned)o[2] | ((unsigned)o[3] << 16), (unsigned)o[4] | ((unsigned)o[5] << 16),
                     (unsigned)o[6] | ((unsigned)o[7] << 16)};
         *reinterpret_cast<u32x4*>(C + i) = pk;
@@ -591,17 +590,16 @@ __global__ __launch_bounds__(256) void gemm_kn_skinny_reduce(const float* __rest
 // C[i] = round(W[0][i] + ... + W[splits - 1][i]) for the few ranges gemm_kn_rows leaves (at most a few dozen):
 // a work-item adds its four outputs' partial sums in the order of the ranges.
 template <bool kF16>
-__global__ __launch_bounds__(256) void gemm_kn_rows_reduce(const float* __restrict__ W, unsigned short* __restrict__ C, long total, int splits) {
+__global__ __launch_bounds__(256) void gemm_kn_rows_reduce(const float* __restrict__ W, unsigned short* __restrict__ C, long total, int splits,
+                                                           const unsigned short* __restrict__ add, long add_period) {
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= total) return;
     f32x4 s = *reinterpret_cast<const f32x4*>(W + i);
     for (int k = 1; k < splits; k++) s += *reinterpret_cast<const f32x4*>(W + (size_t)k * total + i);
+    const unsigned short* ad = add ? add + (add_period ? i % add_period : i) : nullptr;
     unsigned short o[4];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        if constexpr (kF16) o[j] = __builtin_bit_cast(unsigned short, (_Float16)s[j]);
-        else o[j] = round_bf16(s[j]);
-    }
+    for (int j = 0; j < 4; j++) o[j] = round_out<kF16>(s[j], ad, j);
     *reinterpret_cast<u32x2*>(C + i) = u32x2{(unsigned)o[0] | ((unsigned)o[1] << 16), (unsigned)o[2] | ((unsigned)o[3] << 16)};
 }
 
@@ -757,7 +755,7 @@ bool gemm_kn_skinny_plan(long M, long N, long K, long batch, long* splits, long*
 }
 
 int launch_gemm_kn_skinny(void* stream, const void* A, const void* B, void* C, void* W, long M, long N, long K, long splits, long rows_per_group,
-                          bool f16) {
+                          bool f16, const void* add, bool add_is_row) {
     using namespace mrk::dev;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(C)) % 16)
         return (int)hipErrorInvalidValue;
@@ -776,8 +774,10 @@ int launch_gemm_kn_skinny(void* stream, const void* A, const void* B, void* C, v
 #undef MRK_KN
     const long total = M * N;  // (a multiple of 8)
     const unsigned blocks = (unsigned)((total + 63) / 64);
-    if (f16) gemm_kn_skinny_reduce<true><<<blocks, 256, 0, s>>>(w, static_cast<unsigned short*>(C), total, (int)splits);
-    else gemm_kn_skinny_reduce<false><<<blocks, 256, 0, s>>>(w, static_cast<unsigned short*>(C), total, (int)splits);
+    const unsigned short* ad = static_cast<const unsigned short*>(add);
+    const long period = add_is_row ? N : 0;
+    if (f16) gemm_kn_skinny_reduce<true><<<blocks, 256, 0, s>>>(w, static_cast<unsigned short*>(C), total, (int)splits, ad, period);
+    else gemm_kn_skinny_reduce<false><<<blocks, 256, 0, s>>>(w, static_cast<unsigned short*>(C), total, (int)splits, ad, period);
     return (int)hipGetLastError();
 }
 
@@ -804,7 +804,7 @@ bool gemm_kn_rows_plan(long M, long N, long K, long batch, long* splits, long* k
 }
 
 int launch_gemm_kn_rows(void* stream, const void* A, const void* B, void* C, void* W, long M, long N, long K, long splits, long k_per_split,
-                        bool f16) {
+                        bool f16, const void* add, bool add_is_row) {
     using namespace mrk::dev;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(W) | reinterpret_cast<uintptr_t>(C)) % 16)
         return (int)hipErrorInvalidValue;
@@ -815,11 +815,13 @@ int launch_gemm_kn_rows(void* stream, const void* A, const void* B, void* C, voi
     const unsigned short* b = static_cast<const unsigned short*>(B);
     unsigned short* c = static_cast<unsigned short*>(C);
     float* w = splits > 1 ? static_cast<float*>(W) : nullptr;
+    const unsigned short* ad = static_cast<const unsigned short*>(add);
+    const long pitch = add_is_row ? 0 : N;
 #define MRK_KN_ROWS(MT, CB)                                                                                              \
     do {                                                                                                                 \
         const dim3 grid((unsigned)((N + 64 * CB - 1) / (64 * CB)), (unsigned)splits);                                    \
-        if (f16) gemm_kn_rows<MT, CB, true><<<grid, 512, 0, s>>>(a, b, c, w, (int)M, (int)N, (int)K, (int)k_per_split);   \
-        else gemm_kn_rows<MT, CB, false><<<grid, 512, 0, s>>>(a, b, c, w, (int)M, (int)N, (int)K, (int)k_per_split);      \
+        if (f16) gemm_kn_rows<MT, CB, true><<<grid, 512, 0, s>>>(a, b, c, w, (int)M, (int)N, (int)K, (int)k_per_split, ad, pitch);  \
+        else gemm_kn_rows<MT, CB, false><<<grid, 512, 0, s>>>(a, b, c, w, (int)M, (int)N, (int)K, (int)k_per_split, ad, pitch);     \
     } while (0)
     if (M > 32) MRK_KN_ROWS(4, 1);
     else if (M > 16) MRK_KN_ROWS(2, 1);
@@ -829,8 +831,8 @@ int launch_gemm_kn_rows(void* stream, const void* A, const void* B, void* C, voi
     if (splits > 1) {
         const long total = M * N;  // (a multiple of 8)
         const unsigned blocks = (unsigned)((total / 4 + 255) / 256);
-        if (f16) gemm_kn_rows_reduce<true><<<blocks, 256, 0, s>>>(w, c, total, (int)splits);
-        else gemm_kn_rows_reduce<false><<<blocks, 256, 0, s>>>(w, c, total, (int)splits);
+        if (f16) gemm_kn_rows_reduce<true><<<blocks, 256, 0, s>>>(w, c, total, (int)splits, ad, add_is_row ? N : 0);
+        else gemm_kn_rows_reduce<false><<<blocks, 256, 0, s>>>(w, c, total, (int)splits, ad, add_is_row ? N : 0);
     }
     return (int)hipGetLastError();
 }

@@ -47,29 +47,29 @@ int launch_gemm_nt_rows(void* stream, const void* A, const void* Bt, void* C, lo
 // taken this way.  gemm_bf16_workspace_bytes reports splits * M * N * 4 for such shapes.
 bool gemm_kn_skinny_plan(long M, long N, long K, long batch, long* splits, long* rows_per_group);
 int launch_gemm_kn_skinny(void* stream, const void* A, const void* B, void* C, void* W, long M, long N, long K, long splits, long rows_per_group,
-                          bool f16);
+                          bool f16, const void* add = nullptr, bool add_is_row = false);
 // The [K, N] form for up to 16 rows (up to 64 against a weight of at most 4096 columns and 8192 rows) on the matrix
 // pipes (weight blocks through LDS and the transposing read), with the
 // same split into f32 partial sums W[splits][M][N] and the same second kernel; with splits == 1 one launch writes C
 // and W is not used.  N and K multiples of 8, K >= 256, one product.
 bool gemm_kn_rows_plan(long M, long N, long K, long batch, long* splits, long* k_per_split);
 int launch_gemm_kn_rows(void* stream, const void* A, const void* B, void* C, void* W, long M, long N, long K, long splits, long k_per_split,
-                        bool f16);
-// c = bf16(float(bf16(a b)) + float(r)) with r of c's shape, added in the product kernel's epilogue
-// (same bits as the product followed by an elementwise add).  Supported for the shapes the tiled
-// kernels take without split-K; gemm_bf16_residual_supported tells.  r_is_row: r is one row [N] added to every row
-// of c (a Linear layer's bias, tensor/src/nn/linear.rs:39-41) instead of a matrix of c's shape.
+                        bool f16, const void* add = nullptr, bool add_is_row = false);
+// (`add`, for both: a matrix of C's shape or, add_is_row, one row [N] of C's type, added to the rounded result where the
+// second kernel, or the single launch, writes it: the bits of the product followed by the elementwise add)
+// c = bf16(float(bf16(a b)) + float(r)) with r of c's shape, or (r_is_row) one row [N] added to every row of c (a
+// Linear layer's bias, tensor/src/nn/linear.rs:39-41): the same bits as the product followed by an elementwise add.  The
+// product takes the route launch_gemm_bf16 would take (same workspace: gemm_bf16[_nt]_workspace_bytes) and r is added by
+// whichever kernel writes the result: the tiled kernels' residual epilogue, the split-K reduction, the streaming kernels.
+// gemm_bf16_residual_supported: N and K multiples of 8 (the tiled kernels' shapes); with the second operand stored
+// [N, K] also every shape the streaming kernels take (gemm_bf16_bias_supported / _launchable tell, for either operand).
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch);
 int launch_gemm_bf16_residual(void* stream, const void* a, const void* b, const void* r, void* c, long M, long N, long K, long batch,
-                              bool b_transposed = false, bool r_is_row = false);
-// The product with a bias row, whichever kernel takes the shape: the streaming kernels (second operand [N, K], up to 64
-// rows) or the tiled kernels' residual epilogue with a row pitch of zero.  gemm_bf16_bias_supported tells where that is
-// the fast route (shapes that would be spread along K are left out: [K, N] with few rows, more than 64 rows with few
-// tiles); gemm_bf16_bias_launchable every shape launch_gemm_bf16_bias runs.
+                              bool b_transposed = false, bool r_is_row = false, void* workspace = nullptr, size_t workspace_bytes = 0);
 bool gemm_bf16_bias_supported(long M, long N, long K, long batch, bool b_transposed);
 bool gemm_bf16_bias_launchable(long M, long N, long K, long batch, bool b_transposed);
 int launch_gemm_bf16_bias(void* stream, const void* a, const void* b, const void* bias, void* c, long M, long N, long K, long batch,
-                          bool b_transposed);
+                          bool b_transposed, void* workspace = nullptr, size_t workspace_bytes = 0);
 // y[M, N] = bf16(float(bf16(x wt^T)) + float(add)) with wt [N, K] as a Linear layer holds it and `add` either one row
 // [N] (its bias) or a matrix [M, N] (a residual), for the shapes the streaming kernels take (up to 64 rows, K a
 // multiple of 8, one product): added where the kernel writes its result.  Same bits as the product followed by the add.

@@ -1450,9 +1450,9 @@ struct Scheduler {
             const TensorNode* rb = r;
             while (!rb->buffer && rb->kind == TKind::Reshape) rb = rb->src[0].get();
             if (!(rb->buffer || is_boundary_kind(rb) || fusable(rb))) continue;
-            // (a handful of rows against an [N, K] weight: the streaming kernels add the operand where they write their result)
-            const bool streamed = transposed_weight(mm) && gemm_nt_bias_streamed(M, N, K, batch);
-            if (!streamed && (!gemm_bf16_residual_supported(M, N, K, batch) || spread_or_streamed(mm, M, N, K, batch))) continue;
+            // (whichever kernel writes the product adds the operand: a tiled kernel's epilogue, the sum of a product spread
+            // along K, a streaming kernel for a handful of rows)
+            if (!gemm_bf16_bias_supported(M, N, K, batch, transposed_weight(mm) != nullptr)) continue;
             *other = r;
             return mm;
         }
@@ -1556,9 +1556,16 @@ struct Scheduler {
         MRK_TRY(weight_operand(mm, true, &wbuf, &nt));  // (the residual epilogue exists for exactly the shapes the B^T kernels take)
         MRK_TRY(materialize(r));
         auto out = new_buffer(n);
-        const std::vector<int64_t> params = batch == 1 ? std::vector<int64_t>{M, N, K} : std::vector<int64_t>{M, N, K, batch};
         const std::string kind = std::string(nt ? "gemm_bf16_nt_" : "gemm_bf16_") + (is_row ? "bias" : "residual");
-        MRK_TRY(builtin(kind.c_str(), params, {out, mm->hint_inputs[0]->buffer, wbuf, r->buffer}));
+        // few output tiles against a long K: scratch for the partial results, an intermediate of the plan like any other
+        const size_t ws = nt ? gemm_bf16_nt_workspace_bytes(M, N, K, batch) : gemm_bf16_workspace_bytes(M, N, K, batch);
+        if (ws) {
+            auto scratch = std::make_shared<Buffer>(dev->allocator, ws, BufferOptions());
+            MRK_TRY(builtin(kind.c_str(), {M, N, K, batch, static_cast<int64_t>(ws)}, {out, mm->hint_inputs[0]->buffer, wbuf, r->buffer, scratch}));
+        } else {
+            const std::vector<int64_t> params = batch == 1 ? std::vector<int64_t>{M, N, K} : std::vector<int64_t>{M, N, K, batch};
+            MRK_TRY(builtin(kind.c_str(), params, {out, mm->hint_inputs[0]->buffer, wbuf, r->buffer}));
+        }
         n->buffer = out;
         produced.push_back(n);
         return kOk;

@@ -47,14 +47,18 @@ int launch_gemm_bf16_static_ws(void* stream, int, const void*, const void*, void
 bool gemm_nt_bias_streamed(long M, long N, long K, long batch) { return batch == 1 && M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0; }
 bool gemm_bf16_bias_supported(long M, long N, long K, long batch, bool) { return M > 0 && N > 0 && K > 0 && batch > 0 && N % 8 == 0 && K % 8 == 0; }
 bool gemm_bf16_bias_launchable(long M, long N, long K, long batch, bool t) { return gemm_bf16_bias_supported(M, N, K, batch, t); }
-int launch_gemm_bf16_bias(void* stream, const void*, const void*, const void*, void*, long, long, long, long, bool b_transposed) {
+int launch_gemm_bf16_bias(void* stream, const void*, const void*, const void*, void*, long, long, long, long, bool b_transposed, void*, size_t) {
     mrk_shim_note_launch(stream, b_transposed ? "gemm_bf16_nt_bias" : "gemm_bf16_bias");
     return 0;
 }
 bool gemm_bf16_residual_supported(long M, long N, long K, long batch) {
     return M > 0 && N > 0 && K > 0 && batch > 0 && N % 8 == 0 && K % 8 == 0;
 }
-int launch_gemm_bf16_residual(void* stream, const void*, const void*, const void*, void*, long, long, long, long, bool b_transposed, bool) {
+int launch_gemm_bf16_residual(void* stream, const void*, const void*, const void*, void*, long, long, long, long, bool b_transposed, bool r_is_row, void*, size_t) {
+    if (r_is_row) {
+        mrk_shim_note_launch(stream, b_transposed ? "gemm_bf16_nt_bias" : "gemm_bf16_bias");
+        return 0;
+    }
     mrk_shim_note_launch(stream, b_transposed ? "gemm_bf16_nt_residual" : "gemm_bf16_residual");
     return 0;
 }

@@ -58,10 +58,7 @@ def test_attention_over_random_layouts(dev, seed):
 @pytest.mark.parametrize("seed", range(16))
 def test_residual_epilogue_random_shapes(dev, seed):
     rng = np.random.default_rng(7200 + seed)
-    while True:  # shapes the split-K kernel would take have no fused epilogue: draw again
-        M, N, K = int(rng.integers(1, 700)), int(rng.integers(1, 90)) * 8, int(rng.integers(1, 160)) * 8
-        if morok_amd._ffi.lib.mrk_hip_gemm_bf16_workspace_bytes(M, N, K, 1) == 0:
-            break
+    M, N, K = int(rng.integers(1, 700)), int(rng.integers(1, 90)) * 8, int(rng.integers(1, 160)) * 8
     a, b, r = (synth.normal_bf16(sh, 7200 + seed, i) for i, sh in enumerate(((M, K), (K, N), (M, N))))
     ba, bb, br = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (a, b, r))
     bc, bp = dev.buffer(M * N * 2), dev.buffer(M * N * 2)

@@ -243,14 +243,48 @@ def test_gemm_residual_epilogue(dev, oracle, shape):
     assert np.abs(gf - wf).max() <= 2e-2 * np.abs(wf).max()
 
 
-def test_gemm_residual_refuses_split_k_shapes(dev):
+@pytest.mark.parametrize("shape", [(4, 1024, 4096), (1, 4096, 4096), (16, 12288, 512), (40, 4096, 2048), (100, 264, 4104), (200, 520, 8192)])
+def test_gemm_residual_and_bias_where_the_product_is_spread_along_k(dev, shape):
+    """Few output tiles against a long K, either layout of the weight: the product runs as the plain one does (split-K
+    over the tiles, or the streaming kernels for a handful of rows) and the addend joins where the result is written,
+    with the bits of the product followed by the elementwise add.  A matrix of the result's shape and a bias row."""
+    M, N, K = shape
+    a, b = synth.normal_bf16((M, K), 3, 50), synth.normal_bf16((K, N), 3, 51)
+    r, bias = synth.normal_bf16((M, N), 3, 52), synth.normal_bf16((N,), 3, 53)
+    ba, bb, br, bbias = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (a, b, r, bias))
+    bbt = morok_amd.Buffer.from_numpy(np.ascontiguousarray(b.T), dev.device_id)
+    plain, plain_nt = dev.buffer(M * N * 2), dev.buffer(M * N * 2)
+    ops.gemm_bf16(ba, bb, plain, M, N, K, dev.device_id)
+    ops.gemm_bf16_nt(ba, bbt, plain_nt, M, N, K, dev.device_id)
+    p_kn, p_nt = synth.from_bf16(plain.copyout(np.uint16, (M, N))), synth.from_bf16(plain_nt.copyout(np.uint16, (M, N)))
+    bc = morok_amd.Buffer.from_numpy(np.full(M * N + 2048, 0x7FC0, np.uint16), dev.device_id)
+    ops.gemm_bf16_residual(ba, bb, br, bc, M, N, K, dev.device_id)
+    out = bc.copyout(np.uint16)
+    assert np.all(out[M * N:] == 0x7FC0)
+    assert np.array_equal(out[: M * N].reshape(M, N), synth.to_bf16(p_kn + synth.from_bf16(r)))
+    ops.linear_bf16(ba, bbt, bbias, bc, M, N, K, dev.device_id)
+    out = bc.copyout(np.uint16)
+    assert np.all(out[M * N:] == 0x7FC0)
+    assert np.array_equal(out[: M * N].reshape(M, N), synth.to_bf16(p_nt + synth.from_bf16(bias)[None, :]))
+    # as plan items with the plan's scratch, the other two combinations
+    ws = morok_amd._ffi.lib.mrk_hip_gemm_bf16_workspace_bytes(M, N, K, 1)
+    scratch = dev.buffer(max(ws, 16))
+    params, bufs = ([M, N, K, 1, ws], [scratch]) if ws else ([M, N, K], [])
+    morok_amd.Program.builtin("gemm_bf16_bias", params, dev.device_id).execute([bc, ba, bb, bbias] + bufs)
+    assert np.array_equal(bc.copyout(np.uint16)[: M * N].reshape(M, N), synth.to_bf16(p_kn + synth.from_bf16(bias)[None, :]))
+    if M <= 64:
+        morok_amd.Program.builtin("gemm_bf16_nt_residual", [M, N, K], dev.device_id).execute([bc, ba, bbt, br])
+        assert np.array_equal(bc.copyout(np.uint16)[: M * N].reshape(M, N), synth.to_bf16(p_nt + synth.from_bf16(r)))
+
+
+def test_gemm_residual_refusals(dev):
     a = dev.buffer(4 * 4096 * 2)
     b = dev.buffer(4096 * 1024 * 2)
     c = dev.buffer(4 * 1024 * 2)
     with pytest.raises(morok_amd.MorokHipError):
-        ops.gemm_bf16_residual(a, b, c, c, 4, 1024, 4096, dev.device_id)   # few tiles, long K: the split-K shape
-    with pytest.raises(morok_amd.MorokHipError):
         ops.gemm_bf16_residual(a, b, c, c, 4, 1020, 64, dev.device_id)     # N not a multiple of 8
+    with pytest.raises(morok_amd.MorokHipError):
+        ops.gemm_bf16_residual(a, b, c, c, 4, 1024, 60, dev.device_id)     # K not a multiple of 8
 
 
 # ---------------------------------------------------------------- gated epilogue (SwiGLU)
@@ -406,13 +440,16 @@ def test_linear_forward_with_bias(dev, oracle, shape):
 
 
 def test_linear_forward_with_bias_few_tiles_and_refusals(dev, oracle):
-    """More than 64 rows with few output tiles against a long K (the plain product would be spread along K): the
-    bias form runs unsplit; K not a multiple of 8 is refused."""
+    """More than 64 rows with few output tiles against a long K: the product is spread along K as the plain one is and
+    the bias is added where the partial results are summed; K not a multiple of 8 is refused."""
     M, N, K = 100, 264, 4104
     x, w, bias = synth.normal_bf16((M, K), 3, 43), synth.normal_bf16((N, K), 3, 44), synth.normal_bf16((N,), 3, 45)
     bx, bw, bb = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (x, w, bias))
-    by = dev.buffer(M * N * 2)
+    by, bp = dev.buffer(M * N * 2), dev.buffer(M * N * 2)
     ops.linear_bf16(bx, bw, bb, by, M, N, K, dev.device_id)
+    ops.gemm_bf16_nt(bx, bw, bp, M, N, K, dev.device_id)
+    want = synth.to_bf16(synth.from_bf16(bp.copyout(np.uint16, (M, N))) + synth.from_bf16(bias)[None, :])
+    assert np.array_equal(by.copyout(np.uint16, (M, N)), want)
     ref = synth.from_bf16(oracle.gemm_bf16(x, np.ascontiguousarray(w.T))) + synth.from_bf16(bias)[None, :]
     assert np.abs(synth.from_bf16(by.copyout(np.uint16, (M, N))) - ref).max() <= 2e-2 * np.abs(ref).max()
     with pytest.raises(morok_amd.MorokHipError):
