@@ -1088,6 +1088,8 @@ int launch_gemm_bf16_swiglu(void* stream, const void* A, const void* B, void* C,
     if (M <= 0 || F <= 0) return 0;
     if (!gemm_bf16_swiglu_supported(M, F, K, b_transposed)) return (int)hipErrorInvalidValue;
     if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(C)) % 16) return (int)hipErrorInvalidValue;
+    // a handful of rows against a [2F, K] weight: the gated form of the streaming kernel
+    if (b_transposed && gemm_nt_swiglu_streamed(M, F, K)) return launch_gemm_nt_swiglu_streamed(stream, A, B, C, M, F, K);
     hipStream_t s = static_cast<hipStream_t>(stream);
     (void)hipGetLastError();
     const long tn = (F + 127) / 128, tm = (M + kBM - 1) / kBM;

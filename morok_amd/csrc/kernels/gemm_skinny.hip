@@ -183,7 +183,7 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 #define MRK_LDS_PTR(T, p) ((__attribute__((address_space(3))) T*)(p))
 
-template <int kMT, int kRT, int kWaves, bool kF16>
+template <int kMT, int kRT, int kWaves, bool kF16, bool kGate = false>
 __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short* __restrict__ A, const unsigned short* __restrict__ Bt,
                                                              unsigned short* __restrict__ C, int M, int N, int K,
                                                              const unsigned short* __restrict__ add, long add_pitch) {
@@ -192,8 +192,11 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
     constexpr int kRowsPerCopy = 64 / kPieces;     // rows one copy instruction covers
     constexpr int kCopies = 16 / kRowsPerCopy;     // copy instructions per 16-row block
     constexpr int kBlockBytes = 16 * kPieces * 16; // one block's chunk in LDS
-    constexpr int kWaveBytes = (kRT + kMT) * kBlockBytes;
-    constexpr int kTiles = kRT * kMT;
+    // kGate: the weight is [2 N, K], gate rows first; the workgroup owns kRT blocks of gate rows and the kRT blocks of up
+    // rows N rows further down, and writes C[M, N] = silu(a gate) * (a up) (see the end of the kernel)
+    constexpr int kWB = kGate ? 2 * kRT : kRT;     // weight blocks per workgroup
+    constexpr int kWaveBytes = (kWB + kMT) * kBlockBytes;
+    constexpr int kTiles = kWB * kMT;
     constexpr int kSumBytes = kWaves * kTiles * 1024;
     constexpr int kLds = kWaves * kWaveBytes > kSumBytes ? kWaves * kWaveBytes : kSumBytes;
     static_assert(kLds <= 160 * 1024, "LDS");
@@ -202,23 +205,23 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
     const int li = lane & 15, g = lane >> 4;
     const long n0 = (long)blockIdx.x * (16 * kRT);
     A += (size_t)blockIdx.y * M * K;
-    Bt += (size_t)blockIdx.y * N * K;
+    Bt += (size_t)blockIdx.y * (kGate ? 2 : 1) * N * K;
     C += (size_t)blockIdx.y * M * N;
     const char* w_base = reinterpret_cast<const char*>(Bt + (size_t)n0 * K);
     const char* a_base = reinterpret_cast<const char*>(A);
     const unsigned lds_wave = (unsigned)(uintptr_t)MRK_LDS_PTR(char, smem) + wave * kWaveBytes;
     // copy side: lane -> (row of the copy, position in the row); byte offsets of its rows from the bases
     const int pos = lane % kPieces, rsub = lane / kPieces;
-    unsigned w_off[kRT][kCopies], a_off[kMT][kCopies], piece_of[kCopies];
+    unsigned w_off[kWB][kCopies], a_off[kMT][kCopies], piece_of[kCopies];
 #pragma unroll
     for (int i = 0; i < kCopies; i++) {
         const int r = i * kRowsPerCopy + rsub;
         piece_of[i] = (unsigned)(pos ^ ((r >> 1) & 7));
 #pragma unroll
-        for (int t = 0; t < kRT; t++) {
-            long n = n0 + t * 16 + r;
+        for (int t = 0; t < kWB; t++) {
+            long n = n0 + (t % kRT) * 16 + r;
             n = n < N ? n : N - 1;  // a row past the end repeats the last one (not written)
-            w_off[t][i] = (unsigned)(n - n0) * (unsigned)K * 2u;
+            w_off[t][i] = (unsigned)(n - n0 + (t >= kRT ? N : 0)) * (unsigned)K * 2u;
         }
 #pragma unroll
         for (int t = 0; t < kMT; t++) {
@@ -227,9 +230,9 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
             a_off[t][i] = (unsigned)m * (unsigned)K * 2u;
         }
     }
-    f32x4 acc[kRT][kMT];
+    f32x4 acc[kWB][kMT];
 #pragma unroll
-    for (int r = 0; r < kRT; r++)
+    for (int r = 0; r < kWB; r++)
 #pragma unroll
         for (int m = 0; m < kMT; m++) acc[r][m] = f32x4{0.f, 0.f, 0.f, 0.f};
     // read side: row li of a block, piece 4 s + g of the chunk at position (4 s + g) ^ key(li)
@@ -251,7 +254,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
             unsigned piece = (unsigned)p0 + piece_of[i];
             if (!full) piece = piece < (unsigned)pieces ? piece : (unsigned)pieces - 1u;  // any valid piece: zeroed below
 #pragma unroll
-            for (int t = 0; t < kRT; t++)
+            for (int t = 0; t < kWB; t++)
                 asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
                              :
                              : "s"(lds_wave + t * kBlockBytes + i * 1024), "v"(w_off[t][i] + piece * 16u), "s"(w_base)
@@ -260,7 +263,7 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
             for (int t = 0; t < kMT; t++)
                 asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                              :
-                             : "s"(lds_wave + (kRT + t) * kBlockBytes + i * 1024), "v"(a_off[t][i] + piece * 16u), "s"(a_base)
+                             : "s"(lds_wave + (kWB + t) * kBlockBytes + i * 1024), "v"(a_off[t][i] + piece * 16u), "s"(a_base)
                              : "m0", "memory");
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -271,11 +274,11 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
             u32x4 x[kMT];
 #pragma unroll
             for (int t = 0; t < kMT; t++) {
-                x[t] = *MRK_LDS_PTR(u32x4, rd_row + (kRT + t) * kBlockBytes + po);
+                x[t] = *MRK_LDS_PTR(u32x4, rd_row + (kWB + t) * kBlockBytes + po);
                 if (!full) x[t] = in ? x[t] : u32x4{0u, 0u, 0u, 0u};
             }
 #pragma unroll
-            for (int r = 0; r < kRT; r++) {
+            for (int r = 0; r < kWB; r++) {
                 u32x4 w = *MRK_LDS_PTR(u32x4, rd_row + r * kBlockBytes + po);
                 if (!full) w = in ? w : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
@@ -293,12 +296,12 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
     __syncthreads();
     f32x4* partial = reinterpret_cast<f32x4*>(smem);  // [kWaves][kTiles][64]
 #pragma unroll
-    for (int r = 0; r < kRT; r++)
+    for (int r = 0; r < kWB; r++)
 #pragma unroll
         for (int m = 0; m < kMT; m++) partial[(wave * kTiles + r * kMT + m) * 64 + lane] = acc[r][m];
     __syncthreads();
     const bool vec = (N & 3) == 0;
-    for (int e = threadIdx.x; e < kTiles * 64; e += kWaves * 64) {
+    for (int e = threadIdx.x; e < kRT * kMT * 64; e += kWaves * 64) {
         const int tile = e >> 6, l = e & 63;
         f32x4 s = partial[tile * 64 + l];
 #pragma unroll
@@ -307,8 +310,22 @@ __global__ __launch_bounds__(kWaves * 64) void gemm_nt_rows(const unsigned short
         const long n = n0 + r * 16 + 4 * (l >> 4);
         if (m >= M || n >= N) continue;
         unsigned short o[4];
+        if constexpr (kGate) {
+            // the up block's sums, then x * sigmoid(x) * y on the two products rounded as separate kernels would leave them,
+            // in f32 with one rounding: the arithmetic of the generated elementwise kernel this replaces
+            f32x4 u = partial[(tile + kRT * kMT) * 64 + l];
 #pragma unroll
-        for (int i = 0; i < 4; i++) o[i] = round_out<kF16>(s[i], add && n + i < N ? add + (size_t)m * add_pitch : nullptr, n + i);
+            for (int w = 1; w < kWaves; w++) u += partial[(w * kTiles + tile + kRT * kMT) * 64 + l];
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float g = __builtin_bit_cast(float, (unsigned)round_bf16(s[i]) << 16);
+                const float y = __builtin_bit_cast(float, (unsigned)round_bf16(u[i]) << 16);
+                o[i] = round_bf16((g * (1.0f / (1.0f + exp2f(g * -1.44269502f)))) * y);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[i] = round_out<kF16>(s[i], add && n + i < N ? add + (size_t)m * add_pitch : nullptr, n + i);
+        }
         unsigned short* dst = C + (size_t)m * N + n;
         if (vec) {
             *reinterpret_cast<u32x2*>(dst) = u32x2{(unsigned)o[0] | ((unsigned)o[1] << 16), (unsigned)o[2] | ((unsigned)o[3] << 16)};
@@ -715,6 +732,47 @@ int launch_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M,
 
 int launch_gemm_nt_rows(void* stream, const void* A, const void* Bt, void* C, long M, long N, long K, long batch, bool f16) {
     return launch_nt_rows(stream, A, Bt, C, M, N, K, batch, f16, nullptr, 0);
+}
+
+// c[M, F] = silu(a gate) * (a up) over a weight [2 F, K] (gate rows first) for the shapes the matrix-pipe kernel takes,
+// bf16: the gated form of gemm_nt_rows.  Row offsets of the up blocks from the workgroup's first row are 32-bit.
+bool gemm_nt_swiglu_streamed(long M, long F, long K) {
+    return gemm_nt_rows_supported(M, 2 * F, K, 1) && (F + 96) * K * 2 < (1L << 32);
+}
+
+int launch_gemm_nt_swiglu_streamed(void* stream, const void* A, const void* Bt, void* C, long M, long F, long K) {
+    using namespace mrk::dev;
+    if (!gemm_nt_swiglu_streamed(M, F, K)) return (int)hipErrorInvalidValue;
+    if ((reinterpret_cast<uintptr_t>(A) | reinterpret_cast<uintptr_t>(Bt)) % 16 || reinterpret_cast<uintptr_t>(C) % 8) return (int)hipErrorInvalidValue;
+    (void)hipGetLastError();
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const unsigned short* a = static_cast<const unsigned short*>(A);
+    const unsigned short* b = static_cast<const unsigned short*>(Bt);
+    unsigned short* c = static_cast<unsigned short*>(C);
+    const int mt = (int)((M + 15) / 16);
+    // gate and up blocks together: as many weight blocks per workgroup as the plain kernel would take, in pairs
+    int rt = rows_blocks_per_group(2 * F, mt) / 2;
+    rt = rt < 1 ? 1 : rt > 3 ? 3 : rt;
+    if (2 * rt * mt > 18) rt = mt == 4 ? 2 : rt;
+#define MRK_GATE(MT, RT)                                                                                                       \
+    do {                                                                                                                       \
+        const dim3 grid((unsigned)((F + 16 * RT - 1) / (16 * RT)), 1);                                                         \
+        gemm_nt_rows<MT, RT, 8, false, true><<<grid, 512, 0, s>>>(a, b, c, (int)M, (int)F, (int)K, nullptr, 0);                \
+    } while (0)
+#define MRK_GATE_MT(MT)                \
+    do {                               \
+        if (rt == 1) MRK_GATE(MT, 1);  \
+        else if (rt == 2) MRK_GATE(MT, 2); \
+        else MRK_GATE(MT, 3);          \
+    } while (0)
+    if (mt == 1) MRK_GATE_MT(1);
+    else if (mt == 2) MRK_GATE_MT(2);
+    else if (mt == 3) MRK_GATE_MT(3);
+    else if (rt == 1) MRK_GATE(4, 1);
+    else MRK_GATE(4, 2);
+#undef MRK_GATE_MT
+#undef MRK_GATE
+    return (int)hipGetLastError();
 }
 
 bool gemm_nt_bias_streamed(long M, long N, long K, long batch) {

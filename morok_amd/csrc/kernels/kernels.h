@@ -73,6 +73,10 @@ int launch_gemm_bf16_bias(void* stream, const void* a, const void* b, const void
 // y[M, N] = bf16(float(bf16(x wt^T)) + float(add)) with wt [N, K] as a Linear layer holds it and `add` either one row
 // [N] (its bias) or a matrix [M, N] (a residual), for the shapes the streaming kernels take (up to 64 rows, K a
 // multiple of 8, one product): added where the kernel writes its result.  Same bits as the product followed by the add.
+// c[M, F] = silu(a gate) * (a up) over a weight [2 F, K] (gate rows first) with up to 64 rows of a, bf16: the gate applied where
+// the matrix-pipe streaming kernel writes its result (the arithmetic of the generated elementwise kernel it replaces).
+bool gemm_nt_swiglu_streamed(long M, long F, long K);
+int launch_gemm_nt_swiglu_streamed(void* stream, const void* A, const void* Bt, void* C, long M, long F, long K);
 bool gemm_nt_bias_streamed(long M, long N, long K, long batch);
 int launch_gemm_nt_bias_streamed(void* stream, const void* A, const void* Bt, const void* add, void* C, long M, long N, long K, bool f16,
                                  bool add_is_row = true);

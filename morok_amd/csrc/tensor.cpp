@@ -1485,7 +1485,9 @@ struct Scheduler {
             if (!used(mm, 2) || !used(gate, 2) || !used(up, 1) || !used(sw, 1)) continue;
             int64_t Mx, N2, K, batch;
             matmul_extents(mm, &Mx, &N2, &K, &batch);
-            if (batch != 1 || Mx != M || N2 != 2 * F || !gemm_bf16_swiglu_supported(M, F, K) || spread_or_streamed(mm, M, N2, K, 1)) continue;
+            if (batch != 1 || Mx != M || N2 != 2 * F || !gemm_bf16_swiglu_supported(M, F, K)) continue;
+            // (a handful of rows against a [2F, K] weight: the streaming kernel has a gated form of its own)
+            if (spread_or_streamed(mm, M, N2, K, 1) && !(transposed_weight(mm) && gemm_nt_swiglu_streamed(M, F, K))) continue;
             return mm;
         }
         return nullptr;

@@ -44,6 +44,7 @@ int launch_gemm_bf16_static_ws(void* stream, int, const void*, const void*, void
     mrk_shim_note_launch(stream, "gemm_bf16");
     return 0;
 }
+bool gemm_nt_swiglu_streamed(long M, long F, long K) { return M >= 1 && M <= 64 && F >= 1 && K >= 8 && K % 8 == 0; }
 bool gemm_nt_bias_streamed(long M, long N, long K, long batch) { return batch == 1 && M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0; }
 bool gemm_bf16_bias_supported(long M, long N, long K, long batch, bool) { return M > 0 && N > 0 && K > 0 && batch > 0 && N % 8 == 0 && K % 8 == 0; }
 bool gemm_bf16_bias_launchable(long M, long N, long K, long batch, bool t) { return gemm_bf16_bias_supported(M, N, K, batch, t); }

@@ -155,6 +155,63 @@ def test_linear_decode_with_residual_is_one_kernel(T, oracle):
     assert np.abs(synth.from_bf16(got) - ref).max() <= 2e-2 * np.abs(ref).max()
 
 
+@pytest.mark.parametrize("shape", [(1, 4096, 1024), (4, 1024, 512), (16, 11008, 4096), (33, 520, 264), (64, 2816, 1024), (7, 136, 72), (48, 4104, 520)])
+def test_streamed_gated_product(dev, T, shape):
+    """silu(x @ Wg.T) * (x @ Wu.T) over a weight [2F, K] (gate rows first) for a handful of rows: the gated form of the
+    streaming kernel ("gemm_bf16_nt_swiglu").  On small-integer data both products are exact, so the result must be
+    the generated elementwise kernel's on the exact products, bit for bit; on normal data the two may differ where a
+    product's f32 sum rounds the other way (another summation order), i.e. by roundings of single elements."""
+    from morok_amd import uop
+
+    M, F, K = shape
+    rng = np.random.default_rng(11)
+    for exact in (True, False):
+        if exact:
+            x = synth.to_bf16(rng.integers(-2, 3, size=(M, K)).astype(np.float32))
+            w = synth.to_bf16(rng.integers(-2, 3, size=(2 * F, K)).astype(np.float32))
+        else:
+            x, w = synth.normal_bf16((M, K), 13, 40), (synth.from_bf16(synth.normal_bf16((2 * F, K), 13, 41)) / np.sqrt(K)).astype(np.float32)
+            w = synth.to_bf16(w)
+        bx, bw = morok_amd.Buffer.from_numpy(x, dev.device_id), morok_amd.Buffer.from_numpy(w, dev.device_id)
+        bg = dev.buffer((M * F + 2048) * 2)
+        bg.copyin(np.full(M * F + 2048, 0x7FC0, np.uint16))
+        morok_amd.Program.builtin("gemm_bf16_nt_swiglu", [M, F, K], dev.device_id).execute([bg, bx, bw])
+        out = bg.copyout(np.uint16)
+        assert np.all(out[M * F:] == 0x7FC0)
+        got = out[: M * F].reshape(M, F)
+        # the unfused pair: the packed product, then the generated kernel over its two halves
+        bp = dev.buffer(M * 2 * F * 2)
+        ops.gemm_bf16_nt(bx, bw, bp, M, 2 * F, K, dev.device_id)
+        p = T.Tensor.from_numpy(bp.copyout(np.uint16, (M, 2 * F)), uop.BF16)
+        want = p.try_shrink([(0, M), (0, F)]).silu().try_mul(p.try_shrink([(0, M), (F, 2 * F)])).to_numpy()
+        if exact:
+            assert np.array_equal(got, want)
+        else:
+            g, wv = synth.from_bf16(got), synth.from_bf16(want)
+            assert np.all(np.isfinite(g))
+            assert np.mean(got == want) >= 0.97
+            assert np.all(np.abs(g - wv) <= np.abs(wv) * 2.0 ** -6 + 1e-3 * np.abs(wv).max())
+
+
+def test_linear_decode_gate_is_one_kernel(T, oracle):
+    """The gated feed-forward half of a decode step over Linear-layout weights: one streaming kernel."""
+    from morok_amd import uop
+
+    M, K, F = 8, 1024, 1536
+    x, w13 = synth.normal_bf16((M, K), 13, 42), synth.normal_bf16((2 * F, K), 13, 43)
+    tx, tw = T.Tensor.from_numpy(x, uop.BF16), T.Tensor.from_numpy(w13, uop.BF16)
+    T.set_fusion(True)
+    gu = tx.linear(tw)
+    g = gu.try_shrink([(0, M), (0, F)]).silu().try_mul(gu.try_shrink([(0, M), (F, 2 * F)]))
+    got = g.to_numpy()
+    assert g.kernels() == [f"gemm_bf16_nt_swiglu_{M}_{F}_{K}"]
+    ref = oracle.gemm_bf16(x, np.ascontiguousarray(w13.T))
+    gate, up = synth.from_bf16(ref[:, :F]), synth.from_bf16(ref[:, F:])
+    with np.errstate(over="ignore"):
+        want = gate / (1.0 + np.exp(-gate)) * up
+    assert np.abs(synth.from_bf16(got) - want).max() <= 2e-2 * np.abs(want).max()
+
+
 def test_skinny_refusals(dev):
     a, b, c = dev.buffer(72 * 4096 * 2), dev.buffer(4096 * 1024 * 2), dev.buffer(72 * 1024 * 2)
     with pytest.raises(morok_amd.MorokHipError):
