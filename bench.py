@@ -40,7 +40,8 @@ PROFILE_OF = {"softmax": "softmax_rows_in_regs_8192x8192_f32.txt", "gemm": "gemm
               "flash": "flash_fwd_d128_causal_8x32x4096x128.txt", "decoder": "decoder_block_4x2048_h4096.txt",
               "generated_tc": "generated_tensor_core_gemm_4096cubed.txt", "matmul_f32": "generated_f32_matmul_1024cubed.txt",
               "gemm_f16": "gemm_f16_tile256_4096cubed.txt", "flash_options": "flash_fwd_ext_d128_8x32x4096x128.txt",
-              "linear_decode": "gemm_nt_skinny_1x12288x4096_x8.txt", "linear_decode_16": "gemm_nt_rows_16x12288x4096_x8.txt"}
+              "linear_decode": "gemm_nt_skinny_1x12288x4096_x8.txt", "linear_decode_16": "gemm_nt_rows_16x12288x4096_x8.txt",
+              "decoder_decode": "decoder_block_decode_16tokens_linear_layout.txt"}
 
 
 def _profiled_traffic(workload, kernel):
@@ -462,7 +463,7 @@ def bench_decoder_decode(m, dev, steps, warmup, cpu):
            "blocks_per_step": layers, "us_per_block": ms * 1e3 / layers, "tokens_per_s": B * S * layers / (ms * 1e-3), "kernels": len(prof),
            "gemm_us": 1e3 * sum(t for n, t in prof if n.startswith("gemm_bf16")), "other_us": 1e3 * sum(t for n, t in prof if not n.startswith("gemm_bf16")),
            "roofline": {"bound": "hbm", "achieved": gbs, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbs / HBM_PEAK_GBS, "traffic": None,
-                        "traffic_source": "per-kernel figures in profiles/" + PROFILE_OF["linear_decode_16"],
+                        "traffic_source": "per-kernel figures in profiles/" + PROFILE_OF["decoder_decode"],
                         "kernel": "gemm_nt_rows (4 of the %d kernels)" % len(prof), "algorithmic_bytes_per_launch": weight_bytes}}
     if cpu:
         from tests.oracle_lib import Oracle
