@@ -208,6 +208,8 @@ void mrk_hip_program_destroy(mrk_program* p);
  *   "flash_fwd_bf16_strided"  params = {B, H, Sq, Sk, D, causal, f32 bits of scale, element offsets
  *                     of q k v o into their buffers (4), (batch, head, row) element strides of
  *                     q k v o (12)}                                  buffers = {o, q, k, v}
+ *                     (both: optionally one more parameter, the bytes of a scratch buffer that follows v:
+ *                     mrk_hip_flash_attn_workspace_bytes, for a key sequence split over workgroups)
  * Buffer order follows the reference's PARAM numbering: outputs first. */
 int mrk_hip_program_builtin(int device_id, const char* kind, const int64_t* params, size_t nparams, mrk_program** out);
 
@@ -537,9 +539,17 @@ int mrk_hip_gemm_bf16_rope(int device_id, const void* a, const void* b, const vo
  * given and no attn_mask / softcap.  q [B,H,Sq,D], k and v [B,H,Sk,D], o [B,H,Sq,D], row-major
  * bf16, D = 256, 128 or 64 (other head dims: INVALID_ARGUMENT here, the composed graph through the tensor
  * API), scale > 0 (the reference default is 1/sqrt(D), transformer.rs:90-91).
- * Causal rule of the reference: key j is visible to query i iff j <= i (transformer.rs:103-109). */
+ * Causal rule of the reference: key j is visible to query i iff j <= i (transformer.rs:103-109).
+ * Up to 16 queries without the causal rule against 256 keys and more (the decode step of a model that keeps
+ * its keys and values: the same function of the reference, called with a short q) take a kernel that streams
+ * K and V once and splits the key sequence over workgroups where (batch, head) pairs alone would not fill the
+ * chip; the ranges' partial results (f32) are merged by a second kernel in a fixed order.  This call and the
+ * strided one take that scratch from the device's allocator; a builtin Program gets it as a fifth buffer of
+ * mrk_hip_flash_attn_workspace_bytes (0: the shape needs none), its size as one more parameter, and runs the
+ * shape as one key range per pair without it. */
 int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
                                 int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal);
+size_t mrk_hip_flash_attn_workspace_bytes(int64_t batch, int64_t heads, int64_t sq, int64_t sk, int64_t d, int causal);
 /* The same over operands given as views of larger buffers, the way the reference's movement
  * ops hand them over without a copy (tensor/src/transformer.rs:78-137 takes any view; permute /
  * shrink / expand never move data there): strides = (batch, head, row) element strides of q, k,

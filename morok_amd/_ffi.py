@@ -150,6 +150,7 @@ _SIGS = {
     "mrk_hip_gemm_bf16_noalloc": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int64]),
     "mrk_hip_gemm_bf16_noalloc_capacity": (C.c_size_t, []),
     "mrk_hip_gemm_bf16_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64, C.c_int64]),
+    "mrk_hip_flash_attn_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.c_int]),
     "mrk_hip_gemm_bf16_variant": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,
                                             C.c_int64, C.c_int]),
     "mrk_hip_gemm_bf16_residual": (C.c_int, [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64,

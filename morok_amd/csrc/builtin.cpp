@@ -213,32 +213,42 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                       }));
         return kOk;
     }
-    if (k == "flash_fwd_bf16") {
-        MRK_TRY(need(6));
+    if (k == "flash_fwd_bf16") {  // {BH, Sq, Sk, D, causal, scale bits[, workspace bytes]}; buffers {o, q, k, v[, scratch]}
+        if (nparams != 6 && nparams != 7)
+            return failf(kInvalidArgument, "builtin '%s' takes 6 or 7 parameters, got %zu", k.c_str(), nparams);
+        if (p.size() < 7) p.push_back(0);
+        if (p[6] < 0) return fail(kInvalidArgument, "flash_fwd_bf16: negative workspace size");
         if (p[0] < 0 || p[1] < 0 || p[2] <= 0 || (p[3] != 256 && p[3] != 128 && p[3] != 64))
             return fail(kInvalidArgument, "flash_fwd_bf16: bad shape (params BH, Sq, Sk, D = 256, 128 or 64, causal, scale bits)");
         std::string name = "flash_fwd_bf16_" + std::to_string(p[0]) + "_" + std::to_string(p[1]) + "_" + std::to_string(p[2]) + (p[3] != 128 ? "_d" + std::to_string(p[3]) : "");
-        out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
-                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+        // a fifth buffer of p[6] bytes: scratch for the partial results of a key sequence split over workgroups
+        const bool ws = p[6] > 0;
+        out->reset(new BuiltinProgram(device_id, stream, name + (ws ? "_splitkv" : ""), ws ? 5 : 4, p,
+                                      [ws](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
                                           uint32_t bits = static_cast<uint32_t>(q[5]);
                                           float scale;
                                           std::memcpy(&scale, &bits, 4);
                                           return launch_flash_fwd_bf16(s, b[1], b[2], b[3], b[0], q[0], q[1], q[2], q[3],
-                                                                       scale, q[4] != 0);
+                                                                       scale, q[4] != 0, ws ? b[4] : nullptr, ws ? static_cast<size_t>(q[6]) : 0);
                                       }));
         return kOk;
     }
     if (k == "flash_fwd_bf16_strided") {
         // params: B, H, Sq, Sk, D, causal, scale bits, element offsets of q k v o into their
         // buffers (4), then (batch, head, row) element strides of q k v o (12)
-        MRK_TRY(need(23));
+        // optionally a 24th: workspace bytes, with a fifth buffer of that size (scratch for a split key sequence)
+        if (nparams != 23 && nparams != 24)
+            return failf(kInvalidArgument, "builtin '%s' takes 23 or 24 parameters, got %zu", k.c_str(), nparams);
+        if (p.size() < 24) p.push_back(0);
+        if (p[23] < 0) return fail(kInvalidArgument, "flash_fwd_bf16_strided: negative workspace size");
         if (p[0] < 0 || p[1] < 0 || p[2] < 0 || p[3] <= 0 || (p[4] != 256 && p[4] != 128 && p[4] != 64))
             return fail(kInvalidArgument, "flash_fwd_bf16_strided: bad shape (params B, H, Sq, Sk, D = 256, 128 or 64, causal, scale bits, 4 offsets, 12 strides)");
         for (int i = 7; i < 23; i++)
             if (p[i] < 0 || p[i] % 8) return fail(kInvalidArgument, "flash_fwd_bf16_strided: offsets and strides must be non-negative multiples of 8 elements");
         std::string name = "flash_fwd_bf16_strided_" + std::to_string(p[0] * p[1]) + "_" + std::to_string(p[2]) + "_" + std::to_string(p[3]) + (p[4] != 128 ? "_d" + std::to_string(p[4]) : "");
-        out->reset(new BuiltinProgram(device_id, stream, name, 4, p,
-                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+        const bool ws = p[23] > 0;
+        out->reset(new BuiltinProgram(device_id, stream, name + (ws ? "_splitkv" : ""), ws ? 5 : 4, p,
+                                      [ws](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
                                           uint32_t bits = static_cast<uint32_t>(q[6]);
                                           float scale;
                                           std::memcpy(&scale, &bits, 4);
@@ -248,7 +258,8 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                               return static_cast<char*>(b[buf]) + q[7 + which] * 2;
                                           };
                                           return launch_flash_fwd_bf16_strided(s, at(1, 0), at(2, 1), at(3, 2), at(0, 3), q[0], q[1],
-                                                                               q[2], q[3], q[4], scale, q[5] != 0, strides);
+                                                                               q[2], q[3], q[4], scale, q[5] != 0, strides, ws ? b[4] : nullptr,
+                                                                               ws ? static_cast<size_t>(q[23]) : 0);
                                       }));
         return kOk;
     }

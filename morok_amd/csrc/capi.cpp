@@ -1035,9 +1035,21 @@ int mrk_hip_flash_attn_fwd_bf16(int device_id, const void* q, const void* k, con
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_flash_fwd_bf16(dv->allocator->stream(), q, k, v, o, batch * heads, sq, sk, d, scale, causal ? 1 : 0),
-            "flash_attn_fwd launch");
+    // a handful of queries against many keys: the key sequence is split over workgroups, the ranges' partial
+    // results go through scratch from the device's allocator (as for the products' split-K)
+    const size_t ws = flash_fwd_workspace_bytes(batch * heads, sq, sk, d, causal ? 1 : 0);
+    RawBuffer scratch;
+    BufferOptions so;
+    if (ws) MRK_TRY(dv->allocator->alloc(ws, so, &scratch));
+    const int rc = launch_flash_fwd_bf16(dv->allocator->stream(), q, k, v, o, batch * heads, sq, sk, d, scale, causal ? 1 : 0,
+                                         ws ? scratch.ptr : nullptr, ws);
+    if (ws) dv->allocator->free(scratch, so);
+    MRK_HIP(rc, "flash_attn_fwd launch");
     return kOk;
+}
+size_t mrk_hip_flash_attn_workspace_bytes(int64_t batch, int64_t heads, int64_t sq, int64_t sk, int64_t d, int causal) {
+    if (batch <= 0 || heads <= 0) return 0;
+    return flash_fwd_workspace_bytes(batch * heads, sq, sk, d, causal ? 1 : 0);
 }
 
 int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
@@ -1070,8 +1082,14 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_flash_fwd_bf16_strided(dv->allocator->stream(), q, k, v, o, batch, heads, sq, sk, d, scale, causal ? 1 : 0, st),
-            "flash_attn_fwd_strided launch");
+    const size_t ws = flash_fwd_workspace_bytes(batch * heads, sq, sk, d, causal ? 1 : 0);
+    RawBuffer scratch;
+    BufferOptions so;
+    if (ws) MRK_TRY(dv->allocator->alloc(ws, so, &scratch));
+    const int rc = launch_flash_fwd_bf16_strided(dv->allocator->stream(), q, k, v, o, batch, heads, sq, sk, d, scale, causal ? 1 : 0, st,
+                                                 ws ? scratch.ptr : nullptr, ws);
+    if (ws) dv->allocator->free(scratch, so);
+    MRK_HIP(rc, "flash_attn_fwd_strided launch");
     return kOk;
 }
 

@@ -1,0 +1,347 @@
+// Attention for a handful of queries against a long key sequence (a decode step over a key/value cache,
+// tensor/src/transformer.rs:78-137 with Sq of 1 to 16): O = softmax(Q K^T * scale) V is a stream over K and V,
+// 4 * Sk * D bytes per (batch, head) against a few flops per byte, and with few (batch, head) pairs the kernel that
+// gives every pair one workgroup leaves most of the chip without work.  Here the key sequence is split as well:
+// grid = (splits, batch * heads), a workgroup owns a contiguous range of keys, its waves take the range's 32-key
+// chunks in turn.  A wave copies its chunk of K and of V (32 rows each) with direct global -> LDS loads into a
+// region of its own (1 KB per instruction, non-temporal: every byte is read once), so the loop has no barrier,
+// and what streams is bounded by the bytes in flight per CU, i.e. by what the LDS holds.
+// S^T = K Q^T on v_mfma_f32_16x16x32_bf16 (operand A: 16 keys x 32 d read back from LDS, rows swizzled by the key
+// so that the 16 rows of a read fall into different banks; operand B: the queries, 16 columns, loaded once;
+// queries beyond Sq repeat the last one and are not written): a lane then holds, for query l % 16, the keys
+// 4 * (l / 16) + 0..3 of each of the chunk's two 16-key blocks.  Those eight values, exponentiated against the
+// running maximum and rounded to bf16, are directly the lane's operand of O^T += V^T P^T if the instruction's
+// eight k-slots of lane group g are taken to be exactly those keys; V's side follows through the transposing
+// LDS read (ds_read_b64_tr_b16: lane j of a 16-lane group receives column j of the four rows the group's lanes
+// point at), pointed at rows 4 g + 0..3 of either block.  Running maximum and sum per query as in any online
+// softmax; a query's maximum sits in four lanes (l % 16 equal), two exchanges per chunk.
+// At the end the waves' (maximum, sum, O) meet in LDS and are merged in a fixed order; with one split the
+// workgroup writes O, otherwise f32 partial results W[split][batch * head][16][D + 2] (the unnormalised O, then
+// maximum and sum), which flash_decode_merge folds the same way.  Results do not depend on scheduling.
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace mrk::dev {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+#define MRK_FD_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
+
+constexpr int kChunkKeys = 32;  // keys a wave handles per step
+constexpr int kMaxQueries = 16;
+
+struct DecodeLayout {
+    long long q_batch, q_head, k_batch, k_head, v_batch, v_head, o_batch, o_head;  // element strides
+    unsigned q_row, k_row, v_row, o_row;                                           // byte strides of a row
+    int heads;
+};
+
+template <int kD>
+constexpr int decode_waves() {
+    return kD == 256 ? 4 : 8;  // a wave's region is 4 * 32 * kD bytes: 128 KB of LDS for 128 and 256, 64 KB for 64
+}
+
+template <int kD>
+__global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
+    const unsigned short* __restrict__ Q, const unsigned short* __restrict__ K, const unsigned short* __restrict__ V,
+    unsigned short* __restrict__ O, float* __restrict__ W, int Sq, int Sk, int keys_per_split, float scale_log2e, DecodeLayout lay) {
+    constexpr int kWaves = decode_waves<kD>();
+    constexpr int kRowBytes = kD * 2;
+    constexpr int kPieces = kD / 8;                      // 16-byte pieces of a row
+    constexpr int kRowsPerCopy = 1024 / kRowBytes;       // 8, 4, 2
+    constexpr int kCopies = kChunkKeys / kRowsPerCopy;   // per operand and chunk
+    constexpr int kOperandBytes = kChunkKeys * kRowBytes;
+    constexpr int kWaveBytes = 2 * kOperandBytes;
+    constexpr int kSteps = kD / 32;                      // matrix steps of a score block
+    constexpr int kColBlocks = kD / 16;                  // 16-column blocks of O
+    constexpr int kPartBytes = kColBlocks * 1024 + 128;  // a wave's O blocks, then maximum and sum of the 16 queries
+    constexpr int kLds = kWaves * kWaveBytes > kWaves * kPartBytes ? kWaves * kWaveBytes : kWaves * kPartBytes;
+    static_assert(kLds <= 160 * 1024, "LDS");
+    __shared__ __attribute__((aligned(1024))) char smem[kLds];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int jl = lane & 15, blk = lane >> 4;
+    const int bh = blockIdx.y, b = bh / lay.heads, h = bh % lay.heads;
+    const int k_begin = blockIdx.x * keys_per_split;
+    const int k_end = k_begin + keys_per_split < Sk ? k_begin + keys_per_split : Sk;
+    const unsigned lds_k = (unsigned)(uintptr_t)MRK_FD_LDS(char, smem) + wave * kWaveBytes;
+    const unsigned lds_v = lds_k + kOperandBytes;
+    const char* k_head = reinterpret_cast<const char*>(K + b * lay.k_batch + h * lay.k_head);
+    const char* v_head = reinterpret_cast<const char*>(V + b * lay.v_batch + h * lay.v_head);
+
+    // the queries: operand B, query jl (the last one again beyond Sq), eight d at 32 s + 8 blk
+    u32x4 qf[kSteps];
+    {
+        const int qi = jl < Sq ? jl : Sq - 1;
+        const char* qrow = reinterpret_cast<const char*>(Q + b * lay.q_batch + h * lay.q_head) + (size_t)qi * lay.q_row;
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) qf[s] = *reinterpret_cast<const u32x4*>(qrow + 64 * s + 16 * blk);
+    }
+    // copy side: copy i covers rows i * kRowsPerCopy ..; lane -> row rsub of them, position pos of the row in LDS.
+    // K: position p holds piece p ^ key(row), key = row & 15 (rows of 256 bytes and more) or (row >> 1) & 7
+    // (128-byte rows, two to a bank period).  V: 32-byte granule G at granule G ^ key(row), key = row & 7
+    // or (row >> 1) & 3.
+    const int pos = lane % kPieces, rsub = lane / kPieces;
+    unsigned k_piece[kCopies], v_piece[kCopies];
+#pragma unroll
+    for (int i = 0; i < kCopies; i++) {
+        const int r = i * kRowsPerCopy + rsub;
+        const int kk = kD >= 128 ? (r & 15) : ((r >> 1) & 7);
+        const int vk = kD >= 128 ? (r & 7) : ((r >> 1) & 3);
+        k_piece[i] = (unsigned)(pos ^ kk) * 16u;
+        v_piece[i] = (unsigned)((((pos >> 1) ^ vk) << 1) | (pos & 1)) * 16u;
+    }
+    // read side, K: row jl of a 16-key block, piece 4 s + blk of it
+    const unsigned kx = (unsigned)(kD >= 128 ? jl : ((jl >> 1) & 7));
+    const unsigned rd_k = lds_k + jl * kRowBytes;
+    // read side, V: rows 4 blk + (jl >> 2) of either block, 8-byte unit jl & 3 of column block c's granule
+    const int vr = 4 * blk + (jl >> 2);
+    const unsigned vx = (unsigned)(kD >= 128 ? (vr & 7) : ((vr >> 1) & 3));
+    const unsigned rd_v = lds_v + vr * kRowBytes + (jl & 3) * 8;
+
+    f32x4 acc[kColBlocks];
+#pragma unroll
+    for (int c = 0; c < kColBlocks; c++) acc[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.0f;  // l_run: this lane's share of the sum (its eight keys per chunk)
+
+    const int chunks = (k_end - k_begin + kChunkKeys - 1) / kChunkKeys;
+    for (int ci = wave; ci < chunks; ci += kWaves) {
+        const int k0 = k_begin + ci * kChunkKeys;
+        const bool full = k0 + kChunkKeys <= k_end;
+        const int last = k_end - 1 - k0;  // the chunk's last valid row
+        const char* kb = k_head + (size_t)k0 * lay.k_row;
+        const char* vb = v_head + (size_t)k0 * lay.v_row;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");  // the previous chunk's fragment reads are done
+#pragma unroll
+        for (int i = 0; i < kCopies; i++) {
+            int r = i * kRowsPerCopy + rsub;
+            if (!full) r = r < last ? r : last;  // a row past the end repeats the last one (masked below)
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                         :
+                         : "s"(lds_k + i * 1024), "v"((unsigned)r * lay.k_row + k_piece[i]), "s"(kb)
+                         : "m0", "memory");
+        }
+#pragma unroll
+        for (int i = 0; i < kCopies; i++) {
+            int r = i * kRowsPerCopy + rsub;
+            if (!full) r = r < last ? r : last;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+                         :
+                         : "s"(lds_v + i * 1024), "v"((unsigned)r * lay.v_row + v_piece[i]), "s"(vb)
+                         : "m0", "memory");
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        // scores of the two 16-key blocks
+        f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < kSteps; s++) {
+            const unsigned po = (((unsigned)(4 * s + blk)) ^ kx) * 16u;
+            const u32x4 f0 = *MRK_FD_LDS(u32x4, rd_k + po);
+            const u32x4 f1 = *MRK_FD_LDS(u32x4, rd_k + 16 * kRowBytes + po);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, f0), __builtin_bit_cast(bf16x8, qf[s]), s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, f1), __builtin_bit_cast(bf16x8, qf[s]), s1, 0, 0, 0);
+        }
+        float x[8];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            x[r] = s0[r] * scale_log2e;
+            x[4 + r] = s1[r] * scale_log2e;
+        }
+        if (!full) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (4 * blk + r > last) x[r] = -INFINITY;
+                if (16 + 4 * blk + r > last) x[4 + r] = -INFINITY;
+            }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);  // finite: the chunk's first key is valid
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        m_run = m_new;
+        f32x8 p;
+        float psum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 8; r++) {
+            p[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
+            psum += p[r];
+        }
+        l_run = l_run * alpha + psum;
+        const bf16x8 pb = __builtin_convertvector(p, bf16x8);
+#pragma unroll
+        for (int c = 0; c < kColBlocks; c++) {
+            const unsigned off = rd_v + (((unsigned)c ^ vx) << 5);
+            bf16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(MRK_FD_LDS(bf16x4, off));
+            bf16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(MRK_FD_LDS(bf16x4, off + 16 * kRowBytes));
+            if (!full) {
+                // the rows past the end hold copies of the last row; their weights are zero, but a zero times an
+                // infinity or a NaN of that row must not reach the sum
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    if (4 * blk + r > last) lo[r] = (__bf16)0.0f;
+                    if (16 + 4 * blk + r > last) hi[r] = (__bf16)0.0f;
+                }
+            }
+            const bf16x8 vf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb, acc[c] * alpha, 0, 0, 0);
+        }
+    }
+    // a query's sum over the four lanes that share it
+    l_run += __shfl_xor(l_run, 16);
+    l_run += __shfl_xor(l_run, 32);
+
+    // the waves' results meet in LDS, over the copy regions
+    __syncthreads();
+    char* part = smem;  // [kWaves][kPartBytes]
+    {
+        f32x4* po = reinterpret_cast<f32x4*>(part + wave * kPartBytes);
+#pragma unroll
+        for (int c = 0; c < kColBlocks; c++) po[c * 64 + lane] = acc[c];
+        if (blk == 0) {
+            float* ml = reinterpret_cast<float*>(part + wave * kPartBytes + kColBlocks * 1024);
+            ml[jl] = m_run;
+            ml[16 + jl] = l_run;
+        }
+    }
+    __syncthreads();
+    // element e: column block e / 64, lane l = e % 64 of it: query l % 16, columns 16 c + 4 (l / 16) + 0..3
+    for (int e = threadIdx.x; e < kColBlocks * 64; e += kWaves * 64) {
+        const int c = e >> 6, l = e & 63, q = l & 15;
+        if (q >= Sq) continue;
+        float m_tot = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) m_tot = fmaxf(m_tot, reinterpret_cast<const float*>(part + w * kPartBytes + kColBlocks * 1024)[q]);
+        f32x4 o = {0.f, 0.f, 0.f, 0.f};
+        float l_tot = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kWaves; w++) {
+            const float* ml = reinterpret_cast<const float*>(part + w * kPartBytes + kColBlocks * 1024);
+            const float wgt = __builtin_amdgcn_exp2f(ml[q] - m_tot);  // a wave without a chunk: maximum -inf, weight 0
+            o += reinterpret_cast<const f32x4*>(part + w * kPartBytes)[c * 64 + l] * wgt;
+            l_tot += ml[16 + q] * wgt;
+        }
+        const int d = 16 * c + 4 * (l >> 4);
+        if (W) {
+            float* dst = W + (((size_t)blockIdx.x * gridDim.y + bh) * kMaxQueries + q) * (kD + 2);
+            *reinterpret_cast<float2*>(dst + d) = make_float2(o[0], o[1]);
+            *reinterpret_cast<float2*>(dst + d + 2) = make_float2(o[2], o[3]);
+            if (d == 0) {
+                dst[kD] = m_tot;
+                dst[kD + 1] = l_tot;
+            }
+        } else {
+            const float inv = 1.0f / l_tot;
+            const f32x4 v = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
+            char* orow = reinterpret_cast<char*>(O + b * lay.o_batch + h * lay.o_head) + (size_t)q * lay.o_row;
+            *reinterpret_cast<bf16x4*>(orow + d * 2) = __builtin_convertvector(v, bf16x4);
+        }
+    }
+}
+
+// O[bh][q][d] from the splits' partial results: the same merge as inside a workgroup, splits in order.
+// One work-item per four columns; grid = ceil(BH * Sq * D / 4 / 256).
+template <int kD>
+__global__ __launch_bounds__(256) void flash_decode_merge(const float* __restrict__ W, unsigned short* __restrict__ O, int BH, int Sq, int splits,
+                                                          DecodeLayout lay) {
+    const long e = (long)blockIdx.x * 256 + threadIdx.x;
+    constexpr int kQuads = kD / 4;
+    if (e >= (long)BH * Sq * kQuads) return;
+    const int d = (int)(e % kQuads) * 4;
+    const int q = (int)((e / kQuads) % Sq);
+    const int bh = (int)(e / ((long)kQuads * Sq));
+    const size_t slice = (size_t)BH * kMaxQueries * (kD + 2);
+    const float* src = W + ((size_t)bh * kMaxQueries + q) * (kD + 2);
+    float m_tot = -INFINITY;
+    for (int s = 0; s < splits; s++) m_tot = fmaxf(m_tot, src[s * slice + kD]);
+    f32x4 o = {0.f, 0.f, 0.f, 0.f};
+    float l_tot = 0.0f;
+    for (int s = 0; s < splits; s++) {
+        const float* p = src + s * slice;
+        const float wgt = __builtin_amdgcn_exp2f(p[kD] - m_tot);
+        const float2 a = *reinterpret_cast<const float2*>(p + d), c = *reinterpret_cast<const float2*>(p + d + 2);
+        o += f32x4{a.x, a.y, c.x, c.y} * wgt;
+        l_tot += p[kD + 1] * wgt;
+    }
+    const float inv = 1.0f / l_tot;
+    const f32x4 v = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
+    const int b = bh / lay.heads, h = bh % lay.heads;
+    char* orow = reinterpret_cast<char*>(O + b * lay.o_batch + h * lay.o_head) + (size_t)q * lay.o_row;
+    *reinterpret_cast<bf16x4*>(orow + d * 2) = __builtin_convertvector(v, bf16x4);
+}
+
+}  // namespace mrk::dev
+
+namespace mrk {
+using namespace mrk::dev;
+
+// Shapes the split kernel takes and the number of key ranges it uses: up to 16 queries, no causal rule, at
+// least 256 keys.  Measured against one workgroup per 128 queries of a (batch, head) pair it streams K and V
+// faster at every count of pairs (7.0 against 6.1 TB/s with 1024 and more), so the count does not limit it.
+// Ranges are multiples of 32 keys and at least 512 keys long (two chunks per wave and more); about 192
+// workgroups measured best where the pairs alone are fewer (4096 keys, 32 pairs: 41 us in one range, 20 in
+// four to eight, 27 in sixteen: the second kernel and the ranges' fixed cost grow with the count).
+bool flash_decode_plan(long BH, long Sq, long Sk, long D, int causal, long* splits, long* keys_per_split) {
+    if (causal || Sq < 1 || Sq > kMaxQueries || Sk < 256 || Sk > (1L << 24) || BH < 1 || BH > 65535) return false;
+    if (D != 256 && D != 128 && D != 64) return false;
+    const long max_splits = Sk / 512 > 0 ? Sk / 512 : 1;
+    long want = (192 + BH / 2) / BH;
+    want = want < max_splits ? want : max_splits;
+    want = want < 1 ? 1 : want;
+    const long per = ((Sk + want - 1) / want + kChunkKeys - 1) / kChunkKeys * kChunkKeys;
+    *keys_per_split = per;
+    *splits = (Sk + per - 1) / per;
+    return true;
+}
+
+size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal) {
+    long splits = 0, per = 0;
+    if (!flash_decode_plan(BH, Sq, Sk, D, causal, &splits, &per) || splits <= 1) return 0;
+    return (size_t)splits * BH * kMaxQueries * (D + 2) * sizeof(float);
+}
+
+// strides: (batch, head, row) element strides of q, k, v and o (validated by the caller: multiples of 8, rows
+// addressable in 32 bits, pointers 16-byte aligned); W: splits * B * H * 16 * (D + 2) floats, needed with several splits.
+int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
+                        float scale, const long* strides, long splits, long keys_per_split, void* W) {
+    if (B <= 0 || H <= 0 || Sq < 1 || Sq > kMaxQueries || Sk < 1 || splits < 1 || B * H > 65535) return (int)hipErrorInvalidValue;
+    if (keys_per_split < kChunkKeys || keys_per_split % kChunkKeys || splits * keys_per_split < Sk || (splits - 1) * keys_per_split >= Sk)
+        return (int)hipErrorInvalidValue;
+    if (splits > 1 && !W) return (int)hipErrorInvalidValue;
+    DecodeLayout lay;
+    lay.q_batch = strides[0], lay.q_head = strides[1], lay.q_row = (unsigned)(strides[2] * 2);
+    lay.k_batch = strides[3], lay.k_head = strides[4], lay.k_row = (unsigned)(strides[5] * 2);
+    lay.v_batch = strides[6], lay.v_head = strides[7], lay.v_row = (unsigned)(strides[8] * 2);
+    lay.o_batch = strides[9], lay.o_head = strides[10], lay.o_row = (unsigned)(strides[11] * 2);
+    lay.heads = (int)H;
+    const float scale_log2e = scale * 1.4426950408889634f;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)splits, (unsigned)(B * H));
+    float* w = splits > 1 ? static_cast<float*>(W) : nullptr;
+    auto qp = static_cast<const unsigned short*>(q);
+    auto kp = static_cast<const unsigned short*>(k);
+    auto vp = static_cast<const unsigned short*>(v);
+    auto op = static_cast<unsigned short*>(o);
+    (void)hipGetLastError();
+    const long quads = B * H * Sq * (D / 4);
+    const unsigned merge_blocks = (unsigned)((quads + 255) / 256);
+    if (D == 128) {
+        flash_decode_split<128><<<grid, decode_waves<128>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split, scale_log2e, lay);
+        if (w) flash_decode_merge<128><<<merge_blocks, 256, 0, s>>>(w, op, (int)(B * H), (int)Sq, (int)splits, lay);
+    } else if (D == 64) {
+        flash_decode_split<64><<<grid, decode_waves<64>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split, scale_log2e, lay);
+        if (w) flash_decode_merge<64><<<merge_blocks, 256, 0, s>>>(w, op, (int)(B * H), (int)Sq, (int)splits, lay);
+    } else if (D == 256) {
+        flash_decode_split<256><<<grid, decode_waves<256>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split, scale_log2e, lay);
+        if (w) flash_decode_merge<256><<<merge_blocks, 256, 0, s>>>(w, op, (int)(B * H), (int)Sq, (int)splits, lay);
+    } else {
+        return (int)hipErrorInvalidValue;
+    }
+    return (int)hipGetLastError();
+}
+
+}  // namespace mrk

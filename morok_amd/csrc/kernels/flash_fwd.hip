@@ -657,14 +657,37 @@ MRK_FLASH_EXT_KERNEL(flash_fwd_ext_d256_add_cap, 256, 1, 2, true)
 
 namespace mrk {
 
+// A handful of queries against a long key sequence: the kernel that splits the keys (flash_decode.hip), in as many
+// ranges as the workspace allows (one range needs none).
+static bool decode_route(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
+                         float scale, int causal, const long* strides, void* workspace, size_t workspace_bytes, int* rc) {
+    using namespace mrk::dev;
+    long splits = 0, per = 0;
+    if (!flash_decode_plan(B * H, Sq, Sk, D, causal, &splits, &per)) return false;
+    const void* ptrs[4] = {q, k, v, o};
+    for (const void* p : ptrs)
+        if (reinterpret_cast<uintptr_t>(p) % 16) return false;
+    if (splits > 1 && (!workspace || workspace_bytes < flash_fwd_workspace_bytes(B * H, Sq, Sk, D, causal))) {
+        splits = 1;
+        per = (Sk + 31) / 32 * 32;
+    }
+    *rc = launch_flash_decode(stream, q, k, v, o, B, H, Sq, Sk, D, scale, strides, splits, per, workspace);
+    return true;
+}
+
 int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
-                          long D, float scale, int causal) {
+                          long D, float scale, int causal, void* workspace, size_t workspace_bytes) {
     using namespace mrk::dev;
     if (BH <= 0 || Sq <= 0) return 0;
     if ((D != 256 && D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
     if (Sq > (1L << 24) || Sk > (1L << 24) || BH > (1L << 24)) return (int)hipErrorInvalidValue;
     // row offsets inside a head are formed in 32 bits (row * row bytes): the last row must end below 4 GiB
     if (!flash_fwd_rows_addressable(Sq, D * 2, D) || !flash_fwd_rows_addressable(Sk, D * 2, D)) return (int)hipErrorInvalidValue;
+    {
+        const long dense[12] = {Sq * D, 0, D, Sk * D, 0, D, Sk * D, 0, D, Sq * D, 0, D};  // (batch * head, -, row) per operand
+        int rc = 0;
+        if (decode_route(stream, q, k, v, o, BH, 1, Sq, Sk, D, scale, causal, dense, workspace, workspace_bytes, &rc)) return rc;
+    }
     const long q_tiles = (Sq + kQT - 1) / kQT;
     const long units = causal ? (q_tiles + 1) / 2 : q_tiles;
     const long blocks = BH * units;
@@ -679,7 +702,7 @@ int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void
 }
 
 int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq,
-                                  long Sk, long D, float scale, int causal, const long* strides) {
+                                  long Sk, long D, float scale, int causal, const long* strides, void* workspace, size_t workspace_bytes) {
     using namespace mrk::dev;
     if (B < 0 || H < 0 || !strides) return (int)hipErrorInvalidValue;
     const long BH = B * H;
@@ -701,7 +724,11 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
         if (t == 3 && ((Sq > 1 && sr < D) || (H > 1 && sh == 0) || (B > 1 && sb == 0))) return (int)hipErrorInvalidValue;
         dense = dense && sr == D && sh == rows[t] * D && sb == H * rows[t] * D;
     }
-    if (dense) return launch_flash_fwd_bf16(stream, q, k, v, o, BH, Sq, Sk, D, scale, causal);
+    if (dense) return launch_flash_fwd_bf16(stream, q, k, v, o, BH, Sq, Sk, D, scale, causal, workspace, workspace_bytes);
+    {
+        int rc = 0;
+        if (decode_route(stream, q, k, v, o, B, H, Sq, Sk, D, scale, causal, strides, workspace, workspace_bytes, &rc)) return rc;
+    }
     const long q_tiles = (Sq + kQT - 1) / kQT;
     const long units = causal ? (q_tiles + 1) / 2 : q_tiles;
     const long blocks = BH * units;

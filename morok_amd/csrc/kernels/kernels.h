@@ -117,14 +117,23 @@ inline bool flash_fwd_rows_addressable(long rows, long row_bytes, long D) {
 }
 // O = softmax(Q K^T * scale [causal]) V; Q [BH,Sq,D], K/V [BH,Sk,D], O [BH,Sq,D] bf16, D = 256, 128 or 64,
 // scale > 0.  Causal: key j visible to query i iff j <= i.
+// Up to 16 queries without the causal rule against 256 keys and more (a decode step over a key/value cache) take
+// a kernel that also splits the key sequence over workgroups (flash_decode_plan tells how); with several key
+// ranges their f32 partial results go through `workspace` (flash_fwd_workspace_bytes; 0 = one range), which a
+// second kernel merges.  Without a workspace of that size such a shape runs as one range per (batch, head).
+bool flash_decode_plan(long BH, long Sq, long Sk, long D, int causal, long* splits, long* keys_per_split);
+size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal);
+int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
+                        float scale, const long* strides, long splits, long keys_per_split, void* W);
 int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
-                          long D, float scale, int causal);
+                          long D, float scale, int causal, void* workspace = nullptr, size_t workspace_bytes = 0);
 // The same kernel over operands given as views: strides holds (batch, head, row) element
 // strides of q, k, v and o, in that order (12 values); the 128 elements of a row are
 // contiguous.  Strides must be multiples of 8 elements and the pointers 16-byte aligned;
 // zero batch / head strides broadcast an input.  Dense strides take the kernel above.
 int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq,
-                                  long Sk, long D, float scale, int causal, const long* strides);
+                                  long Sk, long D, float scale, int causal, const long* strides, void* workspace = nullptr,
+                                  size_t workspace_bytes = 0);
 
 // The same attention with an attn_mask and / or a softcap (transformer.rs:112-132), operands as
 // views like the strided launcher.  mask_kind 0: none; 1: Bool, one byte per element, nonzero =

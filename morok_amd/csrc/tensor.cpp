@@ -2106,12 +2106,19 @@ struct Scheduler {
             params.insert(params.end(), mask_strides, mask_strides + 3);
             bufs.push_back(has_mask ? mask_buf : bufs[1]);
             MRK_TRY(builtin("flash_fwd_bf16_ext", params, bufs));
-        } else if (dense) {
-            MRK_TRY(builtin("flash_fwd_bf16", {B * H, Sq, Sk, D, att->hint_causal ? 1 : 0, static_cast<int64_t>(bits)}, bufs));
         } else {
-            params = {B, H, Sq, Sk, D, att->hint_causal ? 1 : 0, static_cast<int64_t>(bits), offsets[0], offsets[1], offsets[2], 0};
-            params.insert(params.end(), strides.begin(), strides.end());
-            MRK_TRY(builtin("flash_fwd_bf16_strided", params, bufs));
+            // a handful of queries against a long key sequence: the keys are split over workgroups and the ranges'
+            // partial results go through scratch, an intermediate of the plan like any other
+            const size_t ws = flash_fwd_workspace_bytes(B * H, Sq, Sk, D, att->hint_causal ? 1 : 0);
+            if (ws) bufs.push_back(std::make_shared<Buffer>(dev->allocator, ws, BufferOptions()));
+            if (dense) {
+                params = {B * H, Sq, Sk, D, att->hint_causal ? 1 : 0, static_cast<int64_t>(bits)};
+            } else {
+                params = {B, H, Sq, Sk, D, att->hint_causal ? 1 : 0, static_cast<int64_t>(bits), offsets[0], offsets[1], offsets[2], 0};
+                params.insert(params.end(), strides.begin(), strides.end());
+            }
+            if (ws) params.push_back(static_cast<int64_t>(ws));
+            MRK_TRY(builtin(dense ? "flash_fwd_bf16" : "flash_fwd_bf16_strided", params, bufs));
         }
         dst->buffer = out;
         produced.push_back(dst);

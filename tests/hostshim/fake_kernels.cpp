@@ -75,13 +75,17 @@ int launch_gemm_bf16_rope(void* stream, const void*, const void*, void*, void*, 
     mrk_shim_note_launch(stream, b_transposed ? "gemm_bf16_nt_rope" : "gemm_bf16_rope");
     return 0;
 }
-int launch_flash_fwd_bf16(void* stream, const void*, const void*, const void*, void*, long, long, long, long, float, int) {
-    mrk_shim_note_launch(stream, "flash_fwd_bf16");
+// a handful of queries against many keys with few (batch, head) pairs: scratch for a split key sequence
+size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal) {
+    return !causal && Sq >= 1 && Sq <= 16 && Sk >= 1024 && BH >= 1 && BH <= 96 ? (size_t)2 * BH * 16 * (D + 2) * 4 : 0;
+}
+int launch_flash_fwd_bf16(void* stream, const void*, const void*, const void*, void*, long, long, long, long, float, int, void* ws, size_t) {
+    mrk_shim_note_launch(stream, ws ? "flash_fwd_bf16_splitkv" : "flash_fwd_bf16");
     return 0;
 }
 int launch_flash_fwd_bf16_strided(void* stream, const void*, const void*, const void*, void*, long, long, long, long, long, float,
-                                  int, const long*) {
-    mrk_shim_note_launch(stream, "flash_fwd_bf16_strided");
+                                  int, const long*, void* ws, size_t) {
+    mrk_shim_note_launch(stream, ws ? "flash_fwd_bf16_strided_splitkv" : "flash_fwd_bf16_strided");
     return 0;
 }
 int launch_flash_fwd_bf16_ext(void* stream, const void*, const void*, const void*, void*, long, long, long, long, long, float, int,

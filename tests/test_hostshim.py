@@ -322,6 +322,12 @@ def test_tensor_fused_kernel_selection(T, shim):
     assert f64.kernels() == ["flash_fwd_bf16_2_64_64_d64"]   # head dim 64 has an instantiation of its own
     f256 = bf(1, 2, 64, 256).scaled_dot_product_attention(bf(1, 2, 64, 256), bf(1, 2, 64, 256), is_causal=True).realize()
     assert f256.kernels() == ["flash_fwd_bf16_2_64_64_d256"]  # and so has 256
+    # one query against a long key sequence with few (batch, head) pairs: the key sequence is split over workgroups
+    # and the kernel gets a scratch buffer for the ranges' partial results, an intermediate of the plan
+    dec = bf(1, 8, 1, 128).scaled_dot_product_attention(bf(1, 8, 2048, 128), bf(1, 8, 2048, 128)).realize()
+    assert dec.kernels() == ["flash_fwd_bf16_8_1_2048_splitkv"] and shim.mrk_shim_last_kernel() == b"flash_fwd_bf16_splitkv"
+    dec_c = bf(1, 8, 1, 128).scaled_dot_product_attention(bf(1, 8, 2048, 128), bf(1, 8, 2048, 128), is_causal=True).realize()
+    assert dec_c.kernels() == ["flash_fwd_bf16_8_1_2048"]    # not under the causal rule
     f96 = bf(1, 2, 64, 96).scaled_dot_product_attention(bf(1, 2, 64, 96), bf(1, 2, 64, 96), is_causal=True).realize()
     # other head dims are padded with zero columns to the next instantiation: three padded copies, the
     # fused kernel at 128, the cut back to 96 columns; no reduce kernels, no score matrix
