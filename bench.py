@@ -41,7 +41,7 @@ PROFILE_OF = {"softmax": "softmax_rows_in_regs_8192x8192_f32.txt", "gemm": "gemm
               "generated_tc": "generated_tensor_core_gemm_4096cubed.txt", "matmul_f32": "generated_f32_matmul_1024cubed.txt",
               "gemm_f16": "gemm_f16_tile256_4096cubed.txt", "flash_options": "flash_fwd_ext_d128_8x32x4096x128.txt",
               "linear_decode": "gemm_nt_skinny_1x12288x4096_x8.txt", "linear_decode_16": "gemm_nt_rows_16x12288x4096_x8.txt",
-              "decoder_decode": "decoder_block_decode_16tokens_linear_layout.txt"}
+              "decoder_decode": "decoder_block_decode_16tokens_linear_layout.txt", "flash_decode": "flash_decode_1x32x1x4096_d128_x8.txt"}
 
 
 def _profiled_traffic(workload, kernel):
@@ -655,6 +655,61 @@ def _linear_decode(m, dev, steps, warmup, cpu, M, workload, kernel):
     return rec
 
 
+def bench_flash_decode(m, dev, steps, warmup, cpu):
+    """One new token's attention over the key/value caches of 8 layers (a decode step's eight attention calls):
+    32 heads, 4096 cached keys, head dim 128, batch 1 (and batch 8 beside it): K and V are streamed once."""
+    import numpy as np
+
+    from morok_amd import ops, synth
+
+    layers, H, Sk, D = 8, 32, 4096, 128
+    scale = 1.0 / float(np.sqrt(D))
+
+    def run(B):
+        n_kv, n_q = B * H * Sk * D, B * H * D
+        bq = dev.buffer(n_q * 2).ensure_allocated()
+        ops.fill_normal(bq, n_q, seed=11, tensor_id=0, bf16=True)
+        ks, vs, os_ = [], [], []
+        for i in range(layers):
+            k, v = dev.buffer(n_kv * 2).ensure_allocated(), dev.buffer(n_kv * 2).ensure_allocated()
+            ops.fill_normal(k, n_kv, seed=11, tensor_id=1 + 2 * i, bf16=True)
+            ops.fill_normal(v, n_kv, seed=11, tensor_id=2 + 2 * i, bf16=True)
+            ks.append(k), vs.append(v), os_.append(dev.buffer(n_q * 2).ensure_allocated())
+
+        def step():
+            for k, v, o in zip(ks, vs, os_):
+                ops.flash_attn_fwd_bf16(bq, k, v, o, B, H, 1, Sk, D, scale, False)
+
+        ms, stats = _launch_stats(m, step, max(1, min(steps, 20)), warmup)
+        algo = 2 * n_kv * 2 + 2 * n_q * 2  # per launch: K and V once, q and o
+        return ms, stats, algo, (bq, ks[0], vs[0], os_[0])
+
+    ms, stats, algo_bytes, (bq, k0, v0, o0) = run(1)
+    gbs = layers * algo_bytes / (ms * 1e-3) / 1e9
+    rec = {"metric": "attention decode HBM GB/s", "value": gbs, "unit": "GB/s", "ms_per_step": ms, "dtype": "bf16", **stats,
+           "config": {"workload": "1 query per head x 8 layers' caches [1, 32, 4096, 128] bf16 (K and V), no causal rule, keys split over workgroups"},
+           "launches_per_step": layers, "us_per_launch": ms * 1e3 / layers,
+           "roofline": _roofline("flash_decode", "hbm", gbs, HBM_PEAK_GBS, "GB/s", "flash_decode_split<128>", algorithmic_bytes_per_launch=algo_bytes)}
+    if cpu:
+        from tests.oracle_lib import Oracle
+
+        orc = Oracle()
+        q, k, v = bq.copyout(np.uint16, (1, H, 1, D)), k0.copyout(np.uint16, (1, H, Sk, D)), v0.copyout(np.uint16, (1, H, Sk, D))
+        sec = _cpu_time(lambda: orc.sdpa_bf16(q, k, v, scale, causal=False))
+        got, ref = synth.from_bf16(o0.copyout(np.uint16, (1, H, 1, D))), synth.from_bf16(orc.sdpa_bf16(q, k, v, scale, causal=False))
+        rec["max_rel_err_vs_cpu"] = float(np.abs(got - ref).max() / np.abs(ref).max())
+        rec["cpu_baseline"] = {"value": algo_bytes / sec / 1e9, "unit": "GB/s", "cores": orc.max_threads, "kind": "port",
+                               "sample": "one layer's attention (32 heads x 4096 keys), the oracle's SDPA, min of 3 after 1 warm-up"}
+    del bq, k0, v0, o0
+    dev.synchronize()
+    dev.lru_clear()
+    if REFERENCE_LEGS:  # the same step for a batch of 8 sequences (256 pairs: one key range each, one launch)
+        ms8, _, algo8, _ = run(8)
+        rec["batch_8"] = {"us_per_launch": ms8 * 1e3 / layers, "GB/s": layers * algo8 / (ms8 * 1e-3) / 1e9,
+                          "frac": layers * algo8 / (ms8 * 1e-3) / 1e9 / HBM_PEAK_GBS}
+    return rec
+
+
 def bench_copy(m, dev, steps, warmup, cpu):
     """Calibration only: 256 MiB streaming copy kernel (known traffic 2 x 256 MiB per launch)."""
     from morok_amd import ops
@@ -676,7 +731,7 @@ WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash,
              "matmul_f32": bench_matmul_f32, "generated_tc": bench_generated_tc, "copy": bench_copy, "mfma_ceiling": bench_mfma_ceiling,
              "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16, "flash_options": bench_flash_options,
              "linear_decode": bench_linear_decode, "linear_decode_16": bench_linear_decode_16,
-             "decoder_decode": bench_decoder_decode}
+             "decoder_decode": bench_decoder_decode, "flash_decode": bench_flash_decode}
 PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc", "linear_decode", "linear_decode_16"]
 
 
@@ -722,7 +777,7 @@ def main():
         if "cpu_baseline" in r:
             r["cpu_baseline"]["cpu_model"] = cpu_model
             r["cpu_baseline"]["host_cores"] = os.cpu_count()
-    for k in ("median_ms", "min_ms", "plan_item", "direct_abi_ms_per_step", "vendor_reference", "additive_mask_softcap"):
+    for k in ("median_ms", "min_ms", "plan_item", "direct_abi_ms_per_step", "vendor_reference", "additive_mask_softcap", "batch_8", "launches_per_step", "us_per_launch"):
         if k in primary:
             line[k] = primary[k]
     if "cpu_baseline" in primary:
