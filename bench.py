@@ -732,7 +732,7 @@ WORKLOADS = {"softmax": bench_softmax, "gemm": bench_gemm, "flash": bench_flash,
              "group_reduce": bench_group_reduce, "gemm_f16": bench_gemm_f16, "flash_options": bench_flash_options,
              "linear_decode": bench_linear_decode, "linear_decode_16": bench_linear_decode_16,
              "decoder_decode": bench_decoder_decode, "flash_decode": bench_flash_decode}
-PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc", "linear_decode", "linear_decode_16"]
+PRIMARY_ORDER = ["gemm", "flash", "softmax", "decoder", "matmul_f32", "generated_tc", "linear_decode", "linear_decode_16", "flash_decode"]
 
 
 def main():

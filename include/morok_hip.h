@@ -574,7 +574,11 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
  * takes part in the softmax, exactly as the reference's graph computes it; the kernel then visits
  * every key tile.  A row whose keys are all masked out (no softcap) is NaN, as softmax over -inf
  * only is.  Without mask and softcap this is mrk_hip_flash_attn_fwd_bf16_strided.
- * Builtin Program kind "flash_fwd_bf16_ext" (29 params, buffers {o, q, k, v, mask}). */
+ * A mask without softcap and causal rule over a decode shape (up to 16 queries, 256 keys and more: a batch of
+ * sequences of different lengths decoding under a key-padding mask [batch, 1, 1, sk]) takes the kernel that splits
+ * the key sequence, like the unmasked call; key ranges without a visible key weigh nothing.
+ * Builtin Program kind "flash_fwd_bf16_ext" (29 params, buffers {o, q, k, v, mask}; optionally a 30th, the bytes
+ * of a scratch buffer that follows the mask: mrk_hip_flash_attn_workspace_bytes). */
 int mrk_hip_flash_attn_fwd_bf16_ex(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
                                    int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal,
                                    const int64_t* strides, const void* mask, int mask_kind, const int64_t* mask_strides,

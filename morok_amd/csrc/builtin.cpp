@@ -268,7 +268,11 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
         // softcap bits (0 = none), mask kind (0 none, 1 Bool bytes, 2 additive bf16), element offsets of
         // q k v o mask into their buffers (5), (batch, head, row) element strides of q k v o (12) and of
         // the mask (3).  buffers {o, q, k, v, mask}; without a mask the fifth buffer is not read.
-        MRK_TRY(need(29));
+        // optionally a 30th: workspace bytes, with a sixth buffer of that size (scratch for a split key sequence)
+        if (nparams != 29 && nparams != 30)
+            return failf(kInvalidArgument, "builtin '%s' takes 29 or 30 parameters, got %zu", k.c_str(), nparams);
+        if (p.size() < 30) p.push_back(0);
+        if (p[29] < 0) return fail(kInvalidArgument, "flash_fwd_bf16_ext: negative workspace size");
         if (p[0] < 0 || p[1] < 0 || p[2] < 0 || p[3] <= 0 || (p[4] != 256 && p[4] != 128 && p[4] != 64) || p[8] < 0 || p[8] > 2)
             return fail(kInvalidArgument, "flash_fwd_bf16_ext: bad shape (params B, H, Sq, Sk, D = 256, 128 or 64, causal, scale bits, "
                                           "softcap bits, mask kind 0..2, 5 offsets, 12 strides, 3 mask strides)");
@@ -279,8 +283,9 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
         if (p[8] != 0 && (p[3] % 4 || p[13] % 4)) return fail(kInvalidArgument, "flash_fwd_bf16_ext: with a mask, Sk and the mask offset must be multiples of 4");
         std::string name = std::string("flash_fwd_bf16_ext") + (p[8] == 1 ? "_bool" : p[8] == 2 ? "_add" : "") + (p[7] ? "_cap" : "") + "_" +
                            std::to_string(p[0] * p[1]) + "_" + std::to_string(p[2]) + "_" + std::to_string(p[3]) + (p[4] != 128 ? "_d" + std::to_string(p[4]) : "");
-        out->reset(new BuiltinProgram(device_id, stream, name, 5, p,
-                                      [](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
+        const bool ws = p[29] > 0;
+        out->reset(new BuiltinProgram(device_id, stream, name + (ws ? "_splitkv" : ""), ws ? 6 : 5, p,
+                                      [ws](ffi::Stream s, void* const* b, const std::vector<int64_t>& q) {
                                           uint32_t bits = static_cast<uint32_t>(q[6]), cbits = static_cast<uint32_t>(q[7]);
                                           float scale, cap;
                                           std::memcpy(&scale, &bits, 4);
@@ -292,7 +297,8 @@ int create_builtin_program(int device_id, ffi::Stream stream, const char* kind, 
                                           const int kind = static_cast<int>(q[8]);
                                           const void* mask = kind ? static_cast<char*>(b[4]) + q[13] * (kind == 2 ? 2 : 1) : nullptr;
                                           return launch_flash_fwd_bf16_ext(s, at(1, 0), at(2, 1), at(3, 2), at(0, 3), q[0], q[1], q[2], q[3], q[4],
-                                                                           scale, q[5] != 0, strides, mask, kind, mstrides, cap);
+                                                                           scale, q[5] != 0, strides, mask, kind, mstrides, cap, ws ? b[5] : nullptr,
+                                                                           ws ? static_cast<size_t>(q[29]) : 0);
                                       }));
         return kOk;
     }

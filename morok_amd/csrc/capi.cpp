@@ -1138,8 +1138,15 @@ int mrk_hip_flash_attn_fwd_bf16_ex(int device_id, const void* q, const void* k, 
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    MRK_HIP(launch_flash_fwd_bf16_ext(dv->allocator->stream(), q, k, v, o, batch, heads, sq, sk, d, scale, causal ? 1 : 0, st, mask, mask_kind, mst, softcap),
-            "flash_attn_fwd_ex launch");
+    // (a mask alone over a handful of queries takes the kernel that splits the keys: scratch as in the plain call)
+    const size_t ws = softcap > 0.0f ? 0 : flash_fwd_workspace_bytes(batch * heads, sq, sk, d, causal ? 1 : 0);
+    RawBuffer scratch;
+    BufferOptions so;
+    if (ws) MRK_TRY(dv->allocator->alloc(ws, so, &scratch));
+    const int rc = launch_flash_fwd_bf16_ext(dv->allocator->stream(), q, k, v, o, batch, heads, sq, sk, d, scale, causal ? 1 : 0, st, mask, mask_kind, mst,
+                                             softcap, ws ? scratch.ptr : nullptr, ws);
+    if (ws) dv->allocator->free(scratch, so);
+    MRK_HIP(rc, "flash_attn_fwd_ex launch");
     return kOk;
 }
 

@@ -29,6 +29,7 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x8 __attribute__((ext_vector_type(8)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 #define MRK_FD_LDS(T, p) ((__attribute__((address_space(3))) T*)(p))
 
@@ -41,15 +42,23 @@ struct DecodeLayout {
     int heads;
 };
 
+// attn_mask of the reference (transformer.rs:112-125) as a [batch, head, query, key] view with contiguous keys:
+// element strides per batch, head and query row (0 broadcasts).  Kind 1: Bool bytes, nonzero = attend; 2: additive bf16.
+struct DecodeMask {
+    const void* mask;
+    long long batch, head, row;
+};
+
 template <int kD>
 constexpr int decode_waves() {
     return kD == 256 ? 4 : 8;  // a wave's region is 4 * 32 * kD bytes: 128 KB of LDS for 128 and 256, 64 KB for 64
 }
 
-template <int kD>
+template <int kD, int kMask>
 __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
     const unsigned short* __restrict__ Q, const unsigned short* __restrict__ K, const unsigned short* __restrict__ V,
-    unsigned short* __restrict__ O, float* __restrict__ W, int Sq, int Sk, int keys_per_split, float scale_log2e, DecodeLayout lay) {
+    unsigned short* __restrict__ O, float* __restrict__ W, int Sq, int Sk, int keys_per_split, float scale_log2e, DecodeLayout lay,
+    DecodeMask dm) {
     constexpr int kWaves = decode_waves<kD>();
     constexpr int kRowBytes = kD * 2;
     constexpr int kPieces = kD / 8;                      // 16-byte pieces of a row
@@ -75,8 +84,13 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
 
     // the queries: operand B, query jl (the last one again beyond Sq), eight d at 32 s + 8 blk
     u32x4 qf[kSteps];
+    const int qi = jl < Sq ? jl : Sq - 1;
+    // the mask row of this lane's query: a lane needs the mask of its eight keys per chunk, two groups of four
+    // consecutive ones (the key count is a multiple of 4 under a mask, so a group is inside the sequence or outside)
+    const char* mrow = nullptr;
+    if constexpr (kMask != 0)
+        mrow = static_cast<const char*>(dm.mask) + (b * dm.batch + h * dm.head + qi * dm.row) * (kMask == 2 ? 2 : 1);
     {
-        const int qi = jl < Sq ? jl : Sq - 1;
         const char* qrow = reinterpret_cast<const char*>(Q + b * lay.q_batch + h * lay.q_head) + (size_t)qi * lay.q_row;
 #pragma unroll
         for (int s = 0; s < kSteps; s++) qf[s] = *reinterpret_cast<const u32x4*>(qrow + 64 * s + 16 * blk);
@@ -134,6 +148,19 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
                          : "s"(lds_v + i * 1024), "v"((unsigned)r * lay.v_row + v_piece[i]), "s"(vb)
                          : "m0", "memory");
         }
+        // the mask of this lane's keys, requested together with the copies
+        unsigned mb0 = 0, mb1 = 0;                      // Bool: four bytes per group
+        u32x2 ma0 = {0u, 0u}, ma1 = {0u, 0u};          // additive: four bf16 per group
+        if constexpr (kMask != 0) {
+            const int g0 = k0 + 4 * blk, g1 = g0 + 16;
+            if constexpr (kMask == 1) {
+                if (g0 < k_end) mb0 = *reinterpret_cast<const unsigned*>(mrow + g0);
+                if (g1 < k_end) mb1 = *reinterpret_cast<const unsigned*>(mrow + g1);
+            } else {
+                if (g0 < k_end) ma0 = *reinterpret_cast<const u32x2*>(mrow + 2 * (size_t)g0);
+                if (g1 < k_end) ma1 = *reinterpret_cast<const u32x2*>(mrow + 2 * (size_t)g1);
+            }
+        }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         // scores of the two 16-key blocks
         f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -151,6 +178,22 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
             x[r] = s0[r] * scale_log2e;
             x[4 + r] = s1[r] * scale_log2e;
         }
+        if constexpr (kMask == 1) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                if (((mb0 >> (8 * r)) & 0xffu) == 0u) x[r] = -INFINITY;
+                if (((mb1 >> (8 * r)) & 0xffu) == 0u) x[4 + r] = -INFINITY;
+            }
+        }
+        if constexpr (kMask == 2) {
+            // scale, then the mask (transformer.rs:96-125), both in exp2 units here
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const unsigned w0 = ma0[r >> 1], w1 = ma1[r >> 1];
+                x[r] += __builtin_bit_cast(float, (r & 1) ? (w0 & 0xffff0000u) : (w0 << 16)) * 1.4426950408889634f;
+                x[4 + r] += __builtin_bit_cast(float, (r & 1) ? (w1 & 0xffff0000u) : (w1 << 16)) * 1.4426950408889634f;
+            }
+        }
         if (!full) {
 #pragma unroll
             for (int r = 0; r < 4; r++) {
@@ -161,14 +204,17 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
         float mx = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
         mx = fmaxf(mx, __shfl_xor(mx, 16));
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);  // finite: the chunk's first key is valid
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        const float m_new = fmaxf(m_run, mx);  // without a mask finite: the chunk's first key is valid
+        // under a mask every key so far may be masked out (maximum -inf): such keys weigh nothing, and nothing has been
+        // summed yet; the differences below must not become -inf - -inf
+        const float m_ref = kMask != 0 && m_new == -INFINITY ? 0.0f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
         m_run = m_new;
         f32x8 p;
         float psum = 0.0f;
 #pragma unroll
         for (int r = 0; r < 8; r++) {
-            p[r] = __builtin_amdgcn_exp2f(x[r] - m_new);
+            p[r] = __builtin_amdgcn_exp2f(x[r] - m_ref);
             psum += p[r];
         }
         l_run = l_run * alpha + psum;
@@ -221,7 +267,10 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
 #pragma unroll
         for (int w = 0; w < kWaves; w++) {
             const float* ml = reinterpret_cast<const float*>(part + w * kPartBytes + kColBlocks * 1024);
-            const float wgt = __builtin_amdgcn_exp2f(ml[q] - m_tot);  // a wave without a chunk: maximum -inf, weight 0
+            // a wave without a chunk, or whose keys are all masked out: maximum -inf, weight 0; a workgroup of such waves
+            // only leaves (0, -inf, 0), which weighs nothing among other ranges and ends as 0 / 0 = NaN without them
+            // (the softmax over -inf only of the reference)
+            const float wgt = m_tot == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f(ml[q] - m_tot);
             o += reinterpret_cast<const f32x4*>(part + w * kPartBytes)[c * 64 + l] * wgt;
             l_tot += ml[16 + q] * wgt;
         }
@@ -256,10 +305,13 @@ __global__ __launch_bounds__(256) void flash_decode_merge(const float* __restric
     const int bh = (int)(e / ((long)kQuads * Sq));
     const size_t slice = (size_t)BH * kMaxQueries * (kD + 2);
     const float* src = W + ((size_t)bh * kMaxQueries + q) * (kD + 2);
+    // (both loops unrolled by four: the loads of four ranges are in flight together, the sums keep their order)
     float m_tot = -INFINITY;
+#pragma unroll 4
     for (int s = 0; s < splits; s++) m_tot = fmaxf(m_tot, src[s * slice + kD]);
     f32x4 o = {0.f, 0.f, 0.f, 0.f};
     float l_tot = 0.0f;
+#pragma unroll 4
     for (int s = 0; s < splits; s++) {
         const float* p = src + s * slice;
         const float wgt = __builtin_amdgcn_exp2f(p[kD] - m_tot);
@@ -306,8 +358,11 @@ size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal) 
 
 // strides: (batch, head, row) element strides of q, k, v and o (validated by the caller: multiples of 8, rows
 // addressable in 32 bits, pointers 16-byte aligned); W: splits * B * H * 16 * (D + 2) floats, needed with several splits.
+// mask_kind 0: none; 1: Bool bytes, 2: additive bf16, with (batch, head, query row) element strides that are multiples
+// of 4, a mask pointer aligned to four elements and Sk a multiple of 4 (validated by the caller as well).
 int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
-                        float scale, const long* strides, long splits, long keys_per_split, void* W) {
+                        float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask, int mask_kind,
+                        const long* mask_strides) {
     if (B <= 0 || H <= 0 || Sq < 1 || Sq > kMaxQueries || Sk < 1 || splits < 1 || B * H > 65535) return (int)hipErrorInvalidValue;
     if (keys_per_split < kChunkKeys || keys_per_split % kChunkKeys || splits * keys_per_split < Sk || (splits - 1) * keys_per_split >= Sk)
         return (int)hipErrorInvalidValue;
@@ -318,6 +373,12 @@ int launch_flash_decode(void* stream, const void* q, const void* k, const void* 
     lay.v_batch = strides[6], lay.v_head = strides[7], lay.v_row = (unsigned)(strides[8] * 2);
     lay.o_batch = strides[9], lay.o_head = strides[10], lay.o_row = (unsigned)(strides[11] * 2);
     lay.heads = (int)H;
+    if (mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && (!mask || !mask_strides || Sk % 4))) return (int)hipErrorInvalidValue;
+    DecodeMask dm{};
+    if (mask_kind != 0) {
+        dm.mask = mask;
+        dm.batch = mask_strides[0], dm.head = mask_strides[1], dm.row = mask_strides[2];
+    }
     const float scale_log2e = scale * 1.4426950408889634f;
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)splits, (unsigned)(B * H));
@@ -329,18 +390,21 @@ int launch_flash_decode(void* stream, const void* q, const void* k, const void* 
     (void)hipGetLastError();
     const long quads = B * H * Sq * (D / 4);
     const unsigned merge_blocks = (unsigned)((quads + 255) / 256);
-    if (D == 128) {
-        flash_decode_split<128><<<grid, decode_waves<128>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split, scale_log2e, lay);
-        if (w) flash_decode_merge<128><<<merge_blocks, 256, 0, s>>>(w, op, (int)(B * H), (int)Sq, (int)splits, lay);
-    } else if (D == 64) {
-        flash_decode_split<64><<<grid, decode_waves<64>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split, scale_log2e, lay);
-        if (w) flash_decode_merge<64><<<merge_blocks, 256, 0, s>>>(w, op, (int)(B * H), (int)Sq, (int)splits, lay);
-    } else if (D == 256) {
-        flash_decode_split<256><<<grid, decode_waves<256>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split, scale_log2e, lay);
-        if (w) flash_decode_merge<256><<<merge_blocks, 256, 0, s>>>(w, op, (int)(B * H), (int)Sq, (int)splits, lay);
-    } else {
-        return (int)hipErrorInvalidValue;
-    }
+#define MRK_DECODE(DIM, MASK) \
+    flash_decode_split<DIM, MASK><<<grid, decode_waves<DIM>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split, scale_log2e, lay, dm)
+#define MRK_DECODE_DIM(DIM)                                                                                         \
+    do {                                                                                                            \
+        if (mask_kind == 0) MRK_DECODE(DIM, 0);                                                                     \
+        else if (mask_kind == 1) MRK_DECODE(DIM, 1);                                                                \
+        else MRK_DECODE(DIM, 2);                                                                                    \
+        if (w) flash_decode_merge<DIM><<<merge_blocks, 256, 0, s>>>(w, op, (int)(B * H), (int)Sq, (int)splits, lay); \
+    } while (0)
+    if (D == 128) MRK_DECODE_DIM(128);
+    else if (D == 64) MRK_DECODE_DIM(64);
+    else if (D == 256) MRK_DECODE_DIM(256);
+    else return (int)hipErrorInvalidValue;
+#undef MRK_DECODE_DIM
+#undef MRK_DECODE
     return (int)hipGetLastError();
 }
 

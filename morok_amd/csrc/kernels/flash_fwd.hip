@@ -660,7 +660,8 @@ namespace mrk {
 // A handful of queries against a long key sequence: the kernel that splits the keys (flash_decode.hip), in as many
 // ranges as the workspace allows (one range needs none).
 static bool decode_route(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
-                         float scale, int causal, const long* strides, void* workspace, size_t workspace_bytes, int* rc) {
+                         float scale, int causal, const long* strides, void* workspace, size_t workspace_bytes, int* rc,
+                         const void* mask = nullptr, int mask_kind = 0, const long* mask_strides = nullptr) {
     using namespace mrk::dev;
     long splits = 0, per = 0;
     if (!flash_decode_plan(B * H, Sq, Sk, D, causal, &splits, &per)) return false;
@@ -671,7 +672,7 @@ static bool decode_route(void* stream, const void* q, const void* k, const void*
         splits = 1;
         per = (Sk + 31) / 32 * 32;
     }
-    *rc = launch_flash_decode(stream, q, k, v, o, B, H, Sq, Sk, D, scale, strides, splits, per, workspace);
+    *rc = launch_flash_decode(stream, q, k, v, o, B, H, Sq, Sk, D, scale, strides, splits, per, workspace, mask, mask_kind, mask_strides);
     return true;
 }
 
@@ -752,11 +753,12 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
 
 int launch_flash_fwd_bf16_ext(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk,
                               long D, float scale, int causal, const long* strides, const void* mask, int mask_kind,
-                              const long* mask_strides, float softcap) {
+                              const long* mask_strides, float softcap, void* workspace, size_t workspace_bytes) {
     using namespace mrk::dev;
     if (B < 0 || H < 0 || !strides) return (int)hipErrorInvalidValue;
     if (mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && (!mask || !mask_strides)) || !(softcap >= 0.0f)) return (int)hipErrorInvalidValue;
-    if (mask_kind == 0 && !(softcap > 0.0f)) return launch_flash_fwd_bf16_strided(stream, q, k, v, o, B, H, Sq, Sk, D, scale, causal, strides);
+    if (mask_kind == 0 && !(softcap > 0.0f))
+        return launch_flash_fwd_bf16_strided(stream, q, k, v, o, B, H, Sq, Sk, D, scale, causal, strides, workspace, workspace_bytes);
     const long BH = B * H;
     if (BH == 0 || Sq <= 0) return 0;
     if ((D != 256 && D != 128 && D != 64) || Sk <= 0 || !(scale > 0.0f)) return (int)hipErrorInvalidValue;
@@ -783,6 +785,11 @@ int launch_flash_fwd_bf16_ext(void* stream, const void* q, const void* k, const 
         ext.batch = mask_strides[0], ext.head = mask_strides[1], ext.row = mask_strides[2];
     }
     const bool cap = softcap > 0.0f;
+    if (!cap) {  // a mask alone over a handful of queries: the kernel that splits the keys
+        int rc = 0;
+        if (decode_route(stream, q, k, v, o, B, H, Sq, Sk, D, scale, causal, strides, workspace, workspace_bytes, &rc, mask, mask_kind, mask_strides))
+            return rc;
+    }
     ext.cap = softcap;
     ext.causal_elem = causal ? 1 : 0;
     // under a softcap a causally masked score becomes -cap and still counts: every key tile is visited

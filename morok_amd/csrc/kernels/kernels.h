@@ -124,7 +124,8 @@ inline bool flash_fwd_rows_addressable(long rows, long row_bytes, long D) {
 bool flash_decode_plan(long BH, long Sq, long Sk, long D, int causal, long* splits, long* keys_per_split);
 size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal);
 int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
-                        float scale, const long* strides, long splits, long keys_per_split, void* W);
+                        float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask = nullptr,
+                        int mask_kind = 0, const long* mask_strides = nullptr);
 int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
                           long D, float scale, int causal, void* workspace = nullptr, size_t workspace_bytes = 0);
 // The same kernel over operands given as views: strides holds (batch, head, row) element
@@ -143,9 +144,11 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
 // (causal ones included) turn into -softcap and still take part, as in the reference.  A row
 // whose keys are all masked out (no softcap) comes out as NaN, as the reference's softmax does.
 // Without mask and softcap this is launch_flash_fwd_bf16_strided.
+// A mask without softcap and causal rule over a decode shape (see flash_decode_plan) takes the split kernel as well,
+// with the same workspace.
 int launch_flash_fwd_bf16_ext(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk,
                               long D, float scale, int causal, const long* strides, const void* mask, int mask_kind,
-                              const long* mask_strides, float softcap);
+                              const long* mask_strides, float softcap, void* workspace = nullptr, size_t workspace_bytes = 0);
 
 // Synthetic benchmark inputs. dtype 0 = f32, 1 = bf16; mode 0 = uniform [a, b), 1 = normal(0, a).
 int launch_fill(void* stream, void* out, size_t n, int dtype, int mode, unsigned long long seed,

@@ -89,8 +89,8 @@ int launch_flash_fwd_bf16_strided(void* stream, const void*, const void*, const 
     return 0;
 }
 int launch_flash_fwd_bf16_ext(void* stream, const void*, const void*, const void*, void*, long, long, long, long, long, float, int,
-                              const long*, const void*, int mask_kind, const long*, float softcap) {
-    mrk_shim_note_launch(stream, mask_kind == 0 && !(softcap > 0.0f) ? "flash_fwd_bf16_strided" : "flash_fwd_bf16_ext");
+                              const long*, const void*, int mask_kind, const long*, float softcap, void* ws, size_t) {
+    mrk_shim_note_launch(stream, mask_kind == 0 && !(softcap > 0.0f) ? "flash_fwd_bf16_strided" : ws ? "flash_fwd_bf16_ext_splitkv" : "flash_fwd_bf16_ext");
     return 0;
 }
 int launch_fill(void* stream, void*, size_t, int, int, unsigned long long, unsigned long long, float, float) {

@@ -228,3 +228,102 @@ def test_decode_full_size_properties(dev):
     ou = synth.from_bf16(_attn(dev, q, ku, v, scale))
     mean = synth.from_bf16(v).astype(np.float64).mean(axis=2, keepdims=True)
     assert np.abs(ou - mean).max() <= 1e-2
+
+
+# ---------------------------------------------------------------- attn_mask over a decode shape
+def _mask_for(kind, layout, B, H, Sq, Sk, seed, keep=0.6):
+    """(host array for the oracle, element strides per batch / head / row) of a mask broadcastable to [B, H, Sq, Sk]."""
+    shape = {"b11k": (B, 1, 1, Sk), "bhqk": (B, H, Sq, Sk), "1hqk": (1, H, Sq, Sk), "qk": (Sq, Sk)}[layout]
+    if kind == "bool":
+        m = synth.uniform(shape, seed, 8) < keep
+        m[..., 0] = True  # no empty row
+    else:
+        m = synth.to_bf16((synth.normal(shape, seed, 9) * 2.0).astype(np.float32))
+    full = (1,) * (4 - len(shape)) + shape
+    dense = [full[1] * full[2] * full[3], full[2] * full[3], full[3]]
+    return m, [0 if full[i] == 1 else dense[i] for i in range(3)]
+
+
+def _attn_masked(dev, q, k, v, scale, mask, mstrides, mode="abi"):
+    B, H, Sq, d = q.shape
+    Sk = k.shape[2]
+    bq, bk, bv = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (q, k, v))
+    bo = dev.buffer(q.nbytes)
+    kind = 1 if mask.dtype == np.bool_ else 2
+    bm = morok_amd.Buffer.from_numpy(mask.view(np.uint8) if kind == 1 else mask, dev.device_id)
+    if mode == "abi":
+        ops.flash_attn_fwd_bf16_ex(bq, bk, bv, bo, B, H, Sq, Sk, d, scale, False, bm, kind, mstrides, 0.0, device_id=dev.device_id)
+    else:
+        bits = int(np.float32(scale).view(np.uint32))
+        dense = lambda rows: [H * rows * d, rows * d, d]
+        params = [B, H, Sq, Sk, d, 0, bits, 0, kind, 0, 0, 0, 0, 0, *dense(Sq), *dense(Sk), *dense(Sk), *dense(Sq), *mstrides]
+        ws = lib.mrk_hip_flash_attn_workspace_bytes(B, H, Sq, Sk, d, 0) if mode == "program_ws" else 0
+        if ws:
+            prog = morok_amd.Program.builtin("flash_fwd_bf16_ext", params + [ws], dev.device_id)
+            assert prog.name.endswith("_splitkv")
+            prog.execute([bo, bq, bk, bv, bm, dev.buffer(ws)])
+        else:
+            morok_amd.Program.builtin("flash_fwd_bf16_ext", params, dev.device_id).execute([bo, bq, bk, bv, bm])
+    return bo.copyout(np.uint16, q.shape)
+
+
+@pytest.mark.parametrize("d", [128, 64, 256])
+@pytest.mark.parametrize("kind,layout", [("bool", "b11k"), ("bool", "bhqk"), ("add", "1hqk"), ("add", "bhqk"), ("bool", "qk")])
+@pytest.mark.parametrize("shape", [(2, 4, 1, 1000), (1, 32, 1, 4096), (3, 2, 5, 516), (1, 2, 16, 2052)])
+def test_decode_mask_vs_oracle(dev, oracle, shape, kind, layout, d):
+    """attn_mask (transformer.rs:112-125) over decode shapes: a key-padding mask [B, 1, 1, Sk] is what a batch of
+    sequences of different lengths decodes with.  The oracle's restatement, through the C entry point and through a
+    Program with and without the scratch buffer."""
+    B, H, Sq, Sk = shape
+    q, k, v = _inputs(B, H, Sq, Sk, d, seed=91)
+    mask, mst = _mask_for(kind, layout, B, H, Sq, Sk, 91)
+    scale = float(d) ** -0.5
+    ref = oracle.sdpa_bf16_ex(q, k, v, scale, causal=False, mask=mask, softcap=0.0)
+    got = _attn_masked(dev, q, k, v, scale, mask, mst)
+    _check(got, ref)
+    assert np.array_equal(_attn_masked(dev, q, k, v, scale, mask, mst, mode="program_ws"), got)
+    _check(_attn_masked(dev, q, k, v, scale, mask, mst, mode="program"), ref)
+
+
+def test_decode_mask_ragged_lengths_and_empty_ranges(dev, oracle):
+    """Sequences of different lengths in one batch (keys past a sequence's length masked out): whole chunks, whole
+    waves' shares and whole key ranges without a visible key must weigh nothing; the result is the unmasked attention
+    over each sequence's own keys.  A sequence with no visible key at all is NaN, as the reference's softmax over
+    -inf only is."""
+    B, H, Sq, Smax, d = 4, 8, 1, 4096, 128
+    lengths = [4096, 1, 700, 33]
+    q, k, v = _inputs(B, H, Sq, Smax, d, seed=92)
+    mask = np.zeros((B, 1, 1, Smax), np.bool_)
+    for b, n in enumerate(lengths):
+        mask[b, ..., :n] = True
+    scale = float(d) ** -0.5
+    assert lib.mrk_hip_flash_attn_workspace_bytes(B, H, Sq, Smax, d, 0) > 0   # 32 pairs: several key ranges
+    got = _attn_masked(dev, q, k, v, scale, mask, [Smax, 0, 0])
+    _check(got, oracle.sdpa_bf16_ex(q, k, v, scale, causal=False, mask=mask, softcap=0.0))
+    for b, n in enumerate(lengths):
+        if n >= 256:  # the same keys without a mask, through the same kernel family
+            alone = _attn(dev, q[b:b + 1], np.ascontiguousarray(k[b:b + 1, :, :n]), np.ascontiguousarray(v[b:b + 1, :, :n]), scale)
+            _check(got[b:b + 1], alone)
+    assert np.array_equal(got[1, :, 0], v[1, :, 0])  # one visible key: its row of V
+    # additive -inf does the same as Bool false
+    add = np.where(mask, np.float32(0), np.float32(-np.inf)).astype(np.float32)
+    got_add = _attn_masked(dev, q, k, v, scale, synth.to_bf16(add), [Smax, 0, 0])
+    _check(got_add, got)
+    # a sequence without any visible key
+    mask[2] = False
+    got = synth.from_bf16(_attn_masked(dev, q, k, v, scale, mask, [Smax, 0, 0]))
+    assert np.all(np.isnan(got[2])) and np.all(np.isfinite(got[[0, 1, 3]]))
+
+
+def test_decode_mask_through_the_tensor_api(dev, oracle):
+    from morok_amd import tensor as T, uop
+
+    B, H, Sk, d = 2, 8, 2048, 128
+    q, k, v = _inputs(B, H, 1, Sk, d, seed=93)
+    mask, _ = _mask_for("bool", "b11k", B, H, 1, Sk, 93)
+    t = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(T.Tensor.from_numpy(k, uop.BF16), T.Tensor.from_numpy(v, uop.BF16),
+                                                                      attn_mask=T.Tensor.from_numpy(mask))
+    got = t.to_numpy()
+    names = [n for n in t.kernels() if n.startswith("flash_fwd")]
+    assert len(names) == 1 and names[0].startswith("flash_fwd_bf16_ext_bool") and names[0].endswith("_splitkv"), t.kernels()
+    _check(got, oracle.sdpa_bf16_ex(q, k, v, float(d) ** -0.5, causal=False, mask=mask, softcap=0.0))
