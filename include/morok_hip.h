@@ -574,9 +574,9 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
  * takes part in the softmax, exactly as the reference's graph computes it; the kernel then visits
  * every key tile.  A row whose keys are all masked out (no softcap) is NaN, as softmax over -inf
  * only is.  Without mask and softcap this is mrk_hip_flash_attn_fwd_bf16_strided.
- * A mask without softcap and causal rule over a decode shape (up to 16 queries, 256 keys and more: a batch of
- * sequences of different lengths decoding under a key-padding mask [batch, 1, 1, sk]) takes the kernel that splits
- * the key sequence, like the unmasked call; key ranges without a visible key weigh nothing.
+ * Without the causal rule a decode shape (up to 16 queries, 256 keys and more: a batch of sequences of different
+ * lengths decoding under a key-padding mask [batch, 1, 1, sk]) takes the kernel that splits the key sequence, like
+ * the unmasked call, mask and softcap inside it; key ranges without a visible key weigh nothing.
  * Builtin Program kind "flash_fwd_bf16_ext" (29 params, buffers {o, q, k, v, mask}; optionally a 30th, the bytes
  * of a scratch buffer that follows the mask: mrk_hip_flash_attn_workspace_bytes). */
 int mrk_hip_flash_attn_fwd_bf16_ex(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,

@@ -1138,8 +1138,8 @@ int mrk_hip_flash_attn_fwd_bf16_ex(int device_id, const void* q, const void* k, 
     std::shared_ptr<Device> dv;
     MRK_TRY(get_device(device_id, &dv));
     MRK_HIP(ffi::set_device(device_id), "hipSetDevice");
-    // (a mask alone over a handful of queries takes the kernel that splits the keys: scratch as in the plain call)
-    const size_t ws = softcap > 0.0f ? 0 : flash_fwd_workspace_bytes(batch * heads, sq, sk, d, causal ? 1 : 0);
+    // (a handful of queries without the causal rule take the kernel that splits the keys: scratch as in the plain call)
+    const size_t ws = flash_fwd_workspace_bytes(batch * heads, sq, sk, d, causal ? 1 : 0);
     RawBuffer scratch;
     BufferOptions so;
     if (ws) MRK_TRY(dv->allocator->alloc(ws, so, &scratch));

@@ -47,6 +47,7 @@ struct DecodeLayout {
 struct DecodeMask {
     const void* mask;
     long long batch, head, row;
+    float cap;  // softcap in score units (transformer.rs:128-132), used by the kCap instantiations
 };
 
 template <int kD>
@@ -54,7 +55,7 @@ constexpr int decode_waves() {
     return kD == 256 ? 4 : 8;  // a wave's region is 4 * 32 * kD bytes: 128 KB of LDS for 128 and 256, 64 KB for 64
 }
 
-template <int kD, int kMask>
+template <int kD, int kMask, bool kCap>
 __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
     const unsigned short* __restrict__ Q, const unsigned short* __restrict__ K, const unsigned short* __restrict__ V,
     unsigned short* __restrict__ O, float* __restrict__ W, int Sq, int Sk, int keys_per_split, float scale_log2e, DecodeLayout lay,
@@ -194,7 +195,18 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
                 x[4 + r] += __builtin_bit_cast(float, (r & 1) ? (w1 & 0xffff0000u) : (w1 << 16)) * 1.4426950408889634f;
             }
         }
-        if (!full) {
+        if constexpr (kCap) {
+            // cap * tanh(x / cap) after the mask, with tanh(y) = 1 - 2 / (exp(2 y) + 1); x in exp2 units, so
+            // exp(2 x / cap) = exp2(2 t / cap); a masked score (-inf) becomes -cap and still takes part, as in
+            // the reference's graph
+            const float cap_out = dm.cap * 1.4426950408889634f, cap_in = 2.0f / dm.cap;
+#pragma unroll
+            for (int r = 0; r < 8; r++) {
+                const float z = __builtin_amdgcn_exp2f(x[r] * cap_in);
+                x[r] = cap_out * (1.0f - 2.0f * __builtin_amdgcn_rcpf(z + 1.0f));
+            }
+        }
+        if (!full) {  // keys that do not exist
 #pragma unroll
             for (int r = 0; r < 4; r++) {
                 if (4 * blk + r > last) x[r] = -INFINITY;
@@ -207,7 +219,7 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
         const float m_new = fmaxf(m_run, mx);  // without a mask finite: the chunk's first key is valid
         // under a mask every key so far may be masked out (maximum -inf): such keys weigh nothing, and nothing has been
         // summed yet; the differences below must not become -inf - -inf
-        const float m_ref = kMask != 0 && m_new == -INFINITY ? 0.0f : m_new;
+        const float m_ref = kMask != 0 && !kCap && m_new == -INFINITY ? 0.0f : m_new;
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_ref);
         m_run = m_new;
         f32x8 p;
@@ -359,10 +371,10 @@ size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal) 
 // strides: (batch, head, row) element strides of q, k, v and o (validated by the caller: multiples of 8, rows
 // addressable in 32 bits, pointers 16-byte aligned); W: splits * B * H * 16 * (D + 2) floats, needed with several splits.
 // mask_kind 0: none; 1: Bool bytes, 2: additive bf16, with (batch, head, query row) element strides that are multiples
-// of 4, a mask pointer aligned to four elements and Sk a multiple of 4 (validated by the caller as well).
+// of 4, a mask pointer aligned to four elements and Sk a multiple of 4 (validated by the caller as well).  softcap 0: none.
 int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
                         float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask, int mask_kind,
-                        const long* mask_strides) {
+                        const long* mask_strides, float softcap) {
     if (B <= 0 || H <= 0 || Sq < 1 || Sq > kMaxQueries || Sk < 1 || splits < 1 || B * H > 65535) return (int)hipErrorInvalidValue;
     if (keys_per_split < kChunkKeys || keys_per_split % kChunkKeys || splits * keys_per_split < Sk || (splits - 1) * keys_per_split >= Sk)
         return (int)hipErrorInvalidValue;
@@ -373,8 +385,10 @@ int launch_flash_decode(void* stream, const void* q, const void* k, const void* 
     lay.v_batch = strides[6], lay.v_head = strides[7], lay.v_row = (unsigned)(strides[8] * 2);
     lay.o_batch = strides[9], lay.o_head = strides[10], lay.o_row = (unsigned)(strides[11] * 2);
     lay.heads = (int)H;
-    if (mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && (!mask || !mask_strides || Sk % 4))) return (int)hipErrorInvalidValue;
+    if (mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && (!mask || !mask_strides || Sk % 4)) || !(softcap >= 0.0f)) return (int)hipErrorInvalidValue;
     DecodeMask dm{};
+    dm.cap = softcap;
+    const bool cap = softcap > 0.0f;
     if (mask_kind != 0) {
         dm.mask = mask;
         dm.batch = mask_strides[0], dm.head = mask_strides[1], dm.row = mask_strides[2];
@@ -390,8 +404,15 @@ int launch_flash_decode(void* stream, const void* q, const void* k, const void* 
     (void)hipGetLastError();
     const long quads = B * H * Sq * (D / 4);
     const unsigned merge_blocks = (unsigned)((quads + 255) / 256);
-#define MRK_DECODE(DIM, MASK) \
-    flash_decode_split<DIM, MASK><<<grid, decode_waves<DIM>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split, scale_log2e, lay, dm)
+#define MRK_DECODE(DIM, MASK)                                                                                                                          \
+    do {                                                                                                                                               \
+        if (cap)                                                                                                                                       \
+            flash_decode_split<DIM, MASK, true><<<grid, decode_waves<DIM>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split,     \
+                                                                                           scale_log2e, lay, dm);                                     \
+        else                                                                                                                                           \
+            flash_decode_split<DIM, MASK, false><<<grid, decode_waves<DIM>() * 64, 0, s>>>(qp, kp, vp, op, w, (int)Sq, (int)Sk, (int)keys_per_split,    \
+                                                                                            scale_log2e, lay, dm);                                    \
+    } while (0)
 #define MRK_DECODE_DIM(DIM)                                                                                         \
     do {                                                                                                            \
         if (mask_kind == 0) MRK_DECODE(DIM, 0);                                                                     \

@@ -661,7 +661,7 @@ namespace mrk {
 // ranges as the workspace allows (one range needs none).
 static bool decode_route(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
                          float scale, int causal, const long* strides, void* workspace, size_t workspace_bytes, int* rc,
-                         const void* mask = nullptr, int mask_kind = 0, const long* mask_strides = nullptr) {
+                         const void* mask = nullptr, int mask_kind = 0, const long* mask_strides = nullptr, float softcap = 0.0f) {
     using namespace mrk::dev;
     long splits = 0, per = 0;
     if (!flash_decode_plan(B * H, Sq, Sk, D, causal, &splits, &per)) return false;
@@ -672,7 +672,8 @@ static bool decode_route(void* stream, const void* q, const void* k, const void*
         splits = 1;
         per = (Sk + 31) / 32 * 32;
     }
-    *rc = launch_flash_decode(stream, q, k, v, o, B, H, Sq, Sk, D, scale, strides, splits, per, workspace, mask, mask_kind, mask_strides);
+    *rc = launch_flash_decode(stream, q, k, v, o, B, H, Sq, Sk, D, scale, strides, splits, per, workspace, mask, mask_kind, mask_strides,
+                              softcap);
     return true;
 }
 
@@ -785,9 +786,10 @@ int launch_flash_fwd_bf16_ext(void* stream, const void* q, const void* k, const 
         ext.batch = mask_strides[0], ext.head = mask_strides[1], ext.row = mask_strides[2];
     }
     const bool cap = softcap > 0.0f;
-    if (!cap) {  // a mask alone over a handful of queries: the kernel that splits the keys
+    {  // a handful of queries without the causal rule: the kernel that splits the keys
         int rc = 0;
-        if (decode_route(stream, q, k, v, o, B, H, Sq, Sk, D, scale, causal, strides, workspace, workspace_bytes, &rc, mask, mask_kind, mask_strides))
+        if (decode_route(stream, q, k, v, o, B, H, Sq, Sk, D, scale, causal, strides, workspace, workspace_bytes, &rc, mask, mask_kind, mask_strides,
+                         softcap))
             return rc;
     }
     ext.cap = softcap;

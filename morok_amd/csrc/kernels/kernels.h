@@ -125,7 +125,7 @@ bool flash_decode_plan(long BH, long Sq, long Sk, long D, int causal, long* spli
 size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal);
 int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
                         float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask = nullptr,
-                        int mask_kind = 0, const long* mask_strides = nullptr);
+                        int mask_kind = 0, const long* mask_strides = nullptr, float softcap = 0.0f);
 int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
                           long D, float scale, int causal, void* workspace = nullptr, size_t workspace_bytes = 0);
 // The same kernel over operands given as views: strides holds (batch, head, row) element
@@ -144,8 +144,8 @@ int launch_flash_fwd_bf16_strided(void* stream, const void* q, const void* k, co
 // (causal ones included) turn into -softcap and still take part, as in the reference.  A row
 // whose keys are all masked out (no softcap) comes out as NaN, as the reference's softmax does.
 // Without mask and softcap this is launch_flash_fwd_bf16_strided.
-// A mask without softcap and causal rule over a decode shape (see flash_decode_plan) takes the split kernel as well,
-// with the same workspace.
+// Without the causal rule a decode shape (see flash_decode_plan) takes the split kernel here as well, mask and
+// softcap inside it, with the same workspace.
 int launch_flash_fwd_bf16_ext(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk,
                               long D, float scale, int causal, const long* strides, const void* mask, int mask_kind,
                               const long* mask_strides, float softcap, void* workspace = nullptr, size_t workspace_bytes = 0);

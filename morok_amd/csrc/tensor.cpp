@@ -2105,8 +2105,8 @@ struct Scheduler {
             params.insert(params.end(), strides.begin(), strides.end());
             params.insert(params.end(), mask_strides, mask_strides + 3);
             bufs.push_back(has_mask ? mask_buf : bufs[1]);
-            // a mask alone over a handful of queries: the kernel that splits the keys, with its scratch
-            const size_t ws = att->hint_softcap > 0.0 ? 0 : flash_fwd_workspace_bytes(B * H, Sq, Sk, D, att->hint_causal ? 1 : 0);
+            // a handful of queries without the causal rule: the kernel that splits the keys, with its scratch
+            const size_t ws = flash_fwd_workspace_bytes(B * H, Sq, Sk, D, att->hint_causal ? 1 : 0);
             if (ws) {
                 bufs.push_back(std::make_shared<Buffer>(dev->allocator, ws, BufferOptions()));
                 params.push_back(static_cast<int64_t>(ws));

@@ -244,19 +244,22 @@ def _mask_for(kind, layout, B, H, Sq, Sk, seed, keep=0.6):
     return m, [0 if full[i] == 1 else dense[i] for i in range(3)]
 
 
-def _attn_masked(dev, q, k, v, scale, mask, mstrides, mode="abi"):
+def _attn_masked(dev, q, k, v, scale, mask, mstrides, mode="abi", cap=0.0):
     B, H, Sq, d = q.shape
     Sk = k.shape[2]
     bq, bk, bv = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (q, k, v))
     bo = dev.buffer(q.nbytes)
-    kind = 1 if mask.dtype == np.bool_ else 2
-    bm = morok_amd.Buffer.from_numpy(mask.view(np.uint8) if kind == 1 else mask, dev.device_id)
+    kind = 0 if mask is None else 1 if mask.dtype == np.bool_ else 2
+    bm = morok_amd.Buffer.from_numpy(mask.view(np.uint8) if kind == 1 else mask, dev.device_id) if kind else bq
+    mstrides = mstrides if kind else [0, 0, 0]
     if mode == "abi":
-        ops.flash_attn_fwd_bf16_ex(bq, bk, bv, bo, B, H, Sq, Sk, d, scale, False, bm, kind, mstrides, 0.0, device_id=dev.device_id)
+        ops.flash_attn_fwd_bf16_ex(bq, bk, bv, bo, B, H, Sq, Sk, d, scale, False, bm if kind else None, kind, mstrides, cap,
+                                   device_id=dev.device_id)
     else:
         bits = int(np.float32(scale).view(np.uint32))
+        cbits = int(np.float32(cap).view(np.uint32)) if cap else 0
         dense = lambda rows: [H * rows * d, rows * d, d]
-        params = [B, H, Sq, Sk, d, 0, bits, 0, kind, 0, 0, 0, 0, 0, *dense(Sq), *dense(Sk), *dense(Sk), *dense(Sq), *mstrides]
+        params = [B, H, Sq, Sk, d, 0, bits, cbits, kind, 0, 0, 0, 0, 0, *dense(Sq), *dense(Sk), *dense(Sk), *dense(Sq), *mstrides]
         ws = lib.mrk_hip_flash_attn_workspace_bytes(B, H, Sq, Sk, d, 0) if mode == "program_ws" else 0
         if ws:
             prog = morok_amd.Program.builtin("flash_fwd_bf16_ext", params + [ws], dev.device_id)
@@ -283,6 +286,29 @@ def test_decode_mask_vs_oracle(dev, oracle, shape, kind, layout, d):
     _check(got, ref)
     assert np.array_equal(_attn_masked(dev, q, k, v, scale, mask, mst, mode="program_ws"), got)
     _check(_attn_masked(dev, q, k, v, scale, mask, mst, mode="program"), ref)
+
+
+@pytest.mark.parametrize("d", [128, 64, 256])
+@pytest.mark.parametrize("cap", [1.5, 30.0])
+@pytest.mark.parametrize("kind,layout", [("none", None), ("bool", "b11k"), ("add", "bhqk")])
+def test_decode_softcap_vs_oracle(dev, oracle, kind, layout, cap, d):
+    """softcap (transformer.rs:128-132) inside the split kernel, alone and after a mask: a masked score becomes -cap and
+    still takes part, as in the reference's graph."""
+    B, H, Sq, Sk = 2, 4, 3, 1540
+    q, k, v = _inputs(B, H, Sq, Sk, d, seed=94)
+    mask, mst = (None, None) if kind == "none" else _mask_for(kind, layout, B, H, Sq, Sk, 94)
+    scale = float(d) ** -0.5
+    ref = oracle.sdpa_bf16_ex(q, k, v, scale, causal=False, mask=mask, softcap=cap)
+    got = _attn_masked(dev, q, k, v, scale, mask, mst, cap=cap)
+    _check(got, ref)
+    assert np.array_equal(_attn_masked(dev, q, k, v, scale, mask, mst, mode="program_ws", cap=cap), got)
+    _check(_attn_masked(dev, q, k, v, scale, mask, mst, mode="program", cap=cap), ref)
+    if kind == "bool":
+        # every key masked out under a cap: all scores -cap, the mean of V (not NaN)
+        none = np.zeros_like(mask)
+        o = synth.from_bf16(_attn_masked(dev, q, k, v, scale, none, mst, cap=cap))
+        mean = synth.from_bf16(v).astype(np.float64).mean(axis=2, keepdims=True)
+        assert np.abs(o - mean).max() <= 1e-2
 
 
 def test_decode_mask_ragged_lengths_and_empty_ranges(dev, oracle):
