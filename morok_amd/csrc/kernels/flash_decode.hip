@@ -39,7 +39,8 @@ constexpr int kMaxQueries = 16;
 struct DecodeLayout {
     long long q_batch, q_head, k_batch, k_head, v_batch, v_head, o_batch, o_head;  // element strides
     unsigned q_row, k_row, v_row, o_row;                                           // byte strides of a row
-    int heads;
+    int heads;  // (batch, head) pairs per batch: the head count, or 1 when the heads are folded into one pair
+    int group;  // heads folded into one pair's query slots (they share K and V: zero head strides), 1 = none
 };
 
 // attn_mask of the reference (transformer.rs:112-125) as a [batch, head, query, key] view with contiguous keys:
@@ -84,15 +85,18 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
     const char* v_head = reinterpret_cast<const char*>(V + b * lay.v_batch + h * lay.v_head);
 
     // the queries: operand B, query jl (the last one again beyond Sq), eight d at 32 s + 8 blk
+    // (query slots: head g of a folded group, row r of its Sq rows, slot g * Sq + r)
     u32x4 qf[kSteps];
-    const int qi = jl < Sq ? jl : Sq - 1;
+    const int nq = Sq * lay.group;
+    const int slot = jl < nq ? jl : nq - 1;
+    const int qg = slot / Sq, qi = slot - qg * Sq;
     // the mask row of this lane's query: a lane needs the mask of its eight keys per chunk, two groups of four
     // consecutive ones (the key count is a multiple of 4 under a mask, so a group is inside the sequence or outside)
     const char* mrow = nullptr;
     if constexpr (kMask != 0)
-        mrow = static_cast<const char*>(dm.mask) + (b * dm.batch + h * dm.head + qi * dm.row) * (kMask == 2 ? 2 : 1);
+        mrow = static_cast<const char*>(dm.mask) + (b * dm.batch + (h + qg) * dm.head + qi * dm.row) * (kMask == 2 ? 2 : 1);
     {
-        const char* qrow = reinterpret_cast<const char*>(Q + b * lay.q_batch + h * lay.q_head) + (size_t)qi * lay.q_row;
+        const char* qrow = reinterpret_cast<const char*>(Q + b * lay.q_batch + (h + qg) * lay.q_head) + (size_t)qi * lay.q_row;
 #pragma unroll
         for (int s = 0; s < kSteps; s++) qf[s] = *reinterpret_cast<const u32x4*>(qrow + 64 * s + 16 * blk);
     }
@@ -270,7 +274,7 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
     // element e: column block e / 64, lane l = e % 64 of it: query l % 16, columns 16 c + 4 (l / 16) + 0..3
     for (int e = threadIdx.x; e < kColBlocks * 64; e += kWaves * 64) {
         const int c = e >> 6, l = e & 63, q = l & 15;
-        if (q >= Sq) continue;
+        if (q >= nq) continue;
         float m_tot = -INFINITY;
 #pragma unroll
         for (int w = 0; w < kWaves; w++) m_tot = fmaxf(m_tot, reinterpret_cast<const float*>(part + w * kPartBytes + kColBlocks * 1024)[q]);
@@ -298,23 +302,25 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
         } else {
             const float inv = 1.0f / l_tot;
             const f32x4 v = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
-            char* orow = reinterpret_cast<char*>(O + b * lay.o_batch + h * lay.o_head) + (size_t)q * lay.o_row;
+            const int og = q / Sq, orw = q - og * Sq;
+            char* orow = reinterpret_cast<char*>(O + b * lay.o_batch + (h + og) * lay.o_head) + (size_t)orw * lay.o_row;
             *reinterpret_cast<bf16x4*>(orow + d * 2) = __builtin_convertvector(v, bf16x4);
         }
     }
 }
 
 // O[bh][q][d] from the splits' partial results: the same merge as inside a workgroup, splits in order.
-// One work-item per four columns; grid = ceil(BH * Sq * D / 4 / 256).
+// One work-item per four columns; grid = ceil(pairs * slots * D / 4 / 256) with slots = Sq * group query slots per pair.
 template <int kD>
 __global__ __launch_bounds__(256) void flash_decode_merge(const float* __restrict__ W, unsigned short* __restrict__ O, int BH, int Sq, int splits,
                                                           DecodeLayout lay) {
     const long e = (long)blockIdx.x * 256 + threadIdx.x;
     constexpr int kQuads = kD / 4;
-    if (e >= (long)BH * Sq * kQuads) return;
+    const int nq = Sq * lay.group;
+    if (e >= (long)BH * nq * kQuads) return;
     const int d = (int)(e % kQuads) * 4;
-    const int q = (int)((e / kQuads) % Sq);
-    const int bh = (int)(e / ((long)kQuads * Sq));
+    const int q = (int)((e / kQuads) % nq);
+    const int bh = (int)(e / ((long)kQuads * nq));
     const size_t slice = (size_t)BH * kMaxQueries * (kD + 2);
     const float* src = W + ((size_t)bh * kMaxQueries + q) * (kD + 2);
     // (both loops unrolled by four: the loads of four ranges are in flight together, the sums keep their order)
@@ -333,8 +339,8 @@ __global__ __launch_bounds__(256) void flash_decode_merge(const float* __restric
     }
     const float inv = 1.0f / l_tot;
     const f32x4 v = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
-    const int b = bh / lay.heads, h = bh % lay.heads;
-    char* orow = reinterpret_cast<char*>(O + b * lay.o_batch + h * lay.o_head) + (size_t)q * lay.o_row;
+    const int b = bh / lay.heads, h = bh % lay.heads, og = q / Sq, orw = q - og * Sq;
+    char* orow = reinterpret_cast<char*>(O + b * lay.o_batch + (h + og) * lay.o_head) + (size_t)orw * lay.o_row;
     *reinterpret_cast<bf16x4*>(orow + d * 2) = __builtin_convertvector(v, bf16x4);
 }
 
@@ -362,20 +368,33 @@ bool flash_decode_plan(long BH, long Sq, long Sk, long D, int causal, long* spli
     return true;
 }
 
+// The workspace a caller provides for (batch * heads) pairs: enough for the plan over those pairs and for the plans
+// over fewer pairs that folding heads which share their keys gives (the launchers see the strides, the caller of this
+// function need not).
 size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal) {
-    long splits = 0, per = 0;
-    if (!flash_decode_plan(BH, Sq, Sk, D, causal, &splits, &per) || splits <= 1) return 0;
-    return (size_t)splits * BH * kMaxQueries * (D + 2) * sizeof(float);
+    size_t most = 0;
+    for (long g = 1; g * Sq <= kMaxQueries && g <= BH; g++) {
+        if (BH % g) continue;
+        long splits = 0, per = 0;
+        if (!flash_decode_plan(BH / g, Sq * g, Sk, D, causal, &splits, &per) || splits <= 1) continue;
+        const size_t need = (size_t)splits * (BH / g) * kMaxQueries * (D + 2) * sizeof(float);
+        most = need > most ? need : most;
+    }
+    return most;
 }
 
 // strides: (batch, head, row) element strides of q, k, v and o (validated by the caller: multiples of 8, rows
-// addressable in 32 bits, pointers 16-byte aligned); W: splits * B * H * 16 * (D + 2) floats, needed with several splits.
+// addressable in 32 bits, pointers 16-byte aligned); W: splits * pairs * 16 * (D + 2) floats, needed with several splits
+// (pairs = B * H, or B with fold_heads).
 // mask_kind 0: none; 1: Bool bytes, 2: additive bf16, with (batch, head, query row) element strides that are multiples
 // of 4, a mask pointer aligned to four elements and Sk a multiple of 4 (validated by the caller as well).  softcap 0: none.
 int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
                         float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask, int mask_kind,
-                        const long* mask_strides, float softcap) {
-    if (B <= 0 || H <= 0 || Sq < 1 || Sq > kMaxQueries || Sk < 1 || splits < 1 || B * H > 65535) return (int)hipErrorInvalidValue;
+                        const long* mask_strides, float softcap, bool fold_heads) {
+    // fold_heads: the H heads of a batch share K and V (zero head strides) and become query slots of one pair
+    const long pairs = fold_heads ? B : B * H, slots = fold_heads ? H * Sq : Sq;
+    if (B <= 0 || H <= 0 || Sq < 1 || slots > kMaxQueries || Sk < 1 || splits < 1 || pairs > 65535) return (int)hipErrorInvalidValue;
+    if (fold_heads && (strides[4] != 0 || strides[7] != 0)) return (int)hipErrorInvalidValue;
     if (keys_per_split < kChunkKeys || keys_per_split % kChunkKeys || splits * keys_per_split < Sk || (splits - 1) * keys_per_split >= Sk)
         return (int)hipErrorInvalidValue;
     if (splits > 1 && !W) return (int)hipErrorInvalidValue;
@@ -384,7 +403,8 @@ int launch_flash_decode(void* stream, const void* q, const void* k, const void* 
     lay.k_batch = strides[3], lay.k_head = strides[4], lay.k_row = (unsigned)(strides[5] * 2);
     lay.v_batch = strides[6], lay.v_head = strides[7], lay.v_row = (unsigned)(strides[8] * 2);
     lay.o_batch = strides[9], lay.o_head = strides[10], lay.o_row = (unsigned)(strides[11] * 2);
-    lay.heads = (int)H;
+    lay.heads = fold_heads ? 1 : (int)H;
+    lay.group = fold_heads ? (int)H : 1;
     if (mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && (!mask || !mask_strides || Sk % 4)) || !(softcap >= 0.0f)) return (int)hipErrorInvalidValue;
     DecodeMask dm{};
     dm.cap = softcap;
@@ -395,14 +415,14 @@ int launch_flash_decode(void* stream, const void* q, const void* k, const void* 
     }
     const float scale_log2e = scale * 1.4426950408889634f;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const dim3 grid((unsigned)splits, (unsigned)(B * H));
+    const dim3 grid((unsigned)splits, (unsigned)pairs);
     float* w = splits > 1 ? static_cast<float*>(W) : nullptr;
     auto qp = static_cast<const unsigned short*>(q);
     auto kp = static_cast<const unsigned short*>(k);
     auto vp = static_cast<const unsigned short*>(v);
     auto op = static_cast<unsigned short*>(o);
     (void)hipGetLastError();
-    const long quads = B * H * Sq * (D / 4);
+    const long quads = pairs * slots * (D / 4);
     const unsigned merge_blocks = (unsigned)((quads + 255) / 256);
 #define MRK_DECODE(DIM, MASK)                                                                                                                          \
     do {                                                                                                                                               \
@@ -418,7 +438,7 @@ int launch_flash_decode(void* stream, const void* q, const void* k, const void* 
         if (mask_kind == 0) MRK_DECODE(DIM, 0);                                                                     \
         else if (mask_kind == 1) MRK_DECODE(DIM, 1);                                                                \
         else MRK_DECODE(DIM, 2);                                                                                    \
-        if (w) flash_decode_merge<DIM><<<merge_blocks, 256, 0, s>>>(w, op, (int)(B * H), (int)Sq, (int)splits, lay); \
+        if (w) flash_decode_merge<DIM><<<merge_blocks, 256, 0, s>>>(w, op, (int)pairs, (int)Sq, (int)splits, lay);   \
     } while (0)
     if (D == 128) MRK_DECODE_DIM(128);
     else if (D == 64) MRK_DECODE_DIM(64);

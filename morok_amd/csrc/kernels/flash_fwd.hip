@@ -663,17 +663,25 @@ static bool decode_route(void* stream, const void* q, const void* k, const void*
                          float scale, int causal, const long* strides, void* workspace, size_t workspace_bytes, int* rc,
                          const void* mask = nullptr, int mask_kind = 0, const long* mask_strides = nullptr, float softcap = 0.0f) {
     using namespace mrk::dev;
+    // heads that share K and V (zero head strides) become query slots of one pair: K and V are read once per batch
+    const bool fold = H > 1 && H * Sq <= 16 && strides[4] == 0 && strides[7] == 0;
+    const long pairs = fold ? B : B * H, slots = fold ? H * Sq : Sq;
     long splits = 0, per = 0;
-    if (!flash_decode_plan(B * H, Sq, Sk, D, causal, &splits, &per)) return false;
+    if (!flash_decode_plan(pairs, slots, Sk, D, causal, &splits, &per)) return false;
     const void* ptrs[4] = {q, k, v, o};
     for (const void* p : ptrs)
         if (reinterpret_cast<uintptr_t>(p) % 16) return false;
-    if (splits > 1 && (!workspace || workspace_bytes < flash_fwd_workspace_bytes(B * H, Sq, Sk, D, causal))) {
-        splits = 1;
-        per = (Sk + 31) / 32 * 32;
+    if (splits > 1) {  // as many key ranges as the workspace holds
+        const size_t slice = (size_t)pairs * 16 * (D + 2) * sizeof(float);
+        const long fit = workspace ? (long)(workspace_bytes / slice) : 0;
+        if (fit < splits) {
+            const long want = fit < 2 ? 1 : fit;
+            per = ((Sk + want - 1) / want + 31) / 32 * 32;
+            splits = (Sk + per - 1) / per;
+        }
     }
     *rc = launch_flash_decode(stream, q, k, v, o, B, H, Sq, Sk, D, scale, strides, splits, per, workspace, mask, mask_kind, mask_strides,
-                              softcap);
+                              softcap, fold);
     return true;
 }
 

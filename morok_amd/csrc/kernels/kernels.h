@@ -120,12 +120,15 @@ inline bool flash_fwd_rows_addressable(long rows, long row_bytes, long D) {
 // Up to 16 queries without the causal rule against 256 keys and more (a decode step over a key/value cache) take
 // a kernel that also splits the key sequence over workgroups (flash_decode_plan tells how); with several key
 // ranges their f32 partial results go through `workspace` (flash_fwd_workspace_bytes; 0 = one range), which a
-// second kernel merges.  Without a workspace of that size such a shape runs as one range per (batch, head).
+// second kernel merges.  Without a workspace of that size such a shape runs in as many ranges as the workspace holds.
+// Heads that share their keys and values (zero head strides of k and v: multi-query attention, or grouped-query
+// attention with the groups as batches) are folded into one pair's query slots while heads * Sq <= 16, so that K and
+// V are read once per batch instead of once per head.
 bool flash_decode_plan(long BH, long Sq, long Sk, long D, int causal, long* splits, long* keys_per_split);
 size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal);
 int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
                         float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask = nullptr,
-                        int mask_kind = 0, const long* mask_strides = nullptr, float softcap = 0.0f);
+                        int mask_kind = 0, const long* mask_strides = nullptr, float softcap = 0.0f, bool fold_heads = false);
 int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
                           long D, float scale, int causal, void* workspace = nullptr, size_t workspace_bytes = 0);
 // The same kernel over operands given as views: strides holds (batch, head, row) element

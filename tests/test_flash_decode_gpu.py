@@ -78,10 +78,13 @@ def test_decode_shapes_split_the_keys_where_pairs_are_few():
     ws = lib.mrk_hip_flash_attn_workspace_bytes
     assert ws(1, 32, 1, 4096, 128, 0) > 0 and ws(1, 8, 4, 8192, 64, 0) > 0 and ws(2, 16, 16, 2048, 256, 0) > 0
     assert ws(1, 32, 1, 4096, 128, 0) % (32 * 16 * 130 * 4) == 0  # whole slices of [pairs][16][D + 2] floats
-    # enough pairs by themselves, the causal rule, many queries, few keys, no kernel for the head dim: no scratch
-    for args in ((16, 32, 1, 4096, 128, 0), (1, 32, 1, 4096, 128, 1), (1, 32, 17, 4096, 128, 0), (1, 32, 1, 255, 128, 0),
-                 (1, 32, 1, 4096, 96, 0), (0, 32, 1, 4096, 128, 0)):
+    # the causal rule, many queries, few keys, no kernel for the head dim: no scratch
+    for args in ((1, 32, 1, 4096, 128, 1), (1, 32, 17, 4096, 128, 0), (1, 32, 1, 255, 128, 0), (1, 32, 1, 4096, 96, 0), (0, 32, 1, 4096, 128, 0)):
         assert ws(*args) == 0, args
+    # 512 pairs fill the chip by themselves, but should their heads share K and V (the launchers see the strides, this
+    # query does not) they fold into as few as 32 pairs, which split their keys: a bounded reserve for that
+    assert 0 < ws(16, 32, 1, 4096, 128, 0) <= 4 << 20
+    assert ws(16, 32, 16, 4096, 128, 0) == 0   # 16 queries a head: nothing to fold
 
 
 @pytest.mark.parametrize("d", [128, 64, 256])
@@ -353,3 +356,73 @@ def test_decode_mask_through_the_tensor_api(dev, oracle):
     names = [n for n in t.kernels() if n.startswith("flash_fwd")]
     assert len(names) == 1 and names[0].startswith("flash_fwd_bf16_ext_bool") and names[0].endswith("_splitkv"), t.kernels()
     _check(got, oracle.sdpa_bf16_ex(q, k, v, float(d) ** -0.5, causal=False, mask=mask, softcap=0.0))
+
+
+# ---------------------------------------------------------------- heads that share their keys and values
+def _attn_shared(dev, q, k1, v1, scale, mask=None, mstrides=None):
+    """q [B, H, Sq, d] against k1 / v1 [B, 1, Sk, d] shared by the H heads of a batch (head stride 0: what `expand` over
+    the head axis hands over), through the strided entry point, or the extended one with a mask."""
+    B, H, Sq, d = q.shape
+    Sk = k1.shape[2]
+    strides = [H * Sq * d, Sq * d, d, Sk * d, 0, d, Sk * d, 0, d, H * Sq * d, Sq * d, d]
+    bq, bk, bv = (morok_amd.Buffer.from_numpy(t, dev.device_id) for t in (q, k1, v1))
+    guard = np.full((B * H * Sq + 2, d), 0x7FC0, np.uint16)
+    bo = morok_amd.Buffer.from_numpy(guard, dev.device_id)
+    if mask is None:
+        ops.flash_attn_fwd_bf16_strided(bq, bk, bv, bo, B, H, Sq, Sk, d, scale, strides, [0, 0, 0, 0], False, dev.device_id)
+    else:
+        kind = 1 if mask.dtype == np.bool_ else 2
+        bm = morok_amd.Buffer.from_numpy(mask.view(np.uint8) if kind == 1 else mask, dev.device_id)
+        ops.flash_attn_fwd_bf16_ex(bq, bk, bv, bo, B, H, Sq, Sk, d, scale, False, bm, kind, mstrides, 0.0, strides=strides,
+                                   device_id=dev.device_id)
+    out = bo.copyout(np.uint16, guard.shape)
+    assert np.all(out[B * H * Sq:] == 0x7FC0)
+    return out[:B * H * Sq].reshape(q.shape)
+
+
+@pytest.mark.parametrize("d", [128, 64, 256])
+@pytest.mark.parametrize("shape", [(2, 8, 1, 3000), (1, 16, 1, 4096), (3, 4, 4, 777), (8, 4, 1, 1024), (2, 5, 3, 515), (1, 9, 2, 600)])
+def test_decode_heads_sharing_keys_are_folded(dev, oracle, shape, d):
+    """Multi-query attention (and grouped-query attention with the groups as batches): the heads of a batch read the
+    same K and V; while heads * Sq <= 16 they become query slots of one pass over the keys.  The oracle's values over
+    broadcast copies; (1, 9, 2, 600) has 18 slots and runs head by head."""
+    B, H, Sq, Sk = shape
+    q = synth.normal_bf16((B, H, Sq, d), 95, 0)
+    k1, v1 = synth.normal_bf16((B, 1, Sk, d), 95, 1), synth.normal_bf16((B, 1, Sk, d), 95, 2)
+    kb, vb = (np.ascontiguousarray(np.broadcast_to(t, (B, H, Sk, d))) for t in (k1, v1))
+    scale = float(d) ** -0.5
+    got = _attn_shared(dev, q, k1, v1, scale)
+    ref = oracle.sdpa_bf16(q, kb, vb, scale, causal=False)
+    _check(got, ref)
+    _check(got, _attn(dev, q, kb, vb, scale), tight=1e-2)   # the unfolded kernel over copies
+    assert np.array_equal(_attn_shared(dev, q, k1, v1, scale), got)
+
+
+def test_decode_folded_heads_under_masks(dev, oracle):
+    B, H, Sq, Sk, d = 2, 8, 2, 2052, 128
+    q = synth.normal_bf16((B, H, Sq, d), 96, 0)
+    k1, v1 = synth.normal_bf16((B, 1, Sk, d), 96, 1), synth.normal_bf16((B, 1, Sk, d), 96, 2)
+    kb, vb = (np.ascontiguousarray(np.broadcast_to(t, (B, H, Sk, d))) for t in (k1, v1))
+    scale = float(d) ** -0.5
+    for kind, layout in (("bool", "b11k"), ("bool", "bhqk"), ("add", "1hqk")):
+        mask, mst = _mask_for(kind, layout, B, H, Sq, Sk, 96)
+        got = _attn_shared(dev, q, k1, v1, scale, mask, mst)
+        _check(got, oracle.sdpa_bf16_ex(q, kb, vb, scale, causal=False, mask=mask, softcap=0.0))
+
+
+def test_decode_folded_heads_through_the_tensor_api(dev, oracle):
+    """K and V of one head expanded over the query heads: read in place with a zero head stride, the heads folded."""
+    from morok_amd import tensor as T, uop
+
+    B, H, Sk, d = 2, 8, 2048, 128
+    q = synth.normal_bf16((B, H, 1, d), 97, 0)
+    k1, v1 = synth.normal_bf16((B, 1, Sk, d), 97, 1), synth.normal_bf16((B, 1, Sk, d), 97, 2)
+    tk = T.Tensor.from_numpy(k1, uop.BF16).try_expand([B, H, Sk, d])
+    tv = T.Tensor.from_numpy(v1, uop.BF16).try_expand([B, H, Sk, d])
+    t = T.Tensor.from_numpy(q, uop.BF16).scaled_dot_product_attention(tk, tv)
+    got = t.to_numpy()
+    names = t.kernels()
+    assert len(names) == 1 and names[0].startswith("flash_fwd_bf16_strided"), names
+    kb, vb = (np.ascontiguousarray(np.broadcast_to(x, (B, H, Sk, d))) for x in (k1, v1))
+    _check(got, oracle.sdpa_bf16(q, kb, vb, float(d) ** -0.5, causal=False))
+    assert np.array_equal(got, _attn_shared(dev, q, k1, v1, float(d) ** -0.5))
