@@ -707,6 +707,30 @@ def bench_flash_decode(m, dev, steps, warmup, cpu):
         ms8, _, algo8, _ = run(8)
         rec["batch_8"] = {"us_per_launch": ms8 * 1e3 / layers, "GB/s": layers * algo8 / (ms8 * 1e-3) / 1e9,
                           "frac": layers * algo8 / (ms8 * 1e-3) / 1e9 / HBM_PEAK_GBS}
+        dev.synchronize()
+        dev.lru_clear()
+        # grouped-query attention: a batch of 16 with 8 key heads and 8 query heads each, K and V with a zero head stride
+        # (batch x key heads as batches): one pass over a key head's 4096 keys serves its 8 query heads
+        groups, G = 16 * 8, 8
+        n_kv, n_q = groups * Sk * D, groups * G * D
+        bq, bo = dev.buffer(n_q * 2).ensure_allocated(), dev.buffer(n_q * 2).ensure_allocated()
+        ops.fill_normal(bq, n_q, seed=12, tensor_id=0, bf16=True)
+        kvs = []
+        for i in range(4):
+            k, v = dev.buffer(n_kv * 2).ensure_allocated(), dev.buffer(n_kv * 2).ensure_allocated()
+            ops.fill_normal(k, n_kv, seed=12, tensor_id=1 + 2 * i, bf16=True)
+            ops.fill_normal(v, n_kv, seed=12, tensor_id=2 + 2 * i, bf16=True)
+            kvs.append((k, v))
+        st = [G * D, D, D, Sk * D, 0, D, Sk * D, 0, D, G * D, D, D]
+
+        def gqa_step():
+            for k, v in kvs:
+                ops.flash_attn_fwd_bf16_strided(bq, k, v, bo, groups, G, 1, Sk, D, scale, st, (0, 0, 0, 0), False)
+
+        msg, _ = _launch_stats(m, gqa_step, max(1, min(steps, 20)), warmup)
+        algo_g = 2 * n_kv * 2 + 2 * n_q * 2
+        rec["grouped_query_16x8x8"] = {"us_per_launch": msg * 1e3 / len(kvs), "GB/s": len(kvs) * algo_g / (msg * 1e-3) / 1e9,
+                                        "frac": len(kvs) * algo_g / (msg * 1e-3) / 1e9 / HBM_PEAK_GBS}
     return rec
 
 
@@ -777,7 +801,7 @@ def main():
         if "cpu_baseline" in r:
             r["cpu_baseline"]["cpu_model"] = cpu_model
             r["cpu_baseline"]["host_cores"] = os.cpu_count()
-    for k in ("median_ms", "min_ms", "plan_item", "direct_abi_ms_per_step", "vendor_reference", "additive_mask_softcap", "batch_8", "launches_per_step", "us_per_launch"):
+    for k in ("median_ms", "min_ms", "plan_item", "direct_abi_ms_per_step", "vendor_reference", "additive_mask_softcap", "batch_8", "grouped_query_16x8x8", "launches_per_step", "us_per_launch"):
         if k in primary:
             line[k] = primary[k]
     if "cpu_baseline" in primary:
