@@ -558,8 +558,8 @@ size_t mrk_hip_flash_attn_workspace_bytes(int64_t batch, int64_t heads, int64_t 
  * shares one set of keys between batches or heads; output rows, heads and batches must not
  * overlap.  (rows - 1) * row stride * 2 bytes must stay below 4 GiB per operand.
  * In a decode shape (above) heads whose k and v head strides are both zero are served by one pass over their
- * shared keys while heads * sq <= 16 (multi-query attention; grouped-query attention with batch = batch x key
- * heads and heads = query heads per key head). */
+ * shared keys, up to 16 query rows (runs of consecutive heads) per pass (multi-query attention; grouped-query
+ * attention with batch = batch x key heads and heads = query heads per key head). */
 int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
                                         int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal,
                                         const int64_t* strides);

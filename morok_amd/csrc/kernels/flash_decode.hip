@@ -39,8 +39,8 @@ constexpr int kMaxQueries = 16;
 struct DecodeLayout {
     long long q_batch, q_head, k_batch, k_head, v_batch, v_head, o_batch, o_head;  // element strides
     unsigned q_row, k_row, v_row, o_row;                                           // byte strides of a row
-    int heads;  // (batch, head) pairs per batch: the head count, or 1 when the heads are folded into one pair
-    int group;  // heads folded into one pair's query slots (they share K and V: zero head strides), 1 = none
+    int heads;  // pairs per batch: the head count divided by `group`
+    int group;  // consecutive heads folded into one pair's query slots (they share K and V: zero head strides), 1 = none
 };
 
 // attn_mask of the reference (transformer.rs:112-125) as a [batch, head, query, key] view with contiguous keys:
@@ -76,7 +76,7 @@ __global__ __launch_bounds__(decode_waves<kD>() * 64) void flash_decode_split(
     __shared__ __attribute__((aligned(1024))) char smem[kLds];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int jl = lane & 15, blk = lane >> 4;
-    const int bh = blockIdx.y, b = bh / lay.heads, h = bh % lay.heads;
+    const int bh = blockIdx.y, b = bh / lay.heads, h = (bh % lay.heads) * lay.group;  // h: the pair's first head
     const int k_begin = blockIdx.x * keys_per_split;
     const int k_end = k_begin + keys_per_split < Sk ? k_begin + keys_per_split : Sk;
     const unsigned lds_k = (unsigned)(uintptr_t)MRK_FD_LDS(char, smem) + wave * kWaveBytes;
@@ -339,7 +339,7 @@ __global__ __launch_bounds__(256) void flash_decode_merge(const float* __restric
     }
     const float inv = 1.0f / l_tot;
     const f32x4 v = {o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
-    const int b = bh / lay.heads, h = bh % lay.heads, og = q / Sq, orw = q - og * Sq;
+    const int b = bh / lay.heads, h = (bh % lay.heads) * lay.group, og = q / Sq, orw = q - og * Sq;
     char* orow = reinterpret_cast<char*>(O + b * lay.o_batch + (h + og) * lay.o_head) + (size_t)orw * lay.o_row;
     *reinterpret_cast<bf16x4*>(orow + d * 2) = __builtin_convertvector(v, bf16x4);
 }
@@ -385,16 +385,17 @@ size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal) 
 
 // strides: (batch, head, row) element strides of q, k, v and o (validated by the caller: multiples of 8, rows
 // addressable in 32 bits, pointers 16-byte aligned); W: splits * pairs * 16 * (D + 2) floats, needed with several splits
-// (pairs = B * H, or B with fold_heads).
+// (pairs = B * H / group).
 // mask_kind 0: none; 1: Bool bytes, 2: additive bf16, with (batch, head, query row) element strides that are multiples
 // of 4, a mask pointer aligned to four elements and Sk a multiple of 4 (validated by the caller as well).  softcap 0: none.
 int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
                         float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask, int mask_kind,
-                        const long* mask_strides, float softcap, bool fold_heads) {
-    // fold_heads: the H heads of a batch share K and V (zero head strides) and become query slots of one pair
-    const long pairs = fold_heads ? B : B * H, slots = fold_heads ? H * Sq : Sq;
-    if (B <= 0 || H <= 0 || Sq < 1 || slots > kMaxQueries || Sk < 1 || splits < 1 || pairs > 65535) return (int)hipErrorInvalidValue;
-    if (fold_heads && (strides[4] != 0 || strides[7] != 0)) return (int)hipErrorInvalidValue;
+                        const long* mask_strides, float softcap, long group) {
+    // group > 1: runs of `group` consecutive heads share K and V (zero head strides) and become query slots of one pair
+    if (B <= 0 || H <= 0 || group < 1 || H % group) return (int)hipErrorInvalidValue;
+    const long pairs = B * (H / group), slots = group * Sq;
+    if (Sq < 1 || slots > kMaxQueries || Sk < 1 || splits < 1 || pairs > 65535) return (int)hipErrorInvalidValue;
+    if (group > 1 && (strides[4] != 0 || strides[7] != 0)) return (int)hipErrorInvalidValue;
     if (keys_per_split < kChunkKeys || keys_per_split % kChunkKeys || splits * keys_per_split < Sk || (splits - 1) * keys_per_split >= Sk)
         return (int)hipErrorInvalidValue;
     if (splits > 1 && !W) return (int)hipErrorInvalidValue;
@@ -403,8 +404,8 @@ int launch_flash_decode(void* stream, const void* q, const void* k, const void* 
     lay.k_batch = strides[3], lay.k_head = strides[4], lay.k_row = (unsigned)(strides[5] * 2);
     lay.v_batch = strides[6], lay.v_head = strides[7], lay.v_row = (unsigned)(strides[8] * 2);
     lay.o_batch = strides[9], lay.o_head = strides[10], lay.o_row = (unsigned)(strides[11] * 2);
-    lay.heads = fold_heads ? 1 : (int)H;
-    lay.group = fold_heads ? (int)H : 1;
+    lay.heads = (int)(H / group);
+    lay.group = (int)group;
     if (mask_kind < 0 || mask_kind > 2 || (mask_kind != 0 && (!mask || !mask_strides || Sk % 4)) || !(softcap >= 0.0f)) return (int)hipErrorInvalidValue;
     DecodeMask dm{};
     dm.cap = softcap;

@@ -664,8 +664,15 @@ static bool decode_route(void* stream, const void* q, const void* k, const void*
                          const void* mask = nullptr, int mask_kind = 0, const long* mask_strides = nullptr, float softcap = 0.0f) {
     using namespace mrk::dev;
     // heads that share K and V (zero head strides) become query slots of one pair: K and V are read once per batch
-    const bool fold = H > 1 && H * Sq <= 16 && strides[4] == 0 && strides[7] == 0;
-    const long pairs = fold ? B : B * H, slots = fold ? H * Sq : Sq;
+    // (runs of consecutive heads: the largest divisor of the head count that gives at most 16 slots)
+    long group = 1;
+    if (H > 1 && strides[4] == 0 && strides[7] == 0 && Sq >= 1)
+        for (long g = 16 / Sq; g > 1; g--)
+            if (H % g == 0) {
+                group = g;
+                break;
+            }
+    const long pairs = B * (H / group), slots = group * Sq;
     long splits = 0, per = 0;
     if (!flash_decode_plan(pairs, slots, Sk, D, causal, &splits, &per)) return false;
     const void* ptrs[4] = {q, k, v, o};
@@ -681,7 +688,7 @@ static bool decode_route(void* stream, const void* q, const void* k, const void*
         }
     }
     *rc = launch_flash_decode(stream, q, k, v, o, B, H, Sq, Sk, D, scale, strides, splits, per, workspace, mask, mask_kind, mask_strides,
-                              softcap, fold);
+                              softcap, group);
     return true;
 }
 

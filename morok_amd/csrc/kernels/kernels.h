@@ -122,13 +122,13 @@ inline bool flash_fwd_rows_addressable(long rows, long row_bytes, long D) {
 // ranges their f32 partial results go through `workspace` (flash_fwd_workspace_bytes; 0 = one range), which a
 // second kernel merges.  Without a workspace of that size such a shape runs in as many ranges as the workspace holds.
 // Heads that share their keys and values (zero head strides of k and v: multi-query attention, or grouped-query
-// attention with the groups as batches) are folded into one pair's query slots while heads * Sq <= 16, so that K and
-// V are read once per batch instead of once per head.
+// attention with the groups as batches) are folded into one pair's query slots, as many consecutive heads as give at
+// most 16 slots (a divisor of the head count), so that K and V are read once per such run instead of once per head.
 bool flash_decode_plan(long BH, long Sq, long Sk, long D, int causal, long* splits, long* keys_per_split);
 size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal);
 int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
                         float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask = nullptr,
-                        int mask_kind = 0, const long* mask_strides = nullptr, float softcap = 0.0f, bool fold_heads = false);
+                        int mask_kind = 0, const long* mask_strides = nullptr, float softcap = 0.0f, long group = 1);
 int launch_flash_fwd_bf16(void* stream, const void* q, const void* k, const void* v, void* o, long BH, long Sq, long Sk,
                           long D, float scale, int causal, void* workspace = nullptr, size_t workspace_bytes = 0);
 // The same kernel over operands given as views: strides holds (batch, head, row) element

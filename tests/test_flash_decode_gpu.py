@@ -381,11 +381,13 @@ def _attn_shared(dev, q, k1, v1, scale, mask=None, mstrides=None):
 
 
 @pytest.mark.parametrize("d", [128, 64, 256])
-@pytest.mark.parametrize("shape", [(2, 8, 1, 3000), (1, 16, 1, 4096), (3, 4, 4, 777), (8, 4, 1, 1024), (2, 5, 3, 515), (1, 9, 2, 600)])
+@pytest.mark.parametrize("shape", [(2, 8, 1, 3000), (1, 16, 1, 4096), (3, 4, 4, 777), (8, 4, 1, 1024), (2, 5, 3, 515), (1, 9, 2, 600),
+                                   (2, 32, 1, 2048), (1, 12, 2, 1000), (1, 7, 3, 300)])
 def test_decode_heads_sharing_keys_are_folded(dev, oracle, shape, d):
     """Multi-query attention (and grouped-query attention with the groups as batches): the heads of a batch read the
-    same K and V; while heads * Sq <= 16 they become query slots of one pass over the keys.  The oracle's values over
-    broadcast copies; (1, 9, 2, 600) has 18 slots and runs head by head."""
+    same K and V; runs of consecutive heads become query slots of one pass over the keys, as many as give at most 16
+    slots (32 heads: two runs of 16; 9 heads of two rows: runs of 3; 12 of two: runs of 6; 7 of three: head by head).
+    The oracle's values over broadcast copies."""
     B, H, Sq, Sk = shape
     q = synth.normal_bf16((B, H, Sq, d), 95, 0)
     k1, v1 = synth.normal_bf16((B, 1, Sk, d), 95, 1), synth.normal_bf16((B, 1, Sk, d), 95, 2)
@@ -398,8 +400,9 @@ def test_decode_heads_sharing_keys_are_folded(dev, oracle, shape, d):
     assert np.array_equal(_attn_shared(dev, q, k1, v1, scale), got)
 
 
-def test_decode_folded_heads_under_masks(dev, oracle):
-    B, H, Sq, Sk, d = 2, 8, 2, 2052, 128
+@pytest.mark.parametrize("H", [8, 12, 32])
+def test_decode_folded_heads_under_masks(dev, oracle, H):
+    B, Sq, Sk, d = 2, (1 if H == 32 else 2), 2052, 128
     q = synth.normal_bf16((B, H, Sq, d), 96, 0)
     k1, v1 = synth.normal_bf16((B, 1, Sk, d), 96, 1), synth.normal_bf16((B, 1, Sk, d), 96, 2)
     kb, vb = (np.ascontiguousarray(np.broadcast_to(t, (B, H, Sk, d))) for t in (k1, v1))
