@@ -80,8 +80,9 @@ class DecoderBlock:
     def _norm(self, x, weight):
         return x.rms_norm(-1, self.eps).try_mul(weight).cast(uop.BF16)
 
-    def forward(self, tokens):
-        """tokens: int32 Tensor [batch*seq].  Returns the lazy bf16 [batch*seq, hidden] output."""
+    def forward(self, tokens, with_cache=False):
+        """tokens: int32 Tensor [batch*seq].  Returns the lazy bf16 [batch*seq, hidden] output; with_cache: also the
+        rotated keys and the values as [batch, heads, seq, dim] tensors (what `decode_step` takes as its past)."""
         w, T = self.w, self.batch * self.seq
         h = w["emb"].embedding(tokens).contiguous()
         xn = self._norm(h, w["w_an"])
@@ -112,4 +113,37 @@ class DecoderBlock:
             g = gu.try_shrink([(0, T), (0, self.ffn)]).silu().try_mul(gu.try_shrink([(0, T), (self.ffn, 2 * self.ffn)]))
         else:
             g = self._proj(xn2, "W1").silu().try_mul(self._proj(xn2, "W3"))
-        return h2.try_add(self._proj(g, "W2"))
+        out = h2.try_add(self._proj(g, "W2"))
+        return (out, k.contiguous(), v.contiguous()) if with_cache else out
+
+    def decode_step(self, tokens, past_k, past_v, pos):
+        """One new token per sequence against the keys and values of the `pos` tokens before it, the way the reference
+        carries a cache through its attention operator (onnx/src/registry/transformer.rs:74-75: K = cat(past, new) along
+        the sequence axis, then scaled_dot_product_attention): tokens int32 [batch], past_k / past_v bf16
+        [batch, heads, pos, dim] (keys already rotated), pos the new token's position.  Returns the lazy
+        (output [batch, hidden], keys [batch, heads, pos + 1, dim], values): the row a causal forward pass over
+        pos + 1 tokens would give for the last token.  With Linear-layout weights the projections stream their weights
+        once, and the attention is one query per head over pos + 1 keys."""
+        assert self.fused, "decode_step uses the packed projections"
+        w, B, H, D = self.w, self.batch, self.heads, self.dim
+        cos, sin = rope_tables(pos + 1, D)
+        cos_p = Tensor.from_numpy(np.ascontiguousarray(cos[pos].reshape(1, 1, 1, D // 2)))
+        sin_p = Tensor.from_numpy(np.ascontiguousarray(sin[pos].reshape(1, 1, 1, D // 2)))
+        h = w["emb"].embedding(tokens).contiguous()
+        xn = self._norm(h, w["w_an"])
+        qkv = self._proj(xn, "Wqkv")
+        xv = qkv.try_shrink([(0, B), (2 * self.hidden, 3 * self.hidden)])
+        qk = qkv.try_shrink([(0, B), (0, 2 * self.hidden)]).try_reshape([B, 1, 2 * H, D])
+        qk = qk.apply_rotary_emb(cos_p, sin_p, False).cast(uop.BF16).contiguous()
+        q = qk.try_shrink([(0, B), (0, 1), (0, H), (0, D)]).try_permute([0, 2, 1, 3])
+        k_new = qk.try_shrink([(0, B), (0, 1), (H, 2 * H), (0, D)]).try_permute([0, 2, 1, 3])
+        v_new = xv.try_reshape([B, 1, H, D]).try_permute([0, 2, 1, 3])
+        k_all = Tensor.cat([past_k, k_new], 2).contiguous()
+        v_all = Tensor.cat([past_v, v_new], 2).contiguous()
+        a = q.scaled_dot_product_attention(k_all, v_all)
+        a = a.try_permute([0, 2, 1, 3]).try_reshape([B, self.hidden])
+        h2 = h.try_add(self._proj(a, "Wo")).contiguous()
+        xn2 = self._norm(h2, w["w_fn"])
+        gu = self._proj(xn2, "W13")
+        g = gu.try_shrink([(0, B), (0, self.ffn)]).silu().try_mul(gu.try_shrink([(0, B), (self.ffn, 2 * self.ffn)]))
+        return h2.try_add(self._proj(g, "W2")), k_all, v_all

@@ -174,3 +174,47 @@ def test_memory_planner_on_and_off_give_the_same_bits_in_less_memory(dev, oracle
     monkeypatch.delenv("MOROK_NO_MEMORY_PLANNER")
     _, out3, _ = run_block(cfg, tok, w)
     assert np.array_equal(out3.to_numpy(), planned)
+
+
+@pytest.mark.parametrize("cfg,linear_layout", [
+    (dict(batch=2, seq=300, hidden=512, heads=4, ffn=1280, vocab=777, eps=1e-6), True),
+    (dict(batch=1, seq=600, hidden=1024, heads=8, ffn=2816, vocab=500, eps=1e-6), False),
+    (dict(batch=4, seq=1100, hidden=256, heads=2, ffn=512, vocab=300, eps=1e-6), True),
+], ids=["h512_299past", "h1024_599past", "h256_1099past"])
+def test_decode_step_over_cached_keys_is_the_last_row_of_a_causal_pass(dev, oracle, cfg, linear_layout):
+    """One new token against the cached keys and values of the tokens before it (K = cat(past, new), then attention with
+    one query per head, as the reference's attention operator carries its past: onnx/src/registry/transformer.rs:74-75)
+    gives the row a causal pass over the whole sequence gives for its last token: against the oracle's block over all
+    tokens, and against this library's own full pass.  The attention of the step is the kernel that streams the keys."""
+    from morok_amd import decoder, synth, tensor
+
+    B, S = cfg["batch"], cfg["seq"]
+    w = decoder.synthetic_weights(cfg["hidden"], cfg["ffn"], cfg["vocab"], seed=8)
+    tok = synth.randint((B * S,), 8, 1, cfg["vocab"]).reshape(B, S)
+    # the whole sequence, causal
+    full_cfg = dict(cfg)
+    blk, out, _ = run_block(full_cfg, tok.reshape(-1), w, linear_layout=linear_layout)
+    full = out.to_numpy().reshape(B, S, cfg["hidden"])
+    ref = oracle.decoder_block_bf16(tok.reshape(-1), w, blk.cos_host, blk.sin_host, B, S, cfg["hidden"], cfg["heads"], cfg["ffn"],
+                                    cfg["eps"]).reshape(B, S, cfg["hidden"])
+    # the first S - 1 tokens, keeping their keys and values
+    P = S - 1
+    pre = decoder.DecoderBlock(w, B, P, cfg["hidden"], cfg["heads"], cfg["ffn"], cfg["eps"], linear_layout=linear_layout)
+    o, k, v = pre.forward(tensor.Tensor.from_numpy(np.ascontiguousarray(tok[:, :P]).reshape(-1).astype(np.int32)), with_cache=True)
+    o.realize(), k.realize(), v.realize()
+    assert tuple(k.shape) == (B, cfg["heads"], P, cfg["hidden"] // cfg["heads"])
+    # the last token against that cache
+    step = decoder.DecoderBlock(w, B, 1, cfg["hidden"], cfg["heads"], cfg["ffn"], cfg["eps"], linear_layout=linear_layout)
+    y, k_all, v_all = step.decode_step(tensor.Tensor.from_numpy(np.ascontiguousarray(tok[:, P]).astype(np.int32)), k, v, P)
+    y.realize()
+    kernels = y.kernels()
+    got = y.to_numpy()
+    assert got.shape == (B, cfg["hidden"])
+    assert rel_err(got, ref[:, P]) <= 2e-2
+    assert rel_err(got, full[:, P]) <= 2e-2
+    att = [n for n in kernels if n.startswith("flash_fwd")]
+    assert len(att) == 1 and ("_%d_1_%d" % (B * cfg["heads"], S)) in att[0], kernels   # one query per head over S keys
+    # the cache the step hands on: the past with the new token's key and value appended
+    ka, va = k_all.to_numpy(), v_all.to_numpy()
+    assert ka.shape == (B, cfg["heads"], S, cfg["hidden"] // cfg["heads"])
+    assert np.array_equal(ka[:, :, :P], k.to_numpy()) and np.array_equal(va[:, :, :P], v.to_numpy())
