@@ -2,7 +2,7 @@
 // tensor/src/transformer.rs:78-137 with Sq of 1 to 16): O = softmax(Q K^T * scale) V is a stream over K and V,
 // 4 * Sk * D bytes per (batch, head) against a few flops per byte, and with few (batch, head) pairs the kernel that
 // gives every pair one workgroup leaves most of the chip without work.  Here the key sequence is split as well:
-// grid = (splits, batch * heads), a workgroup owns a contiguous range of keys, its waves take the range's 32-key
+// grid = (splits, pairs), a workgroup owns a contiguous range of keys, its waves take the range's 32-key
 // chunks in turn.  A wave copies its chunk of K and of V (32 rows each) with direct global -> LDS loads into a
 // region of its own (1 KB per instruction, non-temporal: every byte is read once), so the loop has no barrier,
 // and what streams is bounded by the bytes in flight per CU, i.e. by what the LDS holds.
@@ -16,8 +16,13 @@
 // point at), pointed at rows 4 g + 0..3 of either block.  Running maximum and sum per query as in any online
 // softmax; a query's maximum sits in four lanes (l % 16 equal), two exchanges per chunk.
 // At the end the waves' (maximum, sum, O) meet in LDS and are merged in a fixed order; with one split the
-// workgroup writes O, otherwise f32 partial results W[split][batch * head][16][D + 2] (the unnormalised O, then
+// workgroup writes O, otherwise f32 partial results W[split][pair][16][D + 2] (the unnormalised O, then
 // maximum and sum), which flash_decode_merge folds the same way.  Results do not depend on scheduling.
+// A pair is a (batch, head), or a (batch, run of consecutive heads) when those heads share their K and V (zero
+// head strides: multi-query / grouped-query attention): the run's heads then occupy the 16 query slots together
+// and K and V are read once for all of them.  attn_mask (Bool bytes or additive bf16, any broadcast layout) and
+// softcap of the reference (transformer.rs:112-132) are template options: a lane loads the mask of its eight keys
+// with the chunk's copies and applies it, then the cap, to its scores before the maximum.
 #include <hip/hip_runtime.h>
 
 #include "kernels.h"
