@@ -540,7 +540,7 @@ int mrk_hip_gemm_bf16_rope(int device_id, const void* a, const void* b, const vo
  * bf16, D = 256, 128 or 64 (other head dims: INVALID_ARGUMENT here, the composed graph through the tensor
  * API), scale > 0 (the reference default is 1/sqrt(D), transformer.rs:90-91).
  * Causal rule of the reference: key j is visible to query i iff j <= i (transformer.rs:103-109).
- * Up to 16 queries without the causal rule against 256 keys and more (the decode step of a model that keeps
+ * Up to 32 queries without the causal rule against 256 keys and more (the decode step of a model that keeps
  * its keys and values: the same function of the reference, called with a short q) take a kernel that streams
  * K and V once and splits the key sequence over workgroups where (batch, head) pairs alone would not fill the
  * chip; the ranges' partial results (f32) are merged by a second kernel in a fixed order.  This call and the
@@ -558,7 +558,7 @@ size_t mrk_hip_flash_attn_workspace_bytes(int64_t batch, int64_t heads, int64_t 
  * shares one set of keys between batches or heads; output rows, heads and batches must not
  * overlap.  (rows - 1) * row stride * 2 bytes must stay below 4 GiB per operand.
  * In a decode shape (above) heads whose k and v head strides are both zero are served by one pass over their
- * shared keys, up to 16 query rows (runs of consecutive heads) per pass (multi-query attention; grouped-query
+ * shared keys, up to 32 query rows (runs of consecutive heads) per pass (multi-query attention; grouped-query
  * attention with batch = batch x key heads and heads = query heads per key head). */
 int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void* k, const void* v, void* o, int64_t batch,
                                         int64_t heads, int64_t sq, int64_t sk, int64_t d, float scale, int causal,
@@ -577,7 +577,7 @@ int mrk_hip_flash_attn_fwd_bf16_strided(int device_id, const void* q, const void
  * takes part in the softmax, exactly as the reference's graph computes it; the kernel then visits
  * every key tile.  A row whose keys are all masked out (no softcap) is NaN, as softmax over -inf
  * only is.  Without mask and softcap this is mrk_hip_flash_attn_fwd_bf16_strided.
- * Without the causal rule a decode shape (up to 16 queries, 256 keys and more: a batch of sequences of different
+ * Without the causal rule a decode shape (up to 32 queries, 256 keys and more: a batch of sequences of different
  * lengths decoding under a key-padding mask [batch, 1, 1, sk]) takes the kernel that splits the key sequence, like
  * the unmasked call, mask and softcap inside it; key ranges without a visible key weigh nothing.
  * Builtin Program kind "flash_fwd_bf16_ext" (29 params, buffers {o, q, k, v, mask}; optionally a 30th, the bytes

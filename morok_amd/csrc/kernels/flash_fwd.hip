@@ -664,10 +664,10 @@ static bool decode_route(void* stream, const void* q, const void* k, const void*
                          const void* mask = nullptr, int mask_kind = 0, const long* mask_strides = nullptr, float softcap = 0.0f) {
     using namespace mrk::dev;
     // heads that share K and V (zero head strides) become query slots of one pair: K and V are read once per batch
-    // (runs of consecutive heads: the largest divisor of the head count that gives at most 16 slots)
+    // (runs of consecutive heads: the largest divisor of the head count that gives at most 32 slots)
     long group = 1;
     if (H > 1 && strides[4] == 0 && strides[7] == 0 && Sq >= 1)
-        for (long g = 16 / Sq; g > 1; g--)
+        for (long g = 32 / Sq; g > 1; g--)
             if (H % g == 0) {
                 group = g;
                 break;
@@ -679,7 +679,7 @@ static bool decode_route(void* stream, const void* q, const void* k, const void*
     for (const void* p : ptrs)
         if (reinterpret_cast<uintptr_t>(p) % 16) return false;
     if (splits > 1) {  // as many key ranges as the workspace holds
-        const size_t slice = (size_t)pairs * 16 * (D + 2) * sizeof(float);
+        const size_t slice = (size_t)pairs * flash_decode_slot_capacity(slots) * (D + 2) * sizeof(float);
         const long fit = workspace ? (long)(workspace_bytes / slice) : 0;
         if (fit < splits) {
             const long want = fit < 2 ? 1 : fit;

@@ -117,14 +117,15 @@ inline bool flash_fwd_rows_addressable(long rows, long row_bytes, long D) {
 }
 // O = softmax(Q K^T * scale [causal]) V; Q [BH,Sq,D], K/V [BH,Sk,D], O [BH,Sq,D] bf16, D = 256, 128 or 64,
 // scale > 0.  Causal: key j visible to query i iff j <= i.
-// Up to 16 queries without the causal rule against 256 keys and more (a decode step over a key/value cache) take
+// Up to 32 queries without the causal rule against 256 keys and more (a decode step over a key/value cache) take
 // a kernel that also splits the key sequence over workgroups (flash_decode_plan tells how); with several key
 // ranges their f32 partial results go through `workspace` (flash_fwd_workspace_bytes; 0 = one range), which a
 // second kernel merges.  Without a workspace of that size such a shape runs in as many ranges as the workspace holds.
 // Heads that share their keys and values (zero head strides of k and v: multi-query attention, or grouped-query
 // attention with the groups as batches) are folded into one pair's query slots, as many consecutive heads as give at
-// most 16 slots (a divisor of the head count), so that K and V are read once per such run instead of once per head.
+// most 32 slots (a divisor of the head count), so that K and V are read once per such run instead of once per head.
 bool flash_decode_plan(long BH, long Sq, long Sk, long D, int causal, long* splits, long* keys_per_split);
+long flash_decode_slot_capacity(long slots);
 size_t flash_fwd_workspace_bytes(long BH, long Sq, long Sk, long D, int causal);
 int launch_flash_decode(void* stream, const void* q, const void* k, const void* v, void* o, long B, long H, long Sq, long Sk, long D,
                         float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask = nullptr,

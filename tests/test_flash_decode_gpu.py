@@ -54,7 +54,7 @@ def _check(o, ref, tight=8e-3):
 
 
 SHAPES = [(1, 2, 1, 256), (2, 3, 1, 1000), (1, 4, 5, 777), (1, 1, 16, 4100), (1, 32, 1, 4096), (4, 8, 3, 2048), (3, 1, 16, 515),
-          (2, 100, 1, 300), (1, 8, 2, 8192)]
+          (2, 100, 1, 300), (1, 8, 2, 8192), (1, 4, 17, 777), (2, 2, 32, 1000), (1, 8, 24, 4096)]   # 17 and more: two query blocks
 
 
 @pytest.mark.parametrize("d", [128, 64, 256])
@@ -79,12 +79,13 @@ def test_decode_shapes_split_the_keys_where_pairs_are_few():
     assert ws(1, 32, 1, 4096, 128, 0) > 0 and ws(1, 8, 4, 8192, 64, 0) > 0 and ws(2, 16, 16, 2048, 256, 0) > 0
     assert ws(1, 32, 1, 4096, 128, 0) % (32 * 16 * 130 * 4) == 0  # whole slices of [pairs][16][D + 2] floats
     # the causal rule, many queries, few keys, no kernel for the head dim: no scratch
-    for args in ((1, 32, 1, 4096, 128, 1), (1, 32, 17, 4096, 128, 0), (1, 32, 1, 255, 128, 0), (1, 32, 1, 4096, 96, 0), (0, 32, 1, 4096, 128, 0)):
+    for args in ((1, 32, 1, 4096, 128, 1), (1, 32, 33, 4096, 128, 0), (1, 32, 1, 255, 128, 0), (1, 32, 1, 4096, 96, 0), (0, 32, 1, 4096, 128, 0)):
         assert ws(*args) == 0, args
     # 512 pairs fill the chip by themselves, but should their heads share K and V (the launchers see the strides, this
     # query does not) they fold into as few as 32 pairs, which split their keys: a bounded reserve for that
     assert 0 < ws(16, 32, 1, 4096, 128, 0) <= 4 << 20
-    assert ws(16, 32, 16, 4096, 128, 0) == 0   # 16 queries a head: nothing to fold
+    assert ws(16, 32, 32, 4096, 128, 0) == 0   # 32 queries a head: nothing to fold
+    assert ws(1, 32, 17, 4096, 128, 0) == 6 * 32 * 32 * 130 * 4   # 17 and more: 32 slots a pair (six key ranges, 32 pairs)
 
 
 @pytest.mark.parametrize("d", [128, 64, 256])
@@ -128,14 +129,17 @@ def test_decode_rows_past_the_end_do_not_leak(dev, oracle):
 
 @pytest.mark.parametrize("d", [128, 64])
 def test_decode_agrees_with_the_tiled_kernel(dev, d):
-    """17 queries take the tiled kernel, their first 16 alone the split one: the same keys, the same values to
-    the tolerance of either."""
+    """33 queries take the tiled kernel, their first 32 alone and their first 16 alone the split one (two query blocks,
+    one): the same keys, the same values to the tolerance of either; a query's result does not depend on the block
+    it sits in."""
     B, H, Sk = 2, 4, 3000
     scale = float(d) ** -0.5
-    q, k, v = _inputs(B, H, 17, Sk, d, seed=74)
+    q, k, v = _inputs(B, H, 33, Sk, d, seed=74)
     tiled = _attn(dev, q, k, v, scale)
-    split = _attn(dev, np.ascontiguousarray(q[:, :, :16]), k, v, scale)
-    _check(split, tiled[:, :, :16], tight=1e-2)
+    split = _attn(dev, np.ascontiguousarray(q[:, :, :32]), k, v, scale)
+    _check(split, tiled[:, :, :32], tight=1e-2)
+    assert np.array_equal(_attn(dev, np.ascontiguousarray(q[:, :, :16]), k, v, scale), split[:, :, :16])
+    assert np.array_equal(_attn(dev, np.ascontiguousarray(q[:, :, 16:32]), k, v, scale), split[:, :, 16:])
     # and the causal rule keeps the tiled kernel (a single query then sees key 0 only)
     o = _attn(dev, np.ascontiguousarray(q[:, :, :1]), k, v, scale, causal=True)
     assert np.array_equal(o[:, :, 0], v[:, :, 0])
@@ -193,7 +197,7 @@ def test_decode_random_shapes(dev, oracle, seed):
     rng = np.random.default_rng(5000 + seed)
     d = int(rng.choice([64, 128, 256]))
     B, H = int(rng.integers(1, 4)), int(rng.integers(1, 9))
-    Sq, Sk = int(rng.integers(1, 17)), int(rng.integers(256, 3000))
+    Sq, Sk = int(rng.integers(1, 33)), int(rng.integers(256, 3000))
     scale = float(rng.choice([float(d) ** -0.5, 0.05, 0.2]))
     q, k, v = _inputs(B, H, Sq, Sk, d, seed=80 + seed)
     _check(_attn(dev, q, k, v, scale), oracle.sdpa_bf16(q, k, v, scale, causal=False))
@@ -275,7 +279,7 @@ def _attn_masked(dev, q, k, v, scale, mask, mstrides, mode="abi", cap=0.0):
 
 @pytest.mark.parametrize("d", [128, 64, 256])
 @pytest.mark.parametrize("kind,layout", [("bool", "b11k"), ("bool", "bhqk"), ("add", "1hqk"), ("add", "bhqk"), ("bool", "qk")])
-@pytest.mark.parametrize("shape", [(2, 4, 1, 1000), (1, 32, 1, 4096), (3, 2, 5, 516), (1, 2, 16, 2052)])
+@pytest.mark.parametrize("shape", [(2, 4, 1, 1000), (1, 32, 1, 4096), (3, 2, 5, 516), (1, 2, 16, 2052), (1, 2, 20, 516)])
 def test_decode_mask_vs_oracle(dev, oracle, shape, kind, layout, d):
     """attn_mask (transformer.rs:112-125) over decode shapes: a key-padding mask [B, 1, 1, Sk] is what a batch of
     sequences of different lengths decodes with.  The oracle's restatement, through the C entry point and through a
@@ -382,11 +386,12 @@ def _attn_shared(dev, q, k1, v1, scale, mask=None, mstrides=None):
 
 @pytest.mark.parametrize("d", [128, 64, 256])
 @pytest.mark.parametrize("shape", [(2, 8, 1, 3000), (1, 16, 1, 4096), (3, 4, 4, 777), (8, 4, 1, 1024), (2, 5, 3, 515), (1, 9, 2, 600),
-                                   (2, 32, 1, 2048), (1, 12, 2, 1000), (1, 7, 3, 300)])
+                                   (2, 32, 1, 2048), (1, 12, 2, 1000), (1, 7, 3, 300), (1, 64, 1, 1000), (1, 11, 3, 300)])
 def test_decode_heads_sharing_keys_are_folded(dev, oracle, shape, d):
     """Multi-query attention (and grouped-query attention with the groups as batches): the heads of a batch read the
-    same K and V; runs of consecutive heads become query slots of one pass over the keys, as many as give at most 16
-    slots (32 heads: two runs of 16; 9 heads of two rows: runs of 3; 12 of two: runs of 6; 7 of three: head by head).
+    same K and V; runs of consecutive heads become query slots of one pass over the keys, as many as give at most 32
+    slots (64 heads: two runs of 32; 12 heads of two rows: one run of 24 slots; 7 heads of three rows: one run of 21;
+    11 of three: head by head, 33 slots being too many and 11 having no smaller divisor but 1).
     The oracle's values over broadcast copies."""
     B, H, Sq, Sk = shape
     q = synth.normal_bf16((B, H, Sq, d), 95, 0)
