@@ -398,8 +398,11 @@ using namespace mrk::dev;
 bool flash_decode_plan(long BH, long Sq, long Sk, long D, int causal, long* splits, long* keys_per_split) {
     if (causal || Sq < 1 || Sq > kMaxQueries || Sk < 256 || Sk > (1L << 24) || BH < 1 || BH > 65535) return false;
     if (D != 256 && D != 128 && D != 64) return false;
-    const long max_splits = Sk / 512 > 0 ? Sk / 512 : 1;
-    long want = (192 + BH / 2) / BH;
+    // (two chunks per wave and range at least: 512 keys with eight waves, 256 with the four of head dim 256, whose
+    // workgroups, one per CU, measured best at one per CU: 21 against 24 us at [1, 16, 1, 4096], 30 against 33 with 32 pairs)
+    const long min_keys = D == 256 ? 256 : 512, target = D == 256 ? 256 : 192;
+    const long max_splits = Sk / min_keys > 0 ? Sk / min_keys : 1;
+    long want = (target + BH / 2) / BH;
     want = want < max_splits ? want : max_splits;
     want = want < 1 ? 1 : want;
     const long per = ((Sk + want - 1) / want + kChunkKeys - 1) / kChunkKeys * kChunkKeys;
