@@ -60,3 +60,25 @@ def test_compile_error_is_reported():
     with pytest.raises(morok_amd.MorokHipError) as e:
         morok_amd.compile_spec(spec)
     assert e.value.code == 10 and "bad" in e.value.message
+
+
+def test_workspace_queries_are_host_side_and_bounded():
+    """The scratch sizes a caller asks about before it launches are pure functions of the shape (no device needed):
+    zero where the product / attention needs none, whole slices otherwise, at most 16 MiB for attention."""
+    from morok_amd._ffi import lib
+
+    att = lib.mrk_hip_flash_attn_workspace_bytes
+    # one to 32 queries, no causal rule, 256 keys and more: the key sequence may be split over workgroups
+    assert att(1, 32, 1, 4096, 128, 0) == 6 * 32 * 16 * 130 * 4        # six key ranges, 32 pairs, 16 slots of 128 + 2 floats
+    assert att(1, 32, 17, 4096, 128, 0) == 6 * 32 * 32 * 130 * 4       # from 17 queries on 32 slots a pair
+    for args in ((1, 32, 1, 4096, 128, 1), (1, 32, 33, 4096, 128, 0), (1, 32, 1, 255, 128, 0), (1, 32, 1, 4096, 96, 0),
+                 (0, 32, 1, 4096, 128, 0), (8, 32, 4096, 4096, 128, 1)):
+        assert att(*args) == 0, args
+    for b in (1, 2, 3, 7, 16, 64, 1000):
+        for sq in (1, 4, 16, 32):
+            for d in (64, 128, 256):
+                for sk in (256, 1000, 4096, 1 << 17):
+                    ws = att(b, 32, sq, sk, d, 0)
+                    assert ws % ((d + 2) * 4 * 16) == 0 and ws <= 16 << 20, (b, sq, d, sk, ws)
+    gemm = lib.mrk_hip_gemm_bf16_workspace_bytes
+    assert gemm(4096, 4096, 4096, 1) == 0 and gemm(128, 4096, 11008, 1) > 0 and gemm(0, 4096, 4096, 1) == 0
