@@ -434,3 +434,39 @@ def test_decode_folded_heads_through_the_tensor_api(dev, oracle):
     kb, vb = (np.ascontiguousarray(np.broadcast_to(x, (B, H, Sk, d))) for x in (k1, v1))
     _check(got, oracle.sdpa_bf16(q, kb, vb, float(d) ** -0.5, causal=False))
     assert np.array_equal(got, _attn_shared(dev, q, k1, v1, float(d) ** -0.5))
+
+
+def test_decode_attention_in_a_replayed_graph(dev, oracle):
+    """The split kernel and its merge as two kernel nodes of a plan recorded into a HIP graph, the scratch an
+    intermediate of the plan: every replay, with eager work and synchronisations in between and new queries each
+    time, gives what the eager launches give."""
+    from morok_amd import tensor as T, uop
+
+    B, H, Sk, d = 1, 8, 2048, 128
+    q, k, v = _inputs(B, H, 2, Sk, d, seed=98)
+    tq = T.Tensor.from_numpy(q, uop.BF16)
+    out = tq.scaled_dot_product_attention(T.Tensor.from_numpy(k, uop.BF16), T.Tensor.from_numpy(v, uop.BF16))
+    plan = out.prepare()
+    assert out.kernels()[0].endswith("_splitkv")
+    qbuf = tq.buffer()
+
+    def result():
+        dev.synchronize()
+        return out.buffer().copyout(np.uint16, q.shape).copy()
+
+    plan.execute()
+    _check(result(), oracle.sdpa_bf16(q, k, v, float(d) ** -0.5, causal=False))
+    for i in range(4):
+        qi = synth.normal_bf16(q.shape, 99, i)
+        qbuf.copyin(qi)
+        plan.execute()
+        want = result()
+        out.buffer().copyin(np.zeros(q.size, np.uint16))   # the replay must rewrite it
+        plan.execute_graph()
+        got = result()
+        assert np.array_equal(got, want), i
+        _check(got, oracle.sdpa_bf16(qi, k, v, float(d) ** -0.5, causal=False))
+        x = synth.normal((64, 512), 5, i, sigma=1.0)       # unrelated eager work between the replays
+        bx = morok_amd.Buffer.from_numpy(x, dev.device_id)
+        ops.softmax_f32(bx, dev.buffer(x.nbytes), 64, 512, dev.device_id)
+        dev.synchronize()
