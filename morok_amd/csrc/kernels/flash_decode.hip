@@ -438,7 +438,7 @@ int launch_flash_decode(void* stream, const void* q, const void* k, const void* 
                         float scale, const long* strides, long splits, long keys_per_split, void* W, const void* mask, int mask_kind,
                         const long* mask_strides, float softcap, long group) {
     // group > 1: runs of `group` consecutive heads share K and V (zero head strides) and become query slots of one pair
-    if (B <= 0 || H <= 0 || group < 1 || H % group) return (int)hipErrorInvalidValue;
+    if (B <= 0 || H <= 0 || group < 1 || H % group || !strides || !q || !k || !v || !o) return (int)hipErrorInvalidValue;
     const long pairs = B * (H / group), slots = group * Sq;
     if (Sq < 1 || slots > kMaxQueries || Sk < 1 || splits < 1 || pairs > 65535) return (int)hipErrorInvalidValue;
     if (group > 1 && (strides[4] != 0 || strides[7] != 0)) return (int)hipErrorInvalidValue;
